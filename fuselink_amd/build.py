@@ -1,0 +1,94 @@
+"""Builds libnccl-net-fuselink.so (the HIP data path + the net plugin) for gfx950, in-tree.
+
+Run as ``python -m fuselink_amd.build``.  hipcc cross-compiles without a GPU.  The artifact name
+follows the reference's Makefile (``libnccl-net-fuselink.so``, Makefile:8 in the FuseLink tree) so
+that ``NCCL_NET_PLUGIN=fuselink`` finds it.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIBNAME = "libnccl-net-fuselink.so"
+
+SOURCES = ["fl_kernels.hip", "fl_vmm.cc", "fl_monitor.cc", "fl_plugin.cc"]
+
+# -packed-fp32-ops: keep the compiler from forming packed FP32 instructions (none are wanted in a
+# byte mover, and some forms are unreliable on this hardware).
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-pthread",
+    "-Wall", "-Wno-unused-function",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; a ROCm toolchain is required to build the gfx950 library")
+    return exe
+
+
+def lib_path() -> str:
+    return os.path.join(LIBDIR, LIBNAME)
+
+
+def build_library(verbose: bool = True) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    cmd = [hipcc(), *FLAGS, "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, *srcs, "-o", lib_path(), "-ldl"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "packed-fp32-ops"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + err)
+    if verbose and err.strip():
+        print(err)
+    return lib_path()
+
+
+def build_harness(verbose: bool = True) -> str | None:
+    """The C++ plugin harness (dlopen()s the library exactly as a communication library would)."""
+    src = os.path.join(ROOT, "tests", "harness", "plugin_harness.cc")
+    if not os.path.exists(src):
+        return None
+    out = os.path.join(ROOT, "tests", "harness", "plugin_harness")
+    cmd = [hipcc(), "-O2", "-std=c++17", "-pthread", "-I" + os.path.join(ROOT, "include"), src, "-o", out, "-ldl"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("harness build failed:\n" + res.stderr)
+    return out
+
+
+def build_oracle(verbose: bool = True) -> None:
+    """Compiles the CPU oracle (test infrastructure) and, where the reference tree is present,
+    the reference's own monitor client under oracle/_ref."""
+    cmd = ["make", "-C", os.path.join(ROOT, "oracle"), "all"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("oracle build failed:\n" + res.stdout + res.stderr)
+    if verbose:
+        print(res.stdout.strip())
+
+
+def build_all(verbose: bool = True) -> None:
+    build_library(verbose)
+    build_harness(verbose)
+    build_oracle(verbose)
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

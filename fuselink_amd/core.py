@@ -1,0 +1,262 @@
+"""Host-side driver of the gfx950 data path: thin, typed wrappers over the C ABI in
+include/fuselink_hip.h.  PyTorch is used only to own device memory and streams."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import MAX_LANES, ChunkDesc, SchedHdr, SchedParams, SchedState, Windows, check
+
+TILE_BYTES = 32768
+UNIT_BYTES = 2 * 1024 * 1024
+SCHED_RESET_OFFSETS = 1
+SCHED_MIRROR = 2
+SCHED_F_NO_CREDIT = 1
+
+DESC_DTYPE = np.dtype([("src_off", "<u8"), ("win_off", "<u8"), ("len", "<u4"), ("lane", "<u4"),
+                       ("tile_base", "<u4"), ("epoch", "<u4")])
+HDR_DTYPE = np.dtype([("total_bytes", "<u8"), ("total_tiles", "<u4"), ("n_chunks", "<u4"), ("flags", "<u4"),
+                      ("pad", "<u4"), ("lane_bytes", "<u8", (MAX_LANES,)), ("lane_chunks", "<u4", (MAX_LANES,))])
+STATE_DTYPE = np.dtype([("epoch_bytes", "<u8"), ("chunk_index", "<u8"), ("lane_off", "<u8", (MAX_LANES,))])
+assert DESC_DTYPE.itemsize == C.sizeof(ChunkDesc) == 32
+assert HDR_DTYPE.itemsize == C.sizeof(SchedHdr)
+assert STATE_DTYPE.itemsize == C.sizeof(SchedState)
+
+
+def init(device: int = 0) -> None:
+    check(_lib.load().flh_init(device))
+
+
+def tune(key: str, value: int) -> None:
+    check(_lib.load().flh_tune(key.encode(), int(value)))
+
+
+def _stream_ptr(stream: Optional[torch.cuda.Stream]) -> C.c_void_p:
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _dev_bytes(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+@dataclass
+class Schedule:
+    """Device-resident chunk -> lane table and its summary."""
+    table: torch.Tensor      # uint8 [n * 32]
+    hdr: torch.Tensor        # uint8 [sizeof(flh_sched_hdr)]
+    n_chunks: int
+    tile_bytes: int
+
+    def table_numpy(self) -> np.ndarray:
+        raw = self.table[: self.n_chunks * DESC_DTYPE.itemsize].cpu().numpy()
+        return raw.view(DESC_DTYPE).copy()
+
+    def hdr_numpy(self) -> np.ndarray:
+        return self.hdr.cpu().numpy().view(HDR_DTYPE)[0].copy()
+
+
+def new_state(device="cuda") -> torch.Tensor:
+    return torch.zeros(STATE_DTYPE.itemsize, dtype=torch.uint8, device=device)
+
+
+def state_numpy(state: torch.Tensor) -> np.ndarray:
+    return state.cpu().numpy().view(STATE_DTYPE)[0].copy()
+
+
+def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Optional[torch.Tensor] = None,
+             total_bytes: int = 0, chunk_bytes: int = 0, src_off: Optional[torch.Tensor] = None, src_base: int = 0,
+             epoch_len: int = 0, tile_bytes: int = TILE_BYTES, mode: int = 0, state: Optional[torch.Tensor] = None,
+             out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None) -> Schedule:
+    """Launches the scheduler kernel (flh_schedule).  `credits` is a uint32/int32 device tensor of
+    shape [rows, n_lanes]; `sizes` a uint32/int32 device tensor of chunk sizes, or None for the
+    uniform split of `total_bytes` by `chunk_bytes`."""
+    lib = _lib.load()
+    if credits.dim() == 1:
+        credits = credits.view(1, -1)
+    assert credits.is_cuda and credits.dtype in (torch.int32, torch.uint32) and credits.is_contiguous()
+    assert credits.shape[1] == n_lanes
+    if sizes is not None:
+        assert sizes.is_cuda and sizes.dtype in (torch.int32, torch.uint32) and sizes.is_contiguous()
+        n = sizes.numel()
+    else:
+        n = (total_bytes + chunk_bytes - 1) // chunk_bytes if chunk_bytes else 0
+    if src_off is not None:
+        assert src_off.is_cuda and src_off.dtype in (torch.int64, torch.uint64) and src_off.numel() == n
+    dev = credits.device
+    if out is None:
+        out = Schedule(_dev_bytes(n * DESC_DTYPE.itemsize, dev), _dev_bytes(HDR_DTYPE.itemsize, dev), n, tile_bytes)
+    else:
+        assert out.table.numel() >= n * DESC_DTYPE.itemsize
+        out.n_chunks, out.tile_bytes = n, tile_bytes
+    p = SchedParams(_ptr(sizes), total_bytes, chunk_bytes, _ptr(src_off), src_base, n, n_lanes, _ptr(credits),
+                    credits.shape[0], epoch_len, quantum, tile_bytes, mode, _ptr(state), _ptr(out.table), _ptr(out.hdr))
+    check(lib.flh_schedule(C.byref(p), _stream_ptr(stream)))
+    return out
+
+
+def make_windows(bases: Sequence[int], caps: Sequence[int]) -> Windows:
+    w = Windows()
+    w.n_lanes = len(bases)
+    for l, (b, c) in enumerate(zip(bases, caps)):
+        w.base[l] = b
+        w.cap[l] = c
+    return w
+
+
+def windows_from_tensors(tensors: Sequence[torch.Tensor]) -> Windows:
+    return make_windows([t.data_ptr() for t in tensors], [t.numel() * t.element_size() for t in tensors])
+
+
+def new_status(device="cuda") -> torch.Tensor:
+    return torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def stripe(src: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tensor,
+           stream: Optional[torch.cuda.Stream] = None) -> None:
+    check(_lib.load().flh_stripe(_ptr(src), src.numel() * src.element_size(), C.byref(win), _ptr(sched.table),
+                                 _ptr(sched.hdr), sched.n_chunks, sched.tile_bytes, _ptr(status), _stream_ptr(stream)))
+
+
+def reassemble(dst: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tensor,
+               stream: Optional[torch.cuda.Stream] = None) -> None:
+    check(_lib.load().flh_reassemble(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), _ptr(sched.table),
+                                     _ptr(sched.hdr), sched.n_chunks, sched.tile_bytes, _ptr(status),
+                                     _stream_ptr(stream)))
+
+
+def gather_pages(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int, pages_per_chunk: int, win: Windows,
+                 sched: Schedule, status: torch.Tensor, use_lds: bool = False,
+                 stream: Optional[torch.cuda.Stream] = None) -> None:
+    nbytes = pool.numel() * pool.element_size()
+    check(_lib.load().flh_gather_pages(_ptr(pool), nbytes // page_bytes, _ptr(page_table), page_bytes, pages_per_chunk,
+                                       C.byref(win), _ptr(sched.table), sched.n_chunks, int(use_lds), _ptr(status),
+                                       _stream_ptr(stream)))
+
+
+def scatter_pages(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int, pages_per_chunk: int, win: Windows,
+                  sched: Schedule, status: torch.Tensor, use_lds: bool = False,
+                  stream: Optional[torch.cuda.Stream] = None) -> None:
+    nbytes = pool.numel() * pool.element_size()
+    check(_lib.load().flh_scatter_pages(_ptr(pool), nbytes // page_bytes, _ptr(page_table), page_bytes, pages_per_chunk,
+                                        C.byref(win), _ptr(sched.table), sched.n_chunks, int(use_lds), _ptr(status),
+                                        _stream_ptr(stream)))
+
+
+def copy(dst: torch.Tensor, src: torch.Tensor, stream: Optional[torch.cuda.Stream] = None) -> None:
+    nbytes = src.numel() * src.element_size()
+    assert dst.numel() * dst.element_size() >= nbytes
+    check(_lib.load().flh_copy(_ptr(dst), _ptr(src), nbytes, _stream_ptr(stream)))
+
+
+def qp_split(size: int, nqps: int):
+    off = (C.c_int * nqps)()
+    ln = (C.c_int * nqps)()
+    stride = check(_lib.load().flh_qp_split(size, nqps, off, ln))
+    return stride, list(off), list(ln)
+
+
+class Pool:
+    """HIP-VMM pool of 2 MiB staging units (flh_pool_*)."""
+
+    def __init__(self, device: int = 0, units: int = 256):
+        self._h = C.c_void_p()
+        check(_lib.load().flh_pool_create(device, units, C.byref(self._h)))
+        self.units = units
+
+    @property
+    def handle(self) -> C.c_void_p:
+        return self._h
+
+    def free_units(self) -> int:
+        return check(_lib.load().flh_pool_free_units(self._h))
+
+    def granularity(self) -> int:
+        return int(_lib.load().flh_pool_granularity(self._h))
+
+    def slot_of(self, va: int) -> int:
+        return check(_lib.load().flh_pool_slot_of(self._h, C.c_void_p(va)))
+
+    def destroy(self) -> None:
+        if self._h:
+            check(_lib.load().flh_pool_destroy(self._h))
+            self._h = C.c_void_p()
+
+
+class Window:
+    """One lane's staging window: reserved VA whose leading units are bound to pool slots."""
+
+    def __init__(self, pool: Pool, va_bytes: int):
+        self._h = C.c_void_p()
+        self.pool = pool
+        check(_lib.load().flh_window_create(pool.handle, va_bytes, C.byref(self._h)))
+
+    def bind(self, nbytes: int) -> None:
+        check(_lib.load().flh_window_bind(self._h, nbytes))
+
+    def trim(self, nbytes: int) -> None:
+        check(_lib.load().flh_window_trim(self._h, nbytes))
+
+    @property
+    def base(self) -> int:
+        return int(_lib.load().flh_window_base(self._h) or 0)
+
+    @property
+    def bound_bytes(self) -> int:
+        return int(_lib.load().flh_window_bound_bytes(self._h))
+
+    def slots(self):
+        buf = (C.c_int * 4096)()
+        n = check(_lib.load().flh_window_slots(self._h, buf, 4096))
+        return list(buf[: min(n, 4096)])
+
+    def destroy(self) -> None:
+        if self._h:
+            check(_lib.load().flh_window_destroy(self._h))
+            self._h = C.c_void_p()
+
+
+class Region:
+    """regMr-time object: one window per lane for one user allocation, shared by base address."""
+
+    def __init__(self, pool: Pool, base: int, nbytes: int, n_lanes: int, bound_bytes_per_lane: int):
+        self._h = C.c_void_p()
+        check(_lib.load().flh_region_acquire(pool.handle, C.c_void_p(base), nbytes, n_lanes, bound_bytes_per_lane,
+                                             C.byref(self._h)))
+
+    @property
+    def handle_value(self) -> int:
+        return int(self._h.value or 0)
+
+    def refs(self) -> int:
+        return check(_lib.load().flh_region_refs(self._h))
+
+    def windows(self) -> Windows:
+        w = Windows()
+        check(_lib.load().flh_region_windows(self._h, C.byref(w)))
+        return w
+
+    def translate(self, lane: int, data: int) -> int:
+        return int(_lib.load().flh_region_translate(self._h, lane, C.c_void_p(data)) or 0)
+
+    def release(self) -> int:
+        left = check(_lib.load().flh_region_release(self._h))
+        self._h = C.c_void_p()
+        return left
+
+
+def read_window(base: int, nbytes: int, device="cuda") -> torch.Tensor:
+    """Copies `nbytes` at device address `base` into a fresh uint8 tensor (test helper)."""
+    out = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+    if nbytes:
+        check(_lib.load().flh_copy(C.c_void_p(out.data_ptr()), C.c_void_p(base), nbytes, _stream_ptr(None)))
+    return out[:nbytes]

@@ -1,0 +1,841 @@
+// fl_kernels.hip -- gfx950 kernels of the FuseLink data path and their C entry points:
+//   * fl_schedule_kernel : chunk -> (lane, window offset) table, wavefront prefix scans (DPP)
+//   * fl_copy_tiles      : striping (user buffer -> lane windows) and reassembly (windows -> user)
+//   * fl_page_tiles      : paged gather / scatter (non-contiguous pages <-> lane windows)
+//   * fl_plain_copy      : calibration copy with the same inner loop
+// The path is a pure HBM-bound byte mover plus one small integer scan; nothing here contracts, so
+// no MFMA.  Wavefronts are 64 wide; all cross-lane traffic in the scheduler is DPP row shifts and
+// row broadcasts, LDS is used only to pass per-wave totals between the waves of the one workgroup.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "fl_internal.h"
+#include "fuselink_hip.h"
+
+// ------------------------------------------------------------------------------------------------
+// wavefront scan primitives (DPP)
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int kWave = 64;
+
+// DPP controls of the GFX9 ISA: row_shr:n = 0x110+n, row_bcast:15 = 0x142, row_bcast:31 = 0x143.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+template <int CTRL>
+__device__ __forceinline__ uint64_t dpp_u64(uint64_t v) {
+  uint32_t lo = dpp_u32<CTRL>((uint32_t)v);
+  uint32_t hi = dpp_u32<CTRL>((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// One step of a Hillis-Steele scan: lanes for which `take` holds add the value moved in from below.
+#define FL_SCAN_STEP(T, MOVE, CTRL, COND) \
+  { T t = MOVE<CTRL>(v); if (COND) v += t; }
+
+// inclusive sum over the 64 lanes of a wavefront
+__device__ __forceinline__ uint64_t wave_incl_sum_u64(uint64_t v, int lane) {
+  const int r = lane & 15;
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x111, r >= 1)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x112, r >= 2)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x114, r >= 4)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x118, r >= 8)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x142, (lane & 31) >= 16)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x143, lane >= 32)
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_incl_sum_u32(uint32_t v, int lane) {
+  const int r = lane & 15;
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x111, r >= 1)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x112, r >= 2)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x114, r >= 4)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x118, r >= 8)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x142, (lane & 31) >= 16)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x143, lane >= 32)
+  return v;
+}
+#undef FL_SCAN_STEP
+
+// Segmented inclusive sum: f marks "a segment starts at or before me inside my own span"; the
+// combine is (f1,v1)+(f2,v2) = (f1|f2, f2 ? v2 : v1+v2) with operand 1 the lower lanes.
+#define FL_SEG_STEP(CTRL, COND)                                   \
+  {                                                               \
+    uint64_t tv = dpp_u64<CTRL>(v);                               \
+    uint32_t tf = dpp_u32<CTRL>(f);                               \
+    if (COND) { if (!f) v += tv; f |= tf; }                       \
+  }
+__device__ __forceinline__ void wave_incl_segsum_u64(uint64_t& v, uint32_t& f, int lane) {
+  const int r = lane & 15;
+  FL_SEG_STEP(0x111, r >= 1)
+  FL_SEG_STEP(0x112, r >= 2)
+  FL_SEG_STEP(0x114, r >= 4)
+  FL_SEG_STEP(0x118, r >= 8)
+  FL_SEG_STEP(0x142, (lane & 31) >= 16)
+  FL_SEG_STEP(0x143, lane >= 32)
+}
+#undef FL_SEG_STEP
+
+__device__ __forceinline__ uint64_t bcast_lane_u64(uint64_t v, int src_lane) {
+  uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, src_lane);
+  uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), src_lane);
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ uint32_t bcast_lane_u32(uint32_t v, int src_lane) {
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, src_lane);
+}
+
+// value of the lane below (lane 0 gets 0): turns an inclusive scan into an exclusive one
+__device__ __forceinline__ uint64_t wave_shift_up_u64(uint64_t v, int lane) {
+  // wave_shr:1 does not exist on every GFX9 part for 64 lanes; go through a bpermute
+  int src = (lane - 1) << 2;
+  uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)(uint32_t)v);
+  uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)(uint32_t)(v >> 32));
+  uint64_t r = ((uint64_t)hi << 32) | lo;
+  return lane == 0 ? 0 : r;
+}
+__device__ __forceinline__ uint32_t wave_shift_up_u32(uint32_t v, int lane) {
+  uint32_t r = (uint32_t)__builtin_amdgcn_ds_bpermute((lane - 1) << 2, (int)v);
+  return lane == 0 ? 0 : r;
+}
+
+// ------------------------------------------------------------------------------------------------
+// scheduler
+// ------------------------------------------------------------------------------------------------
+constexpr int kItems = 4;          // chunks per thread per pass
+constexpr int kRowCache = 32;      // credit rows kept in LDS
+
+struct SchedArgs {
+  const uint32_t* sizes;
+  uint64_t total_bytes;
+  const uint64_t* src_off;
+  uint64_t src_base;
+  const uint32_t* credits;
+  uint64_t quantum;
+  flh_sched_state* state;
+  flh_chunk_desc* table;
+  flh_sched_hdr* hdr;
+  uint32_t chunk_bytes;
+  uint32_t n;
+  uint32_t n_lanes;
+  uint32_t n_rows;
+  uint32_t epoch_len;
+  uint32_t tile_bytes;
+  uint32_t mode;
+  int32_t quantum_shift;  // >= 0 when quantum is a power of two
+};
+
+template <int NW>
+__global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
+  constexpr int BT = NW * kWave;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const uint32_t L = a.n_lanes;
+
+  // credit rows as inclusive prefixes; row r occupies rowpfx[r][0..L), W = rowpfx[r][L-1]
+  __shared__ uint64_t rowpfx[kRowCache][FLH_MAX_LANES];
+  __shared__ uint64_t w_seg_v[NW];
+  __shared__ uint32_t w_seg_f[NW];
+  __shared__ uint64_t w_run[NW];
+  __shared__ uint32_t w_tiles[NW];
+  __shared__ uint64_t w_lane[NW][FLH_MAX_LANES];
+  __shared__ uint32_t cnt_lane[FLH_MAX_LANES];
+
+  const bool rows_cached = a.n_rows <= (uint32_t)kRowCache;
+  if (rows_cached) {
+    for (uint32_t r = tid; r < a.n_rows; r += BT) {
+      uint64_t k = 0;
+      for (uint32_t l = 0; l < L; ++l) { k += a.credits[(size_t)r * L + l]; rowpfx[r][l] = k; }
+    }
+  }
+  if (tid < FLH_MAX_LANES) cnt_lane[tid] = 0;
+
+  // carried state (identical in every thread)
+  uint64_t k0 = 0, p_carry = 0, run_carry = 0;
+  uint32_t tiles_carry = 0, flags = 0;
+  uint64_t lane_off[FLH_MAX_LANES];
+  uint64_t lane_off0[FLH_MAX_LANES];
+#pragma unroll
+  for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off[l] = 0;
+  if (a.state) {
+    k0 = a.state->chunk_index;
+    p_carry = a.state->epoch_bytes;
+    if (!(a.mode & FLH_SCHED_RESET_OFFSETS)) {
+#pragma unroll
+      for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off[l] = a.state->lane_off[l];
+    }
+  }
+#pragma unroll
+  for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off0[l] = lane_off[l];
+  uint32_t my_cnt[FLH_MAX_LANES];
+#pragma unroll
+  for (int l = 0; l < FLH_MAX_LANES; ++l) my_cnt[l] = 0;
+
+  __syncthreads();
+
+  for (uint32_t pass = 0; pass < a.n; pass += BT * kItems) {
+    const uint32_t i0 = pass + (uint32_t)tid * kItems;
+    uint32_t s[kItems];
+    uint32_t head[kItems];
+    // ---- load sizes, mark epoch heads, thread-local aggregates -----------------------------------
+    uint64_t seg_v = 0;
+    uint32_t seg_f = 0;
+    uint64_t run = 0;
+    uint32_t tiles = 0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+      const uint32_t i = i0 + k;
+      uint32_t sz = 0, hd = 0;
+      if (i < a.n) {
+        if (a.sizes) {
+          sz = a.sizes[i];
+        } else {
+          uint64_t o = (uint64_t)i * a.chunk_bytes;
+          uint64_t rem = o < a.total_bytes ? a.total_bytes - o : 0;
+          sz = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
+        }
+        hd = a.epoch_len && ((k0 + i) % a.epoch_len == 0);
+      }
+      s[k] = sz;
+      head[k] = hd;
+      if (hd) { seg_v = 0; seg_f = 1; }
+      seg_v += sz;
+      run += sz;
+      tiles += (sz + a.tile_bytes - 1) / a.tile_bytes;
+    }
+    // ---- block-wide exclusive prefixes of (segmented bytes, bytes, tiles) --------------------------
+    uint64_t sv = seg_v;
+    uint32_t sf = seg_f;
+    wave_incl_segsum_u64(sv, sf, lane);
+    uint64_t run_incl = wave_incl_sum_u64(run, lane);
+    uint32_t tiles_incl = wave_incl_sum_u32(tiles, lane);
+    uint64_t seg_ex_v = wave_shift_up_u64(sv, lane);
+    uint32_t seg_ex_f = wave_shift_up_u32(sf, lane);
+    uint64_t run_ex = run_incl - run;
+    uint32_t tiles_ex = tiles_incl - tiles;
+    uint64_t tot_seg_v, tot_run;
+    uint32_t tot_seg_f, tot_tiles;
+    if (NW > 1) {
+      if (lane == kWave - 1) { w_seg_v[wave] = sv; w_seg_f[wave] = sf; w_run[wave] = run_incl; w_tiles[wave] = tiles_incl; }
+      __syncthreads();
+      uint64_t pv = 0, pr = 0;
+      uint32_t pf = 0, pt = 0;
+      tot_seg_v = 0; tot_seg_f = 0; tot_run = 0; tot_tiles = 0;
+      for (int w = 0; w < NW; ++w) {
+        if (w == wave) { pv = tot_seg_v; pf = tot_seg_f; pr = tot_run; pt = tot_tiles; }
+        uint64_t wv = w_seg_v[w];
+        uint32_t wf = w_seg_f[w];
+        tot_seg_v = wf ? wv : tot_seg_v + wv;
+        tot_seg_f |= wf;
+        tot_run += w_run[w];
+        tot_tiles += w_tiles[w];
+      }
+      // combine the earlier waves' aggregate with my in-wave exclusive value
+      if (!seg_ex_f) seg_ex_v += pv;
+      seg_ex_f |= pf;
+      run_ex += pr;
+      tiles_ex += pt;
+    } else {
+      tot_seg_v = bcast_lane_u64(sv, kWave - 1);
+      tot_seg_f = bcast_lane_u32(sf, kWave - 1);
+      tot_run = bcast_lane_u64(run_incl, kWave - 1);
+      tot_tiles = bcast_lane_u32(tiles_incl, kWave - 1);
+    }
+    // bytes of my epoch before my first item
+    uint64_t P = seg_ex_f ? seg_ex_v : p_carry + seg_ex_v;
+
+    // ---- lane of each item ----------------------------------------------------------------------------
+    uint32_t ln[kItems];
+    uint32_t ep[kItems];
+    uint64_t acc[FLH_MAX_LANES];
+#pragma unroll
+    for (int l = 0; l < FLH_MAX_LANES; ++l) acc[l] = 0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+      const uint32_t i = i0 + k;
+      ln[k] = 0;
+      ep[k] = 0;
+      if (i < a.n) {
+        if (head[k]) P = 0;
+        const uint64_t g = k0 + i;
+        const uint64_t e = a.epoch_len ? g / a.epoch_len : 0;
+        const uint32_t r = (uint32_t)(e % a.n_rows);
+        uint64_t W;
+        if (rows_cached) {
+          W = rowpfx[r][L - 1];
+        } else {
+          W = 0;
+          for (uint32_t l = 0; l < L; ++l) W += a.credits[(size_t)r * L + l];
+        }
+        uint32_t pick;
+        if (W == 0) {
+          pick = (uint32_t)(g % L);
+          flags |= FLH_SCHED_F_NO_CREDIT;
+        } else {
+          const uint64_t qn = a.quantum_shift >= 0 ? (P >> a.quantum_shift) : (P / a.quantum);
+          const uint64_t slot = (qn >> 32) == 0 && (W >> 32) == 0 ? (uint64_t)((uint32_t)qn % (uint32_t)W) : qn % W;
+          // lane = number of inclusive prefixes <= slot (zero-credit lanes repeat the prefix and are skipped)
+          pick = 0;
+          if (rows_cached) {
+            for (uint32_t l = 0; l + 1 < L; ++l) pick += rowpfx[r][l] <= slot;
+          } else {
+            uint64_t kk = 0;
+            for (uint32_t l = 0; l + 1 < L; ++l) { kk += a.credits[(size_t)r * L + l]; pick += kk <= slot; }
+          }
+        }
+        ln[k] = pick;
+        ep[k] = (uint32_t)e;
+        P += s[k];
+#pragma unroll
+        for (int l = 0; l < FLH_MAX_LANES; ++l) {
+          acc[l] += (pick == (uint32_t)l) ? (uint64_t)s[k] : 0;
+          my_cnt[l] += (pick == (uint32_t)l);
+        }
+      }
+    }
+    // ---- per-lane exclusive prefixes across the block ----------------------------------------------
+    uint64_t base[FLH_MAX_LANES];
+    uint64_t tot_lane[FLH_MAX_LANES];
+#pragma unroll
+    for (int l = 0; l < FLH_MAX_LANES; ++l) {
+      base[l] = 0;
+      tot_lane[l] = 0;
+      if ((uint32_t)l < L) {
+        uint64_t inc = wave_incl_sum_u64(acc[l], lane);
+        base[l] = inc - acc[l];
+        if (NW > 1) {
+          if (lane == kWave - 1) w_lane[wave][l] = inc;
+        } else {
+          tot_lane[l] = bcast_lane_u64(inc, kWave - 1);
+        }
+      }
+    }
+    if (NW > 1) {
+      __syncthreads();
+#pragma unroll
+      for (int l = 0; l < FLH_MAX_LANES; ++l) {
+        if ((uint32_t)l < L) {
+          uint64_t before = 0, tot = 0;
+          for (int w = 0; w < NW; ++w) {
+            uint64_t x = w_lane[w][l];
+            if (w < wave) before += x;
+            tot += x;
+          }
+          base[l] += before;
+          tot_lane[l] = tot;
+        }
+      }
+    }
+    // ---- emit rows ---------------------------------------------------------------------------------------
+    uint64_t run_i = run_carry + run_ex;
+    uint32_t tiles_i = tiles_carry + tiles_ex;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+      const uint32_t i = i0 + k;
+      if (i < a.n) {
+        uint64_t off = 0;
+#pragma unroll
+        for (int l = 0; l < FLH_MAX_LANES; ++l) {
+          if (ln[k] == (uint32_t)l) { off = lane_off[l] + base[l]; base[l] += s[k]; }
+        }
+        flh_chunk_desc d;
+        d.src_off = a.src_off ? a.src_off[i] : a.src_base + run_i;
+        d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : off;
+        d.len = s[k];
+        d.lane = ln[k];
+        d.tile_base = tiles_i;
+        d.epoch = ep[k];
+        a.table[i] = d;
+        run_i += s[k];
+        tiles_i += (s[k] + a.tile_bytes - 1) / a.tile_bytes;
+      }
+    }
+    // ---- carries ---------------------------------------------------------------------------------------------
+    p_carry = tot_seg_f ? tot_seg_v : p_carry + tot_seg_v;
+    run_carry += tot_run;
+    tiles_carry += tot_tiles;
+#pragma unroll
+    for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off[l] += tot_lane[l];
+    if (NW > 1) __syncthreads();  // LDS scratch is reused by the next pass
+  }
+
+  // ---- header and state --------------------------------------------------------------------------------------
+#pragma unroll
+  for (int l = 0; l < FLH_MAX_LANES; ++l) {
+    uint32_t c = wave_incl_sum_u32(my_cnt[l], lane);
+    if (lane == kWave - 1 && c) atomicAdd(&cnt_lane[l], c);
+  }
+  uint32_t any_flags = flags;
+  any_flags = __builtin_amdgcn_ballot_w64(any_flags != 0) ? 1u : 0u;
+  __shared__ uint32_t sh_flags;
+  if (tid == 0) sh_flags = 0;
+  __syncthreads();
+  if (lane == 0 && any_flags) atomicOr(&sh_flags, FLH_SCHED_F_NO_CREDIT);
+  __syncthreads();
+  if (tid == 0) {
+    flh_sched_hdr h;
+    h.total_bytes = run_carry;
+    h.total_tiles = tiles_carry;
+    h.n_chunks = a.n;
+    h.flags = sh_flags;
+    h.pad = 0;
+    for (int l = 0; l < FLH_MAX_LANES; ++l) {
+      h.lane_bytes[l] = lane_off[l] - lane_off0[l];
+      h.lane_chunks[l] = cnt_lane[l];
+    }
+    *a.hdr = h;
+    if (a.state) {
+      a.state->epoch_bytes = p_carry;
+      a.state->chunk_index = k0 + a.n;
+      for (int l = 0; l < FLH_MAX_LANES; ++l) a.state->lane_off[l] = lane_off[l];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// copy kernels
+// ------------------------------------------------------------------------------------------------
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kCopyBlock = 256;
+constexpr int kCopyUnroll = 8;
+
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const u32x4* p) {
+  return NT ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool NT>
+__device__ __forceinline__ void st16(u32x4* p, u32x4 v) {
+  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+}
+
+// Copies `bytes` from src to dst with the whole workgroup.  Fast path: both 16-byte aligned ->
+// dwordx4 loads batched kCopyUnroll deep before the stores.  Equal misalignment: byte head up to
+// the boundary, vectors, byte tail.  Different misalignment: byte copy (correct, not fast).
+template <bool NT>
+__device__ __forceinline__ void block_copy(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
+                                           uint32_t bytes) {
+  const uint32_t tid = threadIdx.x;
+  const uintptr_t sa = (uintptr_t)src, da = (uintptr_t)dst;
+  if (((sa ^ da) & 15) != 0) {
+    for (uint32_t i = tid; i < bytes; i += kCopyBlock) dst[i] = src[i];
+    return;
+  }
+  uint32_t head = (uint32_t)((16 - (sa & 15)) & 15);
+  if (head > bytes) head = bytes;
+  if (tid < head) dst[tid] = src[tid];
+  const uint32_t body = bytes - head;
+  const uint32_t nvec = body >> 4;
+  const u32x4* s = (const u32x4*)(src + head);
+  u32x4* d = (u32x4*)(dst + head);
+  for (uint32_t b = 0; b < nvec; b += kCopyBlock * kCopyUnroll) {
+    u32x4 r[kCopyUnroll];
+#pragma unroll
+    for (int j = 0; j < kCopyUnroll; ++j) {
+      const uint32_t idx = b + j * kCopyBlock + tid;
+      if (idx < nvec) r[j] = ld16<NT>(s + idx);
+    }
+#pragma unroll
+    for (int j = 0; j < kCopyUnroll; ++j) {
+      const uint32_t idx = b + j * kCopyBlock + tid;
+      if (idx < nvec) st16<NT>(d + idx, r[j]);
+    }
+  }
+  const uint32_t tail0 = head + (nvec << 4);
+  const uint32_t tail = bytes - tail0;
+  if (tid < tail) dst[tail0 + tid] = src[tail0 + tid];
+}
+
+struct CopyArgs {
+  uint8_t* user;
+  uint64_t user_bytes;
+  flh_windows win;
+  const flh_chunk_desc* table;
+  const flh_sched_hdr* hdr;
+  int32_t* status;
+  uint32_t n_chunks_max;
+  uint32_t tile_bytes;
+};
+
+// DIR 0: user -> windows (stripe).  DIR 1: windows -> user (reassemble).
+template <int DIR, bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
+  const uint32_t total = a.hdr->total_tiles;
+  uint32_t n = a.hdr->n_chunks;
+  if (n > a.n_chunks_max) n = a.n_chunks_max;
+  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
+    // last row whose tile_base <= t (empty chunks own no tile and are stepped over)
+    uint32_t lo = 0, hi = n;
+    while (hi - lo > 1) {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (a.table[mid].tile_base <= t) lo = mid; else hi = mid;
+    }
+    if (n == 0) break;
+    const flh_chunk_desc d = a.table[lo];
+    const uint64_t off = (uint64_t)(t - d.tile_base) * a.tile_bytes;
+    if (off >= d.len) continue;
+    const uint32_t bytes = (uint32_t)((d.len - off) < a.tile_bytes ? (d.len - off) : a.tile_bytes);
+    // refuse anything that would leave the user buffer or the mapped part of the window
+    bool ok = d.lane < a.win.n_lanes;
+    if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane] && d.src_off + d.len <= a.user_bytes;
+    if (!ok) {
+      if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+      continue;
+    }
+    uint8_t* u = a.user + d.src_off + off;
+    uint8_t* w = (uint8_t*)a.win.base[d.lane] + d.win_off + off;
+    if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+  }
+}
+
+struct PageArgs {
+  uint8_t* pool;
+  uint64_t pool_pages;
+  const uint32_t* page_table;
+  flh_windows win;
+  const flh_chunk_desc* table;
+  int32_t* status;
+  uint32_t n_chunks;
+  uint32_t page_bytes;
+  uint32_t pages_per_chunk;
+  uint32_t sub_bytes;      // bytes of a page handled by one workgroup step
+  uint32_t subs_per_page;
+};
+
+constexpr uint32_t kLdsStage = 16384;
+
+// DIR 0: pool pages -> windows (gather).  DIR 1: windows -> pool pages (scatter).
+// LDS: stage each sub-tile through LDS (coalesced global->LDS, barrier, LDS->global).
+template <int DIR, bool LDS, bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
+  __shared__ u32x4 stage[LDS ? kLdsStage / 16 : 1];
+  const uint64_t total = (uint64_t)a.n_chunks * a.pages_per_chunk * a.subs_per_page;
+  for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
+    const uint32_t sub = (uint32_t)(t % a.subs_per_page);
+    const uint64_t p = t / a.subs_per_page;          // index into the page table
+    const uint32_t c = (uint32_t)(p / a.pages_per_chunk);
+    const uint32_t k = (uint32_t)(p % a.pages_per_chunk);
+    const flh_chunk_desc d = a.table[c];
+    const uint64_t in_chunk = (uint64_t)k * a.page_bytes + (uint64_t)sub * a.sub_bytes;
+    if (in_chunk >= d.len) continue;
+    uint32_t bytes = a.page_bytes - sub * a.sub_bytes;
+    if (bytes > a.sub_bytes) bytes = a.sub_bytes;
+    if (bytes > d.len - in_chunk) bytes = (uint32_t)(d.len - in_chunk);
+    const uint32_t pg = a.page_table[p];
+    bool ok = d.lane < a.win.n_lanes && pg < a.pool_pages;
+    if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane];
+    if (!ok) {
+      if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+      continue;
+    }
+    uint8_t* u = a.pool + (uint64_t)pg * a.page_bytes + (uint64_t)sub * a.sub_bytes;
+    uint8_t* w = (uint8_t*)a.win.base[d.lane] + d.win_off + in_chunk;
+    uint8_t* dst = DIR == 0 ? w : u;
+    const uint8_t* src = DIR == 0 ? u : w;
+    if (LDS && ((((uintptr_t)src | (uintptr_t)dst) & 15) == 0) && (bytes & 15) == 0) {
+      const uint32_t nvec = bytes >> 4;  // <= kLdsStage/16 by construction of sub_bytes
+      const u32x4* s = (const u32x4*)src;
+      u32x4* dd = (u32x4*)dst;
+      for (uint32_t i = threadIdx.x; i < nvec; i += kCopyBlock) stage[i] = ld16<NT>(s + i);
+      __syncthreads();
+      for (uint32_t i = threadIdx.x; i < nvec; i += kCopyBlock) st16<NT>(dd + i, stage[i]);
+      __syncthreads();
+    } else {
+      block_copy<NT>(dst, src, bytes);
+    }
+  }
+}
+
+template <bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const uint8_t* src, uint64_t bytes,
+                                                            uint32_t tile_bytes) {
+  const uint64_t tiles = (bytes + tile_bytes - 1) / tile_bytes;
+  for (uint64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+    const uint64_t off = t * tile_bytes;
+    const uint32_t len = (uint32_t)((bytes - off) < tile_bytes ? (bytes - off) : tile_bytes);
+    block_copy<NT>(dst + off, src + off, len);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+int g_device = -1;
+int g_cus = 0;
+// launch tunables (overridable through NCCL_FUSELINK_* for experiments)
+int g_grid_per_cu = 8;
+int g_nontemporal = 1;
+
+int64_t env_i64(const char* name, int64_t dflt) {
+  const char* v = getenv(name);
+  if (!v || !*v) return dflt;
+  char* end = nullptr;
+  long long x = strtoll(v, &end, 0);
+  return end && *end == 0 ? x : dflt;
+}
+
+}  // namespace
+
+int fl_set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define FL_HIP(call)                                                                         \
+  do {                                                                                       \
+    hipError_t e_ = (call);                                                                  \
+    if (e_ != hipSuccess)                                                                    \
+      return fl_set_error(e_ == hipErrorNoDevice ? FLH_E_NODEV : FLH_E_HIP, "%s failed: %s (%s:%d)", #call, \
+                          hipGetErrorString(e_), __FILE__, __LINE__);                        \
+  } while (0)
+
+extern "C" {
+
+const char* flh_last_error(void) { return g_err; }
+
+int64_t flh_constant(int which) {
+  switch (which) {
+    case 0: return FLH_TILE_BYTES;
+    case 1: return FLH_MAX_LANES;
+    case 2: return FLH_UNIT_BYTES;
+    case 3: return FLH_POOL_UNITS;
+    case 4: return sizeof(flh_chunk_desc);
+    case 5: return sizeof(flh_sched_state);
+    case 6: return sizeof(flh_sched_hdr);
+    case 7: return 1;
+    case 8: return sizeof(flh_windows);
+    case 9: return sizeof(flh_sched_params);
+  }
+  return -1;
+}
+
+int flh_init(int device) {
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count == 0)
+    return fl_set_error(FLH_E_NODEV, "no HIP device: %s", e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+  if (device < 0 || device >= count) return fl_set_error(FLH_E_ARG, "device %d out of range (%d devices)", device, count);
+  FL_HIP(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  FL_HIP(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fl_set_error(FLH_E_NODEV, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+  g_device = device;
+  g_cus = prop.multiProcessorCount;
+  g_grid_per_cu = (int)env_i64("NCCL_FUSELINK_GRID_PER_CU", g_grid_per_cu);
+  g_nontemporal = (int)env_i64("NCCL_FUSELINK_NONTEMPORAL", g_nontemporal);
+  if (g_grid_per_cu < 1) g_grid_per_cu = 1;
+  return FLH_OK;
+}
+
+int flh_tune(const char* key, int64_t value) {
+  if (!key) return fl_set_error(FLH_E_ARG, "null key");
+  if (!strcmp(key, "grid_per_cu")) { if (value < 1) return fl_set_error(FLH_E_ARG, "grid_per_cu < 1"); g_grid_per_cu = (int)value; return FLH_OK; }
+  if (!strcmp(key, "nontemporal")) { g_nontemporal = value != 0; return FLH_OK; }
+  return fl_set_error(FLH_E_ARG, "unknown tunable %s", key);
+}
+
+static int need_init() {
+  if (g_device < 0) {
+    int rc = flh_init((int)env_i64("NCCL_FUSELINK_DEVICE", 0));
+    if (rc) return rc;
+  }
+  return FLH_OK;
+}
+
+int flh_schedule(const flh_sched_params* p, void* stream) {
+  if (!p) return fl_set_error(FLH_E_ARG, "null params");
+  if (p->n_lanes == 0 || p->n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "n_lanes %u not in 1..%d", p->n_lanes, FLH_MAX_LANES);
+  if (p->n_rows == 0 || !p->d_credits) return fl_set_error(FLH_E_ARG, "credit table missing");
+  if (p->quantum == 0) return fl_set_error(FLH_E_ARG, "quantum must be > 0");
+  if (p->tile_bytes == 0 || p->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", p->tile_bytes);
+  if (!p->d_hdr || (p->n_chunks && !p->d_table)) return fl_set_error(FLH_E_ARG, "output pointers missing");
+  if (!p->d_sizes) {
+    if (p->n_chunks && p->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0 for the uniform split");
+    const uint64_t need = p->chunk_bytes ? (p->total_bytes + p->chunk_bytes - 1) / p->chunk_bytes : 0;
+    if (need != p->n_chunks) return fl_set_error(FLH_E_ARG, "n_chunks %u does not match ceil(%llu / %u) = %llu", p->n_chunks,
+                                                (unsigned long long)p->total_bytes, p->chunk_bytes, (unsigned long long)need);
+  }
+  int rc = need_init();
+  if (rc) return rc;
+  SchedArgs a;
+  a.sizes = p->d_sizes;
+  a.total_bytes = p->total_bytes;
+  a.src_off = p->d_src_off;
+  a.src_base = p->src_base;
+  a.credits = p->d_credits;
+  a.quantum = p->quantum;
+  a.state = p->d_state;
+  a.table = p->d_table;
+  a.hdr = p->d_hdr;
+  a.chunk_bytes = p->chunk_bytes;
+  a.n = p->n_chunks;
+  a.n_lanes = p->n_lanes;
+  a.n_rows = p->n_rows;
+  a.epoch_len = p->epoch_len;
+  a.tile_bytes = p->tile_bytes;
+  a.mode = p->mode;
+  a.quantum_shift = (p->quantum & (p->quantum - 1)) == 0 ? __builtin_ctzll(p->quantum) : -1;
+  hipStream_t s = (hipStream_t)stream;
+  if (p->n_chunks <= kWave * kItems) {
+    hipLaunchKernelGGL(fl_schedule_kernel<1>, dim3(1), dim3(kWave), 0, s, a);
+  } else if (p->n_chunks <= 4 * kWave * kItems) {
+    hipLaunchKernelGGL(fl_schedule_kernel<4>, dim3(1), dim3(4 * kWave), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(fl_schedule_kernel<8>, dim3(1), dim3(8 * kWave), 0, s, a);
+  }
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+static int check_windows(const flh_windows* win) {
+  if (!win) return fl_set_error(FLH_E_ARG, "null windows");
+  if (win->n_lanes == 0 || win->n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "windows.n_lanes %u not in 1..%d", win->n_lanes, FLH_MAX_LANES);
+  for (uint32_t l = 0; l < win->n_lanes; ++l)
+    if (!win->base[l] && win->cap[l]) return fl_set_error(FLH_E_ARG, "window %u has capacity but no base", l);
+  return FLH_OK;
+}
+
+static uint32_t copy_grid(uint64_t max_tiles) {
+  uint64_t g = (uint64_t)g_cus * (uint64_t)g_grid_per_cu;
+  if (g > max_tiles) g = max_tiles;
+  if (g < 1) g = 1;
+  return (uint32_t)g;
+}
+
+static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
+                       const flh_sched_hdr* d_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
+  int rc = check_windows(win);
+  if (rc) return rc;
+  if (!d_hdr || !d_status) return fl_set_error(FLH_E_ARG, "d_hdr and d_status are required");
+  if (n_chunks_max && !d_table) return fl_set_error(FLH_E_ARG, "d_table missing");
+  if (tile_bytes == 0 || tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", tile_bytes);
+  if (user_bytes && !user) return fl_set_error(FLH_E_ARG, "user buffer missing");
+  if (n_chunks_max == 0) return FLH_OK;
+  rc = need_init();
+  if (rc) return rc;
+  CopyArgs a;
+  a.user = (uint8_t*)user;
+  a.user_bytes = user_bytes;
+  a.win = *win;
+  a.table = d_table;
+  a.hdr = d_hdr;
+  a.status = d_status;
+  a.n_chunks_max = n_chunks_max;
+  a.tile_bytes = tile_bytes;
+  const uint64_t max_tiles = user_bytes / tile_bytes + n_chunks_max;
+  const uint32_t grid = copy_grid(max_tiles);
+  hipStream_t s = (hipStream_t)stream;
+  if (dir == 0) {
+    if (g_nontemporal) hipLaunchKernelGGL((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    else hipLaunchKernelGGL((fl_copy_tiles<0, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+  } else {
+    if (g_nontemporal) hipLaunchKernelGGL((fl_copy_tiles<1, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    else hipLaunchKernelGGL((fl_copy_tiles<1, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+  }
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
+               const flh_sched_hdr* d_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
+  return launch_copy(0, (void*)d_src, src_bytes, win, d_table, d_hdr, n_chunks_max, tile_bytes, d_status, stream);
+}
+
+int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
+                   const flh_sched_hdr* d_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
+  return launch_copy(1, d_dst, dst_bytes, win, d_table, d_hdr, n_chunks_max, tile_bytes, d_status, stream);
+}
+
+static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                        uint32_t pages_per_chunk, const flh_windows* win, const flh_chunk_desc* d_table, uint32_t n_chunks,
+                        int use_lds, int32_t* d_status, void* stream) {
+  int rc = check_windows(win);
+  if (rc) return rc;
+  if (!pool || !d_page_table || !d_status) return fl_set_error(FLH_E_ARG, "pool, page table and status are required");
+  if (page_bytes == 0 || pages_per_chunk == 0) return fl_set_error(FLH_E_ARG, "page_bytes and pages_per_chunk must be > 0");
+  if (n_chunks == 0) return FLH_OK;
+  if (!d_table) return fl_set_error(FLH_E_ARG, "d_table missing");
+  rc = need_init();
+  if (rc) return rc;
+  PageArgs a;
+  a.pool = (uint8_t*)pool;
+  a.pool_pages = pool_pages;
+  a.page_table = d_page_table;
+  a.win = *win;
+  a.table = d_table;
+  a.status = d_status;
+  a.n_chunks = n_chunks;
+  a.page_bytes = page_bytes;
+  a.pages_per_chunk = pages_per_chunk;
+  const uint32_t sub = use_lds ? kLdsStage : FLH_TILE_BYTES;
+  a.sub_bytes = page_bytes < sub ? page_bytes : sub;
+  a.subs_per_page = (page_bytes + a.sub_bytes - 1) / a.sub_bytes;
+  const uint64_t total = (uint64_t)n_chunks * pages_per_chunk * a.subs_per_page;
+  const uint32_t grid = copy_grid(total);
+  hipStream_t s = (hipStream_t)stream;
+  const bool nt = g_nontemporal != 0;
+#define FL_LAUNCH_PAGES(D, LD, N) hipLaunchKernelGGL((fl_page_tiles<D, LD, N>), dim3(grid), dim3(kCopyBlock), 0, s, a)
+  if (dir == 0) {
+    if (use_lds) { if (nt) FL_LAUNCH_PAGES(0, true, true); else FL_LAUNCH_PAGES(0, true, false); }
+    else { if (nt) FL_LAUNCH_PAGES(0, false, true); else FL_LAUNCH_PAGES(0, false, false); }
+  } else {
+    if (use_lds) { if (nt) FL_LAUNCH_PAGES(1, true, true); else FL_LAUNCH_PAGES(1, true, false); }
+    else { if (nt) FL_LAUNCH_PAGES(1, false, true); else FL_LAUNCH_PAGES(1, false, false); }
+  }
+#undef FL_LAUNCH_PAGES
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_gather_pages(const void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                     uint32_t pages_per_chunk, const flh_windows* win, const flh_chunk_desc* d_table, uint32_t n_chunks,
+                     int use_lds, int32_t* d_status, void* stream) {
+  return launch_pages(0, (void*)d_pool, pool_pages, d_page_table, page_bytes, pages_per_chunk, win, d_table, n_chunks, use_lds, d_status, stream);
+}
+
+int flh_scatter_pages(void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                      uint32_t pages_per_chunk, const flh_windows* win, const flh_chunk_desc* d_table, uint32_t n_chunks,
+                      int use_lds, int32_t* d_status, void* stream) {
+  return launch_pages(1, d_pool, pool_pages, d_page_table, page_bytes, pages_per_chunk, win, d_table, n_chunks, use_lds, d_status, stream);
+}
+
+int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
+  if (bytes == 0) return FLH_OK;
+  if (!d_dst || !d_src) return fl_set_error(FLH_E_ARG, "null pointer");
+  int rc = need_init();
+  if (rc) return rc;
+  const uint32_t tile = FLH_TILE_BYTES;
+  const uint32_t grid = copy_grid((bytes + tile - 1) / tile);
+  hipStream_t s = (hipStream_t)stream;
+  if (g_nontemporal) hipLaunchKernelGGL(fl_plain_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  else hipLaunchKernelGGL(fl_plain_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_qp_split(int size, int nqps, int* off, int* len) {
+  if (nqps < 1 || size < 0 || !off || !len) return fl_set_error(FLH_E_ARG, "bad qp split arguments");
+  // stride = ceil(ceil(size / nqps) / 128) * 128; a piece past the end is an empty work request
+  const int per = (size + nqps - 1) / nqps;
+  const int stride = (per + 127) / 128 * 128;
+  for (int q = 0, o = 0; q < nqps; ++q, o += stride) {
+    int l = size - o;
+    if (l > stride) l = stride;
+    off[q] = o;
+    len[q] = l > 0 ? l : 0;
+  }
+  return stride;
+}
+
+}  // extern "C"

@@ -1,0 +1,203 @@
+/*
+ * fuselink_hip.h -- C ABI of the MI355X (gfx950) FuseLink data path.
+ *
+ * One shared library, libnccl-net-fuselink.so, carries two interfaces:
+ *   1. the NCCL/RCCL net-plugin tables declared in fuselink_net.h (what a communication library
+ *      dlopen()s), and
+ *   2. the entry points below: the chunk -> lane scheduler, the striping / reassembly copy kernels
+ *      and the HIP-VMM staging windows that the plugin is built from.  They are exported so a host
+ *      runtime (or a test harness) can drive the same path without the plugin's request machinery.
+ *
+ * Conventions: plain C types only.  Every function returns 0 on success or a negative FLH_E_* code;
+ * flh_last_error() returns a thread-local message for the last failure.  Pointers named d_* are
+ * device memory on the current HIP device; `stream` is a hipStream_t passed as void* (NULL = the
+ * null stream).  Nothing here blocks on the GPU unless its comment says so.
+ *
+ * Each entry point names the reference code it replaces (paths inside the FuseLink tree).
+ */
+#ifndef FUSELINK_HIP_H_
+#define FUSELINK_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLH_MAX_LANES     16                      /* MAX_NIC_NUM, src/monitor.h:18 */
+#define FLH_UNIT_BYTES    (2u * 1024u * 1024u)    /* BUFFER_UNIT, src/cumem.h:7 */
+#define FLH_POOL_UNITS    256                     /* MAX_MEM_TABLE_SIZE, src/cumem.cu:9 */
+#define FLH_TILE_BYTES    32768u                  /* default copy tile; must be a multiple of 128 */
+
+#define FLH_OK            0
+#define FLH_E_ARG        -1   /* bad argument (shape, alignment, null pointer) */
+#define FLH_E_HIP        -2   /* a HIP runtime call failed; message holds hipGetErrorString */
+#define FLH_E_NODEV      -3   /* no usable GPU */
+#define FLH_E_NOMEM      -4   /* unit pool exhausted (cumem.cu:176-179) */
+#define FLH_E_RANGE      -5   /* a chunk would land outside its staging window */
+#define FLH_E_STATE      -6   /* object used in the wrong state */
+
+/* One row of the chunk -> lane table (32 bytes, device and host layout identical). */
+typedef struct flh_chunk_desc {
+  uint64_t src_off;    /* byte offset of the chunk in the user buffer */
+  uint64_t win_off;    /* byte offset in its lane's staging window */
+  uint32_t len;        /* bytes */
+  uint32_t lane;       /* staging window / virtual NIC index */
+  uint32_t tile_base;  /* exclusive prefix of ceil(len / tile_bytes): first copy tile of the chunk */
+  uint32_t epoch;      /* credit epoch the chunk was scheduled in */
+} flh_chunk_desc;
+
+/* Scheduler state carried from one call to the next (device memory, 144 bytes). */
+typedef struct flh_sched_state {
+  uint64_t epoch_bytes;               /* bytes already scheduled in the current epoch */
+  uint64_t chunk_index;               /* global index of the next chunk */
+  uint64_t lane_off[FLH_MAX_LANES];   /* next free byte of each staging window */
+} flh_sched_state;
+
+/* Summary written by the scheduler next to the table (device memory, 216 bytes). */
+typedef struct flh_sched_hdr {
+  uint64_t total_bytes;
+  uint32_t total_tiles;
+  uint32_t n_chunks;
+  uint32_t flags;                      /* FLH_SCHED_F_* */
+  uint32_t pad;
+  uint64_t lane_bytes[FLH_MAX_LANES];  /* bytes this call put on each lane */
+  uint32_t lane_chunks[FLH_MAX_LANES]; /* chunks this call put on each lane */
+} flh_sched_hdr;
+
+#define FLH_SCHED_F_NO_CREDIT 1u       /* some epoch had all-zero credits: static lane policy used */
+
+/* flh_sched_params.mode */
+#define FLH_SCHED_RESET_OFFSETS 1u     /* start every lane at window offset 0 instead of the state's */
+#define FLH_SCHED_MIRROR        2u     /* win_off = src_off: each window mirrors the user buffer, the
+                                          reference's translation window + (data - start_addr)
+                                          (src/plugin.cc:1582, 1626); windows must be bound that far */
+
+typedef struct flh_sched_params {
+  const uint32_t* d_sizes;     /* n chunk sizes, or NULL for the uniform split of total_bytes */
+  uint64_t total_bytes;        /* used when d_sizes == NULL */
+  uint32_t chunk_bytes;        /* used when d_sizes == NULL */
+  const uint64_t* d_src_off;   /* n explicit source offsets, or NULL for src_base + running sum */
+  uint64_t src_base;
+  uint32_t n_chunks;
+  uint32_t n_lanes;            /* 1..16 */
+  const uint32_t* d_credits;   /* n_rows x n_lanes credit table */
+  uint32_t n_rows;             /* >= 1; epoch e reads row e mod n_rows */
+  uint32_t epoch_len;          /* chunks per credit epoch; 0 = a single epoch */
+  uint64_t quantum;            /* bytes per credit (the nominal chunk size) */
+  uint32_t tile_bytes;         /* copy tile the table is partitioned for (multiple of 128) */
+  uint32_t mode;               /* FLH_SCHED_* bits */
+  flh_sched_state* d_state;    /* in/out, or NULL to start from zero and discard */
+  flh_chunk_desc* d_table;     /* out: n_chunks rows */
+  flh_sched_hdr* d_hdr;        /* out */
+} flh_sched_params;
+
+/* ---- library ------------------------------------------------------------------------------ */
+/* Selects `device`, checks that it is a gfx950 part, loads kernel attributes.  Idempotent. */
+int flh_init(int device);
+const char* flh_last_error(void);
+/* compile-time facts: 0 tile bytes, 1 max lanes, 2 unit bytes, 3 pool units, 4 sizeof(desc),
+ * 5 sizeof(state), 6 sizeof(hdr), 7 ABI version, 8 sizeof(flh_windows), 9 sizeof(flh_sched_params) */
+int64_t flh_constant(int which);
+/* Launch tunables, for experiments (no counterpart in the reference): "grid_per_cu" = copy
+ * workgroups launched per compute unit, "nontemporal" = 0/1 streaming loads and stores.
+ * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL. */
+int flh_tune(const char* key, int64_t value);
+
+/* ---- scheduler ------------------------------------------------------------------------------
+ * Replaces FuseLinkConnManager::refreshRxComm / bidTxChannel (src/fuselink.h:153-156, 230-238) and
+ * the idle-NIC query behind them (src/monitor.h:191-224) with one kernel launch over a whole send
+ * set: an epoch-segmented wavefront prefix scan of the chunk sizes gives each chunk its quantum
+ * slot, the credit row of its epoch maps the slot to a lane, and a per-lane scan gives its offset
+ * in that lane's staging window.  Equal credits and quantum-sized chunks reproduce the reference's
+ * live policy lane = index mod lanes (src/fuselink.h:235). */
+int flh_schedule(const flh_sched_params* p, void* stream);
+
+/* ---- striping / reassembly --------------------------------------------------------------------
+ * flh_stripe replaces the send side of ncclIbMultiSend (src/plugin.cc:1467-1495: per-request split,
+ * RDMA write out of the staged copy at flmr->addr[dev] + (data - start_addr), src/plugin.cc:1582):
+ * every chunk of the table is copied from d_src + src_off into window[lane] + win_off.
+ * flh_reassemble replaces the landing of those writes in the receiver's translated buffer
+ * (src/plugin.cc:1626): window[lane] + win_off is copied to d_dst + src_off.
+ * d_hdr->total_tiles sizes the work; win_cap[l] is the mapped size of window l and a chunk that
+ * would cross it is skipped and reported through *d_status (FLH_E_RANGE), never written.
+ * n_chunks_max bounds the table rows the kernel may read. */
+typedef struct flh_windows {
+  void*    base[FLH_MAX_LANES];
+  uint64_t cap[FLH_MAX_LANES];
+  uint32_t n_lanes;
+  uint32_t pad;
+} flh_windows;
+
+int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win,
+               const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, uint32_t n_chunks_max,
+               uint32_t tile_bytes, int32_t* d_status, void* stream);
+int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
+                   const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, uint32_t n_chunks_max,
+                   uint32_t tile_bytes, int32_t* d_status, void* stream);
+
+/* Paged variants for non-contiguous sources (KV-cache blocks, src/experiments/serving/model.hh:
+ * 198-201 gives the page shape): chunk c of the table stands for pages
+ * d_page_table[c*pages_per_chunk ...] of a pool of page_bytes-sized pages; gather packs them into
+ * the chunk's window slot, scatter puts them back at the same page numbers of d_pool.
+ * use_lds != 0 stages each tile through LDS. */
+int flh_gather_pages(const void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table,
+                     uint32_t page_bytes, uint32_t pages_per_chunk, const flh_windows* win,
+                     const flh_chunk_desc* d_table, uint32_t n_chunks, int use_lds,
+                     int32_t* d_status, void* stream);
+int flh_scatter_pages(void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table,
+                      uint32_t page_bytes, uint32_t pages_per_chunk, const flh_windows* win,
+                      const flh_chunk_desc* d_table, uint32_t n_chunks, int use_lds,
+                      int32_t* d_status, void* stream);
+
+/* Plain device copy with the same inner loop as the striping kernels (roofline calibration). */
+int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream);
+
+/* ---- R2: request -> QP pieces (src/plugin.cc:1467-1495), host arithmetic ------------------------ */
+int flh_qp_split(int size, int nqps, int* off, int* len);
+
+/* ---- staging windows on HIP VMM ------------------------------------------------------------------
+ * Replaces the 2 MiB slot pool of src/cumem.cu (init_cumem 29-57, register_cumem 107-184,
+ * remap_cumem 72-105, free_cumem 60-70) and the per-device windows of FuseLinkMemRegionInit
+ * (src/fuselink.cc:4-59).  A pool owns `units` physical 2 MiB allocations (hipMemCreate); a window
+ * is a virtual range (hipMemAddressReserve) whose leading units are bound to pool slots first-fit
+ * (hipMemMap + hipMemSetAccess).  Unlike the reference, errors come back as codes, not exit(1)
+ * (src/checks.h:17-23). */
+typedef struct flh_pool flh_pool;
+typedef struct flh_window flh_window;
+
+int flh_pool_create(int device, uint32_t units, flh_pool** out);
+int flh_pool_destroy(flh_pool* pool);             /* all windows must be destroyed first */
+int flh_pool_free_units(const flh_pool* pool);    /* number of unbound slots */
+int flh_pool_slot_of(const flh_pool* pool, const void* va); /* ptr2dev analogue (cumem.cu:186-193) */
+uint64_t flh_pool_granularity(const flh_pool* pool);
+
+int flh_window_create(flh_pool* pool, uint64_t va_bytes, flh_window** out);
+/* grow the bound prefix to cover at least `bytes` (rounded up to units); FLH_E_NOMEM if the pool
+ * cannot supply them (slots bound before the failure stay bound, as in cumem.cu:176-179) */
+int flh_window_bind(flh_window* w, uint64_t bytes);
+/* unbind the trailing units so that at most `bytes` stay bound (0 = all); slots return to the pool */
+int flh_window_trim(flh_window* w, uint64_t bytes);
+int flh_window_destroy(flh_window* w);
+void* flh_window_base(const flh_window* w);
+uint64_t flh_window_bound_bytes(const flh_window* w);
+/* slot ids backing the first `max` units, in order; returns the number of bound units */
+int flh_window_slots(const flh_window* w, int* slots, int max);
+
+/* ---- regions: the regMr-time object (src/plugin.cc:1168-1330, 1337-1408; src/fuselink.h:39-52) ---
+ * One region per base allocation, shared and reference-counted by base address; it owns one
+ * staging window per lane.  flh_region_translate is the reference's pointer translation
+ * window_base + (data - start_addr) (src/plugin.cc:1582, 1626). */
+typedef struct flh_region flh_region;
+int flh_region_acquire(flh_pool* pool, void* base, uint64_t bytes, uint32_t n_lanes,
+                       uint64_t bound_bytes_per_lane, flh_region** out);
+int flh_region_release(flh_region* r);            /* returns remaining refs (>= 0) or an error */
+int flh_region_refs(const flh_region* r);
+int flh_region_windows(const flh_region* r, flh_windows* out);
+void* flh_region_translate(const flh_region* r, uint32_t lane, const void* data);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FUSELINK_HIP_H_ */

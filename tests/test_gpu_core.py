@@ -1,0 +1,188 @@
+"""GPU parity of the scheduler and the striping / reassembly kernels against the CPU oracle.
+All calls go through the C ABI of libnccl-net-fuselink.so (fuselink_amd.core is a ctypes shim)."""
+import numpy as np
+import pytest
+
+from tests import oracle_binding as ob
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fl():
+    import torch
+    from fuselink_amd import core
+    core.init(0)
+    return core, torch
+
+
+def _dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _check_schedule(fl, *, n_lanes, credits, quantum, sizes=None, total_bytes=0, chunk_bytes=0, epoch_len=0,
+                    tile_bytes=32768, mode=0, state=None, src_off=None, src_base=0):
+    core, torch = fl
+    credits = np.asarray(credits, dtype=np.uint32).reshape(-1, n_lanes)
+    exp_t, exp_h, exp_s = ob.credit_schedule(n_lanes=n_lanes, credits=credits, quantum=quantum, sizes=sizes,
+                                             total_bytes=total_bytes, chunk_bytes=chunk_bytes, epoch_len=epoch_len,
+                                             tile_bytes=tile_bytes, mode=mode, state=state, src_off=src_off,
+                                             src_base=src_base)
+    d_state = None
+    if state is not None:
+        d_state = _dev(torch, np.array([state], dtype=ob.STATE_DTYPE).view(np.uint8))
+    sched = core.schedule(n_lanes=n_lanes, credits=_dev(torch, credits.view(np.int32)), quantum=quantum,
+                          sizes=None if sizes is None else _dev(torch, np.asarray(sizes, dtype=np.uint32).view(np.int32)),
+                          total_bytes=total_bytes, chunk_bytes=chunk_bytes, epoch_len=epoch_len, tile_bytes=tile_bytes,
+                          mode=mode, state=d_state, src_base=src_base,
+                          src_off=None if src_off is None else _dev(torch, np.asarray(src_off, dtype=np.uint64).view(np.int64)))
+    torch.cuda.synchronize()
+    got_t, got_h = sched.table_numpy(), sched.hdr_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+    for f in ("total_bytes", "total_tiles", "n_chunks", "flags", "lane_bytes", "lane_chunks"):
+        np.testing.assert_array_equal(got_h[f], exp_h[f], err_msg=f"hdr field {f}")
+    if state is not None:
+        got_s = core.state_numpy(d_state)
+        for f in ob.STATE_DTYPE.names:
+            np.testing.assert_array_equal(got_s[f], exp_s[f], err_msg=f"state field {f}")
+    return sched, exp_t, exp_h
+
+
+@pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 2049, 5000, 16384])
+def test_schedule_uniform_sizes(fl, n):
+    chunk = 65536
+    total = n * chunk - (chunk // 3 if n else 0)
+    rng = np.random.default_rng(n)
+    _check_schedule(fl, n_lanes=8, credits=rng.integers(1, 9, size=8), quantum=chunk, total_bytes=total, chunk_bytes=chunk)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_schedule_random_sizes_epochs(fl, seed):
+    rng = np.random.default_rng(100 + seed)
+    n = int(rng.integers(1, 6000))
+    lanes = int(rng.integers(1, 17))
+    rows = int(rng.integers(1, 40))
+    sizes = rng.integers(0, 300000, size=n).astype(np.uint32)
+    credits = rng.integers(0, 9, size=(rows, lanes)).astype(np.uint32)
+    credits[rng.integers(0, rows)] = 0  # an all-busy epoch exercises the static fallback
+    epoch_len = int(rng.choice([0, 1, 7, 8, 100, 1000]))
+    quantum = int(rng.choice([4096, 65536, 100000, 262144]))
+    _check_schedule(fl, n_lanes=lanes, credits=credits, quantum=quantum, sizes=sizes, epoch_len=epoch_len,
+                    tile_bytes=int(rng.choice([4096, 32768])))
+
+
+def test_schedule_state_carry_and_modes(fl):
+    rng = np.random.default_rng(7)
+    st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+    st["epoch_bytes"] = 123456
+    st["chunk_index"] = 37
+    st["lane_off"][:] = rng.integers(0, 1 << 40, size=16)
+    sizes = rng.integers(1, 100000, size=900).astype(np.uint32)
+    credits = rng.integers(1, 5, size=(3, 5)).astype(np.uint32)
+    for mode in (0, ob.SCHED_RESET_OFFSETS, ob.SCHED_MIRROR):
+        _check_schedule(fl, n_lanes=5, credits=credits, quantum=65536, sizes=sizes, epoch_len=50, state=st, mode=mode,
+                        src_base=4096)
+    src_off = np.cumsum(rng.integers(100000, 200000, size=900)).astype(np.uint64)
+    _check_schedule(fl, n_lanes=5, credits=credits, quantum=65536, sizes=sizes, epoch_len=50, src_off=src_off)
+
+
+def test_schedule_equal_credits_is_static_policy(fl):
+    # the reference's live policy: lane = index mod lanes (src/fuselink.h:235)
+    core, torch = fl
+    sched, _, _ = _check_schedule(fl, n_lanes=8, credits=np.ones(8), quantum=262144, total_bytes=64 << 20,
+                                  chunk_bytes=262144)
+    t = sched.table_numpy()
+    np.testing.assert_array_equal(t["lane"], np.arange(256) % 8)
+
+
+def _roundtrip(fl, src_np, *, n_lanes, credits, quantum, sizes=None, chunk_bytes=0, epoch_len=0, tile_bytes=32768,
+               src_off=None, dst_extra=0):
+    core, torch = fl
+    nbytes = src_np.size
+    sched, exp_t, exp_h = _check_schedule(fl, n_lanes=n_lanes, credits=credits, quantum=quantum, sizes=sizes,
+                                          total_bytes=0 if sizes is not None else nbytes, chunk_bytes=chunk_bytes,
+                                          epoch_len=epoch_len, tile_bytes=tile_bytes, src_off=src_off)
+    caps = [int(b) for b in exp_h["lane_bytes"][:n_lanes]]
+    src = _dev(torch, src_np)
+    wins = [torch.zeros(max(c, 1) + 64, dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    core.stripe(src, w, sched, status)
+    dst = torch.zeros(nbytes + dst_extra, dtype=torch.uint8, device="cuda")
+    core.reassemble(dst, w, sched, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    # staged windows equal the host-memcpy windows byte for byte, guard bytes untouched
+    exp_w = ob.cpu_stripe(src_np, exp_t, caps)
+    for l in range(n_lanes):
+        got = wins[l].cpu().numpy()
+        np.testing.assert_array_equal(got[: caps[l]], exp_w[l][: caps[l]], err_msg=f"window {l}")
+        assert not got[caps[l]:].any(), f"window {l} written past its {caps[l]} bytes"
+    exp_dst = ob.cpu_reassemble(nbytes, exp_w, exp_t)
+    got_dst = dst.cpu().numpy()
+    np.testing.assert_array_equal(got_dst[:nbytes], exp_dst)
+    return got_dst
+
+
+def test_roundtrip_cfg1_shape(fl):
+    # 4 MiB uint8, 512 KiB chunks, 2 lanes, equal credits (the reference's operating point)
+    rng = np.random.default_rng(1)
+    src = rng.integers(0, 256, size=4 << 20, dtype=np.uint8)
+    out = _roundtrip(fl, src, n_lanes=2, credits=[1, 1], quantum=512 << 10, chunk_bytes=512 << 10)
+    np.testing.assert_array_equal(out, src)
+
+
+def test_roundtrip_cfg2_shape(fl):
+    # 64 MiB fp16 N(0,1), 256 KiB chunks, 8 lanes, credits uniform in [1,8]
+    rng = np.random.default_rng(2)
+    src = rng.standard_normal(32 << 20, dtype=np.float32).astype(np.float16).view(np.uint8)
+    credits = rng.integers(1, 9, size=8)
+    out = _roundtrip(fl, src, n_lanes=8, credits=credits, quantum=256 << 10, chunk_bytes=256 << 10)
+    np.testing.assert_array_equal(out, src)
+
+
+@pytest.mark.parametrize("nbytes,chunk", [(1, 4096), (15, 4096), (4097, 4096), ((4 << 20) + 1, 512 << 10),
+                                          (1000003, 65536), (3 * 32768, 32768)])
+def test_roundtrip_ragged(fl, nbytes, chunk):
+    rng = np.random.default_rng(nbytes)
+    src = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+    out = _roundtrip(fl, src, n_lanes=3, credits=[2, 1, 3], quantum=chunk, chunk_bytes=chunk)
+    np.testing.assert_array_equal(out, src)
+
+
+def test_roundtrip_odd_sizes_misaligned_windows(fl):
+    # chunk sizes that are not multiples of 16 leave window offsets misaligned against the source
+    rng = np.random.default_rng(11)
+    sizes = rng.integers(1, 70000, size=300).astype(np.uint32)
+    src = rng.integers(0, 256, size=int(sizes.sum()), dtype=np.uint8)
+    out = _roundtrip(fl, src, n_lanes=4, credits=[1, 2, 3, 4], quantum=32768, sizes=sizes, tile_bytes=4096)
+    np.testing.assert_array_equal(out, src)
+
+
+def test_empty_message(fl):
+    core, torch = fl
+    sched, _, exp_h = _check_schedule(fl, n_lanes=4, credits=[1, 1, 1, 1], quantum=4096, total_bytes=0, chunk_bytes=4096)
+    assert exp_h["total_tiles"] == 0
+    w = core.make_windows([0, 0, 0, 0], [0, 0, 0, 0])
+    status = core.new_status()
+    dummy = torch.zeros(1, dtype=torch.uint8, device="cuda")
+    core.stripe(dummy[:0], w, sched, status)
+    core.reassemble(dummy[:0], w, sched, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+
+
+def test_window_overflow_is_refused_not_written(fl):
+    core, torch = fl
+    rng = np.random.default_rng(5)
+    src_np = rng.integers(0, 256, size=1 << 20, dtype=np.uint8)
+    sched, exp_t, exp_h = _check_schedule(fl, n_lanes=2, credits=[1, 1], quantum=65536, total_bytes=1 << 20, chunk_bytes=65536)
+    caps = [int(exp_h["lane_bytes"][0]), int(exp_h["lane_bytes"][1]) - 65536]  # lane 1 is one chunk short
+    wins = [torch.zeros(int(exp_h["lane_bytes"][l]), dtype=torch.uint8, device="cuda") for l in range(2)]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    core.stripe(_dev(torch, src_np), w, sched, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == -5
+    assert not wins[1][caps[1]:].cpu().numpy().any()
