@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the FuseLink data path on one MI355X.
+
+One step = the whole hot path over one message: scheduler kernel (chunk -> lane table), striping
+kernel (user buffer -> per-lane HIP-VMM staging windows) and reassembly kernel (windows -> receive
+buffer).  The workload is the headline configuration: a 64 MiB fp16 gradient-bucket buffer
+(N(0,1), seeded), 256 KiB chunks, 8 lanes, lane credits uniform in [1,8] (seeded).  Inputs are
+resident in HBM before the timed region.  Prints one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: (bytes, chunk bytes, lanes, credit rows, epoch length)
+    "cfg2_grad_bucket_64MiB_256KiB_8lanes": (64 << 20, 256 << 10, 8, 1, 0),
+    "cfg5_stress_1GiB_64KiB_16lanes": (1 << 30, 64 << 10, 16, 17, 1000),
+}
+
+# HBM bytes per launch of the striping kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until such a run has been recorded for the workload.
+MEASURED_TRAFFIC = {}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2_grad_bucket_64MiB_256KiB_8lanes", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-iters", type=int, default=60)
+    ap.add_argument("--graph", type=int, default=0, help="replay the step as a HIP graph (1) or launch eagerly (0)")
+    ap.add_argument("--hint", type=int, default=1, help="pass the host-known header fields to the copy kernels")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (every lane's staging window lives on it); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from fuselink_amd import core
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; there is no CPU fallback for the measured path", file=sys.stderr)
+        return 3
+    core.init(0)
+    dev = torch.device("cuda:0")
+    nbytes, chunk, lanes, rows, epoch_len = WORKLOADS[args.workload]
+    n_chunks = (nbytes + chunk - 1) // chunk
+
+    # ---- synthetic inputs, resident in HBM ------------------------------------------------------
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(20251125)
+    if args.workload.startswith("cfg2"):
+        src = torch.randn(nbytes // 2, dtype=torch.float16, device=dev, generator=gen).view(torch.uint8)
+    else:
+        src = torch.randint(0, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device=dev, generator=gen).view(torch.uint8)
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    rng = np.random.default_rng(20251125)
+    credits_np = rng.integers(1, 9, size=(rows, lanes)).astype(np.int32)
+    credits = torch.from_numpy(credits_np).to(dev)
+
+    # ---- registration-time work (untimed): table once for sizing, windows bound from the VMM pool --
+    stream = torch.cuda.Stream(device=dev)
+    status = core.new_status(dev)
+    with torch.cuda.stream(stream):
+        sched = core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
+                              epoch_len=epoch_len, stream=stream)
+    stream.synchronize()
+    hdr = sched.hdr_numpy()
+    lane_bytes = [int(b) for b in hdr["lane_bytes"][:lanes]]
+    units = sum((b + core.UNIT_BYTES - 1) // core.UNIT_BYTES for b in lane_bytes)
+    pool = core.Pool(0, max(256, units))
+    windows = []
+    for b in lane_bytes:
+        w = core.Window(pool, max(b, 1))
+        w.bind(b)
+        windows.append(w)
+    win = core.make_windows([w.base for w in windows], [w.bound_bytes for w in windows])
+
+    # header fields that follow from the uniform split alone; the kernels then need not wait for d_hdr
+    hint = core.uniform_hint(nbytes, chunk) if args.hint else None
+
+    def step():
+        core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
+                      epoch_len=epoch_len, out=sched, stream=stream)
+        core.stripe(src, win, sched, status, stream=stream, hint=hint)
+        core.reassemble(dst, win, sched, status, stream=stream, hint=hint)
+
+    graph = None
+    if args.graph:
+        # capture the three launches once; a replay is one host call per step
+        step()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            step()
+
+    def run_step():
+        if graph is not None:
+            with torch.cuda.stream(stream):
+                graph.replay()
+        else:
+            step()
+
+    for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    # correctness of what was just timed: bit-exact round trip, no range refusals
+    assert int(status.item()) == 0, "a kernel refused a chunk (window or buffer range)"
+    assert torch.equal(src, dst), "reassembled buffer differs from the source"
+
+    # ---- per-kernel durations: every launch carries its own start/stop HIP events on the launch stream ----
+    def kernel_us(fn, iters):
+        core.prof_enable(True)
+        ts = []
+        for _ in range(iters):
+            fn()
+            ts.append(core.prof_last_us())
+        core.prof_enable(False)
+        return sum(ts) / len(ts), min(ts)
+
+    k_iters = max(20, min(args.steps, 200))
+    sched_us, sched_min = kernel_us(lambda: core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes,
+                                                          chunk_bytes=chunk, epoch_len=epoch_len, out=sched, stream=stream), k_iters)
+    stripe_us, stripe_min = kernel_us(lambda: core.stripe(src, win, sched, status, stream=stream, hint=hint), k_iters)
+    reasm_us, reasm_min = kernel_us(lambda: core.reassemble(dst, win, sched, status, stream=stream, hint=hint), k_iters)
+    copy_us, _ = kernel_us(lambda: core.copy(dst, src, stream=stream), k_iters)
+
+    algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
+    algo_bytes_kernel = 2 * nbytes        # one launch of the copy kernel
+    value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
+    pair_us = stripe_us + reasm_us
+    achieved = algo_bytes_kernel / (stripe_us * 1e-6) / 1e9
+
+    out = {
+        "metric": "stripe+reassemble GB/s, 64 MiB over 8 lanes" if args.workload.startswith("cfg2") else "stripe+reassemble GB/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "bytes": nbytes, "chunk_bytes": chunk, "chunks": n_chunks, "lanes": lanes,
+                   "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
+                   "step": "schedule+stripe+reassemble", "launch": "hipGraph replay" if graph is not None else "eager",
+                   "windows": "HIP VMM, 2 MiB units"},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
+        "kernels_us": {"schedule": round(sched_us, 2), "stripe": round(stripe_us, 2), "reassemble": round(reasm_us, 2),
+                       "stripe_min": round(stripe_min, 2), "reassemble_min": round(reasm_min, 2),
+                       "plain_copy_same_bytes": round(copy_us, 2)},
+        "stripe_reassemble_pair_GBps": round(algo_bytes_step / (pair_us * 1e-6) / 1e9, 1),
+        "scheduler_us_per_1k_chunks": round(sched_us / (n_chunks / 1000.0), 3),
+        "roofline": {"bound": "hbm", "kernel": "fl_copy_tiles<0> (stripe)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get(args.workload)},
+    }
+
+    # ---- CPU baseline: the oracle's host-memcpy striping on a bounded sample ------------------------
+    if not args.no_cpu_baseline:
+        from tests import oracle_binding as ob
+        src_np = src.cpu().numpy()
+        tab, h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits_np, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
+                                       epoch_len=epoch_len)
+        iters = args.cpu_iters if nbytes <= (64 << 20) else max(3, args.cpu_iters // 16)
+        med1, best1 = ob.cpu_baseline(src_np, tab, h, lanes, threads=1, warm=3, iters=iters)
+        cores = ob.lib().fl_cpu_cores()
+        thr = min(lanes, cores, 16)
+        medm, bestm = ob.cpu_baseline(src_np, tab, h, lanes, threads=thr, warm=3, iters=iters)
+        out["cpu_baseline"] = {"value": round(algo_bytes_step / med1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{iters} timed stripe+reassemble passes of the same {nbytes >> 20} MiB message "
+                                         f"(host memcpy per chunk into 2 MiB-aligned lane windows), median; host has {cores} cores"}
+        out["cpu_baseline_per_lane_threads"] = {"value": round(algo_bytes_step / medm / 1e9, 2), "unit": "GB/s", "cores": thr,
+                                                "kind": "port", "sample": "same passes, one pinned thread per lane"}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -21,7 +21,7 @@ class SchedState(C.Structure):
 
 class SchedHdr(C.Structure):
     _fields_ = [("total_bytes", C.c_uint64), ("total_tiles", C.c_uint32), ("n_chunks", C.c_uint32),
-                ("flags", C.c_uint32), ("pad", C.c_uint32), ("lane_bytes", C.c_uint64 * MAX_LANES),
+                ("flags", C.c_uint32), ("uniform_tiles", C.c_uint32), ("lane_bytes", C.c_uint64 * MAX_LANES),
                 ("lane_chunks", C.c_uint32 * MAX_LANES)]
 
 
@@ -44,10 +44,10 @@ SIGNATURES = {
     "flh_last_error": (C.c_char_p, []),
     "flh_constant": (C.c_int64, [C.c_int]),
     "flh_schedule": (C.c_int, [C.POINTER(SchedParams), C.c_void_p]),
-    "flh_stripe": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_uint32,
-                             C.c_uint32, C.c_void_p, C.c_void_p]),
-    "flh_reassemble": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_uint32,
-                                 C.c_uint32, C.c_void_p, C.c_void_p]),
+    "flh_stripe": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p, C.POINTER(SchedHdr),
+                             C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
+    "flh_reassemble": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p,
+                                 C.POINTER(SchedHdr), C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
     "flh_gather_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),
                                    C.c_void_p, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p]),
     "flh_scatter_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),
@@ -73,6 +73,8 @@ SIGNATURES = {
     "flh_region_windows": (C.c_int, [C.c_void_p, C.POINTER(Windows)]),
     "flh_region_translate": (C.c_void_p, [C.c_void_p, C.c_uint32, C.c_void_p]),
     "flh_tune": (C.c_int, [C.c_char_p, C.c_int64]),
+    "flh_prof_enable": (C.c_int, [C.c_int]),
+    "flh_prof_last_us": (C.c_int, [C.POINTER(C.c_double)]),
 }
 
 _lib = None

@@ -21,7 +21,7 @@ SCHED_F_NO_CREDIT = 1
 DESC_DTYPE = np.dtype([("src_off", "<u8"), ("win_off", "<u8"), ("len", "<u4"), ("lane", "<u4"),
                        ("tile_base", "<u4"), ("epoch", "<u4")])
 HDR_DTYPE = np.dtype([("total_bytes", "<u8"), ("total_tiles", "<u4"), ("n_chunks", "<u4"), ("flags", "<u4"),
-                      ("pad", "<u4"), ("lane_bytes", "<u8", (MAX_LANES,)), ("lane_chunks", "<u4", (MAX_LANES,))])
+                      ("uniform_tiles", "<u4"), ("lane_bytes", "<u8", (MAX_LANES,)), ("lane_chunks", "<u4", (MAX_LANES,))])
 STATE_DTYPE = np.dtype([("epoch_bytes", "<u8"), ("chunk_index", "<u8"), ("lane_off", "<u8", (MAX_LANES,))])
 assert DESC_DTYPE.itemsize == C.sizeof(ChunkDesc) == 32
 assert HDR_DTYPE.itemsize == C.sizeof(SchedHdr)
@@ -34,6 +34,16 @@ def init(device: int = 0) -> None:
 
 def tune(key: str, value: int) -> None:
     check(_lib.load().flh_tune(key.encode(), int(value)))
+
+
+def prof_enable(on: bool) -> None:
+    check(_lib.load().flh_prof_enable(int(on)))
+
+
+def prof_last_us() -> float:
+    us = C.c_double()
+    check(_lib.load().flh_prof_last_us(C.byref(us)))
+    return us.value
 
 
 def _stream_ptr(stream: Optional[torch.cuda.Stream]) -> C.c_void_p:
@@ -121,16 +131,34 @@ def new_status(device="cuda") -> torch.Tensor:
     return torch.zeros(1, dtype=torch.int32, device=device)
 
 
+def uniform_hint(total_bytes: int, chunk_bytes: int, tile_bytes: int = TILE_BYTES) -> SchedHdr:
+    """Host copy of the header fields that follow from a uniform split alone (no device read)."""
+    h = SchedHdr()
+    n = (total_bytes + chunk_bytes - 1) // chunk_bytes if chunk_bytes else 0
+    per = (chunk_bytes + tile_bytes - 1) // tile_bytes if n else 0
+    last = total_bytes - (n - 1) * chunk_bytes if n else 0
+    h.total_bytes = total_bytes
+    h.n_chunks = n
+    h.uniform_tiles = per
+    h.total_tiles = (n - 1) * per + (last + tile_bytes - 1) // tile_bytes if n else 0
+    return h
+
+
+def _hint_ref(hint: Optional[SchedHdr]):
+    return C.byref(hint) if hint is not None else None
+
+
 def stripe(src: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tensor,
-           stream: Optional[torch.cuda.Stream] = None) -> None:
+           stream: Optional[torch.cuda.Stream] = None, hint: Optional[SchedHdr] = None) -> None:
     check(_lib.load().flh_stripe(_ptr(src), src.numel() * src.element_size(), C.byref(win), _ptr(sched.table),
-                                 _ptr(sched.hdr), sched.n_chunks, sched.tile_bytes, _ptr(status), _stream_ptr(stream)))
+                                 _ptr(sched.hdr), _hint_ref(hint), sched.n_chunks, sched.tile_bytes, _ptr(status),
+                                 _stream_ptr(stream)))
 
 
 def reassemble(dst: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tensor,
-               stream: Optional[torch.cuda.Stream] = None) -> None:
+               stream: Optional[torch.cuda.Stream] = None, hint: Optional[SchedHdr] = None) -> None:
     check(_lib.load().flh_reassemble(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), _ptr(sched.table),
-                                     _ptr(sched.hdr), sched.n_chunks, sched.tile_bytes, _ptr(status),
+                                     _ptr(sched.hdr), _hint_ref(hint), sched.n_chunks, sched.tile_bytes, _ptr(status),
                                      _stream_ptr(stream)))
 
 

@@ -7,6 +7,7 @@
 // no MFMA.  Wavefronts are 64 wide; all cross-lane traffic in the scheduler is DPP row shifts and
 // row broadcasts, LDS is used only to pass per-wave totals between the waves of the one workgroup.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdio>
@@ -107,7 +108,6 @@ __device__ __forceinline__ uint32_t wave_shift_up_u32(uint32_t v, int lane) {
 // ------------------------------------------------------------------------------------------------
 // scheduler
 // ------------------------------------------------------------------------------------------------
-constexpr int kItems = 4;          // chunks per thread per pass
 constexpr int kRowCache = 32;      // credit rows kept in LDS
 
 struct SchedArgs {
@@ -128,9 +128,56 @@ struct SchedArgs {
   uint32_t tile_bytes;
   uint32_t mode;
   int32_t quantum_shift;  // >= 0 when quantum is a power of two
+  int32_t tile_shift;     // >= 0 when tile_bytes is a power of two
 };
 
-template <int NW>
+// 64-bit division is a long software routine on this ISA and almost every operand here fits 32
+// bits; the wide case is kept out of line so that the kernel stays small enough for the
+// instruction cache (a lone wavefront cannot hide instruction fetch).
+__device__ __attribute__((noinline)) uint64_t div_u64_wide(uint64_t a, uint64_t b) { return a / b; }
+__device__ __forceinline__ uint64_t div_u64(uint64_t a, uint64_t b) {
+  return ((a | b) >> 32) == 0 ? (uint64_t)((uint32_t)a / (uint32_t)b) : div_u64_wide(a, b);
+}
+__device__ __forceinline__ uint64_t mod_u64(uint64_t a, uint64_t b) {
+  return ((a | b) >> 32) == 0 ? (uint64_t)((uint32_t)a % (uint32_t)b) : a - div_u64_wide(a, b) * b;
+}
+
+template <typename T> __device__ __forceinline__ T wave_incl_sum(T v, int lane);
+template <> __device__ __forceinline__ uint32_t wave_incl_sum<uint32_t>(uint32_t v, int lane) { return wave_incl_sum_u32(v, lane); }
+template <> __device__ __forceinline__ uint64_t wave_incl_sum<uint64_t>(uint64_t v, int lane) { return wave_incl_sum_u64(v, lane); }
+
+// In-wavefront part of the window offsets: for every lane l in turn, scan the threads' bytes on l
+// and hand each chunk on l its exclusive position; the wavefront's total per lane goes to LDS.
+// T is the width of the partial sums (32 bits when the whole pass moves less than 4 GiB).
+template <typename T, int K>
+__device__ __forceinline__ void lane_pass(const uint32_t (&s)[K], const uint32_t (&ln)[K], uint32_t L, int lane,
+                                          uint64_t* w_lane_row, uint32_t* cnt_lane, uint64_t (&off)[K]) {
+#pragma unroll 1
+  for (uint32_t l = 0; l < L; ++l) {
+    T v = 0;
+    uint32_t c = 0;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const bool mine = ln[k] == l;
+      v += mine ? (T)s[k] : (T)0;
+      c += (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(mine));
+    }
+    const T inc = wave_incl_sum<T>(v, lane);
+    uint64_t ex = (uint64_t)(inc - v);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      if (ln[k] == l) { off[k] = ex; ex += s[k]; }
+    }
+    if (lane == kWave - 1) w_lane_row[l] = (uint64_t)inc;
+    if (lane == 0 && c) atomicAdd(&cnt_lane[l], c);
+  }
+}
+
+// One workgroup of NW wavefronts walks the chunk list in passes of NW*64*K chunks; thread t owns K
+// consecutive chunks of a pass.  Per pass: thread-local sums, three wavefront scans (epoch-segmented
+// bytes, bytes, tiles), the lane of each chunk from its quantum slot, one wavefront scan per lane
+// for the window offsets.  LDS only carries per-wavefront totals and the running lane offsets.
+template <int NW, int K>
 __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   constexpr int BT = NW * kWave;
   const int tid = threadIdx.x;
@@ -140,260 +187,229 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
 
   // credit rows as inclusive prefixes; row r occupies rowpfx[r][0..L), W = rowpfx[r][L-1]
   __shared__ uint64_t rowpfx[kRowCache][FLH_MAX_LANES];
+  __shared__ uint32_t rowzero[kRowCache];  // the row had no credit at all
   __shared__ uint64_t w_seg_v[NW];
   __shared__ uint32_t w_seg_f[NW];
   __shared__ uint64_t w_run[NW];
   __shared__ uint32_t w_tiles[NW];
-  __shared__ uint64_t w_lane[NW][FLH_MAX_LANES];
+  __shared__ uint64_t w_lane[NW][FLH_MAX_LANES];  // per-wavefront lane totals, then absolute bases
+  __shared__ uint64_t lane_off[FLH_MAX_LANES];    // next free byte of every window
+  __shared__ uint64_t lane_off0[FLH_MAX_LANES];
   __shared__ uint32_t cnt_lane[FLH_MAX_LANES];
+  __shared__ uint32_t sh_flags;
 
+  // One wavefront per row: lanes 0..L-1 load the row in a single access, a scan forms the prefixes.
+  // A row without any credit (every lane busy) is replaced by equal credits -- the round-robin of
+  // the static policy -- and flagged.
   const bool rows_cached = a.n_rows <= (uint32_t)kRowCache;
+  uint32_t flags = 0;
   if (rows_cached) {
-    for (uint32_t r = tid; r < a.n_rows; r += BT) {
-      uint64_t k = 0;
-      for (uint32_t l = 0; l < L; ++l) { k += a.credits[(size_t)r * L + l]; rowpfx[r][l] = k; }
+    for (uint32_t r = wave; r < a.n_rows; r += NW) {
+      const uint32_t c = (uint32_t)lane < L ? a.credits[(size_t)r * L + lane] : 0;
+      uint64_t inc = wave_incl_sum_u64(c, lane);
+      const bool zero = bcast_lane_u64(inc, kWave - 1) == 0;
+      if (zero) inc = (uint32_t)lane < L ? lane + 1 : L;
+      if ((uint32_t)lane < L) rowpfx[r][lane] = inc;
+      if (lane == 0) rowzero[r] = zero;
     }
   }
-  if (tid < FLH_MAX_LANES) cnt_lane[tid] = 0;
-
-  // carried state (identical in every thread)
-  uint64_t k0 = 0, p_carry = 0, run_carry = 0;
-  uint32_t tiles_carry = 0, flags = 0;
-  uint64_t lane_off[FLH_MAX_LANES];
-  uint64_t lane_off0[FLH_MAX_LANES];
-#pragma unroll
-  for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off[l] = 0;
+  uint64_t k0 = 0, p_carry = 0, run_carry = 0;  // carried state, identical in every thread
+  uint32_t tiles_carry = 0;
   if (a.state) {
     k0 = a.state->chunk_index;
     p_carry = a.state->epoch_bytes;
-    if (!(a.mode & FLH_SCHED_RESET_OFFSETS)) {
-#pragma unroll
-      for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off[l] = a.state->lane_off[l];
-    }
   }
-#pragma unroll
-  for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off0[l] = lane_off[l];
-  uint32_t my_cnt[FLH_MAX_LANES];
-#pragma unroll
-  for (int l = 0; l < FLH_MAX_LANES; ++l) my_cnt[l] = 0;
-
+  if (tid < FLH_MAX_LANES) {
+    const uint64_t o = (a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS)) ? a.state->lane_off[tid] : 0;
+    lane_off[tid] = o;
+    lane_off0[tid] = o;
+    cnt_lane[tid] = 0;
+  }
+  if (tid == 0) sh_flags = 0;
   __syncthreads();
 
-  for (uint32_t pass = 0; pass < a.n; pass += BT * kItems) {
-    const uint32_t i0 = pass + (uint32_t)tid * kItems;
-    uint32_t s[kItems];
-    uint32_t head[kItems];
+#pragma unroll 1
+  for (uint32_t pass = 0; pass < a.n; pass += BT * K) {
+    const uint32_t i0 = pass + (uint32_t)tid * K;
+    uint32_t s[K], tl[K], row[K], ep[K], ln[K];
+    bool head[K];
+    // ---- epoch, position in epoch and credit row of my first chunk; the rest follow by counting ----
+    uint64_t e_cur = 0;
+    uint32_t pos = 0, r_cur = 0;
+    if (a.epoch_len) {
+      const uint64_t g0 = k0 + i0;
+      e_cur = div_u64(g0, a.epoch_len);
+      pos = (uint32_t)(g0 - e_cur * a.epoch_len);
+      r_cur = (uint32_t)mod_u64(e_cur, a.n_rows);
+    }
     // ---- load sizes, mark epoch heads, thread-local aggregates -----------------------------------
     uint64_t seg_v = 0;
     uint32_t seg_f = 0;
     uint64_t run = 0;
     uint32_t tiles = 0;
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) {
+    for (int k = 0; k < K; ++k) {
       const uint32_t i = i0 + k;
-      uint32_t sz = 0, hd = 0;
+      uint32_t sz = 0;
+      bool hd = false;
       if (i < a.n) {
         if (a.sizes) {
           sz = a.sizes[i];
         } else {
-          uint64_t o = (uint64_t)i * a.chunk_bytes;
-          uint64_t rem = o < a.total_bytes ? a.total_bytes - o : 0;
+          const uint64_t o = (uint64_t)i * a.chunk_bytes;
+          const uint64_t rem = o < a.total_bytes ? a.total_bytes - o : 0;
           sz = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
         }
-        hd = a.epoch_len && ((k0 + i) % a.epoch_len == 0);
+        hd = a.epoch_len && pos == 0;
       }
       s[k] = sz;
       head[k] = hd;
+      row[k] = r_cur;
+      ep[k] = (uint32_t)e_cur;
+      tl[k] = a.tile_shift >= 0 ? (sz + a.tile_bytes - 1) >> a.tile_shift : (sz + a.tile_bytes - 1) / a.tile_bytes;
       if (hd) { seg_v = 0; seg_f = 1; }
       seg_v += sz;
       run += sz;
-      tiles += (sz + a.tile_bytes - 1) / a.tile_bytes;
+      tiles += tl[k];
+      if (a.epoch_len && ++pos == a.epoch_len) {
+        pos = 0;
+        ++e_cur;
+        if (++r_cur == a.n_rows) r_cur = 0;
+      }
     }
     // ---- block-wide exclusive prefixes of (segmented bytes, bytes, tiles) --------------------------
     uint64_t sv = seg_v;
     uint32_t sf = seg_f;
     wave_incl_segsum_u64(sv, sf, lane);
-    uint64_t run_incl = wave_incl_sum_u64(run, lane);
-    uint32_t tiles_incl = wave_incl_sum_u32(tiles, lane);
+    const uint64_t run_incl = wave_incl_sum_u64(run, lane);
+    const uint32_t tiles_incl = wave_incl_sum_u32(tiles, lane);
     uint64_t seg_ex_v = wave_shift_up_u64(sv, lane);
     uint32_t seg_ex_f = wave_shift_up_u32(sf, lane);
     uint64_t run_ex = run_incl - run;
     uint32_t tiles_ex = tiles_incl - tiles;
-    uint64_t tot_seg_v, tot_run;
-    uint32_t tot_seg_f, tot_tiles;
-    if (NW > 1) {
-      if (lane == kWave - 1) { w_seg_v[wave] = sv; w_seg_f[wave] = sf; w_run[wave] = run_incl; w_tiles[wave] = tiles_incl; }
-      __syncthreads();
+    if (lane == kWave - 1) { w_seg_v[wave] = sv; w_seg_f[wave] = sf; w_run[wave] = run_incl; w_tiles[wave] = tiles_incl; }
+    __syncthreads();
+    uint64_t tot_seg_v = 0, tot_run = 0;
+    uint32_t tot_seg_f = 0, tot_tiles = 0;
+    {
       uint64_t pv = 0, pr = 0;
       uint32_t pf = 0, pt = 0;
-      tot_seg_v = 0; tot_seg_f = 0; tot_run = 0; tot_tiles = 0;
+#pragma unroll
       for (int w = 0; w < NW; ++w) {
         if (w == wave) { pv = tot_seg_v; pf = tot_seg_f; pr = tot_run; pt = tot_tiles; }
-        uint64_t wv = w_seg_v[w];
-        uint32_t wf = w_seg_f[w];
+        const uint64_t wv = w_seg_v[w];
+        const uint32_t wf = w_seg_f[w];
         tot_seg_v = wf ? wv : tot_seg_v + wv;
         tot_seg_f |= wf;
         tot_run += w_run[w];
         tot_tiles += w_tiles[w];
       }
-      // combine the earlier waves' aggregate with my in-wave exclusive value
+      // combine the earlier wavefronts' aggregate with my in-wavefront exclusive value
       if (!seg_ex_f) seg_ex_v += pv;
       seg_ex_f |= pf;
       run_ex += pr;
       tiles_ex += pt;
-    } else {
-      tot_seg_v = bcast_lane_u64(sv, kWave - 1);
-      tot_seg_f = bcast_lane_u32(sf, kWave - 1);
-      tot_run = bcast_lane_u64(run_incl, kWave - 1);
-      tot_tiles = bcast_lane_u32(tiles_incl, kWave - 1);
     }
-    // bytes of my epoch before my first item
+    // bytes of my epoch before my first chunk
     uint64_t P = seg_ex_f ? seg_ex_v : p_carry + seg_ex_v;
 
-    // ---- lane of each item ----------------------------------------------------------------------------
-    uint32_t ln[kItems];
-    uint32_t ep[kItems];
-    uint64_t acc[FLH_MAX_LANES];
+    // ---- lane of each chunk ------------------------------------------------------------------------------
 #pragma unroll
-    for (int l = 0; l < FLH_MAX_LANES; ++l) acc[l] = 0;
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
+    for (int k = 0; k < K; ++k) {
       const uint32_t i = i0 + k;
-      ln[k] = 0;
-      ep[k] = 0;
+      ln[k] = FLH_MAX_LANES;  // matches no lane: chunks past the end count nowhere
       if (i < a.n) {
         if (head[k]) P = 0;
-        const uint64_t g = k0 + i;
-        const uint64_t e = a.epoch_len ? g / a.epoch_len : 0;
-        const uint32_t r = (uint32_t)(e % a.n_rows);
+        const uint32_t r = row[k];
         uint64_t W;
+        bool equal = false;  // no lane has credit: equal credits stand in
         if (rows_cached) {
           W = rowpfx[r][L - 1];
+          if (rowzero[r]) flags |= FLH_SCHED_F_NO_CREDIT;
         } else {
           W = 0;
+#pragma unroll 1
           for (uint32_t l = 0; l < L; ++l) W += a.credits[(size_t)r * L + l];
+          if (W == 0) { W = L; equal = true; flags |= FLH_SCHED_F_NO_CREDIT; }
         }
-        uint32_t pick;
-        if (W == 0) {
-          pick = (uint32_t)(g % L);
-          flags |= FLH_SCHED_F_NO_CREDIT;
+        const uint64_t qn = a.quantum_shift >= 0 ? (P >> a.quantum_shift) : div_u64(P, a.quantum);
+        const uint64_t slot = mod_u64(qn, W);
+        // lane = number of inclusive prefixes <= slot (zero-credit lanes repeat the prefix and are skipped)
+        uint32_t pick = 0;
+        if (rows_cached) {
+#pragma unroll 1
+          for (uint32_t l = 0; l + 1 < L; ++l) pick += rowpfx[r][l] <= slot;
+        } else if (equal) {
+          pick = (uint32_t)slot;
         } else {
-          const uint64_t qn = a.quantum_shift >= 0 ? (P >> a.quantum_shift) : (P / a.quantum);
-          const uint64_t slot = (qn >> 32) == 0 && (W >> 32) == 0 ? (uint64_t)((uint32_t)qn % (uint32_t)W) : qn % W;
-          // lane = number of inclusive prefixes <= slot (zero-credit lanes repeat the prefix and are skipped)
-          pick = 0;
-          if (rows_cached) {
-            for (uint32_t l = 0; l + 1 < L; ++l) pick += rowpfx[r][l] <= slot;
-          } else {
-            uint64_t kk = 0;
-            for (uint32_t l = 0; l + 1 < L; ++l) { kk += a.credits[(size_t)r * L + l]; pick += kk <= slot; }
-          }
+          uint64_t kk = 0;
+#pragma unroll 1
+          for (uint32_t l = 0; l + 1 < L; ++l) { kk += a.credits[(size_t)r * L + l]; pick += kk <= slot; }
         }
         ln[k] = pick;
-        ep[k] = (uint32_t)e;
         P += s[k];
-#pragma unroll
-        for (int l = 0; l < FLH_MAX_LANES; ++l) {
-          acc[l] += (pick == (uint32_t)l) ? (uint64_t)s[k] : 0;
-          my_cnt[l] += (pick == (uint32_t)l);
-        }
       }
     }
-    // ---- per-lane exclusive prefixes across the block ----------------------------------------------
-    uint64_t base[FLH_MAX_LANES];
-    uint64_t tot_lane[FLH_MAX_LANES];
+    // ---- window offsets: in-wavefront scans per lane, then wavefront bases through LDS -----------------
+    uint64_t off[K];
 #pragma unroll
-    for (int l = 0; l < FLH_MAX_LANES; ++l) {
-      base[l] = 0;
-      tot_lane[l] = 0;
-      if ((uint32_t)l < L) {
-        uint64_t inc = wave_incl_sum_u64(acc[l], lane);
-        base[l] = inc - acc[l];
-        if (NW > 1) {
-          if (lane == kWave - 1) w_lane[wave][l] = inc;
-        } else {
-          tot_lane[l] = bcast_lane_u64(inc, kWave - 1);
-        }
-      }
-    }
-    if (NW > 1) {
-      __syncthreads();
+    for (int k = 0; k < K; ++k) off[k] = 0;
+    if ((tot_run >> 32) == 0) lane_pass<uint32_t, K>(s, ln, L, lane, w_lane[wave], cnt_lane, off);
+    else lane_pass<uint64_t, K>(s, ln, L, lane, w_lane[wave], cnt_lane, off);
+    __syncthreads();
+    if ((uint32_t)tid < L) {
+      uint64_t at = lane_off[tid];
 #pragma unroll
-      for (int l = 0; l < FLH_MAX_LANES; ++l) {
-        if ((uint32_t)l < L) {
-          uint64_t before = 0, tot = 0;
-          for (int w = 0; w < NW; ++w) {
-            uint64_t x = w_lane[w][l];
-            if (w < wave) before += x;
-            tot += x;
-          }
-          base[l] += before;
-          tot_lane[l] = tot;
-        }
+      for (int w = 0; w < NW; ++w) {
+        const uint64_t x = w_lane[w][tid];
+        w_lane[w][tid] = at;
+        at += x;
       }
+      lane_off[tid] = at;
     }
+    __syncthreads();
     // ---- emit rows ---------------------------------------------------------------------------------------
     uint64_t run_i = run_carry + run_ex;
     uint32_t tiles_i = tiles_carry + tiles_ex;
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) {
+    for (int k = 0; k < K; ++k) {
       const uint32_t i = i0 + k;
       if (i < a.n) {
-        uint64_t off = 0;
-#pragma unroll
-        for (int l = 0; l < FLH_MAX_LANES; ++l) {
-          if (ln[k] == (uint32_t)l) { off = lane_off[l] + base[l]; base[l] += s[k]; }
-        }
         flh_chunk_desc d;
         d.src_off = a.src_off ? a.src_off[i] : a.src_base + run_i;
-        d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : off;
+        d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : w_lane[wave][ln[k]] + off[k];
         d.len = s[k];
         d.lane = ln[k];
         d.tile_base = tiles_i;
         d.epoch = ep[k];
         a.table[i] = d;
         run_i += s[k];
-        tiles_i += (s[k] + a.tile_bytes - 1) / a.tile_bytes;
+        tiles_i += tl[k];
       }
     }
-    // ---- carries ---------------------------------------------------------------------------------------------
+    // ---- carries -------------------------------------------------------------------------------------------
     p_carry = tot_seg_f ? tot_seg_v : p_carry + tot_seg_v;
     run_carry += tot_run;
     tiles_carry += tot_tiles;
-#pragma unroll
-    for (int l = 0; l < FLH_MAX_LANES; ++l) lane_off[l] += tot_lane[l];
-    if (NW > 1) __syncthreads();  // LDS scratch is reused by the next pass
   }
 
   // ---- header and state --------------------------------------------------------------------------------------
-#pragma unroll
-  for (int l = 0; l < FLH_MAX_LANES; ++l) {
-    uint32_t c = wave_incl_sum_u32(my_cnt[l], lane);
-    if (lane == kWave - 1 && c) atomicAdd(&cnt_lane[l], c);
+  if (__builtin_amdgcn_ballot_w64(flags != 0) && lane == 0) atomicOr(&sh_flags, FLH_SCHED_F_NO_CREDIT);
+  __syncthreads();
+  if (tid < FLH_MAX_LANES) {
+    a.hdr->lane_bytes[tid] = lane_off[tid] - lane_off0[tid];
+    a.hdr->lane_chunks[tid] = cnt_lane[tid];
+    if (a.state) a.state->lane_off[tid] = lane_off[tid];
   }
-  uint32_t any_flags = flags;
-  any_flags = __builtin_amdgcn_ballot_w64(any_flags != 0) ? 1u : 0u;
-  __shared__ uint32_t sh_flags;
-  if (tid == 0) sh_flags = 0;
-  __syncthreads();
-  if (lane == 0 && any_flags) atomicOr(&sh_flags, FLH_SCHED_F_NO_CREDIT);
-  __syncthreads();
   if (tid == 0) {
-    flh_sched_hdr h;
-    h.total_bytes = run_carry;
-    h.total_tiles = tiles_carry;
-    h.n_chunks = a.n;
-    h.flags = sh_flags;
-    h.pad = 0;
-    for (int l = 0; l < FLH_MAX_LANES; ++l) {
-      h.lane_bytes[l] = lane_off[l] - lane_off0[l];
-      h.lane_chunks[l] = cnt_lane[l];
-    }
-    *a.hdr = h;
+    a.hdr->total_bytes = run_carry;
+    a.hdr->total_tiles = tiles_carry;
+    a.hdr->n_chunks = a.n;
+    a.hdr->flags = sh_flags;
+    a.hdr->uniform_tiles = (!a.sizes && a.n) ? (a.chunk_bytes + a.tile_bytes - 1) / a.tile_bytes : 0;
     if (a.state) {
       a.state->epoch_bytes = p_carry;
       a.state->chunk_index = k0 + a.n;
-      for (int l = 0; l < FLH_MAX_LANES; ++l) a.state->lane_off[l] = lane_off[l];
     }
   }
 }
@@ -461,25 +477,52 @@ struct CopyArgs {
   int32_t* status;
   uint32_t n_chunks_max;
   uint32_t tile_bytes;
+  // header fields the host already knows (has_hint != 0): saves one dependent memory round trip
+  uint32_t has_hint, hint_total_tiles, hint_n_chunks, hint_uniform_tiles;
 };
+
+// Row of the table that owns copy tile t: the last row with tile_base <= t (rows of empty chunks own
+// no tile and are stepped over).  A uniform split is answered by one division and one row load; any
+// other table by a 64-ary search in which every lane of the wavefront probes one row per round
+// (three rounds cover 262144 chunks).  The result is wavefront-uniform.
+__device__ __forceinline__ uint32_t find_row(const flh_chunk_desc* __restrict__ table, uint32_t n, uint32_t t,
+                                             uint32_t uniform_tiles, uint32_t tile_bytes) {
+  if (uniform_tiles) {
+    const uint32_t c = t / uniform_tiles;
+    if (c < n) {
+      const uint32_t tb = table[c].tile_base;
+      const uint32_t len = table[c].len;
+      if (t >= tb && (uint64_t)(t - tb) * tile_bytes < len) return c;
+    }
+  }
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint32_t lo = 0, cnt = n;  // the answer lies in [lo, lo + cnt); table[lo].tile_base <= t
+  while (cnt > 1) {
+    const uint32_t step = (cnt + kWave - 1) / kWave;
+    const uint32_t idx = lo + lane * step;
+    const bool le = idx < lo + cnt && table[idx].tile_base <= t;
+    const uint32_t k = (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+    const uint32_t adv = (k ? k - 1 : 0) * step;
+    const uint32_t end = lo + cnt;
+    lo += adv;
+    cnt = end - lo < step ? end - lo : step;
+  }
+  return lo;
+}
 
 // DIR 0: user -> windows (stripe).  DIR 1: windows -> user (reassemble).
 template <int DIR, bool NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
-  const uint32_t total = a.hdr->total_tiles;
-  uint32_t n = a.hdr->n_chunks;
+  const uint32_t total = a.has_hint ? a.hint_total_tiles : a.hdr->total_tiles;
+  const uint32_t uniform_tiles = a.has_hint ? a.hint_uniform_tiles : a.hdr->uniform_tiles;
+  uint32_t n = a.has_hint ? a.hint_n_chunks : a.hdr->n_chunks;
   if (n > a.n_chunks_max) n = a.n_chunks_max;
+  if (n == 0) return;
   for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
-    // last row whose tile_base <= t (empty chunks own no tile and are stepped over)
-    uint32_t lo = 0, hi = n;
-    while (hi - lo > 1) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (a.table[mid].tile_base <= t) lo = mid; else hi = mid;
-    }
-    if (n == 0) break;
-    const flh_chunk_desc d = a.table[lo];
+    const uint32_t c = find_row(a.table, n, t, uniform_tiles, a.tile_bytes);
+    const flh_chunk_desc d = a.table[c];
     const uint64_t off = (uint64_t)(t - d.tile_base) * a.tile_bytes;
-    if (off >= d.len) continue;
+    if (t < d.tile_base || off >= d.len) continue;
     const uint32_t bytes = (uint32_t)((d.len - off) < a.tile_bytes ? (d.len - off) : a.tile_bytes);
     // refuse anything that would leave the user buffer or the mapped part of the window
     bool ok = d.lane < a.win.n_lanes;
@@ -571,7 +614,20 @@ int g_device = -1;
 int g_cus = 0;
 // launch tunables (overridable through NCCL_FUSELINK_* for experiments)
 int g_grid_per_cu = 8;
-int g_nontemporal = 1;
+int g_nontemporal = 0;
+int g_sched_variant = 0;  // 0 = pick the scheduler shape from the chunk count
+
+
+// Per-launch timing: when enabled for the calling thread, every kernel is launched with its own
+// start/stop events (hipExtLaunchKernelGGL), which bracket the kernel alone, not the gaps around it.
+thread_local bool g_prof_on = false;
+thread_local hipEvent_t g_prof_ev0 = nullptr, g_prof_ev1 = nullptr;
+
+#define FL_LAUNCH(kernel, grid, block, shmem, stream, ...)                                              \
+  do {                                                                                                  \
+    if (g_prof_on) hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, g_prof_ev0, g_prof_ev1, 0, __VA_ARGS__); \
+    else hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                           \
+  } while (0)
 
 int64_t env_i64(const char* name, int64_t dflt) {
   const char* v = getenv(name);
@@ -638,10 +694,30 @@ int flh_init(int device) {
   return FLH_OK;
 }
 
+int flh_prof_enable(int on) {
+  if (on && !g_prof_ev0) {
+    FL_HIP(hipEventCreate(&g_prof_ev0));
+    FL_HIP(hipEventCreate(&g_prof_ev1));
+  }
+  g_prof_on = on != 0;
+  return FLH_OK;
+}
+
+int flh_prof_last_us(double* us) {
+  if (!us) return fl_set_error(FLH_E_ARG, "null out");
+  if (!g_prof_ev1) return fl_set_error(FLH_E_STATE, "profiling was never enabled on this thread");
+  FL_HIP(hipEventSynchronize(g_prof_ev1));
+  float ms = 0.f;
+  FL_HIP(hipEventElapsedTime(&ms, g_prof_ev0, g_prof_ev1));
+  *us = (double)ms * 1e3;
+  return FLH_OK;
+}
+
 int flh_tune(const char* key, int64_t value) {
   if (!key) return fl_set_error(FLH_E_ARG, "null key");
   if (!strcmp(key, "grid_per_cu")) { if (value < 1) return fl_set_error(FLH_E_ARG, "grid_per_cu < 1"); g_grid_per_cu = (int)value; return FLH_OK; }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value != 0; return FLH_OK; }
+  if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 5) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..5"); g_sched_variant = (int)value; return FLH_OK; }
   return fl_set_error(FLH_E_ARG, "unknown tunable %s", key);
 }
 
@@ -687,12 +763,19 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   a.mode = p->mode;
   a.quantum_shift = (p->quantum & (p->quantum - 1)) == 0 ? __builtin_ctzll(p->quantum) : -1;
   hipStream_t s = (hipStream_t)stream;
-  if (p->n_chunks <= kWave * kItems) {
-    hipLaunchKernelGGL(fl_schedule_kernel<1>, dim3(1), dim3(kWave), 0, s, a);
-  } else if (p->n_chunks <= 4 * kWave * kItems) {
-    hipLaunchKernelGGL(fl_schedule_kernel<4>, dim3(1), dim3(4 * kWave), 0, s, a);
+  a.tile_shift = (p->tile_bytes & (p->tile_bytes - 1)) == 0 ? __builtin_ctz(p->tile_bytes) : -1;
+  const uint32_t n = p->n_chunks;
+  const int variant = g_sched_variant;
+  if ((variant == 0 && n <= kWave) || variant == 1) {
+    FL_LAUNCH((fl_schedule_kernel<1, 1>), dim3(1), dim3(kWave), 0, s, a);
+  } else if ((variant == 0 && n <= 4 * kWave) || variant == 2) {
+    FL_LAUNCH((fl_schedule_kernel<4, 1>), dim3(1), dim3(4 * kWave), 0, s, a);
+  } else if ((variant == 0 && n <= 16 * kWave) || variant == 3) {
+    FL_LAUNCH((fl_schedule_kernel<16, 1>), dim3(1), dim3(16 * kWave), 0, s, a);
+  } else if (variant == 4) {
+    FL_LAUNCH((fl_schedule_kernel<8, 4>), dim3(1), dim3(8 * kWave), 0, s, a);
   } else {
-    hipLaunchKernelGGL(fl_schedule_kernel<8>, dim3(1), dim3(8 * kWave), 0, s, a);
+    FL_LAUNCH((fl_schedule_kernel<16, 4>), dim3(1), dim3(16 * kWave), 0, s, a);
   }
   FL_HIP(hipGetLastError());
   return FLH_OK;
@@ -714,7 +797,7 @@ static uint32_t copy_grid(uint64_t max_tiles) {
 }
 
 static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
-                       const flh_sched_hdr* d_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
+                       const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
   int rc = check_windows(win);
   if (rc) return rc;
   if (!d_hdr || !d_status) return fl_set_error(FLH_E_ARG, "d_hdr and d_status are required");
@@ -733,28 +816,35 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   a.status = d_status;
   a.n_chunks_max = n_chunks_max;
   a.tile_bytes = tile_bytes;
-  const uint64_t max_tiles = user_bytes / tile_bytes + n_chunks_max;
+  a.has_hint = h_hdr != nullptr;
+  a.hint_total_tiles = h_hdr ? h_hdr->total_tiles : 0;
+  a.hint_n_chunks = h_hdr ? h_hdr->n_chunks : 0;
+  a.hint_uniform_tiles = h_hdr ? h_hdr->uniform_tiles : 0;
+  const uint64_t max_tiles = h_hdr ? h_hdr->total_tiles : user_bytes / tile_bytes + n_chunks_max;
+  if (max_tiles == 0) return FLH_OK;
   const uint32_t grid = copy_grid(max_tiles);
   hipStream_t s = (hipStream_t)stream;
   if (dir == 0) {
-    if (g_nontemporal) hipLaunchKernelGGL((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
-    else hipLaunchKernelGGL((fl_copy_tiles<0, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    if (g_nontemporal) FL_LAUNCH((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_tiles<0, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
   } else {
-    if (g_nontemporal) hipLaunchKernelGGL((fl_copy_tiles<1, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
-    else hipLaunchKernelGGL((fl_copy_tiles<1, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    if (g_nontemporal) FL_LAUNCH((fl_copy_tiles<1, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_tiles<1, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
   }
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }
 
 int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
-               const flh_sched_hdr* d_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
-  return launch_copy(0, (void*)d_src, src_bytes, win, d_table, d_hdr, n_chunks_max, tile_bytes, d_status, stream);
+               const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, uint32_t n_chunks_max, uint32_t tile_bytes,
+               int32_t* d_status, void* stream) {
+  return launch_copy(0, (void*)d_src, src_bytes, win, d_table, d_hdr, h_hdr, n_chunks_max, tile_bytes, d_status, stream);
 }
 
 int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
-                   const flh_sched_hdr* d_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
-  return launch_copy(1, d_dst, dst_bytes, win, d_table, d_hdr, n_chunks_max, tile_bytes, d_status, stream);
+                   const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, uint32_t n_chunks_max, uint32_t tile_bytes,
+                   int32_t* d_status, void* stream) {
+  return launch_copy(1, d_dst, dst_bytes, win, d_table, d_hdr, h_hdr, n_chunks_max, tile_bytes, d_status, stream);
 }
 
 static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
@@ -785,7 +875,7 @@ static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t
   const uint32_t grid = copy_grid(total);
   hipStream_t s = (hipStream_t)stream;
   const bool nt = g_nontemporal != 0;
-#define FL_LAUNCH_PAGES(D, LD, N) hipLaunchKernelGGL((fl_page_tiles<D, LD, N>), dim3(grid), dim3(kCopyBlock), 0, s, a)
+#define FL_LAUNCH_PAGES(D, LD, N) FL_LAUNCH((fl_page_tiles<D, LD, N>), dim3(grid), dim3(kCopyBlock), 0, s, a)
   if (dir == 0) {
     if (use_lds) { if (nt) FL_LAUNCH_PAGES(0, true, true); else FL_LAUNCH_PAGES(0, true, false); }
     else { if (nt) FL_LAUNCH_PAGES(0, false, true); else FL_LAUNCH_PAGES(0, false, false); }
@@ -818,8 +908,8 @@ int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
   const uint32_t tile = FLH_TILE_BYTES;
   const uint32_t grid = copy_grid((bytes + tile - 1) / tile);
   hipStream_t s = (hipStream_t)stream;
-  if (g_nontemporal) hipLaunchKernelGGL(fl_plain_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
-  else hipLaunchKernelGGL(fl_plain_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  if (g_nontemporal) FL_LAUNCH(fl_plain_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  else FL_LAUNCH(fl_plain_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }

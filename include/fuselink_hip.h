@@ -61,7 +61,7 @@ typedef struct flh_sched_hdr {
   uint32_t total_tiles;
   uint32_t n_chunks;
   uint32_t flags;                      /* FLH_SCHED_F_* */
-  uint32_t pad;
+  uint32_t uniform_tiles;              /* tiles per chunk if the split is uniform (d_sizes == NULL), else 0 */
   uint64_t lane_bytes[FLH_MAX_LANES];  /* bytes this call put on each lane */
   uint32_t lane_chunks[FLH_MAX_LANES]; /* chunks this call put on each lane */
 } flh_sched_hdr;
@@ -104,6 +104,12 @@ int64_t flh_constant(int which);
  * workgroups launched per compute unit, "nontemporal" = 0/1 streaming loads and stores.
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL. */
 int flh_tune(const char* key, int64_t value);
+/* Per-kernel timing for measurement code (no counterpart in the reference).  While enabled on the
+ * calling thread, every launch made through this library carries its own start/stop HIP events
+ * that bracket the kernel alone; flh_prof_last_us waits for the last such launch and returns its
+ * duration in microseconds. */
+int flh_prof_enable(int on);
+int flh_prof_last_us(double* us);
 
 /* ---- scheduler ------------------------------------------------------------------------------
  * Replaces FuseLinkConnManager::refreshRxComm / bidTxChannel (src/fuselink.h:153-156, 230-238) and
@@ -122,7 +128,9 @@ int flh_schedule(const flh_sched_params* p, void* stream);
  * (src/plugin.cc:1626): window[lane] + win_off is copied to d_dst + src_off.
  * d_hdr->total_tiles sizes the work; win_cap[l] is the mapped size of window l and a chunk that
  * would cross it is skipped and reported through *d_status (FLH_E_RANGE), never written.
- * n_chunks_max bounds the table rows the kernel may read. */
+ * n_chunks_max bounds the table rows the kernel may read.  h_hdr is optional: a HOST copy of the
+ * header whose total_tiles, n_chunks and uniform_tiles the caller already knows (for a uniform
+ * split they follow from the sizes alone); with it the kernel does not wait for d_hdr. */
 typedef struct flh_windows {
   void*    base[FLH_MAX_LANES];
   uint64_t cap[FLH_MAX_LANES];
@@ -131,11 +139,11 @@ typedef struct flh_windows {
 } flh_windows;
 
 int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win,
-               const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, uint32_t n_chunks_max,
-               uint32_t tile_bytes, int32_t* d_status, void* stream);
+               const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr,
+               uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream);
 int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
-                   const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, uint32_t n_chunks_max,
-                   uint32_t tile_bytes, int32_t* d_status, void* stream);
+                   const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr,
+                   uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream);
 
 /* Paged variants for non-contiguous sources (KV-cache blocks, src/experiments/serving/model.hh:
  * 198-201 gives the page shape): chunk c of the table stands for pages

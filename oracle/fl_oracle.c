@@ -159,14 +159,17 @@ int fl_credit_schedule(const uint32_t* sizes, uint64_t total_bytes, uint32_t chu
     const uint32_t* row = credits + (size_t)(e % n_rows) * n_lanes;
     uint64_t W = 0;
     for (uint32_t l = 0; l < n_lanes; ++l) W += row[l];
-    uint32_t lane;
-    if (W == 0) {
-      lane = (uint32_t)(g % n_lanes);           /* static fallback, fuselink.h:235 */
+    uint32_t ones[FLO_MAX_NIC_NUM];
+    if (W == 0) {                                 /* every lane busy: equal credits stand in, which */
+      for (uint32_t l = 0; l < n_lanes; ++l) ones[l] = 1; /* is the round-robin of fuselink.h:235 */
+      row = ones;
+      W = n_lanes;
       h.flags |= FLO_SCHED_F_NO_CREDIT;
-    } else {
+    }
+    uint32_t lane = 0;
+    {
       uint64_t slot = (P / quantum) % W;
       uint64_t K = 0;
-      lane = 0;
       for (uint32_t l = 0; l < n_lanes; ++l) {
         if (slot >= K && slot < K + row[l]) { lane = l; break; }
         K += row[l];
@@ -188,6 +191,7 @@ int fl_credit_schedule(const uint32_t* sizes, uint64_t total_bytes, uint32_t chu
   h.total_bytes = run;
   h.total_tiles = tiles;
   h.n_chunks = n;
+  h.uniform_tiles = (!sizes && n) ? (chunk_bytes + tile_bytes - 1) / tile_bytes : 0;
   if (hdr) *hdr = h;
   if (state) {
     state->epoch_bytes = P;

@@ -111,8 +111,9 @@ void fl_credits_from_status(const int32_t* status, int n_lanes, int own_lane,
  * state.  For chunk i with global index g = k0 + i:  epoch e = E ? g / E : 0, row r = e mod R,
  * W = sum_l c[r][l],  P_i = bytes of earlier chunks of the same epoch (carry-in included),
  * slot = floor(P_i / q) mod W,  lane_i = the l with K_l <= slot < K_l + c[r][l] (K = exclusive
- * prefix of the row).  W == 0 (no lane has credit) falls back to the static policy g mod L
- * (fuselink.h:235) and raises FLO_SCHED_F_NO_CREDIT.  win_off_i = lane_off_in[lane_i] + bytes of
+ * prefix of the row).  A row with W == 0 (no lane has credit) is replaced by equal credits c = 1,
+ * i.e. round-robin over the lanes as in the static policy (fuselink.h:235), and raises
+ * FLO_SCHED_F_NO_CREDIT.  win_off_i = lane_off_in[lane_i] + bytes of
  * earlier chunks of this call on the same lane.  tile_base_i = sum_{j<i} ceil(s_j / T).
  * src_off_i = src_off[i] if given, else src_base + sum_{j<i} s_j.
  *
@@ -141,7 +142,7 @@ typedef struct {
   uint32_t total_tiles;
   uint32_t n_chunks;
   uint32_t flags;
-  uint32_t pad;
+  uint32_t uniform_tiles;                /* tiles per chunk when the split is uniform (sizes == NULL), else 0 */
   uint64_t lane_bytes[FLO_MAX_NIC_NUM];  /* bytes assigned to each lane by this call */
   uint32_t lane_chunks[FLO_MAX_NIC_NUM]; /* chunks assigned to each lane by this call */
 } fl_sched_hdr_t;

@@ -40,7 +40,7 @@ def _check_schedule(fl, *, n_lanes, credits, quantum, sizes=None, total_bytes=0,
     got_t, got_h = sched.table_numpy(), sched.hdr_numpy()
     for f in ob.DESC_DTYPE.names:
         np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
-    for f in ("total_bytes", "total_tiles", "n_chunks", "flags", "lane_bytes", "lane_chunks"):
+    for f in ("total_bytes", "total_tiles", "n_chunks", "flags", "uniform_tiles", "lane_bytes", "lane_chunks"):
         np.testing.assert_array_equal(got_h[f], exp_h[f], err_msg=f"hdr field {f}")
     if state is not None:
         got_s = core.state_numpy(d_state)
@@ -186,3 +186,46 @@ def test_window_overflow_is_refused_not_written(fl):
     torch.cuda.synchronize()
     assert int(status.item()) == -5
     assert not wins[1][caps[1]:].cpu().numpy().any()
+
+
+def test_roundtrip_many_small_chunks_three_search_rounds(fl):
+    # > 4096 variable-size chunks: the tile -> row search needs three 64-ary rounds
+    rng = np.random.default_rng(13)
+    sizes = (rng.integers(0, 200, size=5000) * 16).astype(np.uint32)
+    src = rng.integers(0, 256, size=int(sizes.sum()), dtype=np.uint8)
+    out = _roundtrip(fl, src, n_lanes=16, credits=rng.integers(0, 4, size=16) + np.eye(16, dtype=np.int64)[3],
+                     quantum=1024, sizes=sizes, tile_bytes=1024)
+    np.testing.assert_array_equal(out, src)
+
+
+def test_host_hint_matches_device_header(fl):
+    core, torch = fl
+    for total, chunk, tile in [(64 << 20, 256 << 10, 32768), ((4 << 20) + 1, 512 << 10, 32768), (5, 4096, 4096), (0, 4096, 4096)]:
+        sched, _, exp_h = _check_schedule(fl, n_lanes=4, credits=[1, 2, 3, 4], quantum=chunk, total_bytes=total,
+                                          chunk_bytes=chunk, tile_bytes=tile)
+        h = core.uniform_hint(total, chunk, tile)
+        assert (h.total_tiles, h.n_chunks, h.uniform_tiles) == (exp_h["total_tiles"], exp_h["n_chunks"], exp_h["uniform_tiles"])
+
+
+def test_roundtrip_with_host_hint(fl):
+    core, torch = fl
+    rng = np.random.default_rng(21)
+    nbytes, chunk = (8 << 20) + 4096 + 7, 256 << 10
+    src_np = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+    sched, exp_t, exp_h = _check_schedule(fl, n_lanes=8, credits=rng.integers(1, 9, size=8), quantum=chunk,
+                                          total_bytes=nbytes, chunk_bytes=chunk)
+    caps = [int(b) for b in exp_h["lane_bytes"][:8]]
+    wins = [torch.zeros(max(c, 1), dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    hint = core.uniform_hint(nbytes, chunk)
+    src = _dev(torch, src_np)
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    core.stripe(src, w, sched, status, hint=hint)
+    core.reassemble(dst, w, sched, status, hint=hint)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    np.testing.assert_array_equal(dst.cpu().numpy(), src_np)
+    exp_w = ob.cpu_stripe(src_np, exp_t, caps)
+    for l in range(8):
+        np.testing.assert_array_equal(wins[l].cpu().numpy()[: caps[l]], exp_w[l][: caps[l]])
