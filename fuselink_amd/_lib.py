@@ -30,7 +30,8 @@ class SchedParams(C.Structure):
                 ("d_src_off", C.c_void_p), ("src_base", C.c_uint64), ("n_chunks", C.c_uint32),
                 ("n_lanes", C.c_uint32), ("d_credits", C.c_void_p), ("n_rows", C.c_uint32),
                 ("epoch_len", C.c_uint32), ("quantum", C.c_uint64), ("tile_bytes", C.c_uint32),
-                ("mode", C.c_uint32), ("d_state", C.c_void_p), ("d_table", C.c_void_p), ("d_hdr", C.c_void_p)]
+                ("mode", C.c_uint32), ("d_state", C.c_void_p), ("d_table", C.c_void_p), ("d_hdr", C.c_void_p),
+                ("inline_credits", C.c_uint32 * MAX_LANES)]
 
 
 class Windows(C.Structure):

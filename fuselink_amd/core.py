@@ -16,6 +16,7 @@ TILE_BYTES = 32768
 UNIT_BYTES = 2 * 1024 * 1024
 SCHED_RESET_OFFSETS = 1
 SCHED_MIRROR = 2
+SCHED_NEW_EPOCH = 4
 SCHED_F_NO_CREDIT = 1
 
 DESC_DTYPE = np.dtype([("src_off", "<u8"), ("win_off", "<u8"), ("len", "<u4"), ("lane", "<u4"),
@@ -91,10 +92,15 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
     shape [rows, n_lanes]; `sizes` a uint32/int32 device tensor of chunk sizes, or None for the
     uniform split of `total_bytes` by `chunk_bytes`."""
     lib = _lib.load()
-    if credits.dim() == 1:
-        credits = credits.view(1, -1)
-    assert credits.is_cuda and credits.dtype in (torch.int32, torch.uint32) and credits.is_contiguous()
-    assert credits.shape[1] == n_lanes
+    inline = None
+    if not isinstance(credits, torch.Tensor):
+        inline = [int(c) for c in credits]  # one row, passed by value in the launch arguments
+        assert len(inline) == n_lanes
+    else:
+        if credits.dim() == 1:
+            credits = credits.view(1, -1)
+        assert credits.is_cuda and credits.dtype in (torch.int32, torch.uint32) and credits.is_contiguous()
+        assert credits.shape[1] == n_lanes
     if sizes is not None:
         assert sizes.is_cuda and sizes.dtype in (torch.int32, torch.uint32) and sizes.is_contiguous()
         n = sizes.numel()
@@ -102,14 +108,18 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
         n = (total_bytes + chunk_bytes - 1) // chunk_bytes if chunk_bytes else 0
     if src_off is not None:
         assert src_off.is_cuda and src_off.dtype in (torch.int64, torch.uint64) and src_off.numel() == n
-    dev = credits.device
+    dev = credits.device if inline is None else torch.device("cuda", torch.cuda.current_device())
     if out is None:
         out = Schedule(_dev_bytes(n * DESC_DTYPE.itemsize, dev), _dev_bytes(HDR_DTYPE.itemsize, dev), n, tile_bytes)
     else:
         assert out.table.numel() >= n * DESC_DTYPE.itemsize
         out.n_chunks, out.tile_bytes = n, tile_bytes
-    p = SchedParams(_ptr(sizes), total_bytes, chunk_bytes, _ptr(src_off), src_base, n, n_lanes, _ptr(credits),
-                    credits.shape[0], epoch_len, quantum, tile_bytes, mode, _ptr(state), _ptr(out.table), _ptr(out.hdr))
+    p = SchedParams(_ptr(sizes), total_bytes, chunk_bytes, _ptr(src_off), src_base, n, n_lanes,
+                    _ptr(credits if inline is None else None), 1 if inline is not None else credits.shape[0], epoch_len,
+                    quantum, tile_bytes, mode, _ptr(state), _ptr(out.table), _ptr(out.hdr))
+    if inline is not None:
+        for l, c in enumerate(inline):
+            p.inline_credits[l] = c
     check(lib.flh_schedule(C.byref(p), _stream_ptr(stream)))
     return out
 

@@ -129,6 +129,7 @@ struct SchedArgs {
   uint32_t mode;
   int32_t quantum_shift;  // >= 0 when quantum is a power of two
   int32_t tile_shift;     // >= 0 when tile_bytes is a power of two
+  uint32_t inline_credits[FLH_MAX_LANES];  // the one credit row when credits == nullptr
 };
 
 // 64-bit division is a long software routine on this ISA and almost every operand here fits 32
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   uint32_t flags = 0;
   if (rows_cached) {
     for (uint32_t r = wave; r < a.n_rows; r += NW) {
-      const uint32_t c = (uint32_t)lane < L ? a.credits[(size_t)r * L + lane] : 0;
+      const uint32_t c = (uint32_t)lane < L ? (a.credits ? a.credits[(size_t)r * L + lane] : a.inline_credits[lane]) : 0;
       uint64_t inc = wave_incl_sum_u64(c, lane);
       const bool zero = bcast_lane_u64(inc, kWave - 1) == 0;
       if (zero) inc = (uint32_t)lane < L ? lane + 1 : L;
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   uint32_t tiles_carry = 0;
   if (a.state) {
     k0 = a.state->chunk_index;
-    p_carry = a.state->epoch_bytes;
+    if (!(a.mode & FLH_SCHED_NEW_EPOCH)) p_carry = a.state->epoch_bytes;
   }
   if (tid < FLH_MAX_LANES) {
     const uint64_t o = (a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS)) ? a.state->lane_off[tid] : 0;
@@ -732,7 +733,8 @@ static int need_init() {
 int flh_schedule(const flh_sched_params* p, void* stream) {
   if (!p) return fl_set_error(FLH_E_ARG, "null params");
   if (p->n_lanes == 0 || p->n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "n_lanes %u not in 1..%d", p->n_lanes, FLH_MAX_LANES);
-  if (p->n_rows == 0 || !p->d_credits) return fl_set_error(FLH_E_ARG, "credit table missing");
+  if (p->n_rows == 0) return fl_set_error(FLH_E_ARG, "credit table missing");
+  if (!p->d_credits && p->n_rows != 1) return fl_set_error(FLH_E_ARG, "inline credits carry exactly one row");
   if (p->quantum == 0) return fl_set_error(FLH_E_ARG, "quantum must be > 0");
   if (p->tile_bytes == 0 || p->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", p->tile_bytes);
   if (!p->d_hdr || (p->n_chunks && !p->d_table)) return fl_set_error(FLH_E_ARG, "output pointers missing");
@@ -761,6 +763,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   a.epoch_len = p->epoch_len;
   a.tile_bytes = p->tile_bytes;
   a.mode = p->mode;
+  for (int l = 0; l < FLH_MAX_LANES; ++l) a.inline_credits[l] = p->inline_credits[l];
   a.quantum_shift = (p->quantum & (p->quantum - 1)) == 0 ? __builtin_ctzll(p->quantum) : -1;
   hipStream_t s = (hipStream_t)stream;
   a.tile_shift = (p->tile_bytes & (p->tile_bytes - 1)) == 0 ? __builtin_ctz(p->tile_bytes) : -1;

@@ -1,0 +1,874 @@
+// fl_plugin.cc -- the ncclNet plugin tables (v8, v7, v6) over an in-process loopback wire.
+//
+// What a request does here, next to what the reference does (FuseLink src/plugin.cc):
+//   irecv  posts a descriptor into the sender's FIFO: address, size, tag, the slot index handshake
+//          idx = tail+1, the lane decision `fuselink_offset`, and -- in the padding the reference
+//          leaves unused -- the receiver's credit row (plugin.cc:1616-1677, 1679-1766).  The lane
+//          decision is refreshed every N_FINISHED_BATCH completions and only when nothing posted is
+//          outstanding (plugin.cc:1700-1716).
+//   isend  matches the FIFO head (plugin.cc:1510-1517), checks sizes (1555-1570), splits the request
+//          over QPs in 128-byte-aligned pieces (1467-1495) and then, instead of posting RDMA writes
+//          out of a remapped buffer, queues on the connection's HIP stream, per wave of chunks:
+//          scheduler kernel -> striping kernel (user buffer -> lane staging windows) -> reassembly
+//          kernel (windows -> the posted receive buffer).  The reassembly launch plays the part of the
+//          RDMA write landing at the receiver; its completion event is the receive completion.
+//   test   polls the request's event (the completion queue of plugin.cc:1801-1955) and, unlike the
+//          reference, reports the byte count of a receive.
+// Staging windows are HIP-VMM mappings from the unit pool, one per lane per connection, bound when
+// device memory is first registered on the send side and reused wave after wave.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <map>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "fl_internal.h"
+#include "fuselink_hip.h"
+#include "fuselink_net.h"
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+// logging and parameters
+// ------------------------------------------------------------------------------------------------
+ncclDebugLogger_t g_log = nullptr;
+#define FL_WARN(...) do { if (g_log) g_log(NCCL_LOG_WARN, NCCL_ALL, __FILE__, __LINE__, __VA_ARGS__); } while (0)
+#define FL_INFO(flags, ...) do { if (g_log) g_log(NCCL_LOG_INFO, (flags), __FILE__, __LINE__, __VA_ARGS__); } while (0)
+
+struct Params {
+  int lanes = 8;                 // virtual NICs = staging lanes (the experiment uses 8 HCAs, run_bw_test.sbatch:43)
+  int priority_dev = 0;          // NCCL_FUSELINK_PRIORITY_DEV, plugin.cc:117
+  int64_t chunk = 512 << 10;     // NCCL_P2P_NET_CHUNKSIZE of the experiment, run_bw_test.sbatch:34
+  int refresh_batch = FL_NET_REFRESH_BATCH;
+  int policy = 1;                // 0 = static lane = channelId % lanes (fuselink.h:235); 1 = credit-weighted
+  int pool_units = FLH_POOL_UNITS;
+  int window_units = 4;          // staging units bound per lane per connection
+  int qps = 1;                   // NCCL_IB_QPS_PER_CONNECTION, plugin.cc:584
+  int split_on_qps = 1;          // NCCL_IB_SPLIT_DATA_ON_QPS, plugin.cc:1410
+  int device = 0;
+  int idle_credit = 4;
+  int max_wave_chunks = 4096;
+};
+Params g_par;
+std::mutex g_init_mu;            // ncclIbLock, plugin.cc:84
+bool g_inited = false;
+
+std::mutex g_credit_mu;
+bool g_credit_override = false;
+uint32_t g_credit_static[FL_NET_MAX_LANES] = {};
+
+std::atomic<int> g_live_links{0};
+flh_pool* g_pool = nullptr;      // staging units of this process's GPU
+std::mutex g_pool_mu;
+
+void parse_credit_env() {
+  const char* v = getenv("NCCL_FUSELINK_CREDITS");
+  if (!v || !*v) return;
+  int n = 0;
+  const char* p = v;
+  while (*p && n < FL_NET_MAX_LANES) {
+    char* end = nullptr;
+    long x = strtol(p, &end, 10);
+    if (end == p) break;
+    g_credit_static[n++] = x < 0 ? 0 : (uint32_t)x;
+    p = *end == ',' ? end + 1 : end;
+  }
+  for (int l = n; l < FL_NET_MAX_LANES; ++l) g_credit_static[l] = 0;
+  g_credit_override = n > 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// objects
+// ------------------------------------------------------------------------------------------------
+enum : int { kReqUnused = 0, kReqSend = 1, kReqRecv = 2, kReqFlush = 3 };  // plugin.cc:462-465
+enum : int { kStPosted = 1, kStLaunched = 2, kStDoneHost = 3 };
+
+struct Link;
+
+struct Request {
+  int type = kReqUnused;
+  std::atomic<int> state{0};
+  Link* link = nullptr;
+  hipEvent_t ev = nullptr;
+  int size = 0;          // bytes moved (reported by test for receives)
+  int fault = 0;         // injected wire fault
+  uint32_t magic = 0;
+};
+constexpr uint32_t kReqMagic = 0x464c5251;   // "FLRQ"
+constexpr uint32_t kCommMagic = 0x464c434d;  // "FLCM"
+constexpr uint32_t kMhMagic = 0x464c4d48;    // "FLMH"
+
+// The descriptor a receiver posts: the reference's ncclIbSendFifo (plugin.cc:487-496), 64 bytes, with
+// the credit row and an epoch flag carried in what is padding there.
+struct FifoWire {
+  uint64_t addr;
+  int32_t size;
+  uint32_t rkey;
+  uint32_t nreqs;
+  uint32_t tag;
+  uint64_t idx;
+  int32_t fuselink_offset;   // >= 0: the whole request goes to this lane; -1: comm's own lane; -2: credit row below
+  uint8_t credits[FL_NET_MAX_LANES];
+  uint32_t flags;            // bit 0: the receiver refreshed its lane decision (new credit epoch)
+  uint8_t pad[8];
+};
+static_assert(sizeof(FifoWire) == 64, "descriptor must stay one 64-byte slot");
+
+struct FifoSlot {
+  FifoWire w;
+  Request* rreq;     // loopback only: the receive request this descriptor belongs to
+  int rtype;         // pointer type of the receive buffer
+};
+
+struct Link {
+  std::mutex mu;
+  int refs = 2;                     // one per side
+  int dev = 0;                      // NIC index the comms were opened on
+  int channelId = 0;                // plugin.cc:693-708
+  int send_ready = 0;               // comm->ready, plugin.cc:1502
+  // sender side
+  FifoSlot fifo[FL_NET_MAX_REQUESTS];
+  uint64_t fifoHead = 0;            // plugin.cc:1510
+  Request sreq[FL_NET_MAX_REQUESTS];
+  int64_t s_finished = 0, s_inflight = 0;
+  // receiver side
+  uint64_t fifoTail = 0;            // plugin.cc:1619
+  Request rreq[FL_NET_MAX_REQUESTS];
+  int64_t r_finished = 0, r_inflight = 0, refreshes = 0;
+  int fuselink_offset = -1;
+  uint8_t credits[FL_NET_MAX_LANES] = {};
+  bool have_decision = false;
+  // GPU side of the connection (created on first use with device memory)
+  bool gpu_ready = false;
+  int hip_device = 0;
+  hipStream_t stream = nullptr;
+  flh_window* win[FL_NET_MAX_LANES] = {};
+  flh_windows wins = {};
+  flh_chunk_desc* d_table = nullptr;
+  flh_sched_hdr* d_hdr = nullptr;
+  flh_sched_state* d_state = nullptr;
+  int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
+  int32_t* d_status = nullptr;
+  uint32_t last_wave_rows = 0;
+};
+
+struct Comm {
+  uint32_t magic = kCommMagic;
+  int is_send = 0;
+  Link* link = nullptr;
+};
+
+struct ListenComm {
+  uint32_t magic = kCommMagic;
+  int dev = 0;
+  int channelId = 0;
+  uint64_t id = 0;
+  std::deque<Link*> pending;   // connects waiting for accept
+};
+
+struct MemHandle {             // FuseLinkMemHandle, fuselink.h:48-52
+  uint32_t magic = kMhMagic;
+  int type = 0;
+  uintptr_t start_addr = 0;
+  size_t size = 0;
+  flh_region* region = nullptr;  // shared per base allocation (device memory only)
+};
+
+struct Handle {                // what listen writes into the caller's 128 bytes (plugin.cc:425-430)
+  uint64_t magic;
+  uint64_t listen_id;
+  int32_t channelId;
+  int32_t dev;
+  int32_t stage;               // 0 start, 1 connect posted (plugin.cc:407-423)
+  int32_t pad;
+  void* stage_link;
+};
+static_assert(sizeof(Handle) < NCCL_NET_HANDLE_MAXSIZE, "handle must fit the caller's buffer");  // plugin.cc:705
+constexpr uint64_t kHandleMagic = 0x4655534c494e4b31ull;
+
+std::mutex g_reg_mu;                        // listen registry + channel counter (plugin.cc:690-698)
+std::map<uint64_t, ListenComm*> g_listens;
+uint64_t g_next_listen = 1;
+int g_channel_counter = 0;
+
+ncclResult_t hip_fail(const char* what, hipError_t e) {
+  FL_WARN("NET/FuseLink : %s failed: %s", what, hipGetErrorString(e));
+  return ncclUnhandledCudaError;   // where the reference exit(1)s (src/checks.h:17-23)
+}
+#define FL_HIPCHECK(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return hip_fail(#call, e_); } while (0)
+#define FL_FLHCHECK(call) do { int rc_ = (call); if (rc_ < 0) { FL_WARN("NET/FuseLink : %s: %s", #call, flh_last_error()); \
+  return rc_ == FLH_E_NOMEM || rc_ == FLH_E_ARG ? ncclInternalError : ncclUnhandledCudaError; } } while (0)
+
+void link_unref(Link* lk) {
+  bool last;
+  {
+    std::lock_guard<std::mutex> g(lk->mu);
+    last = --lk->refs == 0;
+  }
+  if (!last) return;
+  if (lk->gpu_ready) {
+    (void)hipSetDevice(lk->hip_device);
+    (void)hipStreamSynchronize(lk->stream);
+    for (int l = 0; l < FL_NET_MAX_LANES; ++l)
+      if (lk->win[l]) (void)flh_window_destroy(lk->win[l]);
+    (void)hipFree(lk->d_table);
+    (void)hipFree(lk->d_hdr);
+    (void)hipFree(lk->d_state);
+    (void)hipHostFree(lk->h_status);
+    (void)hipStreamDestroy(lk->stream);
+  }
+  for (auto& r : lk->sreq) if (r.ev) (void)hipEventDestroy(r.ev);
+  for (auto& r : lk->rreq) if (r.ev) (void)hipEventDestroy(r.ev);
+  delete lk;
+  g_live_links.fetch_sub(1);
+}
+
+// first free of 256 (ncclIbGetRequest, plugin.cc:1070-1085)
+Request* get_request(Request* tab, Link* lk, int type) {
+  for (int i = 0; i < FL_NET_MAX_REQUESTS; ++i) {
+    Request* r = tab + i;
+    if (r->type == kReqUnused) {
+      r->type = type;
+      r->link = lk;
+      r->size = 0;
+      r->fault = 0;
+      r->magic = kReqMagic;
+      r->state.store(0, std::memory_order_relaxed);
+      return r;
+    }
+  }
+  FL_WARN("NET/FuseLink : unable to allocate requests");
+  return nullptr;
+}
+
+ncclResult_t ensure_pool() {
+  std::lock_guard<std::mutex> g(g_pool_mu);
+  if (g_pool) return ncclSuccess;
+  FL_FLHCHECK(flh_pool_create(g_par.device, (uint32_t)g_par.pool_units, &g_pool));
+  return ncclSuccess;
+}
+
+// Staging side of a connection: stream, one bound window per lane, table / header / state buffers.
+ncclResult_t ensure_link_gpu(Link* lk) {
+  if (lk->gpu_ready) return ncclSuccess;
+  ncclResult_t rc = ensure_pool();
+  if (rc != ncclSuccess) return rc;
+  lk->hip_device = g_par.device;
+  FL_HIPCHECK(hipSetDevice(lk->hip_device));
+  FL_HIPCHECK(hipStreamCreateWithFlags(&lk->stream, hipStreamNonBlocking));
+  const uint64_t cap = (uint64_t)g_par.window_units * FLH_UNIT_BYTES;
+  memset(&lk->wins, 0, sizeof(lk->wins));
+  lk->wins.n_lanes = (uint32_t)g_par.lanes;
+  for (int l = 0; l < g_par.lanes; ++l) {
+    FL_FLHCHECK(flh_window_create(g_pool, cap, &lk->win[l]));
+    FL_FLHCHECK(flh_window_bind(lk->win[l], cap));
+    lk->wins.base[l] = flh_window_base(lk->win[l]);
+    lk->wins.cap[l] = flh_window_bound_bytes(lk->win[l]);
+  }
+  FL_HIPCHECK(hipMalloc((void**)&lk->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
+  FL_HIPCHECK(hipMalloc((void**)&lk->d_hdr, sizeof(flh_sched_hdr)));
+  FL_HIPCHECK(hipMalloc((void**)&lk->d_state, sizeof(flh_sched_state)));
+  FL_HIPCHECK(hipMemsetAsync(lk->d_state, 0, sizeof(flh_sched_state), lk->stream));
+  FL_HIPCHECK(hipHostMalloc((void**)&lk->h_status, sizeof(int32_t), hipHostMallocMapped));
+  *lk->h_status = 0;
+  FL_HIPCHECK(hipHostGetDevicePointer((void**)&lk->d_status, lk->h_status, 0));
+  lk->gpu_ready = true;
+  FL_INFO(NCCL_NET, "NET/FuseLink : channel %d staging ready: %d lanes x %llu bytes", lk->channelId, g_par.lanes, (unsigned long long)cap);
+  return ncclSuccess;
+}
+
+// Credit row the receiver advertises at a refresh.
+void current_credits(int own_lane, uint8_t* out) {
+  uint32_t c[FL_NET_MAX_LANES] = {};
+  {
+    std::lock_guard<std::mutex> g(g_credit_mu);
+    if (g_credit_override) {
+      for (int l = 0; l < g_par.lanes; ++l) c[l] = g_credit_static[l];
+    } else {
+      // the daemon's periodic ageing (monitor.cpp:159-193) happens here, right before the table is read
+      (void)fl_monitor_tick(fl_monitor_now());
+      (void)fl_monitor_credits(g_par.lanes, own_lane, (uint32_t)g_par.idle_credit, c);
+    }
+  }
+  for (int l = 0; l < FL_NET_MAX_LANES; ++l) out[l] = (uint8_t)(c[l] > 255 ? 255 : c[l]);
+}
+
+// Chunks one wave may carry so that no lane can outgrow its window whatever the slot phase is: a lane
+// with credit c sees at most (ceil(n / W) + 1) * c chunks out of n consecutive ones.
+uint32_t wave_chunks(const uint32_t* credits, int lanes, uint64_t chunk, uint64_t cap) {
+  uint64_t W = 0, cmax = 0;
+  for (int l = 0; l < lanes; ++l) { W += credits[l]; if (credits[l] > cmax) cmax = credits[l]; }
+  if (W == 0) { W = (uint64_t)lanes; cmax = 1; }   // no credit anywhere: equal credits stand in
+  const uint64_t per_lane = cap / chunk;           // chunks a window holds
+  if (per_lane == 0) return 0;
+  const uint64_t rounds = per_lane / cmax;         // (ceil(n/W) + 1) <= rounds
+  uint64_t n = rounds >= 2 ? (rounds - 1) * W : 1;
+  if (n > (uint64_t)g_par.max_wave_chunks) n = (uint64_t)g_par.max_wave_chunks;
+  return (uint32_t)n;
+}
+
+// ------------------------------------------------------------------------------------------------
+// plugin entry points (v8 signatures; v7 / v6 adapt)
+// ------------------------------------------------------------------------------------------------
+ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
+  std::lock_guard<std::mutex> g(g_init_mu);
+  g_log = logFunction;
+  if (g_inited) return ncclSuccess;
+  g_par.lanes = (int)fl_param("FUSELINK_LANES", g_par.lanes);
+  g_par.priority_dev = (int)fl_param("FUSELINK_PRIORITY_DEV", g_par.priority_dev);
+  g_par.chunk = fl_param("FUSELINK_CHUNKSIZE", g_par.chunk);
+  g_par.refresh_batch = (int)fl_param("FUSELINK_REFRESH_BATCH", g_par.refresh_batch);
+  g_par.policy = (int)fl_param("FUSELINK_POLICY", g_par.policy);
+  g_par.pool_units = (int)fl_param("FUSELINK_POOL_UNITS", g_par.pool_units);
+  g_par.window_units = (int)fl_param("FUSELINK_WINDOW_UNITS", g_par.window_units);
+  g_par.qps = (int)fl_param("IB_QPS_PER_CONNECTION", g_par.qps);
+  g_par.split_on_qps = (int)fl_param("IB_SPLIT_DATA_ON_QPS", g_par.split_on_qps);
+  g_par.device = (int)fl_param("FUSELINK_DEVICE", g_par.device);
+  g_par.idle_credit = (int)fl_param("FUSELINK_IDLE_CREDIT", g_par.idle_credit);
+  g_par.max_wave_chunks = (int)fl_param("FUSELINK_MAX_WAVE_CHUNKS", g_par.max_wave_chunks);
+  if (g_par.lanes < 1 || g_par.lanes > FL_NET_MAX_LANES) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_LANES must be 1..%d", FL_NET_MAX_LANES); return ncclInvalidArgument; }
+  if (g_par.chunk < 128 || g_par.chunk % 128 || g_par.chunk > (int64_t)1 << 30) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_CHUNKSIZE must be a multiple of 128 up to 1 GiB"); return ncclInvalidArgument; }
+  if (g_par.refresh_batch < 1 || g_par.qps < 1 || g_par.qps > 128 || g_par.window_units < 1 || g_par.pool_units < 1 || g_par.max_wave_chunks < 1) {
+    FL_WARN("NET/FuseLink : parameter out of range");
+    return ncclInvalidArgument;
+  }
+  if ((int64_t)g_par.window_units * FLH_UNIT_BYTES < g_par.chunk) { FL_WARN("NET/FuseLink : a staging window must hold at least one chunk"); return ncclInvalidArgument; }
+  parse_credit_env();
+  g_inited = true;
+  FL_INFO(NCCL_INIT | NCCL_NET, "NET/FuseLink : %d lanes, chunk %lld, policy %s, refresh every %d requests (loopback wire)", g_par.lanes,
+          (long long)g_par.chunk, g_par.policy ? "credits" : "static", g_par.refresh_batch);
+  return ncclSuccess;
+}
+
+ncclResult_t fl_devices(int* ndev) {
+  if (!ndev) return ncclInvalidArgument;
+  *ndev = g_par.lanes;  // one virtual NIC per staging lane
+  return ncclSuccess;
+}
+
+char g_dev_names[FL_NET_MAX_LANES][32];
+
+ncclResult_t fl_get_properties_v8(int dev, ncclNetProperties_v8_t* props) {
+  if (!props || dev < 0 || dev >= g_par.lanes) return ncclInvalidArgument;
+  snprintf(g_dev_names[dev], sizeof(g_dev_names[dev]), "fuselink%d", dev);
+  props->name = g_dev_names[dev];
+  props->pciPath = nullptr;
+  props->guid = (uint64_t)dev;
+  props->ptrSupport = NCCL_PTR_HOST | NCCL_PTR_CUDA;   // plugin.cc:364-370, without DMA-BUF
+  props->regIsGlobal = 1;                              // registrations are keyed by base address, not by comm
+  props->speed = 400000;
+  props->port = 1;
+  props->latency = 0;                                  // plugin.cc:372
+  props->maxComms = 65536;
+  props->maxRecvs = 1;   // the reference advertises 8 (plugin.cc:375) yet rejects grouped receives (plugin.cc:1448-1451)
+  props->netDeviceType = NCCL_NET_DEVICE_HOST;         // plugin.cc:376-377
+  props->netDeviceVersion = NCCL_NET_DEVICE_INVALID_VERSION;
+  return ncclSuccess;
+}
+
+ncclResult_t fl_listen(int dev, void* opaqueHandle, void** listenComm) {
+  if (!opaqueHandle || !listenComm || dev < 0 || dev >= g_par.lanes) return ncclInvalidArgument;
+  ListenComm* lc = new (std::nothrow) ListenComm();
+  if (!lc) return ncclSystemError;
+  Handle* h = (Handle*)opaqueHandle;
+  memset(h, 0, sizeof(Handle));
+  {
+    std::lock_guard<std::mutex> g(g_reg_mu);
+    lc->id = g_next_listen++;
+    lc->channelId = g_channel_counter++;  // ncclIbAllocateChannel, plugin.cc:693-698
+    lc->dev = dev;
+    g_listens[lc->id] = lc;
+  }
+  h->magic = kHandleMagic;
+  h->listen_id = lc->id;
+  h->channelId = lc->channelId;
+  h->dev = dev;
+  *listenComm = lc;
+  FL_INFO(NCCL_INIT | NCCL_NET, "NET/FuseLink : channel id %d listen comm %p dev %d", lc->channelId, (void*)lc, dev);
+  return ncclSuccess;
+}
+
+// Non-blocking, staged like the reference (plugin.cc:407-423, 721-760): the first call posts the
+// connection to the listener and returns NULL; a later call returns the comm once accept() took it.
+ncclResult_t fl_connect(int dev, void* opaqueHandle, void** sendComm, ncclNetDeviceHandle_v8_t** /*sendDevComm*/) {
+  if (!opaqueHandle || !sendComm || dev < 0 || dev >= g_par.lanes) return ncclInvalidArgument;
+  Handle* h = (Handle*)opaqueHandle;
+  *sendComm = nullptr;
+  if (h->magic != kHandleMagic) { FL_WARN("NET/FuseLink : connect with a handle that listen did not produce"); return ncclInternalError; }
+  if (h->stage == 0) {
+    Link* lk = new (std::nothrow) Link();
+    if (!lk) return ncclSystemError;
+    g_live_links.fetch_add(1);
+    lk->dev = dev;
+    lk->channelId = h->channelId;
+    std::lock_guard<std::mutex> g(g_reg_mu);
+    auto it = g_listens.find(h->listen_id);
+    if (it == g_listens.end()) { delete lk; g_live_links.fetch_sub(1); FL_WARN("NET/FuseLink : connect to a closed listen comm"); return ncclSystemError; }
+    it->second->pending.push_back(lk);
+    h->stage = 1;
+    h->stage_link = lk;
+    return ncclSuccess;
+  }
+  Link* lk = (Link*)h->stage_link;
+  {
+    std::lock_guard<std::mutex> g(lk->mu);
+    if (!lk->send_ready) return ncclSuccess;  // accept has not happened yet
+  }
+  Comm* c = new (std::nothrow) Comm();
+  if (!c) return ncclSystemError;
+  c->is_send = 1;
+  c->link = lk;
+  h->stage = 0;
+  h->stage_link = nullptr;
+  *sendComm = c;
+  return ncclSuccess;
+}
+
+ncclResult_t fl_accept(void* listenComm, void** recvComm, ncclNetDeviceHandle_v8_t** /*recvDevComm*/) {
+  if (!listenComm || !recvComm) return ncclInvalidArgument;
+  ListenComm* lc = (ListenComm*)listenComm;
+  *recvComm = nullptr;
+  Link* lk = nullptr;
+  {
+    std::lock_guard<std::mutex> g(g_reg_mu);
+    if (lc->pending.empty()) return ncclSuccess;  // nobody connected yet
+    lk = lc->pending.front();
+    lc->pending.pop_front();
+  }
+  Comm* c = new (std::nothrow) Comm();
+  if (!c) return ncclSystemError;
+  c->is_send = 0;
+  c->link = lk;
+  {
+    std::lock_guard<std::mutex> g(lk->mu);
+    lk->send_ready = 1;
+  }
+  *recvComm = c;
+  return ncclSuccess;
+}
+
+ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uint64_t /*offset*/, int /*fd*/, void** mhandle) {
+  if (!comm || !data || !mhandle || size == 0) return ncclInvalidArgument;
+  Comm* c = (Comm*)comm;
+  if (c->magic != kCommMagic) return ncclInvalidArgument;
+  *mhandle = nullptr;
+  MemHandle* mh = new (std::nothrow) MemHandle();
+  if (!mh) return ncclSystemError;
+  mh->type = type;
+  if (type == NCCL_PTR_CUDA) {
+    // whole allocation around the pointer, as cuMemGetAddressRange in plugin.cc:1194
+    FL_HIPCHECK(hipSetDevice(g_par.device));
+    void* base = nullptr;
+    size_t bsz = 0;
+    hipError_t e = hipMemGetAddressRange((hipDeviceptr_t*)&base, &bsz, (hipDeviceptr_t)data);
+    if (e != hipSuccess) { delete mh; return hip_fail("hipMemGetAddressRange", e); }
+    ncclResult_t rc = ensure_pool();
+    if (rc != ncclSuccess) { delete mh; return rc; }
+    // one shared, reference-counted region per base allocation (plugin.cc:1212-1227, 1326)
+    int frc = flh_region_acquire(g_pool, base, bsz, 0, 0, &mh->region);
+    if (frc < 0) { delete mh; FL_WARN("NET/FuseLink : region: %s", flh_last_error()); return ncclInternalError; }
+    mh->start_addr = (uintptr_t)base;
+    mh->size = bsz;
+    if (c->is_send) {  // staging is bound at registration time, not on the request path
+      std::lock_guard<std::mutex> g(c->link->mu);
+      rc = ensure_link_gpu(c->link);
+      if (rc != ncclSuccess) { (void)flh_region_release(mh->region); delete mh; return rc; }
+    }
+  } else if (type == NCCL_PTR_HOST) {
+    // page-aligned span, plugin.cc:1181-1182, 1206-1209; host memory is not staged
+    const uintptr_t page = 4096;
+    const uintptr_t addr = (uintptr_t)data & ~(page - 1);
+    const size_t pages = ((uintptr_t)data + size - addr + page - 1) / page;
+    mh->start_addr = addr;
+    mh->size = pages * page;
+  } else {
+    delete mh;
+    FL_WARN("NET/FuseLink : unsupported pointer type %d", type);
+    return ncclInvalidArgument;
+  }
+  *mhandle = mh;
+  return ncclSuccess;
+}
+
+ncclResult_t fl_reg_mr_v8(void* comm, void* data, size_t size, int type, void** mhandle) {
+  return fl_reg_mr_dmabuf(comm, data, size, type, 0ull, -1, mhandle);  // plugin.cc:1332-1335
+}
+
+ncclResult_t fl_dereg_mr(void* /*comm*/, void* mhandle) {
+  MemHandle* mh = (MemHandle*)mhandle;
+  if (!mh || mh->magic != kMhMagic) return ncclInvalidArgument;
+  if (mh->region) {
+    int left = flh_region_release(mh->region);  // destroyed on the last reference, plugin.cc:1347-1403
+    if (left < 0) { FL_WARN("NET/FuseLink : region release: %s", flh_last_error()); return ncclInternalError; }
+  }
+  mh->magic = 0;
+  delete mh;
+  return ncclSuccess;
+}
+
+bool in_handle(const MemHandle* mh, const void* p, size_t n) {
+  const uintptr_t a = (uintptr_t)p;
+  return a >= mh->start_addr && a + n <= mh->start_addr + mh->size;
+}
+
+// Queue the GPU work of one matched send on the connection's stream.
+ncclResult_t launch_transfer(Link* lk, const uint8_t* src, uint8_t* dst, int size, const FifoWire& w, Request* sreq, Request* rreq) {
+  FL_HIPCHECK(hipSetDevice(lk->hip_device));
+  uint32_t credits[FLH_MAX_LANES] = {};
+  const int lanes = g_par.lanes;
+  if (w.fuselink_offset == -2) {
+    for (int l = 0; l < lanes; ++l) credits[l] = w.credits[l];
+  } else {
+    // the receiver named one lane (fuselink.h:235-237); -1 means the comm's own NIC (plugin.cc:1539-1540)
+    const int lane = w.fuselink_offset >= 0 ? w.fuselink_offset % lanes : lk->dev % lanes;
+    credits[lane] = 1;
+  }
+  const uint64_t chunk = (uint64_t)g_par.chunk;
+  const uint32_t per_wave = wave_chunks(credits, lanes, chunk, lk->wins.cap[0]);
+  if (per_wave == 0) { FL_WARN("NET/FuseLink : staging window smaller than a chunk"); return ncclInternalError; }
+  // request -> QP pieces (plugin.cc:1467-1495), each piece -> waves of chunks
+  const int nqps = g_par.split_on_qps ? g_par.qps : 1;
+  std::vector<int> qoff(nqps), qlen(nqps);
+  if (flh_qp_split(size, nqps, qoff.data(), qlen.data()) < 0) return ncclInternalError;
+  bool first = true;
+  for (int q = 0; q < nqps; ++q) {
+    uint64_t done = 0;
+    const uint64_t piece = (uint64_t)qlen[q];
+    while (done < piece) {
+      uint64_t wave = (uint64_t)per_wave * chunk;
+      if (wave > piece - done) wave = piece - done;
+      flh_sched_params p;
+      memset(&p, 0, sizeof(p));
+      p.total_bytes = wave;
+      p.chunk_bytes = (uint32_t)chunk;
+      p.src_base = (uint64_t)qoff[q] + done;
+      p.n_chunks = (uint32_t)((wave + chunk - 1) / chunk);
+      p.n_lanes = (uint32_t)lanes;
+      p.n_rows = 1;
+      p.quantum = chunk;
+      p.tile_bytes = FLH_TILE_BYTES;
+      p.mode = FLH_SCHED_RESET_OFFSETS | ((first && (w.flags & 1u)) ? FLH_SCHED_NEW_EPOCH : 0u);
+      p.d_state = lk->d_state;
+      p.d_table = lk->d_table;
+      p.d_hdr = lk->d_hdr;
+      for (int l = 0; l < lanes; ++l) p.inline_credits[l] = credits[l];
+      FL_FLHCHECK(flh_schedule(&p, lk->stream));
+      FL_FLHCHECK(flh_stripe(src, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, nullptr, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
+      FL_FLHCHECK(flh_reassemble(dst, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, nullptr, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
+      lk->last_wave_rows = p.n_chunks;
+      done += wave;
+      first = false;
+    }
+  }
+  FL_HIPCHECK(hipEventRecord(sreq->ev, lk->stream));
+  FL_HIPCHECK(hipEventRecord(rreq->ev, lk->stream));
+  return ncclSuccess;
+}
+
+ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhandle, void** request) {
+  if (!sendComm || !request || !mhandle || size < 0 || (size && !data)) return ncclInvalidArgument;
+  Comm* c = (Comm*)sendComm;
+  MemHandle* mh = (MemHandle*)mhandle;
+  if (c->magic != kCommMagic || !c->is_send || mh->magic != kMhMagic) return ncclInvalidArgument;
+  Link* lk = c->link;
+  *request = nullptr;
+  std::lock_guard<std::mutex> g(lk->mu);
+  if (!lk->send_ready) { FL_WARN("NET/FuseLink: isend() called when comm->ready == 0"); return ncclInternalError; }  // plugin.cc:1502
+  // wait for the receiver to have posted the matching receive (plugin.cc:1510-1514)
+  const int slot = (int)(lk->fifoHead % FL_NET_MAX_REQUESTS);
+  FifoSlot& fs = lk->fifo[slot];
+  if (fs.w.idx != lk->fifoHead + 1) return ncclSuccess;
+  if (fs.w.nreqs != 1) { FL_WARN("NET/FuseLink: multi-send not allowed"); return ncclInternalError; }   // plugin.cc:1448-1451
+  if (fs.w.tag != (uint32_t)tag) return ncclSuccess;                                                     // plugin.cc:1552
+  if (size > fs.w.size) {                                                                                // plugin.cc:1555-1562
+    FL_WARN("NET/FuseLink : req tag %x collective mismatch error, local size %d remote size %d", tag, size, fs.w.size);
+    return ncclInvalidUsage;
+  }
+  if (fs.w.size < 0 || fs.w.addr == 0) {                                                                 // plugin.cc:1563-1570
+    FL_WARN("NET/FuseLink : posted incorrect receive info: size %d addr %llx", fs.w.size, (unsigned long long)fs.w.addr);
+    return ncclInternalError;
+  }
+  if (size && !in_handle(mh, data, (size_t)size)) { FL_WARN("NET/FuseLink : send buffer outside its registration"); return ncclInvalidArgument; }
+  Request* sreq = get_request(lk->sreq, lk, kReqSend);
+  if (!sreq) return ncclInternalError;                                                                   // plugin.cc:1082-1084
+  Request* rreq = fs.rreq;
+  sreq->size = size;
+  rreq->size = size;
+  uint8_t* dst = (uint8_t*)(uintptr_t)fs.w.addr;
+  ncclResult_t rc = ncclSuccess;
+  const bool src_dev = mh->type == NCCL_PTR_CUDA, dst_dev = fs.rtype == NCCL_PTR_CUDA;
+  if (size == 0) {
+    sreq->state.store(kStDoneHost, std::memory_order_release);
+    rreq->state.store(kStDoneHost, std::memory_order_release);
+  } else if (!src_dev && !dst_dev) {
+    memcpy(dst, data, (size_t)size);  // host memory is not staged (fuselink.cc:8-13): the wire is a copy
+    sreq->state.store(kStDoneHost, std::memory_order_release);
+    rreq->state.store(kStDoneHost, std::memory_order_release);
+  } else {
+    rc = ensure_link_gpu(lk);
+    if (rc == ncclSuccess && !sreq->ev) { hipError_t e = hipEventCreateWithFlags(&sreq->ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
+    if (rc == ncclSuccess && !rreq->ev) { hipError_t e = hipEventCreateWithFlags(&rreq->ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
+    if (rc == ncclSuccess) {
+      if (src_dev && dst_dev) {
+        rc = launch_transfer(lk, (const uint8_t*)data, dst, size, fs.w, sreq, rreq);
+      } else {
+        // one side is host memory: the copy engine is the wire, nothing is striped
+        hipError_t e = hipMemcpyAsync(dst, data, (size_t)size, hipMemcpyDefault, lk->stream);
+        if (e == hipSuccess) e = hipEventRecord(sreq->ev, lk->stream);
+        if (e == hipSuccess) e = hipEventRecord(rreq->ev, lk->stream);
+        if (e != hipSuccess) rc = hip_fail("hipMemcpyAsync", e);
+      }
+    }
+    if (rc != ncclSuccess) {
+      sreq->type = kReqUnused;
+      return rc;
+    }
+    sreq->state.store(kStLaunched, std::memory_order_release);
+    rreq->state.store(kStLaunched, std::memory_order_release);
+  }
+  // the comm's own NIC carried traffic (updateTxChannelActive, fuselink.h:247-252)
+  (void)fl_monitor_mark_active(lk->dev % g_par.lanes, 1, fl_monitor_now());
+  memset((void*)&fs.w, 0, sizeof(FifoWire));   // plugin.cc:1605
+  fs.rreq = nullptr;
+  lk->fifoHead++;                              // plugin.cc:1607
+  lk->s_inflight++;
+  *request = sreq;
+  return ncclSuccess;
+}
+
+ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags, void** mhandles, void** request) {
+  if (!recvComm || !request || !data || !sizes || !tags || !mhandles) return ncclInvalidArgument;
+  Comm* c = (Comm*)recvComm;
+  if (c->magic != kCommMagic || c->is_send) return ncclInvalidArgument;
+  *request = nullptr;
+  if (n > FL_NET_MAX_RECVS) return ncclInternalError;                       // plugin.cc:1683
+  if (n != 1) { FL_WARN("NET/FuseLink: multi recv not allowed"); return ncclInternalError; }  // plugin.cc:1873-1880
+  MemHandle* mh = (MemHandle*)mhandles[0];
+  if (!mh || mh->magic != kMhMagic || sizes[0] < 0 || !data[0]) return ncclInvalidArgument;
+  if (sizes[0] && !in_handle(mh, data[0], (size_t)sizes[0])) { FL_WARN("NET/FuseLink : receive buffer outside its registration"); return ncclInvalidArgument; }
+  Link* lk = c->link;
+  std::lock_guard<std::mutex> g(lk->mu);
+  bool refreshed = false;
+  if (lk->r_finished % g_par.refresh_batch == 0 || !lk->have_decision) {   // plugin.cc:1700
+    // only when everything received so far has been consumed (plugin.cc:1704-1709)
+    if (lk->r_inflight != 0) return ncclSuccess;
+    if (g_par.policy == 0) {
+      lk->fuselink_offset = lk->channelId % g_par.lanes;                     // refreshRxComm, fuselink.h:235-237
+    } else {
+      lk->fuselink_offset = -2;
+      current_credits(lk->dev % g_par.lanes, lk->credits);
+    }
+    lk->have_decision = true;
+    lk->refreshes++;
+    refreshed = true;
+  }
+  Request* rreq = get_request(lk->rreq, lk, kReqRecv);
+  if (!rreq) return ncclInternalError;                                         // plugin.cc:1082-1084
+  if (lk->fifoTail - lk->fifoHead >= FL_NET_MAX_REQUESTS) { rreq->type = kReqUnused; return ncclSuccess; }  // descriptor ring full
+  rreq->state.store(kStPosted, std::memory_order_relaxed);
+  // ncclIbPostFifo, plugin.cc:1616-1677
+  const int slot = (int)(lk->fifoTail % FL_NET_MAX_REQUESTS);
+  FifoSlot& fs = lk->fifo[slot];
+  fs.w.addr = (uint64_t)(uintptr_t)data[0];
+  fs.w.size = sizes[0];
+  fs.w.rkey = 1;
+  fs.w.nreqs = (uint32_t)n;
+  fs.w.tag = (uint32_t)tags[0];
+  fs.w.fuselink_offset = lk->fuselink_offset;
+  memcpy(fs.w.credits, lk->credits, sizeof(fs.w.credits));
+  fs.w.flags = refreshed ? 1u : 0u;
+  fs.rreq = rreq;
+  fs.rtype = mh->type;
+  fs.w.idx = lk->fifoTail + 1;   // written last: it is what the sender waits for (plugin.cc:1632)
+  lk->fifoTail++;
+  lk->r_inflight++;
+  *request = rreq;
+  return ncclSuccess;
+}
+
+ncclResult_t fl_iflush(void* recvComm, int /*n*/, void** /*data*/, int* /*sizes*/, void** /*mhandles*/, void** request) {
+  // A receive completes only after its reassembly kernel has finished on the GPU that owns the
+  // buffer, so there is nothing left to flush; the reference too returns without a request when
+  // its flush is disabled, the default (plugin.cc:887, 1772).
+  if (!recvComm || !request) return ncclInvalidArgument;
+  *request = nullptr;
+  return ncclSuccess;
+}
+
+ncclResult_t fl_test(void* request, int* done, int* sizes) {
+  if (!request || !done) return ncclInvalidArgument;
+  Request* r = (Request*)request;
+  if (r->magic != kReqMagic || r->type == kReqUnused) { FL_WARN("NET/FuseLink : test on a request that is not in flight"); return ncclInternalError; }
+  *done = 0;
+  Link* lk = r->link;
+  std::lock_guard<std::mutex> g(lk->mu);
+  const int st = r->state.load(std::memory_order_acquire);
+  if (st == kStPosted || st == 0) return ncclSuccess;   // a receive whose send has not been matched yet
+  if (st == kStLaunched) {
+    hipError_t e = hipEventQuery(r->ev);
+    if (e == hipErrorNotReady) return ncclSuccess;
+    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+    if (lk->h_status && *lk->h_status != 0) {
+      FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", *lk->h_status);
+      return ncclInternalError;
+    }
+  }
+  if (r->fault) {   // failed completion, plugin.cc:1839-1861
+    FL_WARN("NET/FuseLink : Got completion with error (injected), channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
+    return ncclRemoteError;
+  }
+  *done = 1;                                                // plugin.cc:1807-1823
+  if (r->type == kReqSend) { lk->s_finished++; lk->s_inflight--; }
+  if (r->type == kReqRecv) {
+    lk->r_finished++;
+    lk->r_inflight--;
+    if (sizes) sizes[0] = r->size;   // the reference leaves 0 here (plugin.cc:1726, 1882)
+  }
+  r->type = kReqUnused;                                     // ncclIbFreeRequest, plugin.cc:1086-1090
+  return ncclSuccess;
+}
+
+ncclResult_t close_comm(void* comm, int want_send) {
+  Comm* c = (Comm*)comm;
+  if (!c) return ncclSuccess;
+  if (c->magic != kCommMagic || c->is_send != want_send) return ncclInvalidArgument;
+  Link* lk = c->link;
+  c->magic = 0;
+  delete c;
+  link_unref(lk);
+  return ncclSuccess;
+}
+ncclResult_t fl_close_send(void* sendComm) { return close_comm(sendComm, 1); }
+ncclResult_t fl_close_recv(void* recvComm) { return close_comm(recvComm, 0); }
+
+ncclResult_t fl_close_listen(void* listenComm) {
+  ListenComm* lc = (ListenComm*)listenComm;
+  if (!lc) return ncclSuccess;
+  std::vector<Link*> orphans;
+  {
+    std::lock_guard<std::mutex> g(g_reg_mu);
+    g_listens.erase(lc->id);
+    orphans.assign(lc->pending.begin(), lc->pending.end());
+  }
+  for (Link* lk : orphans) {   // connects nobody will accept: drop the listener's share of them
+    link_unref(lk);
+  }
+  delete lc;
+  return ncclSuccess;
+}
+
+// ---- v7 / v6 adapters ---------------------------------------------------------------------------------
+ncclResult_t fl_get_properties_v7(int dev, ncclNetProperties_v7_t* p) {
+  ncclNetProperties_v8_t q;
+  ncclResult_t rc = fl_get_properties_v8(dev, &q);
+  if (rc != ncclSuccess || !p) return rc != ncclSuccess ? rc : ncclInvalidArgument;
+  p->name = q.name; p->pciPath = q.pciPath; p->guid = q.guid; p->ptrSupport = q.ptrSupport; p->speed = q.speed; p->port = q.port;
+  p->latency = q.latency; p->maxComms = q.maxComms; p->maxRecvs = q.maxRecvs; p->netDeviceType = q.netDeviceType;
+  p->netDeviceVersion = q.netDeviceVersion;
+  return ncclSuccess;
+}
+ncclResult_t fl_get_properties_v6(int dev, ncclNetProperties_v6_t* p) {
+  ncclNetProperties_v8_t q;
+  ncclResult_t rc = fl_get_properties_v8(dev, &q);
+  if (rc != ncclSuccess || !p) return rc != ncclSuccess ? rc : ncclInvalidArgument;
+  p->name = q.name; p->pciPath = q.pciPath; p->guid = q.guid; p->ptrSupport = q.ptrSupport; p->speed = q.speed; p->port = q.port;
+  p->latency = q.latency; p->maxComms = q.maxComms; p->maxRecvs = q.maxRecvs;
+  return ncclSuccess;
+}
+ncclResult_t fl_reg_mr_v7(void* comm, void* data, int size, int type, void** mhandle) {
+  if (size <= 0) return ncclInvalidArgument;
+  return fl_reg_mr_dmabuf(comm, data, (size_t)size, type, 0ull, -1, mhandle);
+}
+ncclResult_t fl_connect_v7(int dev, void* handle, void** sendComm, ncclNetDeviceHandle_v7_t** d) { return fl_connect(dev, handle, sendComm, d); }
+ncclResult_t fl_accept_v7(void* listenComm, void** recvComm, ncclNetDeviceHandle_v7_t** d) { return fl_accept(listenComm, recvComm, d); }
+ncclResult_t fl_connect_v6(int dev, void* handle, void** sendComm) { return fl_connect(dev, handle, sendComm, nullptr); }
+ncclResult_t fl_accept_v6(void* listenComm, void** recvComm) { return fl_accept(listenComm, recvComm, nullptr); }
+
+}  // namespace
+
+extern "C" {
+
+__attribute__((visibility("default"))) ncclNet_v8_t ncclNetPlugin_v8 = {
+    "FuseLink", fl_init, fl_devices, fl_get_properties_v8, fl_listen, fl_connect, fl_accept, fl_reg_mr_v8, fl_reg_mr_dmabuf,
+    fl_dereg_mr, fl_isend, fl_irecv, fl_iflush, fl_test, fl_close_send, fl_close_recv, fl_close_listen,
+    nullptr /* getDeviceMr */, nullptr /* irecvConsumed */};
+
+__attribute__((visibility("default"))) ncclNet_v7_t ncclNetPlugin_v7 = {
+    "FuseLink", fl_init, fl_devices, fl_get_properties_v7, fl_listen, fl_connect_v7, fl_accept_v7, fl_reg_mr_v7, fl_reg_mr_dmabuf,
+    fl_dereg_mr, fl_isend, fl_irecv, fl_iflush, fl_test, fl_close_send, fl_close_recv, fl_close_listen,
+    nullptr /* getDeviceMr */, nullptr /* irecvConsumed */};
+
+__attribute__((visibility("default"))) ncclNet_v6_t ncclNetPlugin_v6 = {
+    "FuseLink", fl_init, fl_devices, fl_get_properties_v6, fl_listen, fl_connect_v6, fl_accept_v6, fl_reg_mr_v7, fl_reg_mr_dmabuf,
+    fl_dereg_mr, fl_isend, fl_irecv, fl_iflush, fl_test, fl_close_send, fl_close_recv, fl_close_listen};
+
+int fl_net_set_credits(const uint32_t* credits, int n) {
+  if (n < 0 || n > FL_NET_MAX_LANES || (n && !credits)) return fl_set_error(FLH_E_ARG, "bad credit row");
+  std::lock_guard<std::mutex> g(g_credit_mu);
+  g_credit_override = n > 0;
+  for (int l = 0; l < FL_NET_MAX_LANES; ++l) g_credit_static[l] = l < n ? credits[l] : 0;
+  return FLH_OK;
+}
+
+int fl_net_reset(void) {
+  std::lock_guard<std::mutex> gi(g_init_mu);
+  {
+    std::lock_guard<std::mutex> g(g_reg_mu);
+    if (!g_listens.empty() || g_live_links.load() != 0) return fl_set_error(FLH_E_STATE, "connections are still open");
+  }
+  {
+    std::lock_guard<std::mutex> g(g_pool_mu);
+    if (g_pool) {
+      int rc = flh_pool_destroy(g_pool);
+      if (rc < 0) return rc;
+      g_pool = nullptr;
+    }
+  }
+  g_par = Params();
+  g_inited = false;
+  return FLH_OK;
+}
+
+int fl_net_inject_fault(void* request) {
+  Request* r = (Request*)request;
+  if (!r || r->magic != kReqMagic || r->type == kReqUnused) return fl_set_error(FLH_E_ARG, "not a request in flight");
+  std::lock_guard<std::mutex> g(r->link->mu);
+  r->fault = 1;
+  return FLH_OK;
+}
+
+int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64_t* refreshes) {
+  Comm* c = (Comm*)comm;
+  if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
+  Link* lk = c->link;
+  std::lock_guard<std::mutex> g(lk->mu);
+  if (n_finished) *n_finished = c->is_send ? lk->s_finished : lk->r_finished;
+  if (in_flight) *in_flight = c->is_send ? lk->s_inflight : lk->r_inflight;
+  if (refreshes) *refreshes = lk->refreshes;
+  return FLH_OK;
+}
+
+int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_out) {
+  Comm* c = (Comm*)sendComm;
+  if (!c || c->magic != kCommMagic || !c->is_send) return fl_set_error(FLH_E_ARG, "not a send comm");
+  Link* lk = c->link;
+  std::lock_guard<std::mutex> g(lk->mu);
+  if (!lk->gpu_ready) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
+  if (hipSetDevice(lk->hip_device) != hipSuccess || hipStreamSynchronize(lk->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
+  int rows = (int)lk->last_wave_rows;
+  int take = rows < max_rows ? rows : max_rows;
+  if (take > 0 && rows_out && hipMemcpy(rows_out, lk->d_table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
+    return fl_set_error(FLH_E_HIP, "table copy failed");
+  if (hdr_out && hipMemcpy(hdr_out, lk->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
+    return fl_set_error(FLH_E_HIP, "header copy failed");
+  return rows;
+}
+
+}  // extern "C"

@@ -246,7 +246,7 @@ int flh_region_acquire(flh_pool* pool, void* base, uint64_t bytes, uint32_t n_la
   if (!pool || !base || !out) return fl_set_error(FLH_E_ARG, "null argument");
   *out = nullptr;
   if (bytes == 0) return fl_set_error(FLH_E_ARG, "bytes must be > 0");
-  if (n_lanes == 0 || n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "n_lanes %u not in 1..%d", n_lanes, FLH_MAX_LANES);
+  if (n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "n_lanes %u not in 0..%d", n_lanes, FLH_MAX_LANES);
   std::lock_guard<std::mutex> g(g_region_mu);
   auto it = g_regions.find(base);
   if (it != g_regions.end()) {  // src/plugin.cc:1214-1226: share the region, count the handle

@@ -70,6 +70,7 @@ typedef struct flh_sched_hdr {
 
 /* flh_sched_params.mode */
 #define FLH_SCHED_RESET_OFFSETS 1u     /* start every lane at window offset 0 instead of the state's */
+#define FLH_SCHED_NEW_EPOCH     4u     /* start with zero epoch bytes instead of the state's (credits were refreshed) */
 #define FLH_SCHED_MIRROR        2u     /* win_off = src_off: each window mirrors the user buffer, the
                                           reference's translation window + (data - start_addr)
                                           (src/plugin.cc:1582, 1626); windows must be bound that far */
@@ -82,7 +83,7 @@ typedef struct flh_sched_params {
   uint64_t src_base;
   uint32_t n_chunks;
   uint32_t n_lanes;            /* 1..16 */
-  const uint32_t* d_credits;   /* n_rows x n_lanes credit table */
+  const uint32_t* d_credits;   /* n_rows x n_lanes credit table; NULL = the single row in inline_credits */
   uint32_t n_rows;             /* >= 1; epoch e reads row e mod n_rows */
   uint32_t epoch_len;          /* chunks per credit epoch; 0 = a single epoch */
   uint64_t quantum;            /* bytes per credit (the nominal chunk size) */
@@ -91,6 +92,7 @@ typedef struct flh_sched_params {
   flh_sched_state* d_state;    /* in/out, or NULL to start from zero and discard */
   flh_chunk_desc* d_table;     /* out: n_chunks rows */
   flh_sched_hdr* d_hdr;        /* out */
+  uint32_t inline_credits[FLH_MAX_LANES]; /* one credit row passed by value (used when d_credits == NULL) */
 } flh_sched_params;
 
 /* ---- library ------------------------------------------------------------------------------ */
@@ -198,6 +200,7 @@ int flh_window_slots(const flh_window* w, int* slots, int max);
  * staging window per lane.  flh_region_translate is the reference's pointer translation
  * window_base + (data - start_addr) (src/plugin.cc:1582, 1626). */
 typedef struct flh_region flh_region;
+/* n_lanes may be 0: the region then only keeps the registration (base, size, reference count). */
 int flh_region_acquire(flh_pool* pool, void* base, uint64_t bytes, uint32_t n_lanes,
                        uint64_t bound_bytes_per_lane, flh_region** out);
 int flh_region_release(flh_region* r);            /* returns remaining refs (>= 0) or an error */

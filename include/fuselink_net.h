@@ -1,0 +1,231 @@
+/*
+ * fuselink_net.h -- the NCCL/RCCL network-plugin ABI exported by libnccl-net-fuselink.so.
+ *
+ * Self-contained restatement of the ext-net structures (no nccl.h needed).  The reference exports
+ * `ncclNetPlugin_v7` and aliases `ncclNetPlugin_v6` to it (FuseLink src/plugin.cc:1997-2018; struct
+ * definitions in src/extern/nccl_net.h:24-98 for v7 and :104-163 for v6).  This library exports
+ *     ncclNetPlugin_v8   (primary: what RCCL 2.2x probes first among the versions carried here)
+ *     ncclNetPlugin_v7   (the reference's own version)
+ *     ncclNetPlugin_v6   (a real v6 table; the reference's alias relies on the v7 and v6 layouts
+ *                         agreeing in their leading slots)
+ * v8 differs from v7 in two places only: regMr takes `size_t size` instead of `int size`, and the
+ * properties struct gains `int regIsGlobal` after ptrSupport.
+ *
+ * Calling convention (src/extern/nccl_net.h:53-83): every entry returns ncclResult_t; "would block"
+ * is ncclSuccess with *sendComm / *recvComm / *request left NULL and the call is repeated.
+ */
+#ifndef FUSELINK_NET_H_
+#define FUSELINK_NET_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- result codes (values of rccl.h / nccl.h) ---------------------------------------------- */
+#ifndef NCCL_H_
+typedef enum {
+  ncclSuccess = 0,
+  ncclUnhandledCudaError = 1,
+  ncclSystemError = 2,
+  ncclInternalError = 3,
+  ncclInvalidArgument = 4,
+  ncclInvalidUsage = 5,
+  ncclRemoteError = 6,
+  ncclInProgress = 7,
+  ncclNumResults = 8
+} ncclResult_t;
+#endif
+
+/* ---- logging (nccl_common.h of NCCL 2.19) -------------------------------------------------- */
+typedef enum { NCCL_LOG_NONE = 0, NCCL_LOG_VERSION = 1, NCCL_LOG_WARN = 2, NCCL_LOG_INFO = 3, NCCL_LOG_ABORT = 4, NCCL_LOG_TRACE = 5 } ncclDebugLogLevel;
+typedef enum {
+  NCCL_INIT = 1, NCCL_COLL = 2, NCCL_P2P = 4, NCCL_SHM = 8, NCCL_NET = 16, NCCL_GRAPH = 32, NCCL_TUNING = 64,
+  NCCL_ENV = 128, NCCL_ALLOC = 256, NCCL_CALL = 512, NCCL_PROXY = 1024, NCCL_NVLS = 2048, NCCL_ALL = ~0
+} ncclDebugLogSubSys;
+typedef void (*ncclDebugLogger_t)(ncclDebugLogLevel level, unsigned long flags, const char* file, int line, const char* fmt, ...);
+
+/* ---- constants (src/extern/nccl_net.h:15-22) ----------------------------------------------- */
+#define NCCL_NET_HANDLE_MAXSIZE 128
+#define NCCL_PTR_HOST 0x1
+#define NCCL_PTR_CUDA 0x2
+#define NCCL_PTR_DMABUF 0x4
+#define NCCL_NET_MAX_REQUESTS 32
+
+/* ---- device offload descriptors (net_device.h) ---------------------------------------------- */
+typedef enum { NCCL_NET_DEVICE_HOST = 0, NCCL_NET_DEVICE_UNPACK = 1 } ncclNetDeviceType;
+#define NCCL_NET_DEVICE_INVALID_VERSION 0x0
+typedef struct {
+  ncclNetDeviceType netDeviceType;
+  int netDeviceVersion;
+  void* handle;
+  size_t size;
+  int needsProxyProgress;
+} ncclNetDeviceHandle_v7_t;
+typedef ncclNetDeviceHandle_v7_t ncclNetDeviceHandle_v8_t;
+
+/* ---- properties ------------------------------------------------------------------------------- */
+typedef struct {  /* src/extern/nccl_net.h:105-116 */
+  char* name;
+  char* pciPath;
+  uint64_t guid;
+  int ptrSupport;
+  int speed;
+  int port;
+  float latency;
+  int maxComms;
+  int maxRecvs;
+} ncclNetProperties_v6_t;
+
+typedef struct {  /* src/extern/nccl_net.h:24-37 */
+  char* name;
+  char* pciPath;
+  uint64_t guid;
+  int ptrSupport;
+  int speed;
+  int port;
+  float latency;
+  int maxComms;
+  int maxRecvs;
+  ncclNetDeviceType netDeviceType;
+  int netDeviceVersion;
+} ncclNetProperties_v7_t;
+
+typedef struct {
+  char* name;
+  char* pciPath;
+  uint64_t guid;
+  int ptrSupport;
+  int regIsGlobal;  /* regMr is not tied to a particular comm */
+  int speed;
+  int port;
+  float latency;
+  int maxComms;
+  int maxRecvs;
+  ncclNetDeviceType netDeviceType;
+  int netDeviceVersion;
+} ncclNetProperties_v8_t;
+
+/* ---- function tables ------------------------------------------------------------------------- */
+typedef struct {  /* src/extern/nccl_net.h:118-163 */
+  const char* name;
+  ncclResult_t (*init)(ncclDebugLogger_t logFunction);
+  ncclResult_t (*devices)(int* ndev);
+  ncclResult_t (*getProperties)(int dev, ncclNetProperties_v6_t* props);
+  ncclResult_t (*listen)(int dev, void* handle, void** listenComm);
+  ncclResult_t (*connect)(int dev, void* handle, void** sendComm);
+  ncclResult_t (*accept)(void* listenComm, void** recvComm);
+  ncclResult_t (*regMr)(void* comm, void* data, int size, int type, void** mhandle);
+  ncclResult_t (*regMrDmaBuf)(void* comm, void* data, size_t size, int type, uint64_t offset, int fd, void** mhandle);
+  ncclResult_t (*deregMr)(void* comm, void* mhandle);
+  ncclResult_t (*isend)(void* sendComm, void* data, int size, int tag, void* mhandle, void** request);
+  ncclResult_t (*irecv)(void* recvComm, int n, void** data, int* sizes, int* tags, void** mhandles, void** request);
+  ncclResult_t (*iflush)(void* recvComm, int n, void** data, int* sizes, void** mhandles, void** request);
+  ncclResult_t (*test)(void* request, int* done, int* sizes);
+  ncclResult_t (*closeSend)(void* sendComm);
+  ncclResult_t (*closeRecv)(void* recvComm);
+  ncclResult_t (*closeListen)(void* listenComm);
+} ncclNet_v6_t;
+
+typedef struct {  /* src/extern/nccl_net.h:41-94; instance at src/plugin.cc:1997-2017 */
+  const char* name;
+  ncclResult_t (*init)(ncclDebugLogger_t logFunction);
+  ncclResult_t (*devices)(int* ndev);
+  ncclResult_t (*getProperties)(int dev, ncclNetProperties_v7_t* props);
+  ncclResult_t (*listen)(int dev, void* handle, void** listenComm);
+  ncclResult_t (*connect)(int dev, void* handle, void** sendComm, ncclNetDeviceHandle_v7_t** sendDevComm);
+  ncclResult_t (*accept)(void* listenComm, void** recvComm, ncclNetDeviceHandle_v7_t** recvDevComm);
+  ncclResult_t (*regMr)(void* comm, void* data, int size, int type, void** mhandle);
+  ncclResult_t (*regMrDmaBuf)(void* comm, void* data, size_t size, int type, uint64_t offset, int fd, void** mhandle);
+  ncclResult_t (*deregMr)(void* comm, void* mhandle);
+  ncclResult_t (*isend)(void* sendComm, void* data, int size, int tag, void* mhandle, void** request);
+  ncclResult_t (*irecv)(void* recvComm, int n, void** data, int* sizes, int* tags, void** mhandles, void** request);
+  ncclResult_t (*iflush)(void* recvComm, int n, void** data, int* sizes, void** mhandles, void** request);
+  ncclResult_t (*test)(void* request, int* done, int* sizes);
+  ncclResult_t (*closeSend)(void* sendComm);
+  ncclResult_t (*closeRecv)(void* recvComm);
+  ncclResult_t (*closeListen)(void* listenComm);
+  ncclResult_t (*getDeviceMr)(void* comm, void* mhandle, void** dptr_mhandle);   /* NULL, as src/plugin.cc:2015 */
+  ncclResult_t (*irecvConsumed)(void* recvComm, int n, void* request);          /* NULL, as src/plugin.cc:2016 */
+} ncclNet_v7_t;
+
+typedef struct {
+  const char* name;
+  ncclResult_t (*init)(ncclDebugLogger_t logFunction);
+  ncclResult_t (*devices)(int* ndev);
+  ncclResult_t (*getProperties)(int dev, ncclNetProperties_v8_t* props);
+  ncclResult_t (*listen)(int dev, void* handle, void** listenComm);
+  ncclResult_t (*connect)(int dev, void* handle, void** sendComm, ncclNetDeviceHandle_v8_t** sendDevComm);
+  ncclResult_t (*accept)(void* listenComm, void** recvComm, ncclNetDeviceHandle_v8_t** recvDevComm);
+  ncclResult_t (*regMr)(void* comm, void* data, size_t size, int type, void** mhandle);
+  ncclResult_t (*regMrDmaBuf)(void* comm, void* data, size_t size, int type, uint64_t offset, int fd, void** mhandle);
+  ncclResult_t (*deregMr)(void* comm, void* mhandle);
+  ncclResult_t (*isend)(void* sendComm, void* data, int size, int tag, void* mhandle, void** request);
+  ncclResult_t (*irecv)(void* recvComm, int n, void** data, int* sizes, int* tags, void** mhandles, void** request);
+  ncclResult_t (*iflush)(void* recvComm, int n, void** data, int* sizes, void** mhandles, void** request);
+  ncclResult_t (*test)(void* request, int* done, int* sizes);
+  ncclResult_t (*closeSend)(void* sendComm);
+  ncclResult_t (*closeRecv)(void* recvComm);
+  ncclResult_t (*closeListen)(void* listenComm);
+  ncclResult_t (*getDeviceMr)(void* comm, void* mhandle, void** dptr_mhandle);
+  ncclResult_t (*irecvConsumed)(void* recvComm, int n, void* request);
+} ncclNet_v8_t;
+
+/* the data symbols a communication library resolves with dlsym() */
+extern ncclNet_v8_t ncclNetPlugin_v8;
+extern ncclNet_v7_t ncclNetPlugin_v7;
+extern ncclNet_v6_t ncclNetPlugin_v6;
+
+/* ---- limits restated from the reference -------------------------------------------------------- */
+#define FL_NET_MAX_RECVS        8     /* NCCL_NET_IB_MAX_RECVS, src/plugin.cc:358 */
+#define FL_NET_MAX_REQUESTS     256   /* MAX_REQUESTS = 32 * 8, src/plugin.cc:382 */
+#define FL_NET_REFRESH_BATCH    8     /* N_FINISHED_BATCH, src/plugin.cc:38 */
+#define FL_NET_MAX_LANES        16    /* MAX_NIC_NUM, src/monitor.h:18 */
+#define FL_NET_MONITOR_TIMEOUT_US 160 /* MONITOR_TIMEOUT_US, src/monitor.h:26 */
+
+/* ---- control surface beside the plugin tables (for a harness or a host runtime) ------------------
+ * None of this is needed to use the plugin; it exposes what the reference keeps in its monitor
+ * daemon's shared memory (src/monitor.h:47-55) and a few counters.  All return 0 or a negative
+ * FLH_E_* code (fuselink_hip.h). */
+
+/* Monitor state machine of src/monitor.h:191-250 and src/monitor.cpp:159-193, in-process, with the
+ * clock passed in so that it is deterministic: mark = (timestamp, BUSY); tick = every NIC whose
+ * timestamp + 160 us <= now becomes IDLE; pick = borrow an idle NIC of another group. */
+int fl_monitor_reset(void);
+/* Clock of the plugin's own marks and ticks: manual = 0 (default) reads the steady clock as
+ * get_timestamp() does (src/monitor.h:29-33); manual = 1 freezes it at now_us until the next call,
+ * which makes every lane decision reproducible. */
+int fl_monitor_set_clock(int manual, int64_t now_us);
+int64_t fl_monitor_now(void);
+int fl_monitor_mark_active(int lane, int is_tx, int64_t now_us);
+int fl_monitor_tick(int64_t now_us);
+int fl_monitor_status(int is_tx, int n_lanes, int32_t* status_out);
+/* getIdleNicTx / getIdleNicRx (src/monitor.h:191-224).  `exact` = 0 restates the reference as
+ * written (every idle NIC met is marked BORROWED and the last one is returned); `exact` = 1 borrows
+ * only the first idle NIC, which is what the code evidently meant. */
+int fl_monitor_idle_pick(int is_tx, int group, int mask, int exact);
+/* credits the scheduler will use from the next refresh on: IDLE -> idle_credit, BUSY/BORROWED -> 0,
+ * the comm's own lane never below 1 */
+int fl_monitor_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t* credits_out);
+
+/* Static credits (one value per lane) overriding the monitor-derived ones; n = 0 removes the
+ * override.  The same can be preset with NCCL_FUSELINK_CREDITS="c0,c1,...". */
+int fl_net_set_credits(const uint32_t* credits, int n);
+/* Forget the parameters read at init so that the next init() reads the NCCL_FUSELINK_* environment
+ * again; refused (FLH_E_STATE) while a listen comm or a connection is alive. */
+int fl_net_reset(void);
+/* Make the next completion of `request` fail in test() with ncclRemoteError (wire-fault injection). */
+int fl_net_inject_fault(void* request);
+/* Counters of a send or recv comm: n_finished (src/plugin.cc:517,568), requests in flight, lane refreshes. */
+int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64_t* refreshes);
+/* Chunk -> lane table and header of the last wave a send comm scheduled, copied to host memory
+ * (blocks until that wave has run).  rows_out holds up to max_rows flh_chunk_desc entries.
+ * Returns the number of rows of that wave. */
+int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FUSELINK_NET_H_ */

@@ -144,7 +144,7 @@ int fl_credit_schedule(const uint32_t* sizes, uint64_t total_bytes, uint32_t chu
   if (state) st = *state; else memset(&st, 0, sizeof(st));
   fl_sched_hdr_t h;
   memset(&h, 0, sizeof(h));
-  uint64_t P = st.epoch_bytes;
+  uint64_t P = (mode & FLO_SCHED_NEW_EPOCH) ? 0 : st.epoch_bytes;
   uint64_t run = 0;
   uint64_t lane_off[FLO_MAX_NIC_NUM];
   for (int l = 0; l < FLO_MAX_NIC_NUM; ++l) lane_off[l] = (mode & FLO_SCHED_RESET_OFFSETS) ? 0 : st.lane_off[l];

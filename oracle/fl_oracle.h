@@ -150,6 +150,7 @@ typedef struct {
 #define FLO_SCHED_F_NO_CREDIT 1u
 /* mode bits of the `mode` argument */
 #define FLO_SCHED_RESET_OFFSETS 1u /* ignore state->lane_off on entry: windows are reused from 0 */
+#define FLO_SCHED_NEW_EPOCH     4u /* ignore state->epoch_bytes on entry: a credit refresh starts a new epoch */
 #define FLO_SCHED_MIRROR        2u /* win_off = src_off: the window mirrors the user buffer, which is
                                       the reference's translation window + (data - start_addr),
                                       plugin.cc:1582,1626 */

@@ -1,0 +1,243 @@
+"""The plugin ABI driven the way NCCL's proxy drives it, with host memory (NCCL_PTR_HOST) so that
+the request machinery, the FIFO handshake and the error convention are checked without a GPU.
+Host buffers are never staged (FuseLink src/fuselink.cc:8-13), so no kernel is involved here."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from fuselink_amd import plugin as P
+
+
+@pytest.fixture()
+def net():
+    p = P.NetPlugin(8)
+    assert p.init() == P.ncclSuccess
+    p.lib.fl_monitor_reset()
+    p.set_credits([])
+    return p
+
+
+def _host(n, seed=0):
+    a = np.random.default_rng(seed).integers(0, 256, size=n, dtype=np.uint8)
+    return a, a.ctypes.data
+
+
+def test_library_exports_every_declared_symbol():
+    import re, os
+    lib = C.CDLL(P.lib_path())
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    names = set()
+    for hdr in ("fuselink_hip.h", "fuselink_net.h"):
+        text = open(os.path.join(root, "include", hdr)).read()
+        names |= set(re.findall(r"\b(flh_[a-z0-9_]+|fl_net_[a-z0-9_]+|fl_monitor_[a-z0-9_]+)\s*\(", text))
+        names |= set(re.findall(r"extern\s+\w+\s+(ncclNetPlugin_v\d)\s*;", text))
+    assert len(names) > 40
+    for n in sorted(names):
+        assert hasattr(lib, n), f"{n} is declared in include/ but not exported"
+
+
+@pytest.mark.parametrize("version", [6, 7, 8])
+def test_tables_and_properties(version):
+    p = P.NetPlugin(version)
+    assert p.name == "FuseLink"  # src/plugin.cc:1998
+    assert p.init() == P.ncclSuccess
+    rc, n = p.devices()
+    assert rc == P.ncclSuccess and n == 8
+    rc, props = p.getProperties(3)
+    assert rc == P.ncclSuccess
+    assert props.name == b"fuselink3" and props.guid == 3
+    assert props.ptrSupport == P.NCCL_PTR_HOST | P.NCCL_PTR_CUDA
+    assert props.maxRecvs == 1 and props.latency == 0
+    if version >= 7:
+        assert props.netDeviceType == 0 and props.netDeviceVersion == 0  # src/plugin.cc:376-377
+        assert not p.t.getDeviceMr and not p.t.irecvConsumed            # src/plugin.cc:2015-2016
+    if version == 8:
+        assert props.regIsGlobal == 1
+    assert p.getProperties(99)[0] == P.ncclInvalidArgument
+
+
+def test_connect_accept_are_nonblocking_and_staged(net):
+    rc, handle, lcomm = net.listen(0)
+    assert rc == P.ncclSuccess and lcomm
+    rc, r = net.accept(lcomm)
+    assert rc == P.ncclSuccess and r is None           # nobody connected yet
+    rc, s = net.connect(0, handle)
+    assert rc == P.ncclSuccess and s is None           # posted, peer has not accepted
+    rc, s = net.connect(0, handle)
+    assert rc == P.ncclSuccess and s is None
+    rc, r = net.accept(lcomm)
+    assert rc == P.ncclSuccess and r
+    rc, s = net.connect(0, handle)
+    assert rc == P.ncclSuccess and s
+    assert net.closeSend(s) == 0 and net.closeRecv(r) == 0 and net.closeListen(lcomm) == 0
+
+
+def test_channel_ids_count_up_per_listen(net):
+    # ncclIbListen hands out a global, increasing channelId (src/plugin.cc:693-708); it sits in the handle
+    ids = []
+    comms = []
+    for _ in range(3):
+        rc, handle, lcomm = net.listen(1)
+        ids.append(int.from_bytes(handle.raw[16:20], "little", signed=True))
+        comms.append(lcomm)
+    assert ids[1] == ids[0] + 1 and ids[2] == ids[0] + 2
+    for c in comms:
+        net.closeListen(c)
+
+
+def test_send_recv_roundtrip_and_sizes(net):
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(1 << 20, 1)
+    dst = np.zeros(1 << 20, dtype=np.uint8)
+    rc, smh = net.regMr(s, sp, src.size, P.NCCL_PTR_HOST)
+    assert rc == 0 and smh
+    rc, rmh = net.regMr(r, dst.ctypes.data, dst.size, P.NCCL_PTR_HOST)
+    assert rc == 0 and rmh
+    # the sender cannot proceed before the receive is posted (src/plugin.cc:1510-1514)
+    rc, req = net.isend(s, sp, 4096, 7, smh)
+    assert rc == 0 and req is None
+    rc, rreq = net.irecv(r, [dst.ctypes.data], [1 << 20], [7], [rmh])
+    assert rc == 0 and rreq
+    rc, done, _ = net.test(rreq)
+    assert rc == 0 and done == 0                        # posted, not matched
+    rc, sreq = net.isend(s, sp, 1 << 20, 7, smh)
+    assert rc == 0 and sreq
+    assert net.wait(sreq) is not None
+    assert net.wait(rreq) == 1 << 20                    # byte count of the receive is reported
+    np.testing.assert_array_equal(dst, src)
+    # a shorter send into a larger posted receive is fine and reports the sent size
+    rc, rreq = net.irecv(r, [dst.ctypes.data], [1 << 20], [8], [rmh])
+    rc, sreq = net.isend(s, sp + 100, 1000, 8, smh)
+    assert rc == 0 and sreq
+    net.wait(sreq)
+    assert net.wait(rreq) == 1000
+    np.testing.assert_array_equal(dst[:1000], src[100:1100])
+    st = net.comm_stats(s)
+    assert st["n_finished"] == 2 and st["in_flight"] == 0
+    assert net.deregMr(s, smh) == 0 and net.deregMr(r, rmh) == 0
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_error_convention(net):
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(8192, 2)
+    dst = np.zeros(8192, dtype=np.uint8)
+    _, smh = net.regMr(s, sp, src.size, P.NCCL_PTR_HOST)
+    _, rmh = net.regMr(r, dst.ctypes.data, dst.size, P.NCCL_PTR_HOST)
+    # send larger than the posted receive -> ncclInvalidUsage (src/plugin.cc:1555-1562)
+    rc, rreq = net.irecv(r, [dst.ctypes.data], [1000], [1], [rmh])
+    assert rc == 0 and rreq
+    rc, sreq = net.isend(s, sp, 2000, 1, smh)
+    assert rc == P.ncclInvalidUsage and sreq is None
+    # a send with another tag does not match and would block (src/plugin.cc:1552)
+    rc, sreq = net.isend(s, sp, 500, 2, smh)
+    assert rc == 0 and sreq is None
+    rc, sreq = net.isend(s, sp, 500, 1, smh)
+    assert rc == 0 and sreq
+    net.wait(sreq), net.wait(rreq)
+    # grouped receives are rejected (src/plugin.cc:1448-1451, 1873-1880); more than 8 is an error outright (1683)
+    rc, q = net.irecv(r, [dst.ctypes.data] * 2, [10, 10], [1, 1], [rmh, rmh])
+    assert rc == P.ncclInternalError and q is None
+    rc, q = net.irecv(r, [dst.ctypes.data] * 9, [10] * 9, [1] * 9, [rmh] * 9)
+    assert rc == P.ncclInternalError
+    # buffers outside their registration
+    other = np.zeros(64, dtype=np.uint8)
+    rc, q = net.isend(s, other.ctypes.data + (1 << 30), 16, 1, smh)
+    assert rc in (0, P.ncclInvalidArgument) and q is None
+    # test on a request that already completed
+    rc, _, _ = net.test(sreq)
+    assert rc == P.ncclInternalError
+    # unsupported pointer type
+    rc, mh = net.regMr(s, sp, 16, 64)
+    assert rc == P.ncclInvalidArgument and mh is None
+    net.deregMr(s, smh), net.deregMr(r, rmh)
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_refresh_cadence_gates_posting(net):
+    """Every 8 completions the receiver may change lanes, and only once nothing is outstanding
+    (src/plugin.cc:38, 1700-1712): at those points a second irecv has to wait for the first."""
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(4096, 3)
+    dst = np.zeros(4096, dtype=np.uint8)
+    _, smh = net.regMr(s, sp, src.size, P.NCCL_PTR_HOST)
+    _, rmh = net.regMr(r, dst.ctypes.data, dst.size, P.NCCL_PTR_HOST)
+    tag = 0
+    refreshed_at = []
+    while net.comm_stats(r)["n_finished"] < 40:
+        fin = net.comm_stats(r)["n_finished"]
+        before = net.comm_stats(r)["refreshes"]
+        rc, first = net.irecv(r, [dst.ctypes.data], [64], [tag], [rmh])
+        assert rc == 0 and first
+        if net.comm_stats(r)["refreshes"] != before:
+            refreshed_at.append(fin)
+        # with one receive outstanding a second one is held back exactly on a batch boundary
+        rc, second = net.irecv(r, [dst.ctypes.data + 64], [64], [tag + 1], [rmh])
+        assert rc == 0
+        assert (second is None) == (fin % 8 == 0), fin
+        for q, t in ((first, tag), (second, tag + 1)):
+            if q is None:
+                continue
+            rc, sreq = net.isend(s, sp, 64, t, smh)
+            assert rc == 0 and sreq
+            net.wait(sreq), net.wait(q)
+        tag += 2
+    # refreshes happen on the batch boundaries that an irecv actually met with nothing outstanding
+    assert refreshed_at and all(f % 8 == 0 for f in refreshed_at) and refreshed_at[0] == 0
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_request_slots_run_out_at_256(net):
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(4096, 4)
+    dst = np.zeros(4096, dtype=np.uint8)
+    _, smh = net.regMr(s, sp, src.size, P.NCCL_PTR_HOST)
+    _, rmh = net.regMr(r, dst.ctypes.data, dst.size, P.NCCL_PTR_HOST)
+    # get n_finished off the refresh boundary first
+    _, rreq = net.irecv(r, [dst.ctypes.data], [8], [0], [rmh])
+    _, sreq = net.isend(s, sp, 8, 0, smh)
+    net.wait(sreq), net.wait(rreq)
+    reqs = []
+    for k in range(256):
+        rc, q = net.irecv(r, [dst.ctypes.data], [8], [k], [rmh])
+        assert rc == 0 and q, k
+        reqs.append(q)
+    rc, q = net.irecv(r, [dst.ctypes.data], [8], [999], [rmh])
+    assert rc == P.ncclInternalError and q is None       # src/plugin.cc:1082-1084
+    # requests are slots of a fixed table inside the connection: first free first (src/plugin.cc:1070-1085)
+    assert len(set(reqs)) == 256
+    stride = reqs[1] - reqs[0]
+    assert all(reqs[i + 1] - reqs[i] == stride for i in range(255))
+    for k in range(256):
+        rc, sq = net.isend(s, sp, 8, k, smh)
+        assert rc == 0 and sq
+        net.wait(sq), net.wait(reqs[k])
+    assert net.comm_stats(r)["n_finished"] == 257
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_injected_wire_fault_surfaces_in_test(net):
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(4096, 5)
+    dst = np.zeros(4096, dtype=np.uint8)
+    _, smh = net.regMr(s, sp, src.size, P.NCCL_PTR_HOST)
+    _, rmh = net.regMr(r, dst.ctypes.data, dst.size, P.NCCL_PTR_HOST)
+    _, rreq = net.irecv(r, [dst.ctypes.data], [64], [0], [rmh])
+    _, sreq = net.isend(s, sp, 64, 0, smh)
+    assert net.lib.fl_net_inject_fault(rreq) == 0
+    net.wait(sreq)
+    rc, done, _ = net.test(rreq)
+    assert rc == P.ncclRemoteError and done == 0        # src/plugin.cc:1839-1861
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_cuda_pointer_fails_loudly_without_gpu(net):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(4096, 6)
+    rc, mh = net.regMr(s, sp, 4096, P.NCCL_PTR_CUDA)
+    assert rc == P.ncclUnhandledCudaError and mh is None  # no CPU fallback for device memory
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
