@@ -64,6 +64,14 @@ int fl_monitor_mark_active(int lane, int is_tx, int64_t now_us) {
   return FLH_OK;
 }
 
+int fl_monitor_set_entry(int lane, int is_tx, int32_t status, int64_t last_active_us) {
+  if (lane < 0 || lane >= kGroups || status < kIdle || status > kBorrowed) return fl_set_error(FLH_E_ARG, "bad table entry");
+  std::lock_guard<std::mutex> g(g_mu);
+  g_tab.status[is_tx ? 1 : 0][lane] = status;
+  g_tab.last_active[is_tx ? 1 : 0][lane] = last_active_us;
+  return FLH_OK;
+}
+
 // Monitor::monitorThread body (src/monitor.cpp:164-188): a lane whose last activity is at least the
 // timeout old becomes IDLE, whatever it was (BUSY or BORROWED); a younger one keeps its status.
 int fl_monitor_tick(int64_t now_us) {

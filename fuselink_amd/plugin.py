@@ -71,7 +71,7 @@ def _table(version: int):
 
 
 PLUGIN_SYMBOLS = ["ncclNetPlugin_v8", "ncclNetPlugin_v7", "ncclNetPlugin_v6"]
-CONTROL_SYMBOLS = ["fl_monitor_reset", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
+CONTROL_SYMBOLS = ["fl_monitor_reset", "fl_monitor_set_entry", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
                    "fl_monitor_status", "fl_monitor_idle_pick", "fl_monitor_credits", "fl_net_set_credits",
                    "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_last_table", "fl_net_reset"]
 
@@ -102,6 +102,7 @@ class NetPlugin:
         L.fl_monitor_now.restype = C.c_int64
         L.fl_monitor_mark_active.argtypes = [C.c_int, C.c_int, C.c_int64]
         L.fl_monitor_tick.argtypes = [C.c_int64]
+        L.fl_monitor_set_entry.argtypes = [C.c_int, C.c_int, C.c_int32, C.c_int64]
         L.fl_monitor_status.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_int32)]
         L.fl_monitor_idle_pick.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int]
         L.fl_monitor_credits.argtypes = [C.c_int, C.c_int, C.c_uint32, C.POINTER(C.c_uint32)]

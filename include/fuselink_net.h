@@ -200,6 +200,8 @@ int fl_monitor_reset(void);
 int fl_monitor_set_clock(int manual, int64_t now_us);
 int64_t fl_monitor_now(void);
 int fl_monitor_mark_active(int lane, int is_tx, int64_t now_us);
+/* raw write of one table entry, as any process mapping the reference's shared memory could do */
+int fl_monitor_set_entry(int lane, int is_tx, int32_t status, int64_t last_active_us);
 int fl_monitor_tick(int64_t now_us);
 int fl_monitor_status(int is_tx, int n_lanes, int32_t* status_out);
 /* getIdleNicTx / getIdleNicRx (src/monitor.h:191-224).  `exact` = 0 restates the reference as
