@@ -131,22 +131,29 @@ def main() -> int:
     assert int(status.item()) == 0, "a kernel refused a chunk (window or buffer range)"
     assert torch.equal(src, dst), "reassembled buffer differs from the source"
 
-    # ---- per-kernel durations: every launch carries its own start/stop HIP events on the launch stream ----
-    def kernel_us(fn, iters):
-        core.prof_enable(True)
-        ts = []
-        for _ in range(iters):
-            fn()
-            ts.append(core.prof_last_us())
-        core.prof_enable(False)
-        return sum(ts) / len(ts), min(ts)
+    # ---- per-kernel durations: the same K steps again, every launch carrying its own start/stop HIP
+    # events on the launch stream (they bracket the kernel alone; launches stay back to back) ----------
+    def profiled(fn, launches):
+        core.prof_begin(launches)
+        fn()
+        return core.prof_end(launches)
 
-    k_iters = max(20, min(args.steps, 200))
-    sched_us, sched_min = kernel_us(lambda: core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes,
-                                                          chunk_bytes=chunk, epoch_len=epoch_len, out=sched, stream=stream), k_iters)
-    stripe_us, stripe_min = kernel_us(lambda: core.stripe(src, win, sched, status, stream=stream, hint=hint), k_iters)
-    reasm_us, reasm_min = kernel_us(lambda: core.reassemble(dst, win, sched, status, stream=stream, hint=hint), k_iters)
-    copy_us, _ = kernel_us(lambda: core.copy(dst, src, stream=stream), k_iters)
+    def steps_eager():
+        for _ in range(args.steps):
+            step()
+
+    per = profiled(steps_eager, 4 * args.steps)
+    mean = lambda xs: sum(xs) / len(xs)
+    sched_us, stripe_us, reasm_us = mean(per["schedule"]), mean(per["stripe"]), mean(per["reassemble"])
+    stripe_min, reasm_min = min(per["stripe"]), min(per["reassemble"])
+    n_sched_launches = len(per["schedule"]) // args.steps
+
+    def copies():
+        for _ in range(min(args.steps, 100)):
+            core.copy(dst, src, stream=stream)
+
+    copy_us = mean(profiled(copies, 128)["copy"])
+    assert torch.equal(src, dst)
 
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
     algo_bytes_kernel = 2 * nbytes        # one launch of the copy kernel
@@ -177,7 +184,7 @@ def main() -> int:
                        "stripe_min": round(stripe_min, 2), "reassemble_min": round(reasm_min, 2),
                        "plain_copy_same_bytes": round(copy_us, 2)},
         "stripe_reassemble_pair_GBps": round(algo_bytes_step / (pair_us * 1e-6) / 1e9, 1),
-        "scheduler_us_per_1k_chunks": round(sched_us / (n_chunks / 1000.0), 3),
+        "scheduler_us_per_1k_chunks": round(sched_us * n_sched_launches / (n_chunks / 1000.0), 3),
         "roofline": {"bound": "hbm", "kernel": "fl_copy_tiles<0> (stripe)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC.get(args.workload)},

@@ -74,8 +74,8 @@ SIGNATURES = {
     "flh_region_windows": (C.c_int, [C.c_void_p, C.POINTER(Windows)]),
     "flh_region_translate": (C.c_void_p, [C.c_void_p, C.c_uint32, C.c_void_p]),
     "flh_tune": (C.c_int, [C.c_char_p, C.c_int64]),
-    "flh_prof_enable": (C.c_int, [C.c_int]),
-    "flh_prof_last_us": (C.c_int, [C.POINTER(C.c_double)]),
+    "flh_prof_begin": (C.c_int, [C.c_int]),
+    "flh_prof_end": (C.c_int, [C.POINTER(C.c_double), C.POINTER(C.c_int), C.c_int]),
 }
 
 _lib = None

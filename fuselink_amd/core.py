@@ -37,14 +37,22 @@ def tune(key: str, value: int) -> None:
     check(_lib.load().flh_tune(key.encode(), int(value)))
 
 
-def prof_enable(on: bool) -> None:
-    check(_lib.load().flh_prof_enable(int(on)))
+PROF_KERNELS = {1: "schedule", 2: "stripe", 3: "reassemble", 4: "gather", 5: "scatter", 6: "copy"}
 
 
-def prof_last_us() -> float:
-    us = C.c_double()
-    check(_lib.load().flh_prof_last_us(C.byref(us)))
-    return us.value
+def prof_begin(capacity: int) -> None:
+    check(_lib.load().flh_prof_begin(capacity))
+
+
+def prof_end(capacity: int):
+    """Returns {kernel name: [durations in us]} of the launches made since prof_begin."""
+    us = (C.c_double * capacity)()
+    kid = (C.c_int * capacity)()
+    n = check(_lib.load().flh_prof_end(us, kid, capacity))
+    out = {}
+    for i in range(min(n, capacity)):
+        out.setdefault(PROF_KERNELS.get(kid[i], str(kid[i])), []).append(us[i])
+    return out
 
 
 def _stream_ptr(stream: Optional[torch.cuda.Stream]) -> C.c_void_p:

@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <vector>
 
 #include "fl_internal.h"
 #include "fuselink_hip.h"
@@ -204,9 +205,13 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   // the static policy -- and flagged.
   const bool rows_cached = a.n_rows <= (uint32_t)kRowCache;
   uint32_t flags = 0;
+  __shared__ uint32_t raw[kRowCache * FLH_MAX_LANES];
   if (rows_cached) {
+    // all credit rows in one round trip to memory, then one wavefront scan per row out of LDS
+    for (uint32_t e = tid; e < a.n_rows * L; e += BT) raw[e] = a.credits ? a.credits[e] : a.inline_credits[e];
+    __syncthreads();
     for (uint32_t r = wave; r < a.n_rows; r += NW) {
-      const uint32_t c = (uint32_t)lane < L ? (a.credits ? a.credits[(size_t)r * L + lane] : a.inline_credits[lane]) : 0;
+      const uint32_t c = (uint32_t)lane < L ? raw[r * L + lane] : 0;
       uint64_t inc = wave_incl_sum_u64(c, lane);
       const bool zero = bcast_lane_u64(inc, kWave - 1) == 0;
       if (zero) inc = (uint32_t)lane < L ? lane + 1 : L;
@@ -416,6 +421,196 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// scheduler, uniform split
+// ------------------------------------------------------------------------------------------------
+// When every chunk has the quantum's size (the ordinary message split: sizes == nullptr and
+// quantum == chunk_bytes; only the last chunk may be short) the byte prefix of chunk j of an epoch
+// is j quanta, so its slot is j mod W and nothing has to be scanned: the number of earlier chunks
+// on a lane is a closed form in j,
+//     cnt(row, l, x) = #{ y < x : slot y belongs to lane l } = (x / W) * c_l + clamp(x mod W - K_l, 0, c_l),
+// whole epochs contribute cnt(row, l, E), and because rows repeat with period R those contributions
+// sum in closed form too.  Every chunk is independent, so the table is filled by as many workgroups
+// as it takes; the results are identical to the scan kernel's.
+struct UniTables {
+  uint64_t pfx[kRowCache][FLH_MAX_LANES];   // inclusive credit prefixes (equal credits for an empty row)
+  uint64_t pf[kRowCache + 1][FLH_MAX_LANES];  // pf[r][l] = chunks on lane l in whole epochs of rows < r; pf[R] = one period
+  uint32_t zero[kRowCache];
+};
+
+__device__ __forceinline__ uint64_t uni_cnt(const UniTables& t, uint32_t r, uint32_t l, uint32_t L, uint64_t x) {
+  const uint64_t W = t.pfx[r][L - 1];
+  const uint64_t hi = t.pfx[r][l];
+  const uint64_t K = l ? t.pfx[r][l - 1] : 0;
+  const uint64_t c = hi - K;
+  const uint64_t full = div_u64(x, W);
+  const uint64_t rem = x - full * W;
+  const uint64_t part = rem <= K ? 0 : (rem - K < c ? rem - K : c);
+  return full * c + part;
+}
+
+__device__ __forceinline__ uint32_t uni_lane(const UniTables& t, uint32_t r, uint32_t L, uint64_t j) {
+  const uint64_t slot = mod_u64(j, t.pfx[r][L - 1]);
+  uint32_t pick = 0;
+#pragma unroll 1
+  for (uint32_t l = 0; l + 1 < L; ++l) pick += t.pfx[r][l] <= slot;
+  return pick;
+}
+
+struct UniCtx {
+  uint64_t k0, a0, e0, C;
+  uint32_t pos0, E, R, L;
+};
+
+// chunks of this call, before local index i (0 <= i <= n), that sit on lane l; also returns the lane
+// of chunk i itself through *lane_of_i when asked (l == 0xffffffff means "use chunk i's own lane")
+__device__ __forceinline__ uint64_t uni_before(const UniTables& t, const UniCtx& c, uint64_t i, uint32_t l, uint32_t* lane_of_i,
+                                               uint64_t* epoch_of_i) {
+  if (c.E == 0) {
+    const uint64_t j = c.a0 + i;
+    if (lane_of_i) { *lane_of_i = uni_lane(t, 0, c.L, j); if (l == 0xffffffffu) l = *lane_of_i; }
+    if (epoch_of_i) *epoch_of_i = 0;
+    return uni_cnt(t, 0, l, c.L, j) - uni_cnt(t, 0, l, c.L, c.a0);
+  }
+  const uint64_t g = c.k0 + i;
+  const uint64_t e = div_u64(g, c.E);
+  const uint64_t pos = g - e * c.E;
+  const uint32_t r = (uint32_t)mod_u64(e, c.R);
+  if (epoch_of_i) *epoch_of_i = e;
+  if (e == c.e0) {
+    const uint64_t j = c.a0 + (pos - c.pos0);
+    if (lane_of_i) { *lane_of_i = uni_lane(t, r, c.L, j); if (l == 0xffffffffu) l = *lane_of_i; }
+    return uni_cnt(t, r, l, c.L, j) - uni_cnt(t, r, l, c.L, c.a0);
+  }
+  if (lane_of_i) { *lane_of_i = uni_lane(t, r, c.L, pos); if (l == 0xffffffffu) l = *lane_of_i; }
+  const uint32_t r0 = (uint32_t)mod_u64(c.e0, c.R);
+  const uint64_t m0 = c.E - c.pos0;  // chunks of this call in its first epoch
+  uint64_t before = uni_cnt(t, r0, l, c.L, c.a0 + m0) - uni_cnt(t, r0, l, c.L, c.a0);
+  // whole epochs e0+1 .. e-1: G(e) - G(e0+1), G(z) = (z / R) * period + pf[z mod R]
+  const uint64_t z1 = e, z0 = c.e0 + 1;
+  const uint64_t q1 = div_u64(z1, c.R), q0 = div_u64(z0, c.R);
+  before += q1 * t.pf[c.R][l] + t.pf[z1 - q1 * c.R][l];
+  before -= q0 * t.pf[c.R][l] + t.pf[z0 - q0 * c.R][l];
+  before += uni_cnt(t, r, l, c.L, pos);
+  return before;
+}
+
+constexpr int kUniBlock = 256;
+
+// MODE 0: fill the table; the last workgroup also writes the header and, if the grid is a single
+//         workgroup, the state (in place: every read of the old state precedes the barrier).
+// MODE 1: write the state only (second launch after a multi-workgroup MODE 0, so that no workgroup
+//         can still be reading the old state).
+template <int MODE>
+__global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArgs a) {
+  __shared__ UniTables t;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const uint32_t L = a.n_lanes, R = a.n_rows;
+  // all credit rows in one round trip to memory, then one wavefront scan per row out of LDS
+  __shared__ uint32_t raw[kRowCache * FLH_MAX_LANES];
+  for (uint32_t e = tid; e < R * L; e += kUniBlock) raw[e] = a.credits ? a.credits[e] : a.inline_credits[e];
+  __syncthreads();
+  for (uint32_t r = wave; r < R; r += kUniBlock / kWave) {
+    const uint32_t c = (uint32_t)lane < L ? raw[r * L + lane] : 0;
+    uint64_t inc = wave_incl_sum_u64(c, lane);
+    const bool zero = bcast_lane_u64(inc, kWave - 1) == 0;
+    if (zero) inc = (uint32_t)lane < L ? lane + 1 : L;
+    if ((uint32_t)lane < L) t.pfx[r][lane] = inc;
+    if (lane == 0) t.zero[r] = zero;
+  }
+  __syncthreads();
+  if ((uint32_t)tid < L) {  // chunks per lane of one whole epoch under each row, prefixed over the rows
+    uint64_t run = 0;
+    for (uint32_t r = 0; r < R; ++r) {
+      t.pf[r][tid] = run;
+      if (a.epoch_len) run += uni_cnt(t, r, (uint32_t)tid, L, a.epoch_len);
+    }
+    t.pf[R][tid] = run;
+  }
+  __syncthreads();
+
+  UniCtx c;
+  c.C = a.chunk_bytes;
+  c.E = a.epoch_len;
+  c.R = R;
+  c.L = L;
+  c.k0 = a.state ? a.state->chunk_index : 0;
+  const uint64_t p0 = (a.state && !(a.mode & FLH_SCHED_NEW_EPOCH)) ? a.state->epoch_bytes : 0;
+  c.e0 = c.E ? div_u64(c.k0, c.E) : 0;
+  c.pos0 = c.E ? (uint32_t)(c.k0 - c.e0 * c.E) : 0;
+  // quanta already behind the first chunk inside its epoch; an epoch head starts from zero
+  c.a0 = (c.E && c.pos0 == 0) ? 0 : div_u64(p0, c.C);
+  const bool keep_off = a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS);
+  const uint32_t tpc = a.tile_shift >= 0 ? (a.chunk_bytes + a.tile_bytes - 1) >> a.tile_shift : (a.chunk_bytes + a.tile_bytes - 1) / a.tile_bytes;
+
+  if (MODE == 0) {
+    const uint32_t i = blockIdx.x * kUniBlock + tid;
+    if (i < a.n) {
+      uint32_t ln;
+      uint64_t ep;
+      const uint64_t before = uni_before(t, c, i, 0xffffffffu, &ln, &ep);
+      const uint64_t o = (uint64_t)i * c.C;
+      const uint64_t rem = a.total_bytes - o;
+      flh_chunk_desc d;
+      d.src_off = a.src_base + o;
+      d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : (keep_off ? a.state->lane_off[ln] : 0) + before * c.C;
+      d.len = (uint32_t)(rem < c.C ? rem : c.C);
+      d.lane = ln;
+      d.tile_base = i * tpc;
+      d.epoch = (uint32_t)ep;
+      a.table[i] = d;
+    }
+    if (blockIdx.x != gridDim.x - 1) return;
+  }
+  const bool write_hdr = MODE == 0;
+  const bool write_state = a.state && (MODE == 1 || gridDim.x == 1);
+  const uint64_t last = a.n - 1;
+  const uint64_t len_last = a.total_bytes - last * c.C;
+  uint32_t lane_last;
+  uint64_t ep_last;
+  (void)uni_before(t, c, last, 0xffffffffu, &lane_last, &ep_last);
+  uint64_t chunks = 0, bytes = 0, off_in = 0;
+  if ((uint32_t)tid < L) {
+    chunks = uni_before(t, c, a.n, (uint32_t)tid, nullptr, nullptr);
+    bytes = chunks * c.C - ((uint32_t)tid == lane_last ? c.C - len_last : 0);
+  }
+  if (tid < FLH_MAX_LANES && keep_off) off_in = a.state->lane_off[tid];
+  __syncthreads();  // the old state has been read by everyone who needs it
+  if (tid < FLH_MAX_LANES) {
+    if (write_hdr) {
+      a.hdr->lane_bytes[tid] = bytes;
+      a.hdr->lane_chunks[tid] = (uint32_t)chunks;
+    }
+    if (write_state) a.state->lane_off[tid] = off_in + bytes;
+  }
+  if (tid == 0) {
+    if (write_hdr) {
+      uint32_t flags = 0;
+      const uint64_t n_ep = ep_last - c.e0 + 1;
+      const uint32_t look = n_ep < R ? (uint32_t)n_ep : R;
+      for (uint32_t k = 0; k < look; ++k) flags |= t.zero[(uint32_t)mod_u64(c.e0 + k, R)] ? FLH_SCHED_F_NO_CREDIT : 0;
+      a.hdr->total_bytes = a.total_bytes;
+      a.hdr->total_tiles = (uint32_t)last * tpc + (uint32_t)((len_last + a.tile_bytes - 1) / a.tile_bytes);
+      a.hdr->n_chunks = a.n;
+      a.hdr->flags = flags;
+      a.hdr->uniform_tiles = tpc;
+    }
+    if (write_state) {
+      uint64_t p_end;
+      if (c.E == 0 || ep_last == c.e0) {
+        p_end = ((c.E && c.pos0 == 0) ? 0 : p0) + a.total_bytes;
+      } else {
+        const uint64_t pos_last = (c.k0 + last) - ep_last * c.E;
+        p_end = pos_last * c.C + len_last;
+      }
+      a.state->epoch_bytes = p_end;
+      a.state->chunk_index = c.k0 + a.n;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // copy kernels
 // ------------------------------------------------------------------------------------------------
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -538,6 +733,28 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
   }
 }
 
+// Uniform split with the header known on the host: a two-dimensional grid (tile in chunk, chunk)
+// names the work directly, so a workgroup's only dependent access before its data is the one scalar
+// load of its table row.
+template <int DIR, bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform(CopyArgs a) {
+  const uint32_t c = blockIdx.y;
+  if (c >= a.hint_n_chunks) return;
+  const flh_chunk_desc d = a.table[c];
+  const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
+  if (off >= d.len) return;
+  const uint32_t bytes = (uint32_t)((d.len - off) < a.tile_bytes ? (d.len - off) : a.tile_bytes);
+  bool ok = d.lane < a.win.n_lanes;
+  if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane] && d.src_off + d.len <= a.user_bytes;
+  if (!ok) {
+    if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+    return;
+  }
+  uint8_t* u = a.user + d.src_off + off;
+  uint8_t* w = (uint8_t*)a.win.base[d.lane] + d.win_off + off;
+  if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+}
+
 struct PageArgs {
   uint8_t* pool;
   uint64_t pool_pages;
@@ -617,17 +834,29 @@ int g_cus = 0;
 int g_grid_per_cu = 8;
 int g_nontemporal = 0;
 int g_sched_variant = 0;  // 0 = pick the scheduler shape from the chunk count
+int g_sched_uniform_fast = 1;
+int g_copy_uniform_grid = 1;
 
 
-// Per-launch timing: when enabled for the calling thread, every kernel is launched with its own
-// start/stop events (hipExtLaunchKernelGGL), which bracket the kernel alone, not the gaps around it.
+// Per-launch timing: while a profiling region is open on the calling thread, every kernel is launched
+// with its own start/stop events (hipExtLaunchKernelGGL), which bracket the kernel alone and not the
+// gaps around it.  The events are read back when the region is closed, so the launches themselves
+// stay asynchronous and back to back.
+struct ProfRec { hipEvent_t e0, e1; int kid; };
+thread_local std::vector<ProfRec>* g_prof_ring = nullptr;
+thread_local size_t g_prof_n = 0;
 thread_local bool g_prof_on = false;
-thread_local hipEvent_t g_prof_ev0 = nullptr, g_prof_ev1 = nullptr;
+thread_local int g_prof_kid = 0;   // which entry point is launching: 1 schedule, 2 stripe, 3 reassemble, 4 gather, 5 scatter, 6 copy
 
 #define FL_LAUNCH(kernel, grid, block, shmem, stream, ...)                                              \
   do {                                                                                                  \
-    if (g_prof_on) hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, g_prof_ev0, g_prof_ev1, 0, __VA_ARGS__); \
-    else hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                           \
+    if (g_prof_on && g_prof_n < g_prof_ring->size()) {                                                  \
+      ProfRec& pr_ = (*g_prof_ring)[g_prof_n++];                                                        \
+      pr_.kid = g_prof_kid;                                                                             \
+      hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, pr_.e0, pr_.e1, 0, __VA_ARGS__);        \
+    } else {                                                                                            \
+      hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                              \
+    }                                                                                                   \
   } while (0)
 
 int64_t env_i64(const char* name, int64_t dflt) {
@@ -695,29 +924,45 @@ int flh_init(int device) {
   return FLH_OK;
 }
 
-int flh_prof_enable(int on) {
-  if (on && !g_prof_ev0) {
-    FL_HIP(hipEventCreate(&g_prof_ev0));
-    FL_HIP(hipEventCreate(&g_prof_ev1));
+int flh_prof_begin(int capacity) {
+  if (capacity < 1 || capacity > (1 << 20)) return fl_set_error(FLH_E_ARG, "capacity %d out of range", capacity);
+  if (!g_prof_ring) g_prof_ring = new std::vector<ProfRec>();
+  while (g_prof_ring->size() < (size_t)capacity) {
+    ProfRec r;
+    r.kid = 0;
+    FL_HIP(hipEventCreate(&r.e0));
+    FL_HIP(hipEventCreate(&r.e1));
+    g_prof_ring->push_back(r);
   }
-  g_prof_on = on != 0;
+  g_prof_n = 0;
+  g_prof_on = true;
   return FLH_OK;
 }
 
-int flh_prof_last_us(double* us) {
-  if (!us) return fl_set_error(FLH_E_ARG, "null out");
-  if (!g_prof_ev1) return fl_set_error(FLH_E_STATE, "profiling was never enabled on this thread");
-  FL_HIP(hipEventSynchronize(g_prof_ev1));
-  float ms = 0.f;
-  FL_HIP(hipEventElapsedTime(&ms, g_prof_ev0, g_prof_ev1));
-  *us = (double)ms * 1e3;
-  return FLH_OK;
+int flh_prof_end(double* us_out, int* kernel_out, int max) {
+  g_prof_on = false;
+  if (!g_prof_ring) return fl_set_error(FLH_E_STATE, "no profiling region was opened on this thread");
+  const size_t n = g_prof_n;
+  for (size_t i = 0; i < n; ++i) {
+    ProfRec& r = (*g_prof_ring)[i];
+    FL_HIP(hipEventSynchronize(r.e1));
+    float ms = 0.f;
+    FL_HIP(hipEventElapsedTime(&ms, r.e0, r.e1));
+    if ((int)i < max) {
+      if (us_out) us_out[i] = (double)ms * 1e3;
+      if (kernel_out) kernel_out[i] = r.kid;
+    }
+  }
+  g_prof_n = 0;
+  return (int)n;
 }
 
 int flh_tune(const char* key, int64_t value) {
   if (!key) return fl_set_error(FLH_E_ARG, "null key");
   if (!strcmp(key, "grid_per_cu")) { if (value < 1) return fl_set_error(FLH_E_ARG, "grid_per_cu < 1"); g_grid_per_cu = (int)value; return FLH_OK; }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value != 0; return FLH_OK; }
+  if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
+  if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 5) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..5"); g_sched_variant = (int)value; return FLH_OK; }
   return fl_set_error(FLH_E_ARG, "unknown tunable %s", key);
 }
@@ -746,6 +991,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   }
   int rc = need_init();
   if (rc) return rc;
+  g_prof_kid = 1;
   SchedArgs a;
   a.sizes = p->d_sizes;
   a.total_bytes = p->total_bytes;
@@ -769,6 +1015,15 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   a.tile_shift = (p->tile_bytes & (p->tile_bytes - 1)) == 0 ? __builtin_ctz(p->tile_bytes) : -1;
   const uint32_t n = p->n_chunks;
   const int variant = g_sched_variant;
+  // ordinary message split with quantum-sized chunks: closed form, no scan
+  if (g_sched_uniform_fast && variant == 0 && n > 0 && !p->d_sizes && !p->d_src_off && p->quantum == p->chunk_bytes &&
+      p->n_rows <= (uint32_t)kRowCache) {
+    const uint32_t grid = (n + kUniBlock - 1) / kUniBlock;
+    FL_LAUNCH((fl_schedule_uniform_kernel<0>), dim3(grid), dim3(kUniBlock), 0, s, a);
+    if (grid > 1 && p->d_state) FL_LAUNCH((fl_schedule_uniform_kernel<1>), dim3(1), dim3(kUniBlock), 0, s, a);
+    FL_HIP(hipGetLastError());
+    return FLH_OK;
+  }
   if ((variant == 0 && n <= kWave) || variant == 1) {
     FL_LAUNCH((fl_schedule_kernel<1, 1>), dim3(1), dim3(kWave), 0, s, a);
   } else if ((variant == 0 && n <= 4 * kWave) || variant == 2) {
@@ -810,6 +1065,7 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   if (n_chunks_max == 0) return FLH_OK;
   rc = need_init();
   if (rc) return rc;
+  g_prof_kid = dir == 0 ? 2 : 3;
   CopyArgs a;
   a.user = (uint8_t*)user;
   a.user_bytes = user_bytes;
@@ -825,8 +1081,20 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   a.hint_uniform_tiles = h_hdr ? h_hdr->uniform_tiles : 0;
   const uint64_t max_tiles = h_hdr ? h_hdr->total_tiles : user_bytes / tile_bytes + n_chunks_max;
   if (max_tiles == 0) return FLH_OK;
-  const uint32_t grid = copy_grid(max_tiles);
   hipStream_t s = (hipStream_t)stream;
+  if (h_hdr && h_hdr->uniform_tiles && h_hdr->n_chunks <= 65535 && h_hdr->n_chunks <= n_chunks_max && g_copy_uniform_grid) {
+    const dim3 grid(h_hdr->uniform_tiles, h_hdr->n_chunks);
+    if (dir == 0) {
+      if (g_nontemporal) FL_LAUNCH((fl_copy_uniform<0, true>), grid, dim3(kCopyBlock), 0, s, a);
+      else FL_LAUNCH((fl_copy_uniform<0, false>), grid, dim3(kCopyBlock), 0, s, a);
+    } else {
+      if (g_nontemporal) FL_LAUNCH((fl_copy_uniform<1, true>), grid, dim3(kCopyBlock), 0, s, a);
+      else FL_LAUNCH((fl_copy_uniform<1, false>), grid, dim3(kCopyBlock), 0, s, a);
+    }
+    FL_HIP(hipGetLastError());
+    return FLH_OK;
+  }
+  const uint32_t grid = copy_grid(max_tiles);
   if (dir == 0) {
     if (g_nontemporal) FL_LAUNCH((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
     else FL_LAUNCH((fl_copy_tiles<0, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
@@ -861,6 +1129,7 @@ static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t
   if (!d_table) return fl_set_error(FLH_E_ARG, "d_table missing");
   rc = need_init();
   if (rc) return rc;
+  g_prof_kid = dir == 0 ? 4 : 5;
   PageArgs a;
   a.pool = (uint8_t*)pool;
   a.pool_pages = pool_pages;
@@ -908,6 +1177,7 @@ int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
   if (!d_dst || !d_src) return fl_set_error(FLH_E_ARG, "null pointer");
   int rc = need_init();
   if (rc) return rc;
+  g_prof_kid = 6;
   const uint32_t tile = FLH_TILE_BYTES;
   const uint32_t grid = copy_grid((bytes + tile - 1) / tile);
   hipStream_t s = (hipStream_t)stream;

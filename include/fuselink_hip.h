@@ -106,12 +106,14 @@ int64_t flh_constant(int which);
  * workgroups launched per compute unit, "nontemporal" = 0/1 streaming loads and stores.
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL. */
 int flh_tune(const char* key, int64_t value);
-/* Per-kernel timing for measurement code (no counterpart in the reference).  While enabled on the
- * calling thread, every launch made through this library carries its own start/stop HIP events
- * that bracket the kernel alone; flh_prof_last_us waits for the last such launch and returns its
- * duration in microseconds. */
-int flh_prof_enable(int on);
-int flh_prof_last_us(double* us);
+/* Per-kernel timing for measurement code (no counterpart in the reference).  Between
+ * flh_prof_begin and flh_prof_end every launch this thread makes through the library carries its
+ * own start/stop HIP events that bracket the kernel alone; the launches stay asynchronous.
+ * flh_prof_end waits for them and returns how many were recorded, filling up to `max` durations
+ * (microseconds) and the entry point that launched each: 1 schedule, 2 stripe, 3 reassemble,
+ * 4 gather, 5 scatter, 6 copy.  Launches beyond `capacity` are not timed. */
+int flh_prof_begin(int capacity);
+int flh_prof_end(double* us_out, int* kernel_out, int max);
 
 /* ---- scheduler ------------------------------------------------------------------------------
  * Replaces FuseLinkConnManager::refreshRxComm / bidTxChannel (src/fuselink.h:153-156, 230-238) and

@@ -229,3 +229,59 @@ def test_roundtrip_with_host_hint(fl):
     exp_w = ob.cpu_stripe(src_np, exp_t, caps)
     for l in range(8):
         np.testing.assert_array_equal(wins[l].cpu().numpy()[: caps[l]], exp_w[l][: caps[l]])
+
+
+@pytest.mark.parametrize("fast", [1, 0])
+@pytest.mark.parametrize("seed", range(8))
+def test_schedule_uniform_closed_form_and_scan_agree_with_oracle(fl, seed, fast):
+    """Quantum-sized chunks take the closed-form kernel (fast=1) or are forced through the scan
+    kernel (fast=0); both must equal the oracle, with epochs, empty credit rows, carried state and
+    every mode bit in play."""
+    core, torch = fl
+    core.tune("sched_uniform_fast", fast)
+    try:
+        rng = np.random.default_rng(1000 + seed)
+        lanes = int(rng.integers(1, 17))
+        rows = int(rng.integers(1, 33))
+        chunk = int(rng.choice([128, 4096, 65536, 100 * 128]))
+        n = int(rng.choice([1, 2, 255, 256, 257, 1000, 3000]))
+        total = n * chunk - int(rng.integers(0, chunk))
+        credits = rng.integers(0, 9, size=(rows, lanes)).astype(np.uint32)
+        credits[rng.integers(0, rows)] = 0
+        epoch_len = int(rng.choice([0, 1, 8, 100, 1000]))
+        st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+        st["chunk_index"] = int(rng.integers(0, 5000))
+        st["epoch_bytes"] = int(rng.integers(0, 50)) * chunk + int(rng.integers(0, chunk))
+        st["lane_off"][:] = rng.integers(0, 1 << 36, size=16)
+        for mode in (0, ob.SCHED_RESET_OFFSETS, ob.SCHED_MIRROR, 4, 5):
+            _check_schedule(fl, n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                            epoch_len=epoch_len, state=st, mode=mode, src_base=int(rng.integers(0, 1 << 20)),
+                            tile_bytes=int(rng.choice([128, 4096, 32768, 3 * 128])))
+        _check_schedule(fl, n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk, epoch_len=epoch_len)
+    finally:
+        core.tune("sched_uniform_fast", 1)
+
+
+def test_schedule_chain_of_calls_matches_one_shot(fl):
+    # a message scheduled in pieces with the device-resident state equals the one-shot table
+    core, torch = fl
+    rng = np.random.default_rng(77)
+    chunk, lanes, E = 4096, 5, 37
+    credits = rng.integers(0, 5, size=(3, lanes)).astype(np.uint32)
+    pieces = [10 * chunk, 600 * chunk, chunk, 300 * chunk + 5]
+    whole_t, _, whole_s = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=sum(pieces),
+                                             chunk_bytes=chunk, epoch_len=E)
+    d_credits = _dev(torch, credits.view(np.int32))
+    state = core.new_state()
+    got, base = [], 0
+    for nb in pieces:
+        sched = core.schedule(n_lanes=lanes, credits=d_credits, quantum=chunk, total_bytes=nb, chunk_bytes=chunk, epoch_len=E,
+                              state=state, src_base=base)
+        torch.cuda.synchronize()
+        got.append(sched.table_numpy())
+        base += nb
+    cat = np.concatenate(got)
+    for f in ("src_off", "win_off", "len", "lane", "epoch"):
+        np.testing.assert_array_equal(cat[f], whole_t[f], err_msg=f)
+    s = core.state_numpy(state)
+    assert s["chunk_index"] == whole_s["chunk_index"] and (s["lane_off"] == whole_s["lane_off"]).all()
