@@ -28,9 +28,11 @@ WORKLOADS = {
     "cfg5_stress_1GiB_64KiB_16lanes": (1 << 30, 64 << 10, 16, 17, 1000),
 }
 
-# HBM bytes per launch of the striping kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until such a run has been recorded for the workload.
-MEASURED_TRAFFIC = {}
+# HBM bytes per launch of the striping kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size
+# (fetch x1.9984, write x1.0000): 65666 KiB fetched + 65536 KiB written.  None where no such run
+# has been recorded for the workload.
+MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134350828}
 
 
 def main() -> int:
@@ -185,7 +187,7 @@ def main() -> int:
                        "plain_copy_same_bytes": round(copy_us, 2)},
         "stripe_reassemble_pair_GBps": round(algo_bytes_step / (pair_us * 1e-6) / 1e9, 1),
         "scheduler_us_per_1k_chunks": round(sched_us * n_sched_launches / (n_chunks / 1000.0), 3),
-        "roofline": {"bound": "hbm", "kernel": "fl_copy_tiles<0> (stripe)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": "fl_copy_uniform<0> (stripe)" if hint is not None else "fl_copy_tiles<0> (stripe)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC.get(args.workload)},
     }
