@@ -61,7 +61,11 @@ def build_harness(verbose: bool = True) -> str | None:
     if not os.path.exists(src):
         return None
     out = os.path.join(ROOT, "tests", "harness", "plugin_harness")
-    cmd = [hipcc(), "-O2", "-std=c++17", "-pthread", "-I" + os.path.join(ROOT, "include"), src, "-o", out, "-ldl"]
+    # host code only: the HIP runtime is used for device buffers, no kernels are compiled here
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [shutil.which("g++") or "g++", "-O2", "-std=c++17", "-pthread", "-D__HIP_PLATFORM_AMD__",
+           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(rocm, "include"), src, "-o", out,
+           "-L" + os.path.join(rocm, "lib"), "-Wl,-rpath," + os.path.join(rocm, "lib"), "-lamdhip64", "-ldl"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -1,0 +1,52 @@
+"""The C++ plugin harness (two proxy threads, dlopen + dlsym like a communication library)."""
+import json
+import os
+import subprocess
+
+import pytest
+
+from fuselink_amd import build
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "harness", "plugin_harness")
+
+
+def _run(args, env=None):
+    if not os.path.exists(BIN):
+        build.build_harness(verbose=False)
+    e = dict(os.environ)
+    e.update(env or {})
+    res = subprocess.run([BIN, build.lib_path(), *args], capture_output=True, text=True, timeout=300, env=e)
+    assert res.returncode == 0, res.stderr[-2000:]
+    return json.loads(res.stdout.strip().splitlines()[-1])
+
+
+@pytest.mark.parametrize("version", [6, 7, 8])
+def test_harness_host_memory_two_threads(version):
+    out = _run(["--host", "--bytes", str(16 << 20), "--request", str(1 << 20), "--inflight", "4", "--iters", "2",
+                "--version", str(version)])
+    assert out["bit_exact"] and out["requests"] == 16 and out["name"] == "FuseLink"
+
+
+def test_harness_cfg1_host_reference_operating_point():
+    # 4 MiB uint8 message, 512 KiB requests (one NCCL step each), as the reference's experiment drives the plugin
+    out = _run(["--host", "--bytes", str(4 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "3"],
+               env={"NCCL_FUSELINK_LANES": "2", "NCCL_FUSELINK_CREDITS": "1,1"})
+    assert out["bit_exact"] and out["requests"] == 8 and out["devices"] == 2
+
+
+@pytest.mark.gpu
+def test_harness_device_memory_cfg2_shape():
+    out = _run(["--bytes", str(64 << 20), "--request", str(64 << 20), "--inflight", "1", "--iters", "5"],
+               env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "28",
+                    "NCCL_FUSELINK_CREDITS": "8,6,7,1,8,7,3,3"})
+    assert out["bit_exact"] and out["memory"] == "device"
+    print(out)
+
+
+@pytest.mark.gpu
+def test_harness_device_memory_stress_four_in_flight():
+    out = _run(["--bytes", str(1 << 30), "--request", str(64 << 20), "--inflight", "4", "--iters", "2"],
+               env={"NCCL_FUSELINK_LANES": "16", "NCCL_FUSELINK_CHUNKSIZE": str(64 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "4"})
+    assert out["bit_exact"] and out["requests"] == 16
+    print(out)
