@@ -559,9 +559,16 @@ ncclResult_t launch_transfer(Link* lk, const uint8_t* src, uint8_t* dst, int siz
       p.d_table = lk->d_table;
       p.d_hdr = lk->d_hdr;
       for (int l = 0; l < lanes; ++l) p.inline_credits[l] = credits[l];
+      // what the header will say follows from the split alone, so the copy kernels need not wait for it
+      flh_sched_hdr hint;
+      memset(&hint, 0, sizeof(hint));
+      const uint64_t last_len = wave - (uint64_t)(p.n_chunks - 1) * chunk;
+      hint.n_chunks = p.n_chunks;
+      hint.uniform_tiles = (uint32_t)((chunk + FLH_TILE_BYTES - 1) / FLH_TILE_BYTES);
+      hint.total_tiles = (p.n_chunks - 1) * hint.uniform_tiles + (uint32_t)((last_len + FLH_TILE_BYTES - 1) / FLH_TILE_BYTES);
       FL_FLHCHECK(flh_schedule(&p, lk->stream));
-      FL_FLHCHECK(flh_stripe(src, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, nullptr, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
-      FL_FLHCHECK(flh_reassemble(dst, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, nullptr, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
+      FL_FLHCHECK(flh_stripe(src, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, &hint, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
+      FL_FLHCHECK(flh_reassemble(dst, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, &hint, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
       lk->last_wave_rows = p.n_chunks;
       done += wave;
       first = false;
