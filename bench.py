@@ -1,13 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the FuseLink data path on one MI355X.
 
-One step = the whole hot path over one message: scheduler kernel (chunk -> lane table), striping
-kernel (user buffer -> per-lane HIP-VMM staging windows) and reassembly kernel (windows -> receive
-buffer).  The workload is the headline configuration: a 64 MiB fp16 gradient-bucket buffer
-(N(0,1), seeded), 256 KiB chunks, 8 lanes, lane credits uniform in [1,8] (seeded).  Inputs are
-resident in HBM before the timed region.  Prints one JSON line.
+One step = the whole hot path over one message: chunk -> lane scheduling, striping (user buffer ->
+per-lane HIP-VMM staging windows) and reassembly (windows -> receive buffer).  The default workload
+is the headline configuration: a 64 MiB fp16 gradient-bucket buffer (N(0,1), seeded), 256 KiB chunks,
+8 lanes, lane credits uniform in [1,8] (seeded).  Inputs are resident in HBM before the timed region.
+Prints one JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--path auto|fused|split]
 """
 from __future__ import annotations
 
@@ -23,15 +23,18 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 
 WORKLOADS = {
-    # name: (bytes, chunk bytes, lanes, credit rows, epoch length)
-    "cfg2_grad_bucket_64MiB_256KiB_8lanes": (64 << 20, 256 << 10, 8, 1, 0),
-    "cfg5_stress_1GiB_64KiB_16lanes": (1 << 30, 64 << 10, 16, 17, 1000),
+    # name: (kind, bytes, chunk bytes, lanes, credit rows, epoch length)
+    "cfg2_grad_bucket_64MiB_256KiB_8lanes": ("uniform", 64 << 20, 256 << 10, 8, 1, 0),
+    "cfg5_stress_1GiB_64KiB_16lanes": ("uniform", 1 << 30, 64 << 10, 16, 17, 1000),
+    # 256 variable blocks of 7168-wide bf16 rows, rows ~ Zipf(1.1) capped at 4096; the chunks are the blocks
+    "cfg3_expert_parallel_256_blocks_8lanes": ("blocks", 0, 256 << 10, 8, 1, 0),
+    # K and V pools of 4096 pages of 32 KiB each, seeded page permutation, 128 KiB chunks (4 pages)
+    "cfg4_paged_kv_2x4096_pages_8lanes": ("pages", 2 * 4096 * 32768, 128 << 10, 8, 1, 0),
 }
 
 # HBM bytes per launch of the striping kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
-# WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size
-# (fetch x1.9984, write x1.0000): 65666 KiB fetched + 65536 KiB written.  None where no such run
-# has been recorded for the workload.
+# WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size.
+# None where no such run has been recorded for the workload.
 MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134350828}
 
 
@@ -43,8 +46,10 @@ def main() -> int:
     ap.add_argument("--workload", default="cfg2_grad_bucket_64MiB_256KiB_8lanes", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-iters", type=int, default=60)
-    ap.add_argument("--graph", type=int, default=0, help="replay the step as a HIP graph (1) or launch eagerly (0)")
     ap.add_argument("--hint", type=int, default=1, help="pass the host-known header fields to the copy kernels")
+    ap.add_argument("--path", default="auto", choices=["auto", "fused", "split"],
+                    help="fused: scheduler folded into the striping launch (uniform split, one credit row); split: three launches")
+    ap.add_argument("--lds", type=int, default=0, help="paged workload: stage the gather through LDS")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (every lane's staging window lives on it); "
@@ -61,27 +66,51 @@ def main() -> int:
         return 3
     core.init(0)
     dev = torch.device("cuda:0")
-    nbytes, chunk, lanes, rows, epoch_len = WORKLOADS[args.workload]
-    n_chunks = (nbytes + chunk - 1) // chunk
-
-    # ---- synthetic inputs, resident in HBM ------------------------------------------------------
+    kind, nbytes, chunk, lanes, rows, epoch_len = WORKLOADS[args.workload]
+    rng = np.random.default_rng(20251125)
     gen = torch.Generator(device=dev)
     gen.manual_seed(20251125)
-    if args.workload.startswith("cfg2"):
-        src = torch.randn(nbytes // 2, dtype=torch.float16, device=dev, generator=gen).view(torch.uint8)
-    else:
-        src = torch.randint(0, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device=dev, generator=gen).view(torch.uint8)
-    dst = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
-    rng = np.random.default_rng(20251125)
-    credits_np = rng.integers(1, 9, size=(rows, lanes)).astype(np.int32)
-    credits = torch.from_numpy(credits_np).to(dev)
-
-    # ---- registration-time work (untimed): table once for sizing, windows bound from the VMM pool --
     stream = torch.cuda.Stream(device=dev)
     status = core.new_status(dev)
-    with torch.cuda.stream(stream):
-        sched = core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
-                              epoch_len=epoch_len, stream=stream)
+
+    # ---- synthetic inputs, resident in HBM ------------------------------------------------------
+    sizes_np = None
+    if kind == "blocks":
+        ranks = np.arange(1, 4097, dtype=np.float64)
+        p = ranks ** -1.1
+        rows_per_block = rng.choice(np.arange(1, 4097), size=256, p=p / p.sum())
+        sizes_np = (rows_per_block * 7168 * 2).astype(np.uint32)
+        nbytes = int(sizes_np.sum())
+        credits_np = np.array([[4, 4, 4, 4, 4, 4, 4, 1]], dtype=np.int32)   # one lane at 25 % idleness
+        n_chunks = 256
+    else:
+        credits_np = rng.integers(1, 9, size=(rows, lanes)).astype(np.int32)
+        n_chunks = (nbytes + chunk - 1) // chunk
+    credits = torch.from_numpy(credits_np).to(dev)
+    if args.workload.startswith("cfg2"):
+        src = torch.randn(nbytes // 2, dtype=torch.float16, device=dev, generator=gen).view(torch.uint8)
+    elif kind == "uniform":
+        src = torch.randint(0, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device=dev, generator=gen).view(torch.uint8)
+    else:
+        src = torch.randint(-32768, 32767, (nbytes // 2,), dtype=torch.int16, device=dev, generator=gen).view(torch.uint8)
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    sizes = torch.from_numpy(sizes_np.view(np.int32)).to(dev) if sizes_np is not None else None
+    page_bytes, ppc = 32768, 4
+    tables = None
+    if kind == "pages":
+        half = nbytes // 2
+        tables = [torch.from_numpy(rng.permutation(half // page_bytes).astype(np.int32)).to(dev) for _ in range(2)]
+
+    # ---- registration-time work (untimed): table once for sizing, windows bound from the VMM pool --
+    msg_bytes = nbytes // 2 if kind == "pages" else nbytes    # K and V are two messages over the same windows
+    msg_chunks = n_chunks // 2 if kind == "pages" else n_chunks
+
+    def run_schedule(out=None):
+        return core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, sizes=sizes,
+                             total_bytes=0 if sizes is not None else msg_bytes, chunk_bytes=0 if sizes is not None else chunk,
+                             epoch_len=epoch_len, out=out, stream=stream)
+
+    sched = run_schedule()
     stream.synchronize()
     hdr = sched.hdr_numpy()
     lane_bytes = [int(b) for b in hdr["lane_bytes"][:lanes]]
@@ -95,36 +124,37 @@ def main() -> int:
     win = core.make_windows([w.base for w in windows], [w.bound_bytes for w in windows])
 
     # header fields that follow from the uniform split alone; the kernels then need not wait for d_hdr
-    hint = core.uniform_hint(nbytes, chunk) if args.hint else None
+    hint = core.uniform_hint(msg_bytes, chunk) if (args.hint and kind == "uniform") else None
+    fused = kind == "uniform" and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and n_chunks <= 65535))
+    if fused and (rows != 1 or epoch_len != 0):
+        print("bench.py: the fused path takes a single credit row without epochs", file=sys.stderr)
+        return 2
+    uni = core.uniform_params(nbytes, chunk, credits_np[0].tolist()) if fused else None
 
     def step():
-        core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
-                      epoch_len=epoch_len, out=sched, stream=stream)
-        core.stripe(src, win, sched, status, stream=stream, hint=hint)
-        core.reassemble(dst, win, sched, status, stream=stream, hint=hint)
-
-    graph = None
-    if args.graph:
-        # capture the three launches once; a replay is one host call per step
-        step()
-        stream.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            step()
-
-    def run_step():
-        if graph is not None:
-            with torch.cuda.stream(stream):
-                graph.replay()
+        if kind == "pages":
+            for half_i in range(2):   # K, then V: schedule, gather the pages into the windows, scatter them back out
+                run_schedule(sched)
+                lo = half_i * msg_bytes
+                core.gather_pages(src[lo: lo + msg_bytes], tables[half_i], page_bytes, ppc, win, sched, status,
+                                  use_lds=bool(args.lds), stream=stream)
+                core.scatter_pages(dst[lo: lo + msg_bytes], tables[half_i], page_bytes, ppc, win, sched, status,
+                                   use_lds=bool(args.lds), stream=stream)
+        elif fused:
+            # the striping launch computes each chunk's lane and offset itself and writes the table out
+            core.stripe_uniform(src, win, uni, status, out=sched, stream=stream)
+            core.reassemble_uniform(dst, win, uni, status, stream=stream)
         else:
-            step()
+            run_schedule(sched)
+            core.stripe(src, win, sched, status, stream=stream, hint=hint)
+            core.reassemble(dst, win, sched, status, stream=stream, hint=hint)
 
     for _ in range(args.warmup):
-        run_step()
+        step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        run_step()
+        step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
@@ -140,28 +170,50 @@ def main() -> int:
         fn()
         return core.prof_end(launches)
 
-    def steps_eager():
+    def steps_again():
         for _ in range(args.steps):
             step()
 
-    per = profiled(steps_eager, 4 * args.steps)
+    per = profiled(steps_again, 8 * args.steps)
     mean = lambda xs: sum(xs) / len(xs)
-    sched_us, stripe_us, reasm_us = mean(per["schedule"]), mean(per["stripe"]), mean(per["reassemble"])
-    stripe_min, reasm_min = min(per["stripe"]), min(per["reassemble"])
-    n_sched_launches = len(per["schedule"]) // args.steps
+    out_k, in_k = ("gather", "scatter") if kind == "pages" else ("stripe", "reassemble")
+    stripe_us, reasm_us = mean(per[out_k]), mean(per[in_k])
+    stripe_min, reasm_min = min(per[out_k]), min(per[in_k])
+    launches_per_step = len(per[out_k]) // args.steps
+    if fused:
+        # the table the fused launch wrote must be the scheduler kernel's table
+        fused_table = sched.table_numpy().tobytes()
+
+        def scheds():
+            for _ in range(args.steps):
+                run_schedule(sched)
+
+        per_s = profiled(scheds, 2 * args.steps)
+        assert sched.table_numpy().tobytes() == fused_table, "fused and standalone scheduler tables differ"
+        sched_us, n_sched = mean(per_s["schedule"]), len(per_s["schedule"]) // args.steps
+    else:
+        sched_us, n_sched = mean(per["schedule"]), len(per["schedule"]) // args.steps
 
     def copies():
         for _ in range(min(args.steps, 100)):
-            core.copy(dst, src, stream=stream)
+            core.copy(dst[:msg_bytes], src[:msg_bytes], stream=stream)
 
     copy_us = mean(profiled(copies, 128)["copy"])
     assert torch.equal(src, dst)
 
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
-    algo_bytes_kernel = 2 * nbytes        # one launch of the copy kernel
+    algo_bytes_kernel = 2 * msg_bytes     # one launch of the copy kernel
     value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
-    pair_us = stripe_us + reasm_us
+    pair_us = (stripe_us + reasm_us) * launches_per_step
     achieved = algo_bytes_kernel / (stripe_us * 1e-6) / 1e9
+    if kind == "pages":
+        kernel_name = f"fl_page_tiles<0, lds={args.lds}> (gather)"
+    elif fused:
+        kernel_name = "fl_copy_uniform_fused<0> (stripe)"
+    elif hint is not None:
+        kernel_name = "fl_copy_uniform<0> (stripe)"
+    else:
+        kernel_name = "fl_copy_tiles<0> (stripe)"
 
     out = {
         "metric": "stripe+reassemble GB/s, 64 MiB over 8 lanes" if args.workload.startswith("cfg2") else "stripe+reassemble GB/s",
@@ -176,18 +228,20 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "config": {"workload": args.workload, "bytes": nbytes, "chunk_bytes": chunk, "chunks": n_chunks, "lanes": lanes,
-                   "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
-                   "step": "schedule+stripe+reassemble", "launch": "hipGraph replay" if graph is not None else "eager",
-                   "windows": "HIP VMM, 2 MiB units"},
+        "config": {"workload": args.workload, "bytes": nbytes, "chunk_bytes": chunk if sizes is None else "variable", "chunks": n_chunks,
+                   "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
+                   "step": ("2x(schedule+gather+scatter)" if kind == "pages" else
+                            "stripe(with scheduler folded in)+reassemble" if fused else "schedule+stripe+reassemble"),
+                   "launch": "eager", "windows": "HIP VMM, 2 MiB units"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
-        "kernels_us": {"schedule": round(sched_us, 2), "stripe": round(stripe_us, 2), "reassemble": round(reasm_us, 2),
-                       "stripe_min": round(stripe_min, 2), "reassemble_min": round(reasm_min, 2),
+        "kernels_us": {"schedule": round(sched_us, 2), out_k: round(stripe_us, 2), in_k: round(reasm_us, 2),
+                       out_k + "_min": round(stripe_min, 2), in_k + "_min": round(reasm_min, 2),
                        "plain_copy_same_bytes": round(copy_us, 2)},
         "stripe_reassemble_pair_GBps": round(algo_bytes_step / (pair_us * 1e-6) / 1e9, 1),
-        "scheduler_us_per_1k_chunks": round(sched_us * n_sched_launches / (n_chunks / 1000.0), 3),
-        "roofline": {"bound": "hbm", "kernel": "fl_copy_uniform<0> (stripe)" if hint is not None else "fl_copy_tiles<0> (stripe)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "scheduler_kernel": "standalone launch, not part of the fused step" if fused else "first launch of every message",
+        "scheduler_us_per_1k_chunks": round(sched_us * n_sched / (n_chunks / 1000.0), 3),
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC.get(args.workload)},
     }
@@ -196,18 +250,37 @@ def main() -> int:
     if not args.no_cpu_baseline:
         from tests import oracle_binding as ob
         src_np = src.cpu().numpy()
-        tab, h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits_np, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
-                                       epoch_len=epoch_len)
-        iters = args.cpu_iters if nbytes <= (64 << 20) else max(3, args.cpu_iters // 16)
-        med1, best1 = ob.cpu_baseline(src_np, tab, h, lanes, threads=1, warm=3, iters=iters)
         cores = ob.lib().fl_cpu_cores()
         thr = min(lanes, cores, 16)
-        medm, bestm = ob.cpu_baseline(src_np, tab, h, lanes, threads=thr, warm=3, iters=iters)
-        out["cpu_baseline"] = {"value": round(algo_bytes_step / med1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
-                               "sample": f"{iters} timed stripe+reassemble passes of the same {nbytes >> 20} MiB message "
-                                         f"(host memcpy per chunk into 2 MiB-aligned lane windows), median; host has {cores} cores"}
-        out["cpu_baseline_per_lane_threads"] = {"value": round(algo_bytes_step / medm / 1e9, 2), "unit": "GB/s", "cores": thr,
-                                                "kind": "port", "sample": "same passes, one pinned thread per lane"}
+        if kind == "pages":
+            tab, h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits_np, quantum=chunk, total_bytes=msg_bytes, chunk_bytes=chunk)
+            caps = h["lane_bytes"][:lanes]
+            ts = []
+            for _ in range(max(3, args.cpu_iters // 12)):
+                c0 = time.perf_counter()
+                for half_i in range(2):
+                    half = src_np[half_i * msg_bytes: (half_i + 1) * msg_bytes]
+                    tb = tables[half_i].cpu().numpy().view(np.uint32)
+                    w_ = ob.cpu_gather_pages(half, tb, page_bytes, ppc, tab, caps)
+                    back = ob.cpu_scatter_pages(msg_bytes, tb, page_bytes, ppc, w_, tab)
+                ts.append(time.perf_counter() - c0)
+                assert (back == half).all()
+            med1 = sorted(ts)[len(ts) // 2]
+            out["cpu_baseline"] = {"value": round(algo_bytes_step / med1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                                   "sample": f"{len(ts)} passes of the same K+V gather/scatter (host memcpy per page; includes "
+                                             f"allocating the host windows each pass), median; host has {cores} cores"}
+        else:
+            tab, h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits_np, quantum=chunk, sizes=sizes_np,
+                                           total_bytes=0 if sizes_np is not None else nbytes,
+                                           chunk_bytes=0 if sizes_np is not None else chunk, epoch_len=epoch_len)
+            iters = args.cpu_iters if nbytes <= (64 << 20) else max(3, args.cpu_iters * (64 << 20) // nbytes)
+            med1, _ = ob.cpu_baseline(src_np, tab, h, lanes, threads=1, warm=3, iters=iters)
+            medm, _ = ob.cpu_baseline(src_np, tab, h, lanes, threads=thr, warm=3, iters=iters)
+            out["cpu_baseline"] = {"value": round(algo_bytes_step / med1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                                   "sample": f"{iters} timed stripe+reassemble passes of the same {nbytes >> 20} MiB message "
+                                             f"(host memcpy per chunk into 2 MiB-aligned lane windows), median; host has {cores} cores"}
+            out["cpu_baseline_per_lane_threads"] = {"value": round(algo_bytes_step / medm / 1e9, 2), "unit": "GB/s", "cores": thr,
+                                                    "kind": "port", "sample": "same passes, one pinned thread per lane"}
     print(json.dumps(out))
     return 0
 

@@ -34,6 +34,12 @@ class SchedParams(C.Structure):
                 ("inline_credits", C.c_uint32 * MAX_LANES)]
 
 
+class UniformParams(C.Structure):
+    _fields_ = [("total_bytes", C.c_uint64), ("src_base", C.c_uint64), ("epoch_bytes", C.c_uint64),
+                ("chunk_bytes", C.c_uint32), ("n_lanes", C.c_uint32), ("tile_bytes", C.c_uint32), ("pad", C.c_uint32),
+                ("credits", C.c_uint32 * MAX_LANES)]
+
+
 class Windows(C.Structure):
     _fields_ = [("base", C.c_void_p * MAX_LANES), ("cap", C.c_uint64 * MAX_LANES), ("n_lanes", C.c_uint32),
                 ("pad", C.c_uint32)]
@@ -49,6 +55,10 @@ SIGNATURES = {
                              C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
     "flh_reassemble": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p,
                                  C.POINTER(SchedHdr), C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
+    "flh_stripe_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,
+                                     C.c_void_p, C.c_void_p, C.c_void_p]),
+    "flh_reassemble_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,
+                                         C.c_void_p]),
     "flh_gather_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),
                                    C.c_void_p, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p]),
     "flh_scatter_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),

@@ -10,7 +10,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from ._lib import MAX_LANES, ChunkDesc, SchedHdr, SchedParams, SchedState, Windows, check
+from ._lib import MAX_LANES, ChunkDesc, SchedHdr, SchedParams, SchedState, UniformParams, Windows, check
 
 TILE_BYTES = 32768
 UNIT_BYTES = 2 * 1024 * 1024
@@ -178,6 +178,34 @@ def reassemble(dst: torch.Tensor, win: Windows, sched: Schedule, status: torch.T
     check(_lib.load().flh_reassemble(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), _ptr(sched.table),
                                      _ptr(sched.hdr), _hint_ref(hint), sched.n_chunks, sched.tile_bytes, _ptr(status),
                                      _stream_ptr(stream)))
+
+
+def uniform_params(total_bytes: int, chunk_bytes: int, credits: Sequence[int], *, src_base: int = 0, epoch_bytes: int = 0,
+                   tile_bytes: int = TILE_BYTES) -> UniformParams:
+    u = UniformParams()
+    u.total_bytes, u.src_base, u.epoch_bytes = total_bytes, src_base, epoch_bytes
+    u.chunk_bytes, u.n_lanes, u.tile_bytes = chunk_bytes, len(credits), tile_bytes
+    for l, c in enumerate(credits):
+        u.credits[l] = int(c)
+    return u
+
+
+def new_schedule_buffers(n_chunks: int, tile_bytes: int = TILE_BYTES, device="cuda") -> Schedule:
+    return Schedule(_dev_bytes(n_chunks * DESC_DTYPE.itemsize, device), _dev_bytes(HDR_DTYPE.itemsize, device), n_chunks, tile_bytes)
+
+
+def stripe_uniform(src: torch.Tensor, win: Windows, u: UniformParams, status: torch.Tensor, out: Optional[Schedule] = None,
+                   stream: Optional[torch.cuda.Stream] = None) -> None:
+    """Scheduler + stripe in one launch (flh_stripe_uniform); `out` receives the table and header."""
+    check(_lib.load().flh_stripe_uniform(_ptr(src), src.numel() * src.element_size(), C.byref(win), C.byref(u),
+                                         _ptr(out.table) if out else None, _ptr(out.hdr) if out else None, _ptr(status),
+                                         _stream_ptr(stream)))
+
+
+def reassemble_uniform(dst: torch.Tensor, win: Windows, u: UniformParams, status: torch.Tensor,
+                       stream: Optional[torch.cuda.Stream] = None) -> None:
+    check(_lib.load().flh_reassemble_uniform(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), C.byref(u),
+                                             _ptr(status), _stream_ptr(stream)))
 
 
 def gather_pages(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int, pages_per_chunk: int, win: Windows,

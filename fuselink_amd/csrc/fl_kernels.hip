@@ -755,6 +755,129 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform(CopyArgs a) {
   if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
 }
 
+// Scheduler and copy in one launch, for the ordinary case of a uniform split under one credit row:
+// the workgroup that copies tile k of chunk c works out the chunk's lane and window offset itself
+// from the closed form (no table row to wait for), and the workgroup of tile 0 also writes the row
+// out, so that the table exists for the receiver and for inspection exactly as the scheduler kernel
+// would have produced it.  Window offsets start at zero (the windows are reused message by message).
+struct FusedArgs {
+  uint8_t* user;
+  uint64_t user_bytes;
+  flh_windows win;
+  flh_chunk_desc* table;     // out (stripe only), may be null
+  flh_sched_hdr* hdr;        // out (stripe only), may be null
+  int32_t* status;
+  uint64_t total_bytes;
+  uint64_t src_base;
+  uint64_t quanta_before;    // quanta of the current epoch already behind chunk 0 (epoch bytes / chunk)
+  uint32_t chunk_bytes;
+  uint32_t n_chunks;
+  uint32_t n_lanes;
+  uint32_t tile_bytes;
+  uint32_t tiles_per_chunk;
+  uint32_t credits[FLH_MAX_LANES];
+};
+
+struct FusedRow {  // inclusive credit prefixes of the one row (equal credits if it is empty)
+  uint64_t pfx[FLH_MAX_LANES];
+  uint64_t W;
+  bool zero;
+};
+
+__device__ __forceinline__ void fused_row(const FusedArgs& a, FusedRow& r) {
+  uint64_t run = 0;
+#pragma unroll
+  for (int l = 0; l < FLH_MAX_LANES; ++l) { if ((uint32_t)l < a.n_lanes) run += a.credits[l]; r.pfx[l] = run; }
+  r.zero = run == 0;
+  if (r.zero) {
+#pragma unroll
+    for (int l = 0; l < FLH_MAX_LANES; ++l) r.pfx[l] = (uint32_t)l < a.n_lanes ? l + 1 : a.n_lanes;
+    run = a.n_lanes;
+  }
+  r.W = run;
+}
+
+// slots y < x that belong to the lane with prefix bounds [K, hi)
+__device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t hi, uint64_t x) {
+  const uint64_t c = hi - K;
+  const uint64_t full = div_u64(x, W);
+  const uint64_t rem = x - full * W;
+  const uint64_t part = rem <= K ? 0 : (rem - K < c ? rem - K : c);
+  return full * c + part;
+}
+
+template <int DIR, bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(FusedArgs a) {
+  const uint32_t c = blockIdx.y;
+  if (c >= a.n_chunks) return;
+  FusedRow r;
+  fused_row(a, r);
+  const uint64_t j = a.quanta_before + c;
+  const uint64_t slot = mod_u64(j, r.W);
+  uint32_t lane = 0;
+  uint64_t K = 0, hi = r.pfx[0];
+#pragma unroll
+  for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
+    if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; }
+  }
+  const uint64_t before = fused_cnt(r.W, K, hi, j) - fused_cnt(r.W, K, hi, a.quanta_before);
+  const uint64_t chunk_off = (uint64_t)c * a.chunk_bytes;
+  const uint64_t rem = a.total_bytes - chunk_off;
+  const uint32_t len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
+  const uint64_t src_off = a.src_base + chunk_off;
+  const uint64_t win_off = before * a.chunk_bytes;
+
+  if (DIR == 0 && blockIdx.x == 0 && threadIdx.x == 0 && a.table) {
+    flh_chunk_desc d;
+    d.src_off = src_off;
+    d.win_off = win_off;
+    d.len = len;
+    d.lane = lane;
+    d.tile_base = c * a.tiles_per_chunk;
+    d.epoch = 0;
+    a.table[c] = d;
+  }
+  if (DIR == 0 && blockIdx.x == 0 && c == 0 && a.hdr) {  // header: per-lane totals in closed form
+    const uint32_t t = threadIdx.x;
+    const uint64_t last = a.n_chunks - 1;
+    const uint64_t len_last = a.total_bytes - last * a.chunk_bytes;
+    if (t < FLH_MAX_LANES) {
+      uint64_t chunks = 0, bytes = 0;
+      if (t < a.n_lanes) {
+        uint64_t k_lo = 0, k_hi = 0;  // selected, not indexed: indexing would push the row into scratch memory
+#pragma unroll
+        for (int l = 0; l < FLH_MAX_LANES; ++l) {
+          if ((uint32_t)l == t) { k_hi = r.pfx[l]; k_lo = l ? r.pfx[l > 0 ? l - 1 : 0] : 0; }
+        }
+        chunks = fused_cnt(r.W, k_lo, k_hi, a.quanta_before + a.n_chunks) - fused_cnt(r.W, k_lo, k_hi, a.quanta_before);
+        const uint64_t slot_last = mod_u64(a.quanta_before + last, r.W);
+        const bool mine = slot_last >= k_lo && slot_last < k_hi;
+        bytes = chunks * a.chunk_bytes - (mine ? a.chunk_bytes - len_last : 0);
+      }
+      a.hdr->lane_bytes[t] = bytes;
+      a.hdr->lane_chunks[t] = (uint32_t)chunks;
+    }
+    if (t == 0) {
+      a.hdr->total_bytes = a.total_bytes;
+      a.hdr->total_tiles = (uint32_t)last * a.tiles_per_chunk + (uint32_t)((len_last + a.tile_bytes - 1) / a.tile_bytes);
+      a.hdr->n_chunks = a.n_chunks;
+      a.hdr->flags = r.zero ? FLH_SCHED_F_NO_CREDIT : 0;
+      a.hdr->uniform_tiles = a.tiles_per_chunk;
+    }
+  }
+
+  const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
+  if (off >= len) return;
+  const uint32_t bytes = (uint32_t)((len - off) < a.tile_bytes ? (len - off) : a.tile_bytes);
+  if (win_off + len > a.win.cap[lane] || src_off + len > a.user_bytes) {
+    if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+    return;
+  }
+  uint8_t* u = a.user + src_off + off;
+  uint8_t* w = (uint8_t*)a.win.base[lane] + win_off + off;
+  if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+}
+
 struct PageArgs {
   uint8_t* pool;
   uint64_t pool_pages;
@@ -831,8 +954,8 @@ thread_local char g_err[512] = "";
 int g_device = -1;
 int g_cus = 0;
 // launch tunables (overridable through NCCL_FUSELINK_* for experiments)
-int g_grid_per_cu = 8;
-int g_nontemporal = 0;
+int g_grid_per_cu = 0;     // 0: one workgroup per tile (up to 2^20)
+int g_nontemporal = -1;   // -1: streaming accesses only when the buffers cannot all sit in the Infinity Cache
 int g_sched_variant = 0;  // 0 = pick the scheduler shape from the chunk count
 int g_sched_uniform_fast = 1;
 int g_copy_uniform_grid = 1;
@@ -920,7 +1043,7 @@ int flh_init(int device) {
   g_cus = prop.multiProcessorCount;
   g_grid_per_cu = (int)env_i64("NCCL_FUSELINK_GRID_PER_CU", g_grid_per_cu);
   g_nontemporal = (int)env_i64("NCCL_FUSELINK_NONTEMPORAL", g_nontemporal);
-  if (g_grid_per_cu < 1) g_grid_per_cu = 1;
+  if (g_grid_per_cu < 0) g_grid_per_cu = 0;
   return FLH_OK;
 }
 
@@ -959,8 +1082,8 @@ int flh_prof_end(double* us_out, int* kernel_out, int max) {
 
 int flh_tune(const char* key, int64_t value) {
   if (!key) return fl_set_error(FLH_E_ARG, "null key");
-  if (!strcmp(key, "grid_per_cu")) { if (value < 1) return fl_set_error(FLH_E_ARG, "grid_per_cu < 1"); g_grid_per_cu = (int)value; return FLH_OK; }
-  if (!strcmp(key, "nontemporal")) { g_nontemporal = value != 0; return FLH_OK; }
+  if (!strcmp(key, "grid_per_cu")) { if (value < 0) return fl_set_error(FLH_E_ARG, "grid_per_cu < 0"); g_grid_per_cu = (int)value; return FLH_OK; }
+  if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 5) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..5"); g_sched_variant = (int)value; return FLH_OK; }
@@ -1047,8 +1170,18 @@ static int check_windows(const flh_windows* win) {
   return FLH_OK;
 }
 
+// Non-temporal loads and stores pay off once the working set (the buffers a transfer touches) is well
+// beyond the 256 MB Infinity Cache (measured: +3-5 % at 1 GiB messages) and cost throughput when a
+// good part of it still fits (-8 % at 64 MiB, -20 % on the read-back side at 128 MiB).
+static bool use_nt(uint64_t working_set_bytes) {
+  if (g_nontemporal >= 0) return g_nontemporal != 0;
+  return working_set_bytes > (512ull << 20);
+}
+
 static uint32_t copy_grid(uint64_t max_tiles) {
-  uint64_t g = (uint64_t)g_cus * (uint64_t)g_grid_per_cu;
+  // one workgroup per tile lets the dispatcher overlap loads and stores of different tiles; the
+  // kernels' stride loops only matter beyond the cap (grid_per_cu can lower it for experiments)
+  uint64_t g = g_grid_per_cu > 0 ? (uint64_t)g_cus * (uint64_t)g_grid_per_cu : (1ull << 20);
   if (g > max_tiles) g = max_tiles;
   if (g < 1) g = 1;
   return (uint32_t)g;
@@ -1082,13 +1215,14 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   const uint64_t max_tiles = h_hdr ? h_hdr->total_tiles : user_bytes / tile_bytes + n_chunks_max;
   if (max_tiles == 0) return FLH_OK;
   hipStream_t s = (hipStream_t)stream;
+  const bool nt = use_nt(3 * user_bytes);  // user buffer + windows + the peer's buffer
   if (h_hdr && h_hdr->uniform_tiles && h_hdr->n_chunks <= 65535 && h_hdr->n_chunks <= n_chunks_max && g_copy_uniform_grid) {
     const dim3 grid(h_hdr->uniform_tiles, h_hdr->n_chunks);
     if (dir == 0) {
-      if (g_nontemporal) FL_LAUNCH((fl_copy_uniform<0, true>), grid, dim3(kCopyBlock), 0, s, a);
+      if (nt) FL_LAUNCH((fl_copy_uniform<0, true>), grid, dim3(kCopyBlock), 0, s, a);
       else FL_LAUNCH((fl_copy_uniform<0, false>), grid, dim3(kCopyBlock), 0, s, a);
     } else {
-      if (g_nontemporal) FL_LAUNCH((fl_copy_uniform<1, true>), grid, dim3(kCopyBlock), 0, s, a);
+      if (nt) FL_LAUNCH((fl_copy_uniform<1, true>), grid, dim3(kCopyBlock), 0, s, a);
       else FL_LAUNCH((fl_copy_uniform<1, false>), grid, dim3(kCopyBlock), 0, s, a);
     }
     FL_HIP(hipGetLastError());
@@ -1096,10 +1230,10 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   }
   const uint32_t grid = copy_grid(max_tiles);
   if (dir == 0) {
-    if (g_nontemporal) FL_LAUNCH((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    if (nt) FL_LAUNCH((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
     else FL_LAUNCH((fl_copy_tiles<0, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
   } else {
-    if (g_nontemporal) FL_LAUNCH((fl_copy_tiles<1, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    if (nt) FL_LAUNCH((fl_copy_tiles<1, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
     else FL_LAUNCH((fl_copy_tiles<1, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
   }
   FL_HIP(hipGetLastError());
@@ -1116,6 +1250,61 @@ int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win, cons
                    const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, uint32_t n_chunks_max, uint32_t tile_bytes,
                    int32_t* d_status, void* stream) {
   return launch_copy(1, d_dst, dst_bytes, win, d_table, d_hdr, h_hdr, n_chunks_max, tile_bytes, d_status, stream);
+}
+
+static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_uniform_params* u,
+                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream) {
+  int rc = check_windows(win);
+  if (rc) return rc;
+  if (!u || !d_status) return fl_set_error(FLH_E_ARG, "parameters and d_status are required");
+  if (u->n_lanes == 0 || u->n_lanes > FLH_MAX_LANES || u->n_lanes != win->n_lanes) return fl_set_error(FLH_E_ARG, "n_lanes %u does not match the windows' %u", u->n_lanes, win->n_lanes);
+  if (u->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0");
+  if (u->tile_bytes == 0 || u->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", u->tile_bytes);
+  if (u->total_bytes == 0) return FLH_OK;
+  if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
+  const uint64_t n = (u->total_bytes + u->chunk_bytes - 1) / u->chunk_bytes;
+  if (n > 65535) return fl_set_error(FLH_E_ARG, "%llu chunks exceed the 65535 one launch can name; split the message", (unsigned long long)n);
+  rc = need_init();
+  if (rc) return rc;
+  g_prof_kid = dir == 0 ? 2 : 3;
+  FusedArgs a;
+  a.user = (uint8_t*)user;
+  a.user_bytes = user_bytes;
+  a.win = *win;
+  a.table = dir == 0 ? d_table : nullptr;
+  a.hdr = dir == 0 ? d_hdr : nullptr;
+  a.status = d_status;
+  a.total_bytes = u->total_bytes;
+  a.src_base = u->src_base;
+  a.quanta_before = u->epoch_bytes / u->chunk_bytes;
+  a.chunk_bytes = u->chunk_bytes;
+  a.n_chunks = (uint32_t)n;
+  a.n_lanes = u->n_lanes;
+  a.tile_bytes = u->tile_bytes;
+  a.tiles_per_chunk = (u->chunk_bytes + u->tile_bytes - 1) / u->tile_bytes;
+  for (int l = 0; l < FLH_MAX_LANES; ++l) a.credits[l] = (uint32_t)l < u->n_lanes ? u->credits[l] : 0;
+  const dim3 grid(a.tiles_per_chunk, a.n_chunks);
+  hipStream_t s = (hipStream_t)stream;
+  const bool nt = use_nt(3 * user_bytes);
+  if (dir == 0) {
+    if (nt) FL_LAUNCH((fl_copy_uniform_fused<0, true>), grid, dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_uniform_fused<0, false>), grid, dim3(kCopyBlock), 0, s, a);
+  } else {
+    if (nt) FL_LAUNCH((fl_copy_uniform_fused<1, true>), grid, dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_uniform_fused<1, false>), grid, dim3(kCopyBlock), 0, s, a);
+  }
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_uniform_params* u,
+                       flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
+  return launch_fused(0, (void*)d_src, src_bytes, win, u, d_table_out, d_hdr_out, d_status, stream);
+}
+
+int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_uniform_params* u,
+                           int32_t* d_status, void* stream) {
+  return launch_fused(1, d_dst, dst_bytes, win, u, nullptr, nullptr, d_status, stream);
 }
 
 static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
@@ -1146,7 +1335,7 @@ static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t
   const uint64_t total = (uint64_t)n_chunks * pages_per_chunk * a.subs_per_page;
   const uint32_t grid = copy_grid(total);
   hipStream_t s = (hipStream_t)stream;
-  const bool nt = g_nontemporal != 0;
+  const bool nt = use_nt(3ull * n_chunks * pages_per_chunk * page_bytes);
 #define FL_LAUNCH_PAGES(D, LD, N) FL_LAUNCH((fl_page_tiles<D, LD, N>), dim3(grid), dim3(kCopyBlock), 0, s, a)
   if (dir == 0) {
     if (use_lds) { if (nt) FL_LAUNCH_PAGES(0, true, true); else FL_LAUNCH_PAGES(0, true, false); }
@@ -1181,7 +1370,7 @@ int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
   const uint32_t tile = FLH_TILE_BYTES;
   const uint32_t grid = copy_grid((bytes + tile - 1) / tile);
   hipStream_t s = (hipStream_t)stream;
-  if (g_nontemporal) FL_LAUNCH(fl_plain_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  if (use_nt(2 * bytes)) FL_LAUNCH(fl_plain_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
   else FL_LAUNCH(fl_plain_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
   FL_HIP(hipGetLastError());
   return FLH_OK;

@@ -103,7 +103,8 @@ const char* flh_last_error(void);
  * 5 sizeof(state), 6 sizeof(hdr), 7 ABI version, 8 sizeof(flh_windows), 9 sizeof(flh_sched_params) */
 int64_t flh_constant(int which);
 /* Launch tunables, for experiments (no counterpart in the reference): "grid_per_cu" = copy
- * workgroups launched per compute unit, "nontemporal" = 0/1 streaming loads and stores.
+ * workgroups launched per compute unit (0 = one per tile), "nontemporal" = 0/1 streaming loads and
+ * stores (-1 = only when the buffers exceed the 256 MB Infinity Cache, the default).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL. */
 int flh_tune(const char* key, int64_t value);
 /* Per-kernel timing for measurement code (no counterpart in the reference).  Between
@@ -148,6 +149,31 @@ int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win,
 int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
                    const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr,
                    uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream);
+
+/* Scheduler and copy in one launch, for a uniform split (R1) under a single credit row with
+ * quantum == chunk_bytes and window offsets starting at 0 -- the shape of every request the plugin
+ * issues.  Each workgroup derives its chunk's lane and window offset from the closed form of the
+ * schedule instead of reading a table row; flh_stripe_uniform also writes the table and header (when
+ * the pointers are given), bit-identical to what flh_schedule produces for the same inputs with
+ * FLH_SCHED_RESET_OFFSETS, state {epoch_bytes, 0, ...} and d_sizes == NULL.  Replaces, in one step,
+ * the lane choice (src/fuselink.h:230-238) and the send / landing of src/plugin.cc:1467-1495, 1582, 1626.
+ * At most 65535 chunks per call. */
+typedef struct flh_uniform_params {
+  uint64_t total_bytes;
+  uint64_t src_base;          /* byte offset of chunk 0 in the user buffer */
+  uint64_t epoch_bytes;       /* bytes already scheduled in the current credit epoch (0 after a refresh) */
+  uint32_t chunk_bytes;       /* chunk size = quantum */
+  uint32_t n_lanes;
+  uint32_t tile_bytes;
+  uint32_t pad;
+  uint32_t credits[FLH_MAX_LANES];
+} flh_uniform_params;
+
+int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows* win,
+                       const flh_uniform_params* u, flh_chunk_desc* d_table_out,
+                       flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
+int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
+                           const flh_uniform_params* u, int32_t* d_status, void* stream);
 
 /* Paged variants for non-contiguous sources (KV-cache blocks, src/experiments/serving/model.hh:
  * 198-201 gives the page shape): chunk c of the table stands for pages

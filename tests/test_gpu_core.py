@@ -285,3 +285,68 @@ def test_schedule_chain_of_calls_matches_one_shot(fl):
         np.testing.assert_array_equal(cat[f], whole_t[f], err_msg=f)
     s = core.state_numpy(state)
     assert s["chunk_index"] == whole_s["chunk_index"] and (s["lane_off"] == whole_s["lane_off"]).all()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_fused_schedule_and_stripe_equals_oracle(fl, seed):
+    """flh_stripe_uniform / flh_reassemble_uniform: the table it writes, the staged windows and the
+    reassembled buffer against the oracle, with carried epoch bytes and an empty credit row."""
+    core, torch = fl
+    rng = np.random.default_rng(500 + seed)
+    lanes = int(rng.integers(1, 17))
+    chunk = int(rng.choice([4096, 65536, 256 << 10, 100 * 128]))
+    n = int(rng.choice([1, 2, 7, 64, 257]))
+    total = n * chunk - int(rng.integers(0, chunk))
+    tile = int(rng.choice([4096, 32768, 3 * 128]))
+    credits = rng.integers(0, 9, size=lanes).astype(np.uint32)
+    if seed == 3:
+        credits[:] = 0
+    epoch_bytes = int(rng.integers(0, 40)) * chunk + int(rng.integers(0, chunk))
+    base = int(rng.integers(0, 8)) * 4096
+    st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+    st["epoch_bytes"] = epoch_bytes
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                         tile_bytes=tile, mode=ob.SCHED_RESET_OFFSETS, state=st, src_base=base)
+    src_np = rng.integers(0, 256, size=base + total, dtype=np.uint8)
+    src = _dev(torch, src_np)
+    caps = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    wins = [torch.zeros(max(c, 1) + 64, dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    u = core.uniform_params(total, chunk, credits, src_base=base, epoch_bytes=epoch_bytes, tile_bytes=tile)
+    out = core.new_schedule_buffers(n, tile)
+    core.stripe_uniform(src, w, u, status, out=out)
+    dst = torch.zeros_like(src)
+    core.reassemble_uniform(dst, w, u, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    got_t, got_h = out.table_numpy(), out.hdr_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f)
+    for f in ("total_bytes", "total_tiles", "n_chunks", "flags", "uniform_tiles", "lane_bytes", "lane_chunks"):
+        np.testing.assert_array_equal(got_h[f], exp_h[f], err_msg=f)
+    exp_w = ob.cpu_stripe(src_np, exp_t, caps)
+    for l in range(lanes):
+        got = wins[l].cpu().numpy()
+        np.testing.assert_array_equal(got[: caps[l]], exp_w[l][: caps[l]])
+        assert not got[caps[l]:].any()
+    got_dst = dst.cpu().numpy()
+    np.testing.assert_array_equal(got_dst[base:], src_np[base:])
+    assert not got_dst[:base].any()
+    # the unfused path produces the same windows from the same table
+    sched = core.schedule(n_lanes=lanes, credits=[int(c) for c in credits], quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                          tile_bytes=tile, mode=core.SCHED_RESET_OFFSETS, src_base=base,
+                          state=_dev(torch, np.array([st], dtype=ob.STATE_DTYPE).view(np.uint8)))
+    torch.cuda.synchronize()
+    assert sched.table_numpy().tobytes() == got_t.tobytes()
+
+
+def test_fused_refuses_short_window(fl):
+    core, torch = fl
+    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device="cuda")
+    wins = [torch.zeros(512 << 10, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    w = core.make_windows([t.data_ptr() for t in wins], [512 << 10, (512 << 10) - 65536])
+    status = core.new_status()
+    core.stripe_uniform(src, w, core.uniform_params(1 << 20, 65536, [1, 1]), status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == -5
