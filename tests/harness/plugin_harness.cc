@@ -3,7 +3,8 @@
 // posting irecv and polling test and one sender thread issuing isend and polling test, with a bounded
 // number of requests in flight.  Verifies the received buffer byte for byte and prints one JSON line.
 //
-//   plugin_harness <lib.so> [--bytes N] [--request N] [--inflight K] [--iters I] [--host] [--version 6|7|8]
+//   plugin_harness <lib.so> [--bytes N] [--request N] [--inflight K] [--iters I] [--host] [--version 6|7|8] [--connections C]
+// With --connections C, C connections run concurrently, each with its own pair of proxy threads and buffers.
 #include <dlfcn.h>
 #include <hip/hip_runtime.h>
 
@@ -33,45 +34,21 @@ static void logger(ncclDebugLogLevel level, unsigned long, const char* file, int
 #define CHECK(x) do { ncclResult_t r_ = (x); if (r_ != ncclSuccess) { fprintf(stderr, "%s -> ncclResult %d (line %d)\n", #x, (int)r_, __LINE__); exit(2); } } while (0)
 #define HIP(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { fprintf(stderr, "%s -> %s\n", #x, hipGetErrorString(e_)); exit(3); } } while (0)
 
-int main(int argc, char** argv) {
-  if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [options]\n", argv[0]); return 1; }
-  size_t bytes = 64u << 20, request = 0;
-  int inflight = 4, iters = 5, host = 0, version = 8;
-  for (int i = 2; i < argc; ++i) {
-    std::string a = argv[i];
-    auto val = [&]() { return i + 1 < argc ? strtoull(argv[++i], nullptr, 0) : 0ull; };
-    if (a == "--bytes") bytes = val();
-    else if (a == "--request") request = val();
-    else if (a == "--inflight") inflight = (int)val();
-    else if (a == "--iters") iters = (int)val();
-    else if (a == "--version") version = (int)val();
-    else if (a == "--host") host = 1;
-  }
-  if (!request || request > bytes) request = bytes;
-  if (request > 0x7fffffffull) request = 0x40000000ull;  // isend takes an int size (src/extern/nccl_net.h:74)
-
-  void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
-  if (!lib) { fprintf(stderr, "dlopen: %s\n", dlerror()); return 1; }
-  // the three tables share their leading slots; v8 is used for everything but regMr's size type
-  ncclNet_v8_t* net8 = (ncclNet_v8_t*)dlsym(lib, "ncclNetPlugin_v8");
-  ncclNet_v7_t* net7 = (ncclNet_v7_t*)dlsym(lib, "ncclNetPlugin_v7");
-  ncclNet_v6_t* net6 = (ncclNet_v6_t*)dlsym(lib, "ncclNetPlugin_v6");
-  if (!net8 || !net7 || !net6) { fprintf(stderr, "plugin symbols missing\n"); return 1; }
-  CHECK(net8->init(logger));
-  int ndev = 0;
-  CHECK(net8->devices(&ndev));
-
+static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclNet_v6_t* net6, size_t bytes, size_t request, int inflight,
+                           int iters, int host, int version, double* best_out, double* total_out) {
+  if (!host) HIP(hipSetDevice(0));
+  const int dev = ci % 2;  // spread the connections over two virtual NICs
   char handle[NCCL_NET_HANDLE_MAXSIZE];
   void *lcomm = nullptr, *scomm = nullptr, *rcomm = nullptr;
-  CHECK(net8->listen(0, handle, &lcomm));
+  CHECK(net8->listen(dev, handle, &lcomm));
   for (int spin = 0; spin < 1000 && (!scomm || !rcomm); ++spin) {
-    if (!scomm) { if (version == 6) CHECK(net6->connect(0, handle, &scomm)); else CHECK(net8->connect(0, handle, &scomm, nullptr)); }
+    if (!scomm) { if (version == 6) CHECK(net6->connect(dev, handle, &scomm)); else CHECK(net8->connect(dev, handle, &scomm, nullptr)); }
     if (!rcomm) { if (version == 6) CHECK(net6->accept(lcomm, &rcomm)); else CHECK(net8->accept(lcomm, &rcomm, nullptr)); }
   }
-  if (!scomm || !rcomm) { fprintf(stderr, "connection did not come up\n"); return 2; }
+  if (!scomm || !rcomm) { fprintf(stderr, "connection did not come up\n"); exit(2); }
 
   std::vector<uint8_t> pattern(bytes);
-  uint64_t x = 88172645463325252ull;
+  uint64_t x = 88172645463325252ull + 7919ull * (uint64_t)ci;
   for (size_t i = 0; i < bytes; ++i) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; pattern[i] = (uint8_t)x; }
   uint8_t *src = nullptr, *dst = nullptr;
   const int type = host ? NCCL_PTR_HOST : NCCL_PTR_CUDA;
@@ -142,7 +119,7 @@ int main(int argc, char** argv) {
     if (s < best) best = s;
     std::vector<uint8_t> back(bytes);
     if (host) memcpy(back.data(), dst, bytes); else HIP(hipMemcpy(back.data(), dst, bytes, hipMemcpyDeviceToHost));
-    if (memcmp(back.data(), pattern.data(), bytes) != 0) { fprintf(stderr, "iteration %d: received buffer differs\n", it); return 5; }
+    if (memcmp(back.data(), pattern.data(), bytes) != 0) { fprintf(stderr, "connection %d iteration %d: received buffer differs\n", ci, it); exit(5); }
     if (host) memset(dst, 0, bytes); else HIP(hipMemset(dst, 0, bytes));
   }
   CHECK(net8->deregMr(scomm, smh));
@@ -150,8 +127,49 @@ int main(int argc, char** argv) {
   CHECK(net8->closeSend(scomm));
   CHECK(net8->closeRecv(rcomm));
   CHECK(net8->closeListen(lcomm));
+  if (host) { free(src); free(dst); } else { HIP(hipFree(src)); HIP(hipFree(dst)); }
+  *best_out = best;
+  *total_out = total / iters;
+}
+
+int main(int argc, char** argv) {
+  if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [options]\n", argv[0]); return 1; }
+  size_t bytes = 64u << 20, request = 0;
+  int inflight = 4, iters = 5, host = 0, version = 8, connections = 1;
+  for (int i = 2; i < argc; ++i) {
+    std::string a = argv[i];
+    auto val = [&]() { return i + 1 < argc ? strtoull(argv[++i], nullptr, 0) : 0ull; };
+    if (a == "--bytes") bytes = val();
+    else if (a == "--request") request = val();
+    else if (a == "--inflight") inflight = (int)val();
+    else if (a == "--iters") iters = (int)val();
+    else if (a == "--version") version = (int)val();
+    else if (a == "--host") host = 1;
+    else if (a == "--connections") connections = (int)val();
+  }
+  if (!request || request > bytes) request = bytes;
+  if (request > 0x7fffffffull) request = 0x40000000ull;  // isend takes an int size (src/extern/nccl_net.h:74)
+
+  void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
+  if (!lib) { fprintf(stderr, "dlopen: %s\n", dlerror()); return 1; }
+  // the three tables share their leading slots; v8 is used for everything but regMr's size type
+  ncclNet_v8_t* net8 = (ncclNet_v8_t*)dlsym(lib, "ncclNetPlugin_v8");
+  ncclNet_v7_t* net7 = (ncclNet_v7_t*)dlsym(lib, "ncclNetPlugin_v7");
+  ncclNet_v6_t* net6 = (ncclNet_v6_t*)dlsym(lib, "ncclNetPlugin_v6");
+  if (!net8 || !net7 || !net6) { fprintf(stderr, "plugin symbols missing\n"); return 1; }
+  CHECK(net8->init(logger));
+  int ndev = 0;
+  CHECK(net8->devices(&ndev));
+
+  std::vector<double> bests(connections, 1e30), totals(connections, 0.0);
+  std::vector<std::thread> conns;
+  for (int ci = 0; ci < connections; ++ci) conns.emplace_back([&, ci]() { run_connection(ci, net8, net7, net6, bytes, request, inflight, iters, host, version, &bests[ci], &totals[ci]); });
+  for (auto& t : conns) t.join();
+  double best = 0, total = 0;
+  for (int ci = 0; ci < connections; ++ci) { if (bests[ci] > best) best = bests[ci]; total += totals[ci] / connections; }
+  const size_t n_req = (bytes + request - 1) / request;
   printf("{\"harness\": \"plugin\", \"name\": \"%s\", \"devices\": %d, \"memory\": \"%s\", \"bytes\": %zu, \"request_bytes\": %zu, \"requests\": %zu, "
-         "\"inflight\": %d, \"iters\": %d, \"best_s\": %.9f, \"mean_s\": %.9f, \"GBps_4N_best\": %.1f, \"bit_exact\": true}\n",
-         net8->name, ndev, host ? "host" : "device", bytes, request, n_req, inflight, iters, best, total / iters, 4.0 * bytes / best / 1e9);
+         "\"inflight\": %d, \"iters\": %d, \"connections\": %d, \"best_s\": %.9f, \"mean_s\": %.9f, \"GBps_4N_best\": %.1f, \"bit_exact\": true}\n",
+         net8->name, ndev, host ? "host" : "device", bytes, request, n_req, inflight, iters, connections, best, total, 4.0 * bytes * connections / best / 1e9);
   return 0;
 }

@@ -50,3 +50,29 @@ def test_harness_device_memory_stress_four_in_flight():
                env={"NCCL_FUSELINK_LANES": "16", "NCCL_FUSELINK_CHUNKSIZE": str(64 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "4"})
     assert out["bit_exact"] and out["requests"] == 16
     print(out)
+
+
+def test_harness_host_four_concurrent_connections():
+    out = _run(["--host", "--bytes", str(8 << 20), "--request", str(1 << 20), "--inflight", "4", "--iters", "3", "--connections", "4"])
+    assert out["bit_exact"] and out["connections"] == 4
+
+
+@pytest.mark.gpu
+def test_harness_device_four_concurrent_connections():
+    # four connections stage through the same unit pool and monitor table at once, each on its own stream
+    out = _run(["--bytes", str(128 << 20), "--request", str(16 << 20), "--inflight", "4", "--iters", "3", "--connections", "4"],
+               env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10)})
+    assert out["bit_exact"] and out["connections"] == 4
+    print(out)
+
+
+def test_plugin_host_path_under_thread_sanitizer():
+    """Four connections, eight proxy threads, host memory: the plugin's request tables, FIFO, registry,
+    credit row and monitor table are touched from all of them; ThreadSanitizer must stay silent."""
+    lib, exe = build.build_tsan(verbose=False)
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1 exitcode=66")
+    res = subprocess.run([exe, lib, "--host", "--bytes", str(4 << 20), "--request", str(256 << 10), "--connections", "4",
+                          "--inflight", "4", "--iters", "2"], capture_output=True, text=True, timeout=600, env=env)
+    assert "ThreadSanitizer" not in res.stderr, res.stderr[-3000:]
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert json.loads(res.stdout.strip().splitlines()[-1])["bit_exact"]
