@@ -1378,16 +1378,18 @@ int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
 
 int flh_qp_split(int size, int nqps, int* off, int* len) {
   if (nqps < 1 || size < 0 || !off || !len) return fl_set_error(FLH_E_ARG, "bad qp split arguments");
-  // stride = ceil(ceil(size / nqps) / 128) * 128; a piece past the end is an empty work request
-  const int per = (size + nqps - 1) / nqps;
-  const int stride = (per + 127) / 128 * 128;
-  for (int q = 0, o = 0; q < nqps; ++q, o += stride) {
-    int l = size - o;
+  // stride = ceil(ceil(size / nqps) / 128) * 128; a piece past the end is an empty work request.
+  // 64-bit inside: the reference's `int` expression overflows for sizes within 127 bytes of INT_MAX.
+  const int64_t per = ((int64_t)size + nqps - 1) / nqps;
+  const int64_t stride = (per + 127) / 128 * 128;
+  int64_t o = 0;
+  for (int q = 0; q < nqps; ++q, o += stride) {
+    int64_t l = (int64_t)size - o;
     if (l > stride) l = stride;
-    off[q] = o;
-    len[q] = l > 0 ? l : 0;
+    off[q] = o > 0x7fffffff ? 0x7fffffff : (int)o;
+    len[q] = l > 0 ? (int)l : 0;
   }
-  return stride;
+  return stride > 0x7fffff80 ? 0x7fffff80 : (int)stride;
 }
 
 }  // extern "C"

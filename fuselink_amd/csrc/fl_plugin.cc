@@ -9,8 +9,8 @@
 //   isend  matches the FIFO head (plugin.cc:1510-1517), checks sizes (1555-1570), splits the request
 //          over QPs in 128-byte-aligned pieces (1467-1495) and then, instead of posting RDMA writes
 //          out of a remapped buffer, queues on the connection's HIP stream, per wave of chunks:
-//          scheduler kernel -> striping kernel (user buffer -> lane staging windows) -> reassembly
-//          kernel (windows -> the posted receive buffer).  The reassembly launch plays the part of the
+//          striping kernel (chunk -> lane scheduling folded in; user buffer -> lane staging windows)
+//          -> reassembly kernel (windows -> the posted receive buffer).  The reassembly launch plays the part of the
 //          RDMA write landing at the receiver; its completion event is the receive completion.
 //   test   polls the request's event (the completion queue of plugin.cc:1801-1955) and, unlike the
 //          reference, reports the byte count of a receive.
@@ -153,7 +153,7 @@ struct Link {
   flh_windows wins = {};
   flh_chunk_desc* d_table = nullptr;
   flh_sched_hdr* d_hdr = nullptr;
-  flh_sched_state* d_state = nullptr;
+  uint64_t epoch_bytes = 0;         // bytes scheduled since the last lane-decision refresh (the scheduler's carried prefix)
   int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
   int32_t* d_status = nullptr;
   uint32_t last_wave_rows = 0;
@@ -220,7 +220,6 @@ void link_unref(Link* lk) {
       if (lk->win[l]) (void)flh_window_destroy(lk->win[l]);
     (void)hipFree(lk->d_table);
     (void)hipFree(lk->d_hdr);
-    (void)hipFree(lk->d_state);
     (void)hipHostFree(lk->h_status);
     (void)hipStreamDestroy(lk->stream);
   }
@@ -274,8 +273,6 @@ ncclResult_t ensure_link_gpu(Link* lk) {
   }
   FL_HIPCHECK(hipMalloc((void**)&lk->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
   FL_HIPCHECK(hipMalloc((void**)&lk->d_hdr, sizeof(flh_sched_hdr)));
-  FL_HIPCHECK(hipMalloc((void**)&lk->d_state, sizeof(flh_sched_state)));
-  FL_HIPCHECK(hipMemsetAsync(lk->d_state, 0, sizeof(flh_sched_state), lk->stream));
   FL_HIPCHECK(hipHostMalloc((void**)&lk->h_status, sizeof(int32_t), hipHostMallocMapped));
   *lk->h_status = 0;
   FL_HIPCHECK(hipHostGetDevicePointer((void**)&lk->d_status, lk->h_status, 0));
@@ -544,32 +541,22 @@ ncclResult_t launch_transfer(Link* lk, const uint8_t* src, uint8_t* dst, int siz
     while (done < piece) {
       uint64_t wave = (uint64_t)per_wave * chunk;
       if (wave > piece - done) wave = piece - done;
-      flh_sched_params p;
-      memset(&p, 0, sizeof(p));
-      p.total_bytes = wave;
-      p.chunk_bytes = (uint32_t)chunk;
-      p.src_base = (uint64_t)qoff[q] + done;
-      p.n_chunks = (uint32_t)((wave + chunk - 1) / chunk);
-      p.n_lanes = (uint32_t)lanes;
-      p.n_rows = 1;
-      p.quantum = chunk;
-      p.tile_bytes = FLH_TILE_BYTES;
-      p.mode = FLH_SCHED_RESET_OFFSETS | ((first && (w.flags & 1u)) ? FLH_SCHED_NEW_EPOCH : 0u);
-      p.d_state = lk->d_state;
-      p.d_table = lk->d_table;
-      p.d_hdr = lk->d_hdr;
-      for (int l = 0; l < lanes; ++l) p.inline_credits[l] = credits[l];
-      // what the header will say follows from the split alone, so the copy kernels need not wait for it
-      flh_sched_hdr hint;
-      memset(&hint, 0, sizeof(hint));
-      const uint64_t last_len = wave - (uint64_t)(p.n_chunks - 1) * chunk;
-      hint.n_chunks = p.n_chunks;
-      hint.uniform_tiles = (uint32_t)((chunk + FLH_TILE_BYTES - 1) / FLH_TILE_BYTES);
-      hint.total_tiles = (p.n_chunks - 1) * hint.uniform_tiles + (uint32_t)((last_len + FLH_TILE_BYTES - 1) / FLH_TILE_BYTES);
-      FL_FLHCHECK(flh_schedule(&p, lk->stream));
-      FL_FLHCHECK(flh_stripe(src, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, &hint, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
-      FL_FLHCHECK(flh_reassemble(dst, (uint64_t)size, &lk->wins, lk->d_table, lk->d_hdr, &hint, p.n_chunks, FLH_TILE_BYTES, lk->d_status, lk->stream));
-      lk->last_wave_rows = p.n_chunks;
+      // One credit row, quantum-sized chunks, windows reused from offset 0: the striping launch works out
+      // every chunk's lane and window offset itself (and writes the table), the reassembly launch likewise.
+      if (first && (w.flags & 1u)) lk->epoch_bytes = 0;   // the receiver refreshed its lane decision: new credit epoch
+      flh_uniform_params u;
+      memset(&u, 0, sizeof(u));
+      u.total_bytes = wave;
+      u.src_base = (uint64_t)qoff[q] + done;
+      u.epoch_bytes = lk->epoch_bytes;
+      u.chunk_bytes = (uint32_t)chunk;
+      u.n_lanes = (uint32_t)lanes;
+      u.tile_bytes = FLH_TILE_BYTES;
+      for (int l = 0; l < lanes; ++l) u.credits[l] = credits[l];
+      FL_FLHCHECK(flh_stripe_uniform(src, (uint64_t)size, &lk->wins, &u, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
+      FL_FLHCHECK(flh_reassemble_uniform(dst, (uint64_t)size, &lk->wins, &u, lk->d_status, lk->stream));
+      lk->epoch_bytes += wave;
+      lk->last_wave_rows = (uint32_t)((wave + chunk - 1) / chunk);
       done += wave;
       first = false;
     }

@@ -266,3 +266,52 @@ def test_region_is_shared_and_refcounted(net):
     assert rc == 0
     net.deregMr(r, mh)
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_largest_request_an_int_can_name(net):
+    # isend/irecv sizes are `int` (src/extern/nccl_net.h:74): 2 GiB - 1 bytes in one request, waves reuse the windows
+    import torch
+    size = (1 << 31) - 1
+    net.reconfigure(NCCL_FUSELINK_LANES=16, NCCL_FUSELINK_CHUNKSIZE=512 << 10, NCCL_FUSELINK_WINDOW_UNITS=4)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(9)
+    src = torch.randint(0, 2**31 - 1, ((1 << 31) // 4,), dtype=torch.int32, device="cuda", generator=gen).view(torch.uint8)
+    dst = torch.zeros_like(src)
+    lcomm, s, r = net.connect_pair(0)
+    _, smh = net.regMr(s, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA)
+    _, rmh = net.regMr(r, dst.data_ptr(), dst.numel(), P.NCCL_PTR_CUDA)
+    _send_recv(net, s, r, src, dst, size, 11, smh, rmh)
+    assert torch.equal(src[:size], dst[:size]) and int(dst[size]) == 0
+    net.deregMr(s, smh), net.deregMr(r, rmh)
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_epoch_prefix_carries_across_requests_until_refresh(net):
+    """The byte prefix that picks the slot runs on from request to request and restarts when the receiver
+    refreshes its lane decision (every REFRESH_BATCH completions): tables against the oracle's carried state."""
+    import torch
+    chunk = 64 << 10
+    net.reconfigure(NCCL_FUSELINK_LANES=4, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_REFRESH_BATCH=3)
+    credits = [3, 1, 2, 2]
+    net.set_credits(credits)
+    src = torch.randint(0, 255, (4 << 20,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    lcomm, s, r = net.connect_pair(0)
+    _, smh = net.regMr(s, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA)
+    _, rmh = net.regMr(r, dst.data_ptr(), dst.numel(), P.NCCL_PTR_CUDA)
+    sizes = [5 * chunk, 3 * chunk + 100, 7 * chunk, 2 * chunk, 9 * chunk - 1, chunk, 4 * chunk]
+    prefix = 0
+    for k, size in enumerate(sizes):
+        if k % 3 == 0:
+            prefix = 0                      # refresh: a new credit epoch
+        dst.zero_()
+        _send_recv(net, s, r, src, dst, size, k, smh, rmh)
+        assert torch.equal(src[:size], dst[:size])
+        rows, hdr = net.last_table(s)
+        exp_t, exp_h, _ = ob.credit_schedule(n_lanes=4, credits=credits, quantum=chunk, total_bytes=size, chunk_bytes=chunk,
+                                             mode=ob.SCHED_RESET_OFFSETS, state=_state(prefix, 0))
+        _same_table(rows, exp_t)
+        np.testing.assert_array_equal(hdr["lane_bytes"], exp_h["lane_bytes"])
+        prefix += size
+    net.deregMr(s, smh), net.deregMr(r, rmh)
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
