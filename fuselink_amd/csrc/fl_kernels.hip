@@ -627,6 +627,15 @@ __device__ __forceinline__ void st16(u32x4* p, u32x4 v) {
   if (NT) __builtin_nontemporal_store(v, p); else *p = v;
 }
 
+template <bool NT, int U>
+__device__ __forceinline__ void copy_exact(u32x4* __restrict__ d, const u32x4* __restrict__ s, uint32_t tid) {
+  u32x4 r[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) r[j] = ld16<NT>(s + j * kCopyBlock + tid);
+#pragma unroll
+  for (int j = 0; j < U; ++j) st16<NT>(d + j * kCopyBlock + tid, r[j]);
+}
+
 // Copies `bytes` from src to dst with the whole workgroup.  Fast path: both 16-byte aligned ->
 // dwordx4 loads batched kCopyUnroll deep before the stores.  Equal misalignment: byte head up to
 // the boundary, vectors, byte tail.  Different misalignment: byte copy (correct, not fast).
@@ -646,17 +655,23 @@ __device__ __forceinline__ void block_copy(uint8_t* __restrict__ dst, const uint
   const uint32_t nvec = body >> 4;
   const u32x4* s = (const u32x4*)(src + head);
   u32x4* d = (u32x4*)(dst + head);
-  for (uint32_t b = 0; b < nvec; b += kCopyBlock * kCopyUnroll) {
-    u32x4 r[kCopyUnroll];
+  // whole tiles of the usual sizes: every load of the tile is issued before the first store, unpredicated
+  if (nvec == kCopyBlock * 16) { copy_exact<NT, 16>(d, s, tid); }
+  else if (nvec == kCopyBlock * 8) { copy_exact<NT, 8>(d, s, tid); }
+  else if (nvec == kCopyBlock * 4) { copy_exact<NT, 4>(d, s, tid); }
+  else {
+    for (uint32_t b = 0; b < nvec; b += kCopyBlock * kCopyUnroll) {
+      u32x4 r[kCopyUnroll];
 #pragma unroll
-    for (int j = 0; j < kCopyUnroll; ++j) {
-      const uint32_t idx = b + j * kCopyBlock + tid;
-      if (idx < nvec) r[j] = ld16<NT>(s + idx);
-    }
+      for (int j = 0; j < kCopyUnroll; ++j) {
+        const uint32_t idx = b + j * kCopyBlock + tid;
+        if (idx < nvec) r[j] = ld16<NT>(s + idx);
+      }
 #pragma unroll
-    for (int j = 0; j < kCopyUnroll; ++j) {
-      const uint32_t idx = b + j * kCopyBlock + tid;
-      if (idx < nvec) st16<NT>(d + idx, r[j]);
+      for (int j = 0; j < kCopyUnroll; ++j) {
+        const uint32_t idx = b + j * kCopyBlock + tid;
+        if (idx < nvec) st16<NT>(d + idx, r[j]);
+      }
     }
   }
   const uint32_t tail0 = head + (nvec << 4);
