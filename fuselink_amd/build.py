@@ -99,6 +99,23 @@ def build_tsan(verbose: bool = True):
     return lib, exe
 
 
+def monitor_path() -> str:
+    return os.path.join(LIBDIR, "fuselink-monitor")
+
+
+def build_monitor(verbose: bool = True) -> str:
+    """The lane-idleness daemon (host code only)."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    cmd = [shutil.which("g++") or "g++", "-O2", "-std=c++17", "-pthread", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+           os.path.join(CSRC, "fl_monitor.cc"), os.path.join(CSRC, "fl_monitor_main.cc"), "-o", monitor_path(), "-lrt"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("monitor build failed:\n" + res.stderr)
+    return monitor_path()
+
+
 def build_oracle(verbose: bool = True) -> None:
     """Compiles the CPU oracle (test infrastructure) and, where the reference tree is present,
     the reference's own monitor client under oracle/_ref."""
@@ -114,6 +131,7 @@ def build_oracle(verbose: bool = True) -> None:
 
 def build_all(verbose: bool = True) -> None:
     build_library(verbose)
+    build_monitor(verbose)
     build_harness(verbose)
     build_oracle(verbose)
 

@@ -2,10 +2,20 @@
 //
 // The reference keeps this state in POSIX shared memory owned by a daemon (FuseLink
 // src/monitor.h:47-55, src/monitor.cpp:159-193) and guards every access with a named semaphore.
-// Here the table lives in the plugin's process behind a mutex and the clock is an argument, so the
-// state machine is deterministic: the transport marks a lane active when it puts traffic on it, a
-// tick ages lanes to IDLE after MONITOR_TIMEOUT_US, and the scheduler's credits are read off the
-// statuses at each refresh.
+// The table here has the same layout and can live in two places:
+//   * in the plugin's process behind a mutex (the default), with the clock passed in, so that the
+//     state machine is deterministic;
+//   * in the reference's shared-memory object (`/rdma_monitor_shm`, guarded by the named semaphore
+//     `/rdma_monitor_sem`), after fl_monitor_attach_shm(): then several processes -- this library,
+//     the fuselink-monitor daemon, the reference's own MonitorClient -- see one table.
+// The transport marks a lane active when it puts traffic on it, a tick ages lanes to IDLE after
+// MONITOR_TIMEOUT_US, and the scheduler's credits are read off the statuses at each refresh.
+#include <fcntl.h>
+#include <semaphore.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
 #include <chrono>
 #include <cstring>
 #include <mutex>
@@ -19,19 +29,112 @@ namespace {
 constexpr int kGroups = FL_NET_MAX_LANES;  // NGROUP with NNIC_PER_GROUP == 1 (src/monitor.h:18-20)
 enum : int32_t { kIdle = 0, kBusy = 1, kBorrowed = 2 };  // NicStatus, src/monitor.h:40-44
 
+// struct SharedMemory of src/monitor.h:47-55 with NGROUP = 16, NNIC_PER_GROUP = 1: two status arrays,
+// two timestamp arrays (microseconds of the steady clock), the daemon's running flag.
 struct LaneTable {
-  int32_t status[2][kGroups];        // [0] rx, [1] tx
-  int64_t last_active[2][kGroups];   // microseconds
+  int32_t tx_status[kGroups];
+  int32_t rx_status[kGroups];
+  int64_t tx_last_active[kGroups];
+  int64_t rx_last_active[kGroups];
+  volatile uint8_t running;
 };
+static_assert(offsetof(LaneTable, rx_status) == 64 && offsetof(LaneTable, tx_last_active) == 128 &&
+              offsetof(LaneTable, rx_last_active) == 256 && offsetof(LaneTable, running) == 384 && sizeof(LaneTable) == 392,
+              "layout must match the reference's SharedMemory");
 
-std::mutex g_mu;
-LaneTable g_tab = {};
+std::mutex g_mu;            // guards the pointers below and, in process-local mode, the table
+LaneTable g_local = {};
+LaneTable* g_tab = &g_local;
+sem_t* g_sem = SEM_FAILED;  // the cross-process lock when attached
+int g_shm_fd = -1;
+bool g_owner = false;
+char g_shm_name[64] = "", g_sem_name[64] = "";
 bool g_manual_clock = false;
 int64_t g_manual_now = 0;
+
+// every access to the table goes through one of these
+struct TableLock {
+  std::unique_lock<std::mutex> local;
+  sem_t* sem;
+  TableLock() : local(g_mu), sem(g_sem) {
+    if (sem != SEM_FAILED) {
+      while (sem_wait(sem) != 0) {}
+    }
+  }
+  ~TableLock() {
+    if (sem != SEM_FAILED) sem_post(sem);
+  }
+};
+
+int32_t* status_of(int is_tx) { return is_tx ? g_tab->tx_status : g_tab->rx_status; }
+int64_t* stamp_of(int is_tx) { return is_tx ? g_tab->tx_last_active : g_tab->rx_last_active; }
+
+void detach_locked() {
+  if (g_tab != &g_local) munmap(g_tab, sizeof(LaneTable));
+  g_tab = &g_local;
+  if (g_shm_fd >= 0) close(g_shm_fd);
+  g_shm_fd = -1;
+  if (g_sem != SEM_FAILED) sem_close(g_sem);
+  g_sem = SEM_FAILED;
+  if (g_owner) {
+    shm_unlink(g_shm_name);
+    sem_unlink(g_sem_name);
+  }
+  g_owner = false;
+}
 
 }  // namespace
 
 extern "C" {
+
+int fl_monitor_attach_shm(const char* shm_name, const char* sem_name, int create) {
+  if (!shm_name) shm_name = "/rdma_monitor_shm";  // SHM_NAME, src/monitor.h:23
+  if (!sem_name) sem_name = "/rdma_monitor_sem";  // SEM_NAME, src/monitor.h:24
+  if (strlen(shm_name) >= sizeof(g_shm_name) || strlen(sem_name) >= sizeof(g_sem_name)) return fl_set_error(FLH_E_ARG, "name too long");
+  std::lock_guard<std::mutex> g(g_mu);
+  detach_locked();
+  if (create) {  // the daemon's part (Monitor::setupSharedMemory in src/monitor.cpp)
+    shm_unlink(shm_name);
+    sem_unlink(sem_name);
+  }
+  int fd = shm_open(shm_name, create ? (O_CREAT | O_RDWR) : O_RDWR, 0666);
+  if (fd < 0) return fl_set_error(FLH_E_STATE, "shm_open(%s) failed: is the monitor daemon running?", shm_name);
+  if (create && ftruncate(fd, sizeof(LaneTable)) != 0) { close(fd); return fl_set_error(FLH_E_STATE, "ftruncate failed"); }
+  struct stat st;
+  if (fstat(fd, &st) != 0 || (size_t)st.st_size < sizeof(LaneTable)) { close(fd); return fl_set_error(FLH_E_STATE, "%s is smaller than the monitor table", shm_name); }
+  void* p = mmap(nullptr, sizeof(LaneTable), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+  if (p == MAP_FAILED) { close(fd); return fl_set_error(FLH_E_STATE, "mmap of %s failed", shm_name); }
+  sem_t* sem = create ? sem_open(sem_name, O_CREAT, 0666, 1) : sem_open(sem_name, 0);
+  if (sem == SEM_FAILED) { munmap(p, sizeof(LaneTable)); close(fd); return fl_set_error(FLH_E_STATE, "sem_open(%s) failed", sem_name); }
+  g_tab = (LaneTable*)p;
+  g_shm_fd = fd;
+  g_sem = sem;
+  g_owner = create != 0;
+  strcpy(g_shm_name, shm_name);
+  strcpy(g_sem_name, sem_name);
+  if (create) {
+    memset(g_tab, 0, sizeof(LaneTable));
+    g_tab->running = 1;
+  }
+  return FLH_OK;
+}
+
+int fl_monitor_detach(void) {
+  std::lock_guard<std::mutex> g(g_mu);
+  if (g_owner && g_tab != &g_local) g_tab->running = 0;
+  detach_locked();
+  return FLH_OK;
+}
+
+int fl_monitor_is_shared(void) {
+  std::lock_guard<std::mutex> g(g_mu);
+  return g_tab != &g_local;
+}
+
+int fl_monitor_daemon_running(void) {
+  TableLock l;
+  return g_tab != &g_local && g_tab->running != 0;
+}
 
 int fl_monitor_set_clock(int manual, int64_t now_us) {
   std::lock_guard<std::mutex> g(g_mu);
@@ -40,6 +143,7 @@ int fl_monitor_set_clock(int manual, int64_t now_us) {
   return FLH_OK;
 }
 
+// get_timestamp() of src/monitor.h:29-33 unless a test has frozen the clock
 int64_t fl_monitor_now(void) {
   {
     std::lock_guard<std::mutex> g(g_mu);
@@ -49,44 +153,45 @@ int64_t fl_monitor_now(void) {
 }
 
 int fl_monitor_reset(void) {
-  std::lock_guard<std::mutex> g(g_mu);
-  memset(&g_tab, 0, sizeof(g_tab));
+  TableLock l;
+  const uint8_t running = g_tab->running;
+  memset(g_tab, 0, sizeof(LaneTable));
+  g_tab->running = running;
   return FLH_OK;
 }
 
 // markNicTxAsActive / markNicRxAsActive (src/monitor.h:236-250)
 int fl_monitor_mark_active(int lane, int is_tx, int64_t now_us) {
   if (lane < 0 || lane >= kGroups) return fl_set_error(FLH_E_ARG, "lane %d out of range", lane);
-  std::lock_guard<std::mutex> g(g_mu);
-  const int d = is_tx ? 1 : 0;
-  g_tab.last_active[d][lane] = now_us;
-  g_tab.status[d][lane] = kBusy;
+  TableLock l;
+  stamp_of(is_tx)[lane] = now_us;
+  status_of(is_tx)[lane] = kBusy;
   return FLH_OK;
 }
 
 int fl_monitor_set_entry(int lane, int is_tx, int32_t status, int64_t last_active_us) {
   if (lane < 0 || lane >= kGroups || status < kIdle || status > kBorrowed) return fl_set_error(FLH_E_ARG, "bad table entry");
-  std::lock_guard<std::mutex> g(g_mu);
-  g_tab.status[is_tx ? 1 : 0][lane] = status;
-  g_tab.last_active[is_tx ? 1 : 0][lane] = last_active_us;
+  TableLock l;
+  status_of(is_tx)[lane] = status;
+  stamp_of(is_tx)[lane] = last_active_us;
   return FLH_OK;
 }
 
 // Monitor::monitorThread body (src/monitor.cpp:164-188): a lane whose last activity is at least the
 // timeout old becomes IDLE, whatever it was (BUSY or BORROWED); a younger one keeps its status.
 int fl_monitor_tick(int64_t now_us) {
-  std::lock_guard<std::mutex> g(g_mu);
+  TableLock l;
   for (int d = 0; d < 2; ++d)
     for (int i = 0; i < kGroups; ++i)
-      if (!(g_tab.last_active[d][i] + FL_NET_MONITOR_TIMEOUT_US > now_us)) g_tab.status[d][i] = kIdle;
+      if (!(stamp_of(d)[i] + FL_NET_MONITOR_TIMEOUT_US > now_us)) status_of(d)[i] = kIdle;
   return FLH_OK;
 }
 
 // getNICStatus (src/monitor.h:226-234), for either direction
 int fl_monitor_status(int is_tx, int n_lanes, int32_t* status_out) {
   if (n_lanes < 0 || n_lanes > kGroups || !status_out) return fl_set_error(FLH_E_ARG, "bad status query");
-  std::lock_guard<std::mutex> g(g_mu);
-  for (int i = 0; i < n_lanes; ++i) status_out[i] = g_tab.status[is_tx ? 1 : 0][i];
+  TableLock l;
+  for (int i = 0; i < n_lanes; ++i) status_out[i] = status_of(is_tx)[i];
   return FLH_OK;
 }
 
@@ -94,14 +199,14 @@ int fl_monitor_status(int is_tx, int n_lanes, int32_t* status_out) {
 // the one-iteration inner loop, so the scan goes on: every idle NIC outside `group` that the mask
 // admits is marked BORROWED and the last of them is returned.  exact != 0 stops at the first.
 int fl_monitor_idle_pick(int is_tx, int group, int mask, int exact) {
-  std::lock_guard<std::mutex> g(g_mu);
-  const int d = is_tx ? 1 : 0;
+  TableLock l;
+  int32_t* st = status_of(is_tx);
   int found = -1;
   for (int i = 0; i < kGroups; ++i) {
     if (i == group) continue;
     if (!is_tx && (mask & (1 << i)) == 0) continue;  // only the rx query takes a mask (src/monitor.h:214)
-    if (g_tab.status[d][i] != kIdle) continue;
-    g_tab.status[d][i] = kBorrowed;
+    if (st[i] != kIdle) continue;
+    st[i] = kBorrowed;
     found = i;
     if (exact) break;
   }
@@ -110,8 +215,8 @@ int fl_monitor_idle_pick(int is_tx, int group, int mask, int exact) {
 
 int fl_monitor_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t* credits_out) {
   if (n_lanes < 1 || n_lanes > kGroups || !credits_out) return fl_set_error(FLH_E_ARG, "bad credit query");
-  std::lock_guard<std::mutex> g(g_mu);
-  for (int l = 0; l < n_lanes; ++l) credits_out[l] = g_tab.status[1][l] == kIdle ? idle_credit : 0;
+  TableLock l;
+  for (int i = 0; i < n_lanes; ++i) credits_out[i] = g_tab->tx_status[i] == kIdle ? idle_credit : 0;
   if (own_lane >= 0 && own_lane < n_lanes && credits_out[own_lane] == 0) credits_out[own_lane] = 1;
   return FLH_OK;
 }

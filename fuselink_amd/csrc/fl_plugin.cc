@@ -338,6 +338,11 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   }
   if ((int64_t)g_par.window_units * FLH_UNIT_BYTES < g_par.chunk) { FL_WARN("NET/FuseLink : a staging window must hold at least one chunk"); return ncclInvalidArgument; }
   parse_credit_env();
+  if (fl_param("FUSELINK_MONITOR_SHM", 0)) {
+    // lane statuses come from the daemon's shared table, as in FuseLinkConnManager::SetUpMonitor (fuselink.h:99-101);
+    // an absent daemon is an error here instead of the exception MonitorClient throws (monitor.h:113-131)
+    if (fl_monitor_attach_shm(nullptr, nullptr, 0) != 0) { FL_WARN("NET/FuseLink : %s", flh_last_error()); return ncclSystemError; }
+  }
   g_inited = true;
   FL_INFO(NCCL_INIT | NCCL_NET, "NET/FuseLink : %d lanes, chunk %lld, policy %s, refresh every %d requests (loopback wire)", g_par.lanes,
           (long long)g_par.chunk, g_par.policy ? "credits" : "static", g_par.refresh_batch);
@@ -721,6 +726,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   *done = 1;                                                // plugin.cc:1807-1823
   if (r->type == kReqSend) { lk->s_finished++; lk->s_inflight--; }
   if (r->type == kReqRecv) {
+    (void)fl_monitor_mark_active(lk->dev % g_par.lanes, 0, fl_monitor_now());   // updateRxChannelActive, fuselink.h:254-259
     lk->r_finished++;
     lk->r_inflight--;
     if (sizes) sizes[0] = r->size;   // the reference leaves 0 here (plugin.cc:1726, 1882)
@@ -827,6 +833,7 @@ int fl_net_reset(void) {
   }
   g_par = Params();
   g_inited = false;
+  if (fl_monitor_is_shared()) fl_monitor_detach();  // back to the process-local table until init attaches again
   return FLH_OK;
 }
 

@@ -71,7 +71,7 @@ def _table(version: int):
 
 
 PLUGIN_SYMBOLS = ["ncclNetPlugin_v8", "ncclNetPlugin_v7", "ncclNetPlugin_v6"]
-CONTROL_SYMBOLS = ["fl_monitor_reset", "fl_monitor_set_entry", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
+CONTROL_SYMBOLS = ["fl_monitor_attach_shm", "fl_monitor_detach", "fl_monitor_is_shared", "fl_monitor_daemon_running", "fl_monitor_reset", "fl_monitor_set_entry", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
                    "fl_monitor_status", "fl_monitor_idle_pick", "fl_monitor_credits", "fl_net_set_credits",
                    "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_last_table", "fl_net_reset"]
 
@@ -98,6 +98,7 @@ class NetPlugin:
         self._logger = LOGGER(_logger)
         L = self.lib
         L.fl_monitor_reset.restype = C.c_int
+        L.fl_monitor_attach_shm.argtypes = [C.c_char_p, C.c_char_p, C.c_int]
         L.fl_monitor_set_clock.argtypes = [C.c_int, C.c_int64]
         L.fl_monitor_now.restype = C.c_int64
         L.fl_monitor_mark_active.argtypes = [C.c_int, C.c_int, C.c_int64]

@@ -194,6 +194,16 @@ extern ncclNet_v6_t ncclNetPlugin_v6;
  * clock passed in so that it is deterministic: mark = (timestamp, BUSY); tick = every NIC whose
  * timestamp + 160 us <= now becomes IDLE; pick = borrow an idle NIC of another group. */
 int fl_monitor_reset(void);
+/* Move the table into POSIX shared memory guarded by a named semaphore, the reference's arrangement
+ * (src/monitor.h:23-24, 47-55; NULL names = "/rdma_monitor_shm", "/rdma_monitor_sem").  create = 1
+ * makes and owns the objects (the daemon's part), create = 0 attaches to existing ones as the
+ * reference's MonitorClient constructor does (src/monitor.h:110-133) and fails with FLH_E_STATE when
+ * they are absent.  The layout is the reference's SharedMemory, so its client and this library can
+ * share one table.  fl_monitor_detach returns to the process-local table. */
+int fl_monitor_attach_shm(const char* shm_name, const char* sem_name, int create);
+int fl_monitor_detach(void);
+int fl_monitor_is_shared(void);
+int fl_monitor_daemon_running(void);
 /* Clock of the plugin's own marks and ticks: manual = 0 (default) reads the steady clock as
  * get_timestamp() does (src/monitor.h:29-33); manual = 1 freezes it at now_us until the next call,
  * which makes every lane decision reproducible. */

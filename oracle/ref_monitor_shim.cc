@@ -38,6 +38,22 @@ int ref_mon_open() {
   return 0;
 }
 
+// attach the reference's client to shared memory that somebody else (a daemon) created
+int ref_mon_attach() {
+  if (g_client) return 0;
+  try {
+    g_client = new MonitorClient();
+  } catch (...) {
+    return -5;
+  }
+  return 0;
+}
+
+void ref_mon_detach() {
+  delete g_client;
+  g_client = nullptr;
+}
+
 void ref_mon_close() {
   delete g_client;
   g_client = nullptr;
