@@ -24,6 +24,7 @@
 namespace {
 
 constexpr int kWave = 64;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // DPP controls of the GFX9 ISA: row_shr:n = 0x110+n, row_bcast:15 = 0x142, row_bcast:31 = 0x143.
 template <int CTRL>
@@ -144,35 +145,71 @@ __device__ __forceinline__ uint64_t mod_u64(uint64_t a, uint64_t b) {
   return ((a | b) >> 32) == 0 ? (uint64_t)((uint32_t)a % (uint32_t)b) : a - div_u64_wide(a, b) * b;
 }
 
+// Credit rows -> inclusive prefixes, four rows per wavefront: a row of at most 16 lanes fills one
+// 16-lane DPP row, so four row_shr steps scan it and rows never mix.  `raw` holds the rows in LDS.
+// A row without any credit (every lane busy) is replaced by equal credits -- the round robin of the
+// static policy -- and marked in zero[].
+template <int BT>
+__device__ __forceinline__ void credit_row_prefixes(const uint32_t* raw, uint32_t R, uint32_t L, int tid,
+                                                    uint64_t (*pfx)[FLH_MAX_LANES], uint32_t* zero) {
+  const int lane = tid & (kWave - 1);
+  const uint32_t sub = (uint32_t)lane & 15u;
+#pragma unroll 1
+  for (uint32_t r0 = 0; r0 < R; r0 += BT / 16) {
+    const uint32_t r = r0 + (uint32_t)tid / 16u;
+    const bool live = r < R && sub < L;
+    uint64_t v = live ? raw[r * L + sub] : 0u;
+    { uint64_t t = dpp_u64<0x111>(v); if (sub >= 1) v += t; }
+    { uint64_t t = dpp_u64<0x112>(v); if (sub >= 2) v += t; }
+    { uint64_t t = dpp_u64<0x114>(v); if (sub >= 4) v += t; }
+    { uint64_t t = dpp_u64<0x118>(v); if (sub >= 8) v += t; }
+    const int top = (lane | 15) << 2;
+    const uint32_t wlo = (uint32_t)__builtin_amdgcn_ds_bpermute(top, (int)(uint32_t)v);
+    const uint32_t whi = (uint32_t)__builtin_amdgcn_ds_bpermute(top, (int)(uint32_t)(v >> 32));
+    const bool none = (wlo | whi) == 0;
+    if (none) v = sub + 1;
+    if (live) pfx[r][sub] = v;
+    if (r < R && sub == 0) zero[r] = none;
+  }
+}
+
 template <typename T> __device__ __forceinline__ T wave_incl_sum(T v, int lane);
 template <> __device__ __forceinline__ uint32_t wave_incl_sum<uint32_t>(uint32_t v, int lane) { return wave_incl_sum_u32(v, lane); }
 template <> __device__ __forceinline__ uint64_t wave_incl_sum<uint64_t>(uint64_t v, int lane) { return wave_incl_sum_u64(v, lane); }
 
-// In-wavefront part of the window offsets: for every lane l in turn, scan the threads' bytes on l
-// and hand each chunk on l its exclusive position; the wavefront's total per lane goes to LDS.
+// In-wavefront part of the window offsets: for every lane l, scan the threads' bytes on l and hand
+// each chunk on l its exclusive position.  Four lanes go through the scan side by side so that their
+// DPP chains overlap (a lone wavefront per SIMD has nothing else to hide that latency with).  The
+// wavefront's total of lane l is parked in thread l and goes to LDS once at the end.
 // T is the width of the partial sums (32 bits when the whole pass moves less than 4 GiB).
 template <typename T, int K>
 __device__ __forceinline__ void lane_pass(const uint32_t (&s)[K], const uint32_t (&ln)[K], uint32_t L, int lane,
-                                          uint64_t* w_lane_row, uint32_t* cnt_lane, uint64_t (&off)[K]) {
+                                          uint64_t* w_lane_row, uint64_t (&off)[K]) {
+  constexpr int G = 4;
+  uint64_t my_total = 0;
 #pragma unroll 1
-  for (uint32_t l = 0; l < L; ++l) {
-    T v = 0;
-    uint32_t c = 0;
+  for (uint32_t l0 = 0; l0 < L; l0 += G) {
+    T v[G], inc[G];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-      const bool mine = ln[k] == l;
-      v += mine ? (T)s[k] : (T)0;
-      c += (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(mine));
-    }
-    const T inc = wave_incl_sum<T>(v, lane);
-    uint64_t ex = (uint64_t)(inc - v);
+    for (int g = 0; g < G; ++g) {
+      v[g] = 0;
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-      if (ln[k] == l) { off[k] = ex; ex += s[k]; }
+      for (int k = 0; k < K; ++k) v[g] += ln[k] == l0 + g ? (T)s[k] : (T)0;
     }
-    if (lane == kWave - 1) w_lane_row[l] = (uint64_t)inc;
-    if (lane == 0 && c) atomicAdd(&cnt_lane[l], c);
+#pragma unroll
+    for (int g = 0; g < G; ++g) inc[g] = wave_incl_sum<T>(v[g], lane);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      uint64_t ex = (uint64_t)(inc[g] - v[g]);
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        if (ln[k] == l0 + g) { off[k] = ex; ex += s[k]; }
+      }
+      const uint64_t tot = sizeof(T) == 8 ? bcast_lane_u64((uint64_t)inc[g], kWave - 1) : (uint64_t)bcast_lane_u32((uint32_t)inc[g], kWave - 1);
+      if ((uint32_t)lane == l0 + g) my_total = tot;
+    }
   }
+  if ((uint32_t)lane < L) w_lane_row[lane] = my_total;
 }
 
 // One workgroup of NW wavefronts walks the chunk list in passes of NW*64*K chunks; thread t owns K
@@ -190,6 +227,9 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   // credit rows as inclusive prefixes; row r occupies rowpfx[r][0..L), W = rowpfx[r][L-1]
   __shared__ uint64_t rowpfx[kRowCache][FLH_MAX_LANES];
   __shared__ uint32_t rowzero[kRowCache];  // the row had no credit at all
+  // the same prefixes in 32 bits, entries past L-1 saturated, for rows whose credits sum below 2^32
+  __shared__ __attribute__((aligned(16))) uint32_t rowpfx32[kRowCache][FLH_MAX_LANES];
+  __shared__ uint32_t rows_wide;  // some row sums to 2^32 or more: use the 64-bit prefixes
   __shared__ uint64_t w_seg_v[NW];
   __shared__ uint32_t w_seg_f[NW];
   __shared__ uint64_t w_run[NW];
@@ -209,24 +249,37 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   if (rows_cached) {
     // all credit rows in one round trip to memory, then one wavefront scan per row out of LDS
     for (uint32_t e = tid; e < a.n_rows * L; e += BT) raw[e] = a.credits ? a.credits[e] : a.inline_credits[e];
-    __syncthreads();
-    for (uint32_t r = wave; r < a.n_rows; r += NW) {
-      const uint32_t c = (uint32_t)lane < L ? raw[r * L + lane] : 0;
-      uint64_t inc = wave_incl_sum_u64(c, lane);
-      const bool zero = bcast_lane_u64(inc, kWave - 1) == 0;
-      if (zero) inc = (uint32_t)lane < L ? lane + 1 : L;
-      if ((uint32_t)lane < L) rowpfx[r][lane] = inc;
-      if (lane == 0) rowzero[r] = zero;
-    }
   }
+  // the carried state and the first pass's sizes are requested before anything waits on the credit rows,
+  // so that the kernel pays one round trip to memory, not three in a row
   uint64_t k0 = 0, p_carry = 0, run_carry = 0;  // carried state, identical in every thread
   uint32_t tiles_carry = 0;
   if (a.state) {
     k0 = a.state->chunk_index;
     if (!(a.mode & FLH_SCHED_NEW_EPOCH)) p_carry = a.state->epoch_bytes;
   }
+  uint64_t off_in = 0;
+  if (tid < FLH_MAX_LANES && a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS)) off_in = a.state->lane_off[tid];
+  uint32_t s_next[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const uint32_t i = (uint32_t)tid * K + k;
+    s_next[k] = (a.sizes && i < a.n) ? a.sizes[i] : 0;
+  }
+  if (rows_cached) {
+    __syncthreads();
+    credit_row_prefixes<BT>(raw, a.n_rows, L, tid, rowpfx, rowzero);
+    if (tid == 0) rows_wide = 0;
+    __syncthreads();
+    for (uint32_t e = tid; e < a.n_rows * FLH_MAX_LANES; e += BT) {
+      const uint32_t r = e / FLH_MAX_LANES, l = e % FLH_MAX_LANES;
+      const uint64_t v = l + 1 < L ? rowpfx[r][l] : ~0ull;  // the last prefix is W > slot: never counted
+      rowpfx32[r][l] = v >> 32 ? 0xffffffffu : (uint32_t)v;
+      if (l == L - 1 && (rowpfx[r][l] >> 32)) rows_wide = 1;
+    }
+  }
   if (tid < FLH_MAX_LANES) {
-    const uint64_t o = (a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS)) ? a.state->lane_off[tid] : 0;
+    const uint64_t o = off_in;
     lane_off[tid] = o;
     lane_off0[tid] = o;
     cnt_lane[tid] = 0;
@@ -234,6 +287,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   if (tid == 0) sh_flags = 0;
   __syncthreads();
 
+  const bool wide = rows_cached && rows_wide != 0;
 #pragma unroll 1
   for (uint32_t pass = 0; pass < a.n; pass += BT * K) {
     const uint32_t i0 = pass + (uint32_t)tid * K;
@@ -260,7 +314,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
       bool hd = false;
       if (i < a.n) {
         if (a.sizes) {
-          sz = a.sizes[i];
+          sz = s_next[k];
         } else {
           const uint64_t o = (uint64_t)i * a.chunk_bytes;
           const uint64_t rem = o < a.total_bytes ? a.total_bytes - o : 0;
@@ -281,6 +335,13 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
         pos = 0;
         ++e_cur;
         if (++r_cur == a.n_rows) r_cur = 0;
+      }
+    }
+    if (a.sizes) {  // next pass's sizes travel while this pass computes
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const uint64_t i = (uint64_t)i0 + (uint64_t)BT * K + k;
+        s_next[k] = i < a.n ? a.sizes[i] : 0;
       }
     }
     // ---- block-wide exclusive prefixes of (segmented bytes, bytes, tiles) --------------------------
@@ -342,7 +403,14 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
         const uint64_t slot = mod_u64(qn, W);
         // lane = number of inclusive prefixes <= slot (zero-credit lanes repeat the prefix and are skipped)
         uint32_t pick = 0;
-        if (rows_cached) {
+        if (rows_cached && !wide) {
+          const uint32_t slot32 = (uint32_t)slot;  // slot < W < 2^32
+          const u32x4* pr = reinterpret_cast<const u32x4*>(rowpfx32[r]);
+          const u32x4 p0 = pr[0], p1 = pr[1], p2 = pr[2], p3 = pr[3];
+          pick = (p0.x <= slot32) + (p0.y <= slot32) + (p0.z <= slot32) + (p0.w <= slot32) + (p1.x <= slot32) + (p1.y <= slot32) +
+                 (p1.z <= slot32) + (p1.w <= slot32) + (p2.x <= slot32) + (p2.y <= slot32) + (p2.z <= slot32) + (p2.w <= slot32) +
+                 (p3.x <= slot32) + (p3.y <= slot32) + (p3.z <= slot32) + (p3.w <= slot32);
+        } else if (rows_cached) {
 #pragma unroll 1
           for (uint32_t l = 0; l + 1 < L; ++l) pick += rowpfx[r][l] <= slot;
         } else if (equal) {
@@ -353,6 +421,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
           for (uint32_t l = 0; l + 1 < L; ++l) { kk += a.credits[(size_t)r * L + l]; pick += kk <= slot; }
         }
         ln[k] = pick;
+        atomicAdd(&cnt_lane[pick], 1u);  // LDS counter of chunks per lane
         P += s[k];
       }
     }
@@ -360,8 +429,8 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
     uint64_t off[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) off[k] = 0;
-    if ((tot_run >> 32) == 0) lane_pass<uint32_t, K>(s, ln, L, lane, w_lane[wave], cnt_lane, off);
-    else lane_pass<uint64_t, K>(s, ln, L, lane, w_lane[wave], cnt_lane, off);
+    if ((tot_run >> 32) == 0) lane_pass<uint32_t, K>(s, ln, L, lane, w_lane[wave], off);
+    else lane_pass<uint64_t, K>(s, ln, L, lane, w_lane[wave], off);
     __syncthreads();
     if ((uint32_t)tid < L) {
       uint64_t at = lane_off[tid];
@@ -510,21 +579,25 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
   // all credit rows in one round trip to memory, then one wavefront scan per row out of LDS
   __shared__ uint32_t raw[kRowCache * FLH_MAX_LANES];
   for (uint32_t e = tid; e < R * L; e += kUniBlock) raw[e] = a.credits ? a.credits[e] : a.inline_credits[e];
+  // the carried state is requested before anything waits on the credit rows
+  const uint64_t k0_in = a.state ? a.state->chunk_index : 0;
+  const uint64_t p0 = (a.state && !(a.mode & FLH_SCHED_NEW_EPOCH)) ? a.state->epoch_bytes : 0;
   __syncthreads();
-  for (uint32_t r = wave; r < R; r += kUniBlock / kWave) {
-    const uint32_t c = (uint32_t)lane < L ? raw[r * L + lane] : 0;
-    uint64_t inc = wave_incl_sum_u64(c, lane);
-    const bool zero = bcast_lane_u64(inc, kWave - 1) == 0;
-    if (zero) inc = (uint32_t)lane < L ? lane + 1 : L;
-    if ((uint32_t)lane < L) t.pfx[r][lane] = inc;
-    if (lane == 0) t.zero[r] = zero;
+  credit_row_prefixes<kUniBlock>(raw, R, L, tid, t.pfx, t.zero);
+  __syncthreads();
+  // chunks per lane of one whole epoch under each row (all rows at once), then prefixed over the rows
+  for (uint32_t e = tid; e < R * L; e += kUniBlock) {
+    const uint32_t r = e / L, l = e - r * L;
+    t.pf[r + 1][l] = a.epoch_len ? uni_cnt(t, r, l, L, a.epoch_len) : 0;
   }
   __syncthreads();
-  if ((uint32_t)tid < L) {  // chunks per lane of one whole epoch under each row, prefixed over the rows
+  if ((uint32_t)tid < L) {
     uint64_t run = 0;
+#pragma unroll 1
     for (uint32_t r = 0; r < R; ++r) {
+      const uint64_t x = t.pf[r + 1][tid];
       t.pf[r][tid] = run;
-      if (a.epoch_len) run += uni_cnt(t, r, (uint32_t)tid, L, a.epoch_len);
+      run += x;
     }
     t.pf[R][tid] = run;
   }
@@ -535,8 +608,7 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
   c.E = a.epoch_len;
   c.R = R;
   c.L = L;
-  c.k0 = a.state ? a.state->chunk_index : 0;
-  const uint64_t p0 = (a.state && !(a.mode & FLH_SCHED_NEW_EPOCH)) ? a.state->epoch_bytes : 0;
+  c.k0 = k0_in;
   c.e0 = c.E ? div_u64(c.k0, c.E) : 0;
   c.pos0 = c.E ? (uint32_t)(c.k0 - c.e0 * c.E) : 0;
   // quanta already behind the first chunk inside its epoch; an epoch head starts from zero
@@ -613,7 +685,6 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
 // ------------------------------------------------------------------------------------------------
 // copy kernels
 // ------------------------------------------------------------------------------------------------
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kCopyBlock = 256;
 constexpr int kCopyUnroll = 8;
@@ -1101,7 +1172,7 @@ int flh_tune(const char* key, int64_t value) {
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
-  if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 5) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..5"); g_sched_variant = (int)value; return FLH_OK; }
+  if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 4) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..4"); g_sched_variant = (int)value; return FLH_OK; }
   return fl_set_error(FLH_E_ARG, "unknown tunable %s", key);
 }
 
@@ -1162,16 +1233,15 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     FL_HIP(hipGetLastError());
     return FLH_OK;
   }
+  // one workgroup; more chunks per thread once the per-pass overhead stops dominating
   if ((variant == 0 && n <= kWave) || variant == 1) {
     FL_LAUNCH((fl_schedule_kernel<1, 1>), dim3(1), dim3(kWave), 0, s, a);
-  } else if ((variant == 0 && n <= 4 * kWave) || variant == 2) {
+  } else if ((variant == 0 && n <= 8 * kWave) || variant == 2) {
     FL_LAUNCH((fl_schedule_kernel<4, 1>), dim3(1), dim3(4 * kWave), 0, s, a);
-  } else if ((variant == 0 && n <= 16 * kWave) || variant == 3) {
-    FL_LAUNCH((fl_schedule_kernel<16, 1>), dim3(1), dim3(16 * kWave), 0, s, a);
-  } else if (variant == 4) {
+  } else if ((variant == 0 && n <= 32 * kWave) || variant == 3) {
     FL_LAUNCH((fl_schedule_kernel<8, 4>), dim3(1), dim3(8 * kWave), 0, s, a);
   } else {
-    FL_LAUNCH((fl_schedule_kernel<16, 4>), dim3(1), dim3(16 * kWave), 0, s, a);
+    FL_LAUNCH((fl_schedule_kernel<8, 8>), dim3(1), dim3(8 * kWave), 0, s, a);
   }
   FL_HIP(hipGetLastError());
   return FLH_OK;

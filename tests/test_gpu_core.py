@@ -72,6 +72,18 @@ def test_schedule_random_sizes_epochs(fl, seed):
                     tile_bytes=int(rng.choice([4096, 32768])))
 
 
+@pytest.mark.parametrize("lanes", [3, 16])
+def test_schedule_credit_rows_summing_past_32_bits(fl, lanes):
+    """Credits are u32 each, so a row may sum to 2^32 or more: the 64-bit prefixes must take over."""
+    rng = np.random.default_rng(7 + lanes)
+    credits = rng.integers(0, 9, size=(5, lanes)).astype(np.uint32)
+    credits[1] = rng.integers(2**31, 2**32 - 1, size=lanes)  # W of this row needs more than 32 bits
+    credits[3, 0] = 2**32 - 1
+    sizes = rng.integers(1, 1 << 20, size=1500).astype(np.uint32)
+    _check_schedule(fl, n_lanes=lanes, credits=credits, quantum=4096, sizes=sizes, epoch_len=100)
+    _check_schedule(fl, n_lanes=lanes, credits=credits, quantum=65536, total_bytes=3000 * 65536 - 5, chunk_bytes=65536, epoch_len=100)
+
+
 def test_schedule_state_carry_and_modes(fl):
     rng = np.random.default_rng(7)
     st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
