@@ -156,7 +156,7 @@ struct Link {
   uint64_t epoch_bytes = 0;         // bytes scheduled since the last lane-decision refresh (the scheduler's carried prefix)
   int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
   int32_t* d_status = nullptr;
-  uint32_t last_wave_rows = 0;
+  std::atomic<uint32_t> last_wave_rows{0};
 };
 
 struct Comm {
@@ -466,10 +466,11 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
   mh->type = type;
   if (type == NCCL_PTR_CUDA) {
     // whole allocation around the pointer, as cuMemGetAddressRange in plugin.cc:1194
-    FL_HIPCHECK(hipSetDevice(g_par.device));
     void* base = nullptr;
     size_t bsz = 0;
-    hipError_t e = hipMemGetAddressRange((hipDeviceptr_t*)&base, &bsz, (hipDeviceptr_t)data);
+    hipError_t e = hipSetDevice(g_par.device);
+    if (e != hipSuccess) { delete mh; return hip_fail("hipSetDevice", e); }
+    e = hipMemGetAddressRange((hipDeviceptr_t*)&base, &bsz, (hipDeviceptr_t)data);
     if (e != hipSuccess) { delete mh; return hip_fail("hipMemGetAddressRange", e); }
     ncclResult_t rc = ensure_pool();
     if (rc != ncclSuccess) { delete mh; return rc; }
@@ -578,45 +579,59 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
   if (c->magic != kCommMagic || !c->is_send || mh->magic != kMhMagic) return ncclInvalidArgument;
   Link* lk = c->link;
   *request = nullptr;
-  std::lock_guard<std::mutex> g(lk->mu);
-  if (!lk->send_ready) { FL_WARN("NET/FuseLink: isend() called when comm->ready == 0"); return ncclInternalError; }  // plugin.cc:1502
-  // wait for the receiver to have posted the matching receive (plugin.cc:1510-1514)
-  const int slot = (int)(lk->fifoHead % FL_NET_MAX_REQUESTS);
-  FifoSlot& fs = lk->fifo[slot];
-  if (fs.w.idx != lk->fifoHead + 1) return ncclSuccess;
-  if (fs.w.nreqs != 1) { FL_WARN("NET/FuseLink: multi-send not allowed"); return ncclInternalError; }   // plugin.cc:1448-1451
-  if (fs.w.tag != (uint32_t)tag) return ncclSuccess;                                                     // plugin.cc:1552
-  if (size > fs.w.size) {                                                                                // plugin.cc:1555-1562
-    FL_WARN("NET/FuseLink : req tag %x collective mismatch error, local size %d remote size %d", tag, size, fs.w.size);
-    return ncclInvalidUsage;
-  }
-  if (fs.w.size < 0 || fs.w.addr == 0) {                                                                 // plugin.cc:1563-1570
-    FL_WARN("NET/FuseLink : posted incorrect receive info: size %d addr %llx", fs.w.size, (unsigned long long)fs.w.addr);
-    return ncclInternalError;
-  }
-  if (size && !in_handle(mh, data, (size_t)size)) { FL_WARN("NET/FuseLink : send buffer outside its registration"); return ncclInvalidArgument; }
-  Request* sreq = get_request(lk->sreq, lk, kReqSend);
-  if (!sreq) return ncclInternalError;                                                                   // plugin.cc:1082-1084
-  Request* rreq = fs.rreq;
-  sreq->size = size;
-  rreq->size = size;
-  uint8_t* dst = (uint8_t*)(uintptr_t)fs.w.addr;
+  // The connection's lock covers the descriptor match and the bookkeeping only.  The GPU work is queued
+  // after it is dropped: one thread drives a send comm (as NCCL's proxy does), so launches on the
+  // connection's stream stay in request order, and the receiver's polling never waits behind a launch.
+  FifoWire w;
+  Request *sreq = nullptr, *rreq = nullptr;
+  int rtype = 0;
   ncclResult_t rc = ncclSuccess;
-  const bool src_dev = mh->type == NCCL_PTR_CUDA, dst_dev = fs.rtype == NCCL_PTR_CUDA;
+  {
+    std::lock_guard<std::mutex> g(lk->mu);
+    if (!lk->send_ready) { FL_WARN("NET/FuseLink: isend() called when comm->ready == 0"); return ncclInternalError; }  // plugin.cc:1502
+    // wait for the receiver to have posted the matching receive (plugin.cc:1510-1514)
+    const int slot = (int)(lk->fifoHead % FL_NET_MAX_REQUESTS);
+    FifoSlot& fs = lk->fifo[slot];
+    if (fs.w.idx != lk->fifoHead + 1) return ncclSuccess;
+    if (fs.w.nreqs != 1) { FL_WARN("NET/FuseLink: multi-send not allowed"); return ncclInternalError; }   // plugin.cc:1448-1451
+    if (fs.w.tag != (uint32_t)tag) return ncclSuccess;                                                     // plugin.cc:1552
+    if (size > fs.w.size) {                                                                                // plugin.cc:1555-1562
+      FL_WARN("NET/FuseLink : req tag %x collective mismatch error, local size %d remote size %d", tag, size, fs.w.size);
+      return ncclInvalidUsage;
+    }
+    if (fs.w.size < 0 || fs.w.addr == 0) {                                                                 // plugin.cc:1563-1570
+      FL_WARN("NET/FuseLink : posted incorrect receive info: size %d addr %llx", fs.w.size, (unsigned long long)fs.w.addr);
+      return ncclInternalError;
+    }
+    if (size && !in_handle(mh, data, (size_t)size)) { FL_WARN("NET/FuseLink : send buffer outside its registration"); return ncclInvalidArgument; }
+    sreq = get_request(lk->sreq, lk, kReqSend);
+    if (!sreq) return ncclInternalError;                                                                   // plugin.cc:1082-1084
+    rreq = fs.rreq;
+    rtype = fs.rtype;
+    w = fs.w;
+    sreq->size = size;
+    rreq->size = size;
+    const bool any_dev = mh->type == NCCL_PTR_CUDA || rtype == NCCL_PTR_CUDA;
+    if (size && any_dev) rc = ensure_link_gpu(lk);
+    if (rc != ncclSuccess) { sreq->type = kReqUnused; return rc; }   // nothing consumed: the descriptor stays posted
+    memset((void*)&fs.w, 0, sizeof(FifoWire));   // plugin.cc:1605
+    fs.rreq = nullptr;
+    lk->fifoHead++;                              // plugin.cc:1607
+    lk->s_inflight++;
+  }
+  uint8_t* dst = (uint8_t*)(uintptr_t)w.addr;
+  const bool src_dev = mh->type == NCCL_PTR_CUDA, dst_dev = rtype == NCCL_PTR_CUDA;
+  int final_state = kStDoneHost;
   if (size == 0) {
-    sreq->state.store(kStDoneHost, std::memory_order_release);
-    rreq->state.store(kStDoneHost, std::memory_order_release);
+    // nothing to move
   } else if (!src_dev && !dst_dev) {
     memcpy(dst, data, (size_t)size);  // host memory is not staged (fuselink.cc:8-13): the wire is a copy
-    sreq->state.store(kStDoneHost, std::memory_order_release);
-    rreq->state.store(kStDoneHost, std::memory_order_release);
   } else {
-    rc = ensure_link_gpu(lk);
-    if (rc == ncclSuccess && !sreq->ev) { hipError_t e = hipEventCreateWithFlags(&sreq->ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
+    if (!sreq->ev) { hipError_t e = hipEventCreateWithFlags(&sreq->ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
     if (rc == ncclSuccess && !rreq->ev) { hipError_t e = hipEventCreateWithFlags(&rreq->ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
     if (rc == ncclSuccess) {
       if (src_dev && dst_dev) {
-        rc = launch_transfer(lk, (const uint8_t*)data, dst, size, fs.w, sreq, rreq);
+        rc = launch_transfer(lk, (const uint8_t*)data, dst, size, w, sreq, rreq);
       } else {
         // one side is host memory: the copy engine is the wire, nothing is striped
         hipError_t e = hipMemcpyAsync(dst, data, (size_t)size, hipMemcpyDefault, lk->stream);
@@ -626,18 +641,21 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
       }
     }
     if (rc != ncclSuccess) {
+      // Part of the transfer may already be queued.  The send fails here; the matched receive completes
+      // with an error, as a receive does whose queue pair went into the error state (plugin.cc:1839-1861).
+      std::lock_guard<std::mutex> g(lk->mu);
       sreq->type = kReqUnused;
+      lk->s_inflight--;
+      rreq->fault = 1;
+      rreq->state.store(kStDoneHost, std::memory_order_release);
       return rc;
     }
-    sreq->state.store(kStLaunched, std::memory_order_release);
-    rreq->state.store(kStLaunched, std::memory_order_release);
+    final_state = kStLaunched;
   }
   // the comm's own NIC carried traffic (updateTxChannelActive, fuselink.h:247-252)
   (void)fl_monitor_mark_active(lk->dev % g_par.lanes, 1, fl_monitor_now());
-  memset((void*)&fs.w, 0, sizeof(FifoWire));   // plugin.cc:1605
-  fs.rreq = nullptr;
-  lk->fifoHead++;                              // plugin.cc:1607
-  lk->s_inflight++;
+  sreq->state.store(final_state, std::memory_order_release);
+  rreq->state.store(final_state, std::memory_order_release);
   *request = sreq;
   return ncclSuccess;
 }
@@ -707,18 +725,19 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   if (r->magic != kReqMagic || r->type == kReqUnused) { FL_WARN("NET/FuseLink : test on a request that is not in flight"); return ncclInternalError; }
   *done = 0;
   Link* lk = r->link;
-  std::lock_guard<std::mutex> g(lk->mu);
+  // the event is polled without the connection's lock: only the thread that drives this comm tests its requests
   const int st = r->state.load(std::memory_order_acquire);
   if (st == kStPosted || st == 0) return ncclSuccess;   // a receive whose send has not been matched yet
   if (st == kStLaunched) {
     hipError_t e = hipEventQuery(r->ev);
     if (e == hipErrorNotReady) return ncclSuccess;
     if (e != hipSuccess) return hip_fail("hipEventQuery", e);
-    if (lk->h_status && *lk->h_status != 0) {
+    if (lk->h_status && *(volatile int32_t*)lk->h_status != 0) {
       FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", *lk->h_status);
       return ncclInternalError;
     }
   }
+  std::lock_guard<std::mutex> g(lk->mu);
   if (r->fault) {   // failed completion, plugin.cc:1839-1861
     FL_WARN("NET/FuseLink : Got completion with error (injected), channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
     return ncclRemoteError;
@@ -863,7 +882,7 @@ int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_ou
   std::lock_guard<std::mutex> g(lk->mu);
   if (!lk->gpu_ready) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
   if (hipSetDevice(lk->hip_device) != hipSuccess || hipStreamSynchronize(lk->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
-  int rows = (int)lk->last_wave_rows;
+  int rows = (int)lk->last_wave_rows.load();
   int take = rows < max_rows ? rows : max_rows;
   if (take > 0 && rows_out && hipMemcpy(rows_out, lk->d_table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "table copy failed");

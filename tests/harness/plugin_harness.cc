@@ -4,7 +4,12 @@
 // number of requests in flight.  Verifies the received buffer byte for byte and prints one JSON line.
 //
 //   plugin_harness <lib.so> [--bytes N] [--request N] [--inflight K] [--iters I] [--host] [--version 6|7|8] [--connections C]
+//                  [--handoff batch,blocks_per_req,layers,kv_heads,block_size,head_dim]
 // With --connections C, C connections run concurrently, each with its own pair of proxy threads and buffers.
+// With --handoff the message is the prefill -> decode hand-off of the reference's serving experiment
+// (FuseLink experiments/serving/model.hh:280-309): one group of five sends on one connection -- the context output
+// (int64 per request), the K cache, the V cache, the block table (int64 per request and block) and the allocated-block
+// counts (int64 per request) -- each cut into --request sized pieces as NCCL's proxy would.
 #include <dlfcn.h>
 #include <hip/hip_runtime.h>
 
@@ -34,7 +39,7 @@ static void logger(ncclDebugLogLevel level, unsigned long, const char* file, int
 #define CHECK(x) do { ncclResult_t r_ = (x); if (r_ != ncclSuccess) { fprintf(stderr, "%s -> ncclResult %d (line %d)\n", #x, (int)r_, __LINE__); exit(2); } } while (0)
 #define HIP(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { fprintf(stderr, "%s -> %s\n", #x, hipGetErrorString(e_)); exit(3); } } while (0)
 
-static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclNet_v6_t* net6, size_t bytes, size_t request, int inflight,
+static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclNet_v6_t* net6, const std::vector<size_t>& sizes, size_t request, int inflight,
                            int iters, int host, int version, double* best_out, double* total_out) {
   if (!host) HIP(hipSetDevice(0));
   const int dev = ci % 2;  // spread the connections over two virtual NICs
@@ -47,25 +52,37 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
   }
   if (!scomm || !rcomm) { fprintf(stderr, "connection did not come up\n"); exit(2); }
 
-  std::vector<uint8_t> pattern(bytes);
-  uint64_t x = 88172645463325252ull + 7919ull * (uint64_t)ci;
-  for (size_t i = 0; i < bytes; ++i) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; pattern[i] = (uint8_t)x; }
-  uint8_t *src = nullptr, *dst = nullptr;
+  // the messages of one group, sent in order over this connection
+  struct Msg { size_t bytes; uint8_t *src, *dst; void *smh, *rmh; std::vector<uint8_t> pattern; };
+  std::vector<Msg> msgs(sizes.size());
   const int type = host ? NCCL_PTR_HOST : NCCL_PTR_CUDA;
-  if (host) {
-    src = (uint8_t*)malloc(bytes); dst = (uint8_t*)calloc(bytes, 1);
-    memcpy(src, pattern.data(), bytes);
-  } else {
-    HIP(hipSetDevice(0));
-    HIP(hipMalloc((void**)&src, bytes)); HIP(hipMalloc((void**)&dst, bytes));
-    HIP(hipMemcpy(src, pattern.data(), bytes, hipMemcpyHostToDevice));
-    HIP(hipMemset(dst, 0, bytes));
+  uint64_t x = 88172645463325252ull + 7919ull * (uint64_t)ci;
+  size_t bytes = 0;
+  for (size_t m = 0; m < sizes.size(); ++m) {
+    Msg& g = msgs[m];
+    g.bytes = sizes[m];
+    bytes += g.bytes;
+    g.pattern.resize(g.bytes);
+    for (size_t i = 0; i < g.bytes; ++i) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; g.pattern[i] = (uint8_t)x; }
+    if (host) {
+      g.src = (uint8_t*)malloc(g.bytes); g.dst = (uint8_t*)calloc(g.bytes, 1);
+      memcpy(g.src, g.pattern.data(), g.bytes);
+    } else {
+      HIP(hipSetDevice(0));
+      HIP(hipMalloc((void**)&g.src, g.bytes)); HIP(hipMalloc((void**)&g.dst, g.bytes));
+      HIP(hipMemcpy(g.src, g.pattern.data(), g.bytes, hipMemcpyHostToDevice));
+      HIP(hipMemset(g.dst, 0, g.bytes));
+    }
+    if (version == 8) { CHECK(net8->regMr(scomm, g.src, g.bytes, type, &g.smh)); CHECK(net8->regMr(rcomm, g.dst, g.bytes, type, &g.rmh)); }
+    else { CHECK(net7->regMr(scomm, g.src, (int)g.bytes, type, &g.smh)); CHECK(net7->regMr(rcomm, g.dst, (int)g.bytes, type, &g.rmh)); }
   }
-  void *smh = nullptr, *rmh = nullptr;
-  if (version == 8) { CHECK(net8->regMr(scomm, src, bytes, type, &smh)); CHECK(net8->regMr(rcomm, dst, bytes, type, &rmh)); }
-  else { CHECK(net7->regMr(scomm, src, (int)bytes, type, &smh)); CHECK(net7->regMr(rcomm, dst, (int)bytes, type, &rmh)); }
-
-  const size_t n_req = (bytes + request - 1) / request;
+  // request k of the group: which message, where in it, how long
+  struct Piece { int msg; size_t off; int len; };
+  std::vector<Piece> pieces;
+  for (size_t m = 0; m < msgs.size(); ++m)
+    for (size_t off = 0; off < msgs[m].bytes; off += request)
+      pieces.push_back({(int)m, off, (int)(msgs[m].bytes - off < request ? msgs[m].bytes - off : request)});
+  const size_t n_req = pieces.size();
   double best = 1e30, total = 0;
   for (int it = 0; it < iters; ++it) {
     std::atomic<size_t> posted{0};
@@ -76,19 +93,19 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
       size_t next = 0, finished = 0;
       while (finished < n_req) {
         if (next < n_req && (int)q.size() < inflight) {
-          void* d = dst + next * request;
-          int sz = (int)((next + 1) * request <= bytes ? request : bytes - next * request), tag = (int)next;
+          const Piece& pc = pieces[next];
+          void* d = msgs[pc.msg].dst + pc.off;
+          int sz = pc.len, tag = (int)next;
           void* req = nullptr;
-          CHECK(net8->irecv(rcomm, 1, &d, &sz, &tag, &rmh, &req));
+          CHECK(net8->irecv(rcomm, 1, &d, &sz, &tag, &msgs[pc.msg].rmh, &req));
           if (req) { q.push_back(req); ++next; posted.store(next, std::memory_order_release); }
         }
         if (!q.empty()) {
           int done = 0, got = -1;
           CHECK(net8->test(q.front(), &done, &got));
           if (done) {
-            const size_t k = finished;
-            const int want = (int)((k + 1) * request <= bytes ? request : bytes - k * request);
-            if (got != want) { fprintf(stderr, "receive %zu reported %d bytes, expected %d\n", k, got, want); exit(4); }
+            const int want = pieces[finished].len;
+            if (got != want) { fprintf(stderr, "receive %zu reported %d bytes, expected %d\n", finished, got, want); exit(4); }
             q.pop_front(); ++finished;
           }
         }
@@ -100,9 +117,9 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
       size_t next = 0, finished = 0;
       while (finished < n_req) {
         if (next < n_req && next < posted.load(std::memory_order_acquire) && (int)q.size() < inflight) {
-          int sz = (int)((next + 1) * request <= bytes ? request : bytes - next * request);
+          const Piece& pc = pieces[next];
           void* req = nullptr;
-          CHECK(net8->isend(scomm, src + next * request, sz, (int)next, smh, &req));
+          CHECK(net8->isend(scomm, msgs[pc.msg].src + pc.off, pc.len, (int)next, msgs[pc.msg].smh, &req));
           if (req) { q.push_back(req); ++next; }
         }
         if (!q.empty()) {
@@ -117,17 +134,23 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
     double s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     total += s;
     if (s < best) best = s;
-    std::vector<uint8_t> back(bytes);
-    if (host) memcpy(back.data(), dst, bytes); else HIP(hipMemcpy(back.data(), dst, bytes, hipMemcpyDeviceToHost));
-    if (memcmp(back.data(), pattern.data(), bytes) != 0) { fprintf(stderr, "connection %d iteration %d: received buffer differs\n", ci, it); exit(5); }
-    if (host) memset(dst, 0, bytes); else HIP(hipMemset(dst, 0, bytes));
+    for (size_t m = 0; m < msgs.size(); ++m) {
+      Msg& g = msgs[m];
+      std::vector<uint8_t> back(g.bytes);
+      if (host) memcpy(back.data(), g.dst, g.bytes); else HIP(hipMemcpy(back.data(), g.dst, g.bytes, hipMemcpyDeviceToHost));
+      if (memcmp(back.data(), g.pattern.data(), g.bytes) != 0) { fprintf(stderr, "connection %d iteration %d message %zu: received buffer differs\n", ci, it, m); exit(5); }
+      if (host) memset(g.dst, 0, g.bytes); else HIP(hipMemset(g.dst, 0, g.bytes));
+    }
   }
-  CHECK(net8->deregMr(scomm, smh));
-  CHECK(net8->deregMr(rcomm, rmh));
+  for (Msg& g : msgs) {
+    CHECK(net8->deregMr(scomm, g.smh));
+    CHECK(net8->deregMr(rcomm, g.rmh));
+  }
   CHECK(net8->closeSend(scomm));
   CHECK(net8->closeRecv(rcomm));
   CHECK(net8->closeListen(lcomm));
-  if (host) { free(src); free(dst); } else { HIP(hipFree(src)); HIP(hipFree(dst)); }
+  for (Msg& g : msgs) { if (host) { free(g.src); free(g.dst); } else { HIP(hipFree(g.src)); HIP(hipFree(g.dst)); } }
+  (void)bytes;
   *best_out = best;
   *total_out = total / iters;
 }
@@ -135,7 +158,8 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
 int main(int argc, char** argv) {
   if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [options]\n", argv[0]); return 1; }
   size_t bytes = 64u << 20, request = 0;
-  int inflight = 4, iters = 5, host = 0, version = 8, connections = 1;
+  int inflight = 4, iters = 5, host = 0, version = 8, connections = 1, handoff = 0;
+  long long ho[6] = {0, 0, 0, 0, 0, 0};
   for (int i = 2; i < argc; ++i) {
     std::string a = argv[i];
     auto val = [&]() { return i + 1 < argc ? strtoull(argv[++i], nullptr, 0) : 0ull; };
@@ -146,6 +170,19 @@ int main(int argc, char** argv) {
     else if (a == "--version") version = (int)val();
     else if (a == "--host") host = 1;
     else if (a == "--connections") connections = (int)val();
+    else if (a == "--handoff" && i + 1 < argc) {
+      if (sscanf(argv[++i], "%lld,%lld,%lld,%lld,%lld,%lld", &ho[0], &ho[1], &ho[2], &ho[3], &ho[4], &ho[5]) != 6) { fprintf(stderr, "--handoff takes six numbers\n"); return 1; }
+      handoff = 1;
+    }
+  }
+  std::vector<size_t> sizes{bytes};
+  if (handoff) {
+    // experiments/serving/model.hh:198-201, 283: cache bytes = sizeof(half) * blocks * layers * kv_heads * block_size * head_dim
+    const size_t batch = (size_t)ho[0], blocks = (size_t)(ho[0] * ho[1]);
+    const size_t cache = 2ull * blocks * (size_t)ho[2] * (size_t)ho[3] * (size_t)ho[4] * (size_t)ho[5];
+    sizes = {8 * batch, cache, cache, 8 * blocks, 8 * batch};   // the five sends of model.hh:286-309, in order
+    bytes = 0;
+    for (size_t b : sizes) bytes += b;
   }
   if (!request || request > bytes) request = bytes;
   if (request > 0x7fffffffull) request = 0x40000000ull;  // isend takes an int size (src/extern/nccl_net.h:74)
@@ -163,11 +200,16 @@ int main(int argc, char** argv) {
 
   std::vector<double> bests(connections, 1e30), totals(connections, 0.0);
   std::vector<std::thread> conns;
-  for (int ci = 0; ci < connections; ++ci) conns.emplace_back([&, ci]() { run_connection(ci, net8, net7, net6, bytes, request, inflight, iters, host, version, &bests[ci], &totals[ci]); });
+  for (int ci = 0; ci < connections; ++ci) conns.emplace_back([&, ci]() { run_connection(ci, net8, net7, net6, sizes, request, inflight, iters, host, version, &bests[ci], &totals[ci]); });
   for (auto& t : conns) t.join();
   double best = 0, total = 0;
   for (int ci = 0; ci < connections; ++ci) { if (bests[ci] > best) best = bests[ci]; total += totals[ci] / connections; }
-  const size_t n_req = (bytes + request - 1) / request;
+  size_t n_req = 0;
+  for (size_t b : sizes) n_req += (b + request - 1) / request;
+  if (handoff)
+    printf("{\"harness\": \"kv_handoff\", \"batch\": %lld, \"blocks\": %lld, \"layers\": %lld, \"kv_heads\": %lld, \"block_size\": %lld, \"head_dim\": %lld, "
+           "\"cache_bytes_each\": %zu, \"comm_volume_bytes\": %zu, \"best_s\": %.9f, \"GBps_volume_over_time\": %.1f}\n",
+           ho[0], ho[0] * ho[1], ho[2], ho[3], ho[4], ho[5], sizes[1], bytes, best, (double)bytes * connections / best / 1e9);
   printf("{\"harness\": \"plugin\", \"name\": \"%s\", \"devices\": %d, \"memory\": \"%s\", \"bytes\": %zu, \"request_bytes\": %zu, \"requests\": %zu, "
          "\"inflight\": %d, \"iters\": %d, \"connections\": %d, \"best_s\": %.9f, \"mean_s\": %.9f, \"GBps_4N_best\": %.1f, \"bit_exact\": true}\n",
          net8->name, ndev, host ? "host" : "device", bytes, request, n_req, inflight, iters, connections, best, total, 4.0 * bytes * connections / best / 1e9);

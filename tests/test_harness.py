@@ -18,7 +18,11 @@ def _run(args, env=None):
     e.update(env or {})
     res = subprocess.run([BIN, build.lib_path(), *args], capture_output=True, text=True, timeout=300, env=e)
     assert res.returncode == 0, res.stderr[-2000:]
-    return json.loads(res.stdout.strip().splitlines()[-1])
+    lines = [json.loads(l) for l in res.stdout.strip().splitlines() if l.startswith("{")]
+    out = lines[-1]
+    if len(lines) > 1:
+        out["handoff"] = lines[-2]
+    return out
 
 
 @pytest.mark.parametrize("version", [6, 7, 8])
@@ -64,6 +68,26 @@ def test_harness_device_four_concurrent_connections():
                env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10)})
     assert out["bit_exact"] and out["connections"] == 4
     print(out)
+
+
+def test_harness_kv_handoff_group_host_memory():
+    # the five sends of the serving experiment's prefill -> decode hand-off (experiments/serving/model.hh:286-309):
+    # int64 context output, K cache, V cache, int64 block table, int64 block counts; tiny and large messages mixed
+    out = _run(["--host", "--handoff", "4,8,2,8,16,128", "--request", str(512 << 10), "--inflight", "8", "--iters", "2"])
+    h = out["handoff"]
+    assert out["bit_exact"] and h["cache_bytes_each"] == 2 * 32 * 2 * 8 * 16 * 128
+    assert h["comm_volume_bytes"] == 2 * h["cache_bytes_each"] + 8 * 4 + 8 * 32 + 8 * 4
+    assert out["requests"] == 1 + 4 + 4 + 1 + 1
+
+
+@pytest.mark.gpu
+def test_harness_kv_handoff_group_device_memory():
+    # 8 requests x 64 blocks, 4 layers, 8 KV heads, 16-token blocks, head_dim 128, fp16: 64 MiB each for K and V,
+    # cut into 512 KiB requests (NCCL_P2P_NET_CHUNKSIZE of the experiment), 8 in flight (NCCL_STEPS)
+    out = _run(["--handoff", "8,64,4,8,16,128", "--request", str(512 << 10), "--inflight", "8", "--iters", "3"],
+               env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(64 << 10)})
+    assert out["bit_exact"] and out["handoff"]["cache_bytes_each"] == 64 << 20
+    print(out["handoff"])
 
 
 def test_plugin_host_path_under_thread_sanitizer():
