@@ -50,6 +50,7 @@ def main() -> int:
     ap.add_argument("--path", default="auto", choices=["auto", "fused", "split"],
                     help="fused: scheduler folded into the striping launch (uniform split, one credit row); split: three launches")
     ap.add_argument("--lds", type=int, default=0, help="paged workload: stage the gather through LDS")
+    ap.add_argument("--no-by-lane", action="store_true", help="stripe large messages in chunk order instead of destination order")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (every lane's staging window lives on it); "
@@ -105,10 +106,14 @@ def main() -> int:
     msg_bytes = nbytes // 2 if kind == "pages" else nbytes    # K and V are two messages over the same windows
     msg_chunks = n_chunks // 2 if kind == "pages" else n_chunks
 
+    # a message too large for the Infinity Cache is striped in destination order (windows written front to back):
+    # the scheduler then also emits the table's rows lane by lane
+    by_lane = kind == "uniform" and rows <= 32 and 3 * msg_bytes > (512 << 20) and not args.no_by_lane
+
     def run_schedule(out=None):
         return core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, sizes=sizes,
                              total_bytes=0 if sizes is not None else msg_bytes, chunk_bytes=0 if sizes is not None else chunk,
-                             epoch_len=epoch_len, out=out, stream=stream)
+                             epoch_len=epoch_len, out=out, stream=stream, by_lane=by_lane)
 
     sched = run_schedule()
     stream.synchronize()
@@ -146,7 +151,7 @@ def main() -> int:
             core.reassemble_uniform(dst, win, uni, status, stream=stream)
         else:
             run_schedule(sched)
-            core.stripe(src, win, sched, status, stream=stream, hint=hint)
+            core.stripe(src, win, sched, status, stream=stream, hint=hint, by_lane=by_lane)
             core.reassemble(dst, win, sched, status, stream=stream, hint=hint)
 
     for _ in range(args.warmup):
@@ -232,7 +237,8 @@ def main() -> int:
                    "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
                    "step": ("2x(schedule+gather+scatter)" if kind == "pages" else
                             "stripe(with scheduler folded in)+reassemble" if fused else "schedule+stripe+reassemble"),
-                   "launch": "eager", "windows": "HIP VMM, 2 MiB units"},
+                   "launch": "eager", "windows": "HIP VMM, 2 MiB units",
+                   "stripe_order": "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel past 512 MiB of buffers)" if fused else "chunk"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
         "kernels_us": {"schedule": round(sched_us, 2), out_k: round(stripe_us, 2), in_k: round(reasm_us, 2),

@@ -31,7 +31,7 @@ class SchedParams(C.Structure):
                 ("n_lanes", C.c_uint32), ("d_credits", C.c_void_p), ("n_rows", C.c_uint32),
                 ("epoch_len", C.c_uint32), ("quantum", C.c_uint64), ("tile_bytes", C.c_uint32),
                 ("mode", C.c_uint32), ("d_state", C.c_void_p), ("d_table", C.c_void_p), ("d_hdr", C.c_void_p),
-                ("inline_credits", C.c_uint32 * MAX_LANES)]
+                ("inline_credits", C.c_uint32 * MAX_LANES), ("d_table_by_lane", C.c_void_p)]
 
 
 class UniformParams(C.Structure):

@@ -75,6 +75,7 @@ class Schedule:
     hdr: torch.Tensor        # uint8 [sizeof(flh_sched_hdr)]
     n_chunks: int
     tile_bytes: int
+    table_by_lane: Optional[torch.Tensor] = None   # the same rows in destination order (uniform split only)
 
     def table_numpy(self) -> np.ndarray:
         raw = self.table[: self.n_chunks * DESC_DTYPE.itemsize].cpu().numpy()
@@ -82,6 +83,10 @@ class Schedule:
 
     def hdr_numpy(self) -> np.ndarray:
         return self.hdr.cpu().numpy().view(HDR_DTYPE)[0].copy()
+
+    def table_by_lane_numpy(self) -> np.ndarray:
+        raw = self.table_by_lane[: self.n_chunks * DESC_DTYPE.itemsize].cpu().numpy()
+        return raw.view(DESC_DTYPE).copy()
 
 
 def new_state(device="cuda") -> torch.Tensor:
@@ -95,7 +100,7 @@ def state_numpy(state: torch.Tensor) -> np.ndarray:
 def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Optional[torch.Tensor] = None,
              total_bytes: int = 0, chunk_bytes: int = 0, src_off: Optional[torch.Tensor] = None, src_base: int = 0,
              epoch_len: int = 0, tile_bytes: int = TILE_BYTES, mode: int = 0, state: Optional[torch.Tensor] = None,
-             out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None) -> Schedule:
+             out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None, by_lane: bool = False) -> Schedule:
     """Launches the scheduler kernel (flh_schedule).  `credits` is a uint32/int32 device tensor of
     shape [rows, n_lanes]; `sizes` a uint32/int32 device tensor of chunk sizes, or None for the
     uniform split of `total_bytes` by `chunk_bytes`."""
@@ -122,12 +127,15 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
     else:
         assert out.table.numel() >= n * DESC_DTYPE.itemsize
         out.n_chunks, out.tile_bytes = n, tile_bytes
+    if by_lane and out.table_by_lane is None:
+        out.table_by_lane = _dev_bytes(max(n, 1) * DESC_DTYPE.itemsize, dev)
     p = SchedParams(_ptr(sizes), total_bytes, chunk_bytes, _ptr(src_off), src_base, n, n_lanes,
                     _ptr(credits if inline is None else None), 1 if inline is not None else credits.shape[0], epoch_len,
                     quantum, tile_bytes, mode, _ptr(state), _ptr(out.table), _ptr(out.hdr))
     if inline is not None:
         for l, c in enumerate(inline):
             p.inline_credits[l] = c
+    p.d_table_by_lane = _ptr(out.table_by_lane) if by_lane else None
     check(lib.flh_schedule(C.byref(p), _stream_ptr(stream)))
     return out
 
@@ -167,8 +175,10 @@ def _hint_ref(hint: Optional[SchedHdr]):
 
 
 def stripe(src: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tensor,
-           stream: Optional[torch.cuda.Stream] = None, hint: Optional[SchedHdr] = None) -> None:
-    check(_lib.load().flh_stripe(_ptr(src), src.numel() * src.element_size(), C.byref(win), _ptr(sched.table),
+           stream: Optional[torch.cuda.Stream] = None, hint: Optional[SchedHdr] = None, by_lane: bool = False) -> None:
+    """flh_stripe; with by_lane the rows are taken in destination order (sched.table_by_lane)."""
+    table = sched.table_by_lane if by_lane else sched.table
+    check(_lib.load().flh_stripe(_ptr(src), src.numel() * src.element_size(), C.byref(win), _ptr(table),
                                  _ptr(sched.hdr), _hint_ref(hint), sched.n_chunks, sched.tile_bytes, _ptr(status),
                                  _stream_ptr(stream)))
 

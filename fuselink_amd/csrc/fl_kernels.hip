@@ -132,6 +132,7 @@ struct SchedArgs {
   int32_t quantum_shift;  // >= 0 when quantum is a power of two
   int32_t tile_shift;     // >= 0 when tile_bytes is a power of two
   uint32_t inline_credits[FLH_MAX_LANES];  // the one credit row when credits == nullptr
+  flh_chunk_desc* table_by_lane;           // optional second copy of the rows in destination order (uniform kernel only)
 };
 
 // 64-bit division is a long software routine on this ISA and almost every operand here fits 32
@@ -616,6 +617,32 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
   const bool keep_off = a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS);
   const uint32_t tpc = a.tile_shift >= 0 ? (a.chunk_bytes + a.tile_bytes - 1) >> a.tile_shift : (a.chunk_bytes + a.tile_bytes - 1) / a.tile_bytes;
 
+  // Destination order: rows grouped by lane, the last chunk's lane last (so that a short final chunk stays the
+  // final row).  Every workgroup works out where each lane's group starts from the per-lane chunk totals.
+  __shared__ uint64_t lane_first[FLH_MAX_LANES];
+  __shared__ uint32_t sh_lane_last;
+  if (MODE == 0 && a.table_by_lane) {
+    if ((uint32_t)tid < L) lane_first[tid] = uni_before(t, c, a.n, (uint32_t)tid, nullptr, nullptr);
+    if (tid == kWave) {  // another wavefront than the one busy with the totals
+      uint32_t ll;
+      (void)uni_before(t, c, a.n - 1, 0xffffffffu, &ll, nullptr);
+      sh_lane_last = ll;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint64_t run = 0;
+      uint32_t l = sh_lane_last;
+#pragma unroll 1
+      for (uint32_t k = 0; k < L; ++k) {
+        l = l + 1 == L ? 0 : l + 1;
+        const uint64_t x = lane_first[l];
+        lane_first[l] = run;
+        run += x;
+      }
+    }
+    __syncthreads();
+  }
+
   if (MODE == 0) {
     const uint32_t i = blockIdx.x * kUniBlock + tid;
     if (i < a.n) {
@@ -632,6 +659,11 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
       d.tile_base = i * tpc;
       d.epoch = (uint32_t)ep;
       a.table[i] = d;
+      if (a.table_by_lane) {
+        const uint64_t pos = lane_first[ln] + before;
+        d.tile_base = (uint32_t)pos * tpc;
+        a.table_by_lane[pos] = d;
+      }
     }
     if (blockIdx.x != gridDim.x - 1) return;
   }
@@ -861,6 +893,7 @@ struct FusedArgs {
   uint32_t n_lanes;
   uint32_t tile_bytes;
   uint32_t tiles_per_chunk;
+  uint32_t dest_order;       // stripe only: blockIdx.y counts chunks in destination order (lane by lane)
   uint32_t credits[FLH_MAX_LANES];
 };
 
@@ -894,19 +927,46 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
 
 template <int DIR, bool NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(FusedArgs a) {
-  const uint32_t c = blockIdx.y;
-  if (c >= a.n_chunks) return;
+  if (blockIdx.y >= a.n_chunks) return;
   FusedRow r;
   fused_row(a, r);
-  const uint64_t j = a.quanta_before + c;
-  const uint64_t slot = mod_u64(j, r.W);
-  uint32_t lane = 0;
-  uint64_t K = 0, hi = r.pfx[0];
+  uint32_t c = blockIdx.y, lane = 0;
+  uint64_t K = 0, hi = r.pfx[0], before;
+  if (DIR == 0 && a.dest_order) {
+    // blockIdx.y = k-th chunk in destination order: find the lane whose group holds k, then invert the
+    // closed form -- the j-th slot of a lane with credit c_l and first slot K_l is (j / c_l) * W + K_l + j mod c_l.
+    const uint64_t x0 = a.quanta_before, x1 = a.quanta_before + a.n_chunks;
+    const uint64_t f0 = div_u64(x0, r.W), f1 = div_u64(x1, r.W);
+    const uint64_t r0 = x0 - f0 * r.W, r1 = x1 - f1 * r.W;
+    uint64_t k = blockIdx.y, cnt0 = 0;
+    bool found = false;
+    uint64_t lo = 0;
 #pragma unroll
-  for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
-    if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; }
+    for (int l = 0; l < FLH_MAX_LANES; ++l) {
+      const uint64_t up = r.pfx[l], cl = up - lo;
+      const uint64_t p0 = r0 <= lo ? 0 : (r0 - lo < cl ? r0 - lo : cl);
+      const uint64_t p1 = r1 <= lo ? 0 : (r1 - lo < cl ? r1 - lo : cl);
+      const uint64_t c0 = f0 * cl + p0;             // slots of the lane before this message
+      const uint64_t nl = f1 * cl + p1 - c0;        // chunks of this message on the lane
+      if (!found && (uint32_t)l < a.n_lanes) {
+        if (k < nl) { found = true; lane = l; K = lo; hi = up; cnt0 = c0; } else { k -= nl; }
+      }
+      lo = up;
+    }
+    const uint64_t cl = hi - K;
+    const uint64_t ja = cnt0 + k;                   // index among all slots of the lane in this epoch
+    const uint64_t rnd = div_u64(ja, cl);
+    c = (uint32_t)(rnd * r.W + K + (ja - rnd * cl) - a.quanta_before);
+    before = k;
+  } else {
+    const uint64_t j = a.quanta_before + c;
+    const uint64_t slot = mod_u64(j, r.W);
+#pragma unroll
+    for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
+      if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; }
+    }
+    before = fused_cnt(r.W, K, hi, j) - fused_cnt(r.W, K, hi, a.quanta_before);
   }
-  const uint64_t before = fused_cnt(r.W, K, hi, j) - fused_cnt(r.W, K, hi, a.quanta_before);
   const uint64_t chunk_off = (uint64_t)c * a.chunk_bytes;
   const uint64_t rem = a.total_bytes - chunk_off;
   const uint32_t len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
@@ -923,7 +983,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(FusedArgs a)
     d.epoch = 0;
     a.table[c] = d;
   }
-  if (DIR == 0 && blockIdx.x == 0 && c == 0 && a.hdr) {  // header: per-lane totals in closed form
+  if (DIR == 0 && blockIdx.x == 0 && blockIdx.y == 0 && a.hdr) {  // header: per-lane totals in closed form
     const uint32_t t = threadIdx.x;
     const uint64_t last = a.n_chunks - 1;
     const uint64_t len_last = a.total_bytes - last * a.chunk_bytes;
@@ -1041,6 +1101,8 @@ int g_device = -1;
 int g_cus = 0;
 // launch tunables (overridable through NCCL_FUSELINK_* for experiments)
 int g_grid_per_cu = 0;     // 0: one workgroup per tile (up to 2^20)
+constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // working sets up to this stay largely in the 256 MB Infinity Cache
+int g_dest_order = -1;    // fused striping in destination order: -1 = when the working set exceeds the cache, 0 / 1 force
 int g_nontemporal = -1;   // -1: streaming accesses only when the buffers cannot all sit in the Infinity Cache
 int g_sched_variant = 0;  // 0 = pick the scheduler shape from the chunk count
 int g_sched_uniform_fast = 1;
@@ -1169,6 +1231,7 @@ int flh_prof_end(double* us_out, int* kernel_out, int max) {
 int flh_tune(const char* key, int64_t value) {
   if (!key) return fl_set_error(FLH_E_ARG, "null key");
   if (!strcmp(key, "grid_per_cu")) { if (value < 0) return fl_set_error(FLH_E_ARG, "grid_per_cu < 0"); g_grid_per_cu = (int)value; return FLH_OK; }
+  if (!strcmp(key, "stripe_dest_order")) { g_dest_order = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
@@ -1211,6 +1274,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   a.state = p->d_state;
   a.table = p->d_table;
   a.hdr = p->d_hdr;
+  a.table_by_lane = p->d_table_by_lane;
   a.chunk_bytes = p->chunk_bytes;
   a.n = p->n_chunks;
   a.n_lanes = p->n_lanes;
@@ -1233,6 +1297,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     FL_HIP(hipGetLastError());
     return FLH_OK;
   }
+  if (p->d_table_by_lane && n > 0) return fl_set_error(FLH_E_ARG, "d_table_by_lane needs the uniform closed-form split (no d_sizes, no d_src_off, quantum == chunk_bytes, n_rows <= %d)", kRowCache);
   // one workgroup; more chunks per thread once the per-pass overhead stops dominating
   if ((variant == 0 && n <= kWave) || variant == 1) {
     FL_LAUNCH((fl_schedule_kernel<1, 1>), dim3(1), dim3(kWave), 0, s, a);
@@ -1260,7 +1325,7 @@ static int check_windows(const flh_windows* win) {
 // good part of it still fits (-8 % at 64 MiB, -20 % on the read-back side at 128 MiB).
 static bool use_nt(uint64_t working_set_bytes) {
   if (g_nontemporal >= 0) return g_nontemporal != 0;
-  return working_set_bytes > (512ull << 20);
+  return working_set_bytes > kCacheResidentBytes;
 }
 
 static uint32_t copy_grid(uint64_t max_tiles) {
@@ -1367,6 +1432,8 @@ static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_wind
   a.n_lanes = u->n_lanes;
   a.tile_bytes = u->tile_bytes;
   a.tiles_per_chunk = (u->chunk_bytes + u->tile_bytes - 1) / u->tile_bytes;
+  // once the message no longer fits the Infinity Cache, write every window front to back
+  a.dest_order = dir == 0 && (g_dest_order < 0 ? 3 * u->total_bytes > kCacheResidentBytes : g_dest_order != 0);
   for (int l = 0; l < FLH_MAX_LANES; ++l) a.credits[l] = (uint32_t)l < u->n_lanes ? u->credits[l] : 0;
   const dim3 grid(a.tiles_per_chunk, a.n_chunks);
   hipStream_t s = (hipStream_t)stream;

@@ -93,6 +93,12 @@ typedef struct flh_sched_params {
   flh_chunk_desc* d_table;     /* out: n_chunks rows */
   flh_sched_hdr* d_hdr;        /* out */
   uint32_t inline_credits[FLH_MAX_LANES]; /* one credit row passed by value (used when d_credits == NULL) */
+  flh_chunk_desc* d_table_by_lane; /* optional out: the same n_chunks rows in destination order -- grouped by lane,
+                                      chunk order kept inside a lane, the last chunk's lane last, tile_base =
+                                      position * tiles per chunk.  flh_stripe driven by this copy writes every
+                                      window front to back, which is faster once a message exceeds the Infinity
+                                      Cache.  Uniform closed-form split only (d_sizes == NULL, d_src_off == NULL,
+                                      quantum == chunk_bytes, n_rows <= 32); FLH_E_ARG otherwise. */
 } flh_sched_params;
 
 /* ---- library ------------------------------------------------------------------------------ */
@@ -105,6 +111,8 @@ int64_t flh_constant(int which);
 /* Launch tunables, for experiments (no counterpart in the reference): "grid_per_cu" = copy
  * workgroups launched per compute unit (0 = one per tile), "nontemporal" = 0/1 streaming loads and
  * stores (-1 = only when the buffers exceed the 256 MB Infinity Cache, the default).
+ * "stripe_dest_order" = 0/1: flh_stripe_uniform walks the chunks lane by lane, so that every window is written
+ * front to back (-1 = only when the buffers exceed the Infinity Cache, the default).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL. */
 int flh_tune(const char* key, int64_t value);
 /* Per-kernel timing for measurement code (no counterpart in the reference).  Between

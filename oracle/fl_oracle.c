@@ -201,6 +201,30 @@ int fl_credit_schedule(const uint32_t* sizes, uint64_t total_bytes, uint32_t chu
   return 0;
 }
 
+int fl_table_by_lane(const fl_chunk_desc_t* table, uint32_t n, uint32_t n_lanes, uint32_t tiles_per_chunk,
+                     fl_chunk_desc_t* out) {
+  if (n_lanes == 0 || n_lanes > FLO_MAX_NIC_NUM || (n && (!table || !out))) return -1;
+  if (n == 0) return 0;
+  uint64_t count[FLO_MAX_NIC_NUM] = {0}, base[FLO_MAX_NIC_NUM] = {0};
+  for (uint32_t i = 0; i < n; ++i) {
+    if (table[i].lane >= n_lanes) return -1;
+    count[table[i].lane]++;
+  }
+  const uint32_t lane_last = table[n - 1].lane;
+  uint64_t run = 0;
+  for (uint32_t k = 0; k < n_lanes; ++k) {
+    const uint32_t l = (lane_last + 1 + k) % n_lanes;
+    base[l] = run;
+    run += count[l];
+  }
+  for (uint32_t i = 0; i < n; ++i) {
+    const uint64_t pos = base[table[i].lane]++;
+    out[pos] = table[i];
+    out[pos].tile_base = (uint32_t)(pos * tiles_per_chunk);
+  }
+  return 0;
+}
+
 /* ---- R6 ------------------------------------------------------------------------------------- */
 uint64_t fl_align_up(uint64_t size, uint64_t gran) { return ((size + gran - 1) / gran) * gran; } /* fuselink.cc:29 */
 uint64_t fl_window_units(uint64_t size, uint64_t unit) { return (size + unit - 1) / unit; }      /* cumem.cu:146-147 */

@@ -21,6 +21,8 @@
  *                     libibverbs headers, absent) is restated and pinned by hand vectors.
  *   fl_credit_schedule  build-defined (the reference has no weighted scheduler); pinned by the
  *                     five properties listed at its declaration and brute force on tiny inputs.
+ *   fl_table_by_lane  build-defined reordering of a finished table (destination order for the striping
+ *                     kernel) -- pinned by a stable sort in numpy and the permutation invariants.
  *   fl_align_up / fl_window_layout / fl_translate / fl_relay_gpu / fl_page_span
  *                     fuselink.cc:15-40, plugin.cc:1181-1201,1582,1626 -- closed forms.
  *   fl_pool_*         cumem.cu:107-184 -- bitmap model, exhaustion at slot 257.
@@ -161,6 +163,12 @@ int fl_credit_schedule(const uint32_t* sizes, uint64_t total_bytes, uint32_t chu
                        const uint32_t* credits, uint32_t n_rows, uint32_t epoch_len,
                        uint64_t quantum, uint32_t tile_bytes, uint32_t mode, fl_sched_state_t* state,
                        fl_chunk_desc_t* table, fl_sched_hdr_t* hdr);
+
+/* The same rows in destination order, for the striping side: grouped by lane, chunk order kept
+ * inside a lane (so window offsets ascend), the lane of the last chunk placed last so that a short
+ * final chunk stays the final row; tile_base = position * tiles_per_chunk.  Uniform splits only. */
+int fl_table_by_lane(const fl_chunk_desc_t* table, uint32_t n, uint32_t n_lanes, uint32_t tiles_per_chunk,
+                     fl_chunk_desc_t* out);
 
 /* ---- R6: staging geometry and pointer translation --------------------------------------- */
 /* fuselink.cc:29: aligned = ceil(size / gran) * gran (granularity queried BEFORE use; the

@@ -75,6 +75,7 @@ def lib() -> C.CDLL:
         "fl_credits_from_status": (None, [i32p, C.c_int, C.c_int, C.c_uint32, u32p]),
         "fl_credit_schedule": (C.c_int, [vp, C.c_uint64, C.c_uint32, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp,
                                          C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint32, C.c_uint32, vp, vp, vp]),
+        "fl_table_by_lane": (C.c_int, [vp, C.c_uint32, C.c_uint32, C.c_uint32, vp]),
         "fl_align_up": (C.c_uint64, [C.c_uint64, C.c_uint64]),
         "fl_window_units": (C.c_uint64, [C.c_uint64, C.c_uint64]),
         "fl_translate": (C.c_uint64, [C.c_uint64, C.c_uint64, C.c_uint64]),
@@ -153,6 +154,14 @@ def credit_schedule(*, n_lanes, credits, quantum, sizes=None, total_bytes=0, chu
     if rc != 0:
         raise ValueError("fl_credit_schedule rejected its arguments")
     return table[:n], hdr[0], st[0]
+
+
+def table_by_lane(table: np.ndarray, n_lanes: int, tiles_per_chunk: int) -> np.ndarray:
+    table = np.ascontiguousarray(table)
+    out = np.zeros(max(table.size, 1), dtype=DESC_DTYPE)
+    if lib().fl_table_by_lane(_vp(table), table.size, n_lanes, tiles_per_chunk, _vp(out)) != 0:
+        raise ValueError("fl_table_by_lane rejected its arguments")
+    return out[: table.size]
 
 
 def _window_ptrs(windows):

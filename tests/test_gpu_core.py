@@ -84,6 +84,90 @@ def test_schedule_credit_rows_summing_past_32_bits(fl, lanes):
     _check_schedule(fl, n_lanes=lanes, credits=credits, quantum=65536, total_bytes=3000 * 65536 - 5, chunk_bytes=65536, epoch_len=100)
 
 
+@pytest.mark.parametrize("seed", range(5))
+def test_schedule_table_in_destination_order(fl, seed):
+    core, torch = fl
+    rng = np.random.default_rng(300 + seed)
+    lanes = int(rng.integers(1, 17))
+    rows = int(rng.integers(1, 20))
+    chunk = int(rng.choice([4096, 65536, 98304]))
+    n = int(rng.integers(1, 5000))
+    total = n * chunk - int(rng.integers(0, chunk))
+    epoch_len = int(rng.choice([0, 7, 1000]))
+    credits = rng.integers(0, 9, size=(rows, lanes)).astype(np.uint32)
+    exp_t, _, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                     epoch_len=epoch_len)
+    exp = ob.table_by_lane(exp_t, lanes, (chunk + 32767) // 32768)
+    sched = core.schedule(n_lanes=lanes, credits=_dev(torch, credits.view(np.int32)), quantum=chunk, total_bytes=total,
+                          chunk_bytes=chunk, epoch_len=epoch_len, by_lane=True)
+    torch.cuda.synchronize()
+    got, got_t = sched.table_by_lane_numpy(), sched.table_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+        np.testing.assert_array_equal(got[f], exp[f], err_msg=f"by-lane field {f}")
+    # both copies of the table move the same bytes
+    lane_bytes = [int(b) for b in sched.hdr_numpy()["lane_bytes"][:lanes]]
+    wins = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
+    w = core.make_windows([t.data_ptr() for t in wins], lane_bytes)
+    src = torch.randint(0, 256, (total,), dtype=torch.uint8, device="cuda")
+    status = core.new_status()
+    for hint in (None, core.uniform_hint(total, chunk)):
+        for t in wins:
+            t.zero_()
+        core.stripe(src, w, sched, status, hint=hint, by_lane=True)
+        dst = torch.zeros_like(src)
+        core.reassemble(dst, w, sched, status, hint=hint)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0 and torch.equal(src, dst)
+
+
+def test_schedule_by_lane_needs_the_uniform_split(fl):
+    core, torch = fl
+    sizes = _dev(torch, np.full(10, 4096, dtype=np.int32))
+    with pytest.raises(Exception):
+        core.schedule(n_lanes=4, credits=[1, 1, 1, 1], quantum=4096, sizes=sizes, by_lane=True)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_fused_stripe_in_destination_order_equals_oracle(fl, seed):
+    core, torch = fl
+    rng = np.random.default_rng(400 + seed)
+    lanes = int(rng.integers(1, 17))
+    chunk = int(rng.choice([8192, 65536, 163840]))
+    n = int(rng.integers(1, 700))
+    total = n * chunk - int(rng.integers(0, chunk))
+    credits = rng.integers(0, 9, size=lanes).astype(np.uint32)
+    if seed == 0:
+        credits[:] = 0
+    epoch_bytes = int(rng.integers(0, 50)) * chunk
+    st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+    st["epoch_bytes"] = epoch_bytes
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                         mode=1, state=st)
+    lane_bytes = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+    exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+    src = _dev(torch, src_np)
+    wins = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
+    w = core.make_windows([t.data_ptr() for t in wins], lane_bytes)
+    u = core.uniform_params(total, chunk, credits.tolist(), epoch_bytes=epoch_bytes)
+    out = core.new_schedule_buffers(n)
+    status = core.new_status()
+    core.tune("stripe_dest_order", 1)
+    try:
+        core.stripe_uniform(src, w, u, status, out=out)
+        torch.cuda.synchronize()
+    finally:
+        core.tune("stripe_dest_order", -1)
+    assert int(status.item()) == 0
+    got_t, got_h = out.table_numpy(), out.hdr_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+    np.testing.assert_array_equal(got_h["lane_bytes"], exp_h["lane_bytes"])
+    for l in range(lanes):
+        np.testing.assert_array_equal(wins[l][: lane_bytes[l]].cpu().numpy(), exp_w[l][: lane_bytes[l]])
+
+
 def test_schedule_state_carry_and_modes(fl):
     rng = np.random.default_rng(7)
     st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]

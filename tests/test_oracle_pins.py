@@ -243,6 +243,31 @@ def test_schedule_properties():
         assert (counts[credits == 0] == 0).all()
 
 
+def test_table_by_lane_is_a_stable_sort_with_the_last_lane_last():
+    rng = np.random.default_rng(11)
+    for _ in range(40):
+        L_ = int(rng.integers(1, 17))
+        chunk = int(rng.choice([4096, 65536, 100000]))
+        n = int(rng.integers(1, 400))
+        total = n * chunk - int(rng.integers(0, chunk))
+        credits = rng.integers(0, 6, size=(int(rng.integers(1, 4)), L_))
+        t, h, _ = ob.credit_schedule(n_lanes=L_, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                     epoch_len=int(rng.choice([0, 5, 64])))
+        tpc = (chunk + 32767) // 32768
+        got = ob.table_by_lane(t, L_, tpc)
+        # independent statement: stable sort by the lane's distance behind the last chunk's lane
+        key = (t["lane"].astype(np.int64) - int(t["lane"][-1]) - 1) % L_
+        order = np.argsort(key, kind="stable")
+        for f in ("src_off", "win_off", "len", "lane", "epoch"):
+            np.testing.assert_array_equal(got[f], t[f][order])
+        np.testing.assert_array_equal(got["tile_base"], np.arange(n, dtype=np.uint32) * tpc)
+        # what the striping kernel relies on: the short chunk is the final row, windows are walked front to back
+        assert got["len"][-1] == t["len"][-1] and (got["len"][:-1] == chunk).all()
+        for l in range(L_):
+            w = got["win_off"][got["lane"] == l]
+            assert (np.diff(w.astype(np.int64)) == chunk).all()
+
+
 def test_schedule_state_carry_equals_one_shot():
     rng = np.random.default_rng(6)
     sizes = rng.integers(0, 5000, size=500)
