@@ -108,7 +108,8 @@ def main() -> int:
 
     # a message too large for the Infinity Cache is striped in destination order (windows written front to back):
     # the scheduler then also emits the table's rows lane by lane
-    by_lane = kind == "uniform" and rows <= 32 and 3 * msg_bytes > (512 << 20) and not args.no_by_lane
+    # (measured: no gain for the paged gather, whose reads are scattered either way, so it keeps chunk order)
+    by_lane = kind == "uniform" and rows <= 32 and 3 * nbytes > (512 << 20) and not args.no_by_lane
 
     def run_schedule(out=None):
         return core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, sizes=sizes,
@@ -142,7 +143,7 @@ def main() -> int:
                 run_schedule(sched)
                 lo = half_i * msg_bytes
                 core.gather_pages(src[lo: lo + msg_bytes], tables[half_i], page_bytes, ppc, win, sched, status,
-                                  use_lds=bool(args.lds), stream=stream)
+                                  use_lds=bool(args.lds), stream=stream, by_lane=by_lane)
                 core.scatter_pages(dst[lo: lo + msg_bytes], tables[half_i], page_bytes, ppc, win, sched, status,
                                    use_lds=bool(args.lds), stream=stream)
         elif fused:

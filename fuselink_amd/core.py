@@ -220,10 +220,10 @@ def reassemble_uniform(dst: torch.Tensor, win: Windows, u: UniformParams, status
 
 def gather_pages(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int, pages_per_chunk: int, win: Windows,
                  sched: Schedule, status: torch.Tensor, use_lds: bool = False,
-                 stream: Optional[torch.cuda.Stream] = None) -> None:
+                 stream: Optional[torch.cuda.Stream] = None, by_lane: bool = False) -> None:
     nbytes = pool.numel() * pool.element_size()
     check(_lib.load().flh_gather_pages(_ptr(pool), nbytes // page_bytes, _ptr(page_table), page_bytes, pages_per_chunk,
-                                       C.byref(win), _ptr(sched.table), sched.n_chunks, int(use_lds), _ptr(status),
+                                       C.byref(win), _ptr(sched.table_by_lane if by_lane else sched.table), sched.n_chunks, int(use_lds), _ptr(status),
                                        _stream_ptr(stream)))
 
 

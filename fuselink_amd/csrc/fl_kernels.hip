@@ -1036,6 +1036,7 @@ struct PageArgs {
   uint32_t pages_per_chunk;
   uint32_t sub_bytes;      // bytes of a page handled by one workgroup step
   uint32_t subs_per_page;
+  int32_t page_shift;      // >= 0 when page_bytes is a power of two
 };
 
 constexpr uint32_t kLdsStage = 16384;
@@ -1048,15 +1049,23 @@ __global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
   const uint64_t total = (uint64_t)a.n_chunks * a.pages_per_chunk * a.subs_per_page;
   for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
     const uint32_t sub = (uint32_t)(t % a.subs_per_page);
-    const uint64_t p = t / a.subs_per_page;          // index into the page table
-    const uint32_t c = (uint32_t)(p / a.pages_per_chunk);
-    const uint32_t k = (uint32_t)(p % a.pages_per_chunk);
+    const uint64_t rp = t / a.subs_per_page;         // row-major page counter
+    const uint32_t c = (uint32_t)(rp / a.pages_per_chunk);
+    const uint32_t k = (uint32_t)(rp % a.pages_per_chunk);
     const flh_chunk_desc d = a.table[c];
     const uint64_t in_chunk = (uint64_t)k * a.page_bytes + (uint64_t)sub * a.sub_bytes;
     if (in_chunk >= d.len) continue;
     uint32_t bytes = a.page_bytes - sub * a.sub_bytes;
     if (bytes > a.sub_bytes) bytes = a.sub_bytes;
     if (bytes > d.len - in_chunk) bytes = (uint32_t)(d.len - in_chunk);
+    // the chunk's place in the message comes from its source offset, not from the row's position, so the
+    // rows may come in any order (destination order for the gather)
+    const uint64_t p = (a.page_shift >= 0 ? d.src_off >> a.page_shift : d.src_off / a.page_bytes) + k;
+    const bool aligned = a.page_shift >= 0 ? (d.src_off & (a.page_bytes - 1)) == 0 : d.src_off % a.page_bytes == 0;
+    if (!aligned || p >= (uint64_t)a.n_chunks * a.pages_per_chunk) {
+      if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+      continue;
+    }
     const uint32_t pg = a.page_table[p];
     bool ok = d.lane < a.win.n_lanes && pg < a.pool_pages;
     if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane];
@@ -1484,6 +1493,7 @@ static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t
   const uint32_t sub = use_lds ? kLdsStage : FLH_TILE_BYTES;
   a.sub_bytes = page_bytes < sub ? page_bytes : sub;
   a.subs_per_page = (page_bytes + a.sub_bytes - 1) / a.sub_bytes;
+  a.page_shift = (page_bytes & (page_bytes - 1)) == 0 ? __builtin_ctz(page_bytes) : -1;
   const uint64_t total = (uint64_t)n_chunks * pages_per_chunk * a.subs_per_page;
   const uint32_t grid = copy_grid(total);
   hipStream_t s = (hipStream_t)stream;

@@ -184,10 +184,13 @@ int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* w
                            const flh_uniform_params* u, int32_t* d_status, void* stream);
 
 /* Paged variants for non-contiguous sources (KV-cache blocks, src/experiments/serving/model.hh:
- * 198-201 gives the page shape): chunk c of the table stands for pages
- * d_page_table[c*pages_per_chunk ...] of a pool of page_bytes-sized pages; gather packs them into
- * the chunk's window slot, scatter puts them back at the same page numbers of d_pool.
- * use_lds != 0 stages each tile through LDS. */
+ * 198-201 gives the page shape): a chunk whose row says src_off stands for the pages
+ * d_page_table[src_off / page_bytes ...] (pages_per_chunk of them) of a pool of page_bytes-sized
+ * pages -- for the uniform split from src_base = 0 that is d_page_table[c*pages_per_chunk ...] for
+ * chunk c; gather packs them into the chunk's window slot, scatter puts them back at the same page
+ * numbers of d_pool.  The rows may come in any order (d_table_by_lane for the gather); src_off must
+ * be a multiple of page_bytes and below n_chunks*pages_per_chunk pages, else FLH_E_RANGE is
+ * reported through *d_status.  use_lds != 0 stages each tile through LDS. */
 int flh_gather_pages(const void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table,
                      uint32_t page_bytes, uint32_t pages_per_chunk, const flh_windows* win,
                      const flh_chunk_desc* d_table, uint32_t n_chunks, int use_lds,

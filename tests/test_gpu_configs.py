@@ -172,8 +172,9 @@ def test_cfg3_expert_parallel_send_set(fl):
 
 
 # ---- paged KV-cache gather --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("by_lane", [False, True])
 @pytest.mark.parametrize("use_lds", [False, True])
-def test_cfg4_paged_kv_gather(fl, use_lds):
+def test_cfg4_paged_kv_gather(fl, use_lds, by_lane):
     core, torch = fl
     rng = np.random.default_rng(4)
     n_pages, page = 4096, 16 * 8 * 128 * 2            # 32 KiB pages: 16 tokens x 8 KV heads x 128 dim bf16
@@ -187,14 +188,14 @@ def test_cfg4_paged_kv_gather(fl, use_lds):
         credits = rng.integers(1, 9, size=8).astype(np.uint32)
         exp_t, exp_h, _ = ob.credit_schedule(n_lanes=8, credits=credits, quantum=chunk, total_bytes=n_pages * page, chunk_bytes=chunk)
         sched = core.schedule(n_lanes=8, credits=_dev(torch, credits.view(np.int32)), quantum=chunk,
-                              total_bytes=n_pages * page, chunk_bytes=chunk)
+                              total_bytes=n_pages * page, chunk_bytes=chunk, by_lane=by_lane)
         torch.cuda.synchronize()
         assert sched.table_numpy().tobytes() == exp_t.tobytes()
         caps = [int(b) for b in exp_h["lane_bytes"][:8]]
         wins = [torch.zeros(max(c, 1), dtype=torch.uint8, device="cuda") for c in caps]
         w = core.make_windows([t.data_ptr() for t in wins], caps)
         status = core.new_status()
-        core.gather_pages(pool, table, page, ppc, w, sched, status, use_lds=use_lds)
+        core.gather_pages(pool, table, page, ppc, w, sched, status, use_lds=use_lds, by_lane=by_lane)
         out = torch.zeros_like(pool)
         core.scatter_pages(out, table, page, ppc, w, sched, status, use_lds=use_lds)
         torch.cuda.synchronize()
@@ -217,16 +218,16 @@ def test_paged_gather_ragged_and_bad_page(fl):
     table_np = np.concatenate([table_np, np.zeros(3, dtype=np.uint32)])   # padded to whole chunks
     credits = np.array([1, 3, 2], dtype=np.uint32)
     exp_t, exp_h, _ = ob.credit_schedule(n_lanes=3, credits=credits, quantum=page * ppc, total_bytes=total, chunk_bytes=page * ppc)
-    sched = core.schedule(n_lanes=3, credits=[1, 3, 2], quantum=page * ppc, total_bytes=total, chunk_bytes=page * ppc)
+    sched = core.schedule(n_lanes=3, credits=[1, 3, 2], quantum=page * ppc, total_bytes=total, chunk_bytes=page * ppc, by_lane=True)
     caps = [int(b) for b in exp_h["lane_bytes"][:3]]
     wins = [torch.zeros(max(c, 1) + 32, dtype=torch.uint8, device="cuda") for c in caps]
     w = core.make_windows([t.data_ptr() for t in wins], caps)
     status = core.new_status()
     table = _dev(torch, table_np.view(np.int32))
-    for lds in (False, True):
+    for lds, by_lane in ((False, False), (True, False), (False, True), (True, True)):
         for t in wins:
             t.zero_()
-        core.gather_pages(pool, table, page, ppc, w, sched, status, use_lds=lds)
+        core.gather_pages(pool, table, page, ppc, w, sched, status, use_lds=lds, by_lane=by_lane)
         out = torch.zeros_like(pool)
         core.scatter_pages(out, table, page, ppc, w, sched, status, use_lds=lds)
         torch.cuda.synchronize()
