@@ -895,6 +895,12 @@ struct FusedArgs {
   uint32_t tiles_per_chunk;
   uint32_t dest_order;       // stripe only: blockIdx.y counts chunks in destination order (lane by lane)
   uint32_t credits[FLH_MAX_LANES];
+  // Worked out once on the host when every quantum index and the credit sum W fit 32 bits: the per-workgroup
+  // division by W becomes one multiply-high by magic = ceil(2^64 / W) (exact for 32-bit operands), and the
+  // lane's slots before the message come from cnt0[] instead of a second and third division.
+  uint32_t fast;
+  uint64_t magic;
+  uint32_t cnt0[FLH_MAX_LANES];
 };
 
 struct FusedRow {  // inclusive credit prefixes of the one row (equal credits if it is empty)
@@ -958,6 +964,16 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(FusedArgs a)
     const uint64_t rnd = div_u64(ja, cl);
     c = (uint32_t)(rnd * r.W + K + (ja - rnd * cl) - a.quanta_before);
     before = k;
+  } else if (a.fast) {
+    const uint32_t j = (uint32_t)a.quanta_before + c;
+    const uint32_t full = (uint32_t)__umul64hi((uint64_t)j, a.magic);  // j / W
+    const uint32_t slot = j - full * (uint32_t)r.W;
+    uint32_t c0 = a.cnt0[0];
+#pragma unroll
+    for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
+      if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; c0 = a.cnt0[l + 1]; }
+    }
+    before = (uint64_t)full * (hi - K) + (slot - K) - c0;  // slot lies inside the lane's span [K, hi)
   } else {
     const uint64_t j = a.quanta_before + c;
     const uint64_t slot = mod_u64(j, r.W);
@@ -1112,6 +1128,7 @@ int g_cus = 0;
 int g_grid_per_cu = 0;     // 0: one workgroup per tile (up to 2^20)
 constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // working sets up to this stay largely in the 256 MB Infinity Cache
 int g_dest_order = -1;    // fused striping in destination order: -1 = when the working set exceeds the cache, 0 / 1 force
+int g_fused_fast = 1;     // host-prepared reciprocal for the fused kernels' slot arithmetic (0 = always divide in the kernel)
 int g_nontemporal = -1;   // -1: streaming accesses only when the buffers cannot all sit in the Infinity Cache
 int g_sched_variant = 0;  // 0 = pick the scheduler shape from the chunk count
 int g_sched_uniform_fast = 1;
@@ -1241,6 +1258,7 @@ int flh_tune(const char* key, int64_t value) {
   if (!key) return fl_set_error(FLH_E_ARG, "null key");
   if (!strcmp(key, "grid_per_cu")) { if (value < 0) return fl_set_error(FLH_E_ARG, "grid_per_cu < 0"); g_grid_per_cu = (int)value; return FLH_OK; }
   if (!strcmp(key, "stripe_dest_order")) { g_dest_order = value < 0 ? -1 : (value != 0); return FLH_OK; }
+  if (!strcmp(key, "fused_fast")) { g_fused_fast = value != 0; return FLH_OK; }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
@@ -1444,6 +1462,23 @@ static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_wind
   // once the message no longer fits the Infinity Cache, write every window front to back
   a.dest_order = dir == 0 && (g_dest_order < 0 ? 3 * u->total_bytes > kCacheResidentBytes : g_dest_order != 0);
   for (int l = 0; l < FLH_MAX_LANES; ++l) a.credits[l] = (uint32_t)l < u->n_lanes ? u->credits[l] : 0;
+  {
+    // the row as the kernel sees it (equal credits stand in for an all-zero row), then the host-side constants
+    uint64_t pfx[FLH_MAX_LANES], W = 0;
+    for (uint32_t l = 0; l < u->n_lanes; ++l) { W += u->credits[l]; pfx[l] = W; }
+    if (W == 0) { for (uint32_t l = 0; l < u->n_lanes; ++l) pfx[l] = l + 1; W = u->n_lanes; }
+    a.fast = W >= 2 && W <= 0xffffffffull && a.quanta_before + n <= 0xffffffffull && g_fused_fast;
+    a.magic = a.fast ? ~0ull / W + 1 : 0;
+    for (int l = 0; l < FLH_MAX_LANES; ++l) a.cnt0[l] = 0;
+    if (a.fast) {
+      const uint64_t full = a.quanta_before / W, rem = a.quanta_before % W;
+      for (uint32_t l = 0; l < u->n_lanes; ++l) {
+        const uint64_t K = l ? pfx[l - 1] : 0, cl = pfx[l] - K;
+        const uint64_t part = rem <= K ? 0 : (rem - K < cl ? rem - K : cl);
+        a.cnt0[l] = (uint32_t)(full * cl + part);
+      }
+    }
+  }
   const dim3 grid(a.tiles_per_chunk, a.n_chunks);
   hipStream_t s = (hipStream_t)stream;
   const bool nt = use_nt(3 * user_bytes);

@@ -383,10 +383,22 @@ def test_schedule_chain_of_calls_matches_one_shot(fl):
     assert s["chunk_index"] == whole_s["chunk_index"] and (s["lane_off"] == whole_s["lane_off"]).all()
 
 
-@pytest.mark.parametrize("seed", range(6))
-def test_fused_schedule_and_stripe_equals_oracle(fl, seed):
+@pytest.mark.parametrize("fast", [1, 0])
+@pytest.mark.parametrize("seed", range(7))
+def test_fused_schedule_and_stripe_equals_oracle(fl, seed, fast):
     """flh_stripe_uniform / flh_reassemble_uniform: the table it writes, the staged windows and the
-    reassembled buffer against the oracle, with carried epoch bytes and an empty credit row."""
+    reassembled buffer against the oracle, with carried epoch bytes and an empty credit row; with the
+    host-prepared reciprocal (fast=1), with in-kernel division (fast=0), and with a credit row that
+    sums past 32 bits (seed 6), which must fall back to division by itself."""
+    core, torch = fl
+    core.tune("fused_fast", fast)
+    try:
+        _fused_case(fl, seed)
+    finally:
+        core.tune("fused_fast", 1)
+
+
+def _fused_case(fl, seed):
     core, torch = fl
     rng = np.random.default_rng(500 + seed)
     lanes = int(rng.integers(1, 17))
@@ -397,6 +409,9 @@ def test_fused_schedule_and_stripe_equals_oracle(fl, seed):
     credits = rng.integers(0, 9, size=lanes).astype(np.uint32)
     if seed == 3:
         credits[:] = 0
+    if seed == 6:
+        credits = rng.integers(2**31, 2**32 - 1, size=lanes).astype(np.uint32)
+        credits[0] = 3
     epoch_bytes = int(rng.integers(0, 40)) * chunk + int(rng.integers(0, chunk))
     base = int(rng.integers(0, 8)) * 4096
     st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
