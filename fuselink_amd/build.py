@@ -52,6 +52,11 @@ def build_library(verbose: bool = True) -> str:
         raise RuntimeError("hipcc failed:\n" + err)
     if verbose and err.strip():
         print(err)
+    # RCCL looks a plugin named X up as librccl-net-X.so (NCCL as libnccl-net-X.so): offer both names
+    alias = os.path.join(LIBDIR, "librccl-net-fuselink.so")
+    if os.path.lexists(alias):
+        os.remove(alias)
+    shutil.copy2(lib_path(), alias)   # a copy, not a link: it must survive whatever carries the tree to another machine
     return lib_path()
 
 

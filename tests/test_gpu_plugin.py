@@ -315,3 +315,30 @@ def test_epoch_prefix_carries_across_requests_until_refresh(net):
         prefix += size
     net.deregMr(s, smh), net.deregMr(r, rmh)
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+@pytest.mark.parametrize("name", ["fuselink", "libnccl-net-fuselink.so"])
+def test_rccl_loads_the_plugin_and_probes_every_device(name):
+    """What the reference's README asks of a user (NCCL_NET_PLUGIN=fuselink, README.md:35-40), under this
+    image's RCCL: the library is found by name, its v8 table is taken, init / devices / getProperties run,
+    and RCCL's GPU Direct check registers device memory through a connection it opens on every virtual NIC."""
+    import os
+    import subprocess
+    import sys
+
+    from fuselink_amd import build
+    libdir = os.path.dirname(build.lib_path())
+    if name == "fuselink" and not os.path.exists(os.path.join(libdir, "librccl-net-fuselink.so")):
+        pytest.skip("librccl-net-fuselink.so (RCCL's name for the plugin) not built")
+    env = dict(os.environ, NCCL_NET_PLUGIN=name, NCCL_DEBUG="INFO", NCCL_DEBUG_SUBSYS="INIT,NET",
+               LD_LIBRARY_PATH=libdir + ":" + os.environ.get("LD_LIBRARY_PATH", ""), MASTER_PORT="29541")
+    probe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "rccl_probe.py")
+    res = subprocess.run([sys.executable, probe], capture_output=True, text=True, timeout=110, env=env)
+    log = res.stdout + res.stderr
+    assert res.returncode == 0, log[-3000:]
+    assert "Loaded net plugin FuseLink (v8)" in log, log[-3000:]
+    assert "Using network FuseLink" in log
+    assert "NET/FuseLink : 8 lanes" in log          # the plugin's own init line, through RCCL's logger
+    for dev in range(8):
+        assert f"'fuselink{dev}'" in log           # getProperties of every virtual NIC was read
+    assert "allreduce 1024.0" in log
