@@ -40,6 +40,14 @@ class UniformParams(C.Structure):
                 ("credits", C.c_uint32 * MAX_LANES)]
 
 
+BATCH_MAX = 8
+
+
+class BatchParams(C.Structure):
+    _fields_ = [("u", UniformParams), ("n_req", C.c_uint32), ("pad", C.c_uint32), ("d_src", C.c_void_p * BATCH_MAX),
+                ("d_dst", C.c_void_p * BATCH_MAX), ("bytes", C.c_uint64 * BATCH_MAX)]
+
+
 class Windows(C.Structure):
     _fields_ = [("base", C.c_void_p * MAX_LANES), ("cap", C.c_uint64 * MAX_LANES), ("n_lanes", C.c_uint32),
                 ("pad", C.c_uint32)]
@@ -59,6 +67,8 @@ SIGNATURES = {
                                      C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_reassemble_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,
                                          C.c_void_p]),
+    "flh_stripe_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "flh_reassemble_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p]),
     "flh_gather_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),
                                    C.c_void_p, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p]),
     "flh_scatter_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),

@@ -10,7 +10,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from ._lib import MAX_LANES, ChunkDesc, SchedHdr, SchedParams, SchedState, UniformParams, Windows, check
+from ._lib import MAX_LANES, BatchParams, ChunkDesc, SchedHdr, SchedParams, SchedState, UniformParams, Windows, check
 
 TILE_BYTES = 32768
 UNIT_BYTES = 2 * 1024 * 1024
@@ -216,6 +216,28 @@ def reassemble_uniform(dst: torch.Tensor, win: Windows, u: UniformParams, status
                        stream: Optional[torch.cuda.Stream] = None) -> None:
     check(_lib.load().flh_reassemble_uniform(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), C.byref(u),
                                              _ptr(status), _stream_ptr(stream)))
+
+
+def batch_params(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor], chunk_bytes: int, credits: Sequence[int], *,
+                 epoch_bytes: int = 0, tile_bytes: int = TILE_BYTES) -> BatchParams:
+    """Several requests handled as one message (flh_stripe_batch / flh_reassemble_batch)."""
+    b = BatchParams()
+    sizes = [t.numel() * t.element_size() for t in srcs]
+    b.u = uniform_params(sum(sizes), chunk_bytes, credits, epoch_bytes=epoch_bytes, tile_bytes=tile_bytes)
+    b.n_req = len(srcs)
+    for q, (s, d, n) in enumerate(zip(srcs, dsts, sizes)):
+        b.d_src[q], b.d_dst[q], b.bytes[q] = s.data_ptr(), d.data_ptr(), n
+    return b
+
+
+def stripe_batch(b: BatchParams, win: Windows, status: torch.Tensor, out: Optional[Schedule] = None,
+                 stream: Optional[torch.cuda.Stream] = None) -> None:
+    check(_lib.load().flh_stripe_batch(C.byref(b), C.byref(win), _ptr(out.table) if out else None,
+                                       _ptr(out.hdr) if out else None, _ptr(status), _stream_ptr(stream)))
+
+
+def reassemble_batch(b: BatchParams, win: Windows, status: torch.Tensor, stream: Optional[torch.cuda.Stream] = None) -> None:
+    check(_lib.load().flh_reassemble_batch(C.byref(b), C.byref(win), _ptr(status), _stream_ptr(stream)))
 
 
 def gather_pages(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int, pages_per_chunk: int, win: Windows,

@@ -903,6 +903,17 @@ struct FusedArgs {
   uint32_t cnt0[FLH_MAX_LANES];
 };
 
+// Several requests as one message: chunk c belongs to the request r with first[r] <= c < first[r+1];
+// its bytes live at user[r] + (c - first[r]) * chunk_bytes.
+struct FusedBatchArgs : FusedArgs {
+  uint32_t n_req;
+  uint32_t first[FLH_BATCH_MAX];   // first chunk of each request
+  uint8_t* req_user[FLH_BATCH_MAX];
+  uint64_t req_bytes[FLH_BATCH_MAX];
+};
+template <class A> struct is_batch { static constexpr bool value = false; };
+template <> struct is_batch<FusedBatchArgs> { static constexpr bool value = true; };
+
 struct FusedRow {  // inclusive credit prefixes of the one row (equal credits if it is empty)
   uint64_t pfx[FLH_MAX_LANES];
   uint64_t W;
@@ -931,8 +942,9 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
   return full * c + part;
 }
 
-template <int DIR, bool NT>
-__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(FusedArgs a) {
+template <int DIR, bool NT, class Args>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
+  constexpr bool BATCH = is_batch<Args>::value;
   if (blockIdx.y >= a.n_chunks) return;
   FusedRow r;
   fused_row(a, r);
@@ -988,6 +1000,19 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(FusedArgs a)
   const uint32_t len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
   const uint64_t src_off = a.src_base + chunk_off;
   const uint64_t win_off = before * a.chunk_bytes;
+  // where the chunk's bytes live on the user side: in the one buffer, or in its request's buffer
+  uint8_t* user = a.user;
+  uint64_t user_off = src_off, user_bytes = a.user_bytes;
+  if constexpr (BATCH) {
+    uint32_t first = 0;
+    user = a.req_user[0];
+    user_bytes = a.req_bytes[0];
+#pragma unroll
+    for (int q = 1; q < FLH_BATCH_MAX; ++q) {
+      if ((uint32_t)q < a.n_req && a.first[q] <= c) { first = a.first[q]; user = a.req_user[q]; user_bytes = a.req_bytes[q]; }
+    }
+    user_off = (uint64_t)(c - first) * a.chunk_bytes;
+  }
 
   if (DIR == 0 && blockIdx.x == 0 && threadIdx.x == 0 && a.table) {
     flh_chunk_desc d;
@@ -1031,11 +1056,11 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(FusedArgs a)
   const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
   if (off >= len) return;
   const uint32_t bytes = (uint32_t)((len - off) < a.tile_bytes ? (len - off) : a.tile_bytes);
-  if (win_off + len > a.win.cap[lane] || src_off + len > a.user_bytes) {
+  if (win_off + len > a.win.cap[lane] || user_off + len > user_bytes) {
     if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
     return;
   }
-  uint8_t* u = a.user + src_off + off;
+  uint8_t* u = user + user_off + off;
   uint8_t* w = (uint8_t*)a.win.base[lane] + win_off + off;
   if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
 }
@@ -1429,24 +1454,23 @@ int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win, cons
   return launch_copy(1, d_dst, dst_bytes, win, d_table, d_hdr, h_hdr, n_chunks_max, tile_bytes, d_status, stream);
 }
 
-static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_uniform_params* u,
-                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream) {
+// argument checks and everything of FusedArgs that follows from the parameters; returns 1 when there is nothing to do
+static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_uniform_params* u, flh_chunk_desc* d_table,
+                      flh_sched_hdr* d_hdr, int32_t* d_status) {
   int rc = check_windows(win);
   if (rc) return rc;
   if (!u || !d_status) return fl_set_error(FLH_E_ARG, "parameters and d_status are required");
   if (u->n_lanes == 0 || u->n_lanes > FLH_MAX_LANES || u->n_lanes != win->n_lanes) return fl_set_error(FLH_E_ARG, "n_lanes %u does not match the windows' %u", u->n_lanes, win->n_lanes);
   if (u->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0");
   if (u->tile_bytes == 0 || u->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", u->tile_bytes);
-  if (u->total_bytes == 0) return FLH_OK;
-  if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
+  if (u->total_bytes == 0) return 1;
   const uint64_t n = (u->total_bytes + u->chunk_bytes - 1) / u->chunk_bytes;
   if (n > 65535) return fl_set_error(FLH_E_ARG, "%llu chunks exceed the 65535 one launch can name; split the message", (unsigned long long)n);
   rc = need_init();
   if (rc) return rc;
   g_prof_kid = dir == 0 ? 2 : 3;
-  FusedArgs a;
-  a.user = (uint8_t*)user;
-  a.user_bytes = user_bytes;
+  a.user = nullptr;
+  a.user_bytes = 0;
   a.win = *win;
   a.table = dir == 0 ? d_table : nullptr;
   a.hdr = dir == 0 ? d_hdr : nullptr;
@@ -1479,18 +1503,72 @@ static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_wind
       }
     }
   }
+  return FLH_OK;
+}
+
+extern "C++" {
+template <class Args>
+static int launch_fused_args(int dir, const Args& a, bool nt, void* stream) {
   const dim3 grid(a.tiles_per_chunk, a.n_chunks);
   hipStream_t s = (hipStream_t)stream;
-  const bool nt = use_nt(3 * user_bytes);
   if (dir == 0) {
-    if (nt) FL_LAUNCH((fl_copy_uniform_fused<0, true>), grid, dim3(kCopyBlock), 0, s, a);
-    else FL_LAUNCH((fl_copy_uniform_fused<0, false>), grid, dim3(kCopyBlock), 0, s, a);
+    if (nt) FL_LAUNCH((fl_copy_uniform_fused<0, true, Args>), grid, dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_uniform_fused<0, false, Args>), grid, dim3(kCopyBlock), 0, s, a);
   } else {
-    if (nt) FL_LAUNCH((fl_copy_uniform_fused<1, true>), grid, dim3(kCopyBlock), 0, s, a);
-    else FL_LAUNCH((fl_copy_uniform_fused<1, false>), grid, dim3(kCopyBlock), 0, s, a);
+    if (nt) FL_LAUNCH((fl_copy_uniform_fused<1, true, Args>), grid, dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_uniform_fused<1, false, Args>), grid, dim3(kCopyBlock), 0, s, a);
   }
   FL_HIP(hipGetLastError());
   return FLH_OK;
+}
+}  // extern "C++"
+
+static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_uniform_params* u,
+                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream) {
+  FusedArgs a;
+  const int rc = fill_fused(a, dir, win, u, d_table, d_hdr, d_status);
+  if (rc) return rc < 0 ? rc : FLH_OK;
+  if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
+  a.user = (uint8_t*)user;
+  a.user_bytes = user_bytes;
+  return launch_fused_args(dir, a, use_nt(3 * user_bytes), stream);
+}
+
+static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table, flh_sched_hdr* d_hdr,
+                        int32_t* d_status, void* stream) {
+  if (!b) return fl_set_error(FLH_E_ARG, "null batch");
+  if (b->n_req == 0 || b->n_req > FLH_BATCH_MAX) return fl_set_error(FLH_E_ARG, "n_req %u not in 1..%d", b->n_req, FLH_BATCH_MAX);
+  FusedBatchArgs a;
+  const int rc = fill_fused(a, dir, win, &b->u, d_table, d_hdr, d_status);
+  if (rc) return rc < 0 ? rc : FLH_OK;
+  a.dest_order = 0;
+  a.src_base = 0;
+  a.n_req = b->n_req;
+  uint64_t sum = 0;
+  for (uint32_t q = 0; q < FLH_BATCH_MAX; ++q) {
+    a.first[q] = 0;
+    a.req_user[q] = nullptr;
+    a.req_bytes[q] = 0;
+    if (q >= b->n_req) continue;
+    void* p = dir == 0 ? (void*)b->d_src[q] : b->d_dst[q];
+    if (!p || b->bytes[q] == 0) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer or no bytes", q);
+    if (q + 1 < b->n_req && b->bytes[q] % b->u.chunk_bytes) return fl_set_error(FLH_E_ARG, "request %u of the batch is not a whole number of chunks", q);
+    a.first[q] = (uint32_t)(sum / b->u.chunk_bytes);
+    a.req_user[q] = (uint8_t*)p;
+    a.req_bytes[q] = b->bytes[q];
+    sum += b->bytes[q];
+  }
+  if (sum != b->u.total_bytes) return fl_set_error(FLH_E_ARG, "the requests hold %llu bytes, the parameters say %llu", (unsigned long long)sum, (unsigned long long)b->u.total_bytes);
+  return launch_fused_args(dir, a, use_nt(3 * sum), stream);
+}
+
+int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
+                     int32_t* d_status, void* stream) {
+  return launch_batch(0, b, win, d_table_out, d_hdr_out, d_status, stream);
+}
+
+int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int32_t* d_status, void* stream) {
+  return launch_batch(1, b, win, nullptr, nullptr, d_status, stream);
 }
 
 int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_uniform_params* u,

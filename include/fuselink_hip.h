@@ -183,6 +183,27 @@ int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows*
 int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
                            const flh_uniform_params* u, int32_t* d_status, void* stream);
 
+/* Several requests in one launch: the requests of one connection that are waiting together (NCCL keeps up
+ * to NCCL_STEPS = 8 in flight, src/fuselink.h:14) are scheduled and copied as ONE message -- the
+ * concatenation of their buffers -- so the launch cost is paid once per batch instead of once per
+ * request.  u->total_bytes must equal the sum of bytes[], u->src_base is ignored, every request but
+ * the last must be a whole number of chunks (then the table equals that of a single message of
+ * total_bytes; row src_off is the offset in the concatenation).  No counterpart in the reference,
+ * which posts one RDMA write per request. */
+#define FLH_BATCH_MAX 8
+typedef struct flh_batch_params {
+  flh_uniform_params u;
+  uint32_t n_req;             /* 1..FLH_BATCH_MAX */
+  uint32_t pad;
+  const void* d_src[FLH_BATCH_MAX];
+  void*       d_dst[FLH_BATCH_MAX];
+  uint64_t    bytes[FLH_BATCH_MAX];
+} flh_batch_params;
+
+int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
+                     flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
+int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int32_t* d_status, void* stream);
+
 /* Paged variants for non-contiguous sources (KV-cache blocks, src/experiments/serving/model.hh:
  * 198-201 gives the page shape): a chunk whose row says src_off stands for the pages
  * d_page_table[src_off / page_bytes ...] (pages_per_chunk of them) of a pool of page_bytes-sized

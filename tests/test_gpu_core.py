@@ -461,3 +461,65 @@ def test_fused_refuses_short_window(fl):
     core.stripe_uniform(src, w, core.uniform_params(1 << 20, 65536, [1, 1]), status)
     torch.cuda.synchronize()
     assert int(status.item()) == -5
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_batch_of_requests_is_one_message(fl, seed):
+    """flh_stripe_batch / flh_reassemble_batch: several request buffers scheduled and copied as the
+    concatenation they form.  Table, header and staged windows equal the oracle's for the single
+    message; every destination receives its own source."""
+    core, torch = fl
+    rng = np.random.default_rng(700 + seed)
+    lanes = int(rng.integers(1, 17))
+    chunk = int(rng.choice([4096, 65536, 512 << 10, 100 * 128]))
+    n_req = int(rng.integers(1, 9))
+    sizes = [int(rng.integers(1, 6)) * chunk for _ in range(n_req)]
+    sizes[-1] -= int(rng.integers(0, chunk))            # only the last request may end inside a chunk
+    total = sum(sizes)
+    credits = rng.integers(0, 9, size=lanes).astype(np.uint32)
+    if seed == 2:
+        credits[:] = 0
+    epoch_bytes = int(rng.integers(0, 40)) * chunk
+    st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+    st["epoch_bytes"] = epoch_bytes
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                         mode=ob.SCHED_RESET_OFFSETS, state=st)
+    srcs_np = [rng.integers(0, 256, size=s, dtype=np.uint8) for s in sizes]
+    caps = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    exp_w = ob.cpu_stripe(np.concatenate(srcs_np), exp_t, caps)
+    srcs = [_dev(torch, a) for a in srcs_np]
+    dsts = [torch.zeros(s + 64, dtype=torch.uint8, device="cuda") for s in sizes]
+    wins = [torch.zeros(max(c, 1) + 64, dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    b = core.batch_params(srcs, dsts, chunk, credits.tolist(), epoch_bytes=epoch_bytes)
+    out = core.new_schedule_buffers(len(exp_t))
+    core.stripe_batch(b, w, status, out=out)
+    core.reassemble_batch(b, w, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    got_t, got_h = out.table_numpy(), out.hdr_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f)
+    for f in ("total_bytes", "total_tiles", "n_chunks", "flags", "lane_bytes", "lane_chunks"):
+        np.testing.assert_array_equal(got_h[f], exp_h[f], err_msg=f)
+    for l in range(lanes):
+        got = wins[l].cpu().numpy()
+        np.testing.assert_array_equal(got[: caps[l]], exp_w[l][: caps[l]])
+        assert not got[caps[l]:].any()
+    for q in range(n_req):
+        got = dsts[q].cpu().numpy()
+        np.testing.assert_array_equal(got[: sizes[q]], srcs_np[q])
+        assert not got[sizes[q]:].any()
+
+
+def test_batch_refuses_a_request_that_ends_inside_a_chunk(fl):
+    core, torch = fl
+    chunk = 4096
+    srcs = [torch.zeros(chunk + 1, dtype=torch.uint8, device="cuda"), torch.zeros(chunk, dtype=torch.uint8, device="cuda")]
+    dsts = [torch.zeros_like(t) for t in srcs]
+    wins = [torch.zeros(4 * chunk, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    w = core.make_windows([t.data_ptr() for t in wins], [4 * chunk] * 2)
+    b = core.batch_params(srcs, dsts, chunk, [1, 1])
+    with pytest.raises(Exception, match="whole number of chunks"):
+        core.stripe_batch(b, w, core.new_status())
