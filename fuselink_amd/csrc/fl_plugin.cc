@@ -12,8 +12,12 @@
 //          striping kernel (chunk -> lane scheduling folded in; user buffer -> lane staging windows)
 //          -> reassembly kernel (windows -> the posted receive buffer).  The reassembly launch plays the part of the
 //          RDMA write landing at the receiver; its completion event is the receive completion.
-//   test   polls the request's event (the completion queue of plugin.cc:1801-1955) and, unlike the
-//          reference, reports the byte count of a receive.
+//          The launches are not made inside isend: matched sends wait on the connection until the first
+//          test of one of them (or until NCCL_FUSELINK_BATCH of them wait), and go out together -- requests
+//          that share a credit row as ONE message in one launch pair, which is what keeps the cost of a
+//          launch from bounding the request rate at NCCL's 512 KiB steps.
+//   test   launches whatever waits on the connection, polls the request's event (the completion queue of
+//          plugin.cc:1801-1955) and, unlike the reference, reports the byte count of a receive.
 // Staging windows are HIP-VMM mappings from the unit pool, one per lane per connection, bound when
 // device memory is first registered on the send side and reused wave after wave.
 #include <hip/hip_runtime.h>
@@ -55,6 +59,7 @@ struct Params {
   int device = 0;
   int idle_credit = 4;
   int max_wave_chunks = 4096;
+  int batch = FLH_BATCH_MAX;     // matched sends that may wait for one launch (1 = launch inside isend)
 };
 Params g_par;
 std::mutex g_init_mu;            // ncclIbLock, plugin.cc:84
@@ -88,7 +93,7 @@ void parse_credit_env() {
 // objects
 // ------------------------------------------------------------------------------------------------
 enum : int { kReqUnused = 0, kReqSend = 1, kReqRecv = 2, kReqFlush = 3 };  // plugin.cc:462-465
-enum : int { kStPosted = 1, kStLaunched = 2, kStDoneHost = 3 };
+enum : int { kStPosted = 1, kStLaunched = 2, kStDoneHost = 3, kStQueued = 4 };
 
 struct Link;
 
@@ -96,7 +101,7 @@ struct Request {
   int type = kReqUnused;
   std::atomic<int> state{0};
   Link* link = nullptr;
-  hipEvent_t ev = nullptr;
+  hipEvent_t ev = nullptr;   // completion of the launch that carries this request (owned by the connection's ring)
   int size = 0;          // bytes moved (reported by test for receives)
   int fault = 0;         // injected wire fault
   uint32_t magic = 0;
@@ -125,6 +130,16 @@ struct FifoSlot {
   FifoWire w;
   Request* rreq;     // loopback only: the receive request this descriptor belongs to
   int rtype;         // pointer type of the receive buffer
+};
+
+// a matched send whose GPU work has not been queued yet
+struct Pending {
+  const uint8_t* src;
+  uint8_t* dst;
+  int size;
+  bool src_dev, dst_dev;
+  FifoWire w;
+  Request *sreq, *rreq;
 };
 
 struct Link {
@@ -157,6 +172,13 @@ struct Link {
   int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
   int32_t* d_status = nullptr;
   std::atomic<uint32_t> last_wave_rows{0};
+  // Guards the waiting sends, the event ring and every launch on `stream` (either side's thread may be the
+  // one that launches).  Never taken while `mu` is held by the same thread for long: isend drops `mu` first.
+  std::mutex launch_mu;
+  std::vector<Pending> pending;
+  hipEvent_t evring[FL_NET_MAX_REQUESTS] = {};   // at most that many requests, hence launches, are in flight
+  uint32_t ev_next = 0;
+  int64_t launches = 0, batched_requests = 0;    // launch pairs made, requests that shared one
 };
 
 struct Comm {
@@ -223,8 +245,7 @@ void link_unref(Link* lk) {
     (void)hipHostFree(lk->h_status);
     (void)hipStreamDestroy(lk->stream);
   }
-  for (auto& r : lk->sreq) if (r.ev) (void)hipEventDestroy(r.ev);
-  for (auto& r : lk->rreq) if (r.ev) (void)hipEventDestroy(r.ev);
+  for (auto& e : lk->evring) if (e) (void)hipEventDestroy(e);
   delete lk;
   g_live_links.fetch_sub(1);
 }
@@ -237,6 +258,7 @@ Request* get_request(Request* tab, Link* lk, int type) {
       r->type = type;
       r->link = lk;
       r->size = 0;
+      r->ev = nullptr;
       r->fault = 0;
       r->magic = kReqMagic;
       r->state.store(0, std::memory_order_relaxed);
@@ -330,6 +352,9 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.device = (int)fl_param("FUSELINK_DEVICE", g_par.device);
   g_par.idle_credit = (int)fl_param("FUSELINK_IDLE_CREDIT", g_par.idle_credit);
   g_par.max_wave_chunks = (int)fl_param("FUSELINK_MAX_WAVE_CHUNKS", g_par.max_wave_chunks);
+  g_par.batch = (int)fl_param("FUSELINK_BATCH", g_par.batch);
+  if (g_par.batch < 1) g_par.batch = 1;
+  if (g_par.batch > FLH_BATCH_MAX) g_par.batch = FLH_BATCH_MAX;
   if (g_par.lanes < 1 || g_par.lanes > FL_NET_MAX_LANES) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_LANES must be 1..%d", FL_NET_MAX_LANES); return ncclInvalidArgument; }
   if (g_par.chunk < 128 || g_par.chunk % 128 || g_par.chunk > (int64_t)1 << 30) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_CHUNKSIZE must be a multiple of 128 up to 1 GiB"); return ncclInvalidArgument; }
   if (g_par.refresh_batch < 1 || g_par.qps < 1 || g_par.qps > 128 || g_par.window_units < 1 || g_par.pool_units < 1 || g_par.max_wave_chunks < 1) {
@@ -521,11 +546,10 @@ bool in_handle(const MemHandle* mh, const void* p, size_t n) {
   return a >= mh->start_addr && a + n <= mh->start_addr + mh->size;
 }
 
-// Queue the GPU work of one matched send on the connection's stream.
-ncclResult_t launch_transfer(Link* lk, const uint8_t* src, uint8_t* dst, int size, const FifoWire& w, Request* sreq, Request* rreq) {
-  FL_HIPCHECK(hipSetDevice(lk->hip_device));
-  uint32_t credits[FLH_MAX_LANES] = {};
+// Credit row a descriptor asks for: the receiver's row, or one lane named outright.
+void wire_credits(const Link* lk, const FifoWire& w, uint32_t* credits) {
   const int lanes = g_par.lanes;
+  for (int l = 0; l < FLH_MAX_LANES; ++l) credits[l] = 0;
   if (w.fuselink_offset == -2) {
     for (int l = 0; l < lanes; ++l) credits[l] = w.credits[l];
   } else {
@@ -533,14 +557,31 @@ ncclResult_t launch_transfer(Link* lk, const uint8_t* src, uint8_t* dst, int siz
     const int lane = w.fuselink_offset >= 0 ? w.fuselink_offset % lanes : lk->dev % lanes;
     credits[lane] = 1;
   }
+}
+
+void fill_uniform(flh_uniform_params& u, const Link* lk, const uint32_t* credits, uint64_t bytes, uint64_t src_base) {
+  memset(&u, 0, sizeof(u));
+  u.total_bytes = bytes;
+  u.src_base = src_base;
+  u.epoch_bytes = lk->epoch_bytes;
+  u.chunk_bytes = (uint32_t)g_par.chunk;
+  u.n_lanes = (uint32_t)g_par.lanes;
+  u.tile_bytes = FLH_TILE_BYTES;
+  for (int l = 0; l < g_par.lanes; ++l) u.credits[l] = credits[l];
+}
+
+// Queue the GPU work of one matched send on the connection's stream (launch_mu held).
+ncclResult_t launch_transfer(Link* lk, const Pending& p) {
+  uint32_t credits[FLH_MAX_LANES];
+  wire_credits(lk, p.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
-  const uint32_t per_wave = wave_chunks(credits, lanes, chunk, lk->wins.cap[0]);
+  const uint32_t per_wave = wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0]);
   if (per_wave == 0) { FL_WARN("NET/FuseLink : staging window smaller than a chunk"); return ncclInternalError; }
   // request -> QP pieces (plugin.cc:1467-1495), each piece -> waves of chunks
   const int nqps = g_par.split_on_qps ? g_par.qps : 1;
   std::vector<int> qoff(nqps), qlen(nqps);
-  if (flh_qp_split(size, nqps, qoff.data(), qlen.data()) < 0) return ncclInternalError;
-  bool first = true;
+  if (flh_qp_split(p.size, nqps, qoff.data(), qlen.data()) < 0) return ncclInternalError;
+  if (p.w.flags & 1u) lk->epoch_bytes = 0;   // the receiver refreshed its lane decision: new credit epoch
   for (int q = 0; q < nqps; ++q) {
     uint64_t done = 0;
     const uint64_t piece = (uint64_t)qlen[q];
@@ -549,27 +590,113 @@ ncclResult_t launch_transfer(Link* lk, const uint8_t* src, uint8_t* dst, int siz
       if (wave > piece - done) wave = piece - done;
       // One credit row, quantum-sized chunks, windows reused from offset 0: the striping launch works out
       // every chunk's lane and window offset itself (and writes the table), the reassembly launch likewise.
-      if (first && (w.flags & 1u)) lk->epoch_bytes = 0;   // the receiver refreshed its lane decision: new credit epoch
       flh_uniform_params u;
-      memset(&u, 0, sizeof(u));
-      u.total_bytes = wave;
-      u.src_base = (uint64_t)qoff[q] + done;
-      u.epoch_bytes = lk->epoch_bytes;
-      u.chunk_bytes = (uint32_t)chunk;
-      u.n_lanes = (uint32_t)lanes;
-      u.tile_bytes = FLH_TILE_BYTES;
-      for (int l = 0; l < lanes; ++l) u.credits[l] = credits[l];
-      FL_FLHCHECK(flh_stripe_uniform(src, (uint64_t)size, &lk->wins, &u, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
-      FL_FLHCHECK(flh_reassemble_uniform(dst, (uint64_t)size, &lk->wins, &u, lk->d_status, lk->stream));
+      fill_uniform(u, lk, credits, wave, (uint64_t)qoff[q] + done);
+      FL_FLHCHECK(flh_stripe_uniform(p.src, (uint64_t)p.size, &lk->wins, &u, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
+      FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &lk->wins, &u, lk->d_status, lk->stream));
       lk->epoch_bytes += wave;
       lk->last_wave_rows = (uint32_t)((wave + chunk - 1) / chunk);
+      lk->launches++;
       done += wave;
-      first = false;
     }
   }
-  FL_HIPCHECK(hipEventRecord(sreq->ev, lk->stream));
-  FL_HIPCHECK(hipEventRecord(rreq->ev, lk->stream));
   return ncclSuccess;
+}
+
+// Requests [i, j) of the waiting list as one message in one launch pair (launch_mu held).
+ncclResult_t launch_batch(Link* lk, size_t i, size_t j) {
+  const Pending& p0 = lk->pending[i];
+  uint32_t credits[FLH_MAX_LANES];
+  wire_credits(lk, p0.w, credits);
+  if (p0.w.flags & 1u) lk->epoch_bytes = 0;
+  flh_batch_params b;
+  memset(&b, 0, sizeof(b));
+  uint64_t sum = 0;
+  for (size_t k = i; k < j; ++k) {
+    const Pending& p = lk->pending[k];
+    b.d_src[k - i] = p.src;
+    b.d_dst[k - i] = p.dst;
+    b.bytes[k - i] = (uint64_t)p.size;
+    sum += (uint64_t)p.size;
+  }
+  b.n_req = (uint32_t)(j - i);
+  fill_uniform(b.u, lk, credits, sum, 0);
+  FL_FLHCHECK(flh_stripe_batch(&b, &lk->wins, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
+  FL_FLHCHECK(flh_reassemble_batch(&b, &lk->wins, lk->d_status, lk->stream));
+  lk->epoch_bytes += sum;
+  lk->last_wave_rows = (uint32_t)((sum + (uint64_t)g_par.chunk - 1) / (uint64_t)g_par.chunk);
+  lk->launches++;
+  lk->batched_requests += (int64_t)(j - i);
+  return ncclSuccess;
+}
+
+// How many of the waiting sends from i on can travel as one message: device memory on both sides, the same
+// credit row, no credit refresh after the first, whole chunks in all but the last, one QP piece each, and
+// all of it inside one wave of the staging windows.
+size_t batch_span(const Link* lk, size_t i) {
+  const Pending& p0 = lk->pending[i];
+  if (!(p0.src_dev && p0.dst_dev) || g_par.batch < 2) return 1;
+  if ((g_par.split_on_qps ? g_par.qps : 1) != 1) return 1;
+  uint32_t credits[FLH_MAX_LANES];
+  wire_credits(lk, p0.w, credits);
+  const uint64_t chunk = (uint64_t)g_par.chunk;
+  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0]) * chunk;
+  uint64_t sum = 0;
+  size_t j = i;
+  while (j < lk->pending.size() && j - i < (size_t)FLH_BATCH_MAX) {
+    const Pending& p = lk->pending[j];
+    if (!(p.src_dev && p.dst_dev)) break;
+    if (j > i && ((p.w.flags & 1u) || p.w.fuselink_offset != p0.w.fuselink_offset || memcmp(p.w.credits, p0.w.credits, sizeof(p.w.credits)))) break;
+    if (sum + (uint64_t)p.size > room) break;
+    sum += (uint64_t)p.size;
+    ++j;
+    if ((uint64_t)p.size % chunk) break;   // a request that ends inside a chunk closes the message
+  }
+  return j > i ? j - i : 1;
+}
+
+// Launch everything that waits on the connection, in order (launch_mu held).  A failure completes the requests
+// it touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).
+void flush_pending(Link* lk) {
+  if (lk->pending.empty()) return;
+  bool dev_ok = hipSetDevice(lk->hip_device) == hipSuccess;
+  size_t i = 0;
+  while (i < lk->pending.size()) {
+    const size_t span = batch_span(lk, i);
+    ncclResult_t rc = dev_ok ? ncclSuccess : ncclUnhandledCudaError;
+    hipEvent_t& ev = lk->evring[lk->ev_next % FL_NET_MAX_REQUESTS];
+    if (rc == ncclSuccess && !ev) { hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
+    if (rc == ncclSuccess) {
+      const Pending& p = lk->pending[i];
+      if (span > 1) {
+        rc = launch_batch(lk, i, i + span);
+      } else if (p.src_dev && p.dst_dev) {
+        rc = launch_transfer(lk, p);
+      } else {
+        // one side is host memory: the copy engine is the wire, nothing is striped
+        hipError_t e = hipMemcpyAsync(p.dst, p.src, (size_t)p.size, hipMemcpyDefault, lk->stream);
+        if (e != hipSuccess) rc = hip_fail("hipMemcpyAsync", e);
+      }
+    }
+    if (rc == ncclSuccess) { hipError_t e = hipEventRecord(ev, lk->stream); if (e != hipSuccess) rc = hip_fail("hipEventRecord", e); }
+    for (size_t k = i; k < i + span; ++k) {
+      Pending& p = lk->pending[k];
+      if (rc == ncclSuccess) {
+        p.sreq->ev = ev;
+        p.rreq->ev = ev;
+        p.sreq->state.store(kStLaunched, std::memory_order_release);
+        p.rreq->state.store(kStLaunched, std::memory_order_release);
+      } else {
+        p.sreq->fault = 1;
+        p.rreq->fault = 1;
+        p.sreq->state.store(kStDoneHost, std::memory_order_release);
+        p.rreq->state.store(kStDoneHost, std::memory_order_release);
+      }
+    }
+    if (rc == ncclSuccess) lk->ev_next++;
+    i += span;
+  }
+  lk->pending.clear();
 }
 
 ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhandle, void** request) {
@@ -621,41 +748,30 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
   }
   uint8_t* dst = (uint8_t*)(uintptr_t)w.addr;
   const bool src_dev = mh->type == NCCL_PTR_CUDA, dst_dev = rtype == NCCL_PTR_CUDA;
-  int final_state = kStDoneHost;
-  if (size == 0) {
-    // nothing to move
-  } else if (!src_dev && !dst_dev) {
-    memcpy(dst, data, (size_t)size);  // host memory is not staged (fuselink.cc:8-13): the wire is a copy
-  } else {
-    if (!sreq->ev) { hipError_t e = hipEventCreateWithFlags(&sreq->ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
-    if (rc == ncclSuccess && !rreq->ev) { hipError_t e = hipEventCreateWithFlags(&rreq->ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
-    if (rc == ncclSuccess) {
-      if (src_dev && dst_dev) {
-        rc = launch_transfer(lk, (const uint8_t*)data, dst, size, w, sreq, rreq);
-      } else {
-        // one side is host memory: the copy engine is the wire, nothing is striped
-        hipError_t e = hipMemcpyAsync(dst, data, (size_t)size, hipMemcpyDefault, lk->stream);
-        if (e == hipSuccess) e = hipEventRecord(sreq->ev, lk->stream);
-        if (e == hipSuccess) e = hipEventRecord(rreq->ev, lk->stream);
-        if (e != hipSuccess) rc = hip_fail("hipMemcpyAsync", e);
-      }
-    }
-    if (rc != ncclSuccess) {
-      // Part of the transfer may already be queued.  The send fails here; the matched receive completes
-      // with an error, as a receive does whose queue pair went into the error state (plugin.cc:1839-1861).
-      std::lock_guard<std::mutex> g(lk->mu);
-      sreq->type = kReqUnused;
-      lk->s_inflight--;
-      rreq->fault = 1;
-      rreq->state.store(kStDoneHost, std::memory_order_release);
-      return rc;
-    }
-    final_state = kStLaunched;
-  }
   // the comm's own NIC carried traffic (updateTxChannelActive, fuselink.h:247-252)
   (void)fl_monitor_mark_active(lk->dev % g_par.lanes, 1, fl_monitor_now());
-  sreq->state.store(final_state, std::memory_order_release);
-  rreq->state.store(final_state, std::memory_order_release);
+  if (size == 0 || (!src_dev && !dst_dev)) {
+    // host memory is not staged (fuselink.cc:8-13): the wire is a copy
+    if (size) memcpy(dst, data, (size_t)size);
+    sreq->state.store(kStDoneHost, std::memory_order_release);
+    rreq->state.store(kStDoneHost, std::memory_order_release);
+  } else {
+    // device memory: the launches are made with the other sends that wait on this connection
+    std::lock_guard<std::mutex> g(lk->launch_mu);
+    Pending p;
+    p.src = (const uint8_t*)data;
+    p.dst = dst;
+    p.size = size;
+    p.src_dev = src_dev;
+    p.dst_dev = dst_dev;
+    p.w = w;
+    p.sreq = sreq;
+    p.rreq = rreq;
+    lk->pending.push_back(p);
+    sreq->state.store(kStQueued, std::memory_order_release);
+    rreq->state.store(kStQueued, std::memory_order_release);
+    if ((int)lk->pending.size() >= g_par.batch) flush_pending(lk);
+  }
   *request = sreq;
   return ncclSuccess;
 }
@@ -726,8 +842,13 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   *done = 0;
   Link* lk = r->link;
   // the event is polled without the connection's lock: only the thread that drives this comm tests its requests
-  const int st = r->state.load(std::memory_order_acquire);
+  int st = r->state.load(std::memory_order_acquire);
   if (st == kStPosted || st == 0) return ncclSuccess;   // a receive whose send has not been matched yet
+  if (st == kStQueued) {                                // matched, not launched: everything that waits goes out now
+    std::lock_guard<std::mutex> g(lk->launch_mu);
+    flush_pending(lk);
+    st = r->state.load(std::memory_order_acquire);
+  }
   if (st == kStLaunched) {
     hipError_t e = hipEventQuery(r->ev);
     if (e == hipErrorNotReady) return ncclSuccess;
@@ -875,12 +996,24 @@ int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64
   return FLH_OK;
 }
 
+int fl_net_launch_stats(void* comm, int64_t* launches, int64_t* batched_requests) {
+  Comm* c = (Comm*)comm;
+  if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
+  Link* lk = c->link;
+  std::lock_guard<std::mutex> g(lk->launch_mu);
+  if (launches) *launches = lk->launches;
+  if (batched_requests) *batched_requests = lk->batched_requests;
+  return FLH_OK;
+}
+
 int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_out) {
   Comm* c = (Comm*)sendComm;
   if (!c || c->magic != kCommMagic || !c->is_send) return fl_set_error(FLH_E_ARG, "not a send comm");
   Link* lk = c->link;
   std::lock_guard<std::mutex> g(lk->mu);
   if (!lk->gpu_ready) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
+  std::lock_guard<std::mutex> gl(lk->launch_mu);
+  flush_pending(lk);
   if (hipSetDevice(lk->hip_device) != hipSuccess || hipStreamSynchronize(lk->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
   int rows = (int)lk->last_wave_rows.load();
   int take = rows < max_rows ? rows : max_rows;

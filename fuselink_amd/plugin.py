@@ -73,7 +73,7 @@ def _table(version: int):
 PLUGIN_SYMBOLS = ["ncclNetPlugin_v8", "ncclNetPlugin_v7", "ncclNetPlugin_v6"]
 CONTROL_SYMBOLS = ["fl_monitor_attach_shm", "fl_monitor_detach", "fl_monitor_is_shared", "fl_monitor_daemon_running", "fl_monitor_reset", "fl_monitor_set_entry", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
                    "fl_monitor_status", "fl_monitor_idle_pick", "fl_monitor_credits", "fl_net_set_credits",
-                   "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_last_table", "fl_net_reset"]
+                   "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_launch_stats", "fl_net_last_table", "fl_net_reset"]
 
 
 class NetPlugin:
@@ -110,6 +110,7 @@ class NetPlugin:
         L.fl_net_set_credits.argtypes = [C.POINTER(C.c_uint32), C.c_int]
         L.fl_net_inject_fault.argtypes = [VP]
         L.fl_net_comm_stats.argtypes = [VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+        L.fl_net_launch_stats.argtypes = [VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         L.fl_net_last_table.argtypes = [VP, VP, C.c_int, VP]
 
     # ---- the function table -----------------------------------------------------------------------
@@ -253,6 +254,11 @@ class NetPlugin:
         a, b, c = C.c_int64(), C.c_int64(), C.c_int64()
         assert self.lib.fl_net_comm_stats(comm, C.byref(a), C.byref(b), C.byref(c)) == 0
         return {"n_finished": a.value, "in_flight": b.value, "refreshes": c.value}
+
+    def launch_stats(self, comm):
+        a, b = C.c_int64(), C.c_int64()
+        assert self.lib.fl_net_launch_stats(comm, C.byref(a), C.byref(b)) == 0
+        return {"launches": a.value, "batched_requests": b.value}
 
     def last_table(self, send_comm, max_rows: int = 4096):
         import numpy as np

@@ -232,6 +232,10 @@ int fl_net_reset(void);
 int fl_net_inject_fault(void* request);
 /* Counters of a send or recv comm: n_finished (src/plugin.cc:517,568), requests in flight, lane refreshes. */
 int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64_t* refreshes);
+/* Launch pairs (stripe + reassemble) a connection has queued so far, and how many requests travelled in
+ * a pair shared with others.  Matched sends wait for the first test() of one of them or until
+ * NCCL_FUSELINK_BATCH (default 8, 1 = launch inside isend) of them wait, then go out together. */
+int fl_net_launch_stats(void* comm, int64_t* launches, int64_t* batched_requests);
 /* Chunk -> lane table and header of the last wave a send comm scheduled, copied to host memory
  * (blocks until that wave has run).  rows_out holds up to max_rows flh_chunk_desc entries.
  * Returns the number of rows of that wave. */

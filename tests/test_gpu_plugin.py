@@ -10,7 +10,8 @@ from tests import oracle_binding as ob
 pytestmark = pytest.mark.gpu
 
 ENV_KEYS = ["NCCL_FUSELINK_LANES", "NCCL_FUSELINK_CHUNKSIZE", "NCCL_FUSELINK_POLICY", "NCCL_FUSELINK_WINDOW_UNITS",
-            "NCCL_FUSELINK_POOL_UNITS", "NCCL_FUSELINK_REFRESH_BATCH", "NCCL_IB_QPS_PER_CONNECTION", "NCCL_FUSELINK_CREDITS"]
+            "NCCL_FUSELINK_POOL_UNITS", "NCCL_FUSELINK_REFRESH_BATCH", "NCCL_IB_QPS_PER_CONNECTION", "NCCL_FUSELINK_CREDITS",
+            "NCCL_FUSELINK_BATCH"]
 
 
 @pytest.fixture()
@@ -315,6 +316,57 @@ def test_epoch_prefix_carries_across_requests_until_refresh(net):
         prefix += size
     net.deregMr(s, smh), net.deregMr(r, rmh)
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_sends_that_wait_together_travel_as_one_message(net):
+    """Seven 512 KiB requests posted before anything is tested: one launch pair carries them all, scheduled as
+    the 3.5 MiB message they form (table against the oracle), every receive buffer gets its own data; with
+    NCCL_FUSELINK_BATCH=1 the same traffic takes one launch pair per request and gives the same bytes.
+    (A first request goes alone: on a refresh boundary the reference's gate admits one receive at a time.)"""
+    import torch
+    rng = np.random.default_rng(77)
+    chunk, piece, n_req = 64 << 10, 512 << 10, 7
+    credits = [3, 1, 0, 2, 5, 1, 1, 4]
+    src_np = rng.integers(0, 256, size=(n_req + 1) * piece, dtype=np.uint8)
+    src = torch.from_numpy(src_np).cuda()
+    for batch, exp_launches, exp_batched in ((8, 1, 7), (1, 7, 0), (3, 3, 6)):
+        net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_BATCH=batch)
+        net.set_credits(credits)
+        dst = torch.zeros_like(src)
+        lcomm, s, r = net.connect_pair(0)
+        _, smh = net.regMr(s, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA)
+        _, rmh = net.regMr(r, dst.data_ptr(), dst.numel(), P.NCCL_PTR_CUDA)
+        _send_recv(net, s, r, src, dst, piece, 99, smh, rmh, src_off=n_req * piece, dst_off=n_req * piece)
+        assert net.launch_stats(s) == {"launches": 1, "batched_requests": 0}
+        rreqs, sreqs = [], []
+        # receive buffers in reverse order, so that a batch has to route every request to its own buffer
+        for k in range(n_req):
+            rc, q = net.irecv(r, [dst.data_ptr() + (n_req - 1 - k) * piece], [piece], [k], [rmh])
+            assert rc == 0 and q
+            rreqs.append(q)
+        for k in range(n_req):
+            rc, q = net.isend(s, src.data_ptr() + k * piece, piece, k, smh)
+            assert rc == 0 and q
+            sreqs.append(q)
+        for q in sreqs:
+            net.wait(q)
+        for q in rreqs:
+            assert net.wait(q) == piece
+        st = net.launch_stats(s)
+        assert st == {"launches": 1 + exp_launches, "batched_requests": exp_batched}, st
+        got = dst.cpu().numpy().reshape(n_req + 1, piece)
+        for k in range(n_req):
+            np.testing.assert_array_equal(got[n_req - 1 - k], src_np[k * piece:(k + 1) * piece])
+        np.testing.assert_array_equal(got[n_req], src_np[n_req * piece:])
+        if batch == 8:
+            rows, hdr = net.last_table(s)
+            exp_t, exp_h, _ = ob.credit_schedule(n_lanes=8, credits=credits, quantum=chunk, total_bytes=n_req * piece,
+                                                 chunk_bytes=chunk, mode=ob.SCHED_RESET_OFFSETS, state=_state(piece, 8))
+            _same_table(rows, exp_t)
+            np.testing.assert_array_equal(hdr["lane_bytes"], exp_h["lane_bytes"])
+        net.deregMr(s, smh), net.deregMr(r, rmh)
+        net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+    net.reconfigure(NCCL_FUSELINK_BATCH=None)
 
 
 @pytest.mark.parametrize("name", ["fuselink", "libnccl-net-fuselink.so"])
