@@ -67,6 +67,7 @@ SIGNATURES = {
                                      C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_reassemble_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,
                                          C.c_void_p]),
+    "flh_window_export_dmabuf": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.POINTER(C.c_int)]),
     "flh_stripe_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_reassemble_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p]),
     "flh_gather_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),

@@ -325,6 +325,12 @@ class Window:
         n = check(_lib.load().flh_window_slots(self._h, buf, 4096))
         return list(buf[: min(n, 4096)])
 
+    def export_dmabuf(self, offset: int, nbytes: int) -> int:
+        """DMA-BUF descriptor for part of the bound window (the caller closes it)."""
+        fd = C.c_int(-1)
+        check(_lib.load().flh_window_export_dmabuf(self._h, offset, nbytes, C.byref(fd)))
+        return fd.value
+
     def destroy(self) -> None:
         if self._h:
             check(_lib.load().flh_window_destroy(self._h))

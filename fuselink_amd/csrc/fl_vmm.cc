@@ -8,6 +8,8 @@
 // lane for one user allocation, shared and reference counted by base address
 // (src/plugin.cc:1212-1227, 1337-1408).
 #include <hip/hip_runtime.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <cstdlib>
@@ -239,6 +241,30 @@ int flh_window_slots(const flh_window* w, int* slots, int max) {
   std::lock_guard<std::mutex> g(w->pool->mu);
   for (int k = 0; k < max && k < (int)w->slots.size(); ++k) slots[k] = w->slots[k];
   return (int)w->slots.size();
+}
+
+int flh_window_export_dmabuf(const flh_window* w, uint64_t offset, uint64_t bytes, int* fd_out) {
+  if (!w || !fd_out) return fl_set_error(FLH_E_ARG, "null argument");
+  *fd_out = -1;
+  const uint64_t unit = w->pool->unit_bytes;
+  uint64_t bound;
+  {
+    std::lock_guard<std::mutex> g(w->pool->mu);
+    bound = (uint64_t)w->slots.size() * unit;
+  }
+  // one descriptor covers one physical allocation, i.e. one unit (a longer range comes back truncated to its first unit)
+  if (offset % unit || bytes != unit) return fl_set_error(FLH_E_ARG, "offset must be a multiple of the %llu-byte unit and bytes exactly one unit", (unsigned long long)unit);
+  if (offset + bytes > bound) return fl_set_error(FLH_E_RANGE, "range %llu+%llu lies outside the %llu bound bytes", (unsigned long long)offset, (unsigned long long)bytes, (unsigned long long)bound);
+  int fd = -1;
+  FL_HIP(hipMemGetHandleForAddressRange(&fd, (hipDeviceptr_t)(w->base + offset), bytes, hipMemRangeHandleTypeDmaBufFd, 0));
+  if (fd < 0) return fl_set_error(FLH_E_HIP, "no descriptor came back");
+  struct stat st;
+  if (fstat(fd, &st) != 0 || (uint64_t)st.st_size < bytes) {
+    close(fd);
+    return fl_set_error(FLH_E_HIP, "the descriptor covers less than the %llu bytes asked for", (unsigned long long)bytes);
+  }
+  *fd_out = fd;
+  return FLH_OK;
 }
 
 int flh_region_acquire(flh_pool* pool, void* base, uint64_t bytes, uint32_t n_lanes, uint64_t bound_bytes_per_lane,

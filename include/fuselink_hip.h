@@ -254,6 +254,11 @@ void* flh_window_base(const flh_window* w);
 uint64_t flh_window_bound_bytes(const flh_window* w);
 /* slot ids backing the first `max` units, in order; returns the number of bound units */
 int flh_window_slots(const flh_window* w, int* slots, int max);
+/* DMA-BUF file descriptor for one bound staging unit of the window (`offset` a multiple of the unit, `bytes`
+ * exactly one unit: a descriptor covers one physical allocation): what a NIC driver registers so that it can read a lane's staged data, the
+ * counterpart of the reference handing `fd`/`offset` to ibv_reg_dmabuf_mr for every relay buffer
+ * (src/plugin.cc:1278-1280).  The caller closes the descriptor. */
+int flh_window_export_dmabuf(const flh_window* w, uint64_t offset, uint64_t bytes, int* fd_out);
 
 /* ---- regions: the regMr-time object (src/plugin.cc:1168-1330, 1337-1408; src/fuselink.h:39-52) ---
  * One region per base allocation, shared and reference-counted by base address; it owns one

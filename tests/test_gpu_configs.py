@@ -90,6 +90,44 @@ def test_pool_windows_first_fit_and_exhaustion(fl):
     pool.destroy()
 
 
+def test_window_units_export_as_dmabuf(fl):
+    """What a NIC driver needs to read a lane's staged bytes (ibv_reg_dmabuf_mr in src/plugin.cc:1278-1280):
+    a DMA-BUF descriptor for bound units of a staging window."""
+    import os
+    import stat
+    core, torch = fl
+    pool = core.Pool(0, 8)
+    w = core.Window(pool, 8 * MB)
+    w.bind(4 * MB)
+    fds = []
+    try:
+        fds.append(w.export_dmabuf(0, 2 * MB))            # one unit
+        fds.append(w.export_dmabuf(2 * MB, 2 * MB))       # the next one
+        for fd in fds:
+            assert fd > 2
+            st = os.fstat(fd)
+            assert not stat.S_ISREG(st.st_mode) and not stat.S_ISDIR(st.st_mode)   # an anonymous dma-buf inode
+        with pytest.raises(core._lib.FuseLinkError) as e:
+            w.export_dmabuf(4 * MB, 2 * MB)                 # not bound
+        assert e.value.code == -5
+        with pytest.raises(core._lib.FuseLinkError):
+            w.export_dmabuf(4096, 2 * MB)                   # not on a unit boundary
+        with pytest.raises(core._lib.FuseLinkError):
+            w.export_dmabuf(0, 4 * MB)                      # a descriptor covers one unit
+        for fd in fds:
+            assert os.fstat(fd).st_size == 2 * MB
+        # the window still works after the export
+        src = torch.randint(0, 255, (4 * MB,), dtype=torch.uint8, device="cuda")
+        core.check(core._lib.load().flh_copy(C.c_void_p(w.base), C.c_void_p(src.data_ptr()), 4 * MB, None))
+        torch.cuda.synchronize()
+        assert torch.equal(core.read_window(w.base, 4 * MB), src)
+    finally:
+        for fd in fds:
+            os.close(fd)
+    w.destroy()
+    pool.destroy()
+
+
 def test_region_refcount_translate_and_mirror_mode(fl):
     core, torch = fl
     pool = core.Pool(0, 64)
