@@ -124,7 +124,7 @@ def build_monitor(verbose: bool = True) -> str:
 def build_oracle(verbose: bool = True) -> None:
     """Compiles the CPU oracle (test infrastructure) and, where the reference tree is present,
     the reference's own monitor client under oracle/_ref."""
-    cmd = ["make", "-C", os.path.join(ROOT, "oracle"), "all"]
+    cmd = ["make", "-B", "-C", os.path.join(ROOT, "oracle"), "all"]   # always recompiles, like the library
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
