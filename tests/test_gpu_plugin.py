@@ -155,6 +155,46 @@ def test_busy_lane_gets_no_chunks_after_refresh(net):
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
+def test_scheduler_reads_live_credits_from_pinned_host_memory(net):
+    """The credit row the scheduler kernels read may live in pinned host memory that the monitor side rewrites
+    in place: no copy, no semaphore on the request path.  fl_monitor_credits writes the row straight into the
+    pinned table; the next launch sees it."""
+    import ctypes as C
+
+    import torch
+    from fuselink_amd import core
+    L = net.lib
+    lanes, chunk, total = 8, 64 << 10, 37 * (64 << 10) - 100
+    L.fl_monitor_reset()
+    L.fl_monitor_set_clock(1, 5_000_000)
+    row = torch.zeros(lanes, dtype=torch.int32).pin_memory()       # device-visible host memory
+    row_ptr = C.cast(row.data_ptr(), C.POINTER(C.c_uint32))
+    try:
+        for busy in ([], [1, 6], [0, 1, 2, 3, 4, 5, 6, 7]):
+            L.fl_monitor_reset()
+            for l in busy:
+                L.fl_monitor_mark_active(l, 1, 5_000_000 - 20)
+            assert L.fl_monitor_credits(lanes, 3, 4, row_ptr) == 0    # own lane 3 never drops to zero
+            credits = row.numpy().astype(np.uint32).copy()
+            assert list(credits) == [0 if l in busy and l != 3 else (1 if l == 3 and 3 in busy else 4) for l in range(lanes)]
+            exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk)
+            for fast in (1, 0):                                        # closed-form and scan kernels
+                core.tune("sched_uniform_fast", fast)
+                p = core.SchedParams()
+                out = core.new_schedule_buffers(len(exp_t))
+                p.total_bytes, p.chunk_bytes, p.n_chunks, p.n_lanes = total, chunk, len(exp_t), lanes
+                p.d_credits, p.n_rows, p.quantum, p.tile_bytes = row.data_ptr(), 1, chunk, 32768
+                p.d_table, p.d_hdr = out.table.data_ptr(), out.hdr.data_ptr()
+                core.check(core._lib.load().flh_schedule(C.byref(p), None))
+                torch.cuda.synchronize()
+                _same_table(out.table_numpy(), exp_t)
+                np.testing.assert_array_equal(out.hdr_numpy()["lane_chunks"], exp_h["lane_chunks"])
+    finally:
+        core.tune("sched_uniform_fast", 1)
+        L.fl_monitor_set_clock(0, 0)
+        L.fl_monitor_reset()
+
+
 def test_stress_shape_many_requests_in_flight(net):
     """Shape of the stress configuration at a quarter of its size per step: uint32 payload, 64 KiB
     chunks, 16 lanes, credits redrawn at every refresh, 4 requests in flight, windows reused by every
