@@ -213,6 +213,17 @@ int fl_monitor_idle_pick(int is_tx, int group, int mask, int exact) {
   return found;
 }
 
+// Give a borrowed lane back before its timeout runs out (the reference never does: a BORROWED NIC only
+// returns to IDLE through the daemon's ageing, src/monitor.cpp:171-186).  Only a BORROWED entry changes.
+int fl_monitor_release(int lane, int is_tx) {
+  if (lane < 0 || lane >= kGroups) return fl_set_error(FLH_E_ARG, "lane %d out of range", lane);
+  TableLock l;
+  int32_t* st = status_of(is_tx);
+  if (st[lane] != kBorrowed) return 0;
+  st[lane] = kIdle;
+  return 1;
+}
+
 int fl_monitor_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t* credits_out) {
   if (n_lanes < 1 || n_lanes > kGroups || !credits_out) return fl_set_error(FLH_E_ARG, "bad credit query");
   TableLock l;

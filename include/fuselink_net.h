@@ -218,6 +218,9 @@ int fl_monitor_status(int is_tx, int n_lanes, int32_t* status_out);
  * written (every idle NIC met is marked BORROWED and the last one is returned); `exact` = 1 borrows
  * only the first idle NIC, which is what the code evidently meant. */
 int fl_monitor_idle_pick(int is_tx, int group, int mask, int exact);
+/* Returns a BORROWED lane to IDLE at once (1 if it was borrowed, 0 if not): the release the reference
+ * lacks, where a borrowed NIC only comes back through the daemon's ageing (src/monitor.cpp:171-186). */
+int fl_monitor_release(int lane, int is_tx);
 /* credits the scheduler will use from the next refresh on: IDLE -> idle_credit, BUSY/BORROWED -> 0,
  * the comm's own lane never below 1 */
 int fl_monitor_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t* credits_out);

@@ -86,6 +86,23 @@ def _load_status(L, is_tx, status):
         L.fl_monitor_set_entry(i, is_tx, st, 0)
 
 
+def test_exact_borrow_takes_one_lane_and_release_gives_it_back(net):
+    """The fixed borrow (exact = 1) marks only the first idle lane outside the group, and a release returns
+    it at once instead of after the daemon's timeout; BUSY and IDLE entries are not touched by a release."""
+    L = net.lib
+    for is_tx in (1, 0):
+        _load_status(L, is_tx, [0, 1, 0, 0] + [1] * 12)
+        assert L.fl_monitor_idle_pick(is_tx, 0, 0xFFFF, 1) == 2        # lane 0 is the group's own, lane 1 is busy
+        out = (C.c_int32 * 16)()
+        L.fl_monitor_status(is_tx, 16, out)
+        assert list(out)[:4] == [0, 1, 2, 0]
+        assert L.fl_monitor_release(1, is_tx) == 0 and L.fl_monitor_release(3, is_tx) == 0
+        assert L.fl_monitor_release(2, is_tx) == 1
+        L.fl_monitor_status(is_tx, 16, out)
+        assert list(out)[:4] == [0, 1, 0, 0]
+    assert L.fl_monitor_release(16, 1) < 0
+
+
 def test_monitor_random_sequences_match_oracle(net):
     """Random mark / tick / pick sequences: the product table and the oracle's stay identical."""
     L = net.lib
