@@ -409,6 +409,76 @@ def test_sends_that_wait_together_travel_as_one_message(net):
     net.reconfigure(NCCL_FUSELINK_BATCH=None)
 
 
+@pytest.mark.parametrize("block", range(4))
+def test_random_request_streams(net, block):
+    """Seeded random connections: lanes, chunk size, batching, refresh cadence, window size, QP split, policy,
+    request sizes (whole chunks or arbitrary, zero included) and the interleaving of irecv / isend / test all
+    vary; every byte must arrive, nothing may be written past the last request."""
+    import torch
+    buf_bytes = 24 << 20
+    src = torch.randint(0, 255, (buf_bytes,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    for seed in range(block * 12, block * 12 + 12):
+        rng = np.random.default_rng(600_000 + seed)
+        lanes = int(rng.integers(1, 17))
+        chunk = int(rng.choice([4096, 65536, 256 << 10, 512 << 10, 100 * 128]))
+        env = dict(NCCL_FUSELINK_LANES=lanes, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_BATCH=int(rng.choice([1, 2, 8])),
+                   NCCL_FUSELINK_REFRESH_BATCH=int(rng.choice([1, 3, 8])), NCCL_FUSELINK_WINDOW_UNITS=int(rng.choice([1, 2, 4])),
+                   NCCL_IB_QPS_PER_CONNECTION=int(rng.choice([1, 1, 3])), NCCL_FUSELINK_POLICY=int(rng.choice([0, 1, 1])))
+        net.reconfigure(**env)
+        net.set_credits([int(c) for c in rng.integers(0, 9, size=lanes)] if rng.random() < 0.8 else [])
+        dst.zero_()
+        lcomm, s, r = net.connect_pair(int(rng.integers(0, lanes)))
+        _, smh = net.regMr(s, src.data_ptr(), buf_bytes, P.NCCL_PTR_CUDA)
+        _, rmh = net.regMr(r, dst.data_ptr(), buf_bytes, P.NCCL_PTR_CUDA)
+        n_req = int(rng.integers(1, 30))
+        if rng.random() < 0.5:
+            sizes = [int(rng.integers(1, 9)) * chunk for _ in range(n_req)]
+        else:
+            sizes = [int(rng.integers(0, 1 << 20)) for _ in range(n_req)]
+        while sum(sizes) > buf_bytes:
+            sizes.pop()
+        n_req = len(sizes)
+        offs = np.concatenate([[0], np.cumsum(sizes)[:-1]]).astype(np.int64)
+        inflight_max = int(rng.integers(1, 9))
+        posted = sent = done_r = done_s = spins = 0
+        rq, sq = [], []
+        while done_r < n_req or done_s < n_req:
+            spins += 1
+            assert spins < 2_000_000, f"seed {seed}: no progress"
+            if posted < n_req and posted - done_r < inflight_max:
+                rc, q = net.irecv(r, [dst.data_ptr() + int(offs[posted])], [sizes[posted]], [posted], [rmh])
+                assert rc == 0
+                if q:
+                    rq.append((q, sizes[posted]))
+                    posted += 1
+            if sent < posted and rng.random() < 0.7:
+                rc, q = net.isend(s, src.data_ptr() + int(offs[sent]), sizes[sent], sent, smh)
+                assert rc == 0
+                if q:
+                    sq.append(q)
+                    sent += 1
+            if rq and rng.random() < 0.5:
+                rc, d, sz = net.test(rq[0][0])
+                assert rc == 0
+                if d:
+                    assert sz == rq[0][1]
+                    rq.pop(0)
+                    done_r += 1
+            if sq and rng.random() < 0.5:
+                rc, d, _ = net.test(sq[0])
+                assert rc == 0
+                if d:
+                    sq.pop(0)
+                    done_s += 1
+        torch.cuda.synchronize()
+        tot = int(sum(sizes))
+        assert torch.equal(dst[:tot], src[:tot]), f"seed {seed}: data differs ({env})"
+        assert not dst[tot:tot + 4096].any(), f"seed {seed}: wrote past the end"
+        net.deregMr(s, smh), net.deregMr(r, rmh)
+        net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
 @pytest.mark.parametrize("name", ["fuselink", "libnccl-net-fuselink.so"])
 def test_rccl_loads_the_plugin_and_probes_every_device(name):
     """What the reference's README asks of a user (NCCL_NET_PLUGIN=fuselink, README.md:35-40), under this
