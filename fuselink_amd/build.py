@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libnccl-net-fuselink.so"
 
-SOURCES = ["fl_kernels.hip", "fl_vmm.cc", "fl_monitor.cc", "fl_plugin.cc"]
+SOURCES = ["fl_sched.hip", "fl_copy.hip", "fl_runtime.cc", "fl_vmm.cc", "fl_monitor.cc", "fl_plugin.cc"]
 
 # -packed-fp32-ops: keep the compiler from forming packed FP32 instructions (none are wanted in a
 # byte mover, and some forms are unreliable on this hardware).

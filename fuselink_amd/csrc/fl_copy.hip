@@ -1,0 +1,718 @@
+// fl_copy.hip -- the byte movers and their entry points:
+//   * fl_copy_uniform_fused : scheduling and copy in one launch (uniform split, one credit row), also for a batch of requests
+//   * fl_copy_uniform       : table-driven stripe / reassemble for a uniform split (2-D grid)
+//   * fl_copy_tiles         : the same for any table (tile -> row by a wavefront search)
+//   * fl_page_tiles         : paged gather / scatter (non-contiguous pages <-> lane windows)
+//   * fl_plain_copy         : calibration copy with the same inner loop
+// The path is an HBM-bound byte mover; nothing here contracts, so no MFMA.
+#include <cstring>
+
+#include "fl_device.h"
+#include "fl_launch.h"
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+// copy kernels
+// ------------------------------------------------------------------------------------------------
+
+constexpr int kCopyBlock = 256;
+constexpr int kCopyUnroll = 8;
+
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const u32x4* p) {
+  return NT ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool NT>
+__device__ __forceinline__ void st16(u32x4* p, u32x4 v) {
+  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+}
+
+template <bool NT, int U>
+__device__ __forceinline__ void copy_exact(u32x4* __restrict__ d, const u32x4* __restrict__ s, uint32_t tid) {
+  u32x4 r[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) r[j] = ld16<NT>(s + j * kCopyBlock + tid);
+#pragma unroll
+  for (int j = 0; j < U; ++j) st16<NT>(d + j * kCopyBlock + tid, r[j]);
+}
+
+// Copies `bytes` from src to dst with the whole workgroup.  Fast path: both 16-byte aligned ->
+// dwordx4 loads batched kCopyUnroll deep before the stores.  Equal misalignment: byte head up to
+// the boundary, vectors, byte tail.  Different misalignment: byte copy (correct, not fast).
+template <bool NT>
+__device__ __forceinline__ void block_copy(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
+                                           uint32_t bytes) {
+  const uint32_t tid = threadIdx.x;
+  const uintptr_t sa = (uintptr_t)src, da = (uintptr_t)dst;
+  if (((sa ^ da) & 15) != 0) {
+    for (uint32_t i = tid; i < bytes; i += kCopyBlock) dst[i] = src[i];
+    return;
+  }
+  uint32_t head = (uint32_t)((16 - (sa & 15)) & 15);
+  if (head > bytes) head = bytes;
+  if (tid < head) dst[tid] = src[tid];
+  const uint32_t body = bytes - head;
+  const uint32_t nvec = body >> 4;
+  const u32x4* s = (const u32x4*)(src + head);
+  u32x4* d = (u32x4*)(dst + head);
+  // whole tiles of the usual sizes: every load of the tile is issued before the first store, unpredicated
+  if (nvec == kCopyBlock * 16) { copy_exact<NT, 16>(d, s, tid); }
+  else if (nvec == kCopyBlock * 8) { copy_exact<NT, 8>(d, s, tid); }
+  else if (nvec == kCopyBlock * 4) { copy_exact<NT, 4>(d, s, tid); }
+  else {
+    for (uint32_t b = 0; b < nvec; b += kCopyBlock * kCopyUnroll) {
+      u32x4 r[kCopyUnroll];
+#pragma unroll
+      for (int j = 0; j < kCopyUnroll; ++j) {
+        const uint32_t idx = b + j * kCopyBlock + tid;
+        if (idx < nvec) r[j] = ld16<NT>(s + idx);
+      }
+#pragma unroll
+      for (int j = 0; j < kCopyUnroll; ++j) {
+        const uint32_t idx = b + j * kCopyBlock + tid;
+        if (idx < nvec) st16<NT>(d + idx, r[j]);
+      }
+    }
+  }
+  const uint32_t tail0 = head + (nvec << 4);
+  const uint32_t tail = bytes - tail0;
+  if (tid < tail) dst[tail0 + tid] = src[tail0 + tid];
+}
+
+struct CopyArgs {
+  uint8_t* user;
+  uint64_t user_bytes;
+  flh_windows win;
+  const flh_chunk_desc* table;
+  const flh_sched_hdr* hdr;
+  int32_t* status;
+  uint32_t n_chunks_max;
+  uint32_t tile_bytes;
+  // header fields the host already knows (has_hint != 0): saves one dependent memory round trip
+  uint32_t has_hint, hint_total_tiles, hint_n_chunks, hint_uniform_tiles;
+};
+
+// Row of the table that owns copy tile t: the last row with tile_base <= t (rows of empty chunks own
+// no tile and are stepped over).  A uniform split is answered by one division and one row load; any
+// other table by a 64-ary search in which every lane of the wavefront probes one row per round
+// (three rounds cover 262144 chunks).  The result is wavefront-uniform.
+__device__ __forceinline__ uint32_t find_row(const flh_chunk_desc* __restrict__ table, uint32_t n, uint32_t t,
+                                             uint32_t uniform_tiles, uint32_t tile_bytes) {
+  if (uniform_tiles) {
+    const uint32_t c = t / uniform_tiles;
+    if (c < n) {
+      const uint32_t tb = table[c].tile_base;
+      const uint32_t len = table[c].len;
+      if (t >= tb && (uint64_t)(t - tb) * tile_bytes < len) return c;
+    }
+  }
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint32_t lo = 0, cnt = n;  // the answer lies in [lo, lo + cnt); table[lo].tile_base <= t
+  while (cnt > 1) {
+    const uint32_t step = (cnt + kWave - 1) / kWave;
+    const uint32_t idx = lo + lane * step;
+    const bool le = idx < lo + cnt && table[idx].tile_base <= t;
+    const uint32_t k = (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+    const uint32_t adv = (k ? k - 1 : 0) * step;
+    const uint32_t end = lo + cnt;
+    lo += adv;
+    cnt = end - lo < step ? end - lo : step;
+  }
+  return lo;
+}
+
+// DIR 0: user -> windows (stripe).  DIR 1: windows -> user (reassemble).
+template <int DIR, bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
+  const uint32_t total = a.has_hint ? a.hint_total_tiles : a.hdr->total_tiles;
+  const uint32_t uniform_tiles = a.has_hint ? a.hint_uniform_tiles : a.hdr->uniform_tiles;
+  uint32_t n = a.has_hint ? a.hint_n_chunks : a.hdr->n_chunks;
+  if (n > a.n_chunks_max) n = a.n_chunks_max;
+  if (n == 0) return;
+  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
+    const uint32_t c = find_row(a.table, n, t, uniform_tiles, a.tile_bytes);
+    const flh_chunk_desc d = a.table[c];
+    const uint64_t off = (uint64_t)(t - d.tile_base) * a.tile_bytes;
+    if (t < d.tile_base || off >= d.len) continue;
+    const uint32_t bytes = (uint32_t)((d.len - off) < a.tile_bytes ? (d.len - off) : a.tile_bytes);
+    // refuse anything that would leave the user buffer or the mapped part of the window
+    bool ok = d.lane < a.win.n_lanes;
+    if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane] && d.src_off + d.len <= a.user_bytes;
+    if (!ok) {
+      if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+      continue;
+    }
+    uint8_t* u = a.user + d.src_off + off;
+    uint8_t* w = (uint8_t*)a.win.base[d.lane] + d.win_off + off;
+    if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+  }
+}
+
+// Uniform split with the header known on the host: a two-dimensional grid (tile in chunk, chunk)
+// names the work directly, so a workgroup's only dependent access before its data is the one scalar
+// load of its table row.
+template <int DIR, bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform(CopyArgs a) {
+  const uint32_t c = blockIdx.y;
+  if (c >= a.hint_n_chunks) return;
+  const flh_chunk_desc d = a.table[c];
+  const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
+  if (off >= d.len) return;
+  const uint32_t bytes = (uint32_t)((d.len - off) < a.tile_bytes ? (d.len - off) : a.tile_bytes);
+  bool ok = d.lane < a.win.n_lanes;
+  if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane] && d.src_off + d.len <= a.user_bytes;
+  if (!ok) {
+    if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+    return;
+  }
+  uint8_t* u = a.user + d.src_off + off;
+  uint8_t* w = (uint8_t*)a.win.base[d.lane] + d.win_off + off;
+  if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+}
+
+// Scheduler and copy in one launch, for the ordinary case of a uniform split under one credit row:
+// the workgroup that copies tile k of chunk c works out the chunk's lane and window offset itself
+// from the closed form (no table row to wait for), and the workgroup of tile 0 also writes the row
+// out, so that the table exists for the receiver and for inspection exactly as the scheduler kernel
+// would have produced it.  Window offsets start at zero (the windows are reused message by message).
+struct FusedArgs {
+  uint8_t* user;
+  uint64_t user_bytes;
+  flh_windows win;
+  flh_chunk_desc* table;     // out (stripe only), may be null
+  flh_sched_hdr* hdr;        // out (stripe only), may be null
+  int32_t* status;
+  uint64_t total_bytes;
+  uint64_t src_base;
+  uint64_t quanta_before;    // quanta of the current epoch already behind chunk 0 (epoch bytes / chunk)
+  uint32_t chunk_bytes;
+  uint32_t n_chunks;
+  uint32_t n_lanes;
+  uint32_t tile_bytes;
+  uint32_t tiles_per_chunk;
+  uint32_t dest_order;       // stripe only: blockIdx.y counts chunks in destination order (lane by lane)
+  uint32_t credits[FLH_MAX_LANES];
+  // Worked out once on the host when every quantum index and the credit sum W fit 32 bits: the per-workgroup
+  // division by W becomes one multiply-high by magic = ceil(2^64 / W) (exact for 32-bit operands), and the
+  // lane's slots before the message come from cnt0[] instead of a second and third division.
+  uint32_t fast;
+  uint64_t magic;
+  uint32_t cnt0[FLH_MAX_LANES];
+};
+
+// Several requests as one message: chunk c belongs to the request r with first[r] <= c < first[r+1];
+// its bytes live at user[r] + (c - first[r]) * chunk_bytes.
+struct FusedBatchArgs : FusedArgs {
+  uint32_t n_req;
+  uint32_t first[FLH_BATCH_MAX];   // first chunk of each request
+  uint8_t* req_user[FLH_BATCH_MAX];
+  uint64_t req_bytes[FLH_BATCH_MAX];
+};
+template <class A> struct is_batch { static constexpr bool value = false; };
+template <> struct is_batch<FusedBatchArgs> { static constexpr bool value = true; };
+
+struct FusedRow {  // inclusive credit prefixes of the one row (equal credits if it is empty)
+  uint64_t pfx[FLH_MAX_LANES];
+  uint64_t W;
+  bool zero;
+};
+
+__device__ __forceinline__ void fused_row(const FusedArgs& a, FusedRow& r) {
+  uint64_t run = 0;
+#pragma unroll
+  for (int l = 0; l < FLH_MAX_LANES; ++l) { if ((uint32_t)l < a.n_lanes) run += a.credits[l]; r.pfx[l] = run; }
+  r.zero = run == 0;
+  if (r.zero) {
+#pragma unroll
+    for (int l = 0; l < FLH_MAX_LANES; ++l) r.pfx[l] = (uint32_t)l < a.n_lanes ? l + 1 : a.n_lanes;
+    run = a.n_lanes;
+  }
+  r.W = run;
+}
+
+// slots y < x that belong to the lane with prefix bounds [K, hi)
+__device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t hi, uint64_t x) {
+  const uint64_t c = hi - K;
+  const uint64_t full = div_u64(x, W);
+  const uint64_t rem = x - full * W;
+  const uint64_t part = rem <= K ? 0 : (rem - K < c ? rem - K : c);
+  return full * c + part;
+}
+
+template <int DIR, bool NT, class Args>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
+  constexpr bool BATCH = is_batch<Args>::value;
+  if (blockIdx.y >= a.n_chunks) return;
+  FusedRow r;
+  fused_row(a, r);
+  uint32_t c = blockIdx.y, lane = 0;
+  uint64_t K = 0, hi = r.pfx[0], before;
+  if (DIR == 0 && a.dest_order) {
+    // blockIdx.y = k-th chunk in destination order: find the lane whose group holds k, then invert the
+    // closed form -- the j-th slot of a lane with credit c_l and first slot K_l is (j / c_l) * W + K_l + j mod c_l.
+    const uint64_t x0 = a.quanta_before, x1 = a.quanta_before + a.n_chunks;
+    const uint64_t f0 = div_u64(x0, r.W), f1 = div_u64(x1, r.W);
+    const uint64_t r0 = x0 - f0 * r.W, r1 = x1 - f1 * r.W;
+    uint64_t k = blockIdx.y, cnt0 = 0;
+    bool found = false;
+    uint64_t lo = 0;
+#pragma unroll
+    for (int l = 0; l < FLH_MAX_LANES; ++l) {
+      const uint64_t up = r.pfx[l], cl = up - lo;
+      const uint64_t p0 = r0 <= lo ? 0 : (r0 - lo < cl ? r0 - lo : cl);
+      const uint64_t p1 = r1 <= lo ? 0 : (r1 - lo < cl ? r1 - lo : cl);
+      const uint64_t c0 = f0 * cl + p0;             // slots of the lane before this message
+      const uint64_t nl = f1 * cl + p1 - c0;        // chunks of this message on the lane
+      if (!found && (uint32_t)l < a.n_lanes) {
+        if (k < nl) { found = true; lane = l; K = lo; hi = up; cnt0 = c0; } else { k -= nl; }
+      }
+      lo = up;
+    }
+    const uint64_t cl = hi - K;
+    const uint64_t ja = cnt0 + k;                   // index among all slots of the lane in this epoch
+    const uint64_t rnd = div_u64(ja, cl);
+    c = (uint32_t)(rnd * r.W + K + (ja - rnd * cl) - a.quanta_before);
+    before = k;
+  } else if (a.fast) {
+    const uint32_t j = (uint32_t)a.quanta_before + c;
+    const uint32_t full = (uint32_t)__umul64hi((uint64_t)j, a.magic);  // j / W
+    const uint32_t slot = j - full * (uint32_t)r.W;
+    uint32_t c0 = a.cnt0[0];
+#pragma unroll
+    for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
+      if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; c0 = a.cnt0[l + 1]; }
+    }
+    before = (uint64_t)full * (hi - K) + (slot - K) - c0;  // slot lies inside the lane's span [K, hi)
+  } else {
+    const uint64_t j = a.quanta_before + c;
+    const uint64_t slot = mod_u64(j, r.W);
+#pragma unroll
+    for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
+      if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; }
+    }
+    before = fused_cnt(r.W, K, hi, j) - fused_cnt(r.W, K, hi, a.quanta_before);
+  }
+  const uint64_t chunk_off = (uint64_t)c * a.chunk_bytes;
+  const uint64_t rem = a.total_bytes - chunk_off;
+  const uint32_t len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
+  const uint64_t src_off = a.src_base + chunk_off;
+  const uint64_t win_off = before * a.chunk_bytes;
+  // where the chunk's bytes live on the user side: in the one buffer, or in its request's buffer
+  uint8_t* user = a.user;
+  uint64_t user_off = src_off, user_bytes = a.user_bytes;
+  if constexpr (BATCH) {
+    uint32_t first = 0;
+    user = a.req_user[0];
+    user_bytes = a.req_bytes[0];
+#pragma unroll
+    for (int q = 1; q < FLH_BATCH_MAX; ++q) {
+      if ((uint32_t)q < a.n_req && a.first[q] <= c) { first = a.first[q]; user = a.req_user[q]; user_bytes = a.req_bytes[q]; }
+    }
+    user_off = (uint64_t)(c - first) * a.chunk_bytes;
+  }
+
+  if (DIR == 0 && blockIdx.x == 0 && threadIdx.x == 0 && a.table) {
+    flh_chunk_desc d;
+    d.src_off = src_off;
+    d.win_off = win_off;
+    d.len = len;
+    d.lane = lane;
+    d.tile_base = c * a.tiles_per_chunk;
+    d.epoch = 0;
+    a.table[c] = d;
+  }
+  if (DIR == 0 && blockIdx.x == 0 && blockIdx.y == 0 && a.hdr) {  // header: per-lane totals in closed form
+    const uint32_t t = threadIdx.x;
+    const uint64_t last = a.n_chunks - 1;
+    const uint64_t len_last = a.total_bytes - last * a.chunk_bytes;
+    if (t < FLH_MAX_LANES) {
+      uint64_t chunks = 0, bytes = 0;
+      if (t < a.n_lanes) {
+        uint64_t k_lo = 0, k_hi = 0;  // selected, not indexed: indexing would push the row into scratch memory
+#pragma unroll
+        for (int l = 0; l < FLH_MAX_LANES; ++l) {
+          if ((uint32_t)l == t) { k_hi = r.pfx[l]; k_lo = l ? r.pfx[l > 0 ? l - 1 : 0] : 0; }
+        }
+        chunks = fused_cnt(r.W, k_lo, k_hi, a.quanta_before + a.n_chunks) - fused_cnt(r.W, k_lo, k_hi, a.quanta_before);
+        const uint64_t slot_last = mod_u64(a.quanta_before + last, r.W);
+        const bool mine = slot_last >= k_lo && slot_last < k_hi;
+        bytes = chunks * a.chunk_bytes - (mine ? a.chunk_bytes - len_last : 0);
+      }
+      a.hdr->lane_bytes[t] = bytes;
+      a.hdr->lane_chunks[t] = (uint32_t)chunks;
+    }
+    if (t == 0) {
+      a.hdr->total_bytes = a.total_bytes;
+      a.hdr->total_tiles = (uint32_t)last * a.tiles_per_chunk + (uint32_t)((len_last + a.tile_bytes - 1) / a.tile_bytes);
+      a.hdr->n_chunks = a.n_chunks;
+      a.hdr->flags = r.zero ? FLH_SCHED_F_NO_CREDIT : 0;
+      a.hdr->uniform_tiles = a.tiles_per_chunk;
+    }
+  }
+
+  const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
+  if (off >= len) return;
+  const uint32_t bytes = (uint32_t)((len - off) < a.tile_bytes ? (len - off) : a.tile_bytes);
+  if (win_off + len > a.win.cap[lane] || user_off + len > user_bytes) {
+    if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+    return;
+  }
+  uint8_t* u = user + user_off + off;
+  uint8_t* w = (uint8_t*)a.win.base[lane] + win_off + off;
+  if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+}
+
+struct PageArgs {
+  uint8_t* pool;
+  uint64_t pool_pages;
+  const uint32_t* page_table;
+  flh_windows win;
+  const flh_chunk_desc* table;
+  int32_t* status;
+  uint32_t n_chunks;
+  uint32_t page_bytes;
+  uint32_t pages_per_chunk;
+  uint32_t sub_bytes;      // bytes of a page handled by one workgroup step
+  uint32_t subs_per_page;
+  int32_t page_shift;      // >= 0 when page_bytes is a power of two
+};
+
+constexpr uint32_t kLdsStage = 16384;
+
+// DIR 0: pool pages -> windows (gather).  DIR 1: windows -> pool pages (scatter).
+// LDS: stage each sub-tile through LDS (coalesced global->LDS, barrier, LDS->global).
+template <int DIR, bool LDS, bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
+  __shared__ u32x4 stage[LDS ? kLdsStage / 16 : 1];
+  const uint64_t total = (uint64_t)a.n_chunks * a.pages_per_chunk * a.subs_per_page;
+  for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
+    const uint32_t sub = (uint32_t)(t % a.subs_per_page);
+    const uint64_t rp = t / a.subs_per_page;         // row-major page counter
+    const uint32_t c = (uint32_t)(rp / a.pages_per_chunk);
+    const uint32_t k = (uint32_t)(rp % a.pages_per_chunk);
+    const flh_chunk_desc d = a.table[c];
+    const uint64_t in_chunk = (uint64_t)k * a.page_bytes + (uint64_t)sub * a.sub_bytes;
+    if (in_chunk >= d.len) continue;
+    uint32_t bytes = a.page_bytes - sub * a.sub_bytes;
+    if (bytes > a.sub_bytes) bytes = a.sub_bytes;
+    if (bytes > d.len - in_chunk) bytes = (uint32_t)(d.len - in_chunk);
+    // the chunk's place in the message comes from its source offset, not from the row's position, so the
+    // rows may come in any order (destination order for the gather)
+    const uint64_t p = (a.page_shift >= 0 ? d.src_off >> a.page_shift : d.src_off / a.page_bytes) + k;
+    const bool aligned = a.page_shift >= 0 ? (d.src_off & (a.page_bytes - 1)) == 0 : d.src_off % a.page_bytes == 0;
+    if (!aligned || p >= (uint64_t)a.n_chunks * a.pages_per_chunk) {
+      if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+      continue;
+    }
+    const uint32_t pg = a.page_table[p];
+    bool ok = d.lane < a.win.n_lanes && pg < a.pool_pages;
+    if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane];
+    if (!ok) {
+      if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+      continue;
+    }
+    uint8_t* u = a.pool + (uint64_t)pg * a.page_bytes + (uint64_t)sub * a.sub_bytes;
+    uint8_t* w = (uint8_t*)a.win.base[d.lane] + d.win_off + in_chunk;
+    uint8_t* dst = DIR == 0 ? w : u;
+    const uint8_t* src = DIR == 0 ? u : w;
+    if (LDS && ((((uintptr_t)src | (uintptr_t)dst) & 15) == 0) && (bytes & 15) == 0) {
+      const uint32_t nvec = bytes >> 4;  // <= kLdsStage/16 by construction of sub_bytes
+      const u32x4* s = (const u32x4*)src;
+      u32x4* dd = (u32x4*)dst;
+      for (uint32_t i = threadIdx.x; i < nvec; i += kCopyBlock) stage[i] = ld16<NT>(s + i);
+      __syncthreads();
+      for (uint32_t i = threadIdx.x; i < nvec; i += kCopyBlock) st16<NT>(dd + i, stage[i]);
+      __syncthreads();
+    } else {
+      block_copy<NT>(dst, src, bytes);
+    }
+  }
+}
+
+template <bool NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const uint8_t* src, uint64_t bytes,
+                                                            uint32_t tile_bytes) {
+  const uint64_t tiles = (bytes + tile_bytes - 1) / tile_bytes;
+  for (uint64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+    const uint64_t off = t * tile_bytes;
+    const uint32_t len = (uint32_t)((bytes - off) < tile_bytes ? (bytes - off) : tile_bytes);
+    block_copy<NT>(dst + off, src + off, len);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+static int check_windows(const flh_windows* win) {
+  if (!win) return fl_set_error(FLH_E_ARG, "null windows");
+  if (win->n_lanes == 0 || win->n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "windows.n_lanes %u not in 1..%d", win->n_lanes, FLH_MAX_LANES);
+  for (uint32_t l = 0; l < win->n_lanes; ++l)
+    if (!win->base[l] && win->cap[l]) return fl_set_error(FLH_E_ARG, "window %u has capacity but no base", l);
+  return FLH_OK;
+}
+
+static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
+                       const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream) {
+  int rc = check_windows(win);
+  if (rc) return rc;
+  if (!d_hdr || !d_status) return fl_set_error(FLH_E_ARG, "d_hdr and d_status are required");
+  if (n_chunks_max && !d_table) return fl_set_error(FLH_E_ARG, "d_table missing");
+  if (tile_bytes == 0 || tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", tile_bytes);
+  if (user_bytes && !user) return fl_set_error(FLH_E_ARG, "user buffer missing");
+  if (n_chunks_max == 0) return FLH_OK;
+  rc = fl_need_init();
+  if (rc) return rc;
+  fl_prof().kid = dir == 0 ? 2 : 3;
+  CopyArgs a;
+  a.user = (uint8_t*)user;
+  a.user_bytes = user_bytes;
+  a.win = *win;
+  a.table = d_table;
+  a.hdr = d_hdr;
+  a.status = d_status;
+  a.n_chunks_max = n_chunks_max;
+  a.tile_bytes = tile_bytes;
+  a.has_hint = h_hdr != nullptr;
+  a.hint_total_tiles = h_hdr ? h_hdr->total_tiles : 0;
+  a.hint_n_chunks = h_hdr ? h_hdr->n_chunks : 0;
+  a.hint_uniform_tiles = h_hdr ? h_hdr->uniform_tiles : 0;
+  const uint64_t max_tiles = h_hdr ? h_hdr->total_tiles : user_bytes / tile_bytes + n_chunks_max;
+  if (max_tiles == 0) return FLH_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const bool nt = fl_use_nt(3 * user_bytes);  // user buffer + windows + the peer's buffer
+  if (h_hdr && h_hdr->uniform_tiles && h_hdr->n_chunks <= 65535 && h_hdr->n_chunks <= n_chunks_max && g_copy_uniform_grid) {
+    const dim3 grid(h_hdr->uniform_tiles, h_hdr->n_chunks);
+    if (dir == 0) {
+      if (nt) FL_LAUNCH((fl_copy_uniform<0, true>), grid, dim3(kCopyBlock), 0, s, a);
+      else FL_LAUNCH((fl_copy_uniform<0, false>), grid, dim3(kCopyBlock), 0, s, a);
+    } else {
+      if (nt) FL_LAUNCH((fl_copy_uniform<1, true>), grid, dim3(kCopyBlock), 0, s, a);
+      else FL_LAUNCH((fl_copy_uniform<1, false>), grid, dim3(kCopyBlock), 0, s, a);
+    }
+    FL_HIP(hipGetLastError());
+    return FLH_OK;
+  }
+  const uint32_t grid = fl_copy_grid(max_tiles);
+  if (dir == 0) {
+    if (nt) FL_LAUNCH((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_tiles<0, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+  } else {
+    if (nt) FL_LAUNCH((fl_copy_tiles<1, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_tiles<1, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
+  }
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
+               const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, uint32_t n_chunks_max, uint32_t tile_bytes,
+               int32_t* d_status, void* stream) {
+  return launch_copy(0, (void*)d_src, src_bytes, win, d_table, d_hdr, h_hdr, n_chunks_max, tile_bytes, d_status, stream);
+}
+
+int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_chunk_desc* d_table,
+                   const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, uint32_t n_chunks_max, uint32_t tile_bytes,
+                   int32_t* d_status, void* stream) {
+  return launch_copy(1, d_dst, dst_bytes, win, d_table, d_hdr, h_hdr, n_chunks_max, tile_bytes, d_status, stream);
+}
+
+// argument checks and everything of FusedArgs that follows from the parameters; returns 1 when there is nothing to do
+static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_uniform_params* u, flh_chunk_desc* d_table,
+                      flh_sched_hdr* d_hdr, int32_t* d_status) {
+  int rc = check_windows(win);
+  if (rc) return rc;
+  if (!u || !d_status) return fl_set_error(FLH_E_ARG, "parameters and d_status are required");
+  if (u->n_lanes == 0 || u->n_lanes > FLH_MAX_LANES || u->n_lanes != win->n_lanes) return fl_set_error(FLH_E_ARG, "n_lanes %u does not match the windows' %u", u->n_lanes, win->n_lanes);
+  if (u->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0");
+  if (u->tile_bytes == 0 || u->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", u->tile_bytes);
+  if (u->total_bytes == 0) return 1;
+  const uint64_t n = (u->total_bytes + u->chunk_bytes - 1) / u->chunk_bytes;
+  if (n > 65535) return fl_set_error(FLH_E_ARG, "%llu chunks exceed the 65535 one launch can name; split the message", (unsigned long long)n);
+  rc = fl_need_init();
+  if (rc) return rc;
+  fl_prof().kid = dir == 0 ? 2 : 3;
+  a.user = nullptr;
+  a.user_bytes = 0;
+  a.win = *win;
+  a.table = dir == 0 ? d_table : nullptr;
+  a.hdr = dir == 0 ? d_hdr : nullptr;
+  a.status = d_status;
+  a.total_bytes = u->total_bytes;
+  a.src_base = u->src_base;
+  a.quanta_before = u->epoch_bytes / u->chunk_bytes;
+  a.chunk_bytes = u->chunk_bytes;
+  a.n_chunks = (uint32_t)n;
+  a.n_lanes = u->n_lanes;
+  a.tile_bytes = u->tile_bytes;
+  a.tiles_per_chunk = (u->chunk_bytes + u->tile_bytes - 1) / u->tile_bytes;
+  // once the message no longer fits the Infinity Cache, write every window front to back
+  a.dest_order = dir == 0 && (g_dest_order < 0 ? 3 * u->total_bytes > kCacheResidentBytes : g_dest_order != 0);
+  for (int l = 0; l < FLH_MAX_LANES; ++l) a.credits[l] = (uint32_t)l < u->n_lanes ? u->credits[l] : 0;
+  {
+    // the row as the kernel sees it (equal credits stand in for an all-zero row), then the host-side constants
+    uint64_t pfx[FLH_MAX_LANES], W = 0;
+    for (uint32_t l = 0; l < u->n_lanes; ++l) { W += u->credits[l]; pfx[l] = W; }
+    if (W == 0) { for (uint32_t l = 0; l < u->n_lanes; ++l) pfx[l] = l + 1; W = u->n_lanes; }
+    a.fast = W >= 2 && W <= 0xffffffffull && a.quanta_before + n <= 0xffffffffull && g_fused_fast;
+    a.magic = a.fast ? ~0ull / W + 1 : 0;
+    for (int l = 0; l < FLH_MAX_LANES; ++l) a.cnt0[l] = 0;
+    if (a.fast) {
+      const uint64_t full = a.quanta_before / W, rem = a.quanta_before % W;
+      for (uint32_t l = 0; l < u->n_lanes; ++l) {
+        const uint64_t K = l ? pfx[l - 1] : 0, cl = pfx[l] - K;
+        const uint64_t part = rem <= K ? 0 : (rem - K < cl ? rem - K : cl);
+        a.cnt0[l] = (uint32_t)(full * cl + part);
+      }
+    }
+  }
+  return FLH_OK;
+}
+
+extern "C++" {
+template <class Args>
+static int launch_fused_args(int dir, const Args& a, bool nt, void* stream) {
+  const dim3 grid(a.tiles_per_chunk, a.n_chunks);
+  hipStream_t s = (hipStream_t)stream;
+  if (dir == 0) {
+    if (nt) FL_LAUNCH((fl_copy_uniform_fused<0, true, Args>), grid, dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_uniform_fused<0, false, Args>), grid, dim3(kCopyBlock), 0, s, a);
+  } else {
+    if (nt) FL_LAUNCH((fl_copy_uniform_fused<1, true, Args>), grid, dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_uniform_fused<1, false, Args>), grid, dim3(kCopyBlock), 0, s, a);
+  }
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+}  // extern "C++"
+
+static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_uniform_params* u,
+                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream) {
+  FusedArgs a;
+  const int rc = fill_fused(a, dir, win, u, d_table, d_hdr, d_status);
+  if (rc) return rc < 0 ? rc : FLH_OK;
+  if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
+  a.user = (uint8_t*)user;
+  a.user_bytes = user_bytes;
+  return launch_fused_args(dir, a, fl_use_nt(3 * user_bytes), stream);
+}
+
+static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table, flh_sched_hdr* d_hdr,
+                        int32_t* d_status, void* stream) {
+  if (!b) return fl_set_error(FLH_E_ARG, "null batch");
+  if (b->n_req == 0 || b->n_req > FLH_BATCH_MAX) return fl_set_error(FLH_E_ARG, "n_req %u not in 1..%d", b->n_req, FLH_BATCH_MAX);
+  FusedBatchArgs a;
+  const int rc = fill_fused(a, dir, win, &b->u, d_table, d_hdr, d_status);
+  if (rc) return rc < 0 ? rc : FLH_OK;
+  a.dest_order = 0;
+  a.src_base = 0;
+  a.n_req = b->n_req;
+  uint64_t sum = 0;
+  for (uint32_t q = 0; q < FLH_BATCH_MAX; ++q) {
+    a.first[q] = 0;
+    a.req_user[q] = nullptr;
+    a.req_bytes[q] = 0;
+    if (q >= b->n_req) continue;
+    void* p = dir == 0 ? (void*)b->d_src[q] : b->d_dst[q];
+    if (!p || b->bytes[q] == 0) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer or no bytes", q);
+    if (q + 1 < b->n_req && b->bytes[q] % b->u.chunk_bytes) return fl_set_error(FLH_E_ARG, "request %u of the batch is not a whole number of chunks", q);
+    a.first[q] = (uint32_t)(sum / b->u.chunk_bytes);
+    a.req_user[q] = (uint8_t*)p;
+    a.req_bytes[q] = b->bytes[q];
+    sum += b->bytes[q];
+  }
+  if (sum != b->u.total_bytes) return fl_set_error(FLH_E_ARG, "the requests hold %llu bytes, the parameters say %llu", (unsigned long long)sum, (unsigned long long)b->u.total_bytes);
+  return launch_fused_args(dir, a, fl_use_nt(3 * sum), stream);
+}
+
+int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
+                     int32_t* d_status, void* stream) {
+  return launch_batch(0, b, win, d_table_out, d_hdr_out, d_status, stream);
+}
+
+int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int32_t* d_status, void* stream) {
+  return launch_batch(1, b, win, nullptr, nullptr, d_status, stream);
+}
+
+int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_uniform_params* u,
+                       flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
+  return launch_fused(0, (void*)d_src, src_bytes, win, u, d_table_out, d_hdr_out, d_status, stream);
+}
+
+int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_uniform_params* u,
+                           int32_t* d_status, void* stream) {
+  return launch_fused(1, d_dst, dst_bytes, win, u, nullptr, nullptr, d_status, stream);
+}
+
+static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                        uint32_t pages_per_chunk, const flh_windows* win, const flh_chunk_desc* d_table, uint32_t n_chunks,
+                        int use_lds, int32_t* d_status, void* stream) {
+  int rc = check_windows(win);
+  if (rc) return rc;
+  if (!pool || !d_page_table || !d_status) return fl_set_error(FLH_E_ARG, "pool, page table and status are required");
+  if (page_bytes == 0 || pages_per_chunk == 0) return fl_set_error(FLH_E_ARG, "page_bytes and pages_per_chunk must be > 0");
+  if (n_chunks == 0) return FLH_OK;
+  if (!d_table) return fl_set_error(FLH_E_ARG, "d_table missing");
+  rc = fl_need_init();
+  if (rc) return rc;
+  fl_prof().kid = dir == 0 ? 4 : 5;
+  PageArgs a;
+  a.pool = (uint8_t*)pool;
+  a.pool_pages = pool_pages;
+  a.page_table = d_page_table;
+  a.win = *win;
+  a.table = d_table;
+  a.status = d_status;
+  a.n_chunks = n_chunks;
+  a.page_bytes = page_bytes;
+  a.pages_per_chunk = pages_per_chunk;
+  const uint32_t sub = use_lds ? kLdsStage : FLH_TILE_BYTES;
+  a.sub_bytes = page_bytes < sub ? page_bytes : sub;
+  a.subs_per_page = (page_bytes + a.sub_bytes - 1) / a.sub_bytes;
+  a.page_shift = (page_bytes & (page_bytes - 1)) == 0 ? __builtin_ctz(page_bytes) : -1;
+  const uint64_t total = (uint64_t)n_chunks * pages_per_chunk * a.subs_per_page;
+  const uint32_t grid = fl_copy_grid(total);
+  hipStream_t s = (hipStream_t)stream;
+  const bool nt = fl_use_nt(3ull * n_chunks * pages_per_chunk * page_bytes);
+#define FL_LAUNCH_PAGES(D, LD, N) FL_LAUNCH((fl_page_tiles<D, LD, N>), dim3(grid), dim3(kCopyBlock), 0, s, a)
+  if (dir == 0) {
+    if (use_lds) { if (nt) FL_LAUNCH_PAGES(0, true, true); else FL_LAUNCH_PAGES(0, true, false); }
+    else { if (nt) FL_LAUNCH_PAGES(0, false, true); else FL_LAUNCH_PAGES(0, false, false); }
+  } else {
+    if (use_lds) { if (nt) FL_LAUNCH_PAGES(1, true, true); else FL_LAUNCH_PAGES(1, true, false); }
+    else { if (nt) FL_LAUNCH_PAGES(1, false, true); else FL_LAUNCH_PAGES(1, false, false); }
+  }
+#undef FL_LAUNCH_PAGES
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_gather_pages(const void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                     uint32_t pages_per_chunk, const flh_windows* win, const flh_chunk_desc* d_table, uint32_t n_chunks,
+                     int use_lds, int32_t* d_status, void* stream) {
+  return launch_pages(0, (void*)d_pool, pool_pages, d_page_table, page_bytes, pages_per_chunk, win, d_table, n_chunks, use_lds, d_status, stream);
+}
+
+int flh_scatter_pages(void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                      uint32_t pages_per_chunk, const flh_windows* win, const flh_chunk_desc* d_table, uint32_t n_chunks,
+                      int use_lds, int32_t* d_status, void* stream) {
+  return launch_pages(1, d_pool, pool_pages, d_page_table, page_bytes, pages_per_chunk, win, d_table, n_chunks, use_lds, d_status, stream);
+}
+
+int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
+  if (bytes == 0) return FLH_OK;
+  if (!d_dst || !d_src) return fl_set_error(FLH_E_ARG, "null pointer");
+  int rc = fl_need_init();
+  if (rc) return rc;
+  fl_prof().kid = 6;
+  const uint32_t tile = FLH_TILE_BYTES;
+  const uint32_t grid = fl_copy_grid((bytes + tile - 1) / tile);
+  hipStream_t s = (hipStream_t)stream;
+  if (fl_use_nt(2 * bytes)) FL_LAUNCH(fl_plain_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  else FL_LAUNCH(fl_plain_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,112 @@
+// fl_device.h -- device-side primitives shared by the scheduler and the copy kernels: wavefront scans built on
+// DPP row shifts and row broadcasts (64-wide wavefronts), lane broadcasts and shifts, and the division helpers.
+// Everything sits in an unnamed namespace: each translation unit compiles its own copy.
+#ifndef FL_DEVICE_H_
+#define FL_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// ------------------------------------------------------------------------------------------------
+// wavefront scan primitives (DPP)
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int kWave = 64;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// DPP controls of the GFX9 ISA: row_shr:n = 0x110+n, row_bcast:15 = 0x142, row_bcast:31 = 0x143.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+template <int CTRL>
+__device__ __forceinline__ uint64_t dpp_u64(uint64_t v) {
+  uint32_t lo = dpp_u32<CTRL>((uint32_t)v);
+  uint32_t hi = dpp_u32<CTRL>((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// One step of a Hillis-Steele scan: lanes for which `take` holds add the value moved in from below.
+#define FL_SCAN_STEP(T, MOVE, CTRL, COND) \
+  { T t = MOVE<CTRL>(v); if (COND) v += t; }
+
+// inclusive sum over the 64 lanes of a wavefront
+__device__ __forceinline__ uint64_t wave_incl_sum_u64(uint64_t v, int lane) {
+  const int r = lane & 15;
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x111, r >= 1)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x112, r >= 2)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x114, r >= 4)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x118, r >= 8)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x142, (lane & 31) >= 16)
+  FL_SCAN_STEP(uint64_t, dpp_u64, 0x143, lane >= 32)
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_incl_sum_u32(uint32_t v, int lane) {
+  const int r = lane & 15;
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x111, r >= 1)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x112, r >= 2)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x114, r >= 4)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x118, r >= 8)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x142, (lane & 31) >= 16)
+  FL_SCAN_STEP(uint32_t, dpp_u32, 0x143, lane >= 32)
+  return v;
+}
+#undef FL_SCAN_STEP
+
+// Segmented inclusive sum: f marks "a segment starts at or before me inside my own span"; the
+// combine is (f1,v1)+(f2,v2) = (f1|f2, f2 ? v2 : v1+v2) with operand 1 the lower lanes.
+#define FL_SEG_STEP(CTRL, COND)                                   \
+  {                                                               \
+    uint64_t tv = dpp_u64<CTRL>(v);                               \
+    uint32_t tf = dpp_u32<CTRL>(f);                               \
+    if (COND) { if (!f) v += tv; f |= tf; }                       \
+  }
+__device__ __forceinline__ void wave_incl_segsum_u64(uint64_t& v, uint32_t& f, int lane) {
+  const int r = lane & 15;
+  FL_SEG_STEP(0x111, r >= 1)
+  FL_SEG_STEP(0x112, r >= 2)
+  FL_SEG_STEP(0x114, r >= 4)
+  FL_SEG_STEP(0x118, r >= 8)
+  FL_SEG_STEP(0x142, (lane & 31) >= 16)
+  FL_SEG_STEP(0x143, lane >= 32)
+}
+#undef FL_SEG_STEP
+
+__device__ __forceinline__ uint64_t bcast_lane_u64(uint64_t v, int src_lane) {
+  uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, src_lane);
+  uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), src_lane);
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ uint32_t bcast_lane_u32(uint32_t v, int src_lane) {
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, src_lane);
+}
+
+// value of the lane below (lane 0 gets 0): turns an inclusive scan into an exclusive one
+__device__ __forceinline__ uint64_t wave_shift_up_u64(uint64_t v, int lane) {
+  // wave_shr:1 does not exist on every GFX9 part for 64 lanes; go through a bpermute
+  int src = (lane - 1) << 2;
+  uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)(uint32_t)v);
+  uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)(uint32_t)(v >> 32));
+  uint64_t r = ((uint64_t)hi << 32) | lo;
+  return lane == 0 ? 0 : r;
+}
+__device__ __forceinline__ uint32_t wave_shift_up_u32(uint32_t v, int lane) {
+  uint32_t r = (uint32_t)__builtin_amdgcn_ds_bpermute((lane - 1) << 2, (int)v);
+  return lane == 0 ? 0 : r;
+}
+
+// 64-bit division is a long software routine on this ISA and almost every operand here fits 32
+// bits; the wide case is kept out of line so that the kernel stays small enough for the
+// instruction cache (a lone wavefront cannot hide instruction fetch).
+__device__ __attribute__((noinline)) uint64_t div_u64_wide(uint64_t a, uint64_t b) { return a / b; }
+__device__ __forceinline__ uint64_t div_u64(uint64_t a, uint64_t b) {
+  return ((a | b) >> 32) == 0 ? (uint64_t)((uint32_t)a / (uint32_t)b) : div_u64_wide(a, b);
+}
+__device__ __forceinline__ uint64_t mod_u64(uint64_t a, uint64_t b) {
+  return ((a | b) >> 32) == 0 ? (uint64_t)((uint32_t)a % (uint32_t)b) : a - div_u64_wide(a, b) * b;
+}
+
+}  // namespace
+
+#endif  // FL_DEVICE_H_

@@ -1,0 +1,75 @@
+// fl_launch.h -- host-side state and helpers shared by the translation units that launch kernels: the launch
+// tunables, the per-thread profiling ring behind flh_prof_begin / flh_prof_end, and the launch macro.
+#ifndef FL_LAUNCH_H_
+#define FL_LAUNCH_H_
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <vector>
+
+#include "fl_internal.h"
+#include "fuselink_hip.h"
+
+#define FL_LOCAL __attribute__((visibility("hidden")))
+
+// device the library was initialised on and its compute-unit count (-1 / 0 before flh_init)
+extern FL_LOCAL int g_device;
+extern FL_LOCAL int g_cus;
+// launch tunables (flh_tune; some can be preset through NCCL_FUSELINK_* for experiments)
+extern FL_LOCAL int g_grid_per_cu;         // 0: one workgroup per tile (up to 2^20)
+extern FL_LOCAL int g_dest_order;          // fused striping in destination order: -1 = when the working set exceeds the cache, 0 / 1 force
+extern FL_LOCAL int g_fused_fast;          // host-prepared reciprocal for the fused kernels' slot arithmetic (0 = always divide in the kernel)
+extern FL_LOCAL int g_nontemporal;         // -1: streaming accesses only when the buffers cannot all sit in the Infinity Cache
+extern FL_LOCAL int g_sched_variant;       // 0 = pick the scheduler shape from the chunk count
+extern FL_LOCAL int g_sched_uniform_fast;
+extern FL_LOCAL int g_copy_uniform_grid;
+constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // working sets up to this stay largely in the 256 MB Infinity Cache
+
+// Per-launch timing: while a profiling region is open on the calling thread, every kernel is launched
+// with its own start/stop events (hipExtLaunchKernelGGL), which bracket the kernel alone and not the
+// gaps around it.  The events are read back when the region is closed, so the launches themselves
+// stay asynchronous and back to back.
+struct ProfRec { hipEvent_t e0, e1; int kid; };
+struct ProfState {
+  std::vector<ProfRec>* ring = nullptr;
+  size_t n = 0;
+  bool on = false;
+  int kid = 0;   // which entry point is launching: 1 schedule, 2 stripe, 3 reassemble, 4 gather, 5 scatter, 6 copy
+};
+// The calling thread's state.  Reached through a function, not through an `extern thread_local`: code that uses
+// such a variable from another translation unit tests the address of its (absent, weak, hidden) initialiser,
+// which position-independent code computes relative to the load address, never as null, and then calls it.
+FL_LOCAL ProfState& fl_prof();
+
+#define FL_LAUNCH(kernel, grid, block, shmem, stream, ...)                                              \
+  do {                                                                                                  \
+    ProfState& ps_ = fl_prof();                                                                         \
+    if (ps_.on && ps_.n < ps_.ring->size()) {                                                           \
+      ProfRec& pr_ = (*ps_.ring)[ps_.n++];                                                              \
+      pr_.kid = ps_.kid;                                                                                \
+      hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, pr_.e0, pr_.e1, 0, __VA_ARGS__);        \
+    } else {                                                                                            \
+      hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                              \
+    }                                                                                                   \
+  } while (0)
+
+#define FL_HIP(call)                                                                         \
+  do {                                                                                       \
+    hipError_t e_ = (call);                                                                  \
+    if (e_ != hipSuccess)                                                                    \
+      return fl_set_error(e_ == hipErrorNoDevice ? FLH_E_NODEV : FLH_E_HIP, "%s failed: %s (%s:%d)", #call, \
+                          hipGetErrorString(e_), __FILE__, __LINE__);                        \
+  } while (0)
+
+// flh_init on NCCL_FUSELINK_DEVICE (default 0) if no entry point has initialised the library yet
+FL_LOCAL int fl_need_init();
+// Non-temporal loads and stores pay off once the working set (the buffers a transfer touches) is well
+// beyond the 256 MB Infinity Cache (measured: +3-5 % at 1 GiB messages) and cost throughput when a
+// good part of it still fits (-8 % at 64 MiB, -20 % on the read-back side at 128 MiB).
+FL_LOCAL bool fl_use_nt(uint64_t working_set_bytes);
+// workgroups for a copy over max_tiles tiles: one per tile (the dispatcher then overlaps loads and stores of
+// different tiles); the kernels' stride loops only matter beyond the cap, which grid_per_cu can lower
+FL_LOCAL uint32_t fl_copy_grid(uint64_t max_tiles);
+
+#endif  // FL_LAUNCH_H_

@@ -1,0 +1,165 @@
+// fl_runtime.cc -- library state and the entry points that launch nothing: initialisation, the last error
+// message, launch tunables, per-launch profiling, and the request -> QP split (host arithmetic).
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "fl_launch.h"
+
+namespace {
+thread_local char g_err[512] = "";
+
+int64_t env_i64(const char* name, int64_t dflt) {
+  const char* v = getenv(name);
+  if (!v || !*v) return dflt;
+  char* end = nullptr;
+  long long x = strtoll(v, &end, 0);
+  return end && *end == 0 ? x : dflt;
+}
+}  // namespace
+
+int g_device = -1;
+int g_cus = 0;
+int g_grid_per_cu = 0;
+int g_dest_order = -1;
+int g_fused_fast = 1;
+int g_nontemporal = -1;
+int g_sched_variant = 0;
+int g_sched_uniform_fast = 1;
+int g_copy_uniform_grid = 1;
+
+namespace {
+thread_local ProfState t_prof;
+}
+ProfState& fl_prof() { return t_prof; }
+
+int fl_set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int fl_need_init() {
+  if (g_device < 0) {
+    int rc = flh_init((int)env_i64("NCCL_FUSELINK_DEVICE", 0));
+    if (rc) return rc;
+  }
+  return FLH_OK;
+}
+
+bool fl_use_nt(uint64_t working_set_bytes) {
+  if (g_nontemporal >= 0) return g_nontemporal != 0;
+  return working_set_bytes > kCacheResidentBytes;
+}
+
+uint32_t fl_copy_grid(uint64_t max_tiles) {
+  uint64_t g = g_grid_per_cu > 0 ? (uint64_t)g_cus * (uint64_t)g_grid_per_cu : (1ull << 20);
+  if (g > max_tiles) g = max_tiles;
+  if (g < 1) g = 1;
+  return (uint32_t)g;
+}
+
+extern "C" {
+
+const char* flh_last_error(void) { return g_err; }
+
+int64_t flh_constant(int which) {
+  switch (which) {
+    case 0: return FLH_TILE_BYTES;
+    case 1: return FLH_MAX_LANES;
+    case 2: return FLH_UNIT_BYTES;
+    case 3: return FLH_POOL_UNITS;
+    case 4: return sizeof(flh_chunk_desc);
+    case 5: return sizeof(flh_sched_state);
+    case 6: return sizeof(flh_sched_hdr);
+    case 7: return 1;
+    case 8: return sizeof(flh_windows);
+    case 9: return sizeof(flh_sched_params);
+  }
+  return -1;
+}
+
+int flh_init(int device) {
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count == 0)
+    return fl_set_error(FLH_E_NODEV, "no HIP device: %s", e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+  if (device < 0 || device >= count) return fl_set_error(FLH_E_ARG, "device %d out of range (%d devices)", device, count);
+  FL_HIP(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  FL_HIP(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fl_set_error(FLH_E_NODEV, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+  g_device = device;
+  g_cus = prop.multiProcessorCount;
+  g_grid_per_cu = (int)env_i64("NCCL_FUSELINK_GRID_PER_CU", g_grid_per_cu);
+  g_nontemporal = (int)env_i64("NCCL_FUSELINK_NONTEMPORAL", g_nontemporal);
+  if (g_grid_per_cu < 0) g_grid_per_cu = 0;
+  return FLH_OK;
+}
+
+int flh_prof_begin(int capacity) {
+  if (capacity < 1 || capacity > (1 << 20)) return fl_set_error(FLH_E_ARG, "capacity %d out of range", capacity);
+  if (!t_prof.ring) t_prof.ring = new std::vector<ProfRec>();
+  while (t_prof.ring->size() < (size_t)capacity) {
+    ProfRec r;
+    r.kid = 0;
+    FL_HIP(hipEventCreate(&r.e0));
+    FL_HIP(hipEventCreate(&r.e1));
+    t_prof.ring->push_back(r);
+  }
+  t_prof.n = 0;
+  t_prof.on = true;
+  return FLH_OK;
+}
+
+int flh_prof_end(double* us_out, int* kernel_out, int max) {
+  t_prof.on = false;
+  if (!t_prof.ring) return fl_set_error(FLH_E_STATE, "no profiling region was opened on this thread");
+  const size_t n = t_prof.n;
+  for (size_t i = 0; i < n; ++i) {
+    ProfRec& r = (*t_prof.ring)[i];
+    FL_HIP(hipEventSynchronize(r.e1));
+    float ms = 0.f;
+    FL_HIP(hipEventElapsedTime(&ms, r.e0, r.e1));
+    if ((int)i < max) {
+      if (us_out) us_out[i] = (double)ms * 1e3;
+      if (kernel_out) kernel_out[i] = r.kid;
+    }
+  }
+  t_prof.n = 0;
+  return (int)n;
+}
+
+int flh_tune(const char* key, int64_t value) {
+  if (!key) return fl_set_error(FLH_E_ARG, "null key");
+  if (!strcmp(key, "grid_per_cu")) { if (value < 0) return fl_set_error(FLH_E_ARG, "grid_per_cu < 0"); g_grid_per_cu = (int)value; return FLH_OK; }
+  if (!strcmp(key, "stripe_dest_order")) { g_dest_order = value < 0 ? -1 : (value != 0); return FLH_OK; }
+  if (!strcmp(key, "fused_fast")) { g_fused_fast = value != 0; return FLH_OK; }
+  if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
+  if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
+  if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
+  if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 4) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..4"); g_sched_variant = (int)value; return FLH_OK; }
+  return fl_set_error(FLH_E_ARG, "unknown tunable %s", key);
+}
+
+int flh_qp_split(int size, int nqps, int* off, int* len) {
+  if (nqps < 1 || size < 0 || !off || !len) return fl_set_error(FLH_E_ARG, "bad qp split arguments");
+  // stride = ceil(ceil(size / nqps) / 128) * 128; a piece past the end is an empty work request.
+  // 64-bit inside: the reference's `int` expression overflows for sizes within 127 bytes of INT_MAX.
+  const int64_t per = ((int64_t)size + nqps - 1) / nqps;
+  const int64_t stride = (per + 127) / 128 * 128;
+  int64_t o = 0;
+  for (int q = 0; q < nqps; ++q, o += stride) {
+    int64_t l = (int64_t)size - o;
+    if (l > stride) l = stride;
+    off[q] = o > 0x7fffffff ? 0x7fffffff : (int)o;
+    len[q] = l > 0 ? (int)l : 0;
+  }
+  return stride > 0x7fffff80 ? 0x7fffff80 : (int)stride;
+}
+
+}  // extern "C"

@@ -1,0 +1,677 @@
+// fl_sched.hip -- the chunk -> (lane, window offset) scheduler kernels and flh_schedule:
+//   * fl_schedule_kernel         : any chunk sizes; one workgroup, wavefront prefix scans (DPP)
+//   * fl_schedule_uniform_kernel : uniform split with quantum-sized chunks; closed form, any number of workgroups
+// All cross-lane traffic is DPP row shifts and row broadcasts; LDS only passes per-wavefront totals between the
+// wavefronts of the one workgroup and caches the credit rows.
+#include <cstring>
+
+#include "fl_device.h"
+#include "fl_launch.h"
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+// scheduler
+// ------------------------------------------------------------------------------------------------
+constexpr int kRowCache = 32;      // credit rows kept in LDS
+
+struct SchedArgs {
+  const uint32_t* sizes;
+  uint64_t total_bytes;
+  const uint64_t* src_off;
+  uint64_t src_base;
+  const uint32_t* credits;
+  uint64_t quantum;
+  flh_sched_state* state;
+  flh_chunk_desc* table;
+  flh_sched_hdr* hdr;
+  uint32_t chunk_bytes;
+  uint32_t n;
+  uint32_t n_lanes;
+  uint32_t n_rows;
+  uint32_t epoch_len;
+  uint32_t tile_bytes;
+  uint32_t mode;
+  int32_t quantum_shift;  // >= 0 when quantum is a power of two
+  int32_t tile_shift;     // >= 0 when tile_bytes is a power of two
+  uint32_t inline_credits[FLH_MAX_LANES];  // the one credit row when credits == nullptr
+  flh_chunk_desc* table_by_lane;           // optional second copy of the rows in destination order (uniform kernel only)
+};
+
+
+// Credit rows -> inclusive prefixes, four rows per wavefront: a row of at most 16 lanes fills one
+// 16-lane DPP row, so four row_shr steps scan it and rows never mix.  `raw` holds the rows in LDS.
+// A row without any credit (every lane busy) is replaced by equal credits -- the round robin of the
+// static policy -- and marked in zero[].
+template <int BT>
+__device__ __forceinline__ void credit_row_prefixes(const uint32_t* raw, uint32_t R, uint32_t L, int tid,
+                                                    uint64_t (*pfx)[FLH_MAX_LANES], uint32_t* zero) {
+  const int lane = tid & (kWave - 1);
+  const uint32_t sub = (uint32_t)lane & 15u;
+#pragma unroll 1
+  for (uint32_t r0 = 0; r0 < R; r0 += BT / 16) {
+    const uint32_t r = r0 + (uint32_t)tid / 16u;
+    const bool live = r < R && sub < L;
+    uint64_t v = live ? raw[r * L + sub] : 0u;
+    { uint64_t t = dpp_u64<0x111>(v); if (sub >= 1) v += t; }
+    { uint64_t t = dpp_u64<0x112>(v); if (sub >= 2) v += t; }
+    { uint64_t t = dpp_u64<0x114>(v); if (sub >= 4) v += t; }
+    { uint64_t t = dpp_u64<0x118>(v); if (sub >= 8) v += t; }
+    const int top = (lane | 15) << 2;
+    const uint32_t wlo = (uint32_t)__builtin_amdgcn_ds_bpermute(top, (int)(uint32_t)v);
+    const uint32_t whi = (uint32_t)__builtin_amdgcn_ds_bpermute(top, (int)(uint32_t)(v >> 32));
+    const bool none = (wlo | whi) == 0;
+    if (none) v = sub + 1;
+    if (live) pfx[r][sub] = v;
+    if (r < R && sub == 0) zero[r] = none;
+  }
+}
+
+template <typename T> __device__ __forceinline__ T wave_incl_sum(T v, int lane);
+template <> __device__ __forceinline__ uint32_t wave_incl_sum<uint32_t>(uint32_t v, int lane) { return wave_incl_sum_u32(v, lane); }
+template <> __device__ __forceinline__ uint64_t wave_incl_sum<uint64_t>(uint64_t v, int lane) { return wave_incl_sum_u64(v, lane); }
+
+// In-wavefront part of the window offsets: for every lane l, scan the threads' bytes on l and hand
+// each chunk on l its exclusive position.  Four lanes go through the scan side by side so that their
+// DPP chains overlap (a lone wavefront per SIMD has nothing else to hide that latency with).  The
+// wavefront's total of lane l is parked in thread l and goes to LDS once at the end.
+// T is the width of the partial sums (32 bits when the whole pass moves less than 4 GiB).
+template <typename T, int K>
+__device__ __forceinline__ void lane_pass(const uint32_t (&s)[K], const uint32_t (&ln)[K], uint32_t L, int lane,
+                                          uint64_t* w_lane_row, uint64_t (&off)[K]) {
+  constexpr int G = 4;
+  uint64_t my_total = 0;
+#pragma unroll 1
+  for (uint32_t l0 = 0; l0 < L; l0 += G) {
+    T v[G], inc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      v[g] = 0;
+#pragma unroll
+      for (int k = 0; k < K; ++k) v[g] += ln[k] == l0 + g ? (T)s[k] : (T)0;
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) inc[g] = wave_incl_sum<T>(v[g], lane);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      uint64_t ex = (uint64_t)(inc[g] - v[g]);
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        if (ln[k] == l0 + g) { off[k] = ex; ex += s[k]; }
+      }
+      const uint64_t tot = sizeof(T) == 8 ? bcast_lane_u64((uint64_t)inc[g], kWave - 1) : (uint64_t)bcast_lane_u32((uint32_t)inc[g], kWave - 1);
+      if ((uint32_t)lane == l0 + g) my_total = tot;
+    }
+  }
+  if ((uint32_t)lane < L) w_lane_row[lane] = my_total;
+}
+
+// One workgroup of NW wavefronts walks the chunk list in passes of NW*64*K chunks; thread t owns K
+// consecutive chunks of a pass.  Per pass: thread-local sums, three wavefront scans (epoch-segmented
+// bytes, bytes, tiles), the lane of each chunk from its quantum slot, one wavefront scan per lane
+// for the window offsets.  LDS only carries per-wavefront totals and the running lane offsets.
+template <int NW, int K>
+__global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
+  constexpr int BT = NW * kWave;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const uint32_t L = a.n_lanes;
+
+  // credit rows as inclusive prefixes; row r occupies rowpfx[r][0..L), W = rowpfx[r][L-1]
+  __shared__ uint64_t rowpfx[kRowCache][FLH_MAX_LANES];
+  __shared__ uint32_t rowzero[kRowCache];  // the row had no credit at all
+  // the same prefixes in 32 bits, entries past L-1 saturated, for rows whose credits sum below 2^32
+  __shared__ __attribute__((aligned(16))) uint32_t rowpfx32[kRowCache][FLH_MAX_LANES];
+  __shared__ uint32_t rows_wide;  // some row sums to 2^32 or more: use the 64-bit prefixes
+  __shared__ uint64_t w_seg_v[NW];
+  __shared__ uint32_t w_seg_f[NW];
+  __shared__ uint64_t w_run[NW];
+  __shared__ uint32_t w_tiles[NW];
+  __shared__ uint64_t w_lane[NW][FLH_MAX_LANES];  // per-wavefront lane totals, then absolute bases
+  __shared__ uint64_t lane_off[FLH_MAX_LANES];    // next free byte of every window
+  __shared__ uint64_t lane_off0[FLH_MAX_LANES];
+  __shared__ uint32_t cnt_lane[FLH_MAX_LANES];
+  __shared__ uint32_t sh_flags;
+
+  // One wavefront per row: lanes 0..L-1 load the row in a single access, a scan forms the prefixes.
+  // A row without any credit (every lane busy) is replaced by equal credits -- the round-robin of
+  // the static policy -- and flagged.
+  const bool rows_cached = a.n_rows <= (uint32_t)kRowCache;
+  uint32_t flags = 0;
+  __shared__ uint32_t raw[kRowCache * FLH_MAX_LANES];
+  if (rows_cached) {
+    // all credit rows in one round trip to memory, then one wavefront scan per row out of LDS
+    for (uint32_t e = tid; e < a.n_rows * L; e += BT) raw[e] = a.credits ? a.credits[e] : a.inline_credits[e];
+  }
+  // the carried state and the first pass's sizes are requested before anything waits on the credit rows,
+  // so that the kernel pays one round trip to memory, not three in a row
+  uint64_t k0 = 0, p_carry = 0, run_carry = 0;  // carried state, identical in every thread
+  uint32_t tiles_carry = 0;
+  if (a.state) {
+    k0 = a.state->chunk_index;
+    if (!(a.mode & FLH_SCHED_NEW_EPOCH)) p_carry = a.state->epoch_bytes;
+  }
+  uint64_t off_in = 0;
+  if (tid < FLH_MAX_LANES && a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS)) off_in = a.state->lane_off[tid];
+  uint32_t s_next[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const uint32_t i = (uint32_t)tid * K + k;
+    s_next[k] = (a.sizes && i < a.n) ? a.sizes[i] : 0;
+  }
+  if (rows_cached) {
+    __syncthreads();
+    credit_row_prefixes<BT>(raw, a.n_rows, L, tid, rowpfx, rowzero);
+    if (tid == 0) rows_wide = 0;
+    __syncthreads();
+    for (uint32_t e = tid; e < a.n_rows * FLH_MAX_LANES; e += BT) {
+      const uint32_t r = e / FLH_MAX_LANES, l = e % FLH_MAX_LANES;
+      const uint64_t v = l + 1 < L ? rowpfx[r][l] : ~0ull;  // the last prefix is W > slot: never counted
+      rowpfx32[r][l] = v >> 32 ? 0xffffffffu : (uint32_t)v;
+      if (l == L - 1 && (rowpfx[r][l] >> 32)) rows_wide = 1;
+    }
+  }
+  if (tid < FLH_MAX_LANES) {
+    const uint64_t o = off_in;
+    lane_off[tid] = o;
+    lane_off0[tid] = o;
+    cnt_lane[tid] = 0;
+  }
+  if (tid == 0) sh_flags = 0;
+  __syncthreads();
+
+  const bool wide = rows_cached && rows_wide != 0;
+#pragma unroll 1
+  for (uint32_t pass = 0; pass < a.n; pass += BT * K) {
+    const uint32_t i0 = pass + (uint32_t)tid * K;
+    uint32_t s[K], tl[K], row[K], ep[K], ln[K];
+    bool head[K];
+    // ---- epoch, position in epoch and credit row of my first chunk; the rest follow by counting ----
+    uint64_t e_cur = 0;
+    uint32_t pos = 0, r_cur = 0;
+    if (a.epoch_len) {
+      const uint64_t g0 = k0 + i0;
+      e_cur = div_u64(g0, a.epoch_len);
+      pos = (uint32_t)(g0 - e_cur * a.epoch_len);
+      r_cur = (uint32_t)mod_u64(e_cur, a.n_rows);
+    }
+    // ---- load sizes, mark epoch heads, thread-local aggregates -----------------------------------
+    uint64_t seg_v = 0;
+    uint32_t seg_f = 0;
+    uint64_t run = 0;
+    uint32_t tiles = 0;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const uint32_t i = i0 + k;
+      uint32_t sz = 0;
+      bool hd = false;
+      if (i < a.n) {
+        if (a.sizes) {
+          sz = s_next[k];
+        } else {
+          const uint64_t o = (uint64_t)i * a.chunk_bytes;
+          const uint64_t rem = o < a.total_bytes ? a.total_bytes - o : 0;
+          sz = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
+        }
+        hd = a.epoch_len && pos == 0;
+      }
+      s[k] = sz;
+      head[k] = hd;
+      row[k] = r_cur;
+      ep[k] = (uint32_t)e_cur;
+      tl[k] = a.tile_shift >= 0 ? (sz + a.tile_bytes - 1) >> a.tile_shift : (sz + a.tile_bytes - 1) / a.tile_bytes;
+      if (hd) { seg_v = 0; seg_f = 1; }
+      seg_v += sz;
+      run += sz;
+      tiles += tl[k];
+      if (a.epoch_len && ++pos == a.epoch_len) {
+        pos = 0;
+        ++e_cur;
+        if (++r_cur == a.n_rows) r_cur = 0;
+      }
+    }
+    if (a.sizes) {  // next pass's sizes travel while this pass computes
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const uint64_t i = (uint64_t)i0 + (uint64_t)BT * K + k;
+        s_next[k] = i < a.n ? a.sizes[i] : 0;
+      }
+    }
+    // ---- block-wide exclusive prefixes of (segmented bytes, bytes, tiles) --------------------------
+    uint64_t sv = seg_v;
+    uint32_t sf = seg_f;
+    wave_incl_segsum_u64(sv, sf, lane);
+    const uint64_t run_incl = wave_incl_sum_u64(run, lane);
+    const uint32_t tiles_incl = wave_incl_sum_u32(tiles, lane);
+    uint64_t seg_ex_v = wave_shift_up_u64(sv, lane);
+    uint32_t seg_ex_f = wave_shift_up_u32(sf, lane);
+    uint64_t run_ex = run_incl - run;
+    uint32_t tiles_ex = tiles_incl - tiles;
+    if (lane == kWave - 1) { w_seg_v[wave] = sv; w_seg_f[wave] = sf; w_run[wave] = run_incl; w_tiles[wave] = tiles_incl; }
+    __syncthreads();
+    uint64_t tot_seg_v = 0, tot_run = 0;
+    uint32_t tot_seg_f = 0, tot_tiles = 0;
+    {
+      uint64_t pv = 0, pr = 0;
+      uint32_t pf = 0, pt = 0;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        if (w == wave) { pv = tot_seg_v; pf = tot_seg_f; pr = tot_run; pt = tot_tiles; }
+        const uint64_t wv = w_seg_v[w];
+        const uint32_t wf = w_seg_f[w];
+        tot_seg_v = wf ? wv : tot_seg_v + wv;
+        tot_seg_f |= wf;
+        tot_run += w_run[w];
+        tot_tiles += w_tiles[w];
+      }
+      // combine the earlier wavefronts' aggregate with my in-wavefront exclusive value
+      if (!seg_ex_f) seg_ex_v += pv;
+      seg_ex_f |= pf;
+      run_ex += pr;
+      tiles_ex += pt;
+    }
+    // bytes of my epoch before my first chunk
+    uint64_t P = seg_ex_f ? seg_ex_v : p_carry + seg_ex_v;
+
+    // ---- lane of each chunk ------------------------------------------------------------------------------
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const uint32_t i = i0 + k;
+      ln[k] = FLH_MAX_LANES;  // matches no lane: chunks past the end count nowhere
+      if (i < a.n) {
+        if (head[k]) P = 0;
+        const uint32_t r = row[k];
+        uint64_t W;
+        bool equal = false;  // no lane has credit: equal credits stand in
+        if (rows_cached) {
+          W = rowpfx[r][L - 1];
+          if (rowzero[r]) flags |= FLH_SCHED_F_NO_CREDIT;
+        } else {
+          W = 0;
+#pragma unroll 1
+          for (uint32_t l = 0; l < L; ++l) W += a.credits[(size_t)r * L + l];
+          if (W == 0) { W = L; equal = true; flags |= FLH_SCHED_F_NO_CREDIT; }
+        }
+        const uint64_t qn = a.quantum_shift >= 0 ? (P >> a.quantum_shift) : div_u64(P, a.quantum);
+        const uint64_t slot = mod_u64(qn, W);
+        // lane = number of inclusive prefixes <= slot (zero-credit lanes repeat the prefix and are skipped)
+        uint32_t pick = 0;
+        if (rows_cached && !wide) {
+          const uint32_t slot32 = (uint32_t)slot;  // slot < W < 2^32
+          const u32x4* pr = reinterpret_cast<const u32x4*>(rowpfx32[r]);
+          const u32x4 p0 = pr[0], p1 = pr[1], p2 = pr[2], p3 = pr[3];
+          pick = (p0.x <= slot32) + (p0.y <= slot32) + (p0.z <= slot32) + (p0.w <= slot32) + (p1.x <= slot32) + (p1.y <= slot32) +
+                 (p1.z <= slot32) + (p1.w <= slot32) + (p2.x <= slot32) + (p2.y <= slot32) + (p2.z <= slot32) + (p2.w <= slot32) +
+                 (p3.x <= slot32) + (p3.y <= slot32) + (p3.z <= slot32) + (p3.w <= slot32);
+        } else if (rows_cached) {
+#pragma unroll 1
+          for (uint32_t l = 0; l + 1 < L; ++l) pick += rowpfx[r][l] <= slot;
+        } else if (equal) {
+          pick = (uint32_t)slot;
+        } else {
+          uint64_t kk = 0;
+#pragma unroll 1
+          for (uint32_t l = 0; l + 1 < L; ++l) { kk += a.credits[(size_t)r * L + l]; pick += kk <= slot; }
+        }
+        ln[k] = pick;
+        atomicAdd(&cnt_lane[pick], 1u);  // LDS counter of chunks per lane
+        P += s[k];
+      }
+    }
+    // ---- window offsets: in-wavefront scans per lane, then wavefront bases through LDS -----------------
+    uint64_t off[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) off[k] = 0;
+    if ((tot_run >> 32) == 0) lane_pass<uint32_t, K>(s, ln, L, lane, w_lane[wave], off);
+    else lane_pass<uint64_t, K>(s, ln, L, lane, w_lane[wave], off);
+    __syncthreads();
+    if ((uint32_t)tid < L) {
+      uint64_t at = lane_off[tid];
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const uint64_t x = w_lane[w][tid];
+        w_lane[w][tid] = at;
+        at += x;
+      }
+      lane_off[tid] = at;
+    }
+    __syncthreads();
+    // ---- emit rows ---------------------------------------------------------------------------------------
+    uint64_t run_i = run_carry + run_ex;
+    uint32_t tiles_i = tiles_carry + tiles_ex;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const uint32_t i = i0 + k;
+      if (i < a.n) {
+        flh_chunk_desc d;
+        d.src_off = a.src_off ? a.src_off[i] : a.src_base + run_i;
+        d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : w_lane[wave][ln[k]] + off[k];
+        d.len = s[k];
+        d.lane = ln[k];
+        d.tile_base = tiles_i;
+        d.epoch = ep[k];
+        a.table[i] = d;
+        run_i += s[k];
+        tiles_i += tl[k];
+      }
+    }
+    // ---- carries -------------------------------------------------------------------------------------------
+    p_carry = tot_seg_f ? tot_seg_v : p_carry + tot_seg_v;
+    run_carry += tot_run;
+    tiles_carry += tot_tiles;
+  }
+
+  // ---- header and state --------------------------------------------------------------------------------------
+  if (__builtin_amdgcn_ballot_w64(flags != 0) && lane == 0) atomicOr(&sh_flags, FLH_SCHED_F_NO_CREDIT);
+  __syncthreads();
+  if (tid < FLH_MAX_LANES) {
+    a.hdr->lane_bytes[tid] = lane_off[tid] - lane_off0[tid];
+    a.hdr->lane_chunks[tid] = cnt_lane[tid];
+    if (a.state) a.state->lane_off[tid] = lane_off[tid];
+  }
+  if (tid == 0) {
+    a.hdr->total_bytes = run_carry;
+    a.hdr->total_tiles = tiles_carry;
+    a.hdr->n_chunks = a.n;
+    a.hdr->flags = sh_flags;
+    a.hdr->uniform_tiles = (!a.sizes && a.n) ? (a.chunk_bytes + a.tile_bytes - 1) / a.tile_bytes : 0;
+    if (a.state) {
+      a.state->epoch_bytes = p_carry;
+      a.state->chunk_index = k0 + a.n;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// scheduler, uniform split
+// ------------------------------------------------------------------------------------------------
+// When every chunk has the quantum's size (the ordinary message split: sizes == nullptr and
+// quantum == chunk_bytes; only the last chunk may be short) the byte prefix of chunk j of an epoch
+// is j quanta, so its slot is j mod W and nothing has to be scanned: the number of earlier chunks
+// on a lane is a closed form in j,
+//     cnt(row, l, x) = #{ y < x : slot y belongs to lane l } = (x / W) * c_l + clamp(x mod W - K_l, 0, c_l),
+// whole epochs contribute cnt(row, l, E), and because rows repeat with period R those contributions
+// sum in closed form too.  Every chunk is independent, so the table is filled by as many workgroups
+// as it takes; the results are identical to the scan kernel's.
+struct UniTables {
+  uint64_t pfx[kRowCache][FLH_MAX_LANES];   // inclusive credit prefixes (equal credits for an empty row)
+  uint64_t pf[kRowCache + 1][FLH_MAX_LANES];  // pf[r][l] = chunks on lane l in whole epochs of rows < r; pf[R] = one period
+  uint32_t zero[kRowCache];
+};
+
+__device__ __forceinline__ uint64_t uni_cnt(const UniTables& t, uint32_t r, uint32_t l, uint32_t L, uint64_t x) {
+  const uint64_t W = t.pfx[r][L - 1];
+  const uint64_t hi = t.pfx[r][l];
+  const uint64_t K = l ? t.pfx[r][l - 1] : 0;
+  const uint64_t c = hi - K;
+  const uint64_t full = div_u64(x, W);
+  const uint64_t rem = x - full * W;
+  const uint64_t part = rem <= K ? 0 : (rem - K < c ? rem - K : c);
+  return full * c + part;
+}
+
+__device__ __forceinline__ uint32_t uni_lane(const UniTables& t, uint32_t r, uint32_t L, uint64_t j) {
+  const uint64_t slot = mod_u64(j, t.pfx[r][L - 1]);
+  uint32_t pick = 0;
+#pragma unroll 1
+  for (uint32_t l = 0; l + 1 < L; ++l) pick += t.pfx[r][l] <= slot;
+  return pick;
+}
+
+struct UniCtx {
+  uint64_t k0, a0, e0, C;
+  uint32_t pos0, E, R, L;
+};
+
+// chunks of this call, before local index i (0 <= i <= n), that sit on lane l; also returns the lane
+// of chunk i itself through *lane_of_i when asked (l == 0xffffffff means "use chunk i's own lane")
+__device__ __forceinline__ uint64_t uni_before(const UniTables& t, const UniCtx& c, uint64_t i, uint32_t l, uint32_t* lane_of_i,
+                                               uint64_t* epoch_of_i) {
+  if (c.E == 0) {
+    const uint64_t j = c.a0 + i;
+    if (lane_of_i) { *lane_of_i = uni_lane(t, 0, c.L, j); if (l == 0xffffffffu) l = *lane_of_i; }
+    if (epoch_of_i) *epoch_of_i = 0;
+    return uni_cnt(t, 0, l, c.L, j) - uni_cnt(t, 0, l, c.L, c.a0);
+  }
+  const uint64_t g = c.k0 + i;
+  const uint64_t e = div_u64(g, c.E);
+  const uint64_t pos = g - e * c.E;
+  const uint32_t r = (uint32_t)mod_u64(e, c.R);
+  if (epoch_of_i) *epoch_of_i = e;
+  if (e == c.e0) {
+    const uint64_t j = c.a0 + (pos - c.pos0);
+    if (lane_of_i) { *lane_of_i = uni_lane(t, r, c.L, j); if (l == 0xffffffffu) l = *lane_of_i; }
+    return uni_cnt(t, r, l, c.L, j) - uni_cnt(t, r, l, c.L, c.a0);
+  }
+  if (lane_of_i) { *lane_of_i = uni_lane(t, r, c.L, pos); if (l == 0xffffffffu) l = *lane_of_i; }
+  const uint32_t r0 = (uint32_t)mod_u64(c.e0, c.R);
+  const uint64_t m0 = c.E - c.pos0;  // chunks of this call in its first epoch
+  uint64_t before = uni_cnt(t, r0, l, c.L, c.a0 + m0) - uni_cnt(t, r0, l, c.L, c.a0);
+  // whole epochs e0+1 .. e-1: G(e) - G(e0+1), G(z) = (z / R) * period + pf[z mod R]
+  const uint64_t z1 = e, z0 = c.e0 + 1;
+  const uint64_t q1 = div_u64(z1, c.R), q0 = div_u64(z0, c.R);
+  before += q1 * t.pf[c.R][l] + t.pf[z1 - q1 * c.R][l];
+  before -= q0 * t.pf[c.R][l] + t.pf[z0 - q0 * c.R][l];
+  before += uni_cnt(t, r, l, c.L, pos);
+  return before;
+}
+
+constexpr int kUniBlock = 256;
+
+// MODE 0: fill the table; the last workgroup also writes the header and, if the grid is a single
+//         workgroup, the state (in place: every read of the old state precedes the barrier).
+// MODE 1: write the state only (second launch after a multi-workgroup MODE 0, so that no workgroup
+//         can still be reading the old state).
+template <int MODE>
+__global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArgs a) {
+  __shared__ UniTables t;
+  const int tid = threadIdx.x;
+  const uint32_t L = a.n_lanes, R = a.n_rows;
+  // all credit rows in one round trip to memory, then one wavefront scan per row out of LDS
+  __shared__ uint32_t raw[kRowCache * FLH_MAX_LANES];
+  for (uint32_t e = tid; e < R * L; e += kUniBlock) raw[e] = a.credits ? a.credits[e] : a.inline_credits[e];
+  // the carried state is requested before anything waits on the credit rows
+  const uint64_t k0_in = a.state ? a.state->chunk_index : 0;
+  const uint64_t p0 = (a.state && !(a.mode & FLH_SCHED_NEW_EPOCH)) ? a.state->epoch_bytes : 0;
+  __syncthreads();
+  credit_row_prefixes<kUniBlock>(raw, R, L, tid, t.pfx, t.zero);
+  __syncthreads();
+  // chunks per lane of one whole epoch under each row (all rows at once), then prefixed over the rows
+  for (uint32_t e = tid; e < R * L; e += kUniBlock) {
+    const uint32_t r = e / L, l = e - r * L;
+    t.pf[r + 1][l] = a.epoch_len ? uni_cnt(t, r, l, L, a.epoch_len) : 0;
+  }
+  __syncthreads();
+  if ((uint32_t)tid < L) {
+    uint64_t run = 0;
+#pragma unroll 1
+    for (uint32_t r = 0; r < R; ++r) {
+      const uint64_t x = t.pf[r + 1][tid];
+      t.pf[r][tid] = run;
+      run += x;
+    }
+    t.pf[R][tid] = run;
+  }
+  __syncthreads();
+
+  UniCtx c;
+  c.C = a.chunk_bytes;
+  c.E = a.epoch_len;
+  c.R = R;
+  c.L = L;
+  c.k0 = k0_in;
+  c.e0 = c.E ? div_u64(c.k0, c.E) : 0;
+  c.pos0 = c.E ? (uint32_t)(c.k0 - c.e0 * c.E) : 0;
+  // quanta already behind the first chunk inside its epoch; an epoch head starts from zero
+  c.a0 = (c.E && c.pos0 == 0) ? 0 : div_u64(p0, c.C);
+  const bool keep_off = a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS);
+  const uint32_t tpc = a.tile_shift >= 0 ? (a.chunk_bytes + a.tile_bytes - 1) >> a.tile_shift : (a.chunk_bytes + a.tile_bytes - 1) / a.tile_bytes;
+
+  // Destination order: rows grouped by lane, the last chunk's lane last (so that a short final chunk stays the
+  // final row).  Every workgroup works out where each lane's group starts from the per-lane chunk totals.
+  __shared__ uint64_t lane_first[FLH_MAX_LANES];
+  __shared__ uint32_t sh_lane_last;
+  if (MODE == 0 && a.table_by_lane) {
+    if ((uint32_t)tid < L) lane_first[tid] = uni_before(t, c, a.n, (uint32_t)tid, nullptr, nullptr);
+    if (tid == kWave) {  // another wavefront than the one busy with the totals
+      uint32_t ll;
+      (void)uni_before(t, c, a.n - 1, 0xffffffffu, &ll, nullptr);
+      sh_lane_last = ll;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint64_t run = 0;
+      uint32_t l = sh_lane_last;
+#pragma unroll 1
+      for (uint32_t k = 0; k < L; ++k) {
+        l = l + 1 == L ? 0 : l + 1;
+        const uint64_t x = lane_first[l];
+        lane_first[l] = run;
+        run += x;
+      }
+    }
+    __syncthreads();
+  }
+
+  if (MODE == 0) {
+    const uint32_t i = blockIdx.x * kUniBlock + tid;
+    if (i < a.n) {
+      uint32_t ln;
+      uint64_t ep;
+      const uint64_t before = uni_before(t, c, i, 0xffffffffu, &ln, &ep);
+      const uint64_t o = (uint64_t)i * c.C;
+      const uint64_t rem = a.total_bytes - o;
+      flh_chunk_desc d;
+      d.src_off = a.src_base + o;
+      d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : (keep_off ? a.state->lane_off[ln] : 0) + before * c.C;
+      d.len = (uint32_t)(rem < c.C ? rem : c.C);
+      d.lane = ln;
+      d.tile_base = i * tpc;
+      d.epoch = (uint32_t)ep;
+      a.table[i] = d;
+      if (a.table_by_lane) {
+        const uint64_t pos = lane_first[ln] + before;
+        d.tile_base = (uint32_t)pos * tpc;
+        a.table_by_lane[pos] = d;
+      }
+    }
+    if (blockIdx.x != gridDim.x - 1) return;
+  }
+  const bool write_hdr = MODE == 0;
+  const bool write_state = a.state && (MODE == 1 || gridDim.x == 1);
+  const uint64_t last = a.n - 1;
+  const uint64_t len_last = a.total_bytes - last * c.C;
+  uint32_t lane_last;
+  uint64_t ep_last;
+  (void)uni_before(t, c, last, 0xffffffffu, &lane_last, &ep_last);
+  uint64_t chunks = 0, bytes = 0, off_in = 0;
+  if ((uint32_t)tid < L) {
+    chunks = uni_before(t, c, a.n, (uint32_t)tid, nullptr, nullptr);
+    bytes = chunks * c.C - ((uint32_t)tid == lane_last ? c.C - len_last : 0);
+  }
+  if (tid < FLH_MAX_LANES && keep_off) off_in = a.state->lane_off[tid];
+  __syncthreads();  // the old state has been read by everyone who needs it
+  if (tid < FLH_MAX_LANES) {
+    if (write_hdr) {
+      a.hdr->lane_bytes[tid] = bytes;
+      a.hdr->lane_chunks[tid] = (uint32_t)chunks;
+    }
+    if (write_state) a.state->lane_off[tid] = off_in + bytes;
+  }
+  if (tid == 0) {
+    if (write_hdr) {
+      uint32_t flags = 0;
+      const uint64_t n_ep = ep_last - c.e0 + 1;
+      const uint32_t look = n_ep < R ? (uint32_t)n_ep : R;
+      for (uint32_t k = 0; k < look; ++k) flags |= t.zero[(uint32_t)mod_u64(c.e0 + k, R)] ? FLH_SCHED_F_NO_CREDIT : 0;
+      a.hdr->total_bytes = a.total_bytes;
+      a.hdr->total_tiles = (uint32_t)last * tpc + (uint32_t)((len_last + a.tile_bytes - 1) / a.tile_bytes);
+      a.hdr->n_chunks = a.n;
+      a.hdr->flags = flags;
+      a.hdr->uniform_tiles = tpc;
+    }
+    if (write_state) {
+      uint64_t p_end;
+      if (c.E == 0 || ep_last == c.e0) {
+        p_end = ((c.E && c.pos0 == 0) ? 0 : p0) + a.total_bytes;
+      } else {
+        const uint64_t pos_last = (c.k0 + last) - ep_last * c.E;
+        p_end = pos_last * c.C + len_last;
+      }
+      a.state->epoch_bytes = p_end;
+      a.state->chunk_index = c.k0 + a.n;
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int flh_schedule(const flh_sched_params* p, void* stream) {
+  if (!p) return fl_set_error(FLH_E_ARG, "null params");
+  if (p->n_lanes == 0 || p->n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "n_lanes %u not in 1..%d", p->n_lanes, FLH_MAX_LANES);
+  if (p->n_rows == 0) return fl_set_error(FLH_E_ARG, "credit table missing");
+  if (!p->d_credits && p->n_rows != 1) return fl_set_error(FLH_E_ARG, "inline credits carry exactly one row");
+  if (p->quantum == 0) return fl_set_error(FLH_E_ARG, "quantum must be > 0");
+  if (p->tile_bytes == 0 || p->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", p->tile_bytes);
+  if (!p->d_hdr || (p->n_chunks && !p->d_table)) return fl_set_error(FLH_E_ARG, "output pointers missing");
+  if (!p->d_sizes) {
+    if (p->n_chunks && p->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0 for the uniform split");
+    const uint64_t need = p->chunk_bytes ? (p->total_bytes + p->chunk_bytes - 1) / p->chunk_bytes : 0;
+    if (need != p->n_chunks) return fl_set_error(FLH_E_ARG, "n_chunks %u does not match ceil(%llu / %u) = %llu", p->n_chunks,
+                                                (unsigned long long)p->total_bytes, p->chunk_bytes, (unsigned long long)need);
+  }
+  int rc = fl_need_init();
+  if (rc) return rc;
+  fl_prof().kid = 1;
+  SchedArgs a;
+  a.sizes = p->d_sizes;
+  a.total_bytes = p->total_bytes;
+  a.src_off = p->d_src_off;
+  a.src_base = p->src_base;
+  a.credits = p->d_credits;
+  a.quantum = p->quantum;
+  a.state = p->d_state;
+  a.table = p->d_table;
+  a.hdr = p->d_hdr;
+  a.table_by_lane = p->d_table_by_lane;
+  a.chunk_bytes = p->chunk_bytes;
+  a.n = p->n_chunks;
+  a.n_lanes = p->n_lanes;
+  a.n_rows = p->n_rows;
+  a.epoch_len = p->epoch_len;
+  a.tile_bytes = p->tile_bytes;
+  a.mode = p->mode;
+  for (int l = 0; l < FLH_MAX_LANES; ++l) a.inline_credits[l] = p->inline_credits[l];
+  a.quantum_shift = (p->quantum & (p->quantum - 1)) == 0 ? __builtin_ctzll(p->quantum) : -1;
+  hipStream_t s = (hipStream_t)stream;
+  a.tile_shift = (p->tile_bytes & (p->tile_bytes - 1)) == 0 ? __builtin_ctz(p->tile_bytes) : -1;
+  const uint32_t n = p->n_chunks;
+  const int variant = g_sched_variant;
+  // ordinary message split with quantum-sized chunks: closed form, no scan
+  if (g_sched_uniform_fast && variant == 0 && n > 0 && !p->d_sizes && !p->d_src_off && p->quantum == p->chunk_bytes &&
+      p->n_rows <= (uint32_t)kRowCache) {
+    const uint32_t grid = (n + kUniBlock - 1) / kUniBlock;
+    FL_LAUNCH((fl_schedule_uniform_kernel<0>), dim3(grid), dim3(kUniBlock), 0, s, a);
+    if (grid > 1 && p->d_state) FL_LAUNCH((fl_schedule_uniform_kernel<1>), dim3(1), dim3(kUniBlock), 0, s, a);
+    FL_HIP(hipGetLastError());
+    return FLH_OK;
+  }
+  if (p->d_table_by_lane && n > 0) return fl_set_error(FLH_E_ARG, "d_table_by_lane needs the uniform closed-form split (no d_sizes, no d_src_off, quantum == chunk_bytes, n_rows <= %d)", kRowCache);
+  // one workgroup; more chunks per thread once the per-pass overhead stops dominating
+  if ((variant == 0 && n <= kWave) || variant == 1) {
+    FL_LAUNCH((fl_schedule_kernel<1, 1>), dim3(1), dim3(kWave), 0, s, a);
+  } else if ((variant == 0 && n <= 8 * kWave) || variant == 2) {
+    FL_LAUNCH((fl_schedule_kernel<4, 1>), dim3(1), dim3(4 * kWave), 0, s, a);
+  } else if ((variant == 0 && n <= 32 * kWave) || variant == 3) {
+    FL_LAUNCH((fl_schedule_kernel<8, 4>), dim3(1), dim3(8 * kWave), 0, s, a);
+  } else {
+    FL_LAUNCH((fl_schedule_kernel<8, 8>), dim3(1), dim3(8 * kWave), 0, s, a);
+  }
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+}  // extern "C"
