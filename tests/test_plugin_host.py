@@ -37,6 +37,22 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} is declared in include/ but not exported"
 
 
+def test_library_shares_no_thread_local_variable_between_its_translation_units():
+    """A thread_local variable declared extern in one translation unit and defined in another is reached
+    through a wrapper that tests the address of the variable's (absent) initialiser, a weak hidden symbol;
+    in a shared object that address is computed relative to the load address, is never null, and gets
+    called.  Such state is reached through accessor functions here; the symbol table must show no
+    thread-local initialiser or wrapper."""
+    import shutil
+    import subprocess
+    nm = shutil.which("nm")
+    if not nm:
+        pytest.skip("nm not available")
+    out = subprocess.run([nm, P.lib_path()], capture_output=True, text=True, check=True).stdout
+    bad = [l for l in out.splitlines() if " _ZTH" in l or " _ZTW" in l]
+    assert not bad, bad
+
+
 @pytest.mark.parametrize("version", [6, 7, 8])
 def test_tables_and_properties(version):
     p = P.NetPlugin(version)
