@@ -79,19 +79,21 @@ def build_harness(verbose: bool = True) -> str | None:
     return out
 
 
-def build_tsan(verbose: bool = True):
-    """ThreadSanitizer build of the library's host code and of the harness (CPU-only check of the
-    plugin's locking: device code is compiled as usual, only the host pass is instrumented)."""
-    out_dir = os.path.join(ROOT, "tests", "harness", "tsan")
+def build_tsan(verbose: bool = True, sanitizer: str = "thread"):
+    """Sanitizer build of the library's host code and of the harness (CPU-only check of the plugin's
+    locking with "thread", of its memory handling with "address": device code is compiled as usual,
+    only the host pass is instrumented)."""
+    tag = {"thread": "tsan", "address": "asan"}[sanitizer]
+    out_dir = os.path.join(ROOT, "tests", "harness", tag)
     os.makedirs(out_dir, exist_ok=True)
-    lib = os.path.join(out_dir, "libnccl-net-fuselink-tsan.so")
-    exe = os.path.join(out_dir, "plugin_harness_tsan")
+    lib = os.path.join(out_dir, f"libnccl-net-fuselink-{tag}.so")
+    exe = os.path.join(out_dir, f"plugin_harness_{tag}")
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    flags = [f for f in FLAGS if f != "-O3"] + ["-O1", "-g", "-Xarch_host", "-fsanitize=thread"]
+    flags = [f for f in FLAGS if f != "-O3"] + ["-O1", "-g", "-Xarch_host", "-fsanitize=" + sanitizer]
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     clang = os.path.join(rocm, "llvm", "bin", "clang++")
     cmds = [[hipcc(), *flags, "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, *srcs, "-o", lib, "-ldl"],
-            [clang, "-O1", "-g", "-std=c++17", "-pthread", "-fsanitize=thread", "-D__HIP_PLATFORM_AMD__",
+            [clang, "-O1", "-g", "-std=c++17", "-pthread", "-fsanitize=" + sanitizer, "-D__HIP_PLATFORM_AMD__",
              "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(rocm, "include"),
              os.path.join(ROOT, "tests", "harness", "plugin_harness.cc"), "-o", exe,
              "-L" + os.path.join(rocm, "lib"), "-Wl,-rpath," + os.path.join(rocm, "lib"), "-lamdhip64", "-ldl"]]

@@ -100,3 +100,15 @@ def test_plugin_host_path_under_thread_sanitizer():
     assert "ThreadSanitizer" not in res.stderr, res.stderr[-3000:]
     assert res.returncode == 0, res.stderr[-2000:]
     assert json.loads(res.stdout.strip().splitlines()[-1])["bit_exact"]
+
+
+def test_plugin_host_path_under_address_sanitizer():
+    """The same traffic with AddressSanitizer on the host code (leak check included): connections, requests,
+    memory handles and listen comms are created and released many times over."""
+    lib, exe = build.build_tsan(verbose=False, sanitizer="address")
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:exitcode=67:protect_shadow_gap=0")
+    res = subprocess.run([exe, lib, "--host", "--bytes", str(4 << 20), "--request", str(256 << 10), "--connections", "4",
+                          "--inflight", "4", "--iters", "3"], capture_output=True, text=True, timeout=600, env=env)
+    assert "AddressSanitizer" not in res.stderr and "LeakSanitizer" not in res.stderr, res.stderr[-3000:]
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert json.loads(res.stdout.strip().splitlines()[-1])["bit_exact"]
