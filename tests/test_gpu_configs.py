@@ -330,3 +330,54 @@ def test_cfg5_stress_full_size(fl):
     for w in wins:
         w.destroy()
     pool.destroy()
+
+
+def test_message_beyond_4_gib(fl):
+    """Offsets past 2^32: a 4 GiB + 3 MiB + 5 B message over 8 lanes through the table-driven kernels (chunk order
+    and destination order), the fused kernels (which pick destination order by themselves at this size) and the
+    generic tile-search kernel; the table against the oracle, the round trip bit for bit."""
+    core, torch = fl
+    total, chunk, lanes = (4 << 30) + (3 << 20) + 5, 1 << 20, 8
+    credits = [5, 1, 7, 2, 8, 3, 1, 6]
+    free, _ = torch.cuda.mem_get_info()
+    if free < 4 * total:
+        pytest.skip("not enough device memory for three 4 GiB buffers")
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk)
+    assert int(exp_t["src_off"][-1]) > 2**32 and int(exp_h["lane_bytes"].max()) < 2**32
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(44)
+    src = torch.randint(0, 2**31 - 1, ((total + 3) // 4,), dtype=torch.int32, device="cuda", generator=gen).view(torch.uint8)[:total]
+    dst = torch.empty_like(src)
+    sched = core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk, by_lane=True)
+    torch.cuda.synchronize()
+    assert sched.table_numpy().tobytes() == exp_t.tobytes()
+    caps = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    wins = [torch.empty(c, dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    hint = core.uniform_hint(total, chunk)
+    u = core.uniform_params(total, chunk, credits)
+
+    def check(tag):
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0, tag
+        assert torch.equal(src, dst), tag
+        dst.zero_()
+        for t in wins:
+            t.zero_()
+
+    dst.zero_()
+    core.stripe(src, w, sched, status, hint=hint)
+    core.reassemble(dst, w, sched, status, hint=hint)
+    check("table-driven, chunk order")
+    core.stripe(src, w, sched, status, hint=hint, by_lane=True)
+    core.reassemble(dst, w, sched, status, hint=hint)
+    check("table-driven, destination order")
+    core.stripe(src, w, sched, status)          # no host hint: the tile-search kernel
+    core.reassemble(dst, w, sched, status)
+    check("generic kernel")
+    out = core.new_schedule_buffers(len(exp_t))
+    core.stripe_uniform(src, w, u, status, out=out)
+    core.reassemble_uniform(dst, w, u, status)
+    check("fused")
+    assert out.table_numpy().tobytes() == exp_t.tobytes()

@@ -41,8 +41,9 @@ def _schedule_case(core, torch, seed):
     tile = int(rng.choice([128, 4096, 32768, 3*128]))
     mode = int(rng.choice([0, 1, 4, 5, 2]))
     st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
-    st["chunk_index"] = int(rng.integers(0, 5000)); st["epoch_bytes"] = int(rng.integers(0, 1 << 24))
-    st["lane_off"][:lanes] = rng.integers(0, 1 << 30, size=lanes)
+    st["chunk_index"] = int(rng.integers(0, 5000))
+    st["epoch_bytes"] = int(rng.integers(0, 1 << int(rng.choice([24, 41]))))      # carried prefixes past 32 bits too
+    st["lane_off"][:lanes] = rng.integers(0, 1 << int(rng.choice([30, 45])), size=lanes)
     kind = int(rng.integers(0, 3))
     what = f"seed {seed} kind {kind} lanes {lanes} rows {rows} E {epoch_len} tile {tile} mode {mode}"
     if kind == 0:   # variable sizes, scan kernel
