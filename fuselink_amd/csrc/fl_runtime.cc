@@ -142,7 +142,7 @@ int flh_tune(const char* key, int64_t value) {
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
-  if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 4) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..4"); g_sched_variant = (int)value; return FLH_OK; }
+  if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 6) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..6"); g_sched_variant = (int)value; return FLH_OK; }
   return fl_set_error(FLH_E_ARG, "unknown tunable %s", key);
 }
 

@@ -660,12 +660,16 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     return FLH_OK;
   }
   if (p->d_table_by_lane && n > 0) return fl_set_error(FLH_E_ARG, "d_table_by_lane needs the uniform closed-form split (no d_sizes, no d_src_off, quantum == chunk_bytes, n_rows <= %d)", kRowCache);
-  // one workgroup; more chunks per thread once the per-pass overhead stops dominating
-  if ((variant == 0 && n <= kWave) || variant == 1) {
+  // one workgroup; more wavefronts first, then more chunks per thread, as the chunk count grows (measured best shapes)
+  if ((variant == 0 && n <= kWave && p->n_rows <= 4) || variant == 1) {   // a lone wavefront prefixes four credit rows per turn
     FL_LAUNCH((fl_schedule_kernel<1, 1>), dim3(1), dim3(kWave), 0, s, a);
-  } else if ((variant == 0 && n <= 8 * kWave) || variant == 2) {
+  } else if ((variant == 0 && n <= 4 * kWave) || variant == 2) {
     FL_LAUNCH((fl_schedule_kernel<4, 1>), dim3(1), dim3(4 * kWave), 0, s, a);
-  } else if ((variant == 0 && n <= 32 * kWave) || variant == 3) {
+  } else if ((variant == 0 && n <= 8 * kWave) || variant == 3) {
+    FL_LAUNCH((fl_schedule_kernel<8, 1>), dim3(1), dim3(8 * kWave), 0, s, a);
+  } else if ((variant == 0 && n <= 16 * kWave) || variant == 4) {
+    FL_LAUNCH((fl_schedule_kernel<8, 2>), dim3(1), dim3(8 * kWave), 0, s, a);
+  } else if ((variant == 0 && n <= 32 * kWave) || variant == 5) {
     FL_LAUNCH((fl_schedule_kernel<8, 4>), dim3(1), dim3(8 * kWave), 0, s, a);
   } else {
     FL_LAUNCH((fl_schedule_kernel<8, 8>), dim3(1), dim3(8 * kWave), 0, s, a);
