@@ -106,6 +106,48 @@ __device__ __forceinline__ void lane_pass(const uint32_t (&s)[K], const uint32_t
   if ((uint32_t)lane < L) w_lane_row[lane] = my_total;
 }
 
+// The same result for threads that own several chunks (K >= 4), with work per thread of K + L instead of K * L:
+// every thread keeps one running byte count per lane in its own column of `acc` (LDS, [lane][thread], so the
+// columns never collide and a wavefront's accesses fall on distinct banks), hands each chunk the count found
+// there, then the per-lane scans run over the threads' column totals and their exclusive results are added back.
+// 32-bit sums only: the caller takes the other routine when a pass moves 4 GiB or more.
+template <int K, int BT>
+__device__ __forceinline__ void lane_pass_columns(const uint32_t (&s)[K], const uint32_t (&ln)[K], uint32_t L, int tid, int lane,
+                                                  uint32_t* acc, uint64_t* w_lane_row, uint64_t (&off)[K]) {
+  constexpr int G = 4;
+#pragma unroll 1
+  for (uint32_t l = 0; l < L; ++l) acc[l * BT + tid] = 0;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    if (ln[k] < L) {   // chunks past the end carry the lane "none"
+      uint32_t* p = &acc[ln[k] * BT + tid];
+      const uint32_t o = *p;
+      off[k] = o;
+      *p = o + s[k];
+    }
+  }
+  uint64_t my_total = 0;
+#pragma unroll 1
+  for (uint32_t l0 = 0; l0 < L; l0 += G) {
+    uint32_t v[G], inc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) v[g] = l0 + g < L ? acc[(l0 + g) * BT + tid] : 0;
+#pragma unroll
+    for (int g = 0; g < G; ++g) inc[g] = wave_incl_sum_u32(v[g], lane);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      if (l0 + g < L) acc[(l0 + g) * BT + tid] = inc[g] - v[g];
+      const uint32_t tot = bcast_lane_u32(inc[g], kWave - 1);
+      if ((uint32_t)lane == l0 + g) my_total = tot;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    if (ln[k] < L) off[k] += acc[ln[k] * BT + tid];
+  }
+  if ((uint32_t)lane < L) w_lane_row[lane] = my_total;
+}
+
 // One workgroup of NW wavefronts walks the chunk list in passes of NW*64*K chunks; thread t owns K
 // consecutive chunks of a pass.  Per pass: thread-local sums, three wavefront scans (epoch-segmented
 // bytes, bytes, tiles), the lane of each chunk from its quantum slot, one wavefront scan per lane
@@ -133,6 +175,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   __shared__ uint64_t lane_off0[FLH_MAX_LANES];
   __shared__ uint32_t cnt_lane[FLH_MAX_LANES];
   __shared__ uint32_t sh_flags;
+  __shared__ uint32_t acc[K >= 4 ? FLH_MAX_LANES * BT : 1];   // per-thread, per-lane running byte counts (lane_pass_columns)
 
   // One wavefront per row: lanes 0..L-1 load the row in a single access, a scan forms the prefixes.
   // A row without any credit (every lane busy) is replaced by equal credits -- the round-robin of
@@ -323,8 +366,13 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
     uint64_t off[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) off[k] = 0;
-    if ((tot_run >> 32) == 0) lane_pass<uint32_t, K>(s, ln, L, lane, w_lane[wave], off);
-    else lane_pass<uint64_t, K>(s, ln, L, lane, w_lane[wave], off);
+    if constexpr (K >= 4) {
+      if ((tot_run >> 32) == 0) lane_pass_columns<K, BT>(s, ln, L, tid, lane, acc, w_lane[wave], off);
+      else lane_pass<uint64_t, K>(s, ln, L, lane, w_lane[wave], off);
+    } else {
+      if ((tot_run >> 32) == 0) lane_pass<uint32_t, K>(s, ln, L, lane, w_lane[wave], off);
+      else lane_pass<uint64_t, K>(s, ln, L, lane, w_lane[wave], off);
+    }
     __syncthreads();
     if ((uint32_t)tid < L) {
       uint64_t at = lane_off[tid];
