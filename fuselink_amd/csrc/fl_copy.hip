@@ -19,16 +19,16 @@ namespace {
 constexpr int kCopyBlock = 256;
 constexpr int kCopyUnroll = 8;
 
-template <bool NT>
+template <int NT>
 __device__ __forceinline__ u32x4 ld16(const u32x4* p) {
-  return NT ? __builtin_nontemporal_load(p) : *p;
+  return (NT & 1) ? __builtin_nontemporal_load(p) : *p;   // bit 0 of the streaming mode: loads
 }
-template <bool NT>
+template <int NT>
 __device__ __forceinline__ void st16(u32x4* p, u32x4 v) {
-  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+  if (NT & 2) __builtin_nontemporal_store(v, p); else *p = v;   // bit 1: stores
 }
 
-template <bool NT, int U>
+template <int NT, int U>
 __device__ __forceinline__ void copy_exact(u32x4* __restrict__ d, const u32x4* __restrict__ s, uint32_t tid) {
   u32x4 r[U];
 #pragma unroll
@@ -40,7 +40,7 @@ __device__ __forceinline__ void copy_exact(u32x4* __restrict__ d, const u32x4* _
 // Copies `bytes` from src to dst with the whole workgroup.  Fast path: both 16-byte aligned ->
 // dwordx4 loads batched kCopyUnroll deep before the stores.  Equal misalignment: byte head up to
 // the boundary, vectors, byte tail.  Different misalignment: byte copy (correct, not fast).
-template <bool NT>
+template <int NT>
 __device__ __forceinline__ void block_copy(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
                                            uint32_t bytes) {
   const uint32_t tid = threadIdx.x;
@@ -123,7 +123,7 @@ __device__ __forceinline__ uint32_t find_row(const flh_chunk_desc* __restrict__ 
 }
 
 // DIR 0: user -> windows (stripe).  DIR 1: windows -> user (reassemble).
-template <int DIR, bool NT>
+template <int DIR, int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
   const uint32_t total = a.has_hint ? a.hint_total_tiles : a.hdr->total_tiles;
   const uint32_t uniform_tiles = a.has_hint ? a.hint_uniform_tiles : a.hdr->uniform_tiles;
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
 // Uniform split with the header known on the host: a two-dimensional grid (tile in chunk, chunk)
 // names the work directly, so a workgroup's only dependent access before its data is the one scalar
 // load of its table row.
-template <int DIR, bool NT>
+template <int DIR, int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform(CopyArgs a) {
   const uint32_t c = blockIdx.y;
   if (c >= a.hint_n_chunks) return;
@@ -240,7 +240,7 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
   return full * c + part;
 }
 
-template <int DIR, bool NT, class Args>
+template <int DIR, int NT, class Args>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   constexpr bool BATCH = is_batch<Args>::value;
   if (blockIdx.y >= a.n_chunks) return;
@@ -382,7 +382,7 @@ constexpr uint32_t kLdsStage = 16384;
 
 // DIR 0: pool pages -> windows (gather).  DIR 1: windows -> pool pages (scatter).
 // LDS: stage each sub-tile through LDS (coalesced global->LDS, barrier, LDS->global).
-template <int DIR, bool LDS, bool NT>
+template <int DIR, int NT, bool LDS>
 __global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
   __shared__ u32x4 stage[LDS ? kLdsStage / 16 : 1];
   const uint64_t total = (uint64_t)a.n_chunks * a.pages_per_chunk * a.subs_per_page;
@@ -430,7 +430,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
   }
 }
 
-template <bool NT>
+template <int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const uint8_t* src, uint64_t bytes,
                                                             uint32_t tile_bytes) {
   const uint64_t tiles = (bytes + tile_bytes - 1) / tile_bytes;
@@ -442,6 +442,23 @@ __global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const 
 }
 
 }  // namespace
+
+// One launch per (direction, streaming mode) pair that the policy can ask for: striping / gathering with modes
+// 0, 1, 3, reassembly / scattering with 0, 2, 3 (fl_stream_mode returns no other).  EXTRA carries trailing
+// template arguments.
+#define FL_LAUNCH_COPY(NAME, EXTRA, dir, mode, grid, s, a)                                  \
+  do {                                                                                      \
+    if ((dir) == 0) {                                                                       \
+      if ((mode) == 0) FL_LAUNCH((NAME<0, 0 EXTRA>), grid, dim3(kCopyBlock), 0, s, a);      \
+      else if ((mode) == 1) FL_LAUNCH((NAME<0, 1 EXTRA>), grid, dim3(kCopyBlock), 0, s, a); \
+      else FL_LAUNCH((NAME<0, 3 EXTRA>), grid, dim3(kCopyBlock), 0, s, a);                  \
+    } else {                                                                                \
+      if ((mode) == 0) FL_LAUNCH((NAME<1, 0 EXTRA>), grid, dim3(kCopyBlock), 0, s, a);      \
+      else if ((mode) == 2) FL_LAUNCH((NAME<1, 2 EXTRA>), grid, dim3(kCopyBlock), 0, s, a); \
+      else FL_LAUNCH((NAME<1, 3 EXTRA>), grid, dim3(kCopyBlock), 0, s, a);                  \
+    }                                                                                       \
+  } while (0)
+#define FL_NO_EXTRA
 
 extern "C" {
 
@@ -481,27 +498,15 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   const uint64_t max_tiles = h_hdr ? h_hdr->total_tiles : user_bytes / tile_bytes + n_chunks_max;
   if (max_tiles == 0) return FLH_OK;
   hipStream_t s = (hipStream_t)stream;
-  const bool nt = fl_use_nt(3 * user_bytes);  // user buffer + windows + the peer's buffer
+  const int mode = fl_stream_mode(dir, user_bytes);
   if (h_hdr && h_hdr->uniform_tiles && h_hdr->n_chunks <= 65535 && h_hdr->n_chunks <= n_chunks_max && g_copy_uniform_grid) {
     const dim3 grid(h_hdr->uniform_tiles, h_hdr->n_chunks);
-    if (dir == 0) {
-      if (nt) FL_LAUNCH((fl_copy_uniform<0, true>), grid, dim3(kCopyBlock), 0, s, a);
-      else FL_LAUNCH((fl_copy_uniform<0, false>), grid, dim3(kCopyBlock), 0, s, a);
-    } else {
-      if (nt) FL_LAUNCH((fl_copy_uniform<1, true>), grid, dim3(kCopyBlock), 0, s, a);
-      else FL_LAUNCH((fl_copy_uniform<1, false>), grid, dim3(kCopyBlock), 0, s, a);
-    }
+    FL_LAUNCH_COPY(fl_copy_uniform, FL_NO_EXTRA, dir, mode, grid, s, a);
     FL_HIP(hipGetLastError());
     return FLH_OK;
   }
-  const uint32_t grid = fl_copy_grid(max_tiles);
-  if (dir == 0) {
-    if (nt) FL_LAUNCH((fl_copy_tiles<0, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
-    else FL_LAUNCH((fl_copy_tiles<0, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
-  } else {
-    if (nt) FL_LAUNCH((fl_copy_tiles<1, true>), dim3(grid), dim3(kCopyBlock), 0, s, a);
-    else FL_LAUNCH((fl_copy_tiles<1, false>), dim3(grid), dim3(kCopyBlock), 0, s, a);
-  }
+  const dim3 grid(fl_copy_grid(max_tiles));
+  FL_LAUNCH_COPY(fl_copy_tiles, FL_NO_EXTRA, dir, mode, grid, s, a);
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }
@@ -572,16 +577,12 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
 
 extern "C++" {
 template <class Args>
-static int launch_fused_args(int dir, const Args& a, bool nt, void* stream) {
+static int launch_fused_args(int dir, const Args& a, int mode, void* stream) {
   const dim3 grid(a.tiles_per_chunk, a.n_chunks);
   hipStream_t s = (hipStream_t)stream;
-  if (dir == 0) {
-    if (nt) FL_LAUNCH((fl_copy_uniform_fused<0, true, Args>), grid, dim3(kCopyBlock), 0, s, a);
-    else FL_LAUNCH((fl_copy_uniform_fused<0, false, Args>), grid, dim3(kCopyBlock), 0, s, a);
-  } else {
-    if (nt) FL_LAUNCH((fl_copy_uniform_fused<1, true, Args>), grid, dim3(kCopyBlock), 0, s, a);
-    else FL_LAUNCH((fl_copy_uniform_fused<1, false, Args>), grid, dim3(kCopyBlock), 0, s, a);
-  }
+#define FL_ARGS_EXTRA , Args
+  FL_LAUNCH_COPY(fl_copy_uniform_fused, FL_ARGS_EXTRA, dir, mode, grid, s, a);
+#undef FL_ARGS_EXTRA
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }
@@ -595,7 +596,7 @@ static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_wind
   if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
   a.user = (uint8_t*)user;
   a.user_bytes = user_bytes;
-  return launch_fused_args(dir, a, fl_use_nt(3 * user_bytes), stream);
+  return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream);
 }
 
 static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table, flh_sched_hdr* d_hdr,
@@ -623,7 +624,7 @@ static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* w
     sum += b->bytes[q];
   }
   if (sum != b->u.total_bytes) return fl_set_error(FLH_E_ARG, "the requests hold %llu bytes, the parameters say %llu", (unsigned long long)sum, (unsigned long long)b->u.total_bytes);
-  return launch_fused_args(dir, a, fl_use_nt(3 * sum), stream);
+  return launch_fused_args(dir, a, fl_stream_mode(dir, sum), stream);
 }
 
 int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
@@ -674,16 +675,14 @@ static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t
   const uint64_t total = (uint64_t)n_chunks * pages_per_chunk * a.subs_per_page;
   const uint32_t grid = fl_copy_grid(total);
   hipStream_t s = (hipStream_t)stream;
-  const bool nt = fl_use_nt(3ull * n_chunks * pages_per_chunk * page_bytes);
-#define FL_LAUNCH_PAGES(D, LD, N) FL_LAUNCH((fl_page_tiles<D, LD, N>), dim3(grid), dim3(kCopyBlock), 0, s, a)
-  if (dir == 0) {
-    if (use_lds) { if (nt) FL_LAUNCH_PAGES(0, true, true); else FL_LAUNCH_PAGES(0, true, false); }
-    else { if (nt) FL_LAUNCH_PAGES(0, false, true); else FL_LAUNCH_PAGES(0, false, false); }
-  } else {
-    if (use_lds) { if (nt) FL_LAUNCH_PAGES(1, true, true); else FL_LAUNCH_PAGES(1, true, false); }
-    else { if (nt) FL_LAUNCH_PAGES(1, false, true); else FL_LAUNCH_PAGES(1, false, false); }
-  }
-#undef FL_LAUNCH_PAGES
+  const int mode = fl_stream_mode(dir, (uint64_t)n_chunks * pages_per_chunk * page_bytes);
+  const dim3 grid3(grid);
+#define FL_LDS_ON , true
+#define FL_LDS_OFF , false
+  if (use_lds) FL_LAUNCH_COPY(fl_page_tiles, FL_LDS_ON, dir, mode, grid3, s, a);
+  else FL_LAUNCH_COPY(fl_page_tiles, FL_LDS_OFF, dir, mode, grid3, s, a);
+#undef FL_LDS_ON
+#undef FL_LDS_OFF
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }
@@ -709,8 +708,8 @@ int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
   const uint32_t tile = FLH_TILE_BYTES;
   const uint32_t grid = fl_copy_grid((bytes + tile - 1) / tile);
   hipStream_t s = (hipStream_t)stream;
-  if (fl_use_nt(2 * bytes)) FL_LAUNCH(fl_plain_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
-  else FL_LAUNCH(fl_plain_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  if (fl_use_nt(2 * bytes)) FL_LAUNCH(fl_plain_copy<3>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  else FL_LAUNCH(fl_plain_copy<0>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }

@@ -55,6 +55,13 @@ bool fl_use_nt(uint64_t working_set_bytes) {
   return working_set_bytes > kCacheResidentBytes;
 }
 
+int fl_stream_mode(int dir, uint64_t bytes) {
+  if (g_nontemporal >= 0) return g_nontemporal ? 3 : 0;
+  if (bytes > (320ull << 20)) return 3;                       // the windows no longer fit the Infinity Cache
+  if (dir == 0) return bytes >= (128ull << 20) ? 1 : 0;       // read the user buffer once, keep the windows cacheable
+  return 2;                                                   // windows come from cache, the user buffer is written once
+}
+
 uint32_t fl_copy_grid(uint64_t max_tiles) {
   uint64_t g = g_grid_per_cu > 0 ? (uint64_t)g_cus * (uint64_t)g_grid_per_cu : (1ull << 20);
   if (g > max_tiles) g = max_tiles;
