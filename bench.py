@@ -110,7 +110,7 @@ def main() -> int:
     # a message too large for the Infinity Cache is striped in destination order (windows written front to back):
     # the scheduler then also emits the table's rows lane by lane
     # (measured: no gain for the paged gather, whose reads are scattered either way, so it keeps chunk order)
-    by_lane = kind == "uniform" and rows <= 32 and 3 * nbytes > (512 << 20) and not args.no_by_lane
+    by_lane = kind == "uniform" and rows <= 32 and nbytes > (256 << 20) and not args.no_by_lane
 
     def run_schedule(out=None):
         return core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, sizes=sizes,
@@ -243,7 +243,7 @@ def main() -> int:
                    "step": ("2x(schedule+gather+scatter)" if kind == "pages" else
                             "stripe(with scheduler folded in)+reassemble" if fused else "schedule+stripe+reassemble"),
                    "launch": "eager", "windows": "HIP VMM, 2 MiB units",
-                   "stripe_order": "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel past 512 MiB of buffers)" if fused else "chunk"},
+                   "stripe_order": "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel for messages past 256 MiB)" if fused else "chunk"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
         "kernels_us": {"schedule": round(sched_us, 2), out_k: round(stripe_us, 2), in_k: round(reasm_us, 2),

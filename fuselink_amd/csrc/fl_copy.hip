@@ -553,7 +553,7 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
   a.tile_bytes = u->tile_bytes;
   a.tiles_per_chunk = (u->chunk_bytes + u->tile_bytes - 1) / u->tile_bytes;
   // once the message no longer fits the Infinity Cache, write every window front to back
-  a.dest_order = dir == 0 && (g_dest_order < 0 ? 3 * u->total_bytes > kCacheResidentBytes : g_dest_order != 0);
+  a.dest_order = dir == 0 && (g_dest_order < 0 ? u->total_bytes > kWindowsCacheableBytes : g_dest_order != 0);
   for (int l = 0; l < FLH_MAX_LANES; ++l) a.credits[l] = (uint32_t)l < u->n_lanes ? u->credits[l] : 0;
   {
     // the row as the kernel sees it (equal credits stand in for an all-zero row), then the host-side constants

@@ -24,7 +24,8 @@ extern FL_LOCAL int g_nontemporal;         // -1: streaming accesses only when t
 extern FL_LOCAL int g_sched_variant;       // 0 = pick the scheduler shape from the chunk count
 extern FL_LOCAL int g_sched_uniform_fast;
 extern FL_LOCAL int g_copy_uniform_grid;
-constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // working sets up to this stay largely in the 256 MB Infinity Cache
+constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // plain copy: working sets up to this stay largely in the 256 MB Infinity Cache
+constexpr uint64_t kWindowsCacheableBytes = 256ull << 20;  // a message whose staging windows still fit the Infinity Cache
 
 // Per-launch timing: while a profiling region is open on the calling thread, every kernel is launched
 // with its own start/stop events (hipExtLaunchKernelGGL), which bracket the kernel alone and not the
@@ -72,7 +73,7 @@ FL_LOCAL bool fl_use_nt(uint64_t working_set_bytes);
 // bit 1 = streaming stores.  What is used once streams -- the user buffer read by the striping side from 128 MiB
 // on, the user buffer written by the reassembly side from 80 MiB on -- and the staging windows, written by one
 // launch and read by the next, stay cacheable until they outgrow the 256 MB Infinity Cache (then everything
-// streams).  Measured against all-cached / all-streaming, stripe + reassemble: 64 MiB equal, 96 MiB +4 %,
+// streams; at 320 MiB the cacheable variant already thrashes: reassembly 146 instead of 117 us).  Measured against all-cached / all-streaming, stripe + reassemble: 64 MiB equal, 96 MiB +4 %,
 // 128 MiB +8 %, 192 MiB +11 %, 256 MiB +9 %, 384 MiB and beyond equal.
 FL_LOCAL int fl_stream_mode(int dir, uint64_t bytes);
 // workgroups for a copy over max_tiles tiles: one per tile (the dispatcher then overlaps loads and stores of

@@ -57,7 +57,7 @@ bool fl_use_nt(uint64_t working_set_bytes) {
 
 int fl_stream_mode(int dir, uint64_t bytes) {
   if (g_nontemporal >= 0) return g_nontemporal ? 3 : 0;
-  if (bytes > (320ull << 20)) return 3;                       // the windows no longer fit the Infinity Cache
+  if (bytes > kWindowsCacheableBytes) return 3;               // the windows no longer fit the Infinity Cache
   if (dir == 0) return bytes >= (128ull << 20) ? 1 : 0;       // read the user buffer once, keep the windows cacheable
   return bytes >= (80ull << 20) ? 2 : 0;                      // windows come from cache; write the user buffer past the cache once it is large
 }
