@@ -251,7 +251,9 @@ def main() -> int:
                        "plain_copy_same_bytes": round(copy_us, 2)},
         "stripe_reassemble_pair_GBps": round(algo_bytes_step / (pair_us * 1e-6) / 1e9, 1),
         "scheduler_kernel": "standalone launch, not part of the fused step" if fused else "first launch of every message",
-        "scheduler_us_per_1k_chunks": round(sched_us * n_sched / (n_chunks / 1000.0), 3),
+        # one launch schedules a whole message; below 1000 chunks its cost is the flat launch time, not a per-1k rate
+        "scheduler_launch_us": round(sched_us, 2),
+        "scheduler_us_per_1k_chunks": round(sched_us * n_sched / (n_chunks / 1000.0), 3) if n_chunks >= 1000 else None,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC.get(args.workload)},
