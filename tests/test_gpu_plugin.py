@@ -495,7 +495,7 @@ def test_rccl_loads_the_plugin_and_probes_every_device(name):
     env = dict(os.environ, NCCL_NET_PLUGIN=name, NCCL_DEBUG="INFO", NCCL_DEBUG_SUBSYS="INIT,NET",
                LD_LIBRARY_PATH=libdir + ":" + os.environ.get("LD_LIBRARY_PATH", ""), MASTER_PORT="29541")
     probe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "rccl_probe.py")
-    res = subprocess.run([sys.executable, probe], capture_output=True, text=True, timeout=110, env=env)
+    res = subprocess.run([sys.executable, probe], capture_output=True, text=True, timeout=170, env=env)
     log = res.stdout + res.stderr
     assert res.returncode == 0, log[-3000:]
     assert "Loaded net plugin FuseLink (v8)" in log, log[-3000:]
