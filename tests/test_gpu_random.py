@@ -33,10 +33,12 @@ def _schedule_case(core, torch, seed):
     dev = lambda a: _dev(torch, a)  # noqa: E731
     same = _same
     rng = np.random.default_rng(seed)
-    lanes = int(rng.integers(1, 17)); rows = int(rng.integers(1, 40))
+    lanes = int(rng.integers(1, 17))
+    rows = int(rng.integers(1, 40))
     hi = int(rng.choice([2, 9, 1000, 2**20]))
     credits = rng.integers(0, hi, size=(rows, lanes)).astype(np.uint32)
-    if rng.random() < 0.3: credits[rng.integers(0, rows)] = 0
+    if rng.random() < 0.3:
+        credits[rng.integers(0, rows)] = 0
     epoch_len = int(rng.choice([0, 1, 2, 7, 64, 1000]))
     tile = int(rng.choice([128, 4096, 32768, 3*128]))
     mode = int(rng.choice([0, 1, 4, 5, 2]))
@@ -109,8 +111,10 @@ def _copy_case(core, torch, seed, status):
         pad = [int(rng.integers(0, 16)) for _ in caps]      # misaligned window bases
         wins = [torch.zeros(c + 64, dtype=torch.uint8, device="cuda") for c in caps]
         w = core.make_windows([t.data_ptr() + p for t, p in zip(wins, pad)], caps)
-        src = dev(src_np); dst = torch.zeros_like(src)
-        core.stripe(src, w, sched, status); core.reassemble(dst, w, sched, status)
+        src = dev(src_np)
+        dst = torch.zeros_like(src)
+        core.stripe(src, w, sched, status)
+        core.reassemble(dst, w, sched, status)
         torch.cuda.synchronize()
         exp_w = ob.cpu_stripe(src_np, exp_t, caps)
         for l in range(lanes):
@@ -118,14 +122,16 @@ def _copy_case(core, torch, seed, status):
             assert np.array_equal(got[pad[l]: pad[l] + caps[l]], exp_w[l][: caps[l]]), (what, "window", l)
             assert not got[:pad[l]].any() and not got[pad[l] + caps[l]:].any(), (what, "guard", l)
         exp_dst = np.zeros_like(src_np)
-        for r in exp_t: exp_dst[int(r["src_off"]): int(r["src_off"]) + int(r["len"])] = src_np[int(r["src_off"]): int(r["src_off"]) + int(r["len"])]
+        for r in exp_t:
+            exp_dst[int(r["src_off"]): int(r["src_off"]) + int(r["len"])] = src_np[int(r["src_off"]): int(r["src_off"]) + int(r["len"])]
         assert np.array_equal(dst.cpu().numpy(), exp_dst), (what, "dst")
     else:
         chunk = int(rng.choice([128, 4096, 65536, 100*128, 3*128]))
         n = int(rng.integers(1, 60))
         total = n*chunk - int(rng.integers(0, chunk))
         epoch_bytes = int(rng.integers(0, 30))*chunk
-        st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]; st["epoch_bytes"] = epoch_bytes
+        st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+        st["epoch_bytes"] = epoch_bytes
         base = int(rng.integers(0, 5))*int(rng.choice([1, 16, 4096])) if kind != 3 else 0
         exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk, tile_bytes=tile, mode=1, state=st, src_base=base)
         caps = [int(b) for b in exp_h["lane_bytes"][:lanes]]
@@ -137,9 +143,12 @@ def _copy_case(core, torch, seed, status):
             core.tune("stripe_dest_order", int(rng.integers(0, 2)))
             u = core.uniform_params(total, chunk, credits.tolist(), src_base=base, epoch_bytes=epoch_bytes, tile_bytes=tile)
             out = core.new_schedule_buffers(n, tile)
-            src = dev(src_np); dst = torch.zeros_like(src)
-            core.stripe_uniform(src, w, u, status, out=out); core.reassemble_uniform(dst, w, u, status)
-            torch.cuda.synchronize(); core.tune("stripe_dest_order", -1)
+            src = dev(src_np)
+            dst = torch.zeros_like(src)
+            core.stripe_uniform(src, w, u, status, out=out)
+            core.reassemble_uniform(dst, w, u, status)
+            torch.cuda.synchronize()
+            core.tune("stripe_dest_order", -1)
             assert out.table_numpy().tobytes() == exp_t.tobytes(), (what, "table")
             assert np.array_equal(dst.cpu().numpy()[base:], src_np[base:]) and not dst.cpu().numpy()[:base].any(), (what, "dst")
         elif kind == 2:  # scheduler kernel + table-driven copies, with and without the host hint, rows by lane or by chunk
@@ -147,8 +156,10 @@ def _copy_case(core, torch, seed, status):
             d_state = dev(np.array([st], dtype=ob.STATE_DTYPE).view(np.uint8))
             sched = core.schedule(n_lanes=lanes, credits=credits.tolist(), quantum=chunk, total_bytes=total, chunk_bytes=chunk, tile_bytes=tile, mode=1, state=d_state, src_base=base, by_lane=by_lane)
             hint = core.uniform_hint(total, chunk, tile) if rng.integers(0, 2) else None
-            src = dev(src_np); dst = torch.zeros_like(src)
-            core.stripe(src, w, sched, status, hint=hint, by_lane=by_lane); core.reassemble(dst, w, sched, status, hint=hint)
+            src = dev(src_np)
+            dst = torch.zeros_like(src)
+            core.stripe(src, w, sched, status, hint=hint, by_lane=by_lane)
+            core.reassemble(dst, w, sched, status, hint=hint)
             torch.cuda.synchronize()
             assert np.array_equal(dst.cpu().numpy()[base:], src_np[base:]), (what, "dst")
         else:            # batch of requests
@@ -157,10 +168,12 @@ def _copy_case(core, torch, seed, status):
             bounds = [0] + [c*chunk for c in cuts] + [total]
             sizes = [b - a for a, b in zip(bounds[:-1], bounds[1:])]
             srcs_np = [src_np[a:b] for a, b in zip(bounds[:-1], bounds[1:])]
-            srcs = [dev(x) for x in srcs_np]; dsts = [torch.zeros(s + 16, dtype=torch.uint8, device="cuda") for s in sizes]
+            srcs = [dev(x) for x in srcs_np]
+            dsts = [torch.zeros(s + 16, dtype=torch.uint8, device="cuda") for s in sizes]
             b = core.batch_params(srcs, dsts, chunk, credits.tolist(), epoch_bytes=epoch_bytes, tile_bytes=tile)
             out = core.new_schedule_buffers(n, tile)
-            core.stripe_batch(b, w, status, out=out); core.reassemble_batch(b, w, status)
+            core.stripe_batch(b, w, status, out=out)
+            core.reassemble_batch(b, w, status)
             torch.cuda.synchronize()
             assert out.table_numpy().tobytes() == exp_t.tobytes(), (what, "table")
             exp_w = ob.cpu_stripe(src_np, exp_t, caps)
