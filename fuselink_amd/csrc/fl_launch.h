@@ -71,10 +71,12 @@ FL_LOCAL int fl_need_init();
 FL_LOCAL bool fl_use_nt(uint64_t working_set_bytes);
 // Streaming mode of a striping (dir 0) or reassembly (dir 1) launch that moves `bytes`: bit 0 = streaming loads,
 // bit 1 = streaming stores.  What is used once streams -- the user buffer read by the striping side from 128 MiB
-// on, the user buffer written by the reassembly side from 80 MiB on -- and the staging windows, written by one
+// on, the user buffer written by the reassembly side from 16 MiB on -- and the staging windows, written by one
 // launch and read by the next, stay cacheable until they outgrow the 256 MB Infinity Cache (then everything
-// streams; at 320 MiB the cacheable variant already thrashes: reassembly 146 instead of 117 us).  Measured against all-cached / all-streaming, stripe + reassemble: 64 MiB equal, 96 MiB +4 %,
-// 128 MiB +8 %, 192 MiB +11 %, 256 MiB +9 %, 384 MiB and beyond equal.
+// streams; at 320 MiB the cacheable variant already thrashes: reassembly 146 instead of 117 us).  Measured
+// against all-cached / all-streaming, stripe + reassemble over one pair of user buffers: 64 MiB equal, 96 MiB
+// +4 %, 128 MiB +8 %, 192 MiB +11 %, 256 MiB +9 %, 384 MiB and beyond equal; over user buffers that no cache
+// holds (pairs in rotation): 32 MiB +3 %, 64 MiB +4.5 %, 128 MiB +6 %.
 FL_LOCAL int fl_stream_mode(int dir, uint64_t bytes);
 // workgroups for a copy over max_tiles tiles: one per tile (the dispatcher then overlaps loads and stores of
 // different tiles); the kernels' stride loops only matter beyond the cap, which grid_per_cu can lower

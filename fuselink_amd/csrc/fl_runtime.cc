@@ -55,11 +55,14 @@ bool fl_use_nt(uint64_t working_set_bytes) {
   return working_set_bytes > kCacheResidentBytes;
 }
 
+int g_stream_force[2] = {-1, -1};   // flh_tune("stream_mode_out" / "stream_mode_in"): -1 = the policy below
+
 int fl_stream_mode(int dir, uint64_t bytes) {
+  if (g_stream_force[dir] >= 0) return dir == 0 ? (g_stream_force[0] == 2 ? 3 : g_stream_force[0]) : (g_stream_force[1] == 1 ? 3 : g_stream_force[1]);
   if (g_nontemporal >= 0) return g_nontemporal ? 3 : 0;
   if (bytes > kWindowsCacheableBytes) return 3;               // the windows no longer fit the Infinity Cache
   if (dir == 0) return bytes >= (128ull << 20) ? 1 : 0;       // read the user buffer once, keep the windows cacheable
-  return bytes >= (80ull << 20) ? 2 : 0;                      // windows come from cache; write the user buffer past the cache once it is large
+  return bytes >= (16ull << 20) ? 2 : 0;                      // windows come from cache; the user buffer is written past it
 }
 
 uint32_t fl_copy_grid(uint64_t max_tiles) {
@@ -146,6 +149,11 @@ int flh_tune(const char* key, int64_t value) {
   if (!strcmp(key, "grid_per_cu")) { if (value < 0) return fl_set_error(FLH_E_ARG, "grid_per_cu < 0"); g_grid_per_cu = (int)value; return FLH_OK; }
   if (!strcmp(key, "stripe_dest_order")) { g_dest_order = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "fused_fast")) { g_fused_fast = value != 0; return FLH_OK; }
+  if (!strcmp(key, "stream_mode_out") || !strcmp(key, "stream_mode_in")) {
+    if (value < -1 || value > 3) return fl_set_error(FLH_E_ARG, "%s not in -1..3", key);
+    g_stream_force[key[12] == 'i'] = (int)value;
+    return FLH_OK;
+  }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }

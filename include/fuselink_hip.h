@@ -110,8 +110,10 @@ const char* flh_last_error(void);
 int64_t flh_constant(int which);
 /* Launch tunables, for experiments (no counterpart in the reference): "grid_per_cu" = copy
  * workgroups launched per compute unit (0 = one per tile), "nontemporal" = 0/1 streaming loads and
- * stores everywhere / nowhere (-1, the default: per side -- user buffers stream once a launch moves 80 to 128 MiB,
+ * stores everywhere / nowhere (-1, the default: per side -- user buffers stream once a launch moves 16 (written side) or 128 MiB (read side),
  * the staging windows stay cacheable until a message passes 256 MiB and they outgrow the Infinity Cache).
+ * "stream_mode_out" / "stream_mode_in" = 0..3 force the mode of the striping / reassembly side (bit 0 loads,
+ * bit 1 stores; -1 = the policy).
  * "stripe_dest_order" = 0/1: flh_stripe_uniform walks the chunks lane by lane, so that every window is written
  * front to back (-1 = only for messages past 256 MiB, whose windows no longer fit the Infinity Cache, the default).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL. */

@@ -523,3 +523,46 @@ def test_batch_refuses_a_request_that_ends_inside_a_chunk(fl):
     b = core.batch_params(srcs, dsts, chunk, [1, 1])
     with pytest.raises(Exception, match="whole number of chunks"):
         core.stripe_batch(b, w, core.new_status())
+
+
+@pytest.mark.parametrize("mode_out,mode_in", [(0, 0), (1, 2), (3, 3), (2, 1)])
+def test_forced_streaming_modes_move_the_same_bytes(fl, mode_out, mode_in):
+    """The cache policy of a launch (which side streams past the caches) selects another instantiation of
+    the copy kernels; every one of them must leave the same windows and the same reassembled buffer."""
+    core, torch = fl
+    rng = np.random.default_rng(9100 + 4 * mode_out + mode_in)
+    lanes, chunk = 6, 40960
+    total = 333 * chunk - 777
+    credits = rng.integers(0, 7, size=lanes).astype(np.uint32)
+    credits[2] = 3
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk)
+    lane_bytes = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+    exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+    src = _dev(torch, src_np)
+    core.tune("stream_mode_out", mode_out)
+    core.tune("stream_mode_in", mode_in)
+    try:
+        for fused in (False, True):
+            wins = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
+            w = core.make_windows([t.data_ptr() for t in wins], lane_bytes)
+            status = core.new_status()
+            dst = torch.zeros_like(src)
+            if fused:
+                u = core.uniform_params(total, chunk, credits.tolist())
+                out = core.new_schedule_buffers(len(exp_t))
+                core.stripe_uniform(src, w, u, status, out=out)
+                core.reassemble_uniform(dst, w, u, status)
+            else:
+                sched = core.schedule(n_lanes=lanes, credits=credits.tolist(), quantum=chunk, total_bytes=total, chunk_bytes=chunk)
+                core.stripe(src, w, sched, status)
+                core.reassemble(dst, w, sched, status)
+            torch.cuda.synchronize()
+            assert int(status.item()) == 0
+            for l in range(lanes):
+                if lane_bytes[l]:
+                    np.testing.assert_array_equal(wins[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"lane {l}")
+            assert torch.equal(src, dst)
+    finally:
+        core.tune("stream_mode_out", -1)
+        core.tune("stream_mode_in", -1)
