@@ -56,7 +56,7 @@ struct Params {
   int window_units = 4;          // staging units bound per lane per connection
   int qps = 1;                   // NCCL_IB_QPS_PER_CONNECTION, plugin.cc:584
   int split_on_qps = 1;          // NCCL_IB_SPLIT_DATA_ON_QPS, plugin.cc:1410
-  int device = 0;
+  int device = -1;               // HIP device that stages; -1 = the one that owns the registered memory
   int idle_credit = 4;
   int max_wave_chunks = 4096;
   int batch = FLH_BATCH_MAX;     // matched sends that may wait for one launch (1 = launch inside isend)
@@ -70,8 +70,18 @@ bool g_credit_override = false;
 uint32_t g_credit_static[FL_NET_MAX_LANES] = {};
 
 std::atomic<int> g_live_links{0};
-flh_pool* g_pool = nullptr;      // staging units of this process's GPU
+std::map<int, flh_pool*> g_pools;   // staging units, one pool per HIP device that has registered memory
 std::mutex g_pool_mu;
+
+// The calling thread's current device is put back when a plugin call that had to switch it returns: the
+// proxy thread that calls in keeps the device its communicator set.
+struct DeviceScope {
+  int saved = -1;
+  DeviceScope() { if (hipGetDevice(&saved) != hipSuccess) saved = -1; }
+  ~DeviceScope() { if (saved >= 0) (void)hipSetDevice(saved); }
+  DeviceScope(const DeviceScope&) = delete;
+  DeviceScope& operator=(const DeviceScope&) = delete;
+};
 
 void parse_credit_env() {
   const char* v = getenv("NCCL_FUSELINK_CREDITS");
@@ -130,6 +140,7 @@ struct FifoSlot {
   FifoWire w;
   Request* rreq;     // loopback only: the receive request this descriptor belongs to
   int rtype;         // pointer type of the receive buffer
+  int rdevice;       // HIP device of the receive buffer (-1: host memory)
 };
 
 // a matched send whose GPU work has not been queued yet
@@ -147,7 +158,7 @@ struct Link {
   int refs = 2;                     // one per side
   int dev = 0;                      // NIC index the comms were opened on
   int channelId = 0;                // plugin.cc:693-708
-  int send_ready = 0;               // comm->ready, plugin.cc:1502
+  int send_ready = 0;               // comm->ready, plugin.cc:1502; -1: the listener closed before accepting
   // sender side
   FifoSlot fifo[FL_NET_MAX_REQUESTS];
   uint64_t fifoHead = 0;            // plugin.cc:1510
@@ -201,6 +212,7 @@ struct MemHandle {             // FuseLinkMemHandle, fuselink.h:48-52
   uintptr_t start_addr = 0;
   size_t size = 0;
   flh_region* region = nullptr;  // shared per base allocation (device memory only)
+  int device = -1;               // HIP device that owns the memory (-1: host memory)
 };
 
 struct Handle {                // what listen writes into the caller's 128 bytes (plugin.cc:425-430)
@@ -235,17 +247,18 @@ void link_unref(Link* lk) {
     last = --lk->refs == 0;
   }
   if (!last) return;
-  if (lk->gpu_ready) {
+  if (lk->stream) {   // the staging side was set up, wholly or in part
+    DeviceScope keep;
     (void)hipSetDevice(lk->hip_device);
     (void)hipStreamSynchronize(lk->stream);
     for (int l = 0; l < FL_NET_MAX_LANES; ++l)
       if (lk->win[l]) (void)flh_window_destroy(lk->win[l]);
-    (void)hipFree(lk->d_table);
-    (void)hipFree(lk->d_hdr);
-    (void)hipHostFree(lk->h_status);
+    if (lk->d_table) (void)hipFree(lk->d_table);
+    if (lk->d_hdr) (void)hipFree(lk->d_hdr);
+    if (lk->h_status) (void)hipHostFree(lk->h_status);
+    for (auto& e : lk->evring) if (e) (void)hipEventDestroy(e);
     (void)hipStreamDestroy(lk->stream);
   }
-  for (auto& e : lk->evring) if (e) (void)hipEventDestroy(e);
   delete lk;
   g_live_links.fetch_sub(1);
 }
@@ -269,26 +282,37 @@ Request* get_request(Request* tab, Link* lk, int type) {
   return nullptr;
 }
 
-ncclResult_t ensure_pool() {
+// The pool of the device (created on first use; creating it makes that device current).
+ncclResult_t ensure_pool(int device, flh_pool** out) {
   std::lock_guard<std::mutex> g(g_pool_mu);
-  if (g_pool) return ncclSuccess;
-  FL_FLHCHECK(flh_pool_create(g_par.device, (uint32_t)g_par.pool_units, &g_pool));
+  auto it = g_pools.find(device);
+  if (it == g_pools.end()) {
+    flh_pool* p = nullptr;
+    FL_FLHCHECK(flh_pool_create(device, (uint32_t)g_par.pool_units, &p));
+    it = g_pools.emplace(device, p).first;
+  }
+  *out = it->second;
   return ncclSuccess;
 }
 
 // Staging side of a connection: stream, one bound window per lane, table / header / state buffers.
-ncclResult_t ensure_link_gpu(Link* lk) {
+// `device` owns the buffer that is being registered or sent; the connection stages on it from then on.
+ncclResult_t ensure_link_gpu(Link* lk, int device) {
   if (lk->gpu_ready) return ncclSuccess;
-  ncclResult_t rc = ensure_pool();
+  if (lk->stream) { FL_WARN("NET/FuseLink : channel %d: the staging side failed to set up earlier", lk->channelId); return ncclInternalError; }
+  if (device < 0) { FL_WARN("NET/FuseLink : no HIP device to stage on"); return ncclInternalError; }
+  DeviceScope keep;
+  flh_pool* pool = nullptr;
+  ncclResult_t rc = ensure_pool(device, &pool);
   if (rc != ncclSuccess) return rc;
-  lk->hip_device = g_par.device;
+  lk->hip_device = device;
   FL_HIPCHECK(hipSetDevice(lk->hip_device));
   FL_HIPCHECK(hipStreamCreateWithFlags(&lk->stream, hipStreamNonBlocking));
   const uint64_t cap = (uint64_t)g_par.window_units * FLH_UNIT_BYTES;
   memset(&lk->wins, 0, sizeof(lk->wins));
   lk->wins.n_lanes = (uint32_t)g_par.lanes;
   for (int l = 0; l < g_par.lanes; ++l) {
-    FL_FLHCHECK(flh_window_create(g_pool, cap, &lk->win[l]));
+    FL_FLHCHECK(flh_window_create(pool, cap, &lk->win[l]));
     FL_FLHCHECK(flh_window_bind(lk->win[l], cap));
     lk->wins.base[l] = flh_window_base(lk->win[l]);
     lk->wins.cap[l] = flh_window_bound_bytes(lk->win[l]);
@@ -444,9 +468,18 @@ ncclResult_t fl_connect(int dev, void* opaqueHandle, void** sendComm, ncclNetDev
     return ncclSuccess;
   }
   Link* lk = (Link*)h->stage_link;
+  int ready;
   {
     std::lock_guard<std::mutex> g(lk->mu);
-    if (!lk->send_ready) return ncclSuccess;  // accept has not happened yet
+    ready = lk->send_ready;
+  }
+  if (ready == 0) return ncclSuccess;  // accept has not happened yet
+  if (ready < 0) {                     // the listener went away before it accepted
+    h->stage = 0;
+    h->stage_link = nullptr;
+    link_unref(lk);
+    FL_WARN("NET/FuseLink : connect: the listen comm was closed before it accepted");
+    return ncclSystemError;
   }
   Comm* c = new (std::nothrow) Comm();
   if (!c) return ncclSystemError;
@@ -493,20 +526,26 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
     // whole allocation around the pointer, as cuMemGetAddressRange in plugin.cc:1194
     void* base = nullptr;
     size_t bsz = 0;
-    hipError_t e = hipSetDevice(g_par.device);
+    DeviceScope keep;
+    hipPointerAttribute_t attr;
+    hipError_t e = hipPointerGetAttributes(&attr, data);
+    if (e != hipSuccess) { delete mh; return hip_fail("hipPointerGetAttributes", e); }
+    mh->device = g_par.device >= 0 ? g_par.device : attr.device;
+    e = hipSetDevice(mh->device);
     if (e != hipSuccess) { delete mh; return hip_fail("hipSetDevice", e); }
     e = hipMemGetAddressRange((hipDeviceptr_t*)&base, &bsz, (hipDeviceptr_t)data);
     if (e != hipSuccess) { delete mh; return hip_fail("hipMemGetAddressRange", e); }
-    ncclResult_t rc = ensure_pool();
+    flh_pool* pool = nullptr;
+    ncclResult_t rc = ensure_pool(mh->device, &pool);
     if (rc != ncclSuccess) { delete mh; return rc; }
     // one shared, reference-counted region per base allocation (plugin.cc:1212-1227, 1326)
-    int frc = flh_region_acquire(g_pool, base, bsz, 0, 0, &mh->region);
+    int frc = flh_region_acquire(pool, base, bsz, 0, 0, &mh->region);
     if (frc < 0) { delete mh; FL_WARN("NET/FuseLink : region: %s", flh_last_error()); return ncclInternalError; }
     mh->start_addr = (uintptr_t)base;
     mh->size = bsz;
     if (c->is_send) {  // staging is bound at registration time, not on the request path
       std::lock_guard<std::mutex> g(c->link->mu);
-      rc = ensure_link_gpu(c->link);
+      rc = ensure_link_gpu(c->link, mh->device);
       if (rc != ncclSuccess) { (void)flh_region_release(mh->region); delete mh; return rc; }
     }
   } else if (type == NCCL_PTR_HOST) {
@@ -659,6 +698,7 @@ size_t batch_span(const Link* lk, size_t i) {
 // it touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).
 void flush_pending(Link* lk) {
   if (lk->pending.empty()) return;
+  DeviceScope keep;
   bool dev_ok = hipSetDevice(lk->hip_device) == hipSuccess;
   size_t i = 0;
   while (i < lk->pending.size()) {
@@ -715,7 +755,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
   ncclResult_t rc = ncclSuccess;
   {
     std::lock_guard<std::mutex> g(lk->mu);
-    if (!lk->send_ready) { FL_WARN("NET/FuseLink: isend() called when comm->ready == 0"); return ncclInternalError; }  // plugin.cc:1502
+    if (lk->send_ready <= 0) { FL_WARN("NET/FuseLink: isend() called when comm->ready == 0"); return ncclInternalError; }  // plugin.cc:1502
     // wait for the receiver to have posted the matching receive (plugin.cc:1510-1514)
     const int slot = (int)(lk->fifoHead % FL_NET_MAX_REQUESTS);
     FifoSlot& fs = lk->fifo[slot];
@@ -739,7 +779,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     sreq->size = size;
     rreq->size = size;
     const bool any_dev = mh->type == NCCL_PTR_CUDA || rtype == NCCL_PTR_CUDA;
-    if (size && any_dev) rc = ensure_link_gpu(lk);
+    if (size && any_dev) rc = ensure_link_gpu(lk, mh->type == NCCL_PTR_CUDA ? mh->device : fs.rdevice);
     if (rc != ncclSuccess) { sreq->type = kReqUnused; return rc; }   // nothing consumed: the descriptor stays posted
     memset((void*)&fs.w, 0, sizeof(FifoWire));   // plugin.cc:1605
     fs.rreq = nullptr;
@@ -819,6 +859,7 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
   fs.w.flags = refreshed ? 1u : 0u;
   fs.rreq = rreq;
   fs.rtype = mh->type;
+  fs.rdevice = mh->device;
   fs.w.idx = lk->fifoTail + 1;   // written last: it is what the sender waits for (plugin.cc:1632)
   lk->fifoTail++;
   lk->r_inflight++;
@@ -897,7 +938,11 @@ ncclResult_t fl_close_listen(void* listenComm) {
     g_listens.erase(lc->id);
     orphans.assign(lc->pending.begin(), lc->pending.end());
   }
-  for (Link* lk : orphans) {   // connects nobody will accept: drop the listener's share of them
+  for (Link* lk : orphans) {   // connects nobody will accept: tell the connecting side, drop the listener's share
+    {
+      std::lock_guard<std::mutex> g(lk->mu);
+      lk->send_ready = -1;
+    }
     link_unref(lk);
   }
   delete lc;
@@ -965,10 +1010,9 @@ int fl_net_reset(void) {
   }
   {
     std::lock_guard<std::mutex> g(g_pool_mu);
-    if (g_pool) {
-      int rc = flh_pool_destroy(g_pool);
+    for (auto it = g_pools.begin(); it != g_pools.end(); it = g_pools.erase(it)) {
+      int rc = flh_pool_destroy(it->second);
       if (rc < 0) return rc;
-      g_pool = nullptr;
     }
   }
   g_par = Params();
@@ -1014,6 +1058,7 @@ int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_ou
   if (!lk->gpu_ready) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
   std::lock_guard<std::mutex> gl(lk->launch_mu);
   flush_pending(lk);
+  DeviceScope keep;
   if (hipSetDevice(lk->hip_device) != hipSuccess || hipStreamSynchronize(lk->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
   int rows = (int)lk->last_wave_rows.load();
   int take = rows < max_rows ? rows : max_rows;

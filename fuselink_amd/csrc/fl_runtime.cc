@@ -44,7 +44,9 @@ int fl_set_error(int code, const char* fmt, ...) {
 
 int fl_need_init() {
   if (g_device < 0) {
-    int rc = flh_init((int)env_i64("NCCL_FUSELINK_DEVICE", 0));
+    int device = (int)env_i64("NCCL_FUSELINK_DEVICE", -1);
+    if (device < 0 && hipGetDevice(&device) != hipSuccess) device = 0;   // unset: the caller's current device
+    int rc = flh_init(device);
     if (rc) return rc;
   }
   return FLH_OK;

@@ -89,6 +89,19 @@ def test_connect_accept_are_nonblocking_and_staged(net):
     assert net.closeSend(s) == 0 and net.closeRecv(r) == 0 and net.closeListen(lcomm) == 0
 
 
+def test_connect_learns_that_its_listener_closed(net):
+    # a connect that was posted but never accepted: closing the listen comm must not leave the connecting
+    # side polling for ever, and the connection's memory is released (reset refuses while a link is alive)
+    rc, handle, lcomm = net.listen(0)
+    rc, s = net.connect(0, handle)
+    assert rc == P.ncclSuccess and s is None
+    assert net.closeListen(lcomm) == 0
+    rc, s = net.connect(0, handle)
+    assert rc == P.ncclSystemError and s is None
+    assert net.lib.fl_net_reset() == 0
+    assert net.init() == 0
+
+
 def test_channel_ids_count_up_per_listen(net):
     # ncclIbListen hands out a global, increasing channelId (src/plugin.cc:693-708); it sits in the handle
     ids = []
