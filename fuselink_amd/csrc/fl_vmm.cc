@@ -62,7 +62,7 @@ namespace {
 std::mutex g_region_mu;                      // addr2flmr_lock of src/plugin.cc:34
 std::map<void*, flh_region*> g_regions;      // addr2flmr of src/plugin.cc:33
 
-int64_t cached_param(const char* name, int64_t dflt) {
+int64_t env_param(const char* name, int64_t dflt) {
   const char* v = getenv(name);
   if (!v || !*v) return dflt;
   char* end = nullptr;
@@ -74,7 +74,7 @@ int64_t cached_param(const char* name, int64_t dflt) {
 int64_t fl_param(const char* env_suffix, int64_t dflt) {
   char name[128];
   snprintf(name, sizeof(name), "NCCL_%s", env_suffix);
-  return cached_param(name, dflt);
+  return env_param(name, dflt);
 }
 
 extern "C" {

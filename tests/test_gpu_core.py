@@ -566,3 +566,53 @@ def test_forced_streaming_modes_move_the_same_bytes(fl, mode_out, mode_in):
     finally:
         core.tune("stream_mode_out", -1)
         core.tune("stream_mode_in", -1)
+
+
+def test_launches_record_into_a_hip_graph_and_replay(fl):
+    """No entry point on the data path allocates, clears or synchronizes, so a caller may record
+    schedule -> stripe -> reassemble into a HIP graph.  Every replay, with eager work and synchronizations of
+    the program's own in between, must give what the eager launches give for the source bytes of that moment."""
+    core, torch = fl
+    rng = np.random.default_rng(31337)
+    lanes, chunk = 8, 65536
+    total = 300 * chunk - 4097
+    credits = rng.integers(1, 9, size=lanes).astype(np.uint32)
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk)
+    lane_bytes = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    src = torch.zeros(total, dtype=torch.uint8, device="cuda")
+    dst_fused, dst_table = torch.zeros_like(src), torch.zeros_like(src)
+    wins = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
+    w = core.make_windows([t.data_ptr() for t in wins], lane_bytes)
+    u = core.uniform_params(total, chunk, credits.tolist())
+    out = core.new_schedule_buffers(len(exp_t))
+    sched_out = core.new_schedule_buffers(len(exp_t))
+    d_credits = _dev(torch, credits.view(np.int32))
+    status = core.new_status()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        # fused pair, then the three-launch path over the same windows into a second destination
+        core.stripe_uniform(src, w, u, status, out=out)
+        core.reassemble_uniform(dst_fused, w, u, status)
+        sched = core.schedule(n_lanes=lanes, credits=d_credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk, out=sched_out)
+        core.stripe(src, w, sched, status)
+        core.reassemble(dst_table, w, sched, status)
+    for rep in range(4):
+        src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+        src.copy_(torch.from_numpy(src_np))
+        dst_fused.zero_()
+        dst_table.zero_()
+        for t in wins:
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+        assert torch.equal(dst_fused, src) and torch.equal(dst_table, src), f"replay {rep}"
+        exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+        for l in range(lanes):
+            np.testing.assert_array_equal(wins[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"replay {rep} lane {l}")
+        for f in ob.DESC_DTYPE.names:
+            np.testing.assert_array_equal(out.table_numpy()[f], exp_t[f], err_msg=f"replay {rep} field {f}")
+            np.testing.assert_array_equal(sched_out.table_numpy()[f], exp_t[f], err_msg=f"replay {rep} field {f} (scheduler kernel)")
