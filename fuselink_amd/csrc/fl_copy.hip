@@ -125,6 +125,7 @@ __device__ __forceinline__ uint32_t find_row(const flh_chunk_desc* __restrict__ 
 // DIR 0: user -> windows (stripe).  DIR 1: windows -> user (reassemble).
 template <int DIR, int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
+  warm_kernel_args(a);
   const uint32_t total = a.has_hint ? a.hint_total_tiles : a.hdr->total_tiles;
   const uint32_t uniform_tiles = a.has_hint ? a.hint_uniform_tiles : a.hdr->uniform_tiles;
   uint32_t n = a.has_hint ? a.hint_n_chunks : a.hdr->n_chunks;
@@ -154,6 +155,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
 // load of its table row.
 template <int DIR, int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform(CopyArgs a) {
+  warm_kernel_args(a);
   const uint32_t c = blockIdx.y;
   if (c >= a.hint_n_chunks) return;
   const flh_chunk_desc d = a.table[c];
@@ -196,9 +198,12 @@ struct FusedArgs {
   // Worked out once on the host when every quantum index and the credit sum W fit 32 bits: the per-workgroup
   // division by W becomes one multiply-high by magic = ceil(2^64 / W) (exact for 32-bit operands), and the
   // lane's slots before the message come from cnt0[] instead of a second and third division.
+  // The lane of a slot is then found by a four-step binary search over pfx_ex[] (exclusive credit prefixes,
+  // W from index n_lanes on), read straight from the argument block.
   uint32_t fast;
   uint64_t magic;
   uint32_t cnt0[FLH_MAX_LANES];
+  uint32_t pfx_ex[FLH_MAX_LANES + 1];
 };
 
 // Several requests as one message: chunk c belongs to the request r with first[r] <= c < first[r+1];
@@ -243,12 +248,14 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
 template <int DIR, int NT, class Args>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   constexpr bool BATCH = is_batch<Args>::value;
+  warm_kernel_args(a);
   if (blockIdx.y >= a.n_chunks) return;
-  FusedRow r;
-  fused_row(a, r);
   uint32_t c = blockIdx.y, lane = 0;
-  uint64_t K = 0, hi = r.pfx[0], before;
+  uint64_t before;
   if (DIR == 0 && a.dest_order) {
+    FusedRow r;
+    fused_row(a, r);
+    uint64_t K = 0, hi = r.pfx[0];
     // blockIdx.y = k-th chunk in destination order: find the lane whose group holds k, then invert the
     // closed form -- the j-th slot of a lane with credit c_l and first slot K_l is (j / c_l) * W + K_l + j mod c_l.
     const uint64_t x0 = a.quanta_before, x1 = a.quanta_before + a.n_chunks;
@@ -277,14 +284,19 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   } else if (a.fast) {
     const uint32_t j = (uint32_t)a.quanta_before + c;
     const uint32_t full = (uint32_t)__umul64hi((uint64_t)j, a.magic);  // j / W
-    const uint32_t slot = j - full * (uint32_t)r.W;
-    uint32_t c0 = a.cnt0[0];
-#pragma unroll
-    for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
-      if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; c0 = a.cnt0[l + 1]; }
-    }
+    const uint32_t slot = j - full * a.pfx_ex[FLH_MAX_LANES];  // the last entry is always W
+    // the last lane whose first slot is not beyond this one (lanes without credit share their successor's first slot)
+    static_assert(FLH_MAX_LANES == 16, "the search below takes four steps");
+    if (a.pfx_ex[lane + 8] <= slot) lane += 8;
+    if (a.pfx_ex[lane + 4] <= slot) lane += 4;
+    if (a.pfx_ex[lane + 2] <= slot) lane += 2;
+    if (a.pfx_ex[lane + 1] <= slot) lane += 1;
+    const uint32_t K = a.pfx_ex[lane], hi = a.pfx_ex[lane + 1], c0 = a.cnt0[lane];   // indexed scalar loads from the argument block
     before = (uint64_t)full * (hi - K) + (slot - K) - c0;  // slot lies inside the lane's span [K, hi)
   } else {
+    FusedRow r;
+    fused_row(a, r);
+    uint64_t K = 0, hi = r.pfx[0];
     const uint64_t j = a.quanta_before + c;
     const uint64_t slot = mod_u64(j, r.W);
 #pragma unroll
@@ -323,6 +335,8 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
     a.table[c] = d;
   }
   if (DIR == 0 && blockIdx.x == 0 && blockIdx.y == 0 && a.hdr) {  // header: per-lane totals in closed form
+    FusedRow r;
+    fused_row(a, r);
     const uint32_t t = threadIdx.x;
     const uint64_t last = a.n_chunks - 1;
     const uint64_t len_last = a.total_bytes - last * a.chunk_bytes;
@@ -385,6 +399,7 @@ constexpr uint32_t kLdsStage = 16384;
 template <int DIR, int NT, bool LDS>
 __global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
   __shared__ u32x4 stage[LDS ? kLdsStage / 16 : 1];
+  warm_kernel_args(a);
   const uint64_t total = (uint64_t)a.n_chunks * a.pages_per_chunk * a.subs_per_page;
   for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
     const uint32_t sub = (uint32_t)(t % a.subs_per_page);
@@ -563,6 +578,7 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
     a.fast = W >= 2 && W <= 0xffffffffull && a.quanta_before + n <= 0xffffffffull && g_fused_fast;
     a.magic = a.fast ? ~0ull / W + 1 : 0;
     for (int l = 0; l < FLH_MAX_LANES; ++l) a.cnt0[l] = 0;
+    for (int l = 0; l <= FLH_MAX_LANES; ++l) a.pfx_ex[l] = l == 0 ? 0 : (uint32_t)((uint32_t)l <= u->n_lanes ? pfx[l - 1] : W);
     if (a.fast) {
       const uint64_t full = a.quanta_before / W, rem = a.quanta_before % W;
       for (uint32_t l = 0; l < u->n_lanes; ++l) {

@@ -107,6 +107,20 @@ __device__ __forceinline__ uint64_t mod_u64(uint64_t a, uint64_t b) {
   return ((a | b) >> 32) == 0 ? (uint64_t)((uint32_t)a % (uint32_t)b) : a - div_u64_wide(a, b) * b;
 }
 
+// A kernel's argument block is read with scalar loads, and the compiler places each load next to its first use:
+// behind every branch waits another round trip to memory that the host wrote a moment ago and no cache holds
+// yet.  Reading one word of every 64-byte line of the block first, all in flight together, turns that chain
+// of misses into one miss plus scalar-cache hits.
+template <class Args>
+__device__ __forceinline__ void warm_kernel_args(const Args& a) {
+  const uint32_t* p = reinterpret_cast<const uint32_t*>(&a);
+  constexpr int kDwords = (int)(sizeof(Args) / 4);
+  uint32_t z = p[kDwords - 1];
+#pragma unroll
+  for (int i = 0; i < kDwords; i += 16) z |= p[i];
+  asm volatile("" ::"s"(z));
+}
+
 }  // namespace
 
 #endif  // FL_DEVICE_H_

@@ -154,6 +154,7 @@ __device__ __forceinline__ void lane_pass_columns(const uint32_t (&s)[K], const 
 // for the window offsets.  LDS only carries per-wavefront totals and the running lane offsets.
 template <int NW, int K>
 __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
+  warm_kernel_args(a);
   constexpr int BT = NW * kWave;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -513,6 +514,7 @@ constexpr int kUniBlock = 256;
 //         can still be reading the old state).
 template <int MODE>
 __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArgs a) {
+  warm_kernel_args(a);
   __shared__ UniTables t;
   const int tid = threadIdx.x;
   const uint32_t L = a.n_lanes, R = a.n_rows;
