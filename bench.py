@@ -58,6 +58,8 @@ def main() -> int:
     ap.add_argument("--cold-user-buffers", action="store_true",
                     help="also time the step over source/destination pairs in rotation (1 GiB), so that no user buffer is "
                          "cache-resident; off by default so that a kernel trace of the default run holds the timed loop's launches only")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="set a library tunable (flh_tune) before the run, e.g. --tune copy_rows_per_wg=1; repeatable")
     ap.add_argument("--no-by-lane", action="store_true", help="stripe large messages in chunk order instead of destination order")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -74,6 +76,9 @@ def main() -> int:
         print("bench.py: no GPU visible; there is no CPU fallback for the measured path", file=sys.stderr)
         return 3
     core.init(0)
+    for kv in args.tune:
+        key, _, val = kv.partition("=")
+        core.tune(key, int(val))
     dev = torch.device("cuda:0")
     kind, nbytes, chunk, lanes, rows, epoch_len = WORKLOADS[args.workload]
     rng = np.random.default_rng(20251125)
