@@ -400,12 +400,11 @@ template <int DIR, int NT, bool LDS>
 __global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
   __shared__ u32x4 stage[LDS ? kLdsStage / 16 : 1];
   warm_kernel_args(a);
-  const uint64_t total = (uint64_t)a.n_chunks * a.pages_per_chunk * a.subs_per_page;
-  for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
-    const uint32_t sub = (uint32_t)(t % a.subs_per_page);
-    const uint64_t rp = t / a.subs_per_page;         // row-major page counter
-    const uint32_t c = (uint32_t)(rp / a.pages_per_chunk);
-    const uint32_t k = (uint32_t)(rp % a.pages_per_chunk);
+  // grid: x = (page in chunk, part of page), y = chunk (stepping by the grid's height past 65535 chunks); no
+  // 64-bit division stands between a workgroup and its row
+  const uint32_t k = a.subs_per_page == 1 ? blockIdx.x : blockIdx.x / a.subs_per_page;
+  const uint32_t sub = blockIdx.x - k * a.subs_per_page;
+  for (uint32_t c = blockIdx.y; c < a.n_chunks; c += gridDim.y) {
     const flh_chunk_desc d = a.table[c];
     const uint64_t in_chunk = (uint64_t)k * a.page_bytes + (uint64_t)sub * a.sub_bytes;
     if (in_chunk >= d.len) continue;
@@ -688,11 +687,11 @@ static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t
   a.sub_bytes = page_bytes < sub ? page_bytes : sub;
   a.subs_per_page = (page_bytes + a.sub_bytes - 1) / a.sub_bytes;
   a.page_shift = (page_bytes & (page_bytes - 1)) == 0 ? __builtin_ctz(page_bytes) : -1;
-  const uint64_t total = (uint64_t)n_chunks * pages_per_chunk * a.subs_per_page;
-  const uint32_t grid = fl_copy_grid(total);
+  const uint64_t per_chunk = (uint64_t)pages_per_chunk * a.subs_per_page;
+  if (per_chunk > 0x7fffffffull) return fl_set_error(FLH_E_ARG, "pages_per_chunk %u is too large for one launch", pages_per_chunk);
   hipStream_t s = (hipStream_t)stream;
   const int mode = fl_stream_mode(dir, (uint64_t)n_chunks * pages_per_chunk * page_bytes);
-  const dim3 grid3(grid);
+  const dim3 grid3((uint32_t)per_chunk, n_chunks < 65535 ? n_chunks : 65535);
 #define FL_LDS_ON , true
 #define FL_LDS_OFF , false
   if (use_lds) FL_LAUNCH_COPY(fl_page_tiles, FL_LDS_ON, dir, mode, grid3, s, a);

@@ -246,6 +246,32 @@ def test_cfg4_paged_kv_gather(fl, use_lds, by_lane):
             np.testing.assert_array_equal(wins[l].cpu().numpy()[: caps[l]], exp_w[l][: caps[l]])
 
 
+def test_paged_gather_with_more_chunks_than_the_grid_is_tall(fl):
+    """70 000 one-page chunks: the page kernels' grid is at most 65 535 chunks tall and steps over the rest."""
+    core, torch = fl
+    rng = np.random.default_rng(15)
+    n_pages, page, ppc = 70000, 256, 1
+    total = n_pages * page
+    pool = torch.randint(0, 255, (total,), dtype=torch.uint8, device="cuda")
+    table_np = rng.permutation(n_pages).astype(np.uint32)
+    credits = np.array([2, 1, 3, 1], dtype=np.uint32)
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=4, credits=credits, quantum=page, total_bytes=total, chunk_bytes=page)
+    sched = core.schedule(n_lanes=4, credits=credits.tolist(), quantum=page, total_bytes=total, chunk_bytes=page)
+    caps = [int(b) for b in exp_h["lane_bytes"][:4]]
+    wins = [torch.zeros(c, dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    table = _dev(torch, table_np.view(np.int32))
+    core.gather_pages(pool, table, page, ppc, w, sched, status)
+    out = torch.zeros_like(pool)
+    core.scatter_pages(out, table, page, ppc, w, sched, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0 and torch.equal(out, pool)
+    exp_w = ob.cpu_gather_pages(pool.cpu().numpy(), table_np, page, ppc, exp_t, caps)
+    for l in range(4):
+        np.testing.assert_array_equal(wins[l].cpu().numpy()[: caps[l]], exp_w[l][: caps[l]])
+
+
 def test_paged_gather_ragged_and_bad_page(fl):
     core, torch = fl
     rng = np.random.default_rng(14)
