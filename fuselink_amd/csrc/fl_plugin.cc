@@ -112,6 +112,7 @@ struct Request {
   std::atomic<int> state{0};
   Link* link = nullptr;
   hipEvent_t ev = nullptr;   // completion of the launch that carries this request (owned by the connection's ring)
+  uint64_t seq = 0;          // number of that launch on its connection, counted from 1
   int size = 0;          // bytes moved (reported by test for receives)
   int fault = 0;         // injected wire fault
   uint32_t magic = 0;
@@ -189,6 +190,11 @@ struct Link {
   std::vector<Pending> pending;
   hipEvent_t evring[FL_NET_MAX_REQUESTS] = {};   // at most that many requests, hence launches, are in flight
   uint32_t ev_next = 0;
+  // Highest launch number seen complete.  The connection's launches run in order on one stream, so a request of an
+  // earlier launch is complete too and its test needs no event query (requests that shared a launch, and the
+  // receive side of a send that was already tested, cost no call into the runtime).
+  std::atomic<uint64_t> done_seq{0};
+  uint64_t launch_seq = 0;
   int64_t launches = 0, batched_requests = 0;    // launch pairs made, requests that shared one
 };
 
@@ -272,6 +278,7 @@ Request* get_request(Request* tab, Link* lk, int type) {
       r->link = lk;
       r->size = 0;
       r->ev = nullptr;
+      r->seq = 0;
       r->fault = 0;
       r->magic = kReqMagic;
       r->state.store(0, std::memory_order_relaxed);
@@ -724,6 +731,8 @@ void flush_pending(Link* lk) {
       if (rc == ncclSuccess) {
         p.sreq->ev = ev;
         p.rreq->ev = ev;
+        p.sreq->seq = lk->launch_seq + 1;
+        p.rreq->seq = lk->launch_seq + 1;
         p.sreq->state.store(kStLaunched, std::memory_order_release);
         p.rreq->state.store(kStLaunched, std::memory_order_release);
       } else {
@@ -733,7 +742,7 @@ void flush_pending(Link* lk) {
         p.rreq->state.store(kStDoneHost, std::memory_order_release);
       }
     }
-    if (rc == ncclSuccess) lk->ev_next++;
+    if (rc == ncclSuccess) { lk->ev_next++; lk->launch_seq++; }
     i += span;
   }
   lk->pending.clear();
@@ -891,9 +900,13 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     st = r->state.load(std::memory_order_acquire);
   }
   if (st == kStLaunched) {
-    hipError_t e = hipEventQuery(r->ev);
-    if (e == hipErrorNotReady) return ncclSuccess;
-    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+    if (r->seq > lk->done_seq.load(std::memory_order_acquire)) {
+      hipError_t e = hipEventQuery(r->ev);
+      if (e == hipErrorNotReady) return ncclSuccess;
+      if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+      uint64_t seen = lk->done_seq.load(std::memory_order_relaxed);
+      while (seen < r->seq && !lk->done_seq.compare_exchange_weak(seen, r->seq, std::memory_order_release, std::memory_order_relaxed)) {}
+    }
     if (lk->h_status && *(volatile int32_t*)lk->h_status != 0) {
       FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", *lk->h_status);
       return ncclInternalError;
