@@ -36,7 +36,7 @@ WORKLOADS = {
 # WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size.
 # None where no such run has been recorded for the workload.
 MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134289278, "cfg5_stress_1GiB_64KiB_16lanes": 2151685750,
-                    "cfg3_expert_parallel_256_blocks_8lanes": 1786051408, "cfg4_paged_kv_2x4096_pages_8lanes": 268868847}
+                    "cfg3_expert_parallel_256_blocks_8lanes": 1786051408, "cfg4_paged_kv_2x4096_pages_8lanes": 268854570}
 
 
 def algo_bytes_cold(nbytes: int) -> int:
