@@ -36,7 +36,7 @@ WORKLOADS = {
 # WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size.
 # None where no such run has been recorded for the workload.
 MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134289278, "cfg5_stress_1GiB_64KiB_16lanes": 2151685750,
-                    "cfg3_expert_parallel_256_blocks_8lanes": 1786051408, "cfg4_paged_kv_2x4096_pages_8lanes": 268854570}
+                    "cfg3_expert_parallel_256_blocks_8lanes": 1786051408, "cfg4_paged_kv_2x4096_pages_8lanes": 268684250}
 
 
 def algo_bytes_cold(nbytes: int) -> int:
@@ -144,14 +144,19 @@ def main() -> int:
 
     # header fields that follow from the uniform split alone; the kernels then need not wait for d_hdr
     hint = core.uniform_hint(msg_bytes, chunk) if (args.hint and kind == "uniform") else None
-    fused = kind == "uniform" and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and n_chunks <= 65535))
+    fused = kind in ("uniform", "pages") and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
     if fused and (rows != 1 or epoch_len != 0):
         print("bench.py: the fused path takes a single credit row without epochs", file=sys.stderr)
         return 2
-    uni = core.uniform_params(nbytes, chunk, credits_np[0].tolist()) if fused else None
+    uni = core.uniform_params(msg_bytes, chunk, credits_np[0].tolist()) if fused else None
 
     def step():
-        if kind == "pages":
+        if kind == "pages" and fused:
+            for half_i in range(2):   # K, then V; the gather works each chunk's lane and offset out itself and writes the table
+                lo = half_i * msg_bytes
+                core.gather_pages_uniform(src[lo: lo + msg_bytes], tables[half_i], page_bytes, win, uni, status, out=sched, stream=stream)
+                core.scatter_pages_uniform(dst[lo: lo + msg_bytes], tables[half_i], page_bytes, win, uni, status, stream=stream)
+        elif kind == "pages":
             for half_i in range(2):   # K, then V: schedule, gather the pages into the windows, scatter them back out
                 run_schedule(sched)
                 lo = half_i * msg_bytes
@@ -225,7 +230,7 @@ def main() -> int:
     # (1 GiB of user buffers) every step meets them cold, as a stream of distinct messages would.  Reported
     # beside `value`, never as `value`.
     cold = None
-    if args.cold_user_buffers and fused and nbytes <= (128 << 20):
+    if args.cold_user_buffers and fused and kind == "uniform" and nbytes <= (128 << 20):
         pairs = max(2, (1 << 30) // (2 * nbytes))
         srcs = [src] + [torch.randint(0, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device=dev, generator=gen).view(torch.uint8)
                         for _ in range(pairs - 1)]
@@ -256,7 +261,9 @@ def main() -> int:
     value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
     pair_us = (stripe_us + reasm_us) * launches_per_step
     achieved = algo_bytes_kernel / (stripe_us * 1e-6) / 1e9
-    if kind == "pages":
+    if kind == "pages" and fused:
+        kernel_name = "fl_copy_uniform_fused<0, FusedPageArgs> (gather)"
+    elif kind == "pages":
         kernel_name = f"fl_page_tiles<0, lds={args.lds}> (gather)"
     elif fused:
         kernel_name = "fl_copy_uniform_fused<0> (stripe)"
@@ -283,7 +290,7 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": args.workload, "bytes": nbytes, "chunk_bytes": chunk if sizes is None else "variable", "chunks": n_chunks,
                    "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
-                   "step": ("2x(schedule+gather+scatter)" if kind == "pages" else
+                   "step": ("2x(gather(with scheduler folded in)+scatter)" if (kind == "pages" and fused) else "2x(schedule+gather+scatter)" if kind == "pages" else
                             "stripe(with scheduler folded in)+reassemble" if fused else "schedule+stripe+reassemble"),
                    "launch": "eager", "windows": "HIP VMM, 2 MiB units",
                    "stripe_order": "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel for messages past 256 MiB)" if fused else "chunk"},

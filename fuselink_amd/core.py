@@ -258,6 +258,22 @@ def scatter_pages(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int,
                                         _stream_ptr(stream)))
 
 
+def gather_pages_uniform(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int, win: Windows, u: UniformParams,
+                         status: torch.Tensor, out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None) -> None:
+    """Scheduler + page gather in one launch (flh_gather_pages_uniform); `out` receives the table and header."""
+    nbytes = pool.numel() * pool.element_size()
+    check(_lib.load().flh_gather_pages_uniform(_ptr(pool), nbytes // page_bytes, _ptr(page_table), page_bytes, C.byref(win), C.byref(u),
+                                               _ptr(out.table) if out else None, _ptr(out.hdr) if out else None, _ptr(status),
+                                               _stream_ptr(stream)))
+
+
+def scatter_pages_uniform(pool: torch.Tensor, page_table: torch.Tensor, page_bytes: int, win: Windows, u: UniformParams,
+                          status: torch.Tensor, stream: Optional[torch.cuda.Stream] = None) -> None:
+    nbytes = pool.numel() * pool.element_size()
+    check(_lib.load().flh_scatter_pages_uniform(_ptr(pool), nbytes // page_bytes, _ptr(page_table), page_bytes, C.byref(win), C.byref(u),
+                                                _ptr(status), _stream_ptr(stream)))
+
+
 def copy(dst: torch.Tensor, src: torch.Tensor, stream: Optional[torch.cuda.Stream] = None) -> None:
     nbytes = src.numel() * src.element_size()
     assert dst.numel() * dst.element_size() >= nbytes

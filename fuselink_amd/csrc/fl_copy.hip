@@ -217,6 +217,18 @@ struct FusedBatchArgs : FusedArgs {
 template <class A> struct is_batch { static constexpr bool value = false; };
 template <> struct is_batch<FusedBatchArgs> { static constexpr bool value = true; };
 
+// The message lives in pages of a pool: byte b of it is byte b mod page_bytes of pool page
+// page_table[b / page_bytes].  `user` is the pool; a tile never straddles a page (tile_bytes divides page_bytes).
+struct FusedPageArgs : FusedArgs {
+  const uint32_t* page_table;
+  uint64_t pool_pages;
+  uint64_t n_pages;        // entries of page_table the message covers
+  uint32_t page_bytes;
+  int32_t page_shift;      // >= 0 when page_bytes is a power of two
+};
+template <class A> struct is_paged { static constexpr bool value = false; };
+template <> struct is_paged<FusedPageArgs> { static constexpr bool value = true; };
+
 struct FusedRow {  // inclusive credit prefixes of the one row (equal credits if it is empty)
   uint64_t pfx[FLH_MAX_LANES];
   uint64_t W;
@@ -248,6 +260,7 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
 template <int DIR, int NT, class Args>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   constexpr bool BATCH = is_batch<Args>::value;
+  constexpr bool PAGED = is_paged<Args>::value;
   warm_kernel_args(a);
   if (blockIdx.y >= a.n_chunks) return;
   uint32_t c = blockIdx.y, lane = 0;
@@ -368,11 +381,21 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
   if (off >= len) return;
   const uint32_t bytes = (uint32_t)((len - off) < a.tile_bytes ? (len - off) : a.tile_bytes);
-  if (win_off + len > a.win.cap[lane] || user_off + len > user_bytes) {
+  if (win_off + len > a.win.cap[lane] || (!PAGED && user_off + len > user_bytes)) {
     if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
     return;
   }
   uint8_t* u = user + user_off + off;
+  if constexpr (PAGED) {
+    const uint64_t at = src_off + off;   // the tile's first byte in the message
+    const uint64_t pi = a.page_shift >= 0 ? at >> a.page_shift : at / a.page_bytes;
+    const uint32_t pg = pi < a.n_pages ? a.page_table[pi] : 0xffffffffu;
+    if (pg >= a.pool_pages) {
+      if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+      return;
+    }
+    u = user + (uint64_t)pg * a.page_bytes + (at - pi * a.page_bytes);
+  }
   uint8_t* w = (uint8_t*)a.win.base[lane] + win_off + off;
   if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
 }
@@ -640,6 +663,37 @@ static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* w
   }
   if (sum != b->u.total_bytes) return fl_set_error(FLH_E_ARG, "the requests hold %llu bytes, the parameters say %llu", (unsigned long long)sum, (unsigned long long)b->u.total_bytes);
   return launch_fused_args(dir, a, fl_stream_mode(dir, sum), stream);
+}
+
+static int launch_fused_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                              const flh_windows* win, const flh_uniform_params* u, flh_chunk_desc* d_table, flh_sched_hdr* d_hdr,
+                              int32_t* d_status, void* stream) {
+  FusedPageArgs a;
+  const int rc = fill_fused(a, dir, win, u, d_table, d_hdr, d_status);
+  if (rc) return rc < 0 ? rc : FLH_OK;
+  if (!pool || !d_page_table) return fl_set_error(FLH_E_ARG, "pool and page table are required");
+  if (page_bytes == 0 || page_bytes % u->tile_bytes) return fl_set_error(FLH_E_ARG, "tile_bytes %u must divide page_bytes %u", u->tile_bytes, page_bytes);
+  if (u->chunk_bytes % page_bytes || u->src_base % page_bytes) return fl_set_error(FLH_E_ARG, "chunk_bytes and src_base must be multiples of page_bytes %u", page_bytes);
+  fl_prof().kid = dir == 0 ? 4 : 5;
+  a.user = (uint8_t*)pool;
+  a.user_bytes = pool_pages * (uint64_t)page_bytes;
+  a.page_table = d_page_table;
+  a.pool_pages = pool_pages;
+  a.n_pages = (u->src_base + u->total_bytes + page_bytes - 1) / page_bytes;
+  a.page_bytes = page_bytes;
+  a.page_shift = (page_bytes & (page_bytes - 1)) == 0 ? __builtin_ctz(page_bytes) : -1;
+  return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream);
+}
+
+int flh_gather_pages_uniform(const void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                             const flh_windows* win, const flh_uniform_params* u, flh_chunk_desc* d_table_out,
+                             flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
+  return launch_fused_pages(0, (void*)d_pool, pool_pages, d_page_table, page_bytes, win, u, d_table_out, d_hdr_out, d_status, stream);
+}
+
+int flh_scatter_pages_uniform(void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                              const flh_windows* win, const flh_uniform_params* u, int32_t* d_status, void* stream) {
+  return launch_fused_pages(1, d_pool, pool_pages, d_page_table, page_bytes, win, u, nullptr, nullptr, d_status, stream);
 }
 
 int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,

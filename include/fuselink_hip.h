@@ -225,6 +225,18 @@ int flh_scatter_pages(void* d_pool, uint64_t pool_pages, const uint32_t* d_page_
                       const flh_chunk_desc* d_table, uint32_t n_chunks, int use_lds,
                       int32_t* d_status, void* stream);
 
+/* The paged pair with the scheduler folded in, as flh_stripe_uniform / flh_reassemble_uniform do for a flat buffer:
+ * the message of u->total_bytes bytes is the pages d_page_table[0 .. ceil((src_base + total_bytes) / page_bytes)) of
+ * the pool, in that order; no table has to exist, the gather writes it to d_table_out / d_hdr_out (may be NULL).
+ * u->tile_bytes must divide page_bytes (a copy tile never straddles a page); u->chunk_bytes and u->src_base must be
+ * multiples of page_bytes.  A page number beyond pool_pages reports FLH_E_RANGE through *d_status.  No counterpart in
+ * the reference; the page shape is the serving experiment's KV block (experiments/serving/model.hh:198-201). */
+int flh_gather_pages_uniform(const void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                             const flh_windows* win, const flh_uniform_params* u, flh_chunk_desc* d_table_out,
+                             flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
+int flh_scatter_pages_uniform(void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
+                              const flh_windows* win, const flh_uniform_params* u, int32_t* d_status, void* stream);
+
 /* Plain device copy with the same inner loop as the striping kernels (roofline calibration). */
 int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream);
 

@@ -246,6 +246,81 @@ def test_cfg4_paged_kv_gather(fl, use_lds, by_lane):
             np.testing.assert_array_equal(wins[l].cpu().numpy()[: caps[l]], exp_w[l][: caps[l]])
 
 
+@pytest.mark.parametrize("seed", range(5))
+def test_fused_paged_gather_equals_oracle(fl, seed):
+    """flh_gather_pages_uniform / flh_scatter_pages_uniform: the table the gather writes, the staged windows and
+    the scattered pool against the oracle; page sizes that are and are not powers of two, a ragged last chunk,
+    a pool larger than the message, carried epoch bytes, destination order."""
+    core, torch = fl
+    rng = np.random.default_rng(7000 + seed)
+    lanes = int(rng.integers(1, 17))
+    page = int(rng.choice([256, 4096, 4096 + 512, 32768]))
+    tile = page if page <= 32768 else 32768
+    ppc = int(rng.integers(1, 6))
+    n_pages = int(rng.integers(1, 300))
+    pool_pages = n_pages + int(rng.integers(0, 20))
+    total, chunk = n_pages * page, ppc * page
+    credits = rng.integers(0, 9, size=lanes).astype(np.uint32)
+    if seed == 1:
+        credits[:] = 0
+    epoch_bytes = int(rng.integers(0, 30)) * chunk
+    st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+    st["epoch_bytes"] = epoch_bytes
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                         mode=1, state=st, tile_bytes=tile)
+    caps = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    pool_np = rng.integers(0, 256, size=pool_pages * page, dtype=np.uint8)
+    table_np = rng.permutation(pool_pages).astype(np.uint32)[:n_pages]
+    padded = np.concatenate([table_np, np.zeros((-n_pages) % ppc, dtype=np.uint32)])
+    exp_w = ob.cpu_gather_pages(pool_np, padded, page, ppc, exp_t, caps)
+    pool = _dev(torch, pool_np)
+    table = _dev(torch, table_np.view(np.int32))
+    u = core.uniform_params(total, chunk, credits.tolist(), epoch_bytes=epoch_bytes, tile_bytes=tile)
+    for dest_order in (0, 1):
+        wins = [torch.zeros(max(c, 1), dtype=torch.uint8, device="cuda") for c in caps]
+        w = core.make_windows([t.data_ptr() for t in wins], caps)
+        out = core.new_schedule_buffers(len(exp_t), tile_bytes=tile)
+        status = core.new_status()
+        core.tune("stripe_dest_order", dest_order)
+        try:
+            core.gather_pages_uniform(pool, table, page, w, u, status, out=out)
+        finally:
+            core.tune("stripe_dest_order", -1)
+        back = torch.zeros_like(pool)
+        core.scatter_pages_uniform(back, table, page, w, u, status)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+        got_t = out.table_numpy()
+        for f in ob.DESC_DTYPE.names:
+            np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+        for l in range(lanes):
+            np.testing.assert_array_equal(wins[l].cpu().numpy()[: caps[l]], exp_w[l][: caps[l]], err_msg=f"lane {l}")
+        # the pages the table names came back; every other page of the pool stayed untouched (zero)
+        back_np = back.cpu().numpy().reshape(pool_pages, page)
+        named = np.zeros(pool_pages, dtype=bool)
+        named[table_np] = True
+        np.testing.assert_array_equal(back_np[named], pool_np.reshape(pool_pages, page)[named])
+        assert not back_np[~named].any()
+
+
+def test_fused_paged_gather_refuses_what_it_cannot_name(fl):
+    core, torch = fl
+    page, lanes = 4096, 2
+    pool = torch.zeros(8 * page, dtype=torch.uint8, device="cuda")
+    wins = [torch.zeros(8 * page, dtype=torch.uint8, device="cuda") for _ in range(lanes)]
+    w = core.make_windows([t.data_ptr() for t in wins], [8 * page] * lanes)
+    status = core.new_status()
+    good = _dev(torch, np.arange(8, dtype=np.int32))
+    with pytest.raises(Exception):   # a tile would straddle pages
+        core.gather_pages_uniform(pool, good, page, w, core.uniform_params(8 * page, 2 * page, [1, 1], tile_bytes=8192), status)
+    with pytest.raises(Exception):   # chunks that are not whole pages
+        core.gather_pages_uniform(pool, good, page, w, core.uniform_params(8 * page, page + 128, [1, 1], tile_bytes=128), status)
+    bad = _dev(torch, np.array([0, 1, 2, 3, 4, 5, 6, 99], dtype=np.int32))   # page 99 is not in the pool
+    core.gather_pages_uniform(pool, bad, page, w, core.uniform_params(8 * page, 2 * page, [1, 1], tile_bytes=4096), status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == -5   # FLH_E_RANGE
+
+
 def test_paged_gather_with_more_chunks_than_the_grid_is_tall(fl):
     """70 000 one-page chunks: the page kernels' grid is at most 65 535 chunks tall and steps over the rest."""
     core, torch = fl
