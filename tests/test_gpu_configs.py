@@ -246,7 +246,7 @@ def test_cfg4_paged_kv_gather(fl, use_lds, by_lane):
             np.testing.assert_array_equal(wins[l].cpu().numpy()[: caps[l]], exp_w[l][: caps[l]])
 
 
-@pytest.mark.parametrize("seed", range(5))
+@pytest.mark.parametrize("seed", range(16))
 def test_fused_paged_gather_equals_oracle(fl, seed):
     """flh_gather_pages_uniform / flh_scatter_pages_uniform: the table the gather writes, the staged windows and
     the scattered pool against the oracle; page sizes that are and are not powers of two, a ragged last chunk,
