@@ -16,7 +16,9 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <cerrno>
 #include <chrono>
+#include <ctime>
 #include <cstring>
 #include <mutex>
 
@@ -52,17 +54,28 @@ char g_shm_name[64] = "", g_sem_name[64] = "";
 bool g_manual_clock = false;
 int64_t g_manual_now = 0;
 
-// every access to the table goes through one of these
+// Every access to the table goes through one of these.  The cross-process semaphore is waited for with a
+// bound: a process that died holding it (the reference's sem_wait would then block for ever, src/monitor.h:195)
+// must not stall a transport thread, so after kSemWaitMs the access goes ahead unlocked -- entries are single
+// words, the worst outcome is one stale status -- and the semaphore is not posted.
+constexpr long kSemWaitMs = 200;
 struct TableLock {
   std::unique_lock<std::mutex> local;
   sem_t* sem;
+  bool held = false;
   TableLock() : local(g_mu), sem(g_sem) {
-    if (sem != SEM_FAILED) {
-      while (sem_wait(sem) != 0) {}
-    }
+    if (sem == SEM_FAILED) return;
+    timespec until;
+    clock_gettime(CLOCK_REALTIME, &until);
+    until.tv_nsec += kSemWaitMs * 1000000L;
+    until.tv_sec += until.tv_nsec / 1000000000L;
+    until.tv_nsec %= 1000000000L;
+    int rc;
+    while ((rc = sem_timedwait(sem, &until)) != 0 && errno == EINTR) {}
+    held = rc == 0;
   }
   ~TableLock() {
-    if (sem != SEM_FAILED) sem_post(sem);
+    if (held) sem_post(sem);
   }
 };
 

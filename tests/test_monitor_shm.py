@@ -173,3 +173,31 @@ def test_plugin_reads_credits_from_the_daemon():
         os.environ.pop("NCCL_FUSELINK_MONITOR_SHM", None)
         p.lib.fl_net_reset()
         assert p.init() == P.ncclSuccess
+
+
+def test_a_semaphore_nobody_releases_does_not_stall_the_library():
+    """A process that dies while it holds the named semaphore leaves it at zero for ever; the reference's
+    sem_wait (src/monitor.h:195) then blocks every client.  Here the wait is bounded and the access goes ahead."""
+    shm, sem = f"/fl_shm_dead_{os.getpid()}".encode(), f"/fl_sem_dead_{os.getpid()}".encode()
+    p = _lib()
+    try:
+        assert p.lib.fl_monitor_attach_shm(shm, sem, 1) == 0      # create the table here, as the daemon would
+        assert p.lib.fl_monitor_mark_active(2, 1, 123) == 0
+        # take the semaphore the way a crashed client would have: wait on it and never post
+        libc = C.CDLL(None, use_errno=True)
+        libc.sem_open.restype = C.c_void_p
+        libc.sem_open.argtypes = [C.c_char_p, C.c_int]
+        libc.sem_wait.argtypes = [C.c_void_p]
+        libc.sem_post.argtypes = [C.c_void_p]
+        h = libc.sem_open(sem, 0)
+        assert h and libc.sem_wait(h) == 0
+        t0 = time.time()
+        assert _status(p.lib, 1)[2] == BUSY                        # answered, after the bounded wait
+        waited = time.time() - t0
+        assert 0.1 < waited < 5.0, waited
+        libc.sem_post(h)
+        t0 = time.time()
+        assert _status(p.lib, 1)[2] == BUSY
+        assert time.time() - t0 < 0.1                              # and at once when the semaphore is free again
+    finally:
+        p.lib.fl_monitor_detach()
