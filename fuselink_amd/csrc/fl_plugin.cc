@@ -350,18 +350,37 @@ void current_credits(int own_lane, uint8_t* out) {
   for (int l = 0; l < FL_NET_MAX_LANES; ++l) out[l] = (uint8_t)(c[l] > 255 ? 255 : c[l]);
 }
 
-// Chunks one wave may carry so that no lane can outgrow its window whatever the slot phase is: a lane
-// with credit c sees at most (ceil(n / W) + 1) * c chunks out of n consecutive ones.
-uint32_t wave_chunks(const uint32_t* credits, int lanes, uint64_t chunk, uint64_t cap) {
-  uint64_t W = 0, cmax = 0;
-  for (int l = 0; l < lanes; ++l) { W += credits[l]; if (credits[l] > cmax) cmax = credits[l]; }
-  if (W == 0) { W = (uint64_t)lanes; cmax = 1; }   // no credit anywhere: equal credits stand in
+// Chunks one wave may carry so that no lane outgrows its window: the largest n for which every lane's share
+// of the quanta [before, before + n) -- the scheduler's closed form, (x / W) c + clamp(x mod W - K, 0, c) slots
+// before quantum x for a lane with first slot K and credit c -- still fits.  A bound that holds for any phase,
+// (ceil(n / W) + 1) c chunks for a lane of credit c, is where the search starts.
+uint32_t wave_chunks(const uint32_t* credits, int lanes, uint64_t chunk, uint64_t cap, uint64_t quanta_before) {
+  uint64_t c[FL_NET_MAX_LANES], K[FL_NET_MAX_LANES], W = 0, cmax = 0;
+  for (int l = 0; l < lanes; ++l) W += credits[l];
+  for (int l = 0; l < lanes; ++l) c[l] = W ? credits[l] : 1;   // no credit anywhere: equal credits stand in
+  W = 0;
+  for (int l = 0; l < lanes; ++l) { K[l] = W; W += c[l]; if (c[l] > cmax) cmax = c[l]; }
   const uint64_t per_lane = cap / chunk;           // chunks a window holds
   if (per_lane == 0) return 0;
-  const uint64_t rounds = per_lane / cmax;         // (ceil(n/W) + 1) <= rounds
-  uint64_t n = rounds >= 2 ? (rounds - 1) * W : 1;
-  if (n > (uint64_t)g_par.max_wave_chunks) n = (uint64_t)g_par.max_wave_chunks;
-  return (uint32_t)n;
+  const uint64_t rounds = per_lane / cmax;         // (ceil(n / W) + 1) <= rounds
+  uint64_t lo = rounds >= 2 ? (rounds - 1) * W : 1;
+  uint64_t hi = per_lane * (uint64_t)lanes;        // all windows full
+  if (hi > (uint64_t)g_par.max_wave_chunks) hi = (uint64_t)g_par.max_wave_chunks;
+  if (lo > hi) lo = hi;
+  auto before = [&](int l, uint64_t x) {
+    const uint64_t rem = x % W;
+    return (x / W) * c[l] + (rem <= K[l] ? 0 : (rem - K[l] < c[l] ? rem - K[l] : c[l]));
+  };
+  auto fits = [&](uint64_t n) {
+    for (int l = 0; l < lanes; ++l)
+      if (before(l, quanta_before + n) - before(l, quanta_before) > per_lane) return false;
+    return true;
+  };
+  while (lo < hi) {                                // largest n in [lo, hi] that fits; the shares only grow with n
+    const uint64_t mid = lo + (hi - lo + 1) / 2;
+    if (fits(mid)) lo = mid; else hi = mid - 1;
+  }
+  return (uint32_t)lo;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -621,8 +640,7 @@ ncclResult_t launch_transfer(Link* lk, const Pending& p) {
   uint32_t credits[FLH_MAX_LANES];
   wire_credits(lk, p.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
-  const uint32_t per_wave = wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0]);
-  if (per_wave == 0) { FL_WARN("NET/FuseLink : staging window smaller than a chunk"); return ncclInternalError; }
+  if (lk->wins.cap[0] < chunk) { FL_WARN("NET/FuseLink : staging window smaller than a chunk"); return ncclInternalError; }
   // request -> QP pieces (plugin.cc:1467-1495), each piece -> waves of chunks
   const int nqps = g_par.split_on_qps ? g_par.qps : 1;
   std::vector<int> qoff(nqps), qlen(nqps);
@@ -632,7 +650,7 @@ ncclResult_t launch_transfer(Link* lk, const Pending& p) {
     uint64_t done = 0;
     const uint64_t piece = (uint64_t)qlen[q];
     while (done < piece) {
-      uint64_t wave = (uint64_t)per_wave * chunk;
+      uint64_t wave = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0], lk->epoch_bytes / chunk) * chunk;
       if (wave > piece - done) wave = piece - done;
       // One credit row, quantum-sized chunks, windows reused from offset 0: the striping launch works out
       // every chunk's lane and window offset itself (and writes the table), the reassembly launch likewise.
@@ -686,7 +704,8 @@ size_t batch_span(const Link* lk, size_t i) {
   uint32_t credits[FLH_MAX_LANES];
   wire_credits(lk, p0.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
-  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0]) * chunk;
+  const uint64_t quanta_before = (p0.w.flags & 1u) ? 0 : lk->epoch_bytes / chunk;   // a refreshed decision starts a new epoch
+  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0], quanta_before) * chunk;
   uint64_t sum = 0;
   size_t j = i;
   while (j < lk->pending.size() && j - i < (size_t)FLH_BATCH_MAX) {

@@ -52,11 +52,35 @@ def test_cfg1_shape_on_gpu(net):
     _send_recv(net, s, r, src, dst, 4 << 20, 5, smh, rmh)
     np.testing.assert_array_equal(dst.cpu().numpy(), src_np)
     rows, hdr = net.last_table(s)
-    # a 2 MiB window holds 4 chunks; (ceil(n/2)+1)*1 <= 4 gives waves of 6 chunks: the last wave has 2
-    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=2, credits=[1, 1], quantum=512 << 10, total_bytes=2 * (512 << 10),
-                                         chunk_bytes=512 << 10, src_base=6 * (512 << 10), mode=ob.SCHED_RESET_OFFSETS,
-                                         state=_state(6 * (512 << 10), 6))
+    # a 2 MiB window holds 4 chunks and each lane gets exactly 4 of the 8: the whole request is one wave
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=2, credits=[1, 1], quantum=512 << 10, total_bytes=4 << 20,
+                                         chunk_bytes=512 << 10, mode=ob.SCHED_RESET_OFFSETS)
     _same_table(rows, exp_t)
+    assert [int(b) for b in exp_h["lane_bytes"][:2]] == [2 << 20, 2 << 20]
+    # a second request starts one quantum further on in the slot cycle only if the first left it there: 8 chunks
+    # over 2 lanes end on a whole round, so 5 more chunks (2.5 MiB) go 3 + 2 and still fit one wave
+    src2, dst2 = src[: 5 * (512 << 10)], dst[: 5 * (512 << 10)]
+    dst.zero_()
+    _send_recv(net, s, r, src2, dst2, 5 * (512 << 10), 6, smh, rmh)
+    np.testing.assert_array_equal(dst2.cpu().numpy(), src_np[: 5 * (512 << 10)])
+    rows, hdr = net.last_table(s)
+    exp_t, _, _ = ob.credit_schedule(n_lanes=2, credits=[1, 1], quantum=512 << 10, total_bytes=5 * (512 << 10),
+                                     chunk_bytes=512 << 10, mode=ob.SCHED_RESET_OFFSETS, state=_state(4 << 20, 8))
+    _same_table(rows, exp_t)
+    # 12 chunks do not fit 2 x 4: from quantum 13 on the lanes alternate, so 8 chunks fill both windows and 4 follow
+    big_np = rng.integers(0, 256, size=6 << 20, dtype=np.uint8)
+    big, back = torch.from_numpy(big_np).cuda(), torch.zeros(6 << 20, dtype=torch.uint8, device="cuda")
+    rc, bmh = net.regMr(s, big.data_ptr(), big.numel(), P.NCCL_PTR_CUDA)
+    assert rc == 0
+    rc, kmh = net.regMr(r, back.data_ptr(), back.numel(), P.NCCL_PTR_CUDA)
+    assert rc == 0
+    _send_recv(net, s, r, big, back, 6 << 20, 7, bmh, kmh)
+    np.testing.assert_array_equal(back.cpu().numpy(), big_np)
+    rows, hdr = net.last_table(s)
+    exp_t, _, _ = ob.credit_schedule(n_lanes=2, credits=[1, 1], quantum=512 << 10, total_bytes=4 * (512 << 10), chunk_bytes=512 << 10,
+                                     src_base=8 * (512 << 10), mode=ob.SCHED_RESET_OFFSETS, state=_state(21 * (512 << 10), 21))
+    _same_table(rows, exp_t)
+    assert net.deregMr(s, bmh) == 0 and net.deregMr(r, kmh) == 0
     assert net.deregMr(s, smh) == 0 and net.deregMr(r, rmh) == 0
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
