@@ -616,3 +616,40 @@ def test_launches_record_into_a_hip_graph_and_replay(fl):
         for f in ob.DESC_DTYPE.names:
             np.testing.assert_array_equal(out.table_numpy()[f], exp_t[f], err_msg=f"replay {rep} field {f}")
             np.testing.assert_array_equal(sched_out.table_numpy()[f], exp_t[f], err_msg=f"replay {rep} field {f} (scheduler kernel)")
+
+
+def test_fused_launch_at_and_past_its_chunk_limit(fl):
+    """One fused launch names its chunks through the grid's second dimension: 65 535 of them are taken (and come
+    out as the oracle has them), one more is refused with an error before anything is launched."""
+    core, torch = fl
+    rng = np.random.default_rng(65535)
+    lanes, chunk = 5, 256
+    credits = np.array([3, 1, 0, 2, 2], dtype=np.uint32)
+    for n, ok in ((65535, True), (65536, False)):
+        total = n * chunk - 100
+        src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+        src = _dev(torch, src_np)
+        dst = torch.zeros_like(src)
+        exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                             tile_bytes=256)
+        lane_bytes = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+        wins = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
+        w = core.make_windows([t.data_ptr() for t in wins], lane_bytes)
+        u = core.uniform_params(total, chunk, credits.tolist(), tile_bytes=256)
+        out = core.new_schedule_buffers(n, tile_bytes=256)
+        status = core.new_status()
+        if not ok:
+            with pytest.raises(Exception, match="65535"):
+                core.stripe_uniform(src, w, u, status, out=out)
+            continue
+        core.stripe_uniform(src, w, u, status, out=out)
+        core.reassemble_uniform(dst, w, u, status)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0 and torch.equal(src, dst)
+        got_t = out.table_numpy()
+        for f in ob.DESC_DTYPE.names:
+            np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+        exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+        for l in range(lanes):
+            if lane_bytes[l]:
+                np.testing.assert_array_equal(wins[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"lane {l}")
