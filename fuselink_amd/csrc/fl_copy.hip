@@ -296,7 +296,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
     before = k;
   } else if (a.fast) {
     const uint32_t j = (uint32_t)a.quanta_before + c;
-    const uint32_t full = (uint32_t)__umul64hi((uint64_t)j, a.magic);  // j / W
+    const uint32_t full = a.magic ? (uint32_t)__umul64hi((uint64_t)j, a.magic) : j;  // j / W (magic 0 stands for W = 1)
     const uint32_t slot = j - full * a.pfx_ex[FLH_MAX_LANES];  // the last entry is always W
     // the last lane whose first slot is not beyond this one (lanes without credit share their successor's first slot)
     static_assert(FLH_MAX_LANES == 16, "the search below takes four steps");
@@ -597,8 +597,8 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
     uint64_t pfx[FLH_MAX_LANES], W = 0;
     for (uint32_t l = 0; l < u->n_lanes; ++l) { W += u->credits[l]; pfx[l] = W; }
     if (W == 0) { for (uint32_t l = 0; l < u->n_lanes; ++l) pfx[l] = l + 1; W = u->n_lanes; }
-    a.fast = W >= 2 && W <= 0xffffffffull && a.quanta_before + n <= 0xffffffffull && g_fused_fast;
-    a.magic = a.fast ? ~0ull / W + 1 : 0;
+    a.fast = W <= 0xffffffffull && a.quanta_before + n <= 0xffffffffull && g_fused_fast;
+    a.magic = a.fast && W >= 2 ? ~0ull / W + 1 : 0;   // ceil(2^64 / W); W = 1 (one lane named outright) needs no division
     for (int l = 0; l < FLH_MAX_LANES; ++l) a.cnt0[l] = 0;
     for (int l = 0; l <= FLH_MAX_LANES; ++l) a.pfx_ex[l] = l == 0 ? 0 : (uint32_t)((uint32_t)l <= u->n_lanes ? pfx[l - 1] : W);
     if (a.fast) {
