@@ -653,3 +653,43 @@ def test_fused_launch_at_and_past_its_chunk_limit(fl):
         for l in range(lanes):
             if lane_bytes[l]:
                 np.testing.assert_array_equal(wins[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"lane {l}")
+
+
+@pytest.mark.parametrize("lanes,hot", [(1, 0), (8, 2), (16, 15)])
+def test_fused_pair_with_one_lane_named_outright(fl, lanes, hot):
+    """The static policy (lane = channelId % nNics, FuseLink src/fuselink.h:235) reaches the kernels as a credit row
+    with a single 1: every chunk on that lane, window offsets running, other windows untouched."""
+    core, torch = fl
+    rng = np.random.default_rng(1235 + lanes)
+    chunk = 24576
+    total = 77 * chunk - 5
+    credits = np.zeros(lanes, dtype=np.uint32)
+    credits[hot] = 1
+    epoch_bytes = 9 * chunk
+    st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+    st["epoch_bytes"] = epoch_bytes
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                         mode=1, state=st)
+    assert (exp_t["lane"] == hot).all()
+    src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+    src = _dev(torch, src_np)
+    dst = torch.zeros_like(src)
+    wins = [torch.full((total + 64,), 0xA5, dtype=torch.uint8, device="cuda") for _ in range(lanes)]
+    w = core.make_windows([t.data_ptr() for t in wins], [total] * lanes)
+    u = core.uniform_params(total, chunk, credits.tolist(), epoch_bytes=epoch_bytes)
+    out = core.new_schedule_buffers(len(exp_t))
+    status = core.new_status()
+    core.stripe_uniform(src, w, u, status, out=out)
+    core.reassemble_uniform(dst, w, u, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0 and torch.equal(src, dst)
+    got_t = out.table_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+    for l in range(lanes):
+        got = wins[l].cpu().numpy()
+        if l == hot:
+            np.testing.assert_array_equal(got[:total], src_np)
+            assert (got[total:] == 0xA5).all()
+        else:
+            assert (got == 0xA5).all(), f"lane {l} was written"
