@@ -60,6 +60,12 @@ def main() -> int:
                          "cache-resident; off by default so that a kernel trace of the default run holds the timed loop's launches only")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="set a library tunable (flh_tune) before the run, e.g. --tune copy_rows_per_wg=1; repeatable")
+    ap.add_argument("--blocks", type=int, default=256,
+                    help="blocks workload: number of variable blocks (rows per block ~ Zipf(1.1) capped at 4096 for the 256 blocks of cfg3, "
+                         "at 65536 / blocks otherwise: 65000 blocks are single rows of 14 KiB)")
+    ap.add_argument("--tile-descriptors", type=int, default=-1,
+                    help="blocks workload: let the scheduler expand the table to one descriptor per copy tile (flh_stripe_tiles); "
+                         "-1 = when the blocks average under two copy tiles and there are at least 4096 of them")
     ap.add_argument("--no-by-lane", action="store_true", help="stripe large messages in chunk order instead of destination order")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -90,13 +96,15 @@ def main() -> int:
     # ---- synthetic inputs, resident in HBM ------------------------------------------------------
     sizes_np = None
     if kind == "blocks":
-        ranks = np.arange(1, 4097, dtype=np.float64)
+        # cfg3 proper: 256 blocks of up to 4096 rows; more blocks mean finer dispatch, down to a token (one row) per block
+        max_rows = 4096 if args.blocks == 256 else max(1, 65536 // args.blocks)
+        ranks = np.arange(1, max_rows + 1, dtype=np.float64)
         p = ranks ** -1.1
-        rows_per_block = rng.choice(np.arange(1, 4097), size=256, p=p / p.sum())
+        rows_per_block = rng.choice(np.arange(1, max_rows + 1), size=args.blocks, p=p / p.sum())
         sizes_np = (rows_per_block * 7168 * 2).astype(np.uint32)
         nbytes = int(sizes_np.sum())
         credits_np = np.array([[4, 4, 4, 4, 4, 4, 4, 1]], dtype=np.int32)   # one lane at 25 % idleness
-        n_chunks = 256
+        n_chunks = args.blocks
     else:
         credits_np = rng.integers(1, 9, size=(rows, lanes)).astype(np.int32)
         n_chunks = (nbytes + chunk - 1) // chunk
@@ -124,10 +132,14 @@ def main() -> int:
     # (measured: no gain for the paged gather, whose reads are scattered either way, so it keeps chunk order)
     by_lane = kind == "uniform" and rows <= 32 and nbytes > (256 << 20) and not args.no_by_lane
 
+    use_tiles = kind == "blocks" and (args.tile_descriptors > 0 or
+                                      (args.tile_descriptors < 0 and n_chunks >= 4096 and nbytes < 2 * core.TILE_BYTES * n_chunks))
+    tiles_capacity = nbytes // core.TILE_BYTES + n_chunks if use_tiles else 0
+
     def run_schedule(out=None):
         return core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, sizes=sizes,
                              total_bytes=0 if sizes is not None else msg_bytes, chunk_bytes=0 if sizes is not None else chunk,
-                             epoch_len=epoch_len, out=out, stream=stream, by_lane=by_lane)
+                             epoch_len=epoch_len, out=out, stream=stream, by_lane=by_lane, tiles_capacity=tiles_capacity)
 
     sched = run_schedule()
     stream.synchronize()
@@ -269,6 +281,8 @@ def main() -> int:
         kernel_name = "fl_copy_uniform_fused<0> (stripe)"
     elif hint is not None:
         kernel_name = "fl_copy_uniform<0> (stripe)"
+    elif use_tiles:
+        kernel_name = "fl_copy_desc<0> (stripe)"
     else:
         kernel_name = "fl_copy_tiles<0> (stripe)"
 
@@ -292,7 +306,7 @@ def main() -> int:
                    "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
                    "step": ("2x(gather(with scheduler folded in)+scatter)" if (kind == "pages" and fused) else "2x(schedule+gather+scatter)" if kind == "pages" else
                             "stripe(with scheduler folded in)+reassemble" if fused else "schedule+stripe+reassemble"),
-                   "launch": "eager", "windows": "HIP VMM, 2 MiB units",
+                   "launch": "eager", "windows": "HIP VMM, 2 MiB units", "tile_descriptors": bool(use_tiles),
                    "stripe_order": "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel for messages past 256 MiB)" if fused else "chunk"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
@@ -307,7 +321,7 @@ def main() -> int:
         "cold_user_buffers": cold,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(args.workload)},
+                     "traffic": MEASURED_TRAFFIC.get(args.workload) if (kind != "blocks" or args.blocks == 256) else None},
     }
 
     # ---- CPU baseline: the oracle's host-memcpy striping on a bounded sample ------------------------

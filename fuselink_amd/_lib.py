@@ -31,7 +31,8 @@ class SchedParams(C.Structure):
                 ("n_lanes", C.c_uint32), ("d_credits", C.c_void_p), ("n_rows", C.c_uint32),
                 ("epoch_len", C.c_uint32), ("quantum", C.c_uint64), ("tile_bytes", C.c_uint32),
                 ("mode", C.c_uint32), ("d_state", C.c_void_p), ("d_table", C.c_void_p), ("d_hdr", C.c_void_p),
-                ("inline_credits", C.c_uint32 * MAX_LANES), ("d_table_by_lane", C.c_void_p)]
+                ("inline_credits", C.c_uint32 * MAX_LANES), ("d_table_by_lane", C.c_void_p),
+                ("d_tiles", C.c_void_p), ("tiles_cap", C.c_uint32), ("pad_", C.c_uint32)]
 
 
 class UniformParams(C.Structure):
@@ -63,6 +64,10 @@ SIGNATURES = {
                              C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
     "flh_reassemble": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p,
                                  C.POINTER(SchedHdr), C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
+    "flh_stripe_tiles": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_uint32, C.c_void_p, C.POINTER(SchedHdr),
+                                   C.c_void_p, C.c_void_p]),
+    "flh_reassemble_tiles": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_uint32, C.c_void_p, C.POINTER(SchedHdr),
+                                       C.c_void_p, C.c_void_p]),
     "flh_stripe_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,
                                      C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_reassemble_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,

@@ -23,6 +23,7 @@ DESC_DTYPE = np.dtype([("src_off", "<u8"), ("win_off", "<u8"), ("len", "<u4"), (
                        ("tile_base", "<u4"), ("epoch", "<u4")])
 HDR_DTYPE = np.dtype([("total_bytes", "<u8"), ("total_tiles", "<u4"), ("n_chunks", "<u4"), ("flags", "<u4"),
                       ("uniform_tiles", "<u4"), ("lane_bytes", "<u8", (MAX_LANES,)), ("lane_chunks", "<u4", (MAX_LANES,))])
+TILE_DESC_DTYPE = np.dtype([("src_off", "<u8"), ("win_off", "<u8"), ("len", "<u4"), ("lane", "<u4"), ("row", "<u4"), ("pad", "<u4")])
 STATE_DTYPE = np.dtype([("epoch_bytes", "<u8"), ("chunk_index", "<u8"), ("lane_off", "<u8", (MAX_LANES,))])
 assert DESC_DTYPE.itemsize == C.sizeof(ChunkDesc) == 32
 assert HDR_DTYPE.itemsize == C.sizeof(SchedHdr)
@@ -76,6 +77,11 @@ class Schedule:
     n_chunks: int
     tile_bytes: int
     table_by_lane: Optional[torch.Tensor] = None   # the same rows in destination order (uniform split only)
+    tiles: Optional[torch.Tensor] = None           # uint8 [capacity * 32]: one flh_tile_desc per copy tile
+    tiles_cap: int = 0
+
+    def tiles_numpy(self, n_tiles: int) -> np.ndarray:
+        return self.tiles[: n_tiles * TILE_DESC_DTYPE.itemsize].cpu().numpy().view(TILE_DESC_DTYPE).copy()
 
     def table_numpy(self) -> np.ndarray:
         raw = self.table[: self.n_chunks * DESC_DTYPE.itemsize].cpu().numpy()
@@ -100,7 +106,8 @@ def state_numpy(state: torch.Tensor) -> np.ndarray:
 def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Optional[torch.Tensor] = None,
              total_bytes: int = 0, chunk_bytes: int = 0, src_off: Optional[torch.Tensor] = None, src_base: int = 0,
              epoch_len: int = 0, tile_bytes: int = TILE_BYTES, mode: int = 0, state: Optional[torch.Tensor] = None,
-             out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None, by_lane: bool = False) -> Schedule:
+             out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None, by_lane: bool = False,
+             tiles_capacity: int = 0) -> Schedule:
     """Launches the scheduler kernel (flh_schedule).  `credits` is a uint32/int32 device tensor of
     shape [rows, n_lanes]; `sizes` a uint32/int32 device tensor of chunk sizes, or None for the
     uniform split of `total_bytes` by `chunk_bytes`."""
@@ -136,6 +143,10 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
         for l, c in enumerate(inline):
             p.inline_credits[l] = c
     p.d_table_by_lane = _ptr(out.table_by_lane) if by_lane else None
+    if tiles_capacity:   # per-tile descriptors for stripe / reassemble (pays for tables of many unequal rows)
+        if out.tiles is None or out.tiles_cap < tiles_capacity:
+            out.tiles, out.tiles_cap = _dev_bytes(tiles_capacity * TILE_DESC_DTYPE.itemsize, dev), tiles_capacity
+        p.d_tiles, p.tiles_cap = _ptr(out.tiles), out.tiles_cap
     check(lib.flh_schedule(C.byref(p), _stream_ptr(stream)))
     return out
 
@@ -178,6 +189,10 @@ def stripe(src: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tenso
            stream: Optional[torch.cuda.Stream] = None, hint: Optional[SchedHdr] = None, by_lane: bool = False) -> None:
     """flh_stripe; with by_lane the rows are taken in destination order (sched.table_by_lane)."""
     table = sched.table_by_lane if by_lane else sched.table
+    if sched.tiles is not None and not by_lane:
+        check(_lib.load().flh_stripe_tiles(_ptr(src), src.numel() * src.element_size(), C.byref(win), _ptr(sched.tiles), sched.tiles_cap,
+                                           _ptr(sched.hdr), _hint_ref(hint), _ptr(status), _stream_ptr(stream)))
+        return
     check(_lib.load().flh_stripe(_ptr(src), src.numel() * src.element_size(), C.byref(win), _ptr(table),
                                  _ptr(sched.hdr), _hint_ref(hint), sched.n_chunks, sched.tile_bytes, _ptr(status),
                                  _stream_ptr(stream)))
@@ -185,6 +200,10 @@ def stripe(src: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tenso
 
 def reassemble(dst: torch.Tensor, win: Windows, sched: Schedule, status: torch.Tensor,
                stream: Optional[torch.cuda.Stream] = None, hint: Optional[SchedHdr] = None) -> None:
+    if sched.tiles is not None:
+        check(_lib.load().flh_reassemble_tiles(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), _ptr(sched.tiles), sched.tiles_cap,
+                                               _ptr(sched.hdr), _hint_ref(hint), _ptr(status), _stream_ptr(stream)))
+        return
     check(_lib.load().flh_reassemble(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), _ptr(sched.table),
                                      _ptr(sched.hdr), _hint_ref(hint), sched.n_chunks, sched.tile_bytes, _ptr(status),
                                      _stream_ptr(stream)))

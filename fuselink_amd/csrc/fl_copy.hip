@@ -150,6 +150,41 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
   }
 }
 
+// Any table, expanded beforehand to one descriptor per tile: the workgroup's descriptor is the only thing it waits
+// for before its data (the header, where the host has no copy of it, is read alongside, not before).
+struct DescArgs {
+  uint8_t* user;
+  uint64_t user_bytes;
+  flh_windows win;
+  const flh_tile_desc* tiles;
+  const flh_sched_hdr* hdr;
+  int32_t* status;
+  uint32_t tiles_cap;
+  uint32_t has_hint, hint_total_tiles;
+};
+
+template <int DIR, int NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_desc(DescArgs a) {
+  warm_kernel_args(a);
+  const uint32_t t = blockIdx.x;
+  const flh_tile_desc d = a.tiles[t];
+  const uint32_t total = a.has_hint ? a.hint_total_tiles : a.hdr->total_tiles;
+  if (total > a.tiles_cap) {   // the table did not fit the descriptor array: nothing of it can be trusted
+    if (t == 0 && threadIdx.x == 0) *a.status = FLH_E_RANGE;
+    return;
+  }
+  if (t >= total || d.len == 0) return;
+  bool ok = d.lane < a.win.n_lanes;
+  if (ok) ok = d.win_off + d.len <= a.win.cap[d.lane] && d.src_off + d.len <= a.user_bytes;
+  if (!ok) {
+    if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
+    return;
+  }
+  uint8_t* u = a.user + d.src_off;
+  uint8_t* w = (uint8_t*)a.win.base[d.lane] + d.win_off;
+  if (DIR == 0) block_copy<NT>(w, u, d.len); else block_copy<NT>(u, w, d.len);
+}
+
 // Uniform split with the header known on the host: a two-dimensional grid (tile in chunk, chunk)
 // names the work directly, so a workgroup's only dependent access before its data is the one scalar
 // load of its table row.
@@ -546,6 +581,46 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   FL_LAUNCH_COPY(fl_copy_tiles, FL_NO_EXTRA, dir, mode, grid, s, a);
   FL_HIP(hipGetLastError());
   return FLH_OK;
+}
+
+static int launch_desc(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_tile_desc* d_tiles, uint32_t tiles_cap,
+                       const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, int32_t* d_status, void* stream) {
+  int rc = check_windows(win);
+  if (rc) return rc;
+  if (!d_tiles || tiles_cap == 0) return fl_set_error(FLH_E_ARG, "tile descriptors missing");
+  if (!d_status || (!d_hdr && !h_hdr)) return fl_set_error(FLH_E_ARG, "d_status and a header (device or host copy) are required");
+  if (user_bytes && !user) return fl_set_error(FLH_E_ARG, "user buffer missing");
+  if (h_hdr && h_hdr->total_tiles > tiles_cap) return fl_set_error(FLH_E_RANGE, "the table has %u tiles, the descriptor array holds %u", h_hdr->total_tiles, tiles_cap);
+  const uint32_t grid = h_hdr ? h_hdr->total_tiles : tiles_cap;
+  if (grid == 0) return FLH_OK;
+  rc = fl_need_init();
+  if (rc) return rc;
+  fl_prof().kid = dir == 0 ? 2 : 3;
+  DescArgs a;
+  a.user = (uint8_t*)user;
+  a.user_bytes = user_bytes;
+  a.win = *win;
+  a.tiles = d_tiles;
+  a.hdr = d_hdr;
+  a.status = d_status;
+  a.tiles_cap = tiles_cap;
+  a.has_hint = h_hdr != nullptr;
+  a.hint_total_tiles = h_hdr ? h_hdr->total_tiles : 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int mode = fl_stream_mode(dir, user_bytes);
+  FL_LAUNCH_COPY(fl_copy_desc, FL_NO_EXTRA, dir, mode, dim3(grid), s, a);
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_stripe_tiles(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_tile_desc* d_tiles,
+                     uint32_t tiles_cap, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, int32_t* d_status, void* stream) {
+  return launch_desc(0, (void*)d_src, src_bytes, win, d_tiles, tiles_cap, d_hdr, h_hdr, d_status, stream);
+}
+
+int flh_reassemble_tiles(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_tile_desc* d_tiles,
+                         uint32_t tiles_cap, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, int32_t* d_status, void* stream) {
+  return launch_desc(1, d_dst, dst_bytes, win, d_tiles, tiles_cap, d_hdr, h_hdr, d_status, stream);
 }
 
 int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_chunk_desc* d_table,

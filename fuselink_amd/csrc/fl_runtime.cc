@@ -87,7 +87,8 @@ int64_t flh_constant(int which) {
     case 4: return sizeof(flh_chunk_desc);
     case 5: return sizeof(flh_sched_state);
     case 6: return sizeof(flh_sched_hdr);
-    case 7: return 2;   // ABI version: 2 added flh_sched_params.d_table_by_lane, the batch entry points, the DMA-BUF export
+    case 7: return 3;   // ABI version: 2 added flh_sched_params.d_table_by_lane, the batch entry points, the DMA-BUF export;
+                        // 3 the per-tile descriptors (flh_sched_params.d_tiles, flh_stripe_tiles / flh_reassemble_tiles) and the fused paged pair
     case 8: return sizeof(flh_windows);
     case 9: return sizeof(flh_sched_params);
   }

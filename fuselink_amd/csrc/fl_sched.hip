@@ -657,7 +657,49 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
 
 }  // namespace
 
+// ------------------------------------------------------------------------------------------------
+// table -> per-tile descriptors
+// ------------------------------------------------------------------------------------------------
+// One wavefront per row, its lanes striding over the row's tiles: short rows cost one store, a row of a thousand
+// tiles sixteen per lane.  Runs behind the scheduler kernel on the same stream and reads what that one wrote.
+constexpr int kExpandBlock = 256;
+__global__ __launch_bounds__(kExpandBlock) void fl_expand_tiles(const flh_chunk_desc* __restrict__ table, const flh_sched_hdr* __restrict__ hdr,
+                                                                uint32_t n_max, uint32_t tile_bytes, flh_tile_desc* __restrict__ out, uint32_t cap) {
+  uint32_t n = hdr->n_chunks;
+  if (n > n_max) n = n_max;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t waves = gridDim.x * (kExpandBlock / kWave);
+  for (uint32_t row = blockIdx.x * (kExpandBlock / kWave) + threadIdx.x / kWave; row < n; row += waves) {
+    const flh_chunk_desc d = table[row];
+    const uint32_t nt = (uint32_t)(((uint64_t)d.len + tile_bytes - 1) / tile_bytes);
+    for (uint32_t j = lane; j < nt; j += kWave) {
+      const uint32_t t = d.tile_base + j;
+      if (t >= cap) break;
+      const uint64_t off = (uint64_t)j * tile_bytes;
+      flh_tile_desc o;
+      o.src_off = d.src_off + off;
+      o.win_off = d.win_off + off;
+      o.len = (uint32_t)((d.len - off) < tile_bytes ? (d.len - off) : tile_bytes);
+      o.lane = d.lane;
+      o.row = row;
+      o.pad = 0;
+      out[t] = o;
+    }
+  }
+}
+
 extern "C" {
+
+static int expand_tiles(const flh_sched_params* p, hipStream_t s) {
+  if (!p->d_tiles || p->n_chunks == 0) return FLH_OK;
+  const uint32_t per_block = kExpandBlock / kWave;
+  uint32_t grid = (p->n_chunks + per_block - 1) / per_block;
+  if (grid > 8192) grid = 8192;
+  FL_LAUNCH(fl_expand_tiles, dim3(grid), dim3(kExpandBlock), 0, s, (const flh_chunk_desc*)p->d_table, (const flh_sched_hdr*)p->d_hdr, p->n_chunks,
+            p->tile_bytes, p->d_tiles, p->tiles_cap);
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
 
 int flh_schedule(const flh_sched_params* p, void* stream) {
   if (!p) return fl_set_error(FLH_E_ARG, "null params");
@@ -667,6 +709,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   if (p->quantum == 0) return fl_set_error(FLH_E_ARG, "quantum must be > 0");
   if (p->tile_bytes == 0 || p->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", p->tile_bytes);
   if (!p->d_hdr || (p->n_chunks && !p->d_table)) return fl_set_error(FLH_E_ARG, "output pointers missing");
+  if (p->d_tiles && p->tiles_cap == 0) return fl_set_error(FLH_E_ARG, "d_tiles without tiles_cap");
   if (!p->d_sizes) {
     if (p->n_chunks && p->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0 for the uniform split");
     const uint64_t need = p->chunk_bytes ? (p->total_bytes + p->chunk_bytes - 1) / p->chunk_bytes : 0;
@@ -707,7 +750,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     FL_LAUNCH((fl_schedule_uniform_kernel<0>), dim3(grid), dim3(kUniBlock), 0, s, a);
     if (grid > 1 && p->d_state) FL_LAUNCH((fl_schedule_uniform_kernel<1>), dim3(1), dim3(kUniBlock), 0, s, a);
     FL_HIP(hipGetLastError());
-    return FLH_OK;
+    return expand_tiles(p, s);
   }
   if (p->d_table_by_lane && n > 0) return fl_set_error(FLH_E_ARG, "d_table_by_lane needs the uniform closed-form split (no d_sizes, no d_src_off, quantum == chunk_bytes, n_rows <= %d)", kRowCache);
   // one workgroup; more wavefronts first, then more chunks per thread, as the chunk count grows (measured best shapes)
@@ -725,7 +768,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     FL_LAUNCH((fl_schedule_kernel<8, 8>), dim3(1), dim3(8 * kWave), 0, s, a);
   }
   FL_HIP(hipGetLastError());
-  return FLH_OK;
+  return expand_tiles(p, s);
 }
 
 }  // extern "C"

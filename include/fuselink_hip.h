@@ -55,6 +55,17 @@ typedef struct flh_sched_state {
   uint64_t lane_off[FLH_MAX_LANES];   /* next free byte of each staging window */
 } flh_sched_state;
 
+/* One copy tile of a table: tile_bytes (the last one of a chunk: fewer) bytes at src_off of the user buffer, at
+ * win_off of lane's window; row = the chunk it belongs to. */
+typedef struct flh_tile_desc {
+  uint64_t src_off;
+  uint64_t win_off;
+  uint32_t len;
+  uint32_t lane;
+  uint32_t row;
+  uint32_t pad;
+} flh_tile_desc;
+
 /* Summary written by the scheduler next to the table (device memory, 216 bytes). */
 typedef struct flh_sched_hdr {
   uint64_t total_bytes;
@@ -99,6 +110,12 @@ typedef struct flh_sched_params {
                                       window front to back, which is faster once a message exceeds the Infinity
                                       Cache.  Uniform closed-form split only (d_sizes == NULL, d_src_off == NULL,
                                       quantum == chunk_bytes, n_rows <= 32); FLH_E_ARG otherwise. */
+  struct flh_tile_desc* d_tiles; /* optional out: the table expanded to one descriptor per copy tile (a second launch
+                                    behind the scheduler's), for flh_stripe_tiles / flh_reassemble_tiles: a copy
+                                    workgroup then reads one descriptor instead of searching the table for its row,
+                                    which pays from a few thousand rows of unequal size on */
+  uint32_t tiles_cap;          /* descriptors d_tiles holds; total_bytes / tile_bytes + n_chunks always suffices */
+  uint32_t pad_;
 } flh_sched_params;
 
 /* ---- library ------------------------------------------------------------------------------ */
@@ -161,6 +178,14 @@ int flh_stripe(const void* d_src, uint64_t src_bytes, const flh_windows* win,
 int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
                    const flh_chunk_desc* d_table, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr,
                    uint32_t n_chunks_max, uint32_t tile_bytes, int32_t* d_status, void* stream);
+
+/* The same pair driven by the per-tile descriptors that flh_schedule wrote to d_tiles (tiles_cap entries).  The
+ * number of tiles comes from h_hdr when given, else from d_hdr; a table with more tiles than tiles_cap is refused
+ * through *d_status (FLH_E_RANGE), and so is a descriptor that would leave the buffer or its window. */
+int flh_stripe_tiles(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_tile_desc* d_tiles,
+                     uint32_t tiles_cap, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, int32_t* d_status, void* stream);
+int flh_reassemble_tiles(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_tile_desc* d_tiles,
+                         uint32_t tiles_cap, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, int32_t* d_status, void* stream);
 
 /* Scheduler and copy in one launch, for a uniform split (R1) under a single credit row with
  * quantum == chunk_bytes and window offsets starting at 0 -- the shape of every request the plugin

@@ -693,3 +693,93 @@ def test_fused_pair_with_one_lane_named_outright(fl, lanes, hot):
             assert (got[total:] == 0xA5).all()
         else:
             assert (got == 0xA5).all(), f"lane {l} was written"
+
+
+def _expected_tiles(table, tile):
+    """One descriptor per copy tile, from the table alone: tile j of row r sits at tile_base[r] + j."""
+    rows = []
+    for r, d in enumerate(table):
+        nt = (int(d["len"]) + tile - 1) // tile
+        for j in range(nt):
+            off = j * tile
+            rows.append((int(d["src_off"]) + off, int(d["win_off"]) + off, min(tile, int(d["len"]) - off), int(d["lane"]), r,
+                         int(d["tile_base"]) + j))
+    return rows
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_tile_descriptors_and_the_copies_they_drive_equal_oracle(fl, seed):
+    """flh_schedule with d_tiles, then flh_stripe_tiles / flh_reassemble_tiles: descriptors as the table implies them,
+    windows and reassembled bytes as the oracle's, for variable sizes (empty chunks among them), explicit source
+    offsets with gaps and odd alignment, small and large tiles, with and without the host copy of the header."""
+    core, torch = fl
+    rng = np.random.default_rng(8800 + seed)
+    lanes = int(rng.integers(1, 17))
+    tile = int(rng.choice([128, 4096, 32768]))
+    n = int(rng.integers(1, 1200))
+    sizes = rng.integers(0, int(rng.choice([300, 9000, 70000])), size=n).astype(np.uint32)
+    if seed % 3 == 0:
+        sizes[rng.integers(0, n, size=max(1, n // 7))] = 0
+    credits = rng.integers(0, 9, size=(int(rng.integers(1, 4)), lanes)).astype(np.uint32)
+    epoch_len = int(rng.choice([0, 5, 100]))
+    quantum = int(rng.choice([1, 4096, 65536]))
+    src_off = None
+    if seed % 2:
+        gaps = rng.integers(0, 40, size=n)
+        src_off = np.concatenate([[int(rng.integers(0, 64))], (sizes[:-1] + gaps[:-1])]).cumsum().astype(np.uint64)
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=quantum, sizes=sizes, src_off=src_off,
+                                         epoch_len=epoch_len, tile_bytes=tile)
+    total = int((src_off[-1] + sizes[-1]) if src_off is not None else sizes.sum()) + 8
+    n_tiles = int(exp_h["total_tiles"])
+    cap = n_tiles + int(rng.integers(0, 50))
+    sched = core.schedule(n_lanes=lanes, credits=_dev(torch, credits.view(np.int32)), quantum=quantum, sizes=_dev(torch, sizes.view(np.int32)),
+                          src_off=None if src_off is None else _dev(torch, src_off.view(np.int64)), epoch_len=epoch_len, tile_bytes=tile,
+                          tiles_capacity=max(cap, 1))
+    torch.cuda.synchronize()
+    got_t = sched.table_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+    got = sched.tiles_numpy(n_tiles)
+    want = _expected_tiles(exp_t, tile)
+    assert len(want) == n_tiles
+    for (s_off, w_off, ln, lane, row, t) in want:
+        g = got[t]
+        assert (int(g["src_off"]), int(g["win_off"]), int(g["len"]), int(g["lane"]), int(g["row"])) == (s_off, w_off, ln, lane, row), f"tile {t}"
+    caps = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+    exp_w = ob.cpu_stripe(src_np, exp_t, caps)
+    src = _dev(torch, src_np)
+    hdr = sched.hdr_numpy()
+    hint = core.SchedHdr()
+    hint.total_bytes, hint.total_tiles, hint.n_chunks = int(hdr["total_bytes"]), int(hdr["total_tiles"]), int(hdr["n_chunks"])
+    for h in (None, hint):
+        pad = [int(rng.integers(0, 16)) for _ in caps]      # misaligned window bases
+        wins = [torch.zeros(c + 64, dtype=torch.uint8, device="cuda") for c in caps]
+        w = core.make_windows([t.data_ptr() + p for t, p in zip(wins, pad)], caps)
+        status = core.new_status()
+        dst = torch.zeros_like(src)
+        core.stripe(src, w, sched, status, hint=h)
+        core.reassemble(dst, w, sched, status, hint=h)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+        for l in range(lanes):
+            np.testing.assert_array_equal(wins[l].cpu().numpy()[pad[l]: pad[l] + caps[l]], exp_w[l][:caps[l]], err_msg=f"lane {l}")
+        exp_dst = ob.cpu_reassemble(total, exp_w, exp_t)
+        np.testing.assert_array_equal(dst.cpu().numpy(), exp_dst[:total])
+
+
+def test_tile_descriptor_array_too_small_is_refused(fl):
+    core, torch = fl
+    sizes = np.full(40, 70000, dtype=np.uint32)      # 3 tiles each: 120 tiles
+    sched = core.schedule(n_lanes=2, credits=[1, 1], quantum=70000, sizes=_dev(torch, sizes.view(np.int32)), tiles_capacity=100)
+    src = torch.zeros(40 * 70000, dtype=torch.uint8, device="cuda")
+    wins = [torch.zeros(20 * 70000, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    w = core.make_windows([t.data_ptr() for t in wins], [20 * 70000] * 2)
+    status = core.new_status()
+    core.stripe(src, w, sched, status)                # header only on the device: the kernel finds out
+    torch.cuda.synchronize()
+    assert int(status.item()) == -5                   # FLH_E_RANGE
+    hint = core.SchedHdr()
+    hint.total_tiles, hint.n_chunks = 120, 40
+    with pytest.raises(Exception, match="120 tiles"):
+        core.stripe(src, w, sched, status, hint=hint)  # the host copy of the header says so before anything is launched
