@@ -139,7 +139,8 @@ def main() -> int:
     def run_schedule(out=None):
         return core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, sizes=sizes,
                              total_bytes=0 if sizes is not None else msg_bytes, chunk_bytes=0 if sizes is not None else chunk,
-                             epoch_len=epoch_len, out=out, stream=stream, by_lane=by_lane, tiles_capacity=tiles_capacity)
+                             epoch_len=epoch_len, out=out, stream=stream, by_lane=by_lane, tiles_capacity=tiles_capacity,
+                             workspace=sizes is not None)   # a long variable list is then scanned by several workgroups
 
     sched = run_schedule()
     stream.synchronize()

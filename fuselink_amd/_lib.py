@@ -32,7 +32,8 @@ class SchedParams(C.Structure):
                 ("epoch_len", C.c_uint32), ("quantum", C.c_uint64), ("tile_bytes", C.c_uint32),
                 ("mode", C.c_uint32), ("d_state", C.c_void_p), ("d_table", C.c_void_p), ("d_hdr", C.c_void_p),
                 ("inline_credits", C.c_uint32 * MAX_LANES), ("d_table_by_lane", C.c_void_p),
-                ("d_tiles", C.c_void_p), ("tiles_cap", C.c_uint32), ("pad_", C.c_uint32)]
+                ("d_tiles", C.c_void_p), ("tiles_cap", C.c_uint32), ("pad_", C.c_uint32),
+                ("d_workspace", C.c_void_p), ("workspace_bytes", C.c_uint64)]
 
 
 class UniformParams(C.Structure):
@@ -59,6 +60,7 @@ SIGNATURES = {
     "flh_init": (C.c_int, [C.c_int]),
     "flh_last_error": (C.c_char_p, []),
     "flh_constant": (C.c_int64, [C.c_int]),
+    "flh_schedule_workspace_bytes": (C.c_uint64, [C.c_uint32]),
     "flh_schedule": (C.c_int, [C.POINTER(SchedParams), C.c_void_p]),
     "flh_stripe": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p, C.POINTER(SchedHdr),
                              C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),

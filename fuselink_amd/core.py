@@ -79,6 +79,7 @@ class Schedule:
     table_by_lane: Optional[torch.Tensor] = None   # the same rows in destination order (uniform split only)
     tiles: Optional[torch.Tensor] = None           # uint8 [capacity * 32]: one flh_tile_desc per copy tile
     tiles_cap: int = 0
+    workspace: Optional[torch.Tensor] = None       # scratch for the scan scheduler over several workgroups
 
     def tiles_numpy(self, n_tiles: int) -> np.ndarray:
         return self.tiles[: n_tiles * TILE_DESC_DTYPE.itemsize].cpu().numpy().view(TILE_DESC_DTYPE).copy()
@@ -107,7 +108,7 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
              total_bytes: int = 0, chunk_bytes: int = 0, src_off: Optional[torch.Tensor] = None, src_base: int = 0,
              epoch_len: int = 0, tile_bytes: int = TILE_BYTES, mode: int = 0, state: Optional[torch.Tensor] = None,
              out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None, by_lane: bool = False,
-             tiles_capacity: int = 0) -> Schedule:
+             tiles_capacity: int = 0, workspace: bool = False) -> Schedule:
     """Launches the scheduler kernel (flh_schedule).  `credits` is a uint32/int32 device tensor of
     shape [rows, n_lanes]; `sizes` a uint32/int32 device tensor of chunk sizes, or None for the
     uniform split of `total_bytes` by `chunk_bytes`."""
@@ -147,6 +148,11 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
         if out.tiles is None or out.tiles_cap < tiles_capacity:
             out.tiles, out.tiles_cap = _dev_bytes(tiles_capacity * TILE_DESC_DTYPE.itemsize, dev), tiles_capacity
         p.d_tiles, p.tiles_cap = _ptr(out.tiles), out.tiles_cap
+    if workspace:        # lets a long list that needs the scan be scheduled by several workgroups
+        need = int(lib.flh_schedule_workspace_bytes(n))
+        if out.workspace is None or out.workspace.numel() < need:
+            out.workspace = _dev_bytes(need, dev)
+        p.d_workspace, p.workspace_bytes = _ptr(out.workspace), out.workspace.numel()
     check(lib.flh_schedule(C.byref(p), _stream_ptr(stream)))
     return out
 

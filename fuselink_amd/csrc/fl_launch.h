@@ -23,6 +23,7 @@ extern FL_LOCAL int g_fused_fast;          // host-prepared reciprocal for the f
 extern FL_LOCAL int g_nontemporal;         // -1: streaming accesses only when the buffers cannot all sit in the Infinity Cache
 extern FL_LOCAL int g_sched_variant;       // 0 = pick the scheduler shape from the chunk count
 extern FL_LOCAL int g_sched_uniform_fast;
+extern FL_LOCAL int g_sched_seg_min;
 extern FL_LOCAL int g_copy_uniform_grid;
 constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // plain copy: working sets up to this stay largely in the 256 MB Infinity Cache
 constexpr uint64_t kWindowsCacheableBytes = 256ull << 20;  // a message whose staging windows still fit the Infinity Cache

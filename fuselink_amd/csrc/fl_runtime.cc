@@ -27,6 +27,7 @@ int g_fused_fast = 1;
 int g_nontemporal = -1;
 int g_sched_variant = 0;
 int g_sched_uniform_fast = 1;
+int g_sched_seg_min = 8192;    // flh_tune("sched_seg_min"): chunks from which a workspace turns the scan into several workgroups
 int g_copy_uniform_grid = 1;
 
 namespace {
@@ -159,6 +160,11 @@ int flh_tune(const char* key, int64_t value) {
   }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
+  if (!strcmp(key, "sched_seg_min")) {
+    if (value < 1) return fl_set_error(FLH_E_ARG, "sched_seg_min < 1");
+    g_sched_seg_min = (int)(value > 0x7fffffff ? 0x7fffffff : value);
+    return FLH_OK;
+  }
   if (!strcmp(key, "sched_uniform_fast")) { g_sched_uniform_fast = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_variant")) { if (value < 0 || value > 6) return fl_set_error(FLH_E_ARG, "sched_variant not in 0..6"); g_sched_variant = (int)value; return FLH_OK; }
   return fl_set_error(FLH_E_ARG, "unknown tunable %s", key);

@@ -36,7 +36,34 @@ struct SchedArgs {
   int32_t tile_shift;     // >= 0 when tile_bytes is a power of two
   uint32_t inline_credits[FLH_MAX_LANES];  // the one credit row when credits == nullptr
   flh_chunk_desc* table_by_lane;           // optional second copy of the rows in destination order (uniform kernel only)
+  struct SegHeader* seg;                   // caller's workspace when several workgroups share the scan, else null
 };
+
+// Scan scheduler over several workgroups: the chunk list is cut into segments of kSegChunks, one workgroup each.
+// What a segment needs from the ones before it -- bytes of its epoch so far, bytes and tiles of the call so far --
+// depends on the sizes alone and is summed first (fl_sched_seg_totals); the segments are then scheduled side by
+// side with window offsets counted from zero (fl_schedule_kernel, which leaves its per-lane totals here), and a
+// last launch adds every lane's bytes of the earlier segments to the rows and writes header and state
+// (fl_sched_seg_finish).  Three launches and no waiting between workgroups.
+constexpr uint32_t kSegChunks = 1024;      // = one pass of fl_schedule_kernel<8, 2>
+struct SegPartial {
+  uint64_t bytes;          // of the whole segment
+  uint64_t tail;           // from the segment's last epoch head on (the whole segment if it has none)
+  uint32_t tiles;
+  uint32_t has_head;
+  uint64_t lane_bytes[FLH_MAX_LANES];
+  uint32_t lane_chunks[FLH_MAX_LANES];
+  uint32_t flags;
+  uint32_t pad;
+};
+struct SegHeader {         // the carried state as it was when the call began
+  uint64_t lane_off[FLH_MAX_LANES];
+  uint64_t epoch_bytes;
+  uint64_t chunk_index;
+  SegPartial part[1];      // one per segment follows
+};
+__host__ __device__ inline uint32_t seg_count(uint32_t n) { return (n + kSegChunks - 1) / kSegChunks; }
+
 
 
 // Credit rows -> inclusive prefixes, four rows per wavefront: a row of at most 16 lanes fills one
@@ -198,11 +225,56 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   }
   uint64_t off_in = 0;
   if (tid < FLH_MAX_LANES && a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS)) off_in = a.state->lane_off[tid];
+  // this workgroup's part of the chunk list: all of it, or one segment
+  uint32_t n_loc = a.n, i_base = 0;
+  const uint32_t* sizes_p = a.sizes;
+  const uint64_t* srcoff_p = a.src_off;
+  flh_chunk_desc* table_p = a.table;
+  if (a.seg) {
+    const uint32_t g = blockIdx.x;
+    i_base = g * kSegChunks;
+    n_loc = a.n - i_base < kSegChunks ? a.n - i_base : kSegChunks;
+    if (sizes_p) sizes_p += i_base;
+    if (srcoff_p) srcoff_p += i_base;
+    table_p += i_base;
+    off_in = 0;   // window offsets are counted from zero here; the finishing launch adds what lies before
+    // what the earlier segments hand over: their bytes and tiles, and the bytes since the last epoch head among them
+    __shared__ unsigned long long c_run, c_after;
+    __shared__ uint32_t c_tiles;
+    __shared__ int c_head;
+    if (tid == 0) { c_run = 0; c_after = 0; c_tiles = 0; c_head = -1; }
+    __syncthreads();
+    {
+      unsigned long long r = 0;
+      uint32_t t = 0;
+      int h = -1;
+      for (uint32_t q = tid; q < g; q += BT) {
+        r += a.seg->part[q].bytes;
+        t += a.seg->part[q].tiles;
+        if (a.seg->part[q].has_head) h = (int)q;
+      }
+      if (r) atomicAdd(&c_run, r);
+      if (t) atomicAdd(&c_tiles, t);
+      if (h >= 0) atomicMax(&c_head, h);
+    }
+    __syncthreads();
+    const int h = c_head;
+    {
+      unsigned long long r = 0;
+      for (uint32_t q = (uint32_t)(h + 1) + tid; q < g; q += BT) r += a.seg->part[q].bytes;
+      if (r) atomicAdd(&c_after, r);
+    }
+    __syncthreads();
+    p_carry = (h >= 0 ? a.seg->part[h].tail : p_carry) + c_after;
+    run_carry = c_run;
+    tiles_carry = c_tiles;
+    k0 += i_base;
+  }
   uint32_t s_next[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     const uint32_t i = (uint32_t)tid * K + k;
-    s_next[k] = (a.sizes && i < a.n) ? a.sizes[i] : 0;
+    s_next[k] = (sizes_p && i < n_loc) ? sizes_p[i] : 0;
   }
   if (rows_cached) {
     __syncthreads();
@@ -227,7 +299,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
 
   const bool wide = rows_cached && rows_wide != 0;
 #pragma unroll 1
-  for (uint32_t pass = 0; pass < a.n; pass += BT * K) {
+  for (uint32_t pass = 0; pass < n_loc; pass += BT * K) {
     const uint32_t i0 = pass + (uint32_t)tid * K;
     uint32_t s[K], tl[K], row[K], ep[K], ln[K];
     bool head[K];
@@ -250,11 +322,11 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
       const uint32_t i = i0 + k;
       uint32_t sz = 0;
       bool hd = false;
-      if (i < a.n) {
-        if (a.sizes) {
+      if (i < n_loc) {
+        if (sizes_p) {
           sz = s_next[k];
         } else {
-          const uint64_t o = (uint64_t)i * a.chunk_bytes;
+          const uint64_t o = (uint64_t)(i_base + i) * a.chunk_bytes;
           const uint64_t rem = o < a.total_bytes ? a.total_bytes - o : 0;
           sz = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
         }
@@ -275,11 +347,11 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
         if (++r_cur == a.n_rows) r_cur = 0;
       }
     }
-    if (a.sizes) {  // next pass's sizes travel while this pass computes
+    if (sizes_p) {  // next pass's sizes travel while this pass computes
 #pragma unroll
       for (int k = 0; k < K; ++k) {
         const uint64_t i = (uint64_t)i0 + (uint64_t)BT * K + k;
-        s_next[k] = i < a.n ? a.sizes[i] : 0;
+        s_next[k] = i < n_loc ? sizes_p[i] : 0;
       }
     }
     // ---- block-wide exclusive prefixes of (segmented bytes, bytes, tiles) --------------------------
@@ -323,7 +395,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
     for (int k = 0; k < K; ++k) {
       const uint32_t i = i0 + k;
       ln[k] = FLH_MAX_LANES;  // matches no lane: chunks past the end count nowhere
-      if (i < a.n) {
+      if (i < n_loc) {
         if (head[k]) P = 0;
         const uint32_t r = row[k];
         uint64_t W;
@@ -392,15 +464,15 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
       const uint32_t i = i0 + k;
-      if (i < a.n) {
+      if (i < n_loc) {
         flh_chunk_desc d;
-        d.src_off = a.src_off ? a.src_off[i] : a.src_base + run_i;
+        d.src_off = srcoff_p ? srcoff_p[i] : a.src_base + run_i;
         d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : w_lane[wave][ln[k]] + off[k];
         d.len = s[k];
         d.lane = ln[k];
         d.tile_base = tiles_i;
         d.epoch = ep[k];
-        a.table[i] = d;
+        table_p[i] = d;
         run_i += s[k];
         tiles_i += tl[k];
       }
@@ -414,6 +486,15 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   // ---- header and state --------------------------------------------------------------------------------------
   if (__builtin_amdgcn_ballot_w64(flags != 0) && lane == 0) atomicOr(&sh_flags, FLH_SCHED_F_NO_CREDIT);
   __syncthreads();
+  if (a.seg) {   // one segment of several: its per-lane totals go to the workspace, header and state wait for the last launch
+    SegPartial& me = a.seg->part[blockIdx.x];
+    if (tid < FLH_MAX_LANES) {
+      me.lane_bytes[tid] = lane_off[tid];
+      me.lane_chunks[tid] = cnt_lane[tid];
+    }
+    if (tid == 0) me.flags = sh_flags;
+    return;
+  }
   if (tid < FLH_MAX_LANES) {
     a.hdr->lane_bytes[tid] = lane_off[tid] - lane_off0[tid];
     a.hdr->lane_chunks[tid] = cnt_lane[tid];
@@ -428,6 +509,126 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
     if (a.state) {
       a.state->epoch_bytes = p_carry;
       a.state->chunk_index = k0 + a.n;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// scan scheduler over several workgroups: first and last launch
+// ------------------------------------------------------------------------------------------------
+constexpr int kSegBlock = 256;
+
+__device__ __forceinline__ uint32_t seg_chunk_size(const SchedArgs& a, uint32_t i) {
+  if (a.sizes) return a.sizes[i];
+  const uint64_t o = (uint64_t)i * a.chunk_bytes;
+  const uint64_t rem = o < a.total_bytes ? a.total_bytes - o : 0;
+  return (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
+}
+
+// Per segment: bytes, tiles, and the bytes from its last epoch head on.  Epoch heads sit at fixed chunk indices
+// (multiples of epoch_len counted from the carried chunk index), so the last one inside a segment is a division.
+__global__ __launch_bounds__(kSegBlock) void fl_sched_seg_totals(SchedArgs a) {
+  warm_kernel_args(a);
+  const uint32_t g = blockIdx.x, tid = threadIdx.x;
+  const uint32_t lo = g * kSegChunks;
+  const uint32_t hi = a.n - lo < kSegChunks ? a.n : lo + kSegChunks;
+  const uint64_t k0 = a.state ? a.state->chunk_index : 0;
+  uint32_t has_head = 0, head_i = lo;
+  if (a.epoch_len) {
+    const uint64_t last = div_u64(k0 + hi - 1, a.epoch_len) * a.epoch_len;   // global index of the last head at or below hi - 1
+    if (last >= k0 + lo) { has_head = 1; head_i = (uint32_t)(last - k0); }
+  }
+  __shared__ unsigned long long sh_bytes, sh_tail;
+  __shared__ uint32_t sh_tiles;
+  if (tid == 0) { sh_bytes = 0; sh_tail = 0; sh_tiles = 0; }
+  __syncthreads();
+  unsigned long long b = 0, tl = 0;
+  uint32_t t = 0;
+  for (uint32_t i = lo + tid; i < hi; i += kSegBlock) {
+    const uint32_t sz = seg_chunk_size(a, i);
+    b += sz;
+    if (i >= head_i) tl += sz;
+    t += a.tile_shift >= 0 ? (sz + a.tile_bytes - 1) >> a.tile_shift : (sz + a.tile_bytes - 1) / a.tile_bytes;
+  }
+  if (b) atomicAdd(&sh_bytes, b);
+  if (tl) atomicAdd(&sh_tail, tl);
+  if (t) atomicAdd(&sh_tiles, t);
+  __syncthreads();
+  if (tid == 0) {
+    SegPartial& me = a.seg->part[g];
+    me.bytes = sh_bytes;
+    me.tail = sh_tail;
+    me.tiles = sh_tiles;
+    me.has_head = has_head;
+  }
+  if (g == 0) {   // the state as the call found it, for the launches that follow (the last of them overwrites the state)
+    if (tid < FLH_MAX_LANES) a.seg->lane_off[tid] = (a.state && !(a.mode & FLH_SCHED_RESET_OFFSETS)) ? a.state->lane_off[tid] : 0;
+    if (tid == 0) {
+      a.seg->epoch_bytes = (a.state && !(a.mode & FLH_SCHED_NEW_EPOCH)) ? a.state->epoch_bytes : 0;
+      a.seg->chunk_index = k0;
+    }
+  }
+}
+
+// Window offsets of a segment's rows start where the earlier segments left each lane; the workgroup of the last
+// segment also sums everything up into header and state.
+__global__ __launch_bounds__(kSegBlock) void fl_sched_seg_finish(SchedArgs a) {
+  warm_kernel_args(a);
+  const uint32_t g = blockIdx.x, tid = threadIdx.x, G = gridDim.x;
+  const uint32_t lo = g * kSegChunks;
+  const uint32_t hi = a.n - lo < kSegChunks ? a.n : lo + kSegChunks;
+  __shared__ unsigned long long base[FLH_MAX_LANES];
+  if (tid < FLH_MAX_LANES) base[tid] = a.seg->lane_off[tid];
+  __syncthreads();
+  for (uint32_t e = tid; e < g * FLH_MAX_LANES; e += kSegBlock) {
+    const unsigned long long v = a.seg->part[e / FLH_MAX_LANES].lane_bytes[e % FLH_MAX_LANES];
+    if (v) atomicAdd(&base[e % FLH_MAX_LANES], v);
+  }
+  __syncthreads();
+  if (!(a.mode & FLH_SCHED_MIRROR)) {
+    for (uint32_t i = lo + tid; i < hi; i += kSegBlock) {
+      const uint32_t ln = a.table[i].lane;
+      a.table[i].win_off += base[ln < FLH_MAX_LANES ? ln : 0];
+    }
+  }
+  if (g != G - 1) return;
+  // ---- header and state, from every segment's partials ----------------------------------------------------
+  __shared__ unsigned long long t_bytes, t_after, t_lane[FLH_MAX_LANES];
+  __shared__ uint32_t t_tiles, t_flags, t_cnt[FLH_MAX_LANES];
+  __shared__ int t_head;
+  if (tid < FLH_MAX_LANES) { t_lane[tid] = 0; t_cnt[tid] = 0; }
+  if (tid == 0) { t_bytes = 0; t_after = 0; t_tiles = 0; t_flags = 0; t_head = -1; }
+  __syncthreads();
+  for (uint32_t e = tid; e < G * FLH_MAX_LANES; e += kSegBlock) {
+    const SegPartial& p = a.seg->part[e / FLH_MAX_LANES];
+    const uint32_t l = e % FLH_MAX_LANES;
+    if (p.lane_bytes[l]) atomicAdd(&t_lane[l], (unsigned long long)p.lane_bytes[l]);
+    if (p.lane_chunks[l]) atomicAdd(&t_cnt[l], p.lane_chunks[l]);
+    if (l == 0) {
+      atomicAdd(&t_bytes, (unsigned long long)p.bytes);
+      atomicAdd(&t_tiles, p.tiles);
+      if (p.flags) atomicOr(&t_flags, p.flags);
+      if (p.has_head) atomicMax(&t_head, (int)(e / FLH_MAX_LANES));
+    }
+  }
+  __syncthreads();
+  const int h = t_head;
+  for (uint32_t q = (uint32_t)(h + 1) + tid; q < G; q += kSegBlock) atomicAdd(&t_after, (unsigned long long)a.seg->part[q].bytes);
+  __syncthreads();
+  if (tid < FLH_MAX_LANES) {
+    a.hdr->lane_bytes[tid] = t_lane[tid];
+    a.hdr->lane_chunks[tid] = t_cnt[tid];
+    if (a.state) a.state->lane_off[tid] = a.seg->lane_off[tid] + t_lane[tid];
+  }
+  if (tid == 0) {
+    a.hdr->total_bytes = t_bytes;
+    a.hdr->total_tiles = t_tiles;
+    a.hdr->n_chunks = a.n;
+    a.hdr->flags = t_flags;
+    a.hdr->uniform_tiles = (!a.sizes && a.n) ? (a.chunk_bytes + a.tile_bytes - 1) / a.tile_bytes : 0;
+    if (a.state) {
+      a.state->epoch_bytes = (h >= 0 ? a.seg->part[h].tail : a.seg->epoch_bytes) + t_after;
+      a.state->chunk_index = a.seg->chunk_index + a.n;
     }
   }
 }
@@ -690,6 +891,10 @@ __global__ __launch_bounds__(kExpandBlock) void fl_expand_tiles(const flh_chunk_
 
 extern "C" {
 
+uint64_t flh_schedule_workspace_bytes(uint32_t n_chunks) {
+  return sizeof(SegHeader) + (uint64_t)seg_count(n_chunks) * sizeof(SegPartial);
+}
+
 static int expand_tiles(const flh_sched_params* p, hipStream_t s) {
   if (!p->d_tiles || p->n_chunks == 0) return FLH_OK;
   const uint32_t per_block = kExpandBlock / kWave;
@@ -730,6 +935,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   a.table = p->d_table;
   a.hdr = p->d_hdr;
   a.table_by_lane = p->d_table_by_lane;
+  a.seg = nullptr;
   a.chunk_bytes = p->chunk_bytes;
   a.n = p->n_chunks;
   a.n_lanes = p->n_lanes;
@@ -749,6 +955,19 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     const uint32_t grid = (n + kUniBlock - 1) / kUniBlock;
     FL_LAUNCH((fl_schedule_uniform_kernel<0>), dim3(grid), dim3(kUniBlock), 0, s, a);
     if (grid > 1 && p->d_state) FL_LAUNCH((fl_schedule_uniform_kernel<1>), dim3(1), dim3(kUniBlock), 0, s, a);
+    FL_HIP(hipGetLastError());
+    return expand_tiles(p, s);
+  }
+  // a long list with a workspace: one workgroup per kSegChunks chunks, three launches
+  if (p->d_workspace && variant == 0 && n >= (uint32_t)g_sched_seg_min && p->n_rows <= (uint32_t)kRowCache && !p->d_table_by_lane) {
+    const uint32_t G = seg_count(n);
+    const uint64_t need = flh_schedule_workspace_bytes(n);
+    if (p->workspace_bytes < need) return fl_set_error(FLH_E_ARG, "workspace of %llu bytes, %llu needed for %u chunks", (unsigned long long)p->workspace_bytes,
+                                                        (unsigned long long)need, n);
+    a.seg = (SegHeader*)p->d_workspace;
+    FL_LAUNCH(fl_sched_seg_totals, dim3(G), dim3(kSegBlock), 0, s, a);
+    FL_LAUNCH((fl_schedule_kernel<8, 2>), dim3(G), dim3(8 * kWave), 0, s, a);
+    FL_LAUNCH(fl_sched_seg_finish, dim3(G), dim3(kSegBlock), 0, s, a);
     FL_HIP(hipGetLastError());
     return expand_tiles(p, s);
   }

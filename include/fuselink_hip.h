@@ -116,12 +116,19 @@ typedef struct flh_sched_params {
                                     which pays from a few thousand rows of unequal size on */
   uint32_t tiles_cap;          /* descriptors d_tiles holds; total_bytes / tile_bytes + n_chunks always suffices */
   uint32_t pad_;
+  void* d_workspace;           /* optional: flh_schedule_workspace_bytes(n_chunks) bytes of device memory; with it a
+                                  chunk list of 8192 chunks or more that needs the scan (d_sizes, d_src_off or
+                                  quantum != chunk_bytes) is scheduled by one workgroup per 1024 chunks in three
+                                  launches instead of by one workgroup; same table, header and state */
+  uint64_t workspace_bytes;
 } flh_sched_params;
 
 /* ---- library ------------------------------------------------------------------------------ */
 /* Selects `device`, checks that it is a gfx950 part, loads kernel attributes.  Idempotent. */
 int flh_init(int device);
 const char* flh_last_error(void);
+/* bytes of flh_sched_params.d_workspace that flh_schedule needs for n_chunks chunks */
+uint64_t flh_schedule_workspace_bytes(uint32_t n_chunks);
 /* compile-time facts: 0 tile bytes, 1 max lanes, 2 unit bytes, 3 pool units, 4 sizeof(desc),
  * 5 sizeof(state), 6 sizeof(hdr), 7 ABI version, 8 sizeof(flh_windows), 9 sizeof(flh_sched_params) */
 int64_t flh_constant(int which);

@@ -21,7 +21,7 @@ def _dev(torch, a):
 
 
 def _check_schedule(fl, *, n_lanes, credits, quantum, sizes=None, total_bytes=0, chunk_bytes=0, epoch_len=0,
-                    tile_bytes=32768, mode=0, state=None, src_off=None, src_base=0):
+                    tile_bytes=32768, mode=0, state=None, src_off=None, src_base=0, workspace=False):
     core, torch = fl
     credits = np.asarray(credits, dtype=np.uint32).reshape(-1, n_lanes)
     exp_t, exp_h, exp_s = ob.credit_schedule(n_lanes=n_lanes, credits=credits, quantum=quantum, sizes=sizes,
@@ -34,7 +34,7 @@ def _check_schedule(fl, *, n_lanes, credits, quantum, sizes=None, total_bytes=0,
     sched = core.schedule(n_lanes=n_lanes, credits=_dev(torch, credits.view(np.int32)), quantum=quantum,
                           sizes=None if sizes is None else _dev(torch, np.asarray(sizes, dtype=np.uint32).view(np.int32)),
                           total_bytes=total_bytes, chunk_bytes=chunk_bytes, epoch_len=epoch_len, tile_bytes=tile_bytes,
-                          mode=mode, state=d_state, src_base=src_base,
+                          mode=mode, state=d_state, src_base=src_base, workspace=workspace,
                           src_off=None if src_off is None else _dev(torch, np.asarray(src_off, dtype=np.uint64).view(np.int64)))
     torch.cuda.synchronize()
     got_t, got_h = sched.table_numpy(), sched.hdr_numpy()
@@ -783,3 +783,60 @@ def test_tile_descriptor_array_too_small_is_refused(fl):
     hint.total_tiles, hint.n_chunks = 120, 40
     with pytest.raises(Exception, match="120 tiles"):
         core.stripe(src, w, sched, status, hint=hint)  # the host copy of the header says so before anything is launched
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_scan_scheduler_over_several_workgroups_equals_oracle(fl, seed):
+    """With a workspace a long list is scheduled by one workgroup per 1024 chunks in three launches; table, header
+    and carried state must be the one-workgroup kernel's, i.e. the oracle's: variable and uniform sizes, epochs that
+    start inside, at the edge of and nowhere near a segment, several credit rows (a rowless one among them), explicit
+    source offsets, carried state from an earlier call, every mode bit."""
+    core, torch = fl
+    rng = np.random.default_rng(4100 + seed)
+    lanes = int(rng.integers(1, 17))
+    n = int(rng.choice([1, 700, 1024, 1025, 2048, 3000, 4097, 9000]))
+    rows = int(rng.integers(1, 6))
+    credits = rng.integers(0, 9, size=(rows, lanes)).astype(np.uint32)
+    if seed % 4 == 0 and rows > 1:
+        credits[1, :] = 0
+    epoch_len = int(rng.choice([0, 7, 512, 1024, 1000, 5000]))
+    quantum = int(rng.choice([1, 4096, 65536, 100000]))
+    tile = int(rng.choice([128, 4096, 32768]))
+    mode = int(rng.choice([0, 1, 2, 4, 5]))
+    state = None
+    if seed % 2:
+        state = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+        state["epoch_bytes"] = int(rng.integers(0, 1 << 22))
+        state["chunk_index"] = int(rng.integers(0, 3000))
+        state["lane_off"][:lanes] = rng.integers(0, 1 << 30, size=lanes)
+    kw = dict(n_lanes=lanes, credits=credits, quantum=quantum, epoch_len=epoch_len, tile_bytes=tile, mode=mode, state=state, workspace=True)
+    core.tune("sched_seg_min", 1)
+    try:
+        if seed % 3 == 2:      # uniform sizes that still need the scan (quantum != chunk)
+            chunk = int(rng.choice([4096, 50000]))
+            total = n * chunk - int(rng.integers(0, chunk))
+            if quantum == chunk:
+                kw["quantum"] = chunk + 1
+            _check_schedule(fl, total_bytes=total, chunk_bytes=chunk, src_base=int(rng.integers(0, 1 << 20)), **kw)
+        else:
+            sizes = rng.integers(0, int(rng.choice([300, 9000, 200000])), size=n).astype(np.uint32)
+            src_off = None
+            if seed % 3 == 1:
+                src_off = (np.concatenate([[5], sizes[:-1].astype(np.uint64) + 3]).cumsum()).astype(np.uint64)
+            _check_schedule(fl, sizes=sizes, src_off=src_off, **kw)
+    finally:
+        core.tune("sched_seg_min", 8192)
+
+
+def test_scan_scheduler_workspace_too_small_is_refused(fl):
+    core, torch = fl
+    sizes = _dev(torch, np.full(9000, 4096, dtype=np.int32))
+    out = core.new_schedule_buffers(9000)
+    out.workspace = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    with pytest.raises(Exception, match="workspace"):
+        import ctypes as C
+        from fuselink_amd import _lib
+        p = _lib.SchedParams(sizes.data_ptr(), 0, 0, None, 0, 9000, 2, None, 1, 0, 4096, 32768, 0, None, out.table.data_ptr(), out.hdr.data_ptr())
+        p.inline_credits[0] = p.inline_credits[1] = 1
+        p.d_workspace, p.workspace_bytes = out.workspace.data_ptr(), 64
+        _lib.check(_lib.load().flh_schedule(C.byref(p), None))
