@@ -35,8 +35,8 @@ WORKLOADS = {
 # HBM bytes per launch of the striping kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size.
 # None where no such run has been recorded for the workload.
-MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134289278, "cfg5_stress_1GiB_64KiB_16lanes": 2151685750,
-                    "cfg3_expert_parallel_256_blocks_8lanes": 1786051408, "cfg4_paged_kv_2x4096_pages_8lanes": 268684250}
+MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134288509, "cfg5_stress_1GiB_64KiB_16lanes": 2151675086,
+                    "cfg3_expert_parallel_256_blocks_8lanes": 1786036451, "cfg4_paged_kv_2x4096_pages_8lanes": 268670118}
 
 
 def algo_bytes_cold(nbytes: int) -> int:

@@ -179,7 +179,7 @@ __device__ __forceinline__ void lane_pass_columns(const uint32_t (&s)[K], const 
 // consecutive chunks of a pass.  Per pass: thread-local sums, three wavefront scans (epoch-segmented
 // bytes, bytes, tiles), the lane of each chunk from its quantum slot, one wavefront scan per lane
 // for the window offsets.  LDS only carries per-wavefront totals and the running lane offsets.
-template <int NW, int K>
+template <int NW, int K, bool SEG = false>
 __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   warm_kernel_args(a);
   constexpr int BT = NW * kWave;
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   const uint32_t* sizes_p = a.sizes;
   const uint64_t* srcoff_p = a.src_off;
   flh_chunk_desc* table_p = a.table;
-  if (a.seg) {
+  if constexpr (SEG) {
     const uint32_t g = blockIdx.x;
     i_base = g * kSegChunks;
     n_loc = a.n - i_base < kSegChunks ? a.n - i_base : kSegChunks;
@@ -486,7 +486,7 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   // ---- header and state --------------------------------------------------------------------------------------
   if (__builtin_amdgcn_ballot_w64(flags != 0) && lane == 0) atomicOr(&sh_flags, FLH_SCHED_F_NO_CREDIT);
   __syncthreads();
-  if (a.seg) {   // one segment of several: its per-lane totals go to the workspace, header and state wait for the last launch
+  if constexpr (SEG) {   // one segment of several: its per-lane totals go to the workspace, header and state wait for the last launch
     SegPartial& me = a.seg->part[blockIdx.x];
     if (tid < FLH_MAX_LANES) {
       me.lane_bytes[tid] = lane_off[tid];
@@ -966,7 +966,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
                                                         (unsigned long long)need, n);
     a.seg = (SegHeader*)p->d_workspace;
     FL_LAUNCH(fl_sched_seg_totals, dim3(G), dim3(kSegBlock), 0, s, a);
-    FL_LAUNCH((fl_schedule_kernel<8, 2>), dim3(G), dim3(8 * kWave), 0, s, a);
+    FL_LAUNCH((fl_schedule_kernel<8, 2, true>), dim3(G), dim3(8 * kWave), 0, s, a);
     FL_LAUNCH(fl_sched_seg_finish, dim3(G), dim3(kSegBlock), 0, s, a);
     FL_HIP(hipGetLastError());
     return expand_tiles(p, s);
