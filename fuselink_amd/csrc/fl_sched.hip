@@ -964,6 +964,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     const uint64_t need = flh_schedule_workspace_bytes(n);
     if (p->workspace_bytes < need) return fl_set_error(FLH_E_ARG, "workspace of %llu bytes, %llu needed for %u chunks", (unsigned long long)p->workspace_bytes,
                                                         (unsigned long long)need, n);
+    if ((uintptr_t)p->d_workspace % alignof(SegHeader)) return fl_set_error(FLH_E_ARG, "workspace must be %zu-byte aligned", alignof(SegHeader));
     a.seg = (SegHeader*)p->d_workspace;
     FL_LAUNCH(fl_sched_seg_totals, dim3(G), dim3(kSegBlock), 0, s, a);
     FL_LAUNCH((fl_schedule_kernel<8, 2, true>), dim3(G), dim3(8 * kWave), 0, s, a);

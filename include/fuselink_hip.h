@@ -116,7 +116,7 @@ typedef struct flh_sched_params {
                                     which pays from a few thousand rows of unequal size on */
   uint32_t tiles_cap;          /* descriptors d_tiles holds; total_bytes / tile_bytes + n_chunks always suffices */
   uint32_t pad_;
-  void* d_workspace;           /* optional: flh_schedule_workspace_bytes(n_chunks) bytes of device memory; with it a
+  void* d_workspace;           /* optional: flh_schedule_workspace_bytes(n_chunks) bytes of 8-byte aligned device memory; with it a
                                   chunk list of 8192 chunks or more that needs the scan (d_sizes, d_src_off or
                                   quantum != chunk_bytes) is scheduled by one workgroup per 1024 chunks in three
                                   launches instead of by one workgroup; same table, header and state */
