@@ -840,3 +840,49 @@ def test_scan_scheduler_workspace_too_small_is_refused(fl):
         p.inline_credits[0] = p.inline_credits[1] = 1
         p.d_workspace, p.workspace_bytes = out.workspace.data_ptr(), 64
         _lib.check(_lib.load().flh_schedule(C.byref(p), None))
+
+
+def test_long_variable_list_records_into_a_hip_graph(fl):
+    """The scan over several workgroups, the expansion to tile descriptors and the copies that read them are plain
+    launches too: recorded once, replayed with new sizes and bytes in the same buffers, checked against the oracle."""
+    core, torch = fl
+    rng = np.random.default_rng(2718)
+    lanes, n, tile = 7, 9000, 4096
+    credits = rng.integers(0, 6, size=(3, lanes)).astype(np.uint32)
+    cap_bytes = n * 3000
+    src = torch.zeros(cap_bytes, dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    sizes = torch.zeros(n, dtype=torch.int32, device="cuda")
+    wins = [torch.zeros(cap_bytes, dtype=torch.uint8, device="cuda") for _ in range(lanes)]
+    w = core.make_windows([t.data_ptr() for t in wins], [cap_bytes] * lanes)
+    d_credits = _dev(torch, credits.view(np.int32))
+    status = core.new_status()
+    sched = core.new_schedule_buffers(n, tile_bytes=tile)
+    tiles_capacity = cap_bytes // tile + n
+    # buffers the graph will use must exist before the capture: one eager call allocates workspace and descriptors
+    core.schedule(n_lanes=lanes, credits=d_credits, quantum=2048, sizes=sizes, epoch_len=1000, tile_bytes=tile, out=sched,
+                  tiles_capacity=tiles_capacity, workspace=True)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        core.schedule(n_lanes=lanes, credits=d_credits, quantum=2048, sizes=sizes, epoch_len=1000, tile_bytes=tile, out=sched,
+                      tiles_capacity=tiles_capacity, workspace=True)
+        core.stripe(src, w, sched, status)
+        core.reassemble(dst, w, sched, status)
+    for rep in range(3):
+        sizes_np = rng.integers(0, 3000, size=n).astype(np.uint32)
+        total = int(sizes_np.sum())
+        src_np = rng.integers(0, 256, size=cap_bytes, dtype=np.uint8)
+        sizes.copy_(torch.from_numpy(sizes_np.view(np.int32)))
+        src.copy_(torch.from_numpy(src_np))
+        dst.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+        exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=2048, sizes=sizes_np, epoch_len=1000, tile_bytes=tile)
+        assert sched.table_numpy().tobytes() == exp_t.tobytes(), f"replay {rep}"
+        np.testing.assert_array_equal(dst.cpu().numpy()[:total], src_np[:total], err_msg=f"replay {rep}")
+        assert not dst[total:].any()
