@@ -188,7 +188,9 @@ int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
 
 /* The same pair driven by the per-tile descriptors that flh_schedule wrote to d_tiles (tiles_cap entries).  The
  * number of tiles comes from h_hdr when given, else from d_hdr; a table with more tiles than tiles_cap is refused
- * through *d_status (FLH_E_RANGE), and so is a descriptor that would leave the buffer or its window. */
+ * through *d_status (FLH_E_RANGE), and so is a descriptor that would leave the buffer or its window.  Like the
+ * scheduler itself these have no counterpart in the reference, whose transport posts one contiguous buffer per
+ * request (src/plugin.cc:1467-1495). */
 int flh_stripe_tiles(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_tile_desc* d_tiles,
                      uint32_t tiles_cap, const flh_sched_hdr* d_hdr, const flh_sched_hdr* h_hdr, int32_t* d_status, void* stream);
 int flh_reassemble_tiles(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_tile_desc* d_tiles,
