@@ -50,7 +50,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2_grad_bucket_64MiB_256KiB_8lanes", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-iters", type=int, default=60)
+    ap.add_argument("--cpu-iters", type=int, default=1000, help="timed CPU passes at 64 MiB (scaled down for larger messages): about 5 s of CPU work per figure")
     ap.add_argument("--hint", type=int, default=1, help="pass the host-known header fields to the copy kernels")
     ap.add_argument("--path", default="auto", choices=["auto", "fused", "split"],
                     help="fused: scheduler folded into the striping launch (uniform split, one credit row); split: three launches")
@@ -335,7 +335,7 @@ def main() -> int:
             tab, h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits_np, quantum=chunk, total_bytes=msg_bytes, chunk_bytes=chunk)
             caps = h["lane_bytes"][:lanes]
             ts = []
-            for _ in range(max(3, args.cpu_iters // 12)):
+            for _ in range(max(3, args.cpu_iters // 100)):
                 c0 = time.perf_counter()
                 for half_i in range(2):
                     half = src_np[half_i * msg_bytes: (half_i + 1) * msg_bytes]
