@@ -403,6 +403,7 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.idle_credit = (int)fl_param("FUSELINK_IDLE_CREDIT", g_par.idle_credit);
   g_par.max_wave_chunks = (int)fl_param("FUSELINK_MAX_WAVE_CHUNKS", g_par.max_wave_chunks);
   g_par.batch = (int)fl_param("FUSELINK_BATCH", g_par.batch);
+  if (g_par.max_wave_chunks > 65535) g_par.max_wave_chunks = 65535;   // what one fused launch can name
   if (g_par.batch < 1) g_par.batch = 1;
   if (g_par.batch > FLH_BATCH_MAX) g_par.batch = FLH_BATCH_MAX;
   if (g_par.lanes < 1 || g_par.lanes > FL_NET_MAX_LANES) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_LANES must be 1..%d", FL_NET_MAX_LANES); return ncclInvalidArgument; }
