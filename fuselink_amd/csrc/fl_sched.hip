@@ -967,6 +967,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     if ((uintptr_t)p->d_workspace % alignof(SegHeader)) return fl_set_error(FLH_E_ARG, "workspace must be %zu-byte aligned", alignof(SegHeader));
     a.seg = (SegHeader*)p->d_workspace;
     FL_LAUNCH(fl_sched_seg_totals, dim3(G), dim3(kSegBlock), 0, s, a);
+    static_assert(kSegChunks == 8 * kWave * 2, "a segment is one pass of fl_schedule_kernel<8, 2>");
     FL_LAUNCH((fl_schedule_kernel<8, 2, true>), dim3(G), dim3(8 * kWave), 0, s, a);
     FL_LAUNCH(fl_sched_seg_finish, dim3(G), dim3(kSegBlock), 0, s, a);
     FL_HIP(hipGetLastError());
