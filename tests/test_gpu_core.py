@@ -829,16 +829,20 @@ def test_scan_scheduler_over_several_workgroups_equals_oracle(fl, seed):
 
 
 def test_scan_scheduler_workspace_too_small_is_refused(fl):
+    """A workspace that cannot hold the partials of every segment is an argument error, raised before any launch."""
+    import ctypes as C
+
+    from fuselink_amd import _lib
     core, torch = fl
-    sizes = _dev(torch, np.full(9000, 4096, dtype=np.int32))
-    out = core.new_schedule_buffers(9000)
-    out.workspace = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    n = 9000
+    sizes = _dev(torch, np.full(n, 4096, dtype=np.int32))
+    out = core.new_schedule_buffers(n)
+    small = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    p = _lib.SchedParams(sizes.data_ptr(), 0, 0, None, 0, n, 2, None, 1, 0, 4096, 32768, 0, None, out.table.data_ptr(), out.hdr.data_ptr())
+    p.inline_credits[0] = p.inline_credits[1] = 1
+    p.d_workspace, p.workspace_bytes = small.data_ptr(), small.numel()
+    assert int(_lib.load().flh_schedule_workspace_bytes(n)) > small.numel()
     with pytest.raises(Exception, match="workspace"):
-        import ctypes as C
-        from fuselink_amd import _lib
-        p = _lib.SchedParams(sizes.data_ptr(), 0, 0, None, 0, 9000, 2, None, 1, 0, 4096, 32768, 0, None, out.table.data_ptr(), out.hdr.data_ptr())
-        p.inline_credits[0] = p.inline_credits[1] = 1
-        p.d_workspace, p.workspace_bytes = out.workspace.data_ptr(), 64
         _lib.check(_lib.load().flh_schedule(C.byref(p), None))
 
 
