@@ -2,6 +2,7 @@
 the request machinery, the FIFO handshake and the error convention are checked without a GPU.
 Host buffers are never staged (FuseLink src/fuselink.cc:8-13), so no kernel is involved here."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -270,3 +271,19 @@ def test_cuda_pointer_fails_loudly_without_gpu(net):
     rc, mh = net.regMr(s, sp, 4096, P.NCCL_PTR_CUDA)
     assert rc == P.ncclUnhandledCudaError and mh is None  # no CPU fallback for device memory
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+@pytest.mark.parametrize("header", ["fuselink_hip.h", "fuselink_net.h"])
+def test_headers_are_plain_c(header, tmp_path):
+    """The boundary is a C ABI: both headers must compile as C99 with nothing else included before them."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if not gcc:
+        pytest.skip("no C compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "use.c"
+    src.write_text(f'#include "{header}"\nint main(void) {{ return 0; }}\n')
+    res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I" + os.path.join(root, "include"), str(src)],
+                         capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
