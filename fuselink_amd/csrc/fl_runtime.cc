@@ -27,7 +27,7 @@ int g_fused_fast = 1;
 int g_nontemporal = -1;
 int g_sched_variant = 0;
 int g_sched_uniform_fast = 1;
-int g_sched_seg_min = 8192;    // flh_tune("sched_seg_min"): chunks from which a workspace turns the scan into several workgroups
+int g_sched_seg_min = 4096;    // flh_tune("sched_seg_min"): chunks from which a workspace turns the scan into several workgroups
 int g_copy_uniform_grid = 1;
 
 namespace {

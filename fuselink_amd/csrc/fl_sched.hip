@@ -538,11 +538,10 @@ __global__ __launch_bounds__(kSegBlock) void fl_sched_seg_totals(SchedArgs a) {
     const uint64_t last = div_u64(k0 + hi - 1, a.epoch_len) * a.epoch_len;   // global index of the last head at or below hi - 1
     if (last >= k0 + lo) { has_head = 1; head_i = (uint32_t)(last - k0); }
   }
-  __shared__ unsigned long long sh_bytes, sh_tail;
-  __shared__ uint32_t sh_tiles;
-  if (tid == 0) { sh_bytes = 0; sh_tail = 0; sh_tiles = 0; }
-  __syncthreads();
-  unsigned long long b = 0, tl = 0;
+  constexpr int kWaves = kSegBlock / kWave;
+  __shared__ uint64_t sh_bytes[kWaves], sh_tail[kWaves];
+  __shared__ uint32_t sh_tiles[kWaves];
+  uint64_t b = 0, tl = 0;
   uint32_t t = 0;
   for (uint32_t i = lo + tid; i < hi; i += kSegBlock) {
     const uint32_t sz = seg_chunk_size(a, i);
@@ -550,15 +549,21 @@ __global__ __launch_bounds__(kSegBlock) void fl_sched_seg_totals(SchedArgs a) {
     if (i >= head_i) tl += sz;
     t += a.tile_shift >= 0 ? (sz + a.tile_bytes - 1) >> a.tile_shift : (sz + a.tile_bytes - 1) / a.tile_bytes;
   }
-  if (b) atomicAdd(&sh_bytes, b);
-  if (tl) atomicAdd(&sh_tail, tl);
-  if (t) atomicAdd(&sh_tiles, t);
+  const int lane = tid & (kWave - 1);
+  b = wave_incl_sum_u64(b, lane);
+  tl = wave_incl_sum_u64(tl, lane);
+  t = wave_incl_sum_u32(t, lane);
+  if (lane == kWave - 1) { sh_bytes[tid / kWave] = b; sh_tail[tid / kWave] = tl; sh_tiles[tid / kWave] = t; }
   __syncthreads();
   if (tid == 0) {
     SegPartial& me = a.seg->part[g];
-    me.bytes = sh_bytes;
-    me.tail = sh_tail;
-    me.tiles = sh_tiles;
+    uint64_t sb = 0, st = 0;
+    uint32_t sn = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) { sb += sh_bytes[w]; st += sh_tail[w]; sn += sh_tiles[w]; }
+    me.bytes = sb;
+    me.tail = st;
+    me.tiles = sn;
     me.has_head = has_head;
   }
   if (g == 0) {   // the state as the call found it, for the launches that follow (the last of them overwrites the state)
@@ -577,12 +582,22 @@ __global__ __launch_bounds__(kSegBlock) void fl_sched_seg_finish(SchedArgs a) {
   const uint32_t g = blockIdx.x, tid = threadIdx.x, G = gridDim.x;
   const uint32_t lo = g * kSegChunks;
   const uint32_t hi = a.n - lo < kSegChunks ? a.n : lo + kSegChunks;
-  __shared__ unsigned long long base[FLH_MAX_LANES];
-  if (tid < FLH_MAX_LANES) base[tid] = a.seg->lane_off[tid];
+  // every lane's bytes in the earlier segments: thread (q, l) sums the segments q, q + 16, ... for lane l
+  constexpr int kQ = kSegBlock / FLH_MAX_LANES;
+  __shared__ uint64_t part_sum[kQ][FLH_MAX_LANES];
+  __shared__ uint64_t base[FLH_MAX_LANES];
+  {
+    const uint32_t q = tid / FLH_MAX_LANES, l = tid % FLH_MAX_LANES;
+    uint64_t v = 0;
+    for (uint32_t s = q; s < g; s += kQ) v += a.seg->part[s].lane_bytes[l];
+    part_sum[q][l] = v;
+  }
   __syncthreads();
-  for (uint32_t e = tid; e < g * FLH_MAX_LANES; e += kSegBlock) {
-    const unsigned long long v = a.seg->part[e / FLH_MAX_LANES].lane_bytes[e % FLH_MAX_LANES];
-    if (v) atomicAdd(&base[e % FLH_MAX_LANES], v);
+  if (tid < FLH_MAX_LANES) {
+    uint64_t v = a.seg->lane_off[tid];
+#pragma unroll
+    for (int q = 0; q < kQ; ++q) v += part_sum[q][tid];
+    base[tid] = v;
   }
   __syncthreads();
   if (!(a.mode & FLH_SCHED_MIRROR)) {
@@ -599,21 +614,38 @@ __global__ __launch_bounds__(kSegBlock) void fl_sched_seg_finish(SchedArgs a) {
   if (tid < FLH_MAX_LANES) { t_lane[tid] = 0; t_cnt[tid] = 0; }
   if (tid == 0) { t_bytes = 0; t_after = 0; t_tiles = 0; t_flags = 0; t_head = -1; }
   __syncthreads();
-  for (uint32_t e = tid; e < G * FLH_MAX_LANES; e += kSegBlock) {
-    const SegPartial& p = a.seg->part[e / FLH_MAX_LANES];
-    const uint32_t l = e % FLH_MAX_LANES;
-    if (p.lane_bytes[l]) atomicAdd(&t_lane[l], (unsigned long long)p.lane_bytes[l]);
-    if (p.lane_chunks[l]) atomicAdd(&t_cnt[l], p.lane_chunks[l]);
+  {
+    const uint32_t q = tid / FLH_MAX_LANES, l = tid % FLH_MAX_LANES;
+    unsigned long long lb = 0, by = 0;
+    uint32_t lc = 0, ti = 0, fl = 0;
+    int hd = -1;
+    for (uint32_t s = q; s < G; s += kQ) {
+      const SegPartial& p = a.seg->part[s];
+      lb += p.lane_bytes[l];
+      lc += p.lane_chunks[l];
+      if (l == 0) {
+        by += p.bytes;
+        ti += p.tiles;
+        fl |= p.flags;
+        if (p.has_head) hd = (int)s;
+      }
+    }
+    if (lb) atomicAdd(&t_lane[l], lb);     // sixteen adds per lane at most
+    if (lc) atomicAdd(&t_cnt[l], lc);
     if (l == 0) {
-      atomicAdd(&t_bytes, (unsigned long long)p.bytes);
-      atomicAdd(&t_tiles, p.tiles);
-      if (p.flags) atomicOr(&t_flags, p.flags);
-      if (p.has_head) atomicMax(&t_head, (int)(e / FLH_MAX_LANES));
+      if (by) atomicAdd(&t_bytes, by);
+      if (ti) atomicAdd(&t_tiles, ti);
+      if (fl) atomicOr(&t_flags, fl);
+      if (hd >= 0) atomicMax(&t_head, hd);
     }
   }
   __syncthreads();
   const int h = t_head;
-  for (uint32_t q = (uint32_t)(h + 1) + tid; q < G; q += kSegBlock) atomicAdd(&t_after, (unsigned long long)a.seg->part[q].bytes);
+  {
+    unsigned long long af = 0;
+    for (uint32_t q = (uint32_t)(h + 1) + tid; q < G; q += kSegBlock) af += a.seg->part[q].bytes;
+    if (af) atomicAdd(&t_after, af);
+  }
   __syncthreads();
   if (tid < FLH_MAX_LANES) {
     a.hdr->lane_bytes[tid] = t_lane[tid];

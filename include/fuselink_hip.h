@@ -117,7 +117,7 @@ typedef struct flh_sched_params {
   uint32_t tiles_cap;          /* descriptors d_tiles holds; total_bytes / tile_bytes + n_chunks always suffices */
   uint32_t pad_;
   void* d_workspace;           /* optional: flh_schedule_workspace_bytes(n_chunks) bytes of 8-byte aligned device memory; with it a
-                                  chunk list of 8192 chunks or more that needs the scan (d_sizes, d_src_off or
+                                  chunk list of 4096 chunks or more that needs the scan (d_sizes, d_src_off or
                                   quantum != chunk_bytes) is scheduled by one workgroup per 1024 chunks in three
                                   launches instead of by one workgroup; same table, header and state */
   uint64_t workspace_bytes;
@@ -140,7 +140,7 @@ int64_t flh_constant(int which);
  * bit 1 stores; -1 = the policy).
  * "stripe_dest_order" = 0/1: flh_stripe_uniform walks the chunks lane by lane, so that every window is written
  * front to back (-1 = only for messages past 256 MiB, whose windows no longer fit the Infinity Cache, the default).
- * "sched_seg_min" = chunks from which a lent workspace makes the scan scheduler use several workgroups (8192).
+ * "sched_seg_min" = chunks from which a lent workspace makes the scan scheduler use several workgroups (4096).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL.
  * The tunables are process-wide and read by every launch: set them while no other thread launches. */
 int flh_tune(const char* key, int64_t value);

@@ -825,7 +825,7 @@ def test_scan_scheduler_over_several_workgroups_equals_oracle(fl, seed):
                 src_off = (np.concatenate([[5], sizes[:-1].astype(np.uint64) + 3]).cumsum()).astype(np.uint64)
             _check_schedule(fl, sizes=sizes, src_off=src_off, **kw)
     finally:
-        core.tune("sched_seg_min", 8192)
+        core.tune("sched_seg_min", 4096)
 
 
 def test_scan_scheduler_workspace_too_small_is_refused(fl):
