@@ -238,36 +238,6 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
     if (srcoff_p) srcoff_p += i_base;
     table_p += i_base;
     off_in = 0;   // window offsets are counted from zero here; the finishing launch adds what lies before
-    // what the earlier segments hand over: their bytes and tiles, and the bytes since the last epoch head among them
-    __shared__ unsigned long long c_run, c_after;
-    __shared__ uint32_t c_tiles;
-    __shared__ int c_head;
-    if (tid == 0) { c_run = 0; c_after = 0; c_tiles = 0; c_head = -1; }
-    __syncthreads();
-    {
-      unsigned long long r = 0;
-      uint32_t t = 0;
-      int h = -1;
-      for (uint32_t q = tid; q < g; q += BT) {
-        r += a.seg->part[q].bytes;
-        t += a.seg->part[q].tiles;
-        if (a.seg->part[q].has_head) h = (int)q;
-      }
-      if (r) atomicAdd(&c_run, r);
-      if (t) atomicAdd(&c_tiles, t);
-      if (h >= 0) atomicMax(&c_head, h);
-    }
-    __syncthreads();
-    const int h = c_head;
-    {
-      unsigned long long r = 0;
-      for (uint32_t q = (uint32_t)(h + 1) + tid; q < g; q += BT) r += a.seg->part[q].bytes;
-      if (r) atomicAdd(&c_after, r);
-    }
-    __syncthreads();
-    p_carry = (h >= 0 ? a.seg->part[h].tail : p_carry) + c_after;
-    run_carry = c_run;
-    tiles_carry = c_tiles;
     k0 += i_base;
   }
   uint32_t s_next[K];
@@ -275,6 +245,50 @@ __global__ __launch_bounds__(NW * kWave) void fl_schedule_kernel(SchedArgs a) {
   for (int k = 0; k < K; ++k) {
     const uint32_t i = (uint32_t)tid * K + k;
     s_next[k] = (sizes_p && i < n_loc) ? sizes_p[i] : 0;
+  }
+  if constexpr (SEG) {
+    // What the earlier segments hand over: their bytes and tiles, and the bytes since the last epoch head among
+    // them.  One wavefront reads their partials sixty-four at a time (one round trip for up to 65 536 chunks).
+    const uint32_t g = blockIdx.x;
+    __shared__ uint64_t c_run, c_p;
+    __shared__ uint32_t c_tiles;
+    if (wave == 0) {
+      uint64_t run = 0, after = 0;
+      uint32_t tiles = 0;
+      bool seen_head = false;
+      for (uint32_t base = 0; base < g; base += kWave) {
+        const uint32_t q = base + lane;
+        uint64_t b = 0, tl = 0;
+        uint32_t t = 0, hd = 0;
+        if (q < g) {
+          const SegPartial& pq = a.seg->part[q];
+          b = pq.bytes;
+          tl = pq.tail;
+          t = pq.tiles;
+          hd = pq.has_head;
+        }
+        const uint64_t heads = __builtin_amdgcn_ballot_w64(hd != 0);
+        run += bcast_lane_u64(wave_incl_sum_u64(b, lane), kWave - 1);
+        tiles += bcast_lane_u32(wave_incl_sum_u32(t, lane), kWave - 1);
+        if (heads) {
+          const int hb = 63 - __builtin_clzll(heads);
+          const uint64_t above = bcast_lane_u64(wave_incl_sum_u64(lane > hb ? b : 0, lane), kWave - 1);
+          after = bcast_lane_u64(tl, hb) + above;
+          seen_head = true;
+        } else {
+          after += bcast_lane_u64(wave_incl_sum_u64(b, lane), kWave - 1);
+        }
+      }
+      if (lane == 0) {
+        c_run = run;
+        c_tiles = tiles;
+        c_p = seen_head ? after : p_carry + after;
+      }
+    }
+    __syncthreads();
+    p_carry = c_p;
+    run_carry = c_run;
+    tiles_carry = c_tiles;
   }
   if (rows_cached) {
     __syncthreads();
@@ -893,19 +907,20 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
 // ------------------------------------------------------------------------------------------------
 // table -> per-tile descriptors
 // ------------------------------------------------------------------------------------------------
-// One wavefront per row, its lanes striding over the row's tiles: short rows cost one store, a row of a thousand
-// tiles sixteen per lane.  Runs behind the scheduler kernel on the same stream and reads what that one wrote.
+// Eight lanes per row, striding over the row's tiles: a short row costs one store, a row of a thousand tiles 128 per
+// lane.  Runs behind the scheduler kernel on the same stream and reads what that one wrote.
 constexpr int kExpandBlock = 256;
+constexpr int kExpandLanes = 8;
 __global__ __launch_bounds__(kExpandBlock) void fl_expand_tiles(const flh_chunk_desc* __restrict__ table, const flh_sched_hdr* __restrict__ hdr,
                                                                 uint32_t n_max, uint32_t tile_bytes, flh_tile_desc* __restrict__ out, uint32_t cap) {
   uint32_t n = hdr->n_chunks;
   if (n > n_max) n = n_max;
-  const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint32_t waves = gridDim.x * (kExpandBlock / kWave);
-  for (uint32_t row = blockIdx.x * (kExpandBlock / kWave) + threadIdx.x / kWave; row < n; row += waves) {
+  const uint32_t lane = threadIdx.x & (kExpandLanes - 1);
+  const uint32_t groups = gridDim.x * (kExpandBlock / kExpandLanes);
+  for (uint32_t row = blockIdx.x * (kExpandBlock / kExpandLanes) + threadIdx.x / kExpandLanes; row < n; row += groups) {
     const flh_chunk_desc d = table[row];
     const uint32_t nt = (uint32_t)(((uint64_t)d.len + tile_bytes - 1) / tile_bytes);
-    for (uint32_t j = lane; j < nt; j += kWave) {
+    for (uint32_t j = lane; j < nt; j += kExpandLanes) {
       const uint32_t t = d.tile_base + j;
       if (t >= cap) break;
       const uint64_t off = (uint64_t)j * tile_bytes;
@@ -929,7 +944,7 @@ uint64_t flh_schedule_workspace_bytes(uint32_t n_chunks) {
 
 static int expand_tiles(const flh_sched_params* p, hipStream_t s) {
   if (!p->d_tiles || p->n_chunks == 0) return FLH_OK;
-  const uint32_t per_block = kExpandBlock / kWave;
+  const uint32_t per_block = kExpandBlock / kExpandLanes;
   uint32_t grid = (p->n_chunks + per_block - 1) / per_block;
   if (grid > 8192) grid = 8192;
   FL_LAUNCH(fl_expand_tiles, dim3(grid), dim3(kExpandBlock), 0, s, (const flh_chunk_desc*)p->d_table, (const flh_sched_hdr*)p->d_hdr, p->n_chunks,
