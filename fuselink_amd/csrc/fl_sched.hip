@@ -589,7 +589,7 @@ __global__ __launch_bounds__(kSegBlock) void fl_sched_seg_totals(SchedArgs a) {
   }
 }
 
-// Window offsets of a segment's rows start where the earlier segments left each lane; the workgroup of the last
+// Window offsets of a segment's rows start where the earlier segments left each lane; the workgroup of the first
 // segment also sums everything up into header and state.
 __global__ __launch_bounds__(kSegBlock) void fl_sched_seg_finish(SchedArgs a) {
   warm_kernel_args(a);
@@ -620,7 +620,7 @@ __global__ __launch_bounds__(kSegBlock) void fl_sched_seg_finish(SchedArgs a) {
       a.table[i].win_off += base[ln < FLH_MAX_LANES ? ln : 0];
     }
   }
-  if (g != G - 1) return;
+  if (g != 0) return;   // the first segment's workgroup had nothing to sum for its own rows: it sums up for all
   // ---- header and state, from every segment's partials ----------------------------------------------------
   __shared__ unsigned long long t_bytes, t_after, t_lane[FLH_MAX_LANES];
   __shared__ uint32_t t_tiles, t_flags, t_cnt[FLH_MAX_LANES];
