@@ -64,7 +64,7 @@ FL_LOCAL ProfState& fl_prof();
                           hipGetErrorString(e_), __FILE__, __LINE__);                        \
   } while (0)
 
-// flh_init on NCCL_FUSELINK_DEVICE (default 0) if no entry point has initialised the library yet
+// flh_init on NCCL_FUSELINK_DEVICE (unset: the calling thread's current device) if no entry point has initialised the library yet
 FL_LOCAL int fl_need_init();
 // Non-temporal loads and stores pay off once the working set (the buffers a transfer touches) is well
 // beyond the 256 MB Infinity Cache (measured: +3-5 % at 1 GiB messages) and cost throughput when a
