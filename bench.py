@@ -66,6 +66,9 @@ def main() -> int:
     ap.add_argument("--tile-descriptors", type=int, default=-1,
                     help="blocks workload: let the scheduler expand the table to one descriptor per copy tile (flh_stripe_tiles); "
                          "-1 = when the blocks average under two copy tiles and there are at least 4096 of them")
+    ap.add_argument("--pool-units", type=int, default=0,
+                    help="uniform table-driven workloads: keep the staging windows within a pool of this many 2 MiB units (the reference's "
+                         "holds 256) and move the message in as few waves as that allows, windows reused wave by wave; 0 = windows for the whole message")
     ap.add_argument("--no-by-lane", action="store_true", help="stripe large messages in chunk order instead of destination order")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -147,7 +150,36 @@ def main() -> int:
     hdr = sched.hdr_numpy()
     lane_bytes = [int(b) for b in hdr["lane_bytes"][:lanes]]
     units = sum((b + core.UNIT_BYTES - 1) // core.UNIT_BYTES for b in lane_bytes)
-    pool = core.Pool(0, max(256, units))
+
+    # ---- a fixed pool: the message goes in waves, every wave scheduled from the carried state with window offsets
+    # from zero, and the windows are as large as the fullest wave needs (found here, untimed, from the headers) ----
+    waves = None
+    if args.pool_units > 0:
+        if kind != "uniform" or (rows == 1 and epoch_len == 0 and args.path != "split"):
+            print("bench.py: --pool-units applies to the table-driven uniform workloads (cfg5, or --path split)", file=sys.stderr)
+            return 2
+        state = core.new_state(dev)
+        for k in range(1, 65):
+            per = (n_chunks + k - 1) // k
+            cuts = [(i * per * chunk, min(nbytes, (i + 1) * per * chunk)) for i in range(k) if i * per * chunk < nbytes]
+            with torch.cuda.stream(stream):
+                state.zero_()
+            scheds, need = [], [0] * lanes
+            for lo, hi in cuts:
+                s_w = core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=hi - lo, chunk_bytes=chunk, src_base=lo,
+                                    epoch_len=epoch_len, mode=core.SCHED_RESET_OFFSETS, state=state, stream=stream, by_lane=by_lane)
+                stream.synchronize()
+                need = [max(a_, int(b_)) for a_, b_ in zip(need, s_w.hdr_numpy()["lane_bytes"][:lanes])]
+                scheds.append(s_w)
+            if sum((b_ + core.UNIT_BYTES - 1) // core.UNIT_BYTES for b_ in need) <= args.pool_units:
+                waves = [(lo, hi, s_w, core.uniform_hint(hi - lo, chunk) if args.hint else None) for (lo, hi), s_w in zip(cuts, scheds)]
+                lane_bytes = need
+                units = sum((b_ + core.UNIT_BYTES - 1) // core.UNIT_BYTES for b_ in need)
+                break
+        if waves is None:
+            print("bench.py: the message does not fit that pool in 64 waves", file=sys.stderr)
+            return 2
+    pool = core.Pool(0, args.pool_units if waves else max(256, units))
     windows = []
     for b in lane_bytes:
         w = core.Window(pool, max(b, 1))
@@ -157,7 +189,7 @@ def main() -> int:
 
     # header fields that follow from the uniform split alone; the kernels then need not wait for d_hdr
     hint = core.uniform_hint(msg_bytes, chunk) if (args.hint and kind == "uniform") else None
-    fused = kind in ("uniform", "pages") and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
+    fused = not waves and kind in ("uniform", "pages") and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
     if fused and (rows != 1 or epoch_len != 0):
         print("bench.py: the fused path takes a single credit row without epochs", file=sys.stderr)
         return 2
@@ -177,6 +209,14 @@ def main() -> int:
                                   use_lds=bool(args.lds), stream=stream, by_lane=by_lane)
                 core.scatter_pages(dst[lo: lo + msg_bytes], tables[half_i], page_bytes, ppc, win, sched, status,
                                    use_lds=bool(args.lds), stream=stream)
+        elif waves:
+            with torch.cuda.stream(stream):
+                state.zero_()
+            for lo, hi, s_w, h_w in waves:
+                core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=hi - lo, chunk_bytes=chunk, src_base=lo, epoch_len=epoch_len,
+                              mode=core.SCHED_RESET_OFFSETS, state=state, out=s_w, stream=stream, by_lane=by_lane)
+                core.stripe(src, win, s_w, status, stream=stream, hint=h_w, by_lane=by_lane)
+                core.reassemble(dst, win, s_w, status, stream=stream, hint=h_w)
         elif fused:
             # the striping launch computes each chunk's lane and offset itself and writes the table out
             core.stripe_uniform(src, win, uni, status, out=sched, stream=stream)
@@ -270,7 +310,7 @@ def main() -> int:
         del srcs, dsts
 
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
-    algo_bytes_kernel = 2 * msg_bytes     # one launch of the copy kernel
+    algo_bytes_kernel = 2 * msg_bytes // (len(waves) if waves else 1)    # one launch of the copy kernel (with waves: the average one)
     value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
     pair_us = (stripe_us + reasm_us) * launches_per_step
     achieved = algo_bytes_kernel / (stripe_us * 1e-6) / 1e9
@@ -307,7 +347,7 @@ def main() -> int:
                    "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
                    "step": ("2x(gather(with scheduler folded in)+scatter)" if (kind == "pages" and fused) else "2x(schedule+gather+scatter)" if kind == "pages" else
                             "stripe(with scheduler folded in)+reassemble" if fused else "schedule+stripe+reassemble"),
-                   "launch": "eager", "windows": "HIP VMM, 2 MiB units", "tile_descriptors": bool(use_tiles),
+                   "launch": "eager", "windows": "HIP VMM, 2 MiB units" + (f", pool of {args.pool_units}, {len(waves)} waves" if waves else ""), "tile_descriptors": bool(use_tiles),
                    "stripe_order": "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel for messages past 256 MiB)" if fused else "chunk"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
