@@ -35,12 +35,22 @@ WORKLOADS = {
 # HBM bytes per launch of the striping kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size.
 # None where no such run has been recorded for the workload.
-MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134288509, "cfg5_stress_1GiB_64KiB_16lanes": 2151675086,
+MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134288509, "cfg5_stress_1GiB_64KiB_16lanes": 2151691798,
+                    "cfg5_stress_1GiB_64KiB_16lanes/17 waves": 126496616,
                     "cfg3_expert_parallel_256_blocks_8lanes": 1786036451, "cfg4_paged_kv_2x4096_pages_8lanes": 268670118}
 
 
 def algo_bytes_cold(nbytes: int) -> int:
     return 4 * nbytes   # stripe: read N + write N; reassemble: read N + write N
+
+
+def _state_at(core, dev, epoch_bytes, chunk):
+    """Scheduler state of a message of whole chunks that has `epoch_bytes` bytes of its one epoch behind it."""
+    import numpy as np
+    import torch
+    st = np.zeros(1, dtype=core.STATE_DTYPE)
+    st["epoch_bytes"], st["chunk_index"] = epoch_bytes, epoch_bytes // chunk
+    return torch.from_numpy(st.view(np.uint8)).to(dev)
 
 
 def main() -> int:
@@ -66,6 +76,13 @@ def main() -> int:
     ap.add_argument("--tile-descriptors", type=int, default=-1,
                     help="blocks workload: let the scheduler expand the table to one descriptor per copy tile (flh_stripe_tiles); "
                          "-1 = when the blocks average under two copy tiles and there are at least 4096 of them")
+    ap.add_argument("--cache-waves", type=int, default=-1,
+                    help="uniform workloads past 256 MiB: move the message in waves small enough for the staging windows to stay in the "
+                         "256 MB Infinity Cache (a wave is a credit epoch where the workload has epochs, else 64 MiB), each wave one fused "
+                         "stripe + reassemble pair over the same windows; -1 = do so, 0 = one launch pair for the whole message")
+    ap.add_argument("--wave-epochs", type=int, default=1,
+                    help="workloads with credit epochs: epochs per cache-resident wave.  1 = a fused launch pair per epoch; more = one "
+                         "scheduler launch for the whole message (wave_chunks) and a table-driven launch pair per wave")
     ap.add_argument("--pool-units", type=int, default=0,
                     help="uniform table-driven workloads: keep the staging windows within a pool of this many 2 MiB units (the reference's "
                          "holds 256) and move the message in as few waves as that allows, windows reused wave by wave; 0 = windows for the whole message")
@@ -179,6 +196,45 @@ def main() -> int:
         if waves is None:
             print("bench.py: the message does not fit that pool in 64 waves", file=sys.stderr)
             return 2
+    # ---- waves that keep the windows cache-resident: what one wave stages is read back by its own reassembly launch
+    # before the next wave overwrites it, so the window traffic never reaches HBM ----
+    cwaves = twaves = None
+    wave_chunks = 0
+    if (kind == "uniform" and not waves and args.cache_waves != 0 and args.path in ("auto", "fused") and nbytes > (256 << 20)
+            and epoch_len > 0 and args.wave_epochs > 1 and args.wave_epochs * epoch_len * chunk <= (200 << 20)):
+        # one scheduler launch whose rows restart their window offsets every wave, then a table-driven pair per wave
+        wave_chunks = args.wave_epochs * epoch_len
+        s_all = core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk, epoch_len=epoch_len,
+                              stream=stream, wave_chunks=wave_chunks)
+        stream.synchronize()
+        t_all = s_all.table_numpy()
+        need = [0] * lanes
+        twaves = []
+        for w0 in range(0, n_chunks, wave_chunks):
+            part = t_all[w0: w0 + wave_chunks]
+            by = np.bincount(part["lane"], weights=part["len"].astype(np.float64), minlength=lanes)
+            need = [max(a_, int(b_)) for a_, b_ in zip(need, by[:lanes])]
+            lo, hi = w0 * chunk, min(nbytes, (w0 + wave_chunks) * chunk)
+            twaves.append((w0, min(wave_chunks, n_chunks - w0), core.uniform_hint(hi - lo, chunk)))
+        lane_bytes = need
+        units = sum((b_ + core.UNIT_BYTES - 1) // core.UNIT_BYTES for b_ in need)
+    elif (kind == "uniform" and not waves and args.cache_waves != 0 and args.path in ("auto", "fused") and nbytes > (256 << 20)
+            and (rows == 1 or epoch_len > 0)):
+        per = epoch_len * chunk if epoch_len else max(chunk, (64 << 20) // chunk * chunk)
+        if per <= (96 << 20):
+            cwaves, need = [], [0] * lanes
+            for i, lo in enumerate(range(0, nbytes, per)):
+                hi = min(nbytes, lo + per)
+                row = credits_np[i % rows if epoch_len else 0].tolist()
+                # with epochs every wave starts a new one; without, the quanta carry on from wave to wave
+                u_w = core.uniform_params(hi - lo, chunk, row, src_base=lo, epoch_bytes=0 if epoch_len else lo)
+                s_w = core.schedule(n_lanes=lanes, credits=row, quantum=chunk, total_bytes=hi - lo, chunk_bytes=chunk, stream=stream,
+                                    state=None if epoch_len else _state_at(core, dev, lo, chunk), mode=core.SCHED_RESET_OFFSETS)
+                stream.synchronize()
+                need = [max(a_, int(b_)) for a_, b_ in zip(need, s_w.hdr_numpy()["lane_bytes"][:lanes])]
+                cwaves.append(u_w)
+            lane_bytes = need
+            units = sum((b_ + core.UNIT_BYTES - 1) // core.UNIT_BYTES for b_ in need)
     pool = core.Pool(0, args.pool_units if waves else max(256, units))
     windows = []
     for b in lane_bytes:
@@ -189,7 +245,7 @@ def main() -> int:
 
     # header fields that follow from the uniform split alone; the kernels then need not wait for d_hdr
     hint = core.uniform_hint(msg_bytes, chunk) if (args.hint and kind == "uniform") else None
-    fused = not waves and kind in ("uniform", "pages") and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
+    fused = not waves and not cwaves and not twaves and kind in ("uniform", "pages") and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
     if fused and (rows != 1 or epoch_len != 0):
         print("bench.py: the fused path takes a single credit row without epochs", file=sys.stderr)
         return 2
@@ -209,6 +265,17 @@ def main() -> int:
                                   use_lds=bool(args.lds), stream=stream, by_lane=by_lane)
                 core.scatter_pages(dst[lo: lo + msg_bytes], tables[half_i], page_bytes, ppc, win, sched, status,
                                    use_lds=bool(args.lds), stream=stream)
+        elif twaves:
+            core.schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk, epoch_len=epoch_len,
+                          out=sched, stream=stream, wave_chunks=wave_chunks)
+            for w0, cnt, h_w in twaves:
+                sub = core.Schedule(sched.table[w0 * core.DESC_DTYPE.itemsize:], sched.hdr, cnt, core.TILE_BYTES)
+                core.stripe(src, win, sub, status, stream=stream, hint=h_w)
+                core.reassemble(dst, win, sub, status, stream=stream, hint=h_w)
+        elif cwaves:
+            for u_w in cwaves:
+                core.stripe_uniform(src, win, u_w, status, out=sched, stream=stream)
+                core.reassemble_uniform(dst, win, u_w, status, stream=stream)
         elif waves:
             with torch.cuda.stream(stream):
                 state.zero_()
@@ -251,14 +318,14 @@ def main() -> int:
         for _ in range(args.steps):
             step()
 
-    per = profiled(steps_again, 8 * args.steps)
+    per = profiled(steps_again, (8 + 2 * len(cwaves or ()) + 3 * len(waves or ()) + 2 * len(twaves or ())) * args.steps)
     mean = lambda xs: sum(xs) / len(xs)
     out_k, in_k = ("gather", "scatter") if kind == "pages" else ("stripe", "reassemble")
     stripe_us, reasm_us = mean(per[out_k]), mean(per[in_k])
     stripe_min, reasm_min = min(per[out_k]), min(per[in_k])
     launches_per_step = len(per[out_k]) // args.steps
-    if fused:
-        # the table the fused launch wrote must be the scheduler kernel's table
+    if fused or cwaves:
+        # the table the fused launch wrote must be the scheduler kernel's table (with waves, sched holds the last wave's only)
         fused_table = sched.table_numpy().tobytes()
 
         def scheds():
@@ -266,7 +333,7 @@ def main() -> int:
                 run_schedule(sched)
 
         per_s = profiled(scheds, 2 * args.steps)
-        assert sched.table_numpy().tobytes() == fused_table, "fused and standalone scheduler tables differ"
+        assert cwaves or sched.table_numpy().tobytes() == fused_table, "fused and standalone scheduler tables differ"
         sched_us, n_sched = mean(per_s["schedule"]), len(per_s["schedule"]) // args.steps
     else:
         sched_us, n_sched = mean(per["schedule"]), len(per["schedule"]) // args.steps
@@ -310,7 +377,7 @@ def main() -> int:
         del srcs, dsts
 
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
-    algo_bytes_kernel = 2 * msg_bytes // (len(waves) if waves else 1)    # one launch of the copy kernel (with waves: the average one)
+    algo_bytes_kernel = 2 * msg_bytes // len(waves or cwaves or twaves or (0,))    # one launch of the copy kernel (with waves: the average one)
     value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
     pair_us = (stripe_us + reasm_us) * launches_per_step
     achieved = algo_bytes_kernel / (stripe_us * 1e-6) / 1e9
@@ -318,7 +385,7 @@ def main() -> int:
         kernel_name = "fl_copy_uniform_fused<0, FusedPageArgs> (gather)"
     elif kind == "pages":
         kernel_name = f"fl_page_tiles<0, lds={args.lds}> (gather)"
-    elif fused:
+    elif fused or cwaves:
         kernel_name = "fl_copy_uniform_fused<0> (stripe)"
     elif hint is not None:
         kernel_name = "fl_copy_uniform<0> (stripe)"
@@ -346,23 +413,26 @@ def main() -> int:
         "config": {"workload": args.workload, "bytes": nbytes, "chunk_bytes": chunk if sizes is None else "variable", "chunks": n_chunks,
                    "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
                    "step": ("2x(gather(with scheduler folded in)+scatter)" if (kind == "pages" and fused) else "2x(schedule+gather+scatter)" if kind == "pages" else
-                            "stripe(with scheduler folded in)+reassemble" if fused else "schedule+stripe+reassemble"),
-                   "launch": "eager", "windows": "HIP VMM, 2 MiB units" + (f", pool of {args.pool_units}, {len(waves)} waves" if waves else ""), "tile_descriptors": bool(use_tiles),
-                   "stripe_order": "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel for messages past 256 MiB)" if fused else "chunk"},
+                            "stripe(with scheduler folded in)+reassemble" if fused else
+                            f"{len(cwaves)} waves of stripe(with scheduler folded in)+reassemble over cache-resident windows" if cwaves else
+                            f"schedule, then {len(twaves)} waves of stripe+reassemble over cache-resident windows" if twaves else "schedule+stripe+reassemble"),
+                   "launch": "eager", "windows": f"HIP VMM, {units} units of 2 MiB bound" + (f", pool of {args.pool_units}, {len(waves)} waves" if waves else ""), "tile_descriptors": bool(use_tiles),
+                   "stripe_order": "chunk" if (cwaves or twaves) else "destination (lane by lane)" if (by_lane and not fused) else "chunk (destination order inside the kernel for messages past 256 MiB)" if fused else "chunk"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
         "kernels_us": {"schedule": round(sched_us, 2), out_k: round(stripe_us, 2), in_k: round(reasm_us, 2),
                        out_k + "_min": round(stripe_min, 2), in_k + "_min": round(reasm_min, 2),
                        "plain_copy_same_bytes": round(copy_us, 2)},
         "stripe_reassemble_pair_GBps": round(algo_bytes_step / (pair_us * 1e-6) / 1e9, 1),
-        "scheduler_kernel": "standalone launch, not part of the fused step" if fused else "first launch of every message",
+        "scheduler_kernel": "standalone launch, not part of the fused step" if (fused or cwaves) else "first launch of every message",
         # one launch schedules a whole message; below 1000 chunks its cost is the flat launch time, not a per-1k rate
         "scheduler_launch_us": round(sched_us, 2),
         "scheduler_us_per_1k_chunks": round(sched_us * n_sched / (n_chunks / 1000.0), 3) if n_chunks >= 1000 else None,
         "cold_user_buffers": cold,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(args.workload) if (kind != "blocks" or args.blocks == 256) else None},
+                     "traffic": (MEASURED_TRAFFIC.get(f"{args.workload}/{len(cwaves)} waves") if cwaves else None if (waves or twaves) else
+                                 MEASURED_TRAFFIC.get(args.workload) if (kind != "blocks" or args.blocks == 256) else None)},
     }
 
     # ---- CPU baseline: the oracle's host-memcpy striping on a bounded sample ------------------------

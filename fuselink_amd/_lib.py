@@ -33,7 +33,7 @@ class SchedParams(C.Structure):
                 ("mode", C.c_uint32), ("d_state", C.c_void_p), ("d_table", C.c_void_p), ("d_hdr", C.c_void_p),
                 ("inline_credits", C.c_uint32 * MAX_LANES), ("d_table_by_lane", C.c_void_p),
                 ("d_tiles", C.c_void_p), ("tiles_cap", C.c_uint32), ("pad_", C.c_uint32),
-                ("d_workspace", C.c_void_p), ("workspace_bytes", C.c_uint64)]
+                ("d_workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("wave_chunks", C.c_uint32), ("pad2_", C.c_uint32)]
 
 
 class UniformParams(C.Structure):

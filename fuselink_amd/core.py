@@ -108,7 +108,7 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
              total_bytes: int = 0, chunk_bytes: int = 0, src_off: Optional[torch.Tensor] = None, src_base: int = 0,
              epoch_len: int = 0, tile_bytes: int = TILE_BYTES, mode: int = 0, state: Optional[torch.Tensor] = None,
              out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None, by_lane: bool = False,
-             tiles_capacity: int = 0, workspace: bool = False) -> Schedule:
+             tiles_capacity: int = 0, workspace: bool = False, wave_chunks: int = 0) -> Schedule:
     """Launches the scheduler kernel (flh_schedule).  `credits` is a uint32/int32 device tensor of
     shape [rows, n_lanes]; `sizes` a uint32/int32 device tensor of chunk sizes, or None for the
     uniform split of `total_bytes` by `chunk_bytes`."""
@@ -148,6 +148,7 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
         if out.tiles is None or out.tiles_cap < tiles_capacity:
             out.tiles, out.tiles_cap = _dev_bytes(tiles_capacity * TILE_DESC_DTYPE.itemsize, dev), tiles_capacity
         p.d_tiles, p.tiles_cap = _ptr(out.tiles), out.tiles_cap
+    p.wave_chunks = wave_chunks
     if workspace:        # lets a long list that needs the scan be scheduled by several workgroups
         need = int(lib.flh_schedule_workspace_bytes(n))
         if out.workspace is None or out.workspace.numel() < need:

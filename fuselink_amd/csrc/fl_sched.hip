@@ -37,6 +37,7 @@ struct SchedArgs {
   uint32_t inline_credits[FLH_MAX_LANES];  // the one credit row when credits == nullptr
   flh_chunk_desc* table_by_lane;           // optional second copy of the rows in destination order (uniform kernel only)
   struct SegHeader* seg;                   // caller's workspace when several workgroups share the scan, else null
+  uint32_t wave_chunks;                    // uniform kernel: window offsets restart every so many chunks (0: never)
 };
 
 // Scan scheduler over several workgroups: the chunk list is cut into segments of kSegChunks, one workgroup each.
@@ -836,12 +837,17 @@ __global__ __launch_bounds__(kUniBlock) void fl_schedule_uniform_kernel(SchedArg
     if (i < a.n) {
       uint32_t ln;
       uint64_t ep;
-      const uint64_t before = uni_before(t, c, i, 0xffffffffu, &ln, &ep);
+      uint64_t before = uni_before(t, c, i, 0xffffffffu, &ln, &ep);
+      bool from_zero = !keep_off;
+      if (a.wave_chunks) {   // the windows are reused wave by wave: count from the wave's first chunk, on an empty window
+        const uint32_t w0 = i - i % a.wave_chunks;
+        if (w0) { before -= uni_before(t, c, w0, ln, nullptr, nullptr); from_zero = true; }
+      }
       const uint64_t o = (uint64_t)i * c.C;
       const uint64_t rem = a.total_bytes - o;
       flh_chunk_desc d;
       d.src_off = a.src_base + o;
-      d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : (keep_off ? a.state->lane_off[ln] : 0) + before * c.C;
+      d.win_off = (a.mode & FLH_SCHED_MIRROR) ? d.src_off : (from_zero ? 0 : a.state->lane_off[ln]) + before * c.C;
       d.len = (uint32_t)(rem < c.C ? rem : c.C);
       d.lane = ln;
       d.tile_base = i * tpc;
@@ -962,6 +968,8 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   if (p->tile_bytes == 0 || p->tile_bytes % 128) return fl_set_error(FLH_E_ARG, "tile_bytes %u must be a positive multiple of 128", p->tile_bytes);
   if (!p->d_hdr || (p->n_chunks && !p->d_table)) return fl_set_error(FLH_E_ARG, "output pointers missing");
   if (p->d_tiles && p->tiles_cap == 0) return fl_set_error(FLH_E_ARG, "d_tiles without tiles_cap");
+  if (p->wave_chunks && (p->d_sizes || p->d_src_off || p->quantum != p->chunk_bytes || p->n_rows > (uint32_t)kRowCache || p->d_table_by_lane))
+    return fl_set_error(FLH_E_ARG, "wave_chunks needs the uniform closed-form split (no d_sizes, no d_src_off, quantum == chunk_bytes, n_rows <= %d) and no d_table_by_lane", kRowCache);
   if (!p->d_sizes) {
     if (p->n_chunks && p->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0 for the uniform split");
     const uint64_t need = p->chunk_bytes ? (p->total_bytes + p->chunk_bytes - 1) / p->chunk_bytes : 0;
@@ -983,6 +991,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   a.hdr = p->d_hdr;
   a.table_by_lane = p->d_table_by_lane;
   a.seg = nullptr;
+  a.wave_chunks = p->wave_chunks;
   a.chunk_bytes = p->chunk_bytes;
   a.n = p->n_chunks;
   a.n_lanes = p->n_lanes;
@@ -1005,6 +1014,7 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
     FL_HIP(hipGetLastError());
     return expand_tiles(p, s);
   }
+  if (p->wave_chunks && n > 0) return fl_set_error(FLH_E_ARG, "wave_chunks: the closed-form scheduler is switched off by a tunable");
   // a long list with a workspace: one workgroup per kSegChunks chunks, three launches
   if (p->d_workspace && variant == 0 && n >= (uint32_t)g_sched_seg_min && p->n_rows <= (uint32_t)kRowCache && !p->d_table_by_lane) {
     const uint32_t G = seg_count(n);

@@ -121,6 +121,13 @@ typedef struct flh_sched_params {
                                   quantum != chunk_bytes) is scheduled by one workgroup per 1024 chunks in three
                                   launches instead of by one workgroup; same table, header and state */
   uint64_t workspace_bytes;
+  uint32_t wave_chunks;        /* uniform closed-form split only: the windows are reused every wave_chunks chunks, so a
+                                  row's win_off counts from the first chunk of its wave on an empty window -- the rows
+                                  [w * wave_chunks, (w + 1) * wave_chunks) are the table of wave w as a call for that
+                                  wave alone (RESET_OFFSETS, state carried) would write it.  Header and state are the
+                                  whole call's.  0 = one wave.  One scheduler launch then serves a message that moves
+                                  through windows smaller than itself (src/cumem.cu:9: a 512 MiB pool). */
+  uint32_t pad2_;
 } flh_sched_params;
 
 /* ---- library ------------------------------------------------------------------------------ */

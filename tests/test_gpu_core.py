@@ -890,3 +890,71 @@ def test_long_variable_list_records_into_a_hip_graph(fl):
         assert sched.table_numpy().tobytes() == exp_t.tobytes(), f"replay {rep}"
         np.testing.assert_array_equal(dst.cpu().numpy()[:total], src_np[:total], err_msg=f"replay {rep}")
         assert not dst[total:].any()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_one_scheduler_launch_for_a_message_that_moves_in_waves(fl, seed):
+    """wave_chunks: the rows of wave w are what a call for that wave alone (offsets from zero, state carried from the
+    wave before) writes -- the oracle is run wave by wave -- while header and state are the whole call's; the copies
+    driven wave by wave over windows that hold one wave round-trip the message."""
+    core, torch = fl
+    rng = np.random.default_rng(6200 + seed)
+    lanes = int(rng.integers(1, 17))
+    rows = int(rng.integers(1, 5))
+    credits = rng.integers(0, 9, size=(rows, lanes)).astype(np.uint32)
+    epoch_len = int(rng.choice([0, 7, 50, 1000]))
+    chunk = int(rng.choice([4096, 8192 + 128, 65536]))
+    n = int(rng.integers(1, 900))
+    V = int(rng.choice([1, 5, 64, 100, 1000]))
+    total = n * chunk - int(rng.integers(0, chunk))
+    tile = int(rng.choice([128, 4096, 32768]))
+    st0 = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+    if seed % 2:
+        st0["epoch_bytes"] = int(rng.integers(0, 40)) * chunk
+        st0["chunk_index"] = int(rng.integers(0, 3000))
+        st0["lane_off"][:lanes] = rng.integers(0, 1 << 20, size=lanes)
+    # expectation: the oracle wave by wave
+    st = st0.copy()
+    exp_rows, need = [], np.zeros(lanes, dtype=np.int64)
+    for w0 in range(0, n, V):
+        lo, hi = w0 * chunk, min(total, (w0 + V) * chunk)
+        t_w, h_w, st = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=hi - lo, chunk_bytes=chunk, src_base=lo,
+                                          epoch_len=epoch_len, tile_bytes=tile, mode=(0 if w0 == 0 else ob.SCHED_RESET_OFFSETS), state=st)
+        exp_rows.append(t_w)
+        if w0:
+            need = np.maximum(need, h_w["lane_bytes"][:lanes].astype(np.int64))
+        else:
+            need = np.maximum(need, st0["lane_off"][:lanes].astype(np.int64) + h_w["lane_bytes"][:lanes].astype(np.int64))
+    exp_t = np.concatenate(exp_rows)
+    whole_t, whole_h, whole_s = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                                   epoch_len=epoch_len, tile_bytes=tile, state=st0.copy())
+    d_state = _dev(torch, np.array([st0], dtype=ob.STATE_DTYPE).view(np.uint8))
+    sched = core.schedule(n_lanes=lanes, credits=_dev(torch, credits.view(np.int32)), quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                          epoch_len=epoch_len, tile_bytes=tile, state=d_state, wave_chunks=V)
+    torch.cuda.synchronize()
+    got_t, got_h = sched.table_numpy(), sched.hdr_numpy()
+    for f in ("src_off", "win_off", "len", "lane", "epoch"):
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f"table field {f}")
+    np.testing.assert_array_equal(got_t["tile_base"], whole_t["tile_base"])
+    for f in ("total_bytes", "total_tiles", "n_chunks", "flags", "uniform_tiles", "lane_bytes", "lane_chunks"):
+        np.testing.assert_array_equal(got_h[f], whole_h[f], err_msg=f"hdr field {f}")
+    got_s = core.state_numpy(d_state)
+    for f in ("epoch_bytes", "chunk_index"):
+        assert got_s[f] == whole_s[f], f
+    # the copies, wave by wave, over windows that hold one wave
+    caps = [int(x) for x in need]
+    wins = [torch.zeros(max(c, 1), dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    src = torch.randint(0, 256, (total,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    status = core.new_status()
+    row_bytes = core.DESC_DTYPE.itemsize
+    for w0 in range(0, n, V):
+        cnt = min(V, n - w0)
+        lo, hi = w0 * chunk, min(total, (w0 + V) * chunk)
+        sub = core.Schedule(sched.table[w0 * row_bytes:], sched.hdr, cnt, tile)
+        hint = core.uniform_hint(hi - lo, chunk, tile)
+        core.stripe(src, w, sub, status, hint=hint)
+        core.reassemble(dst, w, sub, status, hint=hint)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0 and torch.equal(src, dst)
