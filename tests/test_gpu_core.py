@@ -941,6 +941,7 @@ def test_one_scheduler_launch_for_a_message_that_moves_in_waves(fl, seed):
     got_s = core.state_numpy(d_state)
     for f in ("epoch_bytes", "chunk_index"):
         assert got_s[f] == whole_s[f], f
+    np.testing.assert_array_equal(got_s["lane_off"], whole_s["lane_off"])
     # the copies, wave by wave, over windows that hold one wave
     caps = [int(x) for x in need]
     wins = [torch.zeros(max(c, 1), dtype=torch.uint8, device="cuda") for c in caps]
