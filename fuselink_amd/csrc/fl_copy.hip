@@ -236,9 +236,14 @@ struct FusedArgs {
   // The lane of a slot is then found by a four-step binary search over pfx_ex[] (exclusive credit prefixes,
   // W from index n_lanes on), read straight from the argument block.
   uint32_t fast;
+  uint32_t stamp_value;      // see stamp
   uint64_t magic;
   uint32_t cnt0[FLH_MAX_LANES];
   uint32_t pfx_ex[FLH_MAX_LANES + 1];
+  // Stripe only, may be null: a host-visible word that the launch's first workgroup sets to stamp_value as it starts.
+  // A kernel starts once everything queued before it on its stream has finished, so a caller that numbers its
+  // launches learns from the word that all earlier ones are complete, without an event behind each of them.
+  uint32_t* stamp;
 };
 
 // Several requests as one message: chunk c belongs to the request r with first[r] <= c < first[r+1];
@@ -382,6 +387,8 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
     d.epoch = 0;
     a.table[c] = d;
   }
+  if (DIR == 0 && blockIdx.x == 0 && blockIdx.y == 0 && a.stamp && threadIdx.x == 0)
+    __hip_atomic_store(a.stamp, a.stamp_value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   if (DIR == 0 && blockIdx.x == 0 && blockIdx.y == 0 && a.hdr) {  // header: per-lane totals in closed form
     FusedRow r;
     fused_row(a, r);
@@ -656,6 +663,9 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
   a.table = dir == 0 ? d_table : nullptr;
   a.hdr = dir == 0 ? d_hdr : nullptr;
   a.status = d_status;
+  a.stamp = nullptr;
+  a.stamp_value = 0;
+  if (dir == 0) fl_take_launch_stamp(&a.stamp, &a.stamp_value);
   a.total_bytes = u->total_bytes;
   a.src_base = u->src_base;
   a.quanta_before = u->epoch_bytes / u->chunk_bytes;

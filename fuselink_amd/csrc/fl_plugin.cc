@@ -60,6 +60,12 @@ struct Params {
   int idle_credit = 4;
   int max_wave_chunks = 4096;
   int batch = FLH_BATCH_MAX;     // matched sends that may wait for one launch (1 = launch inside isend)
+  // How a launch's completion reaches `test`: 0 = an event recorded behind every launch (a barrier packet of its
+  // own, some 4.5 us in which the connection's next kernel does not start), 1 = the event rides on the launch's
+  // last kernel, 2 = no event at all while launches follow each other: every striping kernel, as it starts, stores
+  // the number of the launch before it to a pinned word (a kernel starts once its stream's earlier work is done),
+  // and only a launch that nothing follows gets an event, recorded when it is first polled.
+  int completion = 2;
 };
 Params g_par;
 std::mutex g_init_mu;            // ncclIbLock, plugin.cc:84
@@ -111,7 +117,6 @@ struct Request {
   int type = kReqUnused;
   std::atomic<int> state{0};
   Link* link = nullptr;
-  hipEvent_t ev = nullptr;   // completion of the launch that carries this request (owned by the connection's ring)
   uint64_t seq = 0;          // number of that launch on its connection, counted from 1
   int size = 0;          // bytes moved (reported by test for receives)
   int fault = 0;         // injected wire fault
@@ -183,18 +188,22 @@ struct Link {
   uint64_t epoch_bytes = 0;         // bytes scheduled since the last lane-decision refresh (the scheduler's carried prefix)
   int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
   int32_t* d_status = nullptr;
+  uint32_t* h_stamp = nullptr;      // pinned, device-visible: number of the last launch known complete (completion mode 2)
+  uint32_t* d_stamp = nullptr;
   std::atomic<uint32_t> last_wave_rows{0};
   // Guards the waiting sends, the event ring and every launch on `stream` (either side's thread may be the
   // one that launches).  Never taken while `mu` is held by the same thread for long: isend drops `mu` first.
   std::mutex launch_mu;
   std::vector<Pending> pending;
-  hipEvent_t evring[FL_NET_MAX_REQUESTS] = {};   // at most that many requests, hence launches, are in flight
-  uint32_t ev_next = 0;
+  std::atomic<uint64_t> waiting_bytes{0};   // bytes of the waiting sends, readable without launch_mu
+  hipEvent_t evring[FL_NET_MAX_REQUESTS] = {};   // launch n owns slot (n - 1) % size: at most that many requests, hence launches, are in flight
+  std::atomic<uint8_t> ev_set[FL_NET_MAX_REQUESTS] = {};    // the slot's event has been recorded (or rides on a kernel) for its launch
+  std::atomic<uint8_t> stamps[FL_NET_MAX_REQUESTS] = {};    // the slot's launch starts with a kernel that stamps the launch before it
   // Highest launch number seen complete.  The connection's launches run in order on one stream, so a request of an
   // earlier launch is complete too and its test needs no event query (requests that shared a launch, and the
   // receive side of a send that was already tested, cost no call into the runtime).
   std::atomic<uint64_t> done_seq{0};
-  uint64_t launch_seq = 0;
+  std::atomic<uint64_t> launch_seq{0};   // written under launch_mu
   int64_t launches = 0, batched_requests = 0;    // launch pairs made, requests that shared one
 };
 
@@ -277,7 +286,6 @@ Request* get_request(Request* tab, Link* lk, int type) {
       r->type = type;
       r->link = lk;
       r->size = 0;
-      r->ev = nullptr;
       r->seq = 0;
       r->fault = 0;
       r->magic = kReqMagic;
@@ -326,9 +334,11 @@ ncclResult_t ensure_link_gpu(Link* lk, int device) {
   }
   FL_HIPCHECK(hipMalloc((void**)&lk->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
   FL_HIPCHECK(hipMalloc((void**)&lk->d_hdr, sizeof(flh_sched_hdr)));
-  FL_HIPCHECK(hipHostMalloc((void**)&lk->h_status, sizeof(int32_t), hipHostMallocMapped));
-  *lk->h_status = 0;
+  FL_HIPCHECK(hipHostMalloc((void**)&lk->h_status, 128, hipHostMallocMapped));   // status word and launch stamp, a cache line apart
+  memset(lk->h_status, 0, 128);
   FL_HIPCHECK(hipHostGetDevicePointer((void**)&lk->d_status, lk->h_status, 0));
+  lk->h_stamp = (uint32_t*)((char*)lk->h_status + 64);
+  lk->d_stamp = (uint32_t*)((char*)lk->d_status + 64);
   lk->gpu_ready = true;
   FL_INFO(NCCL_NET, "NET/FuseLink : channel %d staging ready: %d lanes x %llu bytes", lk->channelId, g_par.lanes, (unsigned long long)cap);
   return ncclSuccess;
@@ -403,6 +413,8 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.idle_credit = (int)fl_param("FUSELINK_IDLE_CREDIT", g_par.idle_credit);
   g_par.max_wave_chunks = (int)fl_param("FUSELINK_MAX_WAVE_CHUNKS", g_par.max_wave_chunks);
   g_par.batch = (int)fl_param("FUSELINK_BATCH", g_par.batch);
+  g_par.completion = (int)fl_param("FUSELINK_COMPLETION", g_par.completion);
+  if (g_par.completion < 0 || g_par.completion > 2) g_par.completion = 2;
   if (g_par.max_wave_chunks > 65535) g_par.max_wave_chunks = 65535;   // what one fused launch can name
   if (g_par.batch < 1) g_par.batch = 1;
   if (g_par.batch > FLH_BATCH_MAX) g_par.batch = FLH_BATCH_MAX;
@@ -636,8 +648,9 @@ void fill_uniform(flh_uniform_params& u, const Link* lk, const uint32_t* credits
   for (int l = 0; l < g_par.lanes; ++l) u.credits[l] = credits[l];
 }
 
-// Queue the GPU work of one matched send on the connection's stream (launch_mu held).
-ncclResult_t launch_transfer(Link* lk, const Pending& p) {
+// Queue the GPU work of one matched send on the connection's stream (launch_mu held); the last launch completes `ev`
+// (if one is given).
+ncclResult_t launch_transfer(Link* lk, const Pending& p, hipEvent_t ev) {
   uint32_t credits[FLH_MAX_LANES];
   wire_credits(lk, p.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
@@ -647,6 +660,8 @@ ncclResult_t launch_transfer(Link* lk, const Pending& p) {
   std::vector<int> qoff(nqps), qlen(nqps);
   if (flh_qp_split(p.size, nqps, qoff.data(), qlen.data()) < 0) return ncclInternalError;
   if (p.w.flags & 1u) lk->epoch_bytes = 0;   // the receiver refreshed its lane decision: new credit epoch
+  int last_q = -1;
+  for (int q = 0; q < nqps; ++q) if (qlen[q] > 0) last_q = q;
   for (int q = 0; q < nqps; ++q) {
     uint64_t done = 0;
     const uint64_t piece = (uint64_t)qlen[q];
@@ -658,6 +673,7 @@ ncclResult_t launch_transfer(Link* lk, const Pending& p) {
       flh_uniform_params u;
       fill_uniform(u, lk, credits, wave, (uint64_t)qoff[q] + done);
       FL_FLHCHECK(flh_stripe_uniform(p.src, (uint64_t)p.size, &lk->wins, &u, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
+      if (ev && q == last_q && done + wave == piece) fl_completion_event(ev);
       FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &lk->wins, &u, lk->d_status, lk->stream));
       lk->epoch_bytes += wave;
       lk->last_wave_rows = (uint32_t)((wave + chunk - 1) / chunk);
@@ -669,7 +685,7 @@ ncclResult_t launch_transfer(Link* lk, const Pending& p) {
 }
 
 // Requests [i, j) of the waiting list as one message in one launch pair (launch_mu held).
-ncclResult_t launch_batch(Link* lk, size_t i, size_t j) {
+ncclResult_t launch_batch(Link* lk, size_t i, size_t j, hipEvent_t ev) {
   const Pending& p0 = lk->pending[i];
   uint32_t credits[FLH_MAX_LANES];
   wire_credits(lk, p0.w, credits);
@@ -687,6 +703,7 @@ ncclResult_t launch_batch(Link* lk, size_t i, size_t j) {
   b.n_req = (uint32_t)(j - i);
   fill_uniform(b.u, lk, credits, sum, 0);
   FL_FLHCHECK(flh_stripe_batch(&b, &lk->wins, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
+  if (ev) fl_completion_event(ev);
   FL_FLHCHECK(flh_reassemble_batch(&b, &lk->wins, lk->d_status, lk->stream));
   lk->epoch_bytes += sum;
   lk->last_wave_rows = (uint32_t)((sum + (uint64_t)g_par.chunk - 1) / (uint64_t)g_par.chunk);
@@ -721,6 +738,9 @@ size_t batch_span(const Link* lk, size_t i) {
   return j > i ? j - i : 1;
 }
 
+// From this many bytes on a launch is bound by the GPU and not by the host's calls around it.
+constexpr uint64_t kEarlyLaunchBytes = 8ull << 20;
+
 // Launch everything that waits on the connection, in order (launch_mu held).  A failure completes the requests
 // it touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).
 void flush_pending(Link* lk) {
@@ -731,28 +751,47 @@ void flush_pending(Link* lk) {
   while (i < lk->pending.size()) {
     const size_t span = batch_span(lk, i);
     ncclResult_t rc = dev_ok ? ncclSuccess : ncclUnhandledCudaError;
-    hipEvent_t& ev = lk->evring[lk->ev_next % FL_NET_MAX_REQUESTS];
+    const uint64_t seq = lk->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
+    const size_t slot = (size_t)((seq - 1) % FL_NET_MAX_REQUESTS);
+    hipEvent_t& ev = lk->evring[slot];
     if (rc == ncclSuccess && !ev) { hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
+    bool stamped = false, rides = false;
     if (rc == ncclSuccess) {
       const Pending& p = lk->pending[i];
-      if (span > 1) {
-        rc = launch_batch(lk, i, i + span);
-      } else if (p.src_dev && p.dst_dev) {
-        rc = launch_transfer(lk, p);
+      const bool gpu = span > 1 || (p.src_dev && p.dst_dev);
+      if (gpu) {
+        if (g_par.completion == 2) fl_launch_stamp(lk->d_stamp, (uint32_t)(seq - 1));
+        hipEvent_t on_kernel = g_par.completion == 1 ? ev : nullptr;
+        rc = span > 1 ? launch_batch(lk, i, i + span, on_kernel) : launch_transfer(lk, p, on_kernel);
+        stamped = fl_launch_stamp_taken();
+        rides = fl_completion_event_taken();
       } else {
         // one side is host memory: the copy engine is the wire, nothing is striped
         hipError_t e = hipMemcpyAsync(p.dst, p.src, (size_t)p.size, hipMemcpyDefault, lk->stream);
         if (e != hipSuccess) rc = hip_fail("hipMemcpyAsync", e);
       }
     }
-    if (rc == ncclSuccess) { hipError_t e = hipEventRecord(ev, lk->stream); if (e != hipSuccess) rc = hip_fail("hipEventRecord", e); }
+    // A launch that begins with a stamping kernel needs no event now: the launch after it stamps it complete, or
+    // its first poll records the event if nothing has followed.  Everything else (host memory, nothing to launch,
+    // the other completion modes) gets the event here unless it already rides on the last kernel.
+    // A small launch gets its event at once all the same: its requests are bound by the host's polling, which an
+    // event that is already there serves sooner, not by the queue.
+    uint64_t launch_bytes = 0;
+    for (size_t k = i; k < i + span; ++k) launch_bytes += (uint64_t)lk->pending[k].size;
+    const bool later = stamped && launch_bytes >= kEarlyLaunchBytes;
+    bool recorded = rides;
+    if (rc == ncclSuccess && !rides && !later) {
+      hipError_t e = hipEventRecord(ev, lk->stream);
+      if (e != hipSuccess) rc = hip_fail("hipEventRecord", e);
+      recorded = true;
+    }
+    lk->ev_set[slot].store(recorded ? 1 : 0, std::memory_order_release);
+    lk->stamps[slot].store(stamped ? 1 : 0, std::memory_order_release);
     for (size_t k = i; k < i + span; ++k) {
       Pending& p = lk->pending[k];
       if (rc == ncclSuccess) {
-        p.sreq->ev = ev;
-        p.rreq->ev = ev;
-        p.sreq->seq = lk->launch_seq + 1;
-        p.rreq->seq = lk->launch_seq + 1;
+        p.sreq->seq = seq;
+        p.rreq->seq = seq;
         p.sreq->state.store(kStLaunched, std::memory_order_release);
         p.rreq->state.store(kStLaunched, std::memory_order_release);
       } else {
@@ -762,10 +801,11 @@ void flush_pending(Link* lk) {
         p.rreq->state.store(kStDoneHost, std::memory_order_release);
       }
     }
-    if (rc == ncclSuccess) { lk->ev_next++; lk->launch_seq++; }
+    if (rc == ncclSuccess) lk->launch_seq.store(seq, std::memory_order_release);
     i += span;
   }
   lk->pending.clear();
+  lk->waiting_bytes.store(0, std::memory_order_release);
 }
 
 ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhandle, void** request) {
@@ -837,6 +877,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     p.sreq = sreq;
     p.rreq = rreq;
     lk->pending.push_back(p);
+    lk->waiting_bytes.store(lk->waiting_bytes.load(std::memory_order_relaxed) + (uint64_t)p.size, std::memory_order_release);
     sreq->state.store(kStQueued, std::memory_order_release);
     rreq->state.store(kStQueued, std::memory_order_release);
     if ((int)lk->pending.size() >= g_par.batch) flush_pending(lk);
@@ -905,6 +946,17 @@ ncclResult_t fl_iflush(void* recvComm, int /*n*/, void** /*data*/, int* /*sizes*
   return ncclSuccess;
 }
 
+// Launches of the connection that have been queued and are not known to be complete.
+uint64_t launches_in_queue(const Link* lk) {
+  const uint64_t queued = lk->launch_seq.load(std::memory_order_acquire);
+  uint64_t done = lk->done_seq.load(std::memory_order_acquire);
+  if (lk->h_stamp) {   // the stamp trails the newest launch by a small number
+    const uint32_t behind = (uint32_t)queued - __atomic_load_n(lk->h_stamp, __ATOMIC_ACQUIRE);
+    if (behind <= queued && queued - behind > done) done = queued - behind;
+  }
+  return queued - done;
+}
+
 ncclResult_t fl_test(void* request, int* done, int* sizes) {
   if (!request || !done) return ncclInvalidArgument;
   Request* r = (Request*)request;
@@ -914,18 +966,54 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   // the event is polled without the connection's lock: only the thread that drives this comm tests its requests
   int st = r->state.load(std::memory_order_acquire);
   if (st == kStPosted || st == 0) return ncclSuccess;   // a receive whose send has not been matched yet
-  if (st == kStQueued) {                                // matched, not launched: everything that waits goes out now
+  // Matched sends wait so that those that arrive together can share a launch.  They go out when one of them is
+  // polled.  Large ones (8 MiB and more wait) also go out when any request of the connection is polled while fewer
+  // than two launches are left in the queue: the GPU then does not run dry behind a launch whose requests are still
+  // being polled (measured: 25-30 us of idle queue every third or fourth 64 MiB request otherwise).  Small ones keep
+  // waiting: what they gain from sharing a launch outweighs the idle queue (512 KiB requests: 2.2x).
+  if (st == kStQueued || (lk->waiting_bytes.load(std::memory_order_acquire) >= kEarlyLaunchBytes && launches_in_queue(lk) < 2)) {
     std::lock_guard<std::mutex> g(lk->launch_mu);
     flush_pending(lk);
     st = r->state.load(std::memory_order_acquire);
   }
   if (st == kStLaunched) {
     if (r->seq > lk->done_seq.load(std::memory_order_acquire)) {
-      hipError_t e = hipEventQuery(r->ev);
-      if (e == hipErrorNotReady) return ncclSuccess;
-      if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+      uint64_t upto = 0;   // launches known complete
+      if (lk->h_stamp) {   // a later launch's first kernel has started: everything before it is done
+        const uint32_t stamp = __atomic_load_n(lk->h_stamp, __ATOMIC_ACQUIRE);
+        const int32_t ahead = (int32_t)(stamp - (uint32_t)r->seq);
+        if (ahead >= 0) upto = r->seq + (uint64_t)ahead;
+      }
+      if (!upto) {
+        uint64_t q = r->seq;   // the launch whose event answers for this request
+        const size_t slot = (size_t)((q - 1) % FL_NET_MAX_REQUESTS);
+        if (!lk->ev_set[slot].load(std::memory_order_acquire)) {
+          if (q < lk->launch_seq.load(std::memory_order_acquire)) {
+            // a launch follows: its first kernel will stamp this one, or else its event was recorded behind it
+            const size_t next = (size_t)(q % FL_NET_MAX_REQUESTS);
+            if (lk->stamps[next].load(std::memory_order_acquire) || !lk->ev_set[next].load(std::memory_order_acquire)) return ncclSuccess;
+            q += 1;
+          } else {
+            // nothing follows: the event goes behind the launch now (and delays no kernel, the queue ends here)
+            std::lock_guard<std::mutex> g(lk->launch_mu);
+            if (q == lk->launch_seq.load(std::memory_order_relaxed) && !lk->ev_set[slot].load(std::memory_order_relaxed)) {
+              DeviceScope keep;
+              hipError_t e = hipSetDevice(lk->hip_device);
+              if (e == hipSuccess) e = hipEventRecord(lk->evring[slot], lk->stream);
+              if (e != hipSuccess) return hip_fail("hipEventRecord", e);
+              lk->ev_set[slot].store(1, std::memory_order_release);
+            } else if (!lk->ev_set[slot].load(std::memory_order_relaxed)) {
+              return ncclSuccess;   // a launch went out meanwhile: the next poll looks at it
+            }
+          }
+        }
+        hipError_t e = hipEventQuery(lk->evring[(size_t)((q - 1) % FL_NET_MAX_REQUESTS)]);
+        if (e == hipErrorNotReady) return ncclSuccess;
+        if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+        upto = q;
+      }
       uint64_t seen = lk->done_seq.load(std::memory_order_relaxed);
-      while (seen < r->seq && !lk->done_seq.compare_exchange_weak(seen, r->seq, std::memory_order_release, std::memory_order_relaxed)) {}
+      while (seen < upto && !lk->done_seq.compare_exchange_weak(seen, upto, std::memory_order_release, std::memory_order_relaxed)) {}
     }
     if (lk->h_status && *(volatile int32_t*)lk->h_status != 0) {
       FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", *lk->h_status);

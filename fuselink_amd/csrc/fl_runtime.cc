@@ -34,6 +34,33 @@ namespace {
 thread_local ProfState t_prof;
 }
 ProfState& fl_prof() { return t_prof; }
+void fl_completion_event(void* hip_event) {
+  t_prof.done_ev = (hipEvent_t)hip_event;
+  t_prof.done_handed = hip_event != nullptr;
+}
+bool fl_completion_event_taken() {
+  const bool taken = t_prof.done_handed && t_prof.done_ev == nullptr;
+  t_prof.done_ev = nullptr;
+  t_prof.done_handed = false;
+  return taken;
+}
+
+void fl_launch_stamp(uint32_t* d_word, uint32_t value) {
+  t_prof.stamp = d_word;
+  t_prof.stamp_value = value;
+  t_prof.stamp_handed = d_word != nullptr;
+}
+void fl_take_launch_stamp(uint32_t** word, uint32_t* value) {
+  *word = t_prof.stamp;
+  *value = t_prof.stamp_value;
+  t_prof.stamp = nullptr;
+}
+bool fl_launch_stamp_taken() {
+  const bool taken = t_prof.stamp_handed && t_prof.stamp == nullptr;
+  t_prof.stamp = nullptr;
+  t_prof.stamp_handed = false;
+  return taken;
+}
 
 int fl_set_error(int code, const char* fmt, ...) {
   va_list ap;

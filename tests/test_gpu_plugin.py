@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 ENV_KEYS = ["NCCL_FUSELINK_LANES", "NCCL_FUSELINK_CHUNKSIZE", "NCCL_FUSELINK_POLICY", "NCCL_FUSELINK_WINDOW_UNITS",
             "NCCL_FUSELINK_POOL_UNITS", "NCCL_FUSELINK_REFRESH_BATCH", "NCCL_IB_QPS_PER_CONNECTION", "NCCL_FUSELINK_CREDITS",
-            "NCCL_FUSELINK_BATCH"]
+            "NCCL_FUSELINK_BATCH", "NCCL_FUSELINK_COMPLETION"]
 
 
 @pytest.fixture()
@@ -310,6 +310,79 @@ def test_mixed_host_and_device_buffers(net):
     net.wait(sreq), net.wait(rreq)
     np.testing.assert_array_equal(host, src.cpu().numpy())
     net.deregMr(s, smh), net.deregMr(r, rmh)
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+@pytest.mark.parametrize("completion", [0, 1, 2])
+@pytest.mark.parametrize("batch", [1, 8])
+def test_completion_reaches_test_in_every_mode(net, completion, batch):
+    """How `test` learns that a launch is done -- an event behind every launch, an event on the launch's last kernel,
+    or the stamp the next launch's first kernel leaves (with an event only behind a launch that nothing follows) --
+    must not change what a consumer sees: every receive is compared on torch's own stream, which does not wait for the
+    connection's, the moment `test` reports it done, with requests in flight behind it, empty requests and host
+    buffers mixed in, and a lone request at the end that no other launch follows."""
+    import torch
+    net.reconfigure(NCCL_FUSELINK_LANES=4, NCCL_FUSELINK_CHUNKSIZE=64 << 10, NCCL_FUSELINK_WINDOW_UNITS=1,
+                    NCCL_FUSELINK_BATCH=batch, NCCL_FUSELINK_COMPLETION=completion)
+    net.set_credits([3, 1, 2, 2])
+    rng = np.random.default_rng(900 + completion * 10 + batch)
+    n_req = 120
+    sizes = [int(rng.choice([0, 1, 4096, 64 << 10, 200000, 1 << 20, (3 << 20) + 17])) for _ in range(n_req)]
+    kinds = ["host" if rng.random() < 0.1 else "dev" for _ in range(n_req)]
+    offs = np.concatenate([[0], np.cumsum([(x + 255) // 256 * 256 for x in sizes])])
+    total = int(offs[-1]) + 256
+    src = torch.randint(0, 256, (total,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    host_dst = np.zeros(total, dtype=np.uint8)
+    lcomm, s, r = net.connect_pair(0)
+    _, smh = net.regMr(s, src.data_ptr(), total, P.NCCL_PTR_CUDA)
+    _, rmh = net.regMr(r, dst.data_ptr(), total, P.NCCL_PTR_CUDA)
+    _, hmh = net.regMr(r, host_dst.ctypes.data, total, P.NCCL_PTR_HOST)
+    src_np = src.cpu().numpy()
+    posted = sent = checked = 0
+    rq, sq = [], []
+    depth = 6
+    while checked < n_req:
+        if posted < n_req and len(rq) < depth:
+            k, o = posted, int(offs[posted])
+            if kinds[k] == "host":
+                rc, rreq = net.irecv(r, [host_dst.ctypes.data + o], [sizes[k]], [k], [hmh])
+            else:
+                rc, rreq = net.irecv(r, [dst.data_ptr() + o], [sizes[k]], [k], [rmh])
+            assert rc == 0
+            if rreq:
+                rq.append((k, rreq))
+                posted += 1
+        if sent < posted and len(sq) < depth:
+            rc, sreq = net.isend(s, src.data_ptr() + int(offs[sent]), sizes[sent], sent, smh)
+            assert rc == 0
+            if sreq:
+                sq.append(sreq)
+                sent += 1
+        if sq:
+            rc, done, _ = net.test(sq[0])
+            assert rc == 0
+            if done:
+                sq.pop(0)
+        if rq:
+            k, rreq = rq[0]
+            rc, done, size = net.test(rreq)
+            assert rc == 0
+            if done:
+                assert size == sizes[k]
+                o = int(offs[k])
+                if kinds[k] == "host":
+                    np.testing.assert_array_equal(host_dst[o: o + sizes[k]], src_np[o: o + sizes[k]], err_msg=f"request {k}")
+                else:   # a kernel on another stream, started at once
+                    assert torch.equal(dst[o: o + sizes[k]], src[o: o + sizes[k]]), f"request {k} of {sizes[k]} bytes"
+                rq.pop(0)
+                checked += 1
+    # one request alone on an idle connection: nothing follows its launch
+    for size in (1 << 20, 5):
+        dst.zero_()
+        _send_recv(net, s, r, src, dst, size, 1000 + size, smh, rmh)
+        assert torch.equal(dst[:size], src[:size]) and not dst[size:].any()
+    net.deregMr(s, smh), net.deregMr(r, rmh), net.deregMr(r, hmh)
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
