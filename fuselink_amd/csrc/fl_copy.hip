@@ -91,6 +91,7 @@ struct CopyArgs {
   uint32_t tile_bytes;
   // header fields the host already knows (has_hint != 0): saves one dependent memory round trip
   uint32_t has_hint, hint_total_tiles, hint_n_chunks, hint_uniform_tiles;
+  uint32_t xcd;   // xcd_tile()'s `full` (fl_copy_tiles, one workgroup per tile) or xcd_tile_2d()'s map (fl_copy_uniform); 0 = off
 };
 
 // Row of the table that owns copy tile t: the last row with tile_base <= t (rows of empty chunks own
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_tiles(CopyArgs a) {
   uint32_t n = a.has_hint ? a.hint_n_chunks : a.hdr->n_chunks;
   if (n > a.n_chunks_max) n = a.n_chunks_max;
   if (n == 0) return;
-  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
+  for (uint32_t t = xcd_tile(blockIdx.x, a.xcd); t < total; t += gridDim.x) {
     const uint32_t c = find_row(a.table, n, t, uniform_tiles, a.tile_bytes);
     const flh_chunk_desc d = a.table[c];
     const uint64_t off = (uint64_t)(t - d.tile_base) * a.tile_bytes;
@@ -161,12 +162,13 @@ struct DescArgs {
   int32_t* status;
   uint32_t tiles_cap;
   uint32_t has_hint, hint_total_tiles;
+  uint32_t xcd;   // xcd_tile()'s `full`; 0 = off
 };
 
 template <int DIR, int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_desc(DescArgs a) {
   warm_kernel_args(a);
-  const uint32_t t = blockIdx.x;
+  const uint32_t t = xcd_tile(blockIdx.x, a.xcd);
   const flh_tile_desc d = a.tiles[t];
   const uint32_t total = a.has_hint ? a.hint_total_tiles : a.hdr->total_tiles;
   if (total > a.tiles_cap) {   // the table did not fit the descriptor array: nothing of it can be trusted
@@ -191,10 +193,11 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_desc(DescArgs a) {
 template <int DIR, int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform(CopyArgs a) {
   warm_kernel_args(a);
-  const uint32_t c = blockIdx.y;
+  uint32_t bx = blockIdx.x, c = blockIdx.y;
+  xcd_tile_2d(a.xcd, bx, c);
   if (c >= a.hint_n_chunks) return;
   const flh_chunk_desc d = a.table[c];
-  const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
+  const uint64_t off = (uint64_t)bx * a.tile_bytes;
   if (off >= d.len) return;
   const uint32_t bytes = (uint32_t)((d.len - off) < a.tile_bytes ? (d.len - off) : a.tile_bytes);
   bool ok = d.lane < a.win.n_lanes;
@@ -240,6 +243,7 @@ struct FusedArgs {
   uint64_t magic;
   uint32_t cnt0[FLH_MAX_LANES];
   uint32_t pfx_ex[FLH_MAX_LANES + 1];
+  uint32_t xcd_map;          // xcd_tile_2d()'s map for the grid (tiles per chunk, chunks); 0 = off
   // Stripe only, may be null: a host-visible word that the launch's first workgroup sets to stamp_value as it starts.
   // A kernel starts once everything queued before it on its stream has finished, so a caller that numbers its
   // launches learns from the word that all earlier ones are complete, without an event behind each of them.
@@ -302,19 +306,21 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   constexpr bool BATCH = is_batch<Args>::value;
   constexpr bool PAGED = is_paged<Args>::value;
   warm_kernel_args(a);
-  if (blockIdx.y >= a.n_chunks) return;
-  uint32_t c = blockIdx.y, lane = 0;
+  uint32_t bx = blockIdx.x, by = blockIdx.y;   // tile of the chunk, chunk (in message or destination order)
+  xcd_tile_2d(a.xcd_map, bx, by);
+  if (by >= a.n_chunks) return;
+  uint32_t c = by, lane = 0;
   uint64_t before;
   if (DIR == 0 && a.dest_order) {
     FusedRow r;
     fused_row(a, r);
     uint64_t K = 0, hi = r.pfx[0];
-    // blockIdx.y = k-th chunk in destination order: find the lane whose group holds k, then invert the
+    // by = k-th chunk in destination order: find the lane whose group holds k, then invert the
     // closed form -- the j-th slot of a lane with credit c_l and first slot K_l is (j / c_l) * W + K_l + j mod c_l.
     const uint64_t x0 = a.quanta_before, x1 = a.quanta_before + a.n_chunks;
     const uint64_t f0 = div_u64(x0, r.W), f1 = div_u64(x1, r.W);
     const uint64_t r0 = x0 - f0 * r.W, r1 = x1 - f1 * r.W;
-    uint64_t k = blockIdx.y, cnt0 = 0;
+    uint64_t k = by, cnt0 = 0;
     bool found = false;
     uint64_t lo = 0;
 #pragma unroll
@@ -377,7 +383,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
     user_off = (uint64_t)(c - first) * a.chunk_bytes;
   }
 
-  if (DIR == 0 && blockIdx.x == 0 && threadIdx.x == 0 && a.table) {
+  if (DIR == 0 && bx == 0 && threadIdx.x == 0 && a.table) {
     flh_chunk_desc d;
     d.src_off = src_off;
     d.win_off = win_off;
@@ -387,9 +393,9 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
     d.epoch = 0;
     a.table[c] = d;
   }
-  if (DIR == 0 && blockIdx.x == 0 && blockIdx.y == 0 && a.stamp && threadIdx.x == 0)
+  if (DIR == 0 && bx == 0 && by == 0 && a.stamp && threadIdx.x == 0)
     __hip_atomic_store(a.stamp, a.stamp_value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  if (DIR == 0 && blockIdx.x == 0 && blockIdx.y == 0 && a.hdr) {  // header: per-lane totals in closed form
+  if (DIR == 0 && bx == 0 && by == 0 && a.hdr) {  // header: per-lane totals in closed form
     FusedRow r;
     fused_row(a, r);
     const uint32_t t = threadIdx.x;
@@ -420,7 +426,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
     }
   }
 
-  const uint64_t off = (uint64_t)blockIdx.x * a.tile_bytes;
+  const uint64_t off = (uint64_t)bx * a.tile_bytes;
   if (off >= len) return;
   const uint32_t bytes = (uint32_t)((len - off) < a.tile_bytes ? (len - off) : a.tile_bytes);
   if (win_off + len > a.win.cap[lane] || (!PAGED && user_off + len > user_bytes)) {
@@ -511,9 +517,9 @@ __global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
 
 template <int NT>
 __global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const uint8_t* src, uint64_t bytes,
-                                                            uint32_t tile_bytes) {
+                                                            uint32_t tile_bytes, uint32_t xcd) {
   const uint64_t tiles = (bytes + tile_bytes - 1) / tile_bytes;
-  for (uint64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+  for (uint64_t t = xcd_tile(blockIdx.x, xcd); t < tiles; t += gridDim.x) {
     const uint64_t off = t * tile_bytes;
     const uint32_t len = (uint32_t)((bytes - off) < tile_bytes ? (bytes - off) : tile_bytes);
     block_copy<NT>(dst + off, src + off, len);
@@ -574,17 +580,20 @@ static int launch_copy(int dir, void* user, uint64_t user_bytes, const flh_windo
   a.hint_total_tiles = h_hdr ? h_hdr->total_tiles : 0;
   a.hint_n_chunks = h_hdr ? h_hdr->n_chunks : 0;
   a.hint_uniform_tiles = h_hdr ? h_hdr->uniform_tiles : 0;
+  a.xcd = 0;
   const uint64_t max_tiles = h_hdr ? h_hdr->total_tiles : user_bytes / tile_bytes + n_chunks_max;
   if (max_tiles == 0) return FLH_OK;
   hipStream_t s = (hipStream_t)stream;
   const int mode = fl_stream_mode(dir, user_bytes);
   if (h_hdr && h_hdr->uniform_tiles && h_hdr->n_chunks <= 65535 && h_hdr->n_chunks <= n_chunks_max && g_copy_uniform_grid) {
     const dim3 grid(h_hdr->uniform_tiles, h_hdr->n_chunks);
+    a.xcd = fl_xcd_map(grid.x, grid.y);
     FL_LAUNCH_COPY(fl_copy_uniform, FL_NO_EXTRA, dir, mode, grid, s, a);
     FL_HIP(hipGetLastError());
     return FLH_OK;
   }
   const dim3 grid(fl_copy_grid(max_tiles));
+  a.xcd = grid.x == max_tiles ? fl_xcd_full(grid.x) : 0;   // only with one workgroup per tile
   FL_LAUNCH_COPY(fl_copy_tiles, FL_NO_EXTRA, dir, mode, grid, s, a);
   FL_HIP(hipGetLastError());
   return FLH_OK;
@@ -613,6 +622,7 @@ static int launch_desc(int dir, void* user, uint64_t user_bytes, const flh_windo
   a.tiles_cap = tiles_cap;
   a.has_hint = h_hdr != nullptr;
   a.hint_total_tiles = h_hdr ? h_hdr->total_tiles : 0;
+  a.xcd = fl_xcd_full(grid);
   hipStream_t s = (hipStream_t)stream;
   const int mode = fl_stream_mode(dir, user_bytes);
   FL_LAUNCH_COPY(fl_copy_desc, FL_NO_EXTRA, dir, mode, dim3(grid), s, a);
@@ -674,6 +684,7 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
   a.n_lanes = u->n_lanes;
   a.tile_bytes = u->tile_bytes;
   a.tiles_per_chunk = (u->chunk_bytes + u->tile_bytes - 1) / u->tile_bytes;
+  a.xcd_map = fl_xcd_map(a.tiles_per_chunk, (uint32_t)n);
   // once the message no longer fits the Infinity Cache, write every window front to back
   a.dest_order = dir == 0 && (g_dest_order < 0 ? u->total_bytes > kWindowsCacheableBytes : g_dest_order != 0);
   for (int l = 0; l < FLH_MAX_LANES; ++l) a.credits[l] = (uint32_t)l < u->n_lanes ? u->credits[l] : 0;
@@ -862,8 +873,9 @@ int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
   const uint32_t tile = FLH_TILE_BYTES;
   const uint32_t grid = fl_copy_grid((bytes + tile - 1) / tile);
   hipStream_t s = (hipStream_t)stream;
-  if (fl_use_nt(2 * bytes)) FL_LAUNCH(fl_plain_copy<3>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
-  else FL_LAUNCH(fl_plain_copy<0>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile);
+  const uint32_t xcd = grid == (bytes + tile - 1) / tile ? fl_xcd_full(grid) : 0;   // only with one workgroup per tile
+  if (fl_use_nt(2 * bytes)) FL_LAUNCH(fl_plain_copy<3>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile, xcd);
+  else FL_LAUNCH(fl_plain_copy<0>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile, xcd);
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }

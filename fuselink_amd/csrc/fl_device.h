@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fl_internal.h"
+
 // ------------------------------------------------------------------------------------------------
 // wavefront scan primitives (DPP)
 // ------------------------------------------------------------------------------------------------
@@ -111,6 +113,26 @@ __device__ __forceinline__ uint64_t mod_u64(uint64_t a, uint64_t b) {
 // behind every branch waits another round trip to memory that the host wrote a moment ago and no cache holds
 // yet.  Reading one word of every 64-byte line of the block first, all in flight together, turns that chain
 // of misses into one miss plus scalar-cache hits.
+// Workgroups of a launch are handed to the eight XCDs in turn: workgroup b runs on XCD b mod 8, so with tile = b every
+// XCD touches every eighth tile of the stream.  xcd_tile() gives each XCD runs of 32 consecutive tiles instead (1 MiB
+// at 32 KiB tiles): workgroups 256 k .. 256 k + 255 still cover tiles 256 k .. 256 k + 255, but XCD x takes
+// 256 k + 32 x .. 256 k + 32 x + 31.  On plain copies this takes 3-5 % less time, inside the Infinity Cache and
+// beyond it (64 MiB: 20.1 -> 19.2 us, 1 GiB: 386 -> 360 us; runs of 4 or 256 tiles gain half as much or nothing).
+// `full` is the workgroup count rounded down to a multiple of 256 (0 switches the mapping off); workgroups from
+// there on keep tile = b, so the map is a permutation of the grid.
+__device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t full) {
+  return b < full ? (b & ~(kXcdBlock - 1)) + ((b & 7u) << kXcdRunShift) + ((b >> 3) & ((1u << kXcdRunShift) - 1)) : b;
+}
+// The same for a grid (tiles of a chunk, chunks) whose width is a power of two: xcd_map = full | log2(width).
+// Takes the workgroup's place in the grid, returns the tile of the chunk (x) and the chunk (y) it works on.
+__device__ __forceinline__ void xcd_tile_2d(uint32_t xcd_map, uint32_t& x, uint32_t& y) {
+  if (xcd_map == 0) return;
+  const uint32_t sh = xcd_map & 31u;
+  const uint32_t t = xcd_tile((y << sh) + x, xcd_map & ~(kXcdBlock - 1));
+  x = t & ((1u << sh) - 1);
+  y = t >> sh;
+}
+
 template <class Args>
 __device__ __forceinline__ void warm_kernel_args(const Args& a) {
   const uint32_t* p = reinterpret_cast<const uint32_t*>(&a);

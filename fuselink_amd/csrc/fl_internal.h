@@ -11,6 +11,13 @@ int fl_set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2
 // variables named NCCL_<NAME>, read once and cached.
 int64_t fl_param(const char* env_suffix, int64_t dflt);
 
+// Copy workgroups take their tiles in runs per XCD (xcd_tile() in fl_device.h): tiles per run and per block of 8 runs.
+#ifndef FL_XCD_RUN_SHIFT
+#define FL_XCD_RUN_SHIFT 5
+#endif
+constexpr uint32_t kXcdRunShift = FL_XCD_RUN_SHIFT;   // 32 tiles
+constexpr uint32_t kXcdBlock = 8u << kXcdRunShift;    // 8 XCDs x 32 tiles
+
 // Completion without a packet of its own: the next kernel the calling thread launches through the library carries
 // `hip_event` as its completion event (hipEventQuery / hipEventSynchronize on it then answer for that kernel),
 // which spares the barrier packet of a hipEventRecord behind it, during which the queue's next kernel does not

@@ -25,6 +25,7 @@ extern FL_LOCAL int g_sched_variant;       // 0 = pick the scheduler shape from 
 extern FL_LOCAL int g_sched_uniform_fast;
 extern FL_LOCAL int g_sched_seg_min;
 extern FL_LOCAL int g_copy_uniform_grid;
+extern FL_LOCAL int g_xcd_runs;            // copy workgroups take their tiles in runs per XCD (see xcd_tile)
 constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // plain copy: working sets up to this stay largely in the 256 MB Infinity Cache
 constexpr uint64_t kWindowsCacheableBytes = 256ull << 20;  // a message whose staging windows still fit the Infinity Cache
 
@@ -94,5 +95,10 @@ FL_LOCAL int fl_stream_mode(int dir, uint64_t bytes);
 // workgroups for a copy over max_tiles tiles: one per tile (the dispatcher then overlaps loads and stores of
 // different tiles); the kernels' stride loops only matter beyond the cap, which grid_per_cu can lower
 FL_LOCAL uint32_t fl_copy_grid(uint64_t max_tiles);
+
+// xcd_tile()'s `full` for a one-dimensional grid, and xcd_tile_2d()'s map for a grid (width, height): 0 (off) unless the
+// mapping is switched on, the grid has 256 workgroups or more and, for the latter, the width is a power of two below 2^32 / height.
+FL_LOCAL uint32_t fl_xcd_full(uint64_t grid);
+FL_LOCAL uint32_t fl_xcd_map(uint32_t width, uint32_t height);
 
 #endif  // FL_LAUNCH_H_

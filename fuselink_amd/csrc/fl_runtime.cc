@@ -29,6 +29,7 @@ int g_sched_variant = 0;
 int g_sched_uniform_fast = 1;
 int g_sched_seg_min = 4096;    // flh_tune("sched_seg_min"): chunks from which a workspace turns the scan into several workgroups
 int g_copy_uniform_grid = 1;
+int g_xcd_runs = 1;              // flh_tune("xcd_runs")
 
 namespace {
 thread_local ProfState t_prof;
@@ -93,6 +94,20 @@ int fl_stream_mode(int dir, uint64_t bytes) {
   if (bytes > kWindowsCacheableBytes) return 3;               // the windows no longer fit the Infinity Cache
   if (dir == 0) return bytes >= (128ull << 20) ? 1 : 0;       // read the user buffer once, keep the windows cacheable
   return bytes >= (16ull << 20) ? 2 : 0;                      // windows come from cache; the user buffer is written past it
+}
+
+uint32_t fl_xcd_full(uint64_t grid) {
+  if (!g_xcd_runs || grid < kXcdBlock || grid > 0xffffffffull) return 0;
+  return (uint32_t)grid & ~(kXcdBlock - 1);
+}
+
+uint32_t fl_xcd_map(uint32_t width, uint32_t height) {
+  if (width == 0 || (width & (width - 1)) || (uint64_t)width * height > 0xffffffffull) return 0;
+  const uint32_t full = fl_xcd_full((uint64_t)width * height);
+  if (!full) return 0;
+  uint32_t sh = 0;
+  while ((1u << sh) < width) ++sh;
+  return full | sh;   // full is a multiple of kXcdBlock >= 32, the shift stays below 32
 }
 
 uint32_t fl_copy_grid(uint64_t max_tiles) {
@@ -186,6 +201,7 @@ int flh_tune(const char* key, int64_t value) {
     return FLH_OK;
   }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
+  if (!strcmp(key, "xcd_runs")) { g_xcd_runs = value != 0; return FLH_OK; }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_seg_min")) {
     if (value < 1) return fl_set_error(FLH_E_ARG, "sched_seg_min < 1");

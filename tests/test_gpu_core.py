@@ -959,3 +959,80 @@ def test_one_scheduler_launch_for_a_message_that_moves_in_waves(fl, seed):
         core.reassemble(dst, w, sub, status, hint=hint)
     torch.cuda.synchronize()
     assert int(status.item()) == 0 and torch.equal(src, dst)
+
+
+@pytest.mark.parametrize("xcd_runs", [1, 0])
+@pytest.mark.parametrize("seed", range(6))
+def test_copies_with_tiles_taken_in_runs_per_xcd(fl, seed, xcd_runs):
+    """Grids of 256 workgroups and more hand each XCD runs of 32 consecutive tiles instead of every eighth tile.  The
+    map only changes which workgroup copies which tile: messages of several hundred small tiles (whole blocks of 256
+    and a ragged rest, tile counts per chunk that are powers of two and ones that are not) through the fused pair, the
+    table-driven pair with and without the host's header, the descriptor-driven pair and the plain copy, against the
+    oracle, with the map on and off."""
+    core, torch = fl
+    rng = np.random.default_rng(7300 + seed)
+    core.tune("xcd_runs", xcd_runs)
+    try:
+        lanes = int(rng.integers(1, 17))
+        tile = int(rng.choice([128, 256, 1024]))
+        tpc = int(rng.choice([1, 2, 4, 8, 16, 3, 6]))
+        chunk = tile * tpc
+        n = int(rng.integers(300, 2500)) // tpc + 1
+        total = n * chunk - int(rng.integers(0, chunk))
+        credits = rng.integers(0, 9, size=lanes).astype(np.uint32)
+        credits[int(rng.integers(0, lanes))] = 5
+        exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                             tile_bytes=tile, mode=ob.SCHED_RESET_OFFSETS)
+        assert int(exp_h["total_tiles"]) >= 256
+        src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+        src = _dev(torch, src_np)
+        caps = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+        exp_w = ob.cpu_stripe(src_np, exp_t, caps)
+
+        def fresh():
+            wins = [torch.zeros(max(c, 1) + 64, dtype=torch.uint8, device="cuda") for c in caps]
+            return wins, core.make_windows([t.data_ptr() for t in wins], caps)
+
+        def check(wins, dst, what):
+            torch.cuda.synchronize()
+            assert int(status.item()) == 0, what
+            for l in range(lanes):
+                got = wins[l].cpu().numpy()
+                np.testing.assert_array_equal(got[: caps[l]], exp_w[l][: caps[l]], err_msg=f"{what}, lane {l}")
+                assert not got[caps[l]:].any(), what
+            np.testing.assert_array_equal(dst.cpu().numpy(), src_np, err_msg=what)
+
+        status = core.new_status()
+        # scheduler folded into the copies
+        u = core.uniform_params(total, chunk, credits, tile_bytes=tile)
+        out = core.new_schedule_buffers(n, tile)
+        wins, w = fresh()
+        dst = torch.zeros_like(src)
+        core.stripe_uniform(src, w, u, status, out=out)
+        core.reassemble_uniform(dst, w, u, status)
+        check(wins, dst, "fused")
+        got_t, got_h = out.table_numpy(), out.hdr_numpy()
+        for f in ob.DESC_DTYPE.names:
+            np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f)
+        for f in ("total_bytes", "total_tiles", "n_chunks", "uniform_tiles", "lane_bytes", "lane_chunks"):
+            np.testing.assert_array_equal(got_h[f], exp_h[f], err_msg=f)
+        # table-driven: the search kernel (no host header), the two-dimensional grid (host header), the descriptors
+        sched = core.schedule(n_lanes=lanes, credits=[int(c) for c in credits], quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                              tile_bytes=tile, mode=core.SCHED_RESET_OFFSETS, tiles_capacity=int(exp_h["total_tiles"]) + 3)
+        torch.cuda.synchronize()
+        hint = core.uniform_hint(total, chunk, tile)
+        plain = core.Schedule(sched.table, sched.hdr, n, tile)
+        for what, s_, h_ in (("search", plain, None), ("grid", plain, hint), ("descriptors", sched, hint), ("descriptors, device header", sched, None)):
+            wins, w = fresh()
+            dst = torch.zeros_like(src)
+            core.stripe(src, w, s_, status, hint=h_)
+            core.reassemble(dst, w, s_, status, hint=h_)
+            check(wins, dst, what)
+        # the calibration copy
+        big = torch.randint(0, 256, (300 * core.TILE_BYTES + 77,), dtype=torch.uint8, device="cuda")
+        back = torch.zeros_like(big)
+        core.copy(back, big)
+        torch.cuda.synchronize()
+        assert torch.equal(back, big)
+    finally:
+        core.tune("xcd_runs", 1)
