@@ -35,9 +35,9 @@ WORKLOADS = {
 # HBM bytes per launch of the striping kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size.
 # None where no such run has been recorded for the workload.
-MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134300730, "cfg5_stress_1GiB_64KiB_16lanes": 2151677076,
-                    "cfg5_stress_1GiB_64KiB_16lanes/17 waves": 126497546,
-                    "cfg3_expert_parallel_256_blocks_8lanes": 1786033378, "cfg4_paged_kv_2x4096_pages_8lanes": 268684251}
+MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134300698, "cfg5_stress_1GiB_64KiB_16lanes": 2148002766,
+                    "cfg5_stress_1GiB_64KiB_16lanes/17 waves": 126498495,
+                    "cfg3_expert_parallel_256_blocks_8lanes": 1786036067, "cfg4_paged_kv_2x4096_pages_8lanes": 268550997}
 
 
 def algo_bytes_cold(nbytes: int) -> int:
