@@ -461,6 +461,7 @@ struct PageArgs {
   uint32_t sub_bytes;      // bytes of a page handled by one workgroup step
   uint32_t subs_per_page;
   int32_t page_shift;      // >= 0 when page_bytes is a power of two
+  uint32_t xcd_map;        // xcd_tile_2d()'s map when the grid has one row per chunk; 0 = off
 };
 
 constexpr uint32_t kLdsStage = 16384;
@@ -473,9 +474,11 @@ __global__ __launch_bounds__(kCopyBlock) void fl_page_tiles(PageArgs a) {
   warm_kernel_args(a);
   // grid: x = (page in chunk, part of page), y = chunk (stepping by the grid's height past 65535 chunks); no
   // 64-bit division stands between a workgroup and its row
-  const uint32_t k = a.subs_per_page == 1 ? blockIdx.x : blockIdx.x / a.subs_per_page;
-  const uint32_t sub = blockIdx.x - k * a.subs_per_page;
-  for (uint32_t c = blockIdx.y; c < a.n_chunks; c += gridDim.y) {
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  xcd_tile_2d(a.xcd_map, bx, by);
+  const uint32_t k = a.subs_per_page == 1 ? bx : bx / a.subs_per_page;
+  const uint32_t sub = bx - k * a.subs_per_page;
+  for (uint32_t c = by; c < a.n_chunks; c += gridDim.y) {
     const flh_chunk_desc d = a.table[c];
     const uint64_t in_chunk = (uint64_t)k * a.page_bytes + (uint64_t)sub * a.sub_bytes;
     if (in_chunk >= d.len) continue;
@@ -842,6 +845,7 @@ static int launch_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t
   hipStream_t s = (hipStream_t)stream;
   const int mode = fl_stream_mode(dir, (uint64_t)n_chunks * pages_per_chunk * page_bytes);
   const dim3 grid3((uint32_t)per_chunk, n_chunks < 65535 ? n_chunks : 65535);
+  a.xcd_map = grid3.y == n_chunks ? fl_xcd_map(grid3.x, grid3.y) : 0;   // only with one grid row per chunk
 #define FL_LDS_ON , true
 #define FL_LDS_OFF , false
   if (use_lds) FL_LAUNCH_COPY(fl_page_tiles, FL_LDS_ON, dir, mode, grid3, s, a);
