@@ -119,7 +119,8 @@ __device__ __forceinline__ uint64_t mod_u64(uint64_t a, uint64_t b) {
 // 256 k + 32 x .. 256 k + 32 x + 31.  On plain copies this takes 3-5 % less time, inside the Infinity Cache and
 // beyond it (64 MiB: 20.1 -> 19.2 us, 1 GiB: 386 -> 360 us; runs of 4 or 256 tiles gain half as much or nothing).
 // `full` is the workgroup count rounded down to a multiple of 256 (0 switches the mapping off); workgroups from
-// there on keep tile = b, so the map is a permutation of the grid.
+// there on keep tile = b, so the map is a permutation of the grid (on a partition of the GPU that hands workgroups out
+// differently it stays one, and only the gain is lost).
 __device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t full) {
   return b < full ? (b & ~(kXcdBlock - 1)) + ((b & 7u) << kXcdRunShift) + ((b >> 3) & ((1u << kXcdRunShift) - 1)) : b;
 }
