@@ -62,6 +62,7 @@ SIGNATURES = {
     "flh_constant": (C.c_int64, [C.c_int]),
     "flh_schedule_workspace_bytes": (C.c_uint64, [C.c_uint32]),
     "flh_schedule": (C.c_int, [C.POINTER(SchedParams), C.c_void_p]),
+    "flh_schedule_static": (C.c_int, [C.POINTER(SchedParams), C.c_void_p]),
     "flh_stripe": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p, C.POINTER(SchedHdr),
                              C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
     "flh_reassemble": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.c_void_p, C.c_void_p,

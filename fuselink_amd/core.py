@@ -108,7 +108,7 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
              total_bytes: int = 0, chunk_bytes: int = 0, src_off: Optional[torch.Tensor] = None, src_base: int = 0,
              epoch_len: int = 0, tile_bytes: int = TILE_BYTES, mode: int = 0, state: Optional[torch.Tensor] = None,
              out: Optional[Schedule] = None, stream: Optional[torch.cuda.Stream] = None, by_lane: bool = False,
-             tiles_capacity: int = 0, workspace: bool = False, wave_chunks: int = 0) -> Schedule:
+             tiles_capacity: int = 0, workspace: bool = False, wave_chunks: int = 0, static_workspace: bool = False) -> Schedule:
     """Launches the scheduler kernel (flh_schedule).  `credits` is a uint32/int32 device tensor of
     shape [rows, n_lanes]; `sizes` a uint32/int32 device tensor of chunk sizes, or None for the
     uniform split of `total_bytes` by `chunk_bytes`."""
@@ -154,7 +154,11 @@ def schedule(*, n_lanes: int, credits: torch.Tensor, quantum: int, sizes: Option
         if out.workspace is None or out.workspace.numel() < need:
             out.workspace = _dev_bytes(need, dev)
         p.d_workspace, p.workspace_bytes = _ptr(out.workspace), out.workspace.numel()
-    check(lib.flh_schedule(C.byref(p), _stream_ptr(stream)))
+    if static_workspace:  # the library's own per-device workspace: nothing is allocated by the call (flh_schedule_static)
+        assert not workspace
+        check(lib.flh_schedule_static(C.byref(p), _stream_ptr(stream)))
+    else:
+        check(lib.flh_schedule(C.byref(p), _stream_ptr(stream)))
     return out
 
 

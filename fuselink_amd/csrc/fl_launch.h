@@ -101,4 +101,9 @@ FL_LOCAL uint32_t fl_copy_grid(uint64_t max_tiles);
 FL_LOCAL uint32_t fl_xcd_full(uint64_t grid);
 FL_LOCAL uint32_t fl_xcd_map(uint32_t width, uint32_t height);
 
+// Resolves, once per device and with that device current, the address of the device's copy of the workspace that
+// flh_schedule_static brings along (hipGetSymbolAddress); called by flh_init, and by the entry point's first call on
+// any other device.
+extern "C" FL_LOCAL int fl_sched_scratch_resolve(int device);
+
 #endif  // FL_LAUNCH_H_

@@ -154,7 +154,7 @@ int flh_init(int device) {
   g_grid_per_cu = (int)env_i64("NCCL_FUSELINK_GRID_PER_CU", g_grid_per_cu);
   g_nontemporal = (int)env_i64("NCCL_FUSELINK_NONTEMPORAL", g_nontemporal);
   if (g_grid_per_cu < 0) g_grid_per_cu = 0;
-  return FLH_OK;
+  return fl_sched_scratch_resolve(device);
 }
 
 int flh_prof_begin(int capacity) {

@@ -3,6 +3,7 @@
 //   * fl_schedule_uniform_kernel : uniform split with quantum-sized chunks; closed form, any number of workgroups
 // All cross-lane traffic is DPP row shifts and row broadcasts; LDS only passes per-wavefront totals between the
 // wavefronts of the one workgroup and caches the credit rows.
+#include <atomic>
 #include <cstring>
 
 #include "fl_device.h"
@@ -64,6 +65,16 @@ struct SegHeader {         // the carried state as it was when the call began
   SegPartial part[1];      // one per segment follows
 };
 __host__ __device__ inline uint32_t seg_count(uint32_t n) { return (n + kSegChunks - 1) / kSegChunks; }
+
+// The workspace that flh_schedule_static brings along for callers that cannot allocate one: one copy per GPU, held until
+// the process ends, sized for FLH_SCHED_STATIC_MAX_CHUNKS chunks.  In host code `scratch` is only a handle for
+// hipGetSymbolAddress; the address the kernels get is the per-device one kept in g_scratch_ptr.
+constexpr uint64_t kScratchBytes = sizeof(SegHeader) + (uint64_t)(FLH_SCHED_STATIC_MAX_CHUNKS / kSegChunks) * sizeof(SegPartial);
+static_assert(FLH_SCHED_STATIC_MAX_CHUNKS % kSegChunks == 0, "the limit is a whole number of segments");
+static_assert(kScratchBytes <= 256u * 1024u, "the static workspace is meant to stay modest");
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kScratchDevices = 64;
+std::atomic<void*> g_scratch_ptr[kScratchDevices];
 
 
 
@@ -959,7 +970,9 @@ static int expand_tiles(const flh_sched_params* p, hipStream_t s) {
   return FLH_OK;
 }
 
-int flh_schedule(const flh_sched_params* p, void* stream) {
+// flh_schedule with the workspace named apart from the parameters: the caller's (flh_schedule) or the library's own
+// per-device array (flh_schedule_static).
+static int schedule_with(const flh_sched_params* p, void* stream, void* d_workspace, uint64_t workspace_bytes) {
   if (!p) return fl_set_error(FLH_E_ARG, "null params");
   if (p->n_lanes == 0 || p->n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "n_lanes %u not in 1..%d", p->n_lanes, FLH_MAX_LANES);
   if (p->n_rows == 0) return fl_set_error(FLH_E_ARG, "credit table missing");
@@ -1016,13 +1029,13 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   }
   if (p->wave_chunks && n > 0) return fl_set_error(FLH_E_ARG, "wave_chunks: the closed-form scheduler is switched off by a tunable");
   // a long list with a workspace: one workgroup per kSegChunks chunks, three launches
-  if (p->d_workspace && variant == 0 && n >= (uint32_t)g_sched_seg_min && p->n_rows <= (uint32_t)kRowCache && !p->d_table_by_lane) {
+  if (d_workspace && variant == 0 && n >= (uint32_t)g_sched_seg_min && p->n_rows <= (uint32_t)kRowCache && !p->d_table_by_lane) {
     const uint32_t G = seg_count(n);
     const uint64_t need = flh_schedule_workspace_bytes(n);
-    if (p->workspace_bytes < need) return fl_set_error(FLH_E_ARG, "workspace of %llu bytes, %llu needed for %u chunks", (unsigned long long)p->workspace_bytes,
+    if (workspace_bytes < need) return fl_set_error(FLH_E_ARG, "workspace of %llu bytes, %llu needed for %u chunks", (unsigned long long)workspace_bytes,
                                                         (unsigned long long)need, n);
-    if ((uintptr_t)p->d_workspace % alignof(SegHeader)) return fl_set_error(FLH_E_ARG, "workspace must be %zu-byte aligned", alignof(SegHeader));
-    a.seg = (SegHeader*)p->d_workspace;
+    if ((uintptr_t)d_workspace % alignof(SegHeader)) return fl_set_error(FLH_E_ARG, "workspace must be %zu-byte aligned", alignof(SegHeader));
+    a.seg = (SegHeader*)d_workspace;
     FL_LAUNCH(fl_sched_seg_totals, dim3(G), dim3(kSegBlock), 0, s, a);
     static_assert(kSegChunks == 8 * kWave * 2, "a segment is one pass of fl_schedule_kernel<8, 2>");
     FL_LAUNCH((fl_schedule_kernel<8, 2, true>), dim3(G), dim3(8 * kWave), 0, s, a);
@@ -1047,6 +1060,37 @@ int flh_schedule(const flh_sched_params* p, void* stream) {
   }
   FL_HIP(hipGetLastError());
   return expand_tiles(p, s);
+}
+
+int flh_schedule(const flh_sched_params* p, void* stream) {
+  return schedule_with(p, stream, p ? p->d_workspace : nullptr, p ? p->workspace_bytes : 0);
+}
+
+int fl_sched_scratch_resolve(int device) {
+  if (device < 0 || device >= kScratchDevices) return fl_set_error(FLH_E_ARG, "device %d has no slot for the scheduler's own workspace (%d devices at most)", device, kScratchDevices);
+  if (g_scratch_ptr[device].load(std::memory_order_acquire)) return FLH_OK;
+  int current = -1;
+  FL_HIP(hipGetDevice(&current));
+  if (current != device) return fl_set_error(FLH_E_STATE, "device %d must be current to resolve its copy of the scheduler's workspace (current: %d)", device, current);
+  void* ptr = nullptr;
+  FL_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));   // this device's copy of the array; `scratch` itself is not an address the host may use
+  if (!ptr) return fl_set_error(FLH_E_HIP, "hipGetSymbolAddress returned no address for the scheduler's workspace on device %d", device);
+  g_scratch_ptr[device].store(ptr, std::memory_order_release);
+  return FLH_OK;
+}
+
+int flh_schedule_static(const flh_sched_params* p, void* stream) {
+  if (!p) return fl_set_error(FLH_E_ARG, "null params");
+  if (p->n_chunks > FLH_SCHED_STATIC_MAX_CHUNKS)
+    return fl_set_error(FLH_E_ARG, "%u chunks exceed the %u that the library's own workspace serves; lend one to flh_schedule instead", p->n_chunks,
+                        (unsigned)FLH_SCHED_STATIC_MAX_CHUNKS);
+  int rc = fl_need_init();
+  if (rc) return rc;
+  int device = -1;
+  FL_HIP(hipGetDevice(&device));
+  rc = fl_sched_scratch_resolve(device);   // resolved at flh_init for the device named there; a first call on another device lands here
+  if (rc) return rc;
+  return schedule_with(p, stream, g_scratch_ptr[device].load(std::memory_order_acquire), kScratchBytes);
 }
 
 }  // extern "C"

@@ -171,6 +171,17 @@ int flh_prof_end(double* us_out, int* kernel_out, int max);
  * live policy lane = index mod lanes (src/fuselink.h:235). */
 int flh_schedule(const flh_sched_params* p, void* stream);
 
+/* flh_schedule for callers that cannot allocate and cannot lend a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same parameters, table, header
+ * and state as flh_schedule; p->d_workspace / p->workspace_bytes are ignored, and a chunk list long enough for the scan over
+ * several workgroups uses a workspace of the library's own instead: a static device array of about 224 KiB that every GPU
+ * the library runs on holds until the process ends, which serves lists of up to FLH_SCHED_STATIC_MAX_CHUNKS chunks
+ * (more: FLH_E_ARG, lend a workspace to flh_schedule).  The call allocates and frees nothing.  All calls on one GPU
+ * share that GPU's array: two calls that overlap on one GPU (different streams, or threads) race; calls in stream
+ * order on one stream are safe, every launch rewrites what it reads. */
+#define FLH_SCHED_STATIC_MAX_CHUNKS (1u << 20)
+int flh_schedule_static(const flh_sched_params* p, void* stream);
+
 /* ---- striping / reassembly --------------------------------------------------------------------
  * flh_stripe replaces the send side of ncclIbMultiSend (src/plugin.cc:1467-1495: per-request split,
  * RDMA write out of the staged copy at flmr->addr[dev] + (data - start_addr), src/plugin.cc:1582):
