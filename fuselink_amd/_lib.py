@@ -39,15 +39,21 @@ class SchedParams(C.Structure):
 class UniformParams(C.Structure):
     _fields_ = [("total_bytes", C.c_uint64), ("src_base", C.c_uint64), ("epoch_bytes", C.c_uint64),
                 ("chunk_bytes", C.c_uint32), ("n_lanes", C.c_uint32), ("tile_bytes", C.c_uint32), ("pad", C.c_uint32),
-                ("credits", C.c_uint32 * MAX_LANES)]
+                ("credits", C.c_uint32 * MAX_LANES), ("d_done_word", C.c_void_p), ("d_done_count", C.c_void_p),
+                ("done_value", C.c_uint32), ("pad2", C.c_uint32), ("done_event", C.c_void_p)]
 
 
-BATCH_MAX = 8
+BATCH_MAX = 32
+SEG_MAX = 8
+
+
+class BatchSegment(C.Structure):
+    _fields_ = [("epoch_bytes", C.c_uint64), ("n_req", C.c_uint32), ("pad", C.c_uint32), ("credits", C.c_uint32 * MAX_LANES)]
 
 
 class BatchParams(C.Structure):
-    _fields_ = [("u", UniformParams), ("n_req", C.c_uint32), ("pad", C.c_uint32), ("d_src", C.c_void_p * BATCH_MAX),
-                ("d_dst", C.c_void_p * BATCH_MAX), ("bytes", C.c_uint64 * BATCH_MAX)]
+    _fields_ = [("u", UniformParams), ("n_req", C.c_uint32), ("n_seg", C.c_uint32), ("d_src", C.c_void_p * BATCH_MAX),
+                ("d_dst", C.c_void_p * BATCH_MAX), ("bytes", C.c_uint64 * BATCH_MAX), ("seg", BatchSegment * SEG_MAX)]
 
 
 class Windows(C.Structure):
@@ -78,6 +84,7 @@ SIGNATURES = {
     "flh_window_export_dmabuf": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.POINTER(C.c_int)]),
     "flh_stripe_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_reassemble_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p]),
+    "flh_batch_layout": (C.c_int, [C.POINTER(BatchParams), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "flh_gather_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),
                                    C.c_void_p, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p]),
     "flh_scatter_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),

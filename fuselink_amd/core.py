@@ -249,15 +249,31 @@ def reassemble_uniform(dst: torch.Tensor, win: Windows, u: UniformParams, status
 
 
 def batch_params(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor], chunk_bytes: int, credits: Sequence[int], *,
-                 epoch_bytes: int = 0, tile_bytes: int = TILE_BYTES) -> BatchParams:
-    """Several requests handled as one message (flh_stripe_batch / flh_reassemble_batch)."""
+                 epoch_bytes: int = 0, tile_bytes: int = TILE_BYTES, segments=None) -> BatchParams:
+    """Several requests in one launch (flh_stripe_batch / flh_reassemble_batch).  Without `segments` they form one
+    message under `credits` / `epoch_bytes`; with it, `segments` is a list of (n_req, credits, epoch_bytes), each
+    scheduled as a message of its own."""
     b = BatchParams()
     sizes = [t.numel() * t.element_size() for t in srcs]
     b.u = uniform_params(sum(sizes), chunk_bytes, credits, epoch_bytes=epoch_bytes, tile_bytes=tile_bytes)
     b.n_req = len(srcs)
     for q, (s, d, n) in enumerate(zip(srcs, dsts, sizes)):
         b.d_src[q], b.d_dst[q], b.bytes[q] = s.data_ptr(), d.data_ptr(), n
+    if segments is not None:
+        b.n_seg = len(segments)
+        for k, (n_req, row, eb) in enumerate(segments):
+            b.seg[k].n_req, b.seg[k].epoch_bytes = n_req, eb
+            for l, c in enumerate(row):
+                b.seg[k].credits[l] = int(c)
     return b
+
+
+def batch_layout(b: BatchParams):
+    """flh_batch_layout: where the batch leaves every lane's window, and every segment's lane bases."""
+    ends = (C.c_uint64 * MAX_LANES)()
+    bases = (C.c_uint64 * (8 * MAX_LANES))()
+    check(_lib.load().flh_batch_layout(C.byref(b), ends, bases))
+    return list(ends), [list(bases[k * MAX_LANES:(k + 1) * MAX_LANES]) for k in range(8)]
 
 
 def stripe_batch(b: BatchParams, win: Windows, status: torch.Tensor, out: Optional[Schedule] = None,

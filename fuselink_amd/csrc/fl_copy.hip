@@ -7,6 +7,7 @@
 // The path is an HBM-bound byte mover; nothing here contracts, so no MFMA.
 #include <cstring>
 
+#include "fl_closed_form.h"
 #include "fl_device.h"
 #include "fl_launch.h"
 
@@ -239,25 +240,43 @@ struct FusedArgs {
   // The lane of a slot is then found by a four-step binary search over pfx_ex[] (exclusive credit prefixes,
   // W from index n_lanes on), read straight from the argument block.
   uint32_t fast;
-  uint32_t stamp_value;      // see stamp
+  uint32_t done_value;       // see done_word
   uint64_t magic;
   uint32_t cnt0[FLH_MAX_LANES];
   uint32_t pfx_ex[FLH_MAX_LANES + 1];
   uint32_t xcd_map;          // xcd_tile_2d()'s map for the grid (tiles per chunk, chunks); 0 = off
-  // Stripe only, may be null: a host-visible word that the launch's first workgroup sets to stamp_value as it starts.
-  // A kernel starts once everything queued before it on its stream has finished, so a caller that numbers its
-  // launches learns from the word that all earlier ones are complete, without an event behind each of them.
-  uint32_t* stamp;
+  // Reassembly only, may be null: a host-visible word that the last workgroup to finish sets to done_value, after
+  // every workgroup's stores have been released (counted in *done_count, device memory, zero between launches).
+  uint32_t* done_word;
+  uint32_t* done_count;
 };
 
-// Several requests as one message: chunk c belongs to the request r with first[r] <= c < first[r+1];
-// its bytes live at user[r] + (c - first[r]) * chunk_bytes.
+// Several requests in one launch.  Chunk c (counted over the launch) belongs to the request r with
+// first[r] <= c < first[r + 1]; its bytes live at req_user[r] + (c - first[r]) * chunk_bytes.  Request r belongs to
+// segment seg_of[r], and a segment is scheduled as the one message its requests form, from its own place in its credit
+// epoch under its own credit row (the per-segment constants are those FusedArgs holds for a lone message), into the
+// windows from base128[lane] * 128 on.
+struct BatchSeg {
+  uint64_t magic;                           // ceil(2^64 / W); 0 stands for W == 1
+  uint32_t quanta_before;
+  uint32_t first_chunk;
+  uint32_t pfx_ex[FLH_MAX_LANES + 1];       // exclusive credit prefixes, W from index n_lanes on
+  uint32_t cnt0[FLH_MAX_LANES];             // the lane's slots before the segment
+  uint32_t base128[FLH_MAX_LANES];          // where the segment starts in the lane's window, in units of 128 bytes
+  uint32_t n_chunks;
+  uint32_t short_by;                        // bytes by which its last chunk falls short of chunk_bytes
+  uint32_t zero;                            // the row had no credit (equal credits stand in)
+  uint32_t pad;
+};
 struct FusedBatchArgs : FusedArgs {
-  uint32_t n_req;
-  uint32_t first[FLH_BATCH_MAX];   // first chunk of each request
+  uint32_t n_req, n_seg;
+  uint32_t first[FLH_BATCH_MAX];            // first chunk of each request; 0xffffffff from n_req on
+  uint8_t seg_of[FLH_BATCH_MAX];
   uint8_t* req_user[FLH_BATCH_MAX];
   uint64_t req_bytes[FLH_BATCH_MAX];
+  BatchSeg seg[FLH_SEG_MAX];
 };
+static_assert(sizeof(FusedBatchArgs) <= 4096, "a kernel's argument block holds 4 KiB");
 template <class A> struct is_batch { static constexpr bool value = false; };
 template <> struct is_batch<FusedBatchArgs> { static constexpr bool value = true; };
 
@@ -301,87 +320,106 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
   return full * c + part;
 }
 
+// One workgroup's share of a fused launch: tile bx of the chunk that grid row by stands for.
 template <int DIR, int NT, class Args>
-__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
+__device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by) {
   constexpr bool BATCH = is_batch<Args>::value;
   constexpr bool PAGED = is_paged<Args>::value;
-  warm_kernel_args(a);
-  uint32_t bx = blockIdx.x, by = blockIdx.y;   // tile of the chunk, chunk (in message or destination order)
-  xcd_tile_2d(a.xcd_map, bx, by);
   if (by >= a.n_chunks) return;
   uint32_t c = by, lane = 0;
   uint64_t before;
-  if (DIR == 0 && a.dest_order) {
-    FusedRow r;
-    fused_row(a, r);
-    uint64_t K = 0, hi = r.pfx[0];
-    // by = k-th chunk in destination order: find the lane whose group holds k, then invert the
-    // closed form -- the j-th slot of a lane with credit c_l and first slot K_l is (j / c_l) * W + K_l + j mod c_l.
-    const uint64_t x0 = a.quanta_before, x1 = a.quanta_before + a.n_chunks;
-    const uint64_t f0 = div_u64(x0, r.W), f1 = div_u64(x1, r.W);
-    const uint64_t r0 = x0 - f0 * r.W, r1 = x1 - f1 * r.W;
-    uint64_t k = by, cnt0 = 0;
-    bool found = false;
-    uint64_t lo = 0;
-#pragma unroll
-    for (int l = 0; l < FLH_MAX_LANES; ++l) {
-      const uint64_t up = r.pfx[l], cl = up - lo;
-      const uint64_t p0 = r0 <= lo ? 0 : (r0 - lo < cl ? r0 - lo : cl);
-      const uint64_t p1 = r1 <= lo ? 0 : (r1 - lo < cl ? r1 - lo : cl);
-      const uint64_t c0 = f0 * cl + p0;             // slots of the lane before this message
-      const uint64_t nl = f1 * cl + p1 - c0;        // chunks of this message on the lane
-      if (!found && (uint32_t)l < a.n_lanes) {
-        if (k < nl) { found = true; lane = l; K = lo; hi = up; cnt0 = c0; } else { k -= nl; }
-      }
-      lo = up;
-    }
-    const uint64_t cl = hi - K;
-    const uint64_t ja = cnt0 + k;                   // index among all slots of the lane in this epoch
-    const uint64_t rnd = div_u64(ja, cl);
-    c = (uint32_t)(rnd * r.W + K + (ja - rnd * cl) - a.quanta_before);
-    before = k;
-  } else if (a.fast) {
-    const uint32_t j = (uint32_t)a.quanta_before + c;
-    const uint32_t full = a.magic ? (uint32_t)__umul64hi((uint64_t)j, a.magic) : j;  // j / W (magic 0 stands for W = 1)
-    const uint32_t slot = j - full * a.pfx_ex[FLH_MAX_LANES];  // the last entry is always W
-    // the last lane whose first slot is not beyond this one (lanes without credit share their successor's first slot)
-    static_assert(FLH_MAX_LANES == 16, "the search below takes four steps");
-    if (a.pfx_ex[lane + 8] <= slot) lane += 8;
-    if (a.pfx_ex[lane + 4] <= slot) lane += 4;
-    if (a.pfx_ex[lane + 2] <= slot) lane += 2;
-    if (a.pfx_ex[lane + 1] <= slot) lane += 1;
-    const uint32_t K = a.pfx_ex[lane], hi = a.pfx_ex[lane + 1], c0 = a.cnt0[lane];   // indexed scalar loads from the argument block
-    before = (uint64_t)full * (hi - K) + (slot - K) - c0;  // slot lies inside the lane's span [K, hi)
-  } else {
-    FusedRow r;
-    fused_row(a, r);
-    uint64_t K = 0, hi = r.pfx[0];
-    const uint64_t j = a.quanta_before + c;
-    const uint64_t slot = mod_u64(j, r.W);
-#pragma unroll
-    for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
-      if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; }
-    }
-    before = fused_cnt(r.W, K, hi, j) - fused_cnt(r.W, K, hi, a.quanta_before);
-  }
-  const uint64_t chunk_off = (uint64_t)c * a.chunk_bytes;
-  const uint64_t rem = a.total_bytes - chunk_off;
-  const uint32_t len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
-  const uint64_t src_off = a.src_base + chunk_off;
-  const uint64_t win_off = before * a.chunk_bytes;
-  // where the chunk's bytes live on the user side: in the one buffer, or in its request's buffer
+  // where the chunk's bytes live on the user side (the one buffer, or its request's), its length, its place in the
+  // message for the table, and where its lane's window starts for it
   uint8_t* user = a.user;
-  uint64_t user_off = src_off, user_bytes = a.user_bytes;
+  uint64_t user_off, user_bytes = a.user_bytes, src_off, win_base = 0;
+  uint32_t len;
   if constexpr (BATCH) {
-    uint32_t first = 0;
-    user = a.req_user[0];
-    user_bytes = a.req_bytes[0];
+    static_assert(FLH_BATCH_MAX == 32, "the search below takes five steps");
+    uint32_t r = a.first[16] <= c ? 16 : 0;     // entries from n_req on hold 0xffffffff
+    if (a.first[r + 8] <= c) r += 8;
+    if (a.first[r + 4] <= c) r += 4;
+    if (a.first[r + 2] <= c) r += 2;
+    if (a.first[r + 1] <= c) r += 1;
+    const BatchSeg& g = a.seg[a.seg_of[r]];     // scalar loads from the argument block, register offsets
+    const uint32_t in_seg = c - g.first_chunk;
+    const uint32_t j = g.quanta_before + in_seg;
+    const uint32_t full = g.magic ? (uint32_t)__umul64hi((uint64_t)j, g.magic) : j;
+    const uint32_t slot = j - full * g.pfx_ex[FLH_MAX_LANES];
+    static_assert(FLH_MAX_LANES == 16, "the search below takes four steps");
+    if (g.pfx_ex[lane + 8] <= slot) lane += 8;
+    if (g.pfx_ex[lane + 4] <= slot) lane += 4;
+    if (g.pfx_ex[lane + 2] <= slot) lane += 2;
+    if (g.pfx_ex[lane + 1] <= slot) lane += 1;
+    const uint32_t K = g.pfx_ex[lane], hi = g.pfx_ex[lane + 1];
+    before = (uint64_t)full * (hi - K) + (slot - K) - g.cnt0[lane];
+    win_base = (uint64_t)g.base128[lane] * 128u;
+    user = a.req_user[r];
+    user_bytes = a.req_bytes[r];
+    user_off = (uint64_t)(c - a.first[r]) * a.chunk_bytes;
+    const uint64_t rem = user_bytes - user_off;
+    len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
+    src_off = (uint64_t)in_seg * a.chunk_bytes;
+  } else {
+    if (DIR == 0 && a.dest_order) {
+      FusedRow r;
+      fused_row(a, r);
+      uint64_t K = 0, hi = r.pfx[0];
+      // by = k-th chunk in destination order: find the lane whose group holds k, then invert the
+      // closed form -- the j-th slot of a lane with credit c_l and first slot K_l is (j / c_l) * W + K_l + j mod c_l.
+      const uint64_t x0 = a.quanta_before, x1 = a.quanta_before + a.n_chunks;
+      const uint64_t f0 = div_u64(x0, r.W), f1 = div_u64(x1, r.W);
+      const uint64_t r0 = x0 - f0 * r.W, r1 = x1 - f1 * r.W;
+      uint64_t k = by, cnt0 = 0;
+      bool found = false;
+      uint64_t lo = 0;
 #pragma unroll
-    for (int q = 1; q < FLH_BATCH_MAX; ++q) {
-      if ((uint32_t)q < a.n_req && a.first[q] <= c) { first = a.first[q]; user = a.req_user[q]; user_bytes = a.req_bytes[q]; }
+      for (int l = 0; l < FLH_MAX_LANES; ++l) {
+        const uint64_t up = r.pfx[l], cl = up - lo;
+        const uint64_t p0 = r0 <= lo ? 0 : (r0 - lo < cl ? r0 - lo : cl);
+        const uint64_t p1 = r1 <= lo ? 0 : (r1 - lo < cl ? r1 - lo : cl);
+        const uint64_t c0 = f0 * cl + p0;             // slots of the lane before this message
+        const uint64_t nl = f1 * cl + p1 - c0;        // chunks of this message on the lane
+        if (!found && (uint32_t)l < a.n_lanes) {
+          if (k < nl) { found = true; lane = l; K = lo; hi = up; cnt0 = c0; } else { k -= nl; }
+        }
+        lo = up;
+      }
+      const uint64_t cl = hi - K;
+      const uint64_t ja = cnt0 + k;                   // index among all slots of the lane in this epoch
+      const uint64_t rnd = div_u64(ja, cl);
+      c = (uint32_t)(rnd * r.W + K + (ja - rnd * cl) - a.quanta_before);
+      before = k;
+    } else if (a.fast) {
+      const uint32_t j = (uint32_t)a.quanta_before + c;
+      const uint32_t full = a.magic ? (uint32_t)__umul64hi((uint64_t)j, a.magic) : j;  // j / W (magic 0 stands for W = 1)
+      const uint32_t slot = j - full * a.pfx_ex[FLH_MAX_LANES];  // the last entry is always W
+      // the last lane whose first slot is not beyond this one (lanes without credit share their successor's first slot)
+      static_assert(FLH_MAX_LANES == 16, "the search below takes four steps");
+      if (a.pfx_ex[lane + 8] <= slot) lane += 8;
+      if (a.pfx_ex[lane + 4] <= slot) lane += 4;
+      if (a.pfx_ex[lane + 2] <= slot) lane += 2;
+      if (a.pfx_ex[lane + 1] <= slot) lane += 1;
+      const uint32_t K = a.pfx_ex[lane], hi = a.pfx_ex[lane + 1], c0 = a.cnt0[lane];   // indexed scalar loads from the argument block
+      before = (uint64_t)full * (hi - K) + (slot - K) - c0;  // slot lies inside the lane's span [K, hi)
+    } else {
+      FusedRow r;
+      fused_row(a, r);
+      uint64_t K = 0, hi = r.pfx[0];
+      const uint64_t j = a.quanta_before + c;
+      const uint64_t slot = mod_u64(j, r.W);
+#pragma unroll
+      for (int l = 0; l + 1 < FLH_MAX_LANES; ++l) {
+        if ((uint32_t)(l + 1) < a.n_lanes && r.pfx[l] <= slot) { lane = l + 1; K = r.pfx[l]; hi = r.pfx[l + 1]; }
+      }
+      before = fused_cnt(r.W, K, hi, j) - fused_cnt(r.W, K, hi, a.quanta_before);
     }
-    user_off = (uint64_t)(c - first) * a.chunk_bytes;
+    const uint64_t chunk_off = (uint64_t)c * a.chunk_bytes;
+    const uint64_t rem = a.total_bytes - chunk_off;
+    len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
+    src_off = a.src_base + chunk_off;
+    user_off = src_off;
   }
+  const uint64_t win_off = win_base + before * a.chunk_bytes;
 
   if (DIR == 0 && bx == 0 && threadIdx.x == 0 && a.table) {
     flh_chunk_desc d;
@@ -393,36 +431,73 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
     d.epoch = 0;
     a.table[c] = d;
   }
-  if (DIR == 0 && bx == 0 && by == 0 && a.stamp && threadIdx.x == 0)
-    __hip_atomic_store(a.stamp, a.stamp_value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   if (DIR == 0 && bx == 0 && by == 0 && a.hdr) {  // header: per-lane totals in closed form
-    FusedRow r;
-    fused_row(a, r);
     const uint32_t t = threadIdx.x;
-    const uint64_t last = a.n_chunks - 1;
-    const uint64_t len_last = a.total_bytes - last * a.chunk_bytes;
-    if (t < FLH_MAX_LANES) {
-      uint64_t chunks = 0, bytes = 0;
-      if (t < a.n_lanes) {
-        uint64_t k_lo = 0, k_hi = 0;  // selected, not indexed: indexing would push the row into scratch memory
-#pragma unroll
-        for (int l = 0; l < FLH_MAX_LANES; ++l) {
-          if ((uint32_t)l == t) { k_hi = r.pfx[l]; k_lo = l ? r.pfx[l > 0 ? l - 1 : 0] : 0; }
+    if constexpr (BATCH) {
+      // the launch's totals: every segment's closed form, summed
+      if (t < FLH_MAX_LANES) {
+        uint64_t chunks = 0, bytes = 0;
+        if (t < a.n_lanes) {
+          for (uint32_t s = 0; s < a.n_seg; ++s) {
+            const BatchSeg& g = a.seg[s];
+            const uint32_t W = g.pfx_ex[FLH_MAX_LANES], K = g.pfx_ex[t], cl = g.pfx_ex[t + 1] - K;
+            const uint32_t x1 = g.quanta_before + g.n_chunks;
+            const uint32_t full = g.magic ? (uint32_t)__umul64hi((uint64_t)x1, g.magic) : x1;
+            const uint32_t rem = x1 - full * W;
+            const uint32_t part = rem <= K ? 0 : (rem - K < cl ? rem - K : cl);
+            const uint64_t k = (uint64_t)full * cl + part - g.cnt0[t];
+            const uint32_t xl = x1 - 1;                       // the segment's last chunk: short, and on which lane
+            const uint32_t fl = g.magic ? (uint32_t)__umul64hi((uint64_t)xl, g.magic) : xl;
+            const uint32_t sl = xl - fl * W;
+            chunks += k;
+            bytes += k * a.chunk_bytes - ((g.n_chunks && sl >= K && sl < K + cl) ? g.short_by : 0);
+          }
         }
-        chunks = fused_cnt(r.W, k_lo, k_hi, a.quanta_before + a.n_chunks) - fused_cnt(r.W, k_lo, k_hi, a.quanta_before);
-        const uint64_t slot_last = mod_u64(a.quanta_before + last, r.W);
-        const bool mine = slot_last >= k_lo && slot_last < k_hi;
-        bytes = chunks * a.chunk_bytes - (mine ? a.chunk_bytes - len_last : 0);
+        a.hdr->lane_bytes[t] = bytes;
+        a.hdr->lane_chunks[t] = (uint32_t)chunks;
       }
-      a.hdr->lane_bytes[t] = bytes;
-      a.hdr->lane_chunks[t] = (uint32_t)chunks;
-    }
-    if (t == 0) {
-      a.hdr->total_bytes = a.total_bytes;
-      a.hdr->total_tiles = (uint32_t)last * a.tiles_per_chunk + (uint32_t)((len_last + a.tile_bytes - 1) / a.tile_bytes);
-      a.hdr->n_chunks = a.n_chunks;
-      a.hdr->flags = r.zero ? FLH_SCHED_F_NO_CREDIT : 0;
-      a.hdr->uniform_tiles = a.tiles_per_chunk;
+      if (t == 0) {
+        uint32_t tiles = 0, zero = 0;
+        for (uint32_t s = 0; s < a.n_seg; ++s) {
+          const BatchSeg& g = a.seg[s];
+          if (!g.n_chunks) continue;
+          tiles += (g.n_chunks - 1) * a.tiles_per_chunk + (a.chunk_bytes - g.short_by + a.tile_bytes - 1) / a.tile_bytes;
+          zero |= g.zero;
+        }
+        a.hdr->total_bytes = a.total_bytes;
+        a.hdr->total_tiles = tiles;
+        a.hdr->n_chunks = a.n_chunks;
+        a.hdr->flags = zero ? FLH_SCHED_F_NO_CREDIT : 0;
+        a.hdr->uniform_tiles = a.tiles_per_chunk;
+      }
+    } else {
+      FusedRow r;
+      fused_row(a, r);
+      const uint64_t last = a.n_chunks - 1;
+      const uint64_t len_last = a.total_bytes - last * a.chunk_bytes;
+      if (t < FLH_MAX_LANES) {
+        uint64_t chunks = 0, bytes = 0;
+        if (t < a.n_lanes) {
+          uint64_t k_lo = 0, k_hi = 0;  // selected, not indexed: indexing would push the row into scratch memory
+#pragma unroll
+          for (int l = 0; l < FLH_MAX_LANES; ++l) {
+            if ((uint32_t)l == t) { k_hi = r.pfx[l]; k_lo = l ? r.pfx[l > 0 ? l - 1 : 0] : 0; }
+          }
+          chunks = fused_cnt(r.W, k_lo, k_hi, a.quanta_before + a.n_chunks) - fused_cnt(r.W, k_lo, k_hi, a.quanta_before);
+          const uint64_t slot_last = mod_u64(a.quanta_before + last, r.W);
+          const bool mine = slot_last >= k_lo && slot_last < k_hi;
+          bytes = chunks * a.chunk_bytes - (mine ? a.chunk_bytes - len_last : 0);
+        }
+        a.hdr->lane_bytes[t] = bytes;
+        a.hdr->lane_chunks[t] = (uint32_t)chunks;
+      }
+      if (t == 0) {
+        a.hdr->total_bytes = a.total_bytes;
+        a.hdr->total_tiles = (uint32_t)last * a.tiles_per_chunk + (uint32_t)((len_last + a.tile_bytes - 1) / a.tile_bytes);
+        a.hdr->n_chunks = a.n_chunks;
+        a.hdr->flags = r.zero ? FLH_SCHED_F_NO_CREDIT : 0;
+        a.hdr->uniform_tiles = a.tiles_per_chunk;
+      }
     }
   }
 
@@ -446,6 +521,29 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   }
   uint8_t* w = (uint8_t*)a.win.base[lane] + win_off + off;
   if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+}
+
+template <int DIR, int NT, class Args>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
+  warm_kernel_args(a);
+  uint32_t bx = blockIdx.x, by = blockIdx.y;   // tile of the chunk, chunk (in message or destination order)
+  xcd_tile_2d(a.xcd_map, bx, by);
+  fused_tile<DIR, NT>(a, bx, by);
+  // Completion word.  Every workgroup of the grid comes through here, also those without a tile.  The barrier orders
+  // the workgroup's stores before thread 0's increment, which releases them at agent scope; the workgroup that counts
+  // the last one has thereby acquired every other workgroup's stores, and its store of the word releases all of them
+  // at system scope.  A reader that finds done_value with an acquire load may read the destination.
+  if (DIR == 1 && a.done_word) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const uint32_t total = gridDim.x * gridDim.y;
+      const uint32_t prev = __hip_atomic_fetch_add(a.done_count, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      if (prev + 1 == total) {
+        __hip_atomic_store(a.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(a.done_word, a.done_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
+  }
 }
 
 struct PageArgs {
@@ -676,9 +774,10 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
   a.table = dir == 0 ? d_table : nullptr;
   a.hdr = dir == 0 ? d_hdr : nullptr;
   a.status = d_status;
-  a.stamp = nullptr;
-  a.stamp_value = 0;
-  if (dir == 0) fl_take_launch_stamp(&a.stamp, &a.stamp_value);
+  a.done_word = dir == 1 ? u->d_done_word : nullptr;
+  a.done_count = dir == 1 ? u->d_done_count : nullptr;
+  a.done_value = u->done_value;
+  if (a.done_word && !a.done_count) return fl_set_error(FLH_E_ARG, "d_done_word needs d_done_count");
   a.total_bytes = u->total_bytes;
   a.src_base = u->src_base;
   a.quanta_before = u->epoch_bytes / u->chunk_bytes;
@@ -714,11 +813,20 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
 
 extern "C++" {
 template <class Args>
-static int launch_fused_args(int dir, const Args& a, int mode, void* stream) {
+static int launch_fused_args(int dir, const Args& a, int mode, void* stream, void* done_event) {
   const dim3 grid(a.tiles_per_chunk, a.n_chunks);
   hipStream_t s = (hipStream_t)stream;
+  hipEvent_t ev = dir == 1 ? (hipEvent_t)done_event : nullptr;
 #define FL_ARGS_EXTRA , Args
-  FL_LAUNCH_COPY(fl_copy_uniform_fused, FL_ARGS_EXTRA, dir, mode, grid, s, a);
+  if (dir == 0) {
+    if (mode == 0) FL_LAUNCH((fl_copy_uniform_fused<0, 0 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, a);
+    else if (mode == 1) FL_LAUNCH((fl_copy_uniform_fused<0, 1 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, a);
+    else FL_LAUNCH((fl_copy_uniform_fused<0, 3 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, a);
+  } else {
+    if (mode == 0) FL_LAUNCH_EV((fl_copy_uniform_fused<1, 0 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+    else if (mode == 2) FL_LAUNCH_EV((fl_copy_uniform_fused<1, 2 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+    else FL_LAUNCH_EV((fl_copy_uniform_fused<1, 3 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+  }
 #undef FL_ARGS_EXTRA
   FL_HIP(hipGetLastError());
   return FLH_OK;
@@ -733,35 +841,119 @@ static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_wind
   if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
   a.user = (uint8_t*)user;
   a.user_bytes = user_bytes;
-  return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream);
+  return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream, u->done_event);
+}
+
+// What a batch comes to: its segments as the kernel takes them, and where each lane's window ends up.
+struct BatchPlan {
+  uint32_t n_seg;
+  uint32_t n_chunks;
+  uint32_t first[FLH_BATCH_MAX];
+  uint8_t seg_of[FLH_BATCH_MAX];
+  BatchSeg seg[FLH_SEG_MAX];
+  uint64_t seg_base[FLH_SEG_MAX][FLH_MAX_LANES];
+  uint64_t lane_end[FLH_MAX_LANES];
+};
+
+static int plan_batch(const flh_batch_params* b, BatchPlan& pl) {
+  if (!b) return fl_set_error(FLH_E_ARG, "null batch");
+  if (b->n_req == 0 || b->n_req > FLH_BATCH_MAX) return fl_set_error(FLH_E_ARG, "n_req %u not in 1..%d", b->n_req, FLH_BATCH_MAX);
+  if (b->n_seg > FLH_SEG_MAX) return fl_set_error(FLH_E_ARG, "n_seg %u not in 0..%d", b->n_seg, FLH_SEG_MAX);
+  const flh_uniform_params& u = b->u;
+  if (u.n_lanes == 0 || u.n_lanes > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "n_lanes %u not in 1..%d", u.n_lanes, FLH_MAX_LANES);
+  if (u.chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0");
+  memset(&pl, 0, sizeof(pl));
+  pl.n_seg = b->n_seg ? b->n_seg : 1;
+  uint32_t q = 0, chunk_at = 0;
+  uint64_t sum = 0;
+  for (uint32_t k = 0; k < pl.n_seg; ++k) {
+    const uint32_t nq = b->n_seg ? b->seg[k].n_req : b->n_req;
+    const uint32_t* credits = b->n_seg ? b->seg[k].credits : u.credits;
+    const uint64_t epoch_bytes = b->n_seg ? b->seg[k].epoch_bytes : u.epoch_bytes;
+    if (nq == 0 || q + nq > b->n_req) return fl_set_error(FLH_E_ARG, "segment %u holds %u requests, %u are left", k, nq, b->n_req - q);
+    BatchSeg& g = pl.seg[k];
+    uint64_t seg_bytes = 0;
+    for (uint32_t i = 0; i < nq; ++i, ++q) {
+      if (b->bytes[q] == 0) return fl_set_error(FLH_E_ARG, "request %u of the batch has no bytes", q);
+      if (i + 1 < nq && b->bytes[q] % u.chunk_bytes) return fl_set_error(FLH_E_ARG, "request %u of the batch is not a whole number of chunks", q);
+      pl.first[q] = chunk_at + (uint32_t)(seg_bytes / u.chunk_bytes);
+      pl.seg_of[q] = (uint8_t)k;
+      seg_bytes += b->bytes[q];
+    }
+    const uint64_t n = (seg_bytes + u.chunk_bytes - 1) / u.chunk_bytes;
+    FlCreditRow row;
+    fl_row_make(credits, u.n_lanes, row);
+    const uint64_t x0 = epoch_bytes / u.chunk_bytes;
+    if (row.W > 0xffffffffull || x0 + n > 0xffffffffull || chunk_at + n > 65535)
+      return fl_set_error(FLH_E_ARG, "segment %u: a credit row that sums past 2^32 - 1, a credit epoch of 2^32 quanta or more, or more than 65535 chunks in the launch", k);
+    g.magic = row.W >= 2 ? ~0ull / row.W + 1 : 0;
+    g.quanta_before = (uint32_t)x0;
+    g.first_chunk = chunk_at;
+    g.n_chunks = (uint32_t)n;
+    g.short_by = (uint32_t)(n * u.chunk_bytes - seg_bytes);
+    g.zero = row.zero;
+    for (uint32_t l = 0; l <= FLH_MAX_LANES; ++l) g.pfx_ex[l] = (uint32_t)row.K[l];
+    uint64_t lane_bytes[FLH_MAX_LANES];
+    uint32_t lane_chunks[FLH_MAX_LANES];
+    fl_row_lane_totals(row, x0, seg_bytes, u.chunk_bytes, lane_bytes, lane_chunks);
+    for (uint32_t l = 0; l < FLH_MAX_LANES; ++l) {
+      g.cnt0[l] = l < u.n_lanes ? (uint32_t)fl_row_before(row, l, x0) : 0;
+      const uint64_t base = (pl.lane_end[l] + 127) / 128 * 128;   // the alignment of the reference's per-QP pieces (plugin.cc:1467)
+      if (base / 128 > 0xffffffffull) return fl_set_error(FLH_E_ARG, "segment %u starts beyond 512 GiB in a window", k);
+      g.base128[l] = (uint32_t)(base / 128);
+      pl.seg_base[k][l] = base;
+      if (lane_chunks[l]) pl.lane_end[l] = base + lane_bytes[l];
+    }
+    chunk_at += (uint32_t)n;
+    sum += seg_bytes;
+  }
+  if (q != b->n_req) return fl_set_error(FLH_E_ARG, "the segments hold %u requests, the batch %u", q, b->n_req);
+  if (sum != u.total_bytes) return fl_set_error(FLH_E_ARG, "the requests hold %llu bytes, the parameters say %llu", (unsigned long long)sum, (unsigned long long)u.total_bytes);
+  for (uint32_t r = b->n_req; r < FLH_BATCH_MAX; ++r) pl.first[r] = 0xffffffffu;
+  pl.n_chunks = chunk_at;
+  return FLH_OK;
+}
+
+int flh_batch_layout(const flh_batch_params* b, uint64_t* lane_end, uint64_t* seg_base) {
+  BatchPlan pl;
+  const int rc = plan_batch(b, pl);
+  if (rc) return rc;
+  if (lane_end) memcpy(lane_end, pl.lane_end, sizeof(pl.lane_end));
+  if (seg_base) memcpy(seg_base, pl.seg_base, sizeof(pl.seg_base));
+  return FLH_OK;
 }
 
 static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table, flh_sched_hdr* d_hdr,
                         int32_t* d_status, void* stream) {
-  if (!b) return fl_set_error(FLH_E_ARG, "null batch");
-  if (b->n_req == 0 || b->n_req > FLH_BATCH_MAX) return fl_set_error(FLH_E_ARG, "n_req %u not in 1..%d", b->n_req, FLH_BATCH_MAX);
+  BatchPlan pl;
+  int rc = plan_batch(b, pl);
+  if (rc) return rc;
   FusedBatchArgs a;
-  const int rc = fill_fused(a, dir, win, &b->u, d_table, d_hdr, d_status);
+  // fill_fused sees the launch as one message of n_chunks whole chunks (grid, tiles per chunk, checks); the credit row
+  // it prepares goes unused, every segment brings its own
+  flh_uniform_params u = b->u;
+  u.total_bytes = (uint64_t)pl.n_chunks * b->u.chunk_bytes;
+  u.epoch_bytes = 0;
+  rc = fill_fused(a, dir, win, &u, d_table, d_hdr, d_status);
   if (rc) return rc < 0 ? rc : FLH_OK;
+  a.total_bytes = b->u.total_bytes;
   a.dest_order = 0;
   a.src_base = 0;
   a.n_req = b->n_req;
-  uint64_t sum = 0;
+  a.n_seg = pl.n_seg;
   for (uint32_t q = 0; q < FLH_BATCH_MAX; ++q) {
-    a.first[q] = 0;
+    a.first[q] = pl.first[q];
+    a.seg_of[q] = pl.seg_of[q];
     a.req_user[q] = nullptr;
     a.req_bytes[q] = 0;
     if (q >= b->n_req) continue;
     void* p = dir == 0 ? (void*)b->d_src[q] : b->d_dst[q];
-    if (!p || b->bytes[q] == 0) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer or no bytes", q);
-    if (q + 1 < b->n_req && b->bytes[q] % b->u.chunk_bytes) return fl_set_error(FLH_E_ARG, "request %u of the batch is not a whole number of chunks", q);
-    a.first[q] = (uint32_t)(sum / b->u.chunk_bytes);
+    if (!p) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer", q);
     a.req_user[q] = (uint8_t*)p;
     a.req_bytes[q] = b->bytes[q];
-    sum += b->bytes[q];
   }
-  if (sum != b->u.total_bytes) return fl_set_error(FLH_E_ARG, "the requests hold %llu bytes, the parameters say %llu", (unsigned long long)sum, (unsigned long long)b->u.total_bytes);
-  return launch_fused_args(dir, a, fl_stream_mode(dir, sum), stream);
+  for (uint32_t k = 0; k < FLH_SEG_MAX; ++k) a.seg[k] = pl.seg[k];
+  return launch_fused_args(dir, a, fl_stream_mode(dir, b->u.total_bytes), stream, b->u.done_event);
 }
 
 static int launch_fused_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
@@ -781,7 +973,7 @@ static int launch_fused_pages(int dir, void* pool, uint64_t pool_pages, const ui
   a.n_pages = (u->src_base + u->total_bytes + page_bytes - 1) / page_bytes;
   a.page_bytes = page_bytes;
   a.page_shift = (page_bytes & (page_bytes - 1)) == 0 ? __builtin_ctz(page_bytes) : -1;
-  return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream);
+  return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream, u->done_event);
 }
 
 int flh_gather_pages_uniform(const void* d_pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,

@@ -39,35 +39,30 @@ struct ProfState {
   size_t n = 0;
   bool on = false;
   int kid = 0;   // which entry point is launching: 1 schedule, 2 stripe, 3 reassemble, 4 gather, 5 scatter, 6 copy
-  hipEvent_t done_ev = nullptr;   // handed over by fl_completion_event(): the next launch completes it
-  bool done_handed = false;
-  uint32_t* stamp = nullptr;      // handed over by fl_launch_stamp(): the next fused striping launch writes stamp_value there
-  uint32_t stamp_value = 0;
-  bool stamp_handed = false;
 };
-// what fl_launch_stamp() left for the calling thread's next fused striping launch (null if nothing); takes it
-FL_LOCAL void fl_take_launch_stamp(uint32_t** word, uint32_t* value);
 // The calling thread's state.  Reached through a function, not through an `extern thread_local`: code that uses
 // such a variable from another translation unit tests the address of its (absent, weak, hidden) initialiser,
 // which position-independent code computes relative to the load address, never as null, and then calls it.
 FL_LOCAL ProfState& fl_prof();
 
-#define FL_LAUNCH(kernel, grid, block, shmem, stream, ...)                                              \
+// `ev` (may be null) is completed by the kernel itself; inside a profiling region the launch carries that region's
+// events and `ev` is recorded behind it instead.
+#define FL_LAUNCH_EV(kernel, grid, block, shmem, stream, ev, ...)                                       \
   do {                                                                                                  \
     ProfState& ps_ = fl_prof();                                                                         \
+    hipEvent_t ev_ = (ev);                                                                              \
     if (ps_.on && ps_.n < ps_.ring->size()) {                                                           \
       ProfRec& pr_ = (*ps_.ring)[ps_.n++];                                                              \
       pr_.kid = ps_.kid;                                                                                \
       hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, pr_.e0, pr_.e1, 0, __VA_ARGS__);        \
-    } else if (ps_.done_ev) {                                                                           \
-      hipEvent_t ev_ = ps_.done_ev;                                                                     \
-      ps_.done_ev = nullptr;                                                                            \
+      if (ev_) (void)hipEventRecord(ev_, stream);                                                       \
+    } else if (ev_) {                                                                                   \
       hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, nullptr, ev_, 0, __VA_ARGS__);          \
     } else {                                                                                            \
       hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                              \
     }                                                                                                   \
   } while (0)
-
+#define FL_LAUNCH(kernel, grid, block, shmem, stream, ...) FL_LAUNCH_EV(kernel, grid, block, shmem, stream, (hipEvent_t) nullptr, __VA_ARGS__)
 
 #define FL_HIP(call)                                                                         \
   do {                                                                                       \

@@ -16,11 +16,13 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <atomic>
 #include <cerrno>
 #include <chrono>
 #include <ctime>
 #include <cstring>
 #include <mutex>
+#include <shared_mutex>
 
 #include "fl_internal.h"
 #include "fuselink_hip.h"
@@ -44,27 +46,49 @@ static_assert(offsetof(LaneTable, rx_status) == 64 && offsetof(LaneTable, tx_las
               offsetof(LaneTable, rx_last_active) == 256 && offsetof(LaneTable, running) == 384 && sizeof(LaneTable) == 392,
               "layout must match the reference's SharedMemory");
 
-std::mutex g_mu;            // guards the pointers below and, in process-local mode, the table
+// g_mu guards the pointers below against attach / detach (taken exclusively there).  A table access takes it
+// exclusively in process-local mode, where it is the table's lock, and shared in shared-memory mode, where the
+// cross-process semaphore is: a thread that waits for the semaphore then holds up nobody in this process.
+std::shared_mutex g_mu;
 LaneTable g_local = {};
 LaneTable* g_tab = &g_local;
 sem_t* g_sem = SEM_FAILED;  // the cross-process lock when attached
 int g_shm_fd = -1;
 bool g_owner = false;
 char g_shm_name[64] = "", g_sem_name[64] = "";
-bool g_manual_clock = false;
-int64_t g_manual_now = 0;
+std::atomic<bool> g_manual_clock{false};
+std::atomic<int64_t> g_manual_now{0};
+// Set when a wait for the semaphore ran into its bound: a process died holding it.  From then on an access only tries
+// the semaphore (and clears the flag when it gets it) instead of waiting again.
+std::atomic<bool> g_sem_dead{false};
 
 // Every access to the table goes through one of these.  The cross-process semaphore is waited for with a
 // bound: a process that died holding it (the reference's sem_wait would then block for ever, src/monitor.h:195)
 // must not stall a transport thread, so after kSemWaitMs the access goes ahead unlocked -- entries are single
-// words, the worst outcome is one stale status -- and the semaphore is not posted.
+// words, the worst outcome is one stale status -- and the semaphore is not posted.  Only the first such access pays
+// the wait; the later ones try the semaphore without waiting until it is free again.
 constexpr long kSemWaitMs = 200;
 struct TableLock {
-  std::unique_lock<std::mutex> local;
-  sem_t* sem;
+  std::unique_lock<std::shared_mutex> local;
+  std::shared_lock<std::shared_mutex> shared;
+  sem_t* sem = SEM_FAILED;
   bool held = false;
-  TableLock() : local(g_mu), sem(g_sem) {
-    if (sem == SEM_FAILED) return;
+  TableLock() {
+    shared = std::shared_lock<std::shared_mutex>(g_mu);
+    if (g_sem == SEM_FAILED) {          // process-local table: g_mu is its lock
+      shared.unlock();
+      local = std::unique_lock<std::shared_mutex>(g_mu);
+      if (g_sem == SEM_FAILED) return;
+      local.unlock();                   // attached meanwhile
+      shared = std::shared_lock<std::shared_mutex>(g_mu);
+      if (g_sem == SEM_FAILED) return;  // and detached again: one unlocked access to single words
+    }
+    sem = g_sem;
+    if (g_sem_dead.load(std::memory_order_acquire)) {
+      held = sem_trywait(sem) == 0;
+      if (held) g_sem_dead.store(false, std::memory_order_release);
+      return;
+    }
     timespec until;
     clock_gettime(CLOCK_REALTIME, &until);
     until.tv_nsec += kSemWaitMs * 1000000L;
@@ -73,6 +97,7 @@ struct TableLock {
     int rc;
     while ((rc = sem_timedwait(sem, &until)) != 0 && errno == EINTR) {}
     held = rc == 0;
+    if (!held) g_sem_dead.store(true, std::memory_order_release);
   }
   ~TableLock() {
     if (held) sem_post(sem);
@@ -104,7 +129,8 @@ int fl_monitor_attach_shm(const char* shm_name, const char* sem_name, int create
   if (!shm_name) shm_name = "/rdma_monitor_shm";  // SHM_NAME, src/monitor.h:23
   if (!sem_name) sem_name = "/rdma_monitor_sem";  // SEM_NAME, src/monitor.h:24
   if (strlen(shm_name) >= sizeof(g_shm_name) || strlen(sem_name) >= sizeof(g_sem_name)) return fl_set_error(FLH_E_ARG, "name too long");
-  std::lock_guard<std::mutex> g(g_mu);
+  std::unique_lock<std::shared_mutex> g(g_mu);
+  g_sem_dead.store(false, std::memory_order_release);
   detach_locked();
   if (create) {  // the daemon's part (Monitor::setupSharedMemory in src/monitor.cpp)
     shm_unlink(shm_name);
@@ -133,14 +159,14 @@ int fl_monitor_attach_shm(const char* shm_name, const char* sem_name, int create
 }
 
 int fl_monitor_detach(void) {
-  std::lock_guard<std::mutex> g(g_mu);
+  std::unique_lock<std::shared_mutex> g(g_mu);
   if (g_owner && g_tab != &g_local) g_tab->running = 0;
   detach_locked();
   return FLH_OK;
 }
 
 int fl_monitor_is_shared(void) {
-  std::lock_guard<std::mutex> g(g_mu);
+  std::shared_lock<std::shared_mutex> g(g_mu);
   return g_tab != &g_local;
 }
 
@@ -150,18 +176,14 @@ int fl_monitor_daemon_running(void) {
 }
 
 int fl_monitor_set_clock(int manual, int64_t now_us) {
-  std::lock_guard<std::mutex> g(g_mu);
-  g_manual_clock = manual != 0;
-  g_manual_now = now_us;
+  g_manual_now.store(now_us, std::memory_order_relaxed);
+  g_manual_clock.store(manual != 0, std::memory_order_release);
   return FLH_OK;
 }
 
 // get_timestamp() of src/monitor.h:29-33 unless a test has frozen the clock
 int64_t fl_monitor_now(void) {
-  {
-    std::lock_guard<std::mutex> g(g_mu);
-    if (g_manual_clock) return g_manual_now;
-  }
+  if (g_manual_clock.load(std::memory_order_acquire)) return g_manual_now.load(std::memory_order_relaxed);   // no lock on the request path
   return std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
 

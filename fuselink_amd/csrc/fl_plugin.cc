@@ -12,14 +12,16 @@
 //          striping kernel (chunk -> lane scheduling folded in; user buffer -> lane staging windows)
 //          -> reassembly kernel (windows -> the posted receive buffer).  The reassembly launch plays the part of the
 //          RDMA write landing at the receiver; its completion event is the receive completion.
-//          The launches are not made inside isend: matched sends wait on the connection until the first
-//          test of one of them (or until NCCL_FUSELINK_BATCH of them wait), and go out together -- requests
-//          that share a credit row as ONE message in one launch pair, which is what keeps the cost of a
-//          launch from bounding the request rate at NCCL's 512 KiB steps.
-//   test   launches whatever waits on the connection, polls the request's event (the completion queue of
-//          plugin.cc:1801-1955) and, unlike the reference, reports the byte count of a receive.
-// Staging windows are HIP-VMM mappings from the unit pool, one per lane per connection, bound when
-// device memory is first registered on the send side and reused wave after wave.
+//          The launches are not made inside isend: matched sends of ALL connections that stage on one GPU wait
+//          in one queue (as the reference's channels share one set of per-NIC lane comms, fuselink.h:271-272,
+//          plugin.cc:727-753) until a test finds the GPU's queue short of work (or until NCCL_FUSELINK_BATCH of
+//          them wait), and go out together: up to 32 requests in one launch pair, the requests of a connection
+//          between two refreshes as one message under that connection's credit row, which is what keeps the
+//          cost of a launch from bounding the request rate at NCCL's 512 KiB steps.
+//   test   launches what waits, reads the completion word that the reassembly kernel's last workgroup stores
+//          (the completion queue of plugin.cc:1801-1955) and, unlike the reference, reports the byte count of a receive.
+// Staging windows are HIP-VMM mappings from the unit pool, one per lane per GPU, shared by every connection
+// that stages there, bound when device memory is first registered on a send side and reused launch after launch.
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -33,6 +35,7 @@
 #include <new>
 #include <vector>
 
+#include "fl_closed_form.h"
 #include "fl_internal.h"
 #include "fuselink_hip.h"
 #include "fuselink_net.h"
@@ -61,11 +64,12 @@ struct Params {
   int max_wave_chunks = 4096;
   int batch = FLH_BATCH_MAX;     // matched sends that may wait for one launch (1 = launch inside isend)
   // How a launch's completion reaches `test`: 0 = an event recorded behind every launch (a barrier packet of its
-  // own, some 4.5 us in which the connection's next kernel does not start), 1 = the event rides on the launch's
-  // last kernel, 2 = no event at all while launches follow each other: every striping kernel, as it starts, stores
-  // the number of the launch before it to a pinned word (a kernel starts once its stream's earlier work is done),
-  // and only a launch that nothing follows gets an event, recorded when it is first polled.
+  // own, some 4.5 us in which the stream's next kernel does not start), 1 = the event rides on the launch's last
+  // kernel, 2 = no event and no call into the runtime: the last workgroup of the reassembly kernel to finish stores
+  // the launch's number to a pinned word, after every workgroup's stores have been released (flh_uniform_params).
   int completion = 2;
+  int small_tile = 0;            // copy tile of a launch under 32 MiB (0 = the library's default tile)
+  int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
 Params g_par;
 std::mutex g_init_mu;            // ncclIbLock, plugin.cc:84
@@ -151,12 +155,62 @@ struct FifoSlot {
 
 // a matched send whose GPU work has not been queued yet
 struct Pending {
+  Link* lk;
   const uint8_t* src;
   uint8_t* dst;
   int size;
   bool src_dev, dst_dev;
   FifoWire w;
   Request *sreq, *rreq;
+};
+
+// What one launch pair carried, for inspection (fl_net_last_launch).
+struct LaunchSeg {
+  int channelId;
+  uint32_t first_row, n_rows, n_req;
+  uint64_t epoch_bytes;
+  uint64_t lane_base[FL_NET_MAX_LANES];
+};
+struct LaunchInfo {
+  uint64_t seq = 0;
+  uint32_t n_seg = 0, n_rows = 0;
+  LaunchSeg seg[FLH_SEG_MAX] = {};
+};
+
+constexpr size_t kEventRing = 1024;
+
+// The staging side of one GPU, shared by every connection that stages there, as the reference's per-NIC lane comms
+// are shared by all channels (fuselink.h:271-272; opened once, on the first connect, plugin.cc:727-753): one stream,
+// one staging window per lane, one queue of matched sends, one sequence of launch numbers.
+struct Peer {
+  int hip_device = 0;
+  int links = 0;                    // connections attached (g_peer_mu)
+  bool ready = false;
+  hipStream_t stream = nullptr;
+  flh_window* win[FL_NET_MAX_LANES] = {};
+  flh_windows wins = {};
+  flh_chunk_desc* d_table = nullptr;
+  flh_sched_hdr* d_hdr = nullptr;
+  uint32_t* d_count = nullptr;      // device word in which a reassembly launch counts its finished workgroups
+  int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
+  int32_t* d_status = nullptr;
+  uint32_t* h_done = nullptr;       // pinned, device-visible: number of the last launch whose reassembly has finished (completion mode 2)
+  uint32_t* d_done = nullptr;
+  // matched sends that wait for a launch, in arrival order
+  std::mutex queue_mu;
+  std::vector<Pending> pending;
+  std::atomic<uint32_t> waiting_reqs{0};
+  std::atomic<uint64_t> waiting_bytes{0};
+  // Guards every launch on `stream`, the event ring, the launch numbers, the connections' scheduling state
+  // (epoch_bytes, launch counters, last table) and `last`.  Taken before queue_mu, never the other way round.
+  std::mutex launch_mu;
+  std::vector<Pending> work;        // the waiting sends a flush took over (launch_mu)
+  hipEvent_t evring[kEventRing] = {};              // launch n may own slot (n - 1) % kEventRing
+  std::atomic<uint64_t> ev_seq[kEventRing] = {};   // the launch whose completion the slot's event stands for (0: none)
+  std::atomic<uint64_t> done_seq{0};               // highest launch number known complete; launches run in order on one stream
+  std::atomic<uint64_t> launch_seq{0};             // highest launch number handed out
+  std::atomic<uint64_t> last_event_seq{0};         // highest launch whose completion comes from an event, not from the word
+  LaunchInfo last;
 };
 
 struct Link {
@@ -177,34 +231,13 @@ struct Link {
   int fuselink_offset = -1;
   uint8_t credits[FL_NET_MAX_LANES] = {};
   bool have_decision = false;
-  // GPU side of the connection (created on first use with device memory)
-  bool gpu_ready = false;
-  int hip_device = 0;
-  hipStream_t stream = nullptr;
-  flh_window* win[FL_NET_MAX_LANES] = {};
-  flh_windows wins = {};
-  flh_chunk_desc* d_table = nullptr;
-  flh_sched_hdr* d_hdr = nullptr;
+  // staging side: the GPU's shared one, attached on first use with device memory (set once, under mu)
+  std::atomic<Peer*> peer{nullptr};
+  // scheduling state of the connection (the peer's launch_mu)
   uint64_t epoch_bytes = 0;         // bytes scheduled since the last lane-decision refresh (the scheduler's carried prefix)
-  int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
-  int32_t* d_status = nullptr;
-  uint32_t* h_stamp = nullptr;      // pinned, device-visible: number of the last launch known complete (completion mode 2)
-  uint32_t* d_stamp = nullptr;
-  std::atomic<uint32_t> last_wave_rows{0};
-  // Guards the waiting sends, the event ring and every launch on `stream` (either side's thread may be the
-  // one that launches).  Never taken while `mu` is held by the same thread for long: isend drops `mu` first.
-  std::mutex launch_mu;
-  std::vector<Pending> pending;
-  std::atomic<uint64_t> waiting_bytes{0};   // bytes of the waiting sends, readable without launch_mu
-  hipEvent_t evring[FL_NET_MAX_REQUESTS] = {};   // launch n owns slot (n - 1) % size: at most that many requests, hence launches, are in flight
-  std::atomic<uint8_t> ev_set[FL_NET_MAX_REQUESTS] = {};    // the slot's event has been recorded (or rides on a kernel) for its launch
-  std::atomic<uint8_t> stamps[FL_NET_MAX_REQUESTS] = {};    // the slot's launch starts with a kernel that stamps the launch before it
-  // Highest launch number seen complete.  The connection's launches run in order on one stream, so a request of an
-  // earlier launch is complete too and its test needs no event query (requests that shared a launch, and the
-  // receive side of a send that was already tested, cost no call into the runtime).
-  std::atomic<uint64_t> done_seq{0};
-  std::atomic<uint64_t> launch_seq{0};   // written under launch_mu
-  int64_t launches = 0, batched_requests = 0;    // launch pairs made, requests that shared one
+  uint64_t last_seq = 0;            // launch that carried the connection's latest segment, and that segment's rows in its table
+  uint32_t last_first_row = 0, last_rows = 0;
+  int64_t launches = 0, batched_requests = 0;    // launch pairs that carried its requests, requests that shared a pair with others
 };
 
 struct Comm {
@@ -255,6 +288,26 @@ ncclResult_t hip_fail(const char* what, hipError_t e) {
 #define FL_FLHCHECK(call) do { int rc_ = (call); if (rc_ < 0) { FL_WARN("NET/FuseLink : %s: %s", #call, flh_last_error()); \
   return rc_ == FLH_E_NOMEM || rc_ == FLH_E_ARG ? ncclInternalError : ncclUnhandledCudaError; } } while (0)
 
+std::mutex g_peer_mu;                // the peers, their attachment counts
+std::map<int, Peer*> g_peers;        // one per HIP device that stages
+
+void flush_pending(Peer* pr);
+
+void peer_destroy(Peer* pr) {        // no longer reachable through g_peers
+  DeviceScope keep;
+  (void)hipSetDevice(pr->hip_device);
+  if (pr->stream) (void)hipStreamSynchronize(pr->stream);
+  for (int l = 0; l < FL_NET_MAX_LANES; ++l)
+    if (pr->win[l]) (void)flh_window_destroy(pr->win[l]);
+  if (pr->d_table) (void)hipFree(pr->d_table);
+  if (pr->d_hdr) (void)hipFree(pr->d_hdr);
+  if (pr->d_count) (void)hipFree(pr->d_count);
+  if (pr->h_status) (void)hipHostFree(pr->h_status);
+  for (auto& e : pr->evring) if (e) (void)hipEventDestroy(e);
+  if (pr->stream) (void)hipStreamDestroy(pr->stream);
+  delete pr;
+}
+
 void link_unref(Link* lk) {
   bool last;
   {
@@ -262,17 +315,18 @@ void link_unref(Link* lk) {
     last = --lk->refs == 0;
   }
   if (!last) return;
-  if (lk->stream) {   // the staging side was set up, wholly or in part
-    DeviceScope keep;
-    (void)hipSetDevice(lk->hip_device);
-    (void)hipStreamSynchronize(lk->stream);
-    for (int l = 0; l < FL_NET_MAX_LANES; ++l)
-      if (lk->win[l]) (void)flh_window_destroy(lk->win[l]);
-    if (lk->d_table) (void)hipFree(lk->d_table);
-    if (lk->d_hdr) (void)hipFree(lk->d_hdr);
-    if (lk->h_status) (void)hipHostFree(lk->h_status);
-    for (auto& e : lk->evring) if (e) (void)hipEventDestroy(e);
-    (void)hipStreamDestroy(lk->stream);
+  if (Peer* pr = lk->peer.load(std::memory_order_acquire)) {
+    {   // nothing of this connection may still wait for a launch when it goes away
+      std::lock_guard<std::mutex> g(pr->launch_mu);
+      flush_pending(pr);
+    }
+    bool gone;
+    {
+      std::lock_guard<std::mutex> g(g_peer_mu);
+      gone = --pr->links == 0;
+      if (gone) g_peers.erase(pr->hip_device);
+    }
+    if (gone) peer_destroy(pr);   // the last connection that staged on this GPU: windows and stream go back
   }
   delete lk;
   g_live_links.fetch_sub(1);
@@ -310,37 +364,54 @@ ncclResult_t ensure_pool(int device, flh_pool** out) {
   return ncclSuccess;
 }
 
-// Staging side of a connection: stream, one bound window per lane, table / header / state buffers.
-// `device` owns the buffer that is being registered or sent; the connection stages on it from then on.
-ncclResult_t ensure_link_gpu(Link* lk, int device) {
-  if (lk->gpu_ready) return ncclSuccess;
-  if (lk->stream) { FL_WARN("NET/FuseLink : channel %d: the staging side failed to set up earlier", lk->channelId); return ncclInternalError; }
-  if (device < 0) { FL_WARN("NET/FuseLink : no HIP device to stage on"); return ncclInternalError; }
-  DeviceScope keep;
+// Stream, one bound window per lane, table / header buffers, status and completion words of a new peer.
+ncclResult_t peer_setup(Peer* pr, int device) {
   flh_pool* pool = nullptr;
   ncclResult_t rc = ensure_pool(device, &pool);
   if (rc != ncclSuccess) return rc;
-  lk->hip_device = device;
-  FL_HIPCHECK(hipSetDevice(lk->hip_device));
-  FL_HIPCHECK(hipStreamCreateWithFlags(&lk->stream, hipStreamNonBlocking));
+  pr->hip_device = device;
+  FL_HIPCHECK(hipSetDevice(device));
+  FL_HIPCHECK(hipStreamCreateWithFlags(&pr->stream, hipStreamNonBlocking));
   const uint64_t cap = (uint64_t)g_par.window_units * FLH_UNIT_BYTES;
-  memset(&lk->wins, 0, sizeof(lk->wins));
-  lk->wins.n_lanes = (uint32_t)g_par.lanes;
+  memset(&pr->wins, 0, sizeof(pr->wins));
+  pr->wins.n_lanes = (uint32_t)g_par.lanes;
   for (int l = 0; l < g_par.lanes; ++l) {
-    FL_FLHCHECK(flh_window_create(pool, cap, &lk->win[l]));
-    FL_FLHCHECK(flh_window_bind(lk->win[l], cap));
-    lk->wins.base[l] = flh_window_base(lk->win[l]);
-    lk->wins.cap[l] = flh_window_bound_bytes(lk->win[l]);
+    FL_FLHCHECK(flh_window_create(pool, cap, &pr->win[l]));
+    FL_FLHCHECK(flh_window_bind(pr->win[l], cap));
+    pr->wins.base[l] = flh_window_base(pr->win[l]);
+    pr->wins.cap[l] = flh_window_bound_bytes(pr->win[l]);
   }
-  FL_HIPCHECK(hipMalloc((void**)&lk->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
-  FL_HIPCHECK(hipMalloc((void**)&lk->d_hdr, sizeof(flh_sched_hdr)));
-  FL_HIPCHECK(hipHostMalloc((void**)&lk->h_status, 128, hipHostMallocMapped));   // status word and launch stamp, a cache line apart
-  memset(lk->h_status, 0, 128);
-  FL_HIPCHECK(hipHostGetDevicePointer((void**)&lk->d_status, lk->h_status, 0));
-  lk->h_stamp = (uint32_t*)((char*)lk->h_status + 64);
-  lk->d_stamp = (uint32_t*)((char*)lk->d_status + 64);
-  lk->gpu_ready = true;
-  FL_INFO(NCCL_NET, "NET/FuseLink : channel %d staging ready: %d lanes x %llu bytes", lk->channelId, g_par.lanes, (unsigned long long)cap);
+  FL_HIPCHECK(hipMalloc((void**)&pr->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
+  FL_HIPCHECK(hipMalloc((void**)&pr->d_hdr, sizeof(flh_sched_hdr)));
+  FL_HIPCHECK(hipMalloc((void**)&pr->d_count, 256));
+  FL_HIPCHECK(hipMemset(pr->d_count, 0, 256));
+  FL_HIPCHECK(hipHostMalloc((void**)&pr->h_status, 128, hipHostMallocMapped));   // status word and completion word, a cache line apart
+  memset(pr->h_status, 0, 128);
+  FL_HIPCHECK(hipHostGetDevicePointer((void**)&pr->d_status, pr->h_status, 0));
+  pr->h_done = (uint32_t*)((char*)pr->h_status + 64);
+  pr->d_done = (uint32_t*)((char*)pr->d_status + 64);
+  pr->ready = true;
+  FL_INFO(NCCL_NET, "NET/FuseLink : device %d staging ready: %d lanes x %llu bytes, shared by its connections", device, g_par.lanes, (unsigned long long)cap);
+  return ncclSuccess;
+}
+
+// Attach the connection to the staging side of `device`, which owns the buffer that is being registered or sent
+// (lk->mu held).  The connection stages there from then on.
+ncclResult_t attach_peer(Link* lk, int device) {
+  if (lk->peer.load(std::memory_order_acquire)) return ncclSuccess;
+  if (device < 0) { FL_WARN("NET/FuseLink : no HIP device to stage on"); return ncclInternalError; }
+  DeviceScope keep;
+  std::lock_guard<std::mutex> g(g_peer_mu);
+  auto it = g_peers.find(device);
+  if (it == g_peers.end()) {
+    Peer* pr = new (std::nothrow) Peer();
+    if (!pr) return ncclSystemError;
+    ncclResult_t rc = peer_setup(pr, device);
+    if (rc != ncclSuccess) { peer_destroy(pr); return rc; }
+    it = g_peers.emplace(device, pr).first;
+  }
+  it->second->links++;
+  lk->peer.store(it->second, std::memory_order_release);
   return ncclSuccess;
 }
 
@@ -414,6 +485,9 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.max_wave_chunks = (int)fl_param("FUSELINK_MAX_WAVE_CHUNKS", g_par.max_wave_chunks);
   g_par.batch = (int)fl_param("FUSELINK_BATCH", g_par.batch);
   g_par.completion = (int)fl_param("FUSELINK_COMPLETION", g_par.completion);
+  g_par.small_tile = (int)fl_param("FUSELINK_SMALL_TILE", g_par.small_tile);
+  if (g_par.small_tile < 0 || g_par.small_tile % 128) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_SMALL_TILE must be a multiple of 128"); return ncclInvalidArgument; }
+  g_par.trace = (int)fl_param("FUSELINK_TRACE", g_par.trace);
   if (g_par.completion < 0 || g_par.completion > 2) g_par.completion = 2;
   if (g_par.max_wave_chunks > 65535) g_par.max_wave_chunks = 65535;   // what one fused launch can name
   if (g_par.batch < 1) g_par.batch = 1;
@@ -584,7 +658,7 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
     mh->size = bsz;
     if (c->is_send) {  // staging is bound at registration time, not on the request path
       std::lock_guard<std::mutex> g(c->link->mu);
-      rc = ensure_link_gpu(c->link, mh->device);
+      rc = attach_peer(c->link, mh->device);
       if (rc != ncclSuccess) { (void)flh_region_release(mh->region); delete mh; return rc; }
     }
   } else if (type == NCCL_PTR_HOST) {
@@ -637,175 +711,320 @@ void wire_credits(const Link* lk, const FifoWire& w, uint32_t* credits) {
   }
 }
 
-void fill_uniform(flh_uniform_params& u, const Link* lk, const uint32_t* credits, uint64_t bytes, uint64_t src_base) {
+void fill_uniform(flh_uniform_params& u, const uint32_t* credits, uint64_t bytes, uint64_t src_base, uint64_t epoch_bytes, uint32_t tile) {
   memset(&u, 0, sizeof(u));
   u.total_bytes = bytes;
   u.src_base = src_base;
-  u.epoch_bytes = lk->epoch_bytes;
+  u.epoch_bytes = epoch_bytes;
   u.chunk_bytes = (uint32_t)g_par.chunk;
   u.n_lanes = (uint32_t)g_par.lanes;
-  u.tile_bytes = FLH_TILE_BYTES;
+  u.tile_bytes = tile;
   for (int l = 0; l < g_par.lanes; ++l) u.credits[l] = credits[l];
 }
 
-// Queue the GPU work of one matched send on the connection's stream (launch_mu held); the last launch completes `ev`
-// (if one is given).
-ncclResult_t launch_transfer(Link* lk, const Pending& p, hipEvent_t ev) {
+// copy tile of a launch pair that moves `bytes`: small launches may take a smaller tile, which spreads them over more
+// workgroups than there are compute units
+uint32_t launch_tile(uint64_t bytes) {
+  return g_par.small_tile && bytes < (32ull << 20) ? (uint32_t)g_par.small_tile : FLH_TILE_BYTES;
+}
+
+// How the completion of launch `seq` will reach test(): through the completion word (mode 2), through an event that
+// the reassembly kernel completes (mode 1), or through an event recorded behind the launch (mode 0, and whatever is
+// not a kernel).  Fills the launch's parameters for the first two.
+struct Completion {
+  hipEvent_t ev = nullptr;   // event to record behind the launch (null: not needed)
+  bool rides = false;        // the event was handed to the kernel
+};
+ncclResult_t launch_event(Peer* pr, uint64_t seq, hipEvent_t* out) {
+  const size_t slot = (size_t)((seq - 1) % kEventRing);
+  const uint64_t old = pr->ev_seq[slot].load(std::memory_order_acquire);
+  if (old && old > pr->done_seq.load(std::memory_order_acquire)) {
+    // the ring came round to a launch that nobody has seen complete: wait for it (it is kEventRing launches old)
+    FL_HIPCHECK(hipEventSynchronize(pr->evring[slot]));
+    uint64_t seen = pr->done_seq.load(std::memory_order_relaxed);
+    while (seen < old && !pr->done_seq.compare_exchange_weak(seen, old, std::memory_order_release, std::memory_order_relaxed)) {}
+  }
+  pr->ev_seq[slot].store(0, std::memory_order_release);
+  if (!pr->evring[slot]) FL_HIPCHECK(hipEventCreateWithFlags(&pr->evring[slot], hipEventDisableTiming));
+  *out = pr->evring[slot];
+  return ncclSuccess;
+}
+ncclResult_t prepare_completion(Peer* pr, uint64_t seq, flh_uniform_params& last_u, Completion& c) {
+  if (g_par.completion == 2) {
+    last_u.d_done_word = pr->d_done;
+    last_u.d_done_count = pr->d_count;
+    last_u.done_value = (uint32_t)seq;
+    return ncclSuccess;
+  }
+  ncclResult_t rc = launch_event(pr, seq, &c.ev);
+  if (rc != ncclSuccess) return rc;
+  if (g_par.completion == 1) { last_u.done_event = c.ev; c.rides = true; }
+  return ncclSuccess;
+}
+ncclResult_t finish_completion(Peer* pr, uint64_t seq, const Completion& c) {
+  if (!c.ev) return ncclSuccess;
+  if (!c.rides) FL_HIPCHECK(hipEventRecord(c.ev, pr->stream));
+  pr->ev_seq[(size_t)((seq - 1) % kEventRing)].store(seq, std::memory_order_release);
+  pr->last_event_seq.store(seq, std::memory_order_release);
+  return ncclSuccess;
+}
+
+void note_segment(Peer* pr, uint32_t k, Link* lk, uint32_t first_row, uint32_t n_rows, uint32_t n_req, uint64_t epoch_bytes, const uint64_t* lane_base) {
+  LaunchSeg& sg = pr->last.seg[k];
+  sg.channelId = lk->channelId;
+  sg.first_row = first_row;
+  sg.n_rows = n_rows;
+  sg.n_req = n_req;
+  sg.epoch_bytes = epoch_bytes;
+  for (int l = 0; l < FL_NET_MAX_LANES; ++l) sg.lane_base[l] = lane_base ? lane_base[l] : 0;
+}
+
+// One matched send on its own (launch_mu held): request -> QP pieces (plugin.cc:1467-1495), each piece -> waves of
+// chunks that fit the staging windows, each wave one launch pair.  The last reassembly launch carries the completion.
+ncclResult_t launch_transfer(Peer* pr, const Pending& p, uint64_t seq) {
+  Link* lk = p.lk;
   uint32_t credits[FLH_MAX_LANES];
   wire_credits(lk, p.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
-  if (lk->wins.cap[0] < chunk) { FL_WARN("NET/FuseLink : staging window smaller than a chunk"); return ncclInternalError; }
-  // request -> QP pieces (plugin.cc:1467-1495), each piece -> waves of chunks
+  if (pr->wins.cap[0] < chunk) { FL_WARN("NET/FuseLink : staging window smaller than a chunk"); return ncclInternalError; }
   const int nqps = g_par.split_on_qps ? g_par.qps : 1;
   std::vector<int> qoff(nqps), qlen(nqps);
   if (flh_qp_split(p.size, nqps, qoff.data(), qlen.data()) < 0) return ncclInternalError;
   if (p.w.flags & 1u) lk->epoch_bytes = 0;   // the receiver refreshed its lane decision: new credit epoch
   int last_q = -1;
   for (int q = 0; q < nqps; ++q) if (qlen[q] > 0) last_q = q;
+  Completion comp;
   for (int q = 0; q < nqps; ++q) {
     uint64_t done = 0;
     const uint64_t piece = (uint64_t)qlen[q];
     while (done < piece) {
-      uint64_t wave = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0], lk->epoch_bytes / chunk) * chunk;
+      uint64_t wave = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, pr->wins.cap[0], lk->epoch_bytes / chunk) * chunk;
       if (wave > piece - done) wave = piece - done;
       // One credit row, quantum-sized chunks, windows reused from offset 0: the striping launch works out
       // every chunk's lane and window offset itself (and writes the table), the reassembly launch likewise.
       flh_uniform_params u;
-      fill_uniform(u, lk, credits, wave, (uint64_t)qoff[q] + done);
-      FL_FLHCHECK(flh_stripe_uniform(p.src, (uint64_t)p.size, &lk->wins, &u, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
-      if (ev && q == last_q && done + wave == piece) fl_completion_event(ev);
-      FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &lk->wins, &u, lk->d_status, lk->stream));
+      fill_uniform(u, credits, wave, (uint64_t)qoff[q] + done, lk->epoch_bytes, launch_tile(wave));
+      FL_FLHCHECK(flh_stripe_uniform(p.src, (uint64_t)p.size, &pr->wins, &u, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+      if (q == last_q && done + wave == piece) {
+        ncclResult_t rc = prepare_completion(pr, seq, u, comp);
+        if (rc != ncclSuccess) return rc;
+      }
+      FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &pr->wins, &u, pr->d_status, pr->stream));
+      const uint32_t rows = (uint32_t)((wave + chunk - 1) / chunk);
+      pr->last.seq = seq;
+      pr->last.n_seg = 1;
+      pr->last.n_rows = rows;
+      note_segment(pr, 0, lk, 0, rows, 1, lk->epoch_bytes, nullptr);
+      lk->last_seq = seq;
+      lk->last_first_row = 0;
+      lk->last_rows = rows;
       lk->epoch_bytes += wave;
-      lk->last_wave_rows = (uint32_t)((wave + chunk - 1) / chunk);
       lk->launches++;
       done += wave;
     }
   }
-  return ncclSuccess;
+  return finish_completion(pr, seq, comp);
 }
 
-// Requests [i, j) of the waiting list as one message in one launch pair (launch_mu held).
-ncclResult_t launch_batch(Link* lk, size_t i, size_t j, hipEvent_t ev) {
-  const Pending& p0 = lk->pending[i];
+// Does the send have to travel on its own, wave by wave?  Yes if it is split over QPs or if the staging windows
+// cannot hold it in one wave from where its connection stands in its credit epoch.
+bool needs_waves(const Peer* pr, const Pending& p, uint64_t epoch_bytes) {
+  if ((g_par.split_on_qps ? g_par.qps : 1) != 1) return true;
   uint32_t credits[FLH_MAX_LANES];
-  wire_credits(lk, p0.w, credits);
-  if (p0.w.flags & 1u) lk->epoch_bytes = 0;
-  flh_batch_params b;
-  memset(&b, 0, sizeof(b));
-  uint64_t sum = 0;
-  for (size_t k = i; k < j; ++k) {
-    const Pending& p = lk->pending[k];
-    b.d_src[k - i] = p.src;
-    b.d_dst[k - i] = p.dst;
-    b.bytes[k - i] = (uint64_t)p.size;
-    sum += (uint64_t)p.size;
-  }
-  b.n_req = (uint32_t)(j - i);
-  fill_uniform(b.u, lk, credits, sum, 0);
-  FL_FLHCHECK(flh_stripe_batch(&b, &lk->wins, lk->d_table, lk->d_hdr, lk->d_status, lk->stream));
-  if (ev) fl_completion_event(ev);
-  FL_FLHCHECK(flh_reassemble_batch(&b, &lk->wins, lk->d_status, lk->stream));
-  lk->epoch_bytes += sum;
-  lk->last_wave_rows = (uint32_t)((sum + (uint64_t)g_par.chunk - 1) / (uint64_t)g_par.chunk);
-  lk->launches++;
-  lk->batched_requests += (int64_t)(j - i);
-  return ncclSuccess;
-}
-
-// How many of the waiting sends from i on can travel as one message: device memory on both sides, the same
-// credit row, no credit refresh after the first, whole chunks in all but the last, one QP piece each, and
-// all of it inside one wave of the staging windows.
-size_t batch_span(const Link* lk, size_t i) {
-  const Pending& p0 = lk->pending[i];
-  if (!(p0.src_dev && p0.dst_dev) || g_par.batch < 2) return 1;
-  if ((g_par.split_on_qps ? g_par.qps : 1) != 1) return 1;
-  uint32_t credits[FLH_MAX_LANES];
-  wire_credits(lk, p0.w, credits);
+  wire_credits(p.lk, p.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
-  const uint64_t quanta_before = (p0.w.flags & 1u) ? 0 : lk->epoch_bytes / chunk;   // a refreshed decision starts a new epoch
-  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, lk->wins.cap[0], quanta_before) * chunk;
-  uint64_t sum = 0;
-  size_t j = i;
-  while (j < lk->pending.size() && j - i < (size_t)FLH_BATCH_MAX) {
-    const Pending& p = lk->pending[j];
-    if (!(p.src_dev && p.dst_dev)) break;
-    if (j > i && ((p.w.flags & 1u) || p.w.fuselink_offset != p0.w.fuselink_offset || memcmp(p.w.credits, p0.w.credits, sizeof(p.w.credits)))) break;
-    if (sum + (uint64_t)p.size > room) break;
-    sum += (uint64_t)p.size;
-    ++j;
-    if ((uint64_t)p.size % chunk) break;   // a request that ends inside a chunk closes the message
-  }
-  return j > i ? j - i : 1;
+  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, pr->wins.cap[0], epoch_bytes / chunk) * chunk;
+  return (uint64_t)p.size > room;
 }
 
-// From this many bytes on a launch is bound by the GPU and not by the host's calls around it.
-constexpr uint64_t kEarlyLaunchBytes = 8ull << 20;
+// The waiting sends work[i ..) that go out as one launch pair (launch_mu held): up to FLH_BATCH_MAX requests in up
+// to FLH_SEG_MAX segments.  A segment is a run of requests of one connection under one credit row with no refresh
+// inside, every request but its last a whole number of chunks; the segments follow each other in the shared
+// windows, and the batch ends where the next request would outgrow a window.  Returns the number of requests taken
+// (at least 1: the caller has checked that work[i] alone fits) and fills the batch.
+struct BatchBuild {
+  flh_batch_params b;
+  Link* seg_link[FLH_SEG_MAX];
+  uint64_t link_epoch_after[FLH_SEG_MAX];   // the segment's connection's epoch bytes once the segment is scheduled
+};
+size_t build_batch(Peer* pr, size_t i, BatchBuild& bb) {
+  const std::vector<Pending>& work = pr->work;
+  flh_batch_params& b = bb.b;
+  memset(&b, 0, sizeof(b));
+  const uint64_t chunk = (uint64_t)g_par.chunk;
+  b.u.chunk_bytes = (uint32_t)chunk;
+  b.u.n_lanes = (uint32_t)g_par.lanes;
+  uint64_t closed_end[FLH_MAX_LANES] = {};   // where the closed segments leave every window
+  uint64_t seg_bytes = 0;                    // of the open (last) segment
+  FlCreditRow row;                           // its credit row
+  uint32_t chunks_closed = 0;
+  size_t j = i;
+  while (j < work.size() && b.n_req < (uint32_t)g_par.batch) {
+    const Pending& p = work[j];
+    if (!(p.src_dev && p.dst_dev)) break;
+    // where the request's connection stands in its epoch: behind its earlier segments of this batch, if any
+    uint64_t epoch = p.lk->epoch_bytes;
+    for (uint32_t k = 0; k < b.n_seg; ++k) if (bb.seg_link[k] == p.lk) epoch = bb.link_epoch_after[k];
+    if (p.w.flags & 1u) epoch = 0;
+    uint32_t credits[FLH_MAX_LANES];
+    wire_credits(p.lk, p.w, credits);
+    bool extend = false;
+    if (b.n_seg) {
+      const uint32_t k = b.n_seg - 1;
+      extend = bb.seg_link[k] == p.lk && !(p.w.flags & 1u) && (uint64_t)work[j - 1].size % chunk == 0 &&
+               memcmp(b.seg[k].credits, credits, sizeof(credits)) == 0;
+    }
+    if (!extend && (b.n_seg == FLH_SEG_MAX || needs_waves(pr, p, epoch))) break;
+    // Where would the windows end up?  The open segment grows by the request, or is closed and a new one opens
+    // behind it, on every lane at the next multiple of 128 bytes (flh_batch_layout's rule).
+    uint64_t base_end[FLH_MAX_LANES], lane_bytes[FLH_MAX_LANES];
+    uint32_t lane_chunks[FLH_MAX_LANES];
+    FlCreditRow try_row = row;
+    uint64_t try_bytes, try_epoch;
+    uint32_t chunks_before = chunks_closed;
+    if (extend) {
+      for (int l = 0; l < FLH_MAX_LANES; ++l) base_end[l] = closed_end[l];
+      try_bytes = seg_bytes + (uint64_t)p.size;
+      try_epoch = b.seg[b.n_seg - 1].epoch_bytes;
+    } else {
+      for (int l = 0; l < FLH_MAX_LANES; ++l) base_end[l] = closed_end[l];
+      if (b.n_seg) {   // close the open segment
+        fl_row_lane_totals(row, b.seg[b.n_seg - 1].epoch_bytes / chunk, seg_bytes, chunk, lane_bytes, lane_chunks);
+        for (int l = 0; l < FLH_MAX_LANES; ++l) if (lane_chunks[l]) base_end[l] = (closed_end[l] + 127) / 128 * 128 + lane_bytes[l];
+        chunks_before += (uint32_t)((seg_bytes + chunk - 1) / chunk);
+      }
+      fl_row_make(credits, (uint32_t)g_par.lanes, try_row);
+      try_bytes = (uint64_t)p.size;
+      try_epoch = epoch;
+    }
+    fl_row_lane_totals(try_row, try_epoch / chunk, try_bytes, chunk, lane_bytes, lane_chunks);
+    bool fits = chunks_before + (try_bytes + chunk - 1) / chunk <= (uint64_t)g_par.max_wave_chunks;
+    for (int l = 0; fits && l < g_par.lanes; ++l)
+      if (lane_chunks[l]) fits = (base_end[l] + 127) / 128 * 128 + lane_bytes[l] <= pr->wins.cap[l];
+    if (!fits) break;
+    uint32_t k;
+    if (extend) {
+      k = b.n_seg - 1;
+      b.seg[k].n_req++;
+    } else {
+      for (int l = 0; l < FLH_MAX_LANES; ++l) closed_end[l] = base_end[l];
+      chunks_closed = chunks_before;
+      row = try_row;
+      k = b.n_seg++;
+      b.seg[k].epoch_bytes = epoch;
+      b.seg[k].n_req = 1;
+      memcpy(b.seg[k].credits, credits, sizeof(credits));
+      bb.seg_link[k] = p.lk;
+    }
+    seg_bytes = try_bytes;
+    bb.link_epoch_after[k] = b.seg[k].epoch_bytes + seg_bytes;
+    b.d_src[b.n_req] = p.src;
+    b.d_dst[b.n_req] = p.dst;
+    b.bytes[b.n_req] = (uint64_t)p.size;
+    b.n_req++;
+    b.u.total_bytes += (uint64_t)p.size;
+    ++j;
+  }
+  return j - i;
+}
 
-// Launch everything that waits on the connection, in order (launch_mu held).  A failure completes the requests
-// it touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).
-void flush_pending(Link* lk) {
-  if (lk->pending.empty()) return;
+ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, uint64_t seq) {
+  flh_batch_params& b = bb.b;
+  b.u.tile_bytes = launch_tile(b.u.total_bytes);
+  uint64_t seg_base[FLH_SEG_MAX][FLH_MAX_LANES];
+  FL_FLHCHECK(flh_batch_layout(&b, nullptr, &seg_base[0][0]));
+  FL_FLHCHECK(flh_stripe_batch(&b, &pr->wins, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+  Completion comp;
+  ncclResult_t rc = prepare_completion(pr, seq, b.u, comp);
+  if (rc != ncclSuccess) return rc;
+  FL_FLHCHECK(flh_reassemble_batch(&b, &pr->wins, pr->d_status, pr->stream));
+  rc = finish_completion(pr, seq, comp);
+  if (rc != ncclSuccess) return rc;
+  // bookkeeping: every connection's place in its epoch, what the launch carried
+  const uint64_t chunk = (uint64_t)g_par.chunk;
+  pr->last.seq = seq;
+  pr->last.n_seg = b.n_seg;
+  uint32_t row = 0, q = 0;
+  for (uint32_t k = 0; k < b.n_seg; ++k) {
+    Link* lk = bb.seg_link[k];
+    uint64_t seg_bytes = 0;
+    for (uint32_t r = 0; r < b.seg[k].n_req; ++r) seg_bytes += b.bytes[q++];
+    const uint32_t rows = (uint32_t)((seg_bytes + chunk - 1) / chunk);
+    note_segment(pr, k, lk, row, rows, b.seg[k].n_req, b.seg[k].epoch_bytes, seg_base[k]);
+    if (lk->last_seq != seq) lk->launches++;
+    lk->last_seq = seq;
+    lk->last_first_row = row;
+    lk->last_rows = rows;
+    lk->epoch_bytes = bb.link_epoch_after[k];
+    if (n > 1) lk->batched_requests += b.seg[k].n_req;
+    row += rows;
+  }
+  pr->last.n_rows = row;
+  return ncclSuccess;
+}
+
+// Launch everything that waits on the peer, in order (launch_mu held).  A failure completes the requests it
+// touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).
+void flush_pending(Peer* pr) {
+  {
+    std::lock_guard<std::mutex> g(pr->queue_mu);
+    if (pr->pending.empty()) return;
+    pr->work.clear();
+    pr->work.swap(pr->pending);
+    pr->waiting_reqs.store(0, std::memory_order_release);
+    pr->waiting_bytes.store(0, std::memory_order_release);
+  }
   DeviceScope keep;
-  bool dev_ok = hipSetDevice(lk->hip_device) == hipSuccess;
+  const bool dev_ok = hipSetDevice(pr->hip_device) == hipSuccess;
+  std::vector<Pending>& work = pr->work;
   size_t i = 0;
-  while (i < lk->pending.size()) {
-    const size_t span = batch_span(lk, i);
+  while (i < work.size()) {
     ncclResult_t rc = dev_ok ? ncclSuccess : ncclUnhandledCudaError;
-    const uint64_t seq = lk->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
-    const size_t slot = (size_t)((seq - 1) % FL_NET_MAX_REQUESTS);
-    hipEvent_t& ev = lk->evring[slot];
-    if (rc == ncclSuccess && !ev) { hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming); if (e != hipSuccess) rc = hip_fail("hipEventCreate", e); }
-    bool stamped = false, rides = false;
+    const uint64_t seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
+    pr->launch_seq.store(seq, std::memory_order_release);   // before anything runs: the completion word never runs ahead of it
+    size_t span = 1;
+    const Pending& p = work[i];
     if (rc == ncclSuccess) {
-      const Pending& p = lk->pending[i];
-      const bool gpu = span > 1 || (p.src_dev && p.dst_dev);
-      if (gpu) {
-        if (g_par.completion == 2) fl_launch_stamp(lk->d_stamp, (uint32_t)(seq - 1));
-        hipEvent_t on_kernel = g_par.completion == 1 ? ev : nullptr;
-        rc = span > 1 ? launch_batch(lk, i, i + span, on_kernel) : launch_transfer(lk, p, on_kernel);
-        stamped = fl_launch_stamp_taken();
-        rides = fl_completion_event_taken();
-      } else {
+      if (!(p.src_dev && p.dst_dev)) {
         // one side is host memory: the copy engine is the wire, nothing is striped
-        hipError_t e = hipMemcpyAsync(p.dst, p.src, (size_t)p.size, hipMemcpyDefault, lk->stream);
+        hipEvent_t ev = nullptr;
+        rc = launch_event(pr, seq, &ev);
+        hipError_t e = rc == ncclSuccess ? hipMemcpyAsync(p.dst, p.src, (size_t)p.size, hipMemcpyDefault, pr->stream) : hipSuccess;
         if (e != hipSuccess) rc = hip_fail("hipMemcpyAsync", e);
-      }
-    }
-    // A launch that begins with a stamping kernel needs no event now: the launch after it stamps it complete, or
-    // its first poll records the event if nothing has followed.  Everything else (host memory, nothing to launch,
-    // the other completion modes) gets the event here unless it already rides on the last kernel.
-    // A small launch gets its event at once all the same: its requests are bound by the host's polling, which an
-    // event that is already there serves sooner, not by the queue.
-    uint64_t launch_bytes = 0;
-    for (size_t k = i; k < i + span; ++k) launch_bytes += (uint64_t)lk->pending[k].size;
-    const bool later = stamped && launch_bytes >= kEarlyLaunchBytes;
-    bool recorded = rides;
-    if (rc == ncclSuccess && !rides && !later) {
-      hipError_t e = hipEventRecord(ev, lk->stream);
-      if (e != hipSuccess) rc = hip_fail("hipEventRecord", e);
-      recorded = true;
-    }
-    lk->ev_set[slot].store(recorded ? 1 : 0, std::memory_order_release);
-    lk->stamps[slot].store(stamped ? 1 : 0, std::memory_order_release);
-    for (size_t k = i; k < i + span; ++k) {
-      Pending& p = lk->pending[k];
-      if (rc == ncclSuccess) {
-        p.sreq->seq = seq;
-        p.rreq->seq = seq;
-        p.sreq->state.store(kStLaunched, std::memory_order_release);
-        p.rreq->state.store(kStLaunched, std::memory_order_release);
+        if (rc == ncclSuccess) { Completion c; c.ev = ev; rc = finish_completion(pr, seq, c); }
+      } else if (g_par.batch < 2 || needs_waves(pr, p, (p.w.flags & 1u) ? 0 : p.lk->epoch_bytes)) {
+        rc = launch_transfer(pr, p, seq);
       } else {
-        p.sreq->fault = 1;
-        p.rreq->fault = 1;
-        p.sreq->state.store(kStDoneHost, std::memory_order_release);
-        p.rreq->state.store(kStDoneHost, std::memory_order_release);
+        BatchBuild bb;
+        span = build_batch(pr, i, bb);
+        if (span == 0) { span = 1; rc = launch_transfer(pr, p, seq); }   // cannot happen: the request fits an empty set of windows
+        else rc = launch_batch(pr, i, span, bb, seq);
       }
     }
-    if (rc == ncclSuccess) lk->launch_seq.store(seq, std::memory_order_release);
+    for (size_t k = i; k < i + span; ++k) {
+      Pending& q = work[k];
+      if (rc == ncclSuccess) {
+        q.sreq->seq = seq;
+        q.rreq->seq = seq;
+        q.sreq->state.store(kStLaunched, std::memory_order_release);
+        q.rreq->state.store(kStLaunched, std::memory_order_release);
+      } else {
+        q.sreq->fault = 1;
+        q.rreq->fault = 1;
+        q.sreq->state.store(kStDoneHost, std::memory_order_release);
+        q.rreq->state.store(kStDoneHost, std::memory_order_release);
+      }
+    }
+    if (rc != ncclSuccess) {
+      // whatever part of the launch was queued is waited for here, so that its number counts as complete and the
+      // launches behind it are not held back by one that will never report
+      if (dev_ok) (void)hipStreamSynchronize(pr->stream);
+      uint64_t seen = pr->done_seq.load(std::memory_order_relaxed);
+      while (seen < seq && !pr->done_seq.compare_exchange_weak(seen, seq, std::memory_order_release, std::memory_order_relaxed)) {}
+    }
     i += span;
   }
-  lk->pending.clear();
-  lk->waiting_bytes.store(0, std::memory_order_release);
+  work.clear();
 }
 
 ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhandle, void** request) {
@@ -848,7 +1067,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     sreq->size = size;
     rreq->size = size;
     const bool any_dev = mh->type == NCCL_PTR_CUDA || rtype == NCCL_PTR_CUDA;
-    if (size && any_dev) rc = ensure_link_gpu(lk, mh->type == NCCL_PTR_CUDA ? mh->device : fs.rdevice);
+    if (size && any_dev) rc = attach_peer(lk, mh->type == NCCL_PTR_CUDA ? mh->device : fs.rdevice);
     if (rc != ncclSuccess) { sreq->type = kReqUnused; return rc; }   // nothing consumed: the descriptor stays posted
     memset((void*)&fs.w, 0, sizeof(FifoWire));   // plugin.cc:1605
     fs.rreq = nullptr;
@@ -865,9 +1084,10 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     sreq->state.store(kStDoneHost, std::memory_order_release);
     rreq->state.store(kStDoneHost, std::memory_order_release);
   } else {
-    // device memory: the launches are made with the other sends that wait on this connection
-    std::lock_guard<std::mutex> g(lk->launch_mu);
+    // device memory: the launches are made together with the other sends that wait on this GPU
+    Peer* pr = lk->peer.load(std::memory_order_acquire);
     Pending p;
+    p.lk = lk;
     p.src = (const uint8_t*)data;
     p.dst = dst;
     p.size = size;
@@ -876,11 +1096,20 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     p.w = w;
     p.sreq = sreq;
     p.rreq = rreq;
-    lk->pending.push_back(p);
-    lk->waiting_bytes.store(lk->waiting_bytes.load(std::memory_order_relaxed) + (uint64_t)p.size, std::memory_order_release);
     sreq->state.store(kStQueued, std::memory_order_release);
     rreq->state.store(kStQueued, std::memory_order_release);
-    if ((int)lk->pending.size() >= g_par.batch) flush_pending(lk);
+    uint32_t waiting;
+    {
+      std::lock_guard<std::mutex> g(pr->queue_mu);
+      pr->pending.push_back(p);
+      waiting = pr->waiting_reqs.load(std::memory_order_relaxed) + 1;
+      pr->waiting_reqs.store(waiting, std::memory_order_release);
+      pr->waiting_bytes.store(pr->waiting_bytes.load(std::memory_order_relaxed) + (uint64_t)size, std::memory_order_release);
+    }
+    if ((int)waiting >= g_par.batch) {   // a full launch waits (NCCL_FUSELINK_BATCH=1: every send is launched here)
+      std::lock_guard<std::mutex> g(pr->launch_mu);
+      flush_pending(pr);
+    }
   }
   *request = sreq;
   return ncclSuccess;
@@ -946,15 +1175,47 @@ ncclResult_t fl_iflush(void* recvComm, int /*n*/, void** /*data*/, int* /*sizes*
   return ncclSuccess;
 }
 
-// Launches of the connection that have been queued and are not known to be complete.
-uint64_t launches_in_queue(const Link* lk) {
-  const uint64_t queued = lk->launch_seq.load(std::memory_order_acquire);
-  uint64_t done = lk->done_seq.load(std::memory_order_acquire);
-  if (lk->h_stamp) {   // the stamp trails the newest launch by a small number
-    const uint32_t behind = (uint32_t)queued - __atomic_load_n(lk->h_stamp, __ATOMIC_ACQUIRE);
-    if (behind <= queued && queued - behind > done) done = queued - behind;
+// Is launch `seq` of the peer complete?  Launches run in order on one stream, so a launch is complete once a later
+// one is.  Mode 2 reads the completion word: a plain load of pinned memory.  Launches whose completion is an event
+// (the other modes, and whatever is not a kernel) are asked through the runtime.
+ncclResult_t launch_complete(Peer* pr, uint64_t seq, bool* done) {
+  *done = false;
+  uint64_t seen = pr->done_seq.load(std::memory_order_acquire);
+  if (seq <= seen) { *done = true; return ncclSuccess; }
+  if (g_par.completion == 2) {
+    // The acquire load pairs with the kernel's release store at system scope: what every workgroup of that launch,
+    // and of the launches before it, wrote is visible to this thread and to whatever it starts afterwards.
+    const uint32_t word = __atomic_load_n(pr->h_done, __ATOMIC_ACQUIRE);
+    const uint64_t top = pr->launch_seq.load(std::memory_order_acquire);
+    uint64_t upto = (top & ~0xffffffffull) | word;   // the word holds the low half of a launch number at or below `top`
+    if (upto > top) upto -= 1ull << 32;
+    if (word != 0 && upto > seen && upto <= top) {
+      while (seen < upto && !pr->done_seq.compare_exchange_weak(seen, upto, std::memory_order_release, std::memory_order_relaxed)) {}
+      if (seq <= upto) { *done = true; return ncclSuccess; }
+    }
   }
-  return queued - done;
+  const size_t slot = (size_t)((seq - 1) % kEventRing);
+  if (pr->ev_seq[slot].load(std::memory_order_acquire) != seq) return ncclSuccess;   // no event stands for this launch
+  hipError_t e = hipEventQuery(pr->evring[slot]);
+  if (e == hipErrorNotReady) return ncclSuccess;
+  if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+  seen = pr->done_seq.load(std::memory_order_relaxed);
+  while (seen < seq && !pr->done_seq.compare_exchange_weak(seen, seq, std::memory_order_release, std::memory_order_relaxed)) {}
+  *done = true;
+  return ncclSuccess;
+}
+
+// Launches of the peer that have been queued and are not known to be complete.
+uint64_t launches_in_queue(Peer* pr) {
+  uint64_t done = pr->done_seq.load(std::memory_order_acquire);
+  const uint64_t top = pr->launch_seq.load(std::memory_order_acquire);
+  if (g_par.completion == 2) {
+    const uint32_t word = __atomic_load_n(pr->h_done, __ATOMIC_ACQUIRE);
+    uint64_t upto = (top & ~0xffffffffull) | word;
+    if (upto > top) upto -= 1ull << 32;
+    if (word != 0 && upto > done && upto <= top) done = upto;
+  }
+  return top - done;
 }
 
 ncclResult_t fl_test(void* request, int* done, int* sizes) {
@@ -963,69 +1224,50 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   if (r->magic != kReqMagic || r->type == kReqUnused) { FL_WARN("NET/FuseLink : test on a request that is not in flight"); return ncclInternalError; }
   *done = 0;
   Link* lk = r->link;
-  // the event is polled without the connection's lock: only the thread that drives this comm tests its requests
+  // the request is polled without the connection's lock: only the thread that drives this comm tests its requests
   int st = r->state.load(std::memory_order_acquire);
   if (st == kStPosted || st == 0) return ncclSuccess;   // a receive whose send has not been matched yet
-  // Matched sends wait so that those that arrive together can share a launch.  They go out when one of them is
-  // polled.  Large ones (8 MiB and more wait) also go out when any request of the connection is polled while fewer
-  // than two launches are left in the queue: the GPU then does not run dry behind a launch whose requests are still
-  // being polled (measured: 25-30 us of idle queue every third or fourth 64 MiB request otherwise).  Small ones keep
-  // waiting: what they gain from sharing a launch outweighs the idle queue (512 KiB requests: 2.2x).
-  if (st == kStQueued || (lk->waiting_bytes.load(std::memory_order_acquire) >= kEarlyLaunchBytes && launches_in_queue(lk) < 2)) {
-    std::lock_guard<std::mutex> g(lk->launch_mu);
-    flush_pending(lk);
-    st = r->state.load(std::memory_order_acquire);
+  Peer* pr = lk->peer.load(std::memory_order_acquire);
+  // Matched sends wait so that those that arrive together -- on this connection and on the others that stage on
+  // the same GPU -- can share a launch.  They go out when a test finds the GPU short of work: fewer than two
+  // launches in its queue and something waiting, whichever request is being polled.  While two launches or more are
+  // queued the GPU is not waiting for the host, and holding the sends back costs them nothing but lets the next
+  // launch carry more of them; a full launch's worth (NCCL_FUSELINK_BATCH) never waits (isend launches it).
+  if (pr && pr->waiting_reqs.load(std::memory_order_acquire) != 0) {
+    // a launch whose completion comes from an event is only known complete once its own requests are polled: it
+    // must not hold anything back
+    const bool events_out = pr->last_event_seq.load(std::memory_order_acquire) > pr->done_seq.load(std::memory_order_acquire);
+    if (events_out || g_par.completion != 2 || launches_in_queue(pr) < 2) {
+      if (pr->launch_mu.try_lock()) {   // if another thread is launching, it or the next poll takes care of it
+        flush_pending(pr);
+        pr->launch_mu.unlock();
+      }
+      st = r->state.load(std::memory_order_acquire);
+    }
   }
+  if (st == kStQueued) return ncclSuccess;
   if (st == kStLaunched) {
-    if (r->seq > lk->done_seq.load(std::memory_order_acquire)) {
-      uint64_t upto = 0;   // launches known complete
-      if (lk->h_stamp) {   // a later launch's first kernel has started: everything before it is done
-        const uint32_t stamp = __atomic_load_n(lk->h_stamp, __ATOMIC_ACQUIRE);
-        const int32_t ahead = (int32_t)(stamp - (uint32_t)r->seq);
-        if (ahead >= 0) upto = r->seq + (uint64_t)ahead;
-      }
-      if (!upto) {
-        uint64_t q = r->seq;   // the launch whose event answers for this request
-        const size_t slot = (size_t)((q - 1) % FL_NET_MAX_REQUESTS);
-        if (!lk->ev_set[slot].load(std::memory_order_acquire)) {
-          if (q < lk->launch_seq.load(std::memory_order_acquire)) {
-            // a launch follows: its first kernel will stamp this one, or else its event was recorded behind it
-            const size_t next = (size_t)(q % FL_NET_MAX_REQUESTS);
-            if (lk->stamps[next].load(std::memory_order_acquire) || !lk->ev_set[next].load(std::memory_order_acquire)) return ncclSuccess;
-            q += 1;
-          } else {
-            // nothing follows: the event goes behind the launch now (and delays no kernel, the queue ends here)
-            std::lock_guard<std::mutex> g(lk->launch_mu);
-            if (q == lk->launch_seq.load(std::memory_order_relaxed) && !lk->ev_set[slot].load(std::memory_order_relaxed)) {
-              DeviceScope keep;
-              hipError_t e = hipSetDevice(lk->hip_device);
-              if (e == hipSuccess) e = hipEventRecord(lk->evring[slot], lk->stream);
-              if (e != hipSuccess) return hip_fail("hipEventRecord", e);
-              lk->ev_set[slot].store(1, std::memory_order_release);
-            } else if (!lk->ev_set[slot].load(std::memory_order_relaxed)) {
-              return ncclSuccess;   // a launch went out meanwhile: the next poll looks at it
-            }
-          }
-        }
-        hipError_t e = hipEventQuery(lk->evring[(size_t)((q - 1) % FL_NET_MAX_REQUESTS)]);
-        if (e == hipErrorNotReady) return ncclSuccess;
-        if (e != hipSuccess) return hip_fail("hipEventQuery", e);
-        upto = q;
-      }
-      uint64_t seen = lk->done_seq.load(std::memory_order_relaxed);
-      while (seen < upto && !lk->done_seq.compare_exchange_weak(seen, upto, std::memory_order_release, std::memory_order_relaxed)) {}
-    }
-    if (lk->h_status && *(volatile int32_t*)lk->h_status != 0) {
-      FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", *lk->h_status);
-      return ncclInternalError;
-    }
+    bool complete = false;
+    ncclResult_t rc = launch_complete(pr, r->seq, &complete);
+    if (rc != ncclSuccess || !complete) return rc;
   }
   std::lock_guard<std::mutex> g(lk->mu);
+  ncclResult_t result = ncclSuccess;
   if (r->fault) {   // failed completion, plugin.cc:1839-1861
     FL_WARN("NET/FuseLink : Got completion with error (injected), channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
     return ncclRemoteError;
   }
-  *done = 1;                                                // plugin.cc:1807-1823
+  if (st == kStLaunched && pr && __atomic_load_n(pr->h_status, __ATOMIC_ACQUIRE) != 0) {
+    // A kernel refused a chunk that would have left its window or buffer (the host sizes every launch so that this
+    // cannot happen; the check is the safety net).  The first request completed after the refusal reports it, once,
+    // and is freed like any other; the word is cleared so that later traffic is not condemned with it.
+    const int32_t code = __atomic_exchange_n(pr->h_status, 0, __ATOMIC_ACQ_REL);
+    if (code != 0) {
+      FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", code);
+      result = ncclInternalError;
+    }
+  }
+  *done = result == ncclSuccess ? 1 : 0;                    // plugin.cc:1807-1823
   if (r->type == kReqSend) { lk->s_finished++; lk->s_inflight--; }
   if (r->type == kReqRecv) {
     (void)fl_monitor_mark_active(lk->dev % g_par.lanes, 0, fl_monitor_now());   // updateRxChannelActive, fuselink.h:254-259
@@ -1034,7 +1276,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     if (sizes) sizes[0] = r->size;   // the reference leaves 0 here (plugin.cc:1726, 1882)
   }
   r->type = kReqUnused;                                     // ncclIbFreeRequest, plugin.cc:1086-1090
-  return ncclSuccess;
+  return result;
 }
 
 ncclResult_t close_comm(void* comm, int want_send) {
@@ -1165,9 +1407,23 @@ int fl_net_launch_stats(void* comm, int64_t* launches, int64_t* batched_requests
   Comm* c = (Comm*)comm;
   if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
   Link* lk = c->link;
-  std::lock_guard<std::mutex> g(lk->launch_mu);
+  Peer* pr = lk->peer.load(std::memory_order_acquire);
+  if (!pr) {
+    if (launches) *launches = 0;
+    if (batched_requests) *batched_requests = 0;
+    return FLH_OK;
+  }
+  std::lock_guard<std::mutex> g(pr->launch_mu);
   if (launches) *launches = lk->launches;
   if (batched_requests) *batched_requests = lk->batched_requests;
+  return FLH_OK;
+}
+
+// launch everything that waits and wait for the stream (launch_mu held)
+static int drain_peer(Peer* pr) {
+  flush_pending(pr);
+  DeviceScope keep;
+  if (hipSetDevice(pr->hip_device) != hipSuccess || hipStreamSynchronize(pr->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
   return FLH_OK;
 }
 
@@ -1175,19 +1431,60 @@ int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_ou
   Comm* c = (Comm*)sendComm;
   if (!c || c->magic != kCommMagic || !c->is_send) return fl_set_error(FLH_E_ARG, "not a send comm");
   Link* lk = c->link;
-  std::lock_guard<std::mutex> g(lk->mu);
-  if (!lk->gpu_ready) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
-  std::lock_guard<std::mutex> gl(lk->launch_mu);
-  flush_pending(lk);
+  Peer* pr = lk->peer.load(std::memory_order_acquire);
+  if (!pr) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
+  std::lock_guard<std::mutex> gl(pr->launch_mu);
+  int rc = drain_peer(pr);
+  if (rc) return rc;
+  if (lk->last_seq == 0) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
+  if (lk->last_seq != pr->last.seq) return fl_set_error(FLH_E_STATE, "a later launch of another connection has reused the table");
+  const int rows = (int)lk->last_rows;
+  const int take = rows < max_rows ? rows : max_rows;
   DeviceScope keep;
-  if (hipSetDevice(lk->hip_device) != hipSuccess || hipStreamSynchronize(lk->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
-  int rows = (int)lk->last_wave_rows.load();
-  int take = rows < max_rows ? rows : max_rows;
-  if (take > 0 && rows_out && hipMemcpy(rows_out, lk->d_table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
+  if (hipSetDevice(pr->hip_device) != hipSuccess) return fl_set_error(FLH_E_HIP, "hipSetDevice failed");
+  if (take > 0 && rows_out && hipMemcpy(rows_out, pr->d_table + lk->last_first_row, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "table copy failed");
-  if (hdr_out && hipMemcpy(hdr_out, lk->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
+  if (hdr_out && hipMemcpy(hdr_out, pr->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "header copy failed");
   return rows;
+}
+
+int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, void* rows_out, int max_rows, void* hdr_out) {
+  Comm* c = (Comm*)comm;
+  if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
+  Peer* pr = c->link->peer.load(std::memory_order_acquire);
+  if (!pr) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
+  std::lock_guard<std::mutex> gl(pr->launch_mu);
+  int rc = drain_peer(pr);
+  if (rc) return rc;
+  const LaunchInfo& li = pr->last;
+  for (int k = 0; k < (int)li.n_seg && k < max_segs && segs_out; ++k) {
+    fl_net_launch_seg& o = segs_out[k];
+    o.channel = li.seg[k].channelId;
+    o.first_row = li.seg[k].first_row;
+    o.n_rows = li.seg[k].n_rows;
+    o.n_req = li.seg[k].n_req;
+    o.epoch_bytes = li.seg[k].epoch_bytes;
+    for (int l = 0; l < FL_NET_MAX_LANES; ++l) o.lane_base[l] = li.seg[k].lane_base[l];
+  }
+  const int take = (int)li.n_rows < max_rows ? (int)li.n_rows : max_rows;
+  DeviceScope keep;
+  if (hipSetDevice(pr->hip_device) != hipSuccess) return fl_set_error(FLH_E_HIP, "hipSetDevice failed");
+  if (take > 0 && rows_out && hipMemcpy(rows_out, pr->d_table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
+    return fl_set_error(FLH_E_HIP, "table copy failed");
+  if (hdr_out && hipMemcpy(hdr_out, pr->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
+    return fl_set_error(FLH_E_HIP, "header copy failed");
+  return (int)li.n_seg;
+}
+
+int fl_net_flush(void* comm) {
+  Comm* c = (Comm*)comm;
+  if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
+  Peer* pr = c->link->peer.load(std::memory_order_acquire);
+  if (!pr) return FLH_OK;
+  std::lock_guard<std::mutex> gl(pr->launch_mu);
+  flush_pending(pr);
+  return FLH_OK;
 }
 
 }  // extern "C"

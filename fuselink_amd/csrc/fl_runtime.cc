@@ -35,34 +35,6 @@ namespace {
 thread_local ProfState t_prof;
 }
 ProfState& fl_prof() { return t_prof; }
-void fl_completion_event(void* hip_event) {
-  t_prof.done_ev = (hipEvent_t)hip_event;
-  t_prof.done_handed = hip_event != nullptr;
-}
-bool fl_completion_event_taken() {
-  const bool taken = t_prof.done_handed && t_prof.done_ev == nullptr;
-  t_prof.done_ev = nullptr;
-  t_prof.done_handed = false;
-  return taken;
-}
-
-void fl_launch_stamp(uint32_t* d_word, uint32_t value) {
-  t_prof.stamp = d_word;
-  t_prof.stamp_value = value;
-  t_prof.stamp_handed = d_word != nullptr;
-}
-void fl_take_launch_stamp(uint32_t** word, uint32_t* value) {
-  *word = t_prof.stamp;
-  *value = t_prof.stamp_value;
-  t_prof.stamp = nullptr;
-}
-bool fl_launch_stamp_taken() {
-  const bool taken = t_prof.stamp_handed && t_prof.stamp == nullptr;
-  t_prof.stamp = nullptr;
-  t_prof.stamp_handed = false;
-  return taken;
-}
-
 int fl_set_error(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -130,10 +102,12 @@ int64_t flh_constant(int which) {
     case 4: return sizeof(flh_chunk_desc);
     case 5: return sizeof(flh_sched_state);
     case 6: return sizeof(flh_sched_hdr);
-    case 7: return 3;   // ABI version: 2 added flh_sched_params.d_table_by_lane, the batch entry points, the DMA-BUF export;
-                        // 3 the per-tile descriptors (flh_sched_params.d_tiles, flh_stripe_tiles / flh_reassemble_tiles) and the fused paged pair
+    case 7: return 4;   // ABI version: 2 added flh_sched_params.d_table_by_lane, the batch entry points, the DMA-BUF export;
+                        // 3 the per-tile descriptors (flh_sched_params.d_tiles, flh_stripe_tiles / flh_reassemble_tiles) and the fused paged pair;
+                        // 4 batches of up to 32 requests in segments, the completion word / event in flh_uniform_params, flh_schedule_static
     case 8: return sizeof(flh_windows);
     case 9: return sizeof(flh_sched_params);
+    case 10: return sizeof(flh_batch_params);
   }
   return -1;
 }

@@ -73,7 +73,13 @@ def _table(version: int):
 PLUGIN_SYMBOLS = ["ncclNetPlugin_v8", "ncclNetPlugin_v7", "ncclNetPlugin_v6"]
 CONTROL_SYMBOLS = ["fl_monitor_attach_shm", "fl_monitor_detach", "fl_monitor_is_shared", "fl_monitor_daemon_running", "fl_monitor_reset", "fl_monitor_set_entry", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
                    "fl_monitor_status", "fl_monitor_idle_pick", "fl_monitor_release", "fl_monitor_credits", "fl_net_set_credits",
-                   "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_launch_stats", "fl_net_last_table", "fl_net_reset"]
+                   "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_launch_stats", "fl_net_last_table", "fl_net_last_launch",
+                   "fl_net_flush", "fl_net_reset"]
+
+
+class LaunchSeg(C.Structure):
+    _fields_ = [("channel", C.c_int32), ("first_row", C.c_uint32), ("n_rows", C.c_uint32), ("n_req", C.c_uint32),
+                ("epoch_bytes", C.c_uint64), ("lane_base", C.c_uint64 * 16)]
 
 
 class NetPlugin:
@@ -112,6 +118,8 @@ class NetPlugin:
         L.fl_net_comm_stats.argtypes = [VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         L.fl_net_launch_stats.argtypes = [VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         L.fl_net_last_table.argtypes = [VP, VP, C.c_int, VP]
+        L.fl_net_last_launch.argtypes = [VP, C.POINTER(LaunchSeg), C.c_int, VP, C.c_int, VP]
+        L.fl_net_flush.argtypes = [VP]
 
     # ---- the function table -----------------------------------------------------------------------
     @property
@@ -270,3 +278,22 @@ class NetPlugin:
         if n < 0:
             raise RuntimeError("fl_net_last_table failed")
         return rows[: min(n, max_rows)], hdr[0]
+
+    def last_launch(self, comm, max_rows: int = 4096):
+        """Segments, table and header of the last launch pair on the GPU that `comm` stages on."""
+        import numpy as np
+
+        from .core import DESC_DTYPE, HDR_DTYPE
+        segs = (LaunchSeg * 8)()
+        rows = np.zeros(max_rows, dtype=DESC_DTYPE)
+        hdr = np.zeros(1, dtype=HDR_DTYPE)
+        n = self.lib.fl_net_last_launch(comm, segs, 8, rows.ctypes.data_as(VP), max_rows, hdr.ctypes.data_as(VP))
+        if n < 0:
+            raise RuntimeError("fl_net_last_launch failed")
+        out = [dict(channel=s.channel, first_row=s.first_row, n_rows=s.n_rows, n_req=s.n_req, epoch_bytes=s.epoch_bytes,
+                    lane_base=list(s.lane_base)) for s in segs[:n]]
+        total = sum(s["n_rows"] for s in out)
+        return out, rows[:total], hdr[0]
+
+    def flush(self, comm) -> None:
+        assert self.lib.fl_net_flush(comm) == 0

@@ -137,7 +137,8 @@ const char* flh_last_error(void);
 /* bytes of flh_sched_params.d_workspace that flh_schedule needs for n_chunks chunks */
 uint64_t flh_schedule_workspace_bytes(uint32_t n_chunks);
 /* compile-time facts: 0 tile bytes, 1 max lanes, 2 unit bytes, 3 pool units, 4 sizeof(desc),
- * 5 sizeof(state), 6 sizeof(hdr), 7 ABI version, 8 sizeof(flh_windows), 9 sizeof(flh_sched_params) */
+ * 5 sizeof(state), 6 sizeof(hdr), 7 ABI version, 8 sizeof(flh_windows), 9 sizeof(flh_sched_params),
+ * 10 sizeof(flh_batch_params) */
 int64_t flh_constant(int which);
 /* Launch tunables, for experiments (no counterpart in the reference): "grid_per_cu" = copy
  * workgroups launched per compute unit (0 = one per tile), "nontemporal" = 0/1 streaming loads and
@@ -234,6 +235,21 @@ typedef struct flh_uniform_params {
   uint32_t tile_bytes;
   uint32_t pad;
   uint32_t credits[FLH_MAX_LANES];
+  /* Completion of the reassembly / scatter launch, for callers that poll instead of synchronising (all optional; the
+   * striping side ignores them; no counterpart in the reference, whose completions come from the NIC's queue,
+   * src/plugin.cc:1801-1955).
+   * d_done_word: a host-visible word (e.g. pinned, mapped memory).  The launch counts its finished workgroups in
+   * *d_done_count (device memory, zero before the first use; the kernel leaves it zero) and the last of them stores
+   * done_value to *d_done_word with release semantics at system scope, after every workgroup's stores: a thread that
+   * reads done_value there with acquire semantics may use the destination buffer.  Launches that share a count word
+   * must be ordered (one stream).
+   * done_event: a hipEvent_t that the launch's kernel completes (hipEventQuery then answers for the kernel), which
+   * spares the separate packet of a hipEventRecord behind it. */
+  uint32_t* d_done_word;
+  uint32_t* d_done_count;
+  uint32_t done_value;
+  uint32_t pad2;
+  void* done_event;
 } flh_uniform_params;
 
 int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows* win,
@@ -242,27 +258,49 @@ int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows*
 int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
                            const flh_uniform_params* u, int32_t* d_status, void* stream);
 
-/* Several requests in one launch: the requests of one connection that are waiting together (NCCL keeps up
- * to NCCL_STEPS = 8 in flight, src/fuselink.h:14) are scheduled and copied as ONE message -- the
- * concatenation of their buffers -- so the launch cost is paid once per batch instead of once per
- * request.  u->total_bytes must equal the sum of bytes[], u->src_base is ignored, every request but
- * the last must be a whole number of chunks (then the table equals that of a single message of
- * total_bytes; row src_off is the offset in the concatenation).  No counterpart in the reference,
- * which posts one RDMA write per request. */
-#define FLH_BATCH_MAX 8
+/* Several requests in one launch: requests that are waiting together -- NCCL keeps up to NCCL_STEPS = 8 in flight per
+ * channel (src/fuselink.h:14) and runs several channels to a peer, which all share the per-NIC lane comms
+ * (src/fuselink.h:271-272, src/plugin.cc:727-753) -- are scheduled and copied by ONE launch per direction, so the
+ * launch cost is paid once per batch instead of once per request.  No counterpart in the reference, which posts one
+ * RDMA write per request.
+ *
+ * The requests form 1..FLH_SEG_MAX segments, in order.  A segment is a run of requests that is scheduled as ONE
+ * message -- the concatenation of its buffers -- from its own credit-epoch prefix under its own credit row, exactly as
+ * flh_stripe_uniform schedules a message: the requests of one connection between two lane-decision refreshes.  Every
+ * request of a segment but its last must be a whole number of chunks.  In the staging windows the segments follow each
+ * other: on every lane, segment k starts where segment k - 1 ended, rounded up to 128 bytes (the alignment of the
+ * reference's per-QP pieces, src/plugin.cc:1467).  n_seg == 0 stands for one segment of all requests under u.credits
+ * and u.epoch_bytes.  u.total_bytes must equal the sum of bytes[]; u.src_base is ignored; a credit row must sum below
+ * 2^32.
+ *
+ * Table rows (flh_stripe_batch, when d_table_out is given) are those of each segment's message -- src_off counts from
+ * the segment's first byte -- with the segment's lane base added to win_off and tile_base counted over the whole
+ * launch; the header holds the totals of the launch. */
+#define FLH_BATCH_MAX 32
+#define FLH_SEG_MAX 8
+typedef struct flh_batch_segment {
+  uint64_t epoch_bytes;       /* bytes already scheduled in the segment's credit epoch (0 after a refresh) */
+  uint32_t n_req;             /* requests of the batch, in order, that form this segment */
+  uint32_t pad;
+  uint32_t credits[FLH_MAX_LANES];
+} flh_batch_segment;
 typedef struct flh_batch_params {
   flh_uniform_params u;
   uint32_t n_req;             /* 1..FLH_BATCH_MAX */
-  uint32_t pad;
+  uint32_t n_seg;             /* 0 (one segment, u.credits / u.epoch_bytes) or 1..FLH_SEG_MAX */
   const void* d_src[FLH_BATCH_MAX];
   void*       d_dst[FLH_BATCH_MAX];
   uint64_t    bytes[FLH_BATCH_MAX];
+  flh_batch_segment seg[FLH_SEG_MAX];
 } flh_batch_params;
 
 int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
                      flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
 int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int32_t* d_status, void* stream);
-
+/* Where the batch leaves every staging window: lane_end[l] = first free byte of lane l after the last segment
+ * (host arithmetic, nothing is launched); seg_base, if given, receives FLH_SEG_MAX x FLH_MAX_LANES lane bases, row k
+ * those of segment k.  A caller sizes its batches with it so that no lane outgrows its window. */
+int flh_batch_layout(const flh_batch_params* b, uint64_t* lane_end, uint64_t* seg_base);
 /* Paged variants for non-contiguous sources (KV-cache blocks, src/experiments/serving/model.hh:
  * 198-201 gives the page shape): a chunk whose row says src_off stands for the pages
  * d_page_table[src_off / page_bytes ...] (pages_per_chunk of them) of a pool of page_bytes-sized

@@ -235,14 +235,29 @@ int fl_net_reset(void);
 int fl_net_inject_fault(void* request);
 /* Counters of a send or recv comm: n_finished (src/plugin.cc:517,568), requests in flight, lane refreshes. */
 int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64_t* refreshes);
-/* Launch pairs (stripe + reassemble) a connection has queued so far, and how many requests travelled in
- * a pair shared with others.  Matched sends wait for the first test() of one of them or until
- * NCCL_FUSELINK_BATCH (default 8, 1 = launch inside isend) of them wait, then go out together. */
+/* Launch pairs (stripe + reassemble) that carried requests of the connection so far, and how many of its requests
+ * travelled in a pair shared with other requests (its own or another connection's).  Matched sends of all connections
+ * that stage on one GPU wait in one queue until a test() finds fewer than two launches queued on that GPU, or until
+ * NCCL_FUSELINK_BATCH (default 32, 1 = launch inside isend) of them wait, then go out together. */
 int fl_net_launch_stats(void* comm, int64_t* launches, int64_t* batched_requests);
-/* Chunk -> lane table and header of the last wave a send comm scheduled, copied to host memory
- * (blocks until that wave has run).  rows_out holds up to max_rows flh_chunk_desc entries.
- * Returns the number of rows of that wave. */
+/* Chunk -> lane rows of the connection's latest segment and the header of the launch that carried it, copied to host
+ * memory (launches what waits and blocks until the GPU's queue has run).  rows_out holds up to max_rows
+ * flh_chunk_desc entries.  Returns the number of rows of that segment; FLH_E_STATE if a later launch that did not
+ * carry this connection has reused the table. */
 int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_out);
+/* The last launch pair of the GPU that `comm` stages on: its segments (which connection, which rows of the table, how
+ * many requests, where the connection stood in its credit epoch, where the segment starts in every lane's window),
+ * the whole table and the header.  Returns the number of segments. */
+typedef struct fl_net_launch_seg {
+  int32_t channel;             /* channel id of the connection (src/plugin.cc:693-708) */
+  uint32_t first_row, n_rows;  /* the segment's rows in the launch's table */
+  uint32_t n_req;
+  uint64_t epoch_bytes;        /* bytes of the connection's credit epoch before the segment */
+  uint64_t lane_base[FL_NET_MAX_LANES];
+} fl_net_launch_seg;
+int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, void* rows_out, int max_rows, void* hdr_out);
+/* Launch whatever waits on the GPU that `comm` stages on, without polling a request. */
+int fl_net_flush(void* comm);
 
 #ifdef __cplusplus
 }
