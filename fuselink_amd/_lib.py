@@ -40,7 +40,7 @@ class UniformParams(C.Structure):
     _fields_ = [("total_bytes", C.c_uint64), ("src_base", C.c_uint64), ("epoch_bytes", C.c_uint64),
                 ("chunk_bytes", C.c_uint32), ("n_lanes", C.c_uint32), ("tile_bytes", C.c_uint32), ("pad", C.c_uint32),
                 ("credits", C.c_uint32 * MAX_LANES), ("d_done_word", C.c_void_p), ("d_done_count", C.c_void_p),
-                ("done_value", C.c_uint32), ("pad2", C.c_uint32), ("done_event", C.c_void_p)]
+                ("done_value", C.c_uint32), ("start_value", C.c_uint32), ("done_event", C.c_void_p), ("d_start_word", C.c_void_p)]
 
 
 BATCH_MAX = 32

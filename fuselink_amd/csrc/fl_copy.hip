@@ -249,6 +249,12 @@ struct FusedArgs {
   // every workgroup's stores have been released (counted in *done_count, device memory, zero between launches).
   uint32_t* done_word;
   uint32_t* done_count;
+  // Striping only, may be null: a host-visible word that the launch's first workgroup sets to start_value as it
+  // starts.  A kernel starts once everything queued before it on its stream has finished, so a caller that numbers
+  // its launches learns from the word that all earlier ones are complete.
+  uint32_t* start_word;
+  uint32_t start_value;
+  uint32_t pad_start;
 };
 
 // Several requests in one launch.  Chunk c (counted over the launch) belongs to the request r with
@@ -528,6 +534,8 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   warm_kernel_args(a);
   uint32_t bx = blockIdx.x, by = blockIdx.y;   // tile of the chunk, chunk (in message or destination order)
   xcd_tile_2d(a.xcd_map, bx, by);
+  if (DIR == 0 && a.start_word && bx == 0 && by == 0 && threadIdx.x == 0)
+    __hip_atomic_store(a.start_word, a.start_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   fused_tile<DIR, NT>(a, bx, by);
   // Completion word.  Every workgroup of the grid comes through here, also those without a tile.  The barrier orders
   // the workgroup's stores before thread 0's increment, which releases them at agent scope; the workgroup that counts
@@ -778,6 +786,9 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
   a.done_count = dir == 1 ? u->d_done_count : nullptr;
   a.done_value = u->done_value;
   if (a.done_word && !a.done_count) return fl_set_error(FLH_E_ARG, "d_done_word needs d_done_count");
+  a.start_word = dir == 0 ? u->d_start_word : nullptr;
+  a.start_value = u->start_value;
+  a.pad_start = 0;
   a.total_bytes = u->total_bytes;
   a.src_base = u->src_base;
   a.quanta_before = u->epoch_bytes / u->chunk_bytes;

@@ -56,6 +56,7 @@ sem_t* g_sem = SEM_FAILED;  // the cross-process lock when attached
 int g_shm_fd = -1;
 bool g_owner = false;
 char g_shm_name[64] = "", g_sem_name[64] = "";
+std::atomic<bool> g_attached{false};   // g_sem != SEM_FAILED, readable without the lock
 std::atomic<bool> g_manual_clock{false};
 std::atomic<int64_t> g_manual_now{0};
 // Set when a wait for the semaphore ran into its bound: a process died holding it.  From then on an access only tries
@@ -74,15 +75,13 @@ struct TableLock {
   sem_t* sem = SEM_FAILED;
   bool held = false;
   TableLock() {
-    shared = std::shared_lock<std::shared_mutex>(g_mu);
-    if (g_sem == SEM_FAILED) {          // process-local table: g_mu is its lock
-      shared.unlock();
+    if (!g_attached.load(std::memory_order_acquire)) {   // process-local table: g_mu is its lock
       local = std::unique_lock<std::shared_mutex>(g_mu);
       if (g_sem == SEM_FAILED) return;
       local.unlock();                   // attached meanwhile
-      shared = std::shared_lock<std::shared_mutex>(g_mu);
-      if (g_sem == SEM_FAILED) return;  // and detached again: one unlocked access to single words
     }
+    shared = std::shared_lock<std::shared_mutex>(g_mu);
+    if (g_sem == SEM_FAILED) return;    // detached meanwhile: one unlocked access to single words
     sem = g_sem;
     if (g_sem_dead.load(std::memory_order_acquire)) {
       held = sem_trywait(sem) == 0;
@@ -114,6 +113,7 @@ void detach_locked() {
   g_shm_fd = -1;
   if (g_sem != SEM_FAILED) sem_close(g_sem);
   g_sem = SEM_FAILED;
+  g_attached.store(false, std::memory_order_release);
   if (g_owner) {
     shm_unlink(g_shm_name);
     sem_unlink(g_sem_name);
@@ -148,6 +148,7 @@ int fl_monitor_attach_shm(const char* shm_name, const char* sem_name, int create
   g_tab = (LaneTable*)p;
   g_shm_fd = fd;
   g_sem = sem;
+  g_attached.store(true, std::memory_order_release);
   g_owner = create != 0;
   strcpy(g_shm_name, shm_name);
   strcpy(g_sem_name, sem_name);

@@ -29,6 +29,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <deque>
 #include <map>
 #include <mutex>
@@ -65,14 +66,40 @@ struct Params {
   int batch = FLH_BATCH_MAX;     // matched sends that may wait for one launch (1 = launch inside isend)
   // How a launch's completion reaches `test`: 0 = an event recorded behind every launch (a barrier packet of its
   // own, some 4.5 us in which the stream's next kernel does not start), 1 = the event rides on the launch's last
-  // kernel, 2 = no event and no call into the runtime: the last workgroup of the reassembly kernel to finish stores
-  // the launch's number to a pinned word, after every workgroup's stores have been released (flh_uniform_params).
+  // kernel, 2 = no event and no call into the runtime: pinned words that kernels store launch numbers to
+  // (flh_uniform_params).  Every striping kernel, as it starts, stores its launch's number (the launches before it
+  // are then complete: a stream runs in order); the reassembly kernel of a launch under 8 MiB also stores the number
+  // itself when its last workgroup has finished, after every workgroup's stores have been released, so that a small
+  // launch is seen complete without a successor (in a large launch the per-workgroup release costs more than it
+  // saves).  A large launch that nothing follows gets an event when it is first polled.
   int completion = 2;
   int small_tile = 0;            // copy tile of a launch under 32 MiB (0 = the library's default tile)
+  int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
+  int batch_wait_ns = 3000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
 Params g_par;
 std::mutex g_init_mu;            // ncclIbLock, plugin.cc:84
+
+// NCCL_FUSELINK_TRACE=1: calls and nanoseconds spent inside the entry points and inside the launches they make
+// (fl_net_host_stats).  Off, a probe costs one predictable branch.
+enum : int { kTrIsend = 0, kTrIrecv, kTrTest, kTrTestDone, kTrFlush, kTrLaunch, kTrRequestsLaunched, kTrCount };
+std::atomic<int64_t> g_tr_calls[kTrCount], g_tr_ns[kTrCount];
+inline int64_t tr_now() {
+  timespec t;
+  clock_gettime(CLOCK_MONOTONIC, &t);
+  return (int64_t)t.tv_sec * 1000000000ll + t.tv_nsec;
+}
+struct TraceScope {
+  int what;
+  int64_t t0;
+  explicit TraceScope(int w) : what(w), t0(g_par.trace ? tr_now() : 0) {}
+  ~TraceScope() {
+    if (!t0) return;
+    g_tr_calls[what].fetch_add(1, std::memory_order_relaxed);
+    g_tr_ns[what].fetch_add(tr_now() - t0, std::memory_order_relaxed);
+  }
+};
 bool g_inited = false;
 
 std::mutex g_credit_mu;
@@ -194,13 +221,16 @@ struct Peer {
   uint32_t* d_count = nullptr;      // device word in which a reassembly launch counts its finished workgroups
   int32_t* h_status = nullptr;      // pinned, device-visible: kernels report range refusals here
   int32_t* d_status = nullptr;
-  uint32_t* h_done = nullptr;       // pinned, device-visible: number of the last launch whose reassembly has finished (completion mode 2)
+  uint32_t* h_done = nullptr;       // pinned, device-visible: number of the last launch whose reassembly kernel reported itself finished (completion mode 2)
   uint32_t* d_done = nullptr;
+  uint32_t* h_started = nullptr;    // pinned, device-visible: number of the last launch whose striping kernel has started
+  uint32_t* d_started = nullptr;
   // matched sends that wait for a launch, in arrival order
   std::mutex queue_mu;
   std::vector<Pending> pending;
   std::atomic<uint32_t> waiting_reqs{0};
   std::atomic<uint64_t> waiting_bytes{0};
+  std::atomic<int64_t> waiting_since{0};   // monotonic nanoseconds at which the oldest waiting send arrived
   // Guards every launch on `stream`, the event ring, the launch numbers, the connections' scheduling state
   // (epoch_bytes, launch counters, last table) and `last`.  Taken before queue_mu, never the other way round.
   std::mutex launch_mu;
@@ -385,11 +415,13 @@ ncclResult_t peer_setup(Peer* pr, int device) {
   FL_HIPCHECK(hipMalloc((void**)&pr->d_hdr, sizeof(flh_sched_hdr)));
   FL_HIPCHECK(hipMalloc((void**)&pr->d_count, 256));
   FL_HIPCHECK(hipMemset(pr->d_count, 0, 256));
-  FL_HIPCHECK(hipHostMalloc((void**)&pr->h_status, 128, hipHostMallocMapped));   // status word and completion word, a cache line apart
-  memset(pr->h_status, 0, 128);
+  FL_HIPCHECK(hipHostMalloc((void**)&pr->h_status, 256, hipHostMallocMapped));   // status word and the two completion words, a cache line apart
+  memset(pr->h_status, 0, 256);
   FL_HIPCHECK(hipHostGetDevicePointer((void**)&pr->d_status, pr->h_status, 0));
   pr->h_done = (uint32_t*)((char*)pr->h_status + 64);
   pr->d_done = (uint32_t*)((char*)pr->d_status + 64);
+  pr->h_started = (uint32_t*)((char*)pr->h_status + 128);
+  pr->d_started = (uint32_t*)((char*)pr->d_status + 128);
   pr->ready = true;
   FL_INFO(NCCL_NET, "NET/FuseLink : device %d staging ready: %d lanes x %llu bytes, shared by its connections", device, g_par.lanes, (unsigned long long)cap);
   return ncclSuccess;
@@ -488,6 +520,10 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.small_tile = (int)fl_param("FUSELINK_SMALL_TILE", g_par.small_tile);
   if (g_par.small_tile < 0 || g_par.small_tile % 128) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_SMALL_TILE must be a multiple of 128"); return ncclInvalidArgument; }
   g_par.trace = (int)fl_param("FUSELINK_TRACE", g_par.trace);
+  g_par.batch_wait_ns = (int)fl_param("FUSELINK_BATCH_WAIT_NS", g_par.batch_wait_ns);
+  if (g_par.batch_wait_ns < 0) g_par.batch_wait_ns = 0;
+  g_par.queue_depth = (int)fl_param("FUSELINK_QUEUE_DEPTH", g_par.queue_depth);
+  if (g_par.queue_depth < 1) g_par.queue_depth = 1;
   if (g_par.completion < 0 || g_par.completion > 2) g_par.completion = 2;
   if (g_par.max_wave_chunks > 65535) g_par.max_wave_chunks = 65535;   // what one fused launch can name
   if (g_par.batch < 1) g_par.batch = 1;
@@ -749,11 +785,21 @@ ncclResult_t launch_event(Peer* pr, uint64_t seq, hipEvent_t* out) {
   *out = pr->evring[slot];
   return ncclSuccess;
 }
-ncclResult_t prepare_completion(Peer* pr, uint64_t seq, flh_uniform_params& last_u, Completion& c) {
+// From this many bytes on a launch is bound by the GPU and not by the host's calls around it.
+constexpr uint64_t kEarlyLaunchBytes = 8ull << 20;
+
+void start_stamp(Peer* pr, uint64_t seq, flh_uniform_params& u) {
+  if (g_par.completion != 2) return;
+  u.d_start_word = pr->d_started;
+  u.start_value = (uint32_t)seq;
+}
+ncclResult_t prepare_completion(Peer* pr, uint64_t seq, uint64_t launch_bytes, flh_uniform_params& last_u, Completion& c) {
   if (g_par.completion == 2) {
-    last_u.d_done_word = pr->d_done;
-    last_u.d_done_count = pr->d_count;
-    last_u.done_value = (uint32_t)seq;
+    if (launch_bytes < kEarlyLaunchBytes) {
+      last_u.d_done_word = pr->d_done;
+      last_u.d_done_count = pr->d_count;
+      last_u.done_value = (uint32_t)seq;
+    }
     return ncclSuccess;
   }
   ncclResult_t rc = launch_event(pr, seq, &c.ev);
@@ -804,9 +850,10 @@ ncclResult_t launch_transfer(Peer* pr, const Pending& p, uint64_t seq) {
       // every chunk's lane and window offset itself (and writes the table), the reassembly launch likewise.
       flh_uniform_params u;
       fill_uniform(u, credits, wave, (uint64_t)qoff[q] + done, lk->epoch_bytes, launch_tile(wave));
+      start_stamp(pr, seq, u);
       FL_FLHCHECK(flh_stripe_uniform(p.src, (uint64_t)p.size, &pr->wins, &u, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
       if (q == last_q && done + wave == piece) {
-        ncclResult_t rc = prepare_completion(pr, seq, u, comp);
+        ncclResult_t rc = prepare_completion(pr, seq, wave, u, comp);
         if (rc != ncclSuccess) return rc;
       }
       FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &pr->wins, &u, pr->d_status, pr->stream));
@@ -933,9 +980,10 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, uint64_t
   b.u.tile_bytes = launch_tile(b.u.total_bytes);
   uint64_t seg_base[FLH_SEG_MAX][FLH_MAX_LANES];
   FL_FLHCHECK(flh_batch_layout(&b, nullptr, &seg_base[0][0]));
+  start_stamp(pr, seq, b.u);
   FL_FLHCHECK(flh_stripe_batch(&b, &pr->wins, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
   Completion comp;
-  ncclResult_t rc = prepare_completion(pr, seq, b.u, comp);
+  ncclResult_t rc = prepare_completion(pr, seq, b.u.total_bytes, b.u, comp);
   if (rc != ncclSuccess) return rc;
   FL_FLHCHECK(flh_reassemble_batch(&b, &pr->wins, pr->d_status, pr->stream));
   rc = finish_completion(pr, seq, comp);
@@ -974,9 +1022,11 @@ void flush_pending(Peer* pr) {
     pr->waiting_reqs.store(0, std::memory_order_release);
     pr->waiting_bytes.store(0, std::memory_order_release);
   }
+  TraceScope tr(kTrFlush);
   DeviceScope keep;
   const bool dev_ok = hipSetDevice(pr->hip_device) == hipSuccess;
   std::vector<Pending>& work = pr->work;
+  if (g_par.trace) g_tr_calls[kTrRequestsLaunched].fetch_add((int64_t)work.size(), std::memory_order_relaxed);
   size_t i = 0;
   while (i < work.size()) {
     ncclResult_t rc = dev_ok ? ncclSuccess : ncclUnhandledCudaError;
@@ -997,6 +1047,7 @@ void flush_pending(Peer* pr) {
       } else {
         BatchBuild bb;
         span = build_batch(pr, i, bb);
+        TraceScope trl(kTrLaunch);
         if (span == 0) { span = 1; rc = launch_transfer(pr, p, seq); }   // cannot happen: the request fits an empty set of windows
         else rc = launch_batch(pr, i, span, bb, seq);
       }
@@ -1034,6 +1085,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
   if (c->magic != kCommMagic || !c->is_send || mh->magic != kMhMagic) return ncclInvalidArgument;
   Link* lk = c->link;
   *request = nullptr;
+  TraceScope tr(kTrIsend);
   // The connection's lock covers the descriptor match and the bookkeeping only.  The GPU work is queued
   // after it is dropped: one thread drives a send comm (as NCCL's proxy does), so launches on the
   // connection's stream stay in request order, and the receiver's polling never waits behind a launch.
@@ -1103,12 +1155,18 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
       std::lock_guard<std::mutex> g(pr->queue_mu);
       pr->pending.push_back(p);
       waiting = pr->waiting_reqs.load(std::memory_order_relaxed) + 1;
+      if (waiting == 1 && g_par.batch_wait_ns) pr->waiting_since.store(tr_now(), std::memory_order_relaxed);
       pr->waiting_reqs.store(waiting, std::memory_order_release);
       pr->waiting_bytes.store(pr->waiting_bytes.load(std::memory_order_relaxed) + (uint64_t)size, std::memory_order_release);
     }
     if ((int)waiting >= g_par.batch) {   // a full launch waits (NCCL_FUSELINK_BATCH=1: every send is launched here)
-      std::lock_guard<std::mutex> g(pr->launch_mu);
-      flush_pending(pr);
+      if (g_par.batch < 2) {
+        std::lock_guard<std::mutex> g(pr->launch_mu);
+        flush_pending(pr);
+      } else if (pr->launch_mu.try_lock()) {   // if another thread is launching, the next poll takes care of it
+        flush_pending(pr);
+        pr->launch_mu.unlock();
+      }
     }
   }
   *request = sreq;
@@ -1126,6 +1184,7 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
   if (!mh || mh->magic != kMhMagic || sizes[0] < 0 || !data[0]) return ncclInvalidArgument;
   if (sizes[0] && !in_handle(mh, data[0], (size_t)sizes[0])) { FL_WARN("NET/FuseLink : receive buffer outside its registration"); return ncclInvalidArgument; }
   Link* lk = c->link;
+  TraceScope tr(kTrIrecv);
   std::lock_guard<std::mutex> g(lk->mu);
   bool refreshed = false;
   if (lk->r_finished % g_par.refresh_batch == 0 || !lk->have_decision) {   // plugin.cc:1700
@@ -1178,24 +1237,55 @@ ncclResult_t fl_iflush(void* recvComm, int /*n*/, void** /*data*/, int* /*sizes*
 // Is launch `seq` of the peer complete?  Launches run in order on one stream, so a launch is complete once a later
 // one is.  Mode 2 reads the completion word: a plain load of pinned memory.  Launches whose completion is an event
 // (the other modes, and whatever is not a kernel) are asked through the runtime.
+// Highest launch number that the completion words say is complete: the launch whose reassembly kernel reported itself
+// finished, or the one before the launch whose striping kernel has started, whichever is later.  The acquire loads
+// pair with the kernels' release stores at system scope.
+uint64_t words_complete(Peer* pr) {
+  const uint32_t done = __atomic_load_n(pr->h_done, __ATOMIC_ACQUIRE);
+  const uint32_t started = __atomic_load_n(pr->h_started, __ATOMIC_ACQUIRE);
+  const uint64_t top = pr->launch_seq.load(std::memory_order_acquire);
+  auto lift = [top](uint32_t word) {   // the word holds the low half of a launch number at or below `top`
+    if (word == 0) return (uint64_t)0;
+    uint64_t v = (top & ~0xffffffffull) | word;
+    if (v > top) v = v >= (1ull << 32) ? v - (1ull << 32) : 0;
+    return v;
+  };
+  const uint64_t a = lift(done), b = lift(started);
+  return a > (b ? b - 1 : 0) ? a : (b ? b - 1 : 0);
+}
+
+// Is launch `seq` of the peer complete?  Launches run in order on one stream, so a launch is complete once a later
+// one is.  Mode 2 reads the completion words: plain loads of pinned memory.  Launches whose completion is an event
+// (the other modes, whatever is not a kernel, a large launch that nothing followed) are asked through the runtime.
 ncclResult_t launch_complete(Peer* pr, uint64_t seq, bool* done) {
   *done = false;
   uint64_t seen = pr->done_seq.load(std::memory_order_acquire);
   if (seq <= seen) { *done = true; return ncclSuccess; }
   if (g_par.completion == 2) {
-    // The acquire load pairs with the kernel's release store at system scope: what every workgroup of that launch,
-    // and of the launches before it, wrote is visible to this thread and to whatever it starts afterwards.
-    const uint32_t word = __atomic_load_n(pr->h_done, __ATOMIC_ACQUIRE);
-    const uint64_t top = pr->launch_seq.load(std::memory_order_acquire);
-    uint64_t upto = (top & ~0xffffffffull) | word;   // the word holds the low half of a launch number at or below `top`
-    if (upto > top) upto -= 1ull << 32;
-    if (word != 0 && upto > seen && upto <= top) {
+    const uint64_t upto = words_complete(pr);
+    if (upto > seen) {
       while (seen < upto && !pr->done_seq.compare_exchange_weak(seen, upto, std::memory_order_release, std::memory_order_relaxed)) {}
       if (seq <= upto) { *done = true; return ncclSuccess; }
     }
   }
   const size_t slot = (size_t)((seq - 1) % kEventRing);
-  if (pr->ev_seq[slot].load(std::memory_order_acquire) != seq) return ncclSuccess;   // no event stands for this launch
+  if (pr->ev_seq[slot].load(std::memory_order_acquire) != seq) {
+    // No event stands for this launch.  If it is a large launch of mode 2 and the newest on the stream, nothing will
+    // report it: put an event behind it now (the queue ends there, so the event's packet delays no kernel).
+    if (g_par.completion != 2 || seq != pr->launch_seq.load(std::memory_order_acquire) || !pr->launch_mu.try_lock()) return ncclSuccess;
+    ncclResult_t rc = ncclSuccess;
+    if (seq == pr->launch_seq.load(std::memory_order_relaxed) && pr->ev_seq[slot].load(std::memory_order_relaxed) != seq &&
+        words_complete(pr) < seq) {
+      DeviceScope keep;
+      hipEvent_t ev = nullptr;
+      hipError_t e = hipSetDevice(pr->hip_device);
+      if (e != hipSuccess) rc = hip_fail("hipSetDevice", e);
+      if (rc == ncclSuccess) rc = launch_event(pr, seq, &ev);
+      if (rc == ncclSuccess) { Completion c; c.ev = ev; rc = finish_completion(pr, seq, c); }
+    }
+    pr->launch_mu.unlock();
+    return rc;   // the next poll asks the event (or finds the words)
+  }
   hipError_t e = hipEventQuery(pr->evring[slot]);
   if (e == hipErrorNotReady) return ncclSuccess;
   if (e != hipSuccess) return hip_fail("hipEventQuery", e);
@@ -1210,12 +1300,10 @@ uint64_t launches_in_queue(Peer* pr) {
   uint64_t done = pr->done_seq.load(std::memory_order_acquire);
   const uint64_t top = pr->launch_seq.load(std::memory_order_acquire);
   if (g_par.completion == 2) {
-    const uint32_t word = __atomic_load_n(pr->h_done, __ATOMIC_ACQUIRE);
-    uint64_t upto = (top & ~0xffffffffull) | word;
-    if (upto > top) upto -= 1ull << 32;
-    if (word != 0 && upto > done && upto <= top) done = upto;
+    const uint64_t upto = words_complete(pr);
+    if (upto > done) done = upto;
   }
-  return top - done;
+  return top > done ? top - done : 0;
 }
 
 ncclResult_t fl_test(void* request, int* done, int* sizes) {
@@ -1224,6 +1312,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   if (r->magic != kReqMagic || r->type == kReqUnused) { FL_WARN("NET/FuseLink : test on a request that is not in flight"); return ncclInternalError; }
   *done = 0;
   Link* lk = r->link;
+  TraceScope tr(kTrTest);
   // the request is polled without the connection's lock: only the thread that drives this comm tests its requests
   int st = r->state.load(std::memory_order_acquire);
   if (st == kStPosted || st == 0) return ncclSuccess;   // a receive whose send has not been matched yet
@@ -1237,7 +1326,13 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     // a launch whose completion comes from an event is only known complete once its own requests are polled: it
     // must not hold anything back
     const bool events_out = pr->last_event_seq.load(std::memory_order_acquire) > pr->done_seq.load(std::memory_order_acquire);
-    if (events_out || g_par.completion != 2 || launches_in_queue(pr) < 2) {
+    bool go = events_out || g_par.completion != 2 || launches_in_queue(pr) < (uint64_t)g_par.queue_depth;
+    // small sends wait a moment for company: a launch pair costs the host as much as ten requests do
+    if (go && g_par.batch_wait_ns && pr->waiting_bytes.load(std::memory_order_acquire) < kEarlyLaunchBytes &&
+        pr->waiting_reqs.load(std::memory_order_acquire) < (uint32_t)g_par.batch &&
+        tr_now() - pr->waiting_since.load(std::memory_order_relaxed) < g_par.batch_wait_ns)
+      go = false;
+    if (go) {
       if (pr->launch_mu.try_lock()) {   // if another thread is launching, it or the next poll takes care of it
         flush_pending(pr);
         pr->launch_mu.unlock();
@@ -1251,6 +1346,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     ncclResult_t rc = launch_complete(pr, r->seq, &complete);
     if (rc != ncclSuccess || !complete) return rc;
   }
+  if (g_par.trace) g_tr_calls[kTrTestDone].fetch_add(1, std::memory_order_relaxed);
   std::lock_guard<std::mutex> g(lk->mu);
   ncclResult_t result = ncclSuccess;
   if (r->fault) {   // failed completion, plugin.cc:1839-1861
@@ -1475,6 +1571,14 @@ int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, vo
   if (hdr_out && hipMemcpy(hdr_out, pr->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "header copy failed");
   return (int)li.n_seg;
+}
+
+int fl_net_host_stats(int64_t* calls_out, int64_t* ns_out, int n) {
+  for (int k = 0; k < n && k < kTrCount; ++k) {
+    if (calls_out) calls_out[k] = g_tr_calls[k].load(std::memory_order_relaxed);
+    if (ns_out) ns_out[k] = g_tr_ns[k].load(std::memory_order_relaxed);
+  }
+  return kTrCount;
 }
 
 int fl_net_flush(void* comm) {

@@ -244,12 +244,18 @@ typedef struct flh_uniform_params {
    * reads done_value there with acquire semantics may use the destination buffer.  Launches that share a count word
    * must be ordered (one stream).
    * done_event: a hipEvent_t that the launch's kernel completes (hipEventQuery then answers for the kernel), which
-   * spares the separate packet of a hipEventRecord behind it. */
+   * spares the separate packet of a hipEventRecord behind it.
+   * d_start_word (striping / gather side only): a host-visible word to which the launch's first workgroup stores
+   * start_value as it starts.  Work on a stream runs in order, each kernel after everything before it has finished
+   * and its results are visible on the device, so a caller that numbers its launches learns from the word that all
+   * launches before this one are complete.  The cheapest of the three: one store per launch, but it only says so once
+   * a later launch has begun. */
   uint32_t* d_done_word;
   uint32_t* d_done_count;
   uint32_t done_value;
-  uint32_t pad2;
+  uint32_t start_value;
   void* done_event;
+  uint32_t* d_start_word;
 } flh_uniform_params;
 
 int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows* win,

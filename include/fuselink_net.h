@@ -256,6 +256,11 @@ typedef struct fl_net_launch_seg {
   uint64_t lane_base[FL_NET_MAX_LANES];
 } fl_net_launch_seg;
 int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, void* rows_out, int max_rows, void* hdr_out);
+/* Where the host's time goes (collected only under NCCL_FUSELINK_TRACE=1; process-wide sums over all threads): calls
+ * and nanoseconds, index 0 isend, 1 irecv, 2 test, 3 tests that completed a request (calls only), 4 passes that
+ * launched what waited, 5 launch pairs (time inside the runtime's launch calls and the batch arithmetic before them),
+ * 6 requests those passes launched (calls only).  Returns the number of counters. */
+int fl_net_host_stats(int64_t* calls_out, int64_t* ns_out, int n);
 /* Launch whatever waits on the GPU that `comm` stages on, without polling a request. */
 int fl_net_flush(void* comm);
 

@@ -5,7 +5,9 @@
 //
 //   plugin_harness <lib.so> [--bytes N] [--request N] [--inflight K] [--iters I] [--host] [--version 6|7|8] [--connections C]
 //                  [--handoff batch,blocks_per_req,layers,kv_heads,block_size,head_dim]
-// With --connections C, C connections run concurrently, each with its own pair of proxy threads and buffers.
+// With --connections C, C connections run concurrently, each with its own pair of proxy threads and buffers; every
+// iteration starts on all of them together and is timed from the first start to the last finish, and the received
+// buffers are compared only once all connections have finished it.
 // With --handoff the message is the prefill -> decode hand-off of the reference's serving experiment
 // (FuseLink experiments/serving/model.hh:280-309): one group of five sends on one connection -- the context output
 // (int64 per request), the K cache, the V cache, the block table (int64 per request and block) and the allocated-block
@@ -39,8 +41,24 @@ static void logger(ncclDebugLogLevel level, unsigned long, const char* file, int
 #define CHECK(x) do { ncclResult_t r_ = (x); if (r_ != ncclSuccess) { fprintf(stderr, "%s -> ncclResult %d (line %d)\n", #x, (int)r_, __LINE__); exit(2); } } while (0)
 #define HIP(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { fprintf(stderr, "%s -> %s\n", #x, hipGetErrorString(e_)); exit(3); } } while (0)
 
+// all connections meet here before and after the transfers of an iteration
+struct Barrier {
+  std::atomic<int> arrived{0}, generation{0};
+  int parties = 1;
+  void wait() {
+    const int gen = generation.load(std::memory_order_acquire);
+    if (arrived.fetch_add(1, std::memory_order_acq_rel) + 1 == parties) {
+      arrived.store(0, std::memory_order_relaxed);
+      generation.store(gen + 1, std::memory_order_release);
+    } else {
+      while (generation.load(std::memory_order_acquire) == gen) std::this_thread::yield();
+    }
+  }
+};
+typedef std::chrono::steady_clock::time_point TimePoint;
+
 static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclNet_v6_t* net6, const std::vector<size_t>& sizes, size_t request, int inflight,
-                           int iters, int host, int version, double* best_out, double* total_out) {
+                           int iters, int host, int version, Barrier* barrier, TimePoint* starts, TimePoint* ends) {
   if (!host) HIP(hipSetDevice(0));
   const int dev = ci % 2;  // spread the connections over two virtual NICs
   char handle[NCCL_NET_HANDLE_MAXSIZE];
@@ -83,10 +101,10 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
     for (size_t off = 0; off < msgs[m].bytes; off += request)
       pieces.push_back({(int)m, off, (int)(msgs[m].bytes - off < request ? msgs[m].bytes - off : request)});
   const size_t n_req = pieces.size();
-  double best = 1e30, total = 0;
   for (int it = 0; it < iters; ++it) {
     std::atomic<size_t> posted{0};
-    auto t0 = std::chrono::steady_clock::now();
+    barrier->wait();
+    starts[it] = std::chrono::steady_clock::now();
     std::thread receiver([&]() {
       if (!host) (void)hipSetDevice(0);
       std::deque<void*> q;
@@ -131,9 +149,8 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
     });
     sender.join();
     receiver.join();
-    double s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-    total += s;
-    if (s < best) best = s;
+    ends[it] = std::chrono::steady_clock::now();
+    barrier->wait();
     for (size_t m = 0; m < msgs.size(); ++m) {
       Msg& g = msgs[m];
       std::vector<uint8_t> back(g.bytes);
@@ -151,8 +168,6 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
   CHECK(net8->closeListen(lcomm));
   for (Msg& g : msgs) { if (host) { free(g.src); free(g.dst); } else { HIP(hipFree(g.src)); HIP(hipFree(g.dst)); } }
   (void)bytes;
-  *best_out = best;
-  *total_out = total / iters;
 }
 
 int main(int argc, char** argv) {
@@ -198,12 +213,22 @@ int main(int argc, char** argv) {
   int ndev = 0;
   CHECK(net8->devices(&ndev));
 
-  std::vector<double> bests(connections, 1e30), totals(connections, 0.0);
+  Barrier barrier;
+  barrier.parties = connections;
+  std::vector<std::vector<TimePoint>> starts(connections, std::vector<TimePoint>(iters)), ends(connections, std::vector<TimePoint>(iters));
   std::vector<std::thread> conns;
-  for (int ci = 0; ci < connections; ++ci) conns.emplace_back([&, ci]() { run_connection(ci, net8, net7, net6, sizes, request, inflight, iters, host, version, &bests[ci], &totals[ci]); });
+  for (int ci = 0; ci < connections; ++ci)
+    conns.emplace_back([&, ci]() { run_connection(ci, net8, net7, net6, sizes, request, inflight, iters, host, version, &barrier, starts[ci].data(), ends[ci].data()); });
   for (auto& t : conns) t.join();
-  double best = 0, total = 0;
-  for (int ci = 0; ci < connections; ++ci) { if (bests[ci] > best) best = bests[ci]; total += totals[ci] / connections; }
+  // an iteration lasts from the first connection's start to the last connection's finish
+  double best = 1e30, total = 0;
+  for (int it = 0; it < iters; ++it) {
+    TimePoint first = starts[0][it], last = ends[0][it];
+    for (int ci = 1; ci < connections; ++ci) { if (starts[ci][it] < first) first = starts[ci][it]; if (ends[ci][it] > last) last = ends[ci][it]; }
+    const double sec = std::chrono::duration<double>(last - first).count();
+    if (sec < best) best = sec;
+    total += sec / iters;
+  }
   size_t n_req = 0;
   for (size_t b : sizes) n_req += (b + request - 1) / request;
   if (handoff)
@@ -213,5 +238,19 @@ int main(int argc, char** argv) {
   printf("{\"harness\": \"plugin\", \"name\": \"%s\", \"devices\": %d, \"memory\": \"%s\", \"bytes\": %zu, \"request_bytes\": %zu, \"requests\": %zu, "
          "\"inflight\": %d, \"iters\": %d, \"connections\": %d, \"best_s\": %.9f, \"mean_s\": %.9f, \"GBps_4N_best\": %.1f, \"bit_exact\": true}\n",
          net8->name, ndev, host ? "host" : "device", bytes, request, n_req, inflight, iters, connections, best, total, 4.0 * bytes * connections / best / 1e9);
+  // NCCL_FUSELINK_TRACE=1: where the host's time went, summed over all proxy threads
+  typedef int (*host_stats_fn)(int64_t*, int64_t*, int);
+  host_stats_fn host_stats = (host_stats_fn)dlsym(lib, "fl_net_host_stats");
+  const char* tr = getenv("NCCL_FUSELINK_TRACE");
+  if (host_stats && tr && atoi(tr) > 0) {
+    int64_t calls[8] = {0}, ns[8] = {0};
+    host_stats(calls, ns, 8);
+    const double reqs = (double)n_req * connections * iters;
+    printf("{\"harness\": \"host_trace\", \"requests\": %.0f, \"isend_calls\": %lld, \"isend_us\": %.1f, \"irecv_calls\": %lld, \"irecv_us\": %.1f, "
+           "\"test_calls\": %lld, \"test_us\": %.1f, \"tests_done\": %lld, \"flush_passes\": %lld, \"flush_us\": %.1f, \"launch_pairs\": %lld, \"launch_us\": %.1f, "
+           "\"requests_per_launch\": %.2f, \"launch_us_per_pair\": %.2f}\n",
+           reqs, (long long)calls[0], ns[0] / 1e3, (long long)calls[1], ns[1] / 1e3, (long long)calls[2], ns[2] / 1e3, (long long)calls[3],
+           (long long)calls[4], ns[4] / 1e3, (long long)calls[5], ns[5] / 1e3, calls[5] ? (double)calls[6] / calls[5] : 0.0, calls[5] ? ns[5] / 1e3 / calls[5] : 0.0);
+  }
   return 0;
 }

@@ -513,6 +513,107 @@ def test_batch_of_requests_is_one_message(fl, seed):
         assert not got[sizes[q]:].any()
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_batch_of_segments_equals_the_oracle_segment_by_segment(fl, seed):
+    """flh_stripe_batch / flh_reassemble_batch with several segments: each segment is scheduled as the message its requests
+    form, from its own epoch prefix under its own credit row, and the segments follow each other in the windows at 128-byte
+    boundaries.  Rows, header, flh_batch_layout, the staged bytes and every destination against the oracle."""
+    core, torch = fl
+    rng = np.random.default_rng(8800 + seed)
+    lanes = int(rng.integers(1, 17))
+    chunk = int(rng.choice([4096, 65536, 256 << 10, 100 * 128]))
+    n_seg = int(rng.integers(1, 9))
+    segments, sizes = [], []
+    for k in range(n_seg):
+        room = 32 - len(sizes) - (n_seg - 1 - k)
+        n_req = int(rng.integers(1, max(2, min(6, room + 1))))
+        ss = [int(rng.integers(1, 4)) * chunk for _ in range(n_req)]
+        if rng.random() < 0.6:
+            ss[-1] -= int(rng.integers(1, chunk))            # a segment's last request may end inside a chunk
+        credits = rng.integers(0, 9, size=lanes).astype(np.uint32)
+        if seed == 3 and k == 0:
+            credits[:] = 0                                   # no credit anywhere: the static policy stands in
+        segments.append((n_req, credits, int(rng.integers(0, 50)) * chunk))
+        sizes += ss
+    srcs_np = [rng.integers(0, 256, size=s, dtype=np.uint8) for s in sizes]
+    srcs = [_dev(torch, a) for a in srcs_np]
+    dsts = [torch.zeros(s + 64, dtype=torch.uint8, device="cuda") for s in sizes]
+    b = core.batch_params(srcs, dsts, chunk, [1] * lanes, segments=[(n, c.tolist(), e) for n, c, e in segments])
+    # the oracle, segment by segment; windows as the layout rule says
+    lane_end = np.zeros(16, dtype=np.uint64)
+    exp_rows, exp_bases, staged = [], [], {}
+    lane_bytes_sum, lane_chunks_sum, flags, first_row, q = np.zeros(16, np.uint64), np.zeros(16, np.uint32), 0, 0, 0
+    tiles_per_chunk = (chunk + 32767) // 32768
+    total_tiles = 0
+    for n_req, credits, epoch in segments:
+        seg_np = np.concatenate(srcs_np[q:q + n_req])
+        q += n_req
+        st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+        st["epoch_bytes"] = epoch
+        exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=seg_np.size, chunk_bytes=chunk,
+                                             mode=ob.SCHED_RESET_OFFSETS, state=st)
+        base = (lane_end + np.uint64(127)) // np.uint64(128) * np.uint64(128)
+        exp_bases.append(base.copy())
+        wins_seg = ob.cpu_stripe(seg_np, exp_t, [int(x) for x in exp_h["lane_bytes"][:lanes]])
+        for l in range(lanes):
+            n = int(exp_h["lane_bytes"][l])
+            if n:
+                staged[(len(exp_rows), l)] = (int(base[l]), wins_seg[l][:n])
+        rows = exp_t.copy()
+        rows["win_off"] += base[rows["lane"]]
+        rows["tile_base"] += first_row * tiles_per_chunk
+        exp_rows.append(rows)
+        used = exp_h["lane_chunks"] > 0
+        lane_end[used] = base[used] + exp_h["lane_bytes"][used]
+        lane_bytes_sum += exp_h["lane_bytes"]
+        lane_chunks_sum += exp_h["lane_chunks"]
+        flags |= int(exp_h["flags"])
+        total_tiles += int(exp_h["total_tiles"])
+        first_row += len(exp_t)
+    exp_t = np.concatenate(exp_rows)
+    ends, bases = core.batch_layout(b)
+    np.testing.assert_array_equal(np.array(ends, dtype=np.uint64), lane_end)
+    for k in range(n_seg):
+        np.testing.assert_array_equal(np.array(bases[k], dtype=np.uint64), exp_bases[k], err_msg=f"segment {k} bases")
+    caps = [int(x) for x in lane_end[:lanes]]
+    wins = [torch.zeros(max(c, 1) + 64, dtype=torch.uint8, device="cuda") for c in caps]
+    w = core.make_windows([t.data_ptr() for t in wins], caps)
+    status = core.new_status()
+    out = core.new_schedule_buffers(len(exp_t))
+    core.stripe_batch(b, w, status, out=out)
+    core.reassemble_batch(b, w, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    got_t, got_h = out.table_numpy(), out.hdr_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got_t[f], exp_t[f], err_msg=f)
+    np.testing.assert_array_equal(got_h["lane_bytes"], lane_bytes_sum)
+    np.testing.assert_array_equal(got_h["lane_chunks"], lane_chunks_sum)
+    assert int(got_h["total_bytes"]) == sum(sizes) and int(got_h["n_chunks"]) == len(exp_t)
+    assert int(got_h["flags"]) == flags and int(got_h["total_tiles"]) == total_tiles
+    for (k, l), (off, data) in staged.items():
+        np.testing.assert_array_equal(wins[l].cpu().numpy()[off:off + data.size], data, err_msg=f"segment {k} lane {l}")
+    for i, s in enumerate(sizes):
+        got = dsts[i].cpu().numpy()
+        np.testing.assert_array_equal(got[:s], srcs_np[i])
+        assert not got[s:].any()
+
+
+def test_batch_refuses_segments_that_do_not_add_up(fl):
+    core, torch = fl
+    chunk = 4096
+    srcs = [torch.zeros(chunk, dtype=torch.uint8, device="cuda") for _ in range(3)]
+    dsts = [torch.zeros_like(t) for t in srcs]
+    wins = [torch.zeros(8 * chunk, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    w = core.make_windows([t.data_ptr() for t in wins], [8 * chunk] * 2)
+    b = core.batch_params(srcs, dsts, chunk, [1, 1], segments=[(1, [1, 1], 0), (1, [1, 0], 0)])
+    with pytest.raises(Exception, match="segments hold 2 requests"):
+        core.stripe_batch(b, w, core.new_status())
+    b = core.batch_params(srcs, dsts, chunk, [1, 1], segments=[(2, [1, 1], 0), (2, [1, 0], 0)])
+    with pytest.raises(Exception, match="are left"):
+        core.stripe_batch(b, w, core.new_status())
+
+
 def test_batch_refuses_a_request_that_ends_inside_a_chunk(fl):
     core, torch = fl
     chunk = 4096

@@ -506,6 +506,157 @@ def test_sends_that_wait_together_travel_as_one_message(net):
     net.reconfigure(NCCL_FUSELINK_BATCH=None)
 
 
+def _open(net, dev, src, dst):
+    lcomm, s, r = net.connect_pair(dev)
+    rc, smh = net.regMr(s, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA)
+    assert rc == 0
+    rc, rmh = net.regMr(r, dst.data_ptr(), dst.numel(), P.NCCL_PTR_CUDA)
+    assert rc == 0
+    return dict(l=lcomm, s=s, r=r, smh=smh, rmh=rmh, src=src, dst=dst)
+
+
+def _close(net, c):
+    assert net.deregMr(c["s"], c["smh"]) == 0 and net.deregMr(c["r"], c["rmh"]) == 0
+    net.closeSend(c["s"]), net.closeRecv(c["r"]), net.closeListen(c["l"])
+
+
+def test_requests_of_four_connections_share_one_launch_pair(net):
+    """NCCL's shape: four channels to a peer, eight requests in flight on each (experiments/bw_test/run_bw_test.sbatch:39-44;
+    src/fuselink.h:14), all sharing the lanes (src/fuselink.h:271-272).  The 32 matched sends go out as ONE launch pair of
+    four segments; every segment's rows are the oracle's table for that connection's message -- its own credit row, its own
+    place in its credit epoch -- shifted to where the earlier segments left each lane's window, and every byte arrives."""
+    import torch
+    chunk, piece, n_conn, per_conn = 64 << 10, 128 << 10, 4, 8
+    net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_BATCH=32)
+    rng = np.random.default_rng(4242)
+    rows = [[3, 1, 0, 2, 5, 1, 1, 4], [1, 1, 1, 1, 1, 1, 1, 1], [0, 0, 7, 0, 0, 0, 0, 0], [2, 0, 2, 0, 2, 0, 2, 9]]
+    conns = []
+    for k in range(n_conn):
+        src_np = rng.integers(0, 256, size=(per_conn + 1) * piece, dtype=np.uint8)
+        c = _open(net, k % 8, torch.from_numpy(src_np).cuda(), torch.zeros((per_conn + 1) * piece, dtype=torch.uint8, device="cuda"))
+        c["src_np"] = src_np
+        net.set_credits(rows[k])           # the row this connection's receiver advertises at its first refresh
+        _send_recv(net, c["s"], c["r"], c["src"], c["dst"], piece, 99, c["smh"], c["rmh"], src_off=per_conn * piece, dst_off=per_conn * piece)
+        conns.append(c)
+    rreqs, sreqs = [], []
+    for c in conns:
+        for q in range(per_conn):
+            rc, req = net.irecv(c["r"], [c["dst"].data_ptr() + q * piece], [piece], [q], [c["rmh"]])
+            assert rc == 0 and req
+            rreqs.append(req)
+    for c in conns:                        # the 32nd send fills the launch: it goes out inside that isend
+        for q in range(per_conn):
+            rc, req = net.isend(c["s"], c["src"].data_ptr() + q * piece, piece, q, c["smh"])
+            assert rc == 0 and req
+            sreqs.append(req)
+    segs, got, hdr = net.last_launch(conns[0]["s"])
+    assert len(segs) == n_conn and [s["n_req"] for s in segs] == [per_conn] * n_conn
+    tiles_per_chunk = chunk // 32768
+    lane_end = np.zeros(16, dtype=np.uint64)
+    lane_bytes_sum = np.zeros(16, dtype=np.uint64)
+    first_row = 0
+    for k, sg in enumerate(segs):
+        exp_t, exp_h, _ = ob.credit_schedule(n_lanes=8, credits=rows[k], quantum=chunk, total_bytes=per_conn * piece, chunk_bytes=chunk,
+                                             mode=ob.SCHED_RESET_OFFSETS, state=_state(piece, 0))
+        assert sg["first_row"] == first_row and sg["n_rows"] == len(exp_t) and sg["epoch_bytes"] == piece
+        base = (lane_end + np.uint64(127)) // np.uint64(128) * np.uint64(128)    # where the earlier segments left every lane, 128-byte aligned
+        np.testing.assert_array_equal(np.array(sg["lane_base"], dtype=np.uint64), base)
+        mine = got[first_row:first_row + len(exp_t)]
+        for f in ("src_off", "len", "lane", "epoch"):
+            np.testing.assert_array_equal(mine[f], exp_t[f], err_msg=f"segment {k}: {f}")
+        np.testing.assert_array_equal(mine["win_off"], exp_t["win_off"] + base[exp_t["lane"]], err_msg=f"segment {k}: win_off")
+        np.testing.assert_array_equal(mine["tile_base"], exp_t["tile_base"] + first_row * tiles_per_chunk, err_msg=f"segment {k}: tile_base")
+        used = exp_h["lane_chunks"] > 0
+        lane_end[used] = base[used] + exp_h["lane_bytes"][used]
+        lane_bytes_sum += exp_h["lane_bytes"]
+        first_row += len(exp_t)
+    np.testing.assert_array_equal(hdr["lane_bytes"], lane_bytes_sum)
+    assert int(hdr["n_chunks"]) == first_row and int(hdr["total_bytes"]) == n_conn * per_conn * piece
+    for q in sreqs:
+        net.wait(q)
+    for q in rreqs:
+        assert net.wait(q) == piece
+    for c in conns:
+        np.testing.assert_array_equal(c["dst"].cpu().numpy(), c["src_np"])
+        assert net.launch_stats(c["s"]) == {"launches": 2, "batched_requests": per_conn}
+        _close(net, c)
+
+
+def test_interleaved_connections_fill_launches_segment_by_segment(net):
+    """Sends of three connections arriving in turn: every send opens a segment (the connection changes), eight segments fill a
+    launch, and a connection's later segments carry on from where its earlier ones of the same launch left its epoch."""
+    import torch
+    chunk = 32 << 10
+    net.reconfigure(NCCL_FUSELINK_LANES=5, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_BATCH=32, NCCL_FUSELINK_REFRESH_BATCH=64)
+    net.set_credits([2, 1, 0, 3, 1])
+    rng = np.random.default_rng(515)
+    n_conn, per_conn = 3, 7
+    sizes = [[int(rng.integers(1, 5)) * chunk - (int(rng.integers(1, chunk)) if rng.random() < 0.4 else 0) for _ in range(per_conn)] for _ in range(n_conn)]
+    conns = []
+    for k in range(n_conn):
+        total = sum(sizes[k]) + chunk
+        src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
+        c = _open(net, k, torch.from_numpy(src_np).cuda(), torch.zeros(total, dtype=torch.uint8, device="cuda"))
+        c["src_np"] = src_np
+        _send_recv(net, c["s"], c["r"], c["src"], c["dst"], chunk, 99, c["smh"], c["rmh"], src_off=sum(sizes[k]), dst_off=sum(sizes[k]))
+        conns.append(c)
+    rreqs, sreqs = [], []
+    for q in range(per_conn):
+        for k, c in enumerate(conns):
+            off = sum(sizes[k][:q])
+            rc, req = net.irecv(c["r"], [c["dst"].data_ptr() + off], [sizes[k][q]], [q], [c["rmh"]])
+            assert rc == 0 and req
+            rreqs.append((req, sizes[k][q]))
+    for q in range(per_conn):
+        for k, c in enumerate(conns):
+            off = sum(sizes[k][:q])
+            rc, req = net.isend(c["s"], c["src"].data_ptr() + off, sizes[k][q], q, c["smh"])
+            assert rc == 0 and req
+            sreqs.append(req)
+    net.flush(conns[0]["s"])
+    segs, got, hdr = net.last_launch(conns[0]["s"])
+    assert 1 <= len(segs) <= 8
+    for q in sreqs:
+        net.wait(q)
+    for q, n in rreqs:
+        assert net.wait(q) == n
+    launches = 0
+    for c in conns:
+        np.testing.assert_array_equal(c["dst"].cpu().numpy(), c["src_np"])
+        launches = max(launches, net.launch_stats(c["s"])["launches"])
+        _close(net, c)
+    assert launches <= 1 + 3      # 21 sends, eight segments to a launch: three launches behind the warm-up
+
+
+def test_more_connections_than_a_pool_of_their_own_windows_would_allow(net):
+    """Every connection that stages on a GPU shares that GPU's lane windows (src/fuselink.h:271-272), so the number of
+    connections is not bounded by the unit pool: twelve connections at 8 lanes x 4 units would need 384 units of the
+    reference's 256 (src/cumem.cu:9) if each bound its own."""
+    import torch
+    net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=64 << 10)
+    rng = np.random.default_rng(12)
+    size = 1 << 20
+    conns = []
+    for k in range(12):
+        src_np = rng.integers(0, 256, size=size, dtype=np.uint8)
+        c = _open(net, k % 8, torch.from_numpy(src_np).cuda(), torch.zeros(size, dtype=torch.uint8, device="cuda"))
+        c["src_np"] = src_np
+        conns.append(c)
+    reqs = []
+    for k, c in enumerate(conns):
+        rc, rreq = net.irecv(c["r"], [c["dst"].data_ptr()], [size], [k], [c["rmh"]])
+        assert rc == 0 and rreq
+        rc, sreq = net.isend(c["s"], c["src"].data_ptr(), size, k, c["smh"])
+        assert rc == 0 and sreq
+        reqs.append((sreq, rreq))
+    for sreq, rreq in reqs:
+        net.wait(sreq)
+        assert net.wait(rreq) == size
+    for c in conns:
+        np.testing.assert_array_equal(c["dst"].cpu().numpy(), c["src_np"])
+        _close(net, c)
+
+
 @pytest.mark.parametrize("block", range(4))
 def test_random_request_streams(net, block):
     """Seeded random connections: lanes, chunk size, batching, refresh cadence, window size, QP split, policy,
