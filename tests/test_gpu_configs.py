@@ -385,6 +385,49 @@ def test_paged_gather_ragged_and_bad_page(fl):
 
 
 # ---- stress: 1 GiB, 64 KiB chunks, 16 lanes, credits redrawn every 1000 chunks -----------------------------------
+def test_cfg2_fused_pair_stages_the_oracles_windows(fl):
+    """The bench's default path at its full size: 64 MiB fp16 N(0,1), 256 KiB chunks, 8 lanes, credits seeded in [1,8],
+    through flh_stripe_uniform / flh_reassemble_uniform.  All eight staging windows byte for byte against the oracle's
+    host-memcpy windows, the table and header the striping launch writes against the oracle's, the reassembled buffer
+    against the source."""
+    core, torch = fl
+    rng = np.random.default_rng(2)
+    total, chunk, lanes = 64 << 20, 256 << 10, 8
+    credits = rng.integers(1, 9, size=lanes).astype(np.uint32)
+    src_np = rng.standard_normal(total // 2, dtype=np.float32).astype(np.float16).view(np.uint8)
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk,
+                                         mode=ob.SCHED_RESET_OFFSETS)
+    lane_bytes = [int(b) for b in exp_h["lane_bytes"][:lanes]]
+    exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+    pool = core.Pool(0, sum((b + 2 * MB - 1) // (2 * MB) for b in lane_bytes))
+    wins = []
+    for b in lane_bytes:
+        w = core.Window(pool, b)
+        w.bind(b)
+        wins.append(w)
+    win = core.make_windows([w.base for w in wins], [w.bound_bytes for w in wins])
+    src = _dev(torch, src_np)
+    dst = torch.zeros_like(src)
+    u = core.uniform_params(total, chunk, credits.tolist())
+    out = core.new_schedule_buffers(len(exp_t))
+    status = core.new_status()
+    core.stripe_uniform(src, win, u, status, out=out)
+    core.reassemble_uniform(dst, win, u, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    assert out.table_numpy().tobytes() == exp_t.tobytes()
+    got_h = out.hdr_numpy()
+    for f in ("total_bytes", "total_tiles", "n_chunks", "flags", "uniform_tiles", "lane_bytes", "lane_chunks"):
+        np.testing.assert_array_equal(got_h[f], exp_h[f], err_msg=f)
+    for l in range(lanes):
+        got = core.read_window(wins[l].base, lane_bytes[l]).cpu().numpy()
+        assert got.tobytes() == exp_w[l][: lane_bytes[l]].tobytes(), f"staging window {l} differs from the host-memcpy window"
+    assert torch.equal(src, dst)
+    for w in wins:
+        w.destroy()
+    pool.destroy()
+
+
 def test_cfg5_stress_full_size(fl):
     core, torch = fl
     rng = np.random.default_rng(5)

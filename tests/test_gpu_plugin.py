@@ -506,6 +506,86 @@ def test_sends_that_wait_together_travel_as_one_message(net):
     net.reconfigure(NCCL_FUSELINK_BATCH=None)
 
 
+def test_cfg5_stress_as_the_plugin_is_driven(net):
+    """The stress configuration in the shape a communication library drives it: 1 GiB of uint32 as 16 384 requests of one
+    64 KiB chunk each, 4 outstanding, 16 lanes, the lane decision refreshed every 1000 requests with credits redrawn at
+    every refresh, 4 staging units per lane reused by every launch.  At two refresh boundaries the rows of the
+    connection's latest launch are compared with the oracle's table for the same carried state: the last launch of an
+    epoch (prefix = everything the epoch has scheduled) and the first of the next (prefix 0, new credit row)."""
+    import torch
+    chunk, lanes, refresh, n_req, inflight_max = 64 << 10, 16, 1000, 16384, 4
+    net.reconfigure(NCCL_FUSELINK_LANES=lanes, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_REFRESH_BATCH=refresh,
+                    NCCL_FUSELINK_WINDOW_UNITS=4)
+    rng = np.random.default_rng(5)
+    rows = rng.integers(1, 9, size=(n_req // refresh + 2, lanes))
+    total = n_req * chunk
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    src = torch.randint(0, 2**31 - 1, (total // 4,), dtype=torch.int32, device="cuda", generator=gen).view(torch.uint8)
+    dst = torch.zeros_like(src)
+    c = _open(net, 0, src, dst)
+    s, r = c["s"], c["r"]
+    net.set_credits([int(x) for x in rows[0]])
+    posted = sent = done_r = done_s = 0
+    epoch = -1                       # credit epochs seen so far - 1 = index of the row in force
+    sent_in_epoch = 0
+    rq, sq = [], []
+    checked = []
+    spins = 0
+    while done_r < n_req or done_s < n_req:
+        spins += 1
+        assert spins < 3_000_000, "no progress"
+        # The reference's gate refreshes only when a receive is posted while the completion count stands on a multiple of
+        # the cadence and nothing is outstanding (src/plugin.cc:1700-1712), so the driver drains before every 1000th post.
+        if posted < n_req and posted - done_r < inflight_max and (posted % refresh != 0 or done_r == posted):
+            rc, q = net.irecv(r, [dst.data_ptr() + posted * chunk], [chunk], [posted & 0xffff], [c["rmh"]])
+            assert rc == 0
+            if q:
+                if posted % refresh == 0:      # this receive refreshed the lane decision: the next refresh draws the next row
+                    assert net.comm_stats(r)["refreshes"] == posted // refresh + 1
+                    net.set_credits([int(x) for x in rows[posted // refresh + 1]])
+                rq.append(q)
+                posted += 1
+        if sent < posted:
+            rc, q = net.isend(s, src.data_ptr() + sent * chunk, chunk, sent & 0xffff, c["smh"])
+            assert rc == 0
+            if q:
+                if sent % refresh == 0:
+                    epoch, sent_in_epoch = epoch + 1, 0
+                sq.append(q)
+                sent += 1
+                sent_in_epoch += 1
+                # the last send of epoch 2 and the first of epoch 3; the last of epoch 9 and the first of epoch 10
+                if sent in (3 * refresh, 3 * refresh + 1, 10 * refresh, 10 * refresh + 1):
+                    got, hdr = net.last_table(s)
+                    n = got.size
+                    assert 1 <= n <= inflight_max
+                    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=rows[epoch], quantum=chunk, total_bytes=n * chunk, chunk_bytes=chunk,
+                                                         mode=ob.SCHED_RESET_OFFSETS, state=_state((sent_in_epoch - n) * chunk, 0))
+                    _same_table(got, exp_t)
+                    np.testing.assert_array_equal(hdr["lane_bytes"], exp_h["lane_bytes"])
+                    checked.append((sent, epoch, n))
+        if rq:
+            rc, d, sz = net.test(rq[0])
+            assert rc == 0
+            if d:
+                assert sz == chunk
+                rq.pop(0)
+                done_r += 1
+        if sq:
+            rc, d, _ = net.test(sq[0])
+            assert rc == 0
+            if d:
+                sq.pop(0)
+                done_s += 1
+    assert [x[0] for x in checked] == [3 * refresh, 3 * refresh + 1, 10 * refresh, 10 * refresh + 1]
+    assert checked[1][2] == 1 and checked[3][2] == 1      # a refresh admits one receive at a time: the epoch's first launch carries one request
+    assert net.comm_stats(r)["refreshes"] == (n_req + refresh - 1) // refresh
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+    _close(net, c)
+
+
 def _open(net, dev, src, dst):
     lcomm, s, r = net.connect_pair(dev)
     rc, smh = net.regMr(s, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA)
