@@ -65,9 +65,20 @@ def main() -> int:
     ap.add_argument("--path", default="auto", choices=["auto", "fused", "split"],
                     help="fused: scheduler folded into the striping launch (uniform split, one credit row); split: three launches")
     ap.add_argument("--lds", type=int, default=0, help="paged workload: stage the gather through LDS")
-    ap.add_argument("--cold-user-buffers", action="store_true",
+    ap.add_argument("--cold-user-buffers", type=int, default=1,
                     help="also time the step over source/destination pairs in rotation (1 GiB), so that no user buffer is "
-                         "cache-resident; off by default so that a kernel trace of the default run holds the timed loop's launches only")
+                         "cache-resident (fused uniform workloads up to 128 MiB); it runs after the timed loop and the per-kernel "
+                         "passes, so a kernel trace of the run holds the timed loop's launches first; 0 = skip")
+    ap.add_argument("--scheduler-bench", type=int, default=1,
+                    help="also time the scheduler kernels on the stress configuration's chunk list (16384 chunks, 16 lanes, 17 credit "
+                         "rows, epochs of 1000): closed form, scan on one workgroup, scan on a workgroup per 1024 chunks; 0 = skip")
+    ap.add_argument("--plugin-bench", type=int, default=1,
+                    help="also move the headline message through the plugin ABI in the shape a communication library drives it "
+                         "(tests/harness/plugin_harness as a child process, started before this process touches the GPU): "
+                         "128 requests of 512 KiB, 8 in flight, one connection and four; 0 = skip")
+    ap.add_argument("--ragged", action="store_true",
+                    help="blocks workload: add 1..15 bytes to every block, so that no chunk is a multiple of 16 bytes and source and "
+                         "window offsets are misaligned against each other")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="set a library tunable (flh_tune) before the run, e.g. --tune copy_rows_per_wg=1; repeatable")
     ap.add_argument("--blocks", type=int, default=256,
@@ -92,6 +103,34 @@ def main() -> int:
         print("bench.py: this build runs on exactly one GPU (every lane's staging window lives on it); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         return 2
+
+    # ---- the plugin ABI, driven as a communication library drives it: a child process, before this one uses the GPU ----
+    plugin = None
+    if args.plugin_bench and args.workload.startswith("cfg2"):
+        import subprocess
+
+        from fuselink_amd import build as flbuild
+        harness = os.path.join(ROOT, "tests", "harness", "plugin_harness")
+        if os.path.exists(harness) and os.path.exists(flbuild.lib_path()):
+            env = dict(os.environ, NCCL_FUSELINK_LANES="8", NCCL_FUSELINK_CHUNKSIZE=str(256 << 10))
+            plugin = {"message_bytes": 64 << 20, "request_bytes": 512 << 10, "requests": 128, "inflight": 8, "lanes": 8, "chunk_bytes": 256 << 10,
+                      "accounting": "4 x bytes x connections / wall time of the best of 20 iterations, proxy threads started inside the timed region",
+                      "env": "NCCL_FUSELINK_LANES=8 NCCL_FUSELINK_CHUNKSIZE=262144"}
+            for conns in (1, 4):
+                cmd = [harness, flbuild.lib_path(), "--bytes", str(64 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "20",
+                       "--connections", str(conns)]
+                try:
+                    res = subprocess.run(cmd, capture_output=True, text=True, timeout=120, env=env)
+                    line = json.loads(res.stdout.strip().splitlines()[-1]) if res.returncode == 0 else None
+                except Exception:
+                    line = None
+                key = f"connections_{conns}"
+                if line and line.get("bit_exact"):
+                    plugin[key] = {"GBps_4N": line["GBps_4N_best"], "best_s": line["best_s"], "mean_s": line["mean_s"], "bit_exact": True,
+                                   "us_per_request": round(line["best_s"] * 1e6 / (128 * conns), 3)}
+                else:
+                    plugin[key] = None
+                plugin[key + "_command"] = " ".join(os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd)
 
     import numpy as np
     import torch
@@ -122,6 +161,8 @@ def main() -> int:
         p = ranks ** -1.1
         rows_per_block = rng.choice(np.arange(1, max_rows + 1), size=args.blocks, p=p / p.sum())
         sizes_np = (rows_per_block * 7168 * 2).astype(np.uint32)
+        if args.ragged:
+            sizes_np += rng.integers(1, 16, size=args.blocks).astype(np.uint32)
         nbytes = int(sizes_np.sum())
         credits_np = np.array([[4, 4, 4, 4, 4, 4, 4, 1]], dtype=np.int32)   # one lane at 25 % idleness
         n_chunks = args.blocks
@@ -134,7 +175,7 @@ def main() -> int:
     elif kind == "uniform":
         src = torch.randint(0, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device=dev, generator=gen).view(torch.uint8)
     else:
-        src = torch.randint(-32768, 32767, (nbytes // 2,), dtype=torch.int16, device=dev, generator=gen).view(torch.uint8)
+        src = torch.randint(-32768, 32767, ((nbytes + 1) // 2,), dtype=torch.int16, device=dev, generator=gen).view(torch.uint8)[:nbytes]
     dst = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
     sizes = torch.from_numpy(sizes_np.view(np.int32)).to(dev) if sizes_np is not None else None
     page_bytes, ppc = 32768, 4
@@ -351,6 +392,7 @@ def main() -> int:
     # beside `value`, never as `value`.
     cold = None
     if args.cold_user_buffers and fused and kind == "uniform" and nbytes <= (128 << 20):
+        cold_cmd = "python bench.py" + ("" if args.workload.startswith("cfg2") else f" --workload {args.workload}")
         pairs = max(2, (1 << 30) // (2 * nbytes))
         srcs = [src] + [torch.randint(0, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device=dev, generator=gen).view(torch.uint8)
                         for _ in range(pairs - 1)]
@@ -373,8 +415,42 @@ def main() -> int:
         cold = {"value": round(algo_bytes_cold(nbytes) / (cold_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "ms_per_step": round(cold_ms, 5),
                 "pairs": pairs, "user_buffer_bytes": 2 * pairs * nbytes,
                 "kernels_us": {"stripe": round(mean(per_c["stripe"]), 2), "reassemble": round(mean(per_c["reassemble"]), 2)},
-                "note": "same step, source/destination pairs in rotation so that no user buffer is cache-resident; windows reused"}
+                "pct_of_hbm_peak": round(100.0 * algo_bytes_cold(nbytes) / (cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                "note": "same step, source/destination pairs in rotation so that no user buffer is cache-resident; windows reused",
+                "command": cold_cmd}
         del srcs, dsts
+
+    # ---- the scheduler kernels on a list long enough for a per-1000-chunk rate: the stress configuration's ----
+    sched_bench = None
+    if args.scheduler_bench:
+        sb_n, sb_lanes, sb_rows, sb_epoch, sb_chunk = 16384, 16, 17, 1000, 64 << 10
+        sb_credits = torch.from_numpy(rng.integers(1, 9, size=(sb_rows, sb_lanes)).astype(np.int32)).to(dev)
+        sb_sizes_np = rng.integers(1, 2 * sb_chunk, size=sb_n).astype(np.uint32)      # variable sizes: the scan has to run
+        sb_sizes = torch.from_numpy(sb_sizes_np.view(np.int32)).to(dev)
+        reps = 50
+
+        def sb_run(label, **kw):
+            out_s = core.schedule(n_lanes=sb_lanes, credits=sb_credits, epoch_len=sb_epoch, stream=stream, **kw)   # buffers, untimed
+            stream.synchronize()
+
+            def go():
+                for _ in range(reps):
+                    core.schedule(n_lanes=sb_lanes, credits=sb_credits, epoch_len=sb_epoch, stream=stream, out=out_s, **kw)
+
+            go()
+            us = profiled(go, 4 * reps)["schedule"]
+            launches = len(us) // reps
+            per_call = sum(us) / reps
+            return {"us_per_call": round(per_call, 2), "launches_per_call": launches, "us_per_1k_chunks": round(per_call / (sb_n / 1000.0), 3)}
+
+        sched_bench = {
+            "chunks": sb_n, "lanes": sb_lanes, "credit_rows": sb_rows, "epoch_len": sb_epoch,
+            "closed_form_uniform_64KiB": sb_run("closed", quantum=sb_chunk, total_bytes=sb_n * sb_chunk, chunk_bytes=sb_chunk),
+            "scan_variable_sizes_one_workgroup": sb_run("scan1", quantum=sb_chunk, sizes=sb_sizes),
+            "scan_variable_sizes_workgroup_per_1024_chunks": sb_run("scanN", quantum=sb_chunk, sizes=sb_sizes, workspace=True),
+            "timing": "HIP events around every scheduler launch, summed per call, mean of 50 calls back to back",
+            "command": "python bench.py",
+        }
 
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
     algo_bytes_kernel = 2 * msg_bytes // len(waves or cwaves or twaves or (0,))    # one launch of the copy kernel (with waves: the average one)
@@ -427,8 +503,13 @@ def main() -> int:
         "scheduler_kernel": "standalone launch, not part of the fused step" if (fused or cwaves) else "first launch of every message",
         # one launch schedules a whole message; below 1000 chunks its cost is the flat launch time, not a per-1k rate
         "scheduler_launch_us": round(sched_us, 2),
-        "scheduler_us_per_1k_chunks": round(sched_us * n_sched / (n_chunks / 1000.0), 3) if n_chunks >= 1000 else None,
+        # the rate on a list long enough to have one: the stress configuration's 16384 chunks through the prefix-scan kernels
+        # (a workgroup per 1024 chunks); the other scheduler shapes are in scheduler_bench
+        "scheduler_us_per_1k_chunks": (sched_bench["scan_variable_sizes_workgroup_per_1024_chunks"]["us_per_1k_chunks"] if sched_bench else
+                                       round(sched_us * n_sched / (n_chunks / 1000.0), 3) if n_chunks >= 1000 else None),
+        "scheduler_bench": sched_bench,
         "cold_user_buffers": cold,
+        "plugin_abi": plugin,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": (MEASURED_TRAFFIC.get(f"{args.workload}/{len(cwaves)} waves") if cwaves else None if (waves or twaves) else

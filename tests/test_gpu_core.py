@@ -256,6 +256,35 @@ def test_roundtrip_odd_sizes_misaligned_windows(fl):
     np.testing.assert_array_equal(out, src)
 
 
+@pytest.mark.parametrize("tile", [4096, 32768])
+def test_every_pair_of_misalignments_and_the_edges_of_the_vector_loop(fl, tile):
+    """Source and window misaligned against each other in every combination of the two residues mod 16, with copy
+    lengths around everything the shifted copy treats specially: fewer bytes than a vector, a head only, whole
+    wavefronts of vectors +- 1 (the last lane takes its second source vector by a load of its own), the unrolled
+    block +- 1, a tile +- 1.  One lane, so the window offsets are the running sum of the sizes; explicit source offsets
+    choose the source residue.  Windows and reassembled buffer against the oracle's host memcpy."""
+    rng = np.random.default_rng(1600 + tile)
+    edge = [1, 2, 15, 16, 17, 31, 32, 33, 63 * 16, 64 * 16, 64 * 16 + 5, 65 * 16 + 9, 255 * 16 + 1, 256 * 16, 257 * 16 + 3,
+            2047 * 16 + 7, 2048 * 16, 2048 * 16 + 1, 2049 * 16 + 15, tile - 1, tile, tile + 1, 3 * tile + 11]
+    sizes, src_off, at = [], [], 0
+    for sres in range(16):
+        for dres in range(16):
+            n = int(edge[(sres * 16 + dres) % len(edge)]) if rng.random() < 0.7 else int(rng.integers(1, 70000))
+            # the window stands at residue (sum of the sizes so far) mod 16; steer it to dres with a small filler chunk
+            filler = (dres - sum(sizes)) % 16
+            if filler:
+                sizes.append(filler)
+                src_off.append(at)
+                at += filler + 16
+            at = (at + 15) // 16 * 16 + sres          # the chunk's bytes start at residue sres in the user buffer
+            sizes.append(n)
+            src_off.append(at)
+            at += n + 3
+    src = rng.integers(0, 256, size=at + 64, dtype=np.uint8)
+    _roundtrip(fl, src, n_lanes=1, credits=[1], quantum=32768, sizes=np.array(sizes, dtype=np.uint32), tile_bytes=tile,
+               src_off=np.array(src_off, dtype=np.uint64))
+
+
 def test_empty_message(fl):
     core, torch = fl
     sched, _, exp_h = _check_schedule(fl, n_lanes=4, credits=[1, 1, 1, 1], quantum=4096, total_bytes=0, chunk_bytes=4096)
