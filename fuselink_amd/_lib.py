@@ -84,6 +84,13 @@ SIGNATURES = {
     "flh_window_export_dmabuf": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.POINTER(C.c_int)]),
     "flh_stripe_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_reassemble_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p]),
+    "flh_engine_create": (C.c_int, [C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_void_p)]),
+    "flh_engine_submit": (C.c_int, [C.c_void_p, C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_uint64),
+                                    C.POINTER(C.c_uint64)]),
+    "flh_engine_completed": (C.c_uint64, [C.c_void_p]),
+    "flh_engine_error": (C.c_int, [C.c_void_p]),
+    "flh_engine_launches": (C.c_uint64, [C.c_void_p]),
+    "flh_engine_destroy": (C.c_int, [C.c_void_p]),
     "flh_batch_layout": (C.c_int, [C.POINTER(BatchParams), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "flh_gather_pages": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(Windows),
                                    C.c_void_p, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p]),

@@ -6,6 +6,7 @@
 //   * fl_plain_copy         : calibration copy with the same inner loop
 // The path is an HBM-bound byte mover; nothing here contracts, so no MFMA.
 #include <cstring>
+#include <new>
 
 #include "fl_closed_form.h"
 #include "fl_device.h"
@@ -698,6 +699,225 @@ __global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const 
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// lane engine: a resident kernel that executes batch descriptors
+// ------------------------------------------------------------------------------------------------
+// Launching a stripe + reassemble pair costs the host about ten microseconds, which bounds the request rate at NCCL's
+// 512 KiB steps.  The engine takes the launches off that path: the host writes the descriptor of a batch -- the very
+// argument block the batch kernels take -- into a ring in pinned memory and advances a tail word; one workgroup of the
+// resident kernel (the dispatcher) polls the tail, copies new descriptors into device memory and publishes them, and
+// the other workgroups (the workers) run every batch's tiles through the same routine the launched kernels run
+// (fused_tile): first the striping of their tiles, then the reassembly of the same tiles, so that a tile is read back
+// by the workgroup that staged it and no workgroup waits for another inside a batch.  A batch's tiles go to the
+// workers in turn, starting behind the worker that took the last tile of the batch before, so that small batches
+// run side by side on different workers.  Successive batches rotate through the caller's sets of staging windows,
+// and a worker enters batch k only once every worker has left batch k - sets.  The last worker to leave a batch stores its number to a host-visible word.
+// Every wait in the kernel is bounded: with nothing to do for idle_us the dispatcher takes the engine down (the host
+// starts it again with the next batch), and a wait that outlasts wait_us reports an error and takes it down as well.
+constexpr uint32_t kEngineDevRing = 8;          // descriptors held in device memory; also the most window sets a caller may rotate
+constexpr uint32_t kEngineDescBytes = 4096;
+// A worker takes this many neighbouring copy tiles at a time.  Every worker with a share in a batch pays for an acquire
+// and a release of that batch, so fewer, larger shares serve the engine better than one 32 KiB tile each: 4 MiB batches
+// took 12.8 us with shares of 32 KiB, 9.1 us with 64 KiB, 9.2 us with 128 KiB (16 MiB batches: 22.4, 20.0, 35.7 us).
+constexpr uint32_t kEngineShare = 2;
+
+struct EngineDesc {                              // what the host writes per batch (kEngineDescBytes at most)
+  uint32_t tiles;                                // worker shares of the batch (the slot's first word: the dispatcher's thread 0 has it in hand)
+  uint32_t pad[3];
+  FusedBatchArgs a;                              // as the striping launch would take it (req_user = sources)
+  uint8_t* req_dst[FLH_BATCH_MAX];               // the reassembly side's buffers
+};
+static_assert(sizeof(EngineDesc) <= kEngineDescBytes, "descriptor slot too small");
+
+struct EngineHostCtl {                           // pinned host memory, mapped to the device; one 64-byte line per word
+  alignas(64) uint64_t tail;                     // host: batches submitted so far
+  alignas(64) uint32_t state;                    // 0 down, 1 running, 2 about to go down (device; the host sets 1 when it launches)
+  alignas(64) uint64_t exited_at;                // device: the batch the next engine has to start with
+  alignas(64) uint64_t done;                     // device: batches complete
+  alignas(64) int32_t error;                     // device: a bounded wait ran out (FLH_E_STATE)
+  alignas(64) uint32_t stop;                     // host: go down now
+};
+struct EngineDevCtl {                            // device memory
+  // per ring slot: low half of the number of the batch whose descriptor the slot holds << 32 | the worker that takes
+  // the batch's first share << 20 | its shares; a worker learns from the one word that its batch is there and
+  // which of its shares, if any, are its own
+  alignas(64) uint64_t published[kEngineDevRing];
+  alignas(64) uint32_t quit;                     // workers leave when they reach batch quit_at
+  uint32_t pad;
+  uint64_t quit_at;
+  alignas(64) uint64_t arrive[kEngineDevRing];   // workers that have left the batches of each ring slot, never reset
+};
+struct EngineArgs {
+  const uint8_t* host_ring;                      // kHostRing descriptors, device-visible pinned memory
+  uint32_t host_slots;
+  uint32_t workers;
+  uint32_t sets;                                 // the caller rotates this many window sets: batch k waits for batch k - sets
+  uint32_t pad;
+  EngineHostCtl* hctl;
+  uint8_t* dev_ring;
+  EngineDevCtl* dctl;
+  uint64_t start;                                // first batch to execute
+  uint64_t idle_ticks, wait_ticks;               // of the 100 MHz wall clock
+};
+
+__device__ __forceinline__ void engine_fail(const EngineArgs& e) {
+  __hip_atomic_store(&e.hctl->error, (int32_t)FLH_E_STATE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __hip_atomic_store(&e.dctl->quit_at, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&e.dctl->quit, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
+  __shared__ EngineDesc d;
+  __shared__ uint32_t sh_flag, sh_first;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t W = e.workers;
+  if (blockIdx.x == 0) {
+    // ---- dispatcher ------------------------------------------------------------------------------------------
+    uint64_t k = e.start;
+    uint64_t tail_seen = e.start;   // the host's tail as last read: a burst of batches costs one look across the bus
+    uint32_t first_worker = 0;      // takes the first tile of batch k
+    uint64_t idle_since = wall_clock64(), free_since = idle_since;
+    for (;;) {
+      if (tid == 0) {
+        uint32_t act = 0;   // 0 poll again, 1 copy descriptor k, 2 leave
+        const uint64_t now = wall_clock64();
+        // the device slot of batch k held batch k - ring: every worker must have left that one
+        const uint64_t need = (k / kEngineDevRing) * W;
+        if (__hip_atomic_load(&e.dctl->arrive[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= need) {
+          free_since = now;
+          if (tail_seen <= k) tail_seen = __hip_atomic_load(&e.hctl->tail, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
+          if (tail_seen > k) act = 1;
+        } else if (now - free_since > e.wait_ticks) {
+          engine_fail(e);   // the workers never left the batch that holds the slot
+        }
+        if (act == 1) {
+          idle_since = now;
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the workers' reads of the slot are behind their arrival
+        } else if (__hip_atomic_load(&e.hctl->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) ||
+                   __hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+          act = 2;
+        } else if (now - idle_since > e.idle_ticks) {
+          // Nothing for a while: announce it, then look once more.  The host stores the tail, then reads the state; this
+          // side stores the state, then reads the tail: one of the two sees the other's store.
+          __hip_atomic_store(&e.hctl->state, 2u, __ATOMIC_SEQ_CST, __HIP_MEMORY_SCOPE_SYSTEM);
+          __atomic_thread_fence(__ATOMIC_SEQ_CST);
+          const uint64_t tail = __hip_atomic_load(&e.hctl->tail, __ATOMIC_SEQ_CST, __HIP_MEMORY_SCOPE_SYSTEM);
+          if (tail > k) {
+            __hip_atomic_store(&e.hctl->state, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+            idle_since = now;
+          } else {
+            act = 2;
+          }
+        }
+        sh_flag = act;
+      }
+      __syncthreads();
+      const uint32_t act = sh_flag;
+      __syncthreads();
+      if (act == 2) break;
+      if (act == 0) { __builtin_amdgcn_s_sleep(8); continue; }
+      // descriptor k: pinned host memory -> device ring, sixteen bytes per thread
+      const u32x4* src = (const u32x4*)(e.host_ring + (size_t)(k % e.host_slots) * kEngineDescBytes);
+      u32x4* dst = (u32x4*)(e.dev_ring + (size_t)(k % kEngineDevRing) * kEngineDescBytes);
+      static_assert(kEngineDescBytes == kCopyBlock * 16, "one vector per thread moves a descriptor");
+      const u32x4 v = src[tid];
+      dst[tid] = v;
+      __syncthreads();
+      if (tid == 0) {
+        const uint32_t tiles = v.x < 0xfffffu ? v.x : 0xfffffu;   // EngineDesc::tiles
+        __hip_atomic_store(&e.dctl->published[k % kEngineDevRing], ((uint64_t)(uint32_t)(k + 1) << 32) | ((uint64_t)first_worker << 20) | tiles,
+                           __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        first_worker = (first_worker + tiles) % W;
+      }
+      ++k;
+    }
+    if (tid == 0) {
+      // workers finish what has been published and leave at batch k; the next engine starts there
+      if (!__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+        __hip_atomic_store(&e.dctl->quit_at, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&e.dctl->quit, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __hip_atomic_store(&e.hctl->exited_at, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(&e.hctl->state, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    return;
+  }
+  // ---- worker ----------------------------------------------------------------------------------------------
+  const uint32_t w = blockIdx.x - 1;
+  for (uint64_t k = e.start;; ++k) {
+    if (tid == 0) {
+      uint32_t act = 1;   // 1 run batch k, 2 leave, 3 no tile of batch k is this worker's
+      uint64_t word = 0;
+      const uint64_t t0 = wall_clock64();
+      for (uint32_t spin = 0;; ++spin) {
+        word = __hip_atomic_load(&e.dctl->published[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // the fence below acquires
+        if ((uint32_t)(word >> 32) == (uint32_t)(k + 1)) break;
+        if ((spin & 7) == 7) {   // the flag and the clock now and then: every look is a round trip to memory
+          if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) &&
+              __hip_atomic_load(&e.dctl->quit_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <= k) { act = 2; break; }
+          if (wall_clock64() - t0 > e.wait_ticks + e.idle_ticks) { engine_fail(e); act = 2; break; }
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      // this worker's first tile of the batch: the tiles go round the workers from the batch's first worker on
+      const uint32_t first = (uint32_t)(word >> 20) & 0xfffu;
+      sh_first = (w + W - first) % W;
+      if (act == 1 && sh_first >= (uint32_t)(word & 0xfffffu)) act = 3;
+      if (act == 1 && k >= e.sets) {
+        // batch k reuses the windows of batch k - sets: every worker must have left that one
+        const uint64_t j = k - e.sets;
+        const uint64_t need = (j / kEngineDevRing + 1) * W;
+        const uint64_t t1 = wall_clock64();
+        while (__hip_atomic_load(&e.dctl->arrive[j % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+          if (wall_clock64() - t1 > e.wait_ticks) { engine_fail(e); act = 2; break; }
+          __builtin_amdgcn_s_sleep(1);
+        }
+      }
+      sh_flag = act;
+    }
+    __syncthreads();
+    const uint32_t act = sh_flag, mine = sh_first;
+    __syncthreads();
+    if (act == 2) return;
+    uint64_t* cnt = &e.dctl->arrive[k % kEngineDevRing];
+    if (act == 3) {
+      // nothing read, nothing written: the worker only has to be counted (the last one to leave publishes the batch)
+      if (tid == 0) {
+        const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (before + 1 == (k / kEngineDevRing + 1) * W)
+          __hip_atomic_store(&e.hctl->done, k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+      continue;
+    }
+    // what the batch reads may have been written by anyone, on this GPU or off it, before the host submitted it
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    {
+      const u32x4* src = (const u32x4*)(e.dev_ring + (size_t)(k % kEngineDevRing) * kEngineDescBytes);
+      u32x4* dst = (u32x4*)&d;
+      if (tid * 16 < sizeof(EngineDesc)) dst[tid] = src[tid];
+    }
+    __syncthreads();
+    const uint32_t tpc = d.a.tiles_per_chunk;
+    const uint32_t total = tpc * d.a.n_chunks;
+    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W)                           // this worker's tiles, user buffers -> windows
+      for (uint32_t t = sh * kEngineShare; t < total && t < (sh + 1) * kEngineShare; ++t) fused_tile<0, 0>(d.a, t % tpc, t / tpc);
+    __syncthreads();
+    if (tid < FLH_BATCH_MAX) d.a.req_user[tid] = d.req_dst[tid];                          // the same tiles, windows -> receive buffers
+    if (tid == 0) { d.a.table = nullptr; d.a.hdr = nullptr; }
+    __syncthreads();
+    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W)
+      for (uint32_t t = sh * kEngineShare; t < total && t < (sh + 1) * kEngineShare; ++t) fused_tile<1, 0>(d.a, t % tpc, t / tpc);
+    __syncthreads();
+    if (tid == 0) {
+      // leaving the batch releases this worker's stores; the last one to leave has thereby acquired everybody's and
+      // publishes the batch to the host
+      const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_SYSTEM);
+      if (before + 1 == (k / kEngineDevRing + 1) * W)
+        __hip_atomic_store(&e.hctl->done, k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
+}
+
 }  // namespace
 
 // One launch per (direction, streaming mode) pair that the policy can ask for: striping / gathering with modes
@@ -1132,6 +1352,166 @@ int flh_scatter_pages(void* d_pool, uint64_t pool_pages, const uint32_t* d_page_
                       uint32_t pages_per_chunk, const flh_windows* win, const flh_chunk_desc* d_table, uint32_t n_chunks,
                       int use_lds, int32_t* d_status, void* stream) {
   return launch_pages(1, d_pool, pool_pages, d_page_table, page_bytes, pages_per_chunk, win, d_table, n_chunks, use_lds, d_status, stream);
+}
+
+// ---- lane engine, host side ---------------------------------------------------------------------------------
+struct flh_engine {
+  int device;
+  uint32_t workers;
+  uint32_t host_slots;
+  uint32_t sets;
+  hipStream_t stream;
+  uint8_t* h_ring;          // pinned, mapped
+  uint8_t* d_ring_host;     // the same ring as the device addresses it
+  EngineHostCtl* h_ctl;
+  EngineHostCtl* d_ctl_host;
+  uint8_t* dev_ring;
+  EngineDevCtl* dctl;
+  uint64_t submitted;       // batches written into the ring
+  uint64_t launches;        // engine kernels started
+  uint64_t idle_us, wait_us;
+};
+
+int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_t window_sets, flh_engine** out) {
+  if (!out) return fl_set_error(FLH_E_ARG, "null out pointer");
+  *out = nullptr;
+  int rc = fl_need_init();
+  if (rc) return rc;
+  // Half as many workers as compute units by default.  Every worker that has a tile in a batch pays for an acquire and a
+  // release of that batch, which is what bounds small batches; 128 workers moved 4 MiB batches at 1.3 TB/s and 16 MiB
+  // batches at 3.0 TB/s (4 x bytes), 255 workers at 1.1 and 2.5, 64 at 1.45 and 2.1.
+  if (workgroups == 0) workgroups = (uint32_t)g_cus / 2 + 1;
+  if (window_sets < 1 || window_sets > kEngineDevRing) return fl_set_error(FLH_E_ARG, "an engine rotates 1..%u window sets, not %u", kEngineDevRing, window_sets);
+  if (workgroups < 2 || workgroups > 1024) return fl_set_error(FLH_E_ARG, "an engine takes 2..1024 workgroups (a dispatcher and workers), not %u", workgroups);
+  flh_engine* e = new (std::nothrow) flh_engine();
+  if (!e) return fl_set_error(FLH_E_HIP, "out of host memory");
+  memset(e, 0, sizeof(*e));
+  e->device = device;
+  e->workers = workgroups - 1;
+  e->sets = window_sets;
+  e->host_slots = 64;
+  e->idle_us = idle_us ? idle_us : 200;
+  e->wait_us = 2000000;
+  FL_HIP(hipSetDevice(device));
+  FL_HIP(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
+  FL_HIP(hipHostMalloc((void**)&e->h_ring, (size_t)e->host_slots * kEngineDescBytes, hipHostMallocMapped));
+  FL_HIP(hipHostGetDevicePointer((void**)&e->d_ring_host, e->h_ring, 0));
+  FL_HIP(hipHostMalloc((void**)&e->h_ctl, sizeof(EngineHostCtl), hipHostMallocMapped));
+  memset(e->h_ctl, 0, sizeof(EngineHostCtl));
+  FL_HIP(hipHostGetDevicePointer((void**)&e->d_ctl_host, e->h_ctl, 0));
+  FL_HIP(hipMalloc((void**)&e->dev_ring, (size_t)kEngineDevRing * kEngineDescBytes));
+  FL_HIP(hipMalloc((void**)&e->dctl, sizeof(EngineDevCtl)));
+  FL_HIP(hipMemset(e->dctl, 0, sizeof(EngineDevCtl)));
+  *out = e;
+  return FLH_OK;
+}
+
+// start the resident kernel with the batch the last one stopped at (the stream orders it behind that one's exit)
+static int engine_start(flh_engine* e) {
+  EngineArgs a;
+  a.host_ring = e->d_ring_host;
+  a.host_slots = e->host_slots;
+  a.workers = e->workers;
+  a.sets = e->sets;
+  a.pad = 0;
+  a.hctl = e->d_ctl_host;
+  a.dev_ring = e->dev_ring;
+  a.dctl = e->dctl;
+  a.start = __atomic_load_n(&e->h_ctl->exited_at, __ATOMIC_ACQUIRE);
+  a.idle_ticks = e->idle_us * 100;     // the wall clock counts at 100 MHz
+  a.wait_ticks = e->wait_us * 100;
+  __atomic_store_n(&e->h_ctl->state, 1u, __ATOMIC_RELEASE);
+  FL_HIP(hipMemsetAsync(&e->dctl->quit, 0, sizeof(uint32_t), e->stream));
+  hipLaunchKernelGGL(fl_engine_kernel, dim3(e->workers + 1), dim3(kCopyBlock), 0, e->stream, a);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    __atomic_store_n(&e->h_ctl->state, 0u, __ATOMIC_RELEASE);
+    return fl_set_error(FLH_E_HIP, "engine launch failed: %s", hipGetErrorString(err));
+  }
+  e->launches++;
+  return FLH_OK;
+}
+
+int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
+                      flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out) {
+  if (!e || !seq_out) return fl_set_error(FLH_E_ARG, "null engine or sequence pointer");
+  if (__atomic_load_n(&e->h_ctl->error, __ATOMIC_ACQUIRE)) return fl_set_error(FLH_E_STATE, "the engine went down on a wait that ran out");
+  // the ring slot must be free: its last occupant complete
+  const uint64_t seq = e->submitted;
+  if (seq >= e->host_slots && __atomic_load_n(&e->h_ctl->done, __ATOMIC_ACQUIRE) + e->host_slots <= seq)
+    return fl_set_error(FLH_E_NOMEM, "the engine's descriptor ring is full (%u batches in flight)", e->host_slots);
+  BatchPlan pl;
+  int rc = plan_batch(b, pl);
+  if (rc) return rc;
+  if (seg_base_out) memcpy(seg_base_out, pl.seg_base, sizeof(pl.seg_base));
+  EngineDesc* d = (EngineDesc*)(e->h_ring + (size_t)(seq % e->host_slots) * kEngineDescBytes);
+  flh_uniform_params u = b->u;
+  u.total_bytes = (uint64_t)pl.n_chunks * b->u.chunk_bytes;
+  u.epoch_bytes = 0;
+  u.d_done_word = nullptr;
+  u.d_start_word = nullptr;
+  u.done_event = nullptr;
+  FusedBatchArgs a;
+  rc = fill_fused(a, 0, win, &u, d_table_out, d_hdr_out, d_status);
+  if (rc) return rc < 0 ? rc : fl_set_error(FLH_E_ARG, "empty batch");
+  a.total_bytes = b->u.total_bytes;
+  a.dest_order = 0;
+  a.src_base = 0;
+  a.xcd_map = 0;                        // the engine's workers take tiles by their own stride
+  a.n_req = b->n_req;
+  a.n_seg = pl.n_seg;
+  uint8_t* dsts[FLH_BATCH_MAX];
+  for (uint32_t q = 0; q < FLH_BATCH_MAX; ++q) {
+    a.first[q] = pl.first[q];
+    a.seg_of[q] = pl.seg_of[q];
+    a.req_user[q] = nullptr;
+    a.req_bytes[q] = 0;
+    dsts[q] = nullptr;
+    if (q >= b->n_req) continue;
+    if (!b->d_src[q] || !b->d_dst[q]) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer", q);
+    a.req_user[q] = (uint8_t*)b->d_src[q];
+    a.req_bytes[q] = b->bytes[q];
+    dsts[q] = (uint8_t*)b->d_dst[q];
+  }
+  for (uint32_t k = 0; k < FLH_SEG_MAX; ++k) a.seg[k] = pl.seg[k];
+  memcpy(&d->a, &a, sizeof(a));
+  memcpy(d->req_dst, dsts, sizeof(dsts));
+  d->tiles = (a.n_chunks * a.tiles_per_chunk + kEngineShare - 1) / kEngineShare;
+  e->submitted = seq + 1;
+  *seq_out = seq + 1;
+  // The tail goes out, then the state is read; the dispatcher stores the state, then reads the tail: one of the two
+  // sees the other's store, so a batch is never left behind by an engine that is going down.
+  __atomic_store_n(&e->h_ctl->tail, seq + 1, __ATOMIC_SEQ_CST);
+  __atomic_thread_fence(__ATOMIC_SEQ_CST);
+  uint32_t st = __atomic_load_n(&e->h_ctl->state, __ATOMIC_SEQ_CST);
+  for (int spin = 0; st == 2 && spin < 4000000; ++spin) st = __atomic_load_n(&e->h_ctl->state, __ATOMIC_ACQUIRE);   // it decides within microseconds
+  if (st == 2) return fl_set_error(FLH_E_STATE, "the engine did not finish going down");
+  if (st == 0) return engine_start(e);
+  return FLH_OK;
+}
+
+uint64_t flh_engine_completed(const flh_engine* e) {
+  return e ? __atomic_load_n(&e->h_ctl->done, __ATOMIC_ACQUIRE) : 0;
+}
+
+int flh_engine_error(const flh_engine* e) {
+  return e ? __atomic_load_n(&e->h_ctl->error, __ATOMIC_ACQUIRE) : FLH_E_ARG;
+}
+
+uint64_t flh_engine_launches(const flh_engine* e) { return e ? e->launches : 0; }
+
+int flh_engine_destroy(flh_engine* e) {
+  if (!e) return FLH_OK;
+  (void)hipSetDevice(e->device);
+  __atomic_store_n(&e->h_ctl->stop, 1u, __ATOMIC_RELEASE);
+  if (e->stream) (void)hipStreamSynchronize(e->stream);   // the dispatcher sees the flag within a poll
+  if (e->h_ring) (void)hipHostFree(e->h_ring);
+  if (e->h_ctl) (void)hipHostFree(e->h_ctl);
+  if (e->dev_ring) (void)hipFree(e->dev_ring);
+  if (e->dctl) (void)hipFree(e->dctl);
+  if (e->stream) (void)hipStreamDestroy(e->stream);
+  delete e;
+  return FLH_OK;
 }
 
 int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {

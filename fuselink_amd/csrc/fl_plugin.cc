@@ -50,6 +50,7 @@ ncclDebugLogger_t g_log = nullptr;
 #define FL_WARN(...) do { if (g_log) g_log(NCCL_LOG_WARN, NCCL_ALL, __FILE__, __LINE__, __VA_ARGS__); } while (0)
 #define FL_INFO(flags, ...) do { if (g_log) g_log(NCCL_LOG_INFO, (flags), __FILE__, __LINE__, __VA_ARGS__); } while (0)
 
+constexpr int kEngineSetsMax = 8;
 struct Params {
   int lanes = 8;                 // virtual NICs = staging lanes (the experiment uses 8 HCAs, run_bw_test.sbatch:43)
   int priority_dev = 0;          // NCCL_FUSELINK_PRIORITY_DEV, plugin.cc:117
@@ -74,8 +75,16 @@ struct Params {
   // saves).  A large launch that nothing follows gets an event when it is first polled.
   int completion = 2;
   int small_tile = 0;            // copy tile of a launch under 32 MiB (0 = the library's default tile)
+  // NCCL_FUSELINK_ENGINE=1: batches of small requests go to a resident kernel through a descriptor ring instead of
+  // through a launch pair each (flh_engine_*); 0 = every batch is a launch pair
+  int engine = 1;
+  int engine_units = 1;          // staging units per lane for each of the engine's window sets
+  int engine_sets = 4;           // window sets the engine's batches rotate through = batches it has in flight at once
+  int engine_idle_us = 200;      // the engine goes down after this long without work
+  int engine_workgroups = 0;     // 0 = the library's default
+  int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
-  int batch_wait_ns = 3000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
+  int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
 Params g_par;
@@ -148,7 +157,8 @@ struct Request {
   int type = kReqUnused;
   std::atomic<int> state{0};
   Link* link = nullptr;
-  uint64_t seq = 0;          // number of that launch on its connection, counted from 1
+  uint64_t seq = 0;          // number of the launch (or engine batch) that carries it, counted from 1
+  bool engine = false;       // carried by an engine batch, not by a launch
   int size = 0;          // bytes moved (reported by test for receives)
   int fault = 0;         // injected wire fault
   uint32_t magic = 0;
@@ -199,6 +209,7 @@ struct LaunchSeg {
   uint64_t lane_base[FL_NET_MAX_LANES];
 };
 struct LaunchInfo {
+  bool engine = false;       // an engine batch: its table sits in the engine's slot (seq - 1) % kEngineSlots
   uint64_t seq = 0;
   uint32_t n_seg = 0, n_rows = 0;
   LaunchSeg seg[FLH_SEG_MAX] = {};
@@ -241,7 +252,18 @@ struct Peer {
   std::atomic<uint64_t> launch_seq{0};             // highest launch number handed out
   std::atomic<uint64_t> last_event_seq{0};         // highest launch whose completion comes from an event, not from the word
   LaunchInfo last;
+  // the lane engine (flh_engine_*): a resident kernel that takes batches of small requests from a descriptor ring.
+  // Its batches alternate between two window sets of their own and have their own numbers, tables and headers.
+  flh_engine* engine = nullptr;
+  std::atomic<bool> engine_ok{false};              // cleared for good when the engine reports an error
+  flh_window* ewin[kEngineSetsMax][FL_NET_MAX_LANES] = {};
+  flh_windows ewins[kEngineSetsMax] = {};
+  flh_chunk_desc* d_etable = nullptr;              // kEngineSlots tables of kEngineRows rows
+  flh_sched_hdr* d_ehdr = nullptr;                 // kEngineSlots headers
+  std::atomic<uint64_t> engine_submitted{0};       // batches handed to the engine (written under launch_mu)
 };
+constexpr uint32_t kEngineSlots = 64;              // the engine's descriptor ring
+constexpr uint32_t kEngineRows = 512;              // chunks an engine batch may hold
 
 struct Link {
   std::mutex mu;
@@ -266,6 +288,7 @@ struct Link {
   // scheduling state of the connection (the peer's launch_mu)
   uint64_t epoch_bytes = 0;         // bytes scheduled since the last lane-decision refresh (the scheduler's carried prefix)
   uint64_t last_seq = 0;            // launch that carried the connection's latest segment, and that segment's rows in its table
+  bool last_engine = false;         // ... or engine batch
   uint32_t last_first_row = 0, last_rows = 0;
   int64_t launches = 0, batched_requests = 0;    // launch pairs that carried its requests, requests that shared a pair with others
 };
@@ -326,9 +349,14 @@ void flush_pending(Peer* pr);
 void peer_destroy(Peer* pr) {        // no longer reachable through g_peers
   DeviceScope keep;
   (void)hipSetDevice(pr->hip_device);
+  if (pr->engine) (void)flh_engine_destroy(pr->engine);   // asks the resident kernel down and waits for it
   if (pr->stream) (void)hipStreamSynchronize(pr->stream);
-  for (int l = 0; l < FL_NET_MAX_LANES; ++l)
+  for (int l = 0; l < FL_NET_MAX_LANES; ++l) {
     if (pr->win[l]) (void)flh_window_destroy(pr->win[l]);
+    for (int h = 0; h < kEngineSetsMax; ++h) if (pr->ewin[h][l]) (void)flh_window_destroy(pr->ewin[h][l]);
+  }
+  if (pr->d_etable) (void)hipFree(pr->d_etable);
+  if (pr->d_ehdr) (void)hipFree(pr->d_ehdr);
   if (pr->d_table) (void)hipFree(pr->d_table);
   if (pr->d_hdr) (void)hipFree(pr->d_hdr);
   if (pr->d_count) (void)hipFree(pr->d_count);
@@ -371,6 +399,7 @@ Request* get_request(Request* tab, Link* lk, int type) {
       r->link = lk;
       r->size = 0;
       r->seq = 0;
+      r->engine = false;
       r->fault = 0;
       r->magic = kReqMagic;
       r->state.store(0, std::memory_order_relaxed);
@@ -422,6 +451,26 @@ ncclResult_t peer_setup(Peer* pr, int device) {
   pr->d_done = (uint32_t*)((char*)pr->d_status + 64);
   pr->h_started = (uint32_t*)((char*)pr->h_status + 128);
   pr->d_started = (uint32_t*)((char*)pr->d_status + 128);
+  if (g_par.engine) {
+    const uint64_t ecap = (uint64_t)g_par.engine_units * FLH_UNIT_BYTES;
+    if (ecap < (uint64_t)g_par.chunk) {
+      FL_INFO(NCCL_NET, "NET/FuseLink : the engine's windows (%llu bytes) do not hold a chunk: launches only", (unsigned long long)ecap);
+    } else {
+      for (int h = 0; h < g_par.engine_sets; ++h) {
+        pr->ewins[h].n_lanes = (uint32_t)g_par.lanes;
+        for (int l = 0; l < g_par.lanes; ++l) {
+          FL_FLHCHECK(flh_window_create(pool, ecap, &pr->ewin[h][l]));
+          FL_FLHCHECK(flh_window_bind(pr->ewin[h][l], ecap));
+          pr->ewins[h].base[l] = flh_window_base(pr->ewin[h][l]);
+          pr->ewins[h].cap[l] = flh_window_bound_bytes(pr->ewin[h][l]);
+        }
+      }
+      FL_HIPCHECK(hipMalloc((void**)&pr->d_etable, sizeof(flh_chunk_desc) * (size_t)kEngineSlots * kEngineRows));
+      FL_HIPCHECK(hipMalloc((void**)&pr->d_ehdr, sizeof(flh_sched_hdr) * (size_t)kEngineSlots));
+      FL_FLHCHECK(flh_engine_create(device, (uint32_t)g_par.engine_workgroups, (uint32_t)g_par.engine_idle_us, (uint32_t)g_par.engine_sets, &pr->engine));
+      pr->engine_ok.store(true, std::memory_order_release);
+    }
+  }
   pr->ready = true;
   FL_INFO(NCCL_NET, "NET/FuseLink : device %d staging ready: %d lanes x %llu bytes, shared by its connections", device, g_par.lanes, (unsigned long long)cap);
   return ncclSuccess;
@@ -520,6 +569,14 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.small_tile = (int)fl_param("FUSELINK_SMALL_TILE", g_par.small_tile);
   if (g_par.small_tile < 0 || g_par.small_tile % 128) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_SMALL_TILE must be a multiple of 128"); return ncclInvalidArgument; }
   g_par.trace = (int)fl_param("FUSELINK_TRACE", g_par.trace);
+  g_par.engine = (int)fl_param("FUSELINK_ENGINE", g_par.engine);
+  g_par.engine_units = (int)fl_param("FUSELINK_ENGINE_UNITS", g_par.engine_units);
+  g_par.engine_idle_us = (int)fl_param("FUSELINK_ENGINE_IDLE_US", g_par.engine_idle_us);
+  g_par.engine_sets = (int)fl_param("FUSELINK_ENGINE_SETS", g_par.engine_sets);
+  if (g_par.engine_sets < 1 || g_par.engine_sets > kEngineSetsMax) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_ENGINE_SETS must be 1..%d", kEngineSetsMax); return ncclInvalidArgument; }
+  g_par.engine_workgroups = (int)fl_param("FUSELINK_ENGINE_WORKGROUPS", g_par.engine_workgroups);
+  g_par.engine_max_request = fl_param("FUSELINK_ENGINE_MAX_REQUEST", g_par.engine_max_request);
+  if (g_par.engine_units < 1 || g_par.engine_idle_us < 1 || g_par.engine_workgroups < 0) { FL_WARN("NET/FuseLink : engine parameter out of range"); return ncclInvalidArgument; }
   g_par.batch_wait_ns = (int)fl_param("FUSELINK_BATCH_WAIT_NS", g_par.batch_wait_ns);
   if (g_par.batch_wait_ns < 0) g_par.batch_wait_ns = 0;
   g_par.queue_depth = (int)fl_param("FUSELINK_QUEUE_DEPTH", g_par.queue_depth);
@@ -528,6 +585,7 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   if (g_par.max_wave_chunks > 65535) g_par.max_wave_chunks = 65535;   // what one fused launch can name
   if (g_par.batch < 1) g_par.batch = 1;
   if (g_par.batch > FLH_BATCH_MAX) g_par.batch = FLH_BATCH_MAX;
+  if (g_par.completion != 2 || g_par.batch < 2) g_par.engine = 0;   // the engine reports through its completion word and takes batches
   if (g_par.lanes < 1 || g_par.lanes > FL_NET_MAX_LANES) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_LANES must be 1..%d", FL_NET_MAX_LANES); return ncclInvalidArgument; }
   if (g_par.chunk < 128 || g_par.chunk % 128 || g_par.chunk > (int64_t)1 << 30) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_CHUNKSIZE must be a multiple of 128 up to 1 GiB"); return ncclInvalidArgument; }
   if (g_par.refresh_batch < 1 || g_par.qps < 1 || g_par.qps > 128 || g_par.window_units < 1 || g_par.pool_units < 1 || g_par.max_wave_chunks < 1) {
@@ -859,10 +917,12 @@ ncclResult_t launch_transfer(Peer* pr, const Pending& p, uint64_t seq) {
       FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &pr->wins, &u, pr->d_status, pr->stream));
       const uint32_t rows = (uint32_t)((wave + chunk - 1) / chunk);
       pr->last.seq = seq;
+      pr->last.engine = false;
       pr->last.n_seg = 1;
       pr->last.n_rows = rows;
       note_segment(pr, 0, lk, 0, rows, 1, lk->epoch_bytes, nullptr);
       lk->last_seq = seq;
+      lk->last_engine = false;
       lk->last_first_row = 0;
       lk->last_rows = rows;
       lk->epoch_bytes += wave;
@@ -875,13 +935,20 @@ ncclResult_t launch_transfer(Peer* pr, const Pending& p, uint64_t seq) {
 
 // Does the send have to travel on its own, wave by wave?  Yes if it is split over QPs or if the staging windows
 // cannot hold it in one wave from where its connection stands in its credit epoch.
-bool needs_waves(const Peer* pr, const Pending& p, uint64_t epoch_bytes) {
+bool needs_waves(const flh_windows& wins, const Pending& p, uint64_t epoch_bytes) {
   if ((g_par.split_on_qps ? g_par.qps : 1) != 1) return true;
   uint32_t credits[FLH_MAX_LANES];
   wire_credits(p.lk, p.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
-  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, pr->wins.cap[0], epoch_bytes / chunk) * chunk;
+  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, wins.cap[0], epoch_bytes / chunk) * chunk;
   return (uint64_t)p.size > room;
+}
+
+// May the send travel in an engine batch?  Small requests only (large ones are bound by the GPU, not by the launch),
+// and it must fit one of the engine's window sets in one go.
+bool engine_takes(const Peer* pr, const Pending& p, uint64_t epoch_bytes) {
+  return pr->engine_ok.load(std::memory_order_acquire) && p.src_dev && p.dst_dev && (int64_t)p.size <= g_par.engine_max_request &&
+         !needs_waves(pr->ewins[0], p, epoch_bytes);
 }
 
 // The waiting sends work[i ..) that go out as one launch pair (launch_mu held): up to FLH_BATCH_MAX requests in up
@@ -894,8 +961,10 @@ struct BatchBuild {
   Link* seg_link[FLH_SEG_MAX];
   uint64_t link_epoch_after[FLH_SEG_MAX];   // the segment's connection's epoch bytes once the segment is scheduled
 };
-size_t build_batch(Peer* pr, size_t i, BatchBuild& bb) {
+size_t build_batch(Peer* pr, size_t i, BatchBuild& bb, bool engine) {
   const std::vector<Pending>& work = pr->work;
+  const flh_windows& wins = engine ? pr->ewins[0] : pr->wins;
+  const uint64_t max_chunks = engine ? kEngineRows : (uint64_t)g_par.max_wave_chunks;
   flh_batch_params& b = bb.b;
   memset(&b, 0, sizeof(b));
   const uint64_t chunk = (uint64_t)g_par.chunk;
@@ -921,7 +990,8 @@ size_t build_batch(Peer* pr, size_t i, BatchBuild& bb) {
       extend = bb.seg_link[k] == p.lk && !(p.w.flags & 1u) && (uint64_t)work[j - 1].size % chunk == 0 &&
                memcmp(b.seg[k].credits, credits, sizeof(credits)) == 0;
     }
-    if (!extend && (b.n_seg == FLH_SEG_MAX || needs_waves(pr, p, epoch))) break;
+    if (engine ? !engine_takes(pr, p, epoch) : (!extend && needs_waves(wins, p, epoch))) break;
+    if (!extend && b.n_seg == FLH_SEG_MAX) break;
     // Where would the windows end up?  The open segment grows by the request, or is closed and a new one opens
     // behind it, on every lane at the next multiple of 128 bytes (flh_batch_layout's rule).
     uint64_t base_end[FLH_MAX_LANES], lane_bytes[FLH_MAX_LANES];
@@ -945,9 +1015,9 @@ size_t build_batch(Peer* pr, size_t i, BatchBuild& bb) {
       try_epoch = epoch;
     }
     fl_row_lane_totals(try_row, try_epoch / chunk, try_bytes, chunk, lane_bytes, lane_chunks);
-    bool fits = chunks_before + (try_bytes + chunk - 1) / chunk <= (uint64_t)g_par.max_wave_chunks;
+    bool fits = chunks_before + (try_bytes + chunk - 1) / chunk <= max_chunks;
     for (int l = 0; fits && l < g_par.lanes; ++l)
-      if (lane_chunks[l]) fits = (base_end[l] + 127) / 128 * 128 + lane_bytes[l] <= pr->wins.cap[l];
+      if (lane_chunks[l]) fits = (base_end[l] + 127) / 128 * 128 + lane_bytes[l] <= wins.cap[l];
     if (!fits) break;
     uint32_t k;
     if (extend) {
@@ -975,22 +1045,44 @@ size_t build_batch(Peer* pr, size_t i, BatchBuild& bb) {
   return j - i;
 }
 
-ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, uint64_t seq) {
+// The batch as a launch pair on the peer's stream (engine == false, `seq` its launch number), or handed to the engine
+// (engine == true; `seq` then returns the engine's number for the batch).
+ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool engine, uint64_t& seq) {
   flh_batch_params& b = bb.b;
   b.u.tile_bytes = launch_tile(b.u.total_bytes);
   uint64_t seg_base[FLH_SEG_MAX][FLH_MAX_LANES];
-  FL_FLHCHECK(flh_batch_layout(&b, nullptr, &seg_base[0][0]));
-  start_stamp(pr, seq, b.u);
-  FL_FLHCHECK(flh_stripe_batch(&b, &pr->wins, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
-  Completion comp;
-  ncclResult_t rc = prepare_completion(pr, seq, b.u.total_bytes, b.u, comp);
-  if (rc != ncclSuccess) return rc;
-  FL_FLHCHECK(flh_reassemble_batch(&b, &pr->wins, pr->d_status, pr->stream));
-  rc = finish_completion(pr, seq, comp);
-  if (rc != ncclSuccess) return rc;
+  if (!engine) FL_FLHCHECK(flh_batch_layout(&b, nullptr, &seg_base[0][0]));
+  if (engine) {
+    // batch number k (from 1) takes window set (k - 1) mod sets and slot (k - 1) % kEngineSlots of the tables; the engine
+    // lets it in once batch k - sets, the last to use that window set, is complete
+    const uint64_t k = pr->engine_submitted.load(std::memory_order_relaxed);
+    const uint32_t slot = (uint32_t)(k % kEngineSlots);
+    b.u.tile_bytes = FLH_TILE_BYTES;
+    uint64_t got = 0;
+    const int frc = flh_engine_submit(pr->engine, &b, &pr->ewins[k % (uint64_t)g_par.engine_sets], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot, pr->d_status, &got,
+                                      &seg_base[0][0]);
+    if (frc == FLH_E_NOMEM) return ncclInProgress;   // the descriptor ring is full: the caller takes the launch path for this batch
+    if (frc < 0) {
+      FL_WARN("NET/FuseLink : engine: %s", flh_last_error());
+      pr->engine_ok.store(false, std::memory_order_release);
+      return ncclInProgress;
+    }
+    seq = got;
+    pr->engine_submitted.store(got, std::memory_order_release);
+  } else {
+    start_stamp(pr, seq, b.u);
+    FL_FLHCHECK(flh_stripe_batch(&b, &pr->wins, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+    Completion comp;
+    ncclResult_t rc = prepare_completion(pr, seq, b.u.total_bytes, b.u, comp);
+    if (rc != ncclSuccess) return rc;
+    FL_FLHCHECK(flh_reassemble_batch(&b, &pr->wins, pr->d_status, pr->stream));
+    rc = finish_completion(pr, seq, comp);
+    if (rc != ncclSuccess) return rc;
+  }
   // bookkeeping: every connection's place in its epoch, what the launch carried
   const uint64_t chunk = (uint64_t)g_par.chunk;
   pr->last.seq = seq;
+  pr->last.engine = engine;
   pr->last.n_seg = b.n_seg;
   uint32_t row = 0, q = 0;
   for (uint32_t k = 0; k < b.n_seg; ++k) {
@@ -999,8 +1091,9 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, uint64_t
     for (uint32_t r = 0; r < b.seg[k].n_req; ++r) seg_bytes += b.bytes[q++];
     const uint32_t rows = (uint32_t)((seg_bytes + chunk - 1) / chunk);
     note_segment(pr, k, lk, row, rows, b.seg[k].n_req, b.seg[k].epoch_bytes, seg_base[k]);
-    if (lk->last_seq != seq) lk->launches++;
+    if (lk->last_seq != seq || lk->last_engine != engine) lk->launches++;
     lk->last_seq = seq;
+    lk->last_engine = engine;
     lk->last_first_row = row;
     lk->last_rows = rows;
     lk->epoch_bytes = bb.link_epoch_after[k];
@@ -1030,11 +1123,27 @@ void flush_pending(Peer* pr) {
   size_t i = 0;
   while (i < work.size()) {
     ncclResult_t rc = dev_ok ? ncclSuccess : ncclUnhandledCudaError;
-    const uint64_t seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
-    pr->launch_seq.store(seq, std::memory_order_release);   // before anything runs: the completion word never runs ahead of it
     size_t span = 1;
     const Pending& p = work[i];
-    if (rc == ncclSuccess) {
+    const uint64_t p_epoch = (p.w.flags & 1u) ? 0 : p.lk->epoch_bytes;
+    // small requests in device memory go to the engine, batch by batch: no launch, and a number of the engine's own
+    bool by_engine = false;
+    uint64_t seq = 0;
+    if (rc == ncclSuccess && g_par.batch >= 2 && engine_takes(pr, p, p_epoch)) {
+      BatchBuild bb;
+      const size_t n = build_batch(pr, i, bb, true);
+      if (n) {
+        TraceScope trl(kTrLaunch);
+        const ncclResult_t erc = launch_batch(pr, i, n, bb, true, seq);
+        if (erc == ncclSuccess) { by_engine = true; span = n; }
+        else if (erc != ncclInProgress) rc = erc;    // ncclInProgress: the engine could not take it, a launch pair carries it
+      }
+    }
+    if (!by_engine) {
+      seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
+      pr->launch_seq.store(seq, std::memory_order_release);   // before anything runs: the completion words never run ahead of it
+    }
+    if (rc == ncclSuccess && !by_engine) {
       if (!(p.src_dev && p.dst_dev)) {
         // one side is host memory: the copy engine is the wire, nothing is striped
         hipEvent_t ev = nullptr;
@@ -1042,14 +1151,14 @@ void flush_pending(Peer* pr) {
         hipError_t e = rc == ncclSuccess ? hipMemcpyAsync(p.dst, p.src, (size_t)p.size, hipMemcpyDefault, pr->stream) : hipSuccess;
         if (e != hipSuccess) rc = hip_fail("hipMemcpyAsync", e);
         if (rc == ncclSuccess) { Completion c; c.ev = ev; rc = finish_completion(pr, seq, c); }
-      } else if (g_par.batch < 2 || needs_waves(pr, p, (p.w.flags & 1u) ? 0 : p.lk->epoch_bytes)) {
+      } else if (g_par.batch < 2 || needs_waves(pr->wins, p, p_epoch)) {
         rc = launch_transfer(pr, p, seq);
       } else {
         BatchBuild bb;
-        span = build_batch(pr, i, bb);
+        span = build_batch(pr, i, bb, false);
         TraceScope trl(kTrLaunch);
         if (span == 0) { span = 1; rc = launch_transfer(pr, p, seq); }   // cannot happen: the request fits an empty set of windows
-        else rc = launch_batch(pr, i, span, bb, seq);
+        else rc = launch_batch(pr, i, span, bb, false, seq);
       }
     }
     for (size_t k = i; k < i + span; ++k) {
@@ -1057,6 +1166,8 @@ void flush_pending(Peer* pr) {
       if (rc == ncclSuccess) {
         q.sreq->seq = seq;
         q.rreq->seq = seq;
+        q.sreq->engine = by_engine;
+        q.rreq->engine = by_engine;
         q.sreq->state.store(kStLaunched, std::memory_order_release);
         q.rreq->state.store(kStLaunched, std::memory_order_release);
       } else {
@@ -1066,7 +1177,7 @@ void flush_pending(Peer* pr) {
         q.rreq->state.store(kStDoneHost, std::memory_order_release);
       }
     }
-    if (rc != ncclSuccess) {
+    if (rc != ncclSuccess && !by_engine) {
       // whatever part of the launch was queued is waited for here, so that its number counts as complete and the
       // launches behind it are not held back by one that will never report
       if (dev_ok) (void)hipStreamSynchronize(pr->stream);
@@ -1295,6 +1406,13 @@ ncclResult_t launch_complete(Peer* pr, uint64_t seq, bool* done) {
   return ncclSuccess;
 }
 
+// Engine batches handed over and not yet reported complete.
+uint64_t engine_in_flight(Peer* pr) {
+  if (!pr->engine) return 0;
+  const uint64_t sub = pr->engine_submitted.load(std::memory_order_acquire), done = flh_engine_completed(pr->engine);
+  return sub > done ? sub - done : 0;
+}
+
 // Launches of the peer that have been queued and are not known to be complete.
 uint64_t launches_in_queue(Peer* pr) {
   uint64_t done = pr->done_seq.load(std::memory_order_acquire);
@@ -1326,7 +1444,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     // a launch whose completion comes from an event is only known complete once its own requests are polled: it
     // must not hold anything back
     const bool events_out = pr->last_event_seq.load(std::memory_order_acquire) > pr->done_seq.load(std::memory_order_acquire);
-    bool go = events_out || g_par.completion != 2 || launches_in_queue(pr) < (uint64_t)g_par.queue_depth;
+    bool go = events_out || g_par.completion != 2 || launches_in_queue(pr) + engine_in_flight(pr) < (uint64_t)g_par.queue_depth;
     // small sends wait a moment for company: a launch pair costs the host as much as ten requests do
     if (go && g_par.batch_wait_ns && pr->waiting_bytes.load(std::memory_order_acquire) < kEarlyLaunchBytes &&
         pr->waiting_reqs.load(std::memory_order_acquire) < (uint32_t)g_par.batch &&
@@ -1341,7 +1459,16 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     }
   }
   if (st == kStQueued) return ncclSuccess;
-  if (st == kStLaunched) {
+  if (st == kStLaunched && r->engine) {
+    // the engine stores the number of the last complete batch to a pinned word: a plain load, as for the launches' words
+    if (flh_engine_completed(pr->engine) < r->seq) {
+      if (flh_engine_error(pr->engine) == 0) return ncclSuccess;
+      // the engine went down on a wait that ran out: what it still held is lost, later traffic travels by launches
+      pr->engine_ok.store(false, std::memory_order_release);
+      FL_WARN("NET/FuseLink : the lane engine stopped with an error; channel %d falls back to launches", lk->channelId);
+      r->fault = 1;
+    }
+  } else if (st == kStLaunched) {
     bool complete = false;
     ncclResult_t rc = launch_complete(pr, r->seq, &complete);
     if (rc != ncclSuccess || !complete) return rc;
@@ -1520,7 +1647,25 @@ static int drain_peer(Peer* pr) {
   flush_pending(pr);
   DeviceScope keep;
   if (hipSetDevice(pr->hip_device) != hipSuccess || hipStreamSynchronize(pr->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
+  if (pr->engine) {
+    const int64_t until = tr_now() + 5000000000ll;
+    while (flh_engine_completed(pr->engine) < pr->engine_submitted.load(std::memory_order_acquire)) {
+      if (flh_engine_error(pr->engine) || tr_now() > until) return fl_set_error(FLH_E_STATE, "the lane engine did not finish its batches");
+    }
+  }
   return FLH_OK;
+}
+
+// table and header of the peer's last launch or engine batch (launch_mu held, the peer drained)
+static void last_buffers(const Peer* pr, const flh_chunk_desc** table, const flh_sched_hdr** hdr) {
+  if (pr->last.engine) {
+    const uint32_t slot = (uint32_t)((pr->last.seq - 1) % kEngineSlots);
+    *table = pr->d_etable + (size_t)slot * kEngineRows;
+    *hdr = pr->d_ehdr + slot;
+  } else {
+    *table = pr->d_table;
+    *hdr = pr->d_hdr;
+  }
 }
 
 int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_out) {
@@ -1533,14 +1678,17 @@ int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_ou
   int rc = drain_peer(pr);
   if (rc) return rc;
   if (lk->last_seq == 0) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
-  if (lk->last_seq != pr->last.seq) return fl_set_error(FLH_E_STATE, "a later launch of another connection has reused the table");
+  if (lk->last_seq != pr->last.seq || lk->last_engine != pr->last.engine) return fl_set_error(FLH_E_STATE, "a later launch of another connection has reused the table");
   const int rows = (int)lk->last_rows;
   const int take = rows < max_rows ? rows : max_rows;
+  const flh_chunk_desc* table;
+  const flh_sched_hdr* hdr;
+  last_buffers(pr, &table, &hdr);
   DeviceScope keep;
   if (hipSetDevice(pr->hip_device) != hipSuccess) return fl_set_error(FLH_E_HIP, "hipSetDevice failed");
-  if (take > 0 && rows_out && hipMemcpy(rows_out, pr->d_table + lk->last_first_row, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
+  if (take > 0 && rows_out && hipMemcpy(rows_out, table + lk->last_first_row, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "table copy failed");
-  if (hdr_out && hipMemcpy(hdr_out, pr->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
+  if (hdr_out && hipMemcpy(hdr_out, hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "header copy failed");
   return rows;
 }
@@ -1564,11 +1712,14 @@ int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, vo
     for (int l = 0; l < FL_NET_MAX_LANES; ++l) o.lane_base[l] = li.seg[k].lane_base[l];
   }
   const int take = (int)li.n_rows < max_rows ? (int)li.n_rows : max_rows;
+  const flh_chunk_desc* table;
+  const flh_sched_hdr* hdr;
+  last_buffers(pr, &table, &hdr);
   DeviceScope keep;
   if (hipSetDevice(pr->hip_device) != hipSuccess) return fl_set_error(FLH_E_HIP, "hipSetDevice failed");
-  if (take > 0 && rows_out && hipMemcpy(rows_out, pr->d_table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
+  if (take > 0 && rows_out && hipMemcpy(rows_out, table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "table copy failed");
-  if (hdr_out && hipMemcpy(hdr_out, pr->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
+  if (hdr_out && hipMemcpy(hdr_out, hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
     return fl_set_error(FLH_E_HIP, "header copy failed");
   return (int)li.n_seg;
 }

@@ -307,6 +307,29 @@ int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int3
  * (host arithmetic, nothing is launched); seg_base, if given, receives FLH_SEG_MAX x FLH_MAX_LANES lane bases, row k
  * those of segment k.  A caller sizes its batches with it so that no lane outgrows its window. */
 int flh_batch_layout(const flh_batch_params* b, uint64_t* lane_end, uint64_t* seg_base);
+/* ---- lane engine: batches without a launch per batch ------------------------------------------------------------
+ * A resident kernel -- one dispatcher workgroup, the others workers, by default one worker per two compute units -- that
+ * executes batches as flh_stripe_batch + flh_reassemble_batch would, but takes them from a descriptor ring in pinned
+ * host memory instead of from kernel launches: flh_engine_submit writes the descriptor and advances a tail word (about
+ * a microsecond of host time instead of about ten for a launch pair), the engine stripes every tile into the windows,
+ * reassembles it from there and stores the batch's number to a host-visible word when its last workgroup has left the
+ * batch (flh_engine_completed reads it: no call into the runtime).  Rows, header, staged bytes and received bytes are
+ * those of the launched pair.  Several batches are in flight at once, so successive batches must not share staging
+ * windows: the caller rotates window_sets (1..8) sets of windows, batch number k taking set (k - 1) mod window_sets, and
+ * the engine lets a batch in only once batch k - window_sets is complete.  With nothing to do for idle_us (default 200) the
+ * engine goes down and the next submit starts it again with one launch.  Every wait inside the kernel is bounded;
+ * flh_engine_error reports FLH_E_STATE if one ran out.  No counterpart in the reference, whose NIC plays this part.
+ * flh_engine_submit and flh_engine_destroy are not thread-safe (one submitter at a time); the readers are. */
+typedef struct flh_engine flh_engine;
+int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_t window_sets, flh_engine** out);
+/* *seq_out = the batch's number, from 1; seg_base_out (optional) = the lane bases of its segments, as flh_batch_layout gives them */
+int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
+                      flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out);
+uint64_t flh_engine_completed(const flh_engine* e);   /* batches complete: all with a number up to this one */
+int flh_engine_error(const flh_engine* e);
+uint64_t flh_engine_launches(const flh_engine* e);    /* engine kernels started so far */
+int flh_engine_destroy(flh_engine* e);                /* asks the engine down and waits for it */
+
 /* Paged variants for non-contiguous sources (KV-cache blocks, src/experiments/serving/model.hh:
  * 198-201 gives the page shape): a chunk whose row says src_off stands for the pages
  * d_page_table[src_off / page_bytes ...] (pages_per_chunk of them) of a pool of page_bytes-sized

@@ -1,0 +1,145 @@
+"""The lane engine (flh_engine_*): a resident kernel that executes batches from a descriptor ring instead of from a launch
+pair each.  What it stages and delivers must be what flh_stripe_batch / flh_reassemble_batch stage and deliver, i.e. the
+oracle's tables and bytes; it must go down when idle and come up again with the next batch; bad arguments are refused on
+the host."""
+import ctypes as C
+import time
+
+import numpy as np
+import pytest
+
+from tests import oracle_binding as ob
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fl():
+    import torch
+    from fuselink_amd import _lib, core
+    core.init(0)
+    return core, torch, _lib
+
+
+def _dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _wait(lib, eng, seq, seconds=10.0):
+    deadline = time.time() + seconds
+    while lib.flh_engine_completed(eng) < seq:
+        assert lib.flh_engine_error(eng) == 0, "the engine reported a wait that ran out"
+        assert time.time() < deadline, f"batch {seq} did not complete (completed {lib.flh_engine_completed(eng)})"
+
+
+@pytest.mark.parametrize("sets", [1, 3])
+def test_engine_batches_equal_the_oracle_and_the_engine_restarts_after_idling(fl, sets):
+    core, torch, _lib = fl
+    lib = _lib.load()
+    rng = np.random.default_rng(7300 + sets)
+    lanes, chunk, n_batches = 6, 32 << 10, 7
+    eng = C.c_void_p()
+    _lib.check(lib.flh_engine_create(0, 0, 100, sets, C.byref(eng)))     # idle limit 100 us
+    try:
+        cap = 3 << 20
+        wins = [[torch.zeros(cap + 64, dtype=torch.uint8, device="cuda") for _ in range(lanes)] for _ in range(sets)]
+        W = [core.make_windows([t.data_ptr() for t in ws], [cap] * lanes) for ws in wins]
+        status = core.new_status()
+        batches = []
+        for k in range(n_batches):
+            n_seg = int(rng.integers(1, 4))
+            segments, sizes = [], []
+            for _ in range(n_seg):
+                n_req = int(rng.integers(1, 5))
+                ss = [int(rng.integers(1, 6)) * chunk for _ in range(n_req)]
+                if rng.random() < 0.5:
+                    ss[-1] -= int(rng.integers(1, chunk))
+                segments.append((n_req, rng.integers(0, 6, size=lanes).astype(np.uint32), int(rng.integers(0, 30)) * chunk))
+                sizes += ss
+            srcs_np = [rng.integers(0, 256, size=s, dtype=np.uint8) for s in sizes]
+            srcs = [_dev(torch, a) for a in srcs_np]
+            dsts = [torch.zeros(s + 32, dtype=torch.uint8, device="cuda") for s in sizes]
+            n_rows = sum((s + chunk - 1) // chunk for s in sizes) + len(segments)
+            batches.append(dict(segments=segments, sizes=sizes, srcs_np=srcs_np, srcs=srcs, dsts=dsts, out=core.new_schedule_buffers(n_rows)))
+        torch.cuda.synchronize()
+        seq = C.c_uint64()
+        for k, bt in enumerate(batches):
+            b = core.batch_params(bt["srcs"], bt["dsts"], chunk, [1] * lanes, segments=[(n, c.tolist(), e) for n, c, e in bt["segments"]])
+            _lib.check(lib.flh_engine_submit(eng, C.byref(b), C.byref(W[k % sets]), bt["out"].table.data_ptr(), bt["out"].hdr.data_ptr(),
+                                             status.data_ptr(), C.byref(seq), None))
+            assert seq.value == k + 1
+            if k == 2:
+                _wait(lib, eng, seq.value)
+                time.sleep(0.02)            # far beyond the idle limit: the engine goes down, the next submit starts it again
+                assert int(lib.flh_engine_launches(eng)) == 1
+            if sets == 1:
+                _wait(lib, eng, seq.value)  # one window set: the caller may not have two batches in flight
+        _wait(lib, eng, seq.value)
+        assert int(lib.flh_engine_launches(eng)) == 2 and lib.flh_engine_error(eng) == 0
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+        for k, bt in enumerate(batches):
+            lane_end = np.zeros(16, dtype=np.uint64)
+            rows, first_row, q = [], 0, 0
+            tpc = (chunk + 32767) // 32768
+            staged = []
+            for n_req, credits, epoch in bt["segments"]:
+                seg_np = np.concatenate(bt["srcs_np"][q:q + n_req])
+                q += n_req
+                st = np.zeros(1, dtype=ob.STATE_DTYPE)[0]
+                st["epoch_bytes"] = epoch
+                exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=seg_np.size, chunk_bytes=chunk,
+                                                     mode=ob.SCHED_RESET_OFFSETS, state=st)
+                base = (lane_end + np.uint64(127)) // np.uint64(128) * np.uint64(128)
+                wins_seg = ob.cpu_stripe(seg_np, exp_t, [int(x) for x in exp_h["lane_bytes"][:lanes]])
+                for l in range(lanes):
+                    n = int(exp_h["lane_bytes"][l])
+                    if n:
+                        staged.append((l, int(base[l]), wins_seg[l][:n]))
+                r = exp_t.copy()
+                r["win_off"] += base[r["lane"]]
+                r["tile_base"] += first_row * tpc
+                rows.append(r)
+                used = exp_h["lane_chunks"] > 0
+                lane_end[used] = base[used] + exp_h["lane_bytes"][used]
+                first_row += len(exp_t)
+            exp_rows = np.concatenate(rows)
+            bt["out"].n_chunks = len(exp_rows)
+            got = bt["out"].table_numpy()
+            for f in ob.DESC_DTYPE.names:
+                np.testing.assert_array_equal(got[f], exp_rows[f], err_msg=f"batch {k}: {f}")
+            assert int(bt["out"].hdr_numpy()["n_chunks"]) == len(exp_rows)
+            if k >= n_batches - sets:       # the window sets still hold what their last batch staged
+                for l, off, data in staged:
+                    np.testing.assert_array_equal(wins[k % sets][l].cpu().numpy()[off:off + data.size], data, err_msg=f"batch {k} lane {l}")
+            for i, s in enumerate(bt["sizes"]):
+                g = bt["dsts"][i].cpu().numpy()
+                np.testing.assert_array_equal(g[:s], bt["srcs_np"][i], err_msg=f"batch {k} request {i}")
+                assert not g[s:].any()
+    finally:
+        _lib.check(lib.flh_engine_destroy(eng))
+
+
+def test_engine_refuses_bad_arguments_on_the_host(fl):
+    core, torch, _lib = fl
+    lib = _lib.load()
+    eng = C.c_void_p()
+    assert lib.flh_engine_create(0, 0, 0, 0, C.byref(eng)) == -1       # no window set
+    assert lib.flh_engine_create(0, 0, 0, 9, C.byref(eng)) == -1       # more sets than the engine keeps descriptors for
+    assert lib.flh_engine_create(0, 1, 0, 2, C.byref(eng)) == -1       # a dispatcher without workers
+    _lib.check(lib.flh_engine_create(0, 9, 0, 2, C.byref(eng)))
+    try:
+        chunk = 4096
+        srcs = [torch.zeros(chunk + 1, dtype=torch.uint8, device="cuda"), torch.zeros(chunk, dtype=torch.uint8, device="cuda")]
+        dsts = [torch.zeros_like(t) for t in srcs]
+        wins = [torch.zeros(8 * chunk, dtype=torch.uint8, device="cuda") for _ in range(2)]
+        w = core.make_windows([t.data_ptr() for t in wins], [8 * chunk] * 2)
+        out = core.new_schedule_buffers(8)
+        status = core.new_status()
+        seq = C.c_uint64()
+        b = core.batch_params(srcs, dsts, chunk, [1, 1])
+        with pytest.raises(Exception, match="whole number of chunks"):
+            _lib.check(lib.flh_engine_submit(eng, C.byref(b), C.byref(w), out.table.data_ptr(), out.hdr.data_ptr(), status.data_ptr(), C.byref(seq), None))
+        assert int(lib.flh_engine_launches(eng)) == 0 and int(lib.flh_engine_completed(eng)) == 0
+    finally:
+        _lib.check(lib.flh_engine_destroy(eng))

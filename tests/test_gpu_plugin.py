@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 ENV_KEYS = ["NCCL_FUSELINK_LANES", "NCCL_FUSELINK_CHUNKSIZE", "NCCL_FUSELINK_POLICY", "NCCL_FUSELINK_WINDOW_UNITS",
             "NCCL_FUSELINK_POOL_UNITS", "NCCL_FUSELINK_REFRESH_BATCH", "NCCL_IB_QPS_PER_CONNECTION", "NCCL_FUSELINK_CREDITS",
-            "NCCL_FUSELINK_BATCH", "NCCL_FUSELINK_COMPLETION"]
+            "NCCL_FUSELINK_BATCH", "NCCL_FUSELINK_COMPLETION", "NCCL_FUSELINK_ENGINE", "NCCL_FUSELINK_ENGINE_SETS", "NCCL_FUSELINK_ENGINE_UNITS"]
 
 
 @pytest.fixture()
@@ -313,17 +313,18 @@ def test_mixed_host_and_device_buffers(net):
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
-@pytest.mark.parametrize("completion", [0, 1, 2])
+@pytest.mark.parametrize("completion,engine", [(0, 0), (1, 0), (2, 0), (2, 1)])
 @pytest.mark.parametrize("batch", [1, 8])
-def test_completion_reaches_test_in_every_mode(net, completion, batch):
+def test_completion_reaches_test_in_every_mode(net, completion, engine, batch):
     """How `test` learns that a launch is done -- an event behind every launch, an event on the launch's last kernel,
-    or the stamp the next launch's first kernel leaves (with an event only behind a launch that nothing follows) --
-    must not change what a consumer sees: every receive is compared on torch's own stream, which does not wait for the
+    the words that kernels store launch numbers to (a small launch's reassembly kernel when its last workgroup has
+    finished, every striping kernel as it starts, an event only behind a large launch that nothing follows), or the
+    lane engine's completion word for the small requests it carries -- must not change what a consumer sees: every receive is compared on torch's own stream, which does not wait for the
     connection's, the moment `test` reports it done, with requests in flight behind it, empty requests and host
     buffers mixed in, and a lone request at the end that no other launch follows."""
     import torch
     net.reconfigure(NCCL_FUSELINK_LANES=4, NCCL_FUSELINK_CHUNKSIZE=64 << 10, NCCL_FUSELINK_WINDOW_UNITS=1,
-                    NCCL_FUSELINK_BATCH=batch, NCCL_FUSELINK_COMPLETION=completion)
+                    NCCL_FUSELINK_BATCH=batch, NCCL_FUSELINK_COMPLETION=completion, NCCL_FUSELINK_ENGINE=engine)
     net.set_credits([3, 1, 2, 2])
     rng = np.random.default_rng(900 + completion * 10 + batch)
     n_req = 120
