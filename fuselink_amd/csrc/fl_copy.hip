@@ -390,9 +390,10 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
   return full * c + part;
 }
 
-// One workgroup's share of a fused launch: tile bx of the chunk that grid row by stands for.
+// One workgroup's share of a fused launch: tile bx of the chunk that grid row by stands for (`span` neighbouring tiles
+// of that chunk from bx on, for a caller that hands out larger shares).
 template <int DIR, int NT, class Args>
-__device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by) {
+__device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by, uint32_t span = 1) {
   constexpr bool BATCH = is_batch<Args>::value;
   constexpr bool PAGED = is_paged<Args>::value;
   if (by >= a.n_chunks) return;
@@ -573,7 +574,8 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
 
   const uint64_t off = (uint64_t)bx * a.tile_bytes;
   if (off >= len) return;
-  const uint32_t bytes = (uint32_t)((len - off) < a.tile_bytes ? (len - off) : a.tile_bytes);
+  const uint64_t share = (uint64_t)a.tile_bytes * span;
+  const uint32_t bytes = (uint32_t)((len - off) < share ? (len - off) : share);
   if (win_off + len > a.win.cap[lane] || (!PAGED && user_off + len > user_bytes)) {
     if (threadIdx.x == 0) *a.status = FLH_E_RANGE;
     return;
@@ -776,6 +778,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     uint64_t k = e.start;
     uint64_t tail_seen = e.start;   // the host's tail as last read: a burst of batches costs one look across the bus
     uint32_t first_worker = 0;      // takes the first tile of batch k
+    uint32_t polls = 0;
     uint64_t idle_since = wall_clock64(), free_since = idle_since;
     for (;;) {
       if (tid == 0) {
@@ -793,9 +796,9 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
         if (act == 1) {
           idle_since = now;
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the workers' reads of the slot are behind their arrival
-        } else if (__hip_atomic_load(&e.hctl->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) ||
-                   __hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
-          act = 2;
+        } else if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ||
+                   ((++polls & 31) == 0 && __hip_atomic_load(&e.hctl->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM))) {
+          act = 2;   // (the host's stop flag is a trip across the bus: looked at now and then)
         } else if (now - idle_since > e.idle_ticks) {
           // Nothing for a while: announce it, then look once more.  The host stores the tail, then reads the state; this
           // side stores the state, then reads the tail: one of the two sees the other's store.
@@ -815,7 +818,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
       const uint32_t act = sh_flag;
       __syncthreads();
       if (act == 2) break;
-      if (act == 0) { __builtin_amdgcn_s_sleep(8); continue; }
+      if (act == 0) { __builtin_amdgcn_s_sleep(2); continue; }
       // descriptor k: pinned host memory -> device ring, sixteen bytes per thread
       const u32x4* src = (const u32x4*)(e.host_ring + (size_t)(k % e.host_slots) * kEngineDescBytes);
       u32x4* dst = (u32x4*)(e.dev_ring + (size_t)(k % kEngineDevRing) * kEngineDescBytes);
@@ -899,14 +902,22 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     __syncthreads();
     const uint32_t tpc = d.a.tiles_per_chunk;
     const uint32_t total = tpc * d.a.n_chunks;
-    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W)                           // this worker's tiles, user buffers -> windows
-      for (uint32_t t = sh * kEngineShare; t < total && t < (sh + 1) * kEngineShare; ++t) fused_tile<0, 0>(d.a, t % tpc, t / tpc);
+    // a share is kEngineShare neighbouring tiles: one copy of twice the length when they lie in one chunk
+    const bool whole = tpc % kEngineShare == 0;
+    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {                         // this worker's tiles, user buffers -> windows
+      const uint32_t t0 = sh * kEngineShare;
+      if (whole) fused_tile<0, 0>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
+      else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<0, 0>(d.a, t % tpc, t / tpc);
+    }
     __syncthreads();
     if (tid < FLH_BATCH_MAX) d.a.req_user[tid] = d.req_dst[tid];                          // the same tiles, windows -> receive buffers
     if (tid == 0) { d.a.table = nullptr; d.a.hdr = nullptr; }
     __syncthreads();
-    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W)
-      for (uint32_t t = sh * kEngineShare; t < total && t < (sh + 1) * kEngineShare; ++t) fused_tile<1, 0>(d.a, t % tpc, t / tpc);
+    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
+      const uint32_t t0 = sh * kEngineShare;
+      if (whole) fused_tile<1, 0>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
+      else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<1, 0>(d.a, t % tpc, t / tpc);
+    }
     __syncthreads();
     if (tid == 0) {
       // leaving the batch releases this worker's stores; the last one to leave has thereby acquired everybody's and
@@ -1408,6 +1419,10 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
 
 // start the resident kernel with the batch the last one stopped at (the stream orders it behind that one's exit)
 static int engine_start(flh_engine* e) {
+  int prev = -1;
+  (void)hipGetDevice(&prev);
+  if (prev != e->device) FL_HIP(hipSetDevice(e->device));
+  struct Back { int dev; ~Back() { if (dev >= 0) (void)hipSetDevice(dev); } } back{prev != e->device ? prev : -1};
   EngineArgs a;
   a.host_ring = e->d_ring_host;
   a.host_slots = e->host_slots;

@@ -99,6 +99,22 @@ inline int64_t tr_now() {
   clock_gettime(CLOCK_MONOTONIC, &t);
   return (int64_t)t.tv_sec * 1000000000ll + t.tv_nsec;
 }
+// NCCL_FUSELINK_TRACE=2 also keeps a timeline: (nanoseconds, thread, event, value) of every entry-point event, in a fixed
+// ring that fl_net_timeline() copies out.  Events: 1 irecv posted (value = channel), 2 isend matched (channel),
+// 3 pass that launches begins (requests waiting), 4 batch handed over (requests << 32 | number; bit 31 of the number's
+// word set for engine batches), 5 request seen complete by test (channel << 1 | is-receive).
+struct TimelineEvent { int64_t ns; uint32_t thread; uint32_t event; uint64_t value; };
+constexpr size_t kTimelineCap = 1 << 16;
+TimelineEvent g_timeline[kTimelineCap];
+std::atomic<uint64_t> g_timeline_n{0};
+inline void tl_event(uint32_t event, uint64_t value) {
+  if (g_par.trace < 2) return;
+  static std::atomic<uint32_t> next_thread{0};
+  thread_local uint32_t me = next_thread.fetch_add(1);
+  const uint64_t i = g_timeline_n.fetch_add(1, std::memory_order_relaxed);
+  if (i >= kTimelineCap) return;
+  g_timeline[i] = TimelineEvent{tr_now(), me, event, value};
+}
 struct TraceScope {
   int what;
   int64_t t0;
@@ -127,6 +143,25 @@ struct DeviceScope {
   ~DeviceScope() { if (saved >= 0) (void)hipSetDevice(saved); }
   DeviceScope(const DeviceScope&) = delete;
   DeviceScope& operator=(const DeviceScope&) = delete;
+};
+// The same, but the runtime is only asked once a call that needs the device is about to be made: a pass that hands
+// everything to the lane engine makes none.
+struct LazyDevice {
+  int want, saved = -1;
+  bool switched = false, ok = true;
+  explicit LazyDevice(int device) : want(device) {}
+  bool use() {
+    if (!switched) {
+      switched = true;
+      if (hipGetDevice(&saved) != hipSuccess) saved = -1;
+      ok = saved == want || hipSetDevice(want) == hipSuccess;
+      if (saved == want) saved = -1;   // nothing to put back
+    }
+    return ok;
+  }
+  ~LazyDevice() { if (switched && saved >= 0) (void)hipSetDevice(saved); }
+  LazyDevice(const LazyDevice&) = delete;
+  LazyDevice& operator=(const LazyDevice&) = delete;
 };
 
 void parse_credit_env() {
@@ -1116,13 +1151,13 @@ void flush_pending(Peer* pr) {
     pr->waiting_bytes.store(0, std::memory_order_release);
   }
   TraceScope tr(kTrFlush);
-  DeviceScope keep;
-  const bool dev_ok = hipSetDevice(pr->hip_device) == hipSuccess;
+  LazyDevice dev(pr->hip_device);
   std::vector<Pending>& work = pr->work;
   if (g_par.trace) g_tr_calls[kTrRequestsLaunched].fetch_add((int64_t)work.size(), std::memory_order_relaxed);
+  tl_event(3, (uint64_t)work.size());
   size_t i = 0;
   while (i < work.size()) {
-    ncclResult_t rc = dev_ok ? ncclSuccess : ncclUnhandledCudaError;
+    ncclResult_t rc = ncclSuccess;
     size_t span = 1;
     const Pending& p = work[i];
     const uint64_t p_epoch = (p.w.flags & 1u) ? 0 : p.lk->epoch_bytes;
@@ -1140,6 +1175,7 @@ void flush_pending(Peer* pr) {
       }
     }
     if (!by_engine) {
+      if (rc == ncclSuccess && !dev.use()) rc = ncclUnhandledCudaError;   // launches need the staging device current
       seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
       pr->launch_seq.store(seq, std::memory_order_release);   // before anything runs: the completion words never run ahead of it
     }
@@ -1161,6 +1197,7 @@ void flush_pending(Peer* pr) {
         else rc = launch_batch(pr, i, span, bb, false, seq);
       }
     }
+    tl_event(4, ((uint64_t)span << 32) | (by_engine ? 0x80000000ull : 0) | (seq & 0x7fffffffull));
     for (size_t k = i; k < i + span; ++k) {
       Pending& q = work[k];
       if (rc == ncclSuccess) {
@@ -1180,7 +1217,7 @@ void flush_pending(Peer* pr) {
     if (rc != ncclSuccess && !by_engine) {
       // whatever part of the launch was queued is waited for here, so that its number counts as complete and the
       // launches behind it are not held back by one that will never report
-      if (dev_ok) (void)hipStreamSynchronize(pr->stream);
+      if (dev.use()) (void)hipStreamSynchronize(pr->stream);
       uint64_t seen = pr->done_seq.load(std::memory_order_relaxed);
       while (seen < seq && !pr->done_seq.compare_exchange_weak(seen, seq, std::memory_order_release, std::memory_order_relaxed)) {}
     }
@@ -1261,6 +1298,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     p.rreq = rreq;
     sreq->state.store(kStQueued, std::memory_order_release);
     rreq->state.store(kStQueued, std::memory_order_release);
+    tl_event(2, (uint64_t)lk->channelId);
     uint32_t waiting;
     {
       std::lock_guard<std::mutex> g(pr->queue_mu);
@@ -1329,6 +1367,7 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
   fs.rreq = rreq;
   fs.rtype = mh->type;
   fs.rdevice = mh->device;
+  tl_event(1, (uint64_t)lk->channelId);
   fs.w.idx = lk->fifoTail + 1;   // written last: it is what the sender waits for (plugin.cc:1632)
   lk->fifoTail++;
   lk->r_inflight++;
@@ -1474,6 +1513,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     if (rc != ncclSuccess || !complete) return rc;
   }
   if (g_par.trace) g_tr_calls[kTrTestDone].fetch_add(1, std::memory_order_relaxed);
+  tl_event(5, ((uint64_t)lk->channelId << 1) | (r->type == kReqRecv ? 1u : 0u));
   std::lock_guard<std::mutex> g(lk->mu);
   ncclResult_t result = ncclSuccess;
   if (r->fault) {   // failed completion, plugin.cc:1839-1861
@@ -1730,6 +1770,14 @@ int fl_net_host_stats(int64_t* calls_out, int64_t* ns_out, int n) {
     if (ns_out) ns_out[k] = g_tr_ns[k].load(std::memory_order_relaxed);
   }
   return kTrCount;
+}
+
+int fl_net_timeline(void* out, int max_events) {
+  const uint64_t n = g_timeline_n.load(std::memory_order_acquire);
+  const uint64_t have = n < kTimelineCap ? n : kTimelineCap;
+  const uint64_t take = have < (uint64_t)(max_events > 0 ? max_events : 0) ? have : (uint64_t)(max_events > 0 ? max_events : 0);
+  if (out && take) memcpy(out, g_timeline, take * sizeof(TimelineEvent));
+  return (int)have;
 }
 
 int fl_net_flush(void* comm) {

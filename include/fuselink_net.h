@@ -261,6 +261,11 @@ int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, vo
  * launched what waited, 5 launch pairs (time inside the runtime's launch calls and the batch arithmetic before them),
  * 6 requests those passes launched (calls only).  Returns the number of counters. */
 int fl_net_host_stats(int64_t* calls_out, int64_t* ns_out, int n);
+/* Timeline kept under NCCL_FUSELINK_TRACE=2: up to 65536 events of 24 bytes {int64 nanoseconds (monotonic clock), uint32
+ * thread, uint32 event, uint64 value}; events: 1 receive posted (value = channel), 2 send matched (channel), 3 a pass that
+ * launches begins (requests waiting), 4 batch handed over (requests << 32 | bit 31: engine batch | its number),
+ * 5 request seen complete by test (channel << 1 | is-receive).  Copies up to max_events into `out`, returns how many exist. */
+int fl_net_timeline(void* out, int max_events);
 /* Launch whatever waits on the GPU that `comm` stages on, without polling a request. */
 int fl_net_flush(void* comm);
 

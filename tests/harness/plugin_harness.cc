@@ -252,5 +252,20 @@ int main(int argc, char** argv) {
            reqs, (long long)calls[0], ns[0] / 1e3, (long long)calls[1], ns[1] / 1e3, (long long)calls[2], ns[2] / 1e3, (long long)calls[3],
            (long long)calls[4], ns[4] / 1e3, (long long)calls[5], ns[5] / 1e3, calls[5] ? (double)calls[6] / calls[5] : 0.0, calls[5] ? ns[5] / 1e3 / calls[5] : 0.0);
   }
+  // NCCL_FUSELINK_TRACE=2: the timeline of the entry-point events, one line per event, into the file named by FL_TIMELINE_OUT
+  typedef int (*timeline_fn)(void*, int);
+  timeline_fn timeline = (timeline_fn)dlsym(lib, "fl_net_timeline");
+  const char* tl_out = getenv("FL_TIMELINE_OUT");
+  if (timeline && tr && atoi(tr) > 1 && tl_out) {
+    struct Ev { int64_t ns; uint32_t thread, event; uint64_t value; };
+    std::vector<Ev> ev(65536);
+    const int n = timeline(ev.data(), (int)ev.size());
+    FILE* f = fopen(tl_out, "w");
+    if (f) {
+      for (int i = 0; i < n && i < (int)ev.size(); ++i)
+        fprintf(f, "%lld %u %u %llu\n", (long long)(ev[i].ns - ev[0].ns), ev[i].thread, ev[i].event, (unsigned long long)ev[i].value);
+      fclose(f);
+    }
+  }
   return 0;
 }
