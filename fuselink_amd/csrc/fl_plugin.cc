@@ -78,8 +78,8 @@ struct Params {
   // NCCL_FUSELINK_ENGINE=1: batches of small requests go to a resident kernel through a descriptor ring instead of
   // through a launch pair each (flh_engine_*); 0 = every batch is a launch pair
   int engine = 1;
-  int engine_units = 1;          // staging units per lane for each of the engine's window sets
-  int engine_sets = 4;           // window sets the engine's batches rotate through = batches it has in flight at once
+  int engine_units = 2;          // staging units per lane for each of the engine's window sets
+  int engine_sets = 2;           // window sets the engine's batches rotate through = batches it has in flight at once
   int engine_idle_us = 200;      // the engine goes down after this long without work
   int engine_workgroups = 0;     // 0 = the library's default
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
@@ -271,22 +271,27 @@ struct Peer {
   uint32_t* d_done = nullptr;
   uint32_t* h_started = nullptr;    // pinned, device-visible: number of the last launch whose striping kernel has started
   uint32_t* d_started = nullptr;
-  // matched sends that wait for a launch, in arrival order
-  std::mutex queue_mu;
+  // matched sends that wait for a launch, in arrival order.  (Cache lines: what the senders write, what the pollers
+  // read and what only the thread that launches touches are kept apart; polling threads must not slow a launch down by
+  // pulling its lines away.)
+  alignas(64) std::mutex queue_mu;
   std::vector<Pending> pending;
   std::atomic<uint32_t> waiting_reqs{0};
   std::atomic<uint64_t> waiting_bytes{0};
   std::atomic<int64_t> waiting_since{0};   // monotonic nanoseconds at which the oldest waiting send arrived
   // Guards every launch on `stream`, the event ring, the launch numbers, the connections' scheduling state
   // (epoch_bytes, launch counters, last table) and `last`.  Taken before queue_mu, never the other way round.
-  std::mutex launch_mu;
-  std::vector<Pending> work;        // the waiting sends a flush took over (launch_mu)
+  alignas(64) std::mutex launch_mu;
+  alignas(64) std::atomic<bool> launching{false};   // a thread holds launch_mu for a pass: pollers look here before they try the lock
+  alignas(64) std::vector<Pending> work;        // the waiting sends a flush took over (launch_mu)
+  std::vector<Pending> work_sorted; // scratch of the same pass
+  std::vector<bool> work_taken;
   hipEvent_t evring[kEventRing] = {};              // launch n may own slot (n - 1) % kEventRing
   std::atomic<uint64_t> ev_seq[kEventRing] = {};   // the launch whose completion the slot's event stands for (0: none)
-  std::atomic<uint64_t> done_seq{0};               // highest launch number known complete; launches run in order on one stream
+  alignas(64) std::atomic<uint64_t> done_seq{0};   // highest launch number known complete; launches run in order on one stream
   std::atomic<uint64_t> launch_seq{0};             // highest launch number handed out
   std::atomic<uint64_t> last_event_seq{0};         // highest launch whose completion comes from an event, not from the word
-  LaunchInfo last;
+  alignas(64) LaunchInfo last;
   // the lane engine (flh_engine_*): a resident kernel that takes batches of small requests from a descriptor ring.
   // Its batches alternate between two window sets of their own and have their own numbers, tables and headers.
   flh_engine* engine = nullptr;
@@ -295,7 +300,7 @@ struct Peer {
   flh_windows ewins[kEngineSetsMax] = {};
   flh_chunk_desc* d_etable = nullptr;              // kEngineSlots tables of kEngineRows rows
   flh_sched_hdr* d_ehdr = nullptr;                 // kEngineSlots headers
-  std::atomic<uint64_t> engine_submitted{0};       // batches handed to the engine (written under launch_mu)
+  alignas(64) std::atomic<uint64_t> engine_submitted{0};   // batches handed to the engine (written under launch_mu)
 };
 constexpr uint32_t kEngineSlots = 64;              // the engine's descriptor ring
 constexpr uint32_t kEngineRows = 512;              // chunks an engine batch may hold
@@ -975,8 +980,16 @@ bool needs_waves(const flh_windows& wins, const Pending& p, uint64_t epoch_bytes
   uint32_t credits[FLH_MAX_LANES];
   wire_credits(p.lk, p.w, credits);
   const uint64_t chunk = (uint64_t)g_par.chunk;
-  const uint64_t room = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, wins.cap[0], epoch_bytes / chunk) * chunk;
-  return (uint64_t)p.size > room;
+  if ((((uint64_t)p.size + chunk - 1) / chunk) > (uint64_t)g_par.max_wave_chunks) return true;
+  // where the request's chunks land, from the closed form: it travels in one go if no lane outgrows its window
+  FlCreditRow row;
+  fl_row_make(credits, (uint32_t)g_par.lanes, row);
+  uint64_t lane_bytes[FLH_MAX_LANES];
+  uint32_t lane_chunks[FLH_MAX_LANES];
+  fl_row_lane_totals(row, epoch_bytes / chunk, (uint64_t)p.size, chunk, lane_bytes, lane_chunks);
+  for (int l = 0; l < g_par.lanes; ++l)
+    if (lane_bytes[l] > wins.cap[l]) return true;
+  return false;
 }
 
 // May the send travel in an engine batch?  Small requests only (large ones are bound by the GPU, not by the launch),
@@ -1153,6 +1166,23 @@ void flush_pending(Peer* pr) {
   TraceScope tr(kTrFlush);
   LazyDevice dev(pr->hip_device);
   std::vector<Pending>& work = pr->work;
+  if (work.size() > 2) {
+    // Sends of several connections arrive interleaved, and every change of connection opens a segment: bring each
+    // connection's sends together (in the order the connections first appear, each connection's own order kept), so
+    // that a launch holds four connections' requests in four segments instead of closing after eight requests.
+    // Requests of different connections are independent of each other, so the order among them is free.
+    std::vector<Pending>& sorted = pr->work_sorted;
+    sorted.clear();
+    sorted.reserve(work.size());
+    std::vector<bool>& taken = pr->work_taken;
+    taken.assign(work.size(), false);
+    for (size_t a = 0; a < work.size(); ++a) {
+      if (taken[a]) continue;
+      for (size_t b = a; b < work.size(); ++b)
+        if (!taken[b] && work[b].lk == work[a].lk) { sorted.push_back(work[b]); taken[b] = true; }
+    }
+    work.swap(sorted);
+  }
   if (g_par.trace) g_tr_calls[kTrRequestsLaunched].fetch_add((int64_t)work.size(), std::memory_order_relaxed);
   tl_event(3, (uint64_t)work.size());
   size_t i = 0;
@@ -1312,8 +1342,10 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
       if (g_par.batch < 2) {
         std::lock_guard<std::mutex> g(pr->launch_mu);
         flush_pending(pr);
-      } else if (pr->launch_mu.try_lock()) {   // if another thread is launching, the next poll takes care of it
+      } else if (!pr->launching.load(std::memory_order_relaxed) && pr->launch_mu.try_lock()) {   // if another thread is launching, the next poll takes care of it
+        pr->launching.store(true, std::memory_order_relaxed);
         flush_pending(pr);
+        pr->launching.store(false, std::memory_order_relaxed);
         pr->launch_mu.unlock();
       }
     }
@@ -1489,9 +1521,11 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
         pr->waiting_reqs.load(std::memory_order_acquire) < (uint32_t)g_par.batch &&
         tr_now() - pr->waiting_since.load(std::memory_order_relaxed) < g_par.batch_wait_ns)
       go = false;
-    if (go) {
+    if (go && !pr->launching.load(std::memory_order_relaxed)) {
       if (pr->launch_mu.try_lock()) {   // if another thread is launching, it or the next poll takes care of it
+        pr->launching.store(true, std::memory_order_relaxed);
         flush_pending(pr);
+        pr->launching.store(false, std::memory_order_relaxed);
         pr->launch_mu.unlock();
       }
       st = r->state.load(std::memory_order_acquire);
