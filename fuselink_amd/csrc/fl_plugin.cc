@@ -22,7 +22,11 @@
 //          (the completion queue of plugin.cc:1801-1955) and, unlike the reference, reports the byte count of a receive.
 // Staging windows are HIP-VMM mappings from the unit pool, one per lane per GPU, shared by every connection
 // that stages there, bound when device memory is first registered on a send side and reused launch after launch.
+#include <fcntl.h>
 #include <hip/hip_runtime.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
 #include <atomic>
 #include <cstdarg>
@@ -85,6 +89,7 @@ struct Params {
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
   int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
+  int wire = 0;                  // NCCL_FUSELINK_WIRE: 0 = both ends in this process (loopback), 1 = the other end is another process (shared-memory wire)
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
 Params g_par;
@@ -586,6 +591,472 @@ uint32_t wave_chunks(const uint32_t* credits, int lanes, uint64_t chunk, uint64_
 }
 
 // ------------------------------------------------------------------------------------------------
+// shared-memory wire: sender and receiver in different processes (NCCL_FUSELINK_WIRE=shm)
+// ------------------------------------------------------------------------------------------------
+// The reference's two ends are different processes on different hosts: the receiver writes 64-byte descriptors into a
+// FIFO in the sender's memory by RDMA (ncclIbSendFifo, plugin.cc:487-496, 1616-1677), the sender RDMA-writes the payload
+// out of its staged buffer into the receiver's registered memory and completes it with a WRITE_WITH_IMM
+// (plugin.cc:1453-1495), and the 128-byte handle that listen fills carries what connect needs to reach the listener
+// (plugin.cc:425-430, 776-885).  On one GPU the part of that which can be shown is the process boundary: listen creates a
+// POSIX shared-memory object and names it in the handle; connect, in another process, maps it.  The object holds the
+// descriptor FIFO (receiver writes, sender reads), a ring of wave completions (sender writes, receiver reads: the
+// stand-in for the WRITE_WITH_IMM completions) and the IPC handle of the receiver's landing windows.  A send then runs
+// as in the reference's layers: the striping kernel stages the request's chunks in the sender's lane windows (HIP VMM,
+// from the unit pool); the wire copies every lane's staged bytes into the receiver's landing window for that lane,
+// device memory of the receiver's process that the sender has opened through hipIpcOpenMemHandle (an imported VMM
+// allocation would be the closer analogue; this runtime refuses hipMemImportFromShareableHandle for another process's
+// descriptor, so the landing windows are a plain device allocation); the sender publishes the wave; the receiver's
+// reassembly kernel writes the posted buffer from its landing windows and acknowledges.  One wave is on the wire at a
+// time per connection (the landing windows are reused wave by wave), requests complete in order.
+void fill_uniform(flh_uniform_params& u, const uint32_t* credits, uint64_t bytes, uint64_t src_base, uint64_t epoch_bytes, uint32_t tile);
+
+constexpr uint64_t kHandleMagicShm = 0x4655534c53484d31ull;   // "FUSLSHM1"
+constexpr uint32_t kShmCommMagic = 0x464c5343;                // "FLSC"
+constexpr uint32_t kShmReqMagic = 0x464c5352;                 // "FLSR"
+constexpr uint32_t kShmListenMagic = 0x464c534c;              // "FLSL"
+
+struct ShmWave {                   // one wave of chunks that has landed in the receiver's windows
+  std::atomic<uint64_t> seq;       // wave number + 1, written last
+  uint64_t fifo_idx;               // the descriptor (request) it belongs to
+  uint64_t epoch_bytes;            // the connection's credit-epoch prefix the wave was scheduled from
+  uint64_t offset;                 // byte offset of the wave in the request
+  uint64_t bytes;
+  uint32_t last;                   // the request's last wave
+  uint32_t pad;
+};
+struct ShmWire {
+  uint64_t magic;
+  uint32_t lanes;
+  uint32_t channelId;
+  std::atomic<uint32_t> connected, accepted, send_closed, recv_closed;
+  std::atomic<uint32_t> landing_ready;
+  uint32_t pad0;
+  uint64_t landing_bytes_per_lane;
+  hipIpcMemHandle_t landing;       // lanes x landing_bytes_per_lane of the receiver's device memory
+  alignas(64) FifoWire fifo[FL_NET_MAX_REQUESTS];          // plugin.cc:487-496: written by the receiver, idx last
+  alignas(64) ShmWave wave[FL_NET_MAX_REQUESTS];
+  alignas(64) std::atomic<uint64_t> waves_consumed;        // receiver: waves reassembled so far (the landing windows are free again)
+};
+
+struct ShmRequest {
+  uint32_t magic = 0;
+  int type = kReqUnused;
+  struct ShmComm* comm = nullptr;
+  uint64_t fifo_idx = 0;           // 1-based descriptor number
+  // sender
+  const uint8_t* src = nullptr;
+  uint64_t size = 0, sent = 0;     // bytes of the request, bytes whose waves have been published
+  uint64_t wave_no = 0;            // number of the wave in flight (1-based), 0 = none
+  uint64_t wave_bytes = 0, wave_epoch = 0;
+  int phase = 0;                   // sender: 0 idle, 1 stripe + wire queued, 2 published; receiver: 0 waiting for a wave, 1 reassembly queued
+  uint32_t credits[FLH_MAX_LANES] = {};
+  bool refresh = false;
+  // receiver
+  uint8_t* dst = nullptr;
+  uint64_t received = 0;
+  int done_size = 0;
+};
+
+struct ShmComm {
+  uint32_t magic = kShmCommMagic;
+  int is_send = 0;
+  int dev = 0;
+  ShmWire* w = nullptr;
+  char name[64] = "";
+  bool owner = false;              // the receiver created the object and unlinks it
+  std::mutex mu;
+  ShmRequest reqs[FL_NET_MAX_REQUESTS];
+  uint64_t fifoHead = 0, fifoTail = 0;       // sender: next descriptor to match; receiver: next to post
+  std::deque<ShmRequest*> active;            // requests in flight, in order; only the first makes progress
+  uint64_t epoch_bytes = 0;                  // sender: the scheduler's carried prefix
+  uint64_t waves_published = 0, waves_seen = 0;
+  int64_t r_finished = 0, r_inflight = 0;
+  int fuselink_offset = -1;
+  uint8_t credits[FL_NET_MAX_LANES] = {};
+  bool have_decision = false;
+  // GPU side
+  bool gpu_ready = false;
+  int hip_device = -1;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev = nullptr;
+  flh_window* win[FL_NET_MAX_LANES] = {};    // sender: staging windows
+  flh_windows wins = {};
+  uint8_t* landing = nullptr;                // receiver: its allocation; sender: the same memory opened through IPC
+  flh_windows landing_wins = {};
+  flh_chunk_desc* d_table = nullptr;
+  flh_sched_hdr* d_hdr = nullptr;
+  int32_t *h_status = nullptr, *d_status = nullptr;
+};
+
+struct ShmListen {
+  uint32_t magic = kShmListenMagic;
+  int dev = 0;
+  ShmComm* comm = nullptr;         // becomes the recv comm at accept
+};
+
+std::atomic<uint64_t> g_shm_counter{0};
+
+void shm_comm_free(ShmComm* c) {
+  if (c->stream) {
+    DeviceScope keep;
+    (void)hipSetDevice(c->hip_device);
+    (void)hipStreamSynchronize(c->stream);
+    for (int l = 0; l < FL_NET_MAX_LANES; ++l) if (c->win[l]) (void)flh_window_destroy(c->win[l]);
+    if (c->landing) { if (c->is_send) (void)hipIpcCloseMemHandle(c->landing); else (void)hipFree(c->landing); }
+    if (c->d_table) (void)hipFree(c->d_table);
+    if (c->d_hdr) (void)hipFree(c->d_hdr);
+    if (c->h_status) (void)hipHostFree(c->h_status);
+    if (c->ev) (void)hipEventDestroy(c->ev);
+    (void)hipStreamDestroy(c->stream);
+  }
+  if (c->w) munmap(c->w, sizeof(ShmWire));
+  if (c->owner && c->name[0]) shm_unlink(c->name);
+  delete c;
+}
+
+ncclResult_t shm_listen(int dev, void* opaqueHandle, void** listenComm) {
+  ShmListen* lc = new (std::nothrow) ShmListen();
+  ShmComm* c = new (std::nothrow) ShmComm();
+  if (!lc || !c) { delete lc; delete c; return ncclSystemError; }
+  snprintf(c->name, sizeof(c->name), "/fuselink-wire-%d-%llu", (int)getpid(), (unsigned long long)g_shm_counter.fetch_add(1));
+  int fd = shm_open(c->name, O_CREAT | O_EXCL | O_RDWR, 0600);
+  if (fd < 0 || ftruncate(fd, sizeof(ShmWire)) != 0) { if (fd >= 0) close(fd); FL_WARN("NET/FuseLink : shm_open(%s) failed", c->name); delete lc; delete c; return ncclSystemError; }
+  void* p = mmap(nullptr, sizeof(ShmWire), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+  close(fd);
+  if (p == MAP_FAILED) { shm_unlink(c->name); delete lc; delete c; return ncclSystemError; }
+  memset(p, 0, sizeof(ShmWire));
+  c->w = (ShmWire*)p;
+  c->owner = true;
+  c->dev = dev;
+  c->w->lanes = (uint32_t)g_par.lanes;
+  {
+    std::lock_guard<std::mutex> g(g_reg_mu);
+    c->w->channelId = (uint32_t)g_channel_counter++;
+  }
+  c->w->magic = kHandleMagicShm;
+  lc->dev = dev;
+  lc->comm = c;
+  Handle* h = (Handle*)opaqueHandle;
+  memset(h, 0, NCCL_NET_HANDLE_MAXSIZE);
+  h->magic = kHandleMagicShm;
+  h->channelId = (int32_t)c->w->channelId;
+  h->dev = dev;
+  // the object's name travels in the handle, as the listener's address does in the reference's (plugin.cc:425-430)
+  static_assert(sizeof(Handle) + 64 <= NCCL_NET_HANDLE_MAXSIZE, "the name must fit behind the fixed part of the handle");
+  memcpy((char*)opaqueHandle + sizeof(Handle), c->name, sizeof(c->name));
+  *listenComm = lc;
+  return ncclSuccess;
+}
+
+ncclResult_t shm_connect(int dev, void* opaqueHandle, void** sendComm) {
+  Handle* h = (Handle*)opaqueHandle;
+  *sendComm = nullptr;
+  ShmComm* c = (ShmComm*)h->stage_link;
+  if (h->stage == 0) {
+    char name[64];
+    memcpy(name, (char*)opaqueHandle + sizeof(Handle), sizeof(name));
+    name[63] = 0;
+    int fd = shm_open(name, O_RDWR, 0600);
+    if (fd < 0) { FL_WARN("NET/FuseLink : connect: no shared-memory object %s (is the listener alive?)", name); return ncclSystemError; }
+    void* p = mmap(nullptr, sizeof(ShmWire), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    close(fd);
+    if (p == MAP_FAILED) return ncclSystemError;
+    c = new (std::nothrow) ShmComm();
+    if (!c) { munmap(p, sizeof(ShmWire)); return ncclSystemError; }
+    c->w = (ShmWire*)p;
+    if (c->w->magic != kHandleMagicShm || (int)c->w->lanes != g_par.lanes) {
+      FL_WARN("NET/FuseLink : connect: the listener runs %u lanes, this side %d", c->w->lanes, g_par.lanes);
+      shm_comm_free(c);
+      return ncclInvalidUsage;
+    }
+    c->is_send = 1;
+    c->dev = dev;
+    memcpy(c->name, name, sizeof(name));
+    c->w->connected.store(1, std::memory_order_release);
+    h->stage = 1;
+    h->stage_link = c;
+    return ncclSuccess;
+  }
+  if (!c->w->accepted.load(std::memory_order_acquire)) return ncclSuccess;   // accept has not happened yet
+  h->stage = 0;
+  h->stage_link = nullptr;
+  *sendComm = c;
+  return ncclSuccess;
+}
+
+ncclResult_t shm_accept(ShmListen* lc, void** recvComm) {
+  *recvComm = nullptr;
+  ShmComm* c = lc->comm;
+  if (!c || !c->w->connected.load(std::memory_order_acquire)) return ncclSuccess;   // nobody connected yet
+  c->w->accepted.store(1, std::memory_order_release);
+  shm_unlink(c->name);   // both ends hold their mapping: the name is no longer needed and cannot leak
+  c->owner = false;
+  lc->comm = nullptr;
+  *recvComm = c;
+  return ncclSuccess;
+}
+
+// stream, status word, table buffers; the sender's staging windows or the receiver's landing windows
+ncclResult_t shm_setup_gpu(ShmComm* c, int device) {
+  if (c->gpu_ready) return ncclSuccess;
+  if (c->stream) return ncclInternalError;   // failed earlier
+  DeviceScope keep;
+  c->hip_device = device;
+  FL_HIPCHECK(hipSetDevice(device));
+  FL_HIPCHECK(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+  FL_HIPCHECK(hipEventCreateWithFlags(&c->ev, hipEventDisableTiming));
+  FL_HIPCHECK(hipHostMalloc((void**)&c->h_status, 64, hipHostMallocMapped));
+  memset(c->h_status, 0, 64);
+  FL_HIPCHECK(hipHostGetDevicePointer((void**)&c->d_status, c->h_status, 0));
+  const uint64_t cap = (uint64_t)g_par.window_units * FLH_UNIT_BYTES;
+  if (c->is_send) {
+    flh_pool* pool = nullptr;
+    ncclResult_t rc = ensure_pool(device, &pool);
+    if (rc != ncclSuccess) return rc;
+    c->wins.n_lanes = (uint32_t)g_par.lanes;
+    for (int l = 0; l < g_par.lanes; ++l) {
+      FL_FLHCHECK(flh_window_create(pool, cap, &c->win[l]));
+      FL_FLHCHECK(flh_window_bind(c->win[l], cap));
+      c->wins.base[l] = flh_window_base(c->win[l]);
+      c->wins.cap[l] = flh_window_bound_bytes(c->win[l]);
+    }
+    FL_HIPCHECK(hipMalloc((void**)&c->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
+    FL_HIPCHECK(hipMalloc((void**)&c->d_hdr, sizeof(flh_sched_hdr)));
+  } else {
+    FL_HIPCHECK(hipMalloc((void**)&c->landing, cap * (uint64_t)g_par.lanes));
+    FL_HIPCHECK(hipIpcGetMemHandle(&c->w->landing, c->landing));
+    c->w->landing_bytes_per_lane = cap;
+    c->w->landing_ready.store(1, std::memory_order_release);
+  }
+  if (!c->is_send) {
+    c->landing_wins.n_lanes = (uint32_t)g_par.lanes;
+    for (int l = 0; l < g_par.lanes; ++l) { c->landing_wins.base[l] = c->landing + (uint64_t)l * cap; c->landing_wins.cap[l] = cap; }
+  }
+  c->gpu_ready = true;
+  return ncclSuccess;
+}
+
+ShmRequest* shm_get_request(ShmComm* c, int type) {
+  for (int i = 0; i < FL_NET_MAX_REQUESTS; ++i) {
+    ShmRequest* r = &c->reqs[i];
+    if (r->type == kReqUnused) {
+      *r = ShmRequest();
+      r->magic = kShmReqMagic;
+      r->type = type;
+      r->comm = c;
+      return r;
+    }
+  }
+  FL_WARN("NET/FuseLink : unable to allocate requests");
+  return nullptr;
+}
+
+// Credit row a descriptor asks for (both ends derive it from the descriptor alone, so they agree).
+void shm_wire_credits(const ShmComm* c, const FifoWire& w, uint32_t* credits) {
+  for (int l = 0; l < FLH_MAX_LANES; ++l) credits[l] = 0;
+  if (w.fuselink_offset == -2) { for (int l = 0; l < g_par.lanes; ++l) credits[l] = w.credits[l]; }
+  else credits[w.fuselink_offset >= 0 ? w.fuselink_offset % g_par.lanes : (int)(c->w->channelId % (uint32_t)g_par.lanes)] = 1;
+}
+
+ncclResult_t shm_irecv(ShmComm* c, void* data, int size, int tag, MemHandle* mh, void** request) {
+  *request = nullptr;
+  if (mh->type != NCCL_PTR_CUDA) { FL_WARN("NET/FuseLink : the shared-memory wire carries device memory only"); return ncclInvalidUsage; }
+  std::lock_guard<std::mutex> g(c->mu);
+  ncclResult_t rc = shm_setup_gpu(c, mh->device);
+  if (rc != ncclSuccess) return rc;
+  bool refreshed = false;
+  if (c->r_finished % g_par.refresh_batch == 0 || !c->have_decision) {   // plugin.cc:1700-1712
+    if (c->r_inflight != 0) return ncclSuccess;
+    if (g_par.policy == 0) {
+      c->fuselink_offset = (int)(c->w->channelId % (uint32_t)g_par.lanes);
+    } else {
+      c->fuselink_offset = -2;
+      current_credits(c->dev % g_par.lanes, c->credits);
+    }
+    c->have_decision = true;
+    refreshed = true;
+  }
+  if ((int)c->active.size() >= FL_NET_MAX_REQUESTS - 1) return ncclSuccess;   // the descriptor ring is full
+  ShmRequest* r = shm_get_request(c, kReqRecv);
+  if (!r) return ncclInternalError;
+  r->dst = (uint8_t*)data;
+  r->size = (uint64_t)size;
+  r->fifo_idx = c->fifoTail + 1;
+  FifoWire& w = c->w->fifo[c->fifoTail % FL_NET_MAX_REQUESTS];
+  w.addr = (uint64_t)(uintptr_t)data;
+  w.size = size;
+  w.rkey = 1;
+  w.nreqs = 1;
+  w.tag = (uint32_t)tag;
+  w.fuselink_offset = c->fuselink_offset;
+  memcpy(w.credits, c->credits, sizeof(w.credits));
+  w.flags = refreshed ? 1u : 0u;
+  shm_wire_credits(c, w, r->credits);
+  __atomic_store_n(&w.idx, c->fifoTail + 1, __ATOMIC_RELEASE);   // written last: it is what the sender waits for (plugin.cc:1632)
+  c->fifoTail++;
+  c->r_inflight++;
+  c->active.push_back(r);
+  *request = r;
+  return ncclSuccess;
+}
+
+ncclResult_t shm_isend(ShmComm* c, void* data, int size, int tag, MemHandle* mh, void** request) {
+  *request = nullptr;
+  if (mh->type != NCCL_PTR_CUDA) { FL_WARN("NET/FuseLink : the shared-memory wire carries device memory only"); return ncclInvalidUsage; }
+  std::lock_guard<std::mutex> g(c->mu);
+  FifoWire& fw = c->w->fifo[c->fifoHead % FL_NET_MAX_REQUESTS];
+  if (__atomic_load_n(&fw.idx, __ATOMIC_ACQUIRE) != c->fifoHead + 1) return ncclSuccess;   // not posted yet (plugin.cc:1510-1514)
+  if (fw.nreqs != 1) return ncclInternalError;
+  if (fw.tag != (uint32_t)tag) return ncclSuccess;
+  if (size > fw.size) { FL_WARN("NET/FuseLink : req tag %x collective mismatch error, local size %d remote size %d", tag, size, fw.size); return ncclInvalidUsage; }
+  ncclResult_t rc = shm_setup_gpu(c, mh->device);
+  if (rc != ncclSuccess) return rc;
+  if (!c->landing) {   // the receiver's landing windows, once it has set them up
+    if (!c->w->landing_ready.load(std::memory_order_acquire)) return ncclSuccess;
+    DeviceScope keep;
+    FL_HIPCHECK(hipSetDevice(c->hip_device));
+    FL_HIPCHECK(hipIpcOpenMemHandle((void**)&c->landing, c->w->landing, hipIpcMemLazyEnablePeerAccess));
+    c->landing_wins.n_lanes = (uint32_t)g_par.lanes;
+    for (int l = 0; l < g_par.lanes; ++l) {
+      c->landing_wins.base[l] = c->landing + (uint64_t)l * c->w->landing_bytes_per_lane;
+      c->landing_wins.cap[l] = c->w->landing_bytes_per_lane;
+    }
+    if (c->w->landing_bytes_per_lane < c->wins.cap[0]) { FL_WARN("NET/FuseLink : the receiver's landing windows are smaller than the staging windows"); return ncclInvalidUsage; }
+  }
+  ShmRequest* r = shm_get_request(c, kReqSend);
+  if (!r) return ncclInternalError;
+  r->src = (const uint8_t*)data;
+  r->size = (uint64_t)size;
+  r->fifo_idx = c->fifoHead + 1;
+  r->refresh = (fw.flags & 1u) != 0;
+  shm_wire_credits(c, fw, r->credits);
+  memset((void*)&fw, 0, sizeof(FifoWire));   // plugin.cc:1605
+  c->fifoHead++;
+  c->active.push_back(r);
+  *request = r;
+  return ncclSuccess;
+}
+
+// One step of the connection's first request in flight (c->mu held).
+ncclResult_t shm_progress_send(ShmComm* c, ShmRequest* r) {
+  const uint64_t chunk = (uint64_t)g_par.chunk;
+  DeviceScope keep;
+  if (r->phase == 0) {
+    if (r->size == 0 && r->sent == 0 && r->wave_no == 0) {
+      // nothing to move: the completion alone travels
+    } else if (r->sent >= r->size) {
+      return ncclSuccess;
+    }
+    // the landing windows hold one wave: the previous one must have been reassembled
+    if (c->w->waves_consumed.load(std::memory_order_acquire) < c->waves_published) return ncclSuccess;
+    if (r->refresh && r->sent == 0) c->epoch_bytes = 0;
+    uint64_t wave = (uint64_t)wave_chunks(r->credits, g_par.lanes, chunk, c->wins.cap[0], c->epoch_bytes / chunk) * chunk;
+    if (wave > r->size - r->sent) wave = r->size - r->sent;
+    FL_HIPCHECK(hipSetDevice(c->hip_device));
+    if (wave) {
+      flh_uniform_params u;
+      fill_uniform(u, r->credits, wave, r->sent, c->epoch_bytes, FLH_TILE_BYTES);
+      FL_FLHCHECK(flh_stripe_uniform(r->src, r->size, &c->wins, &u, c->d_table, c->d_hdr, c->d_status, c->stream));
+      // the wire: every lane's staged bytes into the receiver's landing window for that lane
+      FlCreditRow row;
+      fl_row_make(r->credits, (uint32_t)g_par.lanes, row);
+      uint64_t lane_bytes[FLH_MAX_LANES];
+      uint32_t lane_chunks[FLH_MAX_LANES];
+      fl_row_lane_totals(row, c->epoch_bytes / chunk, wave, chunk, lane_bytes, lane_chunks);
+      for (int l = 0; l < g_par.lanes; ++l)
+        if (lane_bytes[l]) FL_FLHCHECK(flh_copy(c->landing_wins.base[l], c->wins.base[l], lane_bytes[l], c->stream));
+    }
+    FL_HIPCHECK(hipEventRecord(c->ev, c->stream));
+    r->wave_bytes = wave;
+    r->wave_epoch = c->epoch_bytes;
+    r->phase = 1;
+    return ncclSuccess;
+  }
+  if (r->phase == 1) {
+    hipError_t e = hipEventQuery(c->ev);
+    if (e == hipErrorNotReady) return ncclSuccess;
+    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+    if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its staging window (status %d)", *c->h_status); return ncclInternalError; }
+    // publish the wave: the stand-in for the WRITE_WITH_IMM completion (plugin.cc:1453-1465)
+    ShmWave& wv = c->w->wave[c->waves_published % FL_NET_MAX_REQUESTS];
+    wv.fifo_idx = r->fifo_idx;
+    wv.epoch_bytes = r->wave_epoch;
+    wv.offset = r->sent;
+    wv.bytes = r->wave_bytes;
+    wv.last = r->sent + r->wave_bytes >= r->size ? 1u : 0u;
+    c->waves_published++;
+    wv.seq.store(c->waves_published, std::memory_order_release);
+    c->epoch_bytes += r->wave_bytes;
+    r->sent += r->wave_bytes;
+    r->wave_no = c->waves_published;
+    r->phase = r->sent >= r->size ? 2 : 0;
+    return ncclSuccess;
+  }
+  return ncclSuccess;
+}
+
+ncclResult_t shm_progress_recv(ShmComm* c, ShmRequest* r) {
+  DeviceScope keep;
+  if (r->phase == 0) {
+    ShmWave& wv = c->w->wave[c->waves_seen % FL_NET_MAX_REQUESTS];
+    if (wv.seq.load(std::memory_order_acquire) != c->waves_seen + 1) return ncclSuccess;   // nothing has landed yet
+    if (wv.fifo_idx != r->fifo_idx) { FL_WARN("NET/FuseLink : a wave of request %llu arrived while %llu is first in line", (unsigned long long)wv.fifo_idx, (unsigned long long)r->fifo_idx); return ncclInternalError; }
+    if (wv.offset + wv.bytes > r->size) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
+    FL_HIPCHECK(hipSetDevice(c->hip_device));
+    if (wv.bytes) {
+      // the credit row this receiver put into the descriptor: the reassembly launch derives the same lanes and offsets
+      flh_uniform_params u;
+      fill_uniform(u, r->credits, wv.bytes, wv.offset, wv.epoch_bytes, FLH_TILE_BYTES);
+      FL_FLHCHECK(flh_reassemble_uniform(r->dst, r->size, &c->landing_wins, &u, c->d_status, c->stream));
+    }
+    FL_HIPCHECK(hipEventRecord(c->ev, c->stream));
+    r->wave_bytes = wv.bytes;
+    r->wave_no = wv.last;
+    r->phase = 1;
+    return ncclSuccess;
+  }
+  hipError_t e = hipEventQuery(c->ev);
+  if (e == hipErrorNotReady) return ncclSuccess;
+  if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+  if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its landing window or buffer (status %d)", *c->h_status); return ncclInternalError; }
+  r->received += r->wave_bytes;
+  c->waves_seen++;
+  c->w->waves_consumed.store(c->waves_seen, std::memory_order_release);   // the landing windows are free again
+  r->phase = r->wave_no ? 2 : 0;
+  return ncclSuccess;
+}
+
+ncclResult_t shm_test(ShmRequest* r, int* done, int* sizes) {
+  *done = 0;
+  ShmComm* c = r->comm;
+  std::lock_guard<std::mutex> g(c->mu);
+  if (c->active.empty() || c->active.front() != r) {
+    // requests complete in order: the first in line is the one that moves
+    if (!c->active.empty()) {
+      ShmRequest* head = c->active.front();
+      ncclResult_t rc = head->type == kReqSend ? shm_progress_send(c, head) : shm_progress_recv(c, head);
+      if (rc != ncclSuccess) return rc;
+    }
+    return ncclSuccess;
+  }
+  ncclResult_t rc = r->type == kReqSend ? shm_progress_send(c, r) : shm_progress_recv(c, r);
+  if (rc != ncclSuccess) return rc;
+  if (r->phase != 2) return ncclSuccess;
+  if (r->type == kReqSend) {
+    // the send is complete once its last wave has been taken out of the landing windows
+    if (c->w->waves_consumed.load(std::memory_order_acquire) < r->wave_no) return ncclSuccess;
+  } else {
+    c->r_finished++;
+    c->r_inflight--;
+    if (sizes) sizes[0] = (int)r->received;
+  }
+  c->active.pop_front();
+  r->type = kReqUnused;
+  *done = 1;
+  return ncclSuccess;
+}
+
+// ------------------------------------------------------------------------------------------------
 // plugin entry points (v8 signatures; v7 / v6 adapt)
 // ------------------------------------------------------------------------------------------------
 ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
@@ -609,6 +1080,10 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.small_tile = (int)fl_param("FUSELINK_SMALL_TILE", g_par.small_tile);
   if (g_par.small_tile < 0 || g_par.small_tile % 128) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_SMALL_TILE must be a multiple of 128"); return ncclInvalidArgument; }
   g_par.trace = (int)fl_param("FUSELINK_TRACE", g_par.trace);
+  {
+    const char* wv = getenv("NCCL_FUSELINK_WIRE");
+    g_par.wire = wv && (!strcmp(wv, "shm") || !strcmp(wv, "1")) ? 1 : 0;
+  }
   g_par.engine = (int)fl_param("FUSELINK_ENGINE", g_par.engine);
   g_par.engine_units = (int)fl_param("FUSELINK_ENGINE_UNITS", g_par.engine_units);
   g_par.engine_idle_us = (int)fl_param("FUSELINK_ENGINE_IDLE_US", g_par.engine_idle_us);
@@ -673,6 +1148,7 @@ ncclResult_t fl_get_properties_v8(int dev, ncclNetProperties_v8_t* props) {
 
 ncclResult_t fl_listen(int dev, void* opaqueHandle, void** listenComm) {
   if (!opaqueHandle || !listenComm || dev < 0 || dev >= g_par.lanes) return ncclInvalidArgument;
+  if (g_par.wire == 1) return shm_listen(dev, opaqueHandle, listenComm);
   ListenComm* lc = new (std::nothrow) ListenComm();
   if (!lc) return ncclSystemError;
   Handle* h = (Handle*)opaqueHandle;
@@ -699,6 +1175,7 @@ ncclResult_t fl_connect(int dev, void* opaqueHandle, void** sendComm, ncclNetDev
   if (!opaqueHandle || !sendComm || dev < 0 || dev >= g_par.lanes) return ncclInvalidArgument;
   Handle* h = (Handle*)opaqueHandle;
   *sendComm = nullptr;
+  if (h->magic == kHandleMagicShm) return shm_connect(dev, opaqueHandle, sendComm);
   if (h->magic != kHandleMagic) { FL_WARN("NET/FuseLink : connect with a handle that listen did not produce"); return ncclInternalError; }
   if (h->stage == 0) {
     Link* lk = new (std::nothrow) Link();
@@ -742,6 +1219,7 @@ ncclResult_t fl_accept(void* listenComm, void** recvComm, ncclNetDeviceHandle_v8
   if (!listenComm || !recvComm) return ncclInvalidArgument;
   ListenComm* lc = (ListenComm*)listenComm;
   *recvComm = nullptr;
+  if (lc->magic == kShmListenMagic) return shm_accept((ShmListen*)listenComm, recvComm);
   Link* lk = nullptr;
   {
     std::lock_guard<std::mutex> g(g_reg_mu);
@@ -764,7 +1242,8 @@ ncclResult_t fl_accept(void* listenComm, void** recvComm, ncclNetDeviceHandle_v8
 ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uint64_t /*offset*/, int /*fd*/, void** mhandle) {
   if (!comm || !data || !mhandle || size == 0) return ncclInvalidArgument;
   Comm* c = (Comm*)comm;
-  if (c->magic != kCommMagic) return ncclInvalidArgument;
+  const bool shm = c->magic == kShmCommMagic;   // the other end is another process: staging is the comm's own
+  if (c->magic != kCommMagic && !shm) return ncclInvalidArgument;
   *mhandle = nullptr;
   MemHandle* mh = new (std::nothrow) MemHandle();
   if (!mh) return ncclSystemError;
@@ -790,7 +1269,7 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
     if (frc < 0) { delete mh; FL_WARN("NET/FuseLink : region: %s", flh_last_error()); return ncclInternalError; }
     mh->start_addr = (uintptr_t)base;
     mh->size = bsz;
-    if (c->is_send) {  // staging is bound at registration time, not on the request path
+    if (c->is_send && !shm) {  // staging is bound at registration time, not on the request path
       std::lock_guard<std::mutex> g(c->link->mu);
       rc = attach_peer(c->link, mh->device);
       if (rc != ncclSuccess) { (void)flh_region_release(mh->region); delete mh; return rc; }
@@ -1260,6 +1739,10 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
   if (!sendComm || !request || !mhandle || size < 0 || (size && !data)) return ncclInvalidArgument;
   Comm* c = (Comm*)sendComm;
   MemHandle* mh = (MemHandle*)mhandle;
+  if (c->magic == kShmCommMagic && mh->magic == kMhMagic && ((ShmComm*)sendComm)->is_send) {
+    if (!request || size < 0 || (!data && size > 0)) return ncclInvalidArgument;
+    return shm_isend((ShmComm*)sendComm, data, size, tag, mh, request);
+  }
   if (c->magic != kCommMagic || !c->is_send || mh->magic != kMhMagic) return ncclInvalidArgument;
   Link* lk = c->link;
   *request = nullptr;
@@ -1357,13 +1840,15 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
 ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags, void** mhandles, void** request) {
   if (!recvComm || !request || !data || !sizes || !tags || !mhandles) return ncclInvalidArgument;
   Comm* c = (Comm*)recvComm;
-  if (c->magic != kCommMagic || c->is_send) return ncclInvalidArgument;
+  const bool shm = c->magic == kShmCommMagic;
+  if ((c->magic != kCommMagic && !shm) || c->is_send) return ncclInvalidArgument;
   *request = nullptr;
   if (n > FL_NET_MAX_RECVS) return ncclInternalError;                       // plugin.cc:1683
   if (n != 1) { FL_WARN("NET/FuseLink: multi recv not allowed"); return ncclInternalError; }  // plugin.cc:1873-1880
   MemHandle* mh = (MemHandle*)mhandles[0];
   if (!mh || mh->magic != kMhMagic || sizes[0] < 0 || !data[0]) return ncclInvalidArgument;
   if (sizes[0] && !in_handle(mh, data[0], (size_t)sizes[0])) { FL_WARN("NET/FuseLink : receive buffer outside its registration"); return ncclInvalidArgument; }
+  if (shm) return shm_irecv((ShmComm*)recvComm, data[0], sizes[0], tags[0], mh, request);
   Link* lk = c->link;
   TraceScope tr(kTrIrecv);
   std::lock_guard<std::mutex> g(lk->mu);
@@ -1497,6 +1982,7 @@ uint64_t launches_in_queue(Peer* pr) {
 
 ncclResult_t fl_test(void* request, int* done, int* sizes) {
   if (!request || !done) return ncclInvalidArgument;
+  if (*(const uint32_t*)request == kShmReqMagic) return shm_test((ShmRequest*)request, done, sizes);   // a Request starts with its small type code
   Request* r = (Request*)request;
   if (r->magic != kReqMagic || r->type == kReqUnused) { FL_WARN("NET/FuseLink : test on a request that is not in flight"); return ncclInternalError; }
   *done = 0;
@@ -1579,6 +2065,13 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
 ncclResult_t close_comm(void* comm, int want_send) {
   Comm* c = (Comm*)comm;
   if (!c) return ncclSuccess;
+  if (c->magic == kShmCommMagic && c->is_send == want_send) {
+    ShmComm* sc = (ShmComm*)comm;
+    (want_send ? sc->w->send_closed : sc->w->recv_closed).store(1, std::memory_order_release);
+    sc->magic = 0;
+    shm_comm_free(sc);
+    return ncclSuccess;
+  }
   if (c->magic != kCommMagic || c->is_send != want_send) return ncclInvalidArgument;
   Link* lk = c->link;
   c->magic = 0;
@@ -1592,6 +2085,13 @@ ncclResult_t fl_close_recv(void* recvComm) { return close_comm(recvComm, 0); }
 ncclResult_t fl_close_listen(void* listenComm) {
   ListenComm* lc = (ListenComm*)listenComm;
   if (!lc) return ncclSuccess;
+  if (lc->magic == kShmListenMagic) {
+    ShmListen* sl = (ShmListen*)listenComm;
+    if (sl->comm) shm_comm_free(sl->comm);   // never accepted: the object goes with it
+    sl->magic = 0;
+    delete sl;
+    return ncclSuccess;
+  }
   std::vector<Link*> orphans;
   {
     std::lock_guard<std::mutex> g(g_reg_mu);

@@ -4,7 +4,12 @@
 // number of requests in flight.  Verifies the received buffer byte for byte and prints one JSON line.
 //
 //   plugin_harness <lib.so> [--bytes N] [--request N] [--inflight K] [--iters I] [--host] [--version 6|7|8] [--connections C]
-//                  [--handoff batch,blocks_per_req,layers,kv_heads,block_size,head_dim]
+//                  [--handoff batch,blocks_per_req,layers,kv_heads,block_size,head_dim] [--two-process]
+// With --two-process the receiver is a child process forked before either side has touched the GPU or loaded the plugin:
+// the child listens and sends the 128-byte handle to the parent over a socket pair (NCCL's bootstrap does that between
+// ranks), the parent connects with it, and from then on the two processes share nothing but what the plugin itself set up
+// behind the handle (NCCL_FUSELINK_WIRE=shm is set for both).  The child checks what it received and reports through its
+// exit status.
 // With --connections C, C connections run concurrently, each with its own pair of proxy threads and buffers; every
 // iteration starts on all of them together and is timed from the first start to the last finish, and the received
 // buffers are compared only once all connections have finished it.
@@ -14,6 +19,10 @@
 // counts (int64 per request) -- each cut into --request sized pieces as NCCL's proxy would.
 #include <dlfcn.h>
 #include <hip/hip_runtime.h>
+#include <signal.h>
+#include <sys/socket.h>
+#include <sys/wait.h>
+#include <unistd.h>
 
 #include <atomic>
 #include <chrono>
@@ -170,10 +179,186 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
   (void)bytes;
 }
 
+// ---- two processes ------------------------------------------------------------------------------------------------
+static void fill_pattern(std::vector<uint8_t>& p, int iteration) {
+  uint64_t x = 88172645463325252ull + 104729ull * (uint64_t)iteration;
+  for (size_t i = 0; i < p.size(); ++i) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; p[i] = (uint8_t)x; }
+}
+static void sock_write(int fd, const void* p, size_t n) {
+  if (write(fd, p, n) != (ssize_t)n) { fprintf(stderr, "socket write failed\n"); exit(6); }
+}
+// blocking read with a deadline, so that neither process outlives the other by more than that
+static void sock_read(int fd, void* p, size_t n, double seconds) {
+  const auto t0 = std::chrono::steady_clock::now();
+  size_t got = 0;
+  while (got < n) {
+    ssize_t k = recv(fd, (char*)p + got, n - got, MSG_DONTWAIT);
+    if (k > 0) { got += (size_t)k; continue; }
+    if (k == 0) { fprintf(stderr, "the other process closed its end\n"); exit(6); }
+    if (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > seconds) { fprintf(stderr, "timed out waiting for the other process\n"); exit(6); }
+    usleep(200);
+  }
+}
+static ncclNet_v8_t* open_plugin(const char* path) {
+  void* lib = dlopen(path, RTLD_NOW | RTLD_LOCAL);
+  if (!lib) { fprintf(stderr, "dlopen: %s\n", dlerror()); exit(1); }
+  ncclNet_v8_t* net8 = (ncclNet_v8_t*)dlsym(lib, "ncclNetPlugin_v8");
+  if (!net8) { fprintf(stderr, "plugin symbols missing\n"); exit(1); }
+  CHECK(net8->init(logger));
+  int ndev = 0;
+  CHECK(net8->devices(&ndev));
+  return net8;
+}
+static const double kDeadline = 90.0;   // seconds any one wait may last
+struct Deadline {
+  std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+  void check(const char* what) const {
+    if (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > kDeadline) { fprintf(stderr, "timed out: %s\n", what); exit(6); }
+  }
+};
+
+static int receiver_process(const char* path, int sock, size_t bytes, size_t request, int inflight, int iters) {
+  ncclNet_v8_t* net = open_plugin(path);
+  char handle[NCCL_NET_HANDLE_MAXSIZE];
+  void *lcomm = nullptr, *rcomm = nullptr;
+  CHECK(net->listen(0, handle, &lcomm));
+  sock_write(sock, handle, sizeof(handle));
+  for (Deadline d; !rcomm; d.check("accept")) { CHECK(net->accept(lcomm, &rcomm, nullptr)); if (!rcomm) usleep(100); }
+  HIP(hipSetDevice(0));
+  uint8_t* dst = nullptr;
+  void* mh = nullptr;
+  HIP(hipMalloc((void**)&dst, bytes));
+  HIP(hipMemset(dst, 0, bytes));
+  CHECK(net->regMr(rcomm, dst, bytes, NCCL_PTR_CUDA, &mh));
+  const size_t n_req = (bytes + request - 1) / request;
+  std::vector<uint8_t> pattern(bytes), back(bytes);
+  for (int it = 0; it < iters; ++it) {
+    char go = 0;
+    sock_read(sock, &go, 1, kDeadline);
+    std::deque<void*> q;
+    size_t next = 0, finished = 0;
+    Deadline d;
+    while (finished < n_req) {
+      if (next < n_req && (int)q.size() < inflight) {
+        void* p = dst + next * request;
+        int sz = (int)(bytes - next * request < request ? bytes - next * request : request), tag = (int)next;
+        void* req = nullptr;
+        CHECK(net->irecv(rcomm, 1, &p, &sz, &tag, &mh, &req));
+        if (req) { q.push_back(req); ++next; }
+      }
+      if (!q.empty()) {
+        int done = 0, got = -1;
+        CHECK(net->test(q.front(), &done, &got));
+        if (done) {
+          const size_t want = bytes - finished * request < request ? bytes - finished * request : request;
+          if ((size_t)got != want) { fprintf(stderr, "receive %zu reported %d bytes, expected %zu\n", finished, got, want); return 4; }
+          q.pop_front(); ++finished;
+        }
+      }
+      d.check("receives");
+    }
+    fill_pattern(pattern, it);
+    HIP(hipMemcpy(back.data(), dst, bytes, hipMemcpyDeviceToHost));
+    if (memcmp(back.data(), pattern.data(), bytes) != 0) {
+      size_t at = 0;
+      while (at < bytes && back[at] == pattern[at]) ++at;
+      fprintf(stderr, "iteration %d: the received buffer differs from what was sent, first at byte %zu\n", it, at);
+      return 5;
+    }
+    HIP(hipMemset(dst, 0, bytes));
+    char ok = 1;
+    sock_write(sock, &ok, 1);
+  }
+  char bye = 0;
+  sock_read(sock, &bye, 1, kDeadline);   // the sender has closed its comm: the landing windows may go
+  CHECK(net->deregMr(rcomm, mh));
+  CHECK(net->closeRecv(rcomm));
+  CHECK(net->closeListen(lcomm));
+  HIP(hipFree(dst));
+  return 0;
+}
+
+static int sender_process(const char* path, int sock, pid_t child, size_t bytes, size_t request, int inflight, int iters) {
+  ncclNet_v8_t* net = open_plugin(path);
+  char handle[NCCL_NET_HANDLE_MAXSIZE];
+  sock_read(sock, handle, sizeof(handle), kDeadline);
+  void* scomm = nullptr;
+  for (Deadline d; !scomm; d.check("connect")) { CHECK(net->connect(1, handle, &scomm, nullptr)); if (!scomm) usleep(100); }
+  HIP(hipSetDevice(0));
+  uint8_t* src = nullptr;
+  void* mh = nullptr;
+  HIP(hipMalloc((void**)&src, bytes));
+  CHECK(net->regMr(scomm, src, bytes, NCCL_PTR_CUDA, &mh));
+  const size_t n_req = (bytes + request - 1) / request;
+  std::vector<uint8_t> pattern(bytes);
+  double best = 1e30, total = 0;
+  for (int it = 0; it < iters; ++it) {
+    fill_pattern(pattern, it);
+    HIP(hipMemcpy(src, pattern.data(), bytes, hipMemcpyHostToDevice));
+    char go = 1;
+    const auto t0 = std::chrono::steady_clock::now();
+    sock_write(sock, &go, 1);
+    std::deque<void*> q;
+    size_t next = 0, finished = 0;
+    Deadline d;
+    while (finished < n_req) {
+      if (next < n_req && (int)q.size() < inflight) {
+        const int sz = (int)(bytes - next * request < request ? bytes - next * request : request);
+        void* req = nullptr;
+        CHECK(net->isend(scomm, src + next * request, sz, (int)next, mh, &req));   // no request: the receive is not posted yet
+        if (req) { q.push_back(req); ++next; }
+      }
+      if (!q.empty()) {
+        int done = 0;
+        CHECK(net->test(q.front(), &done, nullptr));
+        if (done) { q.pop_front(); ++finished; }
+      }
+      d.check("sends");
+    }
+    const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    if (sec < best) best = sec;
+    total += sec / iters;
+    char ok = 0;
+    sock_read(sock, &ok, 1, kDeadline);   // the receiver has compared the buffer
+  }
+  CHECK(net->deregMr(scomm, mh));
+  CHECK(net->closeSend(scomm));
+  HIP(hipFree(src));
+  char bye = 1;
+  sock_write(sock, &bye, 1);
+  int status = 0;
+  Deadline d;
+  while (waitpid(child, &status, WNOHANG) == 0) { usleep(1000); d.check("the receiver's exit"); }
+  if (!WIFEXITED(status) || WEXITSTATUS(status) != 0) { fprintf(stderr, "the receiver process failed (status 0x%x)\n", status); return 5; }
+  printf("{\"harness\": \"plugin_two_process\", \"name\": \"%s\", \"memory\": \"device\", \"bytes\": %zu, \"request_bytes\": %zu, \"requests\": %zu, "
+         "\"inflight\": %d, \"iters\": %d, \"best_s\": %.9f, \"mean_s\": %.9f, \"GBps_payload_best\": %.1f, \"bit_exact\": true}\n",
+         net->name, bytes, request, n_req, inflight, iters, best, total, (double)bytes / best / 1e9);
+  return 0;
+}
+
+static int run_two_processes(const char* path, size_t bytes, size_t request, int inflight, int iters) {
+  setenv("NCCL_FUSELINK_WIRE", "shm", 1);
+  int sv[2];
+  if (socketpair(AF_UNIX, SOCK_STREAM, 0, sv) != 0) { perror("socketpair"); return 1; }
+  fflush(stdout);
+  fflush(stderr);
+  const pid_t child = fork();   // before anything here has loaded the plugin or called HIP
+  if (child < 0) { perror("fork"); return 1; }
+  if (child == 0) {
+    close(sv[0]);
+    const int rc = receiver_process(path, sv[1], bytes, request, inflight, iters);
+    fflush(stderr);
+    _exit(rc);
+  }
+  close(sv[1]);
+  signal(SIGPIPE, SIG_IGN);
+  return sender_process(path, sv[0], child, bytes, request, inflight, iters);
+}
+
 int main(int argc, char** argv) {
   if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [options]\n", argv[0]); return 1; }
   size_t bytes = 64u << 20, request = 0;
-  int inflight = 4, iters = 5, host = 0, version = 8, connections = 1, handoff = 0;
+  int inflight = 4, iters = 5, host = 0, version = 8, connections = 1, handoff = 0, two_process = 0;
   long long ho[6] = {0, 0, 0, 0, 0, 0};
   for (int i = 2; i < argc; ++i) {
     std::string a = argv[i];
@@ -185,6 +370,7 @@ int main(int argc, char** argv) {
     else if (a == "--version") version = (int)val();
     else if (a == "--host") host = 1;
     else if (a == "--connections") connections = (int)val();
+    else if (a == "--two-process") two_process = 1;
     else if (a == "--handoff" && i + 1 < argc) {
       if (sscanf(argv[++i], "%lld,%lld,%lld,%lld,%lld,%lld", &ho[0], &ho[1], &ho[2], &ho[3], &ho[4], &ho[5]) != 6) { fprintf(stderr, "--handoff takes six numbers\n"); return 1; }
       handoff = 1;
@@ -201,6 +387,11 @@ int main(int argc, char** argv) {
   }
   if (!request || request > bytes) request = bytes;
   if (request > 0x7fffffffull) request = 0x40000000ull;  // isend takes an int size (src/extern/nccl_net.h:74)
+
+  if (two_process) {
+    if (host || handoff || connections != 1) { fprintf(stderr, "--two-process runs one connection with device memory\n"); return 1; }
+    return run_two_processes(argv[1], bytes, request, inflight, iters);
+  }
 
   void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
   if (!lib) { fprintf(stderr, "dlopen: %s\n", dlerror()); return 1; }

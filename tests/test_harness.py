@@ -112,3 +112,38 @@ def test_plugin_host_path_under_address_sanitizer():
     assert "AddressSanitizer" not in res.stderr and "LeakSanitizer" not in res.stderr, res.stderr[-3000:]
     assert res.returncode == 0, res.stderr[-2000:]
     assert json.loads(res.stdout.strip().splitlines()[-1])["bit_exact"]
+
+
+# ---- sender and receiver in two processes ----------------------------------------------------------------------------
+# The receiver is a child forked before either side has loaded the plugin or touched the GPU; the two meet through the
+# 128-byte handle alone (a POSIX shared-memory object named in it carries the descriptor ring and the wave completions,
+# the receiver's landing windows are opened by the sender through HIP IPC).  The child compares what it received with
+# the pattern of the iteration and reports through its exit status.
+
+@pytest.mark.gpu
+def test_two_processes_cfg1_shape():
+    # the reference's own experiment: 4 MiB in 512 KiB chunks over 2 lanes, one request per NCCL step
+    out = _run(["--two-process", "--bytes", str(4 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "3"],
+               env={"NCCL_FUSELINK_LANES": "2", "NCCL_FUSELINK_CHUNKSIZE": str(512 << 10), "NCCL_FUSELINK_CREDITS": "1,1"})
+    assert out["harness"] == "plugin_two_process" and out["bit_exact"] and out["requests"] == 8
+    print(out)
+
+
+@pytest.mark.gpu
+def test_two_processes_cfg2_shape():
+    # 64 MiB in 256 KiB chunks over 8 lanes with uneven credits, one request; the windows hold the message in one wave
+    out = _run(["--two-process", "--bytes", str(64 << 20), "--request", str(64 << 20), "--inflight", "1", "--iters", "3"],
+               env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "28",
+                    "NCCL_FUSELINK_CREDITS": "8,6,7,1,8,7,3,3"})
+    assert out["harness"] == "plugin_two_process" and out["bit_exact"] and out["requests"] == 1
+    print(out)
+
+
+@pytest.mark.gpu
+def test_two_processes_requests_larger_than_the_windows_and_a_ragged_tail():
+    # every request takes several waves through the landing windows (4 units per lane), the last request is short and odd
+    out = _run(["--two-process", "--bytes", str((96 << 20) + 12345), "--request", str(32 << 20), "--inflight", "2", "--iters", "2"],
+               env={"NCCL_FUSELINK_LANES": "4", "NCCL_FUSELINK_CHUNKSIZE": str(128 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "4",
+                    "NCCL_FUSELINK_CREDITS": "3,1,2,2"})
+    assert out["bit_exact"] and out["requests"] == 4
+    print(out)

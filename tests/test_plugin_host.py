@@ -287,3 +287,101 @@ def test_headers_are_plain_c(header, tmp_path):
     res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I" + os.path.join(root, "include"), str(src)],
                          capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
+
+
+# ---- the shared-memory wire: the two ends in different processes (NCCL_FUSELINK_WIRE=shm) ---------------------------
+_LISTENER = r"""
+import sys, time
+import numpy as np
+from fuselink_amd import plugin as P
+p = P.NetPlugin(8)
+assert p.init() == P.ncclSuccess
+rc, handle, lcomm = p.listen(0)
+assert rc == P.ncclSuccess
+sys.stdout.write(handle.raw.hex() + "\n"); sys.stdout.flush()
+rcomm = None
+for _ in range(20000):
+    rc, rcomm = p.accept(lcomm)
+    assert rc == P.ncclSuccess
+    if rcomm:
+        break
+    time.sleep(0.001)
+assert rcomm, "nobody connected"
+# host memory does not travel on this wire: registration works, posting a receive is refused
+buf = np.zeros(4096, dtype=np.uint8)
+rc, mh = p.regMr(rcomm, buf.ctypes.data, buf.nbytes, P.NCCL_PTR_HOST)
+assert rc == P.ncclSuccess
+rc, req = p.irecv(rcomm, [buf.ctypes.data], [4096], [7], [mh])
+assert rc == P.ncclInvalidUsage and not req, (rc, req)
+assert p.deregMr(rcomm, mh) == P.ncclSuccess
+sys.stdin.readline()   # the connecting side is done
+assert p.closeRecv(rcomm) == P.ncclSuccess
+assert p.closeListen(lcomm) == P.ncclSuccess
+print("listener ok")
+"""
+
+
+def test_two_processes_meet_through_the_handle_alone():
+    """listen in a child process, connect here with nothing but the 128 bytes it printed (NCCL's bootstrap carries
+    them between ranks): the staged connect returns no comm until the listener has accepted, as the reference's does
+    (FuseLink src/plugin.cc:407-423, 721-760), and the shared-memory object's name is gone once both ends hold it."""
+    import subprocess
+    import sys
+    import time
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, NCCL_FUSELINK_WIRE="shm", PYTHONPATH=root)
+    child = subprocess.Popen([sys.executable, "-c", _LISTENER], stdin=subprocess.PIPE, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                             text=True, env=env, cwd=root)
+    try:
+        line = child.stdout.readline().strip()
+        assert len(line) == 2 * P.NCCL_NET_HANDLE_MAXSIZE, child.stderr.read()
+        handle = C.create_string_buffer(bytes.fromhex(line), P.NCCL_NET_HANDLE_MAXSIZE)
+        name = handle.raw[40:104].split(b"\0")[0].decode()
+        assert name.startswith("/fuselink-wire-")
+        old = os.environ.get("NCCL_FUSELINK_WIRE")
+        p = P.NetPlugin(8)
+        p.reconfigure(NCCL_FUSELINK_WIRE="shm")
+        try:
+            scomm = None
+            for _ in range(20000):
+                rc, scomm = p.connect(1, handle)
+                assert rc == P.ncclSuccess
+                if scomm:
+                    break
+                time.sleep(0.001)
+            assert scomm, "the listener never accepted"
+            assert not os.path.exists("/dev/shm" + name)   # unlinked at accept: nothing is left behind if a process dies
+            buf, ptr = _host(4096)
+            rc, mh = p.regMr(scomm, ptr, buf.nbytes, P.NCCL_PTR_HOST)
+            assert rc == P.ncclSuccess
+            rc, req = p.isend(scomm, ptr, 4096, 7, mh)
+            assert rc == P.ncclInvalidUsage and not req
+            assert p.deregMr(scomm, mh) == P.ncclSuccess
+            assert p.closeSend(scomm) == P.ncclSuccess
+        finally:
+            p.reconfigure(NCCL_FUSELINK_WIRE=old)
+        child.stdin.write("done\n")
+        child.stdin.flush()
+        out, err = child.communicate(timeout=60)
+        assert child.returncode == 0 and "listener ok" in out, err
+    finally:
+        if child.poll() is None:
+            child.kill()
+
+
+def test_a_listener_that_never_accepts_leaves_no_shared_memory_behind():
+    p = P.NetPlugin(8)
+    old = os.environ.get("NCCL_FUSELINK_WIRE")
+    p.reconfigure(NCCL_FUSELINK_WIRE="shm")
+    try:
+        rc, handle, lcomm = p.listen(0)
+        assert rc == P.ncclSuccess
+        name = handle.raw[40:104].split(b"\0")[0].decode()
+        assert os.path.exists("/dev/shm" + name)
+        assert p.closeListen(lcomm) == P.ncclSuccess
+        assert not os.path.exists("/dev/shm" + name)
+        # a connect with the stale handle fails cleanly
+        rc, scomm = p.connect(0, handle)
+        assert rc == P.ncclSystemError and not scomm
+    finally:
+        p.reconfigure(NCCL_FUSELINK_WIRE=old)
