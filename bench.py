@@ -32,12 +32,12 @@ WORKLOADS = {
     "cfg4_paged_kv_2x4096_pages_8lanes": ("pages", 2 * 4096 * 32768, 128 << 10, 8, 1, 0),
 }
 
-# HBM bytes per launch of the striping kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
-# WRITE_SIZE), each scaled by what the same counter reads for the plain copy kernel of known size.
-# None where no such run has been recorded for the workload.
-MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134300698, "cfg5_stress_1GiB_64KiB_16lanes": 2148002766,
-                    "cfg5_stress_1GiB_64KiB_16lanes/17 waves": 126498495,
-                    "cfg3_expert_parallel_256_blocks_8lanes": 1786036067, "cfg4_paged_kv_2x4096_pages_8lanes": 268550997}
+# Bytes per launch of the striping kernel between the L2 caches and the fabric behind them (Infinity Cache, then HBM),
+# from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the plain
+# copy kernel of known size.  None where no such run has been recorded for the workload.
+MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134277565, "cfg5_stress_1GiB_64KiB_16lanes": 2148014006,
+                    "cfg5_stress_1GiB_64KiB_16lanes/17 waves": 126482128,
+                    "cfg3_expert_parallel_256_blocks_8lanes": 1786029836, "cfg4_paged_kv_2x4096_pages_8lanes": 268579065}
 
 
 def algo_bytes_cold(nbytes: int) -> int:
@@ -97,6 +97,8 @@ def main() -> int:
     ap.add_argument("--pool-units", type=int, default=0,
                     help="uniform table-driven workloads: keep the staging windows within a pool of this many 2 MiB units (the reference's "
                          "holds 256) and move the message in as few waves as that allows, windows reused wave by wave; 0 = windows for the whole message")
+    ap.add_argument("--lanes", type=int, default=0,
+                    help="override the workload's number of lanes (staging windows); for measuring what the window count costs, not a bench line")
     ap.add_argument("--no-by-lane", action="store_true", help="stripe large messages in chunk order instead of destination order")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -146,6 +148,8 @@ def main() -> int:
         core.tune(key, int(val))
     dev = torch.device("cuda:0")
     kind, nbytes, chunk, lanes, rows, epoch_len = WORKLOADS[args.workload]
+    if args.lanes:
+        lanes = args.lanes
     rng = np.random.default_rng(20251125)
     gen = torch.Generator(device=dev)
     gen.manual_seed(20251125)
@@ -512,7 +516,7 @@ def main() -> int:
         "plugin_abi": plugin,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": (MEASURED_TRAFFIC.get(f"{args.workload}/{len(cwaves)} waves") if cwaves else None if (waves or twaves) else
+                     "traffic": (None if args.lanes else MEASURED_TRAFFIC.get(f"{args.workload}/{len(cwaves)} waves") if cwaves else None if (waves or twaves) else
                                  MEASURED_TRAFFIC.get(args.workload) if (kind != "blocks" or args.blocks == 256) else None)},
     }
 
