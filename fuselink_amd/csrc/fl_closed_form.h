@@ -48,17 +48,29 @@ inline uint32_t fl_row_lane_of(const FlCreditRow& r, uint64_t x) {
 }
 
 // Bytes and chunks that a message of `bytes` bytes in chunks of `chunk` puts on each lane when `quanta_before` quanta
-// of its credit epoch precede it (only the last chunk may be short).
+// of its credit epoch precede it (only the last chunk may be short).  The two divisions by W are done once, not per
+// lane: this runs for every request that waits for a launch.
 inline void fl_row_lane_totals(const FlCreditRow& r, uint64_t quanta_before, uint64_t bytes, uint64_t chunk, uint64_t* lane_bytes,
                                uint32_t* lane_chunks) {
   const uint64_t n = (bytes + chunk - 1) / chunk;
+  const uint64_t W = r.W, x0 = quanta_before, x1 = quanta_before + n;
+  const uint64_t q0 = x0 / W, r0 = x0 - q0 * W, q1 = x1 / W, r1 = x1 - q1 * W;
+  const uint32_t lanes = r.lanes;
+  uint32_t last_lane = 0;
+  const uint64_t last_slot = r1 ? r1 - 1 : W - 1;   // slot of quantum x1 - 1
   for (uint32_t l = 0; l < FLH_MAX_LANES; ++l) {
     uint64_t k = 0;
-    if (l < r.lanes && n) k = fl_row_before(r, l, quanta_before + n) - fl_row_before(r, l, quanta_before);
+    if (l < lanes && n) {
+      const uint64_t K = r.K[l], c = r.K[l + 1] - K;
+      const uint64_t b1 = q1 * c + (r1 <= K ? 0 : (r1 - K < c ? r1 - K : c));
+      const uint64_t b0 = q0 * c + (r0 <= K ? 0 : (r0 - K < c ? r0 - K : c));
+      k = b1 - b0;
+      if (l + 1 < lanes && r.K[l + 1] <= last_slot) last_lane = l + 1;
+    }
     lane_chunks[l] = (uint32_t)k;
     lane_bytes[l] = k * chunk;
   }
-  if (n) lane_bytes[fl_row_lane_of(r, quanta_before + n - 1)] -= n * chunk - bytes;
+  if (n) lane_bytes[last_lane] -= n * chunk - bytes;
 }
 
 #endif  // FL_CLOSED_FORM_H_

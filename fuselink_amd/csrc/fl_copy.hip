@@ -712,8 +712,11 @@ __global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const 
 // (fused_tile): first the striping of their tiles, then the reassembly of the same tiles, so that a tile is read back
 // by the workgroup that staged it and no workgroup waits for another inside a batch.  A batch's tiles go to the
 // workers in turn, starting behind the worker that took the last tile of the batch before, so that small batches
-// run side by side on different workers.  Successive batches rotate through the caller's sets of staging windows,
-// and a worker enters batch k only once every worker has left batch k - sets.  The last worker to leave a batch stores its number to a host-visible word.
+// run side by side on different workers.  Only the workers with a share in a batch are counted in and out of it: the
+// others pass it by without an atomic or a fence, so what a small batch costs does not grow with the size of the
+// engine.  Successive batches rotate through the caller's sets of staging windows, and a worker enters batch k only
+// once batch k - sets is complete.  The last worker to leave a batch stores its number to a host-visible word of the
+// batch's ring slot; batches of different workers may complete out of order, and the host reports the complete prefix.
 // Every wait in the kernel is bounded: with nothing to do for idle_us the dispatcher takes the engine down (the host
 // starts it again with the next batch), and a wait that outlasts wait_us reports an error and takes it down as well.
 constexpr uint32_t kEngineDevRing = 8;          // descriptors held in device memory; also the most window sets a caller may rotate
@@ -735,26 +738,38 @@ struct EngineHostCtl {                           // pinned host memory, mapped t
   alignas(64) uint64_t tail;                     // host: batches submitted so far
   alignas(64) uint32_t state;                    // 0 down, 1 running, 2 about to go down (device; the host sets 1 when it launches)
   alignas(64) uint64_t exited_at;                // device: the batch the next engine has to start with
-  alignas(64) uint64_t done;                     // device: batches complete
+  alignas(64) uint64_t done[kEngineDevRing];     // device: per ring slot, the number of the last batch of that slot that is complete
   alignas(64) int32_t error;                     // device: a bounded wait ran out (FLH_E_STATE)
   alignas(64) uint32_t stop;                     // host: go down now
 };
 struct EngineDevCtl {                            // device memory
-  // per ring slot: low half of the number of the batch whose descriptor the slot holds << 32 | the worker that takes
-  // the batch's first share << 20 | its shares; a worker learns from the one word that its batch is there and
-  // which of its shares, if any, are its own
+  // per ring slot, one word from which a worker learns that its batch is there, which of its shares (if any) are its
+  // own, when it may enter and whether it is the last to leave (engine_word): the batch's number, the worker that
+  // takes its first share, its shares, and the slot counters' values that mean "this batch is complete" and "the batch
+  // whose windows it reuses is complete"
   alignas(64) uint64_t published[kEngineDevRing];
-  alignas(64) uint32_t quit;                     // workers leave when they reach batch quit_at
+  alignas(64) uint32_t quit;                     // the engine launch (EngineArgs::gen) whose workers leave when they reach batch quit_at; never cleared
   uint32_t pad;
   uint64_t quit_at;
-  alignas(64) uint64_t arrive[kEngineDevRing];   // workers that have left the batches of each ring slot, never reset
+  alignas(64) uint64_t arrive[kEngineDevRing];   // workers with a share that have left the batches of each ring slot, never reset
+  alignas(64) uint64_t target[kEngineDevRing];   // the dispatcher's record: arrive[slot] once the slot's latest batch is complete (kept across engine launches)
 };
+
+// The published word: batch number (16 bits) | first worker (10) | shares, saturated (10) | low 14 bits of the slot
+// counter when this batch is complete | low 14 bits of the counter of slot (k - sets) when that batch is complete.
+// Counters are compared modulo 2^14: a slot's counter is never more than one batch (at most 1023 workers) away from
+// either value while anyone looks.
+constexpr uint32_t kEngineCountMask = 0x3fffu;
+__host__ __device__ inline uint64_t engine_word(uint64_t k, uint32_t first, uint32_t shares, uint64_t own_target, uint64_t wait_target) {
+  return ((uint64_t)(uint16_t)(k + 1) << 48) | ((uint64_t)(first & 0x3ffu) << 38) | ((uint64_t)(shares < 0x3ffu ? shares : 0x3ffu) << 28) |
+         ((own_target & kEngineCountMask) << 14) | (wait_target & kEngineCountMask);
+}
 struct EngineArgs {
   const uint8_t* host_ring;                      // kHostRing descriptors, device-visible pinned memory
   uint32_t host_slots;
   uint32_t workers;
   uint32_t sets;                                 // the caller rotates this many window sets: batch k waits for batch k - sets
-  uint32_t pad;
+  uint32_t gen;                                  // number of this launch of the engine, from 1: what the quit word must hold to mean this one
   EngineHostCtl* hctl;
   uint8_t* dev_ring;
   EngineDevCtl* dctl;
@@ -765,12 +780,14 @@ struct EngineArgs {
 __device__ __forceinline__ void engine_fail(const EngineArgs& e) {
   __hip_atomic_store(&e.hctl->error, (int32_t)FLH_E_STATE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   __hip_atomic_store(&e.dctl->quit_at, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(&e.dctl->quit, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&e.dctl->quit, e.gen, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
   __shared__ EngineDesc d;
   __shared__ uint32_t sh_flag, sh_first;
+  __shared__ uint64_t sh_word;
+  __shared__ uint64_t tgt[kEngineDevRing];
   const uint32_t tid = threadIdx.x;
   const uint32_t W = e.workers;
   if (blockIdx.x == 0) {
@@ -780,13 +797,14 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     uint32_t first_worker = 0;      // takes the first tile of batch k
     uint32_t polls = 0;
     uint64_t idle_since = wall_clock64(), free_since = idle_since;
+    if (tid < kEngineDevRing) tgt[tid] = e.dctl->target[tid];   // where the engine before this one left the slots
+    __syncthreads();
     for (;;) {
       if (tid == 0) {
         uint32_t act = 0;   // 0 poll again, 1 copy descriptor k, 2 leave
         const uint64_t now = wall_clock64();
-        // the device slot of batch k held batch k - ring: every worker must have left that one
-        const uint64_t need = (k / kEngineDevRing) * W;
-        if (__hip_atomic_load(&e.dctl->arrive[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= need) {
+        // the device slot of batch k held batch k - ring: that one must be complete
+        if (__hip_atomic_load(&e.dctl->arrive[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= tgt[k % kEngineDevRing]) {
           free_since = now;
           if (tail_seen <= k) tail_seen = __hip_atomic_load(&e.hctl->tail, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
           if (tail_seen > k) act = 1;
@@ -796,7 +814,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
         if (act == 1) {
           idle_since = now;
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the workers' reads of the slot are behind their arrival
-        } else if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ||
+        } else if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == e.gen ||
                    ((++polls & 31) == 0 && __hip_atomic_load(&e.hctl->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM))) {
           act = 2;   // (the host's stop flag is a trip across the bus: looked at now and then)
         } else if (now - idle_since > e.idle_ticks) {
@@ -827,18 +845,25 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
       dst[tid] = v;
       __syncthreads();
       if (tid == 0) {
-        const uint32_t tiles = v.x < 0xfffffu ? v.x : 0xfffffu;   // EngineDesc::tiles
-        __hip_atomic_store(&e.dctl->published[k % kEngineDevRing], ((uint64_t)(uint32_t)(k + 1) << 32) | ((uint64_t)first_worker << 20) | tiles,
-                           __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        first_worker = (first_worker + tiles) % W;
+        const uint32_t tiles = v.x;                                 // EngineDesc::tiles: the batch's shares
+        const uint32_t slot = (uint32_t)(k % kEngineDevRing);
+        const uint64_t takers = tiles < W ? tiles : W;              // workers with a share in the batch
+        const uint64_t wait_target = k >= e.sets ? tgt[(k - e.sets) % kEngineDevRing] : 0;   // (read before this slot's own entry moves: sets may equal the ring)
+        const uint64_t own_target = tgt[slot] + takers;
+        tgt[slot] = own_target;
+        e.dctl->target[slot] = own_target;
+        __hip_atomic_store(&e.dctl->published[slot], engine_word(k, first_worker, tiles, own_target, wait_target), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        if (takers == 0)   // nothing to move (the host submits no such batch): complete as it stands
+          __hip_atomic_store(&e.hctl->done[slot], k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        first_worker = (uint32_t)((first_worker + tiles) % W);
       }
       ++k;
     }
     if (tid == 0) {
       // workers finish what has been published and leave at batch k; the next engine starts there
-      if (!__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+      if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != e.gen) {
         __hip_atomic_store(&e.dctl->quit_at, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&e.dctl->quit, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&e.dctl->quit, e.gen, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
       }
       __hip_atomic_store(&e.hctl->exited_at, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       __hip_atomic_store(&e.hctl->state, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -849,49 +874,46 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
   const uint32_t w = blockIdx.x - 1;
   for (uint64_t k = e.start;; ++k) {
     if (tid == 0) {
-      uint32_t act = 1;   // 1 run batch k, 2 leave, 3 no tile of batch k is this worker's
+      uint32_t act = 1;   // 1 run batch k, 2 leave, 3 no share of batch k is this worker's
       uint64_t word = 0;
       const uint64_t t0 = wall_clock64();
       for (uint32_t spin = 0;; ++spin) {
         word = __hip_atomic_load(&e.dctl->published[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // the fence below acquires
-        if ((uint32_t)(word >> 32) == (uint32_t)(k + 1)) break;
+        const int16_t ahead = (int16_t)((uint16_t)(word >> 48) - (uint16_t)(k + 1));
+        if (ahead == 0) break;
+        // the slot already holds a later batch: batch k came and went, which it could not have with a share of this worker outstanding
+        if (ahead > 0) { act = 3; break; }
         if ((spin & 7) == 7) {   // the flag and the clock now and then: every look is a round trip to memory
-          if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) &&
+          if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == e.gen &&
               __hip_atomic_load(&e.dctl->quit_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <= k) { act = 2; break; }
           if (wall_clock64() - t0 > e.wait_ticks + e.idle_ticks) { engine_fail(e); act = 2; break; }
         }
         __builtin_amdgcn_s_sleep(1);
       }
-      // this worker's first tile of the batch: the tiles go round the workers from the batch's first worker on
-      const uint32_t first = (uint32_t)(word >> 20) & 0xfffu;
+      // this worker's first share of the batch: the shares go round the workers from the batch's first worker on
+      const uint32_t first = (uint32_t)(word >> 38) & 0x3ffu;
       sh_first = (w + W - first) % W;
-      if (act == 1 && sh_first >= (uint32_t)(word & 0xfffffu)) act = 3;
+      if (act == 1 && sh_first >= ((uint32_t)(word >> 28) & 0x3ffu)) act = 3;
       if (act == 1 && k >= e.sets) {
-        // batch k reuses the windows of batch k - sets: every worker must have left that one
+        // batch k reuses the windows of batch k - sets: that one must be complete
         const uint64_t j = k - e.sets;
-        const uint64_t need = (j / kEngineDevRing + 1) * W;
+        const uint32_t need = (uint32_t)word & kEngineCountMask;
         const uint64_t t1 = wall_clock64();
-        while (__hip_atomic_load(&e.dctl->arrive[j % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+        while ((((uint32_t)__hip_atomic_load(&e.dctl->arrive[j % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - need) & kEngineCountMask) > kEngineCountMask / 2) {
           if (wall_clock64() - t1 > e.wait_ticks) { engine_fail(e); act = 2; break; }
           __builtin_amdgcn_s_sleep(1);
         }
       }
       sh_flag = act;
+      sh_word = word;
     }
     __syncthreads();
     const uint32_t act = sh_flag, mine = sh_first;
+    const uint32_t own_target = (uint32_t)(sh_word >> 14) & kEngineCountMask;
     __syncthreads();
     if (act == 2) return;
+    if (act == 3) continue;   // nothing read, nothing written, nothing to count
     uint64_t* cnt = &e.dctl->arrive[k % kEngineDevRing];
-    if (act == 3) {
-      // nothing read, nothing written: the worker only has to be counted (the last one to leave publishes the batch)
-      if (tid == 0) {
-        const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
-        if (before + 1 == (k / kEngineDevRing + 1) * W)
-          __hip_atomic_store(&e.hctl->done, k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-      }
-      continue;
-    }
     // what the batch reads may have been written by anyone, on this GPU or off it, before the host submitted it
     __atomic_thread_fence(__ATOMIC_ACQUIRE);
     {
@@ -923,8 +945,8 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
       // leaving the batch releases this worker's stores; the last one to leave has thereby acquired everybody's and
       // publishes the batch to the host
       const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_SYSTEM);
-      if (before + 1 == (k / kEngineDevRing + 1) * W)
-        __hip_atomic_store(&e.hctl->done, k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      if ((((uint32_t)before + 1) & kEngineCountMask) == own_target)
+        __hip_atomic_store(&e.hctl->done[k % kEngineDevRing], k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
 }
@@ -1379,6 +1401,7 @@ struct flh_engine {
   uint8_t* dev_ring;
   EngineDevCtl* dctl;
   uint64_t submitted;       // batches written into the ring
+  uint64_t completed;       // batches known complete, in order (atomic; moved forward by whoever looks)
   uint64_t launches;        // engine kernels started
   uint64_t idle_us, wait_us;
 };
@@ -1428,7 +1451,7 @@ static int engine_start(flh_engine* e) {
   a.host_slots = e->host_slots;
   a.workers = e->workers;
   a.sets = e->sets;
-  a.pad = 0;
+  a.gen = (uint32_t)(e->launches % 0xfffffffeull) + 1;   // never 0, which is what the quit word holds before any engine has left
   a.hctl = e->d_ctl_host;
   a.dev_ring = e->dev_ring;
   a.dctl = e->dctl;
@@ -1436,7 +1459,6 @@ static int engine_start(flh_engine* e) {
   a.idle_ticks = e->idle_us * 100;     // the wall clock counts at 100 MHz
   a.wait_ticks = e->wait_us * 100;
   __atomic_store_n(&e->h_ctl->state, 1u, __ATOMIC_RELEASE);
-  FL_HIP(hipMemsetAsync(&e->dctl->quit, 0, sizeof(uint32_t), e->stream));
   hipLaunchKernelGGL(fl_engine_kernel, dim3(e->workers + 1), dim3(kCopyBlock), 0, e->stream, a);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
@@ -1453,7 +1475,7 @@ int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_window
   if (__atomic_load_n(&e->h_ctl->error, __ATOMIC_ACQUIRE)) return fl_set_error(FLH_E_STATE, "the engine went down on a wait that ran out");
   // the ring slot must be free: its last occupant complete
   const uint64_t seq = e->submitted;
-  if (seq >= e->host_slots && __atomic_load_n(&e->h_ctl->done, __ATOMIC_ACQUIRE) + e->host_slots <= seq)
+  if (seq >= e->host_slots && flh_engine_completed(e) + e->host_slots <= seq)
     return fl_set_error(FLH_E_NOMEM, "the engine's descriptor ring is full (%u batches in flight)", e->host_slots);
   BatchPlan pl;
   int rc = plan_batch(b, pl);
@@ -1505,8 +1527,20 @@ int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_window
   return FLH_OK;
 }
 
+// Batches complete, counted in order: batch c is complete once its ring slot reports it or a later batch of the slot
+// (which cannot have started before).  Batches with different workers may finish out of order; the prefix is what a
+// caller that reuses window sets and ring slots in order needs.
 uint64_t flh_engine_completed(const flh_engine* e) {
-  return e ? __atomic_load_n(&e->h_ctl->done, __ATOMIC_ACQUIRE) : 0;
+  if (!e) return 0;
+  uint64_t* known = const_cast<uint64_t*>(&e->completed);
+  uint64_t c = __atomic_load_n(known, __ATOMIC_ACQUIRE);   // pairs with the release below: what the thread that moved it forward had acquired from the device
+  const uint64_t from = c;
+  while (__atomic_load_n(&e->h_ctl->done[c % kEngineDevRing], __ATOMIC_ACQUIRE) >= c + 1) ++c;
+  if (c != from) {
+    uint64_t seen = from;
+    while (seen < c && !__atomic_compare_exchange_n(known, &seen, c, true, __ATOMIC_RELEASE, __ATOMIC_RELAXED)) {}
+  }
+  return c;
 }
 
 int flh_engine_error(const flh_engine* e) {

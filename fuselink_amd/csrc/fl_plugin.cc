@@ -97,7 +97,7 @@ std::mutex g_init_mu;            // ncclIbLock, plugin.cc:84
 
 // NCCL_FUSELINK_TRACE=1: calls and nanoseconds spent inside the entry points and inside the launches they make
 // (fl_net_host_stats).  Off, a probe costs one predictable branch.
-enum : int { kTrIsend = 0, kTrIrecv, kTrTest, kTrTestDone, kTrFlush, kTrLaunch, kTrRequestsLaunched, kTrCount };
+enum : int { kTrIsend = 0, kTrIrecv, kTrTest, kTrTestDone, kTrFlush, kTrLaunch, kTrRequestsLaunched, kTrEngineSubmit, kTrEngineStart, kTrCount };
 std::atomic<int64_t> g_tr_calls[kTrCount], g_tr_ns[kTrCount];
 inline int64_t tr_now() {
   timespec t;
@@ -1517,7 +1517,9 @@ size_t build_batch(Peer* pr, size_t i, BatchBuild& bb, bool engine) {
       extend = bb.seg_link[k] == p.lk && !(p.w.flags & 1u) && (uint64_t)work[j - 1].size % chunk == 0 &&
                memcmp(b.seg[k].credits, credits, sizeof(credits)) == 0;
     }
-    if (engine ? !engine_takes(pr, p, epoch) : (!extend && needs_waves(wins, p, epoch))) break;
+    // (whether the request fits is decided below, against what the batch has put into the windows so far; the caller
+    // has made sure that work[i] fits empty ones)
+    if (engine && (int64_t)p.size > g_par.engine_max_request) break;
     if (!extend && b.n_seg == FLH_SEG_MAX) break;
     // Where would the windows end up?  The open segment grows by the request, or is closed and a new one opens
     // behind it, on every lane at the next multiple of 128 bytes (flh_batch_layout's rule).
@@ -1586,8 +1588,15 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     const uint32_t slot = (uint32_t)(k % kEngineSlots);
     b.u.tile_bytes = FLH_TILE_BYTES;
     uint64_t got = 0;
+    const uint64_t starts_before = g_par.trace ? flh_engine_launches(pr->engine) : 0;
+    const int64_t t_sub = g_par.trace ? tr_now() : 0;
     const int frc = flh_engine_submit(pr->engine, &b, &pr->ewins[k % (uint64_t)g_par.engine_sets], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot, pr->d_status, &got,
                                       &seg_base[0][0]);
+    if (g_par.trace) {   // submits that had to start the resident kernel are counted apart: they pay for a launch
+      const int which = flh_engine_launches(pr->engine) != starts_before ? kTrEngineStart : kTrEngineSubmit;
+      g_tr_calls[which].fetch_add(1, std::memory_order_relaxed);
+      g_tr_ns[which].fetch_add(tr_now() - t_sub, std::memory_order_relaxed);
+    }
     if (frc == FLH_E_NOMEM) return ncclInProgress;   // the descriptor ring is full: the caller takes the launch path for this batch
     if (frc < 0) {
       FL_WARN("NET/FuseLink : engine: %s", flh_last_error());

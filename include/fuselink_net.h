@@ -259,7 +259,9 @@ int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, vo
 /* Where the host's time goes (collected only under NCCL_FUSELINK_TRACE=1; process-wide sums over all threads): calls
  * and nanoseconds, index 0 isend, 1 irecv, 2 test, 3 tests that completed a request (calls only), 4 passes that
  * launched what waited, 5 launch pairs (time inside the runtime's launch calls and the batch arithmetic before them),
- * 6 requests those passes launched (calls only).  Returns the number of counters. */
+ * 6 requests those passes launched (calls only), 7 batches handed to the lane engine (time inside flh_engine_submit),
+ * 8 of those hand-overs that had to start the resident kernel first (counted apart from 7).  Returns the number of
+ * counters. */
 int fl_net_host_stats(int64_t* calls_out, int64_t* ns_out, int n);
 /* Timeline kept under NCCL_FUSELINK_TRACE=2: up to 65536 events of 24 bytes {int64 nanoseconds (monotonic clock), uint32
  * thread, uint32 event, uint64 value}; events: 1 receive posted (value = channel), 2 send matched (channel), 3 a pass that

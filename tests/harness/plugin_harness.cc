@@ -434,14 +434,15 @@ int main(int argc, char** argv) {
   host_stats_fn host_stats = (host_stats_fn)dlsym(lib, "fl_net_host_stats");
   const char* tr = getenv("NCCL_FUSELINK_TRACE");
   if (host_stats && tr && atoi(tr) > 0) {
-    int64_t calls[8] = {0}, ns[8] = {0};
-    host_stats(calls, ns, 8);
+    int64_t calls[16] = {0}, ns[16] = {0};
+    host_stats(calls, ns, 16);
     const double reqs = (double)n_req * connections * iters;
     printf("{\"harness\": \"host_trace\", \"requests\": %.0f, \"isend_calls\": %lld, \"isend_us\": %.1f, \"irecv_calls\": %lld, \"irecv_us\": %.1f, "
            "\"test_calls\": %lld, \"test_us\": %.1f, \"tests_done\": %lld, \"flush_passes\": %lld, \"flush_us\": %.1f, \"launch_pairs\": %lld, \"launch_us\": %.1f, "
-           "\"requests_per_launch\": %.2f, \"launch_us_per_pair\": %.2f}\n",
+           "\"requests_per_launch\": %.2f, \"launch_us_per_pair\": %.2f, \"engine_submits\": %lld, \"engine_submit_us\": %.1f, \"engine_starts\": %lld, \"engine_start_us\": %.1f}\n",
            reqs, (long long)calls[0], ns[0] / 1e3, (long long)calls[1], ns[1] / 1e3, (long long)calls[2], ns[2] / 1e3, (long long)calls[3],
-           (long long)calls[4], ns[4] / 1e3, (long long)calls[5], ns[5] / 1e3, calls[5] ? (double)calls[6] / calls[5] : 0.0, calls[5] ? ns[5] / 1e3 / calls[5] : 0.0);
+           (long long)calls[4], ns[4] / 1e3, (long long)calls[5], ns[5] / 1e3, calls[5] ? (double)calls[6] / calls[5] : 0.0, calls[5] ? ns[5] / 1e3 / calls[5] : 0.0,
+           (long long)calls[7], ns[7] / 1e3, (long long)calls[8], ns[8] / 1e3);
   }
   // NCCL_FUSELINK_TRACE=2: the timeline of the entry-point events, one line per event, into the file named by FL_TIMELINE_OUT
   typedef int (*timeline_fn)(void*, int);
