@@ -80,7 +80,7 @@ def main() -> int:
                     help="blocks workload: add 1..15 bytes to every block, so that no chunk is a multiple of 16 bytes and source and "
                          "window offsets are misaligned against each other")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
-                    help="set a library tunable (flh_tune) before the run, e.g. --tune copy_rows_per_wg=1; repeatable")
+                    help="set a library tunable (flh_tune) before the run, e.g. --tune xcd_runs=0; repeatable")
     ap.add_argument("--blocks", type=int, default=256,
                     help="blocks workload: number of variable blocks (rows per block ~ Zipf(1.1) capped at 4096 for the 256 blocks of cfg3, "
                          "at 65536 / blocks otherwise: 65000 blocks are single rows of 14 KiB)")

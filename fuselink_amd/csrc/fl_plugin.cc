@@ -62,7 +62,7 @@ struct Params {
   int refresh_batch = FL_NET_REFRESH_BATCH;
   int policy = 1;                // 0 = static lane = channelId % lanes (fuselink.h:235); 1 = credit-weighted
   int pool_units = FLH_POOL_UNITS;
-  int window_units = 4;          // staging units bound per lane per connection
+  int window_units = 4;          // staging units bound per lane, once per GPU that stages: every connection to that GPU shares the windows
   int qps = 1;                   // NCCL_IB_QPS_PER_CONNECTION, plugin.cc:584
   int split_on_qps = 1;          // NCCL_IB_SPLIT_DATA_ON_QPS, plugin.cc:1410
   int device = -1;               // HIP device that stages; -1 = the one that owns the registered memory
