@@ -76,6 +76,17 @@ def build_harness(verbose: bool = True) -> str | None:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("harness build failed:\n" + res.stderr)
+    # the lane engine's own latency / rate harness
+    esrc = os.path.join(ROOT, "tests", "harness", "engine_bench.cc")
+    if os.path.exists(esrc):
+        ecmd = cmd[:]
+        ecmd[ecmd.index(src)] = esrc
+        ecmd[ecmd.index(out)] = os.path.join(ROOT, "tests", "harness", "engine_bench")
+        if verbose:
+            print(" ".join(ecmd), flush=True)
+        res = subprocess.run(ecmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("engine harness build failed:\n" + res.stderr)
     return out
 
 

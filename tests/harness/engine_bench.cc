@@ -1,0 +1,99 @@
+// engine_bench.cc -- latency and rate of the lane engine (flh_engine_*) for batches of 512 KiB requests, without the
+// plugin around it: what a batch costs one at a time, what it costs with several in flight, and what a submit costs
+// that has to start the resident kernel again.  dlopen()s the library and prints one JSON line.
+//
+//   engine_bench <lib.so> [--requests N] [--depth D] [--workgroups W] [--batches B]
+// N requests per batch (1..32), D window sets = batches in flight (1..8), W workgroups of the engine (0 = default).
+#include <dlfcn.h>
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "fuselink_hip.h"
+
+#define HIP(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { fprintf(stderr, "%s -> %s\n", #x, hipGetErrorString(e_)); exit(3); } } while (0)
+static double now_us() { return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now().time_since_epoch()).count(); }
+
+int main(int argc, char** argv) {
+  if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [--requests N] [--depth D] [--workgroups W] [--batches B]\n", argv[0]); return 1; }
+  int nreq = 8, depth = 2, wgs = 0, batches = 2000;
+  for (int i = 2; i + 1 < argc; i += 2) {
+    const std::string a = argv[i];
+    const int v = atoi(argv[i + 1]);
+    if (a == "--requests") nreq = v; else if (a == "--depth") depth = v; else if (a == "--workgroups") wgs = v; else if (a == "--batches") batches = v;
+  }
+  if (nreq < 1 || nreq > FLH_BATCH_MAX || depth < 1 || depth > 8 || batches < 1) { fprintf(stderr, "arguments out of range\n"); return 1; }
+  void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
+  if (!lib) { fprintf(stderr, "dlopen: %s\n", dlerror()); return 1; }
+#define SYM(name) decltype(&name) p_##name = (decltype(&name))dlsym(lib, #name); if (!p_##name) { fprintf(stderr, "missing %s\n", #name); return 1; }
+  SYM(flh_init) SYM(flh_last_error) SYM(flh_engine_create) SYM(flh_engine_submit) SYM(flh_engine_completed) SYM(flh_engine_error) SYM(flh_engine_launches) SYM(flh_engine_destroy)
+  HIP(hipSetDevice(0));
+  if (p_flh_init(0)) { fprintf(stderr, "init: %s\n", p_flh_last_error()); return 1; }
+  const size_t req = 512 << 10, lanes = 8, cap = 4 << 20;
+  uint8_t *src, *dst, *win;
+  HIP(hipMalloc((void**)&src, req * nreq)); HIP(hipMalloc((void**)&dst, req * nreq)); HIP(hipMalloc((void**)&win, (size_t)depth * lanes * cap));
+  std::vector<uint8_t> pattern(req * nreq);
+  uint64_t x = 88172645463325252ull;
+  for (auto& b : pattern) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; b = (uint8_t)x; }
+  HIP(hipMemcpy(src, pattern.data(), pattern.size(), hipMemcpyHostToDevice));
+  HIP(hipMemset(dst, 0, req * nreq));
+  flh_chunk_desc* table; flh_sched_hdr* hdr;
+  HIP(hipMalloc((void**)&table, 4096 * sizeof(flh_chunk_desc))); HIP(hipMalloc((void**)&hdr, sizeof(flh_sched_hdr)));
+  int32_t *h_status, *d_status;
+  HIP(hipHostMalloc((void**)&h_status, 64, hipHostMallocMapped)); memset(h_status, 0, 64);
+  HIP(hipHostGetDevicePointer((void**)&d_status, h_status, 0));
+  std::vector<flh_windows> w(depth);
+  for (int h = 0; h < depth; ++h) { memset(&w[h], 0, sizeof(flh_windows)); w[h].n_lanes = lanes; for (size_t l = 0; l < lanes; ++l) { w[h].base[l] = win + ((size_t)h * lanes + l) * cap; w[h].cap[l] = cap; } }
+  flh_batch_params b; memset(&b, 0, sizeof(b));
+  b.u.chunk_bytes = 256 << 10; b.u.n_lanes = lanes; b.u.tile_bytes = FLH_TILE_BYTES; b.u.total_bytes = (uint64_t)nreq * req;
+  const uint32_t credits[8] = {8, 6, 7, 1, 8, 7, 3, 3};
+  for (size_t l = 0; l < lanes; ++l) b.u.credits[l] = credits[l];
+  b.n_req = nreq;
+  for (int q = 0; q < nreq; ++q) { b.d_src[q] = src + q * req; b.d_dst[q] = dst + q * req; b.bytes[q] = req; }
+  flh_engine* e = nullptr;
+  if (p_flh_engine_create(0, wgs, 200, depth, &e)) { fprintf(stderr, "engine: %s\n", p_flh_last_error()); return 1; }
+  uint64_t seq = 0;
+  auto submit = [&](int set) { if (p_flh_engine_submit(e, &b, &w[set], table, hdr, d_status, &seq, nullptr)) { fprintf(stderr, "submit: %s\n", p_flh_last_error()); exit(1); } };
+  auto wait_for = [&](uint64_t upto) {
+    const double deadline = now_us() + 5e6;
+    while (p_flh_engine_completed(e) < upto) if (now_us() > deadline) { fprintf(stderr, "timed out, engine error %d\n", p_flh_engine_error(e)); exit(2); }
+  };
+  for (int i = 0; i < 10; ++i) { submit(i % depth); wait_for(seq); }
+  // the bytes must have arrived
+  std::vector<uint8_t> back(req * nreq);
+  HIP(hipMemcpy(back.data(), dst, back.size(), hipMemcpyDeviceToHost));
+  const bool exact = memcmp(back.data(), pattern.data(), back.size()) == 0 && h_status[0] == 0;
+  // one batch at a time
+  double t0 = now_us(), sub = 0;
+  for (int i = 0; i < batches; ++i) { const double a = now_us(); submit(i % depth); sub += now_us() - a; wait_for(seq); }
+  const double alone = (now_us() - t0) / batches;
+  // `depth` batches in flight
+  t0 = now_us();
+  for (int i = 0; i < batches; ++i) { submit(i % depth); if (seq >= (uint64_t)depth) wait_for(seq - depth + 1); }
+  wait_for(seq);
+  const double piped = (now_us() - t0) / batches;
+  // after the engine has gone down (idle for 1.5 ms)
+  double restart_submit = 0, restart_done = 0;
+  const int R = 20;
+  for (int i = 0; i < R; ++i) {
+    std::this_thread::sleep_for(std::chrono::microseconds(1500));
+    const double a = now_us();
+    submit(0);
+    restart_submit += now_us() - a;
+    wait_for(seq);
+    restart_done += now_us() - a;
+  }
+  printf("{\"harness\": \"engine\", \"requests_per_batch\": %d, \"request_bytes\": %zu, \"window_sets\": %d, \"workgroups\": %d, \"batches\": %d, \"bit_exact\": %s, "
+         "\"one_at_a_time_us_per_batch\": %.2f, \"submit_us\": %.2f, \"in_flight_us_per_batch\": %.2f, \"in_flight_us_per_request\": %.3f, \"in_flight_GBps_4N\": %.0f, "
+         "\"after_idle_submit_us\": %.1f, \"after_idle_batch_us\": %.1f, \"engine_launches\": %llu}\n",
+         nreq, req, depth, wgs, batches, exact ? "true" : "false", alone, sub / batches, piped, piped / nreq, 4.0 * nreq * req / (piped * 1e-6) / 1e9,
+         restart_submit / R, restart_done / R, (unsigned long long)p_flh_engine_launches(e));
+  p_flh_engine_destroy(e);
+  return exact ? 0 : 5;
+}

@@ -143,3 +143,23 @@ def test_engine_refuses_bad_arguments_on_the_host(fl):
         assert int(lib.flh_engine_launches(eng)) == 0 and int(lib.flh_engine_completed(eng)) == 0
     finally:
         _lib.check(lib.flh_engine_destroy(eng))
+
+
+@pytest.mark.gpu
+def test_engine_harness_moves_the_bytes_and_reports_its_latency():
+    """tests/harness/engine_bench drives flh_engine_* from C++ the way the plugin does (a batch at a time, several in
+    flight, after the engine has gone down for lack of work) and compares what arrived with what was sent."""
+    import json
+    import os
+    import subprocess
+    from fuselink_amd import build
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "harness", "engine_bench")
+    if not os.path.exists(exe):
+        build.build_harness(verbose=False)
+    res = subprocess.run([exe, build.lib_path(), "--requests", "5", "--depth", "3", "--batches", "300"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr[-2000:]
+    out = json.loads(res.stdout.strip().splitlines()[-1])
+    assert out["bit_exact"] and out["requests_per_batch"] == 5 and out["engine_launches"] >= 20   # every idle period took it down
+    assert 0 < out["in_flight_us_per_batch"] <= out["one_at_a_time_us_per_batch"] * 1.2
+    print(out)
