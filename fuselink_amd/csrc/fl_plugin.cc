@@ -948,7 +948,10 @@ ncclResult_t shm_progress_send(ShmComm* c, ShmRequest* r) {
       return ncclSuccess;
     }
     // the landing windows hold one wave: the previous one must have been reassembled
-    if (c->w->waves_consumed.load(std::memory_order_acquire) < c->waves_published) return ncclSuccess;
+    if (c->w->waves_consumed.load(std::memory_order_acquire) < c->waves_published) {
+      if (c->w->recv_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding"); return ncclRemoteError; }
+      return ncclSuccess;
+    }
     if (r->refresh && r->sent == 0) c->epoch_bytes = 0;
     uint64_t wave = (uint64_t)wave_chunks(r->credits, g_par.lanes, chunk, c->wins.cap[0], c->epoch_bytes / chunk) * chunk;
     if (wave > r->size - r->sent) wave = r->size - r->sent;
@@ -999,7 +1002,10 @@ ncclResult_t shm_progress_recv(ShmComm* c, ShmRequest* r) {
   DeviceScope keep;
   if (r->phase == 0) {
     ShmWave& wv = c->w->wave[c->waves_seen % FL_NET_MAX_REQUESTS];
-    if (wv.seq.load(std::memory_order_acquire) != c->waves_seen + 1) return ncclSuccess;   // nothing has landed yet
+    if (wv.seq.load(std::memory_order_acquire) != c->waves_seen + 1) {   // nothing has landed yet
+      if (c->w->send_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the sending process closed the connection with a receive outstanding"); return ncclRemoteError; }
+      return ncclSuccess;
+    }
     if (wv.fifo_idx != r->fifo_idx) { FL_WARN("NET/FuseLink : a wave of request %llu arrived while %llu is first in line", (unsigned long long)wv.fifo_idx, (unsigned long long)r->fifo_idx); return ncclInternalError; }
     if (wv.offset + wv.bytes > r->size) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
     FL_HIPCHECK(hipSetDevice(c->hip_device));
@@ -1044,7 +1050,10 @@ ncclResult_t shm_test(ShmRequest* r, int* done, int* sizes) {
   if (r->phase != 2) return ncclSuccess;
   if (r->type == kReqSend) {
     // the send is complete once its last wave has been taken out of the landing windows
-    if (c->w->waves_consumed.load(std::memory_order_acquire) < r->wave_no) return ncclSuccess;
+    if (c->w->waves_consumed.load(std::memory_order_acquire) < r->wave_no) {
+      if (c->w->recv_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding"); return ncclRemoteError; }
+      return ncclSuccess;
+    }
   } else {
     c->r_finished++;
     c->r_inflight--;

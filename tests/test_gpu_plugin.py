@@ -833,3 +833,91 @@ def test_rccl_loads_the_plugin_and_probes_every_device(name):
     for dev in range(8):
         assert f"'fuselink{dev}'" in log           # getProperties of every virtual NIC was read
     assert "allreduce 1024.0" in log
+
+
+@pytest.mark.parametrize("seed", range(int(__import__("os").environ.get("FUSELINK_RANDOM_SEEDS", "10"))))
+def test_random_traffic_of_several_connections_arrives_intact(net, seed):
+    """Random mixes of what the paths distinguish: 1 to 5 connections on one GPU; requests of 0 bytes, a few bytes, ragged
+    lengths, whole chunks, more than the engine takes (launch pairs), more than the windows hold (waves); receives
+    larger than their sends; credit rows that change between refreshes; every completion mode with and without the
+    engine.  One thread posts and polls in random order, as several proxy threads' calls could interleave.  Every
+    destination byte is compared with the source (the rest must stay zero) and every receive reports its send's size."""
+    import torch
+    rng = np.random.default_rng(9100 + seed)
+    lanes = int(rng.choice([1, 2, 3, 5, 8, 16]))
+    chunk = int(rng.choice([4 << 10, 32 << 10, 64 << 10, 256 << 10]))
+    completion, engine = [(2, 1), (2, 1), (2, 0), (1, 0), (0, 0)][seed % 5]
+    cadence = int(rng.choice([2, 8, 1000]))
+    net.reconfigure(NCCL_FUSELINK_LANES=lanes, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_WINDOW_UNITS=int(rng.choice([1, 2, 4])),
+                    NCCL_FUSELINK_REFRESH_BATCH=cadence, NCCL_FUSELINK_COMPLETION=completion, NCCL_FUSELINK_ENGINE=engine,
+                    NCCL_FUSELINK_ENGINE_SETS=int(rng.choice([1, 2, 3])), NCCL_FUSELINK_BATCH=int(rng.choice([2, 8, 32])))
+    net.set_credits([int(c) for c in rng.integers(0, 5, size=lanes)])
+
+    def draw_size():
+        kind = rng.integers(0, 8)
+        if kind == 0:
+            return 0
+        if kind == 1:
+            return int(rng.integers(1, 200))
+        if kind == 2:
+            return int(rng.integers(1, 4 * chunk))                       # ragged
+        if kind == 3:
+            return int(rng.integers(1, 9)) * chunk                      # whole chunks
+        if kind == 4:
+            return int(rng.integers(1, 9)) * chunk + int(rng.integers(1, chunk))
+        if kind == 5:
+            return (1 << 20) + int(rng.integers(1, 1 << 20))             # past what the engine takes
+        if kind == 6:
+            return int(rng.integers(1, 3)) * (6 << 20) + int(rng.integers(0, 4097))   # more than small windows hold
+        return 512 << 10
+
+    n_conn = int(rng.integers(1, 6))
+    conns = []
+    for k in range(n_conn):
+        sizes = [draw_size() for _ in range(int(rng.integers(4, 25)))]
+        slack = [int(rng.integers(0, 300)) if rng.random() < 0.3 else 0 for _ in sizes]     # the receive may be larger than the send
+        offs = np.concatenate([[0], np.cumsum([s + e + int(rng.integers(0, 3)) * 7 for s, e in zip(sizes, slack)])]).astype(np.int64)
+        total = int(offs[-1]) + 64
+        src_np = rng.integers(1, 256, size=total, dtype=np.uint8)       # no zero byte: an unwritten destination byte shows
+        c = _open(net, k % lanes, torch.from_numpy(src_np).cuda(), torch.zeros(total, dtype=torch.uint8, device="cuda"))
+        c.update(src_np=src_np, sizes=sizes, slack=slack, offs=offs, posted=0, sent=0, rq=[], sq=[], window=int(rng.integers(1, 9)))
+        conns.append(c)
+    steps = 0
+    while any(c["sent"] < len(c["sizes"]) or c["rq"] or c["sq"] for c in conns):
+        steps += 1
+        assert steps < 2_000_000, "no progress"
+        c = conns[int(rng.integers(0, n_conn))]
+        act = rng.integers(0, 4)
+        if act == 0 and c["posted"] < len(c["sizes"]) and len(c["rq"]) < c["window"]:
+            q = c["posted"]
+            rc, req = net.irecv(c["r"], [c["dst"].data_ptr() + int(c["offs"][q])], [c["sizes"][q] + c["slack"][q]], [q], [c["rmh"]])
+            assert rc == 0
+            if req:                                                        # none: the refresh gate holds it until the receives in flight are done
+                c["rq"].append((req, c["sizes"][q]))
+                c["posted"] += 1
+        elif act == 1 and c["sent"] < c["posted"]:
+            q = c["sent"]
+            rc, req = net.isend(c["s"], c["src"].data_ptr() + int(c["offs"][q]), c["sizes"][q], q, c["smh"])
+            assert rc == 0 and req
+            c["sq"].append(req)
+            c["sent"] += 1
+        elif act == 2 and c["rq"]:
+            rc, done, got = net.test(c["rq"][0][0])
+            assert rc == 0
+            if done:
+                assert got == c["rq"][0][1]
+                c["rq"].pop(0)
+        elif act == 3 and c["sq"]:
+            rc, done, _ = net.test(c["sq"][0])
+            assert rc == 0
+            if done:
+                c["sq"].pop(0)
+        if rng.random() < 0.002:
+            net.set_credits([int(x) for x in rng.integers(0, 5, size=lanes)])   # taken up at the connections' next refresh
+    for c in conns:
+        exp = np.zeros_like(c["src_np"])
+        for q, n in enumerate(c["sizes"]):
+            o = int(c["offs"][q])
+            exp[o:o + n] = c["src_np"][o:o + n]
+        np.testing.assert_array_equal(c["dst"].cpu().numpy(), exp)
+        _close(net, c)
