@@ -1425,7 +1425,7 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
   e->sets = window_sets;
   e->host_slots = 64;
   e->idle_us = idle_us ? idle_us : 200;
-  e->wait_us = 2000000;
+  e->wait_us = (uint64_t)g_engine_wait_us;   // two seconds unless a test has asked for less (flh_tune "engine_wait_us")
   FL_HIP(hipSetDevice(device));
   FL_HIP(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
   FL_HIP(hipHostMalloc((void**)&e->h_ring, (size_t)e->host_slots * kEngineDescBytes, hipHostMallocMapped));

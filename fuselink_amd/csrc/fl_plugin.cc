@@ -1984,7 +1984,7 @@ ncclResult_t launch_complete(Peer* pr, uint64_t seq, bool* done) {
 
 // Engine batches handed over and not yet reported complete.
 uint64_t engine_in_flight(Peer* pr) {
-  if (!pr->engine) return 0;
+  if (!pr->engine || !pr->engine_ok.load(std::memory_order_acquire)) return 0;   // an engine that went down holds nothing back
   const uint64_t sub = pr->engine_submitted.load(std::memory_order_acquire), done = flh_engine_completed(pr->engine);
   return sub > done ? sub - done : 0;
 }

@@ -151,6 +151,8 @@ int64_t flh_constant(int which);
  * "sched_seg_min" = chunks from which a lent workspace makes the scan scheduler use several workgroups (4096).
  * "xcd_runs" = 1/0: launches of 256 copy workgroups and more hand each of the eight XCDs runs of 32 consecutive
  * tiles (1 MiB) instead of every eighth tile (1, the default; 3-5 % faster copies).
+ * "engine_wait_us" = limit of every wait inside a lane engine created afterwards (2 000 000; tests of the failure
+ * path ask for a microsecond).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL.
  * The tunables are process-wide and read by every launch: set them while no other thread launches. */
 int flh_tune(const char* key, int64_t value);

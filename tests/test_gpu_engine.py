@@ -163,3 +163,44 @@ def test_engine_harness_moves_the_bytes_and_reports_its_latency():
     assert out["bit_exact"] and out["requests_per_batch"] == 5 and out["engine_launches"] >= 20   # every idle period took it down
     assert 0 < out["in_flight_us_per_batch"] <= out["one_at_a_time_us_per_batch"] * 1.2
     print(out)
+
+
+def test_a_wait_that_runs_out_takes_the_engine_down_and_is_reported(fl):
+    """Every wait inside the resident kernel is bounded.  With the bound set to a microsecond and one window set, the
+    workers of a second batch cannot get the windows before the first batch is through: their wait runs out, the kernel
+    reports FLH_E_STATE through the control block and every workgroup leaves (the stream drains, destroy returns);
+    later submits are refused.  No kernel is left spinning."""
+    core, torch, _lib = fl
+    lib = _lib.load()
+    lanes, chunk, n_req = 8, 256 << 10, 32
+    _lib.check(lib.flh_tune(b"engine_wait_us", 1))
+    eng = C.c_void_p()
+    try:
+        _lib.check(lib.flh_engine_create(0, 0, 100000, 1, C.byref(eng)))
+    finally:
+        _lib.check(lib.flh_tune(b"engine_wait_us", 2000000))
+    try:
+        cap = 8 << 20
+        wins = [torch.zeros(cap, dtype=torch.uint8, device="cuda") for _ in range(lanes)]
+        W = core.make_windows([t.data_ptr() for t in wins], [cap] * lanes)
+        status = core.new_status()
+        srcs = [torch.full((512 << 10,), 1 + q, dtype=torch.uint8, device="cuda") for q in range(n_req)]
+        dsts = [torch.zeros(512 << 10, dtype=torch.uint8, device="cuda") for _ in range(n_req)]
+        out = core.new_schedule_buffers(n_req * 2 + 1)
+        b = core.batch_params(srcs, dsts, chunk, [1] * lanes)
+        torch.cuda.synchronize()
+        seq = C.c_uint64()
+        for _ in range(2):   # back to back: the second batch wants the first one's windows
+            _lib.check(lib.flh_engine_submit(eng, C.byref(b), C.byref(W), out.table.data_ptr(), out.hdr.data_ptr(), status.data_ptr(), C.byref(seq), None))
+        deadline = time.time() + 10
+        while lib.flh_engine_error(eng) == 0 and lib.flh_engine_completed(eng) < 2:
+            assert time.time() < deadline, "neither an error nor completion"
+        assert lib.flh_engine_error(eng) == -6    # FLH_E_STATE: an error, not completion
+        assert lib.flh_engine_completed(eng) < 2
+        rc = lib.flh_engine_submit(eng, C.byref(b), C.byref(W), out.table.data_ptr(), out.hdr.data_ptr(), status.data_ptr(), C.byref(seq), None)
+        assert rc < 0 and b"went down" in lib.flh_last_error()
+    finally:
+        t0 = time.time()
+        _lib.check(lib.flh_engine_destroy(eng))     # waits for the kernel: it has left, or leaves at its next poll
+        assert time.time() - t0 < 5
+        torch.cuda.synchronize()

@@ -921,3 +921,58 @@ def test_random_traffic_of_several_connections_arrives_intact(net, seed):
             exp[o:o + n] = c["src_np"][o:o + n]
         np.testing.assert_array_equal(c["dst"].cpu().numpy(), exp)
         _close(net, c)
+
+
+def test_an_engine_that_goes_down_fails_its_requests_and_traffic_falls_back_to_launches(net):
+    """The lane engine's waits are bounded; with the bound at a microsecond and one window set its second batch in a row
+    cannot get the windows in time, the engine reports the failure and goes down.  The requests it held complete with
+    ncclRemoteError (as a queue pair in the error state completes its work requests, src/plugin.cc:1839-1861), nothing
+    hangs, and a connection opened afterwards moves its bytes through launch pairs."""
+    import time
+    import torch
+    piece = 512 << 10
+    net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=256 << 10, NCCL_FUSELINK_BATCH=8, NCCL_FUSELINK_ENGINE=1, NCCL_FUSELINK_ENGINE_SETS=1,
+                    NCCL_FUSELINK_REFRESH_BATCH=1000)
+    net.lib.flh_tune.argtypes = [__import__("ctypes").c_char_p, __import__("ctypes").c_int64]
+    assert net.lib.flh_tune(b"engine_wait_us", 1) == 0
+    try:
+        rng = np.random.default_rng(77)
+        n = 32
+        src_np = rng.integers(1, 256, size=(n + 1) * piece, dtype=np.uint8)
+        c = _open(net, 0, torch.from_numpy(src_np).cuda(), torch.zeros((n + 1) * piece, dtype=torch.uint8, device="cuda"))   # creates the GPU's engine
+    finally:
+        assert net.lib.flh_tune(b"engine_wait_us", 2000000) == 0
+    # one request on its own passes (a first batch waits for nothing) and takes the connection off its refresh boundary
+    _send_recv(net, c["s"], c["r"], c["src"], c["dst"], piece, 99, c["smh"], c["rmh"], src_off=n * piece, dst_off=n * piece)
+    reqs = []
+    for q in range(n):
+        rc, rreq = net.irecv(c["r"], [c["dst"].data_ptr() + q * piece], [piece], [q], [c["rmh"]])
+        assert rc == 0 and rreq
+        reqs.append(rreq)
+    for q in range(n):   # every eighth send fills a batch, which goes out inside that isend: four batches in a row
+        rc, sreq = net.isend(c["s"], c["src"].data_ptr() + q * piece, piece, q, c["smh"])
+        assert rc == 0 and sreq
+        reqs.append(sreq)
+    failed = finished = 0
+    deadline = time.time() + 20
+    pending = list(reqs)
+    while pending:
+        assert time.time() < deadline, "requests neither completed nor failed"
+        rc, done, _ = net.test(pending[0])
+        if rc != 0:
+            assert rc == P.ncclRemoteError
+            failed += 1
+            pending.pop(0)
+        elif done:
+            finished += 1
+            pending.pop(0)
+    assert failed >= 2 and finished + failed == 2 * n     # at least the second batch's requests
+    # the GPU's staging side lives on: new traffic goes by launch pairs and arrives
+    src2_np = rng.integers(0, 256, size=4 * piece, dtype=np.uint8)
+    c2 = _open(net, 1, torch.from_numpy(src2_np).cuda(), torch.zeros(4 * piece, dtype=torch.uint8, device="cuda"))
+    for q in range(4):
+        _send_recv(net, c2["s"], c2["r"], c2["src"], c2["dst"], piece, q, c2["smh"], c2["rmh"], src_off=q * piece, dst_off=q * piece)
+    np.testing.assert_array_equal(c2["dst"].cpu().numpy(), src2_np)
+    assert net.launch_stats(c2["s"])["launches"] >= 1
+    _close(net, c2)
+    _close(net, c)
