@@ -516,6 +516,12 @@ def main() -> int:
         "plugin_abi": plugin,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     # what the fraction means for this workload: cached footprints are served in part by the 256 MB Infinity Cache
+                     "note": ("footprint (source, windows, destination) of %d MiB: %s" % (
+                         3 * nbytes >> 20, "largely resident in the 256 MB Infinity Cache, so this is a fraction of the HBM peak reached with that cache's help; "
+                         "the same kernels with nothing cache-resident reach 0.74-0.76 (bench.py --workload cfg5_stress_1GiB_64KiB_16lanes --cache-waves 0)"
+                         if 3 * nbytes <= (256 << 20) else "beyond the 256 MB Infinity Cache" + (
+                             "; moved in cache-resident waves, the windows' traffic stays in the cache" if cwaves else ": every byte is served by HBM"))) if kind == "uniform" else None,
                      "traffic": (None if args.lanes else MEASURED_TRAFFIC.get(f"{args.workload}/{len(cwaves)} waves") if cwaves else None if (waves or twaves) else
                                  MEASURED_TRAFFIC.get(args.workload) if (kind != "blocks" or args.blocks == 256) else None)},
     }
