@@ -101,6 +101,7 @@ SIGNATURES = {
     "flh_scatter_pages_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint32, C.POINTER(Windows),
                                             C.POINTER(UniformParams), C.c_void_p, C.c_void_p]),
     "flh_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]),
+    "flh_copy_runs": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_uint64), C.c_uint32, C.c_void_p]),
     "flh_qp_split": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "flh_pool_create": (C.c_int, [C.c_int, C.c_uint32, C.POINTER(C.c_void_p)]),
     "flh_pool_destroy": (C.c_int, [C.c_void_p]),

@@ -326,6 +326,15 @@ def copy(dst: torch.Tensor, src: torch.Tensor, stream: Optional[torch.cuda.Strea
     check(_lib.load().flh_copy(_ptr(dst), _ptr(src), nbytes, _stream_ptr(stream)))
 
 
+def copy_runs(dsts, srcs, nbytes, stream: Optional[torch.cuda.Stream] = None) -> None:
+    """Up to 16 independent runs in one launch: run r moves nbytes[r] bytes from srcs[r] to dsts[r] (None for an empty run)."""
+    n = len(nbytes)
+    d = (C.c_void_p * n)(*[_ptr(t) if t is not None else None for t in dsts])
+    s = (C.c_void_p * n)(*[_ptr(t) if t is not None else None for t in srcs])
+    b = (C.c_uint64 * n)(*nbytes)
+    check(_lib.load().flh_copy_runs(d, s, b, n, _stream_ptr(stream)))
+
+
 def qp_split(size: int, nqps: int):
     off = (C.c_int * nqps)()
     ln = (C.c_int * nqps)()

@@ -701,6 +701,34 @@ __global__ __launch_bounds__(kCopyBlock) void fl_plain_copy(uint8_t* dst, const 
   }
 }
 
+// Up to FLH_MAX_LANES independent runs in one launch (flh_copy_runs): a workgroup per copy tile, the run of a tile
+// found by a four-step search over the runs' first tiles in the argument block.
+struct CopyRuns {
+  uint8_t* dst[FLH_MAX_LANES];
+  const uint8_t* src[FLH_MAX_LANES];
+  uint64_t bytes[FLH_MAX_LANES];
+  uint32_t first_tile[FLH_MAX_LANES + 1];   // exclusive prefix of the runs' tile counts; entries past the last run repeat the total
+  uint32_t tile_bytes;
+  uint32_t xcd;
+};
+
+template <int NT>
+__global__ __launch_bounds__(kCopyBlock) void fl_copy_runs(CopyRuns a) {
+  warm_kernel_args(a);
+  const uint32_t t = (uint32_t)xcd_tile(blockIdx.x, a.xcd);
+  static_assert(FLH_MAX_LANES == 16, "the search below takes four steps");
+  uint32_t r = 0;
+  if (a.first_tile[r + 8] <= t) r += 8;
+  if (a.first_tile[r + 4] <= t) r += 4;
+  if (a.first_tile[r + 2] <= t) r += 2;
+  if (a.first_tile[r + 1] <= t) r += 1;
+  const uint64_t off = (uint64_t)(t - a.first_tile[r]) * a.tile_bytes;
+  const uint64_t n = a.bytes[r];
+  if (off >= n) return;
+  const uint32_t len = (uint32_t)((n - off) < a.tile_bytes ? (n - off) : a.tile_bytes);
+  block_copy<NT>(a.dst[r] + off, a.src[r] + off, len);
+}
+
 // ------------------------------------------------------------------------------------------------
 // lane engine: a resident kernel that executes batch descriptors
 // ------------------------------------------------------------------------------------------------
@@ -1575,6 +1603,39 @@ int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream) {
   const uint32_t xcd = grid == (bytes + tile - 1) / tile ? fl_xcd_full(grid) : 0;   // only with one workgroup per tile
   if (fl_use_nt(2 * bytes)) FL_LAUNCH(fl_plain_copy<3>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile, xcd);
   else FL_LAUNCH(fl_plain_copy<0>, dim3(grid), dim3(kCopyBlock), 0, s, (uint8_t*)d_dst, (const uint8_t*)d_src, bytes, tile, xcd);
+  FL_HIP(hipGetLastError());
+  return FLH_OK;
+}
+
+int flh_copy_runs(void* const* d_dst, const void* const* d_src, const uint64_t* bytes, uint32_t n, void* stream) {
+  if (n == 0) return FLH_OK;
+  if (!d_dst || !d_src || !bytes) return fl_set_error(FLH_E_ARG, "null pointer");
+  if (n > FLH_MAX_LANES) return fl_set_error(FLH_E_ARG, "%u runs: at most %d go into one launch", n, FLH_MAX_LANES);
+  int rc = fl_need_init();
+  if (rc) return rc;
+  CopyRuns a;
+  memset(&a, 0, sizeof(a));
+  a.tile_bytes = FLH_TILE_BYTES;
+  uint64_t tiles = 0, total = 0;
+  for (uint32_t r = 0; r < FLH_MAX_LANES; ++r) {
+    a.first_tile[r] = (uint32_t)tiles;
+    if (r >= n || bytes[r] == 0) continue;
+    if (!d_dst[r] || !d_src[r]) return fl_set_error(FLH_E_ARG, "run %u has bytes but no buffer", r);
+    a.dst[r] = (uint8_t*)d_dst[r];
+    a.src[r] = (const uint8_t*)d_src[r];
+    a.bytes[r] = bytes[r];
+    tiles += (bytes[r] + a.tile_bytes - 1) / a.tile_bytes;
+    total += bytes[r];
+    if (tiles > 0x7fffffffull) return fl_set_error(FLH_E_ARG, "too many tiles for one launch");
+  }
+  a.first_tile[FLH_MAX_LANES] = (uint32_t)tiles;
+  if (tiles == 0) return FLH_OK;
+  // empty runs share their successor's first tile, so the search lands on the run that owns the tile
+  a.xcd = fl_xcd_full((uint32_t)tiles);
+  fl_prof().kid = 6;
+  hipStream_t s = (hipStream_t)stream;
+  if (fl_use_nt(2 * total)) FL_LAUNCH(fl_copy_runs<3>, dim3((uint32_t)tiles), dim3(kCopyBlock), 0, s, a);
+  else FL_LAUNCH(fl_copy_runs<0>, dim3((uint32_t)tiles), dim3(kCopyBlock), 0, s, a);
   FL_HIP(hipGetLastError());
   return FLH_OK;
 }

@@ -89,6 +89,7 @@ struct Params {
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
   int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
+  int wire_sets = 2;             // NCCL_FUSELINK_WIRE_SETS: sets of landing windows of a receiver on the shared-memory wire = waves on the wire at once
   int wire = 0;                  // NCCL_FUSELINK_WIRE: 0 = both ends in this process (loopback), 1 = the other end is another process (shared-memory wire)
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
@@ -601,13 +602,14 @@ uint32_t wave_chunks(const uint32_t* credits, int lanes, uint64_t chunk, uint64_
 // POSIX shared-memory object and names it in the handle; connect, in another process, maps it.  The object holds the
 // descriptor FIFO (receiver writes, sender reads), a ring of wave completions (sender writes, receiver reads: the
 // stand-in for the WRITE_WITH_IMM completions) and the IPC handle of the receiver's landing windows.  A send then runs
-// as in the reference's layers: the striping kernel stages the request's chunks in the sender's lane windows (HIP VMM,
-// from the unit pool); the wire copies every lane's staged bytes into the receiver's landing window for that lane,
-// device memory of the receiver's process that the sender has opened through hipIpcOpenMemHandle (an imported VMM
-// allocation would be the closer analogue; this runtime refuses hipMemImportFromShareableHandle for another process's
-// descriptor, so the landing windows are a plain device allocation); the sender publishes the wave; the receiver's
-// reassembly kernel writes the posted buffer from its landing windows and acknowledges.  One wave is on the wire at a
-// time per connection (the landing windows are reused wave by wave), requests complete in order.
+// as in the reference's layers: the striping kernel stages a wave of the request's chunks in the sender's lane windows
+// (HIP VMM, from the unit pool); the wire carries every lane's staged bytes into the receiver's landing window for that
+// lane (one launch, flh_copy_runs), device memory of the receiver's process that the sender has opened through
+// hipIpcOpenMemHandle (an imported VMM allocation would be the closer analogue; this runtime refuses
+// hipMemImportFromShareableHandle for another process's descriptor, so the landing windows are a plain device
+// allocation); the sender publishes the wave; the receiver's reassembly kernel writes the posted buffer from its landing
+// windows and hands them back.  The receiver keeps NCCL_FUSELINK_WIRE_SETS sets of landing windows, so that many waves
+// are on the wire at once; requests start, finish and are reported in order.
 void fill_uniform(flh_uniform_params& u, const uint32_t* credits, uint64_t bytes, uint64_t src_base, uint64_t epoch_bytes, uint32_t tile);
 
 constexpr uint64_t kHandleMagicShm = 0x4655534c53484d31ull;   // "FUSLSHM1"
@@ -615,6 +617,7 @@ constexpr uint32_t kShmCommMagic = 0x464c5343;                // "FLSC"
 constexpr uint32_t kShmReqMagic = 0x464c5352;                 // "FLSR"
 constexpr uint32_t kShmListenMagic = 0x464c534c;              // "FLSL"
 
+constexpr int kShmSetsMax = 8;
 struct ShmWave {                   // one wave of chunks that has landed in the receiver's windows
   std::atomic<uint64_t> seq;       // wave number + 1, written last
   uint64_t fifo_idx;               // the descriptor (request) it belongs to
@@ -622,7 +625,7 @@ struct ShmWave {                   // one wave of chunks that has landed in the 
   uint64_t offset;                 // byte offset of the wave in the request
   uint64_t bytes;
   uint32_t last;                   // the request's last wave
-  uint32_t pad;
+  uint32_t set;                    // the set of landing windows it lies in
 };
 struct ShmWire {
   uint64_t magic;
@@ -630,12 +633,12 @@ struct ShmWire {
   uint32_t channelId;
   std::atomic<uint32_t> connected, accepted, send_closed, recv_closed;
   std::atomic<uint32_t> landing_ready;
-  uint32_t pad0;
+  uint32_t landing_sets;           // sets of landing windows = waves that may be on the wire at once
   uint64_t landing_bytes_per_lane;
-  hipIpcMemHandle_t landing;       // lanes x landing_bytes_per_lane of the receiver's device memory
+  hipIpcMemHandle_t landing;       // sets x lanes x landing_bytes_per_lane of the receiver's device memory
   alignas(64) FifoWire fifo[FL_NET_MAX_REQUESTS];          // plugin.cc:487-496: written by the receiver, idx last
   alignas(64) ShmWave wave[FL_NET_MAX_REQUESTS];
-  alignas(64) std::atomic<uint64_t> waves_consumed;        // receiver: waves reassembled so far (the landing windows are free again)
+  alignas(64) std::atomic<uint64_t> waves_consumed;        // receiver: waves reassembled so far, in order (their landing windows are free again)
 };
 
 struct ShmRequest {
@@ -643,18 +646,24 @@ struct ShmRequest {
   int type = kReqUnused;
   struct ShmComm* comm = nullptr;
   uint64_t fifo_idx = 0;           // 1-based descriptor number
+  uint64_t size = 0;
+  uint32_t credits[FLH_MAX_LANES] = {};
   // sender
   const uint8_t* src = nullptr;
-  uint64_t size = 0, sent = 0;     // bytes of the request, bytes whose waves have been published
-  uint64_t wave_no = 0;            // number of the wave in flight (1-based), 0 = none
-  uint64_t wave_bytes = 0, wave_epoch = 0;
-  int phase = 0;                   // sender: 0 idle, 1 stripe + wire queued, 2 published; receiver: 0 waiting for a wave, 1 reassembly queued
-  uint32_t credits[FLH_MAX_LANES] = {};
+  uint64_t launched = 0;           // bytes whose waves have been queued on the GPU
+  bool all_launched = false;       // (a request of no bytes still takes one wave)
+  uint64_t last_wave = 0;          // number (from 1) of the request's last wave, once all_launched
   bool refresh = false;
   // receiver
   uint8_t* dst = nullptr;
-  uint64_t received = 0;
-  int done_size = 0;
+  uint64_t received = 0;           // bytes reassembled
+  bool complete = false;           // the last wave has been reassembled
+};
+
+struct ShmFlight {                 // a wave whose GPU work is queued: the event of its set tells when it is through
+  ShmRequest* req;
+  uint64_t fifo_idx, epoch_bytes, offset, bytes;
+  uint32_t last, set;
 };
 
 struct ShmComm {
@@ -667,9 +676,13 @@ struct ShmComm {
   std::mutex mu;
   ShmRequest reqs[FL_NET_MAX_REQUESTS];
   uint64_t fifoHead = 0, fifoTail = 0;       // sender: next descriptor to match; receiver: next to post
-  std::deque<ShmRequest*> active;            // requests in flight, in order; only the first makes progress
+  std::deque<ShmRequest*> active;            // requests in flight, in order: they start, finish and are reported in that order
+  size_t cursor = 0;                         // sender: first request of `active` with waves left to launch; receiver: the one the next wave belongs to
+  std::deque<ShmFlight> flights;             // waves queued on the GPU, in order
   uint64_t epoch_bytes = 0;                  // sender: the scheduler's carried prefix
-  uint64_t waves_published = 0, waves_seen = 0;
+  uint64_t waves_launched = 0;               // sender: waves queued on the GPU so far; receiver: waves taken off the wire so far
+  uint64_t waves_published = 0;              // sender: waves announced to the receiver
+  uint64_t waves_done = 0;                   // receiver: waves reassembled (what waves_consumed says)
   int64_t r_finished = 0, r_inflight = 0;
   int fuselink_offset = -1;
   uint8_t credits[FL_NET_MAX_LANES] = {};
@@ -677,12 +690,13 @@ struct ShmComm {
   // GPU side
   bool gpu_ready = false;
   int hip_device = -1;
+  int sets = 0;
   hipStream_t stream = nullptr;
-  hipEvent_t ev = nullptr;
+  hipEvent_t ev[kShmSetsMax] = {};           // one per set of landing windows: the latest wave that uses the set
   flh_window* win[FL_NET_MAX_LANES] = {};    // sender: staging windows
   flh_windows wins = {};
   uint8_t* landing = nullptr;                // receiver: its allocation; sender: the same memory opened through IPC
-  flh_windows landing_wins = {};
+  flh_windows landing_wins[kShmSetsMax] = {};
   flh_chunk_desc* d_table = nullptr;
   flh_sched_hdr* d_hdr = nullptr;
   int32_t *h_status = nullptr, *d_status = nullptr;
@@ -706,7 +720,7 @@ void shm_comm_free(ShmComm* c) {
     if (c->d_table) (void)hipFree(c->d_table);
     if (c->d_hdr) (void)hipFree(c->d_hdr);
     if (c->h_status) (void)hipHostFree(c->h_status);
-    if (c->ev) (void)hipEventDestroy(c->ev);
+    for (hipEvent_t e : c->ev) if (e) (void)hipEventDestroy(e);
     (void)hipStreamDestroy(c->stream);
   }
   if (c->w) munmap(c->w, sizeof(ShmWire));
@@ -796,6 +810,17 @@ ncclResult_t shm_accept(ShmListen* lc, void** recvComm) {
   return ncclSuccess;
 }
 
+// set k, lane l of the landing windows: one allocation, set after set, lane after lane
+void shm_landing_windows(ShmComm* c, uint64_t per_lane) {
+  for (int k = 0; k < c->sets; ++k) {
+    c->landing_wins[k].n_lanes = (uint32_t)g_par.lanes;
+    for (int l = 0; l < g_par.lanes; ++l) {
+      c->landing_wins[k].base[l] = c->landing + ((uint64_t)k * (uint64_t)g_par.lanes + (uint64_t)l) * per_lane;
+      c->landing_wins[k].cap[l] = per_lane;
+    }
+  }
+}
+
 // stream, status word, table buffers; the sender's staging windows or the receiver's landing windows
 ncclResult_t shm_setup_gpu(ShmComm* c, int device) {
   if (c->gpu_ready) return ncclSuccess;
@@ -804,7 +829,6 @@ ncclResult_t shm_setup_gpu(ShmComm* c, int device) {
   c->hip_device = device;
   FL_HIPCHECK(hipSetDevice(device));
   FL_HIPCHECK(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-  FL_HIPCHECK(hipEventCreateWithFlags(&c->ev, hipEventDisableTiming));
   FL_HIPCHECK(hipHostMalloc((void**)&c->h_status, 64, hipHostMallocMapped));
   memset(c->h_status, 0, 64);
   FL_HIPCHECK(hipHostGetDevicePointer((void**)&c->d_status, c->h_status, 0));
@@ -822,15 +846,18 @@ ncclResult_t shm_setup_gpu(ShmComm* c, int device) {
     }
     FL_HIPCHECK(hipMalloc((void**)&c->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
     FL_HIPCHECK(hipMalloc((void**)&c->d_hdr, sizeof(flh_sched_hdr)));
+    // (the landing windows, and with them the number of sets and their events, come with the receiver's first descriptor)
   } else {
-    FL_HIPCHECK(hipMalloc((void**)&c->landing, cap * (uint64_t)g_par.lanes));
+    c->sets = g_par.wire_sets;
+    const uint64_t bytes = cap * (uint64_t)g_par.lanes * (uint64_t)c->sets;
+    if (bytes >= (2ull << 30)) { FL_WARN("NET/FuseLink : %d sets of landing windows take %llu bytes; a shared allocation must stay under 2 GiB", c->sets, (unsigned long long)bytes); return ncclInvalidUsage; }
+    FL_HIPCHECK(hipMalloc((void**)&c->landing, bytes));
     FL_HIPCHECK(hipIpcGetMemHandle(&c->w->landing, c->landing));
     c->w->landing_bytes_per_lane = cap;
+    c->w->landing_sets = (uint32_t)c->sets;
+    for (int k = 0; k < c->sets; ++k) FL_HIPCHECK(hipEventCreateWithFlags(&c->ev[k], hipEventDisableTiming));
+    shm_landing_windows(c, cap);
     c->w->landing_ready.store(1, std::memory_order_release);
-  }
-  if (!c->is_send) {
-    c->landing_wins.n_lanes = (uint32_t)g_par.lanes;
-    for (int l = 0; l < g_par.lanes; ++l) { c->landing_wins.base[l] = c->landing + (uint64_t)l * cap; c->landing_wins.cap[l] = cap; }
   }
   c->gpu_ready = true;
   return ncclSuccess;
@@ -915,13 +942,15 @@ ncclResult_t shm_isend(ShmComm* c, void* data, int size, int tag, MemHandle* mh,
     if (!c->w->landing_ready.load(std::memory_order_acquire)) return ncclSuccess;
     DeviceScope keep;
     FL_HIPCHECK(hipSetDevice(c->hip_device));
-    FL_HIPCHECK(hipIpcOpenMemHandle((void**)&c->landing, c->w->landing, hipIpcMemLazyEnablePeerAccess));
-    c->landing_wins.n_lanes = (uint32_t)g_par.lanes;
-    for (int l = 0; l < g_par.lanes; ++l) {
-      c->landing_wins.base[l] = c->landing + (uint64_t)l * c->w->landing_bytes_per_lane;
-      c->landing_wins.cap[l] = c->w->landing_bytes_per_lane;
+    if (c->w->landing_bytes_per_lane < c->wins.cap[0] || c->w->landing_sets < 1 || c->w->landing_sets > (uint32_t)kShmSetsMax) {
+      FL_WARN("NET/FuseLink : the receiver's landing windows (%u sets of %llu bytes per lane) do not fit this side's staging windows",
+              c->w->landing_sets, (unsigned long long)c->w->landing_bytes_per_lane);
+      return ncclInvalidUsage;
     }
-    if (c->w->landing_bytes_per_lane < c->wins.cap[0]) { FL_WARN("NET/FuseLink : the receiver's landing windows are smaller than the staging windows"); return ncclInvalidUsage; }
+    FL_HIPCHECK(hipIpcOpenMemHandle((void**)&c->landing, c->w->landing, hipIpcMemLazyEnablePeerAccess));
+    c->sets = (int)c->w->landing_sets;
+    for (int k = 0; k < c->sets; ++k) FL_HIPCHECK(hipEventCreateWithFlags(&c->ev[k], hipEventDisableTiming));
+    shm_landing_windows(c, c->w->landing_bytes_per_lane);
   }
   ShmRequest* r = shm_get_request(c, kReqSend);
   if (!r) return ncclInternalError;
@@ -937,98 +966,129 @@ ncclResult_t shm_isend(ShmComm* c, void* data, int size, int tag, MemHandle* mh,
   return ncclSuccess;
 }
 
-// One step of the connection's first request in flight (c->mu held).
-ncclResult_t shm_progress_send(ShmComm* c, ShmRequest* r) {
+// The sender's side of the wire (c->mu held): queue waves on the GPU while sets of landing windows are free, announce
+// the waves whose copies have finished.  A wave is the striping launch into this side's staging windows plus one launch
+// that carries every lane's staged bytes into the receiver's landing windows of the wave's set; launches of one stream
+// run in order, so the next wave's striping cannot overtake the copy that still reads the staging windows.
+ncclResult_t shm_progress_send(ShmComm* c) {
   const uint64_t chunk = (uint64_t)g_par.chunk;
   DeviceScope keep;
-  if (r->phase == 0) {
-    if (r->size == 0 && r->sent == 0 && r->wave_no == 0) {
-      // nothing to move: the completion alone travels
-    } else if (r->sent >= r->size) {
-      return ncclSuccess;
-    }
-    // the landing windows hold one wave: the previous one must have been reassembled
-    if (c->w->waves_consumed.load(std::memory_order_acquire) < c->waves_published) {
+  bool device_set = false;
+  // announce what has landed: the stand-in for the WRITE_WITH_IMM completions (plugin.cc:1453-1465)
+  while (!c->flights.empty()) {
+    const ShmFlight& f = c->flights.front();
+    hipError_t e = hipEventQuery(c->ev[f.set]);
+    if (e == hipErrorNotReady) break;
+    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+    if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its staging window (status %d)", *c->h_status); return ncclInternalError; }
+    ShmWave& wv = c->w->wave[c->waves_published % FL_NET_MAX_REQUESTS];
+    wv.fifo_idx = f.fifo_idx;
+    wv.epoch_bytes = f.epoch_bytes;
+    wv.offset = f.offset;
+    wv.bytes = f.bytes;
+    wv.last = f.last;
+    wv.set = f.set;
+    c->waves_published++;
+    wv.seq.store(c->waves_published, std::memory_order_release);
+    c->flights.pop_front();
+  }
+  // queue further waves: a set of landing windows is free once the wave that used it last has been reassembled
+  while (c->cursor < c->active.size()) {
+    ShmRequest* r = c->active[c->cursor];
+    if (r->all_launched) { c->cursor++; continue; }
+    const uint64_t consumed = c->w->waves_consumed.load(std::memory_order_acquire);
+    if (c->waves_launched - consumed >= (uint64_t)c->sets) {
       if (c->w->recv_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding"); return ncclRemoteError; }
-      return ncclSuccess;
+      break;
     }
-    if (r->refresh && r->sent == 0) c->epoch_bytes = 0;
+    if (r->refresh && r->launched == 0) c->epoch_bytes = 0;
     uint64_t wave = (uint64_t)wave_chunks(r->credits, g_par.lanes, chunk, c->wins.cap[0], c->epoch_bytes / chunk) * chunk;
-    if (wave > r->size - r->sent) wave = r->size - r->sent;
-    FL_HIPCHECK(hipSetDevice(c->hip_device));
+    if (wave > r->size - r->launched) wave = r->size - r->launched;
+    const uint32_t set = (uint32_t)(c->waves_launched % (uint64_t)c->sets);
+    if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
     if (wave) {
       flh_uniform_params u;
-      fill_uniform(u, r->credits, wave, r->sent, c->epoch_bytes, FLH_TILE_BYTES);
+      fill_uniform(u, r->credits, wave, r->launched, c->epoch_bytes, FLH_TILE_BYTES);
       FL_FLHCHECK(flh_stripe_uniform(r->src, r->size, &c->wins, &u, c->d_table, c->d_hdr, c->d_status, c->stream));
-      // the wire: every lane's staged bytes into the receiver's landing window for that lane
+      // the wire: every lane's staged bytes into the receiver's landing window of that lane, one launch for all lanes
       FlCreditRow row;
       fl_row_make(r->credits, (uint32_t)g_par.lanes, row);
       uint64_t lane_bytes[FLH_MAX_LANES];
       uint32_t lane_chunks[FLH_MAX_LANES];
       fl_row_lane_totals(row, c->epoch_bytes / chunk, wave, chunk, lane_bytes, lane_chunks);
-      for (int l = 0; l < g_par.lanes; ++l)
-        if (lane_bytes[l]) FL_FLHCHECK(flh_copy(c->landing_wins.base[l], c->wins.base[l], lane_bytes[l], c->stream));
+      FL_FLHCHECK(flh_copy_runs(c->landing_wins[set].base, c->wins.base, lane_bytes, (uint32_t)g_par.lanes, c->stream));
     }
-    FL_HIPCHECK(hipEventRecord(c->ev, c->stream));
-    r->wave_bytes = wave;
-    r->wave_epoch = c->epoch_bytes;
-    r->phase = 1;
-    return ncclSuccess;
-  }
-  if (r->phase == 1) {
-    hipError_t e = hipEventQuery(c->ev);
-    if (e == hipErrorNotReady) return ncclSuccess;
-    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
-    if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its staging window (status %d)", *c->h_status); return ncclInternalError; }
-    // publish the wave: the stand-in for the WRITE_WITH_IMM completion (plugin.cc:1453-1465)
-    ShmWave& wv = c->w->wave[c->waves_published % FL_NET_MAX_REQUESTS];
-    wv.fifo_idx = r->fifo_idx;
-    wv.epoch_bytes = r->wave_epoch;
-    wv.offset = r->sent;
-    wv.bytes = r->wave_bytes;
-    wv.last = r->sent + r->wave_bytes >= r->size ? 1u : 0u;
-    c->waves_published++;
-    wv.seq.store(c->waves_published, std::memory_order_release);
-    c->epoch_bytes += r->wave_bytes;
-    r->sent += r->wave_bytes;
-    r->wave_no = c->waves_published;
-    r->phase = r->sent >= r->size ? 2 : 0;
-    return ncclSuccess;
+    FL_HIPCHECK(hipEventRecord(c->ev[set], c->stream));
+    ShmFlight f;
+    f.req = r;
+    f.fifo_idx = r->fifo_idx;
+    f.epoch_bytes = c->epoch_bytes;
+    f.offset = r->launched;
+    f.bytes = wave;
+    f.set = set;
+    c->epoch_bytes += wave;
+    r->launched += wave;
+    c->waves_launched++;
+    f.last = r->launched >= r->size ? 1u : 0u;
+    if (f.last) { r->all_launched = true; r->last_wave = c->waves_launched; }
+    c->flights.push_back(f);
   }
   return ncclSuccess;
 }
 
-ncclResult_t shm_progress_recv(ShmComm* c, ShmRequest* r) {
+// The receiver's side (c->mu held): reassemble the waves that have been announced out of their landing windows, and
+// hand the windows back, in order, as the reassembly launches finish.
+ncclResult_t shm_progress_recv(ShmComm* c) {
   DeviceScope keep;
-  if (r->phase == 0) {
-    ShmWave& wv = c->w->wave[c->waves_seen % FL_NET_MAX_REQUESTS];
-    if (wv.seq.load(std::memory_order_acquire) != c->waves_seen + 1) {   // nothing has landed yet
-      if (c->w->send_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the sending process closed the connection with a receive outstanding"); return ncclRemoteError; }
-      return ncclSuccess;
+  bool device_set = false;
+  while (!c->flights.empty()) {
+    const ShmFlight& f = c->flights.front();
+    hipError_t e = hipEventQuery(c->ev[f.set]);
+    if (e == hipErrorNotReady) break;
+    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
+    if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its landing window or buffer (status %d)", *c->h_status); return ncclInternalError; }
+    f.req->received += f.bytes;
+    if (f.last) f.req->complete = true;
+    c->waves_done++;
+    c->w->waves_consumed.store(c->waves_done, std::memory_order_release);   // the set's landing windows are free again
+    c->flights.pop_front();
+  }
+  for (;;) {
+    ShmWave& wv = c->w->wave[c->waves_launched % FL_NET_MAX_REQUESTS];
+    if (wv.seq.load(std::memory_order_acquire) != c->waves_launched + 1) {   // nothing further has landed
+      if (c->cursor < c->active.size() && c->w->send_closed.load(std::memory_order_acquire)) {
+        FL_WARN("NET/FuseLink : the sending process closed the connection with a receive outstanding");
+        return ncclRemoteError;
+      }
+      break;
     }
-    if (wv.fifo_idx != r->fifo_idx) { FL_WARN("NET/FuseLink : a wave of request %llu arrived while %llu is first in line", (unsigned long long)wv.fifo_idx, (unsigned long long)r->fifo_idx); return ncclInternalError; }
-    if (wv.offset + wv.bytes > r->size) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
-    FL_HIPCHECK(hipSetDevice(c->hip_device));
+    if (c->cursor >= c->active.size()) { FL_WARN("NET/FuseLink : a wave arrived that no posted receive is waiting for"); return ncclInternalError; }
+    ShmRequest* r = c->active[c->cursor];
+    if (wv.fifo_idx != r->fifo_idx) {
+      FL_WARN("NET/FuseLink : a wave of request %llu arrived while %llu is next in line", (unsigned long long)wv.fifo_idx, (unsigned long long)r->fifo_idx);
+      return ncclInternalError;
+    }
+    if (wv.offset + wv.bytes > r->size || wv.set >= (uint32_t)c->sets) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
+    if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
     if (wv.bytes) {
       // the credit row this receiver put into the descriptor: the reassembly launch derives the same lanes and offsets
       flh_uniform_params u;
       fill_uniform(u, r->credits, wv.bytes, wv.offset, wv.epoch_bytes, FLH_TILE_BYTES);
-      FL_FLHCHECK(flh_reassemble_uniform(r->dst, r->size, &c->landing_wins, &u, c->d_status, c->stream));
+      FL_FLHCHECK(flh_reassemble_uniform(r->dst, r->size, &c->landing_wins[wv.set], &u, c->d_status, c->stream));
     }
-    FL_HIPCHECK(hipEventRecord(c->ev, c->stream));
-    r->wave_bytes = wv.bytes;
-    r->wave_no = wv.last;
-    r->phase = 1;
-    return ncclSuccess;
+    FL_HIPCHECK(hipEventRecord(c->ev[wv.set], c->stream));
+    ShmFlight f;
+    f.req = r;
+    f.fifo_idx = wv.fifo_idx;
+    f.epoch_bytes = wv.epoch_bytes;
+    f.offset = wv.offset;
+    f.bytes = wv.bytes;
+    f.last = wv.last;
+    f.set = wv.set;
+    c->flights.push_back(f);
+    c->waves_launched++;
+    if (wv.last) c->cursor++;   // the next wave belongs to the next receive
   }
-  hipError_t e = hipEventQuery(c->ev);
-  if (e == hipErrorNotReady) return ncclSuccess;
-  if (e != hipSuccess) return hip_fail("hipEventQuery", e);
-  if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its landing window or buffer (status %d)", *c->h_status); return ncclInternalError; }
-  r->received += r->wave_bytes;
-  c->waves_seen++;
-  c->w->waves_consumed.store(c->waves_seen, std::memory_order_release);   // the landing windows are free again
-  r->phase = r->wave_no ? 2 : 0;
   return ncclSuccess;
 }
 
@@ -1036,30 +1096,26 @@ ncclResult_t shm_test(ShmRequest* r, int* done, int* sizes) {
   *done = 0;
   ShmComm* c = r->comm;
   std::lock_guard<std::mutex> g(c->mu);
-  if (c->active.empty() || c->active.front() != r) {
-    // requests complete in order: the first in line is the one that moves
-    if (!c->active.empty()) {
-      ShmRequest* head = c->active.front();
-      ncclResult_t rc = head->type == kReqSend ? shm_progress_send(c, head) : shm_progress_recv(c, head);
-      if (rc != ncclSuccess) return rc;
-    }
-    return ncclSuccess;
-  }
-  ncclResult_t rc = r->type == kReqSend ? shm_progress_send(c, r) : shm_progress_recv(c, r);
+  ncclResult_t rc = c->is_send ? shm_progress_send(c) : shm_progress_recv(c);
   if (rc != ncclSuccess) return rc;
-  if (r->phase != 2) return ncclSuccess;
+  if (c->active.empty() || c->active.front() != r) return ncclSuccess;   // requests are reported in the order they were made
   if (r->type == kReqSend) {
     // the send is complete once its last wave has been taken out of the landing windows
-    if (c->w->waves_consumed.load(std::memory_order_acquire) < r->wave_no) {
-      if (c->w->recv_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding"); return ncclRemoteError; }
+    if (!r->all_launched || c->w->waves_consumed.load(std::memory_order_acquire) < r->last_wave) {
+      if (r->all_launched && c->w->recv_closed.load(std::memory_order_acquire)) {
+        FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding");
+        return ncclRemoteError;
+      }
       return ncclSuccess;
     }
   } else {
+    if (!r->complete) return ncclSuccess;
     c->r_finished++;
     c->r_inflight--;
     if (sizes) sizes[0] = (int)r->received;
   }
   c->active.pop_front();
+  if (c->cursor) c->cursor--;
   r->type = kReqUnused;
   *done = 1;
   return ncclSuccess;
@@ -1093,6 +1149,9 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
     const char* wv = getenv("NCCL_FUSELINK_WIRE");
     g_par.wire = wv && (!strcmp(wv, "shm") || !strcmp(wv, "1")) ? 1 : 0;
   }
+  g_par.wire_sets = (int)fl_param("FUSELINK_WIRE_SETS", g_par.wire_sets);
+  if (g_par.wire_sets < 1) g_par.wire_sets = 1;
+  if (g_par.wire_sets > kShmSetsMax) g_par.wire_sets = kShmSetsMax;
   g_par.engine = (int)fl_param("FUSELINK_ENGINE", g_par.engine);
   g_par.engine_units = (int)fl_param("FUSELINK_ENGINE_UNITS", g_par.engine_units);
   g_par.engine_idle_us = (int)fl_param("FUSELINK_ENGINE_IDLE_US", g_par.engine_idle_us);

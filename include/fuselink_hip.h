@@ -363,6 +363,10 @@ int flh_scatter_pages_uniform(void* d_pool, uint64_t pool_pages, const uint32_t*
 
 /* Plain device copy with the same inner loop as the striping kernels (roofline calibration). */
 int flh_copy(void* d_dst, const void* d_src, uint64_t bytes, void* stream);
+/* Up to FLH_MAX_LANES independent runs in one launch: run r moves bytes[r] from d_src[r] to d_dst[r] (empty runs are
+ * skipped).  It carries the staged bytes of every lane from a sender's windows into a receiver's, the part a NIC
+ * per lane plays in the reference (one RDMA write per lane comm, src/plugin.cc:1453-1495). */
+int flh_copy_runs(void* const* d_dst, const void* const* d_src, const uint64_t* bytes, uint32_t n, void* stream);
 
 /* ---- R2: request -> QP pieces (src/plugin.cc:1467-1495), host arithmetic ------------------------ */
 int flh_qp_split(int size, int nqps, int* off, int* len);

@@ -1166,3 +1166,32 @@ def test_copies_with_tiles_taken_in_runs_per_xcd(fl, seed, xcd_runs):
         assert torch.equal(back, big)
     finally:
         core.tune("xcd_runs", 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(6))
+def test_runs_of_several_lanes_in_one_launch(fl, seed):
+    """flh_copy_runs: what carries every lane's staged bytes from one set of windows to another in a single launch.
+    Runs of any length (none, a few bytes, ragged, megabytes), misaligned against each other, in any of the 16 slots;
+    every destination is compared with numpy, and the bytes around every run must stay untouched."""
+    core, torch = fl
+    rng = np.random.default_rng(6100 + seed)
+    n = int(rng.integers(1, 17))
+    lens = [int(rng.choice([0, 0, int(rng.integers(1, 100)), int(rng.integers(1, 200000)), int(rng.integers(1, 5)) * (1 << 20) + int(rng.integers(0, 3)) * 7]))
+            for _ in range(n)]
+    if seed == 0:
+        lens = [0] * n            # nothing at all: no launch, no error
+    pad = 64
+    srcs_np = [rng.integers(1, 256, size=ln + 2 * pad, dtype=np.uint8) for ln in lens]
+    so = [int(rng.integers(0, pad)) for _ in lens]
+    do = [int(rng.integers(0, pad)) for _ in lens]
+    srcs = [torch.from_numpy(a).cuda() for a in srcs_np]
+    dsts = [torch.zeros(ln + 2 * pad, dtype=torch.uint8, device="cuda") for ln in lens]
+    core.copy_runs([d[o:] if ln else None for d, o, ln in zip(dsts, do, lens)], [s[o:] if ln else None for s, o, ln in zip(srcs, so, lens)], lens)
+    torch.cuda.synchronize()
+    for k, ln in enumerate(lens):
+        exp = np.zeros(ln + 2 * pad, dtype=np.uint8)
+        exp[do[k]:do[k] + ln] = srcs_np[k][so[k]:so[k] + ln]
+        np.testing.assert_array_equal(dsts[k].cpu().numpy(), exp, err_msg=f"run {k} of {lens}")
+    with pytest.raises(Exception):
+        core.copy_runs([dsts[0]] * 17, [srcs[0]] * 17, [1] * 17)

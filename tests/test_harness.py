@@ -140,10 +140,22 @@ def test_two_processes_cfg2_shape():
 
 
 @pytest.mark.gpu
-def test_two_processes_requests_larger_than_the_windows_and_a_ragged_tail():
-    # every request takes several waves through the landing windows (4 units per lane), the last request is short and odd
+@pytest.mark.parametrize("sets", [1, 2, 5])
+def test_two_processes_requests_larger_than_the_windows_and_a_ragged_tail(sets):
+    # every request takes several waves through the landing windows (4 units per lane; `sets` sets of them, so that many
+    # waves are on the wire at once), the last request is short and odd
     out = _run(["--two-process", "--bytes", str((96 << 20) + 12345), "--request", str(32 << 20), "--inflight", "2", "--iters", "2"],
                env={"NCCL_FUSELINK_LANES": "4", "NCCL_FUSELINK_CHUNKSIZE": str(128 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "4",
-                    "NCCL_FUSELINK_CREDITS": "3,1,2,2"})
+                    "NCCL_FUSELINK_CREDITS": "3,1,2,2", "NCCL_FUSELINK_WIRE_SETS": str(sets)})
     assert out["bit_exact"] and out["requests"] == 4
+    print(out)
+
+
+@pytest.mark.gpu
+def test_two_processes_many_small_requests_in_flight():
+    # NCCL's request shape across the process boundary: 512 KiB requests, 8 in flight, more requests than the descriptor
+    # ring and the wave ring have slots (both wrap)
+    out = _run(["--two-process", "--bytes", str(192 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "2"],
+               env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10), "NCCL_FUSELINK_WIRE_SETS": "4"})
+    assert out["bit_exact"] and out["requests"] == 384
     print(out)
