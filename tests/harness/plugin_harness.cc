@@ -9,7 +9,8 @@
 // the child listens and sends the 128-byte handle to the parent over a socket pair (NCCL's bootstrap does that between
 // ranks), the parent connects with it, and from then on the two processes share nothing but what the plugin itself set up
 // behind the handle (NCCL_FUSELINK_WIRE=shm is set for both).  The child checks what it received and reports through its
-// exit status.
+// exit status.  With --handoff as well, the five messages of the hand-off group cross the process boundary, each a
+// buffer and a registration of its own on either side.
 // With --connections C, C connections run concurrently, each with its own pair of proxy threads and buffers; every
 // iteration starts on all of them together and is timed from the first start to the last finish, and the received
 // buffers are compared only once all connections have finished it.
@@ -217,7 +218,17 @@ struct Deadline {
   }
 };
 
-static int receiver_process(const char* path, int sock, size_t bytes, size_t request, int inflight, int iters) {
+// the requests of a group of messages, in order: message, offset in it, length
+struct WirePiece { int msg; size_t off; int len; };
+static std::vector<WirePiece> wire_pieces(const std::vector<size_t>& sizes, size_t request) {
+  std::vector<WirePiece> pieces;
+  for (size_t m = 0; m < sizes.size(); ++m)
+    for (size_t off = 0; off < sizes[m]; off += request)
+      pieces.push_back({(int)m, off, (int)(sizes[m] - off < request ? sizes[m] - off : request)});
+  return pieces;
+}
+
+static int receiver_process(const char* path, int sock, const std::vector<size_t>& sizes, size_t request, int inflight, int iters) {
   ncclNet_v8_t* net = open_plugin(path);
   char handle[NCCL_NET_HANDLE_MAXSIZE];
   void *lcomm = nullptr, *rcomm = nullptr;
@@ -225,12 +236,19 @@ static int receiver_process(const char* path, int sock, size_t bytes, size_t req
   sock_write(sock, handle, sizeof(handle));
   for (Deadline d; !rcomm; d.check("accept")) { CHECK(net->accept(lcomm, &rcomm, nullptr)); if (!rcomm) usleep(100); }
   HIP(hipSetDevice(0));
-  uint8_t* dst = nullptr;
-  void* mh = nullptr;
-  HIP(hipMalloc((void**)&dst, bytes));
-  HIP(hipMemset(dst, 0, bytes));
-  CHECK(net->regMr(rcomm, dst, bytes, NCCL_PTR_CUDA, &mh));
-  const size_t n_req = (bytes + request - 1) / request;
+  size_t bytes = 0;
+  std::vector<uint8_t*> dst(sizes.size(), nullptr);
+  std::vector<void*> mh(sizes.size(), nullptr);
+  std::vector<size_t> base(sizes.size(), 0);
+  for (size_t m = 0; m < sizes.size(); ++m) {   // every message is a buffer and a registration of its own
+    base[m] = bytes;
+    bytes += sizes[m];
+    HIP(hipMalloc((void**)&dst[m], sizes[m]));
+    HIP(hipMemset(dst[m], 0, sizes[m]));
+    CHECK(net->regMr(rcomm, dst[m], sizes[m], NCCL_PTR_CUDA, &mh[m]));
+  }
+  const std::vector<WirePiece> pieces = wire_pieces(sizes, request);
+  const size_t n_req = pieces.size();
   std::vector<uint8_t> pattern(bytes), back(bytes);
   for (int it = 0; it < iters; ++it) {
     char go = 0;
@@ -240,61 +258,70 @@ static int receiver_process(const char* path, int sock, size_t bytes, size_t req
     Deadline d;
     while (finished < n_req) {
       if (next < n_req && (int)q.size() < inflight) {
-        void* p = dst + next * request;
-        int sz = (int)(bytes - next * request < request ? bytes - next * request : request), tag = (int)next;
+        const WirePiece& pc = pieces[next];
+        void* p = dst[pc.msg] + pc.off;
+        int sz = pc.len, tag = (int)next;
         void* req = nullptr;
-        CHECK(net->irecv(rcomm, 1, &p, &sz, &tag, &mh, &req));
+        CHECK(net->irecv(rcomm, 1, &p, &sz, &tag, &mh[pc.msg], &req));
         if (req) { q.push_back(req); ++next; }
       }
       if (!q.empty()) {
         int done = 0, got = -1;
         CHECK(net->test(q.front(), &done, &got));
         if (done) {
-          const size_t want = bytes - finished * request < request ? bytes - finished * request : request;
-          if ((size_t)got != want) { fprintf(stderr, "receive %zu reported %d bytes, expected %zu\n", finished, got, want); return 4; }
+          if (got != pieces[finished].len) { fprintf(stderr, "receive %zu reported %d bytes, expected %d\n", finished, got, pieces[finished].len); return 4; }
           q.pop_front(); ++finished;
         }
       }
       d.check("receives");
     }
     fill_pattern(pattern, it);
-    HIP(hipMemcpy(back.data(), dst, bytes, hipMemcpyDeviceToHost));
-    if (memcmp(back.data(), pattern.data(), bytes) != 0) {
-      size_t at = 0;
-      while (at < bytes && back[at] == pattern[at]) ++at;
-      fprintf(stderr, "iteration %d: the received buffer differs from what was sent, first at byte %zu\n", it, at);
-      return 5;
+    for (size_t m = 0; m < sizes.size(); ++m) {
+      HIP(hipMemcpy(back.data() + base[m], dst[m], sizes[m], hipMemcpyDeviceToHost));
+      if (memcmp(back.data() + base[m], pattern.data() + base[m], sizes[m]) != 0) {
+        size_t at = 0;
+        while (at < sizes[m] && back[base[m] + at] == pattern[base[m] + at]) ++at;
+        fprintf(stderr, "iteration %d, message %zu: the received buffer differs from what was sent, first at byte %zu\n", it, m, at);
+        return 5;
+      }
+      HIP(hipMemset(dst[m], 0, sizes[m]));
     }
-    HIP(hipMemset(dst, 0, bytes));
     char ok = 1;
     sock_write(sock, &ok, 1);
   }
   char bye = 0;
   sock_read(sock, &bye, 1, kDeadline);   // the sender has closed its comm: the landing windows may go
-  CHECK(net->deregMr(rcomm, mh));
+  for (size_t m = 0; m < sizes.size(); ++m) CHECK(net->deregMr(rcomm, mh[m]));
   CHECK(net->closeRecv(rcomm));
   CHECK(net->closeListen(lcomm));
-  HIP(hipFree(dst));
+  for (uint8_t* p : dst) HIP(hipFree(p));
   return 0;
 }
 
-static int sender_process(const char* path, int sock, pid_t child, size_t bytes, size_t request, int inflight, int iters) {
+static int sender_process(const char* path, int sock, pid_t child, const std::vector<size_t>& sizes, size_t request, int inflight, int iters, int handoff) {
   ncclNet_v8_t* net = open_plugin(path);
   char handle[NCCL_NET_HANDLE_MAXSIZE];
   sock_read(sock, handle, sizeof(handle), kDeadline);
   void* scomm = nullptr;
   for (Deadline d; !scomm; d.check("connect")) { CHECK(net->connect(1, handle, &scomm, nullptr)); if (!scomm) usleep(100); }
   HIP(hipSetDevice(0));
-  uint8_t* src = nullptr;
-  void* mh = nullptr;
-  HIP(hipMalloc((void**)&src, bytes));
-  CHECK(net->regMr(scomm, src, bytes, NCCL_PTR_CUDA, &mh));
-  const size_t n_req = (bytes + request - 1) / request;
+  size_t bytes = 0;
+  std::vector<uint8_t*> src(sizes.size(), nullptr);
+  std::vector<void*> mh(sizes.size(), nullptr);
+  std::vector<size_t> base(sizes.size(), 0);
+  for (size_t m = 0; m < sizes.size(); ++m) {
+    base[m] = bytes;
+    bytes += sizes[m];
+    HIP(hipMalloc((void**)&src[m], sizes[m]));
+    CHECK(net->regMr(scomm, src[m], sizes[m], NCCL_PTR_CUDA, &mh[m]));
+  }
+  const std::vector<WirePiece> pieces = wire_pieces(sizes, request);
+  const size_t n_req = pieces.size();
   std::vector<uint8_t> pattern(bytes);
   double best = 1e30, total = 0;
   for (int it = 0; it < iters; ++it) {
     fill_pattern(pattern, it);
-    HIP(hipMemcpy(src, pattern.data(), bytes, hipMemcpyHostToDevice));
+    for (size_t m = 0; m < sizes.size(); ++m) HIP(hipMemcpy(src[m], pattern.data() + base[m], sizes[m], hipMemcpyHostToDevice));
     char go = 1;
     const auto t0 = std::chrono::steady_clock::now();
     sock_write(sock, &go, 1);
@@ -303,9 +330,9 @@ static int sender_process(const char* path, int sock, pid_t child, size_t bytes,
     Deadline d;
     while (finished < n_req) {
       if (next < n_req && (int)q.size() < inflight) {
-        const int sz = (int)(bytes - next * request < request ? bytes - next * request : request);
+        const WirePiece& pc = pieces[next];
         void* req = nullptr;
-        CHECK(net->isend(scomm, src + next * request, sz, (int)next, mh, &req));   // no request: the receive is not posted yet
+        CHECK(net->isend(scomm, src[pc.msg] + pc.off, pc.len, (int)next, mh[pc.msg], &req));   // no request: the receive is not posted yet
         if (req) { q.push_back(req); ++next; }
       }
       if (!q.empty()) {
@@ -319,24 +346,24 @@ static int sender_process(const char* path, int sock, pid_t child, size_t bytes,
     if (sec < best) best = sec;
     total += sec / iters;
     char ok = 0;
-    sock_read(sock, &ok, 1, kDeadline);   // the receiver has compared the buffer
+    sock_read(sock, &ok, 1, kDeadline);   // the receiver has compared the buffers
   }
-  CHECK(net->deregMr(scomm, mh));
+  for (size_t m = 0; m < sizes.size(); ++m) CHECK(net->deregMr(scomm, mh[m]));
   CHECK(net->closeSend(scomm));
-  HIP(hipFree(src));
+  for (uint8_t* p : src) HIP(hipFree(p));
   char bye = 1;
   sock_write(sock, &bye, 1);
   int status = 0;
   Deadline d;
   while (waitpid(child, &status, WNOHANG) == 0) { usleep(1000); d.check("the receiver's exit"); }
   if (!WIFEXITED(status) || WEXITSTATUS(status) != 0) { fprintf(stderr, "the receiver process failed (status 0x%x)\n", status); return 5; }
-  printf("{\"harness\": \"plugin_two_process\", \"name\": \"%s\", \"memory\": \"device\", \"bytes\": %zu, \"request_bytes\": %zu, \"requests\": %zu, "
+  printf("{\"harness\": \"plugin_two_process\", \"name\": \"%s\", \"memory\": \"device\", \"group\": \"%s\", \"messages\": %zu, \"bytes\": %zu, \"request_bytes\": %zu, \"requests\": %zu, "
          "\"inflight\": %d, \"iters\": %d, \"best_s\": %.9f, \"mean_s\": %.9f, \"GBps_payload_best\": %.1f, \"bit_exact\": true}\n",
-         net->name, bytes, request, n_req, inflight, iters, best, total, (double)bytes / best / 1e9);
+         net->name, handoff ? "kv_handoff" : "one message", sizes.size(), bytes, request, n_req, inflight, iters, best, total, (double)bytes / best / 1e9);
   return 0;
 }
 
-static int run_two_processes(const char* path, size_t bytes, size_t request, int inflight, int iters) {
+static int run_two_processes(const char* path, const std::vector<size_t>& sizes, size_t request, int inflight, int iters, int handoff) {
   setenv("NCCL_FUSELINK_WIRE", "shm", 1);
   int sv[2];
   if (socketpair(AF_UNIX, SOCK_STREAM, 0, sv) != 0) { perror("socketpair"); return 1; }
@@ -346,13 +373,13 @@ static int run_two_processes(const char* path, size_t bytes, size_t request, int
   if (child < 0) { perror("fork"); return 1; }
   if (child == 0) {
     close(sv[0]);
-    const int rc = receiver_process(path, sv[1], bytes, request, inflight, iters);
+    const int rc = receiver_process(path, sv[1], sizes, request, inflight, iters);
     fflush(stderr);
     _exit(rc);
   }
   close(sv[1]);
   signal(SIGPIPE, SIG_IGN);
-  return sender_process(path, sv[0], child, bytes, request, inflight, iters);
+  return sender_process(path, sv[0], child, sizes, request, inflight, iters, handoff);
 }
 
 int main(int argc, char** argv) {
@@ -389,8 +416,8 @@ int main(int argc, char** argv) {
   if (request > 0x7fffffffull) request = 0x40000000ull;  // isend takes an int size (src/extern/nccl_net.h:74)
 
   if (two_process) {
-    if (host || handoff || connections != 1) { fprintf(stderr, "--two-process runs one connection with device memory\n"); return 1; }
-    return run_two_processes(argv[1], bytes, request, inflight, iters);
+    if (host || connections != 1) { fprintf(stderr, "--two-process runs one connection with device memory\n"); return 1; }
+    return run_two_processes(argv[1], sizes, request, inflight, iters, handoff);
   }
 
   void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);

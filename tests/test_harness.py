@@ -159,3 +159,15 @@ def test_two_processes_many_small_requests_in_flight():
                env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10), "NCCL_FUSELINK_WIRE_SETS": "4"})
     assert out["bit_exact"] and out["requests"] == 384
     print(out)
+
+
+@pytest.mark.gpu
+def test_two_processes_kv_handoff_group():
+    # the prefill -> decode hand-off of the serving experiment (experiments/serving/model.hh:286-309), where the two are
+    # different processes: five messages (int64 context output, K cache, V cache, int64 block table, int64 counts), each
+    # a buffer and a registration of its own on either side, tiny and large mixed, cut into 512 KiB requests
+    out = _run(["--two-process", "--handoff", "4,8,2,8,16,128", "--request", str(512 << 10), "--inflight", "8", "--iters", "2"])
+    cache = 2 * 32 * 2 * 8 * 16 * 128
+    assert out["bit_exact"] and out["group"] == "kv_handoff" and out["messages"] == 5
+    assert out["bytes"] == 2 * cache + 8 * 4 + 8 * 32 + 8 * 4 and out["requests"] == 1 + 4 + 4 + 1 + 1
+    print(out)
