@@ -972,9 +972,13 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     if (tid == 0) {
       // leaving the batch releases this worker's stores; the last one to leave has thereby acquired everybody's and
       // publishes the batch to the host
-      const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_SYSTEM);
-      if ((((uint32_t)before + 1) & kEngineCountMask) == own_target)
+      const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      if ((((uint32_t)before + 1) & kEngineCountMask) == own_target) {
+        // only the last one to leave has to have seen the others' releases: a fence behind the read of the count that
+        // they all incremented with release, instead of an acquire (a cache invalidate) in every worker's increment
+        __atomic_thread_fence(__ATOMIC_ACQUIRE);
         __hip_atomic_store(&e.hctl->done[k % kEngineDevRing], k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
     }
   }
 }
