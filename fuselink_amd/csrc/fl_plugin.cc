@@ -1798,6 +1798,7 @@ static void last_buffers(const Peer* pr, const flh_chunk_desc** table, const flh
 
 int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_out) {
   Comm* c = (Comm*)sendComm;
+  if (c && c->magic == kShmCommMagic && c->is_send) return shm_last_table((ShmComm*)sendComm, rows_out, max_rows, hdr_out);
   if (!c || c->magic != kCommMagic || !c->is_send) return fl_set_error(FLH_E_ARG, "not a send comm");
   Link* lk = c->link;
   Peer* pr = lk->peer.load(std::memory_order_acquire);

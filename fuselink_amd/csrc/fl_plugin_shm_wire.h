@@ -94,6 +94,7 @@ struct ShmComm {
   uint64_t waves_launched = 0;               // sender: waves queued on the GPU so far; receiver: waves taken off the wire so far
   uint64_t waves_published = 0;              // sender: waves announced to the receiver
   uint64_t waves_done = 0;                   // receiver: waves reassembled (what waves_consumed says)
+  uint32_t last_rows = 0;                    // sender: chunks of the latest wave (rows of d_table)
   int64_t r_finished = 0, r_inflight = 0;
   int fuselink_offset = -1;
   uint8_t credits[FL_NET_MAX_LANES] = {};
@@ -421,6 +422,7 @@ ncclResult_t shm_progress_send(ShmComm* c) {
       flh_uniform_params u;
       fill_uniform(u, r->credits, wave, r->launched, c->epoch_bytes, FLH_TILE_BYTES);
       FL_FLHCHECK(flh_stripe_uniform(r->src, r->size, &c->wins, &u, c->d_table, c->d_hdr, c->d_status, c->stream));
+      c->last_rows = (uint32_t)((wave + chunk - 1) / chunk);
       // the wire: every lane's staged bytes into the receiver's landing window of that lane, one launch for all lanes
       FlCreditRow row;
       fl_row_make(r->credits, (uint32_t)g_par.lanes, row);
@@ -501,6 +503,21 @@ ncclResult_t shm_progress_recv(ShmComm* c) {
     if (wv.last) c->cursor++;   // the next wave belongs to the next receive
   }
   return ncclSuccess;
+}
+
+// The table and header that the striping launch of the connection's latest wave wrote (control surface, for tests).
+int shm_last_table(ShmComm* c, void* rows_out, int max_rows, void* hdr_out) {
+  std::lock_guard<std::mutex> g(c->mu);
+  if (!c->gpu_ready || c->last_rows == 0) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
+  DeviceScope keep;
+  if (hipSetDevice(c->hip_device) != hipSuccess) return fl_set_error(FLH_E_HIP, "hipSetDevice failed");
+  if (hipStreamSynchronize(c->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
+  const int rows = (int)c->last_rows, take = rows < max_rows ? rows : max_rows;
+  if (take > 0 && rows_out && hipMemcpy(rows_out, c->d_table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
+    return fl_set_error(FLH_E_HIP, "table copy failed");
+  if (hdr_out && hipMemcpy(hdr_out, c->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
+    return fl_set_error(FLH_E_HIP, "header copy failed");
+  return rows;
 }
 
 ncclResult_t shm_test(ShmRequest* r, int* done, int* sizes) {
