@@ -195,6 +195,13 @@ ncclResult_t shm_connect(int dev, void* opaqueHandle, void** sendComm) {
       shm_comm_free(c);
       return ncclInvalidUsage;
     }
+    int listener_pid = -1;
+    if (sscanf(name, "/fuselink-wire-%d-", &listener_pid) == 1 && listener_pid == (int)getpid()) {
+      // the landing windows reach the sender through HIP IPC, which a process cannot open on its own allocations
+      FL_WARN("NET/FuseLink : NCCL_FUSELINK_WIRE=shm connects two processes; this listener lives in the connecting process (unset it for the in-process wire)");
+      shm_comm_free(c);
+      return ncclInvalidUsage;
+    }
     c->is_send = 1;
     c->dev = dev;
     memcpy(c->name, name, sizeof(name));

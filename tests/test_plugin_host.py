@@ -385,3 +385,19 @@ def test_a_listener_that_never_accepts_leaves_no_shared_memory_behind():
         assert rc == P.ncclSystemError and not scomm
     finally:
         p.reconfigure(NCCL_FUSELINK_WIRE=old)
+
+
+def test_the_shared_memory_wire_refuses_a_listener_in_the_connecting_process():
+    p = P.NetPlugin(8)
+    old = os.environ.get("NCCL_FUSELINK_WIRE")
+    p.reconfigure(NCCL_FUSELINK_WIRE="shm")
+    try:
+        rc, handle, lcomm = p.listen(0)
+        assert rc == P.ncclSuccess
+        rc, scomm = p.connect(0, handle)
+        assert rc == P.ncclInvalidUsage and not scomm
+        rc, rcomm = p.accept(lcomm)
+        assert rc == P.ncclSuccess and not rcomm       # nobody connected
+        assert p.closeListen(lcomm) == P.ncclSuccess
+    finally:
+        p.reconfigure(NCCL_FUSELINK_WIRE=old)
