@@ -32,7 +32,7 @@ def _wait(lib, eng, seq, seconds=10.0):
         assert time.time() < deadline, f"batch {seq} did not complete (completed {lib.flh_engine_completed(eng)})"
 
 
-@pytest.mark.parametrize("sets", [1, 3])
+@pytest.mark.parametrize("sets", [1, 2, 3, 8])
 def test_engine_batches_equal_the_oracle_and_the_engine_restarts_after_idling(fl, sets):
     core, torch, _lib = fl
     lib = _lib.load()
