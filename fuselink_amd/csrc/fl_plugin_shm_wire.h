@@ -138,18 +138,20 @@ void shm_comm_free(ShmComm* c) {
   if (c->w) munmap(c->w, sizeof(ShmWire));
   if (c->owner && c->name[0]) shm_unlink(c->name);
   delete c;
+  g_live_links.fetch_sub(1);   // (a reset of the plugin waits for these as for the in-process connections)
 }
 
 ncclResult_t shm_listen(int dev, void* opaqueHandle, void** listenComm) {
   ShmListen* lc = new (std::nothrow) ShmListen();
   ShmComm* c = new (std::nothrow) ShmComm();
   if (!lc || !c) { delete lc; delete c; return ncclSystemError; }
+  g_live_links.fetch_add(1);
   snprintf(c->name, sizeof(c->name), "/fuselink-wire-%d-%llu", (int)getpid(), (unsigned long long)g_shm_counter.fetch_add(1));
   int fd = shm_open(c->name, O_CREAT | O_EXCL | O_RDWR, 0600);
-  if (fd < 0 || ftruncate(fd, sizeof(ShmWire)) != 0) { if (fd >= 0) close(fd); FL_WARN("NET/FuseLink : shm_open(%s) failed", c->name); delete lc; delete c; return ncclSystemError; }
+  if (fd < 0 || ftruncate(fd, sizeof(ShmWire)) != 0) { if (fd >= 0) close(fd); FL_WARN("NET/FuseLink : shm_open(%s) failed", c->name); delete lc; delete c; g_live_links.fetch_sub(1); return ncclSystemError; }
   void* p = mmap(nullptr, sizeof(ShmWire), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
   close(fd);
-  if (p == MAP_FAILED) { shm_unlink(c->name); delete lc; delete c; return ncclSystemError; }
+  if (p == MAP_FAILED) { shm_unlink(c->name); delete lc; delete c; g_live_links.fetch_sub(1); return ncclSystemError; }
   memset(p, 0, sizeof(ShmWire));
   c->w = (ShmWire*)p;
   c->owner = true;
@@ -189,6 +191,7 @@ ncclResult_t shm_connect(int dev, void* opaqueHandle, void** sendComm) {
     if (p == MAP_FAILED) return ncclSystemError;
     c = new (std::nothrow) ShmComm();
     if (!c) { munmap(p, sizeof(ShmWire)); return ncclSystemError; }
+    g_live_links.fetch_add(1);
     c->w = (ShmWire*)p;
     if (c->w->magic != kHandleMagicShm || (int)c->w->lanes != g_par.lanes) {
       FL_WARN("NET/FuseLink : connect: the listener runs %u lanes, this side %d", c->w->lanes, g_par.lanes);

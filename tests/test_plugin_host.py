@@ -378,8 +378,10 @@ def test_a_listener_that_never_accepts_leaves_no_shared_memory_behind():
         assert rc == P.ncclSuccess
         name = handle.raw[40:104].split(b"\0")[0].decode()
         assert os.path.exists("/dev/shm" + name)
+        assert p.lib.fl_net_reset() != 0               # an open listener of this wire holds off a reset too
         assert p.closeListen(lcomm) == P.ncclSuccess
         assert not os.path.exists("/dev/shm" + name)
+        assert p.lib.fl_net_reset() == 0 and p.init() == P.ncclSuccess
         # a connect with the stale handle fails cleanly
         rc, scomm = p.connect(0, handle)
         assert rc == P.ncclSystemError and not scomm
