@@ -153,6 +153,9 @@ int64_t flh_constant(int which);
  * tiles (1 MiB) instead of every eighth tile (1, the default; 3-5 % faster copies).
  * "engine_wait_us" = limit of every wait inside a lane engine created afterwards (2 000 000; tests of the failure
  * path ask for a microsecond).
+ * "engine_inject_fault" = 1: a lane engine that is started (or started again after idling) while this is set reports
+ * a wait that ran out in place of executing its first batch and goes down, every workgroup leaving as after a real
+ * one (0; for tests of the failure path, which cannot count on a healthy GPU to miss a limit).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL.
  * The tunables are process-wide and read by every launch: set them while no other thread launches. */
 int flh_tune(const char* key, int64_t value);

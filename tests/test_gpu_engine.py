@@ -120,6 +120,70 @@ def test_engine_batches_equal_the_oracle_and_the_engine_restarts_after_idling(fl
         _lib.check(lib.flh_engine_destroy(eng))
 
 
+def test_buffers_that_are_used_again_deliver_their_latest_contents(fl):
+    """The workers stay resident, so no kernel boundary brings their view of memory up to date or makes their stores
+    visible: they must read what a kernel on another stream has just written into a source they have read before, and a
+    kernel that starts once a batch is complete must read what they delivered.  The same sources, windows and
+    destinations carry new contents in each of 48 batches (sizes that end in odd bytes among them, so the byte edges
+    and the shifted copy take part); every destination is compared on the GPU, by a kernel, not through a DMA copy.
+    Half-way the batches go two at a time, alternating between two sets of buffers."""
+    core, torch, _lib = fl
+    lib = _lib.load()
+    lanes, chunk, sets = 8, 64 << 10, 2
+    sizes = [512 << 10, (512 << 10) - 7, 100_003, 64 << 10, 33]
+    eng = C.c_void_p()
+    _lib.check(lib.flh_engine_create(0, 0, 200, sets, C.byref(eng)))
+    try:
+        cap = 2 << 20
+        wins = [[torch.zeros(cap, dtype=torch.uint8, device="cuda") for _ in range(lanes)] for _ in range(sets)]
+        W = [core.make_windows([t.data_ptr() for t in ws], [cap] * lanes) for ws in wins]
+        status = core.new_status()
+        bufs = []
+        for _ in range(sets):
+            srcs = [torch.zeros(n, dtype=torch.uint8, device="cuda") for n in sizes]
+            dsts = [torch.zeros(n + 64, dtype=torch.uint8, device="cuda") for n in sizes]
+            # only a segment's last request may end inside a chunk: three segments, each with a credit row of its own
+            segments = [(2, [3, 1, 2, 1, 1, 2, 1, 1], 0), (1, [1, 1, 1, 1, 0, 0, 2, 2], 3 * chunk), (2, [1] * lanes, 0)]
+            bufs.append((srcs, dsts, core.batch_params(srcs, dsts, chunk, [1] * lanes, segments=segments)))
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(4711)
+        seq = C.c_uint64()
+
+        def refill(which):
+            for t in bufs[which][0]:
+                t.copy_(torch.randint(0, 256, t.shape, dtype=torch.uint8, device="cuda", generator=gen))
+            for t in bufs[which][1]:
+                t.fill_(0xEE)
+
+        def submit(which):
+            _lib.check(lib.flh_engine_submit(eng, C.byref(bufs[which][2]), C.byref(W[which]), None, None, status.data_ptr(), C.byref(seq), None))
+            return seq.value
+
+        def check(which, k):
+            for i, n in enumerate(sizes):
+                src, dst = bufs[which][0][i], bufs[which][1][i]
+                assert bool(torch.equal(dst[:n], src)), f"batch {k}, request {i}: stale or missing bytes"
+                assert bool((dst[n:] == 0xEE).all()), f"batch {k}, request {i}: bytes past the end"
+
+        for k in range(24):                 # one at a time, the same buffers every time
+            refill(0)
+            torch.cuda.synchronize()        # the contract of a submit: what it reads has been written
+            _wait(lib, eng, submit(0))
+            check(0, k)
+        for k in range(24, 48, 2):          # two in flight
+            refill(0)
+            refill(1)
+            torch.cuda.synchronize()
+            submit(0)
+            _wait(lib, eng, submit(1))
+            check(0, k)
+            check(1, k + 1)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0 and lib.flh_engine_error(eng) == 0
+    finally:
+        _lib.check(lib.flh_engine_destroy(eng))
+
+
 def test_engine_refuses_bad_arguments_on_the_host(fl):
     core, torch, _lib = fl
     lib = _lib.load()

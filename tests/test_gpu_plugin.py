@@ -924,49 +924,54 @@ def test_random_traffic_of_several_connections_arrives_intact(net, seed):
 
 
 def test_an_engine_that_goes_down_fails_its_requests_and_traffic_falls_back_to_launches(net):
-    """The lane engine's waits are bounded; with the bound at a microsecond and one window set its second batch in a row
-    cannot get the windows in time, the engine reports the failure and goes down.  The requests it held complete with
-    ncclRemoteError (as a queue pair in the error state completes its work requests, src/plugin.cc:1839-1861), nothing
-    hangs, and a connection opened afterwards moves its bytes through launch pairs."""
+    """The lane engine's waits are bounded; when one runs out the engine reports it and goes down.  A healthy GPU misses no
+    two-second limit, so the condition is forced from the host: an engine started while flh_tune("engine_inject_fault")
+    is set reports the failure in place of executing its first batch, and every workgroup leaves.  The requests the
+    engine held complete with ncclRemoteError (as a queue pair in the error state completes its work requests,
+    src/plugin.cc:1839-1861), nothing hangs, later requests of the connection and a connection opened afterwards move
+    their bytes through launch pairs."""
+    import ctypes as C
     import time
     import torch
     piece = 512 << 10
-    net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=256 << 10, NCCL_FUSELINK_BATCH=8, NCCL_FUSELINK_ENGINE=1, NCCL_FUSELINK_ENGINE_SETS=1,
+    net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=256 << 10, NCCL_FUSELINK_BATCH=8, NCCL_FUSELINK_ENGINE=1,
                     NCCL_FUSELINK_REFRESH_BATCH=1000)
-    net.lib.flh_tune.argtypes = [__import__("ctypes").c_char_p, __import__("ctypes").c_int64]
-    assert net.lib.flh_tune(b"engine_wait_us", 1) == 0
-    try:
-        rng = np.random.default_rng(77)
-        n = 32
-        src_np = rng.integers(1, 256, size=(n + 1) * piece, dtype=np.uint8)
-        c = _open(net, 0, torch.from_numpy(src_np).cuda(), torch.zeros((n + 1) * piece, dtype=torch.uint8, device="cuda"))   # creates the GPU's engine
-    finally:
-        assert net.lib.flh_tune(b"engine_wait_us", 2000000) == 0
-    # one request on its own passes (a first batch waits for nothing) and takes the connection off its refresh boundary
+    net.lib.flh_tune.argtypes = [C.c_char_p, C.c_int64]
+    rng = np.random.default_rng(77)
+    n = 32
+    src_np = rng.integers(1, 256, size=(n + 1) * piece, dtype=np.uint8)
+    c = _open(net, 0, torch.from_numpy(src_np).cuda(), torch.zeros((n + 1) * piece, dtype=torch.uint8, device="cuda"))
+    # one request on its own passes through the engine and takes the connection off its refresh boundary
     _send_recv(net, c["s"], c["r"], c["src"], c["dst"], piece, 99, c["smh"], c["rmh"], src_off=n * piece, dst_off=n * piece)
-    reqs = []
-    for q in range(n):
-        rc, rreq = net.irecv(c["r"], [c["dst"].data_ptr() + q * piece], [piece], [q], [c["rmh"]])
-        assert rc == 0 and rreq
-        reqs.append(rreq)
-    for q in range(n):   # every eighth send fills a batch, which goes out inside that isend: four batches in a row
-        rc, sreq = net.isend(c["s"], c["src"].data_ptr() + q * piece, piece, q, c["smh"])
-        assert rc == 0 and sreq
-        reqs.append(sreq)
-    failed = finished = 0
-    deadline = time.time() + 20
-    pending = list(reqs)
-    while pending:
-        assert time.time() < deadline, "requests neither completed nor failed"
-        rc, done, _ = net.test(pending[0])
-        if rc != 0:
-            assert rc == P.ncclRemoteError
-            failed += 1
-            pending.pop(0)
-        elif done:
-            finished += 1
-            pending.pop(0)
-    assert failed >= 2 and finished + failed == 2 * n     # at least the second batch's requests
+    time.sleep(0.05)         # far beyond the engine's idle limit: it has gone down, the next batch starts it again
+    assert net.lib.flh_tune(b"engine_inject_fault", 1) == 0
+    try:
+        reqs = []
+        for q in range(n):
+            rc, rreq = net.irecv(c["r"], [c["dst"].data_ptr() + q * piece], [piece], [q], [c["rmh"]])
+            assert rc == 0 and rreq
+            reqs.append(rreq)
+        for q in range(n):   # every eighth send fills a batch, which goes out inside that isend
+            rc, sreq = net.isend(c["s"], c["src"].data_ptr() + q * piece, piece, q, c["smh"])
+            assert rc == 0 and sreq
+            reqs.append(sreq)
+        failed = finished = 0
+        deadline = time.time() + 20
+        pending = list(reqs)
+        while pending:
+            assert time.time() < deadline, "requests neither completed nor failed"
+            rc, done, _ = net.test(pending[0])
+            if rc != 0:
+                assert rc == P.ncclRemoteError
+                failed += 1
+                pending.pop(0)
+            elif done:
+                finished += 1
+                pending.pop(0)
+    finally:
+        assert net.lib.flh_tune(b"engine_inject_fault", 0) == 0
+    # the first batch's eight sends and eight receives at least; what was sent after the failure showed went by launches
+    assert failed >= 16 and finished + failed == 2 * n
     # the GPU's staging side lives on: new traffic goes by launch pairs and arrives
     src2_np = rng.integers(0, 256, size=4 * piece, dtype=np.uint8)
     c2 = _open(net, 1, torch.from_numpy(src2_np).cuda(), torch.zeros(4 * piece, dtype=torch.uint8, device="cuda"))
