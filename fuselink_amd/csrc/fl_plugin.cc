@@ -38,6 +38,7 @@
 #include <map>
 #include <mutex>
 #include <new>
+#include <thread>
 #include <vector>
 
 #include "fl_closed_form.h"
@@ -94,12 +95,72 @@ struct Params {
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
 Params g_par;
+
+// updateTxChannelActive / updateRxChannelActive (fuselink.h:247-259): every send and every completed receive stamps its
+// NIC's entry of the monitor's table, under the table's lock (a semaphore when the table is shared between processes).
+// With eight proxy threads at a request every microsecond that lock was the busiest line in the process: each stamp
+// cost its caller one to two microseconds.  A NIC's entry is therefore stamped at most once in kMarkEveryUs, a tenth
+// of the monitor's timeout (FL_NET_MONITOR_TIMEOUT_US): the table's time of last activity is at most that much older
+// than the truth, and a NIC in use can never look idle.
+constexpr int64_t kMarkEveryUs = FL_NET_MONITOR_TIMEOUT_US / 10;
+alignas(64) std::atomic<int64_t> g_last_mark[2][FL_NET_MAX_LANES];
+inline void mark_nic_active(int nic, int is_tx) {
+  const int64_t now = fl_monitor_now();
+  std::atomic<int64_t>& cell = g_last_mark[is_tx ? 1 : 0][nic];
+  int64_t last = cell.load(std::memory_order_relaxed);
+  if (last != 0 && now >= last && now - last < kMarkEveryUs) return;
+  if (!cell.compare_exchange_strong(last, now, std::memory_order_relaxed)) return;   // another thread stamps it now
+  (void)fl_monitor_mark_active(nic, is_tx, now);
+}
 std::mutex g_init_mu;            // ncclIbLock, plugin.cc:84
+
+// A lock for sections of a few dozen nanoseconds that two proxy threads enter millions of times a second (a
+// connection's descriptor ring and counters, the peer's queue of waiting sends).  It spins: a std::mutex puts the loser
+// to sleep, and the wake-up costs several microseconds -- with a sender and a receiver thread polling one connection,
+// completions that were already visible were seen 7 us late at the median and 19 us late at the 90th percentile.  After
+// a few thousand tries it yields, for the case that the holder has lost its core.
+class ShortLock {
+  std::atomic<bool> held{false};
+ public:
+  void lock() {
+    for (int spins = 0;;) {
+      if (!held.exchange(true, std::memory_order_acquire)) return;
+      while (held.load(std::memory_order_relaxed)) {
+        if (++spins < 4096) {
+#if defined(__x86_64__) || defined(__i386__)
+          __builtin_ia32_pause();
+#endif
+        } else {
+          std::this_thread::yield();
+          spins = 0;
+        }
+      }
+    }
+  }
+  bool try_lock() { return !held.load(std::memory_order_relaxed) && !held.exchange(true, std::memory_order_acquire); }
+  void unlock() { held.store(false, std::memory_order_release); }
+};
 
 // NCCL_FUSELINK_TRACE=1: calls and nanoseconds spent inside the entry points and inside the launches they make
 // (fl_net_host_stats).  Off, a probe costs one predictable branch.
 enum : int { kTrIsend = 0, kTrIrecv, kTrTest, kTrTestDone, kTrFlush, kTrLaunch, kTrRequestsLaunched, kTrEngineSubmit, kTrEngineStart, kTrCount };
-std::atomic<int64_t> g_tr_calls[kTrCount], g_tr_ns[kTrCount];
+// Every thread counts into a block of its own (the blocks live as long as the process; fl_net_host_stats sums them):
+// counters shared by eight proxy threads that poll every few hundred nanoseconds cost each probe more than what it measures.
+struct TraceCounters { alignas(64) std::atomic<int64_t> calls[kTrCount]; std::atomic<int64_t> ns[kTrCount]; };
+std::mutex g_tr_mu;
+std::vector<TraceCounters*> g_tr_blocks;
+inline void tr_add(int what, int64_t calls, int64_t ns) {
+  thread_local TraceCounters* mine = [] {
+    TraceCounters* t = new TraceCounters();
+    for (int k = 0; k < kTrCount; ++k) { t->calls[k].store(0, std::memory_order_relaxed); t->ns[k].store(0, std::memory_order_relaxed); }
+    std::lock_guard<std::mutex> g(g_tr_mu);
+    g_tr_blocks.push_back(t);
+    return t;
+  }();
+  // one writer per block: a load and a store, no locked instruction
+  mine->calls[what].store(mine->calls[what].load(std::memory_order_relaxed) + calls, std::memory_order_relaxed);
+  if (ns) mine->ns[what].store(mine->ns[what].load(std::memory_order_relaxed) + ns, std::memory_order_relaxed);
+}
 inline int64_t tr_now() {
   timespec t;
   clock_gettime(CLOCK_MONOTONIC, &t);
@@ -108,7 +169,8 @@ inline int64_t tr_now() {
 // NCCL_FUSELINK_TRACE=2 also keeps a timeline: (nanoseconds, thread, event, value) of every entry-point event, in a fixed
 // ring that fl_net_timeline() copies out.  Events: 1 irecv posted (value = channel), 2 isend matched (channel),
 // 3 pass that launches begins (requests waiting), 4 batch handed over (requests << 32 | number; bit 31 of the number's
-// word set for engine batches), 5 request seen complete by test (channel << 1 | is-receive).
+// word set for engine batches), 5 request seen complete by test (its batch's number << 16 | channel << 1 | is-receive),
+// 6 a test call is the first to see the engine's batches complete up to this number.
 struct TimelineEvent { int64_t ns; uint32_t thread; uint32_t event; uint64_t value; };
 constexpr size_t kTimelineCap = 1 << 16;
 TimelineEvent g_timeline[kTimelineCap];
@@ -127,8 +189,7 @@ struct TraceScope {
   explicit TraceScope(int w) : what(w), t0(g_par.trace ? tr_now() : 0) {}
   ~TraceScope() {
     if (!t0) return;
-    g_tr_calls[what].fetch_add(1, std::memory_order_relaxed);
-    g_tr_ns[what].fetch_add(tr_now() - t0, std::memory_order_relaxed);
+    tr_add(what, 1, tr_now() - t0);
   }
 };
 bool g_inited = false;
@@ -280,7 +341,7 @@ struct Peer {
   // matched sends that wait for a launch, in arrival order.  (Cache lines: what the senders write, what the pollers
   // read and what only the thread that launches touches are kept apart; polling threads must not slow a launch down by
   // pulling its lines away.)
-  alignas(64) std::mutex queue_mu;
+  alignas(64) ShortLock queue_mu;
   std::vector<Pending> pending;
   std::atomic<uint32_t> waiting_reqs{0};
   std::atomic<uint64_t> waiting_bytes{0};
@@ -302,6 +363,7 @@ struct Peer {
   // Its batches alternate between two window sets of their own and have their own numbers, tables and headers.
   flh_engine* engine = nullptr;
   std::atomic<bool> engine_ok{false};              // cleared for good when the engine reports an error
+  std::atomic<uint64_t> tl_engine_seen{0};         // timeline only: the engine batches some test call has seen complete
   flh_window* ewin[kEngineSetsMax][FL_NET_MAX_LANES] = {};
   flh_windows ewins[kEngineSetsMax] = {};
   flh_chunk_desc* d_etable = nullptr;              // kEngineSlots tables of kEngineRows rows
@@ -312,7 +374,7 @@ constexpr uint32_t kEngineSlots = 64;              // the engine's descriptor ri
 constexpr uint32_t kEngineRows = 512;              // chunks an engine batch may hold
 
 struct Link {
-  std::mutex mu;
+  ShortLock mu;
   int refs = 2;                     // one per side
   int dev = 0;                      // NIC index the comms were opened on
   int channelId = 0;                // plugin.cc:693-708
@@ -415,7 +477,7 @@ void peer_destroy(Peer* pr) {        // no longer reachable through g_peers
 void link_unref(Link* lk) {
   bool last;
   {
-    std::lock_guard<std::mutex> g(lk->mu);
+    std::lock_guard<ShortLock> g(lk->mu);
     last = --lk->refs == 0;
   }
   if (!last) return;
@@ -737,7 +799,7 @@ ncclResult_t fl_connect(int dev, void* opaqueHandle, void** sendComm, ncclNetDev
   Link* lk = (Link*)h->stage_link;
   int ready;
   {
-    std::lock_guard<std::mutex> g(lk->mu);
+    std::lock_guard<ShortLock> g(lk->mu);
     ready = lk->send_ready;
   }
   if (ready == 0) return ncclSuccess;  // accept has not happened yet
@@ -775,7 +837,7 @@ ncclResult_t fl_accept(void* listenComm, void** recvComm, ncclNetDeviceHandle_v8
   c->is_send = 0;
   c->link = lk;
   {
-    std::lock_guard<std::mutex> g(lk->mu);
+    std::lock_guard<ShortLock> g(lk->mu);
     lk->send_ready = 1;
   }
   *recvComm = c;
@@ -813,7 +875,7 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
     mh->start_addr = (uintptr_t)base;
     mh->size = bsz;
     if (c->is_send && !shm) {  // staging is bound at registration time, not on the request path
-      std::lock_guard<std::mutex> g(c->link->mu);
+      std::lock_guard<ShortLock> g(c->link->mu);
       rc = attach_peer(c->link, mh->device);
       if (rc != ncclSuccess) { (void)flh_region_release(mh->region); delete mh; return rc; }
     }
@@ -1137,8 +1199,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
                                       &seg_base[0][0]);
     if (g_par.trace) {   // submits that had to start the resident kernel are counted apart: they pay for a launch
       const int which = flh_engine_launches(pr->engine) != starts_before ? kTrEngineStart : kTrEngineSubmit;
-      g_tr_calls[which].fetch_add(1, std::memory_order_relaxed);
-      g_tr_ns[which].fetch_add(tr_now() - t_sub, std::memory_order_relaxed);
+      tr_add(which, 1, tr_now() - t_sub);
     }
     if (frc == FLH_E_NOMEM) return ncclInProgress;   // the descriptor ring is full: the caller takes the launch path for this batch
     if (frc < 0) {
@@ -1187,7 +1248,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
 // touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).
 void flush_pending(Peer* pr) {
   {
-    std::lock_guard<std::mutex> g(pr->queue_mu);
+    std::lock_guard<ShortLock> g(pr->queue_mu);
     if (pr->pending.empty()) return;
     pr->work.clear();
     pr->work.swap(pr->pending);
@@ -1214,7 +1275,7 @@ void flush_pending(Peer* pr) {
     }
     work.swap(sorted);
   }
-  if (g_par.trace) g_tr_calls[kTrRequestsLaunched].fetch_add((int64_t)work.size(), std::memory_order_relaxed);
+  if (g_par.trace) tr_add(kTrRequestsLaunched, (int64_t)work.size(), 0);
   tl_event(3, (uint64_t)work.size());
   size_t i = 0;
   while (i < work.size()) {
@@ -1309,7 +1370,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
   int rtype = 0;
   ncclResult_t rc = ncclSuccess;
   {
-    std::lock_guard<std::mutex> g(lk->mu);
+    std::lock_guard<ShortLock> g(lk->mu);
     if (lk->send_ready <= 0) { FL_WARN("NET/FuseLink: isend() called when comm->ready == 0"); return ncclInternalError; }  // plugin.cc:1502
     // wait for the receiver to have posted the matching receive (plugin.cc:1510-1514)
     const int slot = (int)(lk->fifoHead % FL_NET_MAX_REQUESTS);
@@ -1344,7 +1405,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
   uint8_t* dst = (uint8_t*)(uintptr_t)w.addr;
   const bool src_dev = mh->type == NCCL_PTR_CUDA, dst_dev = rtype == NCCL_PTR_CUDA;
   // the comm's own NIC carried traffic (updateTxChannelActive, fuselink.h:247-252)
-  (void)fl_monitor_mark_active(lk->dev % g_par.lanes, 1, fl_monitor_now());
+  mark_nic_active(lk->dev % g_par.lanes, 1);
   if (size == 0 || (!src_dev && !dst_dev)) {
     // host memory is not staged (fuselink.cc:8-13): the wire is a copy
     if (size) memcpy(dst, data, (size_t)size);
@@ -1368,7 +1429,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     tl_event(2, (uint64_t)lk->channelId);
     uint32_t waiting;
     {
-      std::lock_guard<std::mutex> g(pr->queue_mu);
+      std::lock_guard<ShortLock> g(pr->queue_mu);
       pr->pending.push_back(p);
       waiting = pr->waiting_reqs.load(std::memory_order_relaxed) + 1;
       if (waiting == 1 && g_par.batch_wait_ns) pr->waiting_since.store(tr_now(), std::memory_order_relaxed);
@@ -1405,7 +1466,7 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
   if (shm) return shm_irecv((ShmComm*)recvComm, data[0], sizes[0], tags[0], mh, request);
   Link* lk = c->link;
   TraceScope tr(kTrIrecv);
-  std::lock_guard<std::mutex> g(lk->mu);
+  std::lock_guard<ShortLock> g(lk->mu);
   bool refreshed = false;
   if (lk->r_finished % g_par.refresh_batch == 0 || !lk->have_decision) {   // plugin.cc:1700
     // only when everything received so far has been consumed (plugin.cc:1704-1709)
@@ -1574,7 +1635,13 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   if (st == kStQueued) return ncclSuccess;
   if (st == kStLaunched && r->engine) {
     // the engine stores the number of the last complete batch to a pinned word: a plain load, as for the launches' words
-    if (flh_engine_completed(pr->engine) < r->seq) {
+    const uint64_t e_done = flh_engine_completed(pr->engine);
+    if (g_par.trace >= 2) {
+      uint64_t seen = pr->tl_engine_seen.load(std::memory_order_relaxed);
+      while (e_done > seen && !pr->tl_engine_seen.compare_exchange_weak(seen, e_done, std::memory_order_relaxed)) {}
+      if (e_done > seen) tl_event(6, e_done);
+    }
+    if (e_done < r->seq) {
       if (flh_engine_error(pr->engine) == 0) return ncclSuccess;
       // the engine went down on a wait that ran out: what it still held is lost, later traffic travels by launches
       pr->engine_ok.store(false, std::memory_order_release);
@@ -1586,9 +1653,9 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     ncclResult_t rc = launch_complete(pr, r->seq, &complete);
     if (rc != ncclSuccess || !complete) return rc;
   }
-  if (g_par.trace) g_tr_calls[kTrTestDone].fetch_add(1, std::memory_order_relaxed);
-  tl_event(5, ((uint64_t)lk->channelId << 1) | (r->type == kReqRecv ? 1u : 0u));
-  std::lock_guard<std::mutex> g(lk->mu);
+  if (g_par.trace) tr_add(kTrTestDone, 1, 0);
+  tl_event(5, ((uint64_t)r->seq << 16) | ((uint64_t)(lk->channelId & 0x7fff) << 1) | (r->type == kReqRecv ? 1u : 0u));
+  std::lock_guard<ShortLock> g(lk->mu);
   ncclResult_t result = ncclSuccess;
   if (r->fault) {   // failed completion, plugin.cc:1839-1861
     FL_WARN("NET/FuseLink : Got completion with error (injected), channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
@@ -1607,7 +1674,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   *done = result == ncclSuccess ? 1 : 0;                    // plugin.cc:1807-1823
   if (r->type == kReqSend) { lk->s_finished++; lk->s_inflight--; }
   if (r->type == kReqRecv) {
-    (void)fl_monitor_mark_active(lk->dev % g_par.lanes, 0, fl_monitor_now());   // updateRxChannelActive, fuselink.h:254-259
+    mark_nic_active(lk->dev % g_par.lanes, 0);   // updateRxChannelActive, fuselink.h:254-259
     lk->r_finished++;
     lk->r_inflight--;
     if (sizes) sizes[0] = r->size;   // the reference leaves 0 here (plugin.cc:1726, 1882)
@@ -1654,7 +1721,7 @@ ncclResult_t fl_close_listen(void* listenComm) {
   }
   for (Link* lk : orphans) {   // connects nobody will accept: tell the connecting side, drop the listener's share
     {
-      std::lock_guard<std::mutex> g(lk->mu);
+      std::lock_guard<ShortLock> g(lk->mu);
       lk->send_ready = -1;
     }
     link_unref(lk);
@@ -1731,6 +1798,7 @@ int fl_net_reset(void) {
   }
   g_par = Params();
   g_inited = false;
+  for (auto& dir : g_last_mark) for (auto& cell : dir) cell.store(0, std::memory_order_relaxed);
   if (fl_monitor_is_shared()) fl_monitor_detach();  // back to the process-local table until init attaches again
   return FLH_OK;
 }
@@ -1738,7 +1806,7 @@ int fl_net_reset(void) {
 int fl_net_inject_fault(void* request) {
   Request* r = (Request*)request;
   if (!r || r->magic != kReqMagic || r->type == kReqUnused) return fl_set_error(FLH_E_ARG, "not a request in flight");
-  std::lock_guard<std::mutex> g(r->link->mu);
+  std::lock_guard<ShortLock> g(r->link->mu);
   r->fault = 1;
   return FLH_OK;
 }
@@ -1747,7 +1815,7 @@ int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64
   Comm* c = (Comm*)comm;
   if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
   Link* lk = c->link;
-  std::lock_guard<std::mutex> g(lk->mu);
+  std::lock_guard<ShortLock> g(lk->mu);
   if (n_finished) *n_finished = c->is_send ? lk->s_finished : lk->r_finished;
   if (in_flight) *in_flight = c->is_send ? lk->s_inflight : lk->r_inflight;
   if (refreshes) *refreshes = lk->refreshes;
@@ -1854,9 +1922,12 @@ int fl_net_last_launch(void* comm, fl_net_launch_seg* segs_out, int max_segs, vo
 }
 
 int fl_net_host_stats(int64_t* calls_out, int64_t* ns_out, int n) {
+  std::lock_guard<std::mutex> g(g_tr_mu);
   for (int k = 0; k < n && k < kTrCount; ++k) {
-    if (calls_out) calls_out[k] = g_tr_calls[k].load(std::memory_order_relaxed);
-    if (ns_out) ns_out[k] = g_tr_ns[k].load(std::memory_order_relaxed);
+    int64_t calls = 0, ns = 0;
+    for (const TraceCounters* t : g_tr_blocks) { calls += t->calls[k].load(std::memory_order_relaxed); ns += t->ns[k].load(std::memory_order_relaxed); }
+    if (calls_out) calls_out[k] = calls;
+    if (ns_out) ns_out[k] = ns;
   }
   return kTrCount;
 }

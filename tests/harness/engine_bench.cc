@@ -21,12 +21,12 @@
 static double now_us() { return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now().time_since_epoch()).count(); }
 
 int main(int argc, char** argv) {
-  if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [--requests N] [--depth D] [--workgroups W] [--batches B]\n", argv[0]); return 1; }
-  int nreq = 8, depth = 2, wgs = 0, batches = 2000;
+  if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [--requests N] [--depth D] [--workgroups W] [--batches B] [--span-mib S]\n", argv[0]); return 1; }
+  int nreq = 8, depth = 2, wgs = 0, batches = 2000, span_mib = 0;
   for (int i = 2; i + 1 < argc; i += 2) {
     const std::string a = argv[i];
     const int v = atoi(argv[i + 1]);
-    if (a == "--requests") nreq = v; else if (a == "--depth") depth = v; else if (a == "--workgroups") wgs = v; else if (a == "--batches") batches = v;
+    if (a == "--requests") nreq = v; else if (a == "--depth") depth = v; else if (a == "--workgroups") wgs = v; else if (a == "--batches") batches = v; else if (a == "--span-mib") span_mib = v;
   }
   if (nreq < 1 || nreq > FLH_BATCH_MAX || depth < 1 || depth > 8 || batches < 1) { fprintf(stderr, "arguments out of range\n"); return 1; }
   void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
@@ -36,13 +36,18 @@ int main(int argc, char** argv) {
   HIP(hipSetDevice(0));
   if (p_flh_init(0)) { fprintf(stderr, "init: %s\n", p_flh_last_error()); return 1; }
   const size_t req = 512 << 10, lanes = 8, cap = 4 << 20;
+  // --span-mib S: successive batches walk through S MiB of sources and destinations, so that what a batch touches is in
+  // no cache (the plugin's traffic); without it every batch moves the same buffers
+  const size_t batch_bytes = req * nreq;
+  const size_t slots = span_mib > 0 ? (((size_t)span_mib << 20) / batch_bytes ? ((size_t)span_mib << 20) / batch_bytes : 1) : 1;
+  const size_t span = slots * batch_bytes;
   uint8_t *src, *dst, *win;
-  HIP(hipMalloc((void**)&src, req * nreq)); HIP(hipMalloc((void**)&dst, req * nreq)); HIP(hipMalloc((void**)&win, (size_t)depth * lanes * cap));
-  std::vector<uint8_t> pattern(req * nreq);
+  HIP(hipMalloc((void**)&src, span)); HIP(hipMalloc((void**)&dst, span)); HIP(hipMalloc((void**)&win, (size_t)depth * lanes * cap));
+  std::vector<uint8_t> pattern(span);
   uint64_t x = 88172645463325252ull;
-  for (auto& b : pattern) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; b = (uint8_t)x; }
+  for (size_t i = 0; i < span; i += 8) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; memcpy(&pattern[i], &x, 8); }
   HIP(hipMemcpy(src, pattern.data(), pattern.size(), hipMemcpyHostToDevice));
-  HIP(hipMemset(dst, 0, req * nreq));
+  HIP(hipMemset(dst, 0, span));
   flh_chunk_desc* table; flh_sched_hdr* hdr;
   HIP(hipMalloc((void**)&table, 4096 * sizeof(flh_chunk_desc))); HIP(hipMalloc((void**)&hdr, sizeof(flh_sched_hdr)));
   int32_t *h_status, *d_status;
@@ -55,20 +60,20 @@ int main(int argc, char** argv) {
   const uint32_t credits[8] = {8, 6, 7, 1, 8, 7, 3, 3};
   for (size_t l = 0; l < lanes; ++l) b.u.credits[l] = credits[l];
   b.n_req = nreq;
-  for (int q = 0; q < nreq; ++q) { b.d_src[q] = src + q * req; b.d_dst[q] = dst + q * req; b.bytes[q] = req; }
+  for (int q = 0; q < nreq; ++q) b.bytes[q] = req;
+  uint64_t submitted = 0;
   flh_engine* e = nullptr;
   if (p_flh_engine_create(0, wgs, 200, depth, &e)) { fprintf(stderr, "engine: %s\n", p_flh_last_error()); return 1; }
   uint64_t seq = 0;
-  auto submit = [&](int set) { if (p_flh_engine_submit(e, &b, &w[set], table, hdr, d_status, &seq, nullptr)) { fprintf(stderr, "submit: %s\n", p_flh_last_error()); exit(1); } };
+  auto submit = [&](int set) {
+    const size_t at = (size_t)(submitted++ % slots) * batch_bytes;
+    for (int q = 0; q < nreq; ++q) { b.d_src[q] = src + at + q * req; b.d_dst[q] = dst + at + q * req; }
+    if (p_flh_engine_submit(e, &b, &w[set], table, hdr, d_status, &seq, nullptr)) { fprintf(stderr, "submit: %s\n", p_flh_last_error()); exit(1); } };
   auto wait_for = [&](uint64_t upto) {
     const double deadline = now_us() + 5e6;
     while (p_flh_engine_completed(e) < upto) if (now_us() > deadline) { fprintf(stderr, "timed out, engine error %d\n", p_flh_engine_error(e)); exit(2); }
   };
   for (int i = 0; i < 10; ++i) { submit(i % depth); wait_for(seq); }
-  // the bytes must have arrived
-  std::vector<uint8_t> back(req * nreq);
-  HIP(hipMemcpy(back.data(), dst, back.size(), hipMemcpyDeviceToHost));
-  const bool exact = memcmp(back.data(), pattern.data(), back.size()) == 0 && h_status[0] == 0;
   // one batch at a time
   double t0 = now_us(), sub = 0;
   for (int i = 0; i < batches; ++i) { const double a = now_us(); submit(i % depth); sub += now_us() - a; wait_for(seq); }
@@ -89,10 +94,15 @@ int main(int argc, char** argv) {
     wait_for(seq);
     restart_done += now_us() - a;
   }
-  printf("{\"harness\": \"engine\", \"requests_per_batch\": %d, \"request_bytes\": %zu, \"window_sets\": %d, \"workgroups\": %d, \"batches\": %d, \"bit_exact\": %s, "
+  // the bytes must have arrived: every slot of the span that a batch has moved
+  std::vector<uint8_t> back(span);
+  HIP(hipMemcpy(back.data(), dst, span, hipMemcpyDeviceToHost));
+  const size_t moved = (submitted < slots ? (size_t)submitted : slots) * batch_bytes;
+  const bool exact = memcmp(back.data(), pattern.data(), moved) == 0 && h_status[0] == 0;
+  printf("{\"harness\": \"engine\", \"requests_per_batch\": %d, \"request_bytes\": %zu, \"span_MiB\": %zu, \"window_sets\": %d, \"workgroups\": %d, \"batches\": %d, \"bit_exact\": %s, "
          "\"one_at_a_time_us_per_batch\": %.2f, \"submit_us\": %.2f, \"in_flight_us_per_batch\": %.2f, \"in_flight_us_per_request\": %.3f, \"in_flight_GBps_4N\": %.0f, "
          "\"after_idle_submit_us\": %.1f, \"after_idle_batch_us\": %.1f, \"engine_launches\": %llu}\n",
-         nreq, req, depth, wgs, batches, exact ? "true" : "false", alone, sub / batches, piped, piped / nreq, 4.0 * nreq * req / (piped * 1e-6) / 1e9,
+         nreq, req, span >> 20, depth, wgs, batches, exact ? "true" : "false", alone, sub / batches, piped, piped / nreq, 4.0 * nreq * req / (piped * 1e-6) / 1e9,
          restart_submit / R, restart_done / R, (unsigned long long)p_flh_engine_launches(e));
   p_flh_engine_destroy(e);
   return exact ? 0 : 5;
