@@ -903,17 +903,20 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_runs(CopyRuns a) {
 // by the workgroup that staged it and no workgroup waits for another inside a batch.  A batch's tiles go to the
 // workers in turn, starting behind the worker that took the last tile of the batch before, so that small batches
 // run side by side on different workers.  Only the workers with a share in a batch are counted in and out of it: the
-// others pass it by without an atomic or a fence, so what a small batch costs does not grow with the size of the
-// engine.  Successive batches rotate through the caller's sets of staging windows, and a worker enters batch k only
-// once batch k - sets is complete.  The last worker to leave a batch stores its number to a host-visible word of the
+// others pass it by without an atomic, so what a small batch costs does not grow with the size of the engine.  The
+// workers never reach a kernel boundary, which is where a kernel's view of memory is brought up to date and its stores
+// are made visible; they touch memory at system scope instead (streaming modes 4 and 8 of the copies) and so need no
+// cache invalidate or L2 write-back per batch.  Successive batches rotate through the caller's sets of staging windows,
+// and a worker enters batch k only once batch k - sets is complete.  The last worker to leave a batch stores its number to a host-visible word of the
 // batch's ring slot; batches of different workers may complete out of order, and the host reports the complete prefix.
 // Every wait in the kernel is bounded: with nothing to do for idle_us the dispatcher takes the engine down (the host
 // starts it again with the next batch), and a wait that outlasts wait_us reports an error and takes it down as well.
 constexpr uint32_t kEngineDevRing = 8;          // descriptors held in device memory; also the most window sets a caller may rotate
 constexpr uint32_t kEngineDescBytes = 4096;
-// A worker takes this many neighbouring copy tiles at a time.  Every worker with a share in a batch pays for an acquire
-// and a release of that batch, so fewer, larger shares serve the engine better than one 32 KiB tile each: 4 MiB batches
-// took 12.8 us with shares of 32 KiB, 9.1 us with 64 KiB, 9.2 us with 128 KiB (16 MiB batches: 22.4, 20.0, 35.7 us).
+// A worker takes this many neighbouring copy tiles at a time: 64 KiB, what a workgroup has in flight when every thread
+// issues its sixteen loads at once.  With shares of one 32 KiB tile a 4 MiB batch on its own takes 11.3 instead of
+// 12.4 us, but four in flight are served every 6.2 instead of every 3.8 us (twice the workers per batch, so fewer
+// batches side by side), and a 16 MiB batch takes 20.9 instead of 18.4 us.
 constexpr uint32_t kEngineShare = 2;
 
 struct EngineDesc {                              // what the host writes per batch (kEngineDescBytes at most)
@@ -1073,7 +1076,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
       uint64_t word = 0;
       const uint64_t t0 = wall_clock64();
       for (uint32_t spin = 0;; ++spin) {
-        word = __hip_atomic_load(&e.dctl->published[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // the fence below acquires
+        word = __hip_atomic_load(&e.dctl->published[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (what it announces is then loaded at system scope)
         const int16_t ahead = (int16_t)((uint16_t)(word >> 48) - (uint16_t)(k + 1));
         if (ahead == 0) break;
         // the slot already holds a later batch: batch k came and went, which it could not have with a share of this worker outstanding
@@ -1110,11 +1113,12 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     if (act == 3) continue;   // nothing read, nothing written, nothing to count
     uint64_t* cnt = &e.dctl->arrive[k % kEngineDevRing];
     // What the batch reads may have been written by anyone, on this GPU or off it, before the host submitted it, and
-    // what it writes is read by anyone once the host has seen it complete.  A worker therefore touches memory at system
-    // scope only (streaming mode 4: loads from memory, stores written through), the descriptor included, and needs no
-    // cache invalidate on its way into a batch and no L2 write-back on its way out.  Either of the two costs every
-    // workgroup that shares the XCD's L2: with 64 workers per batch fencing, batches of eight 512 KiB requests were
-    // served every 7.4 us, without the fences every 4.3 us.
+    // what it writes is read by anyone once the host has seen it complete.  A worker therefore loads the descriptor and
+    // the sources at system scope (mode 8: from memory, whatever line a cache has kept) and stores at system scope
+    // (mode 4: written through); only the windows are read back plainly, by the workgroup that has just written them,
+    // behind a barrier.  So it needs no cache invalidate on its way into a batch and no L2 write-back on its way out.
+    // Either of the two costs every workgroup that shares the XCD's L2: with 64 workers per batch fencing, batches of
+    // eight 512 KiB requests were served every 7.4 us, now every 3.8 us.
     {
       const VecIn<8> slot((const u32x4*)(e.dev_ring + (size_t)(k % kEngineDevRing) * kEngineDescBytes), kEngineDescBytes / 16);
       u32x4* dst = (u32x4*)&d;
@@ -1615,9 +1619,8 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
   *out = nullptr;
   int rc = fl_need_init();
   if (rc) return rc;
-  // Half as many workers as compute units by default.  Every worker that has a tile in a batch pays for an acquire and a
-  // release of that batch, which is what bounds small batches; 128 workers moved 4 MiB batches at 1.3 TB/s and 16 MiB
-  // batches at 3.0 TB/s (4 x bytes), 255 workers at 1.1 and 2.5, 64 at 1.45 and 2.1.
+  // Half as many workers as compute units by default: 128 workers serve 4 MiB batches, two in flight, every 5.9 us and
+  // 16 MiB batches every 12.2 us (2.8 and 5.5 TB/s, 4 x bytes); 256 workers 6.1 and 12.7 us, 32 workers 10.1 and 31 us.
   if (workgroups == 0) workgroups = (uint32_t)g_cus / 2 + 1;
   if (window_sets < 1 || window_sets > kEngineDevRing) return fl_set_error(FLH_E_ARG, "an engine rotates 1..%u window sets, not %u", kEngineDevRing, window_sets);
   if (workgroups < 2 || workgroups > 1024) return fl_set_error(FLH_E_ARG, "an engine takes 2..1024 workgroups (a dispatcher and workers), not %u", workgroups);

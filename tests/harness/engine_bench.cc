@@ -102,7 +102,7 @@ int main(int argc, char** argv) {
   printf("{\"harness\": \"engine\", \"requests_per_batch\": %d, \"request_bytes\": %zu, \"span_MiB\": %zu, \"window_sets\": %d, \"workgroups\": %d, \"batches\": %d, \"bit_exact\": %s, "
          "\"one_at_a_time_us_per_batch\": %.2f, \"submit_us\": %.2f, \"in_flight_us_per_batch\": %.2f, \"in_flight_us_per_request\": %.3f, \"in_flight_GBps_4N\": %.0f, "
          "\"after_idle_submit_us\": %.1f, \"after_idle_batch_us\": %.1f, \"engine_launches\": %llu}\n",
-         nreq, req, span >> 20, depth, wgs, batches, exact ? "true" : "false", alone, sub / batches, piped, piped / nreq, 4.0 * nreq * req / (piped * 1e-6) / 1e9,
+         nreq, req, span_mib > 0 ? span >> 20 : (size_t)0, depth, wgs, batches, exact ? "true" : "false", alone, sub / batches, piped, piped / nreq, 4.0 * nreq * req / (piped * 1e-6) / 1e9,
          restart_submit / R, restart_done / R, (unsigned long long)p_flh_engine_launches(e));
   p_flh_engine_destroy(e);
   return exact ? 0 : 5;
