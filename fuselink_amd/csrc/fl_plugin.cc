@@ -84,11 +84,15 @@ struct Params {
   // through a launch pair each (flh_engine_*); 0 = every batch is a launch pair
   int engine = 1;
   int engine_units = 2;          // staging units per lane for each of the engine's window sets
-  int engine_sets = 2;           // window sets the engine's batches rotate through = batches it has in flight at once
+  int engine_sets = 3;           // window sets the engine's batches rotate through = batches it has in flight at once
   int engine_idle_us = 200;      // the engine goes down after this long without work
   int engine_workgroups = 0;     // 0 = the library's default
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
+  // NCCL_FUSELINK_EAGER_BATCH: this many waiting requests are a batch worth its own trip through the engine and go out
+  // without a free queue slot, as long as a window set is free (0 = never).  Four connections at NCCL's request shape:
+  // 2 000-2 150 GB/s with three sets and 6, against 1 900-1 930 with two sets and the queue depth alone.
+  int eager_batch = 6;
   int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
   int wire_sets = 2;             // NCCL_FUSELINK_WIRE_SETS: sets of landing windows of a receiver on the shared-memory wire = waves on the wire at once
   int wire = 0;                  // NCCL_FUSELINK_WIRE: 0 = both ends in this process (loopback), 1 = the other end is another process (shared-memory wire)
@@ -169,7 +173,7 @@ inline int64_t tr_now() {
 // NCCL_FUSELINK_TRACE=2 also keeps a timeline: (nanoseconds, thread, event, value) of every entry-point event, in a fixed
 // ring that fl_net_timeline() copies out.  Events: 1 irecv posted (value = channel), 2 isend matched (channel),
 // 3 pass that launches begins (requests waiting), 4 batch handed over (requests << 32 | number; bit 31 of the number's
-// word set for engine batches), 5 request seen complete by test (its batch's number << 16 | channel << 1 | is-receive),
+// word set for engine batches), 5 request seen complete by test (its batch's number << 16 | bit 15: an engine batch | channel << 1 | is-receive),
 // 6 a test call is the first to see the engine's batches complete up to this number.
 struct TimelineEvent { int64_t ns; uint32_t thread; uint32_t event; uint64_t value; };
 constexpr size_t kTimelineCap = 1 << 16;
@@ -366,6 +370,7 @@ struct Peer {
   std::atomic<uint64_t> tl_engine_seen{0};         // timeline only: the engine batches some test call has seen complete
   flh_window* ewin[kEngineSetsMax][FL_NET_MAX_LANES] = {};
   flh_windows ewins[kEngineSetsMax] = {};
+  int engine_sets = 0;             // window sets that were bound (NCCL_FUSELINK_ENGINE_SETS, or as many as the pool held)
   flh_chunk_desc* d_etable = nullptr;              // kEngineSlots tables of kEngineRows rows
   flh_sched_hdr* d_ehdr = nullptr;                 // kEngineSlots headers
   alignas(64) std::atomic<uint64_t> engine_submitted{0};   // batches handed to the engine (written under launch_mu)
@@ -564,19 +569,34 @@ ncclResult_t peer_setup(Peer* pr, int device) {
     if (ecap < (uint64_t)g_par.chunk) {
       FL_INFO(NCCL_NET, "NET/FuseLink : the engine's windows (%llu bytes) do not hold a chunk: launches only", (unsigned long long)ecap);
     } else {
+      // as many window sets as asked for, or as the pool still holds whole: the launches' windows come first
+      int sets = 0;
       for (int h = 0; h < g_par.engine_sets; ++h) {
+        bool whole = true;
+        for (int l = 0; l < g_par.lanes && whole; ++l)
+          whole = flh_window_create(pool, ecap, &pr->ewin[h][l]) >= 0 && flh_window_bind(pr->ewin[h][l], ecap) >= 0;
+        if (!whole) {
+          for (int l = 0; l < g_par.lanes; ++l)
+            if (pr->ewin[h][l]) { (void)flh_window_destroy(pr->ewin[h][l]); pr->ewin[h][l] = nullptr; }
+          break;
+        }
         pr->ewins[h].n_lanes = (uint32_t)g_par.lanes;
         for (int l = 0; l < g_par.lanes; ++l) {
-          FL_FLHCHECK(flh_window_create(pool, ecap, &pr->ewin[h][l]));
-          FL_FLHCHECK(flh_window_bind(pr->ewin[h][l], ecap));
           pr->ewins[h].base[l] = flh_window_base(pr->ewin[h][l]);
           pr->ewins[h].cap[l] = flh_window_bound_bytes(pr->ewin[h][l]);
         }
+        ++sets;
       }
-      FL_HIPCHECK(hipMalloc((void**)&pr->d_etable, sizeof(flh_chunk_desc) * (size_t)kEngineSlots * kEngineRows));
-      FL_HIPCHECK(hipMalloc((void**)&pr->d_ehdr, sizeof(flh_sched_hdr) * (size_t)kEngineSlots));
-      FL_FLHCHECK(flh_engine_create(device, (uint32_t)g_par.engine_workgroups, (uint32_t)g_par.engine_idle_us, (uint32_t)g_par.engine_sets, &pr->engine));
-      pr->engine_ok.store(true, std::memory_order_release);
+      if (sets == 0) {
+        FL_INFO(NCCL_NET, "NET/FuseLink : the pool has no room for a window set of the engine: launches only");
+      } else {
+        if (sets < g_par.engine_sets) FL_INFO(NCCL_NET, "NET/FuseLink : the pool holds %d of the engine's %d window sets", sets, g_par.engine_sets);
+        pr->engine_sets = sets;
+        FL_HIPCHECK(hipMalloc((void**)&pr->d_etable, sizeof(flh_chunk_desc) * (size_t)kEngineSlots * kEngineRows));
+        FL_HIPCHECK(hipMalloc((void**)&pr->d_ehdr, sizeof(flh_sched_hdr) * (size_t)kEngineSlots));
+        FL_FLHCHECK(flh_engine_create(device, (uint32_t)g_par.engine_workgroups, (uint32_t)g_par.engine_idle_us, (uint32_t)sets, &pr->engine));
+        pr->engine_ok.store(true, std::memory_order_release);
+      }
     }
   }
   pr->ready = true;
@@ -700,6 +720,7 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.batch_wait_ns = (int)fl_param("FUSELINK_BATCH_WAIT_NS", g_par.batch_wait_ns);
   if (g_par.batch_wait_ns < 0) g_par.batch_wait_ns = 0;
   g_par.queue_depth = (int)fl_param("FUSELINK_QUEUE_DEPTH", g_par.queue_depth);
+  g_par.eager_batch = (int)fl_param("FUSELINK_EAGER_BATCH", g_par.eager_batch);
   if (g_par.queue_depth < 1) g_par.queue_depth = 1;
   if (g_par.completion < 0 || g_par.completion > 2) g_par.completion = 2;
   if (g_par.max_wave_chunks > 65535) g_par.max_wave_chunks = 65535;   // what one fused launch can name
@@ -1195,7 +1216,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     uint64_t got = 0;
     const uint64_t starts_before = g_par.trace ? flh_engine_launches(pr->engine) : 0;
     const int64_t t_sub = g_par.trace ? tr_now() : 0;
-    const int frc = flh_engine_submit(pr->engine, &b, &pr->ewins[k % (uint64_t)g_par.engine_sets], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot, pr->d_status, &got,
+    const int frc = flh_engine_submit(pr->engine, &b, &pr->ewins[k % (uint64_t)pr->engine_sets], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot, pr->d_status, &got,
                                       &seg_base[0][0]);
     if (g_par.trace) {   // submits that had to start the resident kernel are counted apart: they pay for a launch
       const int which = flh_engine_launches(pr->engine) != starts_before ? kTrEngineStart : kTrEngineSubmit;
@@ -1616,7 +1637,9 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     // a launch whose completion comes from an event is only known complete once its own requests are polled: it
     // must not hold anything back
     const bool events_out = pr->last_event_seq.load(std::memory_order_acquire) > pr->done_seq.load(std::memory_order_acquire);
-    bool go = events_out || g_par.completion != 2 || launches_in_queue(pr) + engine_in_flight(pr) < (uint64_t)g_par.queue_depth;
+    const uint64_t in_flight = launches_in_queue(pr) + engine_in_flight(pr);
+    bool go = events_out || g_par.completion != 2 || in_flight < (uint64_t)g_par.queue_depth ||
+              (g_par.eager_batch > 0 && pr->waiting_reqs.load(std::memory_order_acquire) >= (uint32_t)g_par.eager_batch && in_flight < (uint64_t)pr->engine_sets);
     // small sends wait a moment for company: a launch pair costs the host as much as ten requests do
     if (go && g_par.batch_wait_ns && pr->waiting_bytes.load(std::memory_order_acquire) < kEarlyLaunchBytes &&
         pr->waiting_reqs.load(std::memory_order_acquire) < (uint32_t)g_par.batch &&
@@ -1654,7 +1677,7 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     if (rc != ncclSuccess || !complete) return rc;
   }
   if (g_par.trace) tr_add(kTrTestDone, 1, 0);
-  tl_event(5, ((uint64_t)r->seq << 16) | ((uint64_t)(lk->channelId & 0x7fff) << 1) | (r->type == kReqRecv ? 1u : 0u));
+  tl_event(5, ((uint64_t)r->seq << 16) | (r->engine ? 0x8000u : 0u) | ((uint64_t)(lk->channelId & 0x3fff) << 1) | (r->type == kReqRecv ? 1u : 0u));
   std::lock_guard<ShortLock> g(lk->mu);
   ncclResult_t result = ncclSuccess;
   if (r->fault) {   // failed completion, plugin.cc:1839-1861
