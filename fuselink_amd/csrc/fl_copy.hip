@@ -174,6 +174,8 @@ __device__ __forceinline__ void block_copy_shifted(uint8_t* __restrict__ dst, co
 }
 
 // ---- the same copies in the system-scope modes (bits 2 and 3): vectors through buffer resources, bytes as atomics ----
+// (A second set of routines rather than the first one over accessors: addressing by index off a base instead of by
+// pointer changes the launched kernels' address arithmetic and instruction order, and their code is left as tuned.)
 template <int NT, int U>
 __device__ __forceinline__ void copy_exact_system(const VecOut<NT>& out, const VecIn<NT>& in, uint32_t tid) {
   u32x4 r[U];
