@@ -94,6 +94,7 @@ struct Params {
   // 2 000-2 150 GB/s with three sets and 6, against 1 900-1 930 with two sets and the queue depth alone.
   int eager_batch = 6;
   int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
+  int wire_batch = 4;            // NCCL_FUSELINK_WIRE_BATCH: waiting requests of whole chunks under one credit row that may share a wave of the shared-memory wire (1 = a wave per request)
   int wire_sets = 2;             // NCCL_FUSELINK_WIRE_SETS: sets of landing windows of a receiver on the shared-memory wire = waves on the wire at once
   int wire = 0;                  // NCCL_FUSELINK_WIRE: 0 = both ends in this process (loopback), 1 = the other end is another process (shared-memory wire)
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
@@ -707,6 +708,9 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
     g_par.wire = wv && (!strcmp(wv, "shm") || !strcmp(wv, "1")) ? 1 : 0;
   }
   g_par.wire_sets = (int)fl_param("FUSELINK_WIRE_SETS", g_par.wire_sets);
+  g_par.wire_batch = (int)fl_param("FUSELINK_WIRE_BATCH", g_par.wire_batch);
+  if (g_par.wire_batch < 1) g_par.wire_batch = 1;
+  if (g_par.wire_batch > FLH_BATCH_MAX) g_par.wire_batch = FLH_BATCH_MAX;
   if (g_par.wire_sets < 1) g_par.wire_sets = 1;
   if (g_par.wire_sets > kShmSetsMax) g_par.wire_sets = kShmSetsMax;
   g_par.engine = (int)fl_param("FUSELINK_ENGINE", g_par.engine);

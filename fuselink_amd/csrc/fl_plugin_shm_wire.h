@@ -37,6 +37,11 @@ struct ShmWave {                   // one wave of chunks that has landed in the 
   uint64_t bytes;
   uint32_t last;                   // the request's last wave
   uint32_t set;                    // the set of landing windows it lies in
+  // A wave may instead carry n_req >= 2 whole requests, fifo_idx and the ones behind it, staged as one message of
+  // `bytes` from epoch_bytes on (flh_stripe_batch with one segment); req_bytes are the sends' sizes.
+  uint32_t n_req;
+  uint32_t pad;
+  uint64_t req_bytes[FLH_BATCH_MAX];
 };
 struct ShmWire {
   uint64_t magic;
@@ -75,6 +80,9 @@ struct ShmFlight {                 // a wave whose GPU work is queued: the event
   ShmRequest* req;
   uint64_t fifo_idx, epoch_bytes, offset, bytes;
   uint32_t last, set;
+  uint32_t n_req = 1;              // a wave of several whole requests: req and the ones behind it
+  ShmRequest* batch[FLH_BATCH_MAX];
+  uint64_t req_bytes[FLH_BATCH_MAX];
 };
 
 struct ShmComm {
@@ -410,6 +418,8 @@ ncclResult_t shm_progress_send(ShmComm* c) {
     wv.bytes = f.bytes;
     wv.last = f.last;
     wv.set = f.set;
+    wv.n_req = f.n_req;
+    for (uint32_t q = 0; q < f.n_req && f.n_req > 1; ++q) wv.req_bytes[q] = f.req_bytes[q];
     c->waves_published++;
     wv.seq.store(c->waves_published, std::memory_order_release);
     c->flights.pop_front();
@@ -425,9 +435,68 @@ ncclResult_t shm_progress_send(ShmComm* c) {
     }
     if (r->refresh && r->launched == 0) c->epoch_bytes = 0;
     uint64_t wave = (uint64_t)wave_chunks(r->credits, g_par.lanes, chunk, c->wins.cap[0], c->epoch_bytes / chunk) * chunk;
+    const uint64_t room = wave;
     if (wave > r->size - r->launched) wave = r->size - r->launched;
     const uint32_t set = (uint32_t)(c->waves_launched % (uint64_t)c->sets);
     if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
+    // Requests behind this one that have not started either, under the same credit row and without a refresh of
+    // their own, share the wave while it has room: together they are one message from the carried prefix on (every
+    // request but the last a whole number of chunks), staged by one launch, carried by one, reassembled by one.  At
+    // NCCL's 512 KiB steps a wave per request costs both sides their launches and events for half a megabyte each.
+    uint32_t n_req = 1;
+    uint64_t total = r->size;
+    if (g_par.wire_batch > 1 && r->launched == 0 && r->size > 0 && r->size <= room) {
+      while ((int)n_req < g_par.wire_batch && c->cursor + n_req < c->active.size()) {
+        const ShmRequest* prev = c->active[c->cursor + n_req - 1];
+        const ShmRequest* t = c->active[c->cursor + n_req];
+        if (prev->size % chunk != 0 || t->refresh || t->size == 0 || t->launched != 0 || t->all_launched ||
+            memcmp(t->credits, r->credits, sizeof(r->credits)) != 0 || total + t->size > room)
+          break;
+        total += t->size;
+        ++n_req;
+      }
+    }
+    if (n_req >= 2) {
+      flh_batch_params b;
+      memset(&b, 0, sizeof(b));
+      fill_uniform(b.u, r->credits, total, 0, c->epoch_bytes, FLH_TILE_BYTES);
+      b.n_req = n_req;
+      ShmFlight f;
+      for (uint32_t q = 0; q < n_req; ++q) {
+        ShmRequest* t = c->active[c->cursor + q];
+        b.d_src[q] = t->src;
+        b.bytes[q] = t->size;
+        f.batch[q] = t;
+        f.req_bytes[q] = t->size;
+      }
+      FL_FLHCHECK(flh_stripe_batch(&b, &c->wins, c->d_table, c->d_hdr, c->d_status, c->stream));
+      c->last_rows = (uint32_t)((total + chunk - 1) / chunk);
+      FlCreditRow row;
+      fl_row_make(r->credits, (uint32_t)g_par.lanes, row);
+      uint64_t lane_bytes[FLH_MAX_LANES];
+      uint32_t lane_chunks[FLH_MAX_LANES];
+      fl_row_lane_totals(row, c->epoch_bytes / chunk, total, chunk, lane_bytes, lane_chunks);
+      FL_FLHCHECK(flh_copy_runs(c->landing_wins[set].base, c->wins.base, lane_bytes, (uint32_t)g_par.lanes, c->stream));
+      FL_HIPCHECK(hipEventRecord(c->ev[set], c->stream));
+      f.req = r;
+      f.fifo_idx = r->fifo_idx;
+      f.epoch_bytes = c->epoch_bytes;
+      f.offset = 0;
+      f.bytes = total;
+      f.set = set;
+      f.last = 1;
+      f.n_req = n_req;
+      c->epoch_bytes += total;
+      c->waves_launched++;
+      for (uint32_t q = 0; q < n_req; ++q) {
+        ShmRequest* t = f.batch[q];
+        t->launched = t->size;
+        t->all_launched = true;
+        t->last_wave = c->waves_launched;
+      }
+      c->flights.push_back(f);
+      continue;   // the cursor steps over the requests at the top of the loop
+    }
     if (wave) {
       flh_uniform_params u;
       fill_uniform(u, r->credits, wave, r->launched, c->epoch_bytes, FLH_TILE_BYTES);
@@ -470,8 +539,12 @@ ncclResult_t shm_progress_recv(ShmComm* c) {
     if (e == hipErrorNotReady) break;
     if (e != hipSuccess) return hip_fail("hipEventQuery", e);
     if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its landing window or buffer (status %d)", *c->h_status); return ncclInternalError; }
-    f.req->received += f.bytes;
-    if (f.last) f.req->complete = true;
+    if (f.n_req > 1) {
+      for (uint32_t q = 0; q < f.n_req; ++q) { f.batch[q]->received += f.req_bytes[q]; f.batch[q]->complete = true; }
+    } else {
+      f.req->received += f.bytes;
+      if (f.last) f.req->complete = true;
+    }
     c->waves_done++;
     c->w->waves_consumed.store(c->waves_done, std::memory_order_release);   // the set's landing windows are free again
     c->flights.pop_front();
@@ -491,7 +564,47 @@ ncclResult_t shm_progress_recv(ShmComm* c) {
       FL_WARN("NET/FuseLink : a wave of request %llu arrived while %llu is next in line", (unsigned long long)wv.fifo_idx, (unsigned long long)r->fifo_idx);
       return ncclInternalError;
     }
-    if (wv.offset + wv.bytes > r->size || wv.set >= (uint32_t)c->sets) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
+    if (wv.set >= (uint32_t)c->sets) { FL_WARN("NET/FuseLink : a wave in a set of landing windows that does not exist"); return ncclInvalidUsage; }
+    if (wv.n_req > 1) {
+      // several whole requests in one wave: this receive and the ones posted behind it
+      const uint32_t n_req = wv.n_req;
+      if (n_req > FLH_BATCH_MAX || c->cursor + n_req > c->active.size()) { FL_WARN("NET/FuseLink : a wave of %u requests arrived, %zu receives are posted", n_req, c->active.size() - c->cursor); return ncclInternalError; }
+      if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
+      flh_batch_params b;
+      memset(&b, 0, sizeof(b));
+      fill_uniform(b.u, r->credits, wv.bytes, 0, wv.epoch_bytes, FLH_TILE_BYTES);
+      b.n_req = n_req;
+      ShmFlight f;
+      uint64_t sum = 0;
+      for (uint32_t q = 0; q < n_req; ++q) {
+        ShmRequest* t = c->active[c->cursor + q];
+        if (t->fifo_idx != wv.fifo_idx + q || wv.req_bytes[q] > t->size || memcmp(t->credits, r->credits, sizeof(r->credits)) != 0) {
+          FL_WARN("NET/FuseLink : request %u of a wave does not fit the receive posted for it", q);
+          return ncclInvalidUsage;
+        }
+        b.d_dst[q] = t->dst;
+        b.bytes[q] = wv.req_bytes[q];
+        f.batch[q] = t;
+        f.req_bytes[q] = wv.req_bytes[q];
+        sum += wv.req_bytes[q];
+      }
+      if (sum != wv.bytes) { FL_WARN("NET/FuseLink : a wave's requests do not add up to its bytes"); return ncclInvalidUsage; }
+      FL_FLHCHECK(flh_reassemble_batch(&b, &c->landing_wins[wv.set], c->d_status, c->stream));
+      FL_HIPCHECK(hipEventRecord(c->ev[wv.set], c->stream));
+      f.req = r;
+      f.fifo_idx = wv.fifo_idx;
+      f.epoch_bytes = wv.epoch_bytes;
+      f.offset = 0;
+      f.bytes = wv.bytes;
+      f.last = 1;
+      f.set = wv.set;
+      f.n_req = n_req;
+      c->flights.push_back(f);
+      c->waves_launched++;
+      c->cursor += n_req;
+      continue;
+    }
+    if (wv.offset + wv.bytes > r->size) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
     if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
     if (wv.bytes) {
       // the credit row this receiver put into the descriptor: the reassembly launch derives the same lanes and offsets

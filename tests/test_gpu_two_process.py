@@ -39,18 +39,24 @@ total = sum(sizes)
 dst = torch.zeros(total + 64, dtype=torch.uint8, device="cuda")
 rc, mh = p.regMr(rcomm, dst.data_ptr(), dst.numel(), P.NCCL_PTR_CUDA)
 assert rc == P.ncclSuccess
-off = 0
+ahead = len(sys.argv) > 3 and sys.argv[3] == "ahead"   # after the first request, post every receive before testing any
+off, posted = 0, []
 for q, n in enumerate(sizes):
     req = None
     while not req:                      # (the refresh gate may hold a receive back until the one before it is done)
         rc, req = p.irecv(rcomm, [dst.data_ptr() + off], [n], [q], [mh])
         assert rc == P.ncclSuccess and time.time() < deadline
-    done = 0
-    while not done:
-        rc, done, got = p.test(req)
-        assert rc == P.ncclSuccess and time.time() < deadline
-    assert got == n, (q, got, n)
+    posted.append((q, n, req))
     off += n
+    if ahead and 0 < q < len(sizes) - 1:
+        continue
+    for q2, n2, r2 in posted:
+        done = 0
+        while not done:
+            rc, done, got = p.test(r2)
+            assert rc == P.ncclSuccess and time.time() < deadline
+        assert got == n2, (q2, got, n2)
+    posted = []
 torch.cuda.synchronize()
 exp = np.random.default_rng(seed).integers(1, 256, size=total, dtype=np.uint8)
 back = dst.cpu().numpy()
@@ -174,3 +180,73 @@ def test_waves_through_small_windows_across_two_processes():
     _run_pair({"NCCL_FUSELINK_LANES": 4, "NCCL_FUSELINK_CHUNKSIZE": chunk, "NCCL_FUSELINK_CREDITS": ",".join(map(str, credits)),
                "NCCL_FUSELINK_WINDOW_UNITS": 1, "NCCL_FUSELINK_WIRE_SETS": 3, "NCCL_FUSELINK_REFRESH_BATCH": 1000},
               [20 << 20, (7 << 20) + 4321, 3 * chunk], seed=33, credits=credits, lanes=4, chunk=chunk, window_bytes=2 << 20)
+
+
+def test_requests_that_wait_together_share_a_wave_across_two_processes():
+    """NCCL keeps eight 512 KiB steps in flight; a wave per request would cost both processes their launches and events
+    for half a megabyte each.  Requests that wait together, of whole chunks and under one credit row, travel as one wave:
+    staged by one launch as one message from the carried prefix on, carried by one, reassembled by one.  The receiver
+    posts four receives before it tests any, the sender matches all four before its first test; the table its striping
+    launch wrote must be the oracle's schedule of the 2.5 MiB the four requests make up, the bytes must arrive."""
+    import ctypes as C
+    import torch
+    lanes, chunk = 4, 128 << 10
+    credits = [3, 1, 2, 2]
+    sizes = [3 * chunk, 4 * chunk, 2 * chunk, 8 * chunk, 3 * chunk + 999, chunk]      # first on its own, four together (the last of them ragged), one behind
+    env = dict(os.environ, NCCL_FUSELINK_WIRE="shm", PYTHONPATH=ROOT, NCCL_FUSELINK_LANES=str(lanes), NCCL_FUSELINK_CHUNKSIZE=str(chunk),
+               NCCL_FUSELINK_CREDITS=",".join(map(str, credits)), NCCL_FUSELINK_REFRESH_BATCH="1000", NCCL_FUSELINK_WIRE_BATCH="4")
+    child = subprocess.Popen([sys.executable, "-c", _RECEIVER, json.dumps(sizes), "34", "ahead"], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                             stderr=subprocess.PIPE, text=True, env=env, cwd=ROOT)
+    keys = ["NCCL_FUSELINK_WIRE"] + list(env_keys(env))
+    p = P.NetPlugin(8)
+    try:
+        line = child.stdout.readline().strip()
+        assert len(line) == 2 * P.NCCL_NET_HANDLE_MAXSIZE, child.stderr.read()[-3000:]
+        handle = C.create_string_buffer(bytes.fromhex(line), P.NCCL_NET_HANDLE_MAXSIZE)
+        p.reconfigure(**{k: env[k] for k in keys})
+        scomm, deadline = None, time.time() + 60
+        while not scomm:
+            rc, scomm = p.connect(1, handle)
+            assert rc == P.ncclSuccess and time.time() < deadline
+        total = sum(sizes)
+        src = torch.from_numpy(np.random.default_rng(34).integers(1, 256, size=total, dtype=np.uint8)).cuda()
+        rc, mh = p.regMr(scomm, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA)
+        assert rc == P.ncclSuccess
+        offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+
+        def send(q):
+            req = None
+            while not req:                  # no request while the receive has not been posted
+                rc, req = p.isend(scomm, src.data_ptr() + int(offs[q]), sizes[q], q, mh)
+                assert rc == P.ncclSuccess and time.time() < deadline
+            return req
+
+        def finish(req):
+            done = 0
+            while not done:
+                rc, done, _ = p.test(req)
+                assert rc == P.ncclSuccess and time.time() < deadline
+
+        finish(send(0))
+        together = [send(q) for q in (1, 2, 3, 4)]      # all four matched before anything is tested: one wave
+        for r in together:
+            finish(r)
+        rows, hdr = p.last_table(scomm)
+        n = sum(sizes[1:5])
+        exp, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=n, chunk_bytes=chunk,
+                                           mode=ob.SCHED_RESET_OFFSETS, state=_state(sizes[0], sizes[0] // chunk))
+        assert rows.size == exp.size == (n + chunk - 1) // chunk
+        for f in ("src_off", "win_off", "len", "lane"):
+            np.testing.assert_array_equal(rows[f], exp[f], err_msg=f)
+        np.testing.assert_array_equal(hdr["lane_bytes"][:lanes], exp_h["lane_bytes"][:lanes])
+        finish(send(5))
+        assert child.stdout.readline().strip() == "receiver ok", child.stderr.read()[-3000:]
+        assert p.deregMr(scomm, mh) == P.ncclSuccess and p.closeSend(scomm) == P.ncclSuccess
+        child.stdin.write("closed\n")
+        child.stdin.flush()
+        _, err = child.communicate(timeout=60)
+        assert child.returncode == 0, err[-3000:]
+    finally:
+        if child.poll() is None:
+            child.kill()
+        p.reconfigure(**{k: None for k in keys})
