@@ -75,7 +75,8 @@ def main() -> int:
     ap.add_argument("--plugin-bench", type=int, default=1,
                     help="also move the headline message through the plugin ABI in the shape a communication library drives it "
                          "(tests/harness/plugin_harness as a child process, started before this process touches the GPU): "
-                         "128 requests of 512 KiB, 8 in flight, one connection and four; 0 = skip")
+                         "128 requests of 512 KiB, 8 in flight, one connection and four; the same shape on 256 MiB per connection; "
+                         "one batch of eight requests through the lane engine alone (tests/harness/engine_bench); 0 = skip")
     ap.add_argument("--ragged", action="store_true",
                     help="blocks workload: add 1..15 bytes to every block, so that no chunk is a multiple of 16 bytes and source and "
                          "window offsets are misaligned against each other")
@@ -133,6 +134,38 @@ def main() -> int:
                 else:
                     plugin[key] = None
                 plugin[key + "_command"] = " ".join(os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd)
+            # the same request shape on a message long enough (256 MiB per connection, 512 requests) for the threads' start
+            # and the lane engine's to be a small part of an iteration: the rate the round trip of a request allows
+            for conns in (1, 4):
+                cmd = [harness, flbuild.lib_path(), "--bytes", str(256 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "12",
+                       "--connections", str(conns)]
+                try:
+                    res = subprocess.run(cmd, capture_output=True, text=True, timeout=120, env=env)
+                    line = json.loads(res.stdout.strip().splitlines()[-1]) if res.returncode == 0 else None
+                except Exception:
+                    line = None
+                key = f"long_message_256MiB_connections_{conns}"
+                if line and line.get("bit_exact"):
+                    plugin[key] = {"GBps_4N": line["GBps_4N_best"], "best_s": line["best_s"], "mean_s": line["mean_s"], "bit_exact": True,
+                                   "us_per_request": round(line["best_s"] * 1e6 / (512 * conns), 3)}
+                else:
+                    plugin[key] = None
+                plugin[key + "_command"] = " ".join(os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd)
+            # what one batch costs the lane engine on its own (no plugin around it): eight 512 KiB requests per batch
+            ebench = os.path.join(ROOT, "tests", "harness", "engine_bench")
+            if os.path.exists(ebench):
+                cmd = [ebench, flbuild.lib_path(), "--requests", "8", "--depth", "4", "--span-mib", "1024"]
+                try:
+                    res = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+                    line = json.loads(res.stdout.strip().splitlines()[-1]) if res.returncode == 0 else None
+                except Exception:
+                    line = None
+                if line and line.get("bit_exact"):
+                    plugin["lane_engine_batch_of_8"] = {"one_at_a_time_us": line["one_at_a_time_us_per_batch"], "four_in_flight_us_per_batch": line["in_flight_us_per_batch"],
+                                                        "four_in_flight_GBps_4N": line["in_flight_GBps_4N"], "buffers": "walking through 1 GiB", "bit_exact": True}
+                else:
+                    plugin["lane_engine_batch_of_8"] = None
+                plugin["lane_engine_batch_of_8_command"] = " ".join(os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd)
 
     import numpy as np
     import torch
