@@ -149,6 +149,56 @@ def test_send_recv_roundtrip_and_sizes(net):
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
+def test_a_nic_in_use_is_stamped_at_most_once_in_a_tenth_of_the_monitors_timeout(net):
+    """updateTxChannelActive (src/fuselink.h:247-252) stamps the NIC's table entry on every send; under the table's lock
+    that was the busiest line of a process with eight proxy threads.  The plugin stamps an entry at most once in 16 us
+    (FL_NET_MONITOR_TIMEOUT_US / 10): the recorded time of last activity may be that much older than the truth, never
+    more.  With the clock in hand: a send at t stamps t; one at t + 10 leaves the stamp alone (the entry ages out 160 us
+    after t, not after t + 10); one at t + 200 stamps again."""
+    L = net.lib
+    IDLE, BUSY = 0, 1
+    assert net.reconfigure(NCCL_FUSELINK_LANES=8) is None
+    lcomm, s, r = net.connect_pair(3)                     # NIC 3
+    src, sp = _host(4096, 3)
+    dst = np.zeros(4096, dtype=np.uint8)
+    _, smh = net.regMr(s, sp, src.size, P.NCCL_PTR_HOST)
+    _, rmh = net.regMr(r, dst.ctypes.data, dst.size, P.NCCL_PTR_HOST)
+
+    def send(tag):
+        rc, rreq = net.irecv(r, [dst.ctypes.data], [4096], [tag], [rmh])
+        assert rc == 0 and rreq
+        rc, sreq = net.isend(s, sp, 4096, tag, smh)
+        assert rc == 0 and sreq
+        net.wait(sreq), net.wait(rreq)
+
+    def tx_status():
+        st = (C.c_int32 * 8)()
+        assert L.fl_monitor_status(1, 8, st) == 0
+        return st[3]
+
+    t = 1_000_000
+    try:
+        L.fl_monitor_set_clock(1, t)
+        send(0)
+        assert tx_status() == BUSY
+        L.fl_monitor_set_clock(1, t + 10)
+        send(1)                                           # within 16 us of the stamp: not stamped again
+        L.fl_monitor_tick(t + 165)
+        assert tx_status() == IDLE                        # 165 us after t; a stamp at t + 10 would still be 155 us young
+        L.fl_monitor_set_clock(1, t + 200)
+        send(2)
+        assert tx_status() == BUSY
+        L.fl_monitor_tick(t + 355)
+        assert tx_status() == BUSY                        # stamped at t + 200: 155 us old
+        L.fl_monitor_tick(t + 360)
+        assert tx_status() == IDLE
+    finally:
+        L.fl_monitor_set_clock(0, 0)
+        net.deregMr(s, smh), net.deregMr(r, rmh)
+        net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+        net.reconfigure(NCCL_FUSELINK_LANES=None)
+
+
 def test_error_convention(net):
     lcomm, s, r = net.connect_pair(0)
     src, sp = _host(8192, 2)
