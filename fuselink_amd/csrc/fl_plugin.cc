@@ -93,6 +93,10 @@ struct Params {
   // without a free queue slot, as long as a window set is free (0 = never).  Four connections at NCCL's request shape:
   // 2 000-2 150 GB/s with three sets and 6, against 1 900-1 930 with two sets and the queue depth alone.
   int eager_batch = 6;
+  // NCCL_FUSELINK_LIGHT_LOAD: while the engine's batches in flight hold fewer requests than this, what waits goes out
+  // past the queue depth as well, as long as a window set is free.  One connection keeps eight requests in flight: its
+  // batches of two to three are worth a third slot (850-910 against 740 GB/s); four connections' batches of seven are not.
+  int light_load = 8;
   int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
   int wire_batch = 4;            // NCCL_FUSELINK_WIRE_BATCH: waiting requests of whole chunks under one credit row that may share a wave of the shared-memory wire (1 = a wave per request)
   int wire_sets = 2;             // NCCL_FUSELINK_WIRE_SETS: sets of landing windows of a receiver on the shared-memory wire = waves on the wire at once
@@ -327,6 +331,8 @@ constexpr size_t kEventRing = 1024;
 // The staging side of one GPU, shared by every connection that stages there, as the reference's per-NIC lane comms
 // are shared by all channels (fuselink.h:271-272; opened once, on the first connect, plugin.cc:727-753): one stream,
 // one staging window per lane, one queue of matched sends, one sequence of launch numbers.
+constexpr uint32_t kEngineSlots = 64;              // the engine's descriptor ring
+constexpr uint32_t kEngineRows = 512;              // chunks an engine batch may hold
 struct Peer {
   int hip_device = 0;
   int links = 0;                    // connections attached (g_peer_mu)
@@ -375,9 +381,8 @@ struct Peer {
   flh_chunk_desc* d_etable = nullptr;              // kEngineSlots tables of kEngineRows rows
   flh_sched_hdr* d_ehdr = nullptr;                 // kEngineSlots headers
   alignas(64) std::atomic<uint64_t> engine_submitted{0};   // batches handed to the engine (written under launch_mu)
+  std::atomic<uint64_t> engine_reqs_upto[kEngineSlots] = {};   // requests in batches 1..k, at k mod the ring: what the engine holds is a difference of two
 };
-constexpr uint32_t kEngineSlots = 64;              // the engine's descriptor ring
-constexpr uint32_t kEngineRows = 512;              // chunks an engine batch may hold
 
 struct Link {
   ShortLock mu;
@@ -725,6 +730,7 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   if (g_par.batch_wait_ns < 0) g_par.batch_wait_ns = 0;
   g_par.queue_depth = (int)fl_param("FUSELINK_QUEUE_DEPTH", g_par.queue_depth);
   g_par.eager_batch = (int)fl_param("FUSELINK_EAGER_BATCH", g_par.eager_batch);
+  g_par.light_load = (int)fl_param("FUSELINK_LIGHT_LOAD", g_par.light_load);
   if (g_par.queue_depth < 1) g_par.queue_depth = 1;
   if (g_par.completion < 0 || g_par.completion > 2) g_par.completion = 2;
   if (g_par.max_wave_chunks > 65535) g_par.max_wave_chunks = 65535;   // what one fused launch can name
@@ -1233,6 +1239,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
       return ncclInProgress;
     }
     seq = got;
+    pr->engine_reqs_upto[got % kEngineSlots].store(pr->engine_reqs_upto[(got - 1) % kEngineSlots].load(std::memory_order_relaxed) + b.n_req, std::memory_order_relaxed);
     pr->engine_submitted.store(got, std::memory_order_release);
   } else {
     start_stamp(pr, seq, b.u);
@@ -1609,6 +1616,14 @@ uint64_t engine_in_flight(Peer* pr) {
   return sub > done ? sub - done : 0;
 }
 
+// Requests in the engine batches that are not yet reported complete.
+uint64_t engine_requests_in_flight(Peer* pr) {
+  if (!pr->engine || !pr->engine_ok.load(std::memory_order_acquire)) return 0;
+  const uint64_t sub = pr->engine_submitted.load(std::memory_order_acquire), done = flh_engine_completed(pr->engine);
+  if (sub <= done || sub - done >= kEngineSlots) return 0;
+  return pr->engine_reqs_upto[sub % kEngineSlots].load(std::memory_order_relaxed) - pr->engine_reqs_upto[done % kEngineSlots].load(std::memory_order_relaxed);
+}
+
 // Launches of the peer that have been queued and are not known to be complete.
 uint64_t launches_in_queue(Peer* pr) {
   uint64_t done = pr->done_seq.load(std::memory_order_acquire);
@@ -1643,7 +1658,9 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     const bool events_out = pr->last_event_seq.load(std::memory_order_acquire) > pr->done_seq.load(std::memory_order_acquire);
     const uint64_t in_flight = launches_in_queue(pr) + engine_in_flight(pr);
     bool go = events_out || g_par.completion != 2 || in_flight < (uint64_t)g_par.queue_depth ||
-              (g_par.eager_batch > 0 && pr->waiting_reqs.load(std::memory_order_acquire) >= (uint32_t)g_par.eager_batch && in_flight < (uint64_t)pr->engine_sets);
+              (in_flight < (uint64_t)pr->engine_sets &&
+               ((g_par.eager_batch > 0 && pr->waiting_reqs.load(std::memory_order_acquire) >= (uint32_t)g_par.eager_batch) ||
+                engine_requests_in_flight(pr) < (uint64_t)g_par.light_load));
     // small sends wait a moment for company: a launch pair costs the host as much as ten requests do
     if (go && g_par.batch_wait_ns && pr->waiting_bytes.load(std::memory_order_acquire) < kEarlyLaunchBytes &&
         pr->waiting_reqs.load(std::memory_order_acquire) < (uint32_t)g_par.batch &&
