@@ -194,6 +194,15 @@ ncclResult_t shm_connect(int dev, void* opaqueHandle, void** sendComm) {
     name[63] = 0;
     int fd = shm_open(name, O_RDWR, 0600);
     if (fd < 0) { FL_WARN("NET/FuseLink : connect: no shared-memory object %s (is the listener alive?)", name); return ncclSystemError; }
+    // the object is the other process's: it must be the size this build gives the wire (a listener of another build
+    // lays it out differently, and touching pages beyond a shorter object would raise SIGBUS)
+    struct stat st;
+    if (fstat(fd, &st) != 0 || (size_t)st.st_size != sizeof(ShmWire)) {
+      FL_WARN("NET/FuseLink : connect: the shared-memory object %s holds %lld bytes, this build's wire %zu: the listener runs another build", name,
+              (long long)st.st_size, sizeof(ShmWire));
+      close(fd);
+      return ncclInvalidUsage;
+    }
     void* p = mmap(nullptr, sizeof(ShmWire), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
     close(fd);
     if (p == MAP_FAILED) return ncclSystemError;

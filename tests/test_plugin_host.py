@@ -453,3 +453,27 @@ def test_the_shared_memory_wire_refuses_a_listener_in_the_connecting_process():
         assert p.closeListen(lcomm) == P.ncclSuccess
     finally:
         p.reconfigure(NCCL_FUSELINK_WIRE=old)
+
+
+def test_the_shared_memory_wire_refuses_an_object_of_another_size():
+    """The wire's layout belongs to the build; a listener of another build would lay the object out differently.  A
+    connect that finds an object of another size refuses it instead of mapping it."""
+    p = P.NetPlugin(8)
+    old = os.environ.get("NCCL_FUSELINK_WIRE")
+    p.reconfigure(NCCL_FUSELINK_WIRE="shm")
+    name = "/fuselink-wire-1-999999"
+    path = "/dev/shm" + name
+    try:
+        rc, handle, lcomm = p.listen(0)
+        assert rc == P.ncclSuccess
+        with open(path, "wb") as f:
+            f.write(b"\0" * 4096)
+        forged = C.create_string_buffer(handle.raw, P.NCCL_NET_HANDLE_MAXSIZE)
+        forged[40:104] = name.encode().ljust(64, b"\0")
+        rc, scomm = p.connect(0, forged)
+        assert rc == P.ncclInvalidUsage and not scomm
+        assert p.closeListen(lcomm) == P.ncclSuccess
+    finally:
+        if os.path.exists(path):
+            os.unlink(path)
+        p.reconfigure(NCCL_FUSELINK_WIRE=old)
