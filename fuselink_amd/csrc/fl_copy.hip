@@ -510,9 +510,19 @@ struct FusedBatchArgs : FusedArgs {
   uint64_t req_bytes[FLH_BATCH_MAX];
   BatchSeg seg[FLH_SEG_MAX];
 };
-static_assert(sizeof(FusedBatchArgs) <= 4096, "a kernel's argument block holds 4 KiB");
+// Wire sends: a second set of windows, the receiver's landing windows.  The workgroup that has staged a tile in its
+// lane's window then carries it into the same lane and offset of this set, the part the NIC of that lane plays in the
+// reference (an RDMA write out of the staged copy, plugin.cc:1453-1495, 1582).  Argument blocks of their own, so that
+// the launches without a wire keep theirs as they are.
+struct FusedCarryArgs : FusedArgs { flh_windows carry; };
+struct FusedBatchCarryArgs : FusedBatchArgs { flh_windows carry; };
+static_assert(sizeof(FusedBatchCarryArgs) <= 4096, "a kernel's argument block holds 4 KiB");
 template <class A> struct is_batch { static constexpr bool value = false; };
 template <> struct is_batch<FusedBatchArgs> { static constexpr bool value = true; };
+template <> struct is_batch<FusedBatchCarryArgs> { static constexpr bool value = true; };
+template <class A> struct has_carry { static constexpr bool value = false; };
+template <> struct has_carry<FusedCarryArgs> { static constexpr bool value = true; };
+template <> struct has_carry<FusedBatchCarryArgs> { static constexpr bool value = true; };
 
 // The message lives in pages of a pool: byte b of it is byte b mod page_bytes of pool page
 // page_table[b / page_bytes].  `user` is the pool; a tile never straddles a page (tile_bytes divides page_bytes).
@@ -555,7 +565,8 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
 }
 
 // One workgroup's share of a fused launch: tile bx of the chunk that grid row by stands for (`span` neighbouring tiles
-// of that chunk from bx on, for a caller that hands out larger shares).
+// of that chunk from bx on, for a caller that hands out larger shares).  DIR 0: user buffer -> staging window, 1: window
+// -> user buffer, 2: staging window -> the same lane and offset of the carry windows (the wire).
 template <int DIR, int NT, class Args>
 __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by, uint32_t span = 1) {
   constexpr bool BATCH = is_batch<Args>::value;
@@ -595,7 +606,7 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
     len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
     src_off = (uint64_t)in_seg * a.chunk_bytes;
   } else {
-    if (DIR == 0 && a.dest_order) {
+    if (DIR != 1 && a.dest_order) {
       FusedRow r;
       fused_row(a, r);
       uint64_t K = 0, hi = r.pfx[0];
@@ -756,7 +767,18 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
     u = user + (uint64_t)pg * a.page_bytes + (at - pi * a.page_bytes);
   }
   uint8_t* w = (uint8_t*)a.win.base[lane] + win_off + off;
-  if (DIR == 0) block_copy<NT>(w, u, bytes); else block_copy<NT>(u, w, bytes);
+  if constexpr (DIR == 2) {
+    static_assert(has_carry<Args>::value, "the carry needs landing windows");
+    if (win_off + len > a.carry.cap[lane]) {
+      if (threadIdx.x == 0) st_obj<NT>(a.status, (int32_t)FLH_E_RANGE);
+      return;
+    }
+    block_copy<NT>((uint8_t*)a.carry.base[lane] + win_off + off, w, bytes);
+  } else if constexpr (DIR == 0) {
+    block_copy<NT>(w, u, bytes);
+  } else {
+    block_copy<NT>(u, w, bytes);
+  }
 }
 
 template <int DIR, int NT, class Args>
@@ -764,14 +786,21 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   warm_kernel_args(a);
   uint32_t bx = blockIdx.x, by = blockIdx.y;   // tile of the chunk, chunk (in message or destination order)
   xcd_tile_2d(a.xcd_map, bx, by);
-  if (DIR == 0 && a.start_word && bx == 0 && by == 0 && threadIdx.x == 0)
+  if (a.start_word && bx == 0 && by == 0 && threadIdx.x == 0)
     __hip_atomic_store(a.start_word, a.start_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   fused_tile<DIR, NT>(a, bx, by);
+  if constexpr (DIR == 0 && has_carry<Args>::value) {
+    // the wire: the tile this workgroup has just staged goes on into the landing windows.  The barrier orders the
+    // workgroup's stores before its loads of the same bytes (one compute unit, one L1, the XCD's L2 behind it); the
+    // loads stay cacheable whatever the launch's streaming mode, the stores stream when the staging stores do.
+    __syncthreads();
+    fused_tile<2, (NT & 2)>(a, bx, by);
+  }
   // Completion word.  Every workgroup of the grid comes through here, also those without a tile.  The barrier orders
   // the workgroup's stores before thread 0's increment, which releases them at agent scope; the workgroup that counts
   // the last one has thereby acquired every other workgroup's stores, and its store of the word releases all of them
   // at system scope.  A reader that finds done_value with an acquire load may read the destination.
-  if (DIR == 1 && a.done_word) {
+  if ((DIR == 1 || has_carry<Args>::value) && a.done_word) {
     __syncthreads();
     if (threadIdx.x == 0) {
       const uint32_t total = gridDim.x * gridDim.y;
@@ -921,11 +950,17 @@ constexpr uint32_t kEngineDescBytes = 4096;
 // batches side by side), and a 16 MiB batch takes 20.9 instead of 18.4 us.
 constexpr uint32_t kEngineShare = 2;
 
+// What a batch does with its tiles.  Loop: user buffers -> staging windows -> receive buffers, both ends in this process.
+// Send: user buffers -> staging windows -> the same lane and offset of the landing windows (FusedArgs::carry), which are
+// the receiving process's memory: staging plus the wire.  Receive: landing windows (given as the batch's windows) ->
+// receive buffers.
+enum : uint32_t { kEngineLoop = FLH_ENGINE_LOOP, kEngineSend = FLH_ENGINE_SEND, kEngineRecv = FLH_ENGINE_RECV };
 struct EngineDesc {                              // what the host writes per batch (kEngineDescBytes at most)
   uint32_t tiles;                                // worker shares of the batch (the slot's first word: the dispatcher's thread 0 has it in hand)
-  uint32_t pad[3];
-  FusedBatchArgs a;                              // as the striping launch would take it (req_user = sources)
-  uint8_t* req_dst[FLH_BATCH_MAX];               // the reassembly side's buffers
+  uint32_t kind;
+  uint32_t pad[2];
+  FusedBatchCarryArgs a;                         // as the striping launch would take it (req_user = sources; kEngineRecv: the receive buffers)
+  uint8_t* req_dst[FLH_BATCH_MAX];               // kEngineLoop: the reassembly side's buffers
 };
 static_assert(sizeof(EngineDesc) <= kEngineDescBytes, "descriptor slot too small");
 
@@ -948,6 +983,11 @@ struct EngineDevCtl {                            // device memory
   uint64_t quit_at;
   alignas(64) uint64_t arrive[kEngineDevRing];   // workers with a share that have left the batches of each ring slot, never reset
   alignas(64) uint64_t target[kEngineDevRing];   // the dispatcher's record: arrive[slot] once the slot's latest batch is complete (kept across engine launches)
+  // per ring slot, the number of the last batch of the slot whose completion word has reached the host (stored by the
+  // worker that stored the word, once that store has been acknowledged).  The dispatcher gives a slot to batch k only
+  // once this says k - ring: the completion word of a slot can then never be stored out of order, however long the
+  // last worker of a batch dawdles between counting itself out and storing the word.
+  alignas(64) uint64_t freed[kEngineDevRing];
 };
 
 // The published word: batch number (16 bits) | first worker (10) | shares, saturated (10) | low 14 bits of the slot
@@ -970,6 +1010,7 @@ struct EngineArgs {
   EngineDevCtl* dctl;
   uint64_t start;                                // first batch to execute
   uint64_t idle_ticks, wait_ticks;               // of the 100 MHz wall clock
+  uint64_t resident_ticks;                       // the engine leaves after this long even with work at hand (0: never); the host starts it again
   uint32_t inject_fault;                         // tests of the failure path: fail in place of executing the first batch
 };
 
@@ -993,14 +1034,24 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     uint32_t first_worker = 0;      // takes the first tile of batch k
     uint32_t polls = 0;
     uint64_t idle_since = wall_clock64(), free_since = idle_since;
+    const uint64_t born = idle_since;
     if (tid < kEngineDevRing) tgt[tid] = e.dctl->target[tid];   // where the engine before this one left the slots
     __syncthreads();
     for (;;) {
       if (tid == 0) {
         uint32_t act = 0;   // 0 poll again, 1 copy descriptor k, 2 leave
         const uint64_t now = wall_clock64();
-        // the device slot of batch k held batch k - ring: that one must be complete
-        if (__hip_atomic_load(&e.dctl->arrive[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= tgt[k % kEngineDevRing]) {
+        if (e.resident_ticks && now - born > e.resident_ticks) {
+          // Resident long enough.  A kernel that never ends holds its hardware queue, and whatever the runtime has
+          // put on the same queue behind it (streams outnumber queues) waits for as long as small requests keep
+          // coming.  So the engine leaves between two batches although there may be work, and the host starts the
+          // next one (the submit that finds the state at 0, or flh_engine_poke): the queue drains in between.
+          __hip_atomic_store(&e.hctl->state, 2u, __ATOMIC_SEQ_CST, __HIP_MEMORY_SCOPE_SYSTEM);
+          act = 2;
+        } else
+        // the device slot of batch k held batch k - ring: that one must be complete and its completion word out
+        if (__hip_atomic_load(&e.dctl->arrive[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= tgt[k % kEngineDevRing] &&
+            (k < kEngineDevRing || __hip_atomic_load(&e.dctl->freed[k % kEngineDevRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + kEngineDevRing >= k + 1)) {
           free_since = now;
           if (tail_seen <= k) tail_seen = __hip_atomic_load(&e.hctl->tail, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
           if (tail_seen > k) act = 1;
@@ -1053,8 +1104,11 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
         tgt[slot] = own_target;
         e.dctl->target[slot] = own_target;
         __hip_atomic_store(&e.dctl->published[slot], engine_word(k, first_worker, tiles, own_target, wait_target), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        if (takers == 0)   // nothing to move (the host submits no such batch): complete as it stands
+        if (takers == 0) {   // nothing to move (the host submits no such batch): complete as it stands
           __hip_atomic_store(&e.hctl->done[slot], k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __hip_atomic_store(&e.dctl->freed[slot], k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         first_worker = (uint32_t)((first_worker + tiles) % W);
       }
       ++k;
@@ -1129,21 +1183,42 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     __syncthreads();
     const uint32_t tpc = d.a.tiles_per_chunk;
     const uint32_t total = tpc * d.a.n_chunks;
+    const uint32_t kind = d.kind;
     // a share is kEngineShare neighbouring tiles: one copy of twice the length when they lie in one chunk
     const bool whole = tpc % kEngineShare == 0;
-    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {                         // this worker's tiles, user buffers -> windows
-      const uint32_t t0 = sh * kEngineShare;
-      if (whole) fused_tile<0, 12>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
-      else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<0, 12>(d.a, t % tpc, t / tpc);
+    if (kind != kEngineRecv) {
+      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {                       // this worker's tiles, user buffers -> windows
+        const uint32_t t0 = sh * kEngineShare;
+        if (whole) fused_tile<0, 12>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
+        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<0, 12>(d.a, t % tpc, t / tpc);
+      }
+      __syncthreads();
     }
-    __syncthreads();
-    if (tid < FLH_BATCH_MAX) d.a.req_user[tid] = d.req_dst[tid];                          // the same tiles, windows -> receive buffers
-    if (tid == 0) { d.a.table = nullptr; d.a.hdr = nullptr; }
-    __syncthreads();
-    for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
-      const uint32_t t0 = sh * kEngineShare;
-      if (whole) fused_tile<1, 4>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
-      else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<1, 4>(d.a, t % tpc, t / tpc);
+    if (kind == kEngineLoop) {
+      if (tid < FLH_BATCH_MAX) d.a.req_user[tid] = d.req_dst[tid];                        // the same tiles, windows -> receive buffers
+      if (tid == 0) { d.a.table = nullptr; d.a.hdr = nullptr; }
+      __syncthreads();
+      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
+        const uint32_t t0 = sh * kEngineShare;
+        if (whole) fused_tile<1, 4>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
+        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<1, 4>(d.a, t % tpc, t / tpc);
+      }
+    } else if (kind == kEngineSend) {
+      // the same tiles, this process's windows -> the receiving process's landing windows: read back plainly by the
+      // workgroup that wrote them, stored at system scope, so that they are in memory when the count says so
+      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
+        const uint32_t t0 = sh * kEngineShare;
+        if (whole) fused_tile<2, 4>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
+        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<2, 4>(d.a, t % tpc, t / tpc);
+      }
+    } else {
+      // landing windows -> receive buffers.  Another process's kernel wrote the windows (written through, or written
+      // back at the end of its kernel): loaded at system scope, whatever this XCD's L2 has kept of the set's last use.
+      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
+        const uint32_t t0 = sh * kEngineShare;
+        if (whole) fused_tile<1, 12>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
+        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<1, 12>(d.a, t % tpc, t / tpc);
+      }
     }
     // Every thread waits until its stores have been written through and its loads have returned: the wave's memory
     // counter at zero.  (Written out: no fence stands for exactly this.  A release at workgroup scope waits for nothing,
@@ -1155,8 +1230,13 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     __syncthreads();
     if (tid == 0) {
       const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if ((((uint32_t)before + 1) & kEngineCountMask) == own_target)
+      if ((((uint32_t)before + 1) & kEngineCountMask) == own_target) {
         __hip_atomic_store(&e.hctl->done[k % kEngineDevRing], k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        // once the word is out (the store acknowledged), the slot may go to batch k + ring: the word of a slot is
+        // never stored out of order
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __hip_atomic_store(&e.dctl->freed[k % kEngineDevRing], k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
   }
 }
@@ -1289,9 +1369,15 @@ int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win, cons
 
 // argument checks and everything of FusedArgs that follows from the parameters; returns 1 when there is nothing to do
 static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_uniform_params* u, flh_chunk_desc* d_table,
-                      flh_sched_hdr* d_hdr, int32_t* d_status) {
+                      flh_sched_hdr* d_hdr, int32_t* d_status, const flh_windows* carry = nullptr) {
   int rc = check_windows(win);
   if (rc) return rc;
+  if (carry) {   // (the caller's argument block holds the windows themselves)
+    if (dir != 0) return fl_set_error(FLH_E_ARG, "only the striping side carries its tiles on");
+    rc = check_windows(carry);
+    if (rc) return rc;
+    if (carry->n_lanes != win->n_lanes) return fl_set_error(FLH_E_ARG, "%u landing windows for %u staging windows", carry->n_lanes, win->n_lanes);
+  }
   if (!u || !d_status) return fl_set_error(FLH_E_ARG, "parameters and d_status are required");
   if (u->n_lanes == 0 || u->n_lanes > FLH_MAX_LANES || u->n_lanes != win->n_lanes) return fl_set_error(FLH_E_ARG, "n_lanes %u does not match the windows' %u", u->n_lanes, win->n_lanes);
   if (u->chunk_bytes == 0) return fl_set_error(FLH_E_ARG, "chunk_bytes must be > 0");
@@ -1308,11 +1394,11 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
   a.table = dir == 0 ? d_table : nullptr;
   a.hdr = dir == 0 ? d_hdr : nullptr;
   a.status = d_status;
-  a.done_word = dir == 1 ? u->d_done_word : nullptr;
-  a.done_count = dir == 1 ? u->d_done_count : nullptr;
+  a.done_word = dir == 1 || carry ? u->d_done_word : nullptr;   // the launch that ends the path on this side reports
+  a.done_count = dir == 1 || carry ? u->d_done_count : nullptr;
   a.done_value = u->done_value;
   if (a.done_word && !a.done_count) return fl_set_error(FLH_E_ARG, "d_done_word needs d_done_count");
-  a.start_word = dir == 0 ? u->d_start_word : nullptr;
+  a.start_word = u->d_start_word;
   a.start_value = u->start_value;
   a.pad_start = 0;
   a.total_bytes = u->total_bytes;
@@ -1353,13 +1439,13 @@ template <class Args>
 static int launch_fused_args(int dir, const Args& a, int mode, void* stream, void* done_event) {
   const dim3 grid(a.tiles_per_chunk, a.n_chunks);
   hipStream_t s = (hipStream_t)stream;
-  hipEvent_t ev = dir == 1 ? (hipEvent_t)done_event : nullptr;
+  hipEvent_t ev = dir == 1 || has_carry<Args>::value ? (hipEvent_t)done_event : nullptr;
 #define FL_ARGS_EXTRA , Args
   if (dir == 0) {
-    if (mode == 0) FL_LAUNCH((fl_copy_uniform_fused<0, 0 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, a);
-    else if (mode == 1) FL_LAUNCH((fl_copy_uniform_fused<0, 1 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, a);
-    else FL_LAUNCH((fl_copy_uniform_fused<0, 3 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, a);
-  } else {
+    if (mode == 0) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 0 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+    else if (mode == 1) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 1 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+    else FL_LAUNCH_EV((fl_copy_uniform_fused<0, 3 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+  } else if constexpr (!has_carry<Args>::value) {   // (only the striping side carries)
     if (mode == 0) FL_LAUNCH_EV((fl_copy_uniform_fused<1, 0 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
     else if (mode == 2) FL_LAUNCH_EV((fl_copy_uniform_fused<1, 2 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
     else FL_LAUNCH_EV((fl_copy_uniform_fused<1, 3 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
@@ -1371,13 +1457,15 @@ static int launch_fused_args(int dir, const Args& a, int mode, void* stream, voi
 }  // extern "C++"
 
 static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_uniform_params* u,
-                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream) {
-  FusedArgs a;
-  const int rc = fill_fused(a, dir, win, u, d_table, d_hdr, d_status);
+                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream, const flh_windows* carry = nullptr) {
+  FusedCarryArgs a;
+  const int rc = fill_fused(a, dir, win, u, d_table, d_hdr, d_status, carry);
   if (rc) return rc < 0 ? rc : FLH_OK;
   if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
   a.user = (uint8_t*)user;
   a.user_bytes = user_bytes;
+  if (!carry) return launch_fused_args(dir, static_cast<const FusedArgs&>(a), fl_stream_mode(dir, u->total_bytes), stream, u->done_event);
+  a.carry = *carry;
   return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream, u->done_event);
 }
 
@@ -1461,17 +1549,17 @@ int flh_batch_layout(const flh_batch_params* b, uint64_t* lane_end, uint64_t* se
 }
 
 static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table, flh_sched_hdr* d_hdr,
-                        int32_t* d_status, void* stream) {
+                        int32_t* d_status, void* stream, const flh_windows* carry = nullptr) {
   BatchPlan pl;
   int rc = plan_batch(b, pl);
   if (rc) return rc;
-  FusedBatchArgs a;
+  FusedBatchCarryArgs a;
   // fill_fused sees the launch as one message of n_chunks whole chunks (grid, tiles per chunk, checks); the credit row
   // it prepares goes unused, every segment brings its own
   flh_uniform_params u = b->u;
   u.total_bytes = (uint64_t)pl.n_chunks * b->u.chunk_bytes;
   u.epoch_bytes = 0;
-  rc = fill_fused(a, dir, win, &u, d_table, d_hdr, d_status);
+  rc = fill_fused(a, dir, win, &u, d_table, d_hdr, d_status, carry);
   if (rc) return rc < 0 ? rc : FLH_OK;
   a.total_bytes = b->u.total_bytes;
   a.dest_order = 0;
@@ -1490,6 +1578,8 @@ static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* w
     a.req_bytes[q] = b->bytes[q];
   }
   for (uint32_t k = 0; k < FLH_SEG_MAX; ++k) a.seg[k] = pl.seg[k];
+  if (!carry) return launch_fused_args(dir, static_cast<const FusedBatchArgs&>(a), fl_stream_mode(dir, b->u.total_bytes), stream, b->u.done_event);
+  a.carry = *carry;
   return launch_fused_args(dir, a, fl_stream_mode(dir, b->u.total_bytes), stream, b->u.done_event);
 }
 
@@ -1536,6 +1626,18 @@ int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int3
 int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_uniform_params* u,
                        flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
   return launch_fused(0, (void*)d_src, src_bytes, win, u, d_table_out, d_hdr_out, d_status, stream);
+}
+
+int flh_stripe_uniform_carry(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_windows* landing,
+                             const flh_uniform_params* u, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
+  if (!landing) return fl_set_error(FLH_E_ARG, "null landing windows");
+  return launch_fused(0, (void*)d_src, src_bytes, win, u, d_table_out, d_hdr_out, d_status, stream, landing);
+}
+
+int flh_stripe_batch_carry(const flh_batch_params* b, const flh_windows* win, const flh_windows* landing, flh_chunk_desc* d_table_out,
+                           flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
+  if (!landing) return fl_set_error(FLH_E_ARG, "null landing windows");
+  return launch_batch(0, b, win, d_table_out, d_hdr_out, d_status, stream, landing);
 }
 
 int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win, const flh_uniform_params* u,
@@ -1613,7 +1715,7 @@ struct flh_engine {
   uint64_t submitted;       // batches written into the ring
   uint64_t completed;       // batches known complete, in order (atomic; moved forward by whoever looks)
   uint64_t launches;        // engine kernels started
-  uint64_t idle_us, wait_us;
+  uint64_t idle_us, wait_us, resident_us;
 };
 
 int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_t window_sets, flh_engine** out) {
@@ -1635,22 +1737,36 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
   e->host_slots = 64;
   e->idle_us = idle_us ? idle_us : 200;
   e->wait_us = (uint64_t)g_engine_wait_us;   // two seconds unless a test has asked for less (flh_tune "engine_wait_us")
-  FL_HIP(hipSetDevice(device));
-  FL_HIP(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
-  FL_HIP(hipHostMalloc((void**)&e->h_ring, (size_t)e->host_slots * kEngineDescBytes, hipHostMallocMapped));
-  FL_HIP(hipHostGetDevicePointer((void**)&e->d_ring_host, e->h_ring, 0));
-  FL_HIP(hipHostMalloc((void**)&e->h_ctl, sizeof(EngineHostCtl), hipHostMallocMapped));
-  memset(e->h_ctl, 0, sizeof(EngineHostCtl));
-  FL_HIP(hipHostGetDevicePointer((void**)&e->d_ctl_host, e->h_ctl, 0));
-  FL_HIP(hipMalloc((void**)&e->dev_ring, (size_t)kEngineDevRing * kEngineDescBytes));
-  FL_HIP(hipMalloc((void**)&e->dctl, sizeof(EngineDevCtl)));
-  FL_HIP(hipMemset(e->dctl, 0, sizeof(EngineDevCtl)));
+  e->resident_us = 2000;
+  // whatever has been allocated when a call fails goes back through the one cleanup path (which takes null members)
+  auto build = [&]() -> int {
+    FL_HIP(hipSetDevice(device));
+    FL_HIP(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
+    FL_HIP(hipHostMalloc((void**)&e->h_ring, (size_t)e->host_slots * kEngineDescBytes, hipHostMallocMapped));
+    FL_HIP(hipHostGetDevicePointer((void**)&e->d_ring_host, e->h_ring, 0));
+    FL_HIP(hipHostMalloc((void**)&e->h_ctl, sizeof(EngineHostCtl), hipHostMallocMapped));
+    memset(e->h_ctl, 0, sizeof(EngineHostCtl));
+    FL_HIP(hipHostGetDevicePointer((void**)&e->d_ctl_host, e->h_ctl, 0));
+    FL_HIP(hipMalloc((void**)&e->dev_ring, (size_t)kEngineDevRing * kEngineDescBytes));
+    FL_HIP(hipMalloc((void**)&e->dctl, sizeof(EngineDevCtl)));
+    FL_HIP(hipMemset(e->dctl, 0, sizeof(EngineDevCtl)));
+    return FLH_OK;
+  };
+  rc = build();
+  if (rc) { (void)flh_engine_destroy(e); return rc; }
   *out = e;
+  return FLH_OK;
+}
+
+int flh_engine_set_resident(flh_engine* e, uint32_t resident_us) {
+  if (!e) return fl_set_error(FLH_E_ARG, "null engine");
+  e->resident_us = resident_us;   // read by the next start of the resident kernel
   return FLH_OK;
 }
 
 // start the resident kernel with the batch the last one stopped at (the stream orders it behind that one's exit)
 static int engine_start(flh_engine* e) {
+  if (g_engine_fail_start) return fl_set_error(FLH_E_HIP, "engine launch failed: refused by the engine_fail_start test hook");
   int prev = -1;
   (void)hipGetDevice(&prev);
   if (prev != e->device) FL_HIP(hipSetDevice(e->device));
@@ -1667,6 +1783,7 @@ static int engine_start(flh_engine* e) {
   a.start = __atomic_load_n(&e->h_ctl->exited_at, __ATOMIC_ACQUIRE);
   a.idle_ticks = e->idle_us * 100;     // the wall clock counts at 100 MHz
   a.wait_ticks = e->wait_us * 100;
+  a.resident_ticks = e->resident_us * 100;
   a.inject_fault = g_engine_inject_fault ? 1u : 0u;
   __atomic_store_n(&e->h_ctl->state, 1u, __ATOMIC_RELEASE);
   hipLaunchKernelGGL(fl_engine_kernel, dim3(e->workers + 1), dim3(kCopyBlock), 0, e->stream, a);
@@ -1679,9 +1796,19 @@ static int engine_start(flh_engine* e) {
   return FLH_OK;
 }
 
-int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
-                      flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out) {
+// The engine is down (state 0: the dispatcher has left, and it publishes nothing after that) and never published batch
+// `seq`: take the batch back out of the ring, so that no later engine executes it.  Only then may the caller carry it
+// some other way.
+static void engine_take_back(flh_engine* e, uint64_t seq) {
+  e->submitted = seq;
+  __atomic_store_n(&e->h_ctl->tail, seq, __ATOMIC_SEQ_CST);
+}
+
+static int engine_submit(flh_engine* e, uint32_t kind, const flh_batch_params* b, const flh_windows* win, const flh_windows* landing,
+                         flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out) {
   if (!e || !seq_out) return fl_set_error(FLH_E_ARG, "null engine or sequence pointer");
+  if (kind > kEngineRecv) return fl_set_error(FLH_E_ARG, "unknown kind of batch %u", kind);
+  if ((kind == kEngineSend) != (landing != nullptr)) return fl_set_error(FLH_E_ARG, "landing windows go with FLH_ENGINE_SEND and with nothing else");
   if (__atomic_load_n(&e->h_ctl->error, __ATOMIC_ACQUIRE)) return fl_set_error(FLH_E_STATE, "the engine went down on a wait that ran out");
   // the ring slot must be free: its last occupant complete
   const uint64_t seq = e->submitted;
@@ -1698,9 +1825,11 @@ int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_window
   u.d_done_word = nullptr;
   u.d_start_word = nullptr;
   u.done_event = nullptr;
-  FusedBatchArgs a;
-  rc = fill_fused(a, 0, win, &u, d_table_out, d_hdr_out, d_status);
+  FusedBatchCarryArgs a;
+  rc = fill_fused(a, kind == kEngineRecv ? 1 : 0, win, &u, d_table_out, d_hdr_out, d_status, landing);
   if (rc) return rc < 0 ? rc : fl_set_error(FLH_E_ARG, "empty batch");
+  memset(&a.carry, 0, sizeof(a.carry));
+  if (landing) a.carry = *landing;
   a.total_bytes = b->u.total_bytes;
   a.dest_order = 0;
   a.src_base = 0;
@@ -1715,14 +1844,15 @@ int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_window
     a.req_bytes[q] = 0;
     dsts[q] = nullptr;
     if (q >= b->n_req) continue;
-    if (!b->d_src[q] || !b->d_dst[q]) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer", q);
-    a.req_user[q] = (uint8_t*)b->d_src[q];
+    if ((kind != kEngineRecv && !b->d_src[q]) || (kind != kEngineSend && !b->d_dst[q])) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer", q);
+    a.req_user[q] = kind == kEngineRecv ? (uint8_t*)b->d_dst[q] : (uint8_t*)b->d_src[q];
     a.req_bytes[q] = b->bytes[q];
-    dsts[q] = (uint8_t*)b->d_dst[q];
+    dsts[q] = kind == kEngineLoop ? (uint8_t*)b->d_dst[q] : nullptr;
   }
   for (uint32_t k = 0; k < FLH_SEG_MAX; ++k) a.seg[k] = pl.seg[k];
   memcpy(&d->a, &a, sizeof(a));
   memcpy(d->req_dst, dsts, sizeof(dsts));
+  d->kind = kind;
   d->tiles = (a.n_chunks * a.tiles_per_chunk + kEngineShare - 1) / kEngineShare;
   e->submitted = seq + 1;
   *seq_out = seq + 1;
@@ -1732,9 +1862,55 @@ int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_window
   __atomic_thread_fence(__ATOMIC_SEQ_CST);
   uint32_t st = __atomic_load_n(&e->h_ctl->state, __ATOMIC_SEQ_CST);
   for (int spin = 0; st == 2 && spin < 4000000; ++spin) st = __atomic_load_n(&e->h_ctl->state, __ATOMIC_ACQUIRE);   // it decides within microseconds
-  if (st == 2) return fl_set_error(FLH_E_STATE, "the engine did not finish going down");
-  if (st == 0) return engine_start(e);
+  if (st == 2) {
+    // It has not decided (a dispatcher that lost its compute unit to another process's work can take that long).  An
+    // error from here on must be final -- the caller then carries the batch some other way, and an engine that woke
+    // up later and executed it as well would write into buffers that have since been given away.  So the engine is
+    // told to leave and waited for, every wait inside it being bounded; what it did with the batch is then known.
+    (void)hipSetDevice(e->device);
+    __atomic_store_n(&e->h_ctl->stop, 1u, __ATOMIC_RELEASE);
+    const hipError_t err = hipStreamSynchronize(e->stream);
+    __atomic_store_n(&e->h_ctl->stop, 0u, __ATOMIC_RELEASE);
+    if (err != hipSuccess) return fl_set_error(FLH_E_HIP, "the engine did not go down: %s", hipGetErrorString(err));
+    st = __atomic_load_n(&e->h_ctl->state, __ATOMIC_ACQUIRE);
+  }
+  if (st == 0) {
+    // down: either it took the batch with it (published before it left: its workers finish it), or the batch is still
+    // in the ring and the next engine starts with it
+    if (__atomic_load_n(&e->h_ctl->exited_at, __ATOMIC_ACQUIRE) > seq) return FLH_OK;
+    if (__atomic_load_n(&e->h_ctl->error, __ATOMIC_ACQUIRE)) {
+      engine_take_back(e, seq);
+      return fl_set_error(FLH_E_STATE, "the engine went down on a wait that ran out");
+    }
+    rc = engine_start(e);
+    if (rc) engine_take_back(e, seq);
+    return rc;
+  }
   return FLH_OK;
+}
+
+int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
+                      flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out) {
+  return engine_submit(e, kEngineLoop, b, win, nullptr, d_table_out, d_hdr_out, d_status, seq_out, seg_base_out);
+}
+
+int flh_engine_submit_wire(flh_engine* e, uint32_t kind, const flh_batch_params* b, const flh_windows* win, const flh_windows* landing,
+                           flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out) {
+  if (kind != kEngineSend && kind != kEngineRecv) return fl_set_error(FLH_E_ARG, "a wire batch is FLH_ENGINE_SEND or FLH_ENGINE_RECV");
+  return engine_submit(e, kind, b, win, landing, d_table_out, d_hdr_out, d_status, seq_out, seg_base_out);
+}
+
+// An engine that left with batches still in its ring (its time as a resident was up) and that no submit has started
+// again since: start it.  Cheap to ask -- two loads of host memory -- when there is nothing to do.
+int flh_engine_needs_start(const flh_engine* e) {
+  if (!e) return 0;
+  if (__atomic_load_n(&e->h_ctl->state, __ATOMIC_ACQUIRE) != 0) return 0;
+  return __atomic_load_n(&e->h_ctl->tail, __ATOMIC_ACQUIRE) > __atomic_load_n(&e->h_ctl->exited_at, __ATOMIC_ACQUIRE) &&
+         __atomic_load_n(&e->h_ctl->error, __ATOMIC_ACQUIRE) == 0;
+}
+int flh_engine_poke(flh_engine* e) {
+  if (!flh_engine_needs_start(e)) return FLH_OK;
+  return engine_start(e);
 }
 
 // Batches complete, counted in order: batch c is complete once its ring slot reports it or a later batch of the slot
@@ -1762,7 +1938,7 @@ uint64_t flh_engine_launches(const flh_engine* e) { return e ? e->launches : 0; 
 int flh_engine_destroy(flh_engine* e) {
   if (!e) return FLH_OK;
   (void)hipSetDevice(e->device);
-  __atomic_store_n(&e->h_ctl->stop, 1u, __ATOMIC_RELEASE);
+  if (e->h_ctl) __atomic_store_n(&e->h_ctl->stop, 1u, __ATOMIC_RELEASE);
   if (e->stream) (void)hipStreamSynchronize(e->stream);   // the dispatcher sees the flag within a poll
   if (e->h_ring) (void)hipHostFree(e->h_ring);
   if (e->h_ctl) (void)hipHostFree(e->h_ctl);

@@ -86,6 +86,7 @@ struct Params {
   int engine_units = 2;          // staging units per lane for each of the engine's window sets
   int engine_sets = 3;           // window sets the engine's batches rotate through = batches it has in flight at once
   int engine_idle_us = 200;      // the engine goes down after this long without work
+  int engine_resident_us = 2000; // NCCL_FUSELINK_ENGINE_RESIDENT_US: ... and after this long even with work (0 = never), so that its hardware queue drains; the next batch starts it again
   int engine_workgroups = 0;     // 0 = the library's default
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
@@ -601,6 +602,7 @@ ncclResult_t peer_setup(Peer* pr, int device) {
         FL_HIPCHECK(hipMalloc((void**)&pr->d_etable, sizeof(flh_chunk_desc) * (size_t)kEngineSlots * kEngineRows));
         FL_HIPCHECK(hipMalloc((void**)&pr->d_ehdr, sizeof(flh_sched_hdr) * (size_t)kEngineSlots));
         FL_FLHCHECK(flh_engine_create(device, (uint32_t)g_par.engine_workgroups, (uint32_t)g_par.engine_idle_us, (uint32_t)sets, &pr->engine));
+        FL_FLHCHECK(flh_engine_set_resident(pr->engine, (uint32_t)g_par.engine_resident_us));
         pr->engine_ok.store(true, std::memory_order_release);
       }
     }
@@ -721,6 +723,8 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.engine = (int)fl_param("FUSELINK_ENGINE", g_par.engine);
   g_par.engine_units = (int)fl_param("FUSELINK_ENGINE_UNITS", g_par.engine_units);
   g_par.engine_idle_us = (int)fl_param("FUSELINK_ENGINE_IDLE_US", g_par.engine_idle_us);
+  g_par.engine_resident_us = (int)fl_param("FUSELINK_ENGINE_RESIDENT_US", g_par.engine_resident_us);
+  if (g_par.engine_resident_us < 0) g_par.engine_resident_us = 0;
   g_par.engine_sets = (int)fl_param("FUSELINK_ENGINE_SETS", g_par.engine_sets);
   if (g_par.engine_sets < 1 || g_par.engine_sets > kEngineSetsMax) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_ENGINE_SETS must be 1..%d", kEngineSetsMax); return ncclInvalidArgument; }
   g_par.engine_workgroups = (int)fl_param("FUSELINK_ENGINE_WORKGROUPS", g_par.engine_workgroups);
@@ -1686,7 +1690,16 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
       if (e_done > seen) tl_event(6, e_done);
     }
     if (e_done < r->seq) {
-      if (flh_engine_error(pr->engine) == 0) return ncclSuccess;
+      if (flh_engine_error(pr->engine) == 0) {
+        // an engine whose time as a resident ran out leaves between two batches; with nothing further to submit, the
+        // thread that waits for one of them starts the next engine (two loads of host memory to find out)
+        if (flh_engine_needs_start(pr->engine) && pr->launch_mu.try_lock()) {
+          LazyDevice dev(pr->hip_device);
+          if (dev.use() && flh_engine_poke(pr->engine) < 0) FL_WARN("NET/FuseLink : engine: %s", flh_last_error());
+          pr->launch_mu.unlock();
+        }
+        return ncclSuccess;
+      }
       // the engine went down on a wait that ran out: what it still held is lost, later traffic travels by launches
       pr->engine_ok.store(false, std::memory_order_release);
       FL_WARN("NET/FuseLink : the lane engine stopped with an error; channel %d falls back to launches", lk->channelId);
@@ -1701,11 +1714,14 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
   tl_event(5, ((uint64_t)r->seq << 16) | (r->engine ? 0x8000u : 0u) | ((uint64_t)(lk->channelId & 0x3fff) << 1) | (r->type == kReqRecv ? 1u : 0u));
   std::lock_guard<ShortLock> g(lk->mu);
   ncclResult_t result = ncclSuccess;
-  if (r->fault) {   // failed completion, plugin.cc:1839-1861
-    FL_WARN("NET/FuseLink : Got completion with error (injected), channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
-    return ncclRemoteError;
-  }
-  if (st == kStLaunched && pr && __atomic_load_n(pr->h_status, __ATOMIC_ACQUIRE) != 0) {
+  if (r->fault) {
+    // Failed completion (plugin.cc:1839-1861).  The reference returns here with the request still allocated and its
+    // counters untouched: its communicator is dead from then on.  Here the connection lives on (an engine that went
+    // down hands its traffic to launches), so the request is freed and counted like any other: a request that stayed
+    // in flight would hold every later refresh back (r_inflight != 0 on a batch boundary) and leak its slot.
+    FL_WARN("NET/FuseLink : Got completion with error, channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
+    result = ncclRemoteError;
+  } else if (st == kStLaunched && pr && __atomic_load_n(pr->h_status, __ATOMIC_ACQUIRE) != 0) {
     // A kernel refused a chunk that would have left its window or buffer (the host sizes every launch so that this
     // cannot happen; the check is the safety net).  The first request completed after the refusal reports it, once,
     // and is freed like any other; the word is cleared so that later traffic is not condemned with it.
@@ -1891,6 +1907,7 @@ static int drain_peer(Peer* pr) {
     const int64_t until = tr_now() + 5000000000ll;
     while (flh_engine_completed(pr->engine) < pr->engine_submitted.load(std::memory_order_acquire)) {
       if (flh_engine_error(pr->engine) || tr_now() > until) return fl_set_error(FLH_E_STATE, "the lane engine did not finish its batches");
+      if (flh_engine_needs_start(pr->engine)) (void)flh_engine_poke(pr->engine);
     }
   }
   return FLH_OK;

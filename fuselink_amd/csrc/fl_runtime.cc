@@ -32,6 +32,7 @@ int g_copy_uniform_grid = 1;
 int g_xcd_runs = 1;              // flh_tune("xcd_runs")
 int64_t g_engine_wait_us = 2000000;   // flh_tune("engine_wait_us"): limit of every wait inside a lane engine created afterwards
 int g_engine_inject_fault = 0;        // flh_tune("engine_inject_fault"): an engine started while this is set fails at its first batch
+int g_engine_fail_start = 0;          // flh_tune("engine_fail_start"): starting an engine fails as if the launch had been refused
 
 namespace {
 thread_local ProfState t_prof;
@@ -178,8 +179,14 @@ int flh_tune(const char* key, int64_t value) {
   }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "xcd_runs")) { g_xcd_runs = value != 0; return FLH_OK; }
-  if (!strcmp(key, "engine_wait_us")) { if (value < 1) return fl_set_error(FLH_E_ARG, "engine_wait_us < 1"); g_engine_wait_us = value; return FLH_OK; }
-  if (!strcmp(key, "engine_inject_fault")) { g_engine_inject_fault = value != 0; return FLH_OK; }
+  if (!strncmp(key, "engine_", 7)) {
+    // hooks for tests of the failure paths: a production process cannot reach them by accident
+    const char* hooks = getenv("NCCL_FUSELINK_TEST_HOOKS");
+    if (!hooks || strcmp(hooks, "1")) return fl_set_error(FLH_E_STATE, "%s is a test hook: set NCCL_FUSELINK_TEST_HOOKS=1 to use it", key);
+    if (!strcmp(key, "engine_wait_us")) { if (value < 1) return fl_set_error(FLH_E_ARG, "engine_wait_us < 1"); g_engine_wait_us = value; return FLH_OK; }
+    if (!strcmp(key, "engine_inject_fault")) { g_engine_inject_fault = value != 0; return FLH_OK; }
+    if (!strcmp(key, "engine_fail_start")) { g_engine_fail_start = value != 0; return FLH_OK; }
+  }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_seg_min")) {
     if (value < 1) return fl_set_error(FLH_E_ARG, "sched_seg_min < 1");

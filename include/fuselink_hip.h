@@ -151,11 +151,14 @@ int64_t flh_constant(int which);
  * "sched_seg_min" = chunks from which a lent workspace makes the scan scheduler use several workgroups (4096).
  * "xcd_runs" = 1/0: launches of 256 copy workgroups and more hand each of the eight XCDs runs of 32 consecutive
  * tiles (1 MiB) instead of every eighth tile (1, the default; 3-5 % faster copies).
+ * Test hooks (refused with FLH_E_STATE unless the environment holds NCCL_FUSELINK_TEST_HOOKS=1):
  * "engine_wait_us" = limit of every wait inside a lane engine created afterwards (2 000 000; tests of the failure
  * path ask for a microsecond).
  * "engine_inject_fault" = 1: a lane engine that is started (or started again after idling) while this is set reports
  * a wait that ran out in place of executing its first batch and goes down, every workgroup leaving as after a real
  * one (0; for tests of the failure path, which cannot count on a healthy GPU to miss a limit).
+ * "engine_fail_start" = 1: starting the resident kernel fails as a refused launch would (0; the submit that needed the
+ * start must then return its error with the batch taken back out of the ring).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL.
  * The tunables are process-wide and read by every launch: set them while no other thread launches. */
 int flh_tune(const char* key, int64_t value);
@@ -268,6 +271,16 @@ int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows*
                        flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
 int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
                            const flh_uniform_params* u, int32_t* d_status, void* stream);
+/* flh_stripe_uniform for a sender whose receiver is not this process: the workgroup that has staged a tile in its
+ * lane's window carries it on into the same lane and offset of `landing`, windows of the receiver (its device memory,
+ * opened here), which plays the part of the lane's NIC in the reference -- the RDMA write out of the staged copy into
+ * the receiver's translated buffer (src/plugin.cc:1453-1495, 1582, 1626).  The receiver runs flh_reassemble_uniform
+ * over its landing windows with the same parameters.  landing->cap bounds the carry as win->cap bounds the staging
+ * (FLH_E_RANGE through *d_status).  The completion fields of `u` (done word / event) report this launch, which is the
+ * last of the path on the sending side. */
+int flh_stripe_uniform_carry(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_windows* landing,
+                             const flh_uniform_params* u, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
+                             int32_t* d_status, void* stream);
 
 /* Several requests in one launch: requests that are waiting together -- NCCL keeps up to NCCL_STEPS = 8 in flight per
  * channel (src/fuselink.h:14) and runs several channels to a peer, which all share the per-NIC lane comms
@@ -308,6 +321,9 @@ typedef struct flh_batch_params {
 int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
                      flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
 int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int32_t* d_status, void* stream);
+/* flh_stripe_batch with the carry of flh_stripe_uniform_carry (b->d_dst is not used). */
+int flh_stripe_batch_carry(const flh_batch_params* b, const flh_windows* win, const flh_windows* landing,
+                           flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
 /* Where the batch leaves every staging window: lane_end[l] = first free byte of lane l after the last segment
  * (host arithmetic, nothing is launched); seg_base, if given, receives FLH_SEG_MAX x FLH_MAX_LANES lane bases, row k
  * those of segment k.  A caller sizes its batches with it so that no lane outgrows its window. */
@@ -330,6 +346,27 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
 /* *seq_out = the batch's number, from 1; seg_base_out (optional) = the lane bases of its segments, as flh_batch_layout gives them */
 int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
                       flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out);
+/* The two halves of a batch whose ends are different processes, numbered, ordered and reported like any other batch of
+ * the engine.  FLH_ENGINE_SEND: stripe into `win` (the caller's rotating sets, as for flh_engine_submit) and carry every
+ * tile on into `landing`, as flh_stripe_batch_carry does; b->d_dst is not used.  FLH_ENGINE_RECV: reassemble out of `win`
+ * -- the landing windows a sender has filled -- into b->d_dst; b->d_src, `landing` (NULL) and the table pointers are not
+ * used.  A batch is complete when its bytes are in memory: the landing windows' for a send, the receive buffers' for a
+ * receive.  Stands where the reference's NIC stands on either side (src/plugin.cc:1453-1495 / 1616-1677). */
+#define FLH_ENGINE_LOOP 0u   /* what flh_engine_submit submits: both ends in this process */
+#define FLH_ENGINE_SEND 1u
+#define FLH_ENGINE_RECV 2u
+int flh_engine_submit_wire(flh_engine* e, uint32_t kind, const flh_batch_params* b, const flh_windows* win, const flh_windows* landing,
+                           flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out);
+/* How long the resident kernel stays although work keeps coming (microseconds; 0 = as long as there is work; default
+ * 2000).  A kernel that never ends holds its hardware queue; the runtime puts several streams on one queue when a process
+ * has more streams than queues, and what it has queued behind the engine waits until the engine leaves.  With a bound
+ * the engine leaves between two batches when its time is up, and the next flh_engine_submit -- or flh_engine_poke, for a
+ * caller with batches outstanding and nothing further to submit -- starts it again.  flh_engine_needs_start says
+ * whether flh_engine_poke would start it (two loads of host memory).  flh_engine_poke is not thread-safe against
+ * flh_engine_submit. */
+int flh_engine_set_resident(flh_engine* e, uint32_t resident_us);
+int flh_engine_needs_start(const flh_engine* e);
+int flh_engine_poke(flh_engine* e);
 uint64_t flh_engine_completed(const flh_engine* e);   /* batches complete: all with a number up to this one */
 int flh_engine_error(const flh_engine* e);
 uint64_t flh_engine_launches(const flh_engine* e);    /* engine kernels started so far */

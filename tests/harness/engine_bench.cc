@@ -32,7 +32,7 @@ int main(int argc, char** argv) {
   void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
   if (!lib) { fprintf(stderr, "dlopen: %s\n", dlerror()); return 1; }
 #define SYM(name) decltype(&name) p_##name = (decltype(&name))dlsym(lib, #name); if (!p_##name) { fprintf(stderr, "missing %s\n", #name); return 1; }
-  SYM(flh_init) SYM(flh_last_error) SYM(flh_engine_create) SYM(flh_engine_submit) SYM(flh_engine_completed) SYM(flh_engine_error) SYM(flh_engine_launches) SYM(flh_engine_destroy)
+  SYM(flh_init) SYM(flh_last_error) SYM(flh_engine_create) SYM(flh_engine_submit) SYM(flh_engine_completed) SYM(flh_engine_error) SYM(flh_engine_launches) SYM(flh_engine_destroy) SYM(flh_engine_needs_start) SYM(flh_engine_poke)
   HIP(hipSetDevice(0));
   if (p_flh_init(0)) { fprintf(stderr, "init: %s\n", p_flh_last_error()); return 1; }
   const size_t req = 512 << 10, lanes = 8, cap = 4 << 20;
@@ -71,7 +71,11 @@ int main(int argc, char** argv) {
     if (p_flh_engine_submit(e, &b, &w[set], table, hdr, d_status, &seq, nullptr)) { fprintf(stderr, "submit: %s\n", p_flh_last_error()); exit(1); } };
   auto wait_for = [&](uint64_t upto) {
     const double deadline = now_us() + 5e6;
-    while (p_flh_engine_completed(e) < upto) if (now_us() > deadline) { fprintf(stderr, "timed out, engine error %d\n", p_flh_engine_error(e)); exit(2); }
+    while (p_flh_engine_completed(e) < upto) {
+      // an engine whose time as a resident ran out leaves between two batches; whoever waits for one starts the next
+      if (p_flh_engine_needs_start(e) && p_flh_engine_poke(e)) { fprintf(stderr, "poke: %s\n", p_flh_last_error()); exit(1); }
+      if (now_us() > deadline) { fprintf(stderr, "timed out, engine error %d\n", p_flh_engine_error(e)); exit(2); }
+    }
   };
   for (int i = 0; i < 10; ++i) { submit(i % depth); wait_for(seq); }
   // one batch at a time

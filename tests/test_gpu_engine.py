@@ -40,6 +40,7 @@ def test_engine_batches_equal_the_oracle_and_the_engine_restarts_after_idling(fl
     lanes, chunk, n_batches = 6, 32 << 10, 7
     eng = C.c_void_p()
     _lib.check(lib.flh_engine_create(0, 0, 100, sets, C.byref(eng)))     # idle limit 100 us
+    _lib.check(lib.flh_engine_set_resident(eng, 0))                      # (the launches are counted below: only idling takes it down)
     try:
         cap = 3 << 20
         wins = [[torch.zeros(cap + 64, dtype=torch.uint8, device="cuda") for _ in range(lanes)] for _ in range(sets)]

@@ -129,7 +129,7 @@ def _run_pair(env, sizes, seed, credits, lanes, chunk, window_bytes):
 
 
 def env_keys(env):
-    return [k for k in env if k.startswith("NCCL_FUSELINK_") and k != "NCCL_FUSELINK_WIRE"]
+    return [k for k in env if k.startswith("NCCL_FUSELINK_") and k not in ("NCCL_FUSELINK_WIRE", "NCCL_FUSELINK_TEST_HOOKS")]
 
 
 def _state(epoch_bytes, chunk_index):
