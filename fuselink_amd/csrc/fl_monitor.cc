@@ -268,4 +268,26 @@ int fl_monitor_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t
   return FLH_OK;
 }
 
+// The mask a sender ships with its data (refreshTxUsage, src/fuselink.h:265-267, a placeholder there): bit l set when
+// lane l's send side is IDLE in this host's table, the comm's own lane always, and every bit from n_lanes on.
+int fl_monitor_tx_mask(int n_lanes, int own_lane, uint32_t* mask_out) {
+  if (n_lanes < 1 || n_lanes > kGroups || !mask_out) return fl_set_error(FLH_E_ARG, "bad mask query");
+  TableLock l;
+  uint32_t mask = ~0u << n_lanes;
+  for (int i = 0; i < n_lanes; ++i)
+    if (g_tab->tx_status[i] == kIdle || i == own_lane) mask |= 1u << i;
+  *mask_out = mask;
+  return FLH_OK;
+}
+
+// Credits a receiver advertises at a refresh: the query the reference left commented out in refreshRxComm
+// (src/fuselink.h:240-243: getIdleNicRx(group, priority, txAvailable), whose mask skips NICs, src/monitor.h:214).
+int fl_monitor_rx_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t tx_mask, uint32_t* credits_out) {
+  if (n_lanes < 1 || n_lanes > kGroups || !credits_out) return fl_set_error(FLH_E_ARG, "bad credit query");
+  TableLock l;
+  for (int i = 0; i < n_lanes; ++i) credits_out[i] = g_tab->rx_status[i] == kIdle && ((tx_mask >> i) & 1u) ? idle_credit : 0;
+  if (own_lane >= 0 && own_lane < n_lanes && credits_out[own_lane] == 0) credits_out[own_lane] = 1;
+  return FLH_OK;
+}
+
 }  // extern "C"

@@ -99,8 +99,7 @@ struct Params {
   // batches of two to three are worth a third slot (850-910 against 740 GB/s); four connections' batches of seven are not.
   int light_load = 8;
   int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
-  int wire_batch = 4;            // NCCL_FUSELINK_WIRE_BATCH: waiting requests of whole chunks under one credit row that may share a wave of the shared-memory wire (1 = a wave per request)
-  int wire_sets = 2;             // NCCL_FUSELINK_WIRE_SETS: sets of landing windows of a receiver on the shared-memory wire = waves on the wire at once
+  int wire_sets = 4;             // NCCL_FUSELINK_WIRE_SETS: sets of landing windows a receiving process keeps per sending process and GPU = waves on the wire at once
   int wire = 0;                  // NCCL_FUSELINK_WIRE: 0 = both ends in this process (loopback), 1 = the other end is another process (shared-memory wire)
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
@@ -264,6 +263,8 @@ enum : int { kReqUnused = 0, kReqSend = 1, kReqRecv = 2, kReqFlush = 3 };  // pl
 enum : int { kStPosted = 1, kStLaunched = 2, kStDoneHost = 3, kStQueued = 4 };
 
 struct Link;
+struct WireEnd;
+struct WirePair;
 
 struct Request {
   int type = kReqUnused;
@@ -274,6 +275,8 @@ struct Request {
   int size = 0;          // bytes moved (reported by test for receives)
   int fault = 0;         // injected wire fault
   uint32_t magic = 0;
+  uint32_t imm = 0xffffffffu;   // receive: the sender's lane-availability mask that came with the data (imm_data, plugin.cc:1463, 1884-1885)
+  uint64_t wave = 0;         // send to another process: the wave (of its pair) that must be announced before the send is reported
 };
 constexpr uint32_t kReqMagic = 0x464c5251;   // "FLRQ"
 constexpr uint32_t kCommMagic = 0x464c434d;  // "FLCM"
@@ -310,7 +313,11 @@ struct Pending {
   int size;
   bool src_dev, dst_dev;
   FifoWire w;
-  Request *sreq, *rreq;
+  Request *sreq, *rreq;      // (rreq: null when the receiver is another process)
+  uint32_t imm = 0xffffffffu;   // the sender's lane-availability mask that travels with the request
+  uint64_t fifo_idx = 0;     // the descriptor it answers, from 1
+  int q_next = 0;            // a send to another process that travels wave by wave: the QP piece it has got to ...
+  uint64_t q_done = 0;       // ... and the bytes of that piece that are on their way
 };
 
 // What one launch pair carried, for inspection (fl_net_last_launch).
@@ -403,6 +410,13 @@ struct Link {
   int fuselink_offset = -1;
   uint8_t credits[FL_NET_MAX_LANES] = {};
   bool have_decision = false;
+  // The sender's lane-availability mask (getTxUsage / refreshTxUsage, fuselink.h:261-267): refreshed every
+  // N_FINISHED_BATCH sends (plugin.cc:1441-1447), shipped with every request as its immediate data (plugin.cc:1463).
+  uint32_t tx_mask = 0xffffffffu;   // sender: the cached mask (the reference's placeholder value until the first refresh)
+  int64_t tx_refreshes = 0;
+  uint32_t tx_available = 0xffffffffu;   // receiver: the mask of the latest completed receive (comm->txAvailable, plugin.cc:1884-1885)
+  // the other end is another process (NCCL_FUSELINK_WIRE=shm): this end of the shared-memory wire; null on the loopback
+  WireEnd* wire = nullptr;
   // staging side: the GPU's shared one, attached on first use with device memory (set once, under mu)
   std::atomic<Peer*> peer{nullptr};
   // scheduling state of the connection (the peer's launch_mu)
@@ -465,6 +479,7 @@ std::mutex g_peer_mu;                // the peers, their attachment counts
 std::map<int, Peer*> g_peers;        // one per HIP device that stages
 
 void flush_pending(Peer* pr);
+void wire_end_free(Link* lk);
 
 void peer_destroy(Peer* pr) {        // no longer reachable through g_peers
   DeviceScope keep;
@@ -493,11 +508,28 @@ void link_unref(Link* lk) {
     last = --lk->refs == 0;
   }
   if (!last) return;
-  if (Peer* pr = lk->peer.load(std::memory_order_acquire)) {
-    {   // nothing of this connection may still wait for a launch when it goes away
-      std::lock_guard<std::mutex> g(pr->launch_mu);
-      flush_pending(pr);
+  Peer* const peer = lk->peer.load(std::memory_order_acquire);
+  if (peer) {   // nothing of this connection may still wait for a launch when it goes away
+    std::lock_guard<std::mutex> g(peer->launch_mu);
+    flush_pending(peer);
+    // (sends to another process that found no landing set free stay queued: they go with their connection)
+    std::lock_guard<ShortLock> gq(peer->queue_mu);
+    size_t kept = 0;
+    for (size_t i = 0; i < peer->pending.size(); ++i) {
+      if (peer->pending[i].lk == lk) continue;
+      if (kept != i) peer->pending[kept] = peer->pending[i];
+      ++kept;
     }
+    if (kept != peer->pending.size()) {
+      peer->pending.resize(kept);
+      uint64_t bytes = 0;
+      for (const Pending& q : peer->pending) bytes += (uint64_t)q.size;
+      peer->waiting_reqs.store((uint32_t)kept, std::memory_order_release);
+      peer->waiting_bytes.store(bytes, std::memory_order_release);
+    }
+  }
+  wire_end_free(lk);   // (before the staging side: a receiver's landing windows wait for its stream)
+  if (Peer* pr = peer) {
     bool gone;
     {
       std::lock_guard<std::mutex> g(g_peer_mu);
@@ -632,8 +664,12 @@ ncclResult_t attach_peer(Link* lk, int device) {
   return ncclSuccess;
 }
 
-// Credit row the receiver advertises at a refresh.
-void current_credits(int own_lane, uint8_t* out) {
+// Credit row the receiver advertises at a refresh: refreshRxComm(channelId, txAvailable, ...) of plugin.cc:1710 with the
+// query the reference left commented out (fuselink.h:240-243, getIdleNicRx(group, priority, txAvailable)) -- a lane
+// counts when its receive side is idle in this host's table and the sender's mask admits it.  tx_available is the mask
+// that came with the latest completed receive.  Both ends in one process read one table, so there the receiver also
+// looks at the send statuses as they are now (what the sender's next mask will say).
+void current_credits(int own_lane, uint32_t tx_available, bool same_process, uint8_t* out) {
   uint32_t c[FL_NET_MAX_LANES] = {};
   {
     std::lock_guard<std::mutex> g(g_credit_mu);
@@ -642,10 +678,32 @@ void current_credits(int own_lane, uint8_t* out) {
     } else {
       // the daemon's periodic ageing (monitor.cpp:159-193) happens here, right before the table is read
       (void)fl_monitor_tick(fl_monitor_now());
-      (void)fl_monitor_credits(g_par.lanes, own_lane, (uint32_t)g_par.idle_credit, c);
+      uint32_t mask = tx_available, now_mask = 0xffffffffu;
+      if (same_process && fl_monitor_tx_mask(g_par.lanes, own_lane, &now_mask) == 0) mask &= now_mask;
+      (void)fl_monitor_rx_credits(g_par.lanes, own_lane, (uint32_t)g_par.idle_credit, mask, c);
     }
   }
   for (int l = 0; l < FL_NET_MAX_LANES; ++l) out[l] = (uint8_t)(c[l] > 255 ? 255 : c[l]);
+}
+
+// The mask a sender ships with a request: cached, refreshed when (n_finished + 1) % N_FINISHED_BATCH == 0
+// (plugin.cc:1441-1447; refreshTxUsage / getTxUsage, fuselink.h:261-267, placeholders there).  lk->mu held.
+uint32_t sender_mask(Link* lk) {
+  if ((lk->s_finished + 1) % g_par.refresh_batch == 0) {
+    uint32_t mask = 0xffffffffu;
+    bool forced;
+    {
+      std::lock_guard<std::mutex> g(g_credit_mu);
+      forced = g_credit_override;
+    }
+    if (!forced && g_par.policy != 0) {
+      (void)fl_monitor_tick(fl_monitor_now());
+      (void)fl_monitor_tx_mask(g_par.lanes, lk->dev % g_par.lanes, &mask);
+    }
+    lk->tx_mask = mask;
+    lk->tx_refreshes++;
+  }
+  return lk->tx_mask;
 }
 
 // Chunks one wave may carry so that no lane outgrows its window: the largest n for which every lane's share
@@ -715,9 +773,6 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
     g_par.wire = wv && (!strcmp(wv, "shm") || !strcmp(wv, "1")) ? 1 : 0;
   }
   g_par.wire_sets = (int)fl_param("FUSELINK_WIRE_SETS", g_par.wire_sets);
-  g_par.wire_batch = (int)fl_param("FUSELINK_WIRE_BATCH", g_par.wire_batch);
-  if (g_par.wire_batch < 1) g_par.wire_batch = 1;
-  if (g_par.wire_batch > FLH_BATCH_MAX) g_par.wire_batch = FLH_BATCH_MAX;
   if (g_par.wire_sets < 1) g_par.wire_sets = 1;
   if (g_par.wire_sets > kShmSetsMax) g_par.wire_sets = kShmSetsMax;
   g_par.engine = (int)fl_param("FUSELINK_ENGINE", g_par.engine);
@@ -882,8 +937,8 @@ ncclResult_t fl_accept(void* listenComm, void** recvComm, ncclNetDeviceHandle_v8
 ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uint64_t /*offset*/, int /*fd*/, void** mhandle) {
   if (!comm || !data || !mhandle || size == 0) return ncclInvalidArgument;
   Comm* c = (Comm*)comm;
-  const bool shm = c->magic == kShmCommMagic;   // the other end is another process: staging is the comm's own
-  if (c->magic != kCommMagic && !shm) return ncclInvalidArgument;
+  if (c->magic != kCommMagic) return ncclInvalidArgument;
+  const bool wire = c->link->wire != nullptr;   // the other end is another process
   *mhandle = nullptr;
   MemHandle* mh = new (std::nothrow) MemHandle();
   if (!mh) return ncclSystemError;
@@ -909,9 +964,9 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
     if (frc < 0) { delete mh; FL_WARN("NET/FuseLink : region: %s", flh_last_error()); return ncclInternalError; }
     mh->start_addr = (uintptr_t)base;
     mh->size = bsz;
-    if (c->is_send && !shm) {  // staging is bound at registration time, not on the request path
+    if (c->is_send || wire) {  // staging (a receiver in another process: its landing windows) is bound at registration time, not on the request path
       std::lock_guard<ShortLock> g(c->link->mu);
-      rc = attach_peer(c->link, mh->device);
+      rc = c->is_send ? attach_peer(c->link, mh->device) : wire_recv_setup(c->link, mh->device);
       if (rc != ncclSuccess) { (void)flh_region_release(mh->region); delete mh; return rc; }
     }
   } else if (type == NCCL_PTR_HOST) {
@@ -1092,6 +1147,78 @@ ncclResult_t launch_transfer(Peer* pr, const Pending& p, uint64_t seq) {
   return finish_completion(pr, seq, comp);
 }
 
+// The same for a receiver in another process (launch_mu held): every wave of chunks is one launch that stages the wave in
+// this process's windows and carries it on into a set of the pair's landing windows, a wave of the wire with a launch
+// number and a completion of its own.  A wave needs a free landing set; when there is none the send keeps its place (the
+// QP piece and the offset it has got to) and *parked says so: the caller queues it again, in front.
+ncclResult_t launch_transfer_wire(Peer* pr, Pending& p, WirePair* pair, bool* parked) {
+  Link* lk = p.lk;
+  *parked = false;
+  uint32_t credits[FLH_MAX_LANES];
+  wire_credits(lk, p.w, credits);
+  const uint64_t chunk = (uint64_t)g_par.chunk;
+  if (pr->wins.cap[0] < chunk) { FL_WARN("NET/FuseLink : staging window smaller than a chunk"); return ncclInternalError; }
+  const int nqps = g_par.split_on_qps ? g_par.qps : 1;
+  std::vector<int> qoff(nqps), qlen(nqps);
+  if (flh_qp_split(p.size, nqps, qoff.data(), qlen.data()) < 0) return ncclInternalError;
+  if ((p.w.flags & 1u) && p.q_next == 0 && p.q_done == 0) lk->epoch_bytes = 0;   // the receiver refreshed its lane decision: new credit epoch
+  int last_q = -1;
+  for (int q = 0; q < nqps; ++q) if (qlen[q] > 0) last_q = q;
+  for (; p.q_next < nqps; ++p.q_next, p.q_done = 0) {
+    const int q = p.q_next;
+    const uint64_t piece = (uint64_t)qlen[q];
+    while (p.q_done < piece) {
+      if (!wire_set_free(pair)) { *parked = true; return ncclSuccess; }
+      uint64_t wave = (uint64_t)wave_chunks(credits, g_par.lanes, chunk, pr->wins.cap[0], lk->epoch_bytes / chunk) * chunk;
+      if (wave > piece - p.q_done) wave = piece - p.q_done;
+      const bool last = q == last_q && p.q_done + wave == piece;
+      const uint64_t seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;
+      pr->launch_seq.store(seq, std::memory_order_release);
+      uint64_t wave_no;
+      const uint32_t set = wire_next_set(pair, &wave_no);
+      flh_uniform_params u;
+      fill_uniform(u, credits, wave, (uint64_t)qoff[q] + p.q_done, lk->epoch_bytes, launch_tile(wave));
+      start_stamp(pr, seq, u);
+      Completion comp;
+      ncclResult_t rc = prepare_completion(pr, seq, wave, u, comp);   // the carrying launch is the last of the path on this side
+      if (rc != ncclSuccess) return rc;
+      FL_FLHCHECK(flh_stripe_uniform_carry(p.src, (uint64_t)p.size, &pr->wins, &pair->landing_wins[set], &u, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+      rc = finish_completion(pr, seq, comp);
+      if (rc != ncclSuccess) return rc;
+      WireFlight f;
+      f.engine = false;
+      f.seq = seq;
+      f.rec.set = set;
+      f.rec.n_req = 1;
+      f.rec.n_seg = 1;
+      f.rec.piece = 1;
+      f.rec.offset = (uint64_t)qoff[q] + p.q_done;
+      f.rec.last = last ? 1u : 0u;
+      f.rec.total_bytes = wave;
+      f.rec.req[0] = WaveReq{lk->wire->pair_conn, p.imm, p.fifo_idx, wave};
+      f.rec.seg[0] = WaveSeg{lk->epoch_bytes, 1, 0};
+      wire_push_flight(pair, f);
+      const uint32_t rows = (uint32_t)((wave + chunk - 1) / chunk);
+      pr->last.seq = seq;
+      pr->last.engine = false;
+      pr->last.n_seg = 1;
+      pr->last.n_rows = rows;
+      note_segment(pr, 0, lk, 0, rows, 1, lk->epoch_bytes, nullptr);
+      lk->last_seq = seq;
+      lk->last_engine = false;
+      lk->last_first_row = 0;
+      lk->last_rows = rows;
+      lk->epoch_bytes += wave;
+      lk->launches++;
+      p.q_done += wave;
+      p.sreq->seq = seq;
+      p.sreq->engine = false;
+      p.sreq->wave = wave_no;
+    }
+  }
+  return ncclSuccess;
+}
+
 // Does the send have to travel on its own, wave by wave?  Yes if it is split over QPs or if the staging windows
 // cannot hold it in one wave from where its connection stands in its credit epoch.
 bool needs_waves(const flh_windows& wins, const Pending& p, uint64_t epoch_bytes) {
@@ -1142,9 +1269,11 @@ size_t build_batch(Peer* pr, size_t i, BatchBuild& bb, bool engine) {
   FlCreditRow row;                           // its credit row
   uint32_t chunks_closed = 0;
   size_t j = i;
+  WirePair* const pair = work[i].lk->wire ? work[i].lk->wire->pair : nullptr;   // a batch stays on one wire: this process, or one pair
   while (j < work.size() && b.n_req < (uint32_t)g_par.batch) {
     const Pending& p = work[j];
-    if (!(p.src_dev && p.dst_dev)) break;
+    if (!(p.src_dev && p.dst_dev) || p.size == 0) break;
+    if ((p.lk->wire ? p.lk->wire->pair : nullptr) != pair) break;
     // where the request's connection stands in its epoch: behind its earlier segments of this batch, if any
     uint64_t epoch = p.lk->epoch_bytes;
     for (uint32_t k = 0; k < b.n_seg; ++k) if (bb.seg_link[k] == p.lk) epoch = bb.link_epoch_after[k];
@@ -1221,6 +1350,11 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
   b.u.tile_bytes = launch_tile(b.u.total_bytes);
   uint64_t seg_base[FLH_SEG_MAX][FLH_MAX_LANES];
   if (!engine) FL_FLHCHECK(flh_batch_layout(&b, nullptr, &seg_base[0][0]));
+  // a receiver in another process: the batch is a wave of the pair's wire and lands in one of its sets (the caller has
+  // made sure that one is free)
+  WirePair* const pair = pr->work[i].lk->wire ? pr->work[i].lk->wire->pair : nullptr;
+  uint64_t wave_no = 0;
+  const uint32_t set = pair ? wire_next_set(pair, &wave_no) : 0;
   if (engine) {
     // batch number k (from 1) takes window set (k - 1) mod sets and slot (k - 1) % kEngineSlots of the tables; the engine
     // lets it in once batch k - sets, the last to use that window set, is complete
@@ -1230,8 +1364,10 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     uint64_t got = 0;
     const uint64_t starts_before = g_par.trace ? flh_engine_launches(pr->engine) : 0;
     const int64_t t_sub = g_par.trace ? tr_now() : 0;
-    const int frc = flh_engine_submit(pr->engine, &b, &pr->ewins[k % (uint64_t)pr->engine_sets], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot, pr->d_status, &got,
-                                      &seg_base[0][0]);
+    const flh_windows* ewin = &pr->ewins[k % (uint64_t)pr->engine_sets];
+    const int frc = pair ? flh_engine_submit_wire(pr->engine, FLH_ENGINE_SEND, &b, ewin, &pair->landing_wins[set], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot,
+                                                  pr->d_status, &got, &seg_base[0][0])
+                         : flh_engine_submit(pr->engine, &b, ewin, pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot, pr->d_status, &got, &seg_base[0][0]);
     if (g_par.trace) {   // submits that had to start the resident kernel are counted apart: they pay for a launch
       const int which = flh_engine_launches(pr->engine) != starts_before ? kTrEngineStart : kTrEngineSubmit;
       tr_add(which, 1, tr_now() - t_sub);
@@ -1245,6 +1381,14 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     seq = got;
     pr->engine_reqs_upto[got % kEngineSlots].store(pr->engine_reqs_upto[(got - 1) % kEngineSlots].load(std::memory_order_relaxed) + b.n_req, std::memory_order_relaxed);
     pr->engine_submitted.store(got, std::memory_order_release);
+  } else if (pair) {
+    start_stamp(pr, seq, b.u);
+    Completion comp;
+    ncclResult_t rc = prepare_completion(pr, seq, b.u.total_bytes, b.u, comp);   // the carrying launch is the last of the path on this side
+    if (rc != ncclSuccess) return rc;
+    FL_FLHCHECK(flh_stripe_batch_carry(&b, &pr->wins, &pair->landing_wins[set], pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+    rc = finish_completion(pr, seq, comp);
+    if (rc != ncclSuccess) return rc;
   } else {
     start_stamp(pr, seq, b.u);
     FL_FLHCHECK(flh_stripe_batch(&b, &pr->wins, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
@@ -1254,6 +1398,23 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     FL_FLHCHECK(flh_reassemble_batch(&b, &pr->wins, pr->d_status, pr->stream));
     rc = finish_completion(pr, seq, comp);
     if (rc != ncclSuccess) return rc;
+  }
+  if (pair) {
+    // the wave's record: which receives it answers, each connection's run as one message from its epoch prefix on
+    WireFlight f;
+    f.engine = engine;
+    f.seq = seq;
+    f.rec.set = set;
+    f.rec.n_req = b.n_req;
+    f.rec.n_seg = b.n_seg;
+    f.rec.total_bytes = b.u.total_bytes;
+    for (uint32_t q = 0; q < b.n_req; ++q) {
+      const Pending& p = pr->work[i + q];
+      f.rec.req[q] = WaveReq{p.lk->wire->pair_conn, p.imm, p.fifo_idx, (uint64_t)p.size};
+      p.sreq->wave = wave_no;
+    }
+    for (uint32_t k = 0; k < b.n_seg; ++k) f.rec.seg[k] = WaveSeg{b.seg[k].epoch_bytes, b.seg[k].n_req, 0};
+    wire_push_flight(pair, f);
   }
   // bookkeeping: every connection's place in its epoch, what the launch carried
   const uint64_t chunk = (uint64_t)g_par.chunk;
@@ -1281,7 +1442,9 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
 }
 
 // Launch everything that waits on the peer, in order (launch_mu held).  A failure completes the requests it
-// touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).
+// touches with an error, as a queue pair in the error state would (plugin.cc:1839-1861).  Sends to another process
+// need a free set of their pair's landing windows; where there is none they, and whatever waits behind them for the
+// same pair, go back to the front of the queue.
 void flush_pending(Peer* pr) {
   {
     std::lock_guard<ShortLock> g(pr->queue_mu);
@@ -1313,16 +1476,36 @@ void flush_pending(Peer* pr) {
   }
   if (g_par.trace) tr_add(kTrRequestsLaunched, (int64_t)work.size(), 0);
   tl_event(3, (uint64_t)work.size());
+  std::vector<Pending>& parked = pr->work_sorted;   // (free again) what found no landing set, in order
+  parked.clear();
+  for (const Pending& q : work) if (q.lk->wire && q.lk->wire->pair) q.lk->wire->pair->blocked = false;
   size_t i = 0;
   while (i < work.size()) {
     ncclResult_t rc = ncclSuccess;
     size_t span = 1;
-    const Pending& p = work[i];
+    Pending& p = work[i];
+    WirePair* const pair = p.lk->wire ? p.lk->wire->pair : nullptr;
+    if (pair) {
+      if (pair->w->failed.load(std::memory_order_acquire) || p.lk->wire->w->recv_closed.load(std::memory_order_acquire)) {
+        if (!p.lk->wire->w->recv_closed.load(std::memory_order_acquire)) FL_WARN("NET/FuseLink : a wave to the receiving process was lost: the send fails");
+        else FL_WARN("NET/FuseLink : the receiving process closed the connection with a send outstanding");
+        p.sreq->fault = 1;
+        p.sreq->state.store(kStDoneHost, std::memory_order_release);
+        ++i;
+        continue;
+      }
+      if (pair->blocked || !wire_set_free(pair)) {   // no landing set: it keeps its place, and so does what follows it on this wire
+        pair->blocked = true;
+        parked.push_back(p);
+        ++i;
+        continue;
+      }
+    }
     const uint64_t p_epoch = (p.w.flags & 1u) ? 0 : p.lk->epoch_bytes;
     // small requests in device memory go to the engine, batch by batch: no launch, and a number of the engine's own
-    bool by_engine = false;
+    bool by_engine = false, wave_by_wave = false;
     uint64_t seq = 0;
-    if (rc == ncclSuccess && g_par.batch >= 2 && engine_takes(pr, p, p_epoch)) {
+    if (rc == ncclSuccess && p.size && g_par.batch >= 2 && p.q_next == 0 && p.q_done == 0 && engine_takes(pr, p, p_epoch)) {
       BatchBuild bb;
       const size_t n = build_batch(pr, i, bb, true);
       if (n) {
@@ -1334,27 +1517,59 @@ void flush_pending(Peer* pr) {
     }
     if (!by_engine) {
       if (rc == ncclSuccess && !dev.use()) rc = ncclUnhandledCudaError;   // launches need the staging device current
-      seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
-      pr->launch_seq.store(seq, std::memory_order_release);   // before anything runs: the completion words never run ahead of it
+      if (!pair) {   // (waves to another process take their numbers where they are launched: a send may be several)
+        seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;   // this launch's number
+        pr->launch_seq.store(seq, std::memory_order_release);   // before anything runs: the completion words never run ahead of it
+      }
     }
     if (rc == ncclSuccess && !by_engine) {
-      if (!(p.src_dev && p.dst_dev)) {
+      if (pair && p.size == 0) {
+        // a send of no bytes to another process: a wave with nothing to land, announced in its turn
+        uint64_t wave_no;
+        WireFlight f;
+        f.rec.set = wire_next_set(pair, &wave_no);
+        f.rec.n_req = 1;
+        f.rec.n_seg = 1;
+        f.rec.req[0] = WaveReq{p.lk->wire->pair_conn, p.imm, p.fifo_idx, 0};
+        f.rec.seg[0] = WaveSeg{p_epoch, 1, 0};
+        wire_push_flight(pair, f);
+        p.sreq->wave = wave_no;
+        p.sreq->state.store(kStDoneHost, std::memory_order_release);
+        ++i;
+        continue;
+      } else if (!(p.src_dev && p.dst_dev)) {
         // one side is host memory: the copy engine is the wire, nothing is striped
         hipEvent_t ev = nullptr;
         rc = launch_event(pr, seq, &ev);
         hipError_t e = rc == ncclSuccess ? hipMemcpyAsync(p.dst, p.src, (size_t)p.size, hipMemcpyDefault, pr->stream) : hipSuccess;
         if (e != hipSuccess) rc = hip_fail("hipMemcpyAsync", e);
         if (rc == ncclSuccess) { Completion c; c.ev = ev; rc = finish_completion(pr, seq, c); }
-      } else if (g_par.batch < 2 || needs_waves(pr->wins, p, p_epoch)) {
-        rc = launch_transfer(pr, p, seq);
+      } else if (g_par.batch < 2 || p.q_next || p.q_done || needs_waves(pr->wins, p, p_epoch)) {
+        wave_by_wave = true;
       } else {
         BatchBuild bb;
         span = build_batch(pr, i, bb, false);
         TraceScope trl(kTrLaunch);
         // a request on its own takes the single-message kernels: they carry no per-request search and a tenth of the
         // batch kernels' arguments, which is worth a microsecond per kernel on a 64 MiB request
-        if (span <= 1) { span = 1; rc = launch_transfer(pr, p, seq); }
-        else rc = launch_batch(pr, i, span, bb, false, seq);
+        if (span <= 1) { span = 1; wave_by_wave = true; }
+        else {
+          if (pair) { seq = pr->launch_seq.load(std::memory_order_relaxed) + 1; pr->launch_seq.store(seq, std::memory_order_release); }
+          rc = launch_batch(pr, i, span, bb, false, seq);
+        }
+      }
+      if (wave_by_wave && pair) {
+        bool park = false;
+        rc = launch_transfer_wire(pr, p, pair, &park);   // numbers its launches itself, one per wave
+        seq = p.sreq->seq;
+        if (rc == ncclSuccess && park) {   // part of it is on its way; the rest waits for a landing set, in front
+          pair->blocked = true;
+          parked.push_back(p);
+          ++i;
+          continue;
+        }
+      } else if (wave_by_wave) {
+        rc = launch_transfer(pr, p, seq);
       }
     }
     tl_event(4, ((uint64_t)span << 32) | (by_engine ? 0x80000000ull : 0) | (seq & 0x7fffffffull));
@@ -1362,48 +1577,63 @@ void flush_pending(Peer* pr) {
       Pending& q = work[k];
       if (rc == ncclSuccess) {
         q.sreq->seq = seq;
-        q.rreq->seq = seq;
         q.sreq->engine = by_engine;
-        q.rreq->engine = by_engine;
         q.sreq->state.store(kStLaunched, std::memory_order_release);
-        q.rreq->state.store(kStLaunched, std::memory_order_release);
+        if (q.rreq) {
+          q.rreq->seq = seq;
+          q.rreq->engine = by_engine;
+          q.rreq->state.store(kStLaunched, std::memory_order_release);
+        }
       } else {
         q.sreq->fault = 1;
-        q.rreq->fault = 1;
         q.sreq->state.store(kStDoneHost, std::memory_order_release);
-        q.rreq->state.store(kStDoneHost, std::memory_order_release);
+        if (q.rreq) {
+          q.rreq->fault = 1;
+          q.rreq->state.store(kStDoneHost, std::memory_order_release);
+        }
+        if (pair) pair->w->failed.store(1, std::memory_order_release);   // (its wave, if one was numbered, will never land)
       }
     }
     if (rc != ncclSuccess && !by_engine) {
       // whatever part of the launch was queued is waited for here, so that its number counts as complete and the
       // launches behind it are not held back by one that will never report
       if (dev.use()) (void)hipStreamSynchronize(pr->stream);
+      const uint64_t top = pr->launch_seq.load(std::memory_order_relaxed);
       uint64_t seen = pr->done_seq.load(std::memory_order_relaxed);
-      while (seen < seq && !pr->done_seq.compare_exchange_weak(seen, seq, std::memory_order_release, std::memory_order_relaxed)) {}
+      while (seen < top && !pr->done_seq.compare_exchange_weak(seen, top, std::memory_order_release, std::memory_order_relaxed)) {}
     }
     i += span;
   }
   work.clear();
+  if (!parked.empty()) {
+    std::lock_guard<ShortLock> g(pr->queue_mu);
+    uint64_t bytes = 0;
+    for (const Pending& q : parked) bytes += (uint64_t)q.size;
+    pr->pending.insert(pr->pending.begin(), parked.begin(), parked.end());
+    pr->waiting_reqs.store(pr->waiting_reqs.load(std::memory_order_relaxed) + (uint32_t)parked.size(), std::memory_order_release);
+    pr->waiting_bytes.store(pr->waiting_bytes.load(std::memory_order_relaxed) + bytes, std::memory_order_release);
+    parked.clear();
+  }
 }
 
 ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhandle, void** request) {
   if (!sendComm || !request || !mhandle || size < 0 || (size && !data)) return ncclInvalidArgument;
   Comm* c = (Comm*)sendComm;
   MemHandle* mh = (MemHandle*)mhandle;
-  if (c->magic == kShmCommMagic && mh->magic == kMhMagic && ((ShmComm*)sendComm)->is_send) {
-    if (!request || size < 0 || (!data && size > 0)) return ncclInvalidArgument;
-    return shm_isend((ShmComm*)sendComm, data, size, tag, mh, request);
-  }
   if (c->magic != kCommMagic || !c->is_send || mh->magic != kMhMagic) return ncclInvalidArgument;
   Link* lk = c->link;
+  WireEnd* const wire = lk->wire;   // non-null: the receiver is another process
   *request = nullptr;
   TraceScope tr(kTrIsend);
+  if (wire && mh->type != NCCL_PTR_CUDA) { FL_WARN("NET/FuseLink : the shared-memory wire carries device memory only"); return ncclInvalidUsage; }
   // The connection's lock covers the descriptor match and the bookkeeping only.  The GPU work is queued
   // after it is dropped: one thread drives a send comm (as NCCL's proxy does), so launches on the
   // connection's stream stay in request order, and the receiver's polling never waits behind a launch.
   FifoWire w;
   Request *sreq = nullptr, *rreq = nullptr;
   int rtype = 0;
+  uint32_t imm = 0xffffffffu;
+  uint64_t fifo_idx = 0;
   ncclResult_t rc = ncclSuccess;
   {
     std::lock_guard<ShortLock> g(lk->mu);
@@ -1411,38 +1641,62 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     // wait for the receiver to have posted the matching receive (plugin.cc:1510-1514)
     const int slot = (int)(lk->fifoHead % FL_NET_MAX_REQUESTS);
     FifoSlot& fs = lk->fifo[slot];
-    if (fs.w.idx != lk->fifoHead + 1) return ncclSuccess;
-    if (fs.w.nreqs != 1) { FL_WARN("NET/FuseLink: multi-send not allowed"); return ncclInternalError; }   // plugin.cc:1448-1451
-    if (fs.w.tag != (uint32_t)tag) return ncclSuccess;                                                     // plugin.cc:1552
-    if (size > fs.w.size) {                                                                                // plugin.cc:1555-1562
-      FL_WARN("NET/FuseLink : req tag %x collective mismatch error, local size %d remote size %d", tag, size, fs.w.size);
+    // the descriptor: in this process's ring, or in the shared-memory object the receiving process writes (idx last)
+    FifoWire* const fw = wire ? &wire->w->fifo[slot] : &fs.w;
+    if (__atomic_load_n(&fw->idx, __ATOMIC_ACQUIRE) != lk->fifoHead + 1) {
+      if (wire && wire->w->recv_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the receiving process has closed the connection"); return ncclRemoteError; }
+      return ncclSuccess;
+    }
+    w = *fw;
+    if (w.nreqs != 1) { FL_WARN("NET/FuseLink: multi-send not allowed"); return ncclInternalError; }   // plugin.cc:1448-1451
+    if (w.tag != (uint32_t)tag) return ncclSuccess;                                                     // plugin.cc:1552
+    if (size > w.size) {                                                                                // plugin.cc:1555-1562
+      FL_WARN("NET/FuseLink : req tag %x collective mismatch error, local size %d remote size %d", tag, size, w.size);
       return ncclInvalidUsage;
     }
-    if (fs.w.size < 0 || fs.w.addr == 0) {                                                                 // plugin.cc:1563-1570
-      FL_WARN("NET/FuseLink : posted incorrect receive info: size %d addr %llx", fs.w.size, (unsigned long long)fs.w.addr);
+    if (w.size < 0 || w.addr == 0) {                                                                 // plugin.cc:1563-1570
+      FL_WARN("NET/FuseLink : posted incorrect receive info: size %d addr %llx", w.size, (unsigned long long)w.addr);
       return ncclInternalError;
     }
     if (size && !in_handle(mh, data, (size_t)size)) { FL_WARN("NET/FuseLink : send buffer outside its registration"); return ncclInvalidArgument; }
+    if (wire) {   // the receiver's landing windows, once it has set them up
+      bool ready = false;
+      rc = wire_send_setup(lk, mh->device, &ready);
+      if (rc != ncclSuccess || !ready) return rc;
+    }
     sreq = get_request(lk->sreq, lk, kReqSend);
     if (!sreq) return ncclInternalError;                                                                   // plugin.cc:1082-1084
-    rreq = fs.rreq;
-    rtype = fs.rtype;
-    w = fs.w;
+    if (!wire) {
+      rreq = fs.rreq;
+      rtype = fs.rtype;
+    } else {
+      rtype = NCCL_PTR_CUDA;
+    }
     sreq->size = size;
-    rreq->size = size;
+    if (rreq) rreq->size = size;
     const bool any_dev = mh->type == NCCL_PTR_CUDA || rtype == NCCL_PTR_CUDA;
-    if (size && any_dev) rc = attach_peer(lk, mh->type == NCCL_PTR_CUDA ? mh->device : fs.rdevice);
+    if (size && any_dev && !wire) rc = attach_peer(lk, mh->type == NCCL_PTR_CUDA ? mh->device : fs.rdevice);
     if (rc != ncclSuccess) { sreq->type = kReqUnused; return rc; }   // nothing consumed: the descriptor stays posted
-    memset((void*)&fs.w, 0, sizeof(FifoWire));   // plugin.cc:1605
-    fs.rreq = nullptr;
+    imm = sender_mask(lk);                        // plugin.cc:1441-1447
+    if (rreq) rreq->imm = imm;                    // (the immediate data of the write that completes the receive, plugin.cc:1463)
+    fifo_idx = lk->fifoHead + 1;
+    if (wire) {
+      // plugin.cc:1605; the index goes last: once it reads 0 the slot is the receiver's again, and it writes all of it
+      memset((void*)fw, 0, offsetof(FifoWire, idx));
+      memset((char*)fw + offsetof(FifoWire, idx) + sizeof(uint64_t), 0, sizeof(FifoWire) - offsetof(FifoWire, idx) - sizeof(uint64_t));
+      __atomic_store_n(&fw->idx, (uint64_t)0, __ATOMIC_RELEASE);
+    } else {
+      memset((void*)&fs.w, 0, sizeof(FifoWire));   // plugin.cc:1605
+      fs.rreq = nullptr;
+    }
     lk->fifoHead++;                              // plugin.cc:1607
     lk->s_inflight++;
   }
-  uint8_t* dst = (uint8_t*)(uintptr_t)w.addr;
+  uint8_t* dst = wire ? nullptr : (uint8_t*)(uintptr_t)w.addr;
   const bool src_dev = mh->type == NCCL_PTR_CUDA, dst_dev = rtype == NCCL_PTR_CUDA;
   // the comm's own NIC carried traffic (updateTxChannelActive, fuselink.h:247-252)
   mark_nic_active(lk->dev % g_par.lanes, 1);
-  if (size == 0 || (!src_dev && !dst_dev)) {
+  if (!wire && (size == 0 || (!src_dev && !dst_dev))) {
     // host memory is not staged (fuselink.cc:8-13): the wire is a copy
     if (size) memcpy(dst, data, (size_t)size);
     sreq->state.store(kStDoneHost, std::memory_order_release);
@@ -1460,8 +1714,10 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     p.w = w;
     p.sreq = sreq;
     p.rreq = rreq;
+    p.imm = imm;
+    p.fifo_idx = fifo_idx;
     sreq->state.store(kStQueued, std::memory_order_release);
-    rreq->state.store(kStQueued, std::memory_order_release);
+    if (rreq) rreq->state.store(kStQueued, std::memory_order_release);
     tl_event(2, (uint64_t)lk->channelId);
     uint32_t waiting;
     {
@@ -1491,18 +1747,25 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
 ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags, void** mhandles, void** request) {
   if (!recvComm || !request || !data || !sizes || !tags || !mhandles) return ncclInvalidArgument;
   Comm* c = (Comm*)recvComm;
-  const bool shm = c->magic == kShmCommMagic;
-  if ((c->magic != kCommMagic && !shm) || c->is_send) return ncclInvalidArgument;
+  if (c->magic != kCommMagic || c->is_send) return ncclInvalidArgument;
   *request = nullptr;
   if (n > FL_NET_MAX_RECVS) return ncclInternalError;                       // plugin.cc:1683
   if (n != 1) { FL_WARN("NET/FuseLink: multi recv not allowed"); return ncclInternalError; }  // plugin.cc:1873-1880
   MemHandle* mh = (MemHandle*)mhandles[0];
   if (!mh || mh->magic != kMhMagic || sizes[0] < 0 || !data[0]) return ncclInvalidArgument;
   if (sizes[0] && !in_handle(mh, data[0], (size_t)sizes[0])) { FL_WARN("NET/FuseLink : receive buffer outside its registration"); return ncclInvalidArgument; }
-  if (shm) return shm_irecv((ShmComm*)recvComm, data[0], sizes[0], tags[0], mh, request);
   Link* lk = c->link;
+  WireEnd* const wire = lk->wire;   // non-null: the sender is another process
+  if (wire && mh->type != NCCL_PTR_CUDA) { FL_WARN("NET/FuseLink : the shared-memory wire carries device memory only"); return ncclInvalidUsage; }
   TraceScope tr(kTrIrecv);
+  if (wire && wire->pair) (void)wire_progress_recv(wire->pair);   // landing sets whose waves have been delivered go back
   std::lock_guard<ShortLock> g(lk->mu);
+  if (wire) {
+    ncclResult_t rc = wire_recv_setup(lk, mh->device);
+    if (rc != ncclSuccess) return rc;
+  }
+  const int slot = (int)(lk->fifoTail % FL_NET_MAX_REQUESTS);
+  FifoSlot& fs = lk->fifo[slot];
   bool refreshed = false;
   if (lk->r_finished % g_par.refresh_batch == 0 || !lk->have_decision) {   // plugin.cc:1700
     // only when everything received so far has been consumed (plugin.cc:1704-1709)
@@ -1511,7 +1774,7 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
       lk->fuselink_offset = lk->channelId % g_par.lanes;                     // refreshRxComm, fuselink.h:235-237
     } else {
       lk->fuselink_offset = -2;
-      current_credits(lk->dev % g_par.lanes, lk->credits);
+      current_credits(lk->dev % g_par.lanes, lk->tx_available, wire == nullptr, lk->credits);   // plugin.cc:1710
     }
     lk->have_decision = true;
     lk->refreshes++;
@@ -1519,11 +1782,14 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
   }
   Request* rreq = get_request(lk->rreq, lk, kReqRecv);
   if (!rreq) return ncclInternalError;                                         // plugin.cc:1082-1084
-  if (lk->fifoTail - lk->fifoHead >= FL_NET_MAX_REQUESTS) { rreq->type = kReqUnused; return ncclSuccess; }  // descriptor ring full
+  // descriptor ring full: in this process the head says so; across processes the sender clears a slot when it matches
+  // it (plugin.cc:1605), and this side's note of the slot goes when its wave has been delivered
+  if (wire ? (fs.rreq || __atomic_load_n(&wire->w->fifo[slot].idx, __ATOMIC_ACQUIRE) != 0) : lk->fifoTail - lk->fifoHead >= FL_NET_MAX_REQUESTS) {
+    rreq->type = kReqUnused;
+    return ncclSuccess;
+  }
   rreq->state.store(kStPosted, std::memory_order_relaxed);
   // ncclIbPostFifo, plugin.cc:1616-1677
-  const int slot = (int)(lk->fifoTail % FL_NET_MAX_REQUESTS);
-  FifoSlot& fs = lk->fifo[slot];
   fs.w.addr = (uint64_t)(uintptr_t)data[0];
   fs.w.size = sizes[0];
   fs.w.rkey = 1;
@@ -1536,7 +1802,17 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
   fs.rtype = mh->type;
   fs.rdevice = mh->device;
   tl_event(1, (uint64_t)lk->channelId);
-  fs.w.idx = lk->fifoTail + 1;   // written last: it is what the sender waits for (plugin.cc:1632)
+  if (wire) {
+    // this side keeps its note of the slot (the receive it belongs to, the credit row it asked for); the descriptor
+    // itself goes into the sender's view, its index last
+    FifoWire& out = wire->w->fifo[slot];
+    fs.w.idx = 0;
+    out = fs.w;
+    fs.w.idx = lk->fifoTail + 1;
+    __atomic_store_n(&out.idx, lk->fifoTail + 1, __ATOMIC_RELEASE);   // what the sender waits for (plugin.cc:1632)
+  } else {
+    fs.w.idx = lk->fifoTail + 1;   // written last: it is what the sender waits for (plugin.cc:1632)
+  }
   lk->fifoTail++;
   lk->r_inflight++;
   *request = rreq;
@@ -1639,17 +1915,180 @@ uint64_t launches_in_queue(Peer* pr) {
   return top > done ? top - done : 0;
 }
 
+// Is the wave's GPU work through?  (*rc: the engine that held it went down, or the runtime failed.)
+bool wire_flight_complete(Peer* pr, const WireFlight& f, ncclResult_t* rc) {
+  *rc = ncclSuccess;
+  if (f.seq == 0) return true;
+  if (f.engine) {
+    if (flh_engine_completed(pr->engine) >= f.seq) return true;
+    if (flh_engine_error(pr->engine) == 0) return false;
+    *rc = ncclRemoteError;
+    return true;
+  }
+  bool complete = false;
+  *rc = launch_complete(pr, f.seq, &complete);
+  return complete || *rc != ncclSuccess;
+}
+
+// One announced wave (rx_mu and the staging side's launch_mu held): the receives it answers, the same batch the sender
+// built -- each connection's run as one message from its epoch prefix on, under the credit row this side put into the
+// descriptors -- handed to this process's engine or launched, out of the landing set the wave lies in.
+ncclResult_t wire_deliver(WirePair* p, const ShmWave& wv, WireFlight& f) {
+  Peer* pr = p->peer;
+  const uint32_t n_req = wv.n_req, n_seg = wv.n_seg;
+  if (n_req < 1 || n_req > FLH_BATCH_MAX || n_seg < 1 || n_seg > FLH_SEG_MAX || wv.set >= (uint32_t)p->sets || (wv.piece && n_req != 1)) {
+    FL_WARN("NET/FuseLink : a wave record that makes no sense (%u requests, %u segments, set %u)", n_req, n_seg, wv.set);
+    return ncclInternalError;
+  }
+  flh_batch_params b;
+  memset(&b, 0, sizeof(b));
+  b.u.chunk_bytes = (uint32_t)g_par.chunk;
+  b.u.n_lanes = (uint32_t)g_par.lanes;
+  b.u.tile_bytes = FLH_TILE_BYTES;
+  b.n_req = n_req;
+  b.n_seg = n_seg;
+  Request* reqs[FLH_BATCH_MAX];
+  Link* links[FLH_BATCH_MAX];
+  uint32_t q = 0;
+  uint64_t sum = 0;
+  bool small = true;
+  for (uint32_t k = 0; k < n_seg; ++k) {
+    const uint32_t nq = wv.seg[k].n_req;
+    if (nq == 0 || q + nq > n_req) { FL_WARN("NET/FuseLink : a wave whose segments do not add up to its requests"); return ncclInternalError; }
+    b.seg[k].epoch_bytes = wv.seg[k].epoch_bytes;
+    b.seg[k].n_req = nq;
+    for (uint32_t i = 0; i < nq; ++i, ++q) {
+      const WaveReq& wr = wv.req[q];
+      Link* lk = wr.conn < kPairConns ? p->conns[wr.conn].load(std::memory_order_acquire) : nullptr;
+      if (!lk) { FL_WARN("NET/FuseLink : a wave for connection %u, which this process does not have", wr.conn); return ncclInternalError; }
+      std::lock_guard<ShortLock> g(lk->mu);
+      FifoSlot& fs = lk->fifo[(wr.fifo_idx - 1) % FL_NET_MAX_REQUESTS];
+      if (!fs.rreq || fs.w.idx != wr.fifo_idx) { FL_WARN("NET/FuseLink : a wave of request %llu arrived, which no posted receive is waiting for", (unsigned long long)wr.fifo_idx); return ncclInternalError; }
+      const uint64_t at = wv.piece ? wv.offset : 0;
+      if (at + wr.bytes > (uint64_t)fs.w.size) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
+      uint32_t credits[FLH_MAX_LANES];
+      wire_credits(lk, fs.w, credits);
+      if (i == 0) memcpy(b.seg[k].credits, credits, sizeof(credits));
+      else if (links[q - 1] != lk || memcmp(b.seg[k].credits, credits, sizeof(credits)) != 0) {
+        FL_WARN("NET/FuseLink : request %u of a wave does not belong to its segment's connection and credit row", q);
+        return ncclInvalidUsage;
+      }
+      reqs[q] = fs.rreq;
+      links[q] = lk;
+      b.d_dst[q] = (void*)(uintptr_t)fs.w.addr;
+      b.bytes[q] = wr.bytes;
+      sum += wr.bytes;
+      if ((int64_t)wr.bytes > g_par.engine_max_request) small = false;
+      fs.rreq->size += (int)wr.bytes;
+      fs.rreq->imm = wr.imm;
+      if (!wv.piece || wv.last) { fs.rreq = nullptr; fs.w.idx = 0; }   // the slot's note goes: it may be posted again
+    }
+  }
+  if (q != n_req || sum != wv.total_bytes) { FL_WARN("NET/FuseLink : a wave's requests do not add up to its bytes"); return ncclInvalidUsage; }
+  b.u.total_bytes = sum;
+  const flh_windows* landing = &p->landing_wins[wv.set];
+  const uint64_t chunk = (uint64_t)g_par.chunk;
+  bool by_engine = false;
+  uint64_t seq = 0;
+  ncclResult_t rc = ncclSuccess;
+  if (sum == 0) {
+    // a send of no bytes: nothing to deliver
+  } else {
+    uint64_t rows = 0;
+    for (uint32_t i = 0; i < n_req; ++i) rows += (b.bytes[i] + chunk - 1) / chunk;
+    if (!wv.piece && small && rows <= kEngineRows && pr->engine_ok.load(std::memory_order_acquire)) {
+      uint64_t got = 0;
+      const int frc = flh_engine_submit_wire(pr->engine, FLH_ENGINE_RECV, &b, landing, nullptr, nullptr, nullptr, pr->d_status, &got, nullptr);
+      if (frc == FLH_OK) {
+        by_engine = true;
+        seq = got;
+        pr->engine_reqs_upto[got % kEngineSlots].store(pr->engine_reqs_upto[(got - 1) % kEngineSlots].load(std::memory_order_relaxed) + n_req, std::memory_order_relaxed);
+        pr->engine_submitted.store(got, std::memory_order_release);
+      } else if (frc != FLH_E_NOMEM) {
+        FL_WARN("NET/FuseLink : engine: %s", flh_last_error());
+        pr->engine_ok.store(false, std::memory_order_release);
+      }
+    }
+    if (!by_engine) {
+      DeviceScope keep;
+      hipError_t he = hipSetDevice(pr->hip_device);
+      if (he != hipSuccess) rc = hip_fail("hipSetDevice", he);
+      seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;
+      pr->launch_seq.store(seq, std::memory_order_release);
+      Completion comp;
+      if (rc == ncclSuccess) {
+        if (n_req == 1) {
+          // one request (or a piece of one): the single-message kernel, under the credit row of its descriptor
+          flh_uniform_params u;
+          fill_uniform(u, b.seg[0].credits, sum, wv.piece ? wv.offset : 0, b.seg[0].epoch_bytes, launch_tile(sum));
+          start_stamp(pr, seq, u);
+          rc = prepare_completion(pr, seq, sum, u, comp);
+          const uint64_t posted = (uint64_t)(wv.piece ? wv.offset : 0) + sum;   // (checked against the posted size above)
+          if (rc == ncclSuccess && flh_reassemble_uniform(b.d_dst[0], posted, landing, &u, pr->d_status, pr->stream) < 0) { FL_WARN("NET/FuseLink : %s", flh_last_error()); rc = ncclUnhandledCudaError; }
+        } else {
+          b.u.tile_bytes = launch_tile(sum);
+          start_stamp(pr, seq, b.u);
+          rc = prepare_completion(pr, seq, sum, b.u, comp);
+          if (rc == ncclSuccess && flh_reassemble_batch(&b, landing, pr->d_status, pr->stream) < 0) { FL_WARN("NET/FuseLink : %s", flh_last_error()); rc = ncclUnhandledCudaError; }
+        }
+      }
+      if (rc == ncclSuccess) rc = finish_completion(pr, seq, comp);
+      if (rc != ncclSuccess) {
+        // whatever was queued is waited for, so that the number counts as complete and holds nothing back
+        (void)hipStreamSynchronize(pr->stream);
+        uint64_t seen = pr->done_seq.load(std::memory_order_relaxed);
+        while (seen < seq && !pr->done_seq.compare_exchange_weak(seen, seq, std::memory_order_release, std::memory_order_relaxed)) {}
+      }
+    }
+  }
+  f.engine = by_engine;
+  f.seq = sum == 0 || rc != ncclSuccess ? 0 : seq;
+  if (wv.piece && !wv.last && rc == ncclSuccess) return ncclSuccess;   // the request's later pieces complete it
+  for (uint32_t i = 0; i < n_req; ++i) {
+    Request* r = reqs[i];
+    r->seq = seq;
+    r->engine = by_engine;
+    if (rc != ncclSuccess) r->fault = 1;
+    r->state.store(sum == 0 || rc != ncclSuccess ? kStDoneHost : kStLaunched, std::memory_order_release);
+  }
+  return rc;
+}
+
 ncclResult_t fl_test(void* request, int* done, int* sizes) {
   if (!request || !done) return ncclInvalidArgument;
-  if (*(const uint32_t*)request == kShmReqMagic) return shm_test((ShmRequest*)request, done, sizes);   // a Request starts with its small type code
   Request* r = (Request*)request;
   if (r->magic != kReqMagic || r->type == kReqUnused) { FL_WARN("NET/FuseLink : test on a request that is not in flight"); return ncclInternalError; }
   *done = 0;
   Link* lk = r->link;
   TraceScope tr(kTrTest);
+  WirePair* const pair = lk->wire ? lk->wire->pair : nullptr;   // non-null: the other end is another process
+  // The other end is another process: whoever polls a receive takes the waves that have been announced off the wire,
+  // whoever polls a send announces the waves that have landed -- also while its own request still waits for a landing
+  // set, which only comes back once the receiver has seen the waves before it.
+  if (pair && r->type == kReqRecv) (void)wire_progress_recv(pair);
+  if (pair && r->type == kReqSend) (void)wire_publish(pair);
   // the request is polled without the connection's lock: only the thread that drives this comm tests its requests
   int st = r->state.load(std::memory_order_acquire);
-  if (st == kStPosted || st == 0) return ncclSuccess;   // a receive whose send has not been matched yet
+  if (st == kStPosted || st == 0) {   // a receive whose send has not been matched yet
+    if (!lk->wire) return ncclSuccess;
+    // the sender is another process: has a wave been lost on the way, or has the sender gone?
+    const bool lost = pair && pair->w->failed.load(std::memory_order_acquire);
+    if (!lost) {
+      if (!lk->wire->w->send_closed.load(std::memory_order_acquire)) return ncclSuccess;
+      // (what it announced before it left is still delivered: look once more before giving up)
+      if (pair) (void)wire_progress_recv(pair);
+      st = r->state.load(std::memory_order_acquire);
+      if ((st == kStPosted || st == 0) && pair) {
+        const uint64_t taken = pair->rx_taken.load(std::memory_order_acquire);
+        if (pair->w->wave[taken % kPairWaves].seq.load(std::memory_order_acquire) == taken + 1) return ncclSuccess;   // an announced wave has yet to be taken off the wire
+      }
+    }
+    if (st == kStPosted || st == 0) {
+      FL_WARN("NET/FuseLink : %s", lost ? "a wave from the sending process was lost" : "the sending process closed the connection with a receive outstanding");
+      r->fault = 1;
+      st = kStDoneHost;
+    }
+  }
   Peer* pr = lk->peer.load(std::memory_order_acquire);
   // Matched sends wait so that those that arrive together -- on this connection and on the others that stage on
   // the same GPU -- can share a launch.  They go out when a test finds the GPU short of work: fewer than two
@@ -1710,51 +2149,78 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     ncclResult_t rc = launch_complete(pr, r->seq, &complete);
     if (rc != ncclSuccess || !complete) return rc;
   }
-  if (g_par.trace) tr_add(kTrTestDone, 1, 0);
-  tl_event(5, ((uint64_t)r->seq << 16) | (r->engine ? 0x8000u : 0u) | ((uint64_t)(lk->channelId & 0x3fff) << 1) | (r->type == kReqRecv ? 1u : 0u));
-  std::lock_guard<ShortLock> g(lk->mu);
-  ncclResult_t result = ncclSuccess;
-  if (r->fault) {
-    // Failed completion (plugin.cc:1839-1861).  The reference returns here with the request still allocated and its
-    // counters untouched: its communicator is dead from then on.  Here the connection lives on (an engine that went
-    // down hands its traffic to launches), so the request is freed and counted like any other: a request that stayed
-    // in flight would hold every later refresh back (r_inflight != 0 on a batch boundary) and leak its slot.
-    FL_WARN("NET/FuseLink : Got completion with error, channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
-    result = ncclRemoteError;
-  } else if (st == kStLaunched && pr && __atomic_load_n(pr->h_status, __ATOMIC_ACQUIRE) != 0) {
-    // A kernel refused a chunk that would have left its window or buffer (the host sizes every launch so that this
-    // cannot happen; the check is the safety net).  The first request completed after the refusal reports it, once,
-    // and is freed like any other; the word is cleared so that later traffic is not condemned with it.
-    const int32_t code = __atomic_exchange_n(pr->h_status, 0, __ATOMIC_ACQ_REL);
-    if (code != 0) {
-      FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", code);
-      result = ncclInternalError;
+  if (pair && r->type == kReqSend && !r->fault) {
+    // A send to another process is reported once its wave has been announced there (like an RDMA write, complete when
+    // the bytes are in the receiver's memory, plugin.cc:1453-1465): announce what has landed, in order.
+    ncclResult_t prc = wire_publish(pair);
+    if (prc != ncclSuccess || pair->w->failed.load(std::memory_order_acquire)) {
+      FL_WARN("NET/FuseLink : a wave to the receiving process was lost");
+      r->fault = 1;
+    } else if (pair->tx_published.load(std::memory_order_acquire) < r->wave) {
+      if (!lk->wire->w->recv_closed.load(std::memory_order_acquire)) return ncclSuccess;   // waves before it are still landing
+      FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding");
+      r->fault = 1;
     }
   }
-  *done = result == ncclSuccess ? 1 : 0;                    // plugin.cc:1807-1823
-  if (r->type == kReqSend) { lk->s_finished++; lk->s_inflight--; }
-  if (r->type == kReqRecv) {
-    mark_nic_active(lk->dev % g_par.lanes, 0);   // updateRxChannelActive, fuselink.h:254-259
-    lk->r_finished++;
-    lk->r_inflight--;
-    if (sizes) sizes[0] = r->size;   // the reference leaves 0 here (plugin.cc:1726, 1882)
+  if (g_par.trace) tr_add(kTrTestDone, 1, 0);
+  tl_event(5, ((uint64_t)r->seq << 16) | (r->engine ? 0x8000u : 0u) | ((uint64_t)(lk->channelId & 0x3fff) << 1) | (r->type == kReqRecv ? 1u : 0u));
+  ncclResult_t result = ncclSuccess;
+  {
+    std::lock_guard<ShortLock> g(lk->mu);
+    if (r->fault) {
+      // Failed completion (plugin.cc:1839-1861).  The reference returns here with the request still allocated and its
+      // counters untouched: its communicator is dead from then on.  Here the connection lives on (an engine that went
+      // down hands its traffic to launches), so the request is freed and counted like any other: a request that stayed
+      // in flight would hold every later refresh back (r_inflight != 0 on a batch boundary) and leak its slot.
+      FL_WARN("NET/FuseLink : Got completion with error, channel %d, %s", lk->channelId, r->type == kReqSend ? "Send" : "Recv");
+      result = ncclRemoteError;
+    } else if (st == kStLaunched && pr && __atomic_load_n(pr->h_status, __ATOMIC_ACQUIRE) != 0) {
+      // A kernel refused a chunk that would have left its window or buffer (the host sizes every launch so that this
+      // cannot happen; the check is the safety net).  The first request completed after the refusal reports it, once,
+      // and is freed like any other; the word is cleared so that later traffic is not condemned with it.
+      const int32_t code = __atomic_exchange_n(pr->h_status, 0, __ATOMIC_ACQ_REL);
+      if (code != 0) {
+        FL_WARN("NET/FuseLink : a chunk fell outside its staging window or buffer (status %d)", code);
+        result = ncclInternalError;
+      }
+    }
+    *done = result == ncclSuccess ? 1 : 0;                    // plugin.cc:1807-1823
+    if (r->type == kReqSend) { lk->s_finished++; lk->s_inflight--; }
+    if (r->type == kReqRecv) {
+      mark_nic_active(lk->dev % g_par.lanes, 0);   // updateRxChannelActive, fuselink.h:254-259
+      if (result == ncclSuccess) lk->tx_available = r->imm;   // comm->txAvailable = wc->imm_data, plugin.cc:1884-1885
+      lk->r_finished++;
+      lk->r_inflight--;
+      if (sizes) sizes[0] = r->size;   // the reference leaves 0 here (plugin.cc:1726, 1882)
+    }
+    r->type = kReqUnused;                                     // ncclIbFreeRequest, plugin.cc:1086-1090
   }
-  r->type = kReqUnused;                                     // ncclIbFreeRequest, plugin.cc:1086-1090
+  // a receive that is through frees its wave's landing set at the next look; look now, the sender may be waiting for it
+  if (pair && !lk->wire->is_send) (void)wire_progress_recv(pair);
   return result;
 }
 
 ncclResult_t close_comm(void* comm, int want_send) {
   Comm* c = (Comm*)comm;
   if (!c) return ncclSuccess;
-  if (c->magic == kShmCommMagic && c->is_send == want_send) {
-    ShmComm* sc = (ShmComm*)comm;
-    (want_send ? sc->w->send_closed : sc->w->recv_closed).store(1, std::memory_order_release);
-    sc->magic = 0;
-    shm_comm_free(sc);
-    return ncclSuccess;
-  }
   if (c->magic != kCommMagic || c->is_send != want_send) return ncclInvalidArgument;
   Link* lk = c->link;
+  if (lk->wire && lk->wire->pair) {
+    // what this end still owes the other process goes out before the end is marked closed: a sender announces the
+    // waves that have landed, a receiver hands back the landing sets of the waves it has delivered
+    WirePair* pair = lk->wire->pair;
+    const int64_t until = tr_now() + 2000000000ll;
+    if (want_send) {
+      for (;;) {
+        (void)wire_publish(pair);
+        bool empty;
+        { std::lock_guard<std::mutex> g(pair->tx_mu); empty = pair->tx_flights.empty(); }
+        if (empty || pair->w->failed.load(std::memory_order_acquire) || tr_now() > until) break;
+      }
+    } else {
+      (void)wire_progress_recv(pair);
+    }
+  }
   c->magic = 0;
   delete c;
   link_unref(lk);
@@ -1768,7 +2234,7 @@ ncclResult_t fl_close_listen(void* listenComm) {
   if (!lc) return ncclSuccess;
   if (lc->magic == kShmListenMagic) {
     ShmListen* sl = (ShmListen*)listenComm;
-    if (sl->comm) shm_comm_free(sl->comm);   // never accepted: the object goes with it
+    if (sl->link) link_unref(sl->link);   // never accepted: the object goes with it
     sl->magic = 0;
     delete sl;
     return ncclSuccess;
@@ -1927,7 +2393,6 @@ static void last_buffers(const Peer* pr, const flh_chunk_desc** table, const flh
 
 int fl_net_last_table(void* sendComm, void* rows_out, int max_rows, void* hdr_out) {
   Comm* c = (Comm*)sendComm;
-  if (c && c->magic == kShmCommMagic && c->is_send) return shm_last_table((ShmComm*)sendComm, rows_out, max_rows, hdr_out);
   if (!c || c->magic != kCommMagic || !c->is_send) return fl_set_error(FLH_E_ARG, "not a send comm");
   Link* lk = c->link;
   Peer* pr = lk->peer.load(std::memory_order_acquire);

@@ -1,185 +1,222 @@
 // fl_plugin_shm_wire.h -- the plugin's wire between two processes.  Not a header of its own: fl_plugin.cc includes it
-// inside its unnamed namespace, behind the objects and helpers it uses (Params, FifoWire, MemHandle, Handle, the request
-// type codes, DeviceScope, FL_HIPCHECK / FL_FLHCHECK, ensure_pool, current_credits, wave_chunks) and in front of the
-// entry points that dispatch to it by magic number.
+// inside its unnamed namespace, behind the objects and helpers it uses (Params, FifoWire, Link, Peer, Request, Handle,
+// DeviceScope, FL_HIPCHECK / FL_FLHCHECK, ensure_pool, attach_peer, wire_credits, fill_uniform, the completion helpers)
+// and in front of the entry points that dispatch to it.
 // ------------------------------------------------------------------------------------------------
 // shared-memory wire: sender and receiver in different processes (NCCL_FUSELINK_WIRE=shm)
 // ------------------------------------------------------------------------------------------------
 // The reference's two ends are different processes on different hosts: the receiver writes 64-byte descriptors into a
 // FIFO in the sender's memory by RDMA (ncclIbSendFifo, plugin.cc:487-496, 1616-1677), the sender RDMA-writes the payload
-// out of its staged buffer into the receiver's registered memory and completes it with a WRITE_WITH_IMM
-// (plugin.cc:1453-1495), and the 128-byte handle that listen fills carries what connect needs to reach the listener
-// (plugin.cc:425-430, 776-885).  On one GPU the part of that which can be shown is the process boundary: listen creates a
-// POSIX shared-memory object and names it in the handle; connect, in another process, maps it.  The object holds the
-// descriptor FIFO (receiver writes, sender reads), a ring of wave completions (sender writes, receiver reads: the
-// stand-in for the WRITE_WITH_IMM completions) and the IPC handle of the receiver's landing windows.  A send then runs
-// as in the reference's layers: the striping kernel stages a wave of the request's chunks in the sender's lane windows
-// (HIP VMM, from the unit pool); the wire carries every lane's staged bytes into the receiver's landing window for that
-// lane (one launch, flh_copy_runs), device memory of the receiver's process that the sender has opened through
-// hipIpcOpenMemHandle (an imported VMM allocation would be the closer analogue; this runtime refuses
-// hipMemImportFromShareableHandle for another process's descriptor, so the landing windows are a plain device
-// allocation); the sender publishes the wave; the receiver's reassembly kernel writes the posted buffer from its landing
-// windows and hands them back.  The receiver keeps NCCL_FUSELINK_WIRE_SETS sets of landing windows, so that many waves
-// are on the wire at once; requests start, finish and are reported in order.
-void fill_uniform(flh_uniform_params& u, const uint32_t* credits, uint64_t bytes, uint64_t src_base, uint64_t epoch_bytes, uint32_t tile);
+// out of its staged buffer into the receiver's registered memory and completes it with a WRITE_WITH_IMM whose immediate
+// data is its lane-availability mask (plugin.cc:1441-1465, 1467-1495), and the 128-byte handle that listen fills carries
+// what connect needs to reach the listener (plugin.cc:425-430, 776-885).  On one GPU the part of that which can be shown
+// is the process boundary.
+//
+// Per connection: listen creates a POSIX shared-memory object and names it in the handle; connect, in another process,
+// maps it.  It holds the descriptor FIFO (receiver writes, sender reads).
+// Per pair of processes and GPU: the receiver owns sets of landing windows, one window per lane in each set, device
+// memory that the sender opens through hipIpcOpenMemHandle (an imported VMM allocation would be the closer analogue;
+// this runtime refuses hipMemImportFromShareableHandle for another process's descriptor), and a second shared-memory
+// object with a ring of wave records -- the stand-in for the WRITE_WITH_IMM completions -- shared by every connection
+// between the two processes, as the reference's channels share the per-NIC lane comms (fuselink.h:271-272).
+//
+// A send travels through the sending GPU's staging side like a send whose receiver is in the same process
+// (fl_plugin.cc): matched sends of all connections wait in one queue and go out in batches.  A batch for another
+// process is a *wave*: the lane engine (or, for large requests, one launch) stripes it into this process's staging
+// windows and carries every staged tile on into the same lane and offset of one set of landing windows
+// (FLH_ENGINE_SEND / flh_stripe_*_carry: the NIC's part).  When the engine's completion word -- or the launch's --
+// says the bytes have landed, the sender's test publishes the wave record from the host and reports the sends complete:
+// like an RDMA write, a send is complete once its bytes are in the receiver's memory.  The receiver's test finds the
+// record, builds the same batch from the receives it posted (it wrote their credit rows into the descriptors itself;
+// the record brings the sizes, the epoch prefixes and the sender's masks) and hands it to its own engine
+// (FLH_ENGINE_RECV) or launches the reassembly; when that is complete the landing set goes back to the sender through a
+// counter.  No event is recorded or queried and, for requests the engine takes, nothing is launched on either side.
 
-constexpr uint64_t kHandleMagicShm = 0x4655534c53484d31ull;   // "FUSLSHM1"
-constexpr uint32_t kShmCommMagic = 0x464c5343;                // "FLSC"
-constexpr uint32_t kShmReqMagic = 0x464c5352;                 // "FLSR"
+constexpr uint64_t kHandleMagicShm = 0x4655534c53484d32ull;   // "FUSLSHM2"
+constexpr uint64_t kPairMagic = 0x4655534c50414952ull;        // "FUSLPAIR"
 constexpr uint32_t kShmListenMagic = 0x464c534c;              // "FLSL"
 
 constexpr int kShmSetsMax = 8;
-struct ShmWave {                   // one wave of chunks that has landed in the receiver's windows
-  std::atomic<uint64_t> seq;       // wave number + 1, written last
-  uint64_t fifo_idx;               // the descriptor (request) it belongs to
-  uint64_t epoch_bytes;            // the connection's credit-epoch prefix the wave was scheduled from
-  uint64_t offset;                 // byte offset of the wave in the request
+constexpr uint32_t kPairWaves = 64;      // wave records a pair's ring holds (more than the landing sets there can be)
+constexpr uint32_t kPairConns = 256;     // connections between two processes that share the pair
+
+struct WaveReq {                   // one request of a wave
+  uint32_t conn;                   // the connection's number within the pair
+  uint32_t imm;                    // the sender's lane-availability mask: imm_data of plugin.cc:1441-1447, 1463
+  uint64_t fifo_idx;               // the descriptor it answers, from 1
   uint64_t bytes;
-  uint32_t last;                   // the request's last wave
-  uint32_t set;                    // the set of landing windows it lies in
-  // A wave may instead carry n_req >= 2 whole requests, fifo_idx and the ones behind it, staged as one message of
-  // `bytes` from epoch_bytes on (flh_stripe_batch with one segment); req_bytes are the sends' sizes.
+};
+struct WaveSeg {                   // a run of requests of one connection, scheduled as one message (flh_batch_segment)
+  uint64_t epoch_bytes;            // the connection's credit-epoch prefix the segment was scheduled from
   uint32_t n_req;
   uint32_t pad;
-  uint64_t req_bytes[FLH_BATCH_MAX];
 };
-struct ShmWire {
+struct ShmWave {                   // one wave that has landed in the receiver's windows
+  std::atomic<uint64_t> seq;       // wave number (from 1), written last
+  uint32_t set;                    // the set of landing windows it lies in
+  uint32_t n_req, n_seg;
+  uint32_t piece;                  // 1: part of ONE request that the windows do not hold whole: `offset` and `last` apply
+  uint64_t offset;                 // byte offset of the piece in the request
+  uint32_t last;                   // the request's last piece
+  uint32_t pad;
+  uint64_t total_bytes;
+  WaveReq req[FLH_BATCH_MAX];
+  WaveSeg seg[FLH_SEG_MAX];
+};
+struct ShmPair {                   // one per (sending process, receiving process, GPU of the receiver)
+  uint64_t magic;
+  uint32_t lanes;
+  uint32_t sets;                   // sets of landing windows = waves that may be on the wire at once
+  uint64_t bytes_per_lane;
+  hipIpcMemHandle_t landing;       // sets x lanes x bytes_per_lane of the receiver's device memory
+  std::atomic<uint32_t> sender_mapped;   // the sender holds its mapping: the name is no longer needed
+  std::atomic<uint32_t> failed;          // a wave was lost (the sender's engine went down): every request on the pair fails
+  alignas(64) std::atomic<uint64_t> waves_consumed;   // receiver: waves delivered so far, in order (their landing sets are free again)
+  alignas(64) ShmWave wave[kPairWaves];
+};
+struct ShmWire {                   // one per connection
   uint64_t magic;
   uint32_t lanes;
   uint32_t channelId;
   std::atomic<uint32_t> connected, accepted, send_closed, recv_closed;
-  std::atomic<uint32_t> landing_ready;
-  uint32_t landing_sets;           // sets of landing windows = waves that may be on the wire at once
-  uint64_t landing_bytes_per_lane;
-  hipIpcMemHandle_t landing;       // sets x lanes x landing_bytes_per_lane of the receiver's device memory
-  alignas(64) FifoWire fifo[FL_NET_MAX_REQUESTS];          // plugin.cc:487-496: written by the receiver, idx last
-  alignas(64) ShmWave wave[FL_NET_MAX_REQUESTS];
-  alignas(64) std::atomic<uint64_t> waves_consumed;        // receiver: waves reassembled so far, in order (their landing windows are free again)
+  int32_t sender_pid;              // written by connect
+  std::atomic<uint32_t> landing_ready;   // pair_name and pair_conn are valid
+  uint32_t pair_conn;
+  char pair_name[64];
+  alignas(64) FifoWire fifo[FL_NET_MAX_REQUESTS];   // plugin.cc:487-496: written by the receiver, idx last; cleared by the sender when matched
 };
 
-struct ShmRequest {
-  uint32_t magic = 0;
-  int type = kReqUnused;
-  struct ShmComm* comm = nullptr;
-  uint64_t fifo_idx = 0;           // 1-based descriptor number
-  uint64_t size = 0;
-  uint32_t credits[FLH_MAX_LANES] = {};
-  // sender
-  const uint8_t* src = nullptr;
-  uint64_t launched = 0;           // bytes whose waves have been queued on the GPU
-  bool all_launched = false;       // (a request of no bytes still takes one wave)
-  uint64_t last_wave = 0;          // number (from 1) of the request's last wave, once all_launched
-  bool refresh = false;
-  // receiver
-  uint8_t* dst = nullptr;
-  uint64_t received = 0;           // bytes reassembled
-  bool complete = false;           // the last wave has been reassembled
+struct WireFlight {                // a wave whose GPU work has been handed over
+  bool engine = false;
+  uint64_t seq = 0;                // engine batch or launch that completes it (0: no GPU work, complete as it stands)
+  ShmWave rec;                     // sender: the record to publish
+  WireFlight() { memset((void*)&rec, 0, sizeof(rec)); }
+  WireFlight(const WireFlight& o) : engine(o.engine), seq(o.seq) { memcpy((void*)&rec, (const void*)&o.rec, sizeof(rec)); }
+  WireFlight& operator=(const WireFlight&) = delete;
 };
 
-struct ShmFlight {                 // a wave whose GPU work is queued: the event of its set tells when it is through
-  ShmRequest* req;
-  uint64_t fifo_idx, epoch_bytes, offset, bytes;
-  uint32_t last, set;
-  uint32_t n_req = 1;              // a wave of several whole requests: req and the ones behind it
-  ShmRequest* batch[FLH_BATCH_MAX];
-  uint64_t req_bytes[FLH_BATCH_MAX];
+struct WirePair {                  // this process's end of a pair
+  ShmPair* w = nullptr;
+  char name[64] = "";
+  bool receiver = false;           // this process owns the landing windows and the object
+  bool named = false;              // the name still exists in the file system
+  int peer_pid = 0;
+  int hip_device = -1;
+  int links = 0;                   // connections attached (g_pair_mu)
+  Peer* peer = nullptr;            // this process's staging side of the GPU
+  uint8_t* landing = nullptr;      // receiver: its allocation; sender: the same memory opened through IPC
+  int sets = 0;
+  flh_windows landing_wins[kShmSetsMax] = {};
+  // sender (flights and tx_launched under tx_mu)
+  std::mutex tx_mu;
+  std::deque<WireFlight> tx_flights;
+  uint64_t tx_launched = 0;                     // waves handed to the GPU
+  std::atomic<uint64_t> tx_published{0};        // waves announced to the receiver
+  bool blocked = false;                         // a pass that launches found no free landing set (launch_mu)
+  // receiver (under rx_mu)
+  std::mutex rx_mu;
+  std::deque<WireFlight> rx_flights;
+  std::atomic<uint64_t> rx_taken{0};            // waves taken off the ring
+  uint64_t rx_done = 0;                         // waves delivered
+  std::atomic<Link*> conns[kPairConns] = {};    // this process's end of every connection of the pair, by its number
 };
 
-struct ShmComm {
-  uint32_t magic = kShmCommMagic;
-  int is_send = 0;
-  int dev = 0;
+struct WireEnd {                   // a connection's end of the wire (Link::wire)
   ShmWire* w = nullptr;
   char name[64] = "";
   bool owner = false;              // the receiver created the object and unlinks it
-  std::mutex mu;
-  ShmRequest reqs[FL_NET_MAX_REQUESTS];
-  uint64_t fifoHead = 0, fifoTail = 0;       // sender: next descriptor to match; receiver: next to post
-  std::deque<ShmRequest*> active;            // requests in flight, in order: they start, finish and are reported in that order
-  size_t cursor = 0;                         // sender: first request of `active` with waves left to launch; receiver: the one the next wave belongs to
-  std::deque<ShmFlight> flights;             // waves queued on the GPU, in order
-  uint64_t epoch_bytes = 0;                  // sender: the scheduler's carried prefix
-  uint64_t waves_launched = 0;               // sender: waves queued on the GPU so far; receiver: waves taken off the wire so far
-  uint64_t waves_published = 0;              // sender: waves announced to the receiver
-  uint64_t waves_done = 0;                   // receiver: waves reassembled (what waves_consumed says)
-  uint32_t last_rows = 0;                    // sender: chunks of the latest wave (rows of d_table)
-  int64_t r_finished = 0, r_inflight = 0;
-  int fuselink_offset = -1;
-  uint8_t credits[FL_NET_MAX_LANES] = {};
-  bool have_decision = false;
-  // GPU side
-  bool gpu_ready = false;
-  int hip_device = -1;
-  int sets = 0;
-  hipStream_t stream = nullptr;
-  hipEvent_t ev[kShmSetsMax] = {};           // one per set of landing windows: the latest wave that uses the set
-  flh_window* win[FL_NET_MAX_LANES] = {};    // sender: staging windows
-  flh_windows wins = {};
-  uint8_t* landing = nullptr;                // receiver: its allocation; sender: the same memory opened through IPC
-  flh_windows landing_wins[kShmSetsMax] = {};
-  flh_chunk_desc* d_table = nullptr;
-  flh_sched_hdr* d_hdr = nullptr;
-  int32_t *h_status = nullptr, *d_status = nullptr;
+  bool is_send = false;
+  WirePair* pair = nullptr;
+  uint32_t pair_conn = 0;
 };
 
 struct ShmListen {
   uint32_t magic = kShmListenMagic;
   int dev = 0;
-  ShmComm* comm = nullptr;         // becomes the recv comm at accept
+  Link* link = nullptr;            // becomes the recv comm's at accept
 };
 
 std::atomic<uint64_t> g_shm_counter{0};
+std::mutex g_pair_mu;              // the pairs of this process, their attachment counts and connection tables
+std::vector<WirePair*> g_pairs;
 
-void shm_comm_free(ShmComm* c) {
-  if (c->stream) {
+void wire_pair_destroy(WirePair* p) {   // no longer reachable through g_pairs
+  if (p->landing) {
     DeviceScope keep;
-    (void)hipSetDevice(c->hip_device);
-    (void)hipStreamSynchronize(c->stream);
-    for (int l = 0; l < FL_NET_MAX_LANES; ++l) if (c->win[l]) (void)flh_window_destroy(c->win[l]);
-    if (c->landing) { if (c->is_send) (void)hipIpcCloseMemHandle(c->landing); else (void)hipFree(c->landing); }
-    if (c->d_table) (void)hipFree(c->d_table);
-    if (c->d_hdr) (void)hipFree(c->d_hdr);
-    if (c->h_status) (void)hipHostFree(c->h_status);
-    for (hipEvent_t e : c->ev) if (e) (void)hipEventDestroy(e);
-    (void)hipStreamDestroy(c->stream);
+    (void)hipSetDevice(p->hip_device);
+    if (p->receiver) {
+      // what this process's kernels still read out of the windows must be through before they go
+      if (p->peer && p->peer->stream) (void)hipStreamSynchronize(p->peer->stream);
+      (void)hipFree(p->landing);
+    } else {
+      (void)hipIpcCloseMemHandle(p->landing);
+    }
   }
-  if (c->w) munmap(c->w, sizeof(ShmWire));
-  if (c->owner && c->name[0]) shm_unlink(c->name);
-  delete c;
-  g_live_links.fetch_sub(1);   // (a reset of the plugin waits for these as for the in-process connections)
+  if (p->w) munmap(p->w, sizeof(ShmPair));
+  if (p->receiver && p->named) shm_unlink(p->name);
+  delete p;
+}
+
+// The connection's end goes away (the last reference to the link is being dropped; nothing of it waits for a launch).
+void wire_end_free(Link* lk) {
+  WireEnd* e = lk->wire;
+  if (!e) return;
+  if (e->w) (e->is_send ? e->w->send_closed : e->w->recv_closed).store(1, std::memory_order_release);
+  if (WirePair* p = e->pair) {
+    bool gone;
+    {
+      std::lock_guard<std::mutex> g(g_pair_mu);
+      if (p->receiver) p->conns[e->pair_conn].store(nullptr, std::memory_order_release);
+      gone = --p->links == 0;
+      if (gone) {
+        for (size_t i = 0; i < g_pairs.size(); ++i) if (g_pairs[i] == p) { g_pairs.erase(g_pairs.begin() + (long)i); break; }
+      }
+    }
+    if (gone) wire_pair_destroy(p);
+  }
+  if (e->w) munmap(e->w, sizeof(ShmWire));
+  if (e->owner && e->name[0]) shm_unlink(e->name);
+  delete e;
+  lk->wire = nullptr;
 }
 
 ncclResult_t shm_listen(int dev, void* opaqueHandle, void** listenComm) {
   ShmListen* lc = new (std::nothrow) ShmListen();
-  ShmComm* c = new (std::nothrow) ShmComm();
-  if (!lc || !c) { delete lc; delete c; return ncclSystemError; }
-  g_live_links.fetch_add(1);
-  snprintf(c->name, sizeof(c->name), "/fuselink-wire-%d-%llu", (int)getpid(), (unsigned long long)g_shm_counter.fetch_add(1));
-  int fd = shm_open(c->name, O_CREAT | O_EXCL | O_RDWR, 0600);
-  if (fd < 0 || ftruncate(fd, sizeof(ShmWire)) != 0) { if (fd >= 0) close(fd); FL_WARN("NET/FuseLink : shm_open(%s) failed", c->name); delete lc; delete c; g_live_links.fetch_sub(1); return ncclSystemError; }
+  Link* lk = new (std::nothrow) Link();
+  WireEnd* e = new (std::nothrow) WireEnd();
+  if (!lc || !lk || !e) { delete lc; delete lk; delete e; return ncclSystemError; }
+  snprintf(e->name, sizeof(e->name), "/fuselink-wire-%d-%llu", (int)getpid(), (unsigned long long)g_shm_counter.fetch_add(1));
+  int fd = shm_open(e->name, O_CREAT | O_EXCL | O_RDWR, 0600);
+  if (fd < 0 || ftruncate(fd, sizeof(ShmWire)) != 0) { if (fd >= 0) { close(fd); shm_unlink(e->name); } FL_WARN("NET/FuseLink : shm_open(%s) failed", e->name); delete lc; delete lk; delete e; return ncclSystemError; }
   void* p = mmap(nullptr, sizeof(ShmWire), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
   close(fd);
-  if (p == MAP_FAILED) { shm_unlink(c->name); delete lc; delete c; g_live_links.fetch_sub(1); return ncclSystemError; }
+  if (p == MAP_FAILED) { shm_unlink(e->name); delete lc; delete lk; delete e; return ncclSystemError; }
   memset(p, 0, sizeof(ShmWire));
-  c->w = (ShmWire*)p;
-  c->owner = true;
-  c->dev = dev;
-  c->w->lanes = (uint32_t)g_par.lanes;
+  g_live_links.fetch_add(1);
+  e->w = (ShmWire*)p;
+  e->owner = true;
+  e->is_send = false;
+  e->w->lanes = (uint32_t)g_par.lanes;
   {
     std::lock_guard<std::mutex> g(g_reg_mu);
-    c->w->channelId = (uint32_t)g_channel_counter++;
+    e->w->channelId = (uint32_t)g_channel_counter++;
   }
-  c->w->magic = kHandleMagicShm;
+  e->w->magic = kHandleMagicShm;
+  lk->refs = 1;
+  lk->dev = dev;
+  lk->channelId = (int)e->w->channelId;
+  lk->send_ready = 1;
+  lk->wire = e;
   lc->dev = dev;
-  lc->comm = c;
+  lc->link = lk;
   Handle* h = (Handle*)opaqueHandle;
   memset(h, 0, NCCL_NET_HANDLE_MAXSIZE);
   h->magic = kHandleMagicShm;
-  h->channelId = (int32_t)c->w->channelId;
+  h->channelId = (int32_t)e->w->channelId;
   h->dev = dev;
   // the object's name travels in the handle, as the listener's address does in the reference's (plugin.cc:425-430)
   static_assert(sizeof(Handle) + 64 <= NCCL_NET_HANDLE_MAXSIZE, "the name must fit behind the fixed part of the handle");
-  memcpy((char*)opaqueHandle + sizeof(Handle), c->name, sizeof(c->name));
+  memcpy((char*)opaqueHandle + sizeof(Handle), e->name, sizeof(e->name));
   *listenComm = lc;
   return ncclSuccess;
 }
@@ -187,7 +224,7 @@ ncclResult_t shm_listen(int dev, void* opaqueHandle, void** listenComm) {
 ncclResult_t shm_connect(int dev, void* opaqueHandle, void** sendComm) {
   Handle* h = (Handle*)opaqueHandle;
   *sendComm = nullptr;
-  ShmComm* c = (ShmComm*)h->stage_link;
+  Link* lk = (Link*)h->stage_link;
   if (h->stage == 0) {
     char name[64];
     memcpy(name, (char*)opaqueHandle + sizeof(Handle), sizeof(name));
@@ -206,31 +243,45 @@ ncclResult_t shm_connect(int dev, void* opaqueHandle, void** sendComm) {
     void* p = mmap(nullptr, sizeof(ShmWire), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
     close(fd);
     if (p == MAP_FAILED) return ncclSystemError;
-    c = new (std::nothrow) ShmComm();
-    if (!c) { munmap(p, sizeof(ShmWire)); return ncclSystemError; }
+    lk = new (std::nothrow) Link();
+    WireEnd* e = new (std::nothrow) WireEnd();
+    if (!lk || !e) { delete lk; delete e; munmap(p, sizeof(ShmWire)); return ncclSystemError; }
     g_live_links.fetch_add(1);
-    c->w = (ShmWire*)p;
-    if (c->w->magic != kHandleMagicShm || (int)c->w->lanes != g_par.lanes) {
-      FL_WARN("NET/FuseLink : connect: the listener runs %u lanes, this side %d", c->w->lanes, g_par.lanes);
-      shm_comm_free(c);
+    e->w = (ShmWire*)p;
+    e->is_send = true;
+    memcpy(e->name, name, sizeof(name));
+    lk->refs = 1;
+    lk->dev = dev;
+    lk->channelId = (int)e->w->channelId;
+    lk->send_ready = 1;
+    lk->wire = e;
+    if (e->w->magic != kHandleMagicShm || (int)e->w->lanes != g_par.lanes) {
+      FL_WARN("NET/FuseLink : connect: the listener runs %u lanes, this side %d", e->w->lanes, g_par.lanes);
+      e->w = nullptr;               // not ours to mark closed
+      munmap(p, sizeof(ShmWire));
+      link_unref(lk);
       return ncclInvalidUsage;
     }
     int listener_pid = -1;
     if (sscanf(name, "/fuselink-wire-%d-", &listener_pid) == 1 && listener_pid == (int)getpid()) {
       // the landing windows reach the sender through HIP IPC, which a process cannot open on its own allocations
       FL_WARN("NET/FuseLink : NCCL_FUSELINK_WIRE=shm connects two processes; this listener lives in the connecting process (unset it for the in-process wire)");
-      shm_comm_free(c);
+      e->w = nullptr;
+      munmap(p, sizeof(ShmWire));
+      link_unref(lk);
       return ncclInvalidUsage;
     }
-    c->is_send = 1;
-    c->dev = dev;
-    memcpy(c->name, name, sizeof(name));
-    c->w->connected.store(1, std::memory_order_release);
+    e->w->sender_pid = (int32_t)getpid();
+    e->w->connected.store(1, std::memory_order_release);
     h->stage = 1;
-    h->stage_link = c;
+    h->stage_link = lk;
     return ncclSuccess;
   }
-  if (!c->w->accepted.load(std::memory_order_acquire)) return ncclSuccess;   // accept has not happened yet
+  if (!lk->wire->w->accepted.load(std::memory_order_acquire)) return ncclSuccess;   // accept has not happened yet
+  Comm* c = new (std::nothrow) Comm();
+  if (!c) return ncclSystemError;
+  c->is_send = 1;
+  c->link = lk;
   h->stage = 0;
   h->stage_link = nullptr;
   *sendComm = c;
@@ -239,445 +290,234 @@ ncclResult_t shm_connect(int dev, void* opaqueHandle, void** sendComm) {
 
 ncclResult_t shm_accept(ShmListen* lc, void** recvComm) {
   *recvComm = nullptr;
-  ShmComm* c = lc->comm;
-  if (!c || !c->w->connected.load(std::memory_order_acquire)) return ncclSuccess;   // nobody connected yet
-  c->w->accepted.store(1, std::memory_order_release);
-  shm_unlink(c->name);   // both ends hold their mapping: the name is no longer needed and cannot leak
-  c->owner = false;
-  lc->comm = nullptr;
+  Link* lk = lc->link;
+  if (!lk || !lk->wire->w->connected.load(std::memory_order_acquire)) return ncclSuccess;   // nobody connected yet
+  Comm* c = new (std::nothrow) Comm();
+  if (!c) return ncclSystemError;
+  WireEnd* e = lk->wire;
+  e->w->accepted.store(1, std::memory_order_release);
+  shm_unlink(e->name);   // both ends hold their mapping: the name is no longer needed and cannot leak
+  e->owner = false;
+  lc->link = nullptr;
+  c->is_send = 0;
+  c->link = lk;
   *recvComm = c;
   return ncclSuccess;
 }
 
 // set k, lane l of the landing windows: one allocation, set after set, lane after lane
-void shm_landing_windows(ShmComm* c, uint64_t per_lane) {
-  for (int k = 0; k < c->sets; ++k) {
-    c->landing_wins[k].n_lanes = (uint32_t)g_par.lanes;
+void wire_landing_windows(WirePair* p, uint64_t per_lane) {
+  for (int k = 0; k < p->sets; ++k) {
+    p->landing_wins[k].n_lanes = (uint32_t)g_par.lanes;
     for (int l = 0; l < g_par.lanes; ++l) {
-      c->landing_wins[k].base[l] = c->landing + ((uint64_t)k * (uint64_t)g_par.lanes + (uint64_t)l) * per_lane;
-      c->landing_wins[k].cap[l] = per_lane;
+      p->landing_wins[k].base[l] = p->landing + ((uint64_t)k * (uint64_t)g_par.lanes + (uint64_t)l) * per_lane;
+      p->landing_wins[k].cap[l] = per_lane;
     }
   }
 }
 
-// stream, status word, table buffers; the sender's staging windows or the receiver's landing windows
-ncclResult_t shm_setup_gpu(ShmComm* c, int device) {
-  if (c->gpu_ready) return ncclSuccess;
-  if (c->stream) return ncclInternalError;   // failed earlier
-  DeviceScope keep;
-  c->hip_device = device;
-  FL_HIPCHECK(hipSetDevice(device));
-  FL_HIPCHECK(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-  FL_HIPCHECK(hipHostMalloc((void**)&c->h_status, 64, hipHostMallocMapped));
-  memset(c->h_status, 0, 64);
-  FL_HIPCHECK(hipHostGetDevicePointer((void**)&c->d_status, c->h_status, 0));
-  const uint64_t cap = (uint64_t)g_par.window_units * FLH_UNIT_BYTES;
-  if (c->is_send) {
-    flh_pool* pool = nullptr;
-    ncclResult_t rc = ensure_pool(device, &pool);
-    if (rc != ncclSuccess) return rc;
-    c->wins.n_lanes = (uint32_t)g_par.lanes;
-    for (int l = 0; l < g_par.lanes; ++l) {
-      FL_FLHCHECK(flh_window_create(pool, cap, &c->win[l]));
-      FL_FLHCHECK(flh_window_bind(c->win[l], cap));
-      c->wins.base[l] = flh_window_base(c->win[l]);
-      c->wins.cap[l] = flh_window_bound_bytes(c->win[l]);
-    }
-    FL_HIPCHECK(hipMalloc((void**)&c->d_table, sizeof(flh_chunk_desc) * (size_t)g_par.max_wave_chunks));
-    FL_HIPCHECK(hipMalloc((void**)&c->d_hdr, sizeof(flh_sched_hdr)));
-    // (the landing windows, and with them the number of sets and their events, come with the receiver's first descriptor)
-  } else {
-    c->sets = g_par.wire_sets;
-    const uint64_t bytes = cap * (uint64_t)g_par.lanes * (uint64_t)c->sets;
-    if (bytes >= (2ull << 30)) { FL_WARN("NET/FuseLink : %d sets of landing windows take %llu bytes; a shared allocation must stay under 2 GiB", c->sets, (unsigned long long)bytes); return ncclInvalidUsage; }
-    FL_HIPCHECK(hipMalloc((void**)&c->landing, bytes));
-    FL_HIPCHECK(hipIpcGetMemHandle(&c->w->landing, c->landing));
-    c->w->landing_bytes_per_lane = cap;
-    c->w->landing_sets = (uint32_t)c->sets;
-    for (int k = 0; k < c->sets; ++k) FL_HIPCHECK(hipEventCreateWithFlags(&c->ev[k], hipEventDisableTiming));
-    shm_landing_windows(c, cap);
-    c->w->landing_ready.store(1, std::memory_order_release);
-  }
-  c->gpu_ready = true;
-  return ncclSuccess;
+// what a window of either kind (the launches', the engine's) holds in this process
+uint64_t wire_window_cap() {
+  const uint64_t a = (uint64_t)g_par.window_units * FLH_UNIT_BYTES, b = g_par.engine ? (uint64_t)g_par.engine_units * FLH_UNIT_BYTES : 0;
+  return a > b ? a : b;
 }
 
-ShmRequest* shm_get_request(ShmComm* c, int type) {
-  for (int i = 0; i < FL_NET_MAX_REQUESTS; ++i) {
-    ShmRequest* r = &c->reqs[i];
-    if (r->type == kReqUnused) {
-      *r = ShmRequest();
-      r->magic = kShmReqMagic;
-      r->type = type;
-      r->comm = c;
-      return r;
-    }
-  }
-  FL_WARN("NET/FuseLink : unable to allocate requests");
-  return nullptr;
-}
-
-// Credit row a descriptor asks for (both ends derive it from the descriptor alone, so they agree).
-void shm_wire_credits(const ShmComm* c, const FifoWire& w, uint32_t* credits) {
-  for (int l = 0; l < FLH_MAX_LANES; ++l) credits[l] = 0;
-  if (w.fuselink_offset == -2) { for (int l = 0; l < g_par.lanes; ++l) credits[l] = w.credits[l]; }
-  else credits[w.fuselink_offset >= 0 ? w.fuselink_offset % g_par.lanes : (int)(c->w->channelId % (uint32_t)g_par.lanes)] = 1;
-}
-
-ncclResult_t shm_irecv(ShmComm* c, void* data, int size, int tag, MemHandle* mh, void** request) {
-  *request = nullptr;
-  if (mh->type != NCCL_PTR_CUDA) { FL_WARN("NET/FuseLink : the shared-memory wire carries device memory only"); return ncclInvalidUsage; }
-  std::lock_guard<std::mutex> g(c->mu);
-  ncclResult_t rc = shm_setup_gpu(c, mh->device);
+// Receiver (lk->mu held): the connection joins the pair of its sender's process and this GPU -- the first one creates
+// it, landing windows and all -- and tells the sender where to find it.
+ncclResult_t wire_recv_setup(Link* lk, int device) {
+  WireEnd* e = lk->wire;
+  if (e->pair) return ncclSuccess;
+  ncclResult_t rc = attach_peer(lk, device);   // this process's staging side of the GPU: engine, stream, completion words
   if (rc != ncclSuccess) return rc;
-  bool refreshed = false;
-  if (c->r_finished % g_par.refresh_batch == 0 || !c->have_decision) {   // plugin.cc:1700-1712
-    if (c->r_inflight != 0) return ncclSuccess;
-    if (g_par.policy == 0) {
-      c->fuselink_offset = (int)(c->w->channelId % (uint32_t)g_par.lanes);
-    } else {
-      c->fuselink_offset = -2;
-      current_credits(c->dev % g_par.lanes, c->credits);
-    }
-    c->have_decision = true;
-    refreshed = true;
-  }
-  if ((int)c->active.size() >= FL_NET_MAX_REQUESTS - 1) return ncclSuccess;   // the descriptor ring is full
-  ShmRequest* r = shm_get_request(c, kReqRecv);
-  if (!r) return ncclInternalError;
-  r->dst = (uint8_t*)data;
-  r->size = (uint64_t)size;
-  r->fifo_idx = c->fifoTail + 1;
-  FifoWire& w = c->w->fifo[c->fifoTail % FL_NET_MAX_REQUESTS];
-  w.addr = (uint64_t)(uintptr_t)data;
-  w.size = size;
-  w.rkey = 1;
-  w.nreqs = 1;
-  w.tag = (uint32_t)tag;
-  w.fuselink_offset = c->fuselink_offset;
-  memcpy(w.credits, c->credits, sizeof(w.credits));
-  w.flags = refreshed ? 1u : 0u;
-  shm_wire_credits(c, w, r->credits);
-  __atomic_store_n(&w.idx, c->fifoTail + 1, __ATOMIC_RELEASE);   // written last: it is what the sender waits for (plugin.cc:1632)
-  c->fifoTail++;
-  c->r_inflight++;
-  c->active.push_back(r);
-  *request = r;
-  return ncclSuccess;
-}
-
-ncclResult_t shm_isend(ShmComm* c, void* data, int size, int tag, MemHandle* mh, void** request) {
-  *request = nullptr;
-  if (mh->type != NCCL_PTR_CUDA) { FL_WARN("NET/FuseLink : the shared-memory wire carries device memory only"); return ncclInvalidUsage; }
-  std::lock_guard<std::mutex> g(c->mu);
-  FifoWire& fw = c->w->fifo[c->fifoHead % FL_NET_MAX_REQUESTS];
-  if (__atomic_load_n(&fw.idx, __ATOMIC_ACQUIRE) != c->fifoHead + 1) return ncclSuccess;   // not posted yet (plugin.cc:1510-1514)
-  if (fw.nreqs != 1) return ncclInternalError;
-  if (fw.tag != (uint32_t)tag) return ncclSuccess;
-  if (size > fw.size) { FL_WARN("NET/FuseLink : req tag %x collective mismatch error, local size %d remote size %d", tag, size, fw.size); return ncclInvalidUsage; }
-  ncclResult_t rc = shm_setup_gpu(c, mh->device);
-  if (rc != ncclSuccess) return rc;
-  if (!c->landing) {   // the receiver's landing windows, once it has set them up
-    if (!c->w->landing_ready.load(std::memory_order_acquire)) return ncclSuccess;
+  const int sender = (int)e->w->sender_pid;
+  std::lock_guard<std::mutex> g(g_pair_mu);
+  WirePair* p = nullptr;
+  for (WirePair* q : g_pairs) if (q->receiver && q->peer_pid == sender && q->hip_device == device) { p = q; break; }
+  if (!p) {
+    p = new (std::nothrow) WirePair();
+    if (!p) return ncclSystemError;
+    p->receiver = true;
+    p->peer_pid = sender;
+    p->hip_device = device;
+    p->peer = lk->peer.load(std::memory_order_acquire);
+    snprintf(p->name, sizeof(p->name), "/fuselink-pair-%d-%d-%d-%llu", (int)getpid(), sender, device, (unsigned long long)g_shm_counter.fetch_add(1));
+    int fd = shm_open(p->name, O_CREAT | O_EXCL | O_RDWR, 0600);
+    if (fd < 0 || ftruncate(fd, sizeof(ShmPair)) != 0) { if (fd >= 0) { close(fd); shm_unlink(p->name); } FL_WARN("NET/FuseLink : shm_open(%s) failed", p->name); delete p; return ncclSystemError; }
+    void* m = mmap(nullptr, sizeof(ShmPair), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    close(fd);
+    if (m == MAP_FAILED) { shm_unlink(p->name); delete p; return ncclSystemError; }
+    memset(m, 0, sizeof(ShmPair));
+    p->w = (ShmPair*)m;
+    p->named = true;
+    const uint64_t cap = wire_window_cap();
+    p->sets = g_par.wire_sets;
+    while (p->sets > 1 && cap * (uint64_t)g_par.lanes * (uint64_t)p->sets >= (2ull << 30)) p->sets--;   // a shared allocation must stay under 2 GiB
+    const uint64_t bytes = cap * (uint64_t)g_par.lanes * (uint64_t)p->sets;
     DeviceScope keep;
-    FL_HIPCHECK(hipSetDevice(c->hip_device));
-    if (c->w->landing_bytes_per_lane < c->wins.cap[0] || c->w->landing_sets < 1 || c->w->landing_sets > (uint32_t)kShmSetsMax) {
-      FL_WARN("NET/FuseLink : the receiver's landing windows (%u sets of %llu bytes per lane) do not fit this side's staging windows",
-              c->w->landing_sets, (unsigned long long)c->w->landing_bytes_per_lane);
+    hipError_t he = bytes >= (2ull << 30) ? hipErrorInvalidValue : hipSetDevice(device);
+    if (he == hipSuccess) he = hipMalloc((void**)&p->landing, bytes);
+    if (he == hipSuccess) he = hipIpcGetMemHandle(&p->w->landing, p->landing);
+    if (he != hipSuccess) {
+      FL_WARN("NET/FuseLink : %d sets of landing windows (%llu bytes): %s", p->sets, (unsigned long long)bytes, bytes >= (2ull << 30) ? "a shared allocation must stay under 2 GiB" : hipGetErrorString(he));
+      wire_pair_destroy(p);
+      return bytes >= (2ull << 30) ? ncclInvalidUsage : ncclUnhandledCudaError;
+    }
+    p->w->lanes = (uint32_t)g_par.lanes;
+    p->w->sets = (uint32_t)p->sets;
+    p->w->bytes_per_lane = cap;
+    p->w->magic = kPairMagic;
+    wire_landing_windows(p, cap);
+    g_pairs.push_back(p);
+  }
+  uint32_t id = kPairConns;
+  for (uint32_t i = 0; i < kPairConns && id == kPairConns; ++i) {
+    Link* none = nullptr;
+    if (p->conns[i].compare_exchange_strong(none, lk, std::memory_order_acq_rel)) id = i;
+  }
+  if (id == kPairConns) { FL_WARN("NET/FuseLink : more than %u connections between two processes", kPairConns); if (p->links == 0) { g_pairs.pop_back(); wire_pair_destroy(p); } return ncclInternalError; }
+  p->links++;
+  e->pair = p;
+  e->pair_conn = id;
+  memcpy(e->w->pair_name, p->name, sizeof(p->name));
+  e->w->pair_conn = id;
+  e->w->landing_ready.store(1, std::memory_order_release);
+  return ncclSuccess;
+}
+
+// Sender (lk->mu held): opens the pair the receiver announced.  *ready stays false while the receiver has not got that far.
+ncclResult_t wire_send_setup(Link* lk, int device, bool* ready) {
+  WireEnd* e = lk->wire;
+  *ready = e->pair != nullptr;
+  if (*ready) return ncclSuccess;
+  if (!e->w->landing_ready.load(std::memory_order_acquire)) return ncclSuccess;
+  ncclResult_t rc = attach_peer(lk, device);
+  if (rc != ncclSuccess) return rc;
+  char name[64];
+  memcpy(name, e->w->pair_name, sizeof(name));
+  name[63] = 0;
+  std::lock_guard<std::mutex> g(g_pair_mu);
+  WirePair* p = nullptr;
+  for (WirePair* q : g_pairs) if (!q->receiver && !strcmp(q->name, name)) { p = q; break; }
+  if (!p) {
+    int fd = shm_open(name, O_RDWR, 0600);
+    struct stat st;
+    if (fd < 0 || fstat(fd, &st) != 0 || (size_t)st.st_size != sizeof(ShmPair)) {
+      if (fd >= 0) close(fd);
+      FL_WARN("NET/FuseLink : the receiver's landing windows (%s) cannot be reached, or belong to another build", name);
+      return ncclSystemError;
+    }
+    void* m = mmap(nullptr, sizeof(ShmPair), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    close(fd);
+    if (m == MAP_FAILED) return ncclSystemError;
+    p = new (std::nothrow) WirePair();
+    if (!p) { munmap(m, sizeof(ShmPair)); return ncclSystemError; }
+    p->w = (ShmPair*)m;
+    memcpy(p->name, name, sizeof(name));
+    p->hip_device = device;
+    p->peer = lk->peer.load(std::memory_order_acquire);
+    if (p->w->magic != kPairMagic || (int)p->w->lanes != g_par.lanes || p->w->sets < 1 || p->w->sets > (uint32_t)kShmSetsMax || p->w->bytes_per_lane < wire_window_cap()) {
+      FL_WARN("NET/FuseLink : the receiver's landing windows (%u sets of %llu bytes per lane, %u lanes) do not fit this side's staging windows (%llu bytes, %d lanes)",
+              p->w->sets, (unsigned long long)p->w->bytes_per_lane, p->w->lanes, (unsigned long long)wire_window_cap(), g_par.lanes);
+      wire_pair_destroy(p);
       return ncclInvalidUsage;
     }
-    FL_HIPCHECK(hipIpcOpenMemHandle((void**)&c->landing, c->w->landing, hipIpcMemLazyEnablePeerAccess));
-    c->sets = (int)c->w->landing_sets;
-    for (int k = 0; k < c->sets; ++k) FL_HIPCHECK(hipEventCreateWithFlags(&c->ev[k], hipEventDisableTiming));
-    shm_landing_windows(c, c->w->landing_bytes_per_lane);
+    DeviceScope keep;
+    hipError_t he = hipSetDevice(device);
+    if (he == hipSuccess) he = hipIpcOpenMemHandle((void**)&p->landing, p->w->landing, hipIpcMemLazyEnablePeerAccess);
+    if (he != hipSuccess) { p->landing = nullptr; wire_pair_destroy(p); return hip_fail("hipIpcOpenMemHandle", he); }
+    p->sets = (int)p->w->sets;
+    wire_landing_windows(p, p->w->bytes_per_lane);
+    p->w->sender_mapped.store(1, std::memory_order_release);
+    g_pairs.push_back(p);
   }
-  ShmRequest* r = shm_get_request(c, kReqSend);
-  if (!r) return ncclInternalError;
-  r->src = (const uint8_t*)data;
-  r->size = (uint64_t)size;
-  r->fifo_idx = c->fifoHead + 1;
-  r->refresh = (fw.flags & 1u) != 0;
-  shm_wire_credits(c, fw, r->credits);
-  memset((void*)&fw, 0, sizeof(FifoWire));   // plugin.cc:1605
-  c->fifoHead++;
-  c->active.push_back(r);
-  *request = r;
+  p->links++;
+  e->pair = p;
+  e->pair_conn = e->w->pair_conn;
+  *ready = true;
   return ncclSuccess;
 }
 
-// The sender's side of the wire (c->mu held): queue waves on the GPU while sets of landing windows are free, announce
-// the waves whose copies have finished.  A wave is the striping launch into this side's staging windows plus one launch
-// that carries every lane's staged bytes into the receiver's landing windows of the wave's set; launches of one stream
-// run in order, so the next wave's striping cannot overtake the copy that still reads the staging windows.
-ncclResult_t shm_progress_send(ShmComm* c) {
-  const uint64_t chunk = (uint64_t)g_par.chunk;
-  DeviceScope keep;
-  bool device_set = false;
-  // announce what has landed: the stand-in for the WRITE_WITH_IMM completions (plugin.cc:1453-1465)
-  while (!c->flights.empty()) {
-    const ShmFlight& f = c->flights.front();
-    hipError_t e = hipEventQuery(c->ev[f.set]);
-    if (e == hipErrorNotReady) break;
-    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
-    if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its staging window (status %d)", *c->h_status); return ncclInternalError; }
-    ShmWave& wv = c->w->wave[c->waves_published % FL_NET_MAX_REQUESTS];
-    wv.fifo_idx = f.fifo_idx;
-    wv.epoch_bytes = f.epoch_bytes;
-    wv.offset = f.offset;
-    wv.bytes = f.bytes;
-    wv.last = f.last;
-    wv.set = f.set;
-    wv.n_req = f.n_req;
-    for (uint32_t q = 0; q < f.n_req && f.n_req > 1; ++q) wv.req_bytes[q] = f.req_bytes[q];
-    c->waves_published++;
-    wv.seq.store(c->waves_published, std::memory_order_release);
-    c->flights.pop_front();
+// ---- sender ---------------------------------------------------------------------------------------------------------
+// Is a set of landing windows free?  (launch_mu held: the only place waves are added.)
+bool wire_set_free(WirePair* p) {
+  uint64_t launched;
+  {
+    std::lock_guard<std::mutex> g(p->tx_mu);
+    launched = p->tx_launched;
   }
-  // queue further waves: a set of landing windows is free once the wave that used it last has been reassembled
-  while (c->cursor < c->active.size()) {
-    ShmRequest* r = c->active[c->cursor];
-    if (r->all_launched) { c->cursor++; continue; }
-    const uint64_t consumed = c->w->waves_consumed.load(std::memory_order_acquire);
-    if (c->waves_launched - consumed >= (uint64_t)c->sets) {
-      if (c->w->recv_closed.load(std::memory_order_acquire)) { FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding"); return ncclRemoteError; }
+  return launched - p->w->waves_consumed.load(std::memory_order_acquire) < (uint64_t)p->sets;
+}
+// the set the next wave lands in, and its number (launch_mu held)
+uint32_t wire_next_set(WirePair* p, uint64_t* wave_no) {
+  std::lock_guard<std::mutex> g(p->tx_mu);
+  *wave_no = p->tx_launched + 1;
+  return (uint32_t)(p->tx_launched % (uint64_t)p->sets);
+}
+// the wave's GPU work has been handed over (launch_mu held)
+void wire_push_flight(WirePair* p, const WireFlight& f) {
+  std::lock_guard<std::mutex> g(p->tx_mu);
+  p->tx_flights.push_back(f);
+  p->tx_launched++;
+}
+
+bool wire_flight_complete(Peer* pr, const WireFlight& f, ncclResult_t* rc);
+
+// Announce the waves whose bytes have landed, in order: the stand-in for the WRITE_WITH_IMM completions
+// (plugin.cc:1453-1465).  Any thread that polls a send of the pair comes through here; one at a time does the work.
+ncclResult_t wire_publish(WirePair* p) {
+  if (!p->tx_mu.try_lock()) return ncclSuccess;
+  ncclResult_t rc = ncclSuccess;
+  while (!p->tx_flights.empty()) {
+    const WireFlight& f = p->tx_flights.front();
+    if (!wire_flight_complete(p->peer, f, &rc)) break;
+    if (rc != ncclSuccess) {   // the wave is lost: nothing behind it can be delivered in order
+      p->w->failed.store(1, std::memory_order_release);
       break;
     }
-    if (r->refresh && r->launched == 0) c->epoch_bytes = 0;
-    uint64_t wave = (uint64_t)wave_chunks(r->credits, g_par.lanes, chunk, c->wins.cap[0], c->epoch_bytes / chunk) * chunk;
-    const uint64_t room = wave;
-    if (wave > r->size - r->launched) wave = r->size - r->launched;
-    const uint32_t set = (uint32_t)(c->waves_launched % (uint64_t)c->sets);
-    if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
-    // Requests behind this one that have not started either, under the same credit row and without a refresh of
-    // their own, share the wave while it has room: together they are one message from the carried prefix on (every
-    // request but the last a whole number of chunks), staged by one launch, carried by one, reassembled by one.  At
-    // NCCL's 512 KiB steps a wave per request costs both sides their launches and events for half a megabyte each.
-    uint32_t n_req = 1;
-    uint64_t total = r->size;
-    if (g_par.wire_batch > 1 && r->launched == 0 && r->size > 0 && r->size <= room) {
-      while ((int)n_req < g_par.wire_batch && c->cursor + n_req < c->active.size()) {
-        const ShmRequest* prev = c->active[c->cursor + n_req - 1];
-        const ShmRequest* t = c->active[c->cursor + n_req];
-        if (prev->size % chunk != 0 || t->refresh || t->size == 0 || t->launched != 0 || t->all_launched ||
-            memcmp(t->credits, r->credits, sizeof(r->credits)) != 0 || total + t->size > room)
-          break;
-        total += t->size;
-        ++n_req;
-      }
-    }
-    if (n_req >= 2) {
-      flh_batch_params b;
-      memset(&b, 0, sizeof(b));
-      fill_uniform(b.u, r->credits, total, 0, c->epoch_bytes, FLH_TILE_BYTES);
-      b.n_req = n_req;
-      ShmFlight f;
-      for (uint32_t q = 0; q < n_req; ++q) {
-        ShmRequest* t = c->active[c->cursor + q];
-        b.d_src[q] = t->src;
-        b.bytes[q] = t->size;
-        f.batch[q] = t;
-        f.req_bytes[q] = t->size;
-      }
-      FL_FLHCHECK(flh_stripe_batch(&b, &c->wins, c->d_table, c->d_hdr, c->d_status, c->stream));
-      c->last_rows = (uint32_t)((total + chunk - 1) / chunk);
-      FlCreditRow row;
-      fl_row_make(r->credits, (uint32_t)g_par.lanes, row);
-      uint64_t lane_bytes[FLH_MAX_LANES];
-      uint32_t lane_chunks[FLH_MAX_LANES];
-      fl_row_lane_totals(row, c->epoch_bytes / chunk, total, chunk, lane_bytes, lane_chunks);
-      FL_FLHCHECK(flh_copy_runs(c->landing_wins[set].base, c->wins.base, lane_bytes, (uint32_t)g_par.lanes, c->stream));
-      FL_HIPCHECK(hipEventRecord(c->ev[set], c->stream));
-      f.req = r;
-      f.fifo_idx = r->fifo_idx;
-      f.epoch_bytes = c->epoch_bytes;
-      f.offset = 0;
-      f.bytes = total;
-      f.set = set;
-      f.last = 1;
-      f.n_req = n_req;
-      c->epoch_bytes += total;
-      c->waves_launched++;
-      for (uint32_t q = 0; q < n_req; ++q) {
-        ShmRequest* t = f.batch[q];
-        t->launched = t->size;
-        t->all_launched = true;
-        t->last_wave = c->waves_launched;
-      }
-      c->flights.push_back(f);
-      continue;   // the cursor steps over the requests at the top of the loop
-    }
-    if (wave) {
-      flh_uniform_params u;
-      fill_uniform(u, r->credits, wave, r->launched, c->epoch_bytes, FLH_TILE_BYTES);
-      FL_FLHCHECK(flh_stripe_uniform(r->src, r->size, &c->wins, &u, c->d_table, c->d_hdr, c->d_status, c->stream));
-      c->last_rows = (uint32_t)((wave + chunk - 1) / chunk);
-      // the wire: every lane's staged bytes into the receiver's landing window of that lane, one launch for all lanes
-      FlCreditRow row;
-      fl_row_make(r->credits, (uint32_t)g_par.lanes, row);
-      uint64_t lane_bytes[FLH_MAX_LANES];
-      uint32_t lane_chunks[FLH_MAX_LANES];
-      fl_row_lane_totals(row, c->epoch_bytes / chunk, wave, chunk, lane_bytes, lane_chunks);
-      FL_FLHCHECK(flh_copy_runs(c->landing_wins[set].base, c->wins.base, lane_bytes, (uint32_t)g_par.lanes, c->stream));
-    }
-    FL_HIPCHECK(hipEventRecord(c->ev[set], c->stream));
-    ShmFlight f;
-    f.req = r;
-    f.fifo_idx = r->fifo_idx;
-    f.epoch_bytes = c->epoch_bytes;
-    f.offset = r->launched;
-    f.bytes = wave;
-    f.set = set;
-    c->epoch_bytes += wave;
-    r->launched += wave;
-    c->waves_launched++;
-    f.last = r->launched >= r->size ? 1u : 0u;
-    if (f.last) { r->all_launched = true; r->last_wave = c->waves_launched; }
-    c->flights.push_back(f);
+    const uint64_t n = p->tx_published.load(std::memory_order_relaxed) + 1;
+    ShmWave& wv = p->w->wave[(n - 1) % kPairWaves];
+    memcpy((char*)&wv + sizeof(wv.seq), (const char*)&f.rec + sizeof(f.rec.seq), sizeof(ShmWave) - sizeof(wv.seq));
+    wv.seq.store(n, std::memory_order_release);
+    p->tx_published.store(n, std::memory_order_release);
+    p->tx_flights.pop_front();
   }
-  return ncclSuccess;
+  p->tx_mu.unlock();
+  return rc;
 }
 
-// The receiver's side (c->mu held): reassemble the waves that have been announced out of their landing windows, and
-// hand the windows back, in order, as the reassembly launches finish.
-ncclResult_t shm_progress_recv(ShmComm* c) {
-  DeviceScope keep;
-  bool device_set = false;
-  while (!c->flights.empty()) {
-    const ShmFlight& f = c->flights.front();
-    hipError_t e = hipEventQuery(c->ev[f.set]);
-    if (e == hipErrorNotReady) break;
-    if (e != hipSuccess) return hip_fail("hipEventQuery", e);
-    if (*(volatile int32_t*)c->h_status != 0) { FL_WARN("NET/FuseLink : a chunk fell outside its landing window or buffer (status %d)", *c->h_status); return ncclInternalError; }
-    if (f.n_req > 1) {
-      for (uint32_t q = 0; q < f.n_req; ++q) { f.batch[q]->received += f.req_bytes[q]; f.batch[q]->complete = true; }
-    } else {
-      f.req->received += f.bytes;
-      if (f.last) f.req->complete = true;
-    }
-    c->waves_done++;
-    c->w->waves_consumed.store(c->waves_done, std::memory_order_release);   // the set's landing windows are free again
-    c->flights.pop_front();
+// ---- receiver -------------------------------------------------------------------------------------------------------
+ncclResult_t wire_deliver(WirePair* p, const ShmWave& wv, WireFlight& f);
+
+// Take the waves that have been announced off the ring and hand their delivery to the GPU; give the landing sets of
+// delivered waves back, in order.  Any thread that polls a receive of the pair comes through here; one at a time works.
+ncclResult_t wire_progress_recv(WirePair* p) {
+  if (!p->rx_mu.try_lock()) return ncclSuccess;
+  ncclResult_t rc = ncclSuccess;
+  Peer* pr = p->peer;
+  if (p->named && p->w->sender_mapped.load(std::memory_order_acquire)) {
+    shm_unlink(p->name);   // both ends hold their mapping: the name is no longer needed and cannot leak
+    p->named = false;
+  }
+  while (!p->rx_flights.empty()) {
+    if (!wire_flight_complete(pr, p->rx_flights.front(), &rc)) break;
+    // (a delivery that failed has failed its requests already; its set goes back all the same)
+    rc = ncclSuccess;
+    p->rx_done++;
+    p->w->waves_consumed.store(p->rx_done, std::memory_order_release);
+    p->rx_flights.pop_front();
   }
   for (;;) {
-    ShmWave& wv = c->w->wave[c->waves_launched % FL_NET_MAX_REQUESTS];
-    if (wv.seq.load(std::memory_order_acquire) != c->waves_launched + 1) {   // nothing further has landed
-      if (c->cursor < c->active.size() && c->w->send_closed.load(std::memory_order_acquire)) {
-        FL_WARN("NET/FuseLink : the sending process closed the connection with a receive outstanding");
-        return ncclRemoteError;
-      }
-      break;
-    }
-    if (c->cursor >= c->active.size()) { FL_WARN("NET/FuseLink : a wave arrived that no posted receive is waiting for"); return ncclInternalError; }
-    ShmRequest* r = c->active[c->cursor];
-    if (wv.fifo_idx != r->fifo_idx) {
-      FL_WARN("NET/FuseLink : a wave of request %llu arrived while %llu is next in line", (unsigned long long)wv.fifo_idx, (unsigned long long)r->fifo_idx);
-      return ncclInternalError;
-    }
-    if (wv.set >= (uint32_t)c->sets) { FL_WARN("NET/FuseLink : a wave in a set of landing windows that does not exist"); return ncclInvalidUsage; }
-    if (wv.n_req > 1) {
-      // several whole requests in one wave: this receive and the ones posted behind it
-      const uint32_t n_req = wv.n_req;
-      if (n_req > FLH_BATCH_MAX || c->cursor + n_req > c->active.size()) { FL_WARN("NET/FuseLink : a wave of %u requests arrived, %zu receives are posted", n_req, c->active.size() - c->cursor); return ncclInternalError; }
-      if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
-      flh_batch_params b;
-      memset(&b, 0, sizeof(b));
-      fill_uniform(b.u, r->credits, wv.bytes, 0, wv.epoch_bytes, FLH_TILE_BYTES);
-      b.n_req = n_req;
-      ShmFlight f;
-      uint64_t sum = 0;
-      for (uint32_t q = 0; q < n_req; ++q) {
-        ShmRequest* t = c->active[c->cursor + q];
-        if (t->fifo_idx != wv.fifo_idx + q || wv.req_bytes[q] > t->size || memcmp(t->credits, r->credits, sizeof(r->credits)) != 0) {
-          FL_WARN("NET/FuseLink : request %u of a wave does not fit the receive posted for it", q);
-          return ncclInvalidUsage;
-        }
-        b.d_dst[q] = t->dst;
-        b.bytes[q] = wv.req_bytes[q];
-        f.batch[q] = t;
-        f.req_bytes[q] = wv.req_bytes[q];
-        sum += wv.req_bytes[q];
-      }
-      if (sum != wv.bytes) { FL_WARN("NET/FuseLink : a wave's requests do not add up to its bytes"); return ncclInvalidUsage; }
-      FL_FLHCHECK(flh_reassemble_batch(&b, &c->landing_wins[wv.set], c->d_status, c->stream));
-      FL_HIPCHECK(hipEventRecord(c->ev[wv.set], c->stream));
-      f.req = r;
-      f.fifo_idx = wv.fifo_idx;
-      f.epoch_bytes = wv.epoch_bytes;
-      f.offset = 0;
-      f.bytes = wv.bytes;
-      f.last = 1;
-      f.set = wv.set;
-      f.n_req = n_req;
-      c->flights.push_back(f);
-      c->waves_launched++;
-      c->cursor += n_req;
-      continue;
-    }
-    if (wv.offset + wv.bytes > r->size) { FL_WARN("NET/FuseLink : a wave past the end of the posted buffer"); return ncclInvalidUsage; }
-    if (!device_set) { FL_HIPCHECK(hipSetDevice(c->hip_device)); device_set = true; }
-    if (wv.bytes) {
-      // the credit row this receiver put into the descriptor: the reassembly launch derives the same lanes and offsets
-      flh_uniform_params u;
-      fill_uniform(u, r->credits, wv.bytes, wv.offset, wv.epoch_bytes, FLH_TILE_BYTES);
-      FL_FLHCHECK(flh_reassemble_uniform(r->dst, r->size, &c->landing_wins[wv.set], &u, c->d_status, c->stream));
-    }
-    FL_HIPCHECK(hipEventRecord(c->ev[wv.set], c->stream));
-    ShmFlight f;
-    f.req = r;
-    f.fifo_idx = wv.fifo_idx;
-    f.epoch_bytes = wv.epoch_bytes;
-    f.offset = wv.offset;
-    f.bytes = wv.bytes;
-    f.last = wv.last;
-    f.set = wv.set;
-    c->flights.push_back(f);
-    c->waves_launched++;
-    if (wv.last) c->cursor++;   // the next wave belongs to the next receive
+    const uint64_t taken = p->rx_taken.load(std::memory_order_relaxed);
+    const ShmWave& wv = p->w->wave[taken % kPairWaves];
+    if (wv.seq.load(std::memory_order_acquire) != taken + 1) break;         // nothing further has landed
+    if (!pr->launch_mu.try_lock()) break;                                    // somebody is launching: next poll
+    WireFlight f;
+    rc = wire_deliver(p, wv, f);
+    pr->launch_mu.unlock();
+    p->rx_taken.store(taken + 1, std::memory_order_release);
+    p->rx_flights.push_back(f);
+    if (rc != ncclSuccess) { p->w->failed.store(1, std::memory_order_release); break; }
   }
-  return ncclSuccess;
+  p->rx_mu.unlock();
+  return rc;
 }
-
-// The table and header that the striping launch of the connection's latest wave wrote (control surface, for tests).
-int shm_last_table(ShmComm* c, void* rows_out, int max_rows, void* hdr_out) {
-  std::lock_guard<std::mutex> g(c->mu);
-  if (!c->gpu_ready || c->last_rows == 0) return fl_set_error(FLH_E_STATE, "the connection has not staged anything yet");
-  DeviceScope keep;
-  if (hipSetDevice(c->hip_device) != hipSuccess) return fl_set_error(FLH_E_HIP, "hipSetDevice failed");
-  if (hipStreamSynchronize(c->stream) != hipSuccess) return fl_set_error(FLH_E_HIP, "stream synchronize failed");
-  const int rows = (int)c->last_rows, take = rows < max_rows ? rows : max_rows;
-  if (take > 0 && rows_out && hipMemcpy(rows_out, c->d_table, sizeof(flh_chunk_desc) * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess)
-    return fl_set_error(FLH_E_HIP, "table copy failed");
-  if (hdr_out && hipMemcpy(hdr_out, c->d_hdr, sizeof(flh_sched_hdr), hipMemcpyDeviceToHost) != hipSuccess)
-    return fl_set_error(FLH_E_HIP, "header copy failed");
-  return rows;
-}
-
-ncclResult_t shm_test(ShmRequest* r, int* done, int* sizes) {
-  *done = 0;
-  ShmComm* c = r->comm;
-  std::lock_guard<std::mutex> g(c->mu);
-  ncclResult_t rc = c->is_send ? shm_progress_send(c) : shm_progress_recv(c);
-  if (rc != ncclSuccess) return rc;
-  if (c->active.empty() || c->active.front() != r) return ncclSuccess;   // requests are reported in the order they were made
-  if (r->type == kReqSend) {
-    // the send is complete once its last wave has been taken out of the landing windows
-    if (!r->all_launched || c->w->waves_consumed.load(std::memory_order_acquire) < r->last_wave) {
-      if (r->all_launched && c->w->recv_closed.load(std::memory_order_acquire)) {
-        FL_WARN("NET/FuseLink : the receiving process closed the connection with a wave outstanding");
-        return ncclRemoteError;
-      }
-      return ncclSuccess;
-    }
-  } else {
-    if (!r->complete) return ncclSuccess;
-    c->r_finished++;
-    c->r_inflight--;
-    if (sizes) sizes[0] = (int)r->received;
-  }
-  c->active.pop_front();
-  if (c->cursor) c->cursor--;
-  r->type = kReqUnused;
-  *done = 1;
-  return ncclSuccess;
-}
-

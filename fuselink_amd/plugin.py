@@ -72,7 +72,7 @@ def _table(version: int):
 
 PLUGIN_SYMBOLS = ["ncclNetPlugin_v8", "ncclNetPlugin_v7", "ncclNetPlugin_v6"]
 CONTROL_SYMBOLS = ["fl_monitor_attach_shm", "fl_monitor_detach", "fl_monitor_is_shared", "fl_monitor_daemon_running", "fl_monitor_reset", "fl_monitor_set_entry", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
-                   "fl_monitor_status", "fl_monitor_idle_pick", "fl_monitor_release", "fl_monitor_credits", "fl_net_set_credits",
+                   "fl_monitor_status", "fl_monitor_idle_pick", "fl_monitor_release", "fl_monitor_credits", "fl_monitor_tx_mask", "fl_monitor_rx_credits", "fl_net_set_credits",
                    "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_launch_stats", "fl_net_last_table", "fl_net_last_launch",
                    "fl_net_flush", "fl_net_host_stats", "fl_net_timeline", "fl_net_reset"]
 

@@ -224,6 +224,13 @@ int fl_monitor_release(int lane, int is_tx);
 /* credits the scheduler will use from the next refresh on: IDLE -> idle_credit, BUSY/BORROWED -> 0,
  * the comm's own lane never below 1 */
 int fl_monitor_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t* credits_out);
+/* The two halves of the lane decision as the plugin takes it.  The sender's half: the usage mask that travels with its
+ * data as imm_data (refreshTxUsage, src/fuselink.h:261-267, a placeholder there; src/plugin.cc:1441-1447, 1463) -- bit l
+ * set when lane l's send side is IDLE in this host's table, the comm's own lane always, every bit from n_lanes on.  The
+ * receiver's half, at its refresh (src/plugin.cc:1710; the mask of getIdleNicRx, src/monitor.h:208-224): idle_credit
+ * for a lane whose receive side is IDLE here and that tx_mask admits, 0 otherwise, the own lane never below 1. */
+int fl_monitor_tx_mask(int n_lanes, int own_lane, uint32_t* mask_out);
+int fl_monitor_rx_credits(int n_lanes, int own_lane, uint32_t idle_credit, uint32_t tx_mask, uint32_t* credits_out);
 
 /* Static credits (one value per lane) overriding the monitor-derived ones; n = 0 removes the
  * override.  The same can be preset with NCCL_FUSELINK_CREDITS="c0,c1,...". */

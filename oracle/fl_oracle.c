@@ -131,6 +131,26 @@ void fl_credits_from_status(const int32_t* status, int n_lanes, int own_lane,
   if (own_lane >= 0 && own_lane < n_lanes && credits[own_lane] == 0) credits[own_lane] = 1;
 }
 
+/* refreshTxUsage (fuselink.h:265-267) is a placeholder that returns 0xffffffff; the mask it stands for is read off the
+ * sender's statuses: bit l set when lane l's send side is IDLE, the comm's own lane always, and every bit from n_lanes
+ * on (so that a table in which nothing is busy gives the placeholder's value). */
+uint32_t fl_tx_usage_mask(const int32_t* tx_status, int n_lanes, int own_lane) {
+  uint32_t mask = n_lanes >= 32 ? 0u : ~0u << n_lanes;
+  for (int l = 0; l < n_lanes && l < 32; ++l)
+    if (tx_status[l] == FLO_NIC_IDLE || l == own_lane) mask |= 1u << l;
+  return mask;
+}
+
+/* The receiver's side of the same decision: getIdleNicRx(group, priority, txAvailable) skips every NIC that the mask does
+ * not admit (monitor.h:214, the call commented out at fuselink.h:240-243); as credits, a lane counts when its receive side
+ * is IDLE and the sender's mask admits it; the own lane never drops below 1. */
+void fl_rx_credits_from_status(const int32_t* rx_status, int n_lanes, int own_lane, uint32_t idle_credit,
+                               uint32_t tx_mask, uint32_t* credits) {
+  for (int l = 0; l < n_lanes; ++l)
+    credits[l] = rx_status[l] == FLO_NIC_IDLE && (l >= 32 || ((tx_mask >> l) & 1u)) ? idle_credit : 0;
+  if (own_lane >= 0 && own_lane < n_lanes && credits[own_lane] == 0) credits[own_lane] = 1;
+}
+
 /* ---- R5: build-defined credit schedule ------------------------------------------------------ */
 int fl_credit_schedule(const uint32_t* sizes, uint64_t total_bytes, uint32_t chunk_bytes,
                        const uint64_t* src_off, uint64_t src_base, uint32_t n, uint32_t n_lanes,

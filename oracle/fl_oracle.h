@@ -19,6 +19,9 @@
  *                     own MonitorClient compiled from monitor.h (oracle/_ref) for mark / pick /
  *                     status and the shared-memory layout; the daemon tick (monitor.cpp needs
  *                     libibverbs headers, absent) is restated and pinned by hand vectors.
+ *   fl_tx_usage_mask / fl_rx_credits_from_status  build-defined content of a reference placeholder
+ *                     (fuselink.h:261-267) -- hand vectors; all-idle gives the placeholder's 0xffffffff; an all-ones
+ *                     mask reduces to fl_credits_from_status; brute force over every status pattern of 4 lanes.
  *   fl_credit_schedule  build-defined (the reference has no weighted scheduler); pinned by the
  *                     five properties listed at its declaration and brute force on tiny inputs.
  *   fl_table_by_lane  build-defined reordering of a finished table (destination order for the striping
@@ -105,6 +108,17 @@ void fl_mon_status(const fl_monitor_t* m, int n_nics, int32_t* out);
  * a BUSY or BORROWED lane gets 0, and the comm's own lane never drops below 1. */
 void fl_credits_from_status(const int32_t* status, int n_lanes, int own_lane,
                             uint32_t idle_credit, uint32_t* credits);
+
+/* Build-defined content of the sender's usage mask, which the reference leaves a placeholder (refreshTxUsage,
+ * fuselink.h:261-267, always 0xffffffff; shipped as imm_data, plugin.cc:1441-1447, 1463; kept by the receiver as
+ * txAvailable, plugin.cc:1884-1885): bit l set when lane l's send side is IDLE or l is the comm's own lane; bits from
+ * n_lanes on are set. */
+uint32_t fl_tx_usage_mask(const int32_t* tx_status, int n_lanes, int own_lane);
+/* ... and what the receiver makes of it at its refresh (plugin.cc:1710; getIdleNicRx's mask, monitor.h:208-224): a lane
+ * gets idle_credit when its receive side is IDLE and the mask admits it; the own lane never below 1.  With a mask of all
+ * ones this is fl_credits_from_status over the receive statuses. */
+void fl_rx_credits_from_status(const int32_t* rx_status, int n_lanes, int own_lane, uint32_t idle_credit,
+                               uint32_t tx_mask, uint32_t* credits);
 
 /* ---- R5 (build-defined): credit-weighted chunk -> lane schedule ------------------------- */
 /*

@@ -73,6 +73,8 @@ def lib() -> C.CDLL:
         "fl_mon_idle_pick_rx": (C.c_int, [C.POINTER(Monitor), C.c_int, C.c_int]),
         "fl_mon_status": (None, [C.POINTER(Monitor), C.c_int, i32p]),
         "fl_credits_from_status": (None, [i32p, C.c_int, C.c_int, C.c_uint32, u32p]),
+        "fl_tx_usage_mask": (C.c_uint32, [i32p, C.c_int, C.c_int]),
+        "fl_rx_credits_from_status": (None, [i32p, C.c_int, C.c_int, C.c_uint32, C.c_uint32, u32p]),
         "fl_credit_schedule": (C.c_int, [vp, C.c_uint64, C.c_uint32, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp,
                                          C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint32, C.c_uint32, vp, vp, vp]),
         "fl_table_by_lane": (C.c_int, [vp, C.c_uint32, C.c_uint32, C.c_uint32, vp]),

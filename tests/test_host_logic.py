@@ -142,6 +142,19 @@ def test_monitor_random_sequences_match_oracle(net):
         L.fl_monitor_credits(8, 3, 4, got)
         O.fl_credits_from_status(st, 8, 3, 4, exp)
         assert list(got)[:8] == list(exp)[:8]
+        # the two halves of the lane decision: the sender's mask off the send statuses, the receiver's row off the
+        # receive statuses and a mask
+        rx = (C.c_int32 * 16)()
+        L.fl_monitor_status(0, 16, rx)
+        mask = C.c_uint32()
+        for own in (-1, 0, 5):
+            assert L.fl_monitor_tx_mask(8, own, C.byref(mask)) == 0
+            assert mask.value == O.fl_tx_usage_mask(st, 8, own)
+            for m_ in (0xffffffff, mask.value, int(rng.integers(0, 1 << 8))):
+                assert L.fl_monitor_rx_credits(8, own, 4, m_, got) == 0
+                O.fl_rx_credits_from_status(rx, 8, own, 4, m_, exp)
+                assert list(got)[:8] == list(exp)[:8]
+    assert L.fl_monitor_tx_mask(0, 0, C.byref(mask)) < 0 and L.fl_monitor_rx_credits(17, 0, 4, 0, got) < 0
 
 
 def test_exact_pick_borrows_only_one(net):

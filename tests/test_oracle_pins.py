@@ -169,6 +169,44 @@ def test_credits_from_status():
     assert list(out) == [2, 0, 0, 2]
 
 
+def test_tx_usage_mask_and_rx_credits():
+    """The content of the reference's placeholder mask (refreshTxUsage, fuselink.h:261-267) and what the receiver makes of
+    it (getIdleNicRx's mask, monitor.h:208-224).  Hand vectors; the all-idle table gives the placeholder's own value; an
+    all-ones mask reduces the receiver's half to fl_credits_from_status; and every status pattern of four lanes against
+    the definition evaluated in Python."""
+    IDLE, BUSY, BORROWED = 0, 1, 2
+    st = (C.c_int32 * 4)(IDLE, BUSY, BORROWED, IDLE)
+    assert L.fl_tx_usage_mask(st, 4, 1) == 0xfffffffb          # lane 2 borrowed: out; lane 1 busy but the comm's own: in
+    assert L.fl_tx_usage_mask(st, 4, 0) == 0xfffffff9
+    assert L.fl_tx_usage_mask((C.c_int32 * 8)(), 8, 5) == 0xffffffff   # nothing busy: the placeholder's value (fuselink.h:262)
+    out = (C.c_uint32 * 4)()
+    L.fl_rx_credits_from_status(st, 4, 1, 4, 0xffffffff, out)
+    assert list(out) == [4, 1, 0, 4]
+    L.fl_rx_credits_from_status(st, 4, 1, 4, 0xfffffff6, out)   # the sender's lanes 0 and 3 are busy
+    assert list(out) == [0, 1, 0, 0]
+    L.fl_rx_credits_from_status(st, 4, 3, 2, 0xfffffff7, out)   # a masked own lane still keeps one credit
+    assert list(out) == [2, 0, 0, 1]
+    import itertools
+    ref = (C.c_uint32 * 4)()
+    for pattern in itertools.product((IDLE, BUSY, BORROWED), repeat=4):
+        st = (C.c_int32 * 4)(*pattern)
+        for own in (-1, 0, 2):
+            exp_mask = 0xfffffff0
+            for l, v in enumerate(pattern):
+                if v == IDLE or l == own:
+                    exp_mask |= 1 << l
+            assert L.fl_tx_usage_mask(st, 4, own) == exp_mask
+            L.fl_credits_from_status(st, 4, own, 3, ref)
+            L.fl_rx_credits_from_status(st, 4, own, 3, 0xffffffff, out)
+            assert list(out) == list(ref)
+            for mask in (0x0, 0x5, 0xa, 0xf):
+                L.fl_rx_credits_from_status(st, 4, own, 3, mask, out)
+                exp = [3 if v == IDLE and (mask >> l) & 1 else 0 for l, v in enumerate(pattern)]
+                if 0 <= own < 4 and exp[own] == 0:
+                    exp[own] = 1
+                assert list(out) == exp
+
+
 # ---- R5: credit schedule ---------------------------------------------------------------------------------
 def _run_sched_vector(v, fn):
     kw = dict(n_lanes=v["n_lanes"], credits=v["credits"], quantum=v["quantum"], epoch_len=v["epoch_len"], tile_bytes=v["tile_bytes"])
