@@ -101,6 +101,10 @@ struct Params {
   int batch_wait_ns = 2000;      // NCCL_FUSELINK_BATCH_WAIT_NS: a small matched send waits this long for company before a test launches it
   int wire_sets = 4;             // NCCL_FUSELINK_WIRE_SETS: sets of landing windows a receiving process keeps per sending process and GPU = waves on the wire at once
   int wire = 0;                  // NCCL_FUSELINK_WIRE: 0 = both ends in this process (loopback), 1 = the other end is another process (shared-memory wire)
+  // NCCL_FUSELINK_WIRE_DIRECT: 1 = a receiver exports the allocations it registers (under 2 GiB) and the sender's second
+  // copy writes into the posted buffer itself, as an RDMA write lands in registered memory; 0 = every wave goes through
+  // the landing windows and the receiver's own engine or launches deliver it
+  int wire_direct = 1;
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
 };
 Params g_par;
@@ -318,6 +322,7 @@ struct Pending {
   uint64_t fifo_idx = 0;     // the descriptor it answers, from 1
   int q_next = 0;            // a send to another process that travels wave by wave: the QP piece it has got to ...
   uint64_t q_done = 0;       // ... and the bytes of that piece that are on their way
+  bool direct = false;       // a send to another process whose posted buffer this process can write itself (dst is that mapping)
 };
 
 // What one launch pair carried, for inspection (fl_net_last_launch).
@@ -448,6 +453,10 @@ struct MemHandle {             // FuseLinkMemHandle, fuselink.h:48-52
   size_t size = 0;
   flh_region* region = nullptr;  // shared per base allocation (device memory only)
   int device = -1;               // HIP device that owns the memory (-1: host memory)
+  // registered on a receiving comm whose sender is another process: the key under which that process may write into
+  // the allocation directly (0: it cannot), and the pair of processes the key belongs to
+  WirePair* wire_pair = nullptr;
+  uint32_t rkey = 0;
 };
 
 struct Handle {                // what listen writes into the caller's 128 bytes (plugin.cc:425-430)
@@ -773,6 +782,7 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
     g_par.wire = wv && (!strcmp(wv, "shm") || !strcmp(wv, "1")) ? 1 : 0;
   }
   g_par.wire_sets = (int)fl_param("FUSELINK_WIRE_SETS", g_par.wire_sets);
+  g_par.wire_direct = (int)fl_param("FUSELINK_WIRE_DIRECT", g_par.wire_direct) != 0;
   if (g_par.wire_sets < 1) g_par.wire_sets = 1;
   if (g_par.wire_sets > kShmSetsMax) g_par.wire_sets = kShmSetsMax;
   g_par.engine = (int)fl_param("FUSELINK_ENGINE", g_par.engine);
@@ -968,6 +978,10 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
       std::lock_guard<ShortLock> g(c->link->mu);
       rc = c->is_send ? attach_peer(c->link, mh->device) : wire_recv_setup(c->link, mh->device);
       if (rc != ncclSuccess) { (void)flh_region_release(mh->region); delete mh; return rc; }
+      if (wire && !c->is_send) {   // the sender may write into this allocation itself (plugin.cc:1626, 1655: address and rkey go into the descriptor)
+        mh->wire_pair = c->link->wire->pair;
+        wire_export_mr(mh->wire_pair, base, bsz, &mh->rkey);
+      }
     }
   } else if (type == NCCL_PTR_HOST) {
     // page-aligned span, plugin.cc:1181-1182, 1206-1209; host memory is not staged
@@ -992,6 +1006,7 @@ ncclResult_t fl_reg_mr_v8(void* comm, void* data, size_t size, int type, void** 
 ncclResult_t fl_dereg_mr(void* /*comm*/, void* mhandle) {
   MemHandle* mh = (MemHandle*)mhandle;
   if (!mh || mh->magic != kMhMagic) return ncclInvalidArgument;
+  if (mh->rkey) wire_unexport_mr(mh->wire_pair, mh->rkey);
   if (mh->region) {
     int left = flh_region_release(mh->region);  // destroyed on the last reference, plugin.cc:1347-1403
     if (left < 0) { FL_WARN("NET/FuseLink : region release: %s", flh_last_error()); return ncclInternalError; }
@@ -1269,11 +1284,13 @@ size_t build_batch(Peer* pr, size_t i, BatchBuild& bb, bool engine) {
   FlCreditRow row;                           // its credit row
   uint32_t chunks_closed = 0;
   size_t j = i;
-  WirePair* const pair = work[i].lk->wire ? work[i].lk->wire->pair : nullptr;   // a batch stays on one wire: this process, or one pair
+  // a batch stays on one wire and travels one way: this process, or one pair of processes, into the posted buffers or through the landing windows
+  WirePair* const pair = work[i].lk->wire ? work[i].lk->wire->pair : nullptr;
+  const bool direct = work[i].direct;
   while (j < work.size() && b.n_req < (uint32_t)g_par.batch) {
     const Pending& p = work[j];
     if (!(p.src_dev && p.dst_dev) || p.size == 0) break;
-    if ((p.lk->wire ? p.lk->wire->pair : nullptr) != pair) break;
+    if ((p.lk->wire ? p.lk->wire->pair : nullptr) != pair || p.direct != direct) break;
     // where the request's connection stands in its epoch: behind its earlier segments of this batch, if any
     uint64_t epoch = p.lk->epoch_bytes;
     for (uint32_t k = 0; k < b.n_seg; ++k) if (bb.seg_link[k] == p.lk) epoch = bb.link_epoch_after[k];
@@ -1353,6 +1370,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
   // a receiver in another process: the batch is a wave of the pair's wire and lands in one of its sets (the caller has
   // made sure that one is free)
   WirePair* const pair = pr->work[i].lk->wire ? pr->work[i].lk->wire->pair : nullptr;
+  const bool carry = pair && !pr->work[i].direct;   // (a batch whose posted buffers this process can write itself is staged and delivered here, like a loopback one)
   uint64_t wave_no = 0;
   const uint32_t set = pair ? wire_next_set(pair, &wave_no) : 0;
   if (engine) {
@@ -1365,7 +1383,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     const uint64_t starts_before = g_par.trace ? flh_engine_launches(pr->engine) : 0;
     const int64_t t_sub = g_par.trace ? tr_now() : 0;
     const flh_windows* ewin = &pr->ewins[k % (uint64_t)pr->engine_sets];
-    const int frc = pair ? flh_engine_submit_wire(pr->engine, FLH_ENGINE_SEND, &b, ewin, &pair->landing_wins[set], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot,
+    const int frc = carry ? flh_engine_submit_wire(pr->engine, FLH_ENGINE_SEND, &b, ewin, &pair->landing_wins[set], pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot,
                                                   pr->d_status, &got, &seg_base[0][0])
                          : flh_engine_submit(pr->engine, &b, ewin, pr->d_etable + (size_t)slot * kEngineRows, pr->d_ehdr + slot, pr->d_status, &got, &seg_base[0][0]);
     if (g_par.trace) {   // submits that had to start the resident kernel are counted apart: they pay for a launch
@@ -1381,7 +1399,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     seq = got;
     pr->engine_reqs_upto[got % kEngineSlots].store(pr->engine_reqs_upto[(got - 1) % kEngineSlots].load(std::memory_order_relaxed) + b.n_req, std::memory_order_relaxed);
     pr->engine_submitted.store(got, std::memory_order_release);
-  } else if (pair) {
+  } else if (carry) {
     start_stamp(pr, seq, b.u);
     Completion comp;
     ncclResult_t rc = prepare_completion(pr, seq, b.u.total_bytes, b.u, comp);   // the carrying launch is the last of the path on this side
@@ -1407,6 +1425,7 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     f.rec.set = set;
     f.rec.n_req = b.n_req;
     f.rec.n_seg = b.n_seg;
+    f.rec.direct = carry ? 0u : 1u;
     f.rec.total_bytes = b.u.total_bytes;
     for (uint32_t q = 0; q < b.n_req; ++q) {
       const Pending& p = pr->work[i + q];
@@ -1558,7 +1577,27 @@ void flush_pending(Peer* pr) {
           rc = launch_batch(pr, i, span, bb, false, seq);
         }
       }
-      if (wave_by_wave && pair) {
+      if (wave_by_wave && pair && p.direct) {
+        // its posted buffer is mapped here: waves through this process's windows and straight into it, in stream order,
+        // then one record for the receiver
+        seq = pr->launch_seq.load(std::memory_order_relaxed) + 1;
+        pr->launch_seq.store(seq, std::memory_order_release);
+        rc = launch_transfer(pr, p, seq);
+        if (rc == ncclSuccess) {
+          uint64_t wave_no;
+          WireFlight f;
+          f.seq = seq;
+          f.rec.set = wire_next_set(pair, &wave_no);
+          f.rec.n_req = 1;
+          f.rec.n_seg = 1;
+          f.rec.direct = 1;
+          f.rec.total_bytes = (uint64_t)p.size;
+          f.rec.req[0] = WaveReq{p.lk->wire->pair_conn, p.imm, p.fifo_idx, (uint64_t)p.size};
+          f.rec.seg[0] = WaveSeg{p_epoch, 1, 0};
+          wire_push_flight(pair, f);
+          p.sreq->wave = wave_no;
+        }
+      } else if (wave_by_wave && pair) {
         bool park = false;
         rc = launch_transfer_wire(pr, p, pair, &park);   // numbers its launches itself, one per wave
         seq = p.sreq->seq;
@@ -1692,7 +1731,9 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     lk->fifoHead++;                              // plugin.cc:1607
     lk->s_inflight++;
   }
-  uint8_t* dst = wire ? nullptr : (uint8_t*)(uintptr_t)w.addr;
+  // the receiver's buffer: its address in this process; across processes, where its registration is mapped here (if it
+  // is: otherwise null, and the bytes travel through the landing windows)
+  uint8_t* dst = wire ? (size ? wire_map_mr(wire->pair, w.rkey, w.addr, (uint64_t)size) : nullptr) : (uint8_t*)(uintptr_t)w.addr;
   const bool src_dev = mh->type == NCCL_PTR_CUDA, dst_dev = rtype == NCCL_PTR_CUDA;
   // the comm's own NIC carried traffic (updateTxChannelActive, fuselink.h:247-252)
   mark_nic_active(lk->dev % g_par.lanes, 1);
@@ -1716,6 +1757,7 @@ ncclResult_t fl_isend(void* sendComm, void* data, int size, int tag, void* mhand
     p.rreq = rreq;
     p.imm = imm;
     p.fifo_idx = fifo_idx;
+    p.direct = wire && dst != nullptr;
     sreq->state.store(kStQueued, std::memory_order_release);
     if (rreq) rreq->state.store(kStQueued, std::memory_order_release);
     tl_event(2, (uint64_t)lk->channelId);
@@ -1792,7 +1834,7 @@ ncclResult_t fl_irecv(void* recvComm, int n, void** data, int* sizes, int* tags,
   // ncclIbPostFifo, plugin.cc:1616-1677
   fs.w.addr = (uint64_t)(uintptr_t)data[0];
   fs.w.size = sizes[0];
-  fs.w.rkey = 1;
+  fs.w.rkey = !wire ? 1u : (mh->wire_pair == wire->pair ? mh->rkey : 0u);   // across processes: the key to write the buffer directly, if there is one
   fs.w.nreqs = (uint32_t)n;
   fs.w.tag = (uint32_t)tags[0];
   fs.w.fuselink_offset = lk->fuselink_offset;
@@ -1991,8 +2033,10 @@ ncclResult_t wire_deliver(WirePair* p, const ShmWave& wv, WireFlight& f) {
   bool by_engine = false;
   uint64_t seq = 0;
   ncclResult_t rc = ncclSuccess;
-  if (sum == 0) {
-    // a send of no bytes: nothing to deliver
+  const bool nothing = sum == 0 || wv.direct != 0;
+  if (nothing) {
+    // a send of no bytes, or bytes that the sender has written into the posted buffers itself (they were in memory
+    // before it announced the wave): nothing to deliver
   } else {
     uint64_t rows = 0;
     for (uint32_t i = 0; i < n_req; ++i) rows += (b.bytes[i] + chunk - 1) / chunk;
@@ -2042,14 +2086,14 @@ ncclResult_t wire_deliver(WirePair* p, const ShmWave& wv, WireFlight& f) {
     }
   }
   f.engine = by_engine;
-  f.seq = sum == 0 || rc != ncclSuccess ? 0 : seq;
+  f.seq = nothing || rc != ncclSuccess ? 0 : seq;
   if (wv.piece && !wv.last && rc == ncclSuccess) return ncclSuccess;   // the request's later pieces complete it
   for (uint32_t i = 0; i < n_req; ++i) {
     Request* r = reqs[i];
     r->seq = seq;
     r->engine = by_engine;
     if (rc != ncclSuccess) r->fault = 1;
-    r->state.store(sum == 0 || rc != ncclSuccess ? kStDoneHost : kStLaunched, std::memory_order_release);
+    r->state.store(nothing || rc != ncclSuccess ? kStDoneHost : kStLaunched, std::memory_order_release);
   }
   return rc;
 }

@@ -39,6 +39,7 @@ constexpr uint32_t kShmListenMagic = 0x464c534c;              // "FLSL"
 constexpr int kShmSetsMax = 8;
 constexpr uint32_t kPairWaves = 64;      // wave records a pair's ring holds (more than the landing sets there can be)
 constexpr uint32_t kPairConns = 256;     // connections between two processes that share the pair
+constexpr uint32_t kPairMrs = 64;        // registrations of the receiver that the sender can write into directly
 
 struct WaveReq {                   // one request of a wave
   uint32_t conn;                   // the connection's number within the pair
@@ -58,10 +59,19 @@ struct ShmWave {                   // one wave that has landed in the receiver's
   uint32_t piece;                  // 1: part of ONE request that the windows do not hold whole: `offset` and `last` apply
   uint64_t offset;                 // byte offset of the piece in the request
   uint32_t last;                   // the request's last piece
-  uint32_t pad;
+  uint32_t direct;                 // 1: the bytes are already in the posted buffers (written through the registrations' rkeys): nothing to deliver
   uint64_t total_bytes;
   WaveReq req[FLH_BATCH_MAX];
   WaveSeg seg[FLH_SEG_MAX];
+};
+// A registration of the receiver that the sender may write into directly, as an RDMA write lands in the receiver's
+// registered memory (plugin.cc:1485-1486: remote_addr and rkey come from the descriptor): the whole allocation around
+// the registered buffer, exported through HIP IPC.  The descriptor's rkey names the entry and its generation.
+struct ShmMr {
+  std::atomic<uint32_t> gen;       // odd while the registration stands; moves on when it goes
+  uint32_t pad;
+  uint64_t base, size;             // in the receiver's address space
+  hipIpcMemHandle_t handle;
 };
 struct ShmPair {                   // one per (sending process, receiving process, GPU of the receiver)
   uint64_t magic;
@@ -72,6 +82,7 @@ struct ShmPair {                   // one per (sending process, receiving proces
   std::atomic<uint32_t> sender_mapped;   // the sender holds its mapping: the name is no longer needed
   std::atomic<uint32_t> failed;          // a wave was lost (the sender's engine went down): every request on the pair fails
   alignas(64) std::atomic<uint64_t> waves_consumed;   // receiver: waves delivered so far, in order (their landing sets are free again)
+  alignas(64) ShmMr mr[kPairMrs];
   alignas(64) ShmWave wave[kPairWaves];
 };
 struct ShmWire {                   // one per connection
@@ -119,6 +130,10 @@ struct WirePair {                  // this process's end of a pair
   std::atomic<uint64_t> rx_taken{0};            // waves taken off the ring
   uint64_t rx_done = 0;                         // waves delivered
   std::atomic<Link*> conns[kPairConns] = {};    // this process's end of every connection of the pair, by its number
+  // registrations that can be written directly (mr_mu): the receiver's reference counts by allocation, the sender's mappings
+  std::mutex mr_mu;
+  struct { uint64_t base; int refs; } mr_local[kPairMrs] = {};
+  struct { uint8_t* ptr; uint32_t gen; uint64_t base, size; } mr_map[kPairMrs] = {};
 };
 
 struct WireEnd {                   // a connection's end of the wire (Link::wire)
@@ -141,6 +156,13 @@ std::mutex g_pair_mu;              // the pairs of this process, their attachmen
 std::vector<WirePair*> g_pairs;
 
 void wire_pair_destroy(WirePair* p) {   // no longer reachable through g_pairs
+  for (auto& m : p->mr_map) {
+    if (!m.ptr) continue;
+    DeviceScope keep;
+    (void)hipSetDevice(p->hip_device);
+    (void)hipIpcCloseMemHandle(m.ptr);
+    m.ptr = nullptr;
+  }
   if (p->landing) {
     DeviceScope keep;
     (void)hipSetDevice(p->hip_device);
@@ -435,6 +457,77 @@ ncclResult_t wire_send_setup(Link* lk, int device, bool* ready) {
   e->pair_conn = e->w->pair_conn;
   *ready = true;
   return ncclSuccess;
+}
+
+// ---- registrations the sender writes into directly --------------------------------------------------------------------
+bool wire_pair_alive(WirePair* p) {   // g_pair_mu held
+  for (WirePair* q : g_pairs) if (q == p) return true;
+  return false;
+}
+// Receiver, at regMr: export the allocation [base, base + bytes) to the pair's sender.  *rkey stays 0 when that is not
+// possible (switched off, 2 GiB or more -- what HIP IPC carries reliably here --, memory the runtime cannot export, table
+// full): such a buffer is reached through the landing windows instead.
+void wire_export_mr(WirePair* p, void* base, size_t bytes, uint32_t* rkey) {
+  *rkey = 0;
+  if (!g_par.wire_direct || bytes >= (2ull << 30)) return;
+  std::lock_guard<std::mutex> g(p->mr_mu);
+  int at = -1;
+  for (uint32_t i = 0; i < kPairMrs; ++i) {
+    if (p->mr_local[i].refs > 0 && p->mr_local[i].base == (uint64_t)(uintptr_t)base && p->w->mr[i].size == bytes) {
+      p->mr_local[i].refs++;
+      *rkey = ((p->w->mr[i].gen.load(std::memory_order_relaxed) & 0xffffffu) << 8) | (i + 1);
+      return;
+    }
+    if (at < 0 && p->mr_local[i].refs == 0) at = (int)i;
+  }
+  if (at < 0) return;
+  ShmMr& m = p->w->mr[at];
+  DeviceScope keep;
+  if (hipSetDevice(p->hip_device) != hipSuccess || hipIpcGetMemHandle(&m.handle, base) != hipSuccess) {
+    (void)hipGetLastError();   // not an error of the registration: the landing windows carry it
+    return;
+  }
+  m.base = (uint64_t)(uintptr_t)base;
+  m.size = bytes;
+  const uint32_t old = m.gen.load(std::memory_order_relaxed);
+  const uint32_t gen = (old & 1u) ? old + 2 : old + 1;
+  m.gen.store(gen, std::memory_order_release);   // odd: the entry stands
+  p->mr_local[at].base = m.base;
+  p->mr_local[at].refs = 1;
+  *rkey = ((gen & 0xffffffu) << 8) | ((uint32_t)at + 1);
+}
+void wire_unexport_mr(WirePair* p, uint32_t rkey) {
+  std::lock_guard<std::mutex> ga(g_pair_mu);
+  if (!wire_pair_alive(p)) return;   // the pair went with its last connection, and the table with it
+  const uint32_t i = (rkey & 0xffu) - 1;
+  if (i >= kPairMrs) return;
+  std::lock_guard<std::mutex> g(p->mr_mu);
+  if (p->mr_local[i].refs > 0 && --p->mr_local[i].refs == 0) p->w->mr[i].gen.fetch_add(1, std::memory_order_release);   // even: gone
+}
+// Sender: where `bytes` at the receiver's address `addr` lie in this process, through the registration `rkey` names;
+// null when it cannot be reached that way (the caller then sends through the landing windows).  Opens the receiver's
+// allocation on first use.
+uint8_t* wire_map_mr(WirePair* p, uint32_t rkey, uint64_t addr, uint64_t bytes) {
+  const uint32_t i = (rkey & 0xffu) - 1, gen = rkey >> 8;
+  if (!g_par.wire_direct || rkey == 0 || i >= kPairMrs) return nullptr;
+  std::lock_guard<std::mutex> g(p->mr_mu);
+  auto& m = p->mr_map[i];
+  if (!m.ptr || m.gen != gen) {
+    DeviceScope keep;
+    if (hipSetDevice(p->hip_device) != hipSuccess) return nullptr;
+    if (m.ptr) { (void)hipIpcCloseMemHandle(m.ptr); m.ptr = nullptr; }
+    const ShmMr& sm = p->w->mr[i];
+    const uint32_t now = sm.gen.load(std::memory_order_acquire);
+    if ((now & 0xffffffu) != gen || !(now & 1u) || sm.size >= (2ull << 30)) return nullptr;
+    void* ptr = nullptr;
+    if (hipIpcOpenMemHandle(&ptr, sm.handle, hipIpcMemLazyEnablePeerAccess) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    m.ptr = (uint8_t*)ptr;
+    m.gen = gen;
+    m.base = sm.base;
+    m.size = sm.size;
+  }
+  if (addr < m.base || addr + bytes > m.base + m.size) return nullptr;
+  return m.ptr + (addr - m.base);
 }
 
 // ---- sender ---------------------------------------------------------------------------------------------------------

@@ -157,32 +157,39 @@ def _waves(table, lanes, window_bytes, chunk):
     return starts
 
 
-def test_cfg1_shape_tables_and_bytes_across_two_processes():
+DIRECT = pytest.mark.parametrize("direct", [1, 0])   # written into the posted buffers through their registrations / through the landing windows
+
+
+@DIRECT
+def test_cfg1_shape_tables_and_bytes_across_two_processes(direct):
     # the reference's experiment: 4 MiB in 512 KiB chunks over 2 lanes; then requests that start mid-round and a ragged one
     chunk = 512 << 10
-    _run_pair({"NCCL_FUSELINK_LANES": 2, "NCCL_FUSELINK_CHUNKSIZE": chunk, "NCCL_FUSELINK_CREDITS": "1,1", "NCCL_FUSELINK_REFRESH_BATCH": 1000},
+    _run_pair({"NCCL_FUSELINK_LANES": 2, "NCCL_FUSELINK_CHUNKSIZE": chunk, "NCCL_FUSELINK_CREDITS": "1,1", "NCCL_FUSELINK_REFRESH_BATCH": 1000, "NCCL_FUSELINK_WIRE_DIRECT": direct},
               [4 << 20, 5 * chunk, 3 * chunk + 777, chunk], seed=31, credits=[1, 1], lanes=2, chunk=chunk, window_bytes=8 << 20)
 
 
-def test_cfg2_shape_tables_and_bytes_across_two_processes():
+@DIRECT
+def test_cfg2_shape_tables_and_bytes_across_two_processes(direct):
     # 64 MiB in 256 KiB chunks over 8 lanes with uneven credits; windows of 56 MiB per lane hold the message in one wave
     chunk = 256 << 10
     credits = [8, 6, 7, 1, 8, 7, 3, 3]
     _run_pair({"NCCL_FUSELINK_LANES": 8, "NCCL_FUSELINK_CHUNKSIZE": chunk, "NCCL_FUSELINK_CREDITS": ",".join(map(str, credits)),
-               "NCCL_FUSELINK_WINDOW_UNITS": 28, "NCCL_FUSELINK_REFRESH_BATCH": 1000},
+               "NCCL_FUSELINK_WINDOW_UNITS": 28, "NCCL_FUSELINK_REFRESH_BATCH": 1000, "NCCL_FUSELINK_WIRE_DIRECT": direct},
               [64 << 20, 9 * chunk + 5], seed=32, credits=credits, lanes=8, chunk=chunk, window_bytes=56 << 20)
 
 
-def test_waves_through_small_windows_across_two_processes():
+@DIRECT
+def test_waves_through_small_windows_across_two_processes(direct):
     # 2 MiB windows per lane, three sets of landing windows: requests of several waves, the table is the last wave's
     chunk = 128 << 10
     credits = [3, 1, 2, 2]
     _run_pair({"NCCL_FUSELINK_LANES": 4, "NCCL_FUSELINK_CHUNKSIZE": chunk, "NCCL_FUSELINK_CREDITS": ",".join(map(str, credits)),
-               "NCCL_FUSELINK_WINDOW_UNITS": 1, "NCCL_FUSELINK_WIRE_SETS": 3, "NCCL_FUSELINK_REFRESH_BATCH": 1000},
+               "NCCL_FUSELINK_WINDOW_UNITS": 1, "NCCL_FUSELINK_WIRE_SETS": 3, "NCCL_FUSELINK_REFRESH_BATCH": 1000, "NCCL_FUSELINK_WIRE_DIRECT": direct},
               [20 << 20, (7 << 20) + 4321, 3 * chunk], seed=33, credits=credits, lanes=4, chunk=chunk, window_bytes=2 << 20)
 
 
-def test_requests_that_wait_together_share_a_wave_across_two_processes():
+@DIRECT
+def test_requests_that_wait_together_share_a_wave_across_two_processes(direct):
     """NCCL keeps eight 512 KiB steps in flight; a wave per request would cost both processes their launches and events
     for half a megabyte each.  Requests that wait together, of whole chunks and under one credit row, travel as one wave:
     staged by one launch as one message from the carried prefix on, carried by one, reassembled by one.  The receiver
@@ -194,7 +201,7 @@ def test_requests_that_wait_together_share_a_wave_across_two_processes():
     credits = [3, 1, 2, 2]
     sizes = [3 * chunk, 4 * chunk, 2 * chunk, 8 * chunk, 3 * chunk + 999, chunk]      # first on its own, four together (the last of them ragged), one behind
     env = dict(os.environ, NCCL_FUSELINK_WIRE="shm", PYTHONPATH=ROOT, NCCL_FUSELINK_LANES=str(lanes), NCCL_FUSELINK_CHUNKSIZE=str(chunk),
-               NCCL_FUSELINK_CREDITS=",".join(map(str, credits)), NCCL_FUSELINK_REFRESH_BATCH="1000", NCCL_FUSELINK_WIRE_BATCH="4")
+               NCCL_FUSELINK_CREDITS=",".join(map(str, credits)), NCCL_FUSELINK_REFRESH_BATCH="1000", NCCL_FUSELINK_WIRE_DIRECT=str(direct))
     child = subprocess.Popen([sys.executable, "-c", _RECEIVER, json.dumps(sizes), "34", "ahead"], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
                              stderr=subprocess.PIPE, text=True, env=env, cwd=ROOT)
     keys = ["NCCL_FUSELINK_WIRE"] + list(env_keys(env))

@@ -116,57 +116,65 @@ def test_plugin_host_path_under_address_sanitizer():
 
 # ---- sender and receiver in two processes ----------------------------------------------------------------------------
 # The receiver is a child forked before either side has loaded the plugin or touched the GPU; the two meet through the
-# 128-byte handle alone (a POSIX shared-memory object named in it carries the descriptor ring and the wave completions,
-# the receiver's landing windows are opened by the sender through HIP IPC).  The child compares what it received with
-# the pattern of the iteration and reports through its exit status.
+# 128-byte handle alone (a POSIX shared-memory object named in it carries the descriptor ring; a second one, per pair of
+# processes, the wave completions; the receiver's memory is opened by the sender through HIP IPC).  The child compares
+# what it received with the pattern of the iteration and reports through its exit status.  Every shape runs both ways a
+# wave can travel: written by the sender into the posted buffers through their registrations (NCCL_FUSELINK_WIRE_DIRECT=1,
+# the default) and through the landing windows, delivered by the receiver's own engine or launches (0).
+DIRECT = pytest.mark.parametrize("direct", [1, 0])
+
 
 @pytest.mark.gpu
-def test_two_processes_cfg1_shape():
+@DIRECT
+def test_two_processes_cfg1_shape(direct):
     # the reference's own experiment: 4 MiB in 512 KiB chunks over 2 lanes, one request per NCCL step
     out = _run(["--two-process", "--bytes", str(4 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "3"],
-               env={"NCCL_FUSELINK_LANES": "2", "NCCL_FUSELINK_CHUNKSIZE": str(512 << 10), "NCCL_FUSELINK_CREDITS": "1,1"})
+               env={"NCCL_FUSELINK_LANES": "2", "NCCL_FUSELINK_CHUNKSIZE": str(512 << 10), "NCCL_FUSELINK_CREDITS": "1,1", "NCCL_FUSELINK_WIRE_DIRECT": str(direct)})
     assert out["harness"] == "plugin_two_process" and out["bit_exact"] and out["requests"] == 8
     print(out)
 
 
 @pytest.mark.gpu
-def test_two_processes_cfg2_shape():
+@DIRECT
+def test_two_processes_cfg2_shape(direct):
     # 64 MiB in 256 KiB chunks over 8 lanes with uneven credits, one request; the windows hold the message in one wave
     out = _run(["--two-process", "--bytes", str(64 << 20), "--request", str(64 << 20), "--inflight", "1", "--iters", "3"],
                env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "28",
-                    "NCCL_FUSELINK_CREDITS": "8,6,7,1,8,7,3,3"})
+                    "NCCL_FUSELINK_CREDITS": "8,6,7,1,8,7,3,3", "NCCL_FUSELINK_WIRE_DIRECT": str(direct)})
     assert out["harness"] == "plugin_two_process" and out["bit_exact"] and out["requests"] == 1
     print(out)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("sets", [1, 2, 5])
-def test_two_processes_requests_larger_than_the_windows_and_a_ragged_tail(sets):
+@pytest.mark.parametrize("sets,direct", [(1, 0), (2, 0), (5, 0), (2, 1)])
+def test_two_processes_requests_larger_than_the_windows_and_a_ragged_tail(sets, direct):
     # every request takes several waves through the landing windows (4 units per lane; `sets` sets of them, so that many
     # waves are on the wire at once), the last request is short and odd
     out = _run(["--two-process", "--bytes", str((96 << 20) + 12345), "--request", str(32 << 20), "--inflight", "2", "--iters", "2"],
                env={"NCCL_FUSELINK_LANES": "4", "NCCL_FUSELINK_CHUNKSIZE": str(128 << 10), "NCCL_FUSELINK_WINDOW_UNITS": "4",
-                    "NCCL_FUSELINK_CREDITS": "3,1,2,2", "NCCL_FUSELINK_WIRE_SETS": str(sets)})
+                    "NCCL_FUSELINK_CREDITS": "3,1,2,2", "NCCL_FUSELINK_WIRE_SETS": str(sets), "NCCL_FUSELINK_WIRE_DIRECT": str(direct)})
     assert out["bit_exact"] and out["requests"] == 4
     print(out)
 
 
 @pytest.mark.gpu
-def test_two_processes_many_small_requests_in_flight():
+@DIRECT
+def test_two_processes_many_small_requests_in_flight(direct):
     # NCCL's request shape across the process boundary: 512 KiB requests, 8 in flight, more requests than the descriptor
     # ring and the wave ring have slots (both wrap)
     out = _run(["--two-process", "--bytes", str(192 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "2"],
-               env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10), "NCCL_FUSELINK_WIRE_SETS": "4"})
+               env={"NCCL_FUSELINK_LANES": "8", "NCCL_FUSELINK_CHUNKSIZE": str(256 << 10), "NCCL_FUSELINK_WIRE_SETS": "4", "NCCL_FUSELINK_WIRE_DIRECT": str(direct)})
     assert out["bit_exact"] and out["requests"] == 384
     print(out)
 
 
 @pytest.mark.gpu
-def test_two_processes_kv_handoff_group():
+@DIRECT
+def test_two_processes_kv_handoff_group(direct):
     # the prefill -> decode hand-off of the serving experiment (experiments/serving/model.hh:286-309), where the two are
     # different processes: five messages (int64 context output, K cache, V cache, int64 block table, int64 counts), each
     # a buffer and a registration of its own on either side, tiny and large mixed, cut into 512 KiB requests
-    out = _run(["--two-process", "--handoff", "4,8,2,8,16,128", "--request", str(512 << 10), "--inflight", "8", "--iters", "2"])
+    out = _run(["--two-process", "--handoff", "4,8,2,8,16,128", "--request", str(512 << 10), "--inflight", "8", "--iters", "2"], env={"NCCL_FUSELINK_WIRE_DIRECT": str(direct)})
     cache = 2 * 32 * 2 * 8 * 16 * 128
     assert out["bit_exact"] and out["group"] == "kv_handoff" and out["messages"] == 5
     assert out["bytes"] == 2 * cache + 8 * 4 + 8 * 32 + 8 * 4 and out["requests"] == 1 + 4 + 4 + 1 + 1
