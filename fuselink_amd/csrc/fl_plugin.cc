@@ -676,8 +676,8 @@ ncclResult_t attach_peer(Link* lk, int device) {
 // Credit row the receiver advertises at a refresh: refreshRxComm(channelId, txAvailable, ...) of plugin.cc:1710 with the
 // query the reference left commented out (fuselink.h:240-243, getIdleNicRx(group, priority, txAvailable)) -- a lane
 // counts when its receive side is idle in this host's table and the sender's mask admits it.  tx_available is the mask
-// that came with the latest completed receive.  Both ends in one process read one table, so there the receiver also
-// looks at the send statuses as they are now (what the sender's next mask will say).
+// that came with the latest completed receive.  Both ends in one process read one table: there the receiver reads the
+// send statuses themselves, as they are now, in place of the sender's last report of them (which is up to a batch old).
 void current_credits(int own_lane, uint32_t tx_available, bool same_process, uint8_t* out) {
   uint32_t c[FL_NET_MAX_LANES] = {};
   {
@@ -687,8 +687,8 @@ void current_credits(int own_lane, uint32_t tx_available, bool same_process, uin
     } else {
       // the daemon's periodic ageing (monitor.cpp:159-193) happens here, right before the table is read
       (void)fl_monitor_tick(fl_monitor_now());
-      uint32_t mask = tx_available, now_mask = 0xffffffffu;
-      if (same_process && fl_monitor_tx_mask(g_par.lanes, own_lane, &now_mask) == 0) mask &= now_mask;
+      uint32_t mask = tx_available;
+      if (same_process) (void)fl_monitor_tx_mask(g_par.lanes, own_lane, &mask);
       (void)fl_monitor_rx_credits(g_par.lanes, own_lane, (uint32_t)g_par.idle_credit, mask, c);
     }
   }
