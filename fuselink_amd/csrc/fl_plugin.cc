@@ -2392,6 +2392,27 @@ int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64
   return FLH_OK;
 }
 
+int fl_net_mask_stats(void* comm, uint32_t* mask, int64_t* refreshes) {
+  Comm* c = (Comm*)comm;
+  if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
+  Link* lk = c->link;
+  std::lock_guard<ShortLock> g(lk->mu);
+  if (mask) *mask = c->is_send ? lk->tx_mask : lk->tx_available;
+  if (refreshes) *refreshes = c->is_send ? lk->tx_refreshes : lk->refreshes;
+  return FLH_OK;
+}
+
+int fl_net_free_requests(void* comm) {
+  Comm* c = (Comm*)comm;
+  if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");
+  Link* lk = c->link;
+  std::lock_guard<ShortLock> g(lk->mu);
+  const Request* tab = c->is_send ? lk->sreq : lk->rreq;
+  int n = 0;
+  for (int i = 0; i < FL_NET_MAX_REQUESTS; ++i) n += tab[i].type == kReqUnused;
+  return n;
+}
+
 int fl_net_launch_stats(void* comm, int64_t* launches, int64_t* batched_requests) {
   Comm* c = (Comm*)comm;
   if (!c || c->magic != kCommMagic) return fl_set_error(FLH_E_ARG, "not a send or recv comm");

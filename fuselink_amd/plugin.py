@@ -73,7 +73,7 @@ def _table(version: int):
 PLUGIN_SYMBOLS = ["ncclNetPlugin_v8", "ncclNetPlugin_v7", "ncclNetPlugin_v6"]
 CONTROL_SYMBOLS = ["fl_monitor_attach_shm", "fl_monitor_detach", "fl_monitor_is_shared", "fl_monitor_daemon_running", "fl_monitor_reset", "fl_monitor_set_entry", "fl_monitor_set_clock", "fl_monitor_now", "fl_monitor_mark_active", "fl_monitor_tick",
                    "fl_monitor_status", "fl_monitor_idle_pick", "fl_monitor_release", "fl_monitor_credits", "fl_monitor_tx_mask", "fl_monitor_rx_credits", "fl_net_set_credits",
-                   "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_launch_stats", "fl_net_last_table", "fl_net_last_launch",
+                   "fl_net_inject_fault", "fl_net_comm_stats", "fl_net_mask_stats", "fl_net_free_requests", "fl_net_launch_stats", "fl_net_last_table", "fl_net_last_launch",
                    "fl_net_flush", "fl_net_host_stats", "fl_net_timeline", "fl_net_reset"]
 
 
@@ -117,6 +117,10 @@ class NetPlugin:
         L.fl_net_inject_fault.argtypes = [VP]
         L.fl_net_comm_stats.argtypes = [VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         L.fl_net_launch_stats.argtypes = [VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+        L.fl_net_mask_stats.argtypes = [VP, C.POINTER(C.c_uint32), C.POINTER(C.c_int64)]
+        L.fl_net_free_requests.argtypes = [VP]
+        L.fl_monitor_tx_mask.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_uint32)]
+        L.fl_monitor_rx_credits.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32)]
         L.fl_net_last_table.argtypes = [VP, VP, C.c_int, VP]
         L.fl_net_last_launch.argtypes = [VP, C.POINTER(LaunchSeg), C.c_int, VP, C.c_int, VP]
         L.fl_net_flush.argtypes = [VP]
@@ -262,6 +266,14 @@ class NetPlugin:
         a, b, c = C.c_int64(), C.c_int64(), C.c_int64()
         assert self.lib.fl_net_comm_stats(comm, C.byref(a), C.byref(b), C.byref(c)) == 0
         return {"n_finished": a.value, "in_flight": b.value, "refreshes": c.value}
+
+    def mask_stats(self, comm):
+        m, n = C.c_uint32(), C.c_int64()
+        assert self.lib.fl_net_mask_stats(comm, C.byref(m), C.byref(n)) == 0
+        return {"mask": m.value, "refreshes": n.value}
+
+    def free_requests(self, comm) -> int:
+        return self.lib.fl_net_free_requests(comm)
 
     def launch_stats(self, comm):
         a, b = C.c_int64(), C.c_int64()

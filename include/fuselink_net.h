@@ -242,6 +242,14 @@ int fl_net_reset(void);
 int fl_net_inject_fault(void* request);
 /* Counters of a send or recv comm: n_finished (src/plugin.cc:517,568), requests in flight, lane refreshes. */
 int fl_net_comm_stats(void* comm, int64_t* n_finished, int64_t* in_flight, int64_t* refreshes);
+/* The lane-availability mask of a connection.  On a send comm: the mask it ships with its requests (imm_data of
+ * src/plugin.cc:1463; getTxUsage / refreshTxUsage, src/fuselink.h:261-267) and how often it has been refreshed, which
+ * happens before every send for which (n_finished + 1) % N_FINISHED_BATCH == 0 (src/plugin.cc:1443).  On a recv comm: the
+ * mask that came with the latest completed receive (comm->txAvailable, src/plugin.cc:1884-1885), which its next refresh
+ * ANDs into the credit row (src/plugin.cc:1710), and the number of lane refreshes. */
+int fl_net_mask_stats(void* comm, uint32_t* mask, int64_t* refreshes);
+/* Free slots of the comm's request table (256 when nothing is in flight, src/plugin.cc:382, 1070-1090). */
+int fl_net_free_requests(void* comm);
 /* Launch pairs (stripe + reassemble) that carried requests of the connection so far, and how many of its requests
  * travelled in a pair shared with other requests (its own or another connection's).  Matched sends of all connections
  * that stage on one GPU wait in one queue until a test() finds fewer than two launches queued on that GPU, or until

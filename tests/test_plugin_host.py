@@ -312,6 +312,97 @@ def test_injected_wire_fault_surfaces_in_test(net):
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
+def test_a_failed_request_is_freed_and_the_connection_goes_on(net):
+    """The reference returns from a failed completion with the request still allocated (src/plugin.cc:1839-1861); its
+    communicator is dead after that.  Here the connection lives on, so the request must be freed and counted: with the
+    default cadence of 8 a receive left in flight would hold every later refresh back for ever.  Fault on request 5 of
+    20: its test reports ncclRemoteError once, the 19 others arrive, the refreshes at 8 and 16 happen, and both request
+    tables are back to 256 free slots."""
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(20 * 64, 11)
+    dst = np.zeros(20 * 64, dtype=np.uint8)
+    _, smh = net.regMr(s, sp, src.size, P.NCCL_PTR_HOST)
+    _, rmh = net.regMr(r, dst.ctypes.data, dst.size, P.NCCL_PTR_HOST)
+    assert net.free_requests(s) == 256 and net.free_requests(r) == 256
+    failed = 0
+    for k in range(20):
+        rreq = None
+        for _ in range(1000):
+            rc, rreq = net.irecv(r, [dst.ctypes.data + 64 * k], [64], [k], [rmh])
+            assert rc == 0
+            if rreq:
+                break
+        assert rreq, f"receive {k} was never accepted: the refresh gate stayed shut"
+        rc, sreq = net.isend(s, sp + 64 * k, 64, k, smh)
+        assert rc == 0 and sreq
+        if k == 5:
+            assert net.lib.fl_net_inject_fault(rreq) == 0
+        net.wait(sreq)
+        rc, done, _ = net.test(rreq)
+        if k == 5:
+            assert rc == P.ncclRemoteError and done == 0
+            failed += 1
+            rc, _, _ = net.test(rreq)
+            assert rc == P.ncclInternalError          # the request is no longer in flight
+        else:
+            assert rc == 0 and done == 1
+    assert failed == 1
+    st = net.comm_stats(r)
+    assert st["n_finished"] == 20 and st["in_flight"] == 0 and st["refreshes"] == 3      # at 0, 8 and 16
+    assert net.free_requests(s) == 256 and net.free_requests(r) == 256
+    np.testing.assert_array_equal(dst, src)
+    net.deregMr(s, smh), net.deregMr(r, rmh)
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+
+
+def test_the_senders_mask_is_refreshed_on_the_references_cadence_and_reaches_the_receiver(net):
+    """The sender's lane-availability mask (refreshTxUsage / getTxUsage, src/fuselink.h:261-267, placeholders there) is
+    refreshed before every send for which (n_finished + 1) % 8 == 0 (src/plugin.cc:1441-1447), travels as the request's
+    immediate data (1463) and is kept by the receiver when the receive completes (1884-1885).  With the clock in hand: a
+    lane whose send side is busy drops out of the mask at the next refresh, not before, and comes back at the one after
+    its stamp has aged out."""
+    from tests import oracle_binding as ob
+    O = ob.lib()
+    L = net.lib
+    assert net.reconfigure(NCCL_FUSELINK_LANES=8) is None
+    lcomm, s, r = net.connect_pair(2)                    # the comm's own lane is 2
+    src, sp = _host(64, 12)
+    dst = np.zeros(64, dtype=np.uint8)
+    _, smh = net.regMr(s, sp, 64, P.NCCL_PTR_HOST)
+    _, rmh = net.regMr(r, dst.ctypes.data, 64, P.NCCL_PTR_HOST)
+    t = 3_000_000
+    try:
+        L.fl_monitor_set_clock(1, t)
+        L.fl_monitor_set_entry(5, 1, 1, t + 2000)        # lane 5's send side: BUSY until t + 2160
+        due = 0
+        for k in range(40):
+            if k == 20:
+                L.fl_monitor_set_clock(1, t + 3000)      # ... by now it has aged out
+            before = net.mask_stats(s)
+            rreq = None
+            while not rreq:
+                rc, rreq = net.irecv(r, [dst.ctypes.data], [64], [k], [rmh])
+                assert rc == 0
+            rc, sreq = net.isend(s, sp, 64, k, smh)
+            assert rc == 0 and sreq
+            after = net.mask_stats(s)
+            refreshed = after["refreshes"] - before["refreshes"]
+            assert refreshed == O.fl_refresh_tx_due(k), k                 # n_finished == k here: one request at a time
+            due += refreshed
+            # the placeholder's value until the first refresh, then what the send statuses said at the latest one
+            exp = 0xffffffff if k < 7 else (0xffffffdf if k < 23 else 0xffffffff)
+            assert after["mask"] == exp, (k, hex(after["mask"]))
+            net.wait(sreq), net.wait(rreq)
+            assert net.mask_stats(r)["mask"] == exp                        # comm->txAvailable = imm_data
+        assert due == 5
+    finally:
+        L.fl_monitor_set_clock(0, 0)
+        L.fl_monitor_reset()
+        net.deregMr(s, smh), net.deregMr(r, rmh)
+        net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+        net.reconfigure(NCCL_FUSELINK_LANES=None)
+
+
 def test_cuda_pointer_fails_loudly_without_gpu(net):
     import torch
     if torch.cuda.is_available():
