@@ -38,6 +38,13 @@ WORKLOADS = {
 MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134277565, "cfg5_stress_1GiB_64KiB_16lanes": 2148014006,
                     "cfg5_stress_1GiB_64KiB_16lanes/17 waves": 126482128,
                     "cfg3_expert_parallel_256_blocks_8lanes": 1786029836, "cfg4_paged_kv_2x4096_pages_8lanes": 268579065}
+# ... and the summary under profiles/ that each figure comes from (the counters are not read by this script: `traffic` is
+# a recorded measurement of the same kernel on the same workload, the file holds the commands that made it)
+TRAFFIC_SOURCE = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": "profiles/copy_kernels_cfg2_l2_fabric_traffic.md",
+                  "cfg5_stress_1GiB_64KiB_16lanes": "profiles/copy_kernels_cfg5_l2_fabric_traffic.md",
+                  "cfg5_stress_1GiB_64KiB_16lanes/17 waves": "profiles/copy_kernels_cfg5_l2_fabric_traffic.md",
+                  "cfg3_expert_parallel_256_blocks_8lanes": "profiles/copy_kernels_cfg3_l2_fabric_traffic.md",
+                  "cfg4_paged_kv_2x4096_pages_8lanes": "profiles/page_kernels_cfg4_l2_fabric_traffic.md"}
 
 
 def algo_bytes_cold(nbytes: int) -> int:
@@ -151,6 +158,34 @@ def main() -> int:
                 else:
                     plugin[key] = None
                 plugin[key + "_command"] = " ".join(os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd)
+            # Sender and receiver in different processes (NCCL_FUSELINK_WIRE=shm; the harness forks the receiver before either
+            # side has loaded the plugin or touched the GPU): NCCL's request shape, 64 MiB requests, and the five messages of
+            # the serving experiment's KV hand-off.  Payload bytes over the wall time of the best iteration, as a user of the
+            # connection sees it; "landing_windows" is the same shape with the receiver's registrations not exported.
+            two = {"accounting": "payload bytes / wall time of the best iteration, measured in the sending process from its first isend to its last completed send",
+                   "env": "NCCL_FUSELINK_LANES=8 NCCL_FUSELINK_CHUNKSIZE=262144 (the harness sets NCCL_FUSELINK_WIRE=shm)"}
+            shapes = {
+                "two_process_512KiB_x8_256MiB": (["--two-process", "--bytes", str(256 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "10"], {}),
+                "two_process_64MiB_x4_1GiB": (["--two-process", "--bytes", str(1 << 30), "--request", str(64 << 20), "--inflight", "4", "--iters", "6"], {}),
+                "two_process_kv_handoff": (["--two-process", "--handoff", "8,64,4,8,16,128", "--request", str(512 << 10), "--inflight", "8", "--iters", "6"], {}),
+                "two_process_512KiB_x8_256MiB_landing_windows": (["--two-process", "--bytes", str(256 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "10"],
+                                                                 {"NCCL_FUSELINK_WIRE_DIRECT": "0"}),
+                "two_process_64MiB_x4_1GiB_landing_windows": (["--two-process", "--bytes", str(1 << 30), "--request", str(64 << 20), "--inflight", "4", "--iters", "6"],
+                                                              {"NCCL_FUSELINK_WIRE_DIRECT": "0"}),
+            }
+            for key, (argv, extra) in shapes.items():
+                cmd = [harness, flbuild.lib_path(), *argv]
+                try:
+                    res = subprocess.run(cmd, capture_output=True, text=True, timeout=180, env=dict(env, **extra))
+                    line = json.loads(res.stdout.strip().splitlines()[-1]) if res.returncode == 0 else None
+                except Exception:
+                    line = None
+                if line and line.get("bit_exact"):
+                    two[key] = {"GBps_payload": line["GBps_payload_best"], "best_s": line["best_s"], "mean_s": line["mean_s"], "requests": line["requests"], "bit_exact": True}
+                else:
+                    two[key] = None
+                two[key + "_command"] = " ".join([f"{k}={v}" for k, v in extra.items()] + [os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd])
+            plugin["two_process"] = two
             # what one batch costs the lane engine on its own (no plugin around it): eight 512 KiB requests per batch
             ebench = os.path.join(ROOT, "tests", "harness", "engine_bench")
             if os.path.exists(ebench):
@@ -457,6 +492,55 @@ def main() -> int:
                 "command": cold_cmd}
         del srcs, dsts
 
+    # ---- the same two kernels with HBM as the only server: one launch pair over 1 GiB in 64 KiB chunks on 16 lanes (the
+    # stress configuration's shape under one credit row; 3 GiB of source, windows and destination, so nothing of one
+    # launch is left in the 256 MB Infinity Cache for the next).  Goes into `roofline` beside the headline kernel's
+    # fraction, which the cache helps.
+    hbm_only = None
+    if args.cold_user_buffers and fused and kind == "uniform" and nbytes <= (128 << 20):
+        hb_n, hb_chunk, hb_lanes = 1 << 30, 64 << 10, 16
+        hb_row = rng.integers(1, 9, size=hb_lanes).astype(np.int32).tolist()
+        hb_src = torch.randint(0, 2**31 - 1, (hb_n // 4,), dtype=torch.int32, device=dev, generator=gen).view(torch.uint8)
+        hb_dst = torch.zeros(hb_n, dtype=torch.uint8, device=dev)
+        hb_s = core.schedule(n_lanes=hb_lanes, credits=hb_row, quantum=hb_chunk, total_bytes=hb_n, chunk_bytes=hb_chunk, stream=stream)
+        stream.synchronize()
+        hb_lane_bytes = [int(b) for b in hb_s.hdr_numpy()["lane_bytes"][:hb_lanes]]
+        hb_pool = core.Pool(0, sum((b + core.UNIT_BYTES - 1) // core.UNIT_BYTES for b in hb_lane_bytes))
+        hb_windows = []
+        for b in hb_lane_bytes:
+            w = core.Window(hb_pool, max(b, 1))
+            w.bind(b)
+            hb_windows.append(w)
+        hb_win = core.make_windows([w.base for w in hb_windows], [w.bound_bytes for w in hb_windows])
+        hb_uni = core.uniform_params(hb_n, hb_chunk, hb_row)
+        hb_reps = 8
+
+        def hb_pairs():
+            for _ in range(hb_reps):
+                core.stripe_uniform(hb_src, hb_win, hb_uni, status, stream=stream)
+                core.reassemble_uniform(hb_dst, hb_win, hb_uni, status, stream=stream)
+
+        def hb_copies():
+            for _ in range(hb_reps):
+                core.copy(hb_dst, hb_src, stream=stream)
+
+        hb_pairs()
+        per_h = profiled(hb_pairs, 4 * hb_reps)
+        hb_copy_us = mean(profiled(hb_copies, 2 * hb_reps)["copy"])
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0 and torch.equal(hb_src, hb_dst)
+        hb_frac = lambda us: round(2 * hb_n / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+        hbm_only = {"message_bytes": hb_n, "chunk_bytes": hb_chunk, "lanes": hb_lanes, "footprint_bytes": 3 * hb_n,
+                    "stripe_us": round(mean(per_h["stripe"]), 1), "stripe_frac": hb_frac(mean(per_h["stripe"])),
+                    "reassemble_us": round(mean(per_h["reassemble"]), 1), "reassemble_frac": hb_frac(mean(per_h["reassemble"])),
+                    "plain_copy_us": round(hb_copy_us, 1), "plain_copy_frac": hb_frac(hb_copy_us),
+                    "timing": f"HIP events around every launch, mean of {hb_reps} launch pairs back to back, measured in this run",
+                    "command": "python bench.py"}
+        del hb_src, hb_dst
+        for w in hb_windows:
+            w.destroy()
+        hb_pool.destroy()
+
     # ---- the scheduler kernels on a list long enough for a per-1000-chunk rate: the stress configuration's ----
     sched_bench = None
     if args.scheduler_bench:
@@ -552,12 +636,17 @@ def main() -> int:
                      # what the fraction means for this workload: cached footprints are served in part by the 256 MB Infinity Cache
                      "note": ("footprint (source, windows, destination) of %d MiB: %s" % (
                          3 * nbytes >> 20, "largely resident in the 256 MB Infinity Cache, so this is a fraction of the HBM peak reached with that cache's help; "
-                         "the same kernels with nothing cache-resident reach 0.74-0.76 (bench.py --workload cfg5_stress_1GiB_64KiB_16lanes --cache-waves 0)"
+                         "the same kernels with HBM as the only server are in hbm_only (measured in this run; as a whole workload: bench.py --workload cfg5_stress_1GiB_64KiB_16lanes --cache-waves 0)"
                          if 3 * nbytes <= (256 << 20) else "beyond the 256 MB Infinity Cache" + (
                              "; moved in cache-resident waves, the windows' traffic stays in the cache" if cwaves else ": every byte is served by HBM"))) if kind == "uniform" else None,
                      "traffic": (None if args.lanes else MEASURED_TRAFFIC.get(f"{args.workload}/{len(cwaves)} waves") if cwaves else None if (waves or twaves) else
                                  MEASURED_TRAFFIC.get(args.workload) if (kind != "blocks" or args.blocks == 256) else None)},
     }
+    if out["roofline"]["traffic"] is not None:
+        # a recorded measurement (two rocprofv3 --pmc runs, scaled by a plain copy of known size), not read in this run
+        out["roofline"]["traffic_source"] = TRAFFIC_SOURCE.get(f"{args.workload}/{len(cwaves)} waves" if cwaves else args.workload)
+    if hbm_only is not None:
+        out["roofline"]["hbm_only"] = hbm_only
 
     # ---- CPU baseline: the oracle's host-memcpy striping on a bounded sample ------------------------
     if not args.no_cpu_baseline:

@@ -41,7 +41,10 @@ def lib_path() -> str:
 
 def build_library(verbose: bool = True) -> str:
     os.makedirs(LIBDIR, exist_ok=True)
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    srcs = [os.path.join(CSRC, s) for s in SOURCES]
+    missing = [s for s in srcs if not os.path.exists(s)]
+    if missing:
+        raise RuntimeError("library sources missing: " + ", ".join(missing))
     cmd = [hipcc(), *FLAGS, "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, *srcs, "-o", lib_path(), "-ldl"]
     if verbose:
         print(" ".join(cmd), flush=True)

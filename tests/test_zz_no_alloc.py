@@ -56,6 +56,53 @@ def test_static_workspace_scheduler_equals_lent_workspace_twice_in_a_row():
         state = got_s                                   # the second call carries on from the first
 
 
+def test_static_workspace_scheduler_allocates_nothing_and_replays_from_a_graph():
+    """What the header promises of flh_schedule_static beyond its results: the call takes no device memory (the driver's
+    count of free memory reads the same before and after a run of calls whose buffers all exist beforehand), and it can
+    be recorded into a HIP graph -- a capture refuses any allocation -- and replayed with new sizes in the same buffers,
+    every replay checked against the oracle, with eager work and synchronizations of the program's own in between."""
+    import torch
+
+    from fuselink_amd import _lib, core
+    core.init(0)
+    lib = _lib.load()
+    rng = np.random.default_rng(4711)
+    lanes, n, quantum, tile = 9, 12000, 2048, 4096
+    credits = rng.integers(0, 6, size=(3, lanes)).astype(np.uint32)
+    sizes = torch.zeros(n, dtype=torch.int32, device="cuda")
+    d_credits = _dev(torch, credits.view(np.int32))
+    out = core.new_schedule_buffers(n, tile_bytes=tile)
+    p = _lib.SchedParams()
+    p.d_sizes, p.n_chunks, p.n_lanes = sizes.data_ptr(), n, lanes
+    p.d_credits, p.n_rows, p.epoch_len, p.quantum, p.tile_bytes = d_credits.data_ptr(), 3, 1000, quantum, tile
+    p.d_table, p.d_hdr = out.table.data_ptr(), out.hdr.data_ptr()
+    side = torch.cuda.Stream()
+    s_ptr = C.c_void_p(side.cuda_stream)
+    _lib.check(lib.flh_schedule_static(C.byref(p), s_ptr))      # (first call on the device: the workspace's address is resolved)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(20):
+        _lib.check(lib.flh_schedule_static(C.byref(p), s_ptr))
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"device memory moved by {free_before - free_after} bytes across 20 calls"
+
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _lib.check(lib.flh_schedule_static(C.byref(p), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    for rep in range(4):
+        sizes_np = rng.integers(0, 5000, size=n).astype(np.uint32)
+        sizes.copy_(torch.from_numpy(sizes_np.view(np.int32)))
+        out.table.zero_()                                       # eager work of the program's own between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=quantum, sizes=sizes_np, epoch_len=1000, tile_bytes=tile)
+        assert out.table_numpy().tobytes() == exp_t.tobytes(), f"replay {rep}"
+        np.testing.assert_array_equal(out.hdr_numpy()["lane_bytes"], exp_h["lane_bytes"], err_msg=f"replay {rep}")
+
+
 def test_static_workspace_scheduler_refuses_lists_beyond_its_limit():
     import torch
 
