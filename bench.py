@@ -186,6 +186,22 @@ def main() -> int:
                     two[key] = None
                 two[key + "_command"] = " ".join([f"{k}={v}" for k, v in extra.items()] + [os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd])
             plugin["two_process"] = two
+            # The plugin beside an application's own streams: eight more streams of the process kept busy with small fills
+            # while one connection moves 1 GiB at NCCL's request shape.  More streams than hardware queues, so some share a
+            # queue with the plugin's: how long a fill takes from launch to completion shows how long the plugin's kernels
+            # (the resident lane engine above all) hold a queue.
+            cmd = [harness, flbuild.lib_path(), "--bytes", str(1 << 30), "--request", str(512 << 10), "--inflight", "8", "--iters", "3", "--side-streams", "8"]
+            try:
+                res = subprocess.run(cmd, capture_output=True, text=True, timeout=180, env=env)
+                rows = {l["harness"]: l for l in (json.loads(x) for x in res.stdout.strip().splitlines() if x.startswith("{"))} if res.returncode == 0 else {}
+            except Exception:
+                rows = {}
+            if rows.get("plugin", {}).get("bit_exact") and "side_streams" in rows:
+                plugin["beside_8_busy_streams"] = {"GBps_4N": rows["plugin"]["GBps_4N_best"], "fills": rows["side_streams"]["fills"],
+                                                   "fill_us_mean": rows["side_streams"]["fill_us_mean"], "fill_us_max": rows["side_streams"]["fill_us_max"], "bit_exact": True}
+            else:
+                plugin["beside_8_busy_streams"] = None
+            plugin["beside_8_busy_streams_command"] = " ".join(os.path.relpath(c, ROOT) if os.path.isabs(c) else c for c in cmd)
             # what one batch costs the lane engine on its own (no plugin around it): eight 512 KiB requests per batch
             ebench = os.path.join(ROOT, "tests", "harness", "engine_bench")
             if os.path.exists(ebench):

@@ -86,7 +86,12 @@ struct Params {
   int engine_units = 2;          // staging units per lane for each of the engine's window sets
   int engine_sets = 3;           // window sets the engine's batches rotate through = batches it has in flight at once
   int engine_idle_us = 200;      // the engine goes down after this long without work
-  int engine_resident_us = 2000; // NCCL_FUSELINK_ENGINE_RESIDENT_US: ... and after this long even with work (0 = never), so that its hardware queue drains; the next batch starts it again
+  // NCCL_FUSELINK_ENGINE_RESIDENT_US: ... and after this long even with work (0 = never), so that its hardware queue
+  // drains; the next batch starts it again.  With eight more streams of the process busy beside the plugin's (more streams
+  // than hardware queues), a small fill on one of them waited up to 5.0 ms behind an engine that stayed for as long as
+  // requests came, 2.0 ms with a bound of 2000, 0.85 ms with 500 (0.80 ms with no engine at all); the request rate is the
+  // same within the spread of runs.
+  int engine_resident_us = 500;
   int engine_workgroups = 0;     // 0 = the library's default
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
@@ -106,6 +111,7 @@ struct Params {
   // the landing windows and the receiver's own engine or launches deliver it
   int wire_direct = 1;
   int trace = 0;                 // NCCL_FUSELINK_TRACE=1: time spent inside the entry points (fl_net_host_stats)
+  int test_early_send = 0;       // NCCL_FUSELINK_TEST_EARLY_SEND=1 under NCCL_FUSELINK_TEST_HOOKS=1: timing experiment, see fl_test
 };
 Params g_par;
 
@@ -777,6 +783,10 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.small_tile = (int)fl_param("FUSELINK_SMALL_TILE", g_par.small_tile);
   if (g_par.small_tile < 0 || g_par.small_tile % 128) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_SMALL_TILE must be a multiple of 128"); return ncclInvalidArgument; }
   g_par.trace = (int)fl_param("FUSELINK_TRACE", g_par.trace);
+  {
+    const char* hooks = getenv("NCCL_FUSELINK_TEST_HOOKS");
+    g_par.test_early_send = hooks && !strcmp(hooks, "1") && fl_param("FUSELINK_TEST_EARLY_SEND", 0) != 0;
+  }
   {
     const char* wv = getenv("NCCL_FUSELINK_WIRE");
     g_par.wire = wv && (!strcmp(wv, "shm") || !strcmp(wv, "1")) ? 1 : 0;
@@ -2164,6 +2174,10 @@ ncclResult_t fl_test(void* request, int* done, int* sizes) {
     }
   }
   if (st == kStQueued) return ncclSuccess;
+  // Timing experiment, behind the test-hook switch: report a send complete as soon as its batch has been handed over.
+  // Unsafe for a real caller (the source may still be read), but it bounds from above what any earlier completion of
+  // sends -- when their bytes are staged, say -- could be worth to the request rate.
+  if (g_par.test_early_send && st == kStLaunched && r->type == kReqSend && !pair) st = kStDoneHost;
   if (st == kStLaunched && r->engine) {
     // the engine stores the number of the last complete batch to a pinned word: a plain load, as for the launches' words
     const uint64_t e_done = flh_engine_completed(pr->engine);

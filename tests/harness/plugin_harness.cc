@@ -4,7 +4,11 @@
 // number of requests in flight.  Verifies the received buffer byte for byte and prints one JSON line.
 //
 //   plugin_harness <lib.so> [--bytes N] [--request N] [--inflight K] [--iters I] [--host] [--version 6|7|8] [--connections C]
-//                  [--handoff batch,blocks_per_req,layers,kv_heads,block_size,head_dim] [--two-process]
+//                  [--handoff batch,blocks_per_req,layers,kv_heads,block_size,head_dim] [--two-process] [--side-streams S]
+// With --side-streams S, a thread of the harness keeps S more HIP streams of the process busy with small fills while the
+// connections run -- the application's own compute streams beside the plugin's -- and reports how long a fill took from
+// its launch to its completion (mean and worst).  A process has fewer hardware queues than that many streams, so some of
+// them share a queue with the plugin's streams: what they wait for is how long the plugin's kernels hold a queue.
 // With --two-process the receiver is a child process forked before either side has touched the GPU or loaded the plugin:
 // the child listens and sends the 128-byte handle to the parent over a socket pair (NCCL's bootstrap does that between
 // ranks), the parent connects with it, and from then on the two processes share nothing but what the plugin itself set up
@@ -179,6 +183,44 @@ static void run_connection(int ci, ncclNet_v8_t* net8, ncclNet_v7_t* net7, ncclN
   for (Msg& g : msgs) { if (host) { free(g.src); free(g.dst); } else { HIP(hipFree(g.src)); HIP(hipFree(g.dst)); } }
   (void)bytes;
 }
+
+// ---- the application's own streams beside the plugin's ----------------------------------------------------------------
+struct SideStreams {
+  int n = 0;
+  std::atomic<bool> stop{false};
+  std::thread th;
+  double mean_us = 0, max_us = 0;
+  long ops = 0;
+  void start(int streams) {
+    n = streams;
+    th = std::thread([this]() {
+      HIP(hipSetDevice(0));
+      std::vector<hipStream_t> st(n);
+      std::vector<void*> buf(n);
+      for (int i = 0; i < n; ++i) { HIP(hipStreamCreateWithFlags(&st[i], hipStreamNonBlocking)); HIP(hipMalloc(&buf[i], 4096)); }
+      double sum = 0;
+      while (!stop.load(std::memory_order_acquire)) {
+        for (int i = 0; i < n; ++i) {
+          const auto t0 = std::chrono::steady_clock::now();
+          HIP(hipMemsetAsync(buf[i], i, 4096, st[i]));
+          HIP(hipStreamSynchronize(st[i]));
+          const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+          sum += us;
+          if (us > max_us) max_us = us;
+          ++ops;
+        }
+        std::this_thread::sleep_for(std::chrono::microseconds(50));
+      }
+      mean_us = ops ? sum / ops : 0;
+      for (int i = 0; i < n; ++i) { HIP(hipStreamDestroy(st[i])); HIP(hipFree(buf[i])); }
+    });
+  }
+  void finish() {
+    if (!n) return;
+    stop.store(true, std::memory_order_release);
+    th.join();
+  }
+};
 
 // ---- two processes ------------------------------------------------------------------------------------------------
 static void fill_pattern(std::vector<uint8_t>& p, int iteration) {
@@ -385,7 +427,7 @@ static int run_two_processes(const char* path, const std::vector<size_t>& sizes,
 int main(int argc, char** argv) {
   if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [options]\n", argv[0]); return 1; }
   size_t bytes = 64u << 20, request = 0;
-  int inflight = 4, iters = 5, host = 0, version = 8, connections = 1, handoff = 0, two_process = 0;
+  int inflight = 4, iters = 5, host = 0, version = 8, connections = 1, handoff = 0, two_process = 0, side_streams = 0;
   long long ho[6] = {0, 0, 0, 0, 0, 0};
   for (int i = 2; i < argc; ++i) {
     std::string a = argv[i];
@@ -398,6 +440,7 @@ int main(int argc, char** argv) {
     else if (a == "--host") host = 1;
     else if (a == "--connections") connections = (int)val();
     else if (a == "--two-process") two_process = 1;
+    else if (a == "--side-streams") side_streams = (int)val();
     else if (a == "--handoff" && i + 1 < argc) {
       if (sscanf(argv[++i], "%lld,%lld,%lld,%lld,%lld,%lld", &ho[0], &ho[1], &ho[2], &ho[3], &ho[4], &ho[5]) != 6) { fprintf(stderr, "--handoff takes six numbers\n"); return 1; }
       handoff = 1;
@@ -434,10 +477,13 @@ int main(int argc, char** argv) {
   Barrier barrier;
   barrier.parties = connections;
   std::vector<std::vector<TimePoint>> starts(connections, std::vector<TimePoint>(iters)), ends(connections, std::vector<TimePoint>(iters));
+  SideStreams side;
+  if (side_streams > 0 && !host) side.start(side_streams);
   std::vector<std::thread> conns;
   for (int ci = 0; ci < connections; ++ci)
     conns.emplace_back([&, ci]() { run_connection(ci, net8, net7, net6, sizes, request, inflight, iters, host, version, &barrier, starts[ci].data(), ends[ci].data()); });
   for (auto& t : conns) t.join();
+  side.finish();
   // an iteration lasts from the first connection's start to the last connection's finish
   double best = 1e30, total = 0;
   for (int it = 0; it < iters; ++it) {
@@ -456,6 +502,8 @@ int main(int argc, char** argv) {
   printf("{\"harness\": \"plugin\", \"name\": \"%s\", \"devices\": %d, \"memory\": \"%s\", \"bytes\": %zu, \"request_bytes\": %zu, \"requests\": %zu, "
          "\"inflight\": %d, \"iters\": %d, \"connections\": %d, \"best_s\": %.9f, \"mean_s\": %.9f, \"GBps_4N_best\": %.1f, \"bit_exact\": true}\n",
          net8->name, ndev, host ? "host" : "device", bytes, request, n_req, inflight, iters, connections, best, total, 4.0 * bytes * connections / best / 1e9);
+  if (side.n)
+    printf("{\"harness\": \"side_streams\", \"streams\": %d, \"fills\": %ld, \"fill_us_mean\": %.1f, \"fill_us_max\": %.1f}\n", side.n, side.ops, side.mean_us, side.max_us);
   // NCCL_FUSELINK_TRACE=1: where the host's time went, summed over all proxy threads
   typedef int (*host_stats_fn)(int64_t*, int64_t*, int);
   host_stats_fn host_stats = (host_stats_fn)dlsym(lib, "fl_net_host_stats");

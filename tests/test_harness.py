@@ -114,6 +114,24 @@ def test_plugin_host_path_under_address_sanitizer():
     assert json.loads(res.stdout.strip().splitlines()[-1])["bit_exact"]
 
 
+@pytest.mark.gpu
+def test_the_resident_engine_does_not_hold_a_hardware_queue_for_as_long_as_requests_come():
+    """A process has fewer hardware queues than an application has streams; the runtime puts several streams on one queue,
+    and a kernel that never ends holds its queue.  With eight more streams of the process busy with small fills beside a
+    connection at NCCL's request shape (about 5 ms of uninterrupted small requests per iteration), no fill may wait for
+    the whole of that: the lane engine leaves after NCCL_FUSELINK_ENGINE_RESIDENT_US (500) and is started again."""
+    if not os.path.exists(BIN):
+        build.build_harness(verbose=False)
+    res = subprocess.run([BIN, build.lib_path(), "--bytes", str(1 << 30), "--request", str(512 << 10), "--inflight", "8", "--iters", "3", "--side-streams", "8"],
+                         capture_output=True, text=True, timeout=300,
+                         env=dict(os.environ, NCCL_FUSELINK_LANES="8", NCCL_FUSELINK_CHUNKSIZE=str(256 << 10)))
+    assert res.returncode == 0, res.stderr[-2000:]
+    lines = {l["harness"]: l for l in (json.loads(x) for x in res.stdout.strip().splitlines() if x.startswith("{"))}
+    assert lines["plugin"]["bit_exact"] and lines["side_streams"]["streams"] == 8 and lines["side_streams"]["fills"] > 100
+    print(lines["side_streams"], lines["plugin"]["GBps_4N_best"])
+    assert lines["side_streams"]["fill_us_max"] < 3000, lines["side_streams"]
+
+
 # ---- sender and receiver in two processes ----------------------------------------------------------------------------
 # The receiver is a child forked before either side has loaded the plugin or touched the GPU; the two meet through the
 # 128-byte handle alone (a POSIX shared-memory object named in it carries the descriptor ring; a second one, per pair of
