@@ -463,6 +463,12 @@ struct MemHandle {             // FuseLinkMemHandle, fuselink.h:48-52
   // the allocation directly (0: it cannot), and the pair of processes the key belongs to
   WirePair* wire_pair = nullptr;
   uint32_t rkey = 0;
+  // registered through regMrDmaBuf with a descriptor: this registration's own duplicate of it and the offset that came
+  // with it (what the reference hands to ibv_reg_dmabuf_mr for every relay buffer, plugin.cc:1278-1280), kept for a
+  // wire that registers memory with a NIC; closed when the registration goes
+  int dmabuf_fd = -1;
+  uint64_t dmabuf_offset = 0;
+  ~MemHandle() { if (dmabuf_fd >= 0) close(dmabuf_fd); }
 };
 
 struct Handle {                // what listen writes into the caller's 128 bytes (plugin.cc:425-430)
@@ -849,7 +855,7 @@ ncclResult_t fl_get_properties_v8(int dev, ncclNetProperties_v8_t* props) {
   props->name = g_dev_names[dev];
   props->pciPath = nullptr;
   props->guid = (uint64_t)dev;
-  props->ptrSupport = NCCL_PTR_HOST | NCCL_PTR_CUDA;   // plugin.cc:364-370, without DMA-BUF
+  props->ptrSupport = NCCL_PTR_HOST | NCCL_PTR_CUDA | NCCL_PTR_DMABUF;   // plugin.cc:364-370; regMrDmaBuf checks and keeps the descriptor
   props->regIsGlobal = 1;                              // registrations are keyed by base address, not by comm
   props->speed = 400000;
   props->port = 1;
@@ -954,8 +960,30 @@ ncclResult_t fl_accept(void* listenComm, void** recvComm, ncclNetDeviceHandle_v8
   return ncclSuccess;
 }
 
-ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uint64_t /*offset*/, int /*fd*/, void** mhandle) {
+// Is `fd` a DMA-BUF that holds `size` bytes from `offset` on?  (A dma-buf is a file of the kernel's dmabuf pseudo file
+// system: its link in /proc reads "/dmabuf:<name>", and seeking to its end gives its size.)
+bool dmabuf_covers(int fd, uint64_t offset, size_t size) {
+  char path[64], link[128];
+  snprintf(path, sizeof(path), "/proc/self/fd/%d", fd);
+  const ssize_t n = readlink(path, link, sizeof(link) - 1);
+  if (n <= 0) return false;
+  link[n] = 0;
+  if (strncmp(link, "/dmabuf:", 8) != 0 && strncmp(link, "anon_inode:dmabuf", 17) != 0) return false;
+  const off_t end = lseek(fd, 0, SEEK_END);
+  (void)lseek(fd, 0, SEEK_SET);
+  return end >= 0 && (uint64_t)end >= offset && (uint64_t)end - offset >= size;
+}
+
+ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uint64_t offset, int fd, void** mhandle) {
   if (!comm || !data || !mhandle || size == 0) return ncclInvalidArgument;
+  if (fd >= 0) {
+    // A descriptor came with the buffer (plugin.cc:1168, 1278-1280).  It must be what it claims: device memory exported
+    // as a DMA-BUF that holds the registered range.  Anything else is refused, not ignored.
+    if (type != NCCL_PTR_CUDA || !dmabuf_covers(fd, offset, size)) {
+      FL_WARN("NET/FuseLink : regMrDmaBuf: descriptor %d is not a DMA-BUF of device memory that holds %zu bytes from offset %llu", fd, size, (unsigned long long)offset);
+      return ncclInvalidArgument;
+    }
+  }
   Comm* c = (Comm*)comm;
   if (c->magic != kCommMagic) return ncclInvalidArgument;
   const bool wire = c->link->wire != nullptr;   // the other end is another process
@@ -963,6 +991,11 @@ ncclResult_t fl_reg_mr_dmabuf(void* comm, void* data, size_t size, int type, uin
   MemHandle* mh = new (std::nothrow) MemHandle();
   if (!mh) return ncclSystemError;
   mh->type = type;
+  if (fd >= 0) {
+    mh->dmabuf_fd = dup(fd);   // the caller closes its own
+    mh->dmabuf_offset = offset;
+    if (mh->dmabuf_fd < 0) { delete mh; return ncclSystemError; }
+  }
   if (type == NCCL_PTR_CUDA) {
     // whole allocation around the pointer, as cuMemGetAddressRange in plugin.cc:1194
     void* base = nullptr;

@@ -173,6 +173,11 @@ class NetPlugin:
         rc = self.t.regMrDmaBuf(comm, C.c_void_p(data), size, ptr_type, offset, fd, C.byref(mh))
         return rc, mh.value
 
+    def regMrDmaBuf(self, comm, data: int, size: int, ptr_type: int, offset: int, fd: int):
+        mh = C.c_void_p()
+        rc = self.t.regMrDmaBuf(comm, C.c_void_p(data), size, ptr_type, offset, fd, C.byref(mh))
+        return rc, mh.value
+
     def deregMr(self, comm, mhandle) -> int:
         return self.t.deregMr(comm, mhandle)
 

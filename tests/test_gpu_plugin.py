@@ -127,6 +127,47 @@ def test_cfg2_shape_through_plugin(net):
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
+def test_regMrDmaBuf_takes_a_real_dmabuf_and_checks_its_size(net):
+    """regMrDmaBuf with a descriptor (src/plugin.cc:1168, 1278-1280): a DMA-BUF of device memory that holds the registered
+    range is accepted and the registration works like any other; one that is too short for the range, or for the offset
+    that came with it, is refused.  The descriptor here is the export of a 2 MiB staging unit (flh_window_export_dmabuf)."""
+    import os
+
+    import torch
+    from fuselink_amd import core
+    net.reconfigure(NCCL_FUSELINK_LANES=4, NCCL_FUSELINK_CHUNKSIZE=128 << 10)
+    net.set_credits([1, 2, 1, 1])
+    pool = core.Pool(0, 4)
+    w = core.Window(pool, 2 << 20)
+    w.bind(2 << 20)
+    fd = w.export_dmabuf(0, 2 << 20)
+    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    lcomm, s, r = net.connect_pair(0)
+    try:
+        rc, smh = net.regMrDmaBuf(s, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA, 0, fd)
+        assert rc == 0 and smh
+        rc, bad = net.regMrDmaBuf(s, src.data_ptr(), 4 << 20, P.NCCL_PTR_CUDA, 0, fd)          # 4 MiB do not fit a 2 MiB descriptor
+        assert rc == P.ncclInvalidArgument and bad is None
+        rc, bad = net.regMrDmaBuf(s, src.data_ptr(), src.numel(), P.NCCL_PTR_CUDA, (2 << 20) - 4096, fd)   # nor 1 MiB behind that offset
+        assert rc == P.ncclInvalidArgument and bad is None
+        rc, rmh = net.regMrDmaBuf(r, dst.data_ptr(), dst.numel(), P.NCCL_PTR_CUDA, 0, -1)
+        assert rc == 0 and rmh
+        os.close(fd)                                     # the registration keeps a duplicate of its own
+        fd = -1
+        _send_recv(net, s, r, src, dst, 1 << 20, 3, smh, rmh)
+        assert torch.equal(src, dst)
+        rc, props = net.getProperties(0)
+        assert props.ptrSupport & P.NCCL_PTR_DMABUF
+        assert net.deregMr(s, smh) == 0 and net.deregMr(r, rmh) == 0
+    finally:
+        if fd >= 0:
+            os.close(fd)
+        net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
+        w.destroy()
+        pool.destroy()
+
+
 def test_static_policy_puts_a_channel_on_one_lane(net):
     # the reference's live policy: lane = channelId % nNics (src/fuselink.h:235), receiver decides, sender obeys
     import torch

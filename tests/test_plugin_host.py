@@ -64,7 +64,7 @@ def test_tables_and_properties(version):
     rc, props = p.getProperties(3)
     assert rc == P.ncclSuccess
     assert props.name == b"fuselink3" and props.guid == 3
-    assert props.ptrSupport == P.NCCL_PTR_HOST | P.NCCL_PTR_CUDA
+    assert props.ptrSupport == P.NCCL_PTR_HOST | P.NCCL_PTR_CUDA | P.NCCL_PTR_DMABUF   # src/plugin.cc:364-370
     assert props.maxRecvs == 1 and props.latency == 0
     if version >= 7:
         assert props.netDeviceType == 0 and props.netDeviceVersion == 0  # src/plugin.cc:376-377
@@ -401,6 +401,24 @@ def test_the_senders_mask_is_refreshed_on_the_references_cadence_and_reaches_the
         net.deregMr(s, smh), net.deregMr(r, rmh)
         net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
         net.reconfigure(NCCL_FUSELINK_LANES=None)
+
+
+def test_regMrDmaBuf_refuses_a_descriptor_that_is_not_a_dmabuf(net, tmp_path):
+    """regMrDmaBuf (src/plugin.cc:1168, 1278-1280) gets a descriptor and an offset with the buffer.  No descriptor (-1) is
+    a plain registration; a descriptor that is not a DMA-BUF of device memory holding the range is refused, not ignored."""
+    lcomm, s, r = net.connect_pair(0)
+    src, sp = _host(4096, 13)
+    rc, mh = net.regMrDmaBuf(s, sp, 4096, P.NCCL_PTR_HOST, 0, -1)
+    assert rc == 0 and mh
+    assert net.deregMr(s, mh) == 0
+    f = open(tmp_path / "not_a_dmabuf", "w+b")
+    f.truncate(1 << 20)
+    rc, mh = net.regMrDmaBuf(s, sp, 4096, P.NCCL_PTR_CUDA, 0, f.fileno())      # an ordinary file
+    assert rc == P.ncclInvalidArgument and mh is None
+    rc, mh = net.regMrDmaBuf(s, sp, 4096, P.NCCL_PTR_HOST, 0, f.fileno())      # and host memory takes no descriptor at all
+    assert rc == P.ncclInvalidArgument and mh is None
+    f.close()
+    net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
 def test_cuda_pointer_fails_loudly_without_gpu(net):
