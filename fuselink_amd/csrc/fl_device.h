@@ -121,15 +121,20 @@ __device__ __forceinline__ uint64_t mod_u64(uint64_t a, uint64_t b) {
 // `full` is the workgroup count rounded down to a multiple of 256 (0 switches the mapping off); workgroups from
 // there on keep tile = b, so the map is a permutation of the grid (on a partition of the GPU that hands workgroups out
 // differently it stays one, and only the gain is lost).
+// Bit 5 of `full` (free: full is a multiple of 256) asks for the other extreme instead, for experiments: XCD x takes the
+// x-th eighth of the tiles front to back, so that the eight XCDs work in eight places of the stream that lie far apart.
+constexpr uint32_t kXcdEighths = 32u;
 __device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t full) {
-  return b < full ? (b & ~(kXcdBlock - 1)) + ((b & 7u) << kXcdRunShift) + ((b >> 3) & ((1u << kXcdRunShift) - 1)) : b;
+  const uint32_t n = full & ~(kXcdBlock - 1);
+  if (full & kXcdEighths) return b < n ? (b & 7u) * (n >> 3) + (b >> 3) : b;
+  return b < n ? (b & ~(kXcdBlock - 1)) + ((b & 7u) << kXcdRunShift) + ((b >> 3) & ((1u << kXcdRunShift) - 1)) : b;
 }
 // The same for a grid (tiles of a chunk, chunks) whose width is a power of two: xcd_map = full | log2(width).
 // Takes the workgroup's place in the grid, returns the tile of the chunk (x) and the chunk (y) it works on.
 __device__ __forceinline__ void xcd_tile_2d(uint32_t xcd_map, uint32_t& x, uint32_t& y) {
   if (xcd_map == 0) return;
   const uint32_t sh = xcd_map & 31u;
-  const uint32_t t = xcd_tile((y << sh) + x, xcd_map & ~(kXcdBlock - 1));
+  const uint32_t t = xcd_tile((y << sh) + x, xcd_map & ~31u);
   x = t & ((1u << sh) - 1);
   y = t >> sh;
 }

@@ -73,13 +73,13 @@ int fl_stream_mode(int dir, uint64_t bytes) {
 
 uint32_t fl_xcd_full(uint64_t grid) {
   if (!g_xcd_runs || grid < kXcdBlock || grid > 0xffffffffull) return 0;
-  return (uint32_t)grid & ~(kXcdBlock - 1);
+  return ((uint32_t)grid & ~(kXcdBlock - 1)) | (g_xcd_runs == 2 ? 32u : 0u);   // (bit 5: each XCD an eighth of the grid, an experiment)
 }
 
 uint32_t fl_xcd_map(uint32_t width, uint32_t height) {
   if (width == 0 || (width & (width - 1)) || (uint64_t)width * height > 0xffffffffull) return 0;
   const uint32_t full = fl_xcd_full((uint64_t)width * height);
-  if (!full) return 0;
+  if (full < kXcdBlock) return 0;
   uint32_t sh = 0;
   while ((1u << sh) < width) ++sh;
   return full | sh;   // full is a multiple of kXcdBlock >= 32, the shift stays below 32
@@ -178,7 +178,7 @@ int flh_tune(const char* key, int64_t value) {
     return FLH_OK;
   }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
-  if (!strcmp(key, "xcd_runs")) { g_xcd_runs = value != 0; return FLH_OK; }
+  if (!strcmp(key, "xcd_runs")) { g_xcd_runs = value == 2 ? 2 : value != 0; return FLH_OK; }
   if (!strncmp(key, "engine_", 7)) {
     // hooks for tests of the failure paths: a production process cannot reach them by accident
     const char* hooks = getenv("NCCL_FUSELINK_TEST_HOOKS");

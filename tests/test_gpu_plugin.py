@@ -969,19 +969,19 @@ def test_an_engine_that_goes_down_fails_its_requests_and_traffic_falls_back_to_l
     two-second limit, so the condition is forced from the host: an engine started while flh_tune("engine_inject_fault")
     is set reports the failure in place of executing its first batch, and every workgroup leaves.  The requests the
     engine held complete with ncclRemoteError (as a queue pair in the error state completes its work requests,
-    src/plugin.cc:1839-1861), nothing hangs, later requests of the connection and a connection opened afterwards move
-    their bytes through launch pairs."""
+    src/plugin.cc:1839-1861) and are freed, nothing hangs, and later requests of the same connection -- across its next
+    refresh boundaries, on the default cadence of 8 -- and of a connection opened afterwards move their bytes through
+    launch pairs."""
     import ctypes as C
     import time
     import torch
     piece = 512 << 10
-    net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=256 << 10, NCCL_FUSELINK_BATCH=8, NCCL_FUSELINK_ENGINE=1,
-                    NCCL_FUSELINK_REFRESH_BATCH=1000)
+    net.reconfigure(NCCL_FUSELINK_LANES=8, NCCL_FUSELINK_CHUNKSIZE=256 << 10, NCCL_FUSELINK_BATCH=8, NCCL_FUSELINK_ENGINE=1)
     net.lib.flh_tune.argtypes = [C.c_char_p, C.c_int64]
     rng = np.random.default_rng(77)
-    n = 32
-    src_np = rng.integers(1, 256, size=(n + 1) * piece, dtype=np.uint8)
-    c = _open(net, 0, torch.from_numpy(src_np).cuda(), torch.zeros((n + 1) * piece, dtype=torch.uint8, device="cuda"))
+    n, later = 32, 20
+    src_np = rng.integers(1, 256, size=(n + 1 + later) * piece, dtype=np.uint8)
+    c = _open(net, 0, torch.from_numpy(src_np).cuda(), torch.zeros((n + 1 + later) * piece, dtype=torch.uint8, device="cuda"))
     # one request on its own passes through the engine and takes the connection off its refresh boundary
     _send_recv(net, c["s"], c["r"], c["src"], c["dst"], piece, 99, c["smh"], c["rmh"], src_off=n * piece, dst_off=n * piece)
     time.sleep(0.05)         # far beyond the engine's idle limit: it has gone down, the next batch starts it again
@@ -1013,6 +1013,22 @@ def test_an_engine_that_goes_down_fails_its_requests_and_traffic_falls_back_to_l
         assert net.lib.flh_tune(b"engine_inject_fault", 0) == 0
     # the first batch's eight sends and eight receives at least; what was sent after the failure showed went by launches
     assert failed >= 16 and finished + failed == 2 * n
+    # every request, failed or not, has been freed and counted: the connection's next refreshes (at 40 and 48 completed
+    # receives) are not held back, and its later traffic goes by launch pairs and arrives
+    assert net.free_requests(c["s"]) == 256 and net.free_requests(c["r"]) == 256
+    st = net.comm_stats(c["r"])
+    assert st["n_finished"] == n + 1 and st["in_flight"] == 0
+    for q in range(n + 1, n + 1 + later):
+        rreq, deadline = None, time.time() + 10
+        while not rreq:
+            rc, rreq = net.irecv(c["r"], [c["dst"].data_ptr() + q * piece], [piece], [q], [c["rmh"]])
+            assert rc == 0 and time.time() < deadline, "a later receive was never accepted: the connection stalled at its refresh"
+        rc, sreq = net.isend(c["s"], c["src"].data_ptr() + q * piece, piece, q, c["smh"])
+        assert rc == 0 and sreq
+        net.wait(sreq)
+        assert net.wait(rreq) == piece
+    np.testing.assert_array_equal(c["dst"].cpu().numpy()[(n + 1) * piece:], src_np[(n + 1) * piece:])
+    assert net.comm_stats(c["r"])["refreshes"] >= 3
     # the GPU's staging side lives on: new traffic goes by launch pairs and arrives
     src2_np = rng.integers(0, 256, size=4 * piece, dtype=np.uint8)
     c2 = _open(net, 1, torch.from_numpy(src2_np).cuda(), torch.zeros(4 * piece, dtype=torch.uint8, device="cuda"))

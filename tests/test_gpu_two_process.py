@@ -309,6 +309,20 @@ back = dst.cpu().numpy()
 assert np.array_equal(back[:total], exp), "received bytes differ from what was sent"
 assert not back[total:].any(), "bytes behind the last request were touched"
 print("receiver ok"); sys.stdout.flush()
+if plan.get("orphan"):
+    # one more receive, which the sender never answers: once the sender has closed its end the receive must fail, not hang,
+    # and its request must be freed
+    req = None
+    while not req:
+        rc, req = p.irecv(rcomm, [dst.data_ptr()], [4096], [len(sizes)], [mh])
+        assert rc == P.ncclSuccess and time.time() < deadline
+    rc = P.ncclSuccess
+    while rc == P.ncclSuccess:
+        rc, done, _ = p.test(req)
+        assert not done and time.time() < deadline
+    assert rc == P.ncclRemoteError, rc
+    assert p.free_requests(rcomm) == 256
+    print("orphan failed"); sys.stdout.flush()
 sys.stdin.readline()                    # the sender has closed its comm
 assert p.deregMr(rcomm, mh) == P.ncclSuccess
 assert p.closeRecv(rcomm) == P.ncclSuccess and p.closeListen(lcomm) == P.ncclSuccess
@@ -373,6 +387,8 @@ class _Planned:
             if et is None:
                 assert self.child.stdout.readline().strip() == "receiver ok", self.child.stderr.read()[-3000:]
                 assert self.p.deregMr(self.scomm, self.mh) == P.ncclSuccess and self.p.closeSend(self.scomm) == P.ncclSuccess
+                if self.plan.get("orphan"):
+                    assert self.child.stdout.readline().strip() == "orphan failed", self.child.stderr.read()[-3000:]
                 self.child.stdin.write("closed\n")
                 self.child.stdin.flush()
                 _, err = self.child.communicate(timeout=60)
@@ -465,6 +481,7 @@ def test_a_lane_that_another_process_keeps_busy_gets_no_chunks_after_the_next_re
             return list(out)
 
         with _Planned(env, plan) as run:
+            run.p.set_credits([])                # (no static row left over from another test)
             epoch = chunks = 0
             on_lane = [0, 0, 0]
             row = expected_row([])
@@ -517,6 +534,7 @@ def test_a_lane_that_the_senders_process_masks_out_gets_no_chunks_after_the_next
     with _Planned(env, plan) as run:
         L = run.p.lib
         L.fl_monitor_reset()
+        run.p.set_credits([])                    # (no static row left over from another test: the mask comes off the lane table)
         epoch = chunks = 0
         on_lane = [0, 0, 0]
         row = expected_row(0xffffffff)
@@ -546,3 +564,16 @@ def test_a_lane_that_the_senders_process_masks_out_gets_no_chunks_after_the_next
         st = run.p.mask_stats(run.scomm)
         assert st["refreshes"] == 3 and st["mask"] == 0xffffffff
         L.fl_monitor_reset()
+
+
+@DIRECT
+def test_a_receive_whose_sender_has_gone_fails_and_is_freed(direct):
+    """The other process closes its end with a receive still posted here: test returns ncclRemoteError for it (as a failed
+    completion does, src/plugin.cc:1839-1861) instead of polling for ever, and the request goes back to the table.  And the
+    other way round: a send that finds the receiving process gone fails at once."""
+    lanes, chunk = 4, 128 << 10
+    plan = dict(sizes=[3 * chunk, 5 * chunk + 7], seed=55, orphan=True)
+    env = {"NCCL_FUSELINK_LANES": lanes, "NCCL_FUSELINK_CHUNKSIZE": chunk, "NCCL_FUSELINK_WIRE_DIRECT": direct}
+    with _Planned(env, plan) as run:
+        for q in range(len(plan["sizes"])):
+            run.send(q)
