@@ -69,8 +69,11 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-iters", type=int, default=1000, help="timed CPU passes at 64 MiB (scaled down for larger messages): about 5 s of CPU work per figure")
     ap.add_argument("--hint", type=int, default=1, help="pass the host-known header fields to the copy kernels")
-    ap.add_argument("--path", default="auto", choices=["auto", "fused", "split"],
-                    help="fused: scheduler folded into the striping launch (uniform split, one credit row); split: three launches")
+    ap.add_argument("--path", default="auto", choices=["auto", "fused", "split", "carry"],
+                    help="fused: scheduler folded into the striping launch (uniform split, one credit row); split: three launches; "
+                         "carry: the launches of a transfer whose receiver is another process and has not exported its buffer -- the striping "
+                         "launch also carries every staged tile into a second set of windows (the receiver's landing windows, here a plain "
+                         "allocation of this process), the reassembly reads from those; not a bench line")
     ap.add_argument("--lds", type=int, default=0, help="paged workload: stage the gather through LDS")
     ap.add_argument("--cold-user-buffers", type=int, default=1,
                     help="also time the step over source/destination pairs in rotation (1 GiB), so that no user buffer is "
@@ -374,11 +377,17 @@ def main() -> int:
 
     # header fields that follow from the uniform split alone; the kernels then need not wait for d_hdr
     hint = core.uniform_hint(msg_bytes, chunk) if (args.hint and kind == "uniform") else None
-    fused = not waves and not cwaves and not twaves and kind in ("uniform", "pages") and (args.path == "fused" or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
+    carry = args.path == "carry"
+    if carry and (kind != "uniform" or rows != 1 or epoch_len != 0 or waves or cwaves or twaves):
+        print("bench.py: --path carry takes a uniform workload under one credit row that moves in one launch pair", file=sys.stderr)
+        return 2
+    fused = not waves and not cwaves and not twaves and kind in ("uniform", "pages") and (args.path in ("fused", "carry") or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
     if fused and (rows != 1 or epoch_len != 0):
         print("bench.py: the fused path takes a single credit row without epochs", file=sys.stderr)
         return 2
     uni = core.uniform_params(msg_bytes, chunk, credits_np[0].tolist()) if fused else None
+    landing_bufs = [torch.zeros(max(b, 1), dtype=torch.uint8, device=dev) for b in lane_bytes] if carry else None
+    landing = core.make_windows([t.data_ptr() for t in landing_bufs], lane_bytes) if carry else None
 
     def step():
         if kind == "pages" and fused:
@@ -413,6 +422,10 @@ def main() -> int:
                               mode=core.SCHED_RESET_OFFSETS, state=state, out=s_w, stream=stream, by_lane=by_lane)
                 core.stripe(src, win, s_w, status, stream=stream, hint=h_w, by_lane=by_lane)
                 core.reassemble(dst, win, s_w, status, stream=stream, hint=h_w)
+        elif carry:
+            # staging and the wire in one launch (source -> staging windows -> landing windows), delivery out of the landing windows
+            core.stripe_uniform_carry(src, win, landing, uni, status, out=sched, stream=stream)
+            core.reassemble_uniform(dst, landing, uni, status, stream=stream)
         elif fused:
             # the striping launch computes each chunk's lane and offset itself and writes the table out
             core.stripe_uniform(src, win, uni, status, out=sched, stream=stream)
@@ -591,6 +604,8 @@ def main() -> int:
 
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
     algo_bytes_kernel = 2 * msg_bytes // len(waves or cwaves or twaves or (0,))    # one launch of the copy kernel (with waves: the average one)
+    if carry:
+        algo_bytes_kernel = 3 * msg_bytes   # read N, write N into the staging windows, write N into the landing windows (the re-read of a staged tile by the workgroup that wrote it is served by its L2)
     value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
     pair_us = (stripe_us + reasm_us) * launches_per_step
     achieved = algo_bytes_kernel / (stripe_us * 1e-6) / 1e9
@@ -598,6 +613,8 @@ def main() -> int:
         kernel_name = "fl_copy_uniform_fused<0, FusedPageArgs> (gather)"
     elif kind == "pages":
         kernel_name = f"fl_page_tiles<0, lds={args.lds}> (gather)"
+    elif carry:
+        kernel_name = "fl_copy_uniform_fused<0, FusedCarryArgs> (stripe + carry)"
     elif fused or cwaves:
         kernel_name = "fl_copy_uniform_fused<0> (stripe)"
     elif hint is not None:
@@ -626,6 +643,7 @@ def main() -> int:
         "config": {"workload": args.workload, "bytes": nbytes, "chunk_bytes": chunk if sizes is None else "variable", "chunks": n_chunks,
                    "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
                    "step": ("2x(gather(with scheduler folded in)+scatter)" if (kind == "pages" and fused) else "2x(schedule+gather+scatter)" if kind == "pages" else
+                            "stripe(with scheduler folded in)+carry into landing windows, then reassemble out of them" if carry else
                             "stripe(with scheduler folded in)+reassemble" if fused else
                             f"{len(cwaves)} waves of stripe(with scheduler folded in)+reassemble over cache-resident windows" if cwaves else
                             f"schedule, then {len(twaves)} waves of stripe+reassemble over cache-resident windows" if twaves else "schedule+stripe+reassemble"),

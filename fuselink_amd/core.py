@@ -242,6 +242,14 @@ def stripe_uniform(src: torch.Tensor, win: Windows, u: UniformParams, status: to
                                          _stream_ptr(stream)))
 
 
+def stripe_uniform_carry(src: torch.Tensor, win: Windows, landing: Windows, u: UniformParams, status: torch.Tensor, out: Optional[Schedule] = None,
+                         stream: Optional[torch.cuda.Stream] = None) -> None:
+    """flh_stripe_uniform_carry: stripe into `win` and carry every staged tile on into the same place of `landing`."""
+    check(_lib.load().flh_stripe_uniform_carry(_ptr(src), src.numel() * src.element_size(), C.byref(win), C.byref(landing), C.byref(u),
+                                               _ptr(out.table) if out else None, _ptr(out.hdr) if out else None, _ptr(status),
+                                               _stream_ptr(stream)))
+
+
 def reassemble_uniform(dst: torch.Tensor, win: Windows, u: UniformParams, status: torch.Tensor,
                        stream: Optional[torch.cuda.Stream] = None) -> None:
     check(_lib.load().flh_reassemble_uniform(_ptr(dst), dst.numel() * dst.element_size(), C.byref(win), C.byref(u),

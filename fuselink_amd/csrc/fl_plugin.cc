@@ -189,7 +189,8 @@ inline int64_t tr_now() {
 // ring that fl_net_timeline() copies out.  Events: 1 irecv posted (value = channel), 2 isend matched (channel),
 // 3 pass that launches begins (requests waiting), 4 batch handed over (requests << 32 | number; bit 31 of the number's
 // word set for engine batches), 5 request seen complete by test (its batch's number << 16 | bit 15: an engine batch | channel << 1 | is-receive),
-// 6 a test call is the first to see the engine's batches complete up to this number.
+// 6 a test call is the first to see the engine's batches complete up to this number, 7 wave announced to the receiving process
+// (its number), 8 wave taken off the wire by the receiving process (its number).
 struct TimelineEvent { int64_t ns; uint32_t thread; uint32_t event; uint64_t value; };
 constexpr size_t kTimelineCap = 1 << 16;
 TimelineEvent g_timeline[kTimelineCap];

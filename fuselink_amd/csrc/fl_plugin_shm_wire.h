@@ -572,6 +572,7 @@ ncclResult_t wire_publish(WirePair* p) {
     memcpy((char*)&wv + sizeof(wv.seq), (const char*)&f.rec + sizeof(f.rec.seq), sizeof(ShmWave) - sizeof(wv.seq));
     wv.seq.store(n, std::memory_order_release);
     p->tx_published.store(n, std::memory_order_release);
+    tl_event(7, n);
     p->tx_flights.pop_front();
   }
   p->tx_mu.unlock();
@@ -605,6 +606,7 @@ ncclResult_t wire_progress_recv(WirePair* p) {
     if (wv.seq.load(std::memory_order_acquire) != taken + 1) break;         // nothing further has landed
     if (!pr->launch_mu.try_lock()) break;                                    // somebody is launching: next poll
     WireFlight f;
+    tl_event(8, taken + 1);
     rc = wire_deliver(p, wv, f);
     pr->launch_mu.unlock();
     p->rx_taken.store(taken + 1, std::memory_order_release);

@@ -281,7 +281,10 @@ int fl_net_host_stats(int64_t* calls_out, int64_t* ns_out, int n);
 /* Timeline kept under NCCL_FUSELINK_TRACE=2: up to 65536 events of 24 bytes {int64 nanoseconds (monotonic clock), uint32
  * thread, uint32 event, uint64 value}; events: 1 receive posted (value = channel), 2 send matched (channel), 3 a pass that
  * launches begins (requests waiting), 4 batch handed over (requests << 32 | bit 31: engine batch | its number),
- * 5 request seen complete by test (channel << 1 | is-receive).  Copies up to max_events into `out`, returns how many exist. */
+ * 5 request seen complete by test (its batch's number << 16 | bit 15: an engine batch | channel << 1 | is-receive), 6 the
+ * engine's batches seen complete up to this number, 7 wave announced to the receiving process (its number), 8 wave taken
+ * off the wire by the receiving process (its number).  The clock is the same for every process of the machine.  Copies up
+ * to max_events into `out`, returns how many exist. */
 int fl_net_timeline(void* out, int max_events);
 /* Launch whatever waits on the GPU that `comm` stages on, without polling a request. */
 int fl_net_flush(void* comm);

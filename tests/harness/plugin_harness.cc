@@ -252,6 +252,25 @@ static ncclNet_v8_t* open_plugin(const char* path) {
   CHECK(net8->devices(&ndev));
   return net8;
 }
+// NCCL_FUSELINK_TRACE=2 and FL_TIMELINE_OUT=<file>: the entry-point timeline of this process, one event per line
+// (nanoseconds of the machine's monotonic clock, thread, event, value), into <file><suffix>
+static void dump_timeline(const char* lib_path, const char* suffix) {
+  const char* tr = getenv("NCCL_FUSELINK_TRACE");
+  const char* tl_out = getenv("FL_TIMELINE_OUT");
+  if (!tr || atoi(tr) < 2 || !tl_out) return;
+  void* lib = dlopen(lib_path, RTLD_NOW | RTLD_LOCAL);
+  typedef int (*timeline_fn)(void*, int);
+  timeline_fn timeline = lib ? (timeline_fn)dlsym(lib, "fl_net_timeline") : nullptr;
+  if (!timeline) return;
+  struct Ev { int64_t ns; uint32_t thread, event; uint64_t value; };
+  std::vector<Ev> ev(65536);
+  const int n = timeline(ev.data(), (int)ev.size());
+  FILE* f = fopen((std::string(tl_out) + suffix).c_str(), "w");
+  if (!f) return;
+  for (int i = 0; i < n && i < (int)ev.size(); ++i) fprintf(f, "%lld %u %u %llu\n", (long long)ev[i].ns, ev[i].thread, ev[i].event, (unsigned long long)ev[i].value);
+  fclose(f);
+}
+
 static const double kDeadline = 90.0;   // seconds any one wait may last
 struct Deadline {
   std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
@@ -337,6 +356,7 @@ static int receiver_process(const char* path, int sock, const std::vector<size_t
   CHECK(net->closeRecv(rcomm));
   CHECK(net->closeListen(lcomm));
   for (uint8_t* p : dst) HIP(hipFree(p));
+  dump_timeline(path, ".receiver");
   return 0;
 }
 
@@ -393,6 +413,7 @@ static int sender_process(const char* path, int sock, pid_t child, const std::ve
   for (size_t m = 0; m < sizes.size(); ++m) CHECK(net->deregMr(scomm, mh[m]));
   CHECK(net->closeSend(scomm));
   for (uint8_t* p : src) HIP(hipFree(p));
+  dump_timeline(path, ".sender");
   char bye = 1;
   sock_write(sock, &bye, 1);
   int status = 0;
