@@ -1737,7 +1737,7 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
   e->host_slots = 64;
   e->idle_us = idle_us ? idle_us : 200;
   e->wait_us = (uint64_t)g_engine_wait_us;   // two seconds unless a test has asked for less (flh_tune "engine_wait_us")
-  e->resident_us = 500;
+  e->resident_us = 1000;
   // whatever has been allocated when a call fails goes back through the one cleanup path (which takes null members)
   auto build = [&]() -> int {
     FL_HIP(hipSetDevice(device));

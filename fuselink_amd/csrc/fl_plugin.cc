@@ -88,10 +88,11 @@ struct Params {
   int engine_idle_us = 200;      // the engine goes down after this long without work
   // NCCL_FUSELINK_ENGINE_RESIDENT_US: ... and after this long even with work (0 = never), so that its hardware queue
   // drains; the next batch starts it again.  With eight more streams of the process busy beside the plugin's (more streams
-  // than hardware queues), a small fill on one of them waited up to 5.0 ms behind an engine that stayed for as long as
-  // requests came, 2.0 ms with a bound of 2000, 0.85 ms with 500 (0.80 ms with no engine at all); the request rate is the
-  // same within the spread of runs.
-  int engine_resident_us = 500;
+  // than hardware queues), a small fill on one of them waited up to 4.7 ms behind an engine that stayed for as long as
+  // requests came (1 GiB in 512 KiB requests, about 5 ms), 2.0 ms with a bound of 2000, 1.0 ms with 1000, 0.8 ms with 500
+  // or 250 -- and 0.8 ms with no engine at all.  Every restart costs the transfer a launch: the same 1 GiB moved at
+  // 945-990 GB/s with a bound of 1000 or more and at 780-970 with 500 or 250.
+  int engine_resident_us = 1000;
   int engine_workgroups = 0;     // 0 = the library's default
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU

@@ -358,7 +358,7 @@ int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_window
 int flh_engine_submit_wire(flh_engine* e, uint32_t kind, const flh_batch_params* b, const flh_windows* win, const flh_windows* landing,
                            flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out);
 /* How long the resident kernel stays although work keeps coming (microseconds; 0 = as long as there is work; default
- * 500).  A kernel that never ends holds its hardware queue; the runtime puts several streams on one queue when a process
+ * 1000).  A kernel that never ends holds its hardware queue; the runtime puts several streams on one queue when a process
  * has more streams than queues, and what it has queued behind the engine waits until the engine leaves.  With a bound
  * the engine leaves between two batches when its time is up, and the next flh_engine_submit -- or flh_engine_poke, for a
  * caller with batches outstanding and nothing further to submit -- starts it again.  flh_engine_needs_start says

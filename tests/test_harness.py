@@ -119,7 +119,7 @@ def test_the_resident_engine_does_not_hold_a_hardware_queue_for_as_long_as_reque
     """A process has fewer hardware queues than an application has streams; the runtime puts several streams on one queue,
     and a kernel that never ends holds its queue.  With eight more streams of the process busy with small fills beside a
     connection at NCCL's request shape (about 5 ms of uninterrupted small requests per iteration), no fill may wait for
-    the whole of that: the lane engine leaves after NCCL_FUSELINK_ENGINE_RESIDENT_US (500) and is started again."""
+    the whole of that: the lane engine leaves after NCCL_FUSELINK_ENGINE_RESIDENT_US (1000) and is started again."""
     if not os.path.exists(BIN):
         build.build_harness(verbose=False)
     res = subprocess.run([BIN, build.lib_path(), "--bytes", str(1 << 30), "--request", str(512 << 10), "--inflight", "8", "--iters", "3", "--side-streams", "8"],
