@@ -577,3 +577,45 @@ def test_a_receive_whose_sender_has_gone_fails_and_is_freed(direct):
     with _Planned(env, plan) as run:
         for q in range(len(plan["sizes"])):
             run.send(q)
+
+
+@DIRECT
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_traffic_of_several_connections_both_ways_across_two_processes(direct, seed):
+    """The reference's two ends both send and receive, on several channels at once.  Three connections from this process
+    to the child and two back, 24 requests each from empty to 1.5 MiB (some whole chunks, some a few bytes, one of 7.5 MiB
+    that the windows hold only in pieces), six in flight per connection, posted and tested in a seeded random order by
+    both processes at once: requests of different connections share waves, waves of both directions share each GPU
+    side's queue and engine, the refresh gate closes and opens on the default cadence.  Each process compares what it
+    received with the connection's pattern, and the bytes behind it with zero."""
+    from tests import two_process_peer as peer
+    lanes, chunk = 4, 128 << 10
+    env = dict(os.environ, NCCL_FUSELINK_WIRE="shm", PYTHONPATH=ROOT, NCCL_FUSELINK_LANES=str(lanes), NCCL_FUSELINK_CHUNKSIZE=str(chunk),
+               NCCL_FUSELINK_WINDOW_UNITS="1", NCCL_FUSELINK_WIRE_DIRECT=str(direct))
+    plan = peer.make_plan(seed, n_ab=3, n_ba=2, requests=24, max_bytes=3 << 19, chunk=chunk, inflight=6)
+    child = subprocess.Popen([sys.executable, "-m", "tests.two_process_peer", json.dumps(plan)], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                             stderr=subprocess.PIPE, text=True, env=env, cwd=ROOT)
+    keys = ["NCCL_FUSELINK_WIRE"] + list(env_keys(env))
+    p = P.NetPlugin(8)
+
+    def write_line(s):
+        child.stdin.write(s + "\n")
+        child.stdin.flush()
+
+    try:
+        p.reconfigure(**{k: env[k] for k in keys})
+        p.set_credits([])                # no static row left by an earlier test: the monitor drives
+        n = peer.drive(p, P, plan, "a", child.stdout.readline, write_line, peer_alive=lambda: child.poll() is None)
+        assert n == sum(len(c["sizes"]) for c in plan["conns"])
+        assert child.stdout.readline().strip() == f"peer ok {n}", child.stderr.read()[-3000:]
+        _, err = child.communicate(timeout=60)
+        assert child.returncode == 0, err[-3000:]
+    except AssertionError:
+        if child.poll() is None:
+            child.kill()
+        print(child.stderr.read()[-3000:])
+        raise
+    finally:
+        if child.poll() is None:
+            child.kill()
+        p.reconfigure(**{k: None for k in keys})
