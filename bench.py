@@ -127,7 +127,7 @@ def main() -> int:
         if os.path.exists(harness) and os.path.exists(flbuild.lib_path()):
             env = dict(os.environ, NCCL_FUSELINK_LANES="8", NCCL_FUSELINK_CHUNKSIZE=str(256 << 10))
             plugin = {"message_bytes": 64 << 20, "request_bytes": 512 << 10, "requests": 128, "inflight": 8, "lanes": 8, "chunk_bytes": 256 << 10,
-                      "accounting": "4 x bytes x connections / wall time of the best of 20 iterations, proxy threads started inside the timed region",
+                      "accounting": "4 x bytes x connections / wall time of the best of 20 iterations, proxy threads started inside the timed region.  4 x bytes is the headline metric's accounting (stage: read N + write N, deliver: read N + write N) and what a launch pair moves; the lane engine, which carries requests of up to 1 MiB, stores every loaded vector twice (staging window and receive buffer) and so moves 3 x bytes for the same result: payload rate = GBps_4N / 4",
                       "env": "NCCL_FUSELINK_LANES=8 NCCL_FUSELINK_CHUNKSIZE=262144"}
             for conns in (1, 4):
                 cmd = [harness, flbuild.lib_path(), "--bytes", str(64 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "20",
@@ -605,7 +605,7 @@ def main() -> int:
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
     algo_bytes_kernel = 2 * msg_bytes // len(waves or cwaves or twaves or (0,))    # one launch of the copy kernel (with waves: the average one)
     if carry:
-        algo_bytes_kernel = 3 * msg_bytes   # read N, write N into the staging windows, write N into the landing windows (the re-read of a staged tile by the workgroup that wrote it is served by its L2)
+        algo_bytes_kernel = 3 * msg_bytes   # read N, write N into the staging windows, write N into the landing windows (every vector loaded once, stored twice)
     value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
     pair_us = (stripe_us + reasm_us) * launches_per_step
     achieved = algo_bytes_kernel / (stripe_us * 1e-6) / 1e9

@@ -87,6 +87,7 @@ SIGNATURES = {
     "flh_engine_submit_wire": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(BatchParams), C.POINTER(Windows), C.POINTER(Windows), C.c_void_p, C.c_void_p,
                                          C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "flh_engine_set_resident": (C.c_int, [C.c_void_p, C.c_uint32]),
+    "flh_engine_trace": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint32, C.c_void_p]),
     "flh_engine_needs_start": (C.c_int, [C.c_void_p]),
     "flh_engine_poke": (C.c_int, [C.c_void_p]),
     "flh_window_export_dmabuf": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.POINTER(C.c_int)]),

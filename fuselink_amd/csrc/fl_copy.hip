@@ -8,6 +8,7 @@
 #include <cstring>
 #include <new>
 #include <type_traits>
+#include <vector>
 
 #include "fl_closed_form.h"
 #include "fl_device.h"
@@ -309,6 +310,57 @@ __device__ __forceinline__ void block_copy(uint8_t* __restrict__ dst, const uint
   if (tid < tail) dst[tail0 + tid] = src[tail0 + tid];
 }
 
+// One source, two destinations: every vector is loaded once and stored twice (staging window and the wire's far end,
+// or staging window and receive buffer), so the second copy costs no second read and no barrier between a workgroup's
+// store and its re-load.  When the three addresses are not equally aligned the bytes are copied twice from the source.
+template <int NT>
+__device__ __forceinline__ void block_copy2(uint8_t* __restrict__ d1, uint8_t* __restrict__ d2, const uint8_t* __restrict__ src, uint32_t bytes) {
+  const uintptr_t sa = (uintptr_t)src;
+  if ((((sa ^ (uintptr_t)d1) | (sa ^ (uintptr_t)d2)) & 15) != 0) {
+    block_copy<NT>(d1, src, bytes);
+    block_copy<NT>(d2, src, bytes);
+    return;
+  }
+  const uint32_t tid = threadIdx.x;
+  uint32_t head = (uint32_t)((16 - (sa & 15)) & 15);
+  if (head > bytes) head = bytes;
+  if (tid < head) { copy1<NT>(d1 + tid, src + tid); copy1<NT>(d2 + tid, src + tid); }
+  const uint32_t nvec = (bytes - head) >> 4;
+  const VecIn<NT> in((const u32x4*)(src + head), nvec);
+  const VecOut<NT> out1((u32x4*)(d1 + head), nvec), out2((u32x4*)(d2 + head), nvec);
+  auto exact = [&](auto U_) {
+    constexpr int U = decltype(U_)::value;
+    u32x4 r[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) r[j] = in(j * kCopyBlock + tid);
+#pragma unroll
+    for (int j = 0; j < U; ++j) out1(j * kCopyBlock + tid, r[j]);
+#pragma unroll
+    for (int j = 0; j < U; ++j) out2(j * kCopyBlock + tid, r[j]);
+  };
+  if (nvec == kCopyBlock * 16) exact(std::integral_constant<int, 16>{});
+  else if (nvec == kCopyBlock * 8) exact(std::integral_constant<int, 8>{});
+  else if (nvec == kCopyBlock * 4) exact(std::integral_constant<int, 4>{});
+  else {
+    for (uint32_t b = 0; b < nvec; b += kCopyBlock * kCopyUnroll) {
+      u32x4 r[kCopyUnroll];
+#pragma unroll
+      for (int j = 0; j < kCopyUnroll; ++j) {
+        const uint32_t idx = b + j * kCopyBlock + tid;
+        if (idx < nvec) r[j] = in(idx);
+      }
+#pragma unroll
+      for (int j = 0; j < kCopyUnroll; ++j) {
+        const uint32_t idx = b + j * kCopyBlock + tid;
+        if (idx < nvec) { out1(idx, r[j]); out2(idx, r[j]); }
+      }
+    }
+  }
+  const uint32_t tail0 = head + (nvec << 4);
+  const uint32_t tail = bytes - tail0;
+  if (tid < tail) { copy1<NT>(d1 + tail0 + tid, src + tail0 + tid); copy1<NT>(d2 + tail0 + tid, src + tail0 + tid); }
+}
+
 struct CopyArgs {
   uint8_t* user;
   uint64_t user_bytes;
@@ -566,9 +618,12 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
 
 // One workgroup's share of a fused launch: tile bx of the chunk that grid row by stands for (`span` neighbouring tiles
 // of that chunk from bx on, for a caller that hands out larger shares).  DIR 0: user buffer -> staging window, 1: window
-// -> user buffer, 2: staging window -> the same lane and offset of the carry windows (the wire).
+// -> user buffer, 2: staging window -> the same lane and offset of the carry windows (the wire), 3: user buffer -> staging
+// window and, from the same registers, on to where the staged bytes go next: the same place of the request's buffer in
+// `onward` (one buffer per request of a batch: the receive buffers) or, without one, the same lane and offset of the
+// carry windows.
 template <int DIR, int NT, class Args>
-__device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by, uint32_t span = 1) {
+__device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by, uint32_t span = 1, uint8_t* const* onward = nullptr) {
   constexpr bool BATCH = is_batch<Args>::value;
   constexpr bool PAGED = is_paged<Args>::value;
   if (by >= a.n_chunks) return;
@@ -577,6 +632,7 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
   // where the chunk's bytes live on the user side (the one buffer, or its request's), its length, its place in the
   // message for the table, and where its lane's window starts for it
   uint8_t* user = a.user;
+  uint8_t* onward_user = nullptr;
   uint64_t user_off, user_bytes = a.user_bytes, src_off, win_base = 0;
   uint32_t len;
   if constexpr (BATCH) {
@@ -600,6 +656,7 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
     before = (uint64_t)full * (hi - K) + (slot - K) - g.cnt0[lane];
     win_base = (uint64_t)g.base128[lane] * 128u;
     user = a.req_user[r];
+    if (DIR == 3 && onward) onward_user = onward[r];
     user_bytes = a.req_bytes[r];
     user_off = (uint64_t)(c - a.first[r]) * a.chunk_bytes;
     const uint64_t rem = user_bytes - user_off;
@@ -667,7 +724,7 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
   }
   const uint64_t win_off = win_base + before * a.chunk_bytes;
 
-  if (DIR == 0 && bx == 0 && threadIdx.x == 0 && a.table) {
+  if ((DIR == 0 || DIR == 3) && bx == 0 && threadIdx.x == 0 && a.table) {
     flh_chunk_desc d;
     d.src_off = src_off;
     d.win_off = win_off;
@@ -677,7 +734,7 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
     d.epoch = 0;
     st_obj<NT>(&a.table[c], d);
   }
-  if (DIR == 0 && bx == 0 && by == 0 && a.hdr) {  // header: per-lane totals in closed form
+  if ((DIR == 0 || DIR == 3) && bx == 0 && by == 0 && a.hdr) {  // header: per-lane totals in closed form
     const uint32_t t = threadIdx.x;
     if constexpr (BATCH) {
       // the launch's totals: every segment's closed form, summed
@@ -774,6 +831,17 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
       return;
     }
     block_copy<NT>((uint8_t*)a.carry.base[lane] + win_off + off, w, bytes);
+  } else if constexpr (DIR == 3) {
+    static_assert(has_carry<Args>::value && !PAGED, "the second destination is a receive buffer or a landing window");
+    if (onward_user) {
+      block_copy2<NT>(w, onward_user + user_off + off, u, bytes);
+    } else {
+      if (win_off + len > a.carry.cap[lane]) {   // refused whole: nothing of the chunk is staged either
+        if (threadIdx.x == 0) st_obj<NT>(a.status, (int32_t)FLH_E_RANGE);
+        return;
+      }
+      block_copy2<NT>(w, (uint8_t*)a.carry.base[lane] + win_off + off, u, bytes);
+    }
   } else if constexpr (DIR == 0) {
     block_copy<NT>(w, u, bytes);
   } else {
@@ -788,14 +856,9 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_uniform_fused(Args a) {
   xcd_tile_2d(a.xcd_map, bx, by);
   if (a.start_word && bx == 0 && by == 0 && threadIdx.x == 0)
     __hip_atomic_store(a.start_word, a.start_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-  fused_tile<DIR, NT>(a, bx, by);
-  if constexpr (DIR == 0 && has_carry<Args>::value) {
-    // the wire: the tile this workgroup has just staged goes on into the landing windows.  The barrier orders the
-    // workgroup's stores before its loads of the same bytes (one compute unit, one L1, the XCD's L2 behind it); the
-    // loads stay cacheable whatever the launch's streaming mode, the stores stream when the staging stores do.
-    __syncthreads();
-    fused_tile<2, (NT & 2)>(a, bx, by);
-  }
+  // with a wire: the tile goes into its staging window and, from the same registers, into the landing windows
+  if constexpr (DIR == 0 && has_carry<Args>::value) fused_tile<3, NT>(a, bx, by);
+  else fused_tile<DIR, NT>(a, bx, by);
   // Completion word.  Every workgroup of the grid comes through here, also those without a tile.  The barrier orders
   // the workgroup's stores before thread 0's increment, which releases them at agent scope; the workgroup that counts
   // the last one has thereby acquired every other workgroup's stores, and its store of the word releases all of them
@@ -930,8 +993,9 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_runs(CopyRuns a) {
 // argument block the batch kernels take -- into a ring in pinned memory and advances a tail word; one workgroup of the
 // resident kernel (the dispatcher) polls the tail, copies new descriptors into device memory and publishes them, and
 // the other workgroups (the workers) run every batch's tiles through the same routine the launched kernels run
-// (fused_tile): first the striping of their tiles, then the reassembly of the same tiles, so that a tile is read back
-// by the workgroup that staged it and no workgroup waits for another inside a batch.  A batch's tiles go to the
+// (fused_tile): a tile is loaded once and stored twice, into its lane's staging window and on to where the staged bytes
+// go next (the receive buffer, or the receiving process's landing window), so no workgroup waits for another inside
+// a batch and nothing is read back.  A batch's tiles go to the
 // workers in turn, starting behind the worker that took the last tile of the batch before, so that small batches
 // run side by side on different workers.  Only the workers with a share in a batch are counted in and out of it: the
 // others pass it by without an atomic, so what a small batch costs does not grow with the size of the engine.  The
@@ -944,11 +1008,19 @@ __global__ __launch_bounds__(kCopyBlock) void fl_copy_runs(CopyRuns a) {
 // starts it again with the next batch), and a wait that outlasts wait_us reports an error and takes it down as well.
 constexpr uint32_t kEngineDevRing = 8;          // descriptors held in device memory; also the most window sets a caller may rotate
 constexpr uint32_t kEngineDescBytes = 4096;
-// A worker takes this many neighbouring copy tiles at a time: 64 KiB, what a workgroup has in flight when every thread
-// issues its sixteen loads at once.  With shares of one 32 KiB tile a 4 MiB batch on its own takes 11.3 instead of
-// 12.4 us, but four in flight are served every 6.2 instead of every 3.8 us (twice the workers per batch, so fewer
-// batches side by side), and a 16 MiB batch takes 20.9 instead of 18.4 us.
-constexpr uint32_t kEngineShare = 2;
+// A worker takes one copy tile at a time (32 KiB) from a batch that then still leaves a quarter of the workers to the
+// batches beside it, and two neighbouring tiles (64 KiB, what a workgroup has in flight when every thread issues its
+// sixteen loads at once) from a larger one.  Shares of one tile are latency: a batch of one or four 512 KiB requests on
+// its own takes 10.0 / 10.3 us instead of 12.1, four such in flight are served as fast either way (3.5-3.6 us each).
+// Shares of two are throughput: with one-tile shares a batch of eight spreads over all 128 workers and four in flight
+// are served every 6.1 instead of every 4.1 us.  Under the plugin (batches of three to five requests) a limit of 64, 96,
+// 128 tiles or none gave the same rates within the spread of three runs each, all of them above two-tile shares
+// throughout (one connection 849 against 886-971 GB/s, four 1 980 against 2 083-2 122).
+constexpr uint32_t kEngineShareMax = 2;
+inline uint32_t engine_share(uint32_t batch_tiles, uint32_t workers) {
+  const uint64_t upto = g_lane_share1_tiles < 0 ? (uint64_t)workers * 3 / 4 : (uint64_t)g_lane_share1_tiles;   // flh_tune("lane_share1_tiles")
+  return batch_tiles <= upto ? 1u : kEngineShareMax;
+}
 
 // What a batch does with its tiles.  Loop: user buffers -> staging windows -> receive buffers, both ends in this process.
 // Send: user buffers -> staging windows -> the same lane and offset of the landing windows (FusedArgs::carry), which are
@@ -958,7 +1030,8 @@ enum : uint32_t { kEngineLoop = FLH_ENGINE_LOOP, kEngineSend = FLH_ENGINE_SEND, 
 struct EngineDesc {                              // what the host writes per batch (kEngineDescBytes at most)
   uint32_t tiles;                                // worker shares of the batch (the slot's first word: the dispatcher's thread 0 has it in hand)
   uint32_t kind;
-  uint32_t pad[2];
+  uint32_t share;                                // copy tiles per share (engine_share)
+  uint32_t pad;
   FusedBatchCarryArgs a;                         // as the striping launch would take it (req_user = sources; kEngineRecv: the receive buffers)
   uint8_t* req_dst[FLH_BATCH_MAX];               // kEngineLoop: the reassembly side's buffers
 };
@@ -1012,7 +1085,19 @@ struct EngineArgs {
   uint64_t idle_ticks, wait_ticks;               // of the 100 MHz wall clock
   uint64_t resident_ticks;                       // the engine leaves after this long even with work at hand (0: never); the host starts it again
   uint32_t inject_fault;                         // tests of the failure path: fail in place of executing the first batch
+  uint32_t trace_mask;                           // trace slots - 1 (a power of two of them)
+  uint64_t* trace;                               // null, or kEngineStamps wall-clock stamps per slot: where a batch's time goes (flh_engine_trace)
 };
+
+// Stamps of one batch (100 MHz wall clock): the dispatcher has seen the host's tail beyond it; has published it; the
+// worker with its first share has seen the published word; may enter (the batch whose windows it reuses is complete);
+// has the descriptor in LDS; has moved its shares and its stores are in memory; the last worker out has the completion
+// word's store acknowledged.
+enum : uint32_t { kStampTail, kStampPublished, kStampSeen, kStampEntered, kStampDesc, kStampMoved, kStampDone, kEngineStamps };
+static_assert(kEngineStamps == FLH_ENGINE_STAMPS, "the header's count of stamps");
+__device__ __forceinline__ void engine_stamp(const EngineArgs& e, uint64_t k, uint32_t what) {
+  if (e.trace) __hip_atomic_store(&e.trace[(k & e.trace_mask) * kEngineStamps + what], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 __device__ __forceinline__ void engine_fail(const EngineArgs& e) {
   __hip_atomic_store(&e.hctl->error, (int32_t)FLH_E_STATE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -1064,6 +1149,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
         }
         if (act == 1) {
           idle_since = now;
+          engine_stamp(e, k, kStampTail);
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the workers' reads of the slot are behind their arrival
         } else if (__hip_atomic_load(&e.dctl->quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == e.gen ||
                    ((++polls & 31) == 0 && __hip_atomic_load(&e.hctl->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM))) {
@@ -1104,6 +1190,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
         tgt[slot] = own_target;
         e.dctl->target[slot] = own_target;
         __hip_atomic_store(&e.dctl->published[slot], engine_word(k, first_worker, tiles, own_target, wait_target), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        engine_stamp(e, k, kStampPublished);
         if (takers == 0) {   // nothing to move (the host submits no such batch): complete as it stands
           __hip_atomic_store(&e.hctl->done[slot], k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1148,6 +1235,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
       const uint32_t first = (uint32_t)(word >> 38) & 0x3ffu;
       sh_first = (w + W - first) % W;
       if (act == 1 && sh_first >= ((uint32_t)(word >> 28) & 0x3ffu)) act = 3;
+      if (act == 1 && sh_first == 0) engine_stamp(e, k, kStampSeen);
       if (act == 1 && k >= e.sets) {
         // batch k reuses the windows of batch k - sets: that one must be complete
         const uint64_t j = k - e.sets;
@@ -1158,6 +1246,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
           __builtin_amdgcn_s_sleep(1);
         }
       }
+      if (act == 1 && sh_first == 0) engine_stamp(e, k, kStampEntered);
       sh_flag = act;
       sh_word = word;
     }
@@ -1171,8 +1260,8 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     // What the batch reads may have been written by anyone, on this GPU or off it, before the host submitted it, and
     // what it writes is read by anyone once the host has seen it complete.  A worker therefore loads the descriptor and
     // the sources at system scope (mode 8: from memory, whatever line a cache has kept) and stores at system scope
-    // (mode 4: written through); only the windows are read back plainly, by the workgroup that has just written them,
-    // behind a barrier.  So it needs no cache invalidate on its way into a batch and no L2 write-back on its way out.
+    // (mode 4: written through).  So it needs no cache invalidate on its way into a batch and no L2 write-back on its
+    // way out.
     // Either of the two costs every workgroup that shares the XCD's L2: with 64 workers per batch fencing, batches of
     // eight 512 KiB requests were served every 7.4 us, now every 3.8 us.
     {
@@ -1181,54 +1270,45 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
       if (tid * 16 < sizeof(EngineDesc)) dst[tid] = slot(tid);
     }
     __syncthreads();
+    if (tid == 0 && mine == 0) engine_stamp(e, k, kStampDesc);
     const uint32_t tpc = d.a.tiles_per_chunk;
     const uint32_t total = tpc * d.a.n_chunks;
     const uint32_t kind = d.kind;
-    // a share is kEngineShare neighbouring tiles: one copy of twice the length when they lie in one chunk
-    const bool whole = tpc % kEngineShare == 0;
-    if (kind != kEngineRecv) {
-      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {                       // this worker's tiles, user buffers -> windows
-        const uint32_t t0 = sh * kEngineShare;
-        if (whole) fused_tile<0, 12>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
-        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<0, 12>(d.a, t % tpc, t / tpc);
-      }
-      __syncthreads();
-    }
+    // a share is `share` neighbouring tiles: one copy of that many times the length when they lie in one chunk
+    const uint32_t share = d.share;
+    const bool whole = tpc % share == 0;
     if (kind == kEngineLoop) {
-      if (tid < FLH_BATCH_MAX) d.a.req_user[tid] = d.req_dst[tid];                        // the same tiles, windows -> receive buffers
-      if (tid == 0) { d.a.table = nullptr; d.a.hdr = nullptr; }
-      __syncthreads();
-      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
-        const uint32_t t0 = sh * kEngineShare;
-        if (whole) fused_tile<1, 4>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
-        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<1, 4>(d.a, t % tpc, t / tpc);
+      // user buffers -> staging windows and, from the same registers, -> receive buffers: one pass, nothing read back
+      for (uint32_t sh = mine; sh * share < total; sh += W) {
+        const uint32_t t0 = sh * share;
+        if (whole) fused_tile<3, 12>(d.a, t0 % tpc, t0 / tpc, share, d.req_dst);
+        else for (uint32_t t = t0; t < total && t < t0 + share; ++t) fused_tile<3, 12>(d.a, t % tpc, t / tpc, 1, d.req_dst);
       }
     } else if (kind == kEngineSend) {
-      // the same tiles, this process's windows -> the receiving process's landing windows: read back plainly by the
-      // workgroup that wrote them, stored at system scope, so that they are in memory when the count says so
-      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
-        const uint32_t t0 = sh * kEngineShare;
-        if (whole) fused_tile<2, 4>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
-        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<2, 4>(d.a, t % tpc, t / tpc);
+      // user buffers -> staging windows and -> the same lane and offset of the receiving process's landing windows
+      for (uint32_t sh = mine; sh * share < total; sh += W) {
+        const uint32_t t0 = sh * share;
+        if (whole) fused_tile<3, 12>(d.a, t0 % tpc, t0 / tpc, share);
+        else for (uint32_t t = t0; t < total && t < t0 + share; ++t) fused_tile<3, 12>(d.a, t % tpc, t / tpc);
       }
     } else {
       // landing windows -> receive buffers.  Another process's kernel wrote the windows (written through, or written
       // back at the end of its kernel): loaded at system scope, whatever this XCD's L2 has kept of the set's last use.
-      for (uint32_t sh = mine; sh * kEngineShare < total; sh += W) {
-        const uint32_t t0 = sh * kEngineShare;
-        if (whole) fused_tile<1, 12>(d.a, t0 % tpc, t0 / tpc, kEngineShare);
-        else for (uint32_t t = t0; t < total && t < t0 + kEngineShare; ++t) fused_tile<1, 12>(d.a, t % tpc, t / tpc);
+      for (uint32_t sh = mine; sh * share < total; sh += W) {
+        const uint32_t t0 = sh * share;
+        if (whole) fused_tile<1, 12>(d.a, t0 % tpc, t0 / tpc, share);
+        else for (uint32_t t = t0; t < total && t < t0 + share; ++t) fused_tile<1, 12>(d.a, t % tpc, t / tpc);
       }
     }
     // Every thread waits until its stores have been written through and its loads have returned: the wave's memory
     // counter at zero.  (Written out: no fence stands for exactly this.  A release at workgroup scope waits for nothing,
     // a workgroup's accesses being ordered by the L1 they share; one at agent scope adds the L2 write-back that mode 4
-    // is there to avoid.)  Behind the barrier the whole share is in memory and its windows have been read, and the
-    // count says so.  The last worker to leave has read a count that every other one incremented after the same wait,
+    // is there to avoid.)  Behind the barrier the whole share is in memory, and the count says so.  The last worker to leave has read a count that every other one incremented after the same wait,
     // so the batch is in memory when it tells the host.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
+      if (mine == 0) engine_stamp(e, k, kStampMoved);
       const uint64_t before = __hip_atomic_fetch_add(cnt, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if ((((uint32_t)before + 1) & kEngineCountMask) == own_target) {
         __hip_atomic_store(&e.hctl->done[k % kEngineDevRing], k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -1236,6 +1316,7 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
         // never stored out of order
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __hip_atomic_store(&e.dctl->freed[k % kEngineDevRing], k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        engine_stamp(e, k, kStampDone);
       }
     }
   }
@@ -1716,6 +1797,8 @@ struct flh_engine {
   uint64_t completed;       // batches known complete, in order (atomic; moved forward by whoever looks)
   uint64_t launches;        // engine kernels started
   uint64_t idle_us, wait_us, resident_us;
+  uint64_t* d_trace;        // null unless the engine was created with flh_tune("engine_trace") set
+  uint32_t trace_slots;
 };
 
 int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_t window_sets, flh_engine** out) {
@@ -1750,11 +1833,28 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
     FL_HIP(hipMalloc((void**)&e->dev_ring, (size_t)kEngineDevRing * kEngineDescBytes));
     FL_HIP(hipMalloc((void**)&e->dctl, sizeof(EngineDevCtl)));
     FL_HIP(hipMemset(e->dctl, 0, sizeof(EngineDevCtl)));
+    if (g_engine_trace) {
+      e->trace_slots = 1024;
+      FL_HIP(hipMalloc((void**)&e->d_trace, (size_t)e->trace_slots * kEngineStamps * sizeof(uint64_t)));
+      FL_HIP(hipMemset(e->d_trace, 0, (size_t)e->trace_slots * kEngineStamps * sizeof(uint64_t)));
+    }
     return FLH_OK;
   };
   rc = build();
   if (rc) { (void)flh_engine_destroy(e); return rc; }
   *out = e;
+  return FLH_OK;
+}
+
+int flh_engine_trace(flh_engine* e, uint64_t first_seq, uint32_t n, uint64_t* stamps_out) {
+  if (!e || !stamps_out) return fl_set_error(FLH_E_ARG, "null engine or output");
+  if (!e->d_trace) return fl_set_error(FLH_E_STATE, "the engine keeps no trace: set flh_tune(\"engine_trace\", 1) before flh_engine_create");
+  if (first_seq == 0 || n == 0 || n > e->trace_slots || first_seq - 1 + n > flh_engine_completed(e) || flh_engine_completed(e) - (first_seq - 1) > e->trace_slots)
+    return fl_set_error(FLH_E_ARG, "batches %llu..%llu are not among the last %u complete ones", (unsigned long long)first_seq, (unsigned long long)(first_seq + n - 1), e->trace_slots);
+  std::vector<uint64_t> all((size_t)e->trace_slots * kEngineStamps);
+  FL_HIP(hipMemcpy(all.data(), e->d_trace, all.size() * sizeof(uint64_t), hipMemcpyDeviceToHost));
+  for (uint32_t i = 0; i < n; ++i)
+    memcpy(stamps_out + (size_t)i * kEngineStamps, &all[(size_t)((first_seq - 1 + i) & (e->trace_slots - 1)) * kEngineStamps], kEngineStamps * sizeof(uint64_t));
   return FLH_OK;
 }
 
@@ -1785,6 +1885,8 @@ static int engine_start(flh_engine* e) {
   a.wait_ticks = e->wait_us * 100;
   a.resident_ticks = e->resident_us * 100;
   a.inject_fault = g_engine_inject_fault ? 1u : 0u;
+  a.trace = e->d_trace;
+  a.trace_mask = e->trace_slots ? e->trace_slots - 1 : 0;
   __atomic_store_n(&e->h_ctl->state, 1u, __ATOMIC_RELEASE);
   hipLaunchKernelGGL(fl_engine_kernel, dim3(e->workers + 1), dim3(kCopyBlock), 0, e->stream, a);
   hipError_t err = hipGetLastError();
@@ -1853,7 +1955,8 @@ static int engine_submit(flh_engine* e, uint32_t kind, const flh_batch_params* b
   memcpy(&d->a, &a, sizeof(a));
   memcpy(d->req_dst, dsts, sizeof(dsts));
   d->kind = kind;
-  d->tiles = (a.n_chunks * a.tiles_per_chunk + kEngineShare - 1) / kEngineShare;
+  d->share = engine_share(a.n_chunks * a.tiles_per_chunk, e->workers);
+  d->tiles = (a.n_chunks * a.tiles_per_chunk + d->share - 1) / d->share;
   e->submitted = seq + 1;
   *seq_out = seq + 1;
   // The tail goes out, then the state is read; the dispatcher stores the state, then reads the tail: one of the two
@@ -1944,6 +2047,7 @@ int flh_engine_destroy(flh_engine* e) {
   if (e->h_ctl) (void)hipHostFree(e->h_ctl);
   if (e->dev_ring) (void)hipFree(e->dev_ring);
   if (e->dctl) (void)hipFree(e->dctl);
+  if (e->d_trace) (void)hipFree(e->d_trace);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   delete e;
   return FLH_OK;

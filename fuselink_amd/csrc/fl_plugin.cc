@@ -94,6 +94,7 @@ struct Params {
   // 945-990 GB/s with a bound of 1000 or more and at 780-970 with 500 or 250.
   int engine_resident_us = 1000;
   int engine_workgroups = 0;     // 0 = the library's default
+  int64_t engine_share1_tiles = -1;   // NCCL_FUSELINK_ENGINE_SHARE1_TILES: flh_tune("lane_share1_tiles"), -1 = the library's default
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
   int queue_depth = 2;           // NCCL_FUSELINK_QUEUE_DEPTH: a test launches what waits while fewer launches than this are queued on the GPU
   // NCCL_FUSELINK_EAGER_BATCH: this many waiting requests are a batch worth its own trip through the engine and go out
@@ -811,6 +812,8 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   g_par.engine_sets = (int)fl_param("FUSELINK_ENGINE_SETS", g_par.engine_sets);
   if (g_par.engine_sets < 1 || g_par.engine_sets > kEngineSetsMax) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_ENGINE_SETS must be 1..%d", kEngineSetsMax); return ncclInvalidArgument; }
   g_par.engine_workgroups = (int)fl_param("FUSELINK_ENGINE_WORKGROUPS", g_par.engine_workgroups);
+  g_par.engine_share1_tiles = fl_param("FUSELINK_ENGINE_SHARE1_TILES", g_par.engine_share1_tiles);
+  (void)flh_tune("lane_share1_tiles", g_par.engine_share1_tiles);
   g_par.engine_max_request = fl_param("FUSELINK_ENGINE_MAX_REQUEST", g_par.engine_max_request);
   if (g_par.engine_units < 1 || g_par.engine_idle_us < 1 || g_par.engine_workgroups < 0) { FL_WARN("NET/FuseLink : engine parameter out of range"); return ncclInvalidArgument; }
   g_par.batch_wait_ns = (int)fl_param("FUSELINK_BATCH_WAIT_NS", g_par.batch_wait_ns);

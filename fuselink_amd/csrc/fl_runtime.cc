@@ -30,8 +30,10 @@ int g_sched_uniform_fast = 1;
 int g_sched_seg_min = 4096;    // flh_tune("sched_seg_min"): chunks from which a workspace turns the scan into several workgroups
 int g_copy_uniform_grid = 1;
 int g_xcd_runs = 1;              // flh_tune("xcd_runs")
+int64_t g_lane_share1_tiles = -1;  // flh_tune("lane_share1_tiles"): engine batches of up to this many copy tiles go out in one-tile shares (-1: three quarters of the workers)
 int64_t g_engine_wait_us = 2000000;   // flh_tune("engine_wait_us"): limit of every wait inside a lane engine created afterwards
 int g_engine_inject_fault = 0;        // flh_tune("engine_inject_fault"): an engine started while this is set fails at its first batch
+int g_engine_trace = 0;               // flh_tune("engine_trace"): engines created afterwards keep wall-clock stamps of their batches (flh_engine_trace)
 int g_engine_fail_start = 0;          // flh_tune("engine_fail_start"): starting an engine fails as if the launch had been refused
 
 namespace {
@@ -179,6 +181,7 @@ int flh_tune(const char* key, int64_t value) {
   }
   if (!strcmp(key, "nontemporal")) { g_nontemporal = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "xcd_runs")) { g_xcd_runs = value == 2 ? 2 : value != 0; return FLH_OK; }
+  if (!strcmp(key, "lane_share1_tiles")) { g_lane_share1_tiles = value < 0 ? -1 : value; return FLH_OK; }
   if (!strncmp(key, "engine_", 7)) {
     // hooks for tests of the failure paths: a production process cannot reach them by accident
     const char* hooks = getenv("NCCL_FUSELINK_TEST_HOOKS");
@@ -186,6 +189,7 @@ int flh_tune(const char* key, int64_t value) {
     if (!strcmp(key, "engine_wait_us")) { if (value < 1) return fl_set_error(FLH_E_ARG, "engine_wait_us < 1"); g_engine_wait_us = value; return FLH_OK; }
     if (!strcmp(key, "engine_inject_fault")) { g_engine_inject_fault = value != 0; return FLH_OK; }
     if (!strcmp(key, "engine_fail_start")) { g_engine_fail_start = value != 0; return FLH_OK; }
+    if (!strcmp(key, "engine_trace")) { g_engine_trace = value != 0; return FLH_OK; }
   }
   if (!strcmp(key, "copy_uniform_grid")) { g_copy_uniform_grid = value != 0; return FLH_OK; }
   if (!strcmp(key, "sched_seg_min")) {

@@ -151,6 +151,9 @@ int64_t flh_constant(int which);
  * "sched_seg_min" = chunks from which a lent workspace makes the scan scheduler use several workgroups (4096).
  * "xcd_runs" = 1/0: launches of 256 copy workgroups and more hand each of the eight XCDs runs of 32 consecutive
  * tiles (1 MiB) instead of every eighth tile (1, the default; 3-5 % faster copies).
+ * "lane_share1_tiles" = lane-engine batches of up to this many copy tiles are handed to the workers one tile at a time
+ * (latency), larger ones two neighbouring tiles at a time (throughput); -1 = three quarters of the engine's workers,
+ * the default.
  * Test hooks (refused with FLH_E_STATE unless the environment holds NCCL_FUSELINK_TEST_HOOKS=1):
  * "engine_wait_us" = limit of every wait inside a lane engine created afterwards (2 000 000; tests of the failure
  * path ask for a microsecond).
@@ -159,6 +162,8 @@ int64_t flh_constant(int which);
  * one (0; for tests of the failure path, which cannot count on a healthy GPU to miss a limit).
  * "engine_fail_start" = 1: starting the resident kernel fails as a refused launch would (0; the submit that needed the
  * start must then return its error with the batch taken back out of the ring).
+ * "engine_trace" = 1: lane engines created afterwards stamp every batch's stages with the GPU's wall clock
+ * (flh_engine_trace; 0).
  * The same values can be preset with NCCL_FUSELINK_GRID_PER_CU / NCCL_FUSELINK_NONTEMPORAL.
  * The tunables are process-wide and read by every launch: set them while no other thread launches. */
 int flh_tune(const char* key, int64_t value);
@@ -271,12 +276,13 @@ int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows*
                        flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
 int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* win,
                            const flh_uniform_params* u, int32_t* d_status, void* stream);
-/* flh_stripe_uniform for a sender whose receiver is not this process: the workgroup that has staged a tile in its
- * lane's window carries it on into the same lane and offset of `landing`, windows of the receiver (its device memory,
- * opened here), which plays the part of the lane's NIC in the reference -- the RDMA write out of the staged copy into
- * the receiver's translated buffer (src/plugin.cc:1453-1495, 1582, 1626).  The receiver runs flh_reassemble_uniform
- * over its landing windows with the same parameters.  landing->cap bounds the carry as win->cap bounds the staging
- * (FLH_E_RANGE through *d_status).  The completion fields of `u` (done word / event) report this launch, which is the
+/* flh_stripe_uniform for a sender whose receiver is not this process: the workgroup that stages a tile in its
+ * lane's window writes it, from the same registers, into the same lane and offset of `landing` as well, windows of the
+ * receiver (its device memory, opened here), which plays the part of the lane's NIC in the reference -- the RDMA write
+ * out of the staged copy into the receiver's translated buffer (src/plugin.cc:1453-1495, 1582, 1626).  The receiver
+ * runs flh_reassemble_uniform over its landing windows with the same parameters.  landing->cap bounds the carry as
+ * win->cap bounds the staging (FLH_E_RANGE through *d_status; a chunk that would leave either window is written to
+ * neither).  The completion fields of `u` (done word / event) report this launch, which is the
  * last of the path on the sending side. */
 int flh_stripe_uniform_carry(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_windows* landing,
                              const flh_uniform_params* u, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
@@ -332,10 +338,11 @@ int flh_batch_layout(const flh_batch_params* b, uint64_t* lane_end, uint64_t* se
  * A resident kernel -- one dispatcher workgroup, the others workers, by default one worker per two compute units -- that
  * executes batches as flh_stripe_batch + flh_reassemble_batch would, but takes them from a descriptor ring in pinned
  * host memory instead of from kernel launches: flh_engine_submit writes the descriptor and advances a tail word (about
- * a microsecond of host time instead of about ten for a launch pair), the engine stripes every tile into the windows,
- * reassembles it from there and stores the batch's number to a host-visible word when its last workgroup has left the
- * batch (flh_engine_completed reads it: no call into the runtime).  Rows, header, staged bytes and received bytes are
- * those of the launched pair.  Several batches are in flight at once, so successive batches must not share staging
+ * a microsecond of host time instead of about ten for a launch pair), the engine stripes every tile into the windows
+ * and, from the registers it staged the tile from, writes it on into the receive buffer (nothing is read back: what
+ * the windows hold and what is received are the same loaded bytes), and stores the batch's number to a host-visible
+ * word when its last workgroup has left the batch (flh_engine_completed reads it: no call into the runtime).  Rows,
+ * header, staged bytes and received bytes are those of the launched pair.  Several batches are in flight at once, so successive batches must not share staging
  * windows: the caller rotates window_sets (1..8) sets of windows, batch number k taking set (k - 1) mod window_sets, and
  * the engine lets a batch in only once batch k - window_sets is complete.  With nothing to do for idle_us (default 200) the
  * engine goes down and the next submit starts it again with one launch.  Every wait inside the kernel is bounded;
@@ -347,8 +354,8 @@ int flh_engine_create(int device, uint32_t workgroups, uint32_t idle_us, uint32_
 int flh_engine_submit(flh_engine* e, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
                       flh_sched_hdr* d_hdr_out, int32_t* d_status, uint64_t* seq_out, uint64_t* seg_base_out);
 /* The two halves of a batch whose ends are different processes, numbered, ordered and reported like any other batch of
- * the engine.  FLH_ENGINE_SEND: stripe into `win` (the caller's rotating sets, as for flh_engine_submit) and carry every
- * tile on into `landing`, as flh_stripe_batch_carry does; b->d_dst is not used.  FLH_ENGINE_RECV: reassemble out of `win`
+ * the engine.  FLH_ENGINE_SEND: stripe into `win` (the caller's rotating sets, as for flh_engine_submit) and write every
+ * tile into the same lane and offset of `landing` as well, as flh_stripe_batch_carry does; b->d_dst is not used.  FLH_ENGINE_RECV: reassemble out of `win`
  * -- the landing windows a sender has filled -- into b->d_dst; b->d_src, `landing` (NULL) and the table pointers are not
  * used.  A batch is complete when its bytes are in memory: the landing windows' for a send, the receive buffers' for a
  * receive.  Stands where the reference's NIC stands on either side (src/plugin.cc:1453-1495 / 1616-1677). */
@@ -365,6 +372,15 @@ int flh_engine_submit_wire(flh_engine* e, uint32_t kind, const flh_batch_params*
  * whether flh_engine_poke would start it (two loads of host memory).  flh_engine_poke is not thread-safe against
  * flh_engine_submit. */
 int flh_engine_set_resident(flh_engine* e, uint32_t resident_us);
+/* Measurement (no counterpart in the reference): where the batches first_seq .. first_seq + n - 1 (numbers as
+ * flh_engine_submit returned them, all complete, among the last 1024) spent their time inside the resident kernel.
+ * FLH_ENGINE_STAMPS values of the GPU's 100 MHz wall clock per batch: the dispatcher saw the host's tail beyond the
+ * batch; it published the batch to the workers; the worker with the first share saw that; it was let in (the batch
+ * whose windows this one reuses was complete); it had the descriptor; it had moved its shares (their stores in
+ * memory); the last worker out had the completion word's store acknowledged.  Only for an engine created while flh_tune("engine_trace") was set (FLH_E_STATE otherwise);
+ * synchronous (a device-to-host copy). */
+#define FLH_ENGINE_STAMPS 7
+int flh_engine_trace(flh_engine* e, uint64_t first_seq, uint32_t n, uint64_t* stamps_out);
 int flh_engine_needs_start(const flh_engine* e);
 int flh_engine_poke(flh_engine* e);
 uint64_t flh_engine_completed(const flh_engine* e);   /* batches complete: all with a number up to this one */

@@ -2,11 +2,15 @@
 // plugin around it: what a batch costs one at a time, what it costs with several in flight, and what a submit costs
 // that has to start the resident kernel again.  dlopen()s the library and prints one JSON line.
 //
-//   engine_bench <lib.so> [--requests N] [--depth D] [--workgroups W] [--batches B]
+//   engine_bench <lib.so> [--requests N] [--depth D] [--workgroups W] [--batches B] [--span-mib S] [--trace 1] [--share1-tiles T]
 // N requests per batch (1..32), D window sets = batches in flight (1..8), W workgroups of the engine (0 = default).
+// --trace 1 (needs NCCL_FUSELINK_TEST_HOOKS=1): the engine stamps every batch's stages with the GPU's wall clock; a second
+// JSON line gives the median time between consecutive stamps, for the batches that ran one at a time and for those
+// that ran `depth` at a time, beside the host's submit -> completion seen for the same batches.
 #include <dlfcn.h>
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -22,17 +26,17 @@ static double now_us() { return std::chrono::duration<double, std::micro>(std::c
 
 int main(int argc, char** argv) {
   if (argc < 2) { fprintf(stderr, "usage: %s <libnccl-net-fuselink.so> [--requests N] [--depth D] [--workgroups W] [--batches B] [--span-mib S]\n", argv[0]); return 1; }
-  int nreq = 8, depth = 2, wgs = 0, batches = 2000, span_mib = 0;
+  int nreq = 8, depth = 2, wgs = 0, batches = 2000, span_mib = 0, trace = 0, share1 = -1;
   for (int i = 2; i + 1 < argc; i += 2) {
     const std::string a = argv[i];
     const int v = atoi(argv[i + 1]);
-    if (a == "--requests") nreq = v; else if (a == "--depth") depth = v; else if (a == "--workgroups") wgs = v; else if (a == "--batches") batches = v; else if (a == "--span-mib") span_mib = v;
+    if (a == "--requests") nreq = v; else if (a == "--depth") depth = v; else if (a == "--workgroups") wgs = v; else if (a == "--batches") batches = v; else if (a == "--span-mib") span_mib = v; else if (a == "--trace") trace = v; else if (a == "--share1-tiles") share1 = v;
   }
   if (nreq < 1 || nreq > FLH_BATCH_MAX || depth < 1 || depth > 8 || batches < 1) { fprintf(stderr, "arguments out of range\n"); return 1; }
   void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
   if (!lib) { fprintf(stderr, "dlopen: %s\n", dlerror()); return 1; }
 #define SYM(name) decltype(&name) p_##name = (decltype(&name))dlsym(lib, #name); if (!p_##name) { fprintf(stderr, "missing %s\n", #name); return 1; }
-  SYM(flh_init) SYM(flh_last_error) SYM(flh_engine_create) SYM(flh_engine_submit) SYM(flh_engine_completed) SYM(flh_engine_error) SYM(flh_engine_launches) SYM(flh_engine_destroy) SYM(flh_engine_needs_start) SYM(flh_engine_poke)
+  SYM(flh_init) SYM(flh_last_error) SYM(flh_engine_create) SYM(flh_engine_submit) SYM(flh_engine_completed) SYM(flh_engine_error) SYM(flh_engine_launches) SYM(flh_engine_destroy) SYM(flh_engine_needs_start) SYM(flh_engine_poke) SYM(flh_engine_trace) SYM(flh_tune)
   HIP(hipSetDevice(0));
   if (p_flh_init(0)) { fprintf(stderr, "init: %s\n", p_flh_last_error()); return 1; }
   const size_t req = 512 << 10, lanes = 8, cap = 4 << 20;
@@ -63,6 +67,9 @@ int main(int argc, char** argv) {
   for (int q = 0; q < nreq; ++q) b.bytes[q] = req;
   uint64_t submitted = 0;
   flh_engine* e = nullptr;
+  if (share1 >= 0 && p_flh_tune("lane_share1_tiles", share1)) { fprintf(stderr, "tune: %s\n", p_flh_last_error()); return 1; }
+  if (trace && p_flh_tune("engine_trace", 1)) { fprintf(stderr, "trace: %s\n", p_flh_last_error()); return 1; }
+  if (trace && batches > 400) batches = 400;   // the engine keeps the stamps of its last 1024 batches
   if (p_flh_engine_create(0, wgs, 200, depth, &e)) { fprintf(stderr, "engine: %s\n", p_flh_last_error()); return 1; }
   uint64_t seq = 0;
   auto submit = [&](int set) {
@@ -80,8 +87,11 @@ int main(int argc, char** argv) {
   for (int i = 0; i < 10; ++i) { submit(i % depth); wait_for(seq); }
   // one batch at a time
   double t0 = now_us(), sub = 0;
-  for (int i = 0; i < batches; ++i) { const double a = now_us(); submit(i % depth); sub += now_us() - a; wait_for(seq); }
+  std::vector<double> host_alone;
+  const uint64_t alone_first = seq + 1;
+  for (int i = 0; i < batches; ++i) { const double a = now_us(); submit(i % depth); sub += now_us() - a; wait_for(seq); host_alone.push_back(now_us() - a); }
   const double alone = (now_us() - t0) / batches;
+  const uint64_t piped_first = seq + 1;
   // `depth` batches in flight
   t0 = now_us();
   for (int i = 0; i < batches; ++i) { submit(i % depth); if (seq >= (uint64_t)depth) wait_for(seq - depth + 1); }
@@ -108,6 +118,32 @@ int main(int argc, char** argv) {
          "\"after_idle_submit_us\": %.1f, \"after_idle_batch_us\": %.1f, \"engine_launches\": %llu}\n",
          nreq, req, span_mib > 0 ? span >> 20 : (size_t)0, depth, wgs, batches, exact ? "true" : "false", alone, sub / batches, piped, piped / nreq, 4.0 * nreq * req / (piped * 1e-6) / 1e9,
          restart_submit / R, restart_done / R, (unsigned long long)p_flh_engine_launches(e));
+  if (trace) {
+    // median ticks (10 ns) between consecutive stamps
+    auto stages = [&](uint64_t first, uint32_t n, const char* name) {
+      std::vector<uint64_t> st((size_t)n * FLH_ENGINE_STAMPS);
+      if (p_flh_engine_trace(e, first, n, st.data())) { fprintf(stderr, "trace: %s\n", p_flh_last_error()); exit(1); }
+      printf("\"%s\": {", name);
+      static const char* const what[FLH_ENGINE_STAMPS] = {"", "tail_seen_to_published", "published_to_seen_by_first_worker", "seen_to_let_in", "let_in_to_descriptor_in_lds",
+                                                          "descriptor_to_shares_moved_and_in_memory", "moved_to_completion_word_acknowledged"};
+      for (int k = 1; k <= FLH_ENGINE_STAMPS; ++k) {
+        std::vector<double> d;
+        for (uint32_t i = 0; i < n; ++i) {
+          const uint64_t a = st[(size_t)i * FLH_ENGINE_STAMPS + (k < FLH_ENGINE_STAMPS ? k - 1 : 0)], b = st[(size_t)i * FLH_ENGINE_STAMPS + (k < FLH_ENGINE_STAMPS ? k : FLH_ENGINE_STAMPS - 1)];
+          if (a && b && b >= a) d.push_back((double)(b - a) / 100.0);
+        }
+        std::sort(d.begin(), d.end());
+        printf("\"%s_us\": %.2f, ", k < FLH_ENGINE_STAMPS ? what[k] : "tail_seen_to_completion_word_acknowledged", d.empty() ? -1.0 : d[d.size() / 2]);
+      }
+      printf("\"batches\": %u}", n);
+    };
+    std::sort(host_alone.begin(), host_alone.end());
+    printf("{\"harness\": \"engine_trace\", \"requests_per_batch\": %d, \"window_sets\": %d, \"host_submit_to_completion_seen_one_at_a_time_us\": %.2f, ", nreq, depth, host_alone[host_alone.size() / 2]);
+    stages(alone_first, (uint32_t)batches, "one_at_a_time");
+    printf(", ");
+    stages(piped_first, (uint32_t)batches, "in_flight");
+    printf("}\n");
+  }
   p_flh_engine_destroy(e);
   return exact ? 0 : 5;
 }

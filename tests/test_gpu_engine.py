@@ -271,3 +271,52 @@ def test_a_wait_that_runs_out_takes_the_engine_down_and_is_reported(fl):
         _lib.check(lib.flh_engine_destroy(eng))     # waits for the kernel: it has left, or leaves at its next poll
         assert time.time() - t0 < 5
         torch.cuda.synchronize()
+
+
+def test_the_engine_stamps_the_stages_of_its_batches_when_asked(fl):
+    """Measurement: an engine created while flh_tune("engine_trace") is set stamps every batch's stages with the GPU's wall
+    clock (dispatcher saw the tail, published, first worker saw it, was let in, had the descriptor, had moved its shares,
+    completion word acknowledged).  Stamps of a batch never run backwards, a batch's whole stay in the kernel is
+    microseconds, and an engine created without the switch refuses the call."""
+    core, torch, _lib = fl
+    lib = _lib.load()
+    lib.flh_tune.argtypes = [C.c_char_p, C.c_int64]
+    lanes, chunk, n = 4, 64 << 10, 12
+    plain = C.c_void_p()
+    _lib.check(lib.flh_engine_create(0, 0, 200, 2, C.byref(plain)))
+    assert lib.flh_tune(b"engine_trace", 1) == 0
+    eng = C.c_void_p()
+    try:
+        _lib.check(lib.flh_engine_create(0, 0, 200, 2, C.byref(eng)))
+    finally:
+        assert lib.flh_tune(b"engine_trace", 0) == 0
+    try:
+        cap = 1 << 20
+        wins = [[torch.zeros(cap, dtype=torch.uint8, device="cuda") for _ in range(lanes)] for _ in range(2)]
+        W = [core.make_windows([t.data_ptr() for t in ws], [cap] * lanes) for ws in wins]
+        status = core.new_status()
+        src_np = np.random.default_rng(5).integers(0, 256, size=6 * chunk + 100, dtype=np.uint8)
+        src = _dev(torch, src_np)
+        dsts = [torch.zeros(src_np.size, dtype=torch.uint8, device="cuda") for _ in range(n)]
+        out = core.new_schedule_buffers(8)
+        torch.cuda.synchronize()
+        seq = C.c_uint64()
+        for k in range(n):
+            b = core.batch_params([src], [dsts[k]], chunk, [2, 1, 1, 3])
+            _lib.check(lib.flh_engine_submit(eng, C.byref(b), C.byref(W[k % 2]), out.table.data_ptr(), out.hdr.data_ptr(), status.data_ptr(), C.byref(seq), None))
+            _wait(lib, eng, seq.value)
+        stamps = (C.c_uint64 * (7 * n))()
+        _lib.check(lib.flh_engine_trace(eng, 1, n, stamps))
+        st = np.frombuffer(stamps, dtype=np.uint64).reshape(n, 7).astype(np.int64)
+        assert (st > 0).all()
+        assert (np.diff(st, axis=1) >= 0).all(), st
+        assert ((st[:, -1] - st[:, 0]) < 100 * 1000).all()          # under a millisecond of the 100 MHz clock
+        assert (np.diff(st[:, 0]) > 0).all()                        # batch after batch
+        assert lib.flh_engine_trace(eng, 1, n + 1, stamps) != 0      # not complete yet
+        assert lib.flh_engine_trace(plain, 1, 1, stamps) != 0        # keeps no trace
+        torch.cuda.synchronize()
+        for k in range(n):
+            np.testing.assert_array_equal(dsts[k].cpu().numpy(), src_np)
+    finally:
+        _lib.check(lib.flh_engine_destroy(eng))
+        _lib.check(lib.flh_engine_destroy(plain))
