@@ -69,11 +69,13 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-iters", type=int, default=1000, help="timed CPU passes at 64 MiB (scaled down for larger messages): about 5 s of CPU work per figure")
     ap.add_argument("--hint", type=int, default=1, help="pass the host-known header fields to the copy kernels")
-    ap.add_argument("--path", default="auto", choices=["auto", "fused", "split", "carry"],
+    ap.add_argument("--path", default="auto", choices=["auto", "fused", "split", "carry", "deliver"],
                     help="fused: scheduler folded into the striping launch (uniform split, one credit row); split: three launches; "
                          "carry: the launches of a transfer whose receiver is another process and has not exported its buffer -- the striping "
                          "launch also carries every staged tile into a second set of windows (the receiver's landing windows, here a plain "
-                         "allocation of this process), the reassembly reads from those; not a bench line")
+                         "allocation of this process), the reassembly reads from those; deliver: the one launch of a transfer whose receive buffer the "
+                         "sender can write itself -- staged into the windows and written into the destination from the same registers "
+                         "(flh_stage_deliver_uniform; 3 x bytes per step instead of 4); neither is the bench line")
     ap.add_argument("--lds", type=int, default=0, help="paged workload: stage the gather through LDS")
     ap.add_argument("--cold-user-buffers", type=int, default=1,
                     help="also time the step over source/destination pairs in rotation (1 GiB), so that no user buffer is "
@@ -378,10 +380,11 @@ def main() -> int:
     # header fields that follow from the uniform split alone; the kernels then need not wait for d_hdr
     hint = core.uniform_hint(msg_bytes, chunk) if (args.hint and kind == "uniform") else None
     carry = args.path == "carry"
-    if carry and (kind != "uniform" or rows != 1 or epoch_len != 0 or waves or cwaves or twaves):
-        print("bench.py: --path carry takes a uniform workload under one credit row that moves in one launch pair", file=sys.stderr)
+    deliver = args.path == "deliver"
+    if (carry or deliver) and (kind != "uniform" or rows != 1 or epoch_len != 0 or waves or cwaves or twaves):
+        print("bench.py: --path carry and --path deliver take a uniform workload under one credit row that moves in one launch pair", file=sys.stderr)
         return 2
-    fused = not waves and not cwaves and not twaves and kind in ("uniform", "pages") and (args.path in ("fused", "carry") or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
+    fused = not waves and not cwaves and not twaves and kind in ("uniform", "pages") and (args.path in ("fused", "carry", "deliver") or (args.path == "auto" and rows == 1 and epoch_len == 0 and msg_chunks <= 65535))
     if fused and (rows != 1 or epoch_len != 0):
         print("bench.py: the fused path takes a single credit row without epochs", file=sys.stderr)
         return 2
@@ -422,6 +425,9 @@ def main() -> int:
                               mode=core.SCHED_RESET_OFFSETS, state=state, out=s_w, stream=stream, by_lane=by_lane)
                 core.stripe(src, win, s_w, status, stream=stream, hint=h_w, by_lane=by_lane)
                 core.reassemble(dst, win, s_w, status, stream=stream, hint=h_w)
+        elif deliver:
+            # staging and delivery in one launch (source -> staging windows and destination)
+            core.stage_deliver_uniform(src, dst, win, uni, status, out=sched, stream=stream)
         elif carry:
             # staging and the wire in one launch (source -> staging windows -> landing windows), delivery out of the landing windows
             core.stripe_uniform_carry(src, win, landing, uni, status, out=sched, stream=stream)
@@ -462,7 +468,9 @@ def main() -> int:
 
     per = profiled(steps_again, (8 + 2 * len(cwaves or ()) + 3 * len(waves or ()) + 2 * len(twaves or ())) * args.steps)
     mean = lambda xs: sum(xs) / len(xs)
-    out_k, in_k = ("gather", "scatter") if kind == "pages" else ("stripe", "reassemble")
+    out_k, in_k = ("gather", "scatter") if kind == "pages" else ("stage_deliver", "reassemble") if deliver else ("stripe", "reassemble")
+    if deliver:
+        per.setdefault(in_k, [0.0])   # (no second launch)
     stripe_us, reasm_us = mean(per[out_k]), mean(per[in_k])
     stripe_min, reasm_min = min(per[out_k]), min(per[in_k])
     launches_per_step = len(per[out_k]) // args.steps
@@ -604,7 +612,9 @@ def main() -> int:
 
     algo_bytes_step = 4 * nbytes          # stripe: read N + write N; reassemble: read N + write N
     algo_bytes_kernel = 2 * msg_bytes // len(waves or cwaves or twaves or (0,))    # one launch of the copy kernel (with waves: the average one)
-    if carry:
+    if deliver:
+        algo_bytes_step = 3 * nbytes      # read N, write N into the windows, write N into the destination
+    if carry or deliver:
         algo_bytes_kernel = 3 * msg_bytes   # read N, write N into the staging windows, write N into the landing windows (every vector loaded once, stored twice)
     value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
     pair_us = (stripe_us + reasm_us) * launches_per_step
@@ -613,6 +623,8 @@ def main() -> int:
         kernel_name = "fl_copy_uniform_fused<0, FusedPageArgs> (gather)"
     elif kind == "pages":
         kernel_name = f"fl_page_tiles<0, lds={args.lds}> (gather)"
+    elif deliver:
+        kernel_name = "fl_copy_uniform_fused<0, FusedCarryArgs> (stage + deliver)"
     elif carry:
         kernel_name = "fl_copy_uniform_fused<0, FusedCarryArgs> (stripe + carry)"
     elif fused or cwaves:
@@ -644,6 +656,7 @@ def main() -> int:
                    "lanes": lanes, "credits": credits_np.tolist() if rows == 1 else f"{rows} seeded rows in [1,8]", "epoch_len": epoch_len,
                    "step": ("2x(gather(with scheduler folded in)+scatter)" if (kind == "pages" and fused) else "2x(schedule+gather+scatter)" if kind == "pages" else
                             "stripe(with scheduler folded in)+carry into landing windows, then reassemble out of them" if carry else
+                            "one launch: stage into the windows (scheduler folded in) and deliver into the destination; value counts 3 x bytes" if deliver else
                             "stripe(with scheduler folded in)+reassemble" if fused else
                             f"{len(cwaves)} waves of stripe(with scheduler folded in)+reassemble over cache-resident windows" if cwaves else
                             f"schedule, then {len(twaves)} waves of stripe+reassemble over cache-resident windows" if twaves else "schedule+stripe+reassemble"),

@@ -84,6 +84,9 @@ SIGNATURES = {
     "flh_stripe_uniform_carry": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,
                                            C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_stripe_batch_carry": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "flh_stage_deliver_batch": (C.c_int, [C.POINTER(BatchParams), C.POINTER(Windows), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "flh_stage_deliver_uniform": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64, C.POINTER(Windows), C.POINTER(UniformParams), C.c_void_p,
+                                            C.c_void_p, C.c_void_p, C.c_void_p]),
     "flh_engine_submit_wire": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(BatchParams), C.POINTER(Windows), C.POINTER(Windows), C.c_void_p, C.c_void_p,
                                          C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "flh_engine_set_resident": (C.c_int, [C.c_void_p, C.c_uint32]),

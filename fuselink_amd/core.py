@@ -38,7 +38,7 @@ def tune(key: str, value: int) -> None:
     check(_lib.load().flh_tune(key.encode(), int(value)))
 
 
-PROF_KERNELS = {1: "schedule", 2: "stripe", 3: "reassemble", 4: "gather", 5: "scatter", 6: "copy"}
+PROF_KERNELS = {1: "schedule", 2: "stripe", 3: "reassemble", 4: "gather", 5: "scatter", 6: "copy", 7: "stage_deliver"}
 
 
 def prof_begin(capacity: int) -> None:
@@ -240,6 +240,14 @@ def stripe_uniform(src: torch.Tensor, win: Windows, u: UniformParams, status: to
     check(_lib.load().flh_stripe_uniform(_ptr(src), src.numel() * src.element_size(), C.byref(win), C.byref(u),
                                          _ptr(out.table) if out else None, _ptr(out.hdr) if out else None, _ptr(status),
                                          _stream_ptr(stream)))
+
+
+def stage_deliver_uniform(src: torch.Tensor, dst: torch.Tensor, win: Windows, u: UniformParams, status: torch.Tensor, out: Optional[Schedule] = None,
+                          stream: Optional[torch.cuda.Stream] = None) -> None:
+    """flh_stage_deliver_uniform: stripe into `win` and write every tile into the same place of `dst`, in one launch."""
+    check(_lib.load().flh_stage_deliver_uniform(_ptr(src), src.numel() * src.element_size(), _ptr(dst), dst.numel() * dst.element_size(), C.byref(win),
+                                                C.byref(u), _ptr(out.table) if out else None, _ptr(out.hdr) if out else None, _ptr(status),
+                                                _stream_ptr(stream)))
 
 
 def stripe_uniform_carry(src: torch.Tensor, win: Windows, landing: Windows, u: UniformParams, status: torch.Tensor, out: Optional[Schedule] = None,

@@ -313,21 +313,23 @@ __device__ __forceinline__ void block_copy(uint8_t* __restrict__ dst, const uint
 // One source, two destinations: every vector is loaded once and stored twice (staging window and the wire's far end,
 // or staging window and receive buffer), so the second copy costs no second read and no barrier between a workgroup's
 // store and its re-load.  When the three addresses are not equally aligned the bytes are copied twice from the source.
-template <int NT>
+// NT is the streaming mode of the loads and of the stores to d1, NT2's store bits that of the stores to d2.
+template <int NT, int NT2>
 __device__ __forceinline__ void block_copy2(uint8_t* __restrict__ d1, uint8_t* __restrict__ d2, const uint8_t* __restrict__ src, uint32_t bytes) {
   const uintptr_t sa = (uintptr_t)src;
   if ((((sa ^ (uintptr_t)d1) | (sa ^ (uintptr_t)d2)) & 15) != 0) {
     block_copy<NT>(d1, src, bytes);
-    block_copy<NT>(d2, src, bytes);
+    block_copy<NT2>(d2, src, bytes);
     return;
   }
   const uint32_t tid = threadIdx.x;
   uint32_t head = (uint32_t)((16 - (sa & 15)) & 15);
   if (head > bytes) head = bytes;
-  if (tid < head) { copy1<NT>(d1 + tid, src + tid); copy1<NT>(d2 + tid, src + tid); }
+  if (tid < head) { copy1<NT>(d1 + tid, src + tid); copy1<NT2>(d2 + tid, src + tid); }
   const uint32_t nvec = (bytes - head) >> 4;
   const VecIn<NT> in((const u32x4*)(src + head), nvec);
-  const VecOut<NT> out1((u32x4*)(d1 + head), nvec), out2((u32x4*)(d2 + head), nvec);
+  const VecOut<NT> out1((u32x4*)(d1 + head), nvec);
+  const VecOut<NT2> out2((u32x4*)(d2 + head), nvec);
   auto exact = [&](auto U_) {
     constexpr int U = decltype(U_)::value;
     u32x4 r[U];
@@ -358,7 +360,7 @@ __device__ __forceinline__ void block_copy2(uint8_t* __restrict__ d1, uint8_t* _
   }
   const uint32_t tail0 = head + (nvec << 4);
   const uint32_t tail = bytes - tail0;
-  if (tid < tail) { copy1<NT>(d1 + tail0 + tid, src + tail0 + tid); copy1<NT>(d2 + tail0 + tid, src + tail0 + tid); }
+  if (tid < tail) { copy1<NT>(d1 + tail0 + tid, src + tail0 + tid); copy1<NT2>(d2 + tail0 + tid, src + tail0 + tid); }
 }
 
 struct CopyArgs {
@@ -566,8 +568,11 @@ struct FusedBatchArgs : FusedArgs {
 // lane's window then carries it into the same lane and offset of this set, the part the NIC of that lane plays in the
 // reference (an RDMA write out of the staged copy, plugin.cc:1453-1495, 1582).  Argument blocks of their own, so that
 // the launches without a wire keep theirs as they are.
-struct FusedCarryArgs : FusedArgs { flh_windows carry; };
-struct FusedBatchCarryArgs : FusedBatchArgs { flh_windows carry; };
+// Where a staged tile goes next is either the same lane and offset of `carry` or, when `onward` names a buffer, the
+// same place of that buffer as the tile has in its source: the receive buffer of a receiver whose memory this process
+// can write (itself, or a process that exported the buffer), which is where the reference's RDMA write lands.
+struct FusedCarryArgs : FusedArgs { flh_windows carry; uint8_t* onward; uint64_t onward_bytes; };
+struct FusedBatchCarryArgs : FusedBatchArgs { flh_windows carry; uint8_t* onward[FLH_BATCH_MAX]; };   // one per request, or all null
 static_assert(sizeof(FusedBatchCarryArgs) <= 4096, "a kernel's argument block holds 4 KiB");
 template <class A> struct is_batch { static constexpr bool value = false; };
 template <> struct is_batch<FusedBatchArgs> { static constexpr bool value = true; };
@@ -619,11 +624,10 @@ __device__ __forceinline__ uint64_t fused_cnt(uint64_t W, uint64_t K, uint64_t h
 // One workgroup's share of a fused launch: tile bx of the chunk that grid row by stands for (`span` neighbouring tiles
 // of that chunk from bx on, for a caller that hands out larger shares).  DIR 0: user buffer -> staging window, 1: window
 // -> user buffer, 2: staging window -> the same lane and offset of the carry windows (the wire), 3: user buffer -> staging
-// window and, from the same registers, on to where the staged bytes go next: the same place of the request's buffer in
-// `onward` (one buffer per request of a batch: the receive buffers) or, without one, the same lane and offset of the
-// carry windows.
+// window and, from the same registers, on to where the staged bytes go next: the same place of the arguments' onward
+// buffer (the message's, or the request's in a batch) or, without one, the same lane and offset of the carry windows.
 template <int DIR, int NT, class Args>
-__device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by, uint32_t span = 1, uint8_t* const* onward = nullptr) {
+__device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t by, uint32_t span = 1) {
   constexpr bool BATCH = is_batch<Args>::value;
   constexpr bool PAGED = is_paged<Args>::value;
   if (by >= a.n_chunks) return;
@@ -656,7 +660,7 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
     before = (uint64_t)full * (hi - K) + (slot - K) - g.cnt0[lane];
     win_base = (uint64_t)g.base128[lane] * 128u;
     user = a.req_user[r];
-    if (DIR == 3 && onward) onward_user = onward[r];
+    if constexpr (DIR == 3) onward_user = a.onward[r];
     user_bytes = a.req_bytes[r];
     user_off = (uint64_t)(c - a.first[r]) * a.chunk_bytes;
     const uint64_t rem = user_bytes - user_off;
@@ -721,6 +725,13 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
     len = (uint32_t)(rem < a.chunk_bytes ? rem : a.chunk_bytes);
     src_off = a.src_base + chunk_off;
     user_off = src_off;
+    if constexpr (DIR == 3) {
+      onward_user = a.onward;
+      if (onward_user && user_off + len > a.onward_bytes) {
+        if (bx == 0 && threadIdx.x == 0) st_obj<NT>(a.status, (int32_t)FLH_E_RANGE);
+        return;
+      }
+    }
   }
   const uint64_t win_off = win_base + before * a.chunk_bytes;
 
@@ -833,14 +844,16 @@ __device__ __forceinline__ void fused_tile(const Args& a, uint32_t bx, uint32_t 
     block_copy<NT>((uint8_t*)a.carry.base[lane] + win_off + off, w, bytes);
   } else if constexpr (DIR == 3) {
     static_assert(has_carry<Args>::value && !PAGED, "the second destination is a receive buffer or a landing window");
+    // bit 4 of the mode: the window's stores stream (bit 1 speaks for the stores that go on)
+    constexpr int NTW = (NT & ~(2 | 16)) | ((NT & 16) ? 2 : 0), NTO = NT & ~16;
     if (onward_user) {
-      block_copy2<NT>(w, onward_user + user_off + off, u, bytes);
+      block_copy2<NTW, NTO>(w, onward_user + user_off + off, u, bytes);
     } else {
       if (win_off + len > a.carry.cap[lane]) {   // refused whole: nothing of the chunk is staged either
         if (threadIdx.x == 0) st_obj<NT>(a.status, (int32_t)FLH_E_RANGE);
         return;
       }
-      block_copy2<NT>(w, (uint8_t*)a.carry.base[lane] + win_off + off, u, bytes);
+      block_copy2<NTW, NTO>(w, (uint8_t*)a.carry.base[lane] + win_off + off, u, bytes);
     }
   } else if constexpr (DIR == 0) {
     block_copy<NT>(w, u, bytes);
@@ -1032,8 +1045,7 @@ struct EngineDesc {                              // what the host writes per bat
   uint32_t kind;
   uint32_t share;                                // copy tiles per share (engine_share)
   uint32_t pad;
-  FusedBatchCarryArgs a;                         // as the striping launch would take it (req_user = sources; kEngineRecv: the receive buffers)
-  uint8_t* req_dst[FLH_BATCH_MAX];               // kEngineLoop: the reassembly side's buffers
+  FusedBatchCarryArgs a;                         // as the striping launch would take it (req_user = sources, onward = the receive buffers of a kEngineLoop batch; kEngineRecv: req_user = the receive buffers)
 };
 static_assert(sizeof(EngineDesc) <= kEngineDescBytes, "descriptor slot too small");
 
@@ -1277,15 +1289,10 @@ __global__ __launch_bounds__(kCopyBlock) void fl_engine_kernel(EngineArgs e) {
     // a share is `share` neighbouring tiles: one copy of that many times the length when they lie in one chunk
     const uint32_t share = d.share;
     const bool whole = tpc % share == 0;
-    if (kind == kEngineLoop) {
-      // user buffers -> staging windows and, from the same registers, -> receive buffers: one pass, nothing read back
-      for (uint32_t sh = mine; sh * share < total; sh += W) {
-        const uint32_t t0 = sh * share;
-        if (whole) fused_tile<3, 12>(d.a, t0 % tpc, t0 / tpc, share, d.req_dst);
-        else for (uint32_t t = t0; t < total && t < t0 + share; ++t) fused_tile<3, 12>(d.a, t % tpc, t / tpc, 1, d.req_dst);
-      }
-    } else if (kind == kEngineSend) {
-      // user buffers -> staging windows and -> the same lane and offset of the receiving process's landing windows
+    if (kind != kEngineRecv) {
+      // user buffers -> staging windows and, from the same registers, on: into the receive buffers (kEngineLoop, the
+      // descriptor's onward buffers) or into the same lane and offset of the receiving process's landing windows
+      // (kEngineSend).  One pass, nothing read back.
       for (uint32_t sh = mine; sh * share < total; sh += W) {
         const uint32_t t0 = sh * share;
         if (whole) fused_tile<3, 12>(d.a, t0 % tpc, t0 / tpc, share);
@@ -1450,7 +1457,7 @@ int flh_reassemble(void* d_dst, uint64_t dst_bytes, const flh_windows* win, cons
 
 // argument checks and everything of FusedArgs that follows from the parameters; returns 1 when there is nothing to do
 static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_uniform_params* u, flh_chunk_desc* d_table,
-                      flh_sched_hdr* d_hdr, int32_t* d_status, const flh_windows* carry = nullptr) {
+                      flh_sched_hdr* d_hdr, int32_t* d_status, const flh_windows* carry = nullptr, bool onward = false) {
   int rc = check_windows(win);
   if (rc) return rc;
   if (carry) {   // (the caller's argument block holds the windows themselves)
@@ -1468,15 +1475,17 @@ static int fill_fused(FusedArgs& a, int dir, const flh_windows* win, const flh_u
   if (n > 65535) return fl_set_error(FLH_E_ARG, "%llu chunks exceed the 65535 one launch can name; split the message", (unsigned long long)n);
   rc = fl_need_init();
   if (rc) return rc;
-  fl_prof().kid = dir == 0 ? 2 : 3;
+  if (onward && (dir != 0 || carry)) return fl_set_error(FLH_E_ARG, "a launch delivers into receive buffers or carries into landing windows, from the striping side");
+  fl_prof().kid = dir == 0 ? (onward ? 7 : 2) : 3;
+  const bool last = dir == 1 || carry || onward;   // the launch that ends the path on this side reports
   a.user = nullptr;
   a.user_bytes = 0;
   a.win = *win;
   a.table = dir == 0 ? d_table : nullptr;
   a.hdr = dir == 0 ? d_hdr : nullptr;
   a.status = d_status;
-  a.done_word = dir == 1 || carry ? u->d_done_word : nullptr;   // the launch that ends the path on this side reports
-  a.done_count = dir == 1 || carry ? u->d_done_count : nullptr;
+  a.done_word = last ? u->d_done_word : nullptr;
+  a.done_count = last ? u->d_done_count : nullptr;
   a.done_value = u->done_value;
   if (a.done_word && !a.done_count) return fl_set_error(FLH_E_ARG, "d_done_word needs d_done_count");
   a.start_word = u->d_start_word;
@@ -1525,7 +1534,16 @@ static int launch_fused_args(int dir, const Args& a, int mode, void* stream, voi
   if (dir == 0) {
     if (mode == 0) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 0 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
     else if (mode == 1) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 1 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
-    else FL_LAUNCH_EV((fl_copy_uniform_fused<0, 3 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+    else if (mode == 3) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 3 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+    else if constexpr (has_carry<Args>::value) {
+      // a launch with two destinations: bit 1 for the stores that go on, bit 4 for the stores into the staging windows
+      if (mode == 2) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 2 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+      else if (mode == 16) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 16 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+      else if (mode == 18) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 18 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+      else if (mode == 19) FL_LAUNCH_EV((fl_copy_uniform_fused<0, 19 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
+      else return fl_set_error(FLH_E_ARG, "streaming mode %d of a launch with two destinations is not built", mode);
+    }
+    else return fl_set_error(FLH_E_ARG, "streaming mode %d of a striping launch is not built", mode);
   } else if constexpr (!has_carry<Args>::value) {   // (only the striping side carries)
     if (mode == 0) FL_LAUNCH_EV((fl_copy_uniform_fused<1, 0 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
     else if (mode == 2) FL_LAUNCH_EV((fl_copy_uniform_fused<1, 2 FL_ARGS_EXTRA>), grid, dim3(kCopyBlock), 0, s, ev, a);
@@ -1537,17 +1555,37 @@ static int launch_fused_args(int dir, const Args& a, int mode, void* stream, voi
 }
 }  // extern "C++"
 
+// Streaming mode of a launch that stages and delivers: the windows are written and not read again and the receive
+// buffer is read by whoever comes next, so the stores stream from the size on from which the reassembly's do, the loads
+// from the size on from which the striping's do.
+static int deliver_mode(uint64_t total_bytes) {
+  if (g_stream_force_deliver >= 0) return g_stream_force_deliver;
+  // (the windows stay cacheable for as long as the striping launch's do: rewritten by the next message before the
+  // Infinity Cache has given them up, they cost no traffic to memory at all)
+  const int out = fl_stream_mode(0, total_bytes);
+  return (out & 1) | (fl_stream_mode(1, total_bytes) & 2) | ((out & 2) ? 16 : 0);
+}
+// ... that carries into landing windows, which the receiving process reads next: both kinds of window alike
+static int carry_mode(uint64_t total_bytes) {
+  const int out = fl_stream_mode(0, total_bytes);
+  return out | ((out & 2) ? 16 : 0);
+}
+
 static int launch_fused(int dir, void* user, uint64_t user_bytes, const flh_windows* win, const flh_uniform_params* u,
-                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream, const flh_windows* carry = nullptr) {
+                        flh_chunk_desc* d_table, flh_sched_hdr* d_hdr, int32_t* d_status, void* stream, const flh_windows* carry = nullptr,
+                        void* onward = nullptr, uint64_t onward_bytes = 0) {
   FusedCarryArgs a;
-  const int rc = fill_fused(a, dir, win, u, d_table, d_hdr, d_status, carry);
+  const int rc = fill_fused(a, dir, win, u, d_table, d_hdr, d_status, carry, onward != nullptr);
   if (rc) return rc < 0 ? rc : FLH_OK;
   if (!user) return fl_set_error(FLH_E_ARG, "user buffer missing");
   a.user = (uint8_t*)user;
   a.user_bytes = user_bytes;
-  if (!carry) return launch_fused_args(dir, static_cast<const FusedArgs&>(a), fl_stream_mode(dir, u->total_bytes), stream, u->done_event);
-  a.carry = *carry;
-  return launch_fused_args(dir, a, fl_stream_mode(dir, u->total_bytes), stream, u->done_event);
+  if (!carry && !onward) return launch_fused_args(dir, static_cast<const FusedArgs&>(a), fl_stream_mode(dir, u->total_bytes), stream, u->done_event);
+  memset(&a.carry, 0, sizeof(a.carry));
+  if (carry) a.carry = *carry;
+  a.onward = (uint8_t*)onward;
+  a.onward_bytes = onward_bytes;
+  return launch_fused_args(dir, a, onward ? deliver_mode(u->total_bytes) : carry_mode(u->total_bytes), stream, u->done_event);
 }
 
 // What a batch comes to: its segments as the kernel takes them, and where each lane's window ends up.
@@ -1630,7 +1668,7 @@ int flh_batch_layout(const flh_batch_params* b, uint64_t* lane_end, uint64_t* se
 }
 
 static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table, flh_sched_hdr* d_hdr,
-                        int32_t* d_status, void* stream, const flh_windows* carry = nullptr) {
+                        int32_t* d_status, void* stream, const flh_windows* carry = nullptr, bool onward = false) {
   BatchPlan pl;
   int rc = plan_batch(b, pl);
   if (rc) return rc;
@@ -1640,7 +1678,7 @@ static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* w
   flh_uniform_params u = b->u;
   u.total_bytes = (uint64_t)pl.n_chunks * b->u.chunk_bytes;
   u.epoch_bytes = 0;
-  rc = fill_fused(a, dir, win, &u, d_table, d_hdr, d_status, carry);
+  rc = fill_fused(a, dir, win, &u, d_table, d_hdr, d_status, carry, onward);
   if (rc) return rc < 0 ? rc : FLH_OK;
   a.total_bytes = b->u.total_bytes;
   a.dest_order = 0;
@@ -1652,16 +1690,19 @@ static int launch_batch(int dir, const flh_batch_params* b, const flh_windows* w
     a.seg_of[q] = pl.seg_of[q];
     a.req_user[q] = nullptr;
     a.req_bytes[q] = 0;
+    a.onward[q] = nullptr;
     if (q >= b->n_req) continue;
     void* p = dir == 0 ? (void*)b->d_src[q] : b->d_dst[q];
-    if (!p) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer", q);
+    if (!p || (onward && !b->d_dst[q])) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer", q);
     a.req_user[q] = (uint8_t*)p;
     a.req_bytes[q] = b->bytes[q];
+    if (onward) a.onward[q] = (uint8_t*)b->d_dst[q];
   }
   for (uint32_t k = 0; k < FLH_SEG_MAX; ++k) a.seg[k] = pl.seg[k];
-  if (!carry) return launch_fused_args(dir, static_cast<const FusedBatchArgs&>(a), fl_stream_mode(dir, b->u.total_bytes), stream, b->u.done_event);
-  a.carry = *carry;
-  return launch_fused_args(dir, a, fl_stream_mode(dir, b->u.total_bytes), stream, b->u.done_event);
+  if (!carry && !onward) return launch_fused_args(dir, static_cast<const FusedBatchArgs&>(a), fl_stream_mode(dir, b->u.total_bytes), stream, b->u.done_event);
+  memset(&a.carry, 0, sizeof(a.carry));
+  if (carry) a.carry = *carry;
+  return launch_fused_args(dir, a, onward ? deliver_mode(b->u.total_bytes) : carry_mode(b->u.total_bytes), stream, b->u.done_event);
 }
 
 static int launch_fused_pages(int dir, void* pool, uint64_t pool_pages, const uint32_t* d_page_table, uint32_t page_bytes,
@@ -1709,10 +1750,21 @@ int flh_stripe_uniform(const void* d_src, uint64_t src_bytes, const flh_windows*
   return launch_fused(0, (void*)d_src, src_bytes, win, u, d_table_out, d_hdr_out, d_status, stream);
 }
 
+int flh_stage_deliver_uniform(const void* d_src, uint64_t src_bytes, void* d_dst, uint64_t dst_bytes, const flh_windows* win,
+                              const flh_uniform_params* u, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
+  if (!d_dst) return fl_set_error(FLH_E_ARG, "receive buffer missing");
+  return launch_fused(0, (void*)d_src, src_bytes, win, u, d_table_out, d_hdr_out, d_status, stream, nullptr, d_dst, dst_bytes);
+}
+
 int flh_stripe_uniform_carry(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_windows* landing,
                              const flh_uniform_params* u, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream) {
   if (!landing) return fl_set_error(FLH_E_ARG, "null landing windows");
   return launch_fused(0, (void*)d_src, src_bytes, win, u, d_table_out, d_hdr_out, d_status, stream, landing);
+}
+
+int flh_stage_deliver_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
+                            int32_t* d_status, void* stream) {
+  return launch_batch(0, b, win, d_table_out, d_hdr_out, d_status, stream, nullptr, true);
 }
 
 int flh_stripe_batch_carry(const flh_batch_params* b, const flh_windows* win, const flh_windows* landing, flh_chunk_desc* d_table_out,
@@ -1938,22 +1990,20 @@ static int engine_submit(flh_engine* e, uint32_t kind, const flh_batch_params* b
   a.xcd_map = 0;                        // the engine's workers take tiles by their own stride
   a.n_req = b->n_req;
   a.n_seg = pl.n_seg;
-  uint8_t* dsts[FLH_BATCH_MAX];
   for (uint32_t q = 0; q < FLH_BATCH_MAX; ++q) {
     a.first[q] = pl.first[q];
     a.seg_of[q] = pl.seg_of[q];
     a.req_user[q] = nullptr;
     a.req_bytes[q] = 0;
-    dsts[q] = nullptr;
+    a.onward[q] = nullptr;
     if (q >= b->n_req) continue;
     if ((kind != kEngineRecv && !b->d_src[q]) || (kind != kEngineSend && !b->d_dst[q])) return fl_set_error(FLH_E_ARG, "request %u of the batch has no buffer", q);
     a.req_user[q] = kind == kEngineRecv ? (uint8_t*)b->d_dst[q] : (uint8_t*)b->d_src[q];
     a.req_bytes[q] = b->bytes[q];
-    dsts[q] = kind == kEngineLoop ? (uint8_t*)b->d_dst[q] : nullptr;
+    if (kind == kEngineLoop) a.onward[q] = (uint8_t*)b->d_dst[q];
   }
   for (uint32_t k = 0; k < FLH_SEG_MAX; ++k) a.seg[k] = pl.seg[k];
   memcpy(&d->a, &a, sizeof(a));
-  memcpy(d->req_dst, dsts, sizeof(dsts));
   d->kind = kind;
   d->share = engine_share(a.n_chunks * a.tiles_per_chunk, e->workers);
   d->tiles = (a.n_chunks * a.tiles_per_chunk + d->share - 1) / d->share;

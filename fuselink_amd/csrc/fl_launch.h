@@ -30,6 +30,7 @@ extern FL_LOCAL int g_engine_fail_start;
 extern FL_LOCAL int g_engine_trace;
 extern FL_LOCAL int g_copy_uniform_grid;
 extern FL_LOCAL int64_t g_lane_share1_tiles;
+extern FL_LOCAL int g_stream_force_deliver;
 extern FL_LOCAL int g_xcd_runs;            // copy workgroups take their tiles in runs per XCD (see xcd_tile)
 constexpr uint64_t kCacheResidentBytes = 512ull << 20;  // plain copy: working sets up to this stay largely in the 256 MB Infinity Cache
 constexpr uint64_t kWindowsCacheableBytes = 256ull << 20;  // a message whose staging windows still fit the Infinity Cache

@@ -93,6 +93,10 @@ struct Params {
   // or 250 -- and 0.8 ms with no engine at all.  Every restart costs the transfer a launch: the same 1 GiB moved at
   // 945-990 GB/s with a bound of 1000 or more and at 780-970 with 500 or 250.
   int engine_resident_us = 1000;
+  // NCCL_FUSELINK_ONE_PASS: 1 = a launch that can write the receive buffer itself (receiver in this process, or its
+  // buffer mapped here) stages and delivers in one kernel, every vector loaded once and stored twice, as the engine's
+  // batches do; 0 = a striping launch and a reassembly launch out of the windows
+  int one_pass = 1;
   int engine_workgroups = 0;     // 0 = the library's default
   int64_t engine_share1_tiles = -1;   // NCCL_FUSELINK_ENGINE_SHARE1_TILES: flh_tune("lane_share1_tiles"), -1 = the library's default
   int64_t engine_max_request = 1 << 20;   // requests above this size travel by launches
@@ -811,6 +815,8 @@ ncclResult_t fl_init(ncclDebugLogger_t logFunction) {
   if (g_par.engine_resident_us < 0) g_par.engine_resident_us = 0;
   g_par.engine_sets = (int)fl_param("FUSELINK_ENGINE_SETS", g_par.engine_sets);
   if (g_par.engine_sets < 1 || g_par.engine_sets > kEngineSetsMax) { FL_WARN("NET/FuseLink : NCCL_FUSELINK_ENGINE_SETS must be 1..%d", kEngineSetsMax); return ncclInvalidArgument; }
+  g_par.one_pass = (int)fl_param("FUSELINK_ONE_PASS", g_par.one_pass) != 0;
+  (void)flh_tune("stream_mode_deliver", fl_param("FUSELINK_DELIVER_STREAM_MODE", -1));   // an experiment's knob: see flh_tune
   g_par.engine_workgroups = (int)fl_param("FUSELINK_ENGINE_WORKGROUPS", g_par.engine_workgroups);
   g_par.engine_share1_tiles = fl_param("FUSELINK_ENGINE_SHARE1_TILES", g_par.engine_share1_tiles);
   (void)flh_tune("lane_share1_tiles", g_par.engine_share1_tiles);
@@ -1186,12 +1192,21 @@ ncclResult_t launch_transfer(Peer* pr, const Pending& p, uint64_t seq) {
       flh_uniform_params u;
       fill_uniform(u, credits, wave, (uint64_t)qoff[q] + done, lk->epoch_bytes, launch_tile(wave));
       start_stamp(pr, seq, u);
-      FL_FLHCHECK(flh_stripe_uniform(p.src, (uint64_t)p.size, &pr->wins, &u, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
-      if (q == last_q && done + wave == piece) {
-        ncclResult_t rc = prepare_completion(pr, seq, wave, u, comp);
-        if (rc != ncclSuccess) return rc;
+      if (g_par.one_pass) {
+        // one launch per wave: staged into the windows and written into the receive buffer from the same registers
+        if (q == last_q && done + wave == piece) {
+          ncclResult_t rc = prepare_completion(pr, seq, wave, u, comp);
+          if (rc != ncclSuccess) return rc;
+        }
+        FL_FLHCHECK(flh_stage_deliver_uniform(p.src, (uint64_t)p.size, p.dst, (uint64_t)p.size, &pr->wins, &u, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+      } else {
+        FL_FLHCHECK(flh_stripe_uniform(p.src, (uint64_t)p.size, &pr->wins, &u, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+        if (q == last_q && done + wave == piece) {
+          ncclResult_t rc = prepare_completion(pr, seq, wave, u, comp);
+          if (rc != ncclSuccess) return rc;
+        }
+        FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &pr->wins, &u, pr->d_status, pr->stream));
       }
-      FL_FLHCHECK(flh_reassemble_uniform(p.dst, (uint64_t)p.size, &pr->wins, &u, pr->d_status, pr->stream));
       const uint32_t rows = (uint32_t)((wave + chunk - 1) / chunk);
       pr->last.seq = seq;
       pr->last.engine = false;
@@ -1453,6 +1468,16 @@ ncclResult_t launch_batch(Peer* pr, size_t i, size_t n, BatchBuild& bb, bool eng
     ncclResult_t rc = prepare_completion(pr, seq, b.u.total_bytes, b.u, comp);   // the carrying launch is the last of the path on this side
     if (rc != ncclSuccess) return rc;
     FL_FLHCHECK(flh_stripe_batch_carry(&b, &pr->wins, &pair->landing_wins[set], pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
+    rc = finish_completion(pr, seq, comp);
+    if (rc != ncclSuccess) return rc;
+  } else if (g_par.one_pass) {
+    // one launch stages the batch and writes the receive buffers (this process's, or another's mapped through their
+    // registrations)
+    start_stamp(pr, seq, b.u);
+    Completion comp;
+    ncclResult_t rc = prepare_completion(pr, seq, b.u.total_bytes, b.u, comp);
+    if (rc != ncclSuccess) return rc;
+    FL_FLHCHECK(flh_stage_deliver_batch(&b, &pr->wins, pr->d_table, pr->d_hdr, pr->d_status, pr->stream));
     rc = finish_completion(pr, seq, comp);
     if (rc != ncclSuccess) return rc;
   } else {

@@ -63,6 +63,7 @@ bool fl_use_nt(uint64_t working_set_bytes) {
   return working_set_bytes > kCacheResidentBytes;
 }
 
+int g_stream_force_deliver = -1;    // flh_tune("stream_mode_deliver"): -1 = from the two policies below
 int g_stream_force[2] = {-1, -1};   // flh_tune("stream_mode_out" / "stream_mode_in"): -1 = the policy below
 
 int fl_stream_mode(int dir, uint64_t bytes) {
@@ -174,6 +175,11 @@ int flh_tune(const char* key, int64_t value) {
   if (!strcmp(key, "grid_per_cu")) { if (value < 0) return fl_set_error(FLH_E_ARG, "grid_per_cu < 0"); g_grid_per_cu = (int)value; return FLH_OK; }
   if (!strcmp(key, "stripe_dest_order")) { g_dest_order = value < 0 ? -1 : (value != 0); return FLH_OK; }
   if (!strcmp(key, "fused_fast")) { g_fused_fast = value != 0; return FLH_OK; }
+  if (!strcmp(key, "stream_mode_deliver")) {
+    if (value < -1 || (value & ~19)) return fl_set_error(FLH_E_ARG, "%s: -1, or bits 0 (loads), 1 (stores that go on) and 4 (stores into the windows)", key);
+    g_stream_force_deliver = (int)value;
+    return FLH_OK;
+  }
   if (!strcmp(key, "stream_mode_out") || !strcmp(key, "stream_mode_in")) {
     if (value < -1 || value > 3) return fl_set_error(FLH_E_ARG, "%s not in -1..3", key);
     g_stream_force[key[12] == 'i'] = (int)value;

@@ -145,7 +145,8 @@ int64_t flh_constant(int which);
  * stores everywhere / nowhere (-1, the default: per side -- user buffers stream once a launch moves 16 (written side) or 128 MiB (read side),
  * the staging windows stay cacheable until a message passes 256 MiB and they outgrow the Infinity Cache).
  * "stream_mode_out" / "stream_mode_in" = 0..3 force the mode of the striping / reassembly side (bit 0 loads,
- * bit 1 stores; -1 = the policy).
+ * bit 1 stores; -1 = the policy).  "stream_mode_deliver" = the same for flh_stage_deliver_*, with bit 4 for the stores into
+ * the windows (-1: loads and window stores as the striping side's, the other stores as the reassembly side's).
  * "stripe_dest_order" = 0/1: flh_stripe_uniform walks the chunks lane by lane, so that every window is written
  * front to back (-1 = only for messages past 256 MiB, whose windows no longer fit the Infinity Cache, the default).
  * "sched_seg_min" = chunks from which a lent workspace makes the scan scheduler use several workgroups (4096).
@@ -172,7 +173,7 @@ int flh_tune(const char* key, int64_t value);
  * own start/stop HIP events that bracket the kernel alone; the launches stay asynchronous.
  * flh_prof_end waits for them and returns how many were recorded, filling up to `max` durations
  * (microseconds) and the entry point that launched each: 1 schedule, 2 stripe, 3 reassemble,
- * 4 gather, 5 scatter, 6 copy.  Launches beyond `capacity` are not timed. */
+ * 4 gather, 5 scatter, 6 copy, 7 stage + deliver.  Launches beyond `capacity` are not timed. */
 int flh_prof_begin(int capacity);
 int flh_prof_end(double* us_out, int* kernel_out, int max);
 
@@ -287,6 +288,16 @@ int flh_reassemble_uniform(void* d_dst, uint64_t dst_bytes, const flh_windows* w
 int flh_stripe_uniform_carry(const void* d_src, uint64_t src_bytes, const flh_windows* win, const flh_windows* landing,
                              const flh_uniform_params* u, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
                              int32_t* d_status, void* stream);
+/* flh_stripe_uniform + flh_reassemble_uniform in one launch, for a sender that can write the receive buffer itself
+ * (the receiver is this process, or a process whose registered buffer is mapped here): every workgroup loads its tile
+ * of the message once and stores it twice, into its lane's staging window -- table, header and staged bytes are those
+ * of flh_stripe_uniform -- and at the same offset of d_dst as the tile has in d_src, which is where the reference's
+ * RDMA write out of the staged copy lands (src/plugin.cc:1453-1495: remote_addr + offset).  A chunk that would leave its
+ * window, the source or d_dst (dst_bytes) is written nowhere (FLH_E_RANGE through *d_status).  The completion fields of
+ * `u` report this launch. */
+int flh_stage_deliver_uniform(const void* d_src, uint64_t src_bytes, void* d_dst, uint64_t dst_bytes, const flh_windows* win,
+                              const flh_uniform_params* u, flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out,
+                              int32_t* d_status, void* stream);
 
 /* Several requests in one launch: requests that are waiting together -- NCCL keeps up to NCCL_STEPS = 8 in flight per
  * channel (src/fuselink.h:14) and runs several channels to a peer, which all share the per-NIC lane comms
@@ -327,6 +338,10 @@ typedef struct flh_batch_params {
 int flh_stripe_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
                      flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
 int flh_reassemble_batch(const flh_batch_params* b, const flh_windows* win, int32_t* d_status, void* stream);
+/* flh_stripe_batch + flh_reassemble_batch in one launch, as flh_stage_deliver_uniform: request q's bytes go into the
+ * windows and into b->d_dst[q]. */
+int flh_stage_deliver_batch(const flh_batch_params* b, const flh_windows* win, flh_chunk_desc* d_table_out,
+                            flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);
 /* flh_stripe_batch with the carry of flh_stripe_uniform_carry (b->d_dst is not used). */
 int flh_stripe_batch_carry(const flh_batch_params* b, const flh_windows* win, const flh_windows* landing,
                            flh_chunk_desc* d_table_out, flh_sched_hdr* d_hdr_out, int32_t* d_status, void* stream);

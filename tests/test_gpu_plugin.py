@@ -11,7 +11,8 @@ pytestmark = pytest.mark.gpu
 
 ENV_KEYS = ["NCCL_FUSELINK_LANES", "NCCL_FUSELINK_CHUNKSIZE", "NCCL_FUSELINK_POLICY", "NCCL_FUSELINK_WINDOW_UNITS",
             "NCCL_FUSELINK_POOL_UNITS", "NCCL_FUSELINK_REFRESH_BATCH", "NCCL_IB_QPS_PER_CONNECTION", "NCCL_FUSELINK_CREDITS",
-            "NCCL_FUSELINK_BATCH", "NCCL_FUSELINK_COMPLETION", "NCCL_FUSELINK_ENGINE", "NCCL_FUSELINK_ENGINE_SETS", "NCCL_FUSELINK_ENGINE_UNITS"]
+            "NCCL_FUSELINK_BATCH", "NCCL_FUSELINK_COMPLETION", "NCCL_FUSELINK_ENGINE", "NCCL_FUSELINK_ENGINE_SETS", "NCCL_FUSELINK_ENGINE_UNITS",
+            "NCCL_FUSELINK_ONE_PASS"]
 
 
 @pytest.fixture()
@@ -354,18 +355,19 @@ def test_mixed_host_and_device_buffers(net):
     net.closeSend(s), net.closeRecv(r), net.closeListen(lcomm)
 
 
-@pytest.mark.parametrize("completion,engine", [(0, 0), (1, 0), (2, 0), (2, 1)])
+@pytest.mark.parametrize("completion,engine,one_pass", [(0, 0, 1), (1, 0, 1), (2, 0, 1), (2, 1, 1), (0, 0, 0), (1, 0, 0), (2, 0, 0)])
 @pytest.mark.parametrize("batch", [1, 8])
-def test_completion_reaches_test_in_every_mode(net, completion, engine, batch):
+def test_completion_reaches_test_in_every_mode(net, completion, engine, one_pass, batch):
     """How `test` learns that a launch is done -- an event behind every launch, an event on the launch's last kernel,
     the words that kernels store launch numbers to (a small launch's reassembly kernel when its last workgroup has
     finished, every striping kernel as it starts, an event only behind a large launch that nothing follows), or the
-    lane engine's completion word for the small requests it carries -- must not change what a consumer sees: every receive is compared on torch's own stream, which does not wait for the
+    lane engine's completion word for the small requests it carries -- must not change what a consumer sees, whether a
+    launch stages and delivers in one kernel (one_pass) or a striping and a reassembly kernel do: every receive is compared on torch's own stream, which does not wait for the
     connection's, the moment `test` reports it done, with requests in flight behind it, empty requests and host
     buffers mixed in, and a lone request at the end that no other launch follows."""
     import torch
     net.reconfigure(NCCL_FUSELINK_LANES=4, NCCL_FUSELINK_CHUNKSIZE=64 << 10, NCCL_FUSELINK_WINDOW_UNITS=1,
-                    NCCL_FUSELINK_BATCH=batch, NCCL_FUSELINK_COMPLETION=completion, NCCL_FUSELINK_ENGINE=engine)
+                    NCCL_FUSELINK_BATCH=batch, NCCL_FUSELINK_COMPLETION=completion, NCCL_FUSELINK_ENGINE=engine, NCCL_FUSELINK_ONE_PASS=one_pass)
     net.set_credits([3, 1, 2, 2])
     rng = np.random.default_rng(900 + completion * 10 + batch)
     n_req = 120
@@ -891,7 +893,8 @@ def test_random_traffic_of_several_connections_arrives_intact(net, seed):
     cadence = int(rng.choice([2, 8, 1000]))
     net.reconfigure(NCCL_FUSELINK_LANES=lanes, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_WINDOW_UNITS=int(rng.choice([1, 2, 4])),
                     NCCL_FUSELINK_REFRESH_BATCH=cadence, NCCL_FUSELINK_COMPLETION=completion, NCCL_FUSELINK_ENGINE=engine,
-                    NCCL_FUSELINK_ENGINE_SETS=int(rng.choice([1, 2, 3])), NCCL_FUSELINK_BATCH=int(rng.choice([2, 8, 32])))
+                    NCCL_FUSELINK_ENGINE_SETS=int(rng.choice([1, 2, 3])), NCCL_FUSELINK_BATCH=int(rng.choice([2, 8, 32])),
+                    NCCL_FUSELINK_ONE_PASS=int(seed % 3 != 2))
     net.set_credits([int(c) for c in rng.integers(0, 5, size=lanes)])
 
     def draw_size():

@@ -399,3 +399,112 @@ def test_test_hooks_are_refused_without_their_switch(fl, monkeypatch):
         assert lib.flh_tune(key, 1) == -6
     monkeypatch.setenv("NCCL_FUSELINK_TEST_HOOKS", "1")
     assert lib.flh_tune(b"engine_fail_start", 0) == 0
+
+
+# ---- stage + deliver in one launch: the sender writes the receive buffer itself ---------------------------------------
+
+@pytest.mark.parametrize("nbytes,chunk,lanes,epoch_chunks,src_skew,win_skew,dst_skew", [
+    ((4 << 20) + 4096 + 3, 256 << 10, 8, 0, 0, 0, 0), (64 << 20, 256 << 10, 8, 5, 0, 0, 0), (7 * (96 << 10) + 1, 96 << 10, 3, 2, 0, 0, 0),
+    ((3 << 20) + 77, 128 << 10, 4, 1, 5, 5, 5),   # source, windows and receive buffer equally misaligned: vectors with byte edges
+    ((3 << 20) + 77, 128 << 10, 4, 1, 0, 0, 9),   # the receive buffer misaligned against source and windows: two copies from the source
+    ((1 << 20) + 13, 100 * 128, 5, 3, 3, 0, 3),   # the windows misaligned against source and receive buffer
+    (300 << 20, 1 << 20, 16, 0, 0, 0, 0)])        # past 256 MiB: destination order, streaming loads and stores
+def test_a_launch_that_stages_and_delivers_equals_the_launch_pair(fl, nbytes, chunk, lanes, epoch_chunks, src_skew, win_skew, dst_skew):
+    """flh_stage_deliver_uniform: table, header and windows are flh_stripe_uniform's, the receive buffer
+    flh_reassemble_uniform's -- the oracle's -- and the bytes around the receive buffer stay untouched."""
+    core, torch, _lib = fl
+    lib = _lib.load()
+    rng = np.random.default_rng(nbytes % 9973 + lanes + dst_skew)
+    credits = rng.integers(1, 9, size=lanes).astype(np.uint32)
+    epoch = epoch_chunks * chunk
+    src_np = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+    exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
+                                         mode=ob.SCHED_RESET_OFFSETS, state=_state(epoch))
+    lane_bytes = [int(x) for x in exp_h["lane_bytes"][:lanes]]
+    src_buf = torch.zeros(nbytes + 64, dtype=torch.uint8, device="cuda")
+    src = src_buf[src_skew:src_skew + nbytes]
+    src.copy_(torch.from_numpy(src_np))
+    dst_buf = torch.full((nbytes + 128,), 0xEE, dtype=torch.uint8, device="cuda")
+    dst = dst_buf[32 + dst_skew:32 + dst_skew + nbytes]
+    stage_buf = [torch.zeros(max(b, 1) + 64, dtype=torch.uint8, device="cuda") for b in lane_bytes]
+    stage = [t[win_skew:] for t in stage_buf]
+    W = core.make_windows([t.data_ptr() for t in stage], lane_bytes)
+    status = core.new_status()
+    out = core.new_schedule_buffers(len(exp_t))
+    u = core.uniform_params(nbytes, chunk, credits.tolist(), epoch_bytes=epoch)
+    done = torch.zeros(64, dtype=torch.int32).pin_memory()
+    count = torch.zeros(64, dtype=torch.int32, device="cuda")
+    if nbytes < (8 << 20):
+        u.d_done_word, u.d_done_count, u.done_value = done.data_ptr(), count.data_ptr(), 43
+    core.stage_deliver_uniform(src, dst, W, u, status, out=out)
+    if nbytes < (8 << 20):
+        deadline = time.time() + 10
+        while int(done[0]) != 43:
+            assert time.time() < deadline, "the completion word never came"
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0 and int(count[0].item()) == 0
+    got = out.table_numpy()
+    for f in ob.DESC_DTYPE.names:
+        np.testing.assert_array_equal(got[f], exp_t[f], err_msg=f)
+    np.testing.assert_array_equal(out.hdr_numpy()["lane_bytes"][:lanes], exp_h["lane_bytes"][:lanes])
+    if nbytes <= (64 << 20):
+        exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+        for l in range(lanes):
+            np.testing.assert_array_equal(stage[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"staging window {l}")
+            assert not stage[l].cpu().numpy()[lane_bytes[l]:].any()
+    else:   # the windows, taken apart again by the reassembly launch, give the message back
+        back = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        core.reassemble_uniform(back, W, u, status)
+        torch.cuda.synchronize()
+        assert torch.equal(back, src)
+    back = dst_buf.cpu().numpy()
+    lo = 32 + dst_skew
+    np.testing.assert_array_equal(back[lo:lo + nbytes], src_np)
+    assert (back[:lo] == 0xEE).all() and (back[lo + nbytes:] == 0xEE).all()
+
+
+def test_a_delivery_that_would_leave_the_receive_buffer_is_refused(fl):
+    core, torch, _lib = fl
+    lib = _lib.load()
+    lanes, chunk, nbytes = 2, 64 << 10, 8 * (64 << 10)
+    src = torch.ones(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    stage = [torch.zeros(4 * chunk, dtype=torch.uint8, device="cuda") for _ in range(lanes)]
+    W = core.make_windows([t.data_ptr() for t in stage], [4 * chunk] * lanes)
+    status = core.new_status()
+    u = core.uniform_params(nbytes, chunk, [1, 1])
+    # the receive buffer is said to end one chunk early: the last chunk goes nowhere, not even into its window
+    _lib.check(lib.flh_stage_deliver_uniform(src.data_ptr(), nbytes, dst.data_ptr(), nbytes - chunk, C.byref(W), C.byref(u), None, None, status.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert int(status.item()) == -5                                                   # FLH_E_RANGE
+    d = dst.cpu().numpy()
+    assert d[:nbytes - chunk].all() and not d[nbytes - chunk:].any()
+    assert not stage[1].cpu().numpy()[3 * chunk:].any() and stage[0].cpu().numpy().all()
+    assert lib.flh_stage_deliver_uniform(src.data_ptr(), nbytes, None, nbytes, C.byref(W), C.byref(u), None, None, status.data_ptr(), None) == -1
+
+
+def test_a_batch_launch_that_stages_and_delivers_equals_the_batch_pair(fl):
+    core, torch, _lib = fl
+    lib = _lib.load()
+    rng = np.random.default_rng(812)
+    lanes, chunk, cap = 5, 32 << 10, 3 << 20
+    for _ in range(6):
+        bt = _random_batch(rng, torch, lanes, chunk)
+        stage = [torch.zeros(cap, dtype=torch.uint8, device="cuda") for _ in range(lanes)]
+        W = core.make_windows([t.data_ptr() for t in stage], [cap] * lanes)
+        status = core.new_status()
+        exp_rows, staged = _expect_batch(bt["segments"], bt["srcs_np"], lanes, chunk)
+        out = core.new_schedule_buffers(len(exp_rows))
+        b = core.batch_params(bt["srcs"], bt["dsts"], chunk, [1] * lanes, segments=bt["segments"])
+        _lib.check(lib.flh_stage_deliver_batch(C.byref(b), C.byref(W), out.table.data_ptr(), out.hdr.data_ptr(), status.data_ptr(), None))
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+        got = out.table_numpy()
+        for f in ob.DESC_DTYPE.names:
+            np.testing.assert_array_equal(got[f], exp_rows[f], err_msg=f)
+        for l, off, data in staged:
+            np.testing.assert_array_equal(stage[l].cpu().numpy()[off:off + data.size], data, err_msg=f"staging lane {l}")
+        for i, s in enumerate(bt["sizes"]):
+            g = bt["dsts"][i].cpu().numpy()
+            np.testing.assert_array_equal(g[:s], bt["srcs_np"][i], err_msg=f"request {i}")
+            assert not g[s:].any()
