@@ -129,7 +129,7 @@ def main() -> int:
         if os.path.exists(harness) and os.path.exists(flbuild.lib_path()):
             env = dict(os.environ, NCCL_FUSELINK_LANES="8", NCCL_FUSELINK_CHUNKSIZE=str(256 << 10))
             plugin = {"message_bytes": 64 << 20, "request_bytes": 512 << 10, "requests": 128, "inflight": 8, "lanes": 8, "chunk_bytes": 256 << 10,
-                      "accounting": "4 x bytes x connections / wall time of the best of 20 iterations, proxy threads started inside the timed region.  4 x bytes is the headline metric's accounting (stage: read N + write N, deliver: read N + write N) and what a launch pair moves; the lane engine, which carries requests of up to 1 MiB, stores every loaded vector twice (staging window and receive buffer) and so moves 3 x bytes for the same result: payload rate = GBps_4N / 4",
+                      "accounting": "4 x bytes x connections / wall time of the best of 20 iterations, proxy threads started inside the timed region.  4 x bytes is the headline metric's accounting (stage: read N + write N, deliver: read N + write N) and what a striping and a reassembly launch move; the plugin's engine batches and, by default, its launches load every vector once and store it twice (staging window and receive buffer) and so move 3 x bytes for the same result: payload rate = GBps_4N / 4",
                       "env": "NCCL_FUSELINK_LANES=8 NCCL_FUSELINK_CHUNKSIZE=262144"}
             for conns in (1, 4):
                 cmd = [harness, flbuild.lib_path(), "--bytes", str(64 << 20), "--request", str(512 << 10), "--inflight", "8", "--iters", "20",
