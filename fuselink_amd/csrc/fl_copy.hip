@@ -314,8 +314,23 @@ __device__ __forceinline__ void block_copy(uint8_t* __restrict__ dst, const uint
 // or staging window and receive buffer), so the second copy costs no second read and no barrier between a workgroup's
 // store and its re-load.  When the three addresses are not equally aligned the bytes are copied twice from the source.
 // NT is the streaming mode of the loads and of the stores to d1, NT2's store bits that of the stores to d2.
+template <int NT, int NT2, int U>
+__device__ __forceinline__ void copy2_exact(const VecOut<NT>& out1, const VecOut<NT2>& out2, const VecIn<NT>& in, uint32_t tid) {
+  u32x4 r[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) r[j] = in(j * kCopyBlock + tid);
+#pragma unroll
+  for (int j = 0; j < U; ++j) out1(j * kCopyBlock + tid, r[j]);
+#pragma unroll
+  for (int j = 0; j < U; ++j) out2(j * kCopyBlock + tid, r[j]);
+  // The stores above must stay in this block.  Left to itself the optimizer sinks the trailing stores of this path and
+  // of the predicated loop beside it into one shared block with the vector index as a phi, and the backend then left
+  // the index of the first store undefined on this path (seen in the generated code, and on the GPU as a lost or a wild
+  // store).  A marker that differs from path to path keeps the paths' tails apart.
+  asm volatile("; two-destination copy, %0 vectors per thread" ::"n"(U) : "memory");
+}
 template <int NT, int NT2>
-__device__ __forceinline__ void block_copy2(uint8_t* __restrict__ d1, uint8_t* __restrict__ d2, const uint8_t* __restrict__ src, uint32_t bytes) {
+__device__ __forceinline__ void block_copy2(uint8_t* d1, uint8_t* d2, const uint8_t* src, uint32_t bytes) {
   const uintptr_t sa = (uintptr_t)src;
   if ((((sa ^ (uintptr_t)d1) | (sa ^ (uintptr_t)d2)) & 15) != 0) {
     block_copy<NT>(d1, src, bytes);
@@ -330,32 +345,28 @@ __device__ __forceinline__ void block_copy2(uint8_t* __restrict__ d1, uint8_t* _
   const VecIn<NT> in((const u32x4*)(src + head), nvec);
   const VecOut<NT> out1((u32x4*)(d1 + head), nvec);
   const VecOut<NT2> out2((u32x4*)(d2 + head), nvec);
-  auto exact = [&](auto U_) {
-    constexpr int U = decltype(U_)::value;
-    u32x4 r[U];
-#pragma unroll
-    for (int j = 0; j < U; ++j) r[j] = in(j * kCopyBlock + tid);
-#pragma unroll
-    for (int j = 0; j < U; ++j) out1(j * kCopyBlock + tid, r[j]);
-#pragma unroll
-    for (int j = 0; j < U; ++j) out2(j * kCopyBlock + tid, r[j]);
-  };
-  if (nvec == kCopyBlock * 16) exact(std::integral_constant<int, 16>{});
-  else if (nvec == kCopyBlock * 8) exact(std::integral_constant<int, 8>{});
-  else if (nvec == kCopyBlock * 4) exact(std::integral_constant<int, 4>{});
+  // whole tiles of the usual sizes (one tile, a share of two): every load is issued before the first store, unpredicated
+  if (nvec == kCopyBlock * 16) { copy2_exact<NT, NT2, 16>(out1, out2, in, tid); }
+  else if (nvec == kCopyBlock * 8) { copy2_exact<NT, NT2, 8>(out1, out2, in, tid); }
   else {
     for (uint32_t b = 0; b < nvec; b += kCopyBlock * kCopyUnroll) {
       u32x4 r[kCopyUnroll];
 #pragma unroll
       for (int j = 0; j < kCopyUnroll; ++j) {
         const uint32_t idx = b + j * kCopyBlock + tid;
-        if (idx < nvec) r[j] = in(idx);
+        r[j] = idx < nvec ? in(idx) : u32x4{0, 0, 0, 0};
       }
 #pragma unroll
       for (int j = 0; j < kCopyUnroll; ++j) {
         const uint32_t idx = b + j * kCopyBlock + tid;
-        if (idx < nvec) { out1(idx, r[j]); out2(idx, r[j]); }
+        if (idx < nvec) out1(idx, r[j]);
       }
+#pragma unroll
+      for (int j = 0; j < kCopyUnroll; ++j) {
+        const uint32_t idx = b + j * kCopyBlock + tid;
+        if (idx < nvec) out2(idx, r[j]);
+      }
+      asm volatile("; two-destination copy, predicated" ::: "memory");   // (see copy2_exact)
     }
   }
   const uint32_t tail0 = head + (nvec << 4);

@@ -878,7 +878,10 @@ def test_rccl_loads_the_plugin_and_probes_every_device(name):
     assert "allreduce 1024.0" in log
 
 
-@pytest.mark.parametrize("seed", range(int(__import__("os").environ.get("FUSELINK_RANDOM_SEEDS", "10"))))
+_SEED0 = int(__import__("os").environ.get("FUSELINK_RANDOM_SEED_FIRST", "0"))
+
+
+@pytest.mark.parametrize("seed", range(_SEED0, _SEED0 + int(__import__("os").environ.get("FUSELINK_RANDOM_SEEDS", "10"))))
 def test_random_traffic_of_several_connections_arrives_intact(net, seed):
     """Random mixes of what the paths distinguish: 1 to 5 connections on one GPU; requests of 0 bytes, a few bytes, ragged
     lengths, whole chunks, more than the engine takes (launch pairs), more than the windows hold (waves); receives
@@ -894,7 +897,7 @@ def test_random_traffic_of_several_connections_arrives_intact(net, seed):
     net.reconfigure(NCCL_FUSELINK_LANES=lanes, NCCL_FUSELINK_CHUNKSIZE=chunk, NCCL_FUSELINK_WINDOW_UNITS=int(rng.choice([1, 2, 4])),
                     NCCL_FUSELINK_REFRESH_BATCH=cadence, NCCL_FUSELINK_COMPLETION=completion, NCCL_FUSELINK_ENGINE=engine,
                     NCCL_FUSELINK_ENGINE_SETS=int(rng.choice([1, 2, 3])), NCCL_FUSELINK_BATCH=int(rng.choice([2, 8, 32])),
-                    NCCL_FUSELINK_ONE_PASS=int(seed % 3 != 2))
+                    NCCL_FUSELINK_ONE_PASS=int(__import__("os").environ.get("FUSELINK_RANDOM_ONE_PASS", seed % 3 != 2)))
     net.set_credits([int(c) for c in rng.integers(0, 5, size=lanes)])
 
     def draw_size():
@@ -963,7 +966,15 @@ def test_random_traffic_of_several_connections_arrives_intact(net, seed):
         for q, n in enumerate(c["sizes"]):
             o = int(c["offs"][q])
             exp[o:o + n] = c["src_np"][o:o + n]
-        np.testing.assert_array_equal(c["dst"].cpu().numpy(), exp)
+        got = c["dst"].cpu().numpy()
+        if not np.array_equal(got, exp):    # say where: which request, which of its bytes, what lies there instead
+            bad = np.flatnonzero(got != exp)
+            runs = np.split(bad, np.flatnonzero(np.diff(bad) > 1) + 1)
+            q = int(np.searchsorted(c["offs"], bad[0], side="right")) - 1
+            raise AssertionError(f"seed {seed}: lanes {lanes} chunk {chunk} completion {completion} engine {engine}; connection {conns.index(c)} of {n_conn}: "
+                                 f"{bad.size} bytes differ in {len(runs)} runs, the first [{bad[0]}, {runs[0][-1] + 1}) = request {q} (size {c['sizes'][q]}, "
+                                 f"at {int(c['offs'][q])}) + {bad[0] - int(c['offs'][q])}; sizes {c['sizes']}; got {got[bad[0]:bad[0] + 8].tolist()} "
+                                 f"expected {exp[bad[0]:bad[0] + 8].tolist()}; runs {[(int(r[0]), int(r.size)) for r in runs[:8]]}")
         _close(net, c)
 
 

@@ -408,6 +408,8 @@ def test_test_hooks_are_refused_without_their_switch(fl, monkeypatch):
     ((3 << 20) + 77, 128 << 10, 4, 1, 5, 5, 5),   # source, windows and receive buffer equally misaligned: vectors with byte edges
     ((3 << 20) + 77, 128 << 10, 4, 1, 0, 0, 9),   # the receive buffer misaligned against source and windows: two copies from the source
     ((1 << 20) + 13, 100 * 128, 5, 3, 3, 0, 3),   # the windows misaligned against source and receive buffer
+    (5 * (256 << 10) + 6 * 32768 + 16392, 256 << 10, 5, 0, 0, 0, 0),   # a last tile of 16 KiB and a few bytes: the four-vector path
+    (3 * (64 << 10) + 16384, 64 << 10, 2, 1, 0, 0, 0),
     (300 << 20, 1 << 20, 16, 0, 0, 0, 0)])        # past 256 MiB: destination order, streaming loads and stores
 def test_a_launch_that_stages_and_delivers_equals_the_launch_pair(fl, nbytes, chunk, lanes, epoch_chunks, src_skew, win_skew, dst_skew):
     """flh_stage_deliver_uniform: table, header and windows are flh_stripe_uniform's, the receive buffer
@@ -508,3 +510,86 @@ def test_a_batch_launch_that_stages_and_delivers_equals_the_batch_pair(fl):
             g = bt["dsts"][i].cpu().numpy()
             np.testing.assert_array_equal(g[:s], bt["srcs_np"][i], err_msg=f"request {i}")
             assert not g[s:].any()
+
+
+_LAST = [1, 7, 15, 16, 17, 31, 32, 255, 256, 4095, 4096, 4097, 8191, 8192, 12288, 16383, 16384, 16385, 16392, 16399, 16400, 20480, 24576, 28672,
+         32752, 32760, 32767]
+
+
+@pytest.mark.parametrize("skew", [0, 4])
+def test_every_size_class_of_a_last_tile_reaches_both_destinations(fl, skew):
+    """The copy with two destinations takes different paths by the number of 16-byte vectors in a tile (whole tiles
+    unrolled, anything else in a predicated loop, bytes at either edge).  Messages of a chunk, a tile and a last tile of
+    every size class -- around every power of two, sixteen kilobytes and a few bytes, a tile less a few -- go through the
+    launch that stages and delivers, the launch that stages and carries, and the engine's two kinds of batch that do
+    the same at system scope (one-tile and, with the share limit at 0, two-tile shares); source, windows and
+    destinations share a misalignment of `skew` bytes so that the vector path is the one taken.  Windows, landing
+    windows and destinations must hold exactly the message, and nothing beside it."""
+    core, torch, _lib = fl
+    lib = _lib.load()
+    lib.flh_tune.argtypes = [C.c_char_p, C.c_int64]
+    lanes, chunk = 2, 64 << 10
+    credits = [1, 1]
+    rng = np.random.default_rng(77 + skew)
+    cap = 4 * chunk
+    status = core.new_status()
+
+    def buffers(n, fill):
+        raw = [torch.full((n + 64,), fill, dtype=torch.uint8, device="cuda") for _ in range(lanes)]
+        return raw, [t[skew:skew + n] for t in raw]
+
+    def check(name, last, src_np, exp_w, lane_bytes, stage, land, dst_raw, fill):
+        for l in range(lanes):
+            np.testing.assert_array_equal(stage[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"{name}, last {last}: staging window {l}")
+            assert (stage[l].cpu().numpy()[lane_bytes[l]:] == 0).all(), f"{name}, last {last}: staging window {l} written beyond its bytes"
+            if land is not None:
+                np.testing.assert_array_equal(land[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"{name}, last {last}: landing window {l}")
+                assert (land[l].cpu().numpy()[lane_bytes[l]:] == 0).all(), f"{name}, last {last}: landing window {l} written beyond its bytes"
+        if dst_raw is not None:
+            back = dst_raw.cpu().numpy()
+            np.testing.assert_array_equal(back[32 + skew:32 + skew + src_np.size], src_np, err_msg=f"{name}, last {last}: destination")
+            assert (back[:32 + skew] == fill).all() and (back[32 + skew + src_np.size:] == fill).all(), f"{name}, last {last}: bytes around the destination"
+
+    for share_limit in (-1, 0):
+        _lib.check(lib.flh_tune(b"lane_share1_tiles", share_limit))
+        eng = C.c_void_p()
+        _lib.check(lib.flh_engine_create(0, 0, 200, 1, C.byref(eng)))
+        try:
+            for last in _LAST:
+                nbytes = chunk + 32768 + last
+                src_np = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+                src_raw = torch.zeros(nbytes + 64, dtype=torch.uint8, device="cuda")
+                src = src_raw[skew:skew + nbytes]
+                src.copy_(torch.from_numpy(src_np))
+                exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=np.asarray(credits, dtype=np.uint32), quantum=chunk, total_bytes=nbytes,
+                                                     chunk_bytes=chunk, mode=ob.SCHED_RESET_OFFSETS, state=_state(0))
+                lane_bytes = [int(x) for x in exp_h["lane_bytes"][:lanes]]
+                exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+                u = core.uniform_params(nbytes, chunk, credits)
+                for name in (("deliver", "carry") if share_limit == -1 else ()) + ("engine loop", "engine send"):
+                    _, stage = buffers(cap, 0)
+                    _, land = buffers(cap, 0)
+                    W = core.make_windows([t.data_ptr() for t in stage], [cap] * lanes)
+                    L = core.make_windows([t.data_ptr() for t in land], [cap] * lanes)
+                    dst_raw = torch.full((nbytes + 128,), 0xEE, dtype=torch.uint8, device="cuda")
+                    dst = dst_raw[32 + skew:32 + skew + nbytes]
+                    torch.cuda.synchronize()
+                    if name == "deliver":
+                        core.stage_deliver_uniform(src, dst, W, u, status)
+                    elif name == "carry":
+                        core.stripe_uniform_carry(src, W, L, u, status)
+                    else:
+                        b = core.batch_params([src], [dst], chunk, credits)
+                        seq = C.c_uint64()
+                        if name == "engine loop":
+                            _lib.check(lib.flh_engine_submit(eng, C.byref(b), C.byref(W), None, None, status.data_ptr(), C.byref(seq), None))
+                        else:
+                            _lib.check(lib.flh_engine_submit_wire(eng, SEND, C.byref(b), C.byref(W), C.byref(L), None, None, status.data_ptr(), C.byref(seq), None))
+                        _wait(lib, eng, seq.value)
+                    torch.cuda.synchronize()
+                    assert int(status.item()) == 0
+                    check(name, last, src_np, exp_w, lane_bytes, stage, land if name in ("carry", "engine send") else None,
+                          dst_raw if name in ("deliver", "engine loop") else None, 0xEE)
+        finally:
+            _lib.check(lib.flh_tune(b"lane_share1_tiles", -1))
+            _lib.check(lib.flh_engine_destroy(eng))
