@@ -593,3 +593,76 @@ def test_every_size_class_of_a_last_tile_reaches_both_destinations(fl, skew):
         finally:
             _lib.check(lib.flh_tune(b"lane_share1_tiles", -1))
             _lib.check(lib.flh_engine_destroy(eng))
+
+
+@pytest.mark.parametrize("block", range(int(__import__("os").environ.get("FUSELINK_TWO_DEST_BLOCKS", "2"))))
+def test_random_messages_through_the_two_destination_paths(fl, block):
+    """Seeded random messages -- length, chunk size (any multiple of 128), lanes, credit row, place in the credit epoch, and
+    the misalignments of source, windows and destination against each other -- through the launch that stages and
+    delivers, the launch that stages and carries, and the engine's loop and send batches: windows, landing windows and
+    destination must be the oracle's, byte for byte, and the bytes beside them untouched.  Forty cases per block."""
+    core, torch, _lib = fl
+    lib = _lib.load()
+    rng = np.random.default_rng(31000 + block)
+    status = core.new_status()
+    eng = C.c_void_p()
+    _lib.check(lib.flh_engine_create(0, 0, 200, 1, C.byref(eng)))
+    try:
+        for case in range(40):
+            lanes = int(rng.integers(1, 9))
+            chunk = int(rng.choice([128, 4096, 12800, 32768, 65536, 98304, 262144]))
+            n_chunks = int(rng.integers(1, 24))
+            nbytes = max(1, (n_chunks - 1) * chunk + int(rng.integers(1, chunk + 1)))
+            credits = rng.integers(0, 5, size=lanes).astype(np.uint32)
+            epoch = int(rng.integers(0, 20)) * chunk
+            same = rng.random() < 0.6                       # mostly the vector path: every address misaligned alike
+            s0 = int(rng.integers(0, 16))
+            skews = (s0, s0, s0) if same else tuple(int(x) for x in rng.integers(0, 16, size=3))
+            src_np = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+            exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=nbytes, chunk_bytes=chunk,
+                                                 mode=ob.SCHED_RESET_OFFSETS, state=_state(epoch))
+            lane_bytes = [int(x) for x in exp_h["lane_bytes"][:lanes]]
+            exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
+            src_raw = torch.zeros(nbytes + 64, dtype=torch.uint8, device="cuda")
+            src = src_raw[skews[0]:skews[0] + nbytes]
+            src.copy_(torch.from_numpy(src_np))
+            u = core.uniform_params(nbytes, chunk, credits.tolist(), epoch_bytes=epoch)
+            for name in ("deliver", "carry", "engine loop", "engine send"):
+                if name.startswith("engine") and (n_chunks > 500 or chunk % 128):
+                    continue
+                tag = f"block {block} case {case} {name}: {nbytes} bytes, chunk {chunk}, lanes {lanes}, credits {credits.tolist()}, epoch {epoch}, skews {skews}"
+                stage_raw = [torch.full((b + 64,), 0x5A, dtype=torch.uint8, device="cuda") for b in lane_bytes]
+                land_raw = [torch.full((b + 64,), 0x5A, dtype=torch.uint8, device="cuda") for b in lane_bytes]
+                W = core.make_windows([t.data_ptr() + skews[1] for t in stage_raw], lane_bytes)
+                L = core.make_windows([t.data_ptr() + skews[1] for t in land_raw], lane_bytes)
+                dst_raw = torch.full((nbytes + 128,), 0xEE, dtype=torch.uint8, device="cuda")
+                dst = dst_raw[32 + skews[2]:32 + skews[2] + nbytes]
+                torch.cuda.synchronize()
+                if name == "deliver":
+                    core.stage_deliver_uniform(src, dst, W, u, status)
+                elif name == "carry":
+                    core.stripe_uniform_carry(src, W, L, u, status)
+                else:
+                    b = core.batch_params([src], [dst], chunk, credits.tolist(), epoch_bytes=epoch)
+                    seq = C.c_uint64()
+                    if name == "engine loop":
+                        _lib.check(lib.flh_engine_submit(eng, C.byref(b), C.byref(W), None, None, status.data_ptr(), C.byref(seq), None))
+                    else:
+                        _lib.check(lib.flh_engine_submit_wire(eng, SEND, C.byref(b), C.byref(W), C.byref(L), None, None, status.data_ptr(), C.byref(seq), None))
+                    _wait(lib, eng, seq.value)
+                torch.cuda.synchronize()
+                assert int(status.item()) == 0, tag
+                for l in range(lanes):
+                    for kind, raw in (("staging", stage_raw), ("landing", land_raw)):
+                        if kind == "landing" and name not in ("carry", "engine send"):
+                            continue
+                        g = raw[l].cpu().numpy()
+                        np.testing.assert_array_equal(g[skews[1]:skews[1] + lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"{tag}: {kind} window {l}")
+                        assert (g[:skews[1]] == 0x5A).all() and (g[skews[1] + lane_bytes[l]:] == 0x5A).all(), f"{tag}: bytes beside {kind} window {l}"
+                if name in ("deliver", "engine loop"):
+                    back = dst_raw.cpu().numpy()
+                    lo = 32 + skews[2]
+                    np.testing.assert_array_equal(back[lo:lo + nbytes], src_np, err_msg=f"{tag}: destination")
+                    assert (back[:lo] == 0xEE).all() and (back[lo + nbytes:] == 0xEE).all(), f"{tag}: bytes beside the destination"
+    finally:
+        _lib.check(lib.flh_engine_destroy(eng))
