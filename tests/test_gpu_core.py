@@ -700,8 +700,9 @@ def test_forced_streaming_modes_move_the_same_bytes(fl, mode_out, mode_in):
 
 def test_launches_record_into_a_hip_graph_and_replay(fl):
     """No entry point on the data path allocates, clears or synchronizes, so a caller may record
-    schedule -> stripe -> reassemble into a HIP graph.  Every replay, with eager work and synchronizations of
-    the program's own in between, must give what the eager launches give for the source bytes of that moment."""
+    schedule -> stripe -> reassemble into a HIP graph, and likewise the launch that stages and delivers and the
+    one that stages and carries.  Every replay, with eager work and synchronizations of the program's own in between,
+    must give what the eager launches give for the source bytes of that moment."""
     core, torch = fl
     rng = np.random.default_rng(31337)
     lanes, chunk = 8, 65536
@@ -710,9 +711,13 @@ def test_launches_record_into_a_hip_graph_and_replay(fl):
     exp_t, exp_h, _ = ob.credit_schedule(n_lanes=lanes, credits=credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk)
     lane_bytes = [int(b) for b in exp_h["lane_bytes"][:lanes]]
     src = torch.zeros(total, dtype=torch.uint8, device="cuda")
-    dst_fused, dst_table = torch.zeros_like(src), torch.zeros_like(src)
+    dst_fused, dst_table, dst_deliver = torch.zeros_like(src), torch.zeros_like(src), torch.zeros_like(src)
     wins = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
     w = core.make_windows([t.data_ptr() for t in wins], lane_bytes)
+    wins2 = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
+    land = [torch.zeros(max(b, 1), dtype=torch.uint8, device="cuda") for b in lane_bytes]
+    w2 = core.make_windows([t.data_ptr() for t in wins2], lane_bytes)
+    wl = core.make_windows([t.data_ptr() for t in land], lane_bytes)
     u = core.uniform_params(total, chunk, credits.tolist())
     out = core.new_schedule_buffers(len(exp_t))
     sched_out = core.new_schedule_buffers(len(exp_t))
@@ -728,21 +733,26 @@ def test_launches_record_into_a_hip_graph_and_replay(fl):
         sched = core.schedule(n_lanes=lanes, credits=d_credits, quantum=chunk, total_bytes=total, chunk_bytes=chunk, out=sched_out)
         core.stripe(src, w, sched, status)
         core.reassemble(dst_table, w, sched, status)
+        # one launch that stages and delivers; one that stages and carries into landing windows
+        core.stage_deliver_uniform(src, dst_deliver, w2, u, status)
+        core.stripe_uniform_carry(src, w2, wl, u, status)
     for rep in range(4):
         src_np = rng.integers(0, 256, size=total, dtype=np.uint8)
         src.copy_(torch.from_numpy(src_np))
         dst_fused.zero_()
         dst_table.zero_()
-        for t in wins:
+        dst_deliver.zero_()
+        for t in wins + wins2 + land:
             t.zero_()
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         assert int(status.item()) == 0
-        assert torch.equal(dst_fused, src) and torch.equal(dst_table, src), f"replay {rep}"
+        assert torch.equal(dst_fused, src) and torch.equal(dst_table, src) and torch.equal(dst_deliver, src), f"replay {rep}"
         exp_w = ob.cpu_stripe(src_np, exp_t, lane_bytes)
         for l in range(lanes):
-            np.testing.assert_array_equal(wins[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"replay {rep} lane {l}")
+            for name, ws in (("windows", wins), ("windows of the delivering launch", wins2), ("landing windows", land)):
+                np.testing.assert_array_equal(ws[l].cpu().numpy()[:lane_bytes[l]], exp_w[l][:lane_bytes[l]], err_msg=f"replay {rep} {name} lane {l}")
         for f in ob.DESC_DTYPE.names:
             np.testing.assert_array_equal(out.table_numpy()[f], exp_t[f], err_msg=f"replay {rep} field {f}")
             np.testing.assert_array_equal(sched_out.table_numpy()[f], exp_t[f], err_msg=f"replay {rep} field {f} (scheduler kernel)")
