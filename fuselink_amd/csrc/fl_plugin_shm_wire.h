@@ -40,6 +40,9 @@ constexpr int kShmSetsMax = 8;
 constexpr uint32_t kPairWaves = 64;      // wave records a pair's ring holds (more than the landing sets there can be)
 constexpr uint32_t kPairConns = 256;     // connections between two processes that share the pair
 constexpr uint32_t kPairMrs = 64;        // registrations of the receiver that the sender can write into directly
+// Every wave, whichever way it travels, is numbered only while fewer than `sets` waves are unconsumed (wire_set_free), so
+// a record of the ring is never written again before the receiver has taken it.
+static_assert(kPairWaves > (uint32_t)kShmSetsMax, "the ring of wave records must hold every wave that can be unconsumed");
 
 struct WaveReq {                   // one request of a wave
   uint32_t conn;                   // the connection's number within the pair
