@@ -35,12 +35,16 @@ WORKLOADS = {
 # Bytes per launch of the striping kernel between the L2 caches and the fabric behind them (Infinity Cache, then HBM),
 # from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the plain
 # copy kernel of known size.  None where no such run has been recorded for the workload.
-MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134277565, "cfg5_stress_1GiB_64KiB_16lanes": 2148014006,
+MEASURED_TRAFFIC = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": 134277565,
+                    "cfg2_grad_bucket_64MiB_256KiB_8lanes/carry": 201425313, "cfg2_grad_bucket_64MiB_256KiB_8lanes/deliver": 201554230,
+                    "cfg5_stress_1GiB_64KiB_16lanes": 2148014006,
                     "cfg5_stress_1GiB_64KiB_16lanes/17 waves": 126482128,
                     "cfg3_expert_parallel_256_blocks_8lanes": 1786029836, "cfg4_paged_kv_2x4096_pages_8lanes": 268579065}
 # ... and the summary under profiles/ that each figure comes from (the counters are not read by this script: `traffic` is
 # a recorded measurement of the same kernel on the same workload, the file holds the commands that made it)
 TRAFFIC_SOURCE = {"cfg2_grad_bucket_64MiB_256KiB_8lanes": "profiles/copy_kernels_cfg2_l2_fabric_traffic.md",
+                  "cfg2_grad_bucket_64MiB_256KiB_8lanes/carry": "profiles/copy_kernels_cfg2_l2_fabric_traffic.md",
+                  "cfg2_grad_bucket_64MiB_256KiB_8lanes/deliver": "profiles/copy_kernels_cfg2_l2_fabric_traffic.md",
                   "cfg5_stress_1GiB_64KiB_16lanes": "profiles/copy_kernels_cfg5_l2_fabric_traffic.md",
                   "cfg5_stress_1GiB_64KiB_16lanes/17 waves": "profiles/copy_kernels_cfg5_l2_fabric_traffic.md",
                   "cfg3_expert_parallel_256_blocks_8lanes": "profiles/copy_kernels_cfg3_l2_fabric_traffic.md",
@@ -636,6 +640,15 @@ def main() -> int:
     else:
         kernel_name = "fl_copy_tiles<0> (stripe)"
 
+    # which recorded counter measurement, if any, covers this run's dominant kernel on this workload
+    if args.lanes or waves or twaves or (kind == "blocks" and args.blocks != 256):
+        traffic_key = None
+    elif cwaves:
+        traffic_key = f"{args.workload}/{len(cwaves)} waves"
+    elif carry or deliver:
+        traffic_key = f"{args.workload}/{args.path}"
+    else:
+        traffic_key = args.workload
     out = {
         # the headline metric's own wording for the workload it is quoted on; `value` is its GB/s part, the percentage of the
         # HBM peak and the chunks per second travel as fields of their own (pct_of_hbm_peak, chunks_per_s)
@@ -686,12 +699,11 @@ def main() -> int:
                          "the same kernels with HBM as the only server are in hbm_only (measured in this run; as a whole workload: bench.py --workload cfg5_stress_1GiB_64KiB_16lanes --cache-waves 0)"
                          if 3 * nbytes <= (256 << 20) else "beyond the 256 MB Infinity Cache" + (
                              "; moved in cache-resident waves, the windows' traffic stays in the cache" if cwaves else ": every byte is served by HBM"))) if kind == "uniform" else None,
-                     "traffic": (None if args.lanes else MEASURED_TRAFFIC.get(f"{args.workload}/{len(cwaves)} waves") if cwaves else None if (waves or twaves) else
-                                 MEASURED_TRAFFIC.get(args.workload) if (kind != "blocks" or args.blocks == 256) else None)},
+                     "traffic": MEASURED_TRAFFIC.get(traffic_key) if traffic_key else None},
     }
     if out["roofline"]["traffic"] is not None:
         # a recorded measurement (two rocprofv3 --pmc runs, scaled by a plain copy of known size), not read in this run
-        out["roofline"]["traffic_source"] = TRAFFIC_SOURCE.get(f"{args.workload}/{len(cwaves)} waves" if cwaves else args.workload)
+        out["roofline"]["traffic_source"] = TRAFFIC_SOURCE.get(traffic_key)
     if hbm_only is not None:
         out["roofline"]["hbm_only"] = hbm_only
 
