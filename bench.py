@@ -499,6 +499,24 @@ def main() -> int:
     copy_us = mean(profiled(copies, 128)["copy"])
     assert torch.equal(src, dst)
 
+    def runtime_copy_us(d, s, reps):
+        """The runtime's own device-to-device copy of the same bytes (hipMemcpyAsync, which torch's copy_ issues for
+        contiguous bytes on one device): what a copy that stripes nothing gets from the vendor's path.  HIP events
+        around every copy on the launch stream, back to back, mean -- as the library's per-launch timing does."""
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                d.copy_(s)
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+            for a, b in evs:
+                a.record(stream)
+                d.copy_(s)
+                b.record(stream)
+        stream.synchronize()
+        return mean([a.elapsed_time(b) * 1e3 for a, b in evs])
+
+    rt_copy_us = runtime_copy_us(dst[:msg_bytes], src[:msg_bytes], min(args.steps, 100))
+    assert torch.equal(src, dst)
+
     # ---- the same step over rotating user buffers: the timed loop above re-reads one source and rewrites one
     # destination, which the 256 MB Infinity Cache partly holds from step to step; with enough pairs in rotation
     # (1 GiB of user buffers) every step meets them cold, as a stream of distinct messages would.  Reported
@@ -568,6 +586,7 @@ def main() -> int:
         hb_pairs()
         per_h = profiled(hb_pairs, 4 * hb_reps)
         hb_copy_us = mean(profiled(hb_copies, 2 * hb_reps)["copy"])
+        hb_rt_us = runtime_copy_us(hb_dst, hb_src, hb_reps)
         torch.cuda.synchronize()
         assert int(status.item()) == 0 and torch.equal(hb_src, hb_dst)
         hb_frac = lambda us: round(2 * hb_n / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
@@ -575,6 +594,7 @@ def main() -> int:
                     "stripe_us": round(mean(per_h["stripe"]), 1), "stripe_frac": hb_frac(mean(per_h["stripe"])),
                     "reassemble_us": round(mean(per_h["reassemble"]), 1), "reassemble_frac": hb_frac(mean(per_h["reassemble"])),
                     "plain_copy_us": round(hb_copy_us, 1), "plain_copy_frac": hb_frac(hb_copy_us),
+                    "hipMemcpyAsync_us": round(hb_rt_us, 1), "hipMemcpyAsync_frac": hb_frac(hb_rt_us),
                     "timing": f"HIP events around every launch, mean of {hb_reps} launch pairs back to back, measured in this run",
                     "command": "python bench.py"}
         del hb_src, hb_dst
@@ -679,7 +699,7 @@ def main() -> int:
         "chunks_per_s": round(n_chunks / (ms_per_step * 1e-3), 1),
         "kernels_us": {"schedule": round(sched_us, 2), out_k: round(stripe_us, 2), in_k: round(reasm_us, 2),
                        out_k + "_min": round(stripe_min, 2), in_k + "_min": round(reasm_min, 2),
-                       "plain_copy_same_bytes": round(copy_us, 2)},
+                       "plain_copy_same_bytes": round(copy_us, 2), "hipMemcpyAsync_same_bytes": round(rt_copy_us, 2)},
         "stripe_reassemble_pair_GBps": round(algo_bytes_step / (pair_us * 1e-6) / 1e9, 1),
         "scheduler_kernel": "standalone launch, not part of the fused step" if (fused or cwaves) else "first launch of every message",
         # one launch schedules a whole message; below 1000 chunks its cost is the flat launch time, not a per-1k rate
